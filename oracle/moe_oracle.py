@@ -1,0 +1,337 @@
+"""CPU restatement (NumPy) of the reference's MoE token-dispatch ops.
+
+TEST INFRASTRUCTURE ONLY.  This module is the checker that the HIP path is
+compared against; nothing in the shipped package imports it.  Only tests/,
+__graft_entry__.smoke() and bench.py's cpu_baseline leg may call it.
+
+Every function restates an algorithm of the reference (paths relative to the
+reference tree) and cites the lines it follows.  The style is deliberately the
+one the reference's own test references use (one-hot + cumsum locations and a
+Python scatter loop, tests/python/op/cuda/test_cuda_moe.py:114-137), so that
+timing it gives "the NumPy reference path" of the baseline.
+
+Parity status of each function (what pins it, beyond re-reading the source):
+  capacity            closed form; hand-computed cases in tests/test_oracle_moe.py
+  softmax_rows        scipy.special.softmax / fp64 evaluation at 1e-6
+  select_topk         brute-force Python loop; numpy argmax first-max rule.
+                      TIE-BREAK OF THE REFERENCE IS "parity unpinned": the
+                      reference selects with a TVM-compiled argmax whose source
+                      is absent (3rdparty/tvm is an empty submodule); its tests
+                      only compare against np.argmax on tie-free random input.
+                      We fix ties -> lowest expert index.
+  moe_encode          brute-force token loop (tests), invariants (bijection of
+                      locations onto [0,kept), used_out closed form, rows
+                      bit-equal to source rows), chained-partition identity
+  moe_encode_bpr      brute-force per-expert sort; partition independence of the
+                      drop set.  STABILITY OF THE REFERENCE ARGSORT IS "parity
+                      unpinned" (TVM argsort, source absent); we fix a stable
+                      descending order, ties by ascending token id.
+  moe_merge_masks /
+  moe_redispatch      identity "partitioned == un-partitioned" of
+                      test_cuda_moe.py:384-471
+  moe_encode_top2     dense einsum form of docker/resources/sharded_moe.py:253-324
+                      at tiny sizes; identity with two chained top-1 encodes
+  moe_decode          round trip decode(encode(x), gate=1) == x on kept tokens
+"""
+import numpy as np
+
+F32_EPS = np.float32(1.1920929e-07)  # torch.finfo(torch.float32).eps, sharded_moe.py:310
+
+
+# --------------------------------------------------------------------------
+# T1: shape contract
+# --------------------------------------------------------------------------
+def capacity(S, E, capacity_factor):
+    """C = int(float(cf) * ((S + E - 1) / E)): integer ceil-div, float multiply,
+    truncation.  src/op/dialect/cuda/moe.cc:107-109, src/op/declare/moe.cc:46."""
+    return int(np.float32(capacity_factor) * np.float32((S + E - 1) // E))
+
+
+# --------------------------------------------------------------------------
+# A0: gate softmax (outside the reference op; models/benchmark/pytorch/utils.py:565-573)
+# --------------------------------------------------------------------------
+def softmax_rows(logits):
+    """p[s,:] = exp(x - max) / sum_e exp(x - max), fp32, sum taken in expert order."""
+    x = np.asarray(logits, dtype=np.float32)
+    ex = np.exp(x - x.max(axis=1, keepdims=True), dtype=np.float32)
+    acc = np.zeros(x.shape[0], dtype=np.float32)
+    for j in range(x.shape[1]):  # sequential fp32 sum over experts
+        acc = acc + ex[:, j]
+    return (ex / acc[:, None]).astype(np.float32)
+
+
+# --------------------------------------------------------------------------
+# A1 / A2 front end: top-1 / top-2 selection on the array the op is given
+# --------------------------------------------------------------------------
+def select_topk(gate, k=1, gate_is_logits=False):
+    """Returns (idx [k,S] int32, val [k,S] fp32).
+
+    idx[0] = argmax_e gate[s,e] (first max; src/op/dialect/cuda/moe.cc:177-195,
+    tests/python/op/cuda/test_cuda_moe.py:115).  idx[1] = argmax with idx[0]
+    masked to -inf (docker/resources/sharded_moe.py:275-278, noise dropped).
+    val = gate[s, idx] (moe.cc:232-250: sum_e gate*onehot), or the softmax
+    probability of that expert when the array holds logits."""
+    g = np.asarray(gate, dtype=np.float32)
+    S, E = g.shape
+    rows = np.arange(S)
+    prob = softmax_rows(g) if gate_is_logits else g
+    idx = np.empty((k, S), dtype=np.int32)
+    val = np.empty((k, S), dtype=np.float32)
+    i1 = np.argmax(g, axis=1).astype(np.int32) if S else np.zeros(0, np.int32)
+    idx[0] = i1
+    val[0] = prob[rows, i1]
+    if k == 2:
+        assert E >= 2
+        masked = g.copy()
+        masked[rows, i1] = -np.inf
+        # argmax of a row that is all -inf apart from i1 must not return i1
+        i2 = np.argmax(masked, axis=1).astype(np.int32)
+        clash = i2 == i1
+        if clash.any():
+            i2[clash] = np.where(i1[clash] == 0, 1, 0)
+        idx[1] = i2
+        val[1] = prob[rows, i2]
+    return idx, val
+
+
+def _ranks(idx0, E):
+    """rank[s] = #{t < s : idx0[t] == idx0[s]}, via one-hot cumsum - 1
+    (test_cuda_moe.py:116-123).  idx0 < 0 means "no expert" and gets rank 0."""
+    S = idx0.shape[0]
+    if S == 0:
+        return np.zeros(0, np.int32), np.zeros(E, np.int64)
+    onehot = idx0[:, None] == np.arange(E, dtype=np.int32)[None, :]
+    cums = np.cumsum(onehot, axis=0, dtype=np.int32)
+    safe = np.where(idx0 >= 0, idx0, 0)
+    rank = cums[np.arange(S), safe] - 1
+    rank = np.where(idx0 >= 0, rank, 0).astype(np.int32)
+    return rank, cums[-1].astype(np.int64)
+
+
+# --------------------------------------------------------------------------
+# A3: gen_location (tutel_moe_dispatch.cu:164-212)
+# --------------------------------------------------------------------------
+def gen_location(idx0, used_in, C, M, E):
+    """Returns (idx, loc, used_out, elems).  loc = rank among tokens of the same
+    expert (written for dropped tokens too, :198); dropped <=> loc >= C - used_in
+    (:199-201) -> idx = -1; used_out = min(used_in + cnt, C) (:207-209);
+    elems = (used_out - used_in) * M (:210)."""
+    idx0 = np.asarray(idx0, dtype=np.int32)
+    used_in = np.asarray(used_in, dtype=np.int32)
+    rank, cnt = _ranks(idx0, E)
+    safe = np.where(idx0 >= 0, idx0, 0)
+    drop = (idx0 >= 0) & (rank >= (C - used_in[safe]))
+    idx = np.where(drop, -1, idx0).astype(np.int32)
+    used_out = np.minimum(used_in.astype(np.int64) + cnt, C).astype(np.int32)
+    elems = ((used_out.astype(np.int64) - used_in) * M).astype(np.uint64)
+    return idx, rank, used_out, elems
+
+
+# --------------------------------------------------------------------------
+# A4: encode_forward scatter (tutel_moe_dispatch.cu:61-81, launchers :461-484)
+# --------------------------------------------------------------------------
+def scatter_rows(data, idx, loc, E, C, avail=None):
+    """Zero [E,C,M]; for tokens with 0<=idx<E, 0<=loc<C (and loc < avail[idx] when
+    given): out[idx, loc, :] = data[s, :].  The Python loop is the reference's
+    test reference (test_cuda_moe.py:124-127)."""
+    S, M = data.shape
+    out = np.zeros((E, C, M), dtype=data.dtype)
+    for s in range(S):
+        e, l = int(idx[s]), int(loc[s])
+        if 0 <= e < E and 0 <= l < C and (avail is None or l < avail[e]):
+            out[e, l, :] = data[s, :]
+    return out
+
+
+def scatter_rows_fast(data, idx, loc, E, C):
+    """Vectorised form of scatter_rows (same result; used where the loop is too slow)."""
+    S, M = data.shape
+    out = np.zeros((E, C, M), dtype=data.dtype)
+    ok = (idx >= 0) & (idx < E) & (loc >= 0) & (loc < C)
+    out[idx[ok], loc[ok]] = data[ok]
+    return out
+
+
+# --------------------------------------------------------------------------
+# A.1: raf.op.moe_encode (moe.cc:346-396)
+# --------------------------------------------------------------------------
+def moe_encode(data, gate, used_in, capacity_factor=1.0, gate_is_logits=False,
+               C=None, fast_scatter=False):
+    """Returns the reference 5-tuple (src/op/declare/moe.cc:48-58):
+    gates_s [S] fp32, indices_locations [2,S] int32, used_capacity [E] int32,
+    elements_per_expert [E] uint64, dispatched [E,C,M]."""
+    data = np.asarray(data)
+    S, M = data.shape
+    E = gate.shape[1]
+    if C is None:
+        C = capacity(S, E, capacity_factor)
+    sel, val = select_topk(gate, 1, gate_is_logits)
+    idx, loc, used_out, elems = gen_location(sel[0], used_in, C, M, E)
+    fn = scatter_rows_fast if fast_scatter else scatter_rows
+    disp = fn(data, idx, loc, E, C)
+    return val[0], np.stack([idx, loc]).astype(np.int32), used_out, elems, disp
+
+
+# --------------------------------------------------------------------------
+# A.2: raf.op.moe_encode_batch_prioritized (moe.cc:415-729,
+#      tutel_moe_dispatch.cu:259-363, test reference test_cuda_moe.py:270-309)
+# --------------------------------------------------------------------------
+def moe_encode_bpr(data, gate, n_partitions=1, partition_id=0, capacity_factor=1.0,
+                   gate_is_logits=False, C=None, priorities=None, fast_scatter=False):
+    """`priorities`, when given, replaces gates0 as the sort key (used to re-sort
+    keys a device emitted, since exp() is not bit-portable)."""
+    data = np.asarray(data)
+    S0, M = data.shape
+    E = gate.shape[1]
+    P = int(n_partitions)
+    S = S0 // P
+    if C is None:
+        C = capacity(S, E, capacity_factor)
+    sel, val = select_topk(gate, 1, gate_is_logits)
+    idx0, gates0 = sel[0], val[0]
+    key = gates0 if priorities is None else np.asarray(priorities, dtype=np.float32)
+    # descending, stable: ties keep ascending token order (moe.cc:701-719 argsort,
+    # is_ascend=false; np.argsort(-x) in test_cuda_moe.py:189)
+    order = np.argsort(-key.astype(np.float64), kind="stable")
+    # pass 1 (:276-313): rank within expert in priority order, keep = rank < C
+    rank_sorted, _ = _ranks(idx0[order], E)
+    keep = np.empty(S0, dtype=bool)
+    keep[order] = rank_sorted < C
+    # pass 2 (:317-356): compact locations over this partition's kept tokens
+    lo = partition_id * S
+    pidx0 = idx0[lo:lo + S]
+    pkeep = keep[lo:lo + S]
+    rank_kept, cnt_kept = _ranks(np.where(pkeep, pidx0, -1).astype(np.int32), E)
+    idx = np.where(pkeep, pidx0, -1).astype(np.int32)
+    loc = np.where(pkeep, rank_kept, -1).astype(np.int32)
+    used_out = np.minimum(cnt_kept, C).astype(np.int32)         # :358-360
+    elems = (used_out.astype(np.int64) * M).astype(np.uint64)   # :361
+    fn = scatter_rows_fast if fast_scatter else scatter_rows
+    disp = fn(data[lo:lo + S], idx, loc, E, C)
+    return gates0[lo:lo + S].copy(), np.stack([idx, loc]).astype(np.int32), used_out, elems, disp
+
+
+# --------------------------------------------------------------------------
+# A.3: raf.op.moe_merge_masks (moe.cc:731-823, tutel_moe_dispatch.cu:214-255)
+# --------------------------------------------------------------------------
+def moe_merge_masks(indlocs, E):
+    P = len(indlocs)
+    S = indlocs[0].shape[1]
+    out = np.empty((2, P * S), dtype=np.int32)
+    off = np.zeros(E, dtype=np.int64)
+    for p, il in enumerate(indlocs):
+        idx, loc = il[0], il[1]
+        kept = idx >= 0
+        safe = np.where(kept, idx, 0)
+        out[0, p * S:(p + 1) * S] = np.where(kept, idx, -1)
+        out[1, p * S:(p + 1) * S] = np.where(kept, loc + off[safe], -1)
+        off += np.bincount(idx[kept], minlength=E)[:E]
+    return out
+
+
+# --------------------------------------------------------------------------
+# A.4: raf.op.moe_redispatch (moe.cc:826-943, tutel_moe_dispatch.cu:365-408)
+# --------------------------------------------------------------------------
+def moe_redispatch(bufs, indlocs):
+    """out[e, off_p[e] + r, :] = buf_p[e, r, :] for r < kept_p[e].  Rows the
+    reference leaves uninitialised are defined as zero here."""
+    E, C, M = bufs[0].shape
+    out = np.zeros((E, C, M), dtype=bufs[0].dtype)
+    off = np.zeros(E, dtype=np.int64)
+    for buf, il in zip(bufs, indlocs):
+        idx = il[0]
+        cnt = np.bincount(idx[idx >= 0], minlength=E)[:E]
+        for e in range(E):
+            n = int(min(cnt[e], C - off[e]))
+            if n > 0:
+                out[e, off[e]:off[e] + n] = buf[e, :n]
+        off += cnt
+    return out
+
+
+# --------------------------------------------------------------------------
+# A.5: raf.op.moe_decode (moe.cc:1228-1311, tutel_moe_dispatch.cu:46-55,110-116,
+#      test reference test_cuda_moe.py:1157-1165)
+# --------------------------------------------------------------------------
+def _to_f32(a):
+    return np.asarray(a).astype(np.float32)
+
+
+def moe_decode(expert_out, gates_s, indloc, k=1, round_fn=None):
+    """out[s] = sum over the k slots of gates_s * expert_out[idx, loc]; products and
+    the sum are fp32 (each rounded), one final rounding to the storage dtype via
+    round_fn.  Slot j of token s lives at column j*S + s (slot-major)."""
+    E, C, M = expert_out.shape
+    S = indloc.shape[1] // k
+    acc = np.zeros((S, M), dtype=np.float32)
+    x = _to_f32(expert_out)
+    for j in range(k):
+        idx = indloc[0, j * S:(j + 1) * S]
+        loc = indloc[1, j * S:(j + 1) * S]
+        g = np.asarray(gates_s[j * S:(j + 1) * S], dtype=np.float32)
+        ok = (idx >= 0) & (idx < E) & (loc >= 0) & (loc < C)
+        rows = np.zeros((S, M), dtype=np.float32)
+        rows[ok] = x[idx[ok], loc[ok]] * g[ok, None]
+        acc = rows if j == 0 else (acc + rows).astype(np.float32)
+    return acc if round_fn is None else round_fn(acc)
+
+
+# --------------------------------------------------------------------------
+# A.6: top-2 extension (docker/resources/sharded_moe.py:253-324, no Gumbel noise)
+# --------------------------------------------------------------------------
+def moe_encode_top2(data, gate, used_in, capacity_factor=1.0, gate_is_logits=False,
+                    C=None, fast_scatter=False):
+    """GShard top-2 expressed as two chained reference top-1 encodes, merged:
+    slot 1 with used_in, slot 2 with used_out(slot 1); merged layout is what
+    moe_merge_masks/moe_redispatch give for the two calls.  Capacity follows the
+    reference formula with capacity_factor' = 2*capacity_factor
+    (sharded_moe.py:267).  Combine weights are taken after the drop and
+    normalised by max(g1+g2, eps) (:296-312)."""
+    data = np.asarray(data)
+    S, M = data.shape
+    E = gate.shape[1]
+    if C is None:
+        C = capacity(S, E, 2.0 * capacity_factor)
+    sel, val = select_topk(gate, 2, gate_is_logits)
+    used_in = np.asarray(used_in, dtype=np.int32)
+    i1, l1, used1, _ = gen_location(sel[0], used_in, C, M, E)
+    i2, l2, used2, _ = gen_location(sel[1], used1, C, M, E)
+    merged = moe_merge_masks([np.stack([i1, l1]), np.stack([i2, l2])], E)
+    g1 = np.where(i1 >= 0, val[0], np.float32(0)).astype(np.float32)
+    g2 = np.where(i2 >= 0, val[1], np.float32(0)).astype(np.float32)
+    den = np.maximum((g1 + g2).astype(np.float32), F32_EPS)
+    gates = np.concatenate([g1 / den, g2 / den]).astype(np.float32)
+    fn = scatter_rows_fast if fast_scatter else scatter_rows
+    disp = fn(np.concatenate([data, data]), merged[0], merged[1], E, C)
+    elems = ((used2.astype(np.int64) - used_in) * M).astype(np.uint64)
+    return gates, merged, used2, elems, disp
+
+
+def top2_normalize_gates(raw_gates, merged_idx):
+    """Combine weights from raw per-slot gate values and merged (post-drop) indices."""
+    S = raw_gates.shape[0] // 2
+    g1 = np.where(merged_idx[:S] >= 0, raw_gates[:S], np.float32(0)).astype(np.float32)
+    g2 = np.where(merged_idx[S:] >= 0, raw_gates[S:], np.float32(0)).astype(np.float32)
+    den = np.maximum((g1 + g2).astype(np.float32), F32_EPS)
+    return np.concatenate([g1 / den, g2 / den]).astype(np.float32)
+
+
+# --------------------------------------------------------------------------
+# bf16 helpers (round-to-nearest-even on the fp32 bit pattern)
+# --------------------------------------------------------------------------
+def f32_to_bf16_bits(a):
+    u = np.asarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    rounded = (u + 0x7FFF + ((u >> 16) & 1)) >> 16
+    nan = np.isnan(np.asarray(a, dtype=np.float32))
+    out = rounded.astype(np.uint16)
+    out[nan] = 0x7FC0
+    return out
+
+
+def bf16_bits_to_f32(b):
+    return (np.asarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def round_to_bf16(a):
+    """fp32 -> nearest bf16 value, returned as fp32."""
+    return bf16_bits_to_f32(f32_to_bf16_bits(a))

@@ -1,0 +1,293 @@
+"""Pins the NumPy MoE oracle with checks that do not retype its formulas:
+hand-computed values, brute-force token loops, the dense einsum form of GShard
+top-2, and the reference tests' own identities (partitioned == un-partitioned,
+no expert above capacity, encode->decode round trip)."""
+import numpy as np
+import pytest
+from scipy.special import softmax as sp_softmax
+
+from oracle import moe_oracle as mo
+
+
+def rng_case(seed, S, M, E, dtype=np.float32, ties=False):
+    rng = np.random.default_rng(seed)
+    data = rng.standard_normal((S, M)).astype(dtype)
+    gate = rng.standard_normal((S, E)).astype(np.float32)
+    if ties:
+        gate = np.round(gate * 2) / 2  # many exact ties
+    return data, gate
+
+
+# ---------------------------------------------------------------- capacity
+@pytest.mark.parametrize("S,E,cf,want", [
+    (4096, 8, 1.25, 640),          # BASELINE config 1
+    (16384, 16, 2.0, 2048),        # config 2 (top-2: 2*cf)
+    (32768, 64, 1.25, 640),        # config 3
+    (16384, 32, 10.0, 5120),       # config 4 per partition: 2*1.25*4
+    (65536, 32, 2.5, 5120),        # config 4 un-partitioned
+    (1000, 7, 1.0, 143),           # ceil(1000/7)
+    (10, 4, 1.5, 4),               # int(1.5*3) = 4
+    (10, 4, 0.0, 0),
+    (5, 8, 1.0, 1),
+])
+def test_capacity_hand_cases(S, E, cf, want):
+    assert mo.capacity(S, E, cf) == want
+
+
+# ---------------------------------------------------------------- softmax
+def test_softmax_against_scipy_and_fp64():
+    rng = np.random.default_rng(1)
+    x = (rng.standard_normal((257, 33)) * 4).astype(np.float32)
+    p = mo.softmax_rows(x)
+    ref64 = sp_softmax(x.astype(np.float64), axis=1)
+    np.testing.assert_allclose(p, ref64, rtol=2e-6, atol=0)
+    np.testing.assert_allclose(p.sum(axis=1), 1.0, rtol=1e-6)
+    # shift invariance (closed-form property of softmax)
+    p2 = mo.softmax_rows(x + np.float32(3.0))
+    np.testing.assert_allclose(p, p2, rtol=1e-5)
+
+
+# ---------------------------------------------------------------- selection
+def brute_topk(row, k):
+    order = sorted(range(len(row)), key=lambda j: (-row[j], j))
+    return order[:k]
+
+
+@pytest.mark.parametrize("ties", [False, True])
+def test_select_topk_bruteforce(ties):
+    _, gate = rng_case(2, 300, 1, 9, ties=ties)
+    idx, val = mo.select_topk(gate, 2, False)
+    for s in range(gate.shape[0]):
+        want = brute_topk(list(gate[s]), 2)
+        assert [idx[0, s], idx[1, s]] == want
+        assert val[0, s] == gate[s, want[0]] and val[1, s] == gate[s, want[1]]
+
+
+def test_select_hand_ties():
+    gate = np.array([[5, 5, 3], [3, 5, 5], [5, 3, 3], [3, 5, 3], [1, 1, 1]], dtype=np.float32)
+    idx, _ = mo.select_topk(gate, 2)
+    assert idx[0].tolist() == [0, 1, 0, 1, 0]
+    assert idx[1].tolist() == [1, 2, 1, 0, 1]
+
+
+def test_select_second_choice_when_rest_is_minus_inf():
+    gate = np.array([[1.0, -np.inf, -np.inf], [-np.inf, -np.inf, 2.0]], dtype=np.float32)
+    idx, _ = mo.select_topk(gate, 2)
+    assert idx[0].tolist() == [0, 2]
+    assert idx[1].tolist() == [1, 0]
+
+
+# ---------------------------------------------------------------- encode (A.1)
+def brute_encode(data, gate, used_in, C):
+    S, M = data.shape
+    E = gate.shape[1]
+    counts = [0] * E
+    idx = [0] * S
+    loc = [0] * S
+    buf = np.zeros((E, C, M), data.dtype)
+    for s in range(S):
+        e = brute_topk(list(gate[s]), 1)[0]
+        r = counts[e]
+        counts[e] += 1
+        loc[s] = r
+        if r >= C - used_in[e]:
+            idx[s] = -1
+        else:
+            idx[s] = e
+            buf[e, r] = data[s]
+    used_out = [min(int(used_in[e]) + counts[e], C) for e in range(E)]
+    elems = [(used_out[e] - int(used_in[e])) * M for e in range(E)]
+    return idx, loc, used_out, elems, buf
+
+
+@pytest.mark.parametrize("S,M,E,cf,seed", [(64, 8, 4, 1.0, 0), (257, 4, 8, 1.25, 1), (100, 3, 7, 0.5, 2),
+                                           (33, 2, 1, 1.0, 3), (50, 2, 16, 1.0, 4)])
+def test_encode_bruteforce(S, M, E, cf, seed):
+    data, gate = rng_case(seed, S, M, E, ties=(seed % 2 == 1))
+    rng = np.random.default_rng(seed + 100)
+    C = mo.capacity(S, E, cf)
+    used_in = rng.integers(0, C + 1, size=E).astype(np.int32) if seed % 2 else np.zeros(E, np.int32)
+    g, il, used, elems, disp = mo.moe_encode(data, gate, used_in, cf)
+    bi, bl, bu, be, bb = brute_encode(data, gate, used_in, C)
+    assert il[0].tolist() == bi and il[1].tolist() == bl
+    assert used.tolist() == bu and elems.tolist() == be
+    assert elems.dtype == np.uint64 and il.dtype == np.int32 and g.dtype == np.float32
+    np.testing.assert_array_equal(disp, bb)
+    np.testing.assert_array_equal(g, gate.max(axis=1))
+    # vectorised scatter == loop scatter
+    np.testing.assert_array_equal(mo.scatter_rows_fast(data, il[0], il[1], E, C), disp)
+
+
+def test_encode_invariants_all_tokens_one_expert():
+    S, M, E = 40, 4, 4
+    data, gate = rng_case(5, S, M, E)
+    gate[:, 2] = 100.0
+    C = mo.capacity(S, E, 1.0)  # 10
+    g, il, used, elems, disp = mo.moe_encode(data, gate, np.zeros(E, np.int32), 1.0)
+    assert used.tolist() == [0, 0, 10, 0]
+    assert il[0].tolist() == [2] * 10 + [-1] * 30
+    assert il[1].tolist() == list(range(40))          # stale ranks stay on dropped tokens
+    np.testing.assert_array_equal(disp[2], data[:10])
+    assert not disp[[0, 1, 3]].any()
+
+
+# ---------------------------------------------------------------- chained partitions (A.3/A.4)
+@pytest.mark.parametrize("P", [2, 4])
+@pytest.mark.parametrize("E", [2, 8])
+def test_partitioned_equals_unpartitioned(P, E):
+    """tests/python/op/cuda/test_cuda_moe.py:384-471 protocol."""
+    S0, M = 256, 6
+    data, gate = rng_case(7, S0, M, E)
+    S = S0 // P
+    zero = np.zeros(E, np.int32)
+    rg, ril, rused, _, rdisp = mo.moe_encode(data, gate, zero, 1.0)
+    used = zero
+    ils, bufs, gs = [], [], []
+    for p in range(P):
+        sl = slice(p * S, (p + 1) * S)
+        g, il, used, _, disp = mo.moe_encode(data[sl], gate[sl], used, float(P))
+        assert disp.shape == rdisp.shape
+        ils.append(il), bufs.append(disp), gs.append(g)
+    np.testing.assert_array_equal(used, rused)
+    # no expert above capacity across the chain (test_cuda_moe.py:336-381)
+    cat = np.concatenate([il[0] for il in ils])
+    assert (np.bincount(cat[cat >= 0], minlength=E) <= rdisp.shape[1]).all()
+    merged = mo.moe_merge_masks(ils, E)
+    red = mo.moe_redispatch(bufs, ils)
+    ril = ril.copy()
+    ril[1, ril[0] < 0] = -1            # merge normalises stale locations to -1
+    np.testing.assert_array_equal(merged, ril)
+    np.testing.assert_array_equal(red, rdisp)
+    np.testing.assert_array_equal(np.concatenate(gs), rg)
+
+
+# ---------------------------------------------------------------- BPR (A.2)
+def brute_bpr(gate, C, P, pid):
+    S0, E = gate.shape
+    S = S0 // P
+    idx0 = [brute_topk(list(gate[s]), 1)[0] for s in range(S0)]
+    g0 = [gate[s, idx0[s]] for s in range(S0)]
+    keep = [False] * S0
+    for e in range(E):
+        toks = sorted([s for s in range(S0) if idx0[s] == e], key=lambda s: (-g0[s], s))
+        for s in toks[:C]:
+            keep[s] = True
+    counts = [0] * E
+    idx, loc = [], []
+    for s in range(pid * S, (pid + 1) * S):
+        if keep[s]:
+            idx.append(idx0[s]), loc.append(counts[idx0[s]])
+            counts[idx0[s]] += 1
+        else:
+            idx.append(-1), loc.append(-1)
+    return idx, loc, [min(c, C) for c in counts], keep
+
+
+@pytest.mark.parametrize("S0,E,P,cf,ties", [(128, 4, 1, 1.0, False), (128, 4, 1, 0.5, True), (256, 8, 4, 4.0, False),
+                                            (256, 8, 4, 2.0, True), (96, 3, 2, 1.0, True)])
+def test_bpr_bruteforce(S0, E, P, cf, ties):
+    M = 3
+    data, gate = rng_case(11, S0, M, E, ties=ties)
+    C = mo.capacity(S0 // P, E, cf)
+    kept_total = np.zeros(E, np.int64)
+    for pid in range(P):
+        g, il, used, elems, disp = mo.moe_encode_bpr(data, gate, P, pid, cf)
+        bi, bl, bu, keep = brute_bpr(gate, C, P, pid)
+        assert il[0].tolist() == bi and il[1].tolist() == bl and used.tolist() == bu
+        assert elems.tolist() == [u * M for u in bu]
+        S = S0 // P
+        np.testing.assert_array_equal(g, gate.max(axis=1)[pid * S:(pid + 1) * S])
+        for s in range(S):
+            if bi[s] >= 0:
+                np.testing.assert_array_equal(disp[bi[s], bl[s]], data[pid * S + s])
+        assert np.count_nonzero(disp.any(axis=2)) <= sum(bu)
+        kept_total += used
+    # sum over partitions of kept == min(cnt, C): drop set independent of the partitioning
+    cnt = np.bincount(np.argmax(gate, axis=1), minlength=E)
+    np.testing.assert_array_equal(kept_total, np.minimum(cnt, C))
+
+
+# ---------------------------------------------------------------- top-2 (A.6) vs dense GShard form
+def dense_top2(logits, data, C):
+    """docker/resources/sharded_moe.py:253-324 written with dense masks, no noise."""
+    S, E = logits.shape
+    gates = sp_softmax(logits.astype(np.float64), axis=1)
+    i1 = np.argmax(gates, axis=1)
+    mask1 = np.eye(E, dtype=np.int64)[i1]
+    except1 = np.where(mask1.astype(bool), -np.inf, logits.astype(np.float64))
+    i2 = np.argmax(except1, axis=1)
+    mask2 = np.eye(E, dtype=np.int64)[i2]
+    loc1 = np.cumsum(mask1, axis=0) - 1
+    loc2 = np.cumsum(mask2, axis=0) - 1 + mask1.sum(axis=0, keepdims=True)
+    mask1 = mask1 * (loc1 < C)
+    mask2 = mask2 * (loc2 < C)
+    l1 = (loc1 * mask1).sum(axis=1)
+    l2 = (loc2 * mask2).sum(axis=1)
+    g1 = (gates * mask1).sum(axis=1)
+    g2 = (gates * mask2).sum(axis=1)
+    den = np.maximum(g1 + g2, np.finfo(np.float32).eps)
+    g1, g2 = g1 / den, g2 / den
+    cw = np.zeros((S, E, C))
+    for s in range(S):
+        if mask1[s].any():
+            cw[s, i1[s], l1[s]] += g1[s]
+        if mask2[s].any():
+            cw[s, i2[s], l2[s]] += g2[s]
+    disp = np.einsum("sec,sm->ecm", (cw != 0).astype(np.float64), data.astype(np.float64))
+    return cw, disp
+
+
+@pytest.mark.parametrize("S,E,cf,seed", [(48, 4, 1.0, 0), (64, 8, 0.5, 1), (40, 3, 2.0, 2)])
+def test_top2_matches_dense_gshard(S, E, cf, seed):
+    M = 5
+    data, logits = rng_case(seed, S, M, E)
+    logits[:, 0] += 1.5   # a hot expert so that slot 1 and slot 2 both overflow
+    C = int(np.ceil(2 * S / E * cf))
+    assert C == mo.capacity(S, E, 2 * cf) or (2 * S / E * cf) != int(2 * S / E * cf)
+    gates, il, used, elems, disp = mo.moe_encode_top2(data, logits, np.zeros(E, np.int32), cf,
+                                                      gate_is_logits=True, C=C)
+    cw, ddisp = dense_top2(logits, data, C)
+    mine = np.zeros((S, E, C))
+    for j in range(2):
+        for s in range(S):
+            e, l = il[0, j * S + s], il[1, j * S + s]
+            if e >= 0:
+                mine[s, e, l] += gates[j * S + s]
+    np.testing.assert_allclose(mine, cw, rtol=1e-5, atol=1e-7)
+    np.testing.assert_allclose(disp, ddisp, rtol=0, atol=0)
+    kept = np.bincount(il[0][il[0] >= 0], minlength=E)
+    np.testing.assert_array_equal(used, kept)
+    assert elems.tolist() == (kept * M).tolist()
+    # decode of the identity expert with the combine weights == dense combine
+    out = mo.moe_decode(disp, gates, il, k=2)
+    want = np.einsum("sec,ecm->sm", cw, ddisp)
+    np.testing.assert_allclose(out, want, rtol=1e-5, atol=1e-6)
+
+
+# ---------------------------------------------------------------- decode (A.5)
+def test_decode_roundtrip_and_loop_reference():
+    S, M, E = 120, 6, 5
+    data, gate = rng_case(21, S, M, E)
+    probs = mo.softmax_rows(gate)
+    g, il, used, _, disp = mo.moe_encode(data, probs, np.zeros(E, np.int32), 0.75)
+    out1 = mo.moe_decode(disp, np.ones(S, np.float32), il)
+    kept = il[0] >= 0
+    np.testing.assert_array_equal(out1[kept], data[kept])
+    assert not out1[~kept].any() and (~kept).any()
+    # loop reference of test_cuda_moe.py:1157-1165
+    out = mo.moe_decode(disp, g, il)
+    C = disp.shape[1]
+    for s in range(S):
+        e, l = il[0, s], il[1, s]
+        want = disp[e, l] * g[s] if (0 <= e < E and l < C) else np.zeros(M, np.float32)
+        np.testing.assert_array_equal(out[s], want)
+
+
+def test_bf16_rounding_helpers():
+    x = np.array([1.0, 1.00390625, 1.005859375, -2.5, 3.0e38, 1e-40], dtype=np.float32)
+    # 1.00390625 = 1 + 2^-8 is a tie between bf16 1.0 and 1.0078125 -> even (1.0)
+    r = mo.round_to_bf16(x)
+    assert r[0] == 1.0 and r[1] == 1.0 and r[2] == np.float32(1.0078125) and r[3] == -2.5
+    import torch
+    t = torch.from_numpy(x).to(torch.bfloat16).to(torch.float32).numpy()
+    np.testing.assert_array_equal(r, t)

@@ -1,0 +1,267 @@
+"""Benchmark of the MoE dispatch path and the fused LANS step on one MI355X.
+
+A "step" is one pass of the hot path over one batch of synthetic input: raf.op.moe_encode
+(routing + scatter) followed by raf.op.moe_decode at the headline shape of BASELINE.json
+(S=65536 tokens, M=4096 bf16, E=32 experts, top-2, capacity factor 1.25 -> C=5120), inputs
+resident in HBM.  Prints ONE JSON line (see README / DESIGN.md for the fields).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-lans] [--no-cpu]
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+PKG_NAME = "lancet-accelerating-moe-training-via-whole-graph-computation-communication-overlapping_amd"
+
+HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E bandwidth
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--tokens", type=int, default=65536)
+    ap.add_argument("--hidden", type=int, default=4096)
+    ap.add_argument("--experts", type=int, default=32)
+    ap.add_argument("--no-lans", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--lans-scale", type=float, default=1.0, help="fraction of the 24-layer LANS tensor list")
+    return ap.parse_args()
+
+
+def event_ms(fn, iters):
+    """Average duration in ms of fn() over `iters` calls, HIP events on the launch stream."""
+    import torch
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def lans_shapes(scale=1.0):
+    """BASELINE config 5: 24 layers x {4 x [1024,1024], 4 x [1024] biases, 4 x [1024] norms},
+    12 MoE layers x 16 experts x {[1024,4096],[4096,1024]}, final norm 2 x [1024]:
+    674 tensors, 1.7115e9 parameters."""
+    layers = max(1, int(round(24 * scale)))
+    shapes = []
+    for layer in range(layers):
+        shapes += [(1024, 1024)] * 4 + [(1024,)] * 8
+        if layer % 2 == 1 or layers == 1:
+            shapes += [(1024, 4096), (4096, 1024)] * 16
+    shapes += [(1024,)] * 2
+    return shapes
+
+
+def bench_lans(ops, capi, steps, warmup, scale):
+    import torch
+    shapes = lans_shapes(scale)
+    numels = [int(torch.Size(s).numel()) for s in shapes]
+    total = sum(numels)
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    flat = {}
+    for name, std in (("g", 1e-3), ("p", 0.02)):
+        flat[name] = torch.empty(total, device="cuda").normal_(0, std, generator=gen)
+    flat["m"] = torch.zeros(total, device="cuda")
+    flat["v"] = torch.zeros(total, device="cuda")
+    views = {k: list(torch.split(t, numels)) for k, t in flat.items()}
+    plan = ops.LansPlan(numels)
+    hyper = capi.LansHyper(1e-3, 0.9, 0.999, 1e-6, 1, 0.01, 1, 1, 1)
+    state = {"step": 1}
+
+    def one():
+        plan.step(views["g"], views["p"], views["m"], views["v"], state["step"], hyper)
+        state["step"] += 1
+
+    for _ in range(warmup):
+        one()
+    ms = event_ms(one, steps)
+    plan.close()
+    gbs = 28.0 * total / (ms * 1e-3) / 1e9
+    return {"tensors": len(shapes), "params": total, "ms_per_step": round(ms, 4),
+            "algorithmic_GBps": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+            "bytes_per_param_algorithmic": 28, "bytes_per_param_three_sweep": 52, "steps": steps}
+
+
+def cpu_baseline(S_sample, M, E, cf):
+    """The oracle (NumPy restatement of the reference's test references) timed on a bounded
+    sample of the headline workload: top-2 encode + decode over S_sample tokens."""
+    import numpy as np
+    from oracle import moe_oracle as mo
+    rng = np.random.default_rng(0)
+    data = mo.round_to_bf16(rng.standard_normal((S_sample, M), dtype=np.float32))
+    logits = rng.standard_normal((S_sample, E), dtype=np.float32)
+    used = np.zeros(E, np.int32)
+    t0 = time.perf_counter()
+    g, il, _, _, disp = mo.moe_encode_top2(data, logits, used, cf, gate_is_logits=True)
+    out = mo.moe_decode(disp, g, il, k=2, round_fn=mo.round_to_bf16)
+    dt = time.perf_counter() - t0
+    del out
+    return {"value": round(S_sample / dt, 1), "unit": "tokens/s", "cores": 1, "kind": "port",
+            "sample": "NumPy oracle (one-hot cumsum + Python scatter loop), top-2 encode+decode of "
+                      "%d tokens at M=%d, E=%d, %.2f s" % (S_sample, M, E, dt)}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        log("bench.py measures one GPU's share of the dispatch path; this build has no multi-GPU "
+            "path (no collectives are part of it). Run with --gpus 1.")
+        sys.exit(2)
+    import numpy as np
+    import torch
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    torch.cuda.set_device(0)
+    pkg = importlib.import_module(PKG_NAME)
+    ops, capi = pkg.ops, pkg.capi
+    lib = capi.load()
+    import ctypes as C
+
+    S, M, E, K, cf = args.tokens, args.hidden, args.experts, 2, 1.25
+    b = 2  # bf16
+    Cap = ops.moe_capacity(S, E, 2 * cf)
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    data = torch.empty((S, M), device="cuda").normal_(0, 1, generator=gen).to(torch.bfloat16)
+    logits = torch.empty((S, E), device="cuda").normal_(0, 1, generator=gen)
+    used_in = torch.zeros(E, dtype=torch.int32, device="cuda")
+    outs = (torch.empty(K * S, device="cuda"), torch.empty((2, K * S), dtype=torch.int32, device="cuda"),
+            torch.empty(E, dtype=torch.int32, device="cuda"), torch.empty(E, dtype=torch.int64, device="cuda"),
+            torch.empty((E, Cap, M), dtype=torch.bfloat16, device="cuda"))
+    ws = torch.empty(ops.moe_encode_workspace_bytes(S, E, K), dtype=torch.uint8, device="cuda")
+    dec = torch.empty((S, M), dtype=torch.bfloat16, device="cuda")
+
+    def encode():
+        return ops.moe_encode(data, logits, used_in, cf, top_k=K, gate_is_logits=True, workspace=ws, out=outs)
+
+    def decode():
+        return ops.moe_decode(outs[4], outs[0], outs[1], top_k=K, out=dec)
+
+    def step():
+        encode()
+        decode()
+
+    # ---- parity gate at full size: routing bit-exact against the oracle, rows by properties
+    from oracle import moe_oracle as mo
+    step()
+    torch.cuda.synchronize()
+    h_logits = logits.cpu().numpy()
+    sel, val = mo.select_topk(h_logits, 2, True)
+    zero = np.zeros(E, np.int32)
+    i1, l1, u1, _ = mo.gen_location(sel[0], zero, Cap, M, E)
+    i2, l2, u2, _ = mo.gen_location(sel[1], u1, Cap, M, E)
+    merged = mo.moe_merge_masks([np.stack([i1, l1]), np.stack([i2, l2])], E)
+    il = outs[1].cpu().numpy()
+    assert np.array_equal(il, merged), "routing differs from the oracle at full size"
+    assert np.array_equal(outs[2].cpu().numpy(), u2)
+    kept = int((merged[0] >= 0).sum())
+    il_t = outs[1].long()
+    for j in range(K):
+        idx, loc = il_t[0, j * S:(j + 1) * S], il_t[1, j * S:(j + 1) * S]
+        ok = idx >= 0
+        assert torch.equal(outs[4][idx[ok], loc[ok]], data[ok]), "scattered rows differ from the token rows"
+    used = outs[2].long()
+    tail_mask = torch.arange(Cap, device="cuda")[None, :] >= used[:, None]
+    assert not outs[4][tail_mask].any(), "rows past the used capacity are not zero"
+    either = (il_t[0, :S] >= 0) | (il_t[0, S:] >= 0)
+    # identity expert + normalised weights: decode returns the token (g1 + g2 = 1) within 1 bf16 ulp
+    err = (dec[either].float() - data[either].float()).abs() / data[either].float().abs().clamp_min(1e-30)
+    assert float(err.max()) <= 2 ** -7, "encode -> decode round trip broken"
+    assert not dec[~either].any()
+    log("parity gate ok: S=%d M=%d E=%d C=%d kept=%d of %d slots" % (S, M, E, Cap, kept, K * S))
+
+    # ---- timed region: K steps, wall clock bracketed by synchronisation
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # ---- per-op / per-kernel durations with HIP events on the launch stream
+    n = max(args.steps, 10)
+    ms_enc = event_ms(encode, n)
+    ms_dec = event_ms(decode, n)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    p = lambda t: C.c_void_p(t.data_ptr())
+
+    def scatter_only():
+        st = lib.lancet_moe_scatter(p(data), p(outs[1]), p(used_in), p(outs[2]), S, M, E, Cap, K, capi.BF16,
+                                    p(outs[4]), stream)
+        assert st == 0
+
+    def route_only():
+        st = lib.lancet_moe_route(p(logits), p(used_in), S, M, E, Cap, K, capi.GATE_IS_LOGITS, p(outs[0]),
+                                  p(outs[1]), p(outs[2]), p(outs[3]), p(ws), ws.numel(), stream)
+        assert st == 0
+
+    ms_route = event_ms(route_only, n)
+    encode()
+    ms_scatter = event_ms(scatter_only, n)
+
+    enc_bytes = S * E * 4 + S * M * b + E * Cap * M * b + K * S * 12 + E * 12
+    dec_bytes = kept * M * b + S * M * b + K * S * 12
+    scatter_bytes = S * M * b + E * Cap * M * b + K * S * 8 + E * 8
+    gbs = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9
+    scatter_gbs = gbs(scatter_bytes, ms_scatter)
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "scatter_rows_headline_traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f).get("hbm_bytes_per_launch")
+
+    result = {
+        "metric": "moe_dispatch_tokens_per_sec_encode_plus_decode",
+        "value": round(S / (ms_step * 1e-3), 1),
+        "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "un-partitioned top-2 moe_encode + moe_decode, S=%d M=%d bf16 E=%d C=%d "
+                               "(BASELINE config 4 shape, headline)" % (S, M, E, Cap),
+                   "tokens": S, "hidden": M, "experts": E, "capacity": Cap, "top_k": K,
+                   "kept_slots": kept, "gate": "fp32 logits, softmax fused"},
+        "roofline": {"bound": "hbm", "kernel": "scatter_rows_kernel<u32x4,2> (encode_forward)",
+                     "achieved": round(scatter_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(scatter_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "algorithmic_bytes_per_launch": scatter_bytes, "avg_launch_ms": round(ms_scatter, 4)},
+        "ops": {
+            "encode": {"ms": round(ms_enc, 4), "algorithmic_bytes": enc_bytes,
+                       "GBps": round(gbs(enc_bytes, ms_enc), 1),
+                       "frac": round(gbs(enc_bytes, ms_enc) / HBM_PEAK_GBS, 4)},
+            "decode": {"ms": round(ms_dec, 4), "algorithmic_bytes": dec_bytes,
+                       "GBps": round(gbs(dec_bytes, ms_dec), 1),
+                       "frac": round(gbs(dec_bytes, ms_dec) / HBM_PEAK_GBS, 4)},
+            "route_scan": {"ms": round(ms_route, 4)},
+            "encode_plus_decode_frac": round(gbs(enc_bytes + dec_bytes, ms_enc + ms_dec) / HBM_PEAK_GBS, 4),
+        },
+    }
+    del data, dec, outs
+    torch.cuda.empty_cache()
+    if not args.no_lans:
+        result["lans"] = bench_lans(ops, capi, max(3, min(args.steps, 10)), max(1, min(args.warmup, 2)),
+                                    args.lans_scale)
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(2048, M, E, cf)
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,216 @@
+/*
+ * lancet_hip.h - C ABI of the MI355X (gfx950) implementation of one GPU's share of
+ * the MoE token-dispatch path and the fused LANS step.
+ *
+ * Every entry point replaces one piece of the reference's native launcher surface
+ * (src/op/dialect/cuda/kernels/kernel_util.cuh:25-66) or of the OpEnv that drives it
+ * (src/op/dialect/cuda/moe.cc, src/op/dialect/cuda/lans.cc); the citation on each
+ * declaration names the piece.  Conventions:
+ *
+ *   - plain pointers and sizes only; all data pointers are DEVICE pointers unless a
+ *     parameter is documented as a host array;
+ *   - every call takes the HIP stream to launch on (a hipStream_t passed as void*;
+ *     NULL = the default stream), is asynchronous with respect to the host and
+ *     allocates nothing (the two lans_plan calls excepted, which own small tables);
+ *   - outputs and workspaces are caller-owned; *_workspace_bytes() sizes the
+ *     workspace, whose contents need not be initialised and are not preserved;
+ *   - the return value is a status: 0 = ok, < 0 = rejected argument (nothing was
+ *     launched), > 0 = a hipError_t from the runtime.  Nothing aborts the process
+ *     (the reference CHECK/LOG(FATAL)s, src/common/cuda_utils.h:18-22).
+ *
+ * Token rows are `dtype` (LANCET_F32 / LANCET_BF16 / LANCET_F16); gate values,
+ * gates_s and LANS tensors are fp32; indices/locations/used capacity are int32 and
+ * elements_per_expert is uint64, as in src/op/declare/moe.cc:48-58.
+ */
+#ifndef LANCET_HIP_H_
+#define LANCET_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LANCET_ABI_VERSION 1
+
+/* element type of token rows */
+#define LANCET_F32 0
+#define LANCET_BF16 1
+#define LANCET_F16 2
+
+/* status codes (negative = argument rejected, nothing launched) */
+#define LANCET_OK 0
+#define LANCET_ERR_NULL (-1)      /* a required pointer is NULL */
+#define LANCET_ERR_SHAPE (-2)     /* a size is negative, zero where not allowed, or above a limit */
+#define LANCET_ERR_DTYPE (-3)     /* unknown dtype code */
+#define LANCET_ERR_WORKSPACE (-4) /* workspace missing or too small */
+#define LANCET_ERR_ALIGN (-5)     /* a pointer is not aligned to its element type */
+#define LANCET_ERR_TOPK (-6)      /* top_k not 1 or 2, or top_k = 2 with fewer than 2 experts */
+#define LANCET_ERR_PARTITION (-7) /* bad n_partitions / partition_id */
+#define LANCET_ERR_PLAN (-8)      /* invalid LANS plan handle */
+
+/* limits */
+#define LANCET_MAX_EXPERTS 512
+#define LANCET_MAX_PARTITIONS 64
+
+/* flags of lancet_moe_encode / lancet_moe_encode_bpr / lancet_gate_topk */
+#define LANCET_GATE_IS_LOGITS 1u /* `gate` holds logits: select on them, gates_s = softmax prob */
+
+typedef void* lancet_stream_t;
+
+int lancet_abi_version(void);
+const char* lancet_status_string(int status);
+
+/* Capacity C = int(float(cf) * ((S + E - 1) / E)).
+ * Replaces: src/op/dialect/cuda/moe.cc:107-109, src/op/declare/moe.cc:46, src/op/ty/moe.cc:50. */
+int64_t lancet_moe_capacity(int64_t S, int64_t E, float capacity_factor);
+
+/* ---- routing front end -------------------------------------------------------------
+ * idx[j*S + s], val[j*S + s] for j < top_k: first-max expert of row s of gate[S,E] (slot 2:
+ * with slot 1's expert masked), and gate[s, idx] or its softmax probability.
+ * Replaces: the three TVM-compiled micro-kernels argmax / one_hot / multiply+sum that
+ * MoeEncode runs first (src/op/dialect/cuda/moe.cc:177-250, executed :366-371) and, with
+ * LANCET_GATE_IS_LOGITS, the softmax in front of the op (models/benchmark/pytorch/utils.py:565-573). */
+int lancet_gate_topk(const float* gate, int64_t S, int64_t E, int top_k, unsigned flags,
+                     int32_t* idx, float* val, lancet_stream_t stream);
+
+/* ---- launcher level ----------------------------------------------------------------
+ * Replaces launch_gen_location (kernel_util.cuh:60; tutel_moe_dispatch.cu:164-212,548-553).
+ * indices[S] is mutated (dropped tokens -> -1); locations[S] receives the rank of every token
+ * among the tokens of its expert. */
+size_t lancet_gen_location_workspace_bytes(int64_t S, int64_t E);
+int lancet_launch_gen_location(int32_t* indices, const int32_t* in_capused, int32_t* locations,
+                               int32_t* out_capused, uint64_t* out_elements_per_expert,
+                               int64_t C, int64_t S, int64_t E, int64_t M,
+                               void* workspace, size_t workspace_bytes, lancet_stream_t stream);
+
+/* Replaces both launch_encode_forward overloads (kernel_util.cuh:37-40;
+ * tutel_moe_dispatch.cu:61-81,461-484): capused == NULL is the "_wo_usedcap" overload.
+ * Every byte of dispatched[E,C,M] is written exactly once (rows that receive no token are
+ * zero-filled by the same launch; there is no memset + atomicAdd). */
+int lancet_launch_encode_forward(const int32_t* indices, const int32_t* locations,
+                                 const int32_t* capused, const void* data, void* dispatched,
+                                 int64_t S, int64_t M, int64_t C, int64_t E, int dtype,
+                                 lancet_stream_t stream);
+
+/* ---- raf.op.moe_encode -------------------------------------------------------------
+ * Replaces MoeEncode::Execute (src/op/dialect/cuda/moe.cc:346-396); outputs are the 5-tuple of
+ * src/op/declare/moe.cc:48-58.  top_k = 2 is an extension with GShard semantics
+ * (docker/resources/sharded_moe.py:253-324, no noise): outputs are slot-major
+ * (gates_s[2S], indices_locations[2, 2S]) in the layout moe_merge_masks produces for the two
+ * chained top-1 encodes it is equivalent to, and gates_s holds the normalised combine weights.
+ * used_in may be NULL (= zeros). */
+size_t lancet_moe_encode_workspace_bytes(int64_t S, int64_t E, int top_k);
+int lancet_moe_encode(const void* data, const float* gate, const int32_t* used_in,
+                      int64_t S, int64_t M, int64_t E, int64_t C, int top_k, int dtype,
+                      unsigned flags, float* gates_s, int32_t* indices_locations,
+                      int32_t* used_out, uint64_t* elements_per_expert, void* dispatched,
+                      void* workspace, size_t workspace_bytes, lancet_stream_t stream);
+
+/* The two phases of lancet_moe_encode as separate calls, for callers that overlap the routing of
+ * one token partition with the row movement of another (Lancet's forward pipelining,
+ * src/pass/dist_optimization/partition_exprs.cc:1709-1795):
+ *   lancet_moe_route   = selection + position scan (everything of MoeEncode::Execute up to and
+ *                        including launch_gen_location, moe.cc:366-380); outputs as above
+ *                        except the buffer;
+ *   lancet_moe_scatter = launch_encode_forward (moe.cc:381-395) on routing produced by
+ *                        lancet_moe_route; zero-fills the rows past used_out - used_in. */
+int lancet_moe_route(const float* gate, const int32_t* used_in, int64_t S, int64_t M, int64_t E,
+                     int64_t C, int top_k, unsigned flags, float* gates_s,
+                     int32_t* indices_locations, int32_t* used_out, uint64_t* elements_per_expert,
+                     void* workspace, size_t workspace_bytes, lancet_stream_t stream);
+int lancet_moe_scatter(const void* data, const int32_t* indices_locations, const int32_t* used_in,
+                       const int32_t* used_out, int64_t S, int64_t M, int64_t E, int64_t C, int top_k,
+                       int dtype, void* dispatched, lancet_stream_t stream);
+
+/* ---- raf.op.moe_encode_batch_prioritized --------------------------------------------
+ * Replaces MoeEncodeBatchPrioritized::Execute (moe.cc:543-684), the TVM argsort it calls
+ * (:701-719) and launch_gen_location_bpr (kernel_util.cuh:65; tutel_moe_dispatch.cu:259-363).
+ * data[S0,M], gate[S0,E] are the whole batch; S = S0 / n_partitions tokens of partition
+ * partition_id are encoded.  The per-expert keep set is the C best tokens by
+ * (gate value descending, token index ascending), found with a radix select, not a sort. */
+size_t lancet_moe_encode_bpr_workspace_bytes(int64_t S0, int64_t E, int n_partitions);
+int lancet_moe_encode_bpr(const void* data, const float* gate, int64_t S0, int64_t M, int64_t E,
+                          int64_t C, int n_partitions, int partition_id, int dtype, unsigned flags,
+                          float* gates_s, int32_t* indices_locations, int32_t* used_out,
+                          uint64_t* elements_per_expert, void* dispatched,
+                          void* workspace, size_t workspace_bytes, lancet_stream_t stream);
+
+/* ---- raf.op.moe_decode -------------------------------------------------------------
+ * Replaces MoeDecode::Execute / launch_decode_forward (moe.cc:1262-1291; kernel_util.cuh:45;
+ * tutel_moe_dispatch.cu:46-55,110-116,511-521).  top_k = 2 sums the two slots of the
+ * slot-major layout in fp32 and rounds once. */
+int lancet_moe_decode(const void* expert_out, const float* gates_s,
+                      const int32_t* indices_locations, int64_t S, int64_t M, int64_t E,
+                      int64_t C, int top_k, int dtype, void* out, lancet_stream_t stream);
+
+/* Combine weights of the top-2 extension from raw per-slot gate values and merged indices
+ * (docker/resources/sharded_moe.py:304-312); in place when gates_out == raw_gates. */
+int lancet_moe_top2_normalize_gates(const float* raw_gates, const int32_t* merged_indices,
+                                    int64_t S, float* gates_out, lancet_stream_t stream);
+
+/* ---- raf.op.moe_merge_masks --------------------------------------------------------
+ * Replaces MoeMergeMasks::Execute / launch_merge_masks (moe.cc:772-802; kernel_util.cuh:62;
+ * tutel_moe_dispatch.cu:214-255,555-563).  indices_locations is a HOST array of P device
+ * pointers to [2,S] int32 tensors; out is [2, P*S]. */
+size_t lancet_moe_merge_masks_workspace_bytes(int P, int64_t E);
+int lancet_moe_merge_masks(const int32_t* const* indices_locations, int P, int64_t S, int64_t E,
+                           int32_t* out, void* workspace, size_t workspace_bytes,
+                           lancet_stream_t stream);
+
+/* ---- raf.op.moe_redispatch ---------------------------------------------------------
+ * Replaces MoeRedispatch::Execute / launch_redispatch (moe.cc:881-920; kernel_util.cuh:52;
+ * tutel_moe_dispatch.cu:365-408,572-584).  data / indices_locations are HOST arrays of P
+ * device pointers ([E,C,M] buffers and [2,S] masks).  Rows of out[E,C,M] past the merged
+ * count are zero (the reference leaves them uninitialised). */
+size_t lancet_moe_redispatch_workspace_bytes(int P, int64_t E);
+int lancet_moe_redispatch(const void* const* data, const int32_t* const* indices_locations,
+                          int P, int64_t S, int64_t M, int64_t C, int64_t E, int dtype,
+                          void* out, void* workspace, size_t workspace_bytes,
+                          lancet_stream_t stream);
+
+/* ---- raf.op.lans -------------------------------------------------------------------
+ * Replaces LansImpl (src/op/dialect/cuda/lans.cc:26-180) and multi_tensor_lans_cuda
+ * (kernel_util.cuh:25-33; multi_tensor_lans.cu:401-450).  A plan captures the tensor sizes of
+ * one parameter set (what the LansImpl constructor captures) and owns the chunk tables,
+ * per-chunk partial sums and norm vectors; it is created once and reused every step.
+ * g/p/m/v are HOST arrays of T device pointers to fp32 tensors (the four quarters of the
+ * reference's tensor_list).  p, m, v are updated in place; g is not modified.
+ * step: pass step_host >= 1, or a device pointer step_dev to the fp32 step scalar the
+ * reference passes (read on the device; no host synchronisation). */
+typedef struct lancet_lans_plan* lancet_lans_plan_t;
+
+typedef struct lancet_lans_hyper {
+  float learning_rate;
+  float beta1;
+  float beta2;
+  float eps;
+  int bias_correction;
+  float weight_decay;
+  int grad_averaging;
+  int mode;           /* 0 = L2 into the gradient, 1 = decoupled weight decay */
+  int normalize_grad;
+} lancet_lans_hyper;
+
+int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans_plan_t* plan);
+int lancet_lans_plan_destroy(lancet_lans_plan_t plan);
+int lancet_lans_step(lancet_lans_plan_t plan, const float* const* g, float* const* p,
+                     float* const* m, float* const* v, int step_host, const float* step_dev,
+                     const lancet_lans_hyper* hyper, lancet_stream_t stream);
+/* Copies the four per-tensor norm vectors of the last step (||g||, ||p||, ||u_m||, ||u_g||;
+ * the reference's grad_norm_tensor_ ... q_norm_tensor_ workspaces, lans.cc:77-82) into
+ * norms4xT, a device buffer of 4*T floats, asynchronously on `stream`. */
+int lancet_lans_plan_norms(lancet_lans_plan_t plan, float* norms4xT, lancet_stream_t stream);
+
+/* Test hook: number of polls a workgroup of the position scan waits for a predecessor
+ * before it gives up, flags the workspace and finishes with undefined results
+ * (0 restores the default).  Lets a host test exercise the bounded wait without hanging. */
+void lancet_debug_set_spin_limit(unsigned limit);
+/* Reads (synchronously) the error word a scan workspace carries: 0 = ok, 1 = a wait gave up. */
+int lancet_scan_workspace_error(const void* workspace, lancet_stream_t stream, int* error_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LANCET_HIP_H_ */

@@ -1,0 +1,14 @@
+"""MI355X-native MoE token dispatch and fused LANS behind RAF's operator surface.
+
+  capi  - ctypes bindings of the C ABI (include/lancet_hip.h)
+  ops   - the six RAF operators (moe_encode, moe_encode_batch_prioritized, moe_decode,
+          moe_merge_masks, moe_redispatch, lans) over torch tensors that live on the GPU
+  build - compiles the in-tree libraries with hipcc
+
+torch is used for device memory and streams only; every operator runs hand-written HIP
+kernels through the C ABI and raises when the library is missing.
+"""
+from . import capi  # noqa: F401
+from . import ops  # noqa: F401
+
+__all__ = ["capi", "ops"]

@@ -1,0 +1,105 @@
+"""ctypes bindings of the C ABI declared in include/lancet_hip.h.
+
+The library is loaded from <package>/lib/liblancet_hip.so (built in-tree by build.py).
+There is no fallback: a missing library raises.
+"""
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "liblancet_hip.so")
+
+F32, BF16, F16 = 0, 1, 2
+GATE_IS_LOGITS = 1
+MAX_EXPERTS = 512
+MAX_PARTITIONS = 64
+
+OK = 0
+ERR_NULL, ERR_SHAPE, ERR_DTYPE, ERR_WORKSPACE, ERR_ALIGN, ERR_TOPK, ERR_PARTITION, ERR_PLAN = range(-1, -9, -1)
+
+
+class LansHyper(C.Structure):
+    _fields_ = [("learning_rate", C.c_float), ("beta1", C.c_float), ("beta2", C.c_float),
+                ("eps", C.c_float), ("bias_correction", C.c_int), ("weight_decay", C.c_float),
+                ("grad_averaging", C.c_int), ("mode", C.c_int), ("normalize_grad", C.c_int)]
+
+
+class LancetError(RuntimeError):
+    def __init__(self, status, what):
+        self.status = status
+        super().__init__("%s failed: status %d (%s)" % (what, status, status_string(status)))
+
+
+_vp, _i64, _int, _u32, _sz, _f32 = C.c_void_p, C.c_int64, C.c_int, C.c_uint, C.c_size_t, C.c_float
+
+# name -> (restype, argtypes); every symbol include/lancet_hip.h declares
+SIGNATURES = {
+    "lancet_abi_version": (_int, []),
+    "lancet_status_string": (C.c_char_p, [_int]),
+    "lancet_moe_capacity": (_i64, [_i64, _i64, _f32]),
+    "lancet_gate_topk": (_int, [_vp, _i64, _i64, _int, _u32, _vp, _vp, _vp]),
+    "lancet_gen_location_workspace_bytes": (_sz, [_i64, _i64]),
+    "lancet_launch_gen_location": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _sz, _vp]),
+    "lancet_launch_encode_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
+    "lancet_moe_encode_workspace_bytes": (_sz, [_i64, _i64, _int]),
+    "lancet_moe_encode": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _u32,
+                                 _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "lancet_moe_route": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _u32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "lancet_moe_scatter": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp]),
+    "lancet_moe_encode_bpr_workspace_bytes": (_sz, [_i64, _i64, _int]),
+    "lancet_moe_encode_bpr": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _u32,
+                                     _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "lancet_moe_decode": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp]),
+    "lancet_moe_top2_normalize_gates": (_int, [_vp, _vp, _i64, _vp, _vp]),
+    "lancet_moe_merge_masks_workspace_bytes": (_sz, [_int, _i64]),
+    "lancet_moe_merge_masks": (_int, [C.POINTER(_vp), _int, _i64, _i64, _vp, _vp, _sz, _vp]),
+    "lancet_moe_redispatch_workspace_bytes": (_sz, [_int, _i64]),
+    "lancet_moe_redispatch": (_int, [C.POINTER(_vp), C.POINTER(_vp), _int, _i64, _i64, _i64, _i64, _int,
+                                     _vp, _vp, _sz, _vp]),
+    "lancet_lans_plan_create": (_int, [C.POINTER(_i64), _int, C.POINTER(_vp)]),
+    "lancet_lans_plan_destroy": (_int, [_vp]),
+    "lancet_lans_step": (_int, [_vp, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),
+                                _int, _vp, C.POINTER(LansHyper), _vp]),
+    "lancet_lans_plan_norms": (_int, [_vp, _vp, _vp]),
+    "lancet_debug_set_spin_limit": (None, [_u32]),
+    "lancet_scan_workspace_error": (_int, [_vp, _vp, C.POINTER(_int)]),
+}
+
+_lib = None
+
+
+def load():
+    """Returns the ctypes library with typed entry points; raises if it was not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            "liblancet_hip.so is not built (%s). Run `python %s` first; there is no fallback path."
+            % (LIB_PATH, os.path.join(HERE, "build.py")))
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)   # AttributeError = header and library disagree
+        fn.restype = res
+        fn.argtypes = args
+    got = lib.lancet_abi_version()
+    if got != 1:
+        raise RuntimeError("liblancet_hip.so has ABI version %d, expected 1" % got)
+    _lib = lib
+    return lib
+
+
+def status_string(status):
+    return load().lancet_status_string(int(status)).decode()
+
+
+def check(status, what):
+    if status != 0:
+        raise LancetError(status, what)
+
+
+def ptr_array(ptrs):
+    arr = (_vp * len(ptrs))()
+    for i, p in enumerate(ptrs):
+        arr[i] = p
+    return arr

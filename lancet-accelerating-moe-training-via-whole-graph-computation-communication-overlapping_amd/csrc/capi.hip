@@ -1,0 +1,302 @@
+// C ABI of the MoE dispatch path: argument validation, then kernel launches on the caller's
+// stream.  Nothing here allocates, synchronises or keeps state between calls.
+#include "../../include/lancet_hip.h"
+#include "launchers.hpp"
+
+using namespace lancet;
+
+namespace {
+
+inline hipStream_t S_(lancet_stream_t s) { return static_cast<hipStream_t>(s); }
+inline int rc(hipError_t e) { return static_cast<int>(e); }
+
+inline int elem_bytes(int dtype) {
+  switch (dtype) {
+    case LANCET_F32: return 4;
+    case LANCET_BF16:
+    case LANCET_F16: return 2;
+    default: return 0;
+  }
+}
+
+inline bool misaligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
+
+// S, M, C, E and the products the kernels index with must fit what the kernels assume.
+int check_dims(int64_t S, int64_t M, int64_t E, int64_t C) {
+  if (S < 0 || M < 0 || C < 0 || E < 1) return LANCET_ERR_SHAPE;
+  if (E > LANCET_MAX_EXPERTS) return LANCET_ERR_SHAPE;
+  if (S > 0x3fffffff || M > 0x3fffffff || C > 0x3fffffff) return LANCET_ERR_SHAPE;
+  if (E * C > 0x7fffffff) return LANCET_ERR_SHAPE;
+  return LANCET_OK;
+}
+
+}  // namespace
+
+extern "C" int lancet_abi_version(void) { return LANCET_ABI_VERSION; }
+
+extern "C" const char* lancet_status_string(int status) {
+  switch (status) {
+    case LANCET_OK: return "ok";
+    case LANCET_ERR_NULL: return "required pointer is NULL";
+    case LANCET_ERR_SHAPE: return "bad or unsupported size";
+    case LANCET_ERR_DTYPE: return "unknown dtype";
+    case LANCET_ERR_WORKSPACE: return "workspace missing or too small";
+    case LANCET_ERR_ALIGN: return "pointer not aligned to its element type";
+    case LANCET_ERR_TOPK: return "top_k must be 1 or 2 (2 needs at least two experts)";
+    case LANCET_ERR_PARTITION: return "bad n_partitions / partition_id";
+    case LANCET_ERR_PLAN: return "invalid LANS plan";
+    default: return status > 0 ? hipGetErrorString(static_cast<hipError_t>(status)) : "unknown status";
+  }
+}
+
+extern "C" int64_t lancet_moe_capacity(int64_t S, int64_t E, float capacity_factor) {
+  if (E <= 0 || S < 0) return -1;
+  // float * integer in float, truncated: src/op/dialect/cuda/moe.cc:109
+  return static_cast<int64_t>(static_cast<int>(capacity_factor * static_cast<float>((S + E - 1) / E)));
+}
+
+extern "C" void lancet_debug_set_spin_limit(unsigned limit) { set_spin_limit(limit); }
+
+extern "C" int lancet_scan_workspace_error(const void* workspace, lancet_stream_t stream, int* error_out) {
+  if (!workspace || !error_out) return LANCET_ERR_NULL;
+  uint32_t word = 0;
+  hipError_t e = hipMemcpyAsync(&word, static_cast<const uint32_t*>(workspace) + 1, sizeof(word),
+                                hipMemcpyDeviceToHost, S_(stream));
+  if (e == hipSuccess) e = hipStreamSynchronize(S_(stream));
+  *error_out = static_cast<int>(word);
+  return rc(e);
+}
+
+// ---- routing front end ---------------------------------------------------------------
+extern "C" int lancet_gate_topk(const float* gate, int64_t S, int64_t E, int top_k, unsigned flags,
+                                int32_t* idx, float* val, lancet_stream_t stream) {
+  if (!gate || !idx || !val) return LANCET_ERR_NULL;
+  if (int r = check_dims(S, 0, E, 0)) return r;
+  if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
+  if (top_k == 2 && E < 2) return LANCET_ERR_TOPK;
+  if (misaligned(gate, 4) || misaligned(idx, 4) || misaligned(val, 4)) return LANCET_ERR_ALIGN;
+  return rc(run_gate_topk(gate, static_cast<int>(S), static_cast<int>(E), top_k,
+                          (flags & LANCET_GATE_IS_LOGITS) != 0, idx, val, S_(stream)));
+}
+
+// ---- launcher level ------------------------------------------------------------------
+extern "C" size_t lancet_gen_location_workspace_bytes(int64_t S, int64_t E) {
+  if (S < 0 || E < 1) return 0;
+  return scan_workspace_bytes(S, E, 1);
+}
+
+extern "C" int lancet_launch_gen_location(int32_t* indices, const int32_t* in_capused, int32_t* locations,
+                                          int32_t* out_capused, uint64_t* out_elements_per_expert,
+                                          int64_t C, int64_t S, int64_t E, int64_t M, void* workspace,
+                                          size_t workspace_bytes, lancet_stream_t stream) {
+  if (!indices || !locations || !out_capused || !out_elements_per_expert) return LANCET_ERR_NULL;
+  if (int r = check_dims(S, M, E, C)) return r;
+  if (!workspace || workspace_bytes < lancet_gen_location_workspace_bytes(S, E)) return LANCET_ERR_WORKSPACE;
+  if (misaligned(indices, 4) || misaligned(locations, 4) || misaligned(out_capused, 4) ||
+      misaligned(out_elements_per_expert, 8) || misaligned(workspace, 4) || misaligned(in_capused, 4))
+    return LANCET_ERR_ALIGN;
+  return rc(run_route_scan(nullptr, indices, in_capused, static_cast<int>(S), static_cast<int>(E),
+                           static_cast<int>(C), static_cast<int>(M), 1, false, nullptr, indices, locations,
+                           out_capused, out_elements_per_expert, workspace, S_(stream)));
+}
+
+extern "C" int lancet_launch_encode_forward(const int32_t* indices, const int32_t* locations,
+                                            const int32_t* capused, const void* data, void* dispatched,
+                                            int64_t S, int64_t M, int64_t C, int64_t E, int dtype,
+                                            lancet_stream_t stream) {
+  if (!indices || !locations || !dispatched || (!data && S > 0)) return LANCET_ERR_NULL;
+  const int eb = elem_bytes(dtype);
+  if (!eb) return LANCET_ERR_DTYPE;
+  if (int r = check_dims(S, M, E, C)) return r;
+  if (misaligned(data, eb) || misaligned(dispatched, eb) || misaligned(indices, 4) || misaligned(locations, 4))
+    return LANCET_ERR_ALIGN;
+  // rows filled by an arbitrary (indices, locations) pair need not form a prefix, so the
+  // buffer is cleared first, as the reference launcher does
+  hipError_t e = run_zero_bytes(dispatched, static_cast<size_t>(E) * C * M * eb, S_(stream));
+  if (e != hipSuccess) return rc(e);
+  return rc(run_scatter_rows(data, dispatched, indices, locations, capused, nullptr, nullptr,
+                             static_cast<int>(S), static_cast<int>(M), static_cast<int>(E),
+                             static_cast<int>(C), 1, eb, S_(stream)));
+}
+
+// ---- raf.op.moe_encode ---------------------------------------------------------------
+extern "C" size_t lancet_moe_encode_workspace_bytes(int64_t S, int64_t E, int top_k) {
+  if (S < 0 || E < 1 || (top_k != 1 && top_k != 2)) return 0;
+  return scan_workspace_bytes(S, E, top_k);
+}
+
+extern "C" int lancet_moe_route(const float* gate, const int32_t* used_in, int64_t S, int64_t M, int64_t E,
+                                int64_t C, int top_k, unsigned flags, float* gates_s,
+                                int32_t* indices_locations, int32_t* used_out, uint64_t* elements_per_expert,
+                                void* workspace, size_t workspace_bytes, lancet_stream_t stream) {
+  if (((!gate || !gates_s || !indices_locations) && S > 0) || !used_out || !elements_per_expert)
+    return LANCET_ERR_NULL;
+  if (int r = check_dims(S, M, E, C)) return r;
+  if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
+  if (top_k == 2 && E < 2) return LANCET_ERR_TOPK;
+  if (!workspace || workspace_bytes < lancet_moe_encode_workspace_bytes(S, E, top_k)) return LANCET_ERR_WORKSPACE;
+  if (misaligned(gate, 4) || misaligned(gates_s, 4) || misaligned(indices_locations, 4) || misaligned(used_in, 4) ||
+      misaligned(used_out, 4) || misaligned(elements_per_expert, 8) || misaligned(workspace, 4))
+    return LANCET_ERR_ALIGN;
+  const int s = static_cast<int>(S);
+  return rc(run_route_scan(gate, nullptr, used_in, s, static_cast<int>(E), static_cast<int>(C),
+                           static_cast<int>(M), top_k, (flags & LANCET_GATE_IS_LOGITS) != 0, gates_s,
+                           indices_locations, indices_locations + static_cast<size_t>(top_k) * s, used_out,
+                           elements_per_expert, workspace, S_(stream)));
+}
+
+extern "C" int lancet_moe_scatter(const void* data, const int32_t* indices_locations, const int32_t* used_in,
+                                  const int32_t* used_out, int64_t S, int64_t M, int64_t E, int64_t C, int top_k,
+                                  int dtype, void* dispatched, lancet_stream_t stream) {
+  if ((!data && S > 0 && M > 0) || (!indices_locations && S > 0) || !used_out || (!dispatched && C > 0 && M > 0))
+    return LANCET_ERR_NULL;
+  const int eb = elem_bytes(dtype);
+  if (!eb) return LANCET_ERR_DTYPE;
+  if (int r = check_dims(S, M, E, C)) return r;
+  if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
+  if (misaligned(data, eb) || misaligned(dispatched, eb) || misaligned(indices_locations, 4) ||
+      misaligned(used_in, 4) || misaligned(used_out, 4))
+    return LANCET_ERR_ALIGN;
+  const int s = static_cast<int>(S);
+  return rc(run_scatter_rows(data, dispatched, indices_locations, indices_locations + static_cast<size_t>(top_k) * s,
+                             nullptr, used_in, used_out, s, static_cast<int>(M), static_cast<int>(E),
+                             static_cast<int>(C), top_k, eb, S_(stream)));
+}
+
+extern "C" int lancet_moe_encode(const void* data, const float* gate, const int32_t* used_in, int64_t S,
+                                 int64_t M, int64_t E, int64_t C, int top_k, int dtype, unsigned flags,
+                                 float* gates_s, int32_t* indices_locations, int32_t* used_out,
+                                 uint64_t* elements_per_expert, void* dispatched, void* workspace,
+                                 size_t workspace_bytes, lancet_stream_t stream) {
+  // validate everything before the first launch
+  if ((!data && S > 0 && M > 0) || (!dispatched && C > 0 && M > 0)) return LANCET_ERR_NULL;
+  const int eb = elem_bytes(dtype);
+  if (!eb) return LANCET_ERR_DTYPE;
+  if (misaligned(data, eb) || misaligned(dispatched, eb)) return LANCET_ERR_ALIGN;
+  if (int r = lancet_moe_route(gate, used_in, S, M, E, C, top_k, flags, gates_s, indices_locations, used_out,
+                               elements_per_expert, workspace, workspace_bytes, stream))
+    return r;
+  return lancet_moe_scatter(data, indices_locations, used_in, used_out, S, M, E, C, top_k, dtype, dispatched, stream);
+}
+
+// ---- raf.op.moe_encode_batch_prioritized ----------------------------------------------
+extern "C" size_t lancet_moe_encode_bpr_workspace_bytes(int64_t S0, int64_t E, int n_partitions) {
+  if (S0 < 0 || E < 1 || n_partitions < 1) return 0;
+  return bpr_workspace_bytes(S0, S0 / n_partitions, E);
+}
+
+extern "C" int lancet_moe_encode_bpr(const void* data, const float* gate, int64_t S0, int64_t M, int64_t E,
+                                     int64_t C, int n_partitions, int partition_id, int dtype, unsigned flags,
+                                     float* gates_s, int32_t* indices_locations, int32_t* used_out,
+                                     uint64_t* elements_per_expert, void* dispatched, void* workspace,
+                                     size_t workspace_bytes, lancet_stream_t stream) {
+  if ((!data && S0 > 0 && M > 0) || ((!gate || !gates_s || !indices_locations) && S0 > 0) || !used_out ||
+      !elements_per_expert || (!dispatched && C > 0 && M > 0))
+    return LANCET_ERR_NULL;
+  const int eb = elem_bytes(dtype);
+  if (!eb) return LANCET_ERR_DTYPE;
+  if (int r = check_dims(S0, M, E, C)) return r;
+  // src/op/declare/moe.cc:74-75
+  if (n_partitions < 1 || partition_id < 0 || partition_id >= n_partitions) return LANCET_ERR_PARTITION;
+  if (!workspace || workspace_bytes < lancet_moe_encode_bpr_workspace_bytes(S0, E, n_partitions))
+    return LANCET_ERR_WORKSPACE;
+  if (misaligned(data, eb) || misaligned(dispatched, eb) || misaligned(gate, 4) || misaligned(gates_s, 4) ||
+      misaligned(indices_locations, 4) || misaligned(used_out, 4) || misaligned(elements_per_expert, 8) ||
+      misaligned(workspace, 4))
+    return LANCET_ERR_ALIGN;
+  const int s0 = static_cast<int>(S0);
+  const int s = s0 / n_partitions;
+  int32_t* idx = indices_locations;
+  int32_t* loc = indices_locations + s;
+  hipError_t e = run_bpr_route(gate, s0, static_cast<int>(E), static_cast<int>(C), static_cast<int>(M),
+                               n_partitions, partition_id, (flags & LANCET_GATE_IS_LOGITS) != 0, gates_s, idx,
+                               loc, used_out, elements_per_expert, workspace, S_(stream));
+  if (e != hipSuccess) return rc(e);
+  const char* part = static_cast<const char*>(data) + static_cast<size_t>(partition_id) * s * M * eb;
+  return rc(run_scatter_rows(part, dispatched, idx, loc, nullptr, nullptr, used_out, s, static_cast<int>(M),
+                             static_cast<int>(E), static_cast<int>(C), 1, eb, S_(stream)));
+}
+
+// ---- raf.op.moe_decode ---------------------------------------------------------------
+extern "C" int lancet_moe_decode(const void* expert_out, const float* gates_s, const int32_t* indices_locations,
+                                 int64_t S, int64_t M, int64_t E, int64_t C, int top_k, int dtype, void* out,
+                                 lancet_stream_t stream) {
+  if ((!expert_out && C > 0 && M > 0) || ((!gates_s || !indices_locations) && S > 0) || (!out && S > 0 && M > 0))
+    return LANCET_ERR_NULL;
+  const int eb = elem_bytes(dtype);
+  if (!eb) return LANCET_ERR_DTYPE;
+  if (int r = check_dims(S, M, E, C)) return r;
+  if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
+  if (misaligned(expert_out, eb) || misaligned(out, eb) || misaligned(gates_s, 4) || misaligned(indices_locations, 4))
+    return LANCET_ERR_ALIGN;
+  const int s = static_cast<int>(S);
+  return rc(run_decode_rows(expert_out, gates_s, indices_locations, indices_locations + static_cast<size_t>(top_k) * s,
+                            out, s, static_cast<int>(M), static_cast<int>(E), static_cast<int>(C), top_k, dtype,
+                            S_(stream)));
+}
+
+extern "C" int lancet_moe_top2_normalize_gates(const float* raw_gates, const int32_t* merged_indices, int64_t S,
+                                               float* gates_out, lancet_stream_t stream) {
+  if (S < 0 || S > 0x3fffffff) return LANCET_ERR_SHAPE;
+  if (S == 0) return LANCET_OK;
+  if (!raw_gates || !merged_indices || !gates_out) return LANCET_ERR_NULL;
+  if (misaligned(raw_gates, 4) || misaligned(merged_indices, 4) || misaligned(gates_out, 4)) return LANCET_ERR_ALIGN;
+  return rc(run_top2_normalize(raw_gates, merged_indices, static_cast<int>(S), gates_out, S_(stream)));
+}
+
+// ---- raf.op.moe_merge_masks / raf.op.moe_redispatch -------------------------------------
+static int fill_table(PtrTable& t, const void* const* ptrs, int P, size_t align) {
+  for (int p = 0; p < P; ++p) {
+    if (!ptrs[p]) return LANCET_ERR_NULL;
+    if (misaligned(ptrs[p], align)) return LANCET_ERR_ALIGN;
+    t.p[p] = ptrs[p];
+  }
+  for (int p = P; p < kMaxPartitions; ++p) t.p[p] = nullptr;
+  return LANCET_OK;
+}
+
+extern "C" size_t lancet_moe_merge_masks_workspace_bytes(int P, int64_t E) {
+  if (P < 1 || E < 1) return 0;
+  return static_cast<size_t>(P) * E * sizeof(uint32_t);
+}
+
+extern "C" int lancet_moe_merge_masks(const int32_t* const* indices_locations, int P, int64_t S, int64_t E,
+                                      int32_t* out, void* workspace, size_t workspace_bytes,
+                                      lancet_stream_t stream) {
+  if (!indices_locations || (!out && S > 0)) return LANCET_ERR_NULL;
+  if (P < 1 || P > LANCET_MAX_PARTITIONS) return LANCET_ERR_PARTITION;
+  if (int r = check_dims(S, 0, E, 0)) return r;
+  if (static_cast<int64_t>(P) * S > 0x3fffffff) return LANCET_ERR_SHAPE;
+  if (!workspace || workspace_bytes < lancet_moe_merge_masks_workspace_bytes(P, E)) return LANCET_ERR_WORKSPACE;
+  if (misaligned(out, 4) || misaligned(workspace, 4)) return LANCET_ERR_ALIGN;
+  PtrTable t;
+  if (int r = fill_table(t, reinterpret_cast<const void* const*>(indices_locations), P, 4)) return r;
+  uint32_t* counts = static_cast<uint32_t*>(workspace);
+  hipError_t e = run_count_experts(t, P, static_cast<int>(S), static_cast<int>(E), counts, S_(stream));
+  if (e != hipSuccess) return rc(e);
+  return rc(run_merge_masks(t, P, static_cast<int>(S), static_cast<int>(E), counts, out, S_(stream)));
+}
+
+extern "C" size_t lancet_moe_redispatch_workspace_bytes(int P, int64_t E) {
+  return lancet_moe_merge_masks_workspace_bytes(P, E);
+}
+
+extern "C" int lancet_moe_redispatch(const void* const* data, const int32_t* const* indices_locations, int P,
+                                     int64_t S, int64_t M, int64_t C, int64_t E, int dtype, void* out,
+                                     void* workspace, size_t workspace_bytes, lancet_stream_t stream) {
+  if (!data || !indices_locations || (!out && C > 0 && M > 0)) return LANCET_ERR_NULL;
+  const int eb = elem_bytes(dtype);
+  if (!eb) return LANCET_ERR_DTYPE;
+  if (P < 1 || P > LANCET_MAX_PARTITIONS) return LANCET_ERR_PARTITION;
+  if (int r = check_dims(S, M, E, C)) return r;
+  if (!workspace || workspace_bytes < lancet_moe_redispatch_workspace_bytes(P, E)) return LANCET_ERR_WORKSPACE;
+  if (misaligned(out, eb) || misaligned(workspace, 4)) return LANCET_ERR_ALIGN;
+  PtrTable masks, bufs;
+  if (int r = fill_table(masks, reinterpret_cast<const void* const*>(indices_locations), P, 4)) return r;
+  if (int r = fill_table(bufs, data, P, eb)) return r;
+  uint32_t* counts = static_cast<uint32_t*>(workspace);
+  hipError_t e = run_count_experts(masks, P, static_cast<int>(S), static_cast<int>(E), counts, S_(stream));
+  if (e != hipSuccess) return rc(e);
+  return rc(run_redispatch_rows(bufs, P, static_cast<int>(M), static_cast<int>(C), static_cast<int>(E), counts, out,
+                                eb, S_(stream)));
+}

@@ -1,0 +1,58 @@
+// Host-side launch functions of the kernels; the C ABI (capi.hip) validates arguments and
+// calls these.  All sizes have been checked by the caller: S, M, E, C fit in int32,
+// E <= LANCET_MAX_EXPERTS, pointers are non-null where required.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace lancet {
+
+constexpr int kMaxPartitions = 64;
+
+// ---- routing (moe_route.hip) ------------------------------------------------------
+int64_t scan_num_tiles(int64_t S);
+size_t scan_workspace_bytes(int64_t S, int64_t E, int nsets);
+size_t bpr_workspace_bytes(int64_t S0, int64_t S, int64_t E);
+uint32_t current_spin_limit();
+void set_spin_limit(uint32_t limit);
+
+hipError_t run_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t st);
+hipError_t run_gate_topk(const float* gate, int S, int E, int K, bool is_logits, int32_t* idx,
+                         float* val, hipStream_t st);
+// gate-driven (idx_in == nullptr) or index-driven (gate == nullptr, K == 1) routing + scan.
+// idx_out/loc_out are [K*S] each.
+hipError_t run_route_scan(const float* gate, const int32_t* idx_in, const int32_t* used_in, int S,
+                          int E, int C, int M, int K, bool is_logits, float* gates_s,
+                          int32_t* idx_out, int32_t* loc_out, int32_t* used_out,
+                          uint64_t* elems_out, void* ws, hipStream_t st);
+hipError_t run_bpr_route(const float* gate, int S0, int E, int C, int M, int n_partitions,
+                         int partition_id, bool is_logits, float* gates_s, int32_t* idx_out,
+                         int32_t* loc_out, int32_t* used_out, uint64_t* elems_out, void* ws,
+                         hipStream_t st);
+hipError_t run_top2_normalize(const float* raw, const int32_t* idx, int S, float* out, hipStream_t st);
+
+// ---- row movers (moe_rows.hip) ------------------------------------------------------
+// Scatter of token rows into [E,C,M].  avail_used (may be null): only rows with
+// loc < C - avail_used[idx] are written (the reference's capused test).  When rows_hi is
+// non-null the launch also zero-fills rows [rows_hi[e] - rows_lo[e], C) of every expert
+// (rows_lo may be null = zeros); otherwise the caller has cleared the buffer.
+hipError_t run_scatter_rows(const void* data, void* out, const int32_t* idx, const int32_t* loc,
+                            const int32_t* avail_used, const int32_t* rows_lo, const int32_t* rows_hi,
+                            int S, int M, int E, int C, int K, int elem_bytes, hipStream_t st);
+hipError_t run_zero_bytes(void* p, size_t nbytes, hipStream_t st);
+hipError_t run_decode_rows(const void* expert_out, const float* gates, const int32_t* idx,
+                           const int32_t* loc, void* out, int S, int M, int E, int C, int K,
+                           int dtype, hipStream_t st);
+
+struct PtrTable {
+  const void* p[kMaxPartitions];
+};
+// counts[P][E] (zeroed by the call) = number of tokens of partition p whose index is e
+hipError_t run_count_experts(const PtrTable& indlocs, int P, int S, int E, uint32_t* counts, hipStream_t st);
+hipError_t run_merge_masks(const PtrTable& indlocs, int P, int S, int E, const uint32_t* counts,
+                           int32_t* out, hipStream_t st);
+hipError_t run_redispatch_rows(const PtrTable& bufs, int P, int M, int C, int E, const uint32_t* counts,
+                               void* out, int elem_bytes, hipStream_t st);
+
+}  // namespace lancet

@@ -1,0 +1,489 @@
+// Routing kernels: gate softmax + top-1/top-2 selection fused with the capacity-bounded
+// position scan, the top-2 finalisation, and the batch-prioritised (radix select) variant.
+#include "launchers.hpp"
+#include "scan.hpp"
+#include <algorithm>
+
+namespace lancet {
+
+// ---------------------------------------------------------------------------------------
+// Per-token selection on the array the op is given (first max wins; slot 2 = first max with
+// slot 1's expert excluded).  With logits the returned values are softmax probabilities,
+// exp(x - max) / sum_e exp(x - max), the sum taken in expert order.
+// Replaces the argmax / one_hot / multiply+sum micro-kernels of
+// src/op/dialect/cuda/moe.cc:177-250 (three passes over [S,E] plus an [S,E] workspace).
+// ---------------------------------------------------------------------------------------
+template <int K>
+__device__ __forceinline__ void route_token(const float* __restrict__ row, int E, bool is_logits,
+                                            int (&e)[K], float (&p)[K]) {
+  float v1 = 0.f, v2 = 0.f;
+  int i1 = -1, i2 = -1;
+  for (int j = 0; j < E; ++j) {
+    const float x = row[j];
+    if (i1 < 0 || x > v1) {
+      v2 = v1;
+      i2 = i1;
+      v1 = x;
+      i1 = j;
+    } else if (K == 2 && (i2 < 0 || x > v2)) {
+      v2 = x;
+      i2 = j;
+    }
+  }
+  float inv = 1.f, sum = 0.f;
+  if (is_logits) {
+    for (int j = 0; j < E; ++j) sum += expf(row[j] - v1);
+    inv = sum;
+  }
+  e[0] = i1;
+  p[0] = is_logits ? expf(v1 - v1) / inv : v1;
+  if (K == 2) {
+    e[1] = i2;
+    p[1] = is_logits ? expf(v2 - v1) / inv : v2;
+  }
+}
+
+struct RouteArgs {
+  const float* gate;      // [S,E] (NULL when idx_in is given)
+  const int32_t* idx_in;  // launcher-level entry: expert per token already chosen (may alias idx_out)
+  const int32_t* used_in; // [E] or NULL (= zeros)
+  float* gates_s;         // [K*S] (NULL when idx_in is given)
+  int32_t* idx_out;       // [K*S]
+  int32_t* loc_out;       // [K*S]
+  int32_t* used_out;      // [E]
+  uint64_t* elems_out;    // [E]
+  ScanWs ws;
+  int S, E, C, M;
+  int ntiles;
+  int is_logits;
+  uint32_t spin_limit;
+};
+
+// K = 1: everything is final when the tile knows its prefix.
+// K = 2: ranks of both slots are produced in one pass (2E counters); slot-2 locations need the
+//        slot-1 totals of all tiles, so raw (expert, rank, value) are left in the output arrays
+//        and finalize_top2_kernel completes them.
+template <int K>
+__global__ __launch_bounds__(kTile) void route_scan_kernel(RouteArgs a) {
+  extern __shared__ uint32_t s_cnt[];
+  __shared__ uint32_t s_tile;
+  const int tid = threadIdx.x;
+  if (tid == 0) s_tile = atomicAdd(a.ws.ticket, 1u);
+  __syncthreads();
+  const uint32_t tile = s_tile;
+  const int s = static_cast<int>(tile) * kTile + tid;
+  const bool valid = s < a.S;
+
+  int e[K];
+  float p[K];
+#pragma unroll
+  for (int j = 0; j < K; ++j) {
+    e[j] = -1;
+    p[j] = 0.f;
+  }
+  if (valid) {
+    if (a.idx_in) {
+      const int x = a.idx_in[s];
+      e[0] = (x >= 0 && x < a.E) ? x : -1;
+    } else {
+      route_token<K>(a.gate + static_cast<size_t>(s) * a.E, a.E, a.is_logits != 0, e, p);
+    }
+  }
+  uint32_t rank[K];
+  bool mem[K];
+#pragma unroll
+  for (int j = 0; j < K; ++j) mem[j] = e[j] >= 0;
+  tile_scan<K>(e, mem, a.E, tile, a.ws, s_cnt, a.spin_limit, rank);
+
+  if (K == 1) {
+    if (valid) {
+      if (e[0] >= 0) {
+        const int used = a.used_in ? a.used_in[e[0]] : 0;
+        const int r = static_cast<int>(rank[0]);
+        a.loc_out[s] = r;
+        a.idx_out[s] = (r >= a.C - used) ? -1 : e[0];
+      } else if (!a.idx_in) {
+        a.idx_out[s] = -1;
+        a.loc_out[s] = 0;
+      }
+      if (a.gates_s) a.gates_s[s] = p[0];
+    }
+    if (static_cast<int>(tile) == a.ntiles - 1) {
+      const uint32_t* s_agg = s_cnt + kWavesPerTile * a.E;
+      const uint32_t* s_base = s_agg + a.E;
+      for (int c = tid; c < a.E; c += kTile) {
+        const int64_t used = a.used_in ? a.used_in[c] : 0;
+        const int64_t total = static_cast<int64_t>(s_base[c]) + s_agg[c];
+        const int64_t uo = min(used + total, static_cast<int64_t>(a.C));
+        a.used_out[c] = static_cast<int32_t>(uo);
+        a.elems_out[c] = static_cast<uint64_t>((uo - used) * a.M);
+      }
+    }
+  } else {
+    if (valid) {
+#pragma unroll
+      for (int j = 0; j < K; ++j) {
+        a.idx_out[static_cast<size_t>(j) * a.S + s] = e[j];
+        a.loc_out[static_cast<size_t>(j) * a.S + s] = static_cast<int>(rank[j]);
+        a.gates_s[static_cast<size_t>(j) * a.S + s] = p[j];
+      }
+    }
+  }
+}
+
+// Completes top-2 routing once all tiles are done: slot 1 is an ordinary top-1 encode with
+// used_in; slot 2 is a top-1 encode whose used capacity is slot 1's result; locations are in
+// the merged layout (slot-2 rows follow slot-1 rows of the same expert); combine weights are
+// taken after the drop and normalised (docker/resources/sharded_moe.py:282-312).
+__global__ __launch_bounds__(kTile) void finalize_top2_kernel(RouteArgs a) {
+  const int s = blockIdx.x * kTile + threadIdx.x;
+  const uint32_t* tot = a.ws.incl + static_cast<size_t>(a.ntiles - 1) * 2 * a.E;  // [2][E]
+  if (s < a.S) {
+    const int e1 = a.idx_out[s], e2 = a.idx_out[a.S + s];
+    const int r1 = a.loc_out[s], r2 = a.loc_out[a.S + s];
+    const int u1 = a.used_in ? a.used_in[e1] : 0;
+    const int u2 = a.used_in ? a.used_in[e2] : 0;
+    const bool keep1 = r1 < a.C - u1;
+    const int64_t after1 = min(static_cast<int64_t>(u2) + ld_agent(tot + e2), static_cast<int64_t>(a.C));
+    const bool keep2 = r2 < a.C - after1;
+    a.idx_out[s] = keep1 ? e1 : -1;
+    a.loc_out[s] = keep1 ? r1 : -1;
+    a.idx_out[a.S + s] = keep2 ? e2 : -1;
+    a.loc_out[a.S + s] = keep2 ? r2 + static_cast<int>(after1 - u2) : -1;
+    const float g1 = keep1 ? a.gates_s[s] : 0.f;
+    const float g2 = keep2 ? a.gates_s[a.S + s] : 0.f;
+    const float den = fmaxf(g1 + g2, 1.1920929e-07f);
+    a.gates_s[s] = g1 / den;
+    a.gates_s[a.S + s] = g2 / den;
+  }
+  if (blockIdx.x == 0) {
+    for (int c = threadIdx.x; c < a.E; c += kTile) {
+      const int64_t used = a.used_in ? a.used_in[c] : 0;
+      const int64_t total = static_cast<int64_t>(ld_agent(tot + c)) + ld_agent(tot + a.E + c);
+      const int64_t uo = min(used + total, static_cast<int64_t>(a.C));
+      a.used_out[c] = static_cast<int32_t>(uo);
+      a.elems_out[c] = static_cast<uint64_t>((uo - used) * a.M);
+    }
+  }
+}
+
+// Selection only (no scan).
+template <int K>
+__global__ __launch_bounds__(kTile) void gate_topk_kernel(const float* gate, int S, int E, int is_logits,
+                                                          int32_t* idx, float* val) {
+  const int s = blockIdx.x * kTile + threadIdx.x;
+  if (s >= S) return;
+  int e[K];
+  float p[K];
+  route_token<K>(gate + static_cast<size_t>(s) * E, E, is_logits != 0, e, p);
+#pragma unroll
+  for (int j = 0; j < K; ++j) {
+    idx[static_cast<size_t>(j) * S + s] = e[j];
+    val[static_cast<size_t>(j) * S + s] = p[j];
+  }
+}
+
+__global__ void top2_normalize_kernel(const float* raw, const int32_t* idx, int S, float* out) {
+  const int s = blockIdx.x * blockDim.x + threadIdx.x;
+  if (s >= S) return;
+  const float g1 = idx[s] >= 0 ? raw[s] : 0.f;
+  const float g2 = idx[S + s] >= 0 ? raw[S + s] : 0.f;
+  const float den = fmaxf(g1 + g2, 1.1920929e-07f);
+  out[s] = g1 / den;
+  out[S + s] = g2 / den;
+}
+
+__global__ void fill_u32_kernel(uint32_t* p, size_t n, uint32_t v) {
+  for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < n;
+       i += static_cast<size_t>(gridDim.x) * blockDim.x)
+    p[i] = v;
+}
+
+// ---------------------------------------------------------------------------------------
+// Batch-prioritised routing.
+//   bpr_select_kernel : one workgroup per expert.  Finds, with a 4 x 8-bit radix select on the
+//                       order-preserving integer image of the fp32 priority, the C-th largest
+//                       priority among the expert's tokens (threshold), how many ties at the
+//                       threshold may stay (quota, lowest token ids first) and how many ties
+//                       lie before the partition (ties_before).
+//   bpr_scan_kernel   : tile scan over the partition with two counter sets (tokens above the
+//                       threshold / tokens at the threshold); a token stays iff it is above,
+//                       or at the threshold with global tie rank < quota; its location is
+//                       above_before + min(tie_rank, quota) - min(ties_before, quota).
+// Equivalent to the reference's stable descending argsort + keep-first-C + compaction
+// (src/op/dialect/cuda/moe.cc:638-683, tutel_moe_dispatch.cu:259-363) without sorting.
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t order_key(float x) {
+  if (x == 0.f) x = 0.f;  // -0 and +0 compare equal in a float sort
+  const uint32_t u = __float_as_uint(x);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+struct BprArgs {
+  const int32_t* idx0;   // [S0] expert per token
+  const float* prio;     // [S0] priority (gate value of the chosen expert)
+  uint32_t* thresh;      // [E]
+  int32_t* quota;        // [E]
+  int32_t* ties_before;  // [E]
+  int S0, S, E, C, M;
+  int part_lo;           // first token of the partition
+  int ntiles;
+  float* gates_s;        // [S]
+  int32_t* idx_out;      // [S]
+  int32_t* loc_out;      // [S]
+  int32_t* used_out;     // [E]
+  uint64_t* elems_out;   // [E]
+  ScanWs ws;
+  uint32_t spin_limit;
+};
+
+constexpr int kSelectThreads = 1024;
+
+__global__ __launch_bounds__(kSelectThreads) void bpr_select_kernel(BprArgs a) {
+  __shared__ uint32_t hist[256];
+  __shared__ uint32_t s_prefix, s_need, s_count;
+  const int e = blockIdx.x;
+  const int tid = threadIdx.x;
+  if (tid == 0) s_count = 0;
+  __syncthreads();
+  uint32_t local = 0;
+  for (int s = tid; s < a.S0; s += kSelectThreads) local += (a.idx0[s] == e);
+  if (local) atomicAdd(&s_count, local);
+  __syncthreads();
+  const uint32_t count = s_count;
+  if (a.C <= 0) {
+    // nothing fits: no key is above the largest threshold and the tie quota is zero
+    if (tid == 0) {
+      a.thresh[e] = 0xffffffffu;
+      a.quota[e] = 0;
+      a.ties_before[e] = 0;
+    }
+    return;
+  }
+  if (count <= static_cast<uint32_t>(a.C)) {
+    // everything fits: every key is above threshold 0 or ties with it under an unlimited quota
+    if (tid == 0) {
+      a.thresh[e] = 0u;
+      a.quota[e] = 0x7fffffff;
+      a.ties_before[e] = 0;
+    }
+    return;
+  }
+  if (tid == 0) {
+    s_prefix = 0;
+    s_need = static_cast<uint32_t>(a.C);
+  }
+  for (int pass = 0; pass < 4; ++pass) {
+    const int shift = 24 - 8 * pass;
+    if (tid < 256) hist[tid] = 0;
+    __syncthreads();
+    const uint32_t prefix = s_prefix;
+    for (int s = tid; s < a.S0; s += kSelectThreads) {
+      if (a.idx0[s] != e) continue;
+      const uint32_t k = order_key(a.prio[s]);
+      if (pass == 0 || (k >> (shift + 8)) == prefix) atomicAdd(&hist[(k >> shift) & 0xffu], 1u);
+    }
+    __syncthreads();
+    if (tid == 0) {
+      uint32_t need = s_need;
+      int d = 255;
+      for (; d > 0; --d) {
+        if (need <= hist[d]) break;
+        need -= hist[d];
+      }
+      s_need = need;
+      s_prefix = (prefix << 8) | static_cast<uint32_t>(d);
+    }
+    __syncthreads();
+  }
+  const uint32_t thr = s_prefix;
+  // ties that precede the partition
+  if (tid == 0) s_count = 0;
+  __syncthreads();
+  local = 0;
+  for (int s = tid; s < a.part_lo; s += kSelectThreads)
+    local += (a.idx0[s] == e && order_key(a.prio[s]) == thr);
+  if (local) atomicAdd(&s_count, local);
+  __syncthreads();
+  if (tid == 0) {
+    a.thresh[e] = thr;
+    a.quota[e] = static_cast<int32_t>(s_need);
+    a.ties_before[e] = static_cast<int32_t>(s_count);
+  }
+}
+
+__global__ __launch_bounds__(kTile) void bpr_scan_kernel(BprArgs a) {
+  extern __shared__ uint32_t s_cnt[];
+  __shared__ uint32_t s_tile;
+  const int tid = threadIdx.x;
+  if (tid == 0) s_tile = atomicAdd(a.ws.ticket, 1u);
+  __syncthreads();
+  const uint32_t tile = s_tile;
+  const int sl = static_cast<int>(tile) * kTile + tid;  // token inside the partition
+  const bool valid = sl < a.S;
+  int cls[2] = {-1, -1};
+  bool mem[2] = {false, false};
+  float prio = 0.f;
+  if (valid) {
+    const int s = a.part_lo + sl;
+    const int e = a.idx0[s];
+    prio = a.prio[s];
+    if (e >= 0 && e < a.E) {
+      const uint32_t k = order_key(prio);
+      const uint32_t thr = a.thresh[e];
+      cls[0] = cls[1] = e;
+      mem[0] = k > thr;   // above the threshold: always stays
+      mem[1] = k == thr;  // at the threshold: stays while the quota lasts
+    }
+  }
+  uint32_t rank[2];
+  tile_scan<2>(cls, mem, a.E, tile, a.ws, s_cnt, a.spin_limit, rank);
+  if (valid) {
+    int idx = -1, loc = -1;
+    if (cls[0] >= 0) {
+      const int e = cls[0];
+      const int64_t q = a.quota[e];
+      const int64_t tb = a.ties_before[e];
+      const int64_t tie_rank = tb + rank[1];
+      if (mem[0] || (mem[1] && tie_rank < q)) {
+        idx = e;
+        loc = static_cast<int>(static_cast<int64_t>(rank[0]) + min(tie_rank, q) - min(tb, q));
+      }
+    }
+    a.idx_out[sl] = idx;
+    a.loc_out[sl] = loc;
+    a.gates_s[sl] = prio;
+  }
+  if (static_cast<int>(tile) == a.ntiles - 1) {
+    const uint32_t* s_agg = s_cnt + kWavesPerTile * 2 * a.E;
+    const uint32_t* s_base = s_agg + 2 * a.E;
+    for (int c = tid; c < a.E; c += kTile) {
+      const int64_t q = a.quota[c];
+      const int64_t tb = a.ties_before[c];
+      const int64_t above = static_cast<int64_t>(s_base[c]) + s_agg[c];
+      const int64_t ties = static_cast<int64_t>(s_base[a.E + c]) + s_agg[a.E + c];
+      const int64_t kept = above + min(tb + ties, q) - min(tb, q);
+      const int64_t uo = min(kept, static_cast<int64_t>(a.C));
+      a.used_out[c] = static_cast<int32_t>(uo);
+      a.elems_out[c] = static_cast<uint64_t>(uo * a.M);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------------
+static uint32_t g_spin_limit = 1u << 22;  // ~ seconds of polling; a healthy wait is microseconds
+
+uint32_t current_spin_limit() { return __atomic_load_n(&g_spin_limit, __ATOMIC_RELAXED); }
+void set_spin_limit(uint32_t limit) {
+  __atomic_store_n(&g_spin_limit, limit ? limit : (1u << 22), __ATOMIC_RELAXED);
+}
+
+int64_t scan_num_tiles(int64_t S) { return S > 0 ? (S + kTile - 1) / kTile : 1; }
+
+size_t scan_workspace_bytes(int64_t S, int64_t E, int nsets) {
+  return scan_ws_words(scan_num_tiles(S), nsets * E) * sizeof(uint32_t);
+}
+
+size_t bpr_workspace_bytes(int64_t S0, int64_t S, int64_t E) {
+  return scan_workspace_bytes(S, E, 2) + (2 * static_cast<size_t>(S0) + 3 * static_cast<size_t>(E)) * 4;
+}
+
+hipError_t run_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  const int blocks = static_cast<int>(std::min<size_t>((n + 255) / 256, 1024));
+  fill_u32_kernel<<<blocks, 256, 0, st>>>(p, n, v);
+  return hipGetLastError();
+}
+
+hipError_t run_gate_topk(const float* gate, int S, int E, int K, bool is_logits, int32_t* idx,
+                         float* val, hipStream_t st) {
+  if (S == 0) return hipSuccess;
+  const int blocks = (S + kTile - 1) / kTile;
+  if (K == 1) gate_topk_kernel<1><<<blocks, kTile, 0, st>>>(gate, S, E, is_logits, idx, val);
+  else gate_topk_kernel<2><<<blocks, kTile, 0, st>>>(gate, S, E, is_logits, idx, val);
+  return hipGetLastError();
+}
+
+hipError_t run_route_scan(const float* gate, const int32_t* idx_in, const int32_t* used_in, int S,
+                          int E, int C, int M, int K, bool is_logits, float* gates_s,
+                          int32_t* idx_out, int32_t* loc_out, int32_t* used_out,
+                          uint64_t* elems_out, void* ws, hipStream_t st) {
+  RouteArgs a;
+  a.gate = gate;
+  a.idx_in = idx_in;
+  a.used_in = used_in;
+  a.gates_s = gates_s;
+  a.idx_out = idx_out;
+  a.loc_out = loc_out;
+  a.used_out = used_out;
+  a.elems_out = elems_out;
+  a.S = S;
+  a.E = E;
+  a.C = C;
+  a.M = M;
+  a.ntiles = static_cast<int>(scan_num_tiles(S));
+  a.is_logits = is_logits;
+  a.spin_limit = current_spin_limit();
+  a.ws = scan_ws_view(ws, a.ntiles, K * E);
+  hipError_t err = run_fill_u32(static_cast<uint32_t*>(ws), kScanHeaderWords + a.ntiles, 0u, st);
+  if (err != hipSuccess) return err;
+  const size_t lds = scan_lds_bytes(K * E);
+  if (K == 1) {
+    route_scan_kernel<1><<<a.ntiles, kTile, lds, st>>>(a);
+  } else {
+    route_scan_kernel<2><<<a.ntiles, kTile, lds, st>>>(a);
+    err = hipGetLastError();
+    if (err != hipSuccess) return err;
+    finalize_top2_kernel<<<a.ntiles, kTile, 0, st>>>(a);
+  }
+  return hipGetLastError();
+}
+
+hipError_t run_bpr_route(const float* gate, int S0, int E, int C, int M, int n_partitions,
+                         int partition_id, bool is_logits, float* gates_s, int32_t* idx_out,
+                         int32_t* loc_out, int32_t* used_out, uint64_t* elems_out, void* ws,
+                         hipStream_t st) {
+  const int S = S0 / n_partitions;
+  BprArgs a;
+  a.S0 = S0;
+  a.S = S;
+  a.E = E;
+  a.C = C;
+  a.M = M;
+  a.part_lo = partition_id * S;
+  a.ntiles = static_cast<int>(scan_num_tiles(S));
+  a.ws = scan_ws_view(ws, a.ntiles, 2 * E);
+  uint32_t* extra = static_cast<uint32_t*>(ws) + scan_ws_words(a.ntiles, 2 * E);
+  int32_t* idx0 = reinterpret_cast<int32_t*>(extra);
+  float* prio = reinterpret_cast<float*>(extra + S0);
+  a.idx0 = idx0;
+  a.prio = prio;
+  a.thresh = extra + 2 * static_cast<size_t>(S0);
+  a.quota = reinterpret_cast<int32_t*>(a.thresh + E);
+  a.ties_before = a.quota + E;
+  a.gates_s = gates_s;
+  a.idx_out = idx_out;
+  a.loc_out = loc_out;
+  a.used_out = used_out;
+  a.elems_out = elems_out;
+  a.spin_limit = current_spin_limit();
+  hipError_t err = run_fill_u32(static_cast<uint32_t*>(ws), kScanHeaderWords + a.ntiles, 0u, st);
+  if (err != hipSuccess) return err;
+  err = run_gate_topk(gate, S0, E, 1, is_logits, idx0, prio, st);
+  if (err != hipSuccess) return err;
+  bpr_select_kernel<<<E, kSelectThreads, 0, st>>>(a);
+  err = hipGetLastError();
+  if (err != hipSuccess) return err;
+  bpr_scan_kernel<<<a.ntiles, kTile, scan_lds_bytes(2 * E), st>>>(a);
+  return hipGetLastError();
+}
+
+hipError_t run_top2_normalize(const float* raw, const int32_t* idx, int S, float* out, hipStream_t st) {
+  if (S == 0) return hipSuccess;
+  top2_normalize_kernel<<<(S + 255) / 256, 256, 0, st>>>(raw, idx, S, out);
+  return hipGetLastError();
+}
+
+}  // namespace lancet

@@ -1,0 +1,454 @@
+// Row movers: scatter of token rows into the [E,C,M] expert buffer, weighted gather-combine
+// back, partition merge of masks and buffers.  All are pure HBM streaming: one wave per row,
+// 16-byte accesses, streaming (non-temporal) loads and stores, every output byte written once.
+#include "launchers.hpp"
+#include "common.hpp"
+#include "../../include/lancet_hip.h"
+#include <algorithm>
+
+namespace lancet {
+
+constexpr int kRowsPerBlock = kTile / kWave;  // one wave per row
+constexpr int kTailRows = 16;                 // rows zero-filled by one tail workgroup
+
+// Access granule: 16 bytes when the row size and the pointers allow, else one element.
+template <typename V>
+__device__ __forceinline__ V ldv(const V* p) { return __builtin_nontemporal_load(p); }
+template <typename V>
+__device__ __forceinline__ void stv(V* p, V v) { __builtin_nontemporal_store(v, p); }
+template <typename V>
+__device__ __forceinline__ V zero_v() { return V(0); }
+template <>
+__device__ __forceinline__ u32x4 zero_v<u32x4>() { return u32x4{0u, 0u, 0u, 0u}; }
+
+// ---------------------------------------------------------------------------------------
+// encode_forward: out[idx, loc, :] = data[s, :]; rows no token lands on are zero.
+// Replaces cudaMemsetAsync + atomicAdd per element of
+// src/op/dialect/cuda/kernels/tutel_moe_dispatch.cu:61-81,461-484.
+// ---------------------------------------------------------------------------------------
+template <typename V>
+struct ScatterArgs {
+  const V* data;
+  V* out;
+  const int32_t* idx;         // [K*S]
+  const int32_t* loc;         // [K*S]
+  const int32_t* avail_used;  // [E] or null
+  const int32_t* rows_lo;     // [E] or null
+  const int32_t* rows_hi;     // [E] or null (no tail fill)
+  int S, E, C, K;
+  int row_vecs;               // granules per row
+  int token_blocks;
+  int tail_chunks;            // tail workgroups per expert
+};
+
+template <typename V, int K>
+__global__ __launch_bounds__(kTile) void scatter_rows_kernel(ScatterArgs<V> a) {
+  const int w = threadIdx.x / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  if (static_cast<int>(blockIdx.x) < a.token_blocks) {
+    const int s = blockIdx.x * kRowsPerBlock + w;
+    if (s >= a.S) return;
+    V* dst[K];
+    int nd = 0;
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+      const int e = a.idx[static_cast<size_t>(j) * a.S + s];
+      const int l = a.loc[static_cast<size_t>(j) * a.S + s];
+      bool ok = e >= 0 && e < a.E && l >= 0 && l < a.C;
+      if (ok && a.avail_used) ok = l < a.C - a.avail_used[e];
+      dst[j] = nullptr;
+      if (ok) dst[nd++] = a.out + (static_cast<size_t>(e) * a.C + l) * a.row_vecs;
+    }
+    if (nd == 0) return;
+    const V* src = a.data + static_cast<size_t>(s) * a.row_vecs;
+    int v = lane;
+    for (; v + 3 * kWave < a.row_vecs; v += 4 * kWave) {
+      const V x0 = ldv(src + v), x1 = ldv(src + v + kWave), x2 = ldv(src + v + 2 * kWave),
+              x3 = ldv(src + v + 3 * kWave);
+#pragma unroll
+      for (int j = 0; j < K; ++j) {
+        if (j < nd) {
+          stv(dst[j] + v, x0);
+          stv(dst[j] + v + kWave, x1);
+          stv(dst[j] + v + 2 * kWave, x2);
+          stv(dst[j] + v + 3 * kWave, x3);
+        }
+      }
+    }
+    for (; v < a.row_vecs; v += kWave) {
+      const V x = ldv(src + v);
+#pragma unroll
+      for (int j = 0; j < K; ++j)
+        if (j < nd) stv(dst[j] + v, x);
+    }
+  } else {
+    // tail: zero rows [used, C) of expert e, kTailRows rows per workgroup
+    const int tb = blockIdx.x - a.token_blocks;
+    const int e = tb / a.tail_chunks;
+    const int ch = tb - e * a.tail_chunks;
+    const int used = a.rows_hi[e] - (a.rows_lo ? a.rows_lo[e] : 0);
+    const int first = max(used, 0) + ch * kTailRows;
+    const int last = min(first + kTailRows, a.C);
+    const V z = zero_v<V>();
+    for (int r = first + w; r < last; r += kRowsPerBlock) {
+      V* row = a.out + (static_cast<size_t>(e) * a.C + r) * a.row_vecs;
+      for (int v = lane; v < a.row_vecs; v += kWave) stv(row + v, z);
+    }
+  }
+}
+
+__global__ void zero_bytes_kernel(u32x4* p, size_t nvec, uint8_t* tail, size_t ntail) {
+  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  const u32x4 z = {0u, 0u, 0u, 0u};
+  for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < nvec; i += stride)
+    __builtin_nontemporal_store(z, p + i);
+  if (blockIdx.x == 0 && threadIdx.x < ntail) tail[threadIdx.x] = 0;
+}
+
+// ---------------------------------------------------------------------------------------
+// decode_forward: out[s,:] = sum_j gates[j*S+s] * expert_out[idx, loc, :], fp32 products and
+// sum (no fused multiply-add, so that the result is one well-defined rounding sequence), one
+// rounding to the storage type.  Replaces tutel_moe_dispatch.cu:46-55,110-116,511-521.
+// ---------------------------------------------------------------------------------------
+template <int DT>
+struct Codec;
+template <>
+struct Codec<LANCET_F32> {
+  typedef uint32_t S;  // scalar storage
+  static constexpr int kPerVec = 4;
+  static __device__ __forceinline__ float get(S x) { return __uint_as_float(x); }
+  static __device__ __forceinline__ S put(float f) { return __float_as_uint(f); }
+};
+template <>
+struct Codec<LANCET_BF16> {
+  typedef uint16_t S;
+  static constexpr int kPerVec = 8;
+  static __device__ __forceinline__ float get(S x) { return bf16_to_f32(x); }
+  static __device__ __forceinline__ S put(float f) { return static_cast<S>(f32_to_bf16(f)); }
+};
+template <>
+struct Codec<LANCET_F16> {
+  typedef uint16_t S;
+  static constexpr int kPerVec = 8;
+  static __device__ __forceinline__ float get(S x) { return f16_to_f32(x); }
+  static __device__ __forceinline__ S put(float f) { return static_cast<S>(f32_to_f16(f)); }
+};
+
+template <int DT, int K>
+__device__ __forceinline__ u32x4 combine_vec(const u32x4 (&x)[K], const float (&g)[K]) {
+  typedef Codec<DT> Cd;
+  u32x4 r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if (Cd::kPerVec == 4) {
+      float acc = __fmul_rn(g[0], Cd::get(x[0][i]));
+      if (K == 2) acc = __fadd_rn(acc, __fmul_rn(g[1], Cd::get(x[1][i])));
+      r[i] = Cd::put(acc);
+    } else {
+      float lo = __fmul_rn(g[0], Cd::get(static_cast<typename Cd::S>(x[0][i] & 0xffffu)));
+      float hi = __fmul_rn(g[0], Cd::get(static_cast<typename Cd::S>(x[0][i] >> 16)));
+      if (K == 2) {
+        lo = __fadd_rn(lo, __fmul_rn(g[1], Cd::get(static_cast<typename Cd::S>(x[1][i] & 0xffffu))));
+        hi = __fadd_rn(hi, __fmul_rn(g[1], Cd::get(static_cast<typename Cd::S>(x[1][i] >> 16))));
+      }
+      r[i] = static_cast<uint32_t>(Cd::put(lo)) | (static_cast<uint32_t>(Cd::put(hi)) << 16);
+    }
+  }
+  return r;
+}
+
+struct DecodeArgs {
+  const void* expert_out;
+  const float* gates;    // [K*S]
+  const int32_t* idx;    // [K*S]
+  const int32_t* loc;    // [K*S]
+  void* out;             // [S, M]
+  int S, M, E, C;
+};
+
+template <int DT, int K, bool VEC>
+__global__ __launch_bounds__(kTile) void decode_rows_kernel(DecodeArgs a) {
+  typedef Codec<DT> Cd;
+  const int w = threadIdx.x / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int s = blockIdx.x * kRowsPerBlock + w;
+  if (s >= a.S) return;
+  float g[K];
+  size_t row[K];
+  bool ok[K];
+  bool any = false;
+#pragma unroll
+  for (int j = 0; j < K; ++j) {
+    const int e = a.idx[static_cast<size_t>(j) * a.S + s];
+    const int l = a.loc[static_cast<size_t>(j) * a.S + s];
+    ok[j] = e >= 0 && e < a.E && l >= 0 && l < a.C;
+    g[j] = ok[j] ? a.gates[static_cast<size_t>(j) * a.S + s] : 0.f;
+    row[j] = ok[j] ? (static_cast<size_t>(e) * a.C + l) : 0;
+    any = any || ok[j];
+  }
+  if (VEC) {
+    const int row_vecs = a.M / Cd::kPerVec;
+    u32x4* dst = static_cast<u32x4*>(a.out) + static_cast<size_t>(s) * row_vecs;
+    const u32x4* base = static_cast<const u32x4*>(a.expert_out);
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    if (!any) {
+      for (int v = lane; v < row_vecs; v += kWave) st_stream(dst + v, z);
+      return;
+    }
+    int v = lane;
+    for (; v + kWave < row_vecs; v += 2 * kWave) {  // two granules in flight per slot
+      u32x4 xa[K], xb[K];
+#pragma unroll
+      for (int j = 0; j < K; ++j) {
+        xa[j] = ok[j] ? ld_stream(base + row[j] * row_vecs + v) : z;
+        xb[j] = ok[j] ? ld_stream(base + row[j] * row_vecs + v + kWave) : z;
+      }
+      st_stream(dst + v, combine_vec<DT, K>(xa, g));
+      st_stream(dst + v + kWave, combine_vec<DT, K>(xb, g));
+    }
+    for (; v < row_vecs; v += kWave) {
+      u32x4 xa[K];
+#pragma unroll
+      for (int j = 0; j < K; ++j) xa[j] = ok[j] ? ld_stream(base + row[j] * row_vecs + v) : z;
+      st_stream(dst + v, combine_vec<DT, K>(xa, g));
+    }
+  } else {
+    typedef typename Cd::S St;
+    St* dst = static_cast<St*>(a.out) + static_cast<size_t>(s) * a.M;
+    const St* base = static_cast<const St*>(a.expert_out);
+    for (int i = lane; i < a.M; i += kWave) {
+      float acc = ok[0] ? __fmul_rn(g[0], Cd::get(base[row[0] * a.M + i])) : 0.f;
+      if (K == 2) acc = __fadd_rn(acc, ok[1] ? __fmul_rn(g[1], Cd::get(base[row[1] * a.M + i])) : 0.f);
+      dst[i] = Cd::put(acc);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// merge_masks / redispatch.  Both need kept[p][e] = number of tokens of partition p routed to
+// expert e; one counting pass over the masks (the reference re-counts with a tree reduction in
+// each of its E blocks, tutel_moe_dispatch.cu:238-253,377-392).
+// ---------------------------------------------------------------------------------------
+constexpr int kCountPerThread = 4;
+
+__global__ __launch_bounds__(kTile) void count_experts_kernel(PtrTable t, int S, int E, uint32_t* counts) {
+  extern __shared__ uint32_t hist[];
+  const int p = blockIdx.y;
+  const int32_t* idx = static_cast<const int32_t*>(t.p[p]);
+  for (int c = threadIdx.x; c < E; c += kTile) hist[c] = 0;
+  __syncthreads();
+  const int base = blockIdx.x * kTile * kCountPerThread;
+#pragma unroll
+  for (int k = 0; k < kCountPerThread; ++k) {
+    const int i = base + k * kTile + threadIdx.x;
+    if (i < S) {
+      const int e = idx[i];
+      if (e >= 0 && e < E) atomicAdd(&hist[e], 1u);
+    }
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < E; c += kTile)
+    if (hist[c]) atomicAdd(counts + static_cast<size_t>(p) * E + c, hist[c]);
+}
+
+// out[0, p*S+i] = idx, out[1, p*S+i] = loc + sum_{q<p} kept[q][idx]; dropped -> (-1,-1)
+// (tutel_moe_dispatch.cu:214-236).
+__global__ __launch_bounds__(kTile) void merge_masks_kernel(PtrTable t, int P, int S, int E,
+                                                            const uint32_t* counts, int32_t* out) {
+  extern __shared__ uint32_t s_off[];
+  const int p = blockIdx.y;
+  for (int c = threadIdx.x; c < E; c += kTile) {
+    uint32_t off = 0;
+    for (int q = 0; q < p; ++q) off += counts[static_cast<size_t>(q) * E + c];
+    s_off[c] = off;
+  }
+  __syncthreads();
+  const int i = blockIdx.x * kTile + threadIdx.x;
+  if (i >= S) return;
+  const int32_t* il = static_cast<const int32_t*>(t.p[p]);
+  const int e = il[i];
+  const int l = il[S + i];
+  const bool kept = e >= 0 && e < E;
+  const size_t o = static_cast<size_t>(p) * S + i;
+  out[o] = kept ? e : -1;
+  out[static_cast<size_t>(P) * S + o] = kept ? l + static_cast<int>(s_off[e]) : -1;
+}
+
+// out[e, off_p[e] + r, :] = buf_p[e, r, :] for r < kept[p][e]; other rows zero
+// (tutel_moe_dispatch.cu:365-408, which leaves them uninitialised).
+template <typename V>
+__global__ __launch_bounds__(kTile) void redispatch_rows_kernel(PtrTable bufs, int P, int E, int C,
+                                                                int row_vecs, const uint32_t* counts,
+                                                                V* out) {
+  const int w = threadIdx.x / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  const long r = static_cast<long>(blockIdx.x) * kRowsPerBlock + w;
+  if (r >= static_cast<long>(E) * C) return;
+  const int e = static_cast<int>(r / C);
+  const int c = static_cast<int>(r - static_cast<long>(e) * C);
+  const V* src = nullptr;
+  int off = 0;
+  for (int q = 0; q < P; ++q) {
+    const int k = static_cast<int>(counts[static_cast<size_t>(q) * E + e]);
+    if (c < off + k) {
+      src = static_cast<const V*>(bufs.p[q]) + (static_cast<size_t>(e) * C + (c - off)) * row_vecs;
+      break;
+    }
+    off += k;
+  }
+  V* dst = out + static_cast<size_t>(r) * row_vecs;
+  if (src) {
+    int v = lane;
+    for (; v + 3 * kWave < row_vecs; v += 4 * kWave) {
+      const V x0 = ldv(src + v), x1 = ldv(src + v + kWave), x2 = ldv(src + v + 2 * kWave),
+              x3 = ldv(src + v + 3 * kWave);
+      stv(dst + v, x0);
+      stv(dst + v + kWave, x1);
+      stv(dst + v + 2 * kWave, x2);
+      stv(dst + v + 3 * kWave, x3);
+    }
+    for (; v < row_vecs; v += kWave) stv(dst + v, ldv(src + v));
+  } else {
+    const V z = zero_v<V>();
+    for (int v = lane; v < row_vecs; v += kWave) stv(dst + v, z);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------------
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+template <typename V>
+static hipError_t scatter_launch(const void* data, void* out, const int32_t* idx, const int32_t* loc,
+                                 const int32_t* avail_used, const int32_t* rows_lo,
+                                 const int32_t* rows_hi, int S, int E, int C, int K, int row_vecs,
+                                 hipStream_t st) {
+  ScatterArgs<V> a;
+  a.data = static_cast<const V*>(data);
+  a.out = static_cast<V*>(out);
+  a.idx = idx;
+  a.loc = loc;
+  a.avail_used = avail_used;
+  a.rows_lo = rows_lo;
+  a.rows_hi = rows_hi;
+  a.S = S;
+  a.E = E;
+  a.C = C;
+  a.K = K;
+  a.row_vecs = row_vecs;
+  a.token_blocks = (S + kRowsPerBlock - 1) / kRowsPerBlock;
+  a.tail_chunks = rows_hi ? (C + kTailRows - 1) / kTailRows : 0;
+  const long blocks = static_cast<long>(a.token_blocks) + static_cast<long>(a.tail_chunks) * E;
+  if (blocks == 0) return hipSuccess;
+  if (K == 1) scatter_rows_kernel<V, 1><<<static_cast<unsigned>(blocks), kTile, 0, st>>>(a);
+  else scatter_rows_kernel<V, 2><<<static_cast<unsigned>(blocks), kTile, 0, st>>>(a);
+  return hipGetLastError();
+}
+
+hipError_t run_scatter_rows(const void* data, void* out, const int32_t* idx, const int32_t* loc,
+                            const int32_t* avail_used, const int32_t* rows_lo, const int32_t* rows_hi,
+                            int S, int M, int E, int C, int K, int elem_bytes, hipStream_t st) {
+  const size_t row_bytes = static_cast<size_t>(M) * elem_bytes;
+  if (row_bytes == 0) return hipSuccess;
+  if (row_bytes % 16 == 0 && aligned16(data) && aligned16(out))
+    return scatter_launch<u32x4>(data, out, idx, loc, avail_used, rows_lo, rows_hi, S, E, C, K,
+                                 static_cast<int>(row_bytes / 16), st);
+  if (elem_bytes == 4)
+    return scatter_launch<uint32_t>(data, out, idx, loc, avail_used, rows_lo, rows_hi, S, E, C, K, M, st);
+  return scatter_launch<uint16_t>(data, out, idx, loc, avail_used, rows_lo, rows_hi, S, E, C, K, M, st);
+}
+
+hipError_t run_zero_bytes(void* p, size_t nbytes, hipStream_t st) {
+  if (nbytes == 0) return hipSuccess;
+  uint8_t* b = static_cast<uint8_t*>(p);
+  // head bytes up to 16-byte alignment are cleared together with the tail by a second launch
+  const size_t head = (16 - (reinterpret_cast<uintptr_t>(b) & 15u)) & 15u;
+  const size_t h = std::min(head, nbytes);
+  if (h) {
+    zero_bytes_kernel<<<1, 64, 0, st>>>(nullptr, 0, b, h);
+    b += h;
+    nbytes -= h;
+  }
+  const size_t nvec = nbytes / 16;
+  const size_t ntail = nbytes - nvec * 16;
+  if (nvec || ntail) {
+    const int blocks = static_cast<int>(std::min<size_t>((nvec + 255) / 256 + 1, 8192));
+    zero_bytes_kernel<<<blocks, 256, 0, st>>>(reinterpret_cast<u32x4*>(b), nvec, b + nvec * 16, ntail);
+  }
+  return hipGetLastError();
+}
+
+template <int DT>
+static hipError_t decode_launch(const DecodeArgs& a, int K, bool vec, hipStream_t st) {
+  const int blocks = (a.S + kRowsPerBlock - 1) / kRowsPerBlock;
+  if (blocks == 0 || a.M == 0) return hipSuccess;
+  if (K == 1) {
+    if (vec) decode_rows_kernel<DT, 1, true><<<blocks, kTile, 0, st>>>(a);
+    else decode_rows_kernel<DT, 1, false><<<blocks, kTile, 0, st>>>(a);
+  } else {
+    if (vec) decode_rows_kernel<DT, 2, true><<<blocks, kTile, 0, st>>>(a);
+    else decode_rows_kernel<DT, 2, false><<<blocks, kTile, 0, st>>>(a);
+  }
+  return hipGetLastError();
+}
+
+hipError_t run_decode_rows(const void* expert_out, const float* gates, const int32_t* idx,
+                           const int32_t* loc, void* out, int S, int M, int E, int C, int K,
+                           int dtype, hipStream_t st) {
+  DecodeArgs a;
+  a.expert_out = expert_out;
+  a.gates = gates;
+  a.idx = idx;
+  a.loc = loc;
+  a.out = out;
+  a.S = S;
+  a.M = M;
+  a.E = E;
+  a.C = C;
+  const int per_vec = (dtype == LANCET_F32) ? 4 : 8;
+  const bool vec = (M % per_vec == 0) && aligned16(expert_out) && aligned16(out);
+  switch (dtype) {
+    case LANCET_F32: return decode_launch<LANCET_F32>(a, K, vec, st);
+    case LANCET_BF16: return decode_launch<LANCET_BF16>(a, K, vec, st);
+    default: return decode_launch<LANCET_F16>(a, K, vec, st);
+  }
+}
+
+hipError_t run_count_experts(const PtrTable& indlocs, int P, int S, int E, uint32_t* counts, hipStream_t st) {
+  hipError_t err = run_fill_u32(counts, static_cast<size_t>(P) * E, 0u, st);
+  if (err != hipSuccess || S == 0) return err;
+  dim3 grid((S + kTile * kCountPerThread - 1) / (kTile * kCountPerThread), P);
+  count_experts_kernel<<<grid, kTile, E * sizeof(uint32_t), st>>>(indlocs, S, E, counts);
+  return hipGetLastError();
+}
+
+hipError_t run_merge_masks(const PtrTable& indlocs, int P, int S, int E, const uint32_t* counts,
+                           int32_t* out, hipStream_t st) {
+  if (S == 0) return hipSuccess;
+  dim3 grid((S + kTile - 1) / kTile, P);
+  merge_masks_kernel<<<grid, kTile, E * sizeof(uint32_t), st>>>(indlocs, P, S, E, counts, out);
+  return hipGetLastError();
+}
+
+hipError_t run_redispatch_rows(const PtrTable& bufs, int P, int M, int C, int E, const uint32_t* counts,
+                               void* out, int elem_bytes, hipStream_t st) {
+  const size_t row_bytes = static_cast<size_t>(M) * elem_bytes;
+  const long rows = static_cast<long>(E) * C;
+  if (rows == 0 || row_bytes == 0) return hipSuccess;
+  const unsigned blocks = static_cast<unsigned>((rows + kRowsPerBlock - 1) / kRowsPerBlock);
+  bool vec = row_bytes % 16 == 0 && aligned16(out);
+  for (int p = 0; p < P; ++p) vec = vec && aligned16(bufs.p[p]);
+  if (vec)
+    redispatch_rows_kernel<u32x4><<<blocks, kTile, 0, st>>>(bufs, P, E, C, static_cast<int>(row_bytes / 16),
+                                                            counts, static_cast<u32x4*>(out));
+  else if (elem_bytes == 4)
+    redispatch_rows_kernel<uint32_t><<<blocks, kTile, 0, st>>>(bufs, P, E, C, M, counts,
+                                                               static_cast<uint32_t*>(out));
+  else
+    redispatch_rows_kernel<uint16_t><<<blocks, kTile, 0, st>>>(bufs, P, E, C, M, counts,
+                                                               static_cast<uint16_t*>(out));
+  return hipGetLastError();
+}
+
+}  // namespace lancet

@@ -1,0 +1,312 @@
+"""The six RAF operators of the dispatch/optimizer path over torch tensors on the GPU.
+
+Names, positional argument order and defaults follow the reference's schemas
+(scripts/src_codegen/def_schema.py:642-698, 726-742); output tuples follow
+src/op/declare/moe.cc.  Extensions are trailing keyword arguments only (top_k,
+gate_is_logits, workspace, out).  torch supplies device memory and the current
+stream; all computation is done by the HIP kernels behind the C ABI.
+"""
+import ctypes as C
+
+import torch
+
+from . import capi
+
+_DTYPES = {torch.float32: capi.F32, torch.bfloat16: capi.BF16, torch.float16: capi.F16}
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(None)
+
+
+def _dtype_code(t):
+    if t.dtype not in _DTYPES:
+        raise TypeError("token rows must be float32, bfloat16 or float16, got %s" % t.dtype)
+    return _DTYPES[t.dtype]
+
+
+def _need(cond, msg):
+    if not cond:
+        raise ValueError(msg)
+
+
+def _dev(t, name):
+    _need(t.is_cuda, "%s must live on the GPU" % name)
+    _need(t.is_contiguous(), "%s must be contiguous" % name)
+
+
+def _workspace(nbytes, device, given):
+    if given is not None:
+        _need(given.is_cuda and given.dtype == torch.uint8 and given.numel() >= nbytes,
+              "workspace must be a uint8 GPU tensor of at least %d bytes" % nbytes)
+        return given
+    return torch.empty(max(int(nbytes), 4), dtype=torch.uint8, device=device)
+
+
+def moe_capacity(S, E, capacity_factor):
+    """C = int(float(cf) * ceil(S / E)) (src/op/dialect/cuda/moe.cc:107-109)."""
+    return int(capi.load().lancet_moe_capacity(int(S), int(E), float(capacity_factor)))
+
+
+def _check_encode_inputs(data, gate):
+    _dev(data, "data"), _dev(gate, "gate")
+    _need(data.dim() == 2, "Expected input data to be 2D.")
+    _need(gate.dim() == 2, "Expected input gate to be 2D.")
+    _need(data.shape[0] == gate.shape[0], "Input data and gate should have matching shape in dim 0.")
+    _need(gate.dtype == torch.float32, "gate must be float32")
+    return _dtype_code(data)
+
+
+def moe_encode_workspace_bytes(S, E, top_k=1):
+    return int(capi.load().lancet_moe_encode_workspace_bytes(int(S), int(E), int(top_k)))
+
+
+def moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_logits=False,
+               workspace=None, out=None):
+    """raf.op.moe_encode(data, gate, used_capacity, capacity_factor=1.0).
+
+    Returns (gates_s [k*S] f32, indices_locations [2, k*S] i32, used_capacity [E] i32,
+    elements_per_expert [E] u64, dispatched [E, C, M]).  With top_k = 2 the capacity follows
+    GShard: capacity_factor is doubled before the reference formula is applied."""
+    lib = capi.load()
+    dt = _check_encode_inputs(data, gate)
+    S, M = data.shape
+    E = gate.shape[1]
+    _need(top_k in (1, 2), "top_k must be 1 or 2")
+    cf = float(capacity_factor) * (2.0 if top_k == 2 else 1.0)
+    Cap = moe_capacity(S, E, cf)
+    if used_capacity is not None:
+        _dev(used_capacity, "used_capacity")
+        _need(used_capacity.dim() == 1 and used_capacity.numel() == E and used_capacity.dtype == torch.int32,
+              "Input used_capacity should be 1-D int32 of length E.")
+    dev = data.device
+    if out is None:
+        gates_s = torch.empty(top_k * S, dtype=torch.float32, device=dev)
+        indloc = torch.empty((2, top_k * S), dtype=torch.int32, device=dev)
+        used_out = torch.empty(E, dtype=torch.int32, device=dev)
+        elems = torch.empty(E, dtype=torch.int64, device=dev)
+        disp = torch.empty((E, Cap, M), dtype=data.dtype, device=dev)
+    else:
+        gates_s, indloc, used_out, elems, disp = out
+    ws_bytes = moe_encode_workspace_bytes(S, E, top_k)
+    ws = _workspace(ws_bytes, dev, workspace)
+    st = lib.lancet_moe_encode(_p(data), _p(gate), _p(used_capacity), S, M, E, Cap, top_k, dt,
+                               capi.GATE_IS_LOGITS if gate_is_logits else 0, _p(gates_s), _p(indloc),
+                               _p(used_out), _p(elems), _p(disp), _p(ws), ws.numel(), _stream())
+    capi.check(st, "lancet_moe_encode")
+    return gates_s, indloc, used_out, elems.view(torch.uint64) if elems.dtype == torch.int64 else elems, disp
+
+
+def moe_encode_bpr_workspace_bytes(S0, E, n_partitions=1):
+    return int(capi.load().lancet_moe_encode_bpr_workspace_bytes(int(S0), int(E), int(n_partitions)))
+
+
+def moe_encode_batch_prioritized(data, gate, n_partitions=1, partition_id=0, capacity_factor=1.0,
+                                 gate_is_logits=False, workspace=None, out=None):
+    """raf.op.moe_encode_batch_prioritized(data, gate, n_partitions=1, partition_id=0,
+    capacity_factor=1.0): data/gate are the whole batch, the outputs cover partition
+    partition_id (S = S0 / n_partitions tokens)."""
+    lib = capi.load()
+    dt = _check_encode_inputs(data, gate)
+    S0, M = data.shape
+    E = gate.shape[1]
+    _need(n_partitions > 0, "n_partitions should be greater than 0.")
+    _need(0 <= partition_id < n_partitions, "partition_id should be less than n_partitions.")
+    S = S0 // n_partitions
+    Cap = moe_capacity(S, E, capacity_factor)
+    dev = data.device
+    if out is None:
+        gates_s = torch.empty(S, dtype=torch.float32, device=dev)
+        indloc = torch.empty((2, S), dtype=torch.int32, device=dev)
+        used_out = torch.empty(E, dtype=torch.int32, device=dev)
+        elems = torch.empty(E, dtype=torch.int64, device=dev)
+        disp = torch.empty((E, Cap, M), dtype=data.dtype, device=dev)
+    else:
+        gates_s, indloc, used_out, elems, disp = out
+    ws_bytes = moe_encode_bpr_workspace_bytes(S0, E, n_partitions)
+    ws = _workspace(ws_bytes, dev, workspace)
+    st = lib.lancet_moe_encode_bpr(_p(data), _p(gate), S0, M, E, Cap, n_partitions, partition_id, dt,
+                                   capi.GATE_IS_LOGITS if gate_is_logits else 0, _p(gates_s), _p(indloc),
+                                   _p(used_out), _p(elems), _p(disp), _p(ws), ws.numel(), _stream())
+    capi.check(st, "lancet_moe_encode_bpr")
+    return gates_s, indloc, used_out, elems.view(torch.uint64) if elems.dtype == torch.int64 else elems, disp
+
+
+def moe_decode(data, gate, indices_locations, top_k=1, out=None):
+    """raf.op.moe_decode(data [E,C,M], gate [k*S] f32, indices_locations [2, k*S]) -> [S, M]."""
+    lib = capi.load()
+    _dev(data, "data"), _dev(gate, "gate"), _dev(indices_locations, "indices_locations")
+    _need(data.dim() == 3, "Expected input data to be 3D.")
+    _need(gate.dim() == 1, "Expected input gate to be 1D.")
+    _need(gate.dtype == torch.float32, "gate must be float32")
+    _need(indices_locations.dtype == torch.int32 and indices_locations.dim() == 2 and
+          indices_locations.shape[0] == 2 and indices_locations.shape[1] == gate.shape[0],
+          "indices_locations must be int32 [2, k*S]")
+    dt = _dtype_code(data)
+    E, Cap, M = data.shape
+    _need(gate.shape[0] % top_k == 0, "gate length must be a multiple of top_k")
+    S = gate.shape[0] // top_k
+    if out is None:
+        out = torch.empty((S, M), dtype=data.dtype, device=data.device)
+    st = lib.lancet_moe_decode(_p(data), _p(gate), _p(indices_locations), S, M, E, Cap, top_k, dt, _p(out),
+                               _stream())
+    capi.check(st, "lancet_moe_decode")
+    return out
+
+
+def moe_top2_normalize_gates(raw_gates, merged_indices_locations):
+    """Combine weights of the top-2 extension from per-slot raw gate values [2S] and the merged
+    indices_locations [2, 2S]."""
+    lib = capi.load()
+    S = raw_gates.shape[0] // 2
+    out = torch.empty_like(raw_gates)
+    st = lib.lancet_moe_top2_normalize_gates(_p(raw_gates), _p(merged_indices_locations), S, _p(out), _stream())
+    capi.check(st, "lancet_moe_top2_normalize_gates")
+    return out
+
+
+def moe_merge_masks(indices_locations, n_experts, workspace=None, out=None):
+    """raf.op.moe_merge_masks(indices_locations: tuple of [2,S], n_experts) -> [2, P*S]."""
+    lib = capi.load()
+    P = len(indices_locations)
+    _need(P >= 1, "need at least one partition")
+    for il in indices_locations:
+        _dev(il, "indices_locations")
+        _need(il.dim() == 2 and il.shape == indices_locations[0].shape and il.dtype == torch.int32,
+              "Expected input indices_locations to be 2D int32 of equal shape.")
+    S = indices_locations[0].shape[1]
+    dev = indices_locations[0].device
+    if out is None:
+        out = torch.empty((2, P * S), dtype=torch.int32, device=dev)
+    ws_bytes = int(lib.lancet_moe_merge_masks_workspace_bytes(P, n_experts))
+    ws = _workspace(ws_bytes, dev, workspace)
+    ptrs = capi.ptr_array([il.data_ptr() for il in indices_locations])
+    st = lib.lancet_moe_merge_masks(ptrs, P, S, n_experts, _p(out), _p(ws), ws.numel(), _stream())
+    capi.check(st, "lancet_moe_merge_masks")
+    return out
+
+
+def moe_redispatch(data, indices_locations, workspace=None, out=None):
+    """raf.op.moe_redispatch(data: tuple of [E,C,M], indices_locations: tuple of [2,S]) -> [E,C,M]."""
+    lib = capi.load()
+    P = len(indices_locations)
+    _need(P >= 1 and len(data) == P, "data and indices_locations must have one entry per partition")
+    for d in data:
+        _dev(d, "data")
+        _need(d.dim() in (3, 4) and d.shape == data[0].shape and d.dtype == data[0].dtype,
+              "Expected input data to be 3 or 4D of equal shape.")
+    for il in indices_locations:
+        _dev(il, "indices_locations")
+        _need(il.dim() == 2 and il.dtype == torch.int32, "Expected input indices_locations to be 2D.")
+    shape = tuple(data[0].shape)
+    if len(shape) == 4:   # [G, LE, C, M]
+        E, Cap, M = shape[0] * shape[1], shape[2], shape[3]
+    else:
+        E, Cap, M = shape
+    S = indices_locations[0].shape[1]
+    dt = _dtype_code(data[0])
+    dev = data[0].device
+    if out is None:
+        out = torch.empty(shape, dtype=data[0].dtype, device=dev)
+    ws_bytes = int(lib.lancet_moe_redispatch_workspace_bytes(P, E))
+    ws = _workspace(ws_bytes, dev, workspace)
+    dptrs = capi.ptr_array([d.data_ptr() for d in data])
+    iptrs = capi.ptr_array([il.data_ptr() for il in indices_locations])
+    st = lib.lancet_moe_redispatch(dptrs, iptrs, P, S, M, Cap, E, dt, _p(out), _p(ws), ws.numel(), _stream())
+    capi.check(st, "lancet_moe_redispatch")
+    return out
+
+
+# ------------------------------------------------------------------------------------ LANS
+class LansPlan:
+    """Owns the native plan of one parameter set (what the reference's LansImpl constructor
+    captures, src/op/dialect/cuda/lans.cc:28-83)."""
+
+    def __init__(self, numels):
+        lib = capi.load()
+        self.numels = [int(n) for n in numels]
+        arr = (C.c_int64 * len(self.numels))(*self.numels)
+        handle = C.c_void_p()
+        capi.check(lib.lancet_lans_plan_create(arr, len(self.numels), C.byref(handle)), "lancet_lans_plan_create")
+        self._h = handle
+        self._lib = lib
+
+    def close(self):
+        if self._h is not None:
+            self._lib.lancet_lans_plan_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def step(self, g, p, m, v, step, hyper, step_dev=None):
+        T = len(self.numels)
+        _need(len(g) == len(p) == len(m) == len(v) == T, "tensor lists must have one entry per planned tensor")
+        for lst in (g, p, m, v):
+            for t, n in zip(lst, self.numels):
+                _need(t.is_cuda and t.is_contiguous() and t.dtype == torch.float32 and t.numel() == n,
+                      "LANS tensors must be contiguous float32 GPU tensors of the planned sizes")
+        arrs = [capi.ptr_array([t.data_ptr() for t in lst]) for lst in (g, p, m, v)]
+        st = self._lib.lancet_lans_step(self._h, arrs[0], arrs[1], arrs[2], arrs[3], int(step),
+                                        _p(step_dev), C.byref(hyper), _stream())
+        capi.check(st, "lancet_lans_step")
+
+    def norms(self):
+        """[4, T] float32: (||g||, ||p||, ||u_m||, ||u_g||) of the last step."""
+        out = torch.empty((4, len(self.numels)), dtype=torch.float32, device="cuda")
+        capi.check(self._lib.lancet_lans_plan_norms(self._h, _p(out), _stream()), "lancet_lans_plan_norms")
+        return out
+
+
+_PLANS = {}
+
+
+def lans(tensor_list, step, learning_rate, beta1, beta2, eps, bias_correction, weight_decay, grad_averaging,
+         mode, normalize_grad):
+    """raf.op.lans(tensor_list, step, learning_rate, beta1, beta2, eps, bias_correction,
+    weight_decay, grad_averaging, mode, normalize_grad).
+
+    tensor_list = [g.. | p.. | m.. | v..] (python/raf/optim/lans.py:76-103); p, m, v are updated
+    in place and returned (src/op/declare/optimizer.cc:46-62).  `step` is a Python number or a
+    0-dim float32 GPU tensor (the reference passes a tensor; it is read on the device)."""
+    n = len(tensor_list)
+    _need(n % 4 == 0 and n > 0, "tensor_list must hold 4 lists of equal length")
+    T = n // 4
+    g, p, m, v = (list(tensor_list[i * T:(i + 1) * T]) for i in range(4))
+    key = (tuple(t.numel() for t in g), g[0].device.index)
+    plan = _PLANS.get(key)
+    if plan is None:
+        plan = _PLANS[key] = LansPlan(key[0])
+    hyper = capi.LansHyper(float(learning_rate), float(beta1), float(beta2), float(eps), int(bias_correction),
+                           float(weight_decay), int(grad_averaging), int(mode), int(bool(normalize_grad)))
+    if torch.is_tensor(step):
+        _need(step.is_cuda and step.dtype == torch.float32 and step.numel() == 1, "step tensor must be a float32 GPU scalar")
+        plan.step(g, p, m, v, 0, hyper, step_dev=step)
+    else:
+        plan.step(g, p, m, v, int(step), hyper)
+    return tuple(p + m + v)
+
+
+class LansStepper:
+    """Minimal counterpart of raf.optim.lans.LANS (python/raf/optim/lans.py:44-103): owns m, v and
+    the step counter (starting at 1) and feeds [g.., p.., m.., v..] in the reference's order."""
+
+    def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), eps=1e-6, weight_decay=0.01, bias_correction=True,
+                 grad_averaging=True, mode=True, normalize_grad=True):
+        self.params = list(params)
+        self.m = [torch.zeros_like(p) for p in self.params]
+        self.v = [torch.zeros_like(p) for p in self.params]
+        self.hyper = (lr, betas[0], betas[1], eps, int(bias_correction), weight_decay, int(grad_averaging),
+                      int(mode), bool(normalize_grad))
+        self._step = 1
+
+    def step(self, grads):
+        lans(list(grads) + self.params + self.m + self.v, self._step, *self.hyper)
+        self._step += 1

@@ -1,0 +1,128 @@
+"""GPU parity tests of the fused multi-tensor LANS step against the NumPy oracle.
+
+Bar (BASELINE.json): parameters within 1e-6 relative after 10 steps.  Relative is taken per
+tensor against the largest parameter magnitude (an elementwise relative error is undefined
+for parameters that pass through zero); m and v are checked at 1e-5."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import lans_oracle as lo
+from tests.gpu_util import dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+P_RTOL = 1e-6
+
+
+def make_state(seed, shapes):
+    rng = np.random.default_rng(seed)
+    p = [rng.normal(0, 0.02, s).astype(np.float32) for s in shapes]
+    m = [np.zeros(s, np.float32) for s in shapes]
+    v = [np.zeros(s, np.float32) for s in shapes]
+    return rng, p, m, v
+
+
+def assert_close_scaled(got, want, rtol, what):
+    scale = np.abs(want).max()
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64)).max()
+    assert err <= rtol * max(scale, 1e-30), "%s: max err %.3e vs scale %.3e" % (what, err, scale)
+
+
+def run_both(pkg, shapes, steps, seed=0, **hyper):
+    rng, p, m, v = make_state(seed, shapes)
+    dp, dm, dv = [dev(a) for a in p], [dev(a) for a in m], [dev(a) for a in v]
+    args = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-6, bias_correction=1, weight_decay=0.01,
+                grad_averaging=1, mode=1, normalize_grad=True)
+    args.update(hyper)
+    for step in range(1, steps + 1):
+        g = [rng.normal(0, 1e-3, s).astype(np.float32) for s in shapes]
+        dg = [dev(a) for a in g]
+        lo.lans_step(g, p, m, v, step, **args)
+        pkg.ops.lans(dg + dp + dm + dv, step, args["lr"], args["beta1"], args["beta2"], args["eps"],
+                     args["bias_correction"], args["weight_decay"], args["grad_averaging"], args["mode"],
+                     args["normalize_grad"])
+        for a, b in zip(dg, g):   # g is not modified
+            np.testing.assert_array_equal(to_np(a), b)
+    for i in range(len(shapes)):
+        assert_close_scaled(to_np(dp[i]), p[i], P_RTOL, "p[%d]" % i)
+        assert_close_scaled(to_np(dm[i]), m[i], 1e-5, "m[%d]" % i)
+        assert_close_scaled(to_np(dv[i]), v[i], 1e-5, "v[%d]" % i)
+    return dp, dm, dv
+
+
+def test_lans_gpt2_like_list_ten_steps(pkg):
+    # a scaled-down slice of BASELINE config 5: matrices, biases/norms, sizes that are not a
+    # multiple of 4 or of the chunk, a tensor spanning several chunks
+    shapes = [(256, 256), (256, 1024), (1024, 256), (256,), (256,), (1000, 33), (7,), (1,), (16384 * 3 + 5,)]
+    run_both(pkg, shapes, 10)
+
+
+def test_lans_reference_test_shapes(pkg):
+    # tests/python/optim/test_lans.py:140-161 (one 2x2 tensor, 4 steps) and :94-137
+    # (conv 6x3x5x5, bn w/b 6, linear w/b: the >= 3 tensor case)
+    run_both(pkg, [(2, 2)], 4, seed=1)
+    run_both(pkg, [(6, 3, 5, 5), (6,), (6,), (10, 84), (10,)], 2, seed=2)
+
+
+@pytest.mark.parametrize("hyper", [
+    dict(mode=0), dict(weight_decay=0.0), dict(normalize_grad=False), dict(bias_correction=0),
+    dict(grad_averaging=0), dict(mode=0, weight_decay=0.0, normalize_grad=False),
+    dict(lr=5e-2, beta1=0.8, beta2=0.99, eps=1e-8),
+])
+def test_lans_flags(pkg, hyper):
+    run_both(pkg, [(300, 40), (129,), (64, 64)], 5, seed=3, **hyper)
+
+
+def test_lans_zero_norm_special_cases(pkg):
+    """||g|| == 0 (no normalisation, u = wd*p) and ||p|| == 0 (ratio = lr)."""
+    shapes = [(50,), (60,)]
+    p = [np.linspace(-1, 1, 50).astype(np.float32), np.zeros(60, np.float32)]
+    g = [np.zeros(50, np.float32), np.linspace(-1, 1, 60).astype(np.float32)]
+    m = [np.zeros(s, np.float32) for s in shapes]
+    v = [np.zeros(s, np.float32) for s in shapes]
+    dg, dp, dm, dv = ([dev(a) for a in l] for l in (g, p, m, v))
+    lo.lans_step(g, p, m, v, 1)
+    pkg.ops.lans(dg + dp + dm + dv, 1, 1e-3, 0.9, 0.999, 1e-6, 1, 0.01, 1, 1, True)
+    for i in range(2):
+        assert_close_scaled(to_np(dp[i]), p[i], P_RTOL, "p[%d]" % i)
+    np.testing.assert_allclose(to_np(dp[0]), np.linspace(-1, 1, 50) * (1 - 1e-3), rtol=1e-6, atol=1e-9)
+
+
+def test_lans_unaligned_tensors_and_device_step(pkg):
+    """Tensors that start 4 bytes past a 16-byte boundary take the scalar path; the step may be
+    a device scalar (as the reference passes it)."""
+    n = 5000
+    rng = np.random.default_rng(9)
+    host = [rng.normal(0, s, n).astype(np.float32) for s in (1e-3, 0.02)]
+    g, p = host[0].copy(), host[1].copy()
+    m, v = np.zeros(n, np.float32), np.zeros(n, np.float32)
+    store = [torch.zeros(n + 1, device="cuda") for _ in range(4)]
+    views = [s[1:] for s in store]
+    for t, a in zip(views, (g, p, m, v)):
+        t.copy_(torch.from_numpy(a))
+    assert views[0].data_ptr() % 16 == 4
+    step = torch.tensor(3.0, device="cuda")
+    lo.lans_step([g], [p], [m], [v], 3)
+    pkg.ops.lans(views, step, 1e-3, 0.9, 0.999, 1e-6, 1, 0.01, 1, 1, True)
+    assert_close_scaled(to_np(views[1]), p, P_RTOL, "p")
+    assert_close_scaled(to_np(views[2]), m, 1e-5, "m")
+
+
+def test_lans_norms_and_plan_reuse(pkg):
+    shapes = [(64, 64), (100,)]
+    rng, p, m, v = make_state(5, shapes)
+    g = [rng.normal(0, 1e-3, s).astype(np.float32) for s in shapes]
+    plan = pkg.ops.LansPlan([a.size for a in p])
+    hyper = pkg.capi.LansHyper(1e-3, 0.9, 0.999, 1e-6, 1, 0.01, 1, 1, 1)
+    dg, dp, dm, dv = ([dev(a) for a in l] for l in (g, p, m, v))
+    want = lo.lans_step(g, p, m, v, 1)
+    plan.step(dg, dp, dm, dv, 1, hyper)
+    np.testing.assert_allclose(to_np(plan.norms()).T, np.array(want, np.float32), rtol=2e-6)
+    # new gradient tensors (different pointers) on the second step
+    g2 = [rng.normal(0, 1e-3, s).astype(np.float32) for s in shapes]
+    lo.lans_step(g2, p, m, v, 2)
+    plan.step([dev(a) for a in g2], dp, dm, dv, 2, hyper)
+    for i in range(2):
+        assert_close_scaled(to_np(dp[i]), p[i], P_RTOL, "p[%d]" % i)
+    plan.close()

@@ -1,0 +1,316 @@
+"""GPU parity tests of the MoE dispatch path: HIP kernels (through the C ABI) against the
+NumPy oracle on the same seeded inputs.
+
+Bar: expert indices, locations, used capacity, elements_per_expert and scattered rows
+bit-exact; softmax gate values within 1e-5 relative; decode bit-exact in fp32 (the kernel
+rounds exactly like the oracle: fp32 products, fp32 sum, no fused multiply-add) and within
+1 bf16/fp16 ulp for 16-bit rows.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as mo
+from tests.gpu_util import dev, make_inputs, rows_as_oracle, rows_to_torch, to_np
+
+pytestmark = pytest.mark.gpu
+
+GATE_RTOL = 1e-5
+
+
+def check_encode(got, want, gate_exact):
+    g, il, used, elems, disp = got
+    wg, wil, wused, welems, wdisp = want
+    np.testing.assert_array_equal(to_np(il), wil)
+    np.testing.assert_array_equal(to_np(used), wused)
+    np.testing.assert_array_equal(to_np(elems), welems)
+    if gate_exact:
+        np.testing.assert_array_equal(to_np(g), wg)
+    else:
+        np.testing.assert_allclose(to_np(g), wg, rtol=GATE_RTOL, atol=0)
+    np.testing.assert_array_equal(to_np(disp), wdisp)
+
+
+# ----------------------------------------------------------------------------- moe_encode, top-1
+@pytest.mark.parametrize("S,M,E,cf", [
+    (1024, 128, 32, 1.0), (2048, 128, 64, 1.0),      # reference test shapes (test_cuda_moe.py:88-91)
+    (4096, 768, 8, 1.25),                             # BASELINE config 1
+    (1000, 36, 7, 0.5), (255, 8, 3, 1.0), (257, 12, 5, 2.0), (1, 4, 2, 1.0), (64, 4, 1, 1.0),
+    (3000, 16, 128, 1.5), (777, 20, 200, 3.0),
+])
+@pytest.mark.parametrize("is_logits", [False, True])
+def test_encode_top1(pkg, S, M, E, cf, is_logits):
+    data, logits = make_inputs(S * 7 + E, S, M, E)
+    gate = logits if is_logits else mo.softmax_rows(logits)
+    used0 = np.zeros(E, np.int32)
+    want = mo.moe_encode(data, gate, used0, cf, gate_is_logits=is_logits, fast_scatter=True)
+    got = pkg.ops.moe_encode(dev(data), dev(gate), dev(used0), cf, gate_is_logits=is_logits)
+    check_encode(got, want, gate_exact=not is_logits)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+def test_encode_top1_16bit_rows(pkg, dt):
+    S, M, E = 1500, 96, 16
+    data, logits = make_inputs(3, S, M, E)
+    gate = mo.softmax_rows(logits)
+    used0 = np.zeros(E, np.int32)
+    want = mo.moe_encode(rows_as_oracle(data, dt), gate, used0, 1.0, fast_scatter=True)
+    got = pkg.ops.moe_encode(rows_to_torch(data, dt), dev(gate), dev(used0), 1.0)
+    check_encode(got, want, gate_exact=True)
+
+
+def test_encode_rows_not_16_byte_multiple(pkg):
+    """M*4 = 20 bytes and M*2 = 10 bytes per row take the element-granular path."""
+    S, M, E = 600, 5, 6
+    data, logits = make_inputs(4, S, M, E)
+    gate = mo.softmax_rows(logits)
+    used0 = np.zeros(E, np.int32)
+    for dt in ("f32", "bf16"):
+        want = mo.moe_encode(rows_as_oracle(data, dt), gate, used0, 1.0, fast_scatter=True)
+        got = pkg.ops.moe_encode(rows_to_torch(data, dt), dev(gate), dev(used0), 1.0)
+        check_encode(got, want, gate_exact=True)
+
+
+def test_encode_edge_routing(pkg):
+    S, M, E = 900, 8, 8
+    data, logits = make_inputs(5, S, M, E, ties=True)
+    # ties, an expert nobody chooses, an expert that is full on entry, one that overflows
+    logits[:, 3] = -50.0
+    logits[::3, 1] = 40.0
+    C = mo.capacity(S, E, 1.0)
+    used_in = np.array([0, 5, C, 0, C // 2, 1, C - 1, C], np.int32)
+    want = mo.moe_encode(data, logits, used_in, 1.0, fast_scatter=True)
+    got = pkg.ops.moe_encode(dev(data), dev(logits), dev(used_in), 1.0)
+    check_encode(got, want, gate_exact=True)
+    # capacity 0: everything dropped, empty buffer
+    want = mo.moe_encode(data, logits, np.zeros(E, np.int32), 0.0, fast_scatter=True)
+    got = pkg.ops.moe_encode(dev(data), dev(logits), dev(np.zeros(E, np.int32)), 0.0)
+    assert got[4].shape == (E, 0, M)
+    check_encode(got, want, gate_exact=True)
+    # all tokens to one expert
+    logits[:, 2] = 99.0
+    want = mo.moe_encode(data, logits, np.zeros(E, np.int32), 1.0, fast_scatter=True)
+    got = pkg.ops.moe_encode(dev(data), dev(logits), None, 1.0)
+    check_encode(got, want, gate_exact=True)
+
+
+def test_encode_empty_batch(pkg):
+    E, M = 4, 8
+    got = pkg.ops.moe_encode(torch.empty((0, M), device="cuda"), torch.empty((0, E), device="cuda"),
+                             dev(np.array([1, 0, 2, 0], np.int32)), 1.0)
+    assert got[0].numel() == 0 and got[1].shape == (2, 0) and got[4].shape == (E, 0, M)
+    np.testing.assert_array_equal(to_np(got[2]), [0, 0, 0, 0])   # min(used_in + 0, C = 0)
+
+
+# ----------------------------------------------------------------------------- chained partitions
+@pytest.mark.parametrize("P,E,S0,M", [(2, 2, 1024, 512), (4, 2, 1024, 512), (4, 16, 2048, 64), (3, 5, 999, 8)])
+def test_partitioned_encode_merge_redispatch(pkg, P, E, S0, M):
+    """tests/python/op/cuda/test_cuda_moe.py:384-471: partitioned == un-partitioned."""
+    ops = pkg.ops
+    data, logits = make_inputs(17 + P, S0, M, E)
+    gate = mo.softmax_rows(logits)
+    S = S0 // P
+    d_data, d_gate = dev(data), dev(gate)
+    used = dev(np.zeros(E, np.int32))
+    ils, bufs, gs, o_ils, o_bufs = [], [], [], [], []
+    o_used = np.zeros(E, np.int32)
+    for p in range(P):
+        sl = slice(p * S, (p + 1) * S)
+        g, il, used, elems, disp = ops.moe_encode(d_data[sl].contiguous(), d_gate[sl].contiguous(), used, float(P))
+        og, oil, o_used, oelems, odisp = mo.moe_encode(data[sl], gate[sl], o_used, float(P), fast_scatter=True)
+        check_encode((g, il, used, elems, disp), (og, oil, o_used, oelems, odisp), gate_exact=True)
+        ils.append(il), bufs.append(disp), gs.append(g), o_ils.append(oil), o_bufs.append(odisp)
+    merged = ops.moe_merge_masks(ils, E)
+    red = ops.moe_redispatch(bufs, ils)
+    np.testing.assert_array_equal(to_np(merged), mo.moe_merge_masks(o_ils, E))
+    np.testing.assert_array_equal(to_np(red), mo.moe_redispatch(o_bufs, o_ils))
+    if S * P == S0:
+        # against the un-partitioned op (same capacity: cf*P per partition == cf on the whole batch
+        # whenever ceil(S/E)*P == ceil(S0/E))
+        ref = mo.moe_encode(data, gate, np.zeros(E, np.int32), 1.0, fast_scatter=True)
+        if ref[4].shape == tuple(red.shape):
+            ril = ref[1].copy()
+            ril[1, ril[0] < 0] = -1
+            np.testing.assert_array_equal(to_np(merged), ril)
+            np.testing.assert_array_equal(to_np(red), ref[4])
+
+
+# ----------------------------------------------------------------------------- top-2 extension
+@pytest.mark.parametrize("S,M,E,cf,dt", [(2048, 64, 16, 1.0, "f32"), (2048, 64, 16, 1.0, "bf16"),
+                                         (1111, 24, 5, 0.6, "f32"), (4096, 32, 32, 1.25, "bf16"),
+                                         (300, 8, 2, 1.0, "f32")])
+def test_encode_top2(pkg, S, M, E, cf, dt):
+    data, logits = make_inputs(S + E, S, M, E, zipf_bias=True)
+    used0 = np.zeros(E, np.int32)
+    want = mo.moe_encode_top2(rows_as_oracle(data, dt), logits, used0, cf, gate_is_logits=True, fast_scatter=True)
+    got = pkg.ops.moe_encode(rows_to_torch(data, dt), dev(logits), dev(used0), cf, top_k=2, gate_is_logits=True)
+    check_encode(got, want, gate_exact=False)
+    assert (want[1][0] < 0).any(), "config must drop tokens"
+
+
+def test_top2_equals_two_chained_top1_encodes(pkg):
+    """The identity that defines the extension: top-2 == encode(choice 1) -> encode(choice 2,
+    used = out 1) -> merge_masks -> redispatch with the reference's top-1 semantics."""
+    ops = pkg.ops
+    S, M, E, cf = 1536, 32, 8, 0.75
+    data, logits = make_inputs(99, S, M, E, zipf_bias=True)
+    probs = mo.softmax_rows(logits)
+    sel, val = mo.select_topk(logits, 2, True)
+    # gate arrays whose argmax is the k-th choice and whose max is that choice's probability
+    gates = []
+    for j in range(2):
+        g = np.full((S, E), -1.0, np.float32)
+        g[np.arange(S), sel[j]] = val[j]
+        gates.append(g)
+    d_data = dev(data)
+    used = dev(np.zeros(E, np.int32))
+    ils, bufs, raw = [], [], []
+    for j in range(2):
+        g, il, used, elems, disp = ops.moe_encode(d_data, dev(gates[j]), used, 2 * cf)
+        ils.append(il), bufs.append(disp), raw.append(g)
+    merged = ops.moe_merge_masks(ils, E)
+    red = ops.moe_redispatch(bufs, ils)
+    weights = ops.moe_top2_normalize_gates(torch.cat(raw), merged)
+    fused = ops.moe_encode(d_data, dev(logits), dev(np.zeros(E, np.int32)), cf, top_k=2, gate_is_logits=True)
+    np.testing.assert_array_equal(to_np(merged), to_np(fused[1]))
+    np.testing.assert_array_equal(to_np(red), to_np(fused[4]))
+    np.testing.assert_array_equal(to_np(used), to_np(fused[2]))
+    np.testing.assert_allclose(to_np(weights), to_np(fused[0]), rtol=GATE_RTOL)
+    del probs
+
+
+# ----------------------------------------------------------------------------- batch prioritised
+@pytest.mark.parametrize("S0,M,E,P,cf,ties", [
+    (1024, 128, 32, 1, 1.0, False), (2048, 128, 64, 1, 1.0, False),   # test_cuda_moe.py:160-163
+    (1024, 512, 16, 4, 4.0, False),                                    # test_cuda_moe.py:1316
+    (2000, 16, 8, 1, 0.5, True), (1536, 8, 6, 3, 1.5, True), (4096, 8, 64, 4, 2.0, False),
+    (700, 4, 3, 1, 5.0, False),                                        # nothing dropped
+])
+def test_encode_bpr(pkg, S0, M, E, P, cf, ties):
+    data, logits = make_inputs(S0 + P, S0, M, E, logit_scale=2.0, ties=ties)
+    gate = mo.softmax_rows(logits)
+    if ties:
+        gate = (np.round(gate * 16) / 16).astype(np.float32)   # many equal priorities
+    d_data, d_gate = dev(data), dev(gate)
+    for pid in range(P):
+        want = mo.moe_encode_bpr(data, gate, P, pid, cf, fast_scatter=True)
+        got = pkg.ops.moe_encode_batch_prioritized(d_data, d_gate, P, pid, cf)
+        check_encode(got, want, gate_exact=True)
+
+
+def test_encode_bpr_on_logits_resorts_emitted_priorities(pkg):
+    """With logits the priorities are softmax values computed on the device; exp() is not
+    bit-portable, so the oracle re-sorts the priorities the device emitted (checked at 1e-5)."""
+    S0, M, E = 4096, 16, 16
+    data, logits = make_inputs(7, S0, M, E, logit_scale=2.0)
+    got = pkg.ops.moe_encode_batch_prioritized(dev(data), dev(logits), 1, 0, 0.5, gate_is_logits=True)
+    prio = to_np(got[0])
+    want = mo.moe_encode_bpr(data, logits, 1, 0, 0.5, gate_is_logits=True, priorities=prio, fast_scatter=True)
+    np.testing.assert_allclose(prio, want[0], rtol=GATE_RTOL)
+    np.testing.assert_array_equal(to_np(got[1]), want[1])
+    np.testing.assert_array_equal(to_np(got[2]), want[2])
+    np.testing.assert_array_equal(to_np(got[4]), want[4])
+
+
+# ----------------------------------------------------------------------------- decode
+@pytest.mark.parametrize("dt", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("k", [1, 2])
+@pytest.mark.parametrize("S,M,E", [(1024, 128, 32), (777, 40, 6), (300, 5, 4)])
+def test_decode(pkg, dt, k, S, M, E):
+    ops = pkg.ops
+    data, logits = make_inputs(S + k, S, M, E, zipf_bias=True)
+    rows = rows_as_oracle(data, dt)
+    used0 = np.zeros(E, np.int32)
+    if k == 1:
+        g, il, _, _, disp = mo.moe_encode(rows, mo.softmax_rows(logits), used0, 0.8, fast_scatter=True)
+    else:
+        g, il, _, _, disp = mo.moe_encode_top2(rows, logits, used0, 0.8, gate_is_logits=True, fast_scatter=True)
+    # an "expert" that is not the identity, so that the two slots carry different rows
+    expert_out = rows_as_oracle((disp * np.float32(1.5) + np.float32(0.25)).astype(np.float32), dt)
+    want32 = mo.moe_decode(expert_out, g, il, k=k)
+    got = ops.moe_decode(rows_to_torch(expert_out, dt), dev(g), dev(il), top_k=k)
+    if dt == "f32":
+        np.testing.assert_array_equal(to_np(got), want32)
+    else:
+        tdt = torch.bfloat16 if dt == "bf16" else torch.float16
+        want = torch.from_numpy(want32).to(tdt)
+        # same fp32 value rounded once on both sides: identical bits expected; the documented
+        # tolerance is 1 ulp of the storage type
+        a = got.cpu().view(torch.int16).to(torch.int32)
+        b = want.view(torch.int16).to(torch.int32)
+        assert int((a - b).abs().max()) <= 1
+    dropped = (il[0, :S] < 0) if k == 1 else ((il[0, :S] < 0) & (il[0, S:] < 0))
+    assert dropped.any() and not to_np(got)[dropped].any()
+
+
+def test_decode_roundtrip_identity_expert(pkg):
+    """decode(encode(x), gate = 1) == x on kept tokens, 0 on dropped ones (bit-exact)."""
+    ops = pkg.ops
+    S, M, E = 2048, 128, 32
+    data, logits = make_inputs(123, S, M, E)
+    d_data = dev(data)
+    g, il, used, elems, disp = ops.moe_encode(d_data, dev(mo.softmax_rows(logits)), None, 0.9)
+    out = ops.moe_decode(disp, torch.ones_like(g), il)
+    kept = (il[0] >= 0)
+    assert torch.equal(out[kept], d_data[kept]) and not out[~kept].any() and (~kept).any()
+
+
+# ----------------------------------------------------------------------------- launcher level
+def test_launch_gen_location_and_encode_forward(pkg):
+    import ctypes as C
+    lib = pkg.capi.load()
+    S, M, E, cf = 3000, 16, 12, 0.7
+    data, logits = make_inputs(31, S, M, E)
+    Cap = mo.capacity(S, E, cf)
+    idx0 = np.argmax(logits, axis=1).astype(np.int32)
+    used_in = np.array([0, 3] * (E // 2), np.int32)
+    widx, wloc, wused, welems = mo.gen_location(idx0, used_in, Cap, M, E)
+    d_idx, d_used = dev(idx0), dev(used_in)
+    d_loc = torch.empty(S, dtype=torch.int32, device="cuda")
+    d_uo = torch.empty(E, dtype=torch.int32, device="cuda")
+    d_el = torch.empty(E, dtype=torch.int64, device="cuda")
+    nws = lib.lancet_gen_location_workspace_bytes(S, E)
+    ws = torch.empty(nws, dtype=torch.uint8, device="cuda")
+    p = lambda t: C.c_void_p(t.data_ptr())
+    st = lib.lancet_launch_gen_location(p(d_idx), p(d_used), p(d_loc), p(d_uo), p(d_el), Cap, S, E, M, p(ws), nws, None)
+    assert st == 0
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(to_np(d_idx), widx)
+    np.testing.assert_array_equal(to_np(d_loc), wloc)
+    np.testing.assert_array_equal(to_np(d_uo), wused)
+    np.testing.assert_array_equal(to_np(d_el).astype(np.uint64), welems)
+    # scatter with and without the used-capacity test
+    d_data = dev(data)
+    for capused in (d_used, None):
+        out = torch.full((E, Cap, M), 7.0, device="cuda")
+        st = lib.lancet_launch_encode_forward(p(d_idx), p(d_loc), p(capused) if capused is not None else None,
+                                              p(d_data), p(out), S, M, Cap, E, pkg.capi.F32, None)
+        assert st == 0
+        torch.cuda.synchronize()
+        avail = (Cap - used_in) if capused is not None else None
+        np.testing.assert_array_equal(to_np(out), mo.scatter_rows(data, widx, wloc, E, Cap, avail))
+
+
+def test_bounded_wait_flags_the_workspace(pkg):
+    """A spin limit of 1 makes look-back waits give up at once: the kernel must still finish and
+    flag the workspace; the default limit must leave the flag clear."""
+    import ctypes as C
+    lib = pkg.capi.load()
+    S, M, E = 65536, 4, 8
+    data, logits = make_inputs(1, S, M, E)
+    d_data, d_gate = dev(data), dev(logits)
+    ws = torch.empty(pkg.ops.moe_encode_workspace_bytes(S, E, 1), dtype=torch.uint8, device="cuda")
+    err = C.c_int(-1)
+    pkg.ops.moe_encode(d_data, d_gate, None, 1.0, workspace=ws)
+    assert lib.lancet_scan_workspace_error(C.c_void_p(ws.data_ptr()), None, C.byref(err)) == 0 and err.value == 0
+    lib.lancet_debug_set_spin_limit(1)
+    try:
+        pkg.ops.moe_encode(d_data, d_gate, None, 1.0, workspace=ws)
+        torch.cuda.synchronize()   # terminates
+        assert lib.lancet_scan_workspace_error(C.c_void_p(ws.data_ptr()), None, C.byref(err)) == 0
+        assert err.value in (0, 1)   # 1 whenever a predecessor was not ready at the first poll
+    finally:
+        lib.lancet_debug_set_spin_limit(0)
+    want = mo.moe_encode(data, logits, np.zeros(E, np.int32), 1.0, fast_scatter=True)
+    got = pkg.ops.moe_encode(d_data, d_gate, None, 1.0, workspace=ws)
+    np.testing.assert_array_equal(to_np(got[1]), want[1])

@@ -14,32 +14,58 @@ namespace lancet {
 // src/op/dialect/cuda/moe.cc:177-250 (three passes over [S,E] plus an [S,E] workspace).
 // ---------------------------------------------------------------------------------------
 template <int K>
+__device__ __forceinline__ void consider(float x, int j, float& v1, int& i1, float& v2, int& i2) {
+  if (i1 < 0 || x > v1) {
+    v2 = v1;
+    i2 = i1;
+    v1 = x;
+    i1 = j;
+  } else if (K == 2 && (i2 < 0 || x > v2)) {
+    v2 = x;
+    i2 = j;
+  }
+}
+
+template <int K>
 __device__ __forceinline__ void route_token(const float* __restrict__ row, int E, bool is_logits,
                                             int (&e)[K], float (&p)[K]) {
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
   float v1 = 0.f, v2 = 0.f;
   int i1 = -1, i2 = -1;
-  for (int j = 0; j < E; ++j) {
-    const float x = row[j];
-    if (i1 < 0 || x > v1) {
-      v2 = v1;
-      i2 = i1;
-      v1 = x;
-      i1 = j;
-    } else if (K == 2 && (i2 < 0 || x > v2)) {
-      v2 = x;
-      i2 = j;
+  const bool vec = ((E & 3) == 0) && ((reinterpret_cast<uintptr_t>(row) & 15u) == 0);
+  if (vec) {
+    const f32x4* r4 = reinterpret_cast<const f32x4*>(row);
+    for (int j = 0; j < E / 4; ++j) {
+      const f32x4 x = r4[j];
+      consider<K>(x.x, 4 * j, v1, i1, v2, i2);
+      consider<K>(x.y, 4 * j + 1, v1, i1, v2, i2);
+      consider<K>(x.z, 4 * j + 2, v1, i1, v2, i2);
+      consider<K>(x.w, 4 * j + 3, v1, i1, v2, i2);
+    }
+  } else {
+    for (int j = 0; j < E; ++j) consider<K>(row[j], j, v1, i1, v2, i2);
+  }
+  float sum = 1.f;
+  if (is_logits) {
+    sum = 0.f;  // sequential sum in expert order
+    if (vec) {
+      const f32x4* r4 = reinterpret_cast<const f32x4*>(row);
+      for (int j = 0; j < E / 4; ++j) {
+        const f32x4 x = r4[j];
+        sum += expf(x.x - v1);
+        sum += expf(x.y - v1);
+        sum += expf(x.z - v1);
+        sum += expf(x.w - v1);
+      }
+    } else {
+      for (int j = 0; j < E; ++j) sum += expf(row[j] - v1);
     }
   }
-  float inv = 1.f, sum = 0.f;
-  if (is_logits) {
-    for (int j = 0; j < E; ++j) sum += expf(row[j] - v1);
-    inv = sum;
-  }
   e[0] = i1;
-  p[0] = is_logits ? expf(v1 - v1) / inv : v1;
+  p[0] = is_logits ? expf(v1 - v1) / sum : v1;
   if (K == 2) {
     e[1] = i2;
-    p[1] = is_logits ? expf(v2 - v1) / inv : v2;
+    p[1] = is_logits ? expf(v2 - v1) / sum : v2;
   }
 }
 
@@ -137,14 +163,15 @@ __global__ __launch_bounds__(kTile) void route_scan_kernel(RouteArgs a) {
 // taken after the drop and normalised (docker/resources/sharded_moe.py:282-312).
 __global__ __launch_bounds__(kTile) void finalize_top2_kernel(RouteArgs a) {
   const int s = blockIdx.x * kTile + threadIdx.x;
-  const uint32_t* tot = a.ws.incl + static_cast<size_t>(a.ntiles - 1) * 2 * a.E;  // [2][E]
+  // totals of both slots = the last tile's inclusive descriptors, [2][E]
+  const uint32_t* tot = a.ws.desc + static_cast<size_t>(a.ntiles - 1) * 2 * a.E;
   if (s < a.S) {
     const int e1 = a.idx_out[s], e2 = a.idx_out[a.S + s];
     const int r1 = a.loc_out[s], r2 = a.loc_out[a.S + s];
     const int u1 = a.used_in ? a.used_in[e1] : 0;
     const int u2 = a.used_in ? a.used_in[e2] : 0;
     const bool keep1 = r1 < a.C - u1;
-    const int64_t after1 = min(static_cast<int64_t>(u2) + ld_agent(tot + e2), static_cast<int64_t>(a.C));
+    const int64_t after1 = min(static_cast<int64_t>(u2) + (ld_agent(tot + e2) & kDescCountMask), static_cast<int64_t>(a.C));
     const bool keep2 = r2 < a.C - after1;
     a.idx_out[s] = keep1 ? e1 : -1;
     a.loc_out[s] = keep1 ? r1 : -1;
@@ -159,7 +186,7 @@ __global__ __launch_bounds__(kTile) void finalize_top2_kernel(RouteArgs a) {
   if (blockIdx.x == 0) {
     for (int c = threadIdx.x; c < a.E; c += kTile) {
       const int64_t used = a.used_in ? a.used_in[c] : 0;
-      const int64_t total = static_cast<int64_t>(ld_agent(tot + c)) + ld_agent(tot + a.E + c);
+      const int64_t total = static_cast<int64_t>(ld_agent(tot + c) & kDescCountMask) + (ld_agent(tot + a.E + c) & kDescCountMask);
       const int64_t uo = min(used + total, static_cast<int64_t>(a.C));
       a.used_out[c] = static_cast<int32_t>(uo);
       a.elems_out[c] = static_cast<uint64_t>((uo - used) * a.M);
@@ -426,8 +453,8 @@ hipError_t run_route_scan(const float* gate, const int32_t* idx_in, const int32_
   a.ntiles = static_cast<int>(scan_num_tiles(S));
   a.is_logits = is_logits;
   a.spin_limit = current_spin_limit();
-  a.ws = scan_ws_view(ws, a.ntiles, K * E);
-  hipError_t err = run_fill_u32(static_cast<uint32_t*>(ws), kScanHeaderWords + a.ntiles, 0u, st);
+  a.ws = scan_ws_view(ws);
+  hipError_t err = run_fill_u32(static_cast<uint32_t*>(ws), scan_ws_words(a.ntiles, K * E), 0u, st);
   if (err != hipSuccess) return err;
   const size_t lds = scan_lds_bytes(K * E);
   if (K == 1) {
@@ -454,7 +481,7 @@ hipError_t run_bpr_route(const float* gate, int S0, int E, int C, int M, int n_p
   a.M = M;
   a.part_lo = partition_id * S;
   a.ntiles = static_cast<int>(scan_num_tiles(S));
-  a.ws = scan_ws_view(ws, a.ntiles, 2 * E);
+  a.ws = scan_ws_view(ws);
   uint32_t* extra = static_cast<uint32_t*>(ws) + scan_ws_words(a.ntiles, 2 * E);
   int32_t* idx0 = reinterpret_cast<int32_t*>(extra);
   float* prio = reinterpret_cast<float*>(extra + S0);
@@ -469,7 +496,7 @@ hipError_t run_bpr_route(const float* gate, int S0, int E, int C, int M, int n_p
   a.used_out = used_out;
   a.elems_out = elems_out;
   a.spin_limit = current_spin_limit();
-  hipError_t err = run_fill_u32(static_cast<uint32_t*>(ws), kScanHeaderWords + a.ntiles, 0u, st);
+  hipError_t err = run_fill_u32(static_cast<uint32_t*>(ws), scan_ws_words(a.ntiles, 2 * E), 0u, st);
   if (err != hipSuccess) return err;
   err = run_gate_topk(gate, S0, E, 1, is_logits, idx0, prio, st);
   if (err != hipSuccess) return err;

@@ -134,22 +134,34 @@ struct Codec<LANCET_F16> {
   static __device__ __forceinline__ S put(float f) { return static_cast<S>(f32_to_f16(f)); }
 };
 
+// One IEEE multiply / add each, never contracted into a fused multiply-add (the operators of
+// the HIP headers' __fmul_rn/__fadd_rn carry the translation unit's contraction setting).
+__device__ __forceinline__ float mul_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a * b;
+}
+__device__ __forceinline__ float add_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a + b;
+}
+
 template <int DT, int K>
 __device__ __forceinline__ u32x4 combine_vec(const u32x4 (&x)[K], const float (&g)[K]) {
+#pragma clang fp contract(off)
   typedef Codec<DT> Cd;
   u32x4 r;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     if (Cd::kPerVec == 4) {
-      float acc = __fmul_rn(g[0], Cd::get(x[0][i]));
-      if (K == 2) acc = __fadd_rn(acc, __fmul_rn(g[1], Cd::get(x[1][i])));
+      float acc = mul_rn(g[0], Cd::get(x[0][i]));
+      if (K == 2) acc = add_rn(acc, mul_rn(g[1], Cd::get(x[1][i])));
       r[i] = Cd::put(acc);
     } else {
-      float lo = __fmul_rn(g[0], Cd::get(static_cast<typename Cd::S>(x[0][i] & 0xffffu)));
-      float hi = __fmul_rn(g[0], Cd::get(static_cast<typename Cd::S>(x[0][i] >> 16)));
+      float lo = mul_rn(g[0], Cd::get(static_cast<typename Cd::S>(x[0][i] & 0xffffu)));
+      float hi = mul_rn(g[0], Cd::get(static_cast<typename Cd::S>(x[0][i] >> 16)));
       if (K == 2) {
-        lo = __fadd_rn(lo, __fmul_rn(g[1], Cd::get(static_cast<typename Cd::S>(x[1][i] & 0xffffu))));
-        hi = __fadd_rn(hi, __fmul_rn(g[1], Cd::get(static_cast<typename Cd::S>(x[1][i] >> 16))));
+        lo = add_rn(lo, mul_rn(g[1], Cd::get(static_cast<typename Cd::S>(x[1][i] & 0xffffu))));
+        hi = add_rn(hi, mul_rn(g[1], Cd::get(static_cast<typename Cd::S>(x[1][i] >> 16))));
       }
       r[i] = static_cast<uint32_t>(Cd::put(lo)) | (static_cast<uint32_t>(Cd::put(hi)) << 16);
     }
@@ -217,8 +229,9 @@ __global__ __launch_bounds__(kTile) void decode_rows_kernel(DecodeArgs a) {
     St* dst = static_cast<St*>(a.out) + static_cast<size_t>(s) * a.M;
     const St* base = static_cast<const St*>(a.expert_out);
     for (int i = lane; i < a.M; i += kWave) {
-      float acc = ok[0] ? __fmul_rn(g[0], Cd::get(base[row[0] * a.M + i])) : 0.f;
-      if (K == 2) acc = __fadd_rn(acc, ok[1] ? __fmul_rn(g[1], Cd::get(base[row[1] * a.M + i])) : 0.f);
+#pragma clang fp contract(off)
+      float acc = ok[0] ? mul_rn(g[0], Cd::get(base[row[0] * a.M + i])) : 0.f;
+      if (K == 2) acc = add_rn(acc, ok[1] ? mul_rn(g[1], Cd::get(base[row[1] * a.M + i])) : 0.f);
       dst[i] = Cd::put(acc);
     }
   }

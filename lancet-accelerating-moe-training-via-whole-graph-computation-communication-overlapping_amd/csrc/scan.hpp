@@ -3,13 +3,17 @@
 //   1. wave level  - match lanes with the same expert by ballots over the bits of the expert
 //                    id; rank inside the wave = popcount of the peer mask below the lane;
 //   2. tile level  - per-wave counts in LDS, exclusive scan over the waves of the tile;
-//   3. across tiles - decoupled look-back over a [tiles][counters] descriptor table: a tile
-//                    publishes its aggregate, then sums the aggregates of its predecessors
-//                    (in parallel over predecessors and counters) back to the nearest tile
-//                    that has already published an inclusive prefix.
+//   3. across tiles - decoupled look-back over a [tiles][counters] descriptor table.  Every
+//                    descriptor is ONE 32-bit word: 2 status bits (1 = the tile's own count,
+//                    2 = inclusive prefix over all tiles up to it) above a 30-bit count, so a
+//                    word is self-validating and no fence separates "data" from "flag".  A
+//                    tile publishes its counts, then reads the words of its predecessors, a
+//                    window of rows at a time, all (row, counter) pairs in parallel, and stops
+//                    per counter at the nearest row that already holds an inclusive prefix.
 // Tiles are numbered by an atomic ticket, so a tile only ever waits for tiles that are
-// already running.  All cross-workgroup traffic uses agent-scope atomics and fences: the
-// eight XCDs of the chip have private L2 caches.
+// already running, and it only waits for their own counts, never for their prefixes: the
+// look-back is one round of parallel loads, not a serial chain.  Descriptor words are read
+// and written with agent-scope atomics (the eight XCDs of the chip have private L2 caches).
 //
 // Replaces the per-expert serial Blelloch scan of the reference
 // (src/op/dialect/cuda/kernels/tutel_moe_dispatch.cu:164-212: grid = E blocks, each
@@ -23,35 +27,39 @@ namespace lancet {
 struct ScanWs {
   uint32_t* ticket;  // [1]  next tile number
   uint32_t* error;   // [1]  set to 1 when a bounded wait gave up
-  uint32_t* status;  // [T]  0 = nothing, 1 = aggregate published, 2 = inclusive prefix published
-  uint32_t* agg;     // [T][NC] per-tile counts
-  uint32_t* incl;    // [T][NC] inclusive prefix over tiles
+  uint32_t* desc;    // [T][NC] descriptor words, zero before the launch
 };
 
-constexpr uint32_t kScanHeaderWords = 2;  // ticket, error (zeroed together with status)
+constexpr uint32_t kScanHeaderWords = 2;  // ticket, error
+constexpr uint32_t kDescCountMask = 0x3fffffffu;
+constexpr uint32_t kDescAggregate = 1u << 30;
+constexpr uint32_t kDescInclusive = 2u << 30;
 
+// words that must be zero when the kernel starts
 __host__ __device__ inline size_t scan_ws_words(int64_t ntiles, int64_t ncounters) {
-  return kScanHeaderWords + static_cast<size_t>(ntiles) * (1 + 2 * static_cast<size_t>(ncounters));
+  return kScanHeaderWords + static_cast<size_t>(ntiles) * static_cast<size_t>(ncounters);
 }
 
-inline ScanWs scan_ws_view(void* base, int64_t ntiles, int64_t ncounters) {
+inline ScanWs scan_ws_view(void* base) {
   uint32_t* w = static_cast<uint32_t*>(base);
   ScanWs ws;
   ws.ticket = w;
   ws.error = w + 1;
-  ws.status = w + kScanHeaderWords;
-  ws.agg = ws.status + ntiles;
-  ws.incl = ws.agg + ntiles * ncounters;
+  ws.desc = w + kScanHeaderWords;
   return ws;
 }
 
-// LDS layout used by tile_scan: (kWavesPerTile + 2) rows of NC words:
+// LDS layout used by tile_scan: (kWavesPerTile + 3) rows of NC words:
 //   rows 0..3 : per-wave counts, turned into exclusive prefixes over the waves of the tile
 //   row  4    : tile aggregate
 //   row  5    : exclusive prefix of the tile over all earlier tiles
+//   row  6    : per counter, the nearest look-back row that held an inclusive prefix
+constexpr int kScanLdsRows = kWavesPerTile + 3;
 __host__ __device__ inline size_t scan_lds_bytes(int ncounters) {
-  return static_cast<size_t>(kWavesPerTile + 2) * ncounters * sizeof(uint32_t);
+  return static_cast<size_t>(kScanLdsRows) * ncounters * sizeof(uint32_t);
 }
+
+constexpr int kLookbackLoads = 8;  // descriptor words in flight per thread and window
 
 // cls[j] in [0, E) is the class whose running count the token asks for in counter set j
 // (negative = none); mem[j] says whether the token itself counts in that set.
@@ -62,14 +70,15 @@ template <int NSETS>
 __device__ __forceinline__ void tile_scan(const int (&cls)[NSETS], const bool (&mem)[NSETS], int E,
                                           uint32_t tile, const ScanWs& ws, uint32_t* s_cnt,
                                           uint32_t spin_limit, uint32_t (&rank)[NSETS]) {
-  __shared__ int s_nearest;
+  __shared__ int s_open;  // counters whose look-back has not reached an inclusive prefix yet
   const int tid = threadIdx.x;
   const int w = tid / kWave;
   const int NC = NSETS * E;
   uint32_t* s_agg = s_cnt + kWavesPerTile * NC;
   uint32_t* s_base = s_agg + NC;
+  uint32_t* s_stop = s_base + NC;
 
-  for (int c = tid; c < (kWavesPerTile + 2) * NC; c += kTile) s_cnt[c] = 0;
+  for (int c = tid; c < kScanLdsRows * NC; c += kTile) s_cnt[c] = 0;
   __syncthreads();
 
   // 1. wave level
@@ -90,7 +99,7 @@ __device__ __forceinline__ void tile_scan(const int (&cls)[NSETS], const bool (&
   }
   __syncthreads();
 
-  // 2. tile level: exclusive scan over the waves, publish the aggregate
+  // 2. tile level: exclusive scan over the waves, publish the tile's counts
   for (int c = tid; c < NC; c += kTile) {
     uint32_t run = 0;
 #pragma unroll
@@ -100,57 +109,78 @@ __device__ __forceinline__ void tile_scan(const int (&cls)[NSETS], const bool (&
       run += t;
     }
     s_agg[c] = run;
-    st_agent(ws.agg + static_cast<size_t>(tile) * NC + c, run);
-    if (tile == 0) st_agent(ws.incl + c, run);
+    st_agent(ws.desc + static_cast<size_t>(tile) * NC + c, (tile == 0 ? kDescInclusive : kDescAggregate) | run);
   }
-  __threadfence();
-  __syncthreads();
-  if (tid == 0) st_release_agent(ws.status + tile, tile == 0 ? 2u : 1u);
 
   // 3. decoupled look-back
   if (tile > 0) {
-    int newest = static_cast<int>(tile) - 1;  // newest predecessor not yet accounted for
+    if (tid == 0) s_open = NC;
+    for (int c = tid; c < NC; c += kTile) s_stop[c] = 0xffffffffu;
+    __syncthreads();
+    const int win_rows = max(1, (kTile * kLookbackLoads) / NC);  // rows examined per window
+    int newest = static_cast<int>(tile) - 1;                      // newest row of the window
     while (true) {
-      const int nwin = min(kTile, newest + 1);
-      if (tid == 0) s_nearest = nwin;
-      __syncthreads();
-      if (tid < nwin) {
-        const uint32_t* st_ptr = ws.status + (newest - tid);
-        uint32_t st = ld_acquire_agent(st_ptr);
-        uint32_t spins = 0;
-        while (st == 0) {
-          if (++spins > spin_limit) {  // bounded wait: flag and carry on with what is there
-            st_agent(ws.error, 1u);
-            st = 1;
-            break;
-          }
-          __builtin_amdgcn_s_sleep(2);
-          st = ld_acquire_agent(st_ptr);
+      const int nrows = min(win_rows, newest + 1);
+      const int npairs = nrows * NC;
+      uint32_t word[kLookbackLoads];
+      // issue all loads of the window, then wait for the ones that are not published yet
+#pragma unroll
+      for (int k = 0; k < kLookbackLoads; ++k) {
+        const int i = tid + k * kTile;
+        word[k] = kDescAggregate;
+        if (i < npairs) {
+          const int l = i / NC;
+          word[k] = ld_agent(ws.desc + static_cast<size_t>(newest - l) * NC + (i - l * NC));
         }
-        if (st == 2) atomicMin(&s_nearest, tid);
+      }
+#pragma unroll
+      for (int k = 0; k < kLookbackLoads; ++k) {
+        const int i = tid + k * kTile;
+        if (i < npairs && word[k] == 0) {
+          const int l = i / NC;
+          const uint32_t* ptr = ws.desc + static_cast<size_t>(newest - l) * NC + (i - l * NC);
+          uint32_t spins = 0;
+          do {
+            if (++spins > spin_limit) {  // bounded wait: flag the workspace, carry on
+              st_agent(ws.error, 1u);
+              word[k] = kDescAggregate;
+              break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+            word[k] = ld_agent(ptr);
+          } while (word[k] == 0);
+        }
+        if (i < npairs && (word[k] & kDescInclusive)) {
+          const int l = i / NC;
+          atomicMin(&s_stop[i - l * NC], static_cast<uint32_t>(static_cast<int>(tile) - 1 - (newest - l)));
+        }
       }
       __syncthreads();
-      __threadfence();
-      const int nearest = s_nearest;
-      const bool found = nearest < nwin;
-      const int nrows = found ? nearest + 1 : nwin;
-      for (int i = tid; i < nrows * NC; i += kTile) {
-        const int l = i / NC;
-        const int c = i - l * NC;
-        const size_t off = static_cast<size_t>(newest - l) * NC + c;
-        const uint32_t v = (found && l == nearest) ? ld_agent(ws.incl + off) : ld_agent(ws.agg + off);
-        if (v) atomicAdd(&s_base[c], v);
+      // add what counts: rows newer than the counter's stop row, and the stop row itself
+#pragma unroll
+      for (int k = 0; k < kLookbackLoads; ++k) {
+        const int i = tid + k * kTile;
+        if (i < npairs) {
+          const int l = i / NC;
+          const int c = i - l * NC;
+          const uint32_t depth = static_cast<uint32_t>(static_cast<int>(tile) - 1 - (newest - l));
+          const uint32_t stop = s_stop[c];
+          if (depth <= stop) {
+            const uint32_t v = word[k] & kDescCountMask;
+            if (v) atomicAdd(&s_base[c], v);
+            if (depth == stop) atomicSub(&s_open, 1);
+          }
+        }
       }
       __syncthreads();
-      if (found || newest - nwin < 0) break;
-      newest -= nwin;
+      if (s_open <= 0 || newest - nrows < 0) break;
+      newest -= nrows;
+      __syncthreads();
     }
     for (int c = tid; c < NC; c += kTile)
-      st_agent(ws.incl + static_cast<size_t>(tile) * NC + c, s_base[c] + s_agg[c]);
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) st_release_agent(ws.status + tile, 2u);
+      st_agent(ws.desc + static_cast<size_t>(tile) * NC + c, kDescInclusive | ((s_base[c] + s_agg[c]) & kDescCountMask));
   }
+  __syncthreads();
 
 #pragma unroll
   for (int j = 0; j < NSETS; ++j) {

@@ -138,7 +138,7 @@ def test_partitioned_encode_merge_redispatch(pkg, P, E, S0, M):
 # ----------------------------------------------------------------------------- top-2 extension
 @pytest.mark.parametrize("S,M,E,cf,dt", [(2048, 64, 16, 1.0, "f32"), (2048, 64, 16, 1.0, "bf16"),
                                          (1111, 24, 5, 0.6, "f32"), (4096, 32, 32, 1.25, "bf16"),
-                                         (300, 8, 2, 1.0, "f32")])
+                                         (300, 8, 2, 0.5, "f32")])
 def test_encode_top2(pkg, S, M, E, cf, dt):
     data, logits = make_inputs(S + E, S, M, E, zipf_bias=True)
     used0 = np.zeros(E, np.int32)

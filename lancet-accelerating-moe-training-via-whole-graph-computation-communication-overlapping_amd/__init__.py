@@ -3,6 +3,8 @@
   capi  - ctypes bindings of the C ABI (include/lancet_hip.h)
   ops   - the six RAF operators (moe_encode, moe_encode_batch_prioritized, moe_decode,
           moe_merge_masks, moe_redispatch, lans) over torch tensors that live on the GPU
+  raf_executor - a minimal executor over the C++ op layer (raf_hip/: OpEnv, dialect registry,
+          dispatch), the path a RAF build would take
   build - compiles the in-tree libraries with hipcc
 
 torch is used for device memory and streams only; every operator runs hand-written HIP
@@ -10,5 +12,6 @@ kernels through the C ABI and raises when the library is missing.
 """
 from . import capi  # noqa: F401
 from . import ops  # noqa: F401
+from . import raf_executor  # noqa: F401
 
-__all__ = ["capi", "ops"]
+__all__ = ["capi", "ops", "raf_executor"]

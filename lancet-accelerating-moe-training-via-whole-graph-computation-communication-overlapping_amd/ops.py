@@ -274,7 +274,7 @@ def lans(tensor_list, step, learning_rate, beta1, beta2, eps, bias_correction, w
     weight_decay, grad_averaging, mode, normalize_grad).
 
     tensor_list = [g.. | p.. | m.. | v..] (python/raf/optim/lans.py:76-103); p, m, v are updated
-    in place and returned (src/op/declare/optimizer.cc:46-62).  `step` is a Python number or a
+    in place and the output tuple aliases the inputs (src/op/declare/optimizer.cc:46-62).  `step` is a Python number or a
     0-dim float32 GPU tensor (the reference passes a tensor; it is read on the device)."""
     n = len(tensor_list)
     _need(n % 4 == 0 and n > 0, "tensor_list must hold 4 lists of equal length")
@@ -291,7 +291,7 @@ def lans(tensor_list, step, learning_rate, beta1, beta2, eps, bias_correction, w
         plan.step(g, p, m, v, 0, hyper, step_dev=step)
     else:
         plan.step(g, p, m, v, int(step), hyper)
-    return tuple(p + m + v)
+    return tuple(tensor_list)
 
 
 class LansStepper:

@@ -1,0 +1,104 @@
+// raf.op.lans in the "hip" dialect.  Counterparts in the reference: LansDecl
+// (src/op/declare/optimizer.cc:46-62: the output tuple aliases the 4T input tensors, in place)
+// and LansImpl (src/op/dialect/cuda/lans.cc:26-180).
+//
+// The constructor captures hyper-parameters and tensor sizes and creates the native plan (chunk
+// tables, partial sums, norm vectors): this replaces the q workspace of sum(numel) floats, the
+// per-chunk partials and the four norm vectors the reference requests (lans.cc:56-82); the update
+// vectors are recomputed instead of stored, so there is no q buffer and none of its offset
+// arithmetic (lans.cc:126-129).  The step scalar is read on the device (no host synchronisation,
+// unlike lans.cc:102-107); a host integer is accepted as well.
+#include <string>
+#include <vector>
+
+#include "lancet_hip.h"
+#include "op.h"
+
+namespace raf {
+namespace op {
+namespace hip {
+
+void LansDeclare(CallValues& call) {
+  RAF_CHECK(call.args.size() == 11,
+            "lans(tensor_list, step, learning_rate, beta1, beta2, eps, bias_correction, weight_decay, "
+            "grad_averaging, mode, normalize_grad)");
+  const auto& list = call.args[0].AsTuple();
+  RAF_CHECK(!list.empty() && list.size() % 4 == 0, "tensor_list must hold 4 lists of equal length");
+  call.device_id = list[0].AsTensor().device_id;
+  call.out = Value::MakeTuple(list);  // in place: outputs alias the inputs
+}
+
+class LansImpl : public OpEnv {
+ public:
+  explicit LansImpl(const CallValues& cv) {
+    const auto& list = cv.args[0].AsTuple();
+    RAF_CHECK(!list.empty() && list.size() % 4 == 0, "tensor_list must hold 4 lists of equal length");
+    const Tensor& t0 = list[0].AsTensor();
+    RAF_CHECK(t0.dtype.code == DTypeCode::kFloat && t0.dtype.bits == 32,
+              "lans is implemented for float32 (the reference's fp16 path is a LOG(FATAL), lans.cc:143-146)");
+    param_group_n_ = static_cast<int>(list.size() / 4);
+    hyper_.learning_rate = static_cast<float>(cv.args[2].AsFloat());
+    hyper_.beta1 = static_cast<float>(cv.args[3].AsFloat());
+    hyper_.beta2 = static_cast<float>(cv.args[4].AsFloat());
+    hyper_.eps = static_cast<float>(cv.args[5].AsFloat());
+    hyper_.bias_correction = static_cast<int>(cv.args[6].AsInt());
+    hyper_.weight_decay = static_cast<float>(cv.args[7].AsFloat());
+    hyper_.grad_averaging = static_cast<int>(cv.args[8].AsInt());
+    hyper_.mode = static_cast<int>(cv.args[9].AsInt());
+    hyper_.normalize_grad = cv.args[10].AsInt() != 0;
+    for (int i = 0; i < param_group_n_; ++i) numels_.push_back(list[i].AsTensor().numel());
+    for (int q = 1; q < 4; ++q)
+      for (int i = 0; i < param_group_n_; ++i)
+        RAF_CHECK(list[q * param_group_n_ + i].AsTensor().numel() == numels_[i], "the four lists must have matching sizes");
+    device_id_ = t0.device_id;
+    int st = lancet_lans_plan_create(numels_.data(), param_group_n_, &plan_);
+    if (st != LANCET_OK) throw Error(std::string("lancet_lans_plan_create failed: ") + lancet_status_string(st));
+    this->arg_indices = {0, 1};  // tensor_list, step
+  }
+
+  ~LansImpl() override {
+    if (plan_) lancet_lans_plan_destroy(plan_);
+  }
+
+  void Execute(const CallValues& cv) override { Execute({cv.args[0], cv.args[1]}, cv.out); }
+
+  void Execute(const std::vector<Value>& inputs, Value /*output*/) override {
+    const auto& list = inputs[0].AsTuple();
+    RAF_CHECK(static_cast<int>(list.size()) == 4 * param_group_n_, "tensor_list length changed");
+    std::vector<float*> ptrs;
+    for (const auto& v : list) ptrs.push_back(static_cast<float*>(v.AsTensor().data));
+    const int n = param_group_n_;
+    int step_host = 0;
+    const float* step_dev = nullptr;
+    if (inputs[1].kind == Value::kTensor) {
+      const Tensor& ts = inputs[1].AsTensor();
+      RAF_CHECK(ts.numel() == 1 && ts.dtype.code == DTypeCode::kFloat && ts.dtype.bits == 32,
+                "step must be a float32 scalar tensor");
+      step_dev = static_cast<const float*>(ts.data);
+    } else {
+      step_host = static_cast<int>(inputs[1].AsInt());
+    }
+    int st = lancet_lans_step(plan_, ptrs.data(), ptrs.data() + n, ptrs.data() + 2 * n, ptrs.data() + 3 * n,
+                              step_host, step_dev, &hyper_, GetStream(device_id_));
+    if (st != LANCET_OK)
+      throw Error(std::string("lancet_lans_step failed: ") + lancet_status_string(st) + " (status " + std::to_string(st) + ")");
+  }
+
+  std::string name() const override { return "raf.op.hip.lans"; }
+  static OpEnv* make(const CallValues& cv) { return new LansImpl(cv); }
+
+ private:
+  lancet_lans_hyper hyper_;
+  std::vector<int64_t> numels_;
+  int param_group_n_ = 0;
+  int device_id_ = 0;
+  lancet_lans_plan_t plan_ = nullptr;
+};
+
+RAF_OP_DECLARE("raf.op.lans", LansDeclare);
+RAF_REGISTER_DIALECT_OP(hip, lans, 20);
+RAF_OP_ENV_MAKER("raf.op.hip.lans", LansImpl::make);
+
+}  // namespace hip
+}  // namespace op
+}  // namespace raf

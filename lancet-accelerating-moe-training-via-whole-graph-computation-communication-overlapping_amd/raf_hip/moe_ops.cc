@@ -1,0 +1,416 @@
+// The MoE dispatch operators of the "hip" dialect: Declare functions (output shapes and dtypes)
+// and one OpEnv per operator, registered under RAF's base-op names with RAF's argument schemas
+// (scripts/src_codegen/def_schema.py:642-698).  Each OpEnv captures shapes and attributes in its
+// constructor, requests its workspace from the executor and, in Execute, hands raw pointers to
+// the C ABI (include/lancet_hip.h) on the executor's current stream.
+//
+// Counterparts in the reference: src/op/declare/moe.cc:26-213 (Declare) and
+// src/op/dialect/cuda/moe.cc:330-412 (MoeEncode), :415-729 (MoeEncodeBatchPrioritized),
+// :731-823 (MoeMergeMasks), :826-943 (MoeRedispatch), :1228-1311 (MoeDecode).
+//
+// Extensions are trailing, defaulted arguments only:
+//   moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_logits=false)
+//   moe_encode_batch_prioritized(..., capacity_factor=1.0, gate_is_logits=false)
+//   moe_decode(data, gate, indices_locations, top_k=1)
+#include <string>
+#include <vector>
+
+#include "lancet_hip.h"
+#include "op.h"
+
+namespace raf {
+namespace op {
+namespace hip {
+
+namespace {
+
+int DTypeToLancet(const DType& dt) {
+  if (dt.code == DTypeCode::kFloat && dt.bits == 32) return LANCET_F32;
+  if (dt.code == DTypeCode::kFloat && dt.bits == 16) return LANCET_F16;
+  if (dt.code == DTypeCode::kBFloat && dt.bits == 16) return LANCET_BF16;
+  throw Error("token rows must be float32, float16 or bfloat16");
+}
+
+bool IsF32(const DType& dt) { return dt.code == DTypeCode::kFloat && dt.bits == 32; }
+bool IsI32(const DType& dt) { return dt.code == DTypeCode::kInt && dt.bits == 32; }
+
+void CheckStatus(int status, const char* what) {
+  if (status != LANCET_OK)
+    throw Error(std::string(what) + " failed: " + lancet_status_string(status) + " (status " +
+                std::to_string(status) + ")");
+}
+
+Tensor MakeOut(int device_id, DTypeCode code, int bits, std::vector<int64_t> shape) {
+  Tensor t;
+  t.device_id = device_id;
+  t.dtype.code = code;
+  t.dtype.bits = bits;
+  t.shape = std::move(shape);
+  return t;
+}
+
+int64_t OptInt(const CallValues& cv, size_t i, int64_t dflt) {
+  return cv.args.size() > i && cv.args[i].kind != Value::kNone ? cv.args[i].AsInt() : dflt;
+}
+double OptFloat(const CallValues& cv, size_t i, double dflt) {
+  return cv.args.size() > i && cv.args[i].kind != Value::kNone ? cv.args[i].AsFloat() : dflt;
+}
+
+struct EncodeShape {
+  int64_t S, M, E, C;
+};
+
+// dim checks of MoeEncodeDeclare / MoeEncodeInitBody (declare/moe.cc:32-46, cuda/moe.cc:95-121)
+EncodeShape CheckEncodeInputs(const Tensor& data, const Tensor& gate, int64_t n_partitions, float cf) {
+  RAF_CHECK(data.shape.size() == 2, "Input data should be 2-D.");
+  RAF_CHECK(gate.shape.size() == 2, "Input gate should be 2-D.");
+  RAF_CHECK(data.shape[0] == gate.shape[0], "Input data and gate should have matching shape in dim 0.");
+  RAF_CHECK(IsF32(gate.dtype), "gate must be float32 in the hip dialect");
+  DTypeToLancet(data.dtype);
+  EncodeShape s;
+  s.S = data.shape[0] / n_partitions;
+  s.M = data.shape[1];
+  s.E = gate.shape[1];
+  s.C = lancet_moe_capacity(s.S, s.E, cf);
+  RAF_CHECK(s.C >= 0, "bad capacity");
+  return s;
+}
+
+// the 5-tuple of declare/moe.cc:48-58; gates_s is fp32, the buffer has the data dtype
+Value EncodeOutputs(const Tensor& data, const EncodeShape& s, int64_t k) {
+  std::vector<Value> ret;
+  ret.push_back(Value::MakeTensor(MakeOut(data.device_id, DTypeCode::kFloat, 32, {k * s.S})));
+  ret.push_back(Value::MakeTensor(MakeOut(data.device_id, DTypeCode::kInt, 32, {2, k * s.S})));
+  ret.push_back(Value::MakeTensor(MakeOut(data.device_id, DTypeCode::kInt, 32, {s.E})));
+  ret.push_back(Value::MakeTensor(MakeOut(data.device_id, DTypeCode::kUInt, 64, {s.E})));
+  Tensor buf = MakeOut(data.device_id, data.dtype.code, data.dtype.bits, {s.E, s.C, s.M});
+  ret.push_back(Value::MakeTensor(buf));
+  return Value::MakeTuple(std::move(ret));
+}
+
+}  // namespace
+
+// =====================================================================================
+// raf.op.moe_encode
+// =====================================================================================
+void MoeEncodeDeclare(CallValues& call) {
+  RAF_CHECK(call.args.size() >= 3, "moe_encode(data, gate, used_capacity, capacity_factor=1.0)");
+  const Tensor& data = call.args[0].AsTensor();
+  const Tensor& gate = call.args[1].AsTensor();
+  const Tensor& used = call.args[2].AsTensor();
+  RAF_CHECK(used.shape.size() == 1, "Input used_capacity should be 1-D.");
+  const int64_t k = OptInt(call, 4, 1);
+  RAF_CHECK(k == 1 || k == 2, "top_k must be 1 or 2");
+  const float cf = static_cast<float>(OptFloat(call, 3, 1.0)) * (k == 2 ? 2.0f : 1.0f);
+  const EncodeShape s = CheckEncodeInputs(data, gate, 1, cf);
+  RAF_CHECK(used.shape[0] == s.E && IsI32(used.dtype), "used_capacity must be int32 [E]");
+  call.out = EncodeOutputs(data, s, k);
+  call.device_id = data.device_id;
+}
+
+class MoeEncode : public OpEnv {
+ public:
+  explicit MoeEncode(const CallValues& cv) {
+    const Tensor& data = cv.args[0].AsTensor();
+    top_k_ = static_cast<int>(OptInt(cv, 4, 1));
+    const float cf = static_cast<float>(OptFloat(cv, 3, 1.0)) * (top_k_ == 2 ? 2.0f : 1.0f);
+    shape_ = CheckEncodeInputs(data, cv.args[1].AsTensor(), 1, cf);
+    flags_ = OptInt(cv, 5, 0) ? LANCET_GATE_IS_LOGITS : 0u;
+    dtype_ = DTypeToLancet(data.dtype);
+    device_id_ = data.device_id;
+    RAF_CHECK(cv.out.kind == Value::kTuple && cv.out.fields.size() == 5, "Expected output to be a 5-Tuple");
+    ws_bytes_ = lancet_moe_encode_workspace_bytes(shape_.S, shape_.E, top_k_);
+    RequestWorkspace(&ws_, device_id_, static_cast<int64_t>(ws_bytes_));
+    this->arg_indices = {0, 1, 2};  // data, gate, used_capacity
+  }
+
+  void Execute(const CallValues& cv) override { Execute({cv.args[0], cv.args[1], cv.args[2]}, cv.out); }
+
+  void Execute(const std::vector<Value>& inputs, Value output) override {
+    const Tensor& data = inputs[0].AsTensor();
+    const Tensor& gate = inputs[1].AsTensor();
+    const Tensor& used = inputs[2].AsTensor();
+    const auto& out = output.AsTuple();
+    RAF_CHECK(out.size() == 5, "Expected output to be a 5-Tuple");
+    CheckStatus(lancet_moe_encode(data.data, static_cast<const float*>(gate.data),
+                                  static_cast<const int32_t*>(used.data), shape_.S, shape_.M, shape_.E, shape_.C,
+                                  top_k_, dtype_, flags_, static_cast<float*>(out[0].AsTensor().data),
+                                  static_cast<int32_t*>(out[1].AsTensor().data),
+                                  static_cast<int32_t*>(out[2].AsTensor().data),
+                                  static_cast<uint64_t*>(out[3].AsTensor().data), out[4].AsTensor().data, ws_,
+                                  ws_bytes_, GetStream(device_id_)),
+                "lancet_moe_encode");
+  }
+
+  std::string name() const override { return "raf.op.hip.moe_encode"; }
+  static OpEnv* make(const CallValues& cv) { return new MoeEncode(cv); }
+
+ private:
+  EncodeShape shape_;
+  int top_k_, dtype_, device_id_;
+  unsigned flags_;
+  void* ws_ = nullptr;
+  size_t ws_bytes_ = 0;
+};
+
+// =====================================================================================
+// raf.op.moe_encode_batch_prioritized
+// =====================================================================================
+void MoeEncodeBatchPrioritizedDeclare(CallValues& call) {
+  RAF_CHECK(call.args.size() >= 2, "moe_encode_batch_prioritized(data, gate, n_partitions=1, partition_id=0, capacity_factor=1.0)");
+  const Tensor& data = call.args[0].AsTensor();
+  const int64_t n_part = OptInt(call, 2, 1), pid = OptInt(call, 3, 0);
+  RAF_CHECK(n_part > 0, "n_partitions should be greater than 0.");
+  RAF_CHECK(pid >= 0 && pid < n_part, "partition_id should be less than n_partitions.");
+  const EncodeShape s = CheckEncodeInputs(data, call.args[1].AsTensor(), n_part,
+                                          static_cast<float>(OptFloat(call, 4, 1.0)));
+  call.out = EncodeOutputs(data, s, 1);
+  call.device_id = data.device_id;
+}
+
+class MoeEncodeBatchPrioritized : public OpEnv {
+ public:
+  explicit MoeEncodeBatchPrioritized(const CallValues& cv) {
+    const Tensor& data = cv.args[0].AsTensor();
+    n_partitions_ = static_cast<int>(OptInt(cv, 2, 1));
+    partition_id_ = static_cast<int>(OptInt(cv, 3, 0));
+    RAF_CHECK(n_partitions_ > 0 && partition_id_ >= 0 && partition_id_ < n_partitions_, "bad partition");
+    shape_ = CheckEncodeInputs(data, cv.args[1].AsTensor(), n_partitions_, static_cast<float>(OptFloat(cv, 4, 1.0)));
+    orig_S_ = data.shape[0];
+    flags_ = OptInt(cv, 5, 0) ? LANCET_GATE_IS_LOGITS : 0u;
+    dtype_ = DTypeToLancet(data.dtype);
+    device_id_ = data.device_id;
+    // sorted indices, dropping mask, indices and gate buffers of the reference (cuda/moe.cc:512-520)
+    // are replaced by one workspace for the radix select and the scan
+    ws_bytes_ = lancet_moe_encode_bpr_workspace_bytes(orig_S_, shape_.E, n_partitions_);
+    RequestWorkspace(&ws_, device_id_, static_cast<int64_t>(ws_bytes_));
+    this->arg_indices = {0, 1};
+  }
+
+  void Execute(const CallValues& cv) override { Execute({cv.args[0], cv.args[1]}, cv.out); }
+
+  void Execute(const std::vector<Value>& inputs, Value output) override {
+    const auto& out = output.AsTuple();
+    RAF_CHECK(out.size() == 5, "Expected output to be a 5-Tuple");
+    CheckStatus(lancet_moe_encode_bpr(inputs[0].AsTensor().data, static_cast<const float*>(inputs[1].AsTensor().data),
+                                      orig_S_, shape_.M, shape_.E, shape_.C, n_partitions_, partition_id_, dtype_,
+                                      flags_, static_cast<float*>(out[0].AsTensor().data),
+                                      static_cast<int32_t*>(out[1].AsTensor().data),
+                                      static_cast<int32_t*>(out[2].AsTensor().data),
+                                      static_cast<uint64_t*>(out[3].AsTensor().data), out[4].AsTensor().data, ws_,
+                                      ws_bytes_, GetStream(device_id_)),
+                "lancet_moe_encode_bpr");
+  }
+
+  std::string name() const override { return "raf.op.hip.moe_encode_batch_prioritized"; }
+  static OpEnv* make(const CallValues& cv) { return new MoeEncodeBatchPrioritized(cv); }
+
+ private:
+  EncodeShape shape_;
+  int64_t orig_S_;
+  int n_partitions_, partition_id_, dtype_, device_id_;
+  unsigned flags_;
+  void* ws_ = nullptr;
+  size_t ws_bytes_ = 0;
+};
+
+// =====================================================================================
+// raf.op.moe_merge_masks
+// =====================================================================================
+void MoeMergeMasksDeclare(CallValues& call) {
+  RAF_CHECK(call.args.size() == 2, "moe_merge_masks(indices_locations, n_experts)");
+  const auto& masks = call.args[0].AsTuple();
+  RAF_CHECK(!masks.empty(), "indices_locations must not be empty");
+  const Tensor& m0 = masks[0].AsTensor();
+  RAF_CHECK(m0.shape.size() == 2, "Input indices_locations should be 2-D.");
+  const int64_t P = static_cast<int64_t>(masks.size());
+  call.out = Value::MakeTensor(MakeOut(m0.device_id, DTypeCode::kInt, 32, {2, m0.shape[1] * P}));
+  call.device_id = m0.device_id;
+}
+
+class MoeMergeMasks : public OpEnv {
+ public:
+  explicit MoeMergeMasks(const CallValues& cv) {
+    const auto& masks = cv.args[0].AsTuple();
+    n_partitions_ = static_cast<int>(masks.size());
+    RAF_CHECK(n_partitions_ >= 1 && n_partitions_ <= LANCET_MAX_PARTITIONS, "unsupported number of partitions");
+    const Tensor& m0 = masks[0].AsTensor();
+    RAF_CHECK(m0.shape.size() == 2 && m0.shape[0] == 2, "Expected input indices_locations to be [2, S].");
+    dim_S_ = m0.shape[1];
+    dim_E_ = cv.args[1].AsInt();
+    device_id_ = m0.device_id;
+    // the reference keeps a pinned host table and a device table of 2P pointers
+    // (cuda/moe.cc:751-755); pointer tables travel as kernel arguments here
+    ws_bytes_ = lancet_moe_merge_masks_workspace_bytes(n_partitions_, dim_E_);
+    RequestWorkspace(&ws_, device_id_, static_cast<int64_t>(ws_bytes_));
+    this->arg_indices = {0};
+  }
+
+  void Execute(const CallValues& cv) override { Execute({cv.args[0]}, cv.out); }
+
+  void Execute(const std::vector<Value>& inputs, Value output) override {
+    const auto& masks = inputs[0].AsTuple();
+    RAF_CHECK(static_cast<int>(masks.size()) == n_partitions_, "partition count changed");
+    std::vector<const int32_t*> ptrs;
+    for (const auto& m : masks) {
+      const Tensor& t = m.AsTensor();
+      RAF_CHECK(IsI32(t.dtype) && t.shape.size() == 2 && t.shape[1] == dim_S_, "indices_locations must be int32 [2, S]");
+      ptrs.push_back(static_cast<const int32_t*>(t.data));
+    }
+    CheckStatus(lancet_moe_merge_masks(ptrs.data(), n_partitions_, dim_S_, dim_E_,
+                                       static_cast<int32_t*>(output.AsTensor().data), ws_, ws_bytes_,
+                                       GetStream(device_id_)),
+                "lancet_moe_merge_masks");
+  }
+
+  std::string name() const override { return "raf.op.hip.moe_merge_masks"; }
+  static OpEnv* make(const CallValues& cv) { return new MoeMergeMasks(cv); }
+
+ private:
+  int64_t dim_S_, dim_E_;
+  int n_partitions_, device_id_;
+  void* ws_ = nullptr;
+  size_t ws_bytes_ = 0;
+};
+
+// =====================================================================================
+// raf.op.moe_redispatch
+// =====================================================================================
+void MoeRedispatchDeclare(CallValues& call) {
+  RAF_CHECK(call.args.size() == 2, "moe_redispatch(data, indices_locations)");
+  const auto& bufs = call.args[0].AsTuple();
+  const auto& masks = call.args[1].AsTuple();
+  RAF_CHECK(!bufs.empty() && bufs.size() == masks.size(), "data and indices_locations must have one entry per partition");
+  const Tensor& d0 = bufs[0].AsTensor();
+  RAF_CHECK(d0.shape.size() == 3 || d0.shape.size() == 4, "Input data should be 3 or 4-D.");
+  RAF_CHECK(masks[0].AsTensor().shape.size() == 2, "Input indices_locations should be 2-D.");
+  // data dtype, as the type relation says (src/op/ty/moe.cc:141); Declare hard-codes float32
+  // (declare/moe.cc:136), which cannot hold for 16-bit buffers
+  call.out = Value::MakeTensor(MakeOut(d0.device_id, d0.dtype.code, d0.dtype.bits, d0.shape));
+  call.device_id = d0.device_id;
+}
+
+class MoeRedispatch : public OpEnv {
+ public:
+  explicit MoeRedispatch(const CallValues& cv) {
+    const auto& bufs = cv.args[0].AsTuple();
+    const auto& masks = cv.args[1].AsTuple();
+    n_partitions_ = static_cast<int>(masks.size());
+    RAF_CHECK(n_partitions_ >= 1 && n_partitions_ <= LANCET_MAX_PARTITIONS, "unsupported number of partitions");
+    const Tensor& d0 = bufs[0].AsTensor();
+    if (d0.shape.size() == 3) {  // [E, C, M]
+      dim_E_ = d0.shape[0], dim_C_ = d0.shape[1], dim_M_ = d0.shape[2];
+    } else {                     // [G, LE, C, M]
+      RAF_CHECK(d0.shape.size() == 4, "Expected input data to be 3 or 4D.");
+      dim_E_ = d0.shape[0] * d0.shape[1], dim_C_ = d0.shape[2], dim_M_ = d0.shape[3];
+    }
+    dim_S_ = masks[0].AsTensor().shape[1];
+    dtype_ = DTypeToLancet(d0.dtype);
+    device_id_ = d0.device_id;
+    ws_bytes_ = lancet_moe_redispatch_workspace_bytes(n_partitions_, dim_E_);
+    RequestWorkspace(&ws_, device_id_, static_cast<int64_t>(ws_bytes_));
+    this->arg_indices = {0, 1};
+  }
+
+  void Execute(const CallValues& cv) override { Execute({cv.args[0], cv.args[1]}, cv.out); }
+
+  void Execute(const std::vector<Value>& inputs, Value output) override {
+    const auto& bufs = inputs[0].AsTuple();
+    const auto& masks = inputs[1].AsTuple();
+    RAF_CHECK(static_cast<int>(masks.size()) == n_partitions_ && bufs.size() == masks.size(), "partition count changed");
+    std::vector<const void*> dptrs;
+    std::vector<const int32_t*> mptrs;
+    for (int i = 0; i < n_partitions_; ++i) {
+      dptrs.push_back(bufs[i].AsTensor().data);
+      mptrs.push_back(static_cast<const int32_t*>(masks[i].AsTensor().data));
+    }
+    CheckStatus(lancet_moe_redispatch(dptrs.data(), mptrs.data(), n_partitions_, dim_S_, dim_M_, dim_C_, dim_E_,
+                                      dtype_, output.AsTensor().data, ws_, ws_bytes_, GetStream(device_id_)),
+                "lancet_moe_redispatch");
+  }
+
+  std::string name() const override { return "raf.op.hip.moe_redispatch"; }
+  static OpEnv* make(const CallValues& cv) { return new MoeRedispatch(cv); }
+
+ private:
+  int64_t dim_S_, dim_E_, dim_C_, dim_M_;
+  int n_partitions_, dtype_, device_id_;
+  void* ws_ = nullptr;
+  size_t ws_bytes_ = 0;
+};
+
+// =====================================================================================
+// raf.op.moe_decode
+// =====================================================================================
+void MoeDecodeDeclare(CallValues& call) {
+  RAF_CHECK(call.args.size() >= 3, "moe_decode(data, gate, indices_locations)");
+  const Tensor& data = call.args[0].AsTensor();
+  const Tensor& gate = call.args[1].AsTensor();
+  RAF_CHECK(data.shape.size() == 3, "Input data should be 3-D.");
+  RAF_CHECK(gate.shape.size() == 1, "Input gate should be 1-D.");
+  DTypeToLancet(data.dtype);
+  const int64_t k = OptInt(call, 3, 1);
+  RAF_CHECK(k == 1 || k == 2, "top_k must be 1 or 2");
+  RAF_CHECK(gate.shape[0] % k == 0, "gate length must be a multiple of top_k");
+  call.out = Value::MakeTensor(MakeOut(data.device_id, data.dtype.code, data.dtype.bits, {gate.shape[0] / k, data.shape[2]}));
+  call.device_id = data.device_id;
+}
+
+class MoeDecode : public OpEnv {
+ public:
+  explicit MoeDecode(const CallValues& cv) {
+    const Tensor& data = cv.args[0].AsTensor();
+    const Tensor& gate = cv.args[1].AsTensor();
+    RAF_CHECK(data.shape.size() == 3, "Expected input data to be 3D.");
+    RAF_CHECK(gate.shape.size() == 1, "Expected input gate to be 1D.");
+    RAF_CHECK(IsF32(gate.dtype), "gate must be float32 in the hip dialect");
+    top_k_ = static_cast<int>(OptInt(cv, 3, 1));
+    dim_S_ = gate.shape[0] / top_k_;
+    dim_E_ = data.shape[0], dim_C_ = data.shape[1], dim_M_ = data.shape[2];
+    dtype_ = DTypeToLancet(data.dtype);
+    device_id_ = data.device_id;
+    this->arg_indices = {0, 1, 2};
+  }
+
+  void Execute(const CallValues& cv) override { Execute({cv.args[0], cv.args[1], cv.args[2]}, cv.out); }
+
+  void Execute(const std::vector<Value>& inputs, Value output) override {
+    const Tensor& il = inputs[2].AsTensor();
+    RAF_CHECK(IsI32(il.dtype) && il.shape.size() == 2 && il.shape[1] == dim_S_ * top_k_, "indices_locations must be int32 [2, k*S]");
+    CheckStatus(lancet_moe_decode(inputs[0].AsTensor().data, static_cast<const float*>(inputs[1].AsTensor().data),
+                                  static_cast<const int32_t*>(il.data), dim_S_, dim_M_, dim_E_, dim_C_, top_k_,
+                                  dtype_, output.AsTensor().data, GetStream(device_id_)),
+                "lancet_moe_decode");
+  }
+
+  std::string name() const override { return "raf.op.hip.moe_decode"; }
+  static OpEnv* make(const CallValues& cv) { return new MoeDecode(cv); }
+
+ private:
+  int64_t dim_S_, dim_E_, dim_C_, dim_M_;
+  int top_k_, dtype_, device_id_;
+};
+
+// ---- registration (cuda/cuda_utils.cc:17; cuda/moe.cc:411-412,728-729,822-823,942-943,1310-1311) ----
+RAF_REGISTER_DIALECT("hip").set_enable("hip");
+
+RAF_OP_DECLARE("raf.op.moe_encode", MoeEncodeDeclare);
+RAF_OP_DECLARE("raf.op.moe_encode_batch_prioritized", MoeEncodeBatchPrioritizedDeclare);
+RAF_OP_DECLARE("raf.op.moe_merge_masks", MoeMergeMasksDeclare);
+RAF_OP_DECLARE("raf.op.moe_redispatch", MoeRedispatchDeclare);
+RAF_OP_DECLARE("raf.op.moe_decode", MoeDecodeDeclare);
+
+RAF_REGISTER_DIALECT_OP(hip, moe_encode, 20);
+RAF_OP_ENV_MAKER("raf.op.hip.moe_encode", MoeEncode::make);
+RAF_REGISTER_DIALECT_OP(hip, moe_encode_batch_prioritized, 20);
+RAF_OP_ENV_MAKER("raf.op.hip.moe_encode_batch_prioritized", MoeEncodeBatchPrioritized::make);
+RAF_REGISTER_DIALECT_OP(hip, moe_merge_masks, 20);
+RAF_OP_ENV_MAKER("raf.op.hip.moe_merge_masks", MoeMergeMasks::make);
+RAF_REGISTER_DIALECT_OP(hip, moe_redispatch, 20);
+RAF_OP_ENV_MAKER("raf.op.hip.moe_redispatch", MoeRedispatch::make);
+RAF_REGISTER_DIALECT_OP(hip, moe_decode, 20);
+RAF_OP_ENV_MAKER("raf.op.hip.moe_decode", MoeDecode::make);
+
+}  // namespace hip
+}  // namespace op
+}  // namespace raf

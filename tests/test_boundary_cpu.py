@@ -1,0 +1,158 @@
+"""CPU-side checks of the drop-in boundary: the C-ABI library exports every symbol the header
+declares, rejects bad arguments with a status (never aborts), and the C++ op layer registers the
+six operators under RAF's names with RAF's output contract.  No kernel is launched."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_symbols():
+    text = open(os.path.join(ROOT, "include", "lancet_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(lancet_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(pkg):
+    lib = pkg.capi.load()
+    names = header_symbols()
+    assert len(names) >= 25
+    for n in names:
+        assert hasattr(lib, n), "liblancet_hip.so does not export %s" % n
+    assert sorted(pkg.capi.SIGNATURES) == names, "capi.SIGNATURES and the header disagree"
+    assert lib.lancet_abi_version() == 1
+
+
+def test_capacity_formula(pkg):
+    cap = pkg.ops.moe_capacity
+    assert cap(4096, 8, 1.25) == 640 and cap(16384, 16, 2.0) == 2048 and cap(32768, 64, 1.25) == 640
+    assert cap(65536, 32, 2.5) == 5120 and cap(16384, 32, 10.0) == 5120 and cap(10, 4, 1.5) == 4
+
+
+def test_workspace_sizes_and_argument_rejection(pkg):
+    lib, capi = pkg.capi.load(), pkg.capi
+    assert lib.lancet_moe_encode_workspace_bytes(65536, 32, 2) == (2 + 256 * 64) * 4
+    assert lib.lancet_moe_encode_workspace_bytes(0, 4, 1) == (2 + 1 * 4) * 4
+    assert lib.lancet_moe_encode_workspace_bytes(10, 0, 1) == 0
+    one = C.c_void_p(16)  # never dereferenced: every call below is rejected before any launch
+    st = lib.lancet_moe_encode(one, one, None, 8, 4, 2, 4, 1, 99, 0, one, one, one, one, one, one, 1 << 20, None)
+    assert st == capi.ERR_DTYPE
+    st = lib.lancet_moe_encode(one, one, None, 8, 4, 2, 4, 3, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
+    assert st == capi.ERR_TOPK
+    st = lib.lancet_moe_encode(one, one, None, 8, 4, 1, 4, 2, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
+    assert st == capi.ERR_TOPK                      # top-2 needs two experts
+    st = lib.lancet_moe_encode(one, one, None, 8, 4, 2, 4, 1, capi.F32, 0, one, one, one, one, one, one, 8, None)
+    assert st == capi.ERR_WORKSPACE
+    st = lib.lancet_moe_encode(one, one, None, 8, 4, 2, 4, 1, capi.F32, 0, one, None, one, one, one, one, 1 << 20, None)
+    assert st == capi.ERR_NULL
+    st = lib.lancet_moe_encode(one, one, None, -1, 4, 2, 4, 1, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
+    assert st == capi.ERR_SHAPE
+    st = lib.lancet_moe_encode(one, one, None, 8, 4, 1000, 4, 1, capi.F32, 0, one, one, one, one, one, one, 1 << 30, None)
+    assert st == capi.ERR_SHAPE                     # more experts than LANCET_MAX_EXPERTS
+    st = lib.lancet_moe_encode(C.c_void_p(18), one, None, 8, 4, 2, 4, 1, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
+    assert st == capi.ERR_ALIGN
+    st = lib.lancet_moe_encode_bpr(one, one, 8, 4, 2, 4, 2, 2, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
+    assert st == capi.ERR_PARTITION
+    ptrs = capi.ptr_array([16] * 70)
+    assert lib.lancet_moe_merge_masks(ptrs, 70, 8, 2, one, one, 1 << 20, None) == capi.ERR_PARTITION
+    assert lib.lancet_lans_plan_destroy(None) == capi.ERR_PLAN
+    assert "workspace" in capi.status_string(capi.ERR_WORKSPACE)
+
+
+# ----------------------------------------------------------------------------- C++ op layer
+def _declare(rx, op, pushes):
+    lib = rx.load()
+    h = lib.raf_hip_call_create(op.encode())
+    for kind, val in pushes:
+        if kind == "t":
+            dtype, shape = val
+            code, bits = dtype
+            arr = (C.c_int64 * len(shape))(*shape)
+            assert lib.raf_hip_push_tensor(h, C.c_void_p(256), 0, code, bits, len(shape), arr) == 0
+        elif kind == "i":
+            assert lib.raf_hip_push_int(h, val) == 0
+        elif kind == "f":
+            assert lib.raf_hip_push_float(h, val) == 0
+        elif kind == "(":
+            assert lib.raf_hip_begin_tuple(h) == 0
+        elif kind == ")":
+            assert lib.raf_hip_end_tuple(h) == 0
+    rc = lib.raf_hip_declare(h)
+    outs = []
+    if rc == 0:
+        for i in range(lib.raf_hip_num_outputs(h)):
+            code, bits, data = C.c_int(), C.c_int(), C.c_void_p()
+            shape = (C.c_int64 * 8)()
+            nd = lib.raf_hip_output_info(h, i, C.byref(code), C.byref(bits), shape, C.byref(data))
+            outs.append(((code.value, bits.value), tuple(shape[d] for d in range(nd))))
+    return h, rc, outs
+
+
+F32, BF16, I32, U64 = (2, 32), (4, 16), (0, 32), (1, 64)
+
+
+def test_op_layer_registers_the_six_operators(pkg):
+    rx = pkg.raf_executor
+    ops = rx.registered_ops()
+    for name in ("moe_encode", "moe_encode_batch_prioritized", "moe_decode", "moe_merge_masks", "moe_redispatch", "lans"):
+        assert "raf.op." + name in ops
+        assert rx.dispatch_list("raf.op." + name) == [("raf.op.hip." + name, 20)]   # plevel 20 as cuda/moe.cc:411
+    with rx.dialect_preference(["cuda"]):
+        assert rx.dispatch_list("raf.op.moe_encode") == []
+    with rx.dialect_preference(["cuda", "hip"]):
+        assert rx.dispatch_list("raf.op.moe_encode") == [("raf.op.hip.moe_encode", 20)]
+
+
+def test_declare_reproduces_the_output_contract(pkg):
+    """src/op/declare/moe.cc:26-213 / src/op/ty/moe.cc: shapes and dtypes of every output."""
+    rx = pkg.raf_executor
+    lib = rx.load()
+    S, M, E = 4096, 768, 8
+    h, rc, outs = _declare(rx, "raf.op.moe_encode", [("t", (F32, (S, M))), ("t", (F32, (S, E))), ("t", (I32, (E,))), ("f", 1.25)])
+    assert rc == 0 and outs == [(F32, (S,)), (I32, (2, S)), (I32, (E,)), (U64, (E,)), (F32, (E, 640, M))]
+    assert lib.raf_hip_dispatch(h) == 0 and lib.raf_hip_env_name(h) == b"raf.op.hip.moe_encode"
+    assert lib.raf_hip_num_workspaces(h) == 1
+    assert lib.raf_hip_workspace_bytes(h, 0) == pkg.capi.load().lancet_moe_encode_workspace_bytes(S, E, 1)
+    assert [lib.raf_hip_arg_index(h, i) for i in range(lib.raf_hip_num_arg_indices(h))] == [0, 1, 2]
+    lib.raf_hip_call_destroy(h)
+    # top-2 extension: slot-major outputs, doubled capacity factor, bf16 buffer
+    h, rc, outs = _declare(rx, "raf.op.moe_encode", [("t", (BF16, (16384, 1024))), ("t", (F32, (16384, 16))),
+                                                     ("t", (I32, (16,))), ("f", 1.0), ("i", 2), ("i", 1)])
+    assert rc == 0 and outs == [(F32, (32768,)), (I32, (2, 32768)), (I32, (16,)), (U64, (16,)), (BF16, (16, 2048, 1024))]
+    lib.raf_hip_call_destroy(h)
+    h, rc, outs = _declare(rx, "raf.op.moe_encode_batch_prioritized",
+                           [("t", (BF16, (32768, 2048))), ("t", (F32, (32768, 64))), ("i", 4), ("i", 1), ("f", 5.0)])
+    assert rc == 0 and outs == [(F32, (8192,)), (I32, (2, 8192)), (I32, (64,)), (U64, (64,)), (BF16, (64, 640, 2048))]
+    lib.raf_hip_call_destroy(h)
+    h, rc, outs = _declare(rx, "raf.op.moe_merge_masks", [("(", 0)] + [("t", (I32, (2, 100)))] * 4 + [(")", 0), ("i", 8)])
+    assert rc == 0 and outs == [(I32, (2, 400))]
+    lib.raf_hip_call_destroy(h)
+    h, rc, outs = _declare(rx, "raf.op.moe_redispatch", [("(", 0)] + [("t", (BF16, (8, 50, 64)))] * 2 + [(")", 0), ("(", 0)] +
+                           [("t", (I32, (2, 100)))] * 2 + [(")", 0)])
+    assert rc == 0 and outs == [(BF16, (8, 50, 64))]
+    lib.raf_hip_call_destroy(h)
+    h, rc, outs = _declare(rx, "raf.op.moe_decode", [("t", (F32, (8, 50, 64))), ("t", (F32, (100,))), ("t", (I32, (2, 100)))])
+    assert rc == 0 and outs == [(F32, (100, 64))]
+    lib.raf_hip_call_destroy(h)
+
+
+def test_op_layer_errors_are_reported_not_fatal(pkg):
+    rx = pkg.raf_executor
+    lib = rx.load()
+    h, rc, _ = _declare(rx, "raf.op.moe_encode", [("t", (F32, (10, 4))), ("t", (F32, (11, 2))), ("t", (I32, (2,)))])
+    assert rc != 0 and b"matching shape in dim 0" in lib.raf_hip_last_error()
+    lib.raf_hip_call_destroy(h)
+    h, rc, _ = _declare(rx, "raf.op.moe_encode_batch_prioritized", [("t", (F32, (10, 4))), ("t", (F32, (10, 2))), ("i", 2), ("i", 2)])
+    assert rc != 0 and b"partition_id should be less than n_partitions" in lib.raf_hip_last_error()
+    lib.raf_hip_call_destroy(h)
+    h, rc, _ = _declare(rx, "raf.op.not_an_op", [])
+    assert rc != 0 and b"no FRAFDeclare" in lib.raf_hip_last_error()
+    lib.raf_hip_call_destroy(h)
+    with rx.dialect_preference(["cuda"]):
+        h, rc, _ = _declare(rx, "raf.op.moe_decode", [("t", (F32, (8, 50, 64))), ("t", (F32, (100,))), ("t", (I32, (2, 100)))])
+        assert rc == 0 and lib.raf_hip_dispatch(h) != 0
+        assert b"Cannot find a valid dispatch" in lib.raf_hip_last_error()
+        lib.raf_hip_call_destroy(h)

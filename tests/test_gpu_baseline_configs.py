@@ -1,0 +1,156 @@
+"""The BASELINE.json configurations at their full sizes.
+
+Routing integers are compared with the oracle bit for bit at full size.  The [E,C,M] buffers and
+the recombined [S,M] outputs are compared through properties that hold at any size and are
+evaluated on the GPU: every kept token's row is found bit-equal at its (expert, location), rows
+past the used capacity are zero, decode(identity expert) returns the token scaled by its combine
+weight(s).  (The oracle's own buffers are compared directly at the reduced sizes of
+test_gpu_moe.py.)"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as mo
+from tests.gpu_util import dev, make_inputs, rows_to_torch, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def check_buffer_properties(data_t, il_t, used_t, disp_t, k):
+    S = data_t.shape[0]
+    E, Cap, M = disp_t.shape
+    il = il_t.long()
+    for j in range(k):
+        idx, loc = il[0, j * S:(j + 1) * S], il[1, j * S:(j + 1) * S]
+        ok = idx >= 0
+        assert torch.equal(disp_t[idx[ok], loc[ok]], data_t[ok])
+    # kept rows per expert = used (used_in = 0), rows past them are zero
+    kept = torch.bincount(il[0][il[0] >= 0], minlength=E)
+    assert torch.equal(kept, used_t.long())
+    tail = torch.arange(Cap, device="cuda")[None, :] >= used_t.long()[:, None]
+    assert not disp_t[tail].any()
+
+
+def test_config1_switch_top1_fp32(pkg):
+    """S=4096, M=768 fp32, E=8, top-1, C=640, combine weight = top-1 softmax prob, seed 0."""
+    S, M, E, cf = 4096, 768, 8, 1.25
+    data, logits = make_inputs(0, S, M, E)
+    want = mo.moe_encode(data, logits, np.zeros(E, np.int32), cf, gate_is_logits=True, fast_scatter=True)
+    got = pkg.ops.moe_encode(dev(data), dev(logits), None, cf, gate_is_logits=True)
+    assert got[4].shape == (E, 640, M)
+    np.testing.assert_array_equal(to_np(got[1]), want[1])
+    np.testing.assert_array_equal(to_np(got[2]), want[2])
+    np.testing.assert_array_equal(to_np(got[3]), want[3])
+    np.testing.assert_allclose(to_np(got[0]), want[0], rtol=1e-5)
+    np.testing.assert_array_equal(to_np(got[4]), want[4])
+    out = pkg.ops.moe_decode(got[4], got[0], got[1])
+    np.testing.assert_array_equal(to_np(out), mo.moe_decode(want[4], to_np(got[0]), want[1]))
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_config2_gshard_top2_zipf(pkg, dt):
+    """S=16384, M=1024, E=16, top-2, capacity factor 1.0 (C=2048), Zipf(1.2) expert bias."""
+    S, M, E, cf = 16384, 1024, 16, 1.0
+    data, logits = make_inputs(0, S, M, E, zipf_bias=True)
+    sel, val = mo.select_topk(logits, 2, True)
+    zero = np.zeros(E, np.int32)
+    Cap = mo.capacity(S, E, 2 * cf)
+    assert Cap == 2048
+    i1, l1, u1, _ = mo.gen_location(sel[0], zero, Cap, M, E)
+    i2, l2, u2, _ = mo.gen_location(sel[1], u1, Cap, M, E)
+    merged = mo.moe_merge_masks([np.stack([i1, l1]), np.stack([i2, l2])], E)
+    d_data = rows_to_torch(data, dt)
+    got = pkg.ops.moe_encode(d_data, dev(logits), None, cf, top_k=2, gate_is_logits=True)
+    np.testing.assert_array_equal(to_np(got[1]), merged)
+    np.testing.assert_array_equal(to_np(got[2]), u2)
+    assert (merged[0] < 0).sum() > 1000, "hot experts must overflow"
+    raw = np.concatenate([val[0], val[1]])
+    np.testing.assert_allclose(to_np(got[0]), mo.top2_normalize_gates(raw, merged[0]), rtol=1e-5)
+    check_buffer_properties(d_data, got[1], got[2], got[4], 2)
+    out = pkg.ops.moe_decode(got[4], got[0], got[1], top_k=2)
+    # identity expert: out = (g1 + g2) * x with g1 + g2 = 1 where any slot was kept, else 0
+    either = (got[1][0, :S] >= 0) | (got[1][0, S:] >= 0)
+    x = d_data.float()
+    tol = 2e-6 if dt == "f32" else 2 ** -7
+    assert float(((out.float() - x)[either].abs() / x[either].abs().clamp_min(1e-20)).max()) <= tol
+    assert not out[~either].any() and (~either).any()
+
+
+@pytest.mark.parametrize("P", [1, 4])
+@pytest.mark.parametrize("hot_experts", [False, True])
+def test_config3_batch_prioritized_bf16(pkg, P, hot_experts):
+    """S=32768, M=2048 bf16, E=64, top-1, cf=1.25 (C=640), logits ~ 2*N(0,1); the drop set of the
+    sort+scan is reproduced exactly, for the whole batch and for 4 partitions.  With the
+    configuration's balanced logits no expert reaches its capacity (512 +- 22 tokens against
+    640), so the same shape is also run with a Zipf expert bias that makes hot experts overflow."""
+    S0, M, E, cf = 32768, 2048, 64, 1.25
+    data, logits = make_inputs(0, S0, M, E, logit_scale=2.0, zipf_bias=hot_experts)
+    gate = mo.softmax_rows(logits)           # priorities: fp32 softmax prob of the top expert
+    d_data, d_gate = rows_to_torch(data, "bf16"), dev(gate)
+    S = S0 // P
+    kept_total = np.zeros(E, np.int64)
+    for pid in range(P):
+        want = mo.moe_encode_bpr(np.zeros((S0, 1), np.float32), gate, P, pid, cf * P, fast_scatter=True)
+        got = pkg.ops.moe_encode_batch_prioritized(d_data, d_gate, P, pid, cf * P)
+        assert got[4].shape == (E, 640, M)
+        np.testing.assert_array_equal(to_np(got[1]), want[1])
+        np.testing.assert_array_equal(to_np(got[2]), want[2])
+        np.testing.assert_array_equal(to_np(got[0]), want[0])
+        check_buffer_properties(d_data[pid * S:(pid + 1) * S], got[1], got[2], got[4], 1)
+        kept_total += want[2]
+    cnt = np.bincount(np.argmax(gate, axis=1), minlength=E)
+    np.testing.assert_array_equal(kept_total, np.minimum(cnt, 640))
+    assert bool((cnt > 640).any()) == hot_experts
+
+
+def test_config4_lancet_forward_pipeline_bf16(pkg):
+    """S=65536 (4 partitions of 16384), M=4096 bf16, E=32, top-2, cf=1.25 -> C=5120: encode per
+    (slot, partition) in capacity order s1p0..s1p3, s2p0..s2p3 with chained used capacity, then
+    moe_merge_masks + moe_redispatch, then moe_decode; must equal the un-partitioned top-2 op."""
+    ops = pkg.ops
+    S0, M, E, cf, P = 65536, 4096, 32, 1.25, 4
+    S = S0 // P
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    data = torch.empty((S0, M), device="cuda").normal_(0, 1, generator=gen).to(torch.bfloat16)
+    logits = torch.empty((S0, E), device="cuda").normal_(0, 1, generator=gen)
+    logits[:, :4] += 0.75            # some pressure so that slot 2 overflows
+    fused = ops.moe_encode(data, logits, None, cf, top_k=2, gate_is_logits=True)
+    assert fused[4].shape == (E, 5120, M)
+    # per-slot gate arrays: argmax = the slot's expert, max = its softmax probability
+    lib = pkg.capi.load()
+    import ctypes as C
+    sel = torch.empty((2, S0), dtype=torch.int32, device="cuda")
+    val = torch.empty((2, S0), dtype=torch.float32, device="cuda")
+    assert lib.lancet_gate_topk(C.c_void_p(logits.data_ptr()), S0, E, 2, pkg.capi.GATE_IS_LOGITS,
+                                C.c_void_p(sel.data_ptr()), C.c_void_p(val.data_ptr()), None) == 0
+    used = torch.zeros(E, dtype=torch.int32, device="cuda")
+    ils, bufs, raws = [], [], []
+    for slot in range(2):
+        for p in range(P):
+            sl = slice(p * S, (p + 1) * S)
+            gate = torch.full((S, E), -1.0, device="cuda")
+            gate.scatter_(1, sel[slot, sl].long()[:, None], val[slot, sl][:, None])
+            g, il, used, elems, disp = ops.moe_encode(data[sl], gate, used, 2 * cf * P)
+            assert disp.shape == (E, 5120, M)
+            ils.append(il), bufs.append(disp), raws.append(g)
+    merged = ops.moe_merge_masks(ils, E)                 # [2, 8*S] = slot-major [2, 2*S0]
+    red = ops.moe_redispatch(bufs, ils)
+    del bufs
+    weights = ops.moe_top2_normalize_gates(torch.cat(raws), merged)
+    assert torch.equal(merged, fused[1])
+    assert torch.equal(used, fused[2])
+    assert torch.equal(red, fused[4])
+    np.testing.assert_allclose(to_np(weights), to_np(fused[0]), rtol=1e-5)
+    assert int((merged[0] < 0).sum()) > 0
+    out_p = ops.moe_decode(red, weights, merged, top_k=2)
+    out_f = ops.moe_decode(fused[4], fused[0], fused[1], top_k=2)
+    diff = (out_p.view(torch.int16).int() - out_f.view(torch.int16).int()).abs().max()
+    assert int(diff) <= 1
+    # routing at full size against the oracle
+    h_logits = logits.cpu().numpy()
+    osel, _ = mo.select_topk(h_logits, 2, True)
+    zero = np.zeros(E, np.int32)
+    i1, l1, u1, _ = mo.gen_location(osel[0], zero, 5120, M, E)
+    i2, l2, u2, _ = mo.gen_location(osel[1], u1, 5120, M, E)
+    np.testing.assert_array_equal(to_np(merged), mo.moe_merge_masks([np.stack([i1, l1]), np.stack([i2, l2])], E))
+    check_buffer_properties(data, merged, used, red, 2)

@@ -37,6 +37,8 @@ def parse():
     ap.add_argument("--no-lans", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--lans-scale", type=float, default=1.0, help="fraction of the 24-layer LANS tensor list")
+    ap.add_argument("--only", default="all", choices=["all", "scatter", "decode", "route", "copy", "lans"],
+                    help="profiling aid: run just one kernel family (prints a short JSON line)")
     return ap.parse_args()
 
 
@@ -172,6 +174,22 @@ def main():
     lib = capi.load()
     import ctypes as C
 
+    if args.only == "copy":
+        # calibration for the HBM byte counters: a plain copy of known size (1 GiB read + 1 GiB written)
+        n = 1 << 30
+        src = torch.zeros(n, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(args.warmup):
+            dst.copy_(src)
+        ms = event_ms(lambda: dst.copy_(src), args.steps)
+        print(json.dumps({"only": "copy", "bytes_read": n, "bytes_written": n, "ms": round(ms, 4),
+                          "GBps": round(2 * n / ms / 1e6, 1)}), flush=True)
+        return
+    if args.only == "lans":
+        print(json.dumps({"only": "lans", "lans": bench_lans(ops, capi, args.steps, args.warmup, args.lans_scale)}),
+              flush=True)
+        return
+
     S, M, E, K, cf = args.tokens, args.hidden, args.experts, 2, 1.25
     b = 2  # bf16
     Cap = ops.moe_capacity(S, E, 2 * cf)
@@ -251,6 +269,13 @@ def main():
                                   p(outs[1]), p(outs[2]), p(outs[3]), p(ws), ws.numel(), stream)
         assert st == 0
 
+    if args.only in ("scatter", "decode", "route"):
+        fn = {"scatter": scatter_only, "decode": decode, "route": route_only}[args.only]
+        for _ in range(args.warmup):
+            fn()
+        ms = event_ms(fn, args.steps)
+        print(json.dumps({"only": args.only, "ms": round(ms, 4), "steps": args.steps}), flush=True)
+        return
     ms_route = event_ms(route_only, n)
     encode()
     ms_scatter = event_ms(scatter_only, n)

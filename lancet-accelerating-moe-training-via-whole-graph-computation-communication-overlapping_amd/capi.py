@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(HERE, "lib", "liblancet_hip.so")
 
 F32, BF16, F16 = 0, 1, 2
 GATE_IS_LOGITS = 1
+LANS_SWEEPS, LANS_PIPELINED = 0, 1
 MAX_EXPERTS = 512
 MAX_PARTITIONS = 64
 
@@ -61,6 +62,9 @@ SIGNATURES = {
     "lancet_lans_step": (_int, [_vp, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),
                                 _int, _vp, C.POINTER(LansHyper), _vp]),
     "lancet_lans_plan_norms": (_int, [_vp, _vp, _vp]),
+    "lancet_lans_plan_set_schedule": (_int, [_vp, _int]),
+    "lancet_lans_plan_error": (_int, [_vp, _vp, C.POINTER(_int)]),
+    "lancet_lans_debug_task_queue": (_i64, [C.POINTER(_i64), _int, _vp, _vp, _i64]),
     "lancet_debug_set_spin_limit": (None, [_u32]),
     "lancet_scan_workspace_error": (_int, [_vp, _vp, C.POINTER(_int)]),
 }

@@ -226,7 +226,7 @@ class LansPlan:
     """Owns the native plan of one parameter set (what the reference's LansImpl constructor
     captures, src/op/dialect/cuda/lans.cc:28-83)."""
 
-    def __init__(self, numels):
+    def __init__(self, numels, schedule=None):
         lib = capi.load()
         self.numels = [int(n) for n in numels]
         arr = (C.c_int64 * len(self.numels))(*self.numels)
@@ -234,6 +234,17 @@ class LansPlan:
         capi.check(lib.lancet_lans_plan_create(arr, len(self.numels), C.byref(handle)), "lancet_lans_plan_create")
         self._h = handle
         self._lib = lib
+        if schedule is not None:
+            self.set_schedule(schedule)
+
+    def set_schedule(self, schedule):
+        """capi.LANS_SWEEPS (default) or capi.LANS_PIPELINED."""
+        capi.check(self._lib.lancet_lans_plan_set_schedule(self._h, int(schedule)), "lancet_lans_plan_set_schedule")
+
+    def error(self):
+        err = C.c_int(-1)
+        capi.check(self._lib.lancet_lans_plan_error(self._h, _stream(), C.byref(err)), "lancet_lans_plan_error")
+        return err.value
 
     def close(self):
         if self._h is not None:

@@ -156,3 +156,52 @@ def test_op_layer_errors_are_reported_not_fatal(pkg):
         assert rc == 0 and lib.raf_hip_dispatch(h) != 0
         assert b"Cannot find a valid dispatch" in lib.raf_hip_last_error()
         lib.raf_hip_call_destroy(h)
+
+
+# ----------------------------------------------------------------------------- LANS task queue
+def _task_queue(pkg, numels):
+    import numpy as np
+    lib = pkg.capi.load()
+    arr = (C.c_int64 * len(numels))(*numels)
+    n = lib.lancet_lans_debug_task_queue(arr, len(numels), None, None, 0)
+    tasks = np.empty(n, np.uint32)
+    ctensor = np.empty(max(n // 3, 1), np.int32)
+    assert lib.lancet_lans_debug_task_queue(arr, len(numels), tasks.ctypes.data_as(C.c_void_p),
+                                            ctensor.ctypes.data_as(C.c_void_p), n) == n
+    return tasks, ctensor[:n // 3]
+
+
+@pytest.mark.parametrize("case", ["config5", "random", "tiny", "one_big"])
+def test_lans_task_queue_never_waits_on_a_later_task(pkg, case):
+    """The persistent LANS kernel is deadlock-free iff every task of phase k of a tensor comes before
+    every task of phase k+1 of the same tensor (a waiting task then only waits for tasks that running
+    workgroups already took) and every (phase, chunk) pair appears exactly once."""
+    import numpy as np
+    import bench
+    rng = np.random.default_rng(0)
+    if case == "config5":
+        numels = [int(np.prod(s)) for s in bench.lans_shapes()]
+    elif case == "random":
+        numels = [int(x) for x in rng.integers(0, 3_000_000, 200)] + [0, 1, 8192, 8193]
+    elif case == "tiny":
+        numels = [1, 2, 3]
+    else:
+        numels = [50_000_000, 5, 9_000_000]
+    tasks, ctensor = _task_queue(pkg, numels)
+    nchunks = sum((n + 8191) // 8192 for n in numels)
+    assert len(tasks) == 3 * nchunks and len(ctensor) == nchunks
+    phase = (tasks >> 30).astype(np.int64)
+    chunk = (tasks & 0x3FFFFFFF).astype(np.int64)
+    assert chunk.max() < nchunks and phase.max() <= 2
+    assert len(np.unique(phase * nchunks + chunk)) == 3 * nchunks          # each pair exactly once
+    tensor = ctensor[chunk]
+    pos = np.arange(len(tasks))
+    T = len(numels)
+    last = np.full((3, T), -1, np.int64)
+    first = np.full((3, T), len(tasks), np.int64)
+    for ph in range(3):
+        sel = phase == ph
+        np.maximum.at(last[ph], tensor[sel], pos[sel])
+        np.minimum.at(first[ph], tensor[sel], pos[sel])
+    has = np.array([(n + 8191) // 8192 > 0 for n in numels])
+    assert (last[0][has] < first[1][has]).all() and (last[1][has] < first[2][has]).all()

@@ -126,3 +126,28 @@ def test_lans_norms_and_plan_reuse(pkg):
     for i in range(2):
         assert_close_scaled(to_np(dp[i]), p[i], P_RTOL, "p[%d]" % i)
     plan.close()
+
+
+def test_lans_pipelined_schedule_gives_the_same_bits(pkg):
+    """The opt-in persistent-kernel schedule must terminate, leave its error word clear and
+    produce exactly what the default three-sweep schedule produces."""
+    capi = pkg.capi
+    numels = [1000, 70000, 5, 1 << 20, 3 * 8192, 8193, 1, (4 << 20) + 17, 1024, 1024, 2 << 20]
+    results = []
+    for schedule in (capi.LANS_SWEEPS, capi.LANS_PIPELINED):
+        gen = torch.Generator(device="cuda").manual_seed(7)
+        total = sum(numels)
+        flat = [torch.empty(total, device="cuda").normal_(0, s, generator=gen) for s in (1e-3, 0.02)]
+        flat += [torch.zeros(total, device="cuda") for _ in range(2)]
+        views = [list(torch.split(t, numels)) for t in flat]
+        plan = pkg.ops.LansPlan(numels, schedule=schedule)
+        hyper = capi.LansHyper(1e-3, 0.9, 0.999, 1e-6, 1, 0.01, 1, 1, 1)
+        for step in (1, 2, 3):
+            plan.step(*views, step, hyper)
+        torch.cuda.synchronize()
+        assert plan.error() == 0
+        results.append((flat, plan.norms()))
+        plan.close()
+    for a, b in zip(results[0][0], results[1][0]):
+        assert torch.equal(a, b)
+    assert torch.equal(results[0][1], results[1][1])

@@ -145,6 +145,35 @@ int lancet_moe_decode(const void* expert_out, const float* gates_s,
                       const int32_t* indices_locations, int64_t S, int64_t M, int64_t E,
                       int64_t C, int top_k, int dtype, void* out, lancet_stream_t stream);
 
+/* ---- backward ops (raf.op.moe_encode_dx / _dg, raf.op.moe_decode_dx / _dg) ------------------
+ * Gradients wired by src/op/grad/moe.cc:30-93.  Gate-side gradients are fp32 like gates_s; top_k = 2
+ * takes the slot-major layout of the forward ops.
+ *
+ * moe_encode_dx: dx[s,:] = sum over slots of dy[idx, loc, :] (0 for dropped slots).  Replaces
+ * MoeEncodeDx / launch_encode_backward_data (moe.cc:1075-1153; kernel_util.cuh:41;
+ * tutel_moe_dispatch.cu:88-94,486-497). */
+int lancet_moe_encode_dx(const void* dy, const int32_t* indices_locations, int64_t S, int64_t M,
+                         int64_t E, int64_t C, int top_k, int dtype, void* dx, lancet_stream_t stream);
+/* moe_encode_dg: grad_gates[S,E] = 0 except grad_gates[s, idx] = dy_gates_s of that slot.  Replaces
+ * MoeEncodeDg / launch_encode_backward_gate (moe.cc:1155-1225; kernel_util.cuh:43;
+ * tutel_moe_dispatch.cu:96-105,499-506). */
+int lancet_moe_encode_dg(const float* dy_gates_s, const int32_t* indices_locations, int64_t S,
+                         int64_t E, int top_k, float* grad_gates, lancet_stream_t stream);
+/* moe_decode_dx: grad_expert_out[idx, loc, :] = gates_s * dy[s, :], zero elsewhere.  Replaces
+ * MoeDecodeDx / launch_decode_backward_data (moe.cc:1313-1395; kernel_util.cuh:47;
+ * tutel_moe_dispatch.cu:118-124,523-533).  Workspace: an [E*C] int32 row -> token map. */
+size_t lancet_moe_decode_dx_workspace_bytes(int64_t E, int64_t C);
+int lancet_moe_decode_dx(const void* dy, const float* gates_s, const int32_t* indices_locations,
+                         int64_t S, int64_t M, int64_t E, int64_t C, int top_k, int dtype,
+                         void* grad_expert_out, void* workspace, size_t workspace_bytes,
+                         lancet_stream_t stream);
+/* moe_decode_dg: grad_gates_s[slot-token] = <expert_out[idx, loc, :], dy[s, :]>, 0 for dropped slots.
+ * Replaces MoeDecodeDg / launch_decode_backward_gate (moe.cc:1397-1481; kernel_util.cuh:49;
+ * tutel_moe_dispatch.cu:126-157,535-546). */
+int lancet_moe_decode_dg(const void* dy, const void* expert_out, const int32_t* indices_locations,
+                         int64_t S, int64_t M, int64_t E, int64_t C, int top_k, int dtype,
+                         float* grad_gates_s, lancet_stream_t stream);
+
 /* Combine weights of the top-2 extension from raw per-slot gate values and merged indices
  * (docker/resources/sharded_moe.py:304-312); in place when gates_out == raw_gates. */
 int lancet_moe_top2_normalize_gates(const float* raw_gates, const int32_t* merged_indices,

@@ -235,6 +235,70 @@ extern "C" int lancet_moe_decode(const void* expert_out, const float* gates_s, c
                             S_(stream)));
 }
 
+// ---- backward ops -------------------------------------------------------------------
+extern "C" int lancet_moe_encode_dx(const void* dy, const int32_t* indices_locations, int64_t S, int64_t M,
+                                    int64_t E, int64_t C, int top_k, int dtype, void* dx, lancet_stream_t stream) {
+  if ((!dy && C > 0 && M > 0) || (!indices_locations && S > 0) || (!dx && S > 0 && M > 0)) return LANCET_ERR_NULL;
+  const int eb = elem_bytes(dtype);
+  if (!eb) return LANCET_ERR_DTYPE;
+  if (int r = check_dims(S, M, E, C)) return r;
+  if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
+  if (misaligned(dy, eb) || misaligned(dx, eb) || misaligned(indices_locations, 4)) return LANCET_ERR_ALIGN;
+  const int s = static_cast<int>(S);
+  return rc(run_decode_rows(dy, nullptr, indices_locations, indices_locations + static_cast<size_t>(top_k) * s, dx, s,
+                            static_cast<int>(M), static_cast<int>(E), static_cast<int>(C), top_k, dtype, S_(stream)));
+}
+
+extern "C" int lancet_moe_encode_dg(const float* dy_gates_s, const int32_t* indices_locations, int64_t S, int64_t E,
+                                    int top_k, float* grad_gates, lancet_stream_t stream) {
+  if (S > 0 && (!dy_gates_s || !indices_locations || !grad_gates)) return LANCET_ERR_NULL;
+  if (int r = check_dims(S, 0, E, 0)) return r;
+  if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
+  if (misaligned(dy_gates_s, 4) || misaligned(indices_locations, 4) || misaligned(grad_gates, 4)) return LANCET_ERR_ALIGN;
+  return rc(run_encode_dg(dy_gates_s, indices_locations, static_cast<int>(S), static_cast<int>(E), top_k, grad_gates,
+                          S_(stream)));
+}
+
+extern "C" size_t lancet_moe_decode_dx_workspace_bytes(int64_t E, int64_t C) {
+  if (E < 1 || C < 0) return 0;
+  return static_cast<size_t>(E) * static_cast<size_t>(C) * sizeof(int32_t);
+}
+
+extern "C" int lancet_moe_decode_dx(const void* dy, const float* gates_s, const int32_t* indices_locations, int64_t S,
+                                    int64_t M, int64_t E, int64_t C, int top_k, int dtype, void* grad_expert_out,
+                                    void* workspace, size_t workspace_bytes, lancet_stream_t stream) {
+  if (((!dy && M > 0) || !gates_s || !indices_locations) && S > 0) return LANCET_ERR_NULL;
+  if (!grad_expert_out && C > 0 && M > 0) return LANCET_ERR_NULL;
+  const int eb = elem_bytes(dtype);
+  if (!eb) return LANCET_ERR_DTYPE;
+  if (int r = check_dims(S, M, E, C)) return r;
+  if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
+  if (C > 0 && (!workspace || workspace_bytes < lancet_moe_decode_dx_workspace_bytes(E, C))) return LANCET_ERR_WORKSPACE;
+  if (misaligned(dy, eb) || misaligned(grad_expert_out, eb) || misaligned(gates_s, 4) ||
+      misaligned(indices_locations, 4) || misaligned(workspace, 4))
+    return LANCET_ERR_ALIGN;
+  const int s = static_cast<int>(S);
+  return rc(run_decode_dx(dy, gates_s, indices_locations, indices_locations + static_cast<size_t>(top_k) * s,
+                          grad_expert_out, static_cast<int32_t*>(workspace), s, static_cast<int>(M),
+                          static_cast<int>(E), static_cast<int>(C), top_k, dtype, S_(stream)));
+}
+
+extern "C" int lancet_moe_decode_dg(const void* dy, const void* expert_out, const int32_t* indices_locations, int64_t S,
+                                    int64_t M, int64_t E, int64_t C, int top_k, int dtype, float* grad_gates_s,
+                                    lancet_stream_t stream) {
+  if (S > 0 && (!indices_locations || !grad_gates_s || ((!dy || !expert_out) && M > 0))) return LANCET_ERR_NULL;
+  const int eb = elem_bytes(dtype);
+  if (!eb) return LANCET_ERR_DTYPE;
+  if (int r = check_dims(S, M, E, C)) return r;
+  if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
+  if (misaligned(dy, eb) || misaligned(expert_out, eb) || misaligned(grad_gates_s, 4) || misaligned(indices_locations, 4))
+    return LANCET_ERR_ALIGN;
+  const int s = static_cast<int>(S);
+  return rc(run_decode_dg(dy, expert_out, indices_locations, indices_locations + static_cast<size_t>(top_k) * s,
+                          grad_gates_s, s, static_cast<int>(M), static_cast<int>(E), static_cast<int>(C), top_k, dtype,
+                          S_(stream)));
+}
+
 extern "C" int lancet_moe_top2_normalize_gates(const float* raw_gates, const int32_t* merged_indices, int64_t S,
                                                float* gates_out, lancet_stream_t stream) {
   if (S < 0 || S > 0x3fffffff) return LANCET_ERR_SHAPE;

@@ -45,6 +45,13 @@ hipError_t run_decode_rows(const void* expert_out, const float* gates, const int
                            const int32_t* loc, void* out, int S, int M, int E, int C, int K,
                            int dtype, hipStream_t st);
 
+// backward (gates == nullptr in run_decode_rows gives moe_encode_dx)
+hipError_t run_encode_dg(const float* dy, const int32_t* idx, int S, int E, int K, float* grad_gates, hipStream_t st);
+hipError_t run_decode_dx(const void* dy, const float* gates, const int32_t* idx, const int32_t* loc, void* out,
+                         int32_t* src_map, int S, int M, int E, int C, int K, int dtype, hipStream_t st);
+hipError_t run_decode_dg(const void* dy, const void* expert_out, const int32_t* idx, const int32_t* loc, float* out,
+                         int S, int M, int E, int C, int K, int dtype, hipStream_t st);
+
 struct PtrTable {
   const void* p[kMaxPartitions];
 };

@@ -171,7 +171,7 @@ __device__ __forceinline__ u32x4 combine_vec(const u32x4 (&x)[K], const float (&
 
 struct DecodeArgs {
   const void* expert_out;
-  const float* gates;    // [K*S]
+  const float* gates;    // [K*S]; null = all ones (moe_encode_dx)
   const int32_t* idx;    // [K*S]
   const int32_t* loc;    // [K*S]
   void* out;             // [S, M]
@@ -194,7 +194,7 @@ __global__ __launch_bounds__(kTile) void decode_rows_kernel(DecodeArgs a) {
     const int e = a.idx[static_cast<size_t>(j) * a.S + s];
     const int l = a.loc[static_cast<size_t>(j) * a.S + s];
     ok[j] = e >= 0 && e < a.E && l >= 0 && l < a.C;
-    g[j] = ok[j] ? a.gates[static_cast<size_t>(j) * a.S + s] : 0.f;
+    g[j] = ok[j] ? (a.gates ? a.gates[static_cast<size_t>(j) * a.S + s] : 1.f) : 0.f;
     row[j] = ok[j] ? (static_cast<size_t>(e) * a.C + l) : 0;
     any = any || ok[j];
   }
@@ -325,6 +325,126 @@ __global__ __launch_bounds__(kTile) void redispatch_rows_kernel(PtrTable bufs, i
     const V z = zero_v<V>();
     for (int v = lane; v < row_vecs; v += kWave) stv(dst + v, z);
   }
+}
+
+// ---------------------------------------------------------------------------------------
+// backward kernels.  moe_encode_dx is decode_rows_kernel with unit gates
+// (encode_backward_data_kernel, tutel_moe_dispatch.cu:88-94).
+// ---------------------------------------------------------------------------------------
+// grad_gates[s, e] = dy[j*S+s] where e is token s's expert in slot j, else 0: the memset + scatter of
+// encode_backward_gate_kernel (tutel_moe_dispatch.cu:96-105, 499-506) as one pass that writes every
+// element once.
+template <int K>
+__global__ __launch_bounds__(kTile) void encode_dg_kernel(const float* dy, const int32_t* idx, int S, int E,
+                                                          float* grad_gates) {
+  const size_t n = static_cast<size_t>(S) * E;
+  for (size_t i = blockIdx.x * static_cast<size_t>(kTile) + threadIdx.x; i < n;
+       i += static_cast<size_t>(gridDim.x) * kTile) {
+    const int s = static_cast<int>(i / E);
+    const int e = static_cast<int>(i - static_cast<size_t>(s) * E);
+    float v = 0.f;
+    if (idx[s] == e) v = dy[s];
+    if (K == 2 && idx[S + s] == e) v = dy[S + s];
+    grad_gates[i] = v;
+  }
+}
+
+// src[e*C + l] = slot-token id (j*S + s) of the token that owns row (e, l); src is -1 elsewhere.
+__global__ __launch_bounds__(kTile) void inverse_map_kernel(const int32_t* idx, const int32_t* loc, int n, int E,
+                                                            int C, int32_t* src) {
+  const int i = blockIdx.x * kTile + threadIdx.x;
+  if (i >= n) return;
+  const int e = idx[i], l = loc[i];
+  if (e >= 0 && e < E && l >= 0 && l < C) src[static_cast<size_t>(e) * C + l] = i;
+}
+
+// grad_expert_out[e, l, :] = gates[i] * dy[s, :] for the slot-token i = src[e*C+l] (s = i mod S), zero
+// for rows nobody owns: decode_backward_data_kernel (tutel_moe_dispatch.cu:118-124, 523-533) without
+// the memset + atomicAdd; every output byte is written once.
+template <int DT, bool VEC>
+__global__ __launch_bounds__(kTile) void decode_dx_rows_kernel(const void* dy, const float* gates,
+                                                               const int32_t* src, void* out, int S, int M,
+                                                               long rows) {
+  typedef Codec<DT> Cd;
+  const int w = threadIdx.x / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  const long r = static_cast<long>(blockIdx.x) * kRowsPerBlock + w;
+  if (r >= rows) return;
+  const int i = src[r];
+  const float g1[1] = {i >= 0 ? gates[i] : 0.f};
+  const size_t s = i >= 0 ? static_cast<size_t>(i % S) : 0;
+  if (VEC) {
+    const int row_vecs = M / Cd::kPerVec;
+    u32x4* dst = static_cast<u32x4*>(out) + static_cast<size_t>(r) * row_vecs;
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    if (i < 0) {
+      for (int v = lane; v < row_vecs; v += kWave) st_stream(dst + v, z);
+      return;
+    }
+    const u32x4* sp = static_cast<const u32x4*>(dy) + s * row_vecs;
+    int v = lane;
+    for (; v + kWave < row_vecs; v += 2 * kWave) {
+      const u32x4 xa[1] = {ld_stream(sp + v)};
+      const u32x4 xb[1] = {ld_stream(sp + v + kWave)};
+      st_stream(dst + v, combine_vec<DT, 1>(xa, g1));
+      st_stream(dst + v + kWave, combine_vec<DT, 1>(xb, g1));
+    }
+    for (; v < row_vecs; v += kWave) {
+      const u32x4 xa[1] = {ld_stream(sp + v)};
+      st_stream(dst + v, combine_vec<DT, 1>(xa, g1));
+    }
+  } else {
+    typedef typename Cd::S St;
+    St* dst = static_cast<St*>(out) + static_cast<size_t>(r) * M;
+    const St* sp = static_cast<const St*>(dy) + s * M;
+    for (int k = lane; k < M; k += kWave) dst[k] = i >= 0 ? Cd::put(mul_rn(g1[0], Cd::get(sp[k]))) : Cd::put(0.f);
+  }
+}
+
+// grad_gates_s[i] = <expert_out[idx, loc, :], dy[s, :]> for slot-token i, 0 when the slot is dropped
+// (decode_backward_gate_kernel, tutel_moe_dispatch.cu:126-157): one wave per slot-token, fp32 partial
+// sums per lane, xor-tree over the wave.
+template <int DT, bool VEC>
+__global__ __launch_bounds__(kTile) void decode_dg_kernel(const void* dy, const void* expert_out,
+                                                          const int32_t* idx, const int32_t* loc, float* out,
+                                                          int S, int M, int E, int C, int n) {
+  typedef Codec<DT> Cd;
+  const int w = threadIdx.x / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int i = blockIdx.x * kRowsPerBlock + w;
+  if (i >= n) return;
+  const int e = idx[i], l = loc[i];
+  if (!(e >= 0 && e < E && l >= 0 && l < C)) {
+    if (lane == 0) out[i] = 0.f;
+    return;
+  }
+  const size_t s = static_cast<size_t>(i % S);
+  const size_t row = static_cast<size_t>(e) * C + l;
+  float acc = 0.f;
+  if (VEC) {
+    const int row_vecs = M / Cd::kPerVec;
+    const u32x4* a = static_cast<const u32x4*>(expert_out) + row * row_vecs;
+    const u32x4* b = static_cast<const u32x4*>(dy) + s * row_vecs;
+    for (int v = lane; v < row_vecs; v += kWave) {
+      const u32x4 x = ld_stream(a + v), y = ld_stream(b + v);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (Cd::kPerVec == 4) {
+          acc += Cd::get(x[k]) * Cd::get(y[k]);
+        } else {
+          acc += Cd::get(static_cast<typename Cd::S>(x[k] & 0xffffu)) * Cd::get(static_cast<typename Cd::S>(y[k] & 0xffffu));
+          acc += Cd::get(static_cast<typename Cd::S>(x[k] >> 16)) * Cd::get(static_cast<typename Cd::S>(y[k] >> 16));
+        }
+      }
+    }
+  } else {
+    typedef typename Cd::S St;
+    const St* a = static_cast<const St*>(expert_out) + row * M;
+    const St* b = static_cast<const St*>(dy) + s * M;
+    for (int k = lane; k < M; k += kWave) acc += Cd::get(a[k]) * Cd::get(b[k]);
+  }
+  acc = wave_sum(acc);
+  if (lane == 0) out[i] = acc;
 }
 
 // ---------------------------------------------------------------------------------------
@@ -462,6 +582,67 @@ hipError_t run_redispatch_rows(const PtrTable& bufs, int P, int M, int C, int E,
     redispatch_rows_kernel<uint16_t><<<blocks, kTile, 0, st>>>(bufs, P, E, C, M, counts,
                                                                static_cast<uint16_t*>(out));
   return hipGetLastError();
+}
+
+hipError_t run_encode_dg(const float* dy, const int32_t* idx, int S, int E, int K, float* grad_gates, hipStream_t st) {
+  const size_t n = static_cast<size_t>(S) * E;
+  if (n == 0) return hipSuccess;
+  const int blocks = static_cast<int>(std::min<size_t>((n + kTile - 1) / kTile, 65536));
+  if (K == 1) encode_dg_kernel<1><<<blocks, kTile, 0, st>>>(dy, idx, S, E, grad_gates);
+  else encode_dg_kernel<2><<<blocks, kTile, 0, st>>>(dy, idx, S, E, grad_gates);
+  return hipGetLastError();
+}
+
+template <int DT>
+static hipError_t decode_dx_launch(const void* dy, const float* gates, const int32_t* src, void* out, int S, int M,
+                                   long rows, bool vec, hipStream_t st) {
+  const unsigned blocks = static_cast<unsigned>((rows + kRowsPerBlock - 1) / kRowsPerBlock);
+  if (vec) decode_dx_rows_kernel<DT, true><<<blocks, kTile, 0, st>>>(dy, gates, src, out, S, M, rows);
+  else decode_dx_rows_kernel<DT, false><<<blocks, kTile, 0, st>>>(dy, gates, src, out, S, M, rows);
+  return hipGetLastError();
+}
+
+hipError_t run_decode_dx(const void* dy, const float* gates, const int32_t* idx, const int32_t* loc, void* out,
+                         int32_t* src_map, int S, int M, int E, int C, int K, int dtype, hipStream_t st) {
+  const long rows = static_cast<long>(E) * C;
+  if (rows == 0 || M == 0) return hipSuccess;
+  hipError_t err = run_fill_u32(reinterpret_cast<uint32_t*>(src_map), static_cast<size_t>(rows), 0xffffffffu, st);
+  if (err != hipSuccess) return err;
+  const int n = K * S;
+  if (n > 0) {
+    inverse_map_kernel<<<(n + kTile - 1) / kTile, kTile, 0, st>>>(idx, loc, n, E, C, src_map);
+    err = hipGetLastError();
+    if (err != hipSuccess) return err;
+  }
+  const int per_vec = (dtype == LANCET_F32) ? 4 : 8;
+  const bool vec = (M % per_vec == 0) && aligned16(dy) && aligned16(out);
+  switch (dtype) {
+    case LANCET_F32: return decode_dx_launch<LANCET_F32>(dy, gates, src_map, out, S, M, rows, vec, st);
+    case LANCET_BF16: return decode_dx_launch<LANCET_BF16>(dy, gates, src_map, out, S, M, rows, vec, st);
+    default: return decode_dx_launch<LANCET_F16>(dy, gates, src_map, out, S, M, rows, vec, st);
+  }
+}
+
+template <int DT>
+static hipError_t decode_dg_launch(const void* dy, const void* expert_out, const int32_t* idx, const int32_t* loc,
+                                   float* out, int S, int M, int E, int C, int n, bool vec, hipStream_t st) {
+  const int blocks = (n + kRowsPerBlock - 1) / kRowsPerBlock;
+  if (vec) decode_dg_kernel<DT, true><<<blocks, kTile, 0, st>>>(dy, expert_out, idx, loc, out, S, M, E, C, n);
+  else decode_dg_kernel<DT, false><<<blocks, kTile, 0, st>>>(dy, expert_out, idx, loc, out, S, M, E, C, n);
+  return hipGetLastError();
+}
+
+hipError_t run_decode_dg(const void* dy, const void* expert_out, const int32_t* idx, const int32_t* loc, float* out,
+                         int S, int M, int E, int C, int K, int dtype, hipStream_t st) {
+  const int n = K * S;
+  if (n == 0) return hipSuccess;
+  const int per_vec = (dtype == LANCET_F32) ? 4 : 8;
+  const bool vec = (M % per_vec == 0) && aligned16(dy) && aligned16(expert_out);
+  switch (dtype) {
+    case LANCET_F32: return decode_dg_launch<LANCET_F32>(dy, expert_out, idx, loc, out, S, M, E, C, n, vec, st);
+    case LANCET_BF16: return decode_dg_launch<LANCET_BF16>(dy, expert_out, idx, loc, out, S, M, E, C, n, vec, st);
+    default: return decode_dg_launch<LANCET_F16>(dy, expert_out, idx, loc, out, S, M, E, C, n, vec, st);
+  }
 }
 
 }  // namespace lancet

@@ -1,4 +1,5 @@
-"""The six RAF operators of the dispatch/optimizer path over torch tensors on the GPU.
+"""The RAF operators of the dispatch/optimizer path (six forward ops, four MoE backward ops) over
+torch tensors on the GPU.
 
 Names, positional argument order and defaults follow the reference's schemas
 (scripts/src_codegen/def_schema.py:642-698, 726-742); output tuples follow
@@ -155,6 +156,78 @@ def moe_decode(data, gate, indices_locations, top_k=1, out=None):
     st = lib.lancet_moe_decode(_p(data), _p(gate), _p(indices_locations), S, M, E, Cap, top_k, dt, _p(out),
                                _stream())
     capi.check(st, "lancet_moe_decode")
+    return out
+
+
+def _check_indloc(indices_locations, top_k):
+    _dev(indices_locations, "indices_locations")
+    _need(indices_locations.dtype == torch.int32 and indices_locations.dim() == 2 and indices_locations.shape[0] == 2,
+          "indices_locations must be int32 [2, k*S]")
+    _need(top_k in (1, 2) and indices_locations.shape[1] % top_k == 0, "top_k must be 1 or 2 and divide the mask length")
+    return indices_locations.shape[1] // top_k
+
+
+def moe_encode_dx(dy, indices_locations, top_k=1, out=None):
+    """raf.op.moe_encode_dx(dy [E,C,M], indices_locations [2, k*S]) -> [S, M]."""
+    lib = capi.load()
+    _dev(dy, "dy")
+    _need(dy.dim() == 3, "Input dy should be 3-D.")
+    S = _check_indloc(indices_locations, top_k)
+    E, Cap, M = dy.shape
+    if out is None:
+        out = torch.empty((S, M), dtype=dy.dtype, device=dy.device)
+    st = lib.lancet_moe_encode_dx(_p(dy), _p(indices_locations), S, M, E, Cap, top_k, _dtype_code(dy), _p(out), _stream())
+    capi.check(st, "lancet_moe_encode_dx")
+    return out
+
+
+def moe_encode_dg(dy, indices_locations, n_experts, top_k=1, out=None):
+    """raf.op.moe_encode_dg(dy [k*S] f32, indices_locations, n_experts) -> [S, E] f32."""
+    lib = capi.load()
+    _dev(dy, "dy")
+    _need(dy.dim() == 1 and dy.dtype == torch.float32, "Input dy should be 1-D float32.")
+    S = _check_indloc(indices_locations, top_k)
+    _need(dy.shape[0] == top_k * S, "dy and indices_locations disagree")
+    if out is None:
+        out = torch.empty((S, n_experts), dtype=torch.float32, device=dy.device)
+    st = lib.lancet_moe_encode_dg(_p(dy), _p(indices_locations), S, n_experts, top_k, _p(out), _stream())
+    capi.check(st, "lancet_moe_encode_dg")
+    return out
+
+
+def moe_decode_dx(dy, gate, indices_locations, n_experts, capacity, top_k=1, workspace=None, out=None):
+    """raf.op.moe_decode_dx(dy [S,M], gate [k*S] f32, indices_locations, n_experts, capacity) -> [E, C, M]."""
+    lib = capi.load()
+    _dev(dy, "dy"), _dev(gate, "gate")
+    _need(dy.dim() == 2, "Input dy should be 2-D.")
+    _need(gate.dim() == 1 and gate.dtype == torch.float32, "gate must be 1-D float32")
+    S = _check_indloc(indices_locations, top_k)
+    _need(dy.shape[0] == S and gate.shape[0] == top_k * S, "dy, gate and indices_locations disagree")
+    M = dy.shape[1]
+    if out is None:
+        out = torch.empty((n_experts, capacity, M), dtype=dy.dtype, device=dy.device)
+    ws_bytes = int(lib.lancet_moe_decode_dx_workspace_bytes(n_experts, capacity))
+    ws = _workspace(ws_bytes, dy.device, workspace)
+    st = lib.lancet_moe_decode_dx(_p(dy), _p(gate), _p(indices_locations), S, M, n_experts, capacity, top_k,
+                                  _dtype_code(dy), _p(out), _p(ws), ws.numel(), _stream())
+    capi.check(st, "lancet_moe_decode_dx")
+    return out
+
+
+def moe_decode_dg(dy, data, indices_locations, top_k=1, out=None):
+    """raf.op.moe_decode_dg(dy [S,M], data [E,C,M], indices_locations) -> [k*S] f32."""
+    lib = capi.load()
+    _dev(dy, "dy"), _dev(data, "data")
+    _need(dy.dim() == 2 and data.dim() == 3 and dy.dtype == data.dtype and dy.shape[1] == data.shape[2],
+          "dy must be [S,M] and data [E,C,M] of one dtype")
+    S = _check_indloc(indices_locations, top_k)
+    _need(dy.shape[0] == S, "dy and indices_locations disagree")
+    E, Cap, M = data.shape
+    if out is None:
+        out = torch.empty(top_k * S, dtype=torch.float32, device=dy.device)
+    st = lib.lancet_moe_decode_dg(_p(dy), _p(data), _p(indices_locations), S, M, E, Cap, top_k, _dtype_code(dy),
+                                  _p(out), _stream())
+    capi.check(st, "lancet_moe_decode_dg")
     return out
 
 

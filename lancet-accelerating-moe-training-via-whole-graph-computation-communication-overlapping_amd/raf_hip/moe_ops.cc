@@ -391,6 +391,185 @@ class MoeDecode : public OpEnv {
   int top_k_, dtype_, device_id_;
 };
 
+// =====================================================================================
+// backward ops: raf.op.moe_encode_dx / moe_encode_dg / moe_decode_dx / moe_decode_dg
+// (src/op/declare/moe.cc:165-247; src/op/dialect/cuda/moe.cc:1075-1225, 1313-1481; gradients wired in
+// src/op/grad/moe.cc:30-93).  Gate-side tensors are float32; an optional trailing top_k selects the
+// slot-major two-slot layout.
+// =====================================================================================
+namespace {
+int64_t MaskTokens(const Tensor& il, int64_t k) {
+  RAF_CHECK(IsI32(il.dtype) && il.shape.size() == 2 && il.shape[0] == 2, "Input indices_locations should be int32 [2, k*S].");
+  RAF_CHECK(k == 1 || k == 2, "top_k must be 1 or 2");
+  RAF_CHECK(il.shape[1] % k == 0, "mask length must be a multiple of top_k");
+  return il.shape[1] / k;
+}
+}  // namespace
+
+void MoeEncodeDxDeclare(CallValues& call) {
+  RAF_CHECK(call.args.size() >= 2, "moe_encode_dx(dy, indices_locations)");
+  const Tensor& dy = call.args[0].AsTensor();
+  RAF_CHECK(dy.shape.size() == 3, "Input dy should be 3-D.");
+  DTypeToLancet(dy.dtype);
+  const int64_t S = MaskTokens(call.args[1].AsTensor(), OptInt(call, 2, 1));
+  call.out = Value::MakeTensor(MakeOut(dy.device_id, dy.dtype.code, dy.dtype.bits, {S, dy.shape[2]}));
+  call.device_id = dy.device_id;
+}
+
+class MoeEncodeDx : public OpEnv {
+ public:
+  explicit MoeEncodeDx(const CallValues& cv) {
+    const Tensor& dy = cv.args[0].AsTensor();
+    RAF_CHECK(dy.shape.size() == 3, "Expected input dy to be 3D.");
+    top_k_ = static_cast<int>(OptInt(cv, 2, 1));
+    dim_S_ = MaskTokens(cv.args[1].AsTensor(), top_k_);
+    dim_E_ = dy.shape[0], dim_C_ = dy.shape[1], dim_M_ = dy.shape[2];
+    dtype_ = DTypeToLancet(dy.dtype);
+    device_id_ = dy.device_id;
+    this->arg_indices = {0, 1};
+  }
+  void Execute(const CallValues& cv) override { Execute({cv.args[0], cv.args[1]}, cv.out); }
+  void Execute(const std::vector<Value>& inputs, Value output) override {
+    CheckStatus(lancet_moe_encode_dx(inputs[0].AsTensor().data, static_cast<const int32_t*>(inputs[1].AsTensor().data),
+                                     dim_S_, dim_M_, dim_E_, dim_C_, top_k_, dtype_, output.AsTensor().data,
+                                     GetStream(device_id_)),
+                "lancet_moe_encode_dx");
+  }
+  std::string name() const override { return "raf.op.hip.moe_encode_dx"; }
+  static OpEnv* make(const CallValues& cv) { return new MoeEncodeDx(cv); }
+
+ private:
+  int64_t dim_S_, dim_E_, dim_C_, dim_M_;
+  int top_k_, dtype_, device_id_;
+};
+
+void MoeEncodeDgDeclare(CallValues& call) {
+  RAF_CHECK(call.args.size() >= 3, "moe_encode_dg(dy, indices_locations, n_experts)");
+  const Tensor& dy = call.args[0].AsTensor();
+  RAF_CHECK(dy.shape.size() == 1, "Input dy should be 1-D.");
+  RAF_CHECK(IsF32(dy.dtype), "dy of moe_encode_dg must be float32 in the hip dialect");
+  const int64_t S = MaskTokens(call.args[1].AsTensor(), OptInt(call, 3, 1));
+  call.out = Value::MakeTensor(MakeOut(dy.device_id, DTypeCode::kFloat, 32, {S, call.args[2].AsInt()}));
+  call.device_id = dy.device_id;
+}
+
+class MoeEncodeDg : public OpEnv {
+ public:
+  explicit MoeEncodeDg(const CallValues& cv) {
+    const Tensor& dy = cv.args[0].AsTensor();
+    RAF_CHECK(dy.shape.size() == 1 && IsF32(dy.dtype), "Expected input dy to be 1D float32.");
+    top_k_ = static_cast<int>(OptInt(cv, 3, 1));
+    dim_S_ = MaskTokens(cv.args[1].AsTensor(), top_k_);
+    RAF_CHECK(dy.shape[0] == dim_S_ * top_k_, "dy and indices_locations disagree");
+    dim_E_ = cv.args[2].AsInt();
+    device_id_ = dy.device_id;
+    this->arg_indices = {0, 1};
+  }
+  void Execute(const CallValues& cv) override { Execute({cv.args[0], cv.args[1]}, cv.out); }
+  void Execute(const std::vector<Value>& inputs, Value output) override {
+    CheckStatus(lancet_moe_encode_dg(static_cast<const float*>(inputs[0].AsTensor().data),
+                                     static_cast<const int32_t*>(inputs[1].AsTensor().data), dim_S_, dim_E_, top_k_,
+                                     static_cast<float*>(output.AsTensor().data), GetStream(device_id_)),
+                "lancet_moe_encode_dg");
+  }
+  std::string name() const override { return "raf.op.hip.moe_encode_dg"; }
+  static OpEnv* make(const CallValues& cv) { return new MoeEncodeDg(cv); }
+
+ private:
+  int64_t dim_S_, dim_E_;
+  int top_k_, device_id_;
+};
+
+void MoeDecodeDxDeclare(CallValues& call) {
+  RAF_CHECK(call.args.size() >= 5, "moe_decode_dx(dy, gate, indices_locations, n_experts, capacity)");
+  const Tensor& dy = call.args[0].AsTensor();
+  RAF_CHECK(dy.shape.size() == 2, "Input dy should be 2-D.");
+  DTypeToLancet(dy.dtype);
+  call.out = Value::MakeTensor(MakeOut(dy.device_id, dy.dtype.code, dy.dtype.bits,
+                                       {call.args[3].AsInt(), call.args[4].AsInt(), dy.shape[1]}));
+  call.device_id = dy.device_id;
+}
+
+class MoeDecodeDx : public OpEnv {
+ public:
+  explicit MoeDecodeDx(const CallValues& cv) {
+    const Tensor& dy = cv.args[0].AsTensor();
+    const Tensor& gate = cv.args[1].AsTensor();
+    RAF_CHECK(dy.shape.size() == 2, "Expected input dy to be 2D.");
+    RAF_CHECK(gate.shape.size() == 1 && IsF32(gate.dtype), "Expected input gate to be 1D float32.");
+    top_k_ = static_cast<int>(OptInt(cv, 5, 1));
+    dim_S_ = MaskTokens(cv.args[2].AsTensor(), top_k_);
+    RAF_CHECK(dy.shape[0] == dim_S_ && gate.shape[0] == dim_S_ * top_k_, "dy, gate and indices_locations disagree");
+    dim_M_ = dy.shape[1];
+    dim_E_ = cv.args[3].AsInt();
+    dim_C_ = cv.args[4].AsInt();
+    dtype_ = DTypeToLancet(dy.dtype);
+    device_id_ = dy.device_id;
+    ws_bytes_ = lancet_moe_decode_dx_workspace_bytes(dim_E_, dim_C_);
+    RequestWorkspace(&ws_, device_id_, static_cast<int64_t>(ws_bytes_));
+    this->arg_indices = {0, 1, 2};
+  }
+  void Execute(const CallValues& cv) override { Execute({cv.args[0], cv.args[1], cv.args[2]}, cv.out); }
+  void Execute(const std::vector<Value>& inputs, Value output) override {
+    CheckStatus(lancet_moe_decode_dx(inputs[0].AsTensor().data, static_cast<const float*>(inputs[1].AsTensor().data),
+                                     static_cast<const int32_t*>(inputs[2].AsTensor().data), dim_S_, dim_M_, dim_E_,
+                                     dim_C_, top_k_, dtype_, output.AsTensor().data, ws_, ws_bytes_,
+                                     GetStream(device_id_)),
+                "lancet_moe_decode_dx");
+  }
+  std::string name() const override { return "raf.op.hip.moe_decode_dx"; }
+  static OpEnv* make(const CallValues& cv) { return new MoeDecodeDx(cv); }
+
+ private:
+  int64_t dim_S_, dim_E_, dim_C_, dim_M_;
+  int top_k_, dtype_, device_id_;
+  void* ws_ = nullptr;
+  size_t ws_bytes_ = 0;
+};
+
+void MoeDecodeDgDeclare(CallValues& call) {
+  RAF_CHECK(call.args.size() >= 3, "moe_decode_dg(dy, data, indices_locations)");
+  const Tensor& dy = call.args[0].AsTensor();
+  RAF_CHECK(dy.shape.size() == 2, "Input dy should be 2-D.");
+  DTypeToLancet(dy.dtype);
+  const int64_t k = OptInt(call, 3, 1);
+  const int64_t S = MaskTokens(call.args[2].AsTensor(), k);
+  call.out = Value::MakeTensor(MakeOut(dy.device_id, DTypeCode::kFloat, 32, {k * S}));
+  call.device_id = dy.device_id;
+}
+
+class MoeDecodeDg : public OpEnv {
+ public:
+  explicit MoeDecodeDg(const CallValues& cv) {
+    const Tensor& dy = cv.args[0].AsTensor();
+    const Tensor& data = cv.args[1].AsTensor();
+    RAF_CHECK(dy.shape.size() == 2, "Expected input dy to be 2D.");
+    RAF_CHECK(data.shape.size() == 3, "Expected input data to be 3D.");
+    RAF_CHECK(dy.dtype == data.dtype && dy.shape[1] == data.shape[2], "dy and data must agree in dtype and model dim");
+    top_k_ = static_cast<int>(OptInt(cv, 3, 1));
+    dim_S_ = MaskTokens(cv.args[2].AsTensor(), top_k_);
+    RAF_CHECK(dy.shape[0] == dim_S_, "dy and indices_locations disagree");
+    dim_E_ = data.shape[0], dim_C_ = data.shape[1], dim_M_ = data.shape[2];
+    dtype_ = DTypeToLancet(dy.dtype);
+    device_id_ = dy.device_id;
+    this->arg_indices = {0, 1, 2};
+  }
+  void Execute(const CallValues& cv) override { Execute({cv.args[0], cv.args[1], cv.args[2]}, cv.out); }
+  void Execute(const std::vector<Value>& inputs, Value output) override {
+    CheckStatus(lancet_moe_decode_dg(inputs[0].AsTensor().data, inputs[1].AsTensor().data,
+                                     static_cast<const int32_t*>(inputs[2].AsTensor().data), dim_S_, dim_M_, dim_E_,
+                                     dim_C_, top_k_, dtype_, static_cast<float*>(output.AsTensor().data),
+                                     GetStream(device_id_)),
+                "lancet_moe_decode_dg");
+  }
+  std::string name() const override { return "raf.op.hip.moe_decode_dg"; }
+  static OpEnv* make(const CallValues& cv) { return new MoeDecodeDg(cv); }
+
+ private:
+  int64_t dim_S_, dim_E_, dim_C_, dim_M_;
+  int top_k_, dtype_, device_id_;
+};
+
 // ---- registration (cuda/cuda_utils.cc:17; cuda/moe.cc:411-412,728-729,822-823,942-943,1310-1311) ----
 RAF_REGISTER_DIALECT("hip").set_enable("hip");
 
@@ -410,6 +589,19 @@ RAF_REGISTER_DIALECT_OP(hip, moe_redispatch, 20);
 RAF_OP_ENV_MAKER("raf.op.hip.moe_redispatch", MoeRedispatch::make);
 RAF_REGISTER_DIALECT_OP(hip, moe_decode, 20);
 RAF_OP_ENV_MAKER("raf.op.hip.moe_decode", MoeDecode::make);
+
+RAF_OP_DECLARE("raf.op.moe_encode_dx", MoeEncodeDxDeclare);
+RAF_OP_DECLARE("raf.op.moe_encode_dg", MoeEncodeDgDeclare);
+RAF_OP_DECLARE("raf.op.moe_decode_dx", MoeDecodeDxDeclare);
+RAF_OP_DECLARE("raf.op.moe_decode_dg", MoeDecodeDgDeclare);
+RAF_REGISTER_DIALECT_OP(hip, moe_encode_dx, 20);
+RAF_OP_ENV_MAKER("raf.op.hip.moe_encode_dx", MoeEncodeDx::make);
+RAF_REGISTER_DIALECT_OP(hip, moe_encode_dg, 20);
+RAF_OP_ENV_MAKER("raf.op.hip.moe_encode_dg", MoeEncodeDg::make);
+RAF_REGISTER_DIALECT_OP(hip, moe_decode_dx, 20);
+RAF_OP_ENV_MAKER("raf.op.hip.moe_decode_dx", MoeDecodeDx::make);
+RAF_REGISTER_DIALECT_OP(hip, moe_decode_dg, 20);
+RAF_OP_ENV_MAKER("raf.op.hip.moe_decode_dg", MoeDecodeDg::make);
 
 }  // namespace hip
 }  // namespace op

@@ -335,3 +335,57 @@ def bf16_bits_to_f32(b):
 def round_to_bf16(a):
     """fp32 -> nearest bf16 value, returned as fp32."""
     return bf16_bits_to_f32(f32_to_bf16_bits(a))
+
+
+# --------------------------------------------------------------------------
+# backward ops (gradients wired by src/op/grad/moe.cc:30-93)
+# Pinned in tests/test_oracle_moe.py against torch autograd of the dense einsum forms.
+# --------------------------------------------------------------------------
+def _valid(indloc, k, E, C):
+    idx, loc = indloc[0], indloc[1]
+    return (idx >= 0) & (idx < E) & (loc >= 0) & (loc < C)
+
+
+def moe_encode_dx(dy, indloc, k=1):
+    """dx[s] = sum over slots of dy[idx, loc] (encode_backward_data_kernel,
+    tutel_moe_dispatch.cu:46-55,88-94); products with the unit gate are exact."""
+    E, C, M = dy.shape
+    S = indloc.shape[1] // k
+    return moe_decode(dy, np.ones(k * S, np.float32), indloc, k=k)
+
+
+def moe_encode_dg(dy_gates_s, indloc, n_experts, k=1):
+    """grad_gates[S,E]: zero, then grad[s, idx] = dy (encode_backward_gate_kernel, :96-105,499-506)."""
+    S = indloc.shape[1] // k
+    out = np.zeros((S, n_experts), np.float32)
+    for j in range(k):
+        idx = indloc[0, j * S:(j + 1) * S]
+        ok = (idx >= 0) & (idx < n_experts)
+        out[np.arange(S)[ok], idx[ok]] = dy_gates_s[j * S:(j + 1) * S][ok]
+    return out
+
+
+def moe_decode_dx(dy, gates_s, indloc, n_experts, capacity, k=1, round_fn=None):
+    """grad_expert_out[idx, loc] = gates_s * dy[s], zero elsewhere (decode_backward_data_kernel,
+    :118-124,523-533: memset + atomicAdd onto distinct rows)."""
+    S, M = dy.shape
+    out = np.zeros((n_experts, capacity, M), np.float32)
+    ok = _valid(indloc, k, n_experts, capacity)
+    tok = np.tile(np.arange(S), k)
+    g = np.asarray(gates_s, np.float32)
+    out[indloc[0][ok], indloc[1][ok]] = _to_f32(dy)[tok[ok]] * g[ok, None]
+    return out if round_fn is None else round_fn(out)
+
+
+def moe_decode_dg(dy, expert_out, indloc, k=1):
+    """grad_gates_s[i] = <expert_out[idx, loc], dy[s]> (decode_backward_gate_kernel, :126-157), 0 for
+    dropped slots.  fp64 accumulation here; the device sums fp32 partials in a tree."""
+    E, C, M = expert_out.shape
+    S = dy.shape[0]
+    ok = _valid(indloc, k, E, C)
+    tok = np.tile(np.arange(S), k)
+    out = np.zeros(k * S, np.float64)
+    a = _to_f32(expert_out).astype(np.float64)
+    b = _to_f32(dy).astype(np.float64)
+    out[ok] = np.einsum("nm,nm->n", a[indloc[0][ok], indloc[1][ok]], b[tok[ok]])
+    return out.astype(np.float32)

@@ -97,7 +97,8 @@ F32, BF16, I32, U64 = (2, 32), (4, 16), (0, 32), (1, 64)
 def test_op_layer_registers_the_six_operators(pkg):
     rx = pkg.raf_executor
     ops = rx.registered_ops()
-    for name in ("moe_encode", "moe_encode_batch_prioritized", "moe_decode", "moe_merge_masks", "moe_redispatch", "lans"):
+    for name in ("moe_encode", "moe_encode_batch_prioritized", "moe_decode", "moe_merge_masks", "moe_redispatch", "lans",
+                 "moe_encode_dx", "moe_encode_dg", "moe_decode_dx", "moe_decode_dg"):
         assert "raf.op." + name in ops
         assert rx.dispatch_list("raf.op." + name) == [("raf.op.hip." + name, 20)]   # plevel 20 as cuda/moe.cc:411
     with rx.dialect_preference(["cuda"]):
@@ -136,6 +137,20 @@ def test_declare_reproduces_the_output_contract(pkg):
     lib.raf_hip_call_destroy(h)
     h, rc, outs = _declare(rx, "raf.op.moe_decode", [("t", (F32, (8, 50, 64))), ("t", (F32, (100,))), ("t", (I32, (2, 100)))])
     assert rc == 0 and outs == [(F32, (100, 64))]
+    lib.raf_hip_call_destroy(h)
+    # backward ops (src/op/declare/moe.cc:165-247)
+    h, rc, outs = _declare(rx, "raf.op.moe_encode_dx", [("t", (BF16, (8, 50, 64))), ("t", (I32, (2, 100)))])
+    assert rc == 0 and outs == [(BF16, (100, 64))]
+    lib.raf_hip_call_destroy(h)
+    h, rc, outs = _declare(rx, "raf.op.moe_encode_dg", [("t", (F32, (100,))), ("t", (I32, (2, 100))), ("i", 8)])
+    assert rc == 0 and outs == [(F32, (100, 8))]
+    lib.raf_hip_call_destroy(h)
+    h, rc, outs = _declare(rx, "raf.op.moe_decode_dx", [("t", (BF16, (100, 64))), ("t", (F32, (100,))), ("t", (I32, (2, 100))), ("i", 8), ("i", 50)])
+    assert rc == 0 and outs == [(BF16, (8, 50, 64))]
+    assert lib.raf_hip_dispatch(h) == 0 and lib.raf_hip_workspace_bytes(h, 0) == 8 * 50 * 4
+    lib.raf_hip_call_destroy(h)
+    h, rc, outs = _declare(rx, "raf.op.moe_decode_dg", [("t", (F32, (100, 64))), ("t", (F32, (8, 50, 64))), ("t", (I32, (2, 100)))])
+    assert rc == 0 and outs == [(F32, (100,))]
     lib.raf_hip_call_destroy(h)
 
 

@@ -1,0 +1,98 @@
+"""GPU parity tests of the MoE backward ops (moe_encode_dx/dg, moe_decode_dx/dg) against the NumPy
+oracle (itself pinned against torch autograd in tests/test_oracle_moe.py).
+
+Bar: encode_dx, encode_dg and fp32 decode_dx are copies or single fp32 products -> bit-exact;
+16-bit decode_dx within 1 ulp; decode_dg is a length-M dot product summed in a different order than
+the oracle's fp64 sum -> 1e-5 of sum|a_i*b_i|."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as mo
+from tests.gpu_util import dev, make_inputs, rows_as_oracle, rows_to_torch, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def routed(S, M, E, k, dt, seed):
+    data, logits = make_inputs(seed, S, M, E, zipf_bias=True)
+    rows = rows_as_oracle(data, dt)
+    used0 = np.zeros(E, np.int32)
+    if k == 1:
+        return rows, mo.moe_encode(rows, mo.softmax_rows(logits), used0, 0.7, fast_scatter=True)
+    return rows, mo.moe_encode_top2(rows, logits, used0, 0.7, gate_is_logits=True, fast_scatter=True)
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("k", [1, 2])
+@pytest.mark.parametrize("S,M,E", [(1024, 128, 32), (777, 40, 6), (300, 5, 4)])
+def test_backward_ops(pkg, dt, k, S, M, E):
+    ops = pkg.ops
+    rows, (g, il, used, elems, disp) = routed(S, M, E, k, dt, S + 3 * k)
+    C = disp.shape[1]
+    rng = np.random.default_rng(S)
+    dy_buf = rows_as_oracle(rng.standard_normal(disp.shape, dtype=np.float32), dt)
+    dy_tok = rows_as_oracle(rng.standard_normal((S, M), dtype=np.float32), dt)
+    dy_gate = rng.standard_normal(k * S, dtype=np.float32)
+    d_il, d_g = dev(il), dev(g)
+    assert (il[0] < 0).any()
+    # encode_dx: gather (k = 2: fp32 sum of two rows, rounded once)
+    got = ops.moe_encode_dx(rows_to_torch(dy_buf, dt), d_il, top_k=k)
+    want = mo.moe_encode_dx(dy_buf, il, k)
+    if dt == "f32" or k == 1:
+        np.testing.assert_array_equal(to_np(got), rows_as_oracle(want, dt))
+    else:
+        tdt = torch.bfloat16 if dt == "bf16" else torch.float16
+        diff = (got.cpu().view(torch.int16).int() - torch.from_numpy(want).to(tdt).view(torch.int16).int()).abs().max()
+        assert int(diff) <= 1
+    # encode_dg
+    got = ops.moe_encode_dg(dev(dy_gate), d_il, E, top_k=k)
+    np.testing.assert_array_equal(to_np(got), mo.moe_encode_dg(dy_gate, il, E, k))
+    # decode_dx
+    got = ops.moe_decode_dx(rows_to_torch(dy_tok, dt), d_g, d_il, E, C, top_k=k)
+    want = mo.moe_decode_dx(dy_tok, g, il, E, C, k)
+    if dt == "f32":
+        np.testing.assert_array_equal(to_np(got), want)
+    else:
+        tdt = torch.bfloat16 if dt == "bf16" else torch.float16
+        diff = (got.cpu().view(torch.int16).int() - torch.from_numpy(want).to(tdt).view(torch.int16).int()).abs().max()
+        assert int(diff) <= 1
+    # decode_dg
+    got = to_np(ops.moe_decode_dg(rows_to_torch(dy_tok, dt), rows_to_torch(disp, dt), d_il, top_k=k))
+    want = mo.moe_decode_dg(dy_tok, disp, il, k)
+    ok = (il[0] >= 0)
+    tok = np.tile(np.arange(S), k)
+    scale = np.zeros(k * S)
+    scale[ok] = np.abs(disp[il[0][ok], il[1][ok]].astype(np.float64) * dy_tok[tok[ok]]).sum(axis=1)
+    assert (np.abs(got.astype(np.float64) - want) <= 1e-5 * scale + 1e-30).all()
+    assert not got[~ok].any()
+
+
+def test_backward_matches_autograd_through_forward_ops(pkg):
+    """End to end: gradients of sum(decode(expert(encode(x))) * Y) with an elementwise expert, taken
+    with the backward ops, against torch autograd of the same computation written with torch indexing."""
+    ops = pkg.ops
+    S, M, E = 512, 64, 8
+    data, logits = make_inputs(5, S, M, E)
+    x = dev(data)
+    gate = dev(mo.softmax_rows(logits))
+    g, il, used, elems, disp = ops.moe_encode(x, gate, None, 0.8)
+    C = disp.shape[1]
+    y = ops.moe_decode(disp * 2.0, g, il)
+    Y = torch.randn_like(y)
+    # backward with the ops
+    d_expert_out = ops.moe_decode_dx(Y, g, il, E, C)
+    d_gates_s = ops.moe_decode_dg(Y, disp * 2.0, il)
+    d_x = ops.moe_encode_dx(d_expert_out * 2.0, il)
+    d_gate = ops.moe_encode_dg(d_gates_s, il, E)
+    # autograd reference
+    xr = x.clone().double().requires_grad_(True)
+    gr = gate.clone().double().requires_grad_(True)
+    idx, loc = il[0].long(), il[1].long()
+    kept = idx >= 0
+    gs = gr[torch.arange(S, device="cuda"), idx.clamp_min(0)]
+    yr = torch.zeros((S, M), dtype=torch.float64, device="cuda")
+    yr[kept] = xr[kept] * 2.0 * gs[kept, None]
+    (yr * Y.double()).sum().backward()
+    torch.testing.assert_close(d_x.double(), xr.grad, rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(d_gate.double(), gr.grad, rtol=1e-5, atol=1e-5)

@@ -291,3 +291,57 @@ def test_bf16_rounding_helpers():
     import torch
     t = torch.from_numpy(x).to(torch.bfloat16).to(torch.float32).numpy()
     np.testing.assert_array_equal(r, t)
+
+
+# ---------------------------------------------------------------- backward ops vs torch autograd
+@pytest.mark.parametrize("k", [1, 2])
+def test_backward_ops_match_autograd_of_dense_forms(k):
+    """Dense forms: dispatched = einsum('sec,sm->ecm', mask, x), gates_s = gate[s, idx];
+    combined = einsum('sec,ecm->sm', weight_sec, expert_out).  torch autograd of those gives the four
+    gradients without using the oracle's backward formulas."""
+    import torch
+    S, M, E = 40, 6, 4
+    data, logits = rng_case(31 + k, S, M, E)
+    logits[:, 0] += 1.0
+    probs = mo.softmax_rows(logits)
+    if k == 1:
+        g, il, used, _, disp = mo.moe_encode(data, probs, np.zeros(E, np.int32), 0.75)
+    else:
+        g, il, used, _, disp = mo.moe_encode_top2(data, logits, np.zeros(E, np.int32), 0.75, gate_is_logits=True)
+    C = disp.shape[1]
+    mask = np.zeros((k, S, E, C), np.float64)
+    for j in range(k):
+        for s in range(S):
+            e, l = il[0, j * S + s], il[1, j * S + s]
+            if e >= 0:
+                mask[j, s, e, l] = 1.0
+    rng = np.random.default_rng(5)
+    # --- encode: loss = <dispatched, W> + <gates_s, w>
+    W = rng.standard_normal(disp.shape)
+    w = rng.standard_normal(k * S)
+    x = torch.tensor(data.astype(np.float64), requires_grad=True)
+    gate = torch.tensor(probs.astype(np.float64), requires_grad=True)
+    tmask = torch.tensor(mask)
+    dispatched = torch.einsum("jsec,sm->ecm", tmask, x)
+    onehot = torch.zeros((k, S, E), dtype=torch.float64)
+    sel, _ = mo.select_topk(logits, k, True)
+    for j in range(k):
+        kept = il[0, j * S:(j + 1) * S] >= 0
+        onehot[j, np.arange(S)[kept], sel[j][kept]] = 1.0     # dropped slots get no gate gradient
+    gates_s = (gate[None] * onehot).sum(dim=2).reshape(-1)
+    loss = (dispatched * torch.tensor(W)).sum() + (gates_s * torch.tensor(w)).sum()
+    loss.backward()
+    np.testing.assert_array_equal(disp, dispatched.detach().numpy().astype(np.float32))
+    np.testing.assert_allclose(mo.moe_encode_dx(W.astype(np.float32), il, k), x.grad.numpy(), rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(mo.moe_encode_dg(w.astype(np.float32), il, E, k), gate.grad.numpy(), rtol=1e-6, atol=1e-7)
+    # --- decode: loss = <combined, Y>
+    Y = rng.standard_normal((S, M))
+    eo = torch.tensor((disp * 1.5 + 0.1).astype(np.float64), requires_grad=True)
+    gs = torch.tensor(g.astype(np.float64), requires_grad=True)
+    weight = (tmask * gs.reshape(k, S, 1, 1)).sum(dim=0)
+    combined = torch.einsum("sec,ecm->sm", weight, eo)
+    (combined * torch.tensor(Y)).sum().backward()
+    eo32 = eo.detach().numpy().astype(np.float32)
+    np.testing.assert_allclose(mo.moe_decode(eo32, g, il, k=k), combined.detach().numpy(), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(mo.moe_decode_dx(Y.astype(np.float32), g, il, E, C, k), eo.grad.numpy(), rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(mo.moe_decode_dg(Y.astype(np.float32), eo32, il, k), gs.grad.numpy(), rtol=1e-5, atol=1e-6)

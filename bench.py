@@ -159,6 +159,99 @@ def cpu_baseline_lans(hyper_steps=2):
             "kind": "port", "sample": "C/OpenMP restatement, one MoE layer's 32 expert tensors"}
 
 
+def bench_config4_partitioned(ops, lib, capi, data, logits, S, M, E, cf, iters):
+    """BASELINE config 4 as configured: 4 token partitions x 2 slots encoded in capacity order
+    (s1p0..s1p3, s2p0..s2p3) with chained used capacity, moe_merge_masks, moe_redispatch, moe_decode.
+    Per-slot gate arrays are prepared outside the timed region."""
+    import ctypes as C
+    import torch
+    P = 4
+    Sp = S // P
+    sel = torch.empty((2, S), dtype=torch.int32, device="cuda")
+    val = torch.empty((2, S), dtype=torch.float32, device="cuda")
+    assert lib.lancet_gate_topk(C.c_void_p(logits.data_ptr()), S, E, 2, capi.GATE_IS_LOGITS,
+                                C.c_void_p(sel.data_ptr()), C.c_void_p(val.data_ptr()), None) == 0
+    gates, parts = [], []
+    for slot in range(2):
+        for pi in range(P):
+            sl = slice(pi * Sp, (pi + 1) * Sp)
+            g = torch.full((Sp, E), -1.0, device="cuda")
+            g.scatter_(1, sel[slot, sl].long()[:, None], val[slot, sl][:, None])
+            gates.append(g)
+            parts.append(data[sl])
+    Cap = ops.moe_capacity(Sp, E, 2 * cf * P)
+    outs = [(torch.empty(Sp, device="cuda"), torch.empty((2, Sp), dtype=torch.int32, device="cuda"),
+             torch.empty(E, dtype=torch.int32, device="cuda"), torch.empty(E, dtype=torch.int64, device="cuda"),
+             torch.empty((E, Cap, M), dtype=data.dtype, device="cuda")) for _ in range(2 * P)]
+    ws = torch.empty(ops.moe_encode_workspace_bytes(Sp, E, 1), dtype=torch.uint8, device="cuda")
+    zero = torch.zeros(E, dtype=torch.int32, device="cuda")
+    merged = torch.empty((2, 2 * S), dtype=torch.int32, device="cuda")
+    red = torch.empty((E, Cap, M), dtype=data.dtype, device="cuda")
+    dec = torch.empty((S, M), dtype=data.dtype, device="cuda")
+    mws = torch.empty(1 << 16, dtype=torch.uint8, device="cuda")
+
+    def encodes():
+        used = zero
+        for i in range(2 * P):
+            ops.moe_encode(parts[i], gates[i], used, 2 * cf * P, zero_tail=False, workspace=ws, out=outs[i])
+            used = outs[i][2]
+
+    ils = [o[1] for o in outs]
+    bufs = [o[4] for o in outs]
+
+    def merge():
+        ops.moe_merge_masks(ils, E, workspace=mws, out=merged)
+
+    def redispatch():
+        ops.moe_redispatch(bufs, ils, workspace=mws, out=red)
+
+    encodes(), merge(), redispatch()
+    weights = ops.moe_top2_normalize_gates(torch.cat([o[0] for o in outs]), merged)
+
+    def decode():
+        ops.moe_decode(red, weights, merged, top_k=2, out=dec)
+
+    t = {name: event_ms(fn, iters) for name, fn in (("encode_x8", encodes), ("merge_masks", merge),
+                                                     ("redispatch", redispatch), ("decode", decode))}
+    kept = int((merged[0] >= 0).sum())
+    b = data.element_size()
+    # SURVEY 8(d): partition encodes S*E*4 + S*M*b (each token row once per slot here: x2) + kept*M*b,
+    # merge 2*(kS)*8, redispatch kept*M*b + E*C*M*b, decode kept*M*b + S*M*b + kS*12
+    alg = (S * E * 4 + S * M * b + kept * M * b) + 2 * (2 * S) * 8 + (kept * M * b + E * Cap * M * b) + \
+          (kept * M * b + S * M * b + 2 * S * 12)
+    total = sum(t.values())
+    return {"workload": "4 partitions x 2 slots -> merge_masks -> redispatch -> decode, S=%d M=%d E=%d C=%d" % (S, M, E, Cap),
+            "ms": {k: round(v, 4) for k, v in t.items()}, "ms_total": round(total, 4),
+            "tokens_per_s": round(S / (total * 1e-3), 1), "algorithmic_bytes": alg,
+            "frac_of_hbm_peak": round(alg / (total * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "note": "token rows are read once per slot (two passes) in this call pattern; "
+                    "partition encodes write used rows only (zero_tail=False), redispatch zero-fills the merged tail"}
+
+
+def bench_backward(ops, data, outs, dec, S, M, E, Cap, K, kept, iters):
+    """The four backward ops at the headline shape (dy buffers reuse forward tensors as values)."""
+    import torch
+    b = data.element_size()
+    g, il, disp = outs[0], outs[1], outs[4]
+    dx = torch.empty_like(data)
+    dgate = torch.empty((S, E), device="cuda")
+    dbuf = torch.empty_like(disp)
+    dgs = torch.empty(K * S, device="cuda")
+    ws = torch.empty(E * Cap * 4, dtype=torch.uint8, device="cuda")
+    res = {}
+    for name, fn, nbytes in (
+            ("encode_dx", lambda: ops.moe_encode_dx(disp, il, top_k=K, out=dx), kept * M * b + S * M * b + K * S * 8),
+            ("encode_dg", lambda: ops.moe_encode_dg(g, il, E, top_k=K, out=dgate), S * E * 4 + K * S * 8),
+            ("decode_dx", lambda: ops.moe_decode_dx(dec, g, il, E, Cap, top_k=K, workspace=ws, out=dbuf),
+             kept * M * b + E * Cap * M * b + K * S * 12 + 2 * E * Cap * 4),
+            ("decode_dg", lambda: ops.moe_decode_dg(dec, disp, il, top_k=K, out=dgs), 2 * kept * M * b + K * S * 12)):
+        fn()
+        ms = event_ms(fn, iters)
+        res[name] = {"ms": round(ms, 4), "algorithmic_bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1),
+                     "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    return res
+
+
 def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -260,7 +353,7 @@ def main():
     p = lambda t: C.c_void_p(t.data_ptr())
 
     def scatter_only():
-        st = lib.lancet_moe_scatter(p(data), p(outs[1]), p(used_in), p(outs[2]), S, M, E, Cap, K, capi.BF16,
+        st = lib.lancet_moe_scatter(p(data), p(outs[1]), p(used_in), p(outs[2]), S, M, E, Cap, K, capi.BF16, 0,
                                     p(outs[4]), stream)
         assert st == 0
 
@@ -318,7 +411,11 @@ def main():
             "encode_plus_decode_frac": round(gbs(enc_bytes + dec_bytes, ms_enc + ms_dec) / HBM_PEAK_GBS, 4),
         },
     }
-    del data, dec, outs
+    result["backward"] = bench_backward(ops, data, outs, dec, S, M, E, Cap, K, kept, n)
+    del dec, outs
+    torch.cuda.empty_cache()
+    result["config4_partitioned"] = bench_config4_partitioned(ops, lib, capi, data, logits, S, M, E, cf, max(5, n // 2))
+    del data
     torch.cuda.empty_cache()
     if not args.no_lans:
         result["lans"] = bench_lans(ops, capi, max(3, min(args.steps, 10)), max(1, min(args.warmup, 2)),

@@ -56,6 +56,12 @@ extern "C" {
 
 /* flags of lancet_moe_encode / lancet_moe_encode_bpr / lancet_gate_topk */
 #define LANCET_GATE_IS_LOGITS 1u /* `gate` holds logits: select on them, gates_s = softmax prob */
+/* lancet_moe_encode / lancet_moe_encode_bpr / lancet_moe_scatter: leave the rows past the used
+ * capacity unwritten instead of zero-filling them.  For partition buffers that only feed
+ * moe_redispatch (which reads the used rows and zero-fills the merged tail itself); it is what the
+ * reference's own cost for this pattern, a full memset per partition buffer
+ * (tutel_moe_dispatch.cu:466), is spent on. */
+#define LANCET_NO_TAIL_ZERO 2u
 
 typedef void* lancet_stream_t;
 
@@ -122,7 +128,7 @@ int lancet_moe_route(const float* gate, const int32_t* used_in, int64_t S, int64
                      void* workspace, size_t workspace_bytes, lancet_stream_t stream);
 int lancet_moe_scatter(const void* data, const int32_t* indices_locations, const int32_t* used_in,
                        const int32_t* used_out, int64_t S, int64_t M, int64_t E, int64_t C, int top_k,
-                       int dtype, void* dispatched, lancet_stream_t stream);
+                       int dtype, unsigned flags, void* dispatched, lancet_stream_t stream);
 
 /* ---- raf.op.moe_encode_batch_prioritized --------------------------------------------
  * Replaces MoeEncodeBatchPrioritized::Execute (moe.cc:543-684), the TVM argsort it calls

@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(HERE, "lib", "liblancet_hip.so")
 
 F32, BF16, F16 = 0, 1, 2
 GATE_IS_LOGITS = 1
+NO_TAIL_ZERO = 2
 LANS_SWEEPS, LANS_PIPELINED = 0, 1
 MAX_EXPERTS = 512
 MAX_PARTITIONS = 64
@@ -46,7 +47,7 @@ SIGNATURES = {
     "lancet_moe_encode": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _u32,
                                  _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "lancet_moe_route": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _u32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
-    "lancet_moe_scatter": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp]),
+    "lancet_moe_scatter": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _u32, _vp, _vp]),
     "lancet_moe_encode_bpr_workspace_bytes": (_sz, [_i64, _i64, _int]),
     "lancet_moe_encode_bpr": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _u32,
                                      _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),

@@ -147,7 +147,7 @@ extern "C" int lancet_moe_route(const float* gate, const int32_t* used_in, int64
 
 extern "C" int lancet_moe_scatter(const void* data, const int32_t* indices_locations, const int32_t* used_in,
                                   const int32_t* used_out, int64_t S, int64_t M, int64_t E, int64_t C, int top_k,
-                                  int dtype, void* dispatched, lancet_stream_t stream) {
+                                  int dtype, unsigned flags, void* dispatched, lancet_stream_t stream) {
   if ((!data && S > 0 && M > 0) || (!indices_locations && S > 0) || !used_out || (!dispatched && C > 0 && M > 0))
     return LANCET_ERR_NULL;
   const int eb = elem_bytes(dtype);
@@ -158,9 +158,10 @@ extern "C" int lancet_moe_scatter(const void* data, const int32_t* indices_locat
       misaligned(used_in, 4) || misaligned(used_out, 4))
     return LANCET_ERR_ALIGN;
   const int s = static_cast<int>(S);
+  const bool tail = !(flags & LANCET_NO_TAIL_ZERO);
   return rc(run_scatter_rows(data, dispatched, indices_locations, indices_locations + static_cast<size_t>(top_k) * s,
-                             nullptr, used_in, used_out, s, static_cast<int>(M), static_cast<int>(E),
-                             static_cast<int>(C), top_k, eb, S_(stream)));
+                             nullptr, tail ? used_in : nullptr, tail ? used_out : nullptr, s, static_cast<int>(M),
+                             static_cast<int>(E), static_cast<int>(C), top_k, eb, S_(stream)));
 }
 
 extern "C" int lancet_moe_encode(const void* data, const float* gate, const int32_t* used_in, int64_t S,
@@ -176,7 +177,8 @@ extern "C" int lancet_moe_encode(const void* data, const float* gate, const int3
   if (int r = lancet_moe_route(gate, used_in, S, M, E, C, top_k, flags, gates_s, indices_locations, used_out,
                                elements_per_expert, workspace, workspace_bytes, stream))
     return r;
-  return lancet_moe_scatter(data, indices_locations, used_in, used_out, S, M, E, C, top_k, dtype, dispatched, stream);
+  return lancet_moe_scatter(data, indices_locations, used_in, used_out, S, M, E, C, top_k, dtype, flags, dispatched,
+                            stream);
 }
 
 // ---- raf.op.moe_encode_batch_prioritized ----------------------------------------------
@@ -213,7 +215,8 @@ extern "C" int lancet_moe_encode_bpr(const void* data, const float* gate, int64_
                                loc, used_out, elements_per_expert, workspace, S_(stream));
   if (e != hipSuccess) return rc(e);
   const char* part = static_cast<const char*>(data) + static_cast<size_t>(partition_id) * s * M * eb;
-  return rc(run_scatter_rows(part, dispatched, idx, loc, nullptr, nullptr, used_out, s, static_cast<int>(M),
+  return rc(run_scatter_rows(part, dispatched, idx, loc, nullptr, nullptr,
+                             (flags & LANCET_NO_TAIL_ZERO) ? nullptr : used_out, s, static_cast<int>(M),
                              static_cast<int>(E), static_cast<int>(C), 1, eb, S_(stream)));
 }
 

@@ -66,13 +66,18 @@ def moe_encode_workspace_bytes(S, E, top_k=1):
     return int(capi.load().lancet_moe_encode_workspace_bytes(int(S), int(E), int(top_k)))
 
 
+def _flags(gate_is_logits, zero_tail):
+    return (capi.GATE_IS_LOGITS if gate_is_logits else 0) | (0 if zero_tail else capi.NO_TAIL_ZERO)
+
+
 def moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_logits=False,
-               workspace=None, out=None):
+               zero_tail=True, workspace=None, out=None):
     """raf.op.moe_encode(data, gate, used_capacity, capacity_factor=1.0).
 
     Returns (gates_s [k*S] f32, indices_locations [2, k*S] i32, used_capacity [E] i32,
     elements_per_expert [E] u64, dispatched [E, C, M]).  With top_k = 2 the capacity follows
-    GShard: capacity_factor is doubled before the reference formula is applied."""
+    GShard: capacity_factor is doubled before the reference formula is applied.  zero_tail=False
+    leaves rows past the used capacity unwritten (partition buffers that only feed moe_redispatch)."""
     lib = capi.load()
     dt = _check_encode_inputs(data, gate)
     S, M = data.shape
@@ -96,7 +101,7 @@ def moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_
     ws_bytes = moe_encode_workspace_bytes(S, E, top_k)
     ws = _workspace(ws_bytes, dev, workspace)
     st = lib.lancet_moe_encode(_p(data), _p(gate), _p(used_capacity), S, M, E, Cap, top_k, dt,
-                               capi.GATE_IS_LOGITS if gate_is_logits else 0, _p(gates_s), _p(indloc),
+                               _flags(gate_is_logits, zero_tail), _p(gates_s), _p(indloc),
                                _p(used_out), _p(elems), _p(disp), _p(ws), ws.numel(), _stream())
     capi.check(st, "lancet_moe_encode")
     return gates_s, indloc, used_out, elems.view(torch.uint64) if elems.dtype == torch.int64 else elems, disp
@@ -107,7 +112,7 @@ def moe_encode_bpr_workspace_bytes(S0, E, n_partitions=1):
 
 
 def moe_encode_batch_prioritized(data, gate, n_partitions=1, partition_id=0, capacity_factor=1.0,
-                                 gate_is_logits=False, workspace=None, out=None):
+                                 gate_is_logits=False, zero_tail=True, workspace=None, out=None):
     """raf.op.moe_encode_batch_prioritized(data, gate, n_partitions=1, partition_id=0,
     capacity_factor=1.0): data/gate are the whole batch, the outputs cover partition
     partition_id (S = S0 / n_partitions tokens)."""
@@ -131,7 +136,7 @@ def moe_encode_batch_prioritized(data, gate, n_partitions=1, partition_id=0, cap
     ws_bytes = moe_encode_bpr_workspace_bytes(S0, E, n_partitions)
     ws = _workspace(ws_bytes, dev, workspace)
     st = lib.lancet_moe_encode_bpr(_p(data), _p(gate), S0, M, E, Cap, n_partitions, partition_id, dt,
-                                   capi.GATE_IS_LOGITS if gate_is_logits else 0, _p(gates_s), _p(indloc),
+                                   _flags(gate_is_logits, zero_tail), _p(gates_s), _p(indloc),
                                    _p(used_out), _p(elems), _p(disp), _p(ws), ws.numel(), _stream())
     capi.check(st, "lancet_moe_encode_bpr")
     return gates_s, indloc, used_out, elems.view(torch.uint64) if elems.dtype == torch.int64 else elems, disp

@@ -9,8 +9,8 @@
 // :731-823 (MoeMergeMasks), :826-943 (MoeRedispatch), :1228-1311 (MoeDecode).
 //
 // Extensions are trailing, defaulted arguments only:
-//   moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_logits=false)
-//   moe_encode_batch_prioritized(..., capacity_factor=1.0, gate_is_logits=false)
+//   moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_logits=false, zero_tail=true)
+//   moe_encode_batch_prioritized(..., capacity_factor=1.0, gate_is_logits=false, zero_tail=true)
 //   moe_decode(data, gate, indices_locations, top_k=1)
 #include <string>
 #include <vector>
@@ -115,7 +115,7 @@ class MoeEncode : public OpEnv {
     top_k_ = static_cast<int>(OptInt(cv, 4, 1));
     const float cf = static_cast<float>(OptFloat(cv, 3, 1.0)) * (top_k_ == 2 ? 2.0f : 1.0f);
     shape_ = CheckEncodeInputs(data, cv.args[1].AsTensor(), 1, cf);
-    flags_ = OptInt(cv, 5, 0) ? LANCET_GATE_IS_LOGITS : 0u;
+    flags_ = (OptInt(cv, 5, 0) ? LANCET_GATE_IS_LOGITS : 0u) | (OptInt(cv, 6, 1) ? 0u : LANCET_NO_TAIL_ZERO);
     dtype_ = DTypeToLancet(data.dtype);
     device_id_ = data.device_id;
     RAF_CHECK(cv.out.kind == Value::kTuple && cv.out.fields.size() == 5, "Expected output to be a 5-Tuple");
@@ -177,7 +177,7 @@ class MoeEncodeBatchPrioritized : public OpEnv {
     RAF_CHECK(n_partitions_ > 0 && partition_id_ >= 0 && partition_id_ < n_partitions_, "bad partition");
     shape_ = CheckEncodeInputs(data, cv.args[1].AsTensor(), n_partitions_, static_cast<float>(OptFloat(cv, 4, 1.0)));
     orig_S_ = data.shape[0];
-    flags_ = OptInt(cv, 5, 0) ? LANCET_GATE_IS_LOGITS : 0u;
+    flags_ = (OptInt(cv, 5, 0) ? LANCET_GATE_IS_LOGITS : 0u) | (OptInt(cv, 6, 1) ? 0u : LANCET_NO_TAIL_ZERO);
     dtype_ = DTypeToLancet(data.dtype);
     device_id_ = data.device_id;
     // sorted indices, dropping mask, indices and gate buffers of the reference (cuda/moe.cc:512-520)

@@ -314,3 +314,31 @@ def test_bounded_wait_flags_the_workspace(pkg):
     want = mo.moe_encode(data, logits, np.zeros(E, np.int32), 1.0, fast_scatter=True)
     got = pkg.ops.moe_encode(d_data, d_gate, None, 1.0, workspace=ws)
     np.testing.assert_array_equal(to_np(got[1]), want[1])
+
+
+def test_encode_without_tail_zero_fill_feeds_redispatch(pkg):
+    """zero_tail=False writes the used rows only: they equal the zero-filled encode's rows, the rest of
+    the buffer keeps what it held, and moe_redispatch over such partition buffers is unchanged."""
+    ops = pkg.ops
+    S0, M, E, P = 2048, 64, 8, 4
+    data, logits = make_inputs(77, S0, M, E, zipf_bias=True)
+    gate = dev(mo.softmax_rows(logits))
+    d_data = dev(data)
+    S = S0 // P
+    Cap = ops.moe_capacity(S, E, float(P))
+    used_a = used_b = None
+    ils, bufs_a, bufs_b = [], [], []
+    for p_ in range(P):
+        sl = slice(p_ * S, (p_ + 1) * S)
+        a = ops.moe_encode(d_data[sl], gate[sl], used_a, float(P))
+        out_b = (torch.empty(S, device="cuda"), torch.empty((2, S), dtype=torch.int32, device="cuda"),
+                 torch.empty(E, dtype=torch.int32, device="cuda"), torch.empty(E, dtype=torch.int64, device="cuda"),
+                 torch.full((E, Cap, M), 7.0, device="cuda"))
+        b = ops.moe_encode(d_data[sl], gate[sl], used_b, float(P), zero_tail=False, out=out_b)
+        kept = (a[2] - (used_a if used_a is not None else 0)).long()
+        rows = torch.arange(Cap, device="cuda")[None, :] < kept[:, None]
+        assert torch.equal(a[1], b[1]) and torch.equal(a[2], b[2])
+        assert torch.equal(a[4][rows], b[4][rows]) and bool((b[4][~rows] == 7.0).all())
+        used_a, used_b = a[2], b[2]
+        ils.append(a[1]), bufs_a.append(a[4]), bufs_b.append(b[4])
+    assert torch.equal(ops.moe_redispatch(bufs_a, ils), ops.moe_redispatch(bufs_b, ils))

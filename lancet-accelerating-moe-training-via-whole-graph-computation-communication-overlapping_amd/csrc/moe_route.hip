@@ -13,37 +13,48 @@ namespace lancet {
 // Replaces the argmax / one_hot / multiply+sum micro-kernels of
 // src/op/dialect/cuda/moe.cc:177-250 (three passes over [S,E] plus an [S,E] workspace).
 // ---------------------------------------------------------------------------------------
-template <int K>
-__device__ __forceinline__ void consider(float x, int j, float& v1, int& i1, float& v2, int& i2) {
-  if (i1 < 0 || x > v1) {
-    v2 = v1;
-    i2 = i1;
-    v1 = x;
-    i1 = j;
-  } else if (K == 2 && (i2 < 0 || x > v2)) {
-    v2 = x;
-    i2 = j;
-  }
-}
+// Running first-max / second-max of a row, all in scalars (no arrays, no references: the state has
+// to stay in registers).  Branch-free: a lane either takes a new first choice (the old one becomes
+// the second), or a new second choice, or nothing.
+struct TopState {
+  float v1, v2;
+  int i1, i2;
+};
 
 template <int K>
-__device__ __forceinline__ void route_token(const float* __restrict__ row, int E, bool is_logits,
-                                            int (&e)[K], float (&p)[K]) {
+__device__ __forceinline__ TopState consider(TopState t, float x, int j) {
+  const bool first = (t.i1 < 0) | (x > t.v1);
+  if (K == 2) {
+    const bool second = !first & ((t.i2 < 0) | (x > t.v2));
+    t.v2 = first ? t.v1 : (second ? x : t.v2);
+    t.i2 = first ? t.i1 : (second ? j : t.i2);
+  }
+  t.v1 = first ? x : t.v1;
+  t.i1 = first ? j : t.i1;
+  return t;
+}
+
+struct Routed {
+  int e0, e1;
+  float p0, p1;
+};
+
+template <int K>
+__device__ __forceinline__ Routed route_token(const float* __restrict__ row, int E, bool is_logits) {
   typedef float f32x4 __attribute__((ext_vector_type(4)));
-  float v1 = 0.f, v2 = 0.f;
-  int i1 = -1, i2 = -1;
+  TopState t = {0.f, 0.f, -1, -1};
   const bool vec = ((E & 3) == 0) && ((reinterpret_cast<uintptr_t>(row) & 15u) == 0);
   if (vec) {
     const f32x4* r4 = reinterpret_cast<const f32x4*>(row);
     for (int j = 0; j < E / 4; ++j) {
       const f32x4 x = r4[j];
-      consider<K>(x.x, 4 * j, v1, i1, v2, i2);
-      consider<K>(x.y, 4 * j + 1, v1, i1, v2, i2);
-      consider<K>(x.z, 4 * j + 2, v1, i1, v2, i2);
-      consider<K>(x.w, 4 * j + 3, v1, i1, v2, i2);
+      t = consider<K>(t, x.x, 4 * j);
+      t = consider<K>(t, x.y, 4 * j + 1);
+      t = consider<K>(t, x.z, 4 * j + 2);
+      t = consider<K>(t, x.w, 4 * j + 3);
     }
   } else {
-    for (int j = 0; j < E; ++j) consider<K>(row[j], j, v1, i1, v2, i2);
+    for (int j = 0; j < E; ++j) t = consider<K>(t, row[j], j);
   }
   float sum = 1.f;
   if (is_logits) {
@@ -52,21 +63,21 @@ __device__ __forceinline__ void route_token(const float* __restrict__ row, int E
       const f32x4* r4 = reinterpret_cast<const f32x4*>(row);
       for (int j = 0; j < E / 4; ++j) {
         const f32x4 x = r4[j];
-        sum += expf(x.x - v1);
-        sum += expf(x.y - v1);
-        sum += expf(x.z - v1);
-        sum += expf(x.w - v1);
+        sum += expf(x.x - t.v1);
+        sum += expf(x.y - t.v1);
+        sum += expf(x.z - t.v1);
+        sum += expf(x.w - t.v1);
       }
     } else {
-      for (int j = 0; j < E; ++j) sum += expf(row[j] - v1);
+      for (int j = 0; j < E; ++j) sum += expf(row[j] - t.v1);
     }
   }
-  e[0] = i1;
-  p[0] = is_logits ? expf(v1 - v1) / sum : v1;
-  if (K == 2) {
-    e[1] = i2;
-    p[1] = is_logits ? expf(v2 - v1) / sum : v2;
-  }
+  Routed r;
+  r.e0 = t.i1;
+  r.p0 = is_logits ? expf(t.v1 - t.v1) / sum : t.v1;
+  r.e1 = K == 2 ? t.i2 : -1;
+  r.p1 = K == 2 ? (is_logits ? expf(t.v2 - t.v1) / sum : t.v2) : 0.f;
+  return r;
 }
 
 struct RouteArgs {
@@ -112,7 +123,13 @@ __global__ __launch_bounds__(kTile) void route_scan_kernel(RouteArgs a) {
       const int x = a.idx_in[s];
       e[0] = (x >= 0 && x < a.E) ? x : -1;
     } else {
-      route_token<K>(a.gate + static_cast<size_t>(s) * a.E, a.E, a.is_logits != 0, e, p);
+      const Routed r = route_token<K>(a.gate + static_cast<size_t>(s) * a.E, a.E, a.is_logits != 0);
+      e[0] = r.e0;
+      p[0] = r.p0;
+      if (K == 2) {
+        e[K - 1] = r.e1;
+        p[K - 1] = r.p1;
+      }
     }
   }
   uint32_t rank[K];
@@ -200,13 +217,12 @@ __global__ __launch_bounds__(kTile) void gate_topk_kernel(const float* gate, int
                                                           int32_t* idx, float* val) {
   const int s = blockIdx.x * kTile + threadIdx.x;
   if (s >= S) return;
-  int e[K];
-  float p[K];
-  route_token<K>(gate + static_cast<size_t>(s) * E, E, is_logits != 0, e, p);
-#pragma unroll
-  for (int j = 0; j < K; ++j) {
-    idx[static_cast<size_t>(j) * S + s] = e[j];
-    val[static_cast<size_t>(j) * S + s] = p[j];
+  const Routed r = route_token<K>(gate + static_cast<size_t>(s) * E, E, is_logits != 0);
+  idx[s] = r.e0;
+  val[s] = r.p0;
+  if (K == 2) {
+    idx[static_cast<size_t>(S) + s] = r.e1;
+    val[static_cast<size_t>(S) + s] = r.p1;
   }
 }
 

@@ -151,6 +151,18 @@ int lancet_moe_decode(const void* expert_out, const float* gates_s,
                       const int32_t* indices_locations, int64_t S, int64_t M, int64_t E,
                       int64_t C, int top_k, int dtype, void* out, lancet_stream_t stream);
 
+/* ---- raf.op.moe_redispatch_expert_input ------------------------------------------------
+ * Replaces MoeRedispatchExpertInput::Execute / launch_redispatch_expert_input (moe.cc:945-1073;
+ * kernel_util.cuh:55; tutel_moe_dispatch.cu:436-456,586-598): merge, for one local expert, of the
+ * all-to-all outputs of P token partitions.  data: HOST array of P device pointers to [C, G, M]
+ * buffers (capacity row, source GPU, model dim); recv_cnts: HOST array of P device pointers to
+ * uint64 [G * n_local_experts] received element counts (the elements_per_expert side channel of the
+ * all-to-allv).  Rows of out[C, G, M] past the merged stream are zero. */
+int lancet_moe_redispatch_expert_input(const void* const* data, const uint64_t* const* recv_cnts, int P,
+                                       int local_expert_id, int n_local_experts, int64_t C, int64_t M,
+                                       int64_t G, int recv_cnts_scale, int dtype, void* out,
+                                       lancet_stream_t stream);
+
 /* ---- backward ops (raf.op.moe_encode_dx / _dg, raf.op.moe_decode_dx / _dg) ------------------
  * Gradients wired by src/op/grad/moe.cc:30-93.  Gate-side gradients are fp32 like gates_s; top_k = 2
  * takes the slot-major layout of the forward ops.

@@ -30,6 +30,16 @@ int check_dims(int64_t S, int64_t M, int64_t E, int64_t C) {
   return LANCET_OK;
 }
 
+int fill_table(PtrTable& t, const void* const* ptrs, int P, size_t align) {
+  for (int p = 0; p < P; ++p) {
+    if (!ptrs[p]) return LANCET_ERR_NULL;
+    if (misaligned(ptrs[p], align)) return LANCET_ERR_ALIGN;
+    t.p[p] = ptrs[p];
+  }
+  for (int p = P; p < kMaxPartitions; ++p) t.p[p] = nullptr;
+  return LANCET_OK;
+}
+
 }  // namespace
 
 extern "C" int lancet_abi_version(void) { return LANCET_ABI_VERSION; }
@@ -238,6 +248,29 @@ extern "C" int lancet_moe_decode(const void* expert_out, const float* gates_s, c
                             S_(stream)));
 }
 
+extern "C" int lancet_moe_redispatch_expert_input(const void* const* data, const uint64_t* const* recv_cnts, int P,
+                                                  int local_expert_id, int n_local_experts, int64_t C, int64_t M,
+                                                  int64_t G, int recv_cnts_scale, int dtype, void* out,
+                                                  lancet_stream_t stream) {
+  if (!data || !recv_cnts || (!out && C > 0 && M > 0 && G > 0)) return LANCET_ERR_NULL;
+  const int eb = elem_bytes(dtype);
+  if (!eb) return LANCET_ERR_DTYPE;
+  if (P < 1 || P > LANCET_MAX_PARTITIONS) return LANCET_ERR_PARTITION;
+  if (C < 0 || M < 0 || G < 1 || n_local_experts < 1 || local_expert_id < 0 || local_expert_id >= n_local_experts ||
+      recv_cnts_scale < 1 || C > 0x3fffffff || M > 0x3fffffff || G > 0x3fffffff || C * G > 0x7fffffff)
+    return LANCET_ERR_SHAPE;
+  if (misaligned(out, eb)) return LANCET_ERR_ALIGN;
+  PtrTable bufs;
+  if (int r = fill_table(bufs, data, P, eb)) return r;
+  for (int p = 0; p < P; ++p) {
+    if (!recv_cnts[p]) return LANCET_ERR_NULL;
+    if (misaligned(recv_cnts[p], 8)) return LANCET_ERR_ALIGN;
+  }
+  return rc(run_redispatch_expert_input(bufs, reinterpret_cast<const void* const*>(recv_cnts), P, local_expert_id,
+                                        n_local_experts, static_cast<int>(C), static_cast<int>(M), static_cast<int>(G),
+                                        static_cast<uint64_t>(recv_cnts_scale), out, eb, S_(stream)));
+}
+
 // ---- backward ops -------------------------------------------------------------------
 extern "C" int lancet_moe_encode_dx(const void* dy, const int32_t* indices_locations, int64_t S, int64_t M,
                                     int64_t E, int64_t C, int top_k, int dtype, void* dx, lancet_stream_t stream) {
@@ -312,15 +345,6 @@ extern "C" int lancet_moe_top2_normalize_gates(const float* raw_gates, const int
 }
 
 // ---- raf.op.moe_merge_masks / raf.op.moe_redispatch -------------------------------------
-static int fill_table(PtrTable& t, const void* const* ptrs, int P, size_t align) {
-  for (int p = 0; p < P; ++p) {
-    if (!ptrs[p]) return LANCET_ERR_NULL;
-    if (misaligned(ptrs[p], align)) return LANCET_ERR_ALIGN;
-    t.p[p] = ptrs[p];
-  }
-  for (int p = P; p < kMaxPartitions; ++p) t.p[p] = nullptr;
-  return LANCET_OK;
-}
 
 extern "C" size_t lancet_moe_merge_masks_workspace_bytes(int P, int64_t E) {
   if (P < 1 || E < 1) return 0;

@@ -62,4 +62,9 @@ hipError_t run_merge_masks(const PtrTable& indlocs, int P, int S, int E, const u
 hipError_t run_redispatch_rows(const PtrTable& bufs, int P, int M, int C, int E, const uint32_t* counts,
                                void* out, int elem_bytes, hipStream_t st);
 
+// merge of P partitions of one local expert's all-to-all output, layout [C, G, M]; cnt_ptrs are P device
+// arrays of uint64 [G*LE]
+hipError_t run_redispatch_expert_input(const PtrTable& bufs, const void* const* cnt_ptrs, int P, int le, int LE, int C,
+                                       int M, int G, uint64_t scale, void* out, int elem_bytes, hipStream_t st);
+
 }  // namespace lancet

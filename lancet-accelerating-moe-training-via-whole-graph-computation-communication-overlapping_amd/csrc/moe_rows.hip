@@ -328,6 +328,90 @@ __global__ __launch_bounds__(kTile) void redispatch_rows_kernel(PtrTable bufs, i
 }
 
 // ---------------------------------------------------------------------------------------
+// redispatch_expert_input: merge of P partitions of one local expert's all-to-all output, layout
+// [C, G, M] (capacity row, source GPU, model dim).  For source g the partitions' received element
+// streams (recv_cnts_p[g*LE + le] * scale elements each, stored from row 0 of partition p) are
+// concatenated: stream element x lands at out[x / M, g, x % M]
+// (redispatch_expert_input_kernel_CGM, tutel_moe_dispatch.cu:436-456, 586-598).  Rows past the merged
+// stream are zero-filled (the reference leaves them as they were).  One wave per output row (c, g);
+// whole rows are moved in 16-byte granules when every count is a multiple of M.
+// ---------------------------------------------------------------------------------------
+struct CountTable {
+  const uint64_t* p[kMaxPartitions];
+};
+
+// EL = element storage type; VEC = rows and pointers allow 16-byte granules (the row-aligned case then
+// moves whole rows with them; streams that are not row aligned always take the element path).
+template <typename EL, bool VEC>
+__global__ __launch_bounds__(kTile) void redispatch_expert_input_kernel(PtrTable bufs, CountTable cnts, int P,
+                                                                        int le, int LE, int C, int M, int G,
+                                                                        uint64_t scale, EL* out) {
+  const int w = threadIdx.x / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  const long r = static_cast<long>(blockIdx.x) * kRowsPerBlock + w;  // output row index c*G + g
+  if (r >= static_cast<long>(C) * G) return;
+  const int c = static_cast<int>(r / G);
+  const int g = static_cast<int>(r - static_cast<long>(c) * G);
+  EL* dst = out + static_cast<size_t>(r) * M;
+  const uint64_t x0 = static_cast<uint64_t>(c) * M;  // first stream element of this row
+  uint64_t cum = 0, cum0 = 0;
+  int p0 = -1;
+  bool rows_only = true;
+  for (int q = 0; q < P; ++q) {
+    const uint64_t n = cnts.p[q][static_cast<size_t>(g) * LE + le] * scale;
+    rows_only = rows_only && (n % M == 0);
+    if (p0 < 0 && x0 < cum + n) {
+      p0 = q;
+      cum0 = cum;
+    }
+    cum += n;
+  }
+  const uint64_t total = cum;
+  constexpr int kPer = 16 / sizeof(EL);
+  if (x0 >= total) {  // past the merged stream
+    if (VEC) {
+      const u32x4 z = {0u, 0u, 0u, 0u};
+      for (int v = lane; v < M / kPer; v += kWave) st_stream(reinterpret_cast<u32x4*>(dst) + v, z);
+    } else {
+      for (int i = lane; i < M; i += kWave) dst[i] = EL(0);
+    }
+    return;
+  }
+  if (rows_only) {
+    const uint64_t src_row = (x0 - cum0) / M;
+    const bool readable = src_row < static_cast<uint64_t>(C);  // counts larger than the buffer read nothing
+    const EL* src = static_cast<const EL*>(bufs.p[p0]) + (readable ? (src_row * G + g) * M : 0);
+    if (VEC) {
+      const u32x4 z = {0u, 0u, 0u, 0u};
+      for (int v = lane; v < M / kPer; v += kWave)
+        st_stream(reinterpret_cast<u32x4*>(dst) + v, readable ? ld_stream(reinterpret_cast<const u32x4*>(src) + v) : z);
+    } else {
+      for (int i = lane; i < M; i += kWave) dst[i] = readable ? src[i] : EL(0);
+    }
+    return;
+  }
+  // element-granular streams: every element finds its partition
+  for (int i = lane; i < M; i += kWave) {
+    const uint64_t x = x0 + i;
+    EL val = EL(0);
+    if (x < total) {
+      uint64_t run = 0;
+      for (int q = 0; q < P; ++q) {
+        const uint64_t n = cnts.p[q][static_cast<size_t>(g) * LE + le] * scale;
+        if (x < run + n) {
+          const uint64_t y = x - run;
+          const uint64_t sr = y / M;
+          if (sr < static_cast<uint64_t>(C)) val = static_cast<const EL*>(bufs.p[q])[(sr * G + g) * M + (y - sr * M)];
+          break;
+        }
+        run += n;
+      }
+    }
+    dst[i] = val;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // backward kernels.  moe_encode_dx is decode_rows_kernel with unit gates
 // (encode_backward_data_kernel, tutel_moe_dispatch.cu:88-94).
 // ---------------------------------------------------------------------------------------
@@ -643,6 +727,26 @@ hipError_t run_decode_dg(const void* dy, const void* expert_out, const int32_t* 
     case LANCET_BF16: return decode_dg_launch<LANCET_BF16>(dy, expert_out, idx, loc, out, S, M, E, C, n, vec, st);
     default: return decode_dg_launch<LANCET_F16>(dy, expert_out, idx, loc, out, S, M, E, C, n, vec, st);
   }
+}
+
+hipError_t run_redispatch_expert_input(const PtrTable& bufs, const void* const* cnt_ptrs, int P, int le, int LE, int C,
+                                       int M, int G, uint64_t scale, void* out, int elem_bytes, hipStream_t st) {
+  const long rows = static_cast<long>(C) * G;
+  if (rows == 0 || M == 0) return hipSuccess;
+  CountTable ct;
+  for (int q = 0; q < kMaxPartitions; ++q) ct.p[q] = q < P ? static_cast<const uint64_t*>(cnt_ptrs[q]) : nullptr;
+  const unsigned blocks = static_cast<unsigned>((rows + kRowsPerBlock - 1) / kRowsPerBlock);
+  const size_t row_bytes = static_cast<size_t>(M) * elem_bytes;
+  bool vec = row_bytes % 16 == 0 && aligned16(out);
+  for (int q = 0; q < P; ++q) vec = vec && aligned16(bufs.p[q]);
+  if (elem_bytes == 4) {
+    if (vec) redispatch_expert_input_kernel<uint32_t, true><<<blocks, kTile, 0, st>>>(bufs, ct, P, le, LE, C, M, G, scale, static_cast<uint32_t*>(out));
+    else redispatch_expert_input_kernel<uint32_t, false><<<blocks, kTile, 0, st>>>(bufs, ct, P, le, LE, C, M, G, scale, static_cast<uint32_t*>(out));
+  } else {
+    if (vec) redispatch_expert_input_kernel<uint16_t, true><<<blocks, kTile, 0, st>>>(bufs, ct, P, le, LE, C, M, G, scale, static_cast<uint16_t*>(out));
+    else redispatch_expert_input_kernel<uint16_t, false><<<blocks, kTile, 0, st>>>(bufs, ct, P, le, LE, C, M, G, scale, static_cast<uint16_t*>(out));
+  }
+  return hipGetLastError();
 }
 
 }  // namespace lancet

@@ -299,6 +299,42 @@ def moe_redispatch(data, indices_locations, workspace=None, out=None):
     return out
 
 
+def moe_redispatch_expert_input(data, recv_cnts, local_expert_id, n_local_experts, recv_cnts_scale=1, out=None):
+    """raf.op.moe_redispatch_expert_input(data: tuple, recv_cnts: tuple, local_expert_id, n_local_experts,
+    recv_cnts_scale=1): data[p] is [C, G, M] (or [C, 1, G, M] / [C*G, M]), recv_cnts[p] uint64 [G*LE]."""
+    lib = capi.load()
+    P = len(data)
+    _need(P >= 1 and len(recv_cnts) == P, "data and recv_cnts must have one entry per partition")
+    for d in data:
+        _dev(d, "data")
+        _need(d.shape == data[0].shape and d.dtype == data[0].dtype, "partition buffers must agree")
+    for c in recv_cnts:
+        _dev(c, "recv_cnts")
+        _need(c.dim() == 1 and c.dtype in (torch.int64, getattr(torch, "uint64", torch.int64)) and
+              c.shape == recv_cnts[0].shape, "Expected recv_cnts to be 1-D 64-bit counts of equal length.")
+    shape = tuple(data[0].shape)
+    n = recv_cnts[0].shape[0]
+    _need(n % n_local_experts == 0, "recv_cnts length must be G x n_local_experts")
+    if len(shape) == 4:      # [C, 1, G, M]
+        _need(shape[1] == 1, "4D Input data should have dim 1 at axis 1.")
+        Cap, G, M = shape[0], shape[2], shape[3]
+    elif len(shape) == 3:    # [C, G, M]
+        Cap, G, M = shape
+    else:                    # [C x G, M]
+        _need(len(shape) == 2, "Input data should be 2,3 or 4-D.")
+        G = n // n_local_experts
+        Cap, M = shape[0] // G, shape[1]
+    _need(n // G == n_local_experts, "Expected input recv_cnts to be 1D of size G x LE.")
+    if out is None:
+        out = torch.empty(shape, dtype=data[0].dtype, device=data[0].device)
+    dptrs = capi.ptr_array([d.data_ptr() for d in data])
+    cptrs = capi.ptr_array([c.data_ptr() for c in recv_cnts])
+    st = lib.lancet_moe_redispatch_expert_input(dptrs, cptrs, P, int(local_expert_id), int(n_local_experts), Cap, M, G,
+                                                int(recv_cnts_scale), _dtype_code(data[0]), _p(out), _stream())
+    capi.check(st, "lancet_moe_redispatch_expert_input")
+    return out
+
+
 # ------------------------------------------------------------------------------------ LANS
 class LansPlan:
     """Owns the native plan of one parameter set (what the reference's LansImpl constructor

@@ -392,6 +392,88 @@ class MoeDecode : public OpEnv {
 };
 
 // =====================================================================================
+// raf.op.moe_redispatch_expert_input(data, recv_cnts, local_expert_id, n_local_experts, recv_cnts_scale=1)
+// (src/op/declare/moe.cc:140-163; src/op/dialect/cuda/moe.cc:945-1073)
+// =====================================================================================
+namespace {
+struct ExpertInputShape {
+  int64_t C, G, M;
+};
+ExpertInputShape ExpertInputDims(const Tensor& d0, const Tensor& c0, int64_t LE) {
+  RAF_CHECK(c0.shape.size() == 1, "Expected input recv_cnts to be 1D.");
+  RAF_CHECK((c0.dtype.code == DTypeCode::kUInt || c0.dtype.code == DTypeCode::kInt) && c0.dtype.bits == 64,
+            "recv_cnts must be 64-bit counts");
+  ExpertInputShape s;
+  if (d0.shape.size() == 4) {  // [C, 1, G, M]
+    RAF_CHECK(d0.shape[1] == 1, "4D Input data should have dim 1 at axis 1.");
+    s.C = d0.shape[0], s.G = d0.shape[2], s.M = d0.shape[3];
+  } else if (d0.shape.size() == 3) {  // [C, G, M]
+    s.C = d0.shape[0], s.G = d0.shape[1], s.M = d0.shape[2];
+  } else {  // [C x G, M]
+    RAF_CHECK(d0.shape.size() == 2, "Input data should be 2,3 or 4-D.");
+    RAF_CHECK(LE > 0 && c0.shape[0] >= LE, "bad n_local_experts");
+    s.G = c0.shape[0] / LE;
+    s.C = d0.shape[0] / s.G, s.M = d0.shape[1];
+  }
+  RAF_CHECK(s.G > 0 && c0.shape[0] / s.G == LE, "Expected input recv_cnts to be 1D of size G x LE.");
+  return s;
+}
+}  // namespace
+
+void MoeRedispatchExpertInputDeclare(CallValues& call) {
+  RAF_CHECK(call.args.size() >= 4, "moe_redispatch_expert_input(data, recv_cnts, local_expert_id, n_local_experts, recv_cnts_scale=1)");
+  const auto& bufs = call.args[0].AsTuple();
+  const auto& cnts = call.args[1].AsTuple();
+  RAF_CHECK(!bufs.empty() && bufs.size() == cnts.size(), "data and recv_cnts must have one entry per partition");
+  const Tensor& d0 = bufs[0].AsTensor();
+  ExpertInputDims(d0, cnts[0].AsTensor(), call.args[3].AsInt());
+  DTypeToLancet(d0.dtype);
+  // data dtype (Declare hard-codes float32, declare/moe.cc:161, which cannot hold for 16-bit buffers)
+  call.out = Value::MakeTensor(MakeOut(d0.device_id, d0.dtype.code, d0.dtype.bits, d0.shape));
+  call.device_id = d0.device_id;
+}
+
+class MoeRedispatchExpertInput : public OpEnv {
+ public:
+  explicit MoeRedispatchExpertInput(const CallValues& cv) {
+    const auto& bufs = cv.args[0].AsTuple();
+    const auto& cnts = cv.args[1].AsTuple();
+    n_partitions_ = static_cast<int>(cnts.size());
+    RAF_CHECK(n_partitions_ >= 1 && n_partitions_ <= LANCET_MAX_PARTITIONS, "unsupported number of partitions");
+    local_expert_id_ = static_cast<int>(cv.args[2].AsInt());
+    dim_LE_ = static_cast<int>(cv.args[3].AsInt());
+    recv_cnts_scale_ = static_cast<int>(OptInt(cv, 4, 1));
+    const Tensor& d0 = bufs[0].AsTensor();
+    shape_ = ExpertInputDims(d0, cnts[0].AsTensor(), dim_LE_);
+    dtype_ = DTypeToLancet(d0.dtype);
+    device_id_ = d0.device_id;
+    this->arg_indices = {0, 1};
+  }
+  void Execute(const CallValues& cv) override { Execute({cv.args[0], cv.args[1]}, cv.out); }
+  void Execute(const std::vector<Value>& inputs, Value output) override {
+    const auto& bufs = inputs[0].AsTuple();
+    const auto& cnts = inputs[1].AsTuple();
+    RAF_CHECK(static_cast<int>(cnts.size()) == n_partitions_ && bufs.size() == cnts.size(), "partition count changed");
+    std::vector<const void*> dptrs;
+    std::vector<const uint64_t*> cptrs;
+    for (int i = 0; i < n_partitions_; ++i) {
+      dptrs.push_back(bufs[i].AsTensor().data);
+      cptrs.push_back(static_cast<const uint64_t*>(cnts[i].AsTensor().data));
+    }
+    CheckStatus(lancet_moe_redispatch_expert_input(dptrs.data(), cptrs.data(), n_partitions_, local_expert_id_, dim_LE_,
+                                                   shape_.C, shape_.M, shape_.G, recv_cnts_scale_, dtype_,
+                                                   output.AsTensor().data, GetStream(device_id_)),
+                "lancet_moe_redispatch_expert_input");
+  }
+  std::string name() const override { return "raf.op.hip.moe_redispatch_expert_input"; }
+  static OpEnv* make(const CallValues& cv) { return new MoeRedispatchExpertInput(cv); }
+
+ private:
+  ExpertInputShape shape_;
+  int n_partitions_, local_expert_id_, dim_LE_, recv_cnts_scale_, dtype_, device_id_;
+};
+
+// =====================================================================================
 // backward ops: raf.op.moe_encode_dx / moe_encode_dg / moe_decode_dx / moe_decode_dg
 // (src/op/declare/moe.cc:165-247; src/op/dialect/cuda/moe.cc:1075-1225, 1313-1481; gradients wired in
 // src/op/grad/moe.cc:30-93).  Gate-side tensors are float32; an optional trailing top_k selects the
@@ -590,6 +672,9 @@ RAF_OP_ENV_MAKER("raf.op.hip.moe_redispatch", MoeRedispatch::make);
 RAF_REGISTER_DIALECT_OP(hip, moe_decode, 20);
 RAF_OP_ENV_MAKER("raf.op.hip.moe_decode", MoeDecode::make);
 
+RAF_OP_DECLARE("raf.op.moe_redispatch_expert_input", MoeRedispatchExpertInputDeclare);
+RAF_REGISTER_DIALECT_OP(hip, moe_redispatch_expert_input, 20);
+RAF_OP_ENV_MAKER("raf.op.hip.moe_redispatch_expert_input", MoeRedispatchExpertInput::make);
 RAF_OP_DECLARE("raf.op.moe_encode_dx", MoeEncodeDxDeclare);
 RAF_OP_DECLARE("raf.op.moe_encode_dg", MoeEncodeDgDeclare);
 RAF_OP_DECLARE("raf.op.moe_decode_dx", MoeDecodeDxDeclare);

@@ -389,3 +389,26 @@ def moe_decode_dg(dy, expert_out, indloc, k=1):
     b = _to_f32(dy).astype(np.float64)
     out[ok] = np.einsum("nm,nm->n", a[indloc[0][ok], indloc[1][ok]], b[tok[ok]])
     return out.astype(np.float32)
+
+
+# --------------------------------------------------------------------------
+# moe_redispatch_expert_input (moe.cc:945-1073, tutel_moe_dispatch.cu:436-456)
+# Pinned in tests/test_oracle_moe.py by the reference's own protocol: the merge of P row-compacted
+# partitions equals the un-partitioned buffer on the received rows.
+# --------------------------------------------------------------------------
+def moe_redispatch_expert_input(bufs, recv_cnts, local_expert_id, n_local_experts, scale=1):
+    """bufs[p]: [C, G, M]; recv_cnts[p]: uint64 [G*LE] element counts.  For source g the element
+    streams of the partitions are concatenated; stream element x -> out[x // M, g, x % M].  Rows the
+    reference leaves untouched are zero here."""
+    C, G, M = bufs[0].shape
+    out = np.zeros((C, G, M), bufs[0].dtype)
+    for g in range(G):
+        stream = []
+        for buf, cnt in zip(bufs, recv_cnts):
+            n = int(cnt[g * n_local_experts + local_expert_id]) * scale
+            stream.append(buf[:, g, :].reshape(-1)[:n])
+        flat = np.concatenate(stream)[:C * M]
+        col = np.zeros(C * M, bufs[0].dtype)
+        col[:flat.size] = flat
+        out[:, g, :] = col.reshape(C, M)
+    return out

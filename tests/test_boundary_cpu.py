@@ -98,7 +98,7 @@ def test_op_layer_registers_the_six_operators(pkg):
     rx = pkg.raf_executor
     ops = rx.registered_ops()
     for name in ("moe_encode", "moe_encode_batch_prioritized", "moe_decode", "moe_merge_masks", "moe_redispatch", "lans",
-                 "moe_encode_dx", "moe_encode_dg", "moe_decode_dx", "moe_decode_dg"):
+                 "moe_encode_dx", "moe_encode_dg", "moe_decode_dx", "moe_decode_dg", "moe_redispatch_expert_input"):
         assert "raf.op." + name in ops
         assert rx.dispatch_list("raf.op." + name) == [("raf.op.hip." + name, 20)]   # plevel 20 as cuda/moe.cc:411
     with rx.dialect_preference(["cuda"]):

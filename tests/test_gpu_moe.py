@@ -342,3 +342,44 @@ def test_encode_without_tail_zero_fill_feeds_redispatch(pkg):
         used_a, used_b = a[2], b[2]
         ils.append(a[1]), bufs_a.append(a[4]), bufs_b.append(b[4])
     assert torch.equal(ops.moe_redispatch(bufs_a, ils), ops.moe_redispatch(bufs_b, ils))
+
+
+# ----------------------------------------------------------------------------- redispatch_expert_input
+@pytest.mark.parametrize("dt,M", [("f32", 64), ("bf16", 128), ("f32", 5)])
+@pytest.mark.parametrize("P", [2, 4])
+def test_redispatch_expert_input(pkg, dt, M, P):
+    """tests/python/distributed/test_partitioned_moe.py:99-196 with synthetic all-to-all outputs: every
+    source GPU's received rows are split over P partitions; the merge restores them.  Also counts that
+    are not a multiple of M (element-granular streams) and a scale factor."""
+    ops = pkg.ops
+    rng = np.random.default_rng(P * 10 + M)
+    C, G, LE, le = 40, 8, 2, 1
+    whole = rows_as_oracle(rng.standard_normal((C, G, M), dtype=np.float32), dt)
+    rows_total = rng.integers(0, C + 1, G)
+    rows_total[0], rows_total[1] = 0, C
+    bufs = [rows_as_oracle(rng.standard_normal((C, G, M), dtype=np.float32), dt) for _ in range(P)]
+    cnts = [np.zeros(G * LE, np.uint64) for _ in range(P)]
+    for g in range(G):
+        edges = [0] + list(np.sort(rng.integers(0, rows_total[g] + 1, P - 1))) + [rows_total[g]]
+        for p in range(P):
+            n = edges[p + 1] - edges[p]
+            bufs[p][:n, g, :] = whole[edges[p]:edges[p + 1], g, :]
+            cnts[p][g * LE + le] = n * M
+            cnts[p][g * LE + (1 - le)] = 7 * M
+    d_bufs = [rows_to_torch(b, dt) for b in bufs]
+    d_cnts = [dev(c.astype(np.int64)) for c in cnts]
+    want = mo.moe_redispatch_expert_input(bufs, cnts, le, LE)
+    got = ops.moe_redispatch_expert_input(d_bufs, d_cnts, le, LE)
+    np.testing.assert_array_equal(to_np(got), want)
+    for g in range(G):
+        np.testing.assert_array_equal(want[:rows_total[g], g], whole[:rows_total[g], g])
+    # through the op layer, 4-D [C, 1, G, M] form
+    ex = pkg.raf_executor.Executor()
+    got4 = ex("raf.op.moe_redispatch_expert_input", [b.reshape(C, 1, G, M) for b in d_bufs], d_cnts, le, LE)
+    assert tuple(got4.shape) == (C, 1, G, M)
+    np.testing.assert_array_equal(to_np(got4).reshape(C, G, M), want)
+    # element-granular streams with a scale factor
+    cnts2 = [rng.integers(0, (C * M) // (2 * P), G * LE).astype(np.uint64) for _ in range(P)]
+    want2 = mo.moe_redispatch_expert_input(bufs, cnts2, 0, LE, scale=2)
+    got2 = ops.moe_redispatch_expert_input(d_bufs, [dev(c.astype(np.int64)) for c in cnts2], 0, LE, recv_cnts_scale=2)
+    np.testing.assert_array_equal(to_np(got2), want2)

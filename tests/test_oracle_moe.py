@@ -345,3 +345,34 @@ def test_backward_ops_match_autograd_of_dense_forms(k):
     np.testing.assert_allclose(mo.moe_decode(eo32, g, il, k=k), combined.detach().numpy(), rtol=1e-5, atol=1e-6)
     np.testing.assert_allclose(mo.moe_decode_dx(Y.astype(np.float32), g, il, E, C, k), eo.grad.numpy(), rtol=1e-6, atol=1e-7)
     np.testing.assert_allclose(mo.moe_decode_dg(Y.astype(np.float32), eo32, il, k), gs.grad.numpy(), rtol=1e-5, atol=1e-6)
+
+
+# ---------------------------------------------------------------- redispatch_expert_input
+@pytest.mark.parametrize("P", [2, 4])
+def test_redispatch_expert_input_partitioned_equals_whole(P):
+    """tests/python/distributed/test_partitioned_moe.py:99-196: split every source GPU's received rows
+    into P partitions (each compacted from row 0 of its own buffer); the merge restores the whole."""
+    rng = np.random.default_rng(P)
+    C, G, M, LE, le = 12, 3, 4, 2, 1
+    whole = rng.standard_normal((C, G, M)).astype(np.float32)
+    rows_total = rng.integers(0, C + 1, G)
+    bufs = [np.full((C, G, M), 99.0, np.float32) for _ in range(P)]
+    cnts = [np.zeros(G * LE, np.uint64) for _ in range(P)]
+    for g in range(G):
+        cuts = np.sort(rng.integers(0, rows_total[g] + 1, P - 1))
+        edges = [0] + list(cuts) + [rows_total[g]]
+        for p in range(P):
+            n = edges[p + 1] - edges[p]
+            bufs[p][:n, g, :] = whole[edges[p]:edges[p + 1], g, :]
+            cnts[p][g * LE + le] = n * M
+            cnts[p][g * LE + (1 - le)] = 12345          # the other local expert's count must be ignored
+    out = mo.moe_redispatch_expert_input(bufs, cnts, le, LE)
+    for g in range(G):
+        np.testing.assert_array_equal(out[:rows_total[g], g], whole[:rows_total[g], g])
+        assert not out[rows_total[g]:, g].any()
+    # element-granular counts (not a multiple of M) and the scale factor
+    cnts2 = [np.array([3, 0, 5, 0, 0, 0], np.uint64), np.array([2, 0, 1, 0, 4, 0], np.uint64)]
+    out2 = mo.moe_redispatch_expert_input(bufs[:2], cnts2, 0, LE, scale=2)
+    want_g0 = np.concatenate([bufs[0][:, 0].reshape(-1)[:6], bufs[1][:, 0].reshape(-1)[:4]])
+    np.testing.assert_array_equal(out2[:, 0].reshape(-1)[:10], want_g0)
+    assert not out2[:, 0].reshape(-1)[10:].any()

@@ -62,6 +62,7 @@ extern "C" {
  * reference's own cost for this pattern, a full memset per partition buffer
  * (tutel_moe_dispatch.cu:466), is spent on. */
 #define LANCET_NO_TAIL_ZERO 2u
+#define LANCET_ZERO_TAIL 4u /* lancet_memcpy_cont_to_sparse_3d: clear what the copy leaves untouched */
 
 typedef void* lancet_stream_t;
 
@@ -162,6 +163,26 @@ int lancet_moe_redispatch_expert_input(const void* const* data, const uint64_t* 
                                        int local_expert_id, int n_local_experts, int64_t C, int64_t M,
                                        int64_t G, int recv_cnts_scale, int dtype, void* out,
                                        lancet_stream_t stream);
+
+/* ---- sparse <-> packed copies ------------------------------------------------------------
+ * Replace launch_memcpy_sparse_to_cont_3d / launch_memcpy_cont_to_sparse_3d (kernel_util.cuh:69-79;
+ * sparse_memcpy.cu:11-96).  Block b along `axis` (0 or 1) of the [dim0, dim1, dim2] buffer holds
+ * n_b = nelements_per_dim[b*stride + offset] * scale / shrink valid elements (in the block's own
+ * row-major order: [dim1, dim2] for axis 0, [dim0, dim2] for axis 1); the packed side is their
+ * concatenation.  n_counts = length of nelements_per_dim, dst_elems / src_elems = length of the packed
+ * array (both bound what the kernels touch; the reference takes neither).  Counts that exceed a block
+ * or the packed array are clipped.  cont_to_sparse leaves the rest of each block untouched, as the
+ * reference does, unless flags has LANCET_ZERO_TAIL. */
+int lancet_memcpy_sparse_to_cont_3d(const void* src, void* dst, const uint64_t* nelements_per_dim,
+                                    int64_t n_counts, int nelements_stride, int nelements_offset, int axis,
+                                    int64_t dim0, int64_t dim1, int64_t dim2, int64_t dst_elems,
+                                    int scale_element_size_by, int shrink_element_size_by, int dtype,
+                                    lancet_stream_t stream);
+int lancet_memcpy_cont_to_sparse_3d(const void* src, void* dst, const uint64_t* nelements_per_dim,
+                                    int64_t n_counts, int nelements_stride, int nelements_offset, int axis,
+                                    int64_t dim0, int64_t dim1, int64_t dim2, int64_t src_elems,
+                                    int scale_element_size_by, int shrink_element_size_by, int dtype,
+                                    unsigned flags, lancet_stream_t stream);
 
 /* ---- backward ops (raf.op.moe_encode_dx / _dg, raf.op.moe_decode_dx / _dg) ------------------
  * Gradients wired by src/op/grad/moe.cc:30-93.  Gate-side gradients are fp32 like gates_s; top_k = 2

@@ -12,6 +12,7 @@ LIB_PATH = os.path.join(HERE, "lib", "liblancet_hip.so")
 F32, BF16, F16 = 0, 1, 2
 GATE_IS_LOGITS = 1
 NO_TAIL_ZERO = 2
+ZERO_TAIL = 4
 LANS_SWEEPS, LANS_PIPELINED = 0, 1
 MAX_EXPERTS = 512
 MAX_PARTITIONS = 64
@@ -54,6 +55,10 @@ SIGNATURES = {
     "lancet_moe_decode": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp]),
     "lancet_moe_redispatch_expert_input": (_int, [C.POINTER(_vp), C.POINTER(_vp), _int, _int, _int, _i64, _i64, _i64,
                                                   _int, _int, _vp, _vp]),
+    "lancet_memcpy_sparse_to_cont_3d": (_int, [_vp, _vp, _vp, _i64, _int, _int, _int, _i64, _i64, _i64, _i64, _int, _int,
+                                               _int, _vp]),
+    "lancet_memcpy_cont_to_sparse_3d": (_int, [_vp, _vp, _vp, _i64, _int, _int, _int, _i64, _i64, _i64, _i64, _int, _int,
+                                               _int, _u32, _vp]),
     "lancet_moe_encode_dx": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp]),
     "lancet_moe_encode_dg": (_int, [_vp, _vp, _i64, _i64, _int, _vp, _vp]),
     "lancet_moe_decode_dx_workspace_bytes": (_sz, [_i64, _i64]),

@@ -271,6 +271,49 @@ extern "C" int lancet_moe_redispatch_expert_input(const void* const* data, const
                                         static_cast<uint64_t>(recv_cnts_scale), out, eb, S_(stream)));
 }
 
+// ---- sparse <-> packed copies ---------------------------------------------------------------
+namespace {
+int sparse_copy(const void* src, void* dst, const uint64_t* counts, int64_t n_counts, int stride, int offset, int axis,
+                int64_t dim0, int64_t dim1, int64_t dim2, int64_t cont_elems, int scale, int shrink, int dtype,
+                unsigned flags, bool to_cont, lancet_stream_t stream) {
+  const int eb = elem_bytes(dtype);
+  if (!eb) return LANCET_ERR_DTYPE;
+  if (axis != 0 && axis != 1) return LANCET_ERR_SHAPE;
+  if (dim0 < 0 || dim1 < 0 || dim2 < 0 || cont_elems < 0 || scale < 1 || shrink < 1 || stride < 1 || offset < 0)
+    return LANCET_ERR_SHAPE;
+  if (dim0 > 0x7fffffff || dim1 > 0x7fffffff || dim2 > 0x7fffffff) return LANCET_ERR_SHAPE;
+  const int64_t nblocks = axis == 0 ? dim0 : dim1;
+  const int64_t other = axis == 0 ? dim1 : dim0;
+  if (other > 0 && dim2 > 0x7fffffff / other) return LANCET_ERR_SHAPE;  // one block's elements fit in 31 bits
+  if (nblocks > 65535) return LANCET_ERR_SHAPE;                         // grid y
+  if (nblocks == 0 || other * dim2 == 0) return LANCET_OK;
+  if (!src || !dst || !counts) return LANCET_ERR_NULL;
+  if ((nblocks - 1) * stride + offset >= n_counts) return LANCET_ERR_SHAPE;
+  if (misaligned(src, eb) || misaligned(dst, eb) || misaligned(counts, 8)) return LANCET_ERR_ALIGN;
+  return rc(run_sparse_copy_3d(src, dst, counts, stride, offset, axis, static_cast<int>(dim0), static_cast<int>(dim1),
+                               static_cast<int>(dim2), static_cast<uint64_t>(cont_elems), static_cast<uint64_t>(scale),
+                               static_cast<uint64_t>(shrink), to_cont, (flags & LANCET_ZERO_TAIL) != 0, eb, S_(stream)));
+}
+}  // namespace
+
+extern "C" int lancet_memcpy_sparse_to_cont_3d(const void* src, void* dst, const uint64_t* nelements_per_dim,
+                                               int64_t n_counts, int nelements_stride, int nelements_offset, int axis,
+                                               int64_t dim0, int64_t dim1, int64_t dim2, int64_t dst_elems,
+                                               int scale_element_size_by, int shrink_element_size_by, int dtype,
+                                               lancet_stream_t stream) {
+  return sparse_copy(src, dst, nelements_per_dim, n_counts, nelements_stride, nelements_offset, axis, dim0, dim1, dim2,
+                     dst_elems, scale_element_size_by, shrink_element_size_by, dtype, 0u, true, stream);
+}
+
+extern "C" int lancet_memcpy_cont_to_sparse_3d(const void* src, void* dst, const uint64_t* nelements_per_dim,
+                                               int64_t n_counts, int nelements_stride, int nelements_offset, int axis,
+                                               int64_t dim0, int64_t dim1, int64_t dim2, int64_t src_elems,
+                                               int scale_element_size_by, int shrink_element_size_by, int dtype,
+                                               unsigned flags, lancet_stream_t stream) {
+  return sparse_copy(src, dst, nelements_per_dim, n_counts, nelements_stride, nelements_offset, axis, dim0, dim1, dim2,
+                     src_elems, scale_element_size_by, shrink_element_size_by, dtype, flags, false, stream);
+}
+
 // ---- backward ops -------------------------------------------------------------------
 extern "C" int lancet_moe_encode_dx(const void* dy, const int32_t* indices_locations, int64_t S, int64_t M,
                                     int64_t E, int64_t C, int top_k, int dtype, void* dx, lancet_stream_t stream) {

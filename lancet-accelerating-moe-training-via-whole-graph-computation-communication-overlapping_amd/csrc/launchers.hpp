@@ -67,4 +67,11 @@ hipError_t run_redispatch_rows(const PtrTable& bufs, int P, int M, int C, int E,
 hipError_t run_redispatch_expert_input(const PtrTable& bufs, const void* const* cnt_ptrs, int P, int le, int LE, int C,
                                        int M, int G, uint64_t scale, void* out, int elem_bytes, hipStream_t st);
 
+// ---- sparse <-> packed copies (sparse_copy.hip) -----------------------------------------
+// counts[b*stride + offset] elements of block b along `axis` (0 or 1) of a [dim0, dim1, dim2] buffer;
+// cont_cap = elements the packed stream holds.  to_cont: buffer -> stream.
+hipError_t run_sparse_copy_3d(const void* src, void* dst, const uint64_t* counts, int stride, int offset, int axis,
+                              int dim0, int dim1, int dim2, uint64_t cont_cap, uint64_t scale, uint64_t shrink,
+                              bool to_cont, bool zero_tail, int elem_bytes, hipStream_t st);
+
 }  // namespace lancet

@@ -335,6 +335,44 @@ def moe_redispatch_expert_input(data, recv_cnts, local_expert_id, n_local_expert
     return out
 
 
+def _sparse_copy_args(buf, packed, nelements_per_dim, nelements_stride, nelements_offset, axis):
+    _dev(buf, "sparse buffer"), _dev(packed, "packed array"), _dev(nelements_per_dim, "nelements_per_dim")
+    _need(buf.dim() == 3, "the sparse buffer must be 3-D")
+    _need(axis in (0, 1), "Axis %d not supported." % axis)
+    _need(buf.dtype == packed.dtype and buf.is_contiguous() and packed.is_contiguous(), "dtype / layout mismatch")
+    _need(nelements_per_dim.dtype in (torch.int64, getattr(torch, "uint64", torch.int64)) and
+          nelements_per_dim.is_contiguous(), "nelements_per_dim must be contiguous 64-bit counts")
+    return tuple(buf.shape), packed.numel(), nelements_per_dim.numel()
+
+
+def memcpy_sparse_to_cont_3d(src, dst, nelements_per_dim, nelements_stride=1, nelements_offset=0, axis=0,
+                             scale_element_size_by=1, shrink_element_size_by=1):
+    """launch_memcpy_sparse_to_cont_3d (src/op/dialect/cuda/kernels/sparse_memcpy.cu:62-85): packs the valid
+    elements of every block along `axis` of src[dim0, dim1, dim2] into dst (written in place, returned)."""
+    lib = capi.load()
+    (d0, d1, d2), n_dst, n_cnt = _sparse_copy_args(src, dst, nelements_per_dim, nelements_stride, nelements_offset, axis)
+    st = lib.lancet_memcpy_sparse_to_cont_3d(_p(src), _p(dst), _p(nelements_per_dim), n_cnt, int(nelements_stride),
+                                             int(nelements_offset), int(axis), d0, d1, d2, n_dst,
+                                             int(scale_element_size_by), int(shrink_element_size_by), _dtype_code(src),
+                                             _stream())
+    capi.check(st, "lancet_memcpy_sparse_to_cont_3d")
+    return dst
+
+
+def memcpy_cont_to_sparse_3d(src, dst, nelements_per_dim, nelements_stride=1, nelements_offset=0, axis=0,
+                             scale_element_size_by=1, shrink_element_size_by=1, zero_tail=False):
+    """launch_memcpy_cont_to_sparse_3d (sparse_memcpy.cu:62-85): the inverse; dst[dim0, dim1, dim2] is written in
+    place.  zero_tail clears the part of every block the copy does not reach (the reference leaves it)."""
+    lib = capi.load()
+    (d0, d1, d2), n_src, n_cnt = _sparse_copy_args(dst, src, nelements_per_dim, nelements_stride, nelements_offset, axis)
+    st = lib.lancet_memcpy_cont_to_sparse_3d(_p(src), _p(dst), _p(nelements_per_dim), n_cnt, int(nelements_stride),
+                                             int(nelements_offset), int(axis), d0, d1, d2, n_src,
+                                             int(scale_element_size_by), int(shrink_element_size_by), _dtype_code(dst),
+                                             capi.ZERO_TAIL if zero_tail else 0, _stream())
+    capi.check(st, "lancet_memcpy_cont_to_sparse_3d")
+    return dst
+
+
 # ------------------------------------------------------------------------------------ LANS
 class LansPlan:
     """Owns the native plan of one parameter set (what the reference's LansImpl constructor

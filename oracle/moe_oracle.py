@@ -412,3 +412,55 @@ def moe_redispatch_expert_input(bufs, recv_cnts, local_expert_id, n_local_expert
         col[:flat.size] = flat
         out[:, g, :] = col.reshape(C, M)
     return out
+
+
+# ----------------------------------------------------------------------------- sparse <-> packed copies
+def sparse_copy_extents(nelements_per_dim, stride, offset, nblocks, scale=1, shrink=1):
+    """(off_b, n_b) of sparse_memcpy.cu:16-36: the counts of the blocks before b are summed first and the sum
+    is then scaled; the block's own count is scaled by itself."""
+    c = [int(nelements_per_dim[b * stride + offset]) for b in range(nblocks)]
+    offs, run = [], 0
+    for b in range(nblocks):
+        offs.append(run * scale // shrink)
+        run += c[b]
+    return offs, [x * scale // shrink for x in c]
+
+
+def _sparse_block_view(buf, axis, b):
+    # the block's elements in stream order: INDEX3Ddim0 / INDEX3Ddim1, sparse_memcpy.cu:43-46
+    return buf[b].reshape(-1) if axis == 0 else buf[:, b, :].reshape(-1)
+
+
+def memcpy_sparse_to_cont_3d(src, dst, nelements_per_dim, stride=1, offset=0, axis=0, scale=1, shrink=1):
+    """memcpy_sparse_to_cont_3d_dim{0,1}_kernel, sparse_memcpy.cu:48-53: returns dst (1-D) with the packed
+    stream written; what the stream does not cover keeps dst's values.  Counts are clipped to the block and
+    to dst (the source would run out of bounds)."""
+    out = np.array(dst, copy=True).reshape(-1)
+    nb = src.shape[axis]
+    offs, ns = sparse_copy_extents(nelements_per_dim, stride, offset, nb, scale, shrink)
+    for b in range(nb):
+        blk = _sparse_block_view(src, axis, b)
+        n = max(0, min(ns[b], blk.size, out.size - offs[b]))
+        out[offs[b]:offs[b] + n] = blk[:n]
+    return out
+
+
+def memcpy_cont_to_sparse_3d(src, dst, nelements_per_dim, stride=1, offset=0, axis=0, scale=1, shrink=1,
+                             zero_tail=False):
+    """memcpy_cont_to_sparse_3d_dim{0,1}_kernel, sparse_memcpy.cu:55-60: returns dst (3-D) with every block's
+    first n_b elements taken from the packed stream; the rest keeps dst's values (zero with zero_tail)."""
+    out = np.array(dst, copy=True)
+    flat = np.asarray(src).reshape(-1)
+    nb = out.shape[axis]
+    offs, ns = sparse_copy_extents(nelements_per_dim, stride, offset, nb, scale, shrink)
+    for b in range(nb):
+        blk = np.array(_sparse_block_view(out, axis, b), copy=True)
+        n = max(0, min(ns[b], blk.size, flat.size - offs[b]))
+        blk[:n] = flat[offs[b]:offs[b] + n]
+        if zero_tail:
+            blk[n:] = 0
+        if axis == 0:
+            out[b] = blk.reshape(out.shape[1], out.shape[2])
+        else:
+            out[:, b, :] = blk.reshape(out.shape[0], out.shape[2])
+    return out

@@ -58,6 +58,13 @@ def test_workspace_sizes_and_argument_rejection(pkg):
     assert st == capi.ERR_PARTITION
     ptrs = capi.ptr_array([16] * 70)
     assert lib.lancet_moe_merge_masks(ptrs, 70, 8, 2, one, one, 1 << 20, None) == capi.ERR_PARTITION
+    # sparse <-> packed copies: axis 2 is not supported (sparse_memcpy.cu:78-81), counts must cover every block
+    assert lib.lancet_memcpy_sparse_to_cont_3d(one, one, one, 8, 1, 0, 2, 4, 4, 4, 64, 1, 1, capi.F32, None) == capi.ERR_SHAPE
+    assert lib.lancet_memcpy_sparse_to_cont_3d(one, one, one, 4, 2, 0, 0, 4, 4, 4, 64, 1, 1, capi.F32, None) == capi.ERR_SHAPE
+    assert lib.lancet_memcpy_sparse_to_cont_3d(one, one, one, 8, 1, 0, 0, 4, 4, 4, 64, 0, 1, capi.F32, None) == capi.ERR_SHAPE
+    assert lib.lancet_memcpy_cont_to_sparse_3d(one, None, one, 8, 1, 0, 0, 4, 4, 4, 64, 1, 1, capi.F32, 0, None) == capi.ERR_NULL
+    assert lib.lancet_memcpy_cont_to_sparse_3d(one, one, C.c_void_p(12), 8, 1, 0, 1, 4, 4, 4, 64, 1, 1, capi.BF16, 0, None) == capi.ERR_ALIGN
+    assert lib.lancet_memcpy_cont_to_sparse_3d(one, one, one, 8, 1, 0, 1, 4, 0, 4, 64, 1, 1, capi.BF16, 0, None) == capi.OK
     assert lib.lancet_lans_plan_destroy(None) == capi.ERR_PLAN
     assert "workspace" in capi.status_string(capi.ERR_WORKSPACE)
 

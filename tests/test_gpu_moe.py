@@ -383,3 +383,72 @@ def test_redispatch_expert_input(pkg, dt, M, P):
     want2 = mo.moe_redispatch_expert_input(bufs, cnts2, 0, LE, scale=2)
     got2 = ops.moe_redispatch_expert_input(d_bufs, [dev(c.astype(np.int64)) for c in cnts2], 0, LE, recv_cnts_scale=2)
     np.testing.assert_array_equal(to_np(got2), want2)
+
+
+# ----------------------------------------------------------------------------- sparse <-> packed copies
+@pytest.mark.parametrize("dt,dims", [("f32", (6, 10, 16)), ("bf16", (8, 12, 24)), ("bf16", (5, 7, 9)), ("f32", (3, 4, 5))])
+@pytest.mark.parametrize("axis", [0, 1])
+@pytest.mark.parametrize("aligned", [True, False])
+def test_sparse_packed_copies(pkg, dt, dims, axis, aligned):
+    """memcpy_sparse_to_cont_3d / memcpy_cont_to_sparse_3d (sparse_memcpy.cu:11-96) against the oracle, with
+    counts read through a stride and an offset; `aligned` makes every count a multiple of dim2 (whole rows, what
+    elements_per_expert holds), otherwise counts are arbitrary and block offsets fall inside 16-byte granules."""
+    ops = pkg.ops
+    rng = np.random.default_rng(sum(dims) + axis + 2 * aligned)
+    d0, d1, d2 = dims
+    nb = dims[axis]
+    rows = d1 if axis == 0 else d0
+    stride, offset = 3, 2
+    cnt = rng.integers(0, 1000, nb * stride).astype(np.uint64)
+    picked = rng.integers(0, rows + 1, nb) * d2 if aligned else rng.integers(0, rows * d2 + 1, nb)
+    picked[0] = 0 if nb > 1 else picked[0]
+    picked[-1] = rows * d2
+    cnt[offset::stride] = picked
+    total = int(picked.sum())
+    src = rows_as_oracle(rng.standard_normal(dims, dtype=np.float32), dt)
+    dst0 = rows_as_oracle(rng.standard_normal(total + 5, dtype=np.float32), dt)
+    d_cnt = dev(cnt.astype(np.int64))
+    want = mo.memcpy_sparse_to_cont_3d(src, dst0, cnt, stride, offset, axis)
+    got = ops.memcpy_sparse_to_cont_3d(rows_to_torch(src, dt), rows_to_torch(dst0, dt), d_cnt, stride, offset, axis)
+    np.testing.assert_array_equal(to_np(got), want)
+    for zero_tail in (False, True):
+        buf0 = rows_as_oracle(rng.standard_normal(dims, dtype=np.float32), dt)
+        want3 = mo.memcpy_cont_to_sparse_3d(want, buf0, cnt, stride, offset, axis, zero_tail=zero_tail)
+        got3 = ops.memcpy_cont_to_sparse_3d(rows_to_torch(want, dt), rows_to_torch(buf0, dt), d_cnt, stride, offset,
+                                            axis, zero_tail=zero_tail)
+        np.testing.assert_array_equal(to_np(got3), want3)
+    # a packed array shorter than the counts say: the copy stops at its end
+    short = max(total - d2 - 1, 0)
+    want_s = mo.memcpy_sparse_to_cont_3d(src, dst0[:short], cnt, stride, offset, axis)
+    got_s = ops.memcpy_sparse_to_cont_3d(rows_to_torch(src, dt), rows_to_torch(dst0[:short].copy(), dt), d_cnt, stride,
+                                         offset, axis)
+    np.testing.assert_array_equal(to_np(got_s), want_s)
+
+
+def test_sparse_packed_copies_scale_and_encode_counts(pkg):
+    """Counts straight from an encode (elements_per_expert) pack the dispatched buffer; scale/shrink reinterpret
+    the counts for another element size (sparse_memcpy.cu:33-36)."""
+    ops = pkg.ops
+    rng = np.random.default_rng(11)
+    S, M, E = 4096, 256, 16
+    x = rng.standard_normal((S, M), dtype=np.float32)
+    gate = mo.softmax_rows(rng.standard_normal((S, E), dtype=np.float32) * 2)
+    gates_s, indloc, used, elems, disp = ops.moe_encode(dev(x), dev(gate), torch.zeros(E, dtype=torch.int32, device="cuda"), 0.8)
+    kept = int(used.sum().item())
+    assert kept < S
+    packed = ops.memcpy_sparse_to_cont_3d(disp, torch.empty(kept * M, device="cuda"), elems)
+    want = np.concatenate([to_np(disp)[e, :int(used[e])].reshape(-1) for e in range(E)])
+    np.testing.assert_array_equal(to_np(packed), want)
+    back = ops.memcpy_cont_to_sparse_3d(packed, torch.full_like(disp, 3.0), elems, zero_tail=True)
+    np.testing.assert_array_equal(to_np(back), to_np(disp))
+    # the same counts, read as fp32 elements, drive a bf16 buffer of twice the width (scale 2)
+    disp16 = rows_as_oracle(rng.standard_normal((E, disp.shape[1], 2 * M), dtype=np.float32), "bf16")
+    cnt = to_np(elems).astype(np.uint64)
+    want16 = mo.memcpy_sparse_to_cont_3d(disp16, np.zeros(2 * kept * M, disp16.dtype), cnt, scale=2)
+    got16 = ops.memcpy_sparse_to_cont_3d(rows_to_torch(disp16, "bf16"), rows_to_torch(np.zeros(2 * kept * M, disp16.dtype), "bf16"),
+                                         elems, scale_element_size_by=2)
+    np.testing.assert_array_equal(to_np(got16), want16)
+    want_h = mo.memcpy_sparse_to_cont_3d(disp16, np.zeros(kept * M, disp16.dtype), cnt, scale=1, shrink=2)
+    got_h = ops.memcpy_sparse_to_cont_3d(rows_to_torch(disp16, "bf16"), rows_to_torch(np.zeros(kept * M, disp16.dtype), "bf16"),
+                                         elems, shrink_element_size_by=2)
+    np.testing.assert_array_equal(to_np(got_h), want_h)

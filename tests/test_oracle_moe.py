@@ -376,3 +376,62 @@ def test_redispatch_expert_input_partitioned_equals_whole(P):
     want_g0 = np.concatenate([bufs[0][:, 0].reshape(-1)[:6], bufs[1][:, 0].reshape(-1)[:4]])
     np.testing.assert_array_equal(out2[:, 0].reshape(-1)[:10], want_g0)
     assert not out2[:, 0].reshape(-1)[10:].any()
+
+
+# ----------------------------------------------------------------------------- sparse <-> packed copies
+def _brute_sparse_to_cont(src, dst, cnt, stride, offset, axis, scale, shrink):
+    """Element-by-element restatement of the copy as one thread would do it (block offset = scaled sum of the
+    earlier counts; 3-D position from the flat stream position), independent of the oracle's slicing."""
+    d0, d1, d2 = src.shape
+    out = dst.copy()
+    for b in range(src.shape[axis]):
+        before = sum(int(cnt[j * stride + offset]) for j in range(b)) * scale // shrink
+        n = int(cnt[b * stride + offset]) * scale // shrink
+        for t in range(n):
+            if axis == 0:
+                v = src[b, t // d2, t % d2]
+            else:
+                v = src[t // d2, b, t % d2]
+            out[before + t] = v
+    return out
+
+
+@pytest.mark.parametrize("axis", [0, 1])
+@pytest.mark.parametrize("scale,shrink", [(1, 1), (2, 1), (1, 2), (3, 2)])
+def test_sparse_copy_matches_elementwise_definition(axis, scale, shrink):
+    rng = np.random.default_rng(axis * 7 + scale + shrink)
+    d0, d1, d2, stride, offset = 5, 4, 6, 3, 1
+    src = rng.standard_normal((d0, d1, d2)).astype(np.float32)
+    nb = src.shape[axis]
+    cap = (d1 if axis == 0 else d0) * d2
+    cnt = np.zeros(nb * stride, np.uint64)
+    cnt[offset::stride] = rng.integers(0, cap * shrink // scale + 1, nb)
+    cnt[(offset + 1) % stride::stride] = 999          # other columns must not be read
+    total = sum(int(c) for c in cnt[offset::stride]) * scale // shrink
+    dst = np.full(total + 3, -7.0, np.float32)
+    got = mo.memcpy_sparse_to_cont_3d(src, dst, cnt, stride, offset, axis, scale, shrink)
+    np.testing.assert_array_equal(got, _brute_sparse_to_cont(src, dst, cnt, stride, offset, axis, scale, shrink))
+    # inverse: the valid part of every block comes back, the rest keeps the destination's bytes
+    back = mo.memcpy_cont_to_sparse_3d(got, np.full_like(src, 5.0), cnt, stride, offset, axis, scale, shrink)
+    offs, ns = mo.sparse_copy_extents(cnt, stride, offset, nb, scale, shrink)
+    for b in range(nb):
+        a = (src[b] if axis == 0 else src[:, b, :]).reshape(-1)
+        r = (back[b] if axis == 0 else back[:, b, :]).reshape(-1)
+        np.testing.assert_array_equal(r[:ns[b]], a[:ns[b]])
+        assert (r[ns[b]:] == 5.0).all()
+    z = mo.memcpy_cont_to_sparse_3d(got, np.full_like(src, 5.0), cnt, stride, offset, axis, scale, shrink, zero_tail=True)
+    assert ((z == back) | (z == 0)).all() and (z[back == 5.0] == 0).all()
+
+
+def test_sparse_copy_packs_encode_output():
+    """elements_per_expert of an encode is exactly the count array the copy is keyed by: packing [E, C, M]
+    along axis 0 gives the kept rows of every expert back to back, and unpacking restores the buffer."""
+    rng = np.random.default_rng(3)
+    S, M, E = 96, 8, 4
+    x = rng.standard_normal((S, M)).astype(np.float32)
+    gate = mo.softmax_rows(rng.standard_normal((S, E)).astype(np.float32))
+    _, _, used, elems, disp = mo.moe_encode(x, gate, np.zeros(E, np.int32), 0.75)
+    packed = mo.memcpy_sparse_to_cont_3d(disp, np.zeros(int(elems.sum()), np.float32), elems)
+    want = np.concatenate([disp[e, :used[e]].reshape(-1) for e in range(E)])
+    np.testing.assert_array_equal(packed, want)
+    np.testing.assert_array_equal(mo.memcpy_cont_to_sparse_3d(packed, np.zeros_like(disp), elems), disp)

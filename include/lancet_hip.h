@@ -266,14 +266,18 @@ int lancet_lans_plan_destroy(lancet_lans_plan_t plan);
 int lancet_lans_step(lancet_lans_plan_t plan, const float* const* g, float* const* p,
                      float* const* m, float* const* v, int step_host, const float* step_dev,
                      const lancet_lans_hyper* hyper, lancet_stream_t stream);
-/* Schedules of the step; both give the same bits.  LANCET_LANS_SWEEPS (default): three whole-state
- * sweeps with two per-tensor reductions between them.  LANCET_LANS_PIPELINED: one persistent kernel
- * that runs the three phases of neighbouring tensor bundles concurrently (slower on MI355X today:
- * the cross-XCD release fence it needs per task outweighs the cache reuse it is after). */
+/* Schedules of the step.  LANCET_LANS_SWEEPS (default): three whole-state sweeps with two per-tensor
+ * reductions between them (52 B/param of traffic).  LANCET_LANS_RESIDENT: one persistent kernel that keeps
+ * each chunk on chip across the two reductions (28 B/param); every tensor must fit on the chip at once
+ * (lancet_lans_plan_resident_capacity), else set_schedule returns LANCET_ERR_SHAPE and the plan keeps its
+ * schedule.  Each schedule is deterministic; the two agree to fp32 rounding of the per-chunk sums. */
 #define LANCET_LANS_SWEEPS 0
-#define LANCET_LANS_PIPELINED 1
+#define LANCET_LANS_RESIDENT 1
 int lancet_lans_plan_set_schedule(lancet_lans_plan_t plan, int schedule);
-/* Reads (synchronously) the plan's error word: 1 when a bounded wait of the pipelined schedule
+/* workgroups: chunks (of 8192 parameters) the resident schedule holds at once on this device = the
+ * largest tensor it accepts; max_tensor_chunks: chunks of the plan's largest tensor.  Either may be NULL. */
+int lancet_lans_plan_resident_capacity(lancet_lans_plan_t plan, int* workgroups, int* max_tensor_chunks);
+/* Reads (synchronously) the plan's error word: 1 when a bounded wait of the resident schedule
  * gave up (results of that step are undefined). */
 int lancet_lans_plan_error(lancet_lans_plan_t plan, lancet_stream_t stream, int* error_out);
 
@@ -282,11 +286,9 @@ int lancet_lans_plan_error(lancet_lans_plan_t plan, lancet_stream_t stream, int*
  * norms4xT, a device buffer of 4*T floats, asynchronously on `stream`. */
 int lancet_lans_plan_norms(lancet_lans_plan_t plan, float* norms4xT, lancet_stream_t stream);
 
-/* Host-only view of what a plan builds for `numels` (no device needed): the task queue of the
- * pipelined schedule (phase << 30 | chunk) and the chunk -> tensor map.  Returns the number of
- * tasks (3 x chunks); fills at most `capacity` entries of each output (either may be NULL). */
-int64_t lancet_lans_debug_task_queue(const int64_t* numels, int T, uint32_t* tasks_out,
-                                     int32_t* chunk_tensor_out, int64_t capacity);
+/* Host-only view of what a plan builds for `numels` (no device needed): the chunk -> tensor map.
+ * Returns the number of chunks; fills at most `capacity` entries (chunk_tensor_out may be NULL). */
+int64_t lancet_lans_debug_chunk_table(const int64_t* numels, int T, int32_t* chunk_tensor_out, int64_t capacity);
 
 /* Test hook: number of polls a workgroup of the position scan waits for a predecessor
  * before it gives up, flags the workspace and finishes with undefined results

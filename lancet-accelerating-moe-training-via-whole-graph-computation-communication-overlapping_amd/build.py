@@ -44,7 +44,7 @@ def build_hip(verbose=True):
     objs = []
     for src in HIP_SOURCES:
         obj = os.path.join(LIBDIR, src.replace(".hip", ".o"))
-        _run([_hipcc()] + HIP_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj])
+        _run([_hipcc()] + HIP_FLAGS + os.environ.get("LANCET_EXTRA_HIPFLAGS", "").split() + ["-c", os.path.join(CSRC, src), "-o", obj])
         objs.append(obj)
     out = os.path.join(LIBDIR, "liblancet_hip.so")
     _run([_hipcc(), "-shared", "-fPIC", "--offload-arch=gfx950", "-o", out] + objs)

@@ -4,27 +4,25 @@
 //   phase 1  reads g, p            -> per-chunk sums of g^2 and p^2
 //   phase 2  reads g, p, m, v      -> writes m, v; per-chunk sums of u_m^2 and u_g^2
 //   phase 3  reads g, p, m, v      -> recomputes u_m, u_g (never stored) and writes p
-// and two schedules that give the same bits:
+// and two schedules:
 //   * sweeps (default): three plain launches + two tiny per-tensor reductions.  Real HBM traffic
 //     is 52 B/param (g, p read three times, m, v twice) and each sweep streams at the rate a plain
 //     copy reaches on this chip.
-//   * pipelined (opt-in): ONE persistent kernel.  Workgroups pull (phase, chunk) tasks from a
-//     queue built once per parameter set, ordered so that phase 2 of a bundle of tensors (about
-//     4M parameters, 64 MB of state) runs while phase 1 of the next bundle and phase 3 of the
-//     previous one run, with the aim of re-reading a tensor while it is still in the 256 MB
-//     Infinity Cache.  A task that needs a per-tensor norm waits for the chunk partials of that
-//     tensor, which are self-validating 64-bit words (step epoch in the high half, fp32 sum in
-//     the low half) published with one agent-scope atomic store each: no counters, nothing to
-//     clear between steps.  Tasks only ever wait for tasks that are earlier in the queue (already
-//     taken by a running workgroup) and phase-1 tasks never wait, so the queue always drains;
-//     waits are bounded.  m and v cross workgroups (and XCDs, whose L2s are private) between
-//     phase 2 and phase 3, which costs one release fence per phase-2 task and one acquire per
-//     phase-3 task; on MI355X the release (an L2 write-back) makes this schedule about 3x slower
-//     than the sweeps, which is why it is not the default.
+//   * resident (opt-in): ONE persistent kernel in which a workgroup takes a chunk through all three
+//     phases and keeps it on chip in between (g, then u_m and u_g, in registers; p in LDS), so every
+//     array is read once and written once: 28 B/param.  Between phases the workgroups of a tensor
+//     exchange chunk partials as self-validating 64-bit words (step epoch in the high half, fp32 sum
+//     in the low half, one agent-scope atomic store each); the workgroup that arrives last at a
+//     per-tensor counter sums them in a fixed order and publishes the norm the same way.  Nothing
+//     else crosses workgroups, so no fences are needed.  Chunks are handed out in list order by a
+//     ticket; a workgroup only ever waits for chunks of its own tensor, so the kernel drains as long
+//     as the chunks of one tensor all fit on the chip at once, which set_schedule checks (the limit
+//     is the register file: about 4M parameters per tensor on 256 CUs).  Waits are bounded.
 // Work is cut into fixed-size chunks described by device-resident tables built once per
 // parameter set, instead of kernel arguments re-packed for every launch
 // (multi_tensor_apply.cuh:39-92).  Chunk partials are combined in a fixed order in double
-// precision, so results are deterministic and identical between the two schedules.
+// precision, so each schedule is deterministic (the two differ in the last bits: a chunk's own sum is
+// accumulated in a different order).
 #include "launchers.hpp"
 #include "common.hpp"
 #include "../../include/lancet_hip.h"
@@ -47,10 +45,9 @@ struct LansTables {
   const int32_t* chunk_tensor; // [nchunks]
   const int32_t* tensor_first; // [T+1] first chunk of each tensor
   float* partial;              // [2][nchunks]      (sweeps schedule)
-  uint64_t* part_word;         // [4][nchunks]      (pipelined schedule: epoch | fp32 bits)
-  uint64_t* norm_word;         // [4][T]            (pipelined schedule: published norms)
-  const uint32_t* tasks;       // [3*nchunks]       (pipelined schedule: phase << 30 | chunk)
-  uint32_t* ticket;            // [1] next task; [1] error flag
+  uint64_t* part_word;         // [4][nchunks]      (resident schedule: epoch | fp32 sum of squares)
+  uint64_t* norm_word;         // [4][T]            (resident schedule: epoch | fp32 norm)
+  uint32_t* ticket;            // [1] next task; [1] error flag; [2][T] arrivals (resident schedule)
   float* norms;                // [4][T]: g, p, u_m, u_g
   float* consts;               // [2]: bias_correction1, bias_correction2
   int T;
@@ -343,7 +340,7 @@ __global__ __launch_bounds__(kLansThreads) void lans_update_kernel(LansTables t,
 }
 
 // =======================================================================================
-// schedule "pipelined": one persistent kernel over a task queue
+// words published between workgroups: step epoch in the high half, fp32 value in the low half
 // =======================================================================================
 __device__ __forceinline__ uint64_t ld_word(const uint64_t* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -353,93 +350,218 @@ __device__ __forceinline__ void st_word(uint64_t* p, uint32_t epoch, float v) {
                      __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Norm `which` (0 g, 1 p, 2 u_m, 3 u_g) of a tensor, called by the first wave of the workgroup.
-// Uses the published norm word when some workgroup has already summed the partials of this step,
-// else waits for the partials (bounded) and sums them itself, then publishes.
-__device__ __forceinline__ float pipeline_norm(const LansTables& t, const LansScalars& sc, int which, int tensor) {
-  uint64_t* nw = t.norm_word + static_cast<size_t>(which) * t.T + tensor;
-  const uint64_t w = ld_word(nw);
-  // one value for the whole wave, whatever each lane's load returned
-  const uint32_t w_hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(w >> 32));
-  const uint32_t w_lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(w));
-  if (w_hi == sc.epoch) return __uint_as_float(w_lo);
-  const uint64_t* part = t.part_word + static_cast<size_t>(which) * t.nchunks;
-  const int lo = t.tensor_first[tensor], hi = t.tensor_first[tensor + 1];
-  const float n = wave_norm(lo, hi, [&](int c) {
-    uint64_t x = ld_word(part + c);
-    uint32_t spins = 0;
-    while (static_cast<uint32_t>(x >> 32) != sc.epoch) {
-      if (++spins > sc.spin_limit) {  // bounded wait: flag the plan, carry on
-        st_agent(t.ticket + 1, 1u);
-        break;
-      }
-      __builtin_amdgcn_s_sleep(8);
-      x = ld_word(part + c);
+// =======================================================================================
+// schedule "resident": one persistent kernel; a workgroup keeps its chunk in registers across
+// the two per-tensor reductions, so every array is read once and written once (28 B/param)
+// =======================================================================================
+constexpr int kVecPerThread = kLansChunk / 4 / kLansThreads;  // float4 per thread and array
+
+__device__ __forceinline__ f32x4 ld4(const float* a, int e) { return *reinterpret_cast<const f32x4*>(a + e); }
+__device__ __forceinline__ void st4(float* a, int e, f32x4 x) { *reinterpret_cast<f32x4*>(a + e) = x; }
+
+constexpr int kMaxResidentChunks = 512;  // chunks of one tensor the resident schedule can gather
+
+struct ResidentShared {
+  f32x4 p[kVecPerThread][kLansThreads];  // the chunk's parameters, one private slot per thread and float4
+  float part[2][kMaxResidentChunks];     // gathered chunk partials of the tensor
+  float red[kLansThreads / kWave];
+  float norm[4];
+  int chunk;
+  int last;
+};
+
+__device__ __forceinline__ uint64_t wait_word(const LansTables& t, const LansScalars& sc, const uint64_t* src) {
+  uint64_t x = ld_word(src);
+  uint32_t spins = 0;
+  while (static_cast<uint32_t>(x >> 32) != sc.epoch) {
+    if (++spins > sc.spin_limit) {  // bounded: flag the plan, carry on
+      st_agent(t.ticket + 1, 1u);
+      break;
     }
-    return __uint_as_float(static_cast<uint32_t>(x));
-  });
-  if (lane_id() == 0) {
-    st_word(nw, sc.epoch, n);
-    t.norms[which * t.T + tensor] = n;
+    __builtin_amdgcn_s_sleep(2);
+    x = ld_word(src);
   }
-  return n;
+  return x;
 }
 
-__global__ __launch_bounds__(kLansThreads) void lans_pipeline_kernel(LansTables t, LansScalars sc) {
-  __shared__ float s_red[kLansThreads / kWave];
-  __shared__ uint32_t s_task;
-  __shared__ float s_norm[4];
+// Norms `first` and `first`+1 of the tensor from the partials its workgroups publish (this one has
+// published its own, a0 and a1, just before).  The workgroup that arrives last (a per-tensor counter,
+// cleared by the host before the step) gathers the partials into LDS, sums them in the fixed order of
+// wave_norm and publishes the two norms as self-validating words; every other workgroup waits for those
+// two words only.  Waits are bounded.
+__device__ __forceinline__ void resident_norms(const LansTables& t, const LansScalars& sc, int first, int tensor,
+                                               float a0, float a1, ResidentShared& sh) {
+  const int lo = t.tensor_first[tensor];
+  const int nc = t.tensor_first[tensor + 1] - lo;
+  const int w = threadIdx.x / kWave;
+  if (nc == 1) {
+    if (threadIdx.x == 0) {
+      sh.part[0][0] = a0;
+      sh.part[1][0] = a1;
+    }
+    __syncthreads();
+  } else {
+    if (threadIdx.x == 0) {
+      uint32_t* arrive = t.ticket + 2 + static_cast<size_t>(first / 2) * t.T + tensor;
+      const uint32_t old = __hip_atomic_fetch_add(arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      sh.last = old == static_cast<uint32_t>(nc - 1);
+    }
+    __syncthreads();
+    if (!sh.last) {
+      if (w < 2 && lane_id() == 0) {
+        const uint64_t x = wait_word(t, sc, t.norm_word + static_cast<size_t>(first + w) * t.T + tensor);
+        sh.norm[first + w] = __uint_as_float(static_cast<uint32_t>(x));
+      }
+      __syncthreads();
+      return;
+    }
+    for (int idx = threadIdx.x; idx < 2 * nc; idx += kLansThreads) {
+      const int which = idx >= nc ? 1 : 0;
+      const uint64_t x = wait_word(t, sc, t.part_word + static_cast<size_t>(first + which) * t.nchunks + lo + (idx - which * nc));
+      sh.part[which][idx - which * nc] = __uint_as_float(static_cast<uint32_t>(x));
+    }
+    __syncthreads();
+  }
+  if (w < 2) {
+    const float n = wave_norm(0, nc, [&](int c) { return sh.part[w][c]; });
+    if (lane_id() == 0) {
+      sh.norm[first + w] = n;
+      if (nc > 1) st_word(t.norm_word + static_cast<size_t>(first + w) * t.T + tensor, sc.epoch, n);
+    }
+  }
+  __syncthreads();
+}
+
+// One whole chunk of 16-byte aligned arrays through the three phases, every access an unconditional
+// float4.  g and then the updates u_m, u_g stay in registers, p in LDS: each array is read once and
+// written once.
+__device__ __forceinline__ void resident_chunk(const LansTables& t, const LansScalars& sc, const ChunkView& c, int chunk,
+                                               float bc1, float bc2, ResidentShared& sh) {
+  const float* g = t.g[c.tensor] + c.begin;
+  float* p = t.p[c.tensor] + c.begin;
+  float* m = t.m[c.tensor] + c.begin;
+  float* v = t.v[c.tensor] + c.begin;
+  f32x4 xg[kVecPerThread], xu[kVecPerThread];
+  // phase 1
+  float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+  for (int k = 0; k < kVecPerThread; ++k) {
+    const int e = 4 * (threadIdx.x + k * kLansThreads);
+    xg[k] = ld4(g, e);
+    const f32x4 xp = ld4(p, e);
+    sh.p[k][threadIdx.x] = xp;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      a0 += xg[k][j] * xg[k][j];
+      a1 += xp[j] * xp[j];
+    }
+  }
+  a0 = block_sum(a0, sh.red);
+  a1 = block_sum(a1, sh.red);
+  if (threadIdx.x == 0) {
+    st_word(t.part_word + chunk, sc.epoch, a0);
+    st_word(t.part_word + t.nchunks + chunk, sc.epoch, a1);
+  }
+  resident_norms(t, sc, 0, c.tensor, a0, a1, sh);
+  // phase 2: m, v get their final values; u_g takes the registers of g
+  const LansElem el = make_elem(sc, sh.norm[0], bc1, bc2);
+  a0 = 0.f, a1 = 0.f;
+#pragma unroll
+  for (int k = 0; k < kVecPerThread; ++k) {
+    const int e = 4 * (threadIdx.x + k * kLansThreads);
+    f32x4 xm = ld4(m, e), xv = ld4(v, e);
+    const f32x4 xp = sh.p[k][threadIdx.x];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float sg = el.scaled_grad(xg[k][j], xp[j]);
+      float mm = xm[j], vv = xv[j], u0, u1;
+      el.moments(sg, mm, vv);
+      el.updates(sg, xp[j], mm, vv, u0, u1);
+      xm[j] = mm;
+      xv[j] = vv;
+      xu[k][j] = u0;
+      xg[k][j] = u1;
+      a0 += u0 * u0;
+      a1 += u1 * u1;
+    }
+    st4(m, e, xm);
+    st4(v, e, xv);
+  }
+  a0 = block_sum(a0, sh.red);
+  a1 = block_sum(a1, sh.red);
+  if (threadIdx.x == 0) {
+    st_word(t.part_word + 2 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a0);
+    st_word(t.part_word + 3 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a1);
+  }
+  resident_norms(t, sc, 2, c.tensor, a0, a1, sh);
+  if (threadIdx.x == 0 && chunk == t.tensor_first[c.tensor]) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) t.norms[k * t.T + c.tensor] = sh.norm[k];
+  }
+  // phase 3
+  const float pn = sh.norm[1], umn = sh.norm[2], ugn = sh.norm[3];
+  float ratio_m = (umn != 0.f && pn != 0.f) ? sc.lr * (pn / umn) : sc.lr;
+  float ratio_g = (ugn != 0.f && pn != 0.f) ? sc.lr * (pn / ugn) : sc.lr;
+  ratio_m *= sc.beta1;
+  ratio_g *= sc.beta3;
+#pragma unroll
+  for (int k = 0; k < kVecPerThread; ++k) {
+    const int e = 4 * (threadIdx.x + k * kLansThreads);
+    f32x4 xp = sh.p[k][threadIdx.x];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma clang fp contract(off)
+      xp[j] = xp[j] - (ratio_m * xu[k][j]) - (ratio_g * xg[k][j]);
+    }
+    st4(p, e, xp);
+  }
+}
+
+// A partial or unaligned chunk through the same three phases with the streaming chunk functions of the
+// sweeps (nothing held in registers; m and v written in phase 2 are read back by the thread that wrote
+// them).  At most one chunk per tensor takes this path when arrays are aligned.
+__device__ __forceinline__ void resident_chunk_streamed(const LansTables& t, const LansScalars& sc, const ChunkView& c,
+                                                        int chunk, float bc1, float bc2, ResidentShared& sh) {
+  float a0, a1;
+  chunk_norm_gp(t, c, sh.red, a0, a1);
+  if (threadIdx.x == 0) {
+    st_word(t.part_word + chunk, sc.epoch, a0);
+    st_word(t.part_word + t.nchunks + chunk, sc.epoch, a1);
+  }
+  resident_norms(t, sc, 0, c.tensor, a0, a1, sh);
+  const LansElem el = make_elem(sc, sh.norm[0], bc1, bc2);
+  chunk_moments(t, c, el, sh.red, a0, a1);
+  if (threadIdx.x == 0) {
+    st_word(t.part_word + 2 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a0);
+    st_word(t.part_word + 3 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a1);
+  }
+  resident_norms(t, sc, 2, c.tensor, a0, a1, sh);
+  if (threadIdx.x == 0 && chunk == t.tensor_first[c.tensor]) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) t.norms[k * t.T + c.tensor] = sh.norm[k];
+  }
+  chunk_update(t, c, el, sc, sh.norm[1], sh.norm[2], sh.norm[3]);
+}
+
+// WAVES = waves per SIMD the kernel is compiled for, i.e. workgroups per CU: 3 keeps everything in
+// registers; 4 holds two of the largest supported tensors at once (1024 chunks on 256 CUs) at the price
+// of some register spills, which pays when single tensors fill half the chip.
+template <int WAVES>
+__global__ __launch_bounds__(kLansThreads, WAVES) void lans_resident_kernel(LansTables t, LansScalars sc) {
+  __shared__ ResidentShared sh;
   float bc1, bc2;
   bias_corrections(sc, bc1, bc2);
-  const uint32_t ntasks = 3u * static_cast<uint32_t>(t.nchunks);
   while (true) {
-    __syncthreads();  // s_task / s_norm of the previous task are no longer read
-    if (threadIdx.x == 0) s_task = atomicAdd(t.ticket, 1u);
+    __syncthreads();  // shared words of the previous chunk are no longer read
+    if (threadIdx.x == 0) sh.chunk = static_cast<int>(atomicAdd(t.ticket, 1u));
     __syncthreads();
-    const uint32_t slot = s_task;
-    if (slot >= ntasks) break;  // every workgroup reaches this: the queue is finite
-    const uint32_t task = t.tasks[slot];
-    const int phase = static_cast<int>(task >> 30);
-    const int chunk = static_cast<int>(task & 0x3fffffffu);
+    const int chunk = sh.chunk;
+    if (chunk >= t.nchunks) break;  // every workgroup reaches this: chunks are finite
     const ChunkView c = chunk_view(t, chunk);
-    if (phase == 0) {
-      float sg, sp;
-      chunk_norm_gp(t, c, s_red, sg, sp);
-      if (threadIdx.x == 0) {
-        st_word(t.part_word + chunk, sc.epoch, sg);
-        st_word(t.part_word + t.nchunks + chunk, sc.epoch, sp);
-      }
-    } else if (phase == 1) {
-      if (threadIdx.x < kWave) {
-        const float gn = pipeline_norm(t, sc, 0, c.tensor);
-        if (threadIdx.x == 0) s_norm[0] = gn;
-      }
-      __syncthreads();
-      const LansElem el = make_elem(sc, s_norm[0], bc1, bc2);
-      float sm, sg;
-      chunk_moments(t, c, el, s_red, sm, sg);
-      // m and v of this chunk are read in phase 3 by another workgroup, possibly on another XCD
-      // (private L2): make them visible device-wide before the words that announce them
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-      __syncthreads();
-      if (threadIdx.x == 0) {
-        st_word(t.part_word + 2 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, sm);
-        st_word(t.part_word + 3 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, sg);
-      }
-    } else {
-      if (threadIdx.x < kWave) {
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const float n = pipeline_norm(t, sc, k, c.tensor);
-          if (threadIdx.x == 0) s_norm[k] = n;
-        }
-      }
-      __syncthreads();
-      // pairs with the release above: drop stale cached copies of m and v
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-      const LansElem el = make_elem(sc, s_norm[0], bc1, bc2);
-      chunk_update(t, c, el, sc, s_norm[1], s_norm[2], s_norm[3]);
-    }
+    const bool full = c.n == kLansChunk &&
+                      vec_ok(t.g[c.tensor], t.p[c.tensor], t.m[c.tensor], t.v[c.tensor]);
+    if (full) resident_chunk(t, sc, c, chunk, bc1, bc2, sh);
+    else resident_chunk_streamed(t, sc, c, chunk, bc1, bc2, sh);
   }
 }
 
@@ -462,53 +584,18 @@ struct lancet_lans_plan {
   hipEvent_t upload_done;
   bool upload_pending;
   LansTables tables;
-  int schedule;        // LANCET_LANS_SWEEPS or LANCET_LANS_PIPELINED
-  int grid;            // workgroups of the persistent kernel
-  uint32_t epoch;      // step counter that tags the words of the pipelined schedule
+  int schedule;           // LANCET_LANS_SWEEPS or LANCET_LANS_RESIDENT
+  int resident_waves;     // kernel variant of the resident schedule (workgroups per CU)
+  int resident_grid;      // workgroups of that variant the device runs at once
+  int max_tensor_chunks;  // chunks of the largest tensor
+  uint32_t epoch;         // step counter that tags the words of the resident schedule
   size_t words_offset; // part_word + norm_word inside dev_block
   size_t words_bytes;
 };
 
-// Tensors are taken in list order and bundled until a bundle holds this many elements; the
-// pipelined schedule keeps about three bundles (x 16 B/element) in flight.
-static constexpr int64_t kBundleElems = 4 << 20;
-
 static constexpr uint32_t kPlanMagic = 0x4c414e53u;  // "LANS"
 
 static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
-
-// Task queue of the pipelined schedule: stage s runs phase 3 of bundle s-2, phase 2 of bundle
-// s-1 and phase 1 of bundle s, interleaved chunk by chunk.  Every task of phase k of a tensor
-// therefore precedes every task of phase k+1 of the same tensor: the order a waiting task relies on.
-static void build_task_queue(const int64_t* numels, int T, const std::vector<int32_t>& first,
-                             std::vector<uint32_t>& tasks) {
-  std::vector<std::pair<int, int>> bundles;  // [first chunk, last chunk)
-  int64_t acc = 0;
-  int start = 0;
-  for (int i = 0; i < T; ++i) {
-    acc += numels[i];
-    if (acc >= kBundleElems || i == T - 1) {
-      if (first[i + 1] > start) bundles.emplace_back(start, first[i + 1]);
-      start = first[i + 1];
-      acc = 0;
-    }
-  }
-  tasks.clear();
-  tasks.reserve(3 * static_cast<size_t>(first[T]));
-  const int nb = static_cast<int>(bundles.size());
-  for (int sidx = 0; sidx < nb + 2; ++sidx) {
-    int lo[3], hi[3];
-    for (int ph = 0; ph < 3; ++ph) {  // phase ph works on bundle sidx - ph
-      const int b = sidx - ph;
-      lo[ph] = (b >= 0 && b < nb) ? bundles[b].first : 0;
-      hi[ph] = (b >= 0 && b < nb) ? bundles[b].second : 0;
-    }
-    const int longest = std::max(hi[0] - lo[0], std::max(hi[1] - lo[1], hi[2] - lo[2]));
-    for (int k = 0; k < longest; ++k)
-      for (int ph = 2; ph >= 0; --ph)
-        if (lo[ph] + k < hi[ph]) tasks.push_back((static_cast<uint32_t>(ph) << 30) | static_cast<uint32_t>(lo[ph] + k));
-  }
-}
 
 static void chunk_tables(const int64_t* numels, int T, std::vector<int32_t>& ctensor, std::vector<int32_t>& first) {
   first.assign(T + 1, 0);
@@ -523,20 +610,15 @@ static void chunk_tables(const int64_t* numels, int T, std::vector<int32_t>& cte
   first[T] = c;
 }
 
-// Host-only view of the tables a plan would build (no device needed): the chunk -> tensor map and
-// the task queue.  Returns the number of tasks; fills at most `capacity` entries of each array.
-extern "C" int64_t lancet_lans_debug_task_queue(const int64_t* numels, int T, uint32_t* tasks_out,
-                                                int32_t* chunk_tensor_out, int64_t capacity) {
+// Host-only view of the chunk -> tensor map a plan builds for `numels` (no device needed).
+extern "C" int64_t lancet_lans_debug_chunk_table(const int64_t* numels, int T, int32_t* chunk_tensor_out,
+                                                 int64_t capacity) {
   if (!numels || T <= 0) return -1;
   std::vector<int32_t> ctensor, first;
   chunk_tables(numels, T, ctensor, first);
-  std::vector<uint32_t> tasks;
-  build_task_queue(numels, T, first, tasks);
-  for (int64_t i = 0; i < capacity && i < static_cast<int64_t>(tasks.size()); ++i)
-    if (tasks_out) tasks_out[i] = tasks[i];
   for (int64_t i = 0; i < capacity && i < static_cast<int64_t>(ctensor.size()); ++i)
     if (chunk_tensor_out) chunk_tensor_out[i] = ctensor[i];
-  return static_cast<int64_t>(tasks.size());
+  return static_cast<int64_t>(ctensor.size());
 }
 
 extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans_plan_t* out) {
@@ -571,15 +653,27 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
   const size_t o_norms = off;     off = align_up(off + 4 * T * sizeof(float), 256);
   const size_t o_consts = off;    off = align_up(off + 2 * sizeof(float), 256);
   const size_t o_words = off;     off = align_up(off + 4 * ((n ? n : 1) + T) * sizeof(uint64_t), 256);
-  const size_t o_tasks = off;     off = align_up(off + 3 * (n ? n : 1) * sizeof(uint32_t), 256);
-  const size_t o_ticket = off;    off = align_up(off + 2 * sizeof(uint32_t), 256);
+  const size_t o_ticket = off;    off = align_up(off + (2 + 2 * static_cast<size_t>(T)) * sizeof(uint32_t), 256);
   pl->schedule = LANCET_LANS_SWEEPS;
   pl->epoch = 0;
   pl->words_offset = o_words;
   pl->words_bytes = 4 * ((n ? n : 1) + T) * sizeof(uint64_t);
   int cus = 256;
   if (err == hipSuccess) err = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, pl->device);
-  pl->grid = static_cast<int>(std::min<size_t>(3 * n, static_cast<size_t>(cus) * 4));
+  pl->resident_grid = 0;
+  pl->max_tensor_chunks = 0;
+  for (int i = 0; i < T; ++i)
+    pl->max_tensor_chunks = std::max<int>(pl->max_tensor_chunks, static_cast<int>((numels[i] + kLansChunk - 1) / kLansChunk));
+  if (err == hipSuccess) {
+    // the variant with more workgroups per CU only when one tensor would take more than half the chip
+    int per_cu3 = 0, per_cu4 = 0;
+    err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu3, lans_resident_kernel<3>, kLansThreads, 0);
+    if (err == hipSuccess)
+      err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu4, lans_resident_kernel<4>, kLansThreads, 0);
+    const bool wide = 2 * pl->max_tensor_chunks > per_cu3 * cus;
+    pl->resident_waves = wide ? 4 : 3;
+    pl->resident_grid = (wide ? per_cu4 : per_cu3) * cus;
+  }
   if (err == hipSuccess) err = hipMalloc(&pl->dev_block, off);
   if (err == hipSuccess) err = hipHostMalloc(reinterpret_cast<void**>(&pl->h_ptrs), 4 * T * sizeof(void*), hipHostMallocDefault);
   if (err == hipSuccess) err = hipEventCreateWithFlags(&pl->upload_done, hipEventDisableTiming);
@@ -592,14 +686,9 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
     if (err == hipSuccess) err = hipMemcpy(base + o_first, first.data(), (T + 1) * sizeof(int32_t), hipMemcpyHostToDevice);
     if (err == hipSuccess) err = hipMemset(base + o_norms, 0, 4 * T * sizeof(float));
     if (err == hipSuccess) err = hipMemset(base + o_words, 0, pl->words_bytes);
-    std::vector<uint32_t> tasks;
-    build_task_queue(numels, T, first, tasks);
-    if (err == hipSuccess && !tasks.empty())
-      err = hipMemcpy(base + o_tasks, tasks.data(), tasks.size() * sizeof(uint32_t), hipMemcpyHostToDevice);
     LansTables& t = pl->tables;
     t.part_word = reinterpret_cast<uint64_t*>(base + o_words);
     t.norm_word = t.part_word + 4 * (n ? n : 1);
-    t.tasks = reinterpret_cast<const uint32_t*>(base + o_tasks);
     t.ticket = reinterpret_cast<uint32_t*>(base + o_ticket);
     void** dptrs = reinterpret_cast<void**>(base + o_ptrs);
     t.g = reinterpret_cast<const float* const*>(dptrs);
@@ -696,16 +785,18 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
   sc.step_dev = step_dev;
   const LansTables& t = pl->tables;
   sc.spin_limit = current_spin_limit();
-  if (pl->schedule == LANCET_LANS_PIPELINED) {
-    if (++pl->epoch == 0) {  // tag wrapped: forget every word of earlier steps
+  if (pl->schedule == LANCET_LANS_RESIDENT) {
+    if (++pl->epoch == 0) {
       err = hipMemsetAsync(static_cast<char*>(pl->dev_block) + pl->words_offset, 0, pl->words_bytes, st);
       if (err != hipSuccess) return static_cast<int>(err);
       pl->epoch = 1;
     }
     sc.epoch = pl->epoch;
-    err = run_fill_u32(t.ticket, 2, 0u, st);
+    err = run_fill_u32(t.ticket, 2 + 2 * static_cast<size_t>(T), 0u, st);
     if (err != hipSuccess) return static_cast<int>(err);
-    lans_pipeline_kernel<<<pl->grid, kLansThreads, 0, st>>>(t, sc);
+    const int grid = std::min(pl->resident_grid, t.nchunks);
+    if (pl->resident_waves == 4) lans_resident_kernel<4><<<grid, kLansThreads, 0, st>>>(t, sc);
+    else lans_resident_kernel<3><<<grid, kLansThreads, 0, st>>>(t, sc);
     return static_cast<int>(hipGetLastError());
   }
   sc.epoch = 0;
@@ -721,8 +812,18 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
 
 extern "C" int lancet_lans_plan_set_schedule(lancet_lans_plan_t pl, int schedule) {
   if (!pl || pl->magic != kPlanMagic) return LANCET_ERR_PLAN;
-  if (schedule != LANCET_LANS_PIPELINED && schedule != LANCET_LANS_SWEEPS) return LANCET_ERR_SHAPE;
+  if (schedule != LANCET_LANS_SWEEPS && schedule != LANCET_LANS_RESIDENT) return LANCET_ERR_SHAPE;
+  // a tensor's chunks must all be held by running workgroups at once
+  if (schedule == LANCET_LANS_RESIDENT && pl->max_tensor_chunks > std::min(pl->resident_grid, kMaxResidentChunks))
+    return LANCET_ERR_SHAPE;
   pl->schedule = schedule;
+  return LANCET_OK;
+}
+
+extern "C" int lancet_lans_plan_resident_capacity(lancet_lans_plan_t pl, int* workgroups, int* max_tensor_chunks) {
+  if (!pl || pl->magic != kPlanMagic) return LANCET_ERR_PLAN;
+  if (workgroups) *workgroups = std::min(pl->resident_grid, kMaxResidentChunks);
+  if (max_tensor_chunks) *max_tensor_chunks = pl->max_tensor_chunks;
   return LANCET_OK;
 }
 

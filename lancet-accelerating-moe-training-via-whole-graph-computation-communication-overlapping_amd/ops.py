@@ -390,8 +390,15 @@ class LansPlan:
             self.set_schedule(schedule)
 
     def set_schedule(self, schedule):
-        """capi.LANS_SWEEPS (default) or capi.LANS_PIPELINED."""
+        """capi.LANS_SWEEPS (default) or capi.LANS_RESIDENT (raises when a tensor is too large for it)."""
         capi.check(self._lib.lancet_lans_plan_set_schedule(self._h, int(schedule)), "lancet_lans_plan_set_schedule")
+
+    def resident_capacity(self):
+        """(chunks the resident schedule holds at once, chunks of this plan's largest tensor)."""
+        wg, mx = C.c_int(0), C.c_int(0)
+        capi.check(self._lib.lancet_lans_plan_resident_capacity(self._h, C.byref(wg), C.byref(mx)),
+                   "lancet_lans_plan_resident_capacity")
+        return wg.value, mx.value
 
     def error(self):
         err = C.c_int(-1)

@@ -5,6 +5,7 @@ import ctypes as C
 import os
 import re
 
+import numpy as np
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -181,49 +182,70 @@ def test_op_layer_errors_are_reported_not_fatal(pkg):
 
 
 # ----------------------------------------------------------------------------- LANS task queue
-def _task_queue(pkg, numels):
-    import numpy as np
+def _chunk_table(pkg, numels):
     lib = pkg.capi.load()
     arr = (C.c_int64 * len(numels))(*numels)
-    n = lib.lancet_lans_debug_task_queue(arr, len(numels), None, None, 0)
-    tasks = np.empty(n, np.uint32)
-    ctensor = np.empty(max(n // 3, 1), np.int32)
-    assert lib.lancet_lans_debug_task_queue(arr, len(numels), tasks.ctypes.data_as(C.c_void_p),
-                                            ctensor.ctypes.data_as(C.c_void_p), n) == n
-    return tasks, ctensor[:n // 3]
+    n = lib.lancet_lans_debug_chunk_table(arr, len(numels), None, 0)
+    ctensor = np.empty(max(n, 1), np.int32)
+    assert lib.lancet_lans_debug_chunk_table(arr, len(numels), ctensor.ctypes.data_as(C.c_void_p), n) == n
+    return ctensor[:n]
 
 
-@pytest.mark.parametrize("case", ["config5", "random", "tiny", "one_big"])
-def test_lans_task_queue_never_waits_on_a_later_task(pkg, case):
-    """The persistent LANS kernel is deadlock-free iff every task of phase k of a tensor comes before
-    every task of phase k+1 of the same tensor (a waiting task then only waits for tasks that running
-    workgroups already took) and every (phase, chunk) pair appears exactly once."""
-    import numpy as np
+def _simulate_resident(ctensor, workers, rng):
+    """The resident LANS schedule as a state machine: `workers` workgroups take chunks in list order from a
+    ticket; a workgroup publishes its phase-1 partial when it takes the chunk, moves to phase 2 once every
+    chunk of the tensor has published phase 1, publishes phase 2, and finishes once every chunk of the tensor
+    has published phase 2.  Workgroups are advanced in random order.  Returns True when every chunk finishes,
+    False when no workgroup can move."""
+    n = len(ctensor)
+    size = np.bincount(ctensor, minlength=int(ctensor.max()) + 1 if n else 1)
+    pub1 = np.zeros_like(size)
+    pub2 = np.zeros_like(size)
+    ticket, done = 0, 0
+    held = [None] * workers          # (tensor, phase) of the chunk a workgroup holds
+    while done < n:
+        moved = False
+        for w in rng.permutation(workers):
+            if held[w] is None:
+                if ticket < n:
+                    t = int(ctensor[ticket])
+                    ticket += 1
+                    pub1[t] += 1
+                    held[w] = (t, 1)
+                    moved = True
+            else:
+                t, ph = held[w]
+                if ph == 1 and pub1[t] == size[t]:
+                    pub2[t] += 1
+                    held[w] = (t, 2)
+                    moved = True
+                elif ph == 2 and pub2[t] == size[t]:
+                    held[w] = None
+                    done += 1
+                    moved = True
+        if not moved:
+            return False
+    return True
+
+
+@pytest.mark.parametrize("case", ["config5", "random", "tiny"])
+def test_lans_resident_schedule_drains(pkg, case):
+    """A workgroup of the resident schedule waits only for chunks of its own tensor, and chunks are handed
+    out in list order, so the kernel drains whenever the workgroups on the chip are at least as many as the
+    chunks of the largest tensor (what lancet_lans_plan_set_schedule checks) and can stall with fewer."""
     import bench
     rng = np.random.default_rng(0)
     if case == "config5":
-        numels = [int(np.prod(s)) for s in bench.lans_shapes()]
+        numels = [int(np.prod(s)) for s in bench.lans_shapes()][:40]
     elif case == "random":
-        numels = [int(x) for x in rng.integers(0, 3_000_000, 200)] + [0, 1, 8192, 8193]
-    elif case == "tiny":
-        numels = [1, 2, 3]
+        numels = [int(x) for x in rng.integers(0, 600_000, 60)] + [0, 1, 8192, 8193]
     else:
-        numels = [50_000_000, 5, 9_000_000]
-    tasks, ctensor = _task_queue(pkg, numels)
-    nchunks = sum((n + 8191) // 8192 for n in numels)
-    assert len(tasks) == 3 * nchunks and len(ctensor) == nchunks
-    phase = (tasks >> 30).astype(np.int64)
-    chunk = (tasks & 0x3FFFFFFF).astype(np.int64)
-    assert chunk.max() < nchunks and phase.max() <= 2
-    assert len(np.unique(phase * nchunks + chunk)) == 3 * nchunks          # each pair exactly once
-    tensor = ctensor[chunk]
-    pos = np.arange(len(tasks))
-    T = len(numels)
-    last = np.full((3, T), -1, np.int64)
-    first = np.full((3, T), len(tasks), np.int64)
-    for ph in range(3):
-        sel = phase == ph
-        np.maximum.at(last[ph], tensor[sel], pos[sel])
-        np.minimum.at(first[ph], tensor[sel], pos[sel])
-    has = np.array([(n + 8191) // 8192 > 0 for n in numels])
-    assert (last[0][has] < first[1][has]).all() and (last[1][has] < first[2][has]).all()
+        numels = [1, 2, 3]
+    ctensor = _chunk_table(pkg, numels)
+    assert len(ctensor) == sum((n + 8191) // 8192 for n in numels)
+    assert (np.diff(ctensor) >= 0).all()                       # chunks of a tensor are consecutive tickets
+    largest = int(np.bincount(ctensor).max())
+    for workers in (largest, largest + 3, 4 * largest):
+        assert _simulate_resident(ctensor, workers, rng)
+    if largest > 1:
+        assert not _simulate_resident(ctensor, largest - 1, rng)

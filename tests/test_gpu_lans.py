@@ -128,13 +128,14 @@ def test_lans_norms_and_plan_reuse(pkg):
     plan.close()
 
 
-def test_lans_pipelined_schedule_gives_the_same_bits(pkg):
-    """The opt-in persistent-kernel schedule must terminate, leave its error word clear and
-    produce exactly what the default three-sweep schedule produces."""
+def test_lans_resident_schedule(pkg):
+    """The opt-in persistent-kernel schedule must terminate, leave its error word clear, be reproducible and
+    agree with the default three-sweep schedule to fp32 rounding of the per-chunk sums (whole and partial
+    chunks, tensors of one chunk and of many, an unaligned tensor)."""
     capi = pkg.capi
-    numels = [1000, 70000, 5, 1 << 20, 3 * 8192, 8193, 1, (4 << 20) + 17, 1024, 1024, 2 << 20]
+    numels = [1000, 70000, 5, 1 << 20, 3 * 8192, 8193, 1, (2 << 20) + 17, 1024, 1024, 4 << 20, 2 << 20]
     results = []
-    for schedule in (capi.LANS_SWEEPS, capi.LANS_PIPELINED):
+    for schedule in (capi.LANS_SWEEPS, capi.LANS_RESIDENT, capi.LANS_RESIDENT):
         gen = torch.Generator(device="cuda").manual_seed(7)
         total = sum(numels)
         flat = [torch.empty(total, device="cuda").normal_(0, s, generator=gen) for s in (1e-3, 0.02)]
@@ -148,6 +149,45 @@ def test_lans_pipelined_schedule_gives_the_same_bits(pkg):
         assert plan.error() == 0
         results.append((flat, plan.norms()))
         plan.close()
-    for a, b in zip(results[0][0], results[1][0]):
+    for a, b in zip(results[1][0], results[2][0]):          # run to run: the same bits
         assert torch.equal(a, b)
-    assert torch.equal(results[0][1], results[1][1])
+    assert torch.equal(results[1][1], results[2][1])
+    for name, a, b in zip("gpmv", results[0][0], results[1][0]):
+        scale = a.abs().max().item()
+        assert (a - b).abs().max().item() <= 2e-6 * scale, name
+    torch.testing.assert_close(results[0][1], results[1][1], rtol=2e-6, atol=0)
+
+
+def test_lans_resident_schedule_against_oracle(pkg):
+    capi = pkg.capi
+    rng = np.random.default_rng(5)
+    shapes = [(300, 100), (8192,), (17,), (4, 8192), (8192 * 2 + 3,)]
+    g = [rng.normal(0, 1e-3, s).astype(np.float32) for s in shapes]
+    p = [rng.normal(0, 0.02, s).astype(np.float32) for s in shapes]
+    m = [np.zeros(s, np.float32) for s in shapes]
+    v = [np.zeros(s, np.float32) for s in shapes]
+    dg, dp, dm, dv = ([dev(a) for a in lst] for lst in (g, p, m, v))
+    plan = pkg.ops.LansPlan([a.size for a in g], schedule=capi.LANS_RESIDENT)
+    hyper = capi.LansHyper(1e-3, 0.9, 0.999, 1e-6, 1, 0.01, 1, 1, 1)
+    for step in range(1, 11):
+        lo.lans_step(g, p, m, v, step)
+        plan.step(dg, dp, dm, dv, step, hyper)
+    assert plan.error() == 0
+    for i in range(len(shapes)):
+        assert_close_scaled(to_np(dp[i]), p[i], P_RTOL, "p[%d]" % i)
+        assert_close_scaled(to_np(dm[i]), m[i], P_RTOL, "m[%d]" % i)
+        assert_close_scaled(to_np(dv[i]), v[i], P_RTOL, "v[%d]" % i)
+    plan.close()
+
+
+def test_lans_resident_schedule_rejects_a_tensor_that_does_not_fit(pkg):
+    capi = pkg.capi
+    plan = pkg.ops.LansPlan([1024, 1024])
+    workgroups, largest = plan.resident_capacity()
+    plan.close()
+    assert largest == 1 and workgroups >= 256
+    big = pkg.ops.LansPlan([(workgroups + 1) * 8192])       # no memory is touched by creating a plan
+    assert big.resident_capacity()[1] == workgroups + 1
+    with pytest.raises(RuntimeError):
+        big.set_schedule(capi.LANS_RESIDENT)
+    big.close()

@@ -232,7 +232,7 @@ def bench_config4_partitioned(ops, lib, capi, data, logits, S, M, E, cf, iters):
                                                      ("redispatch", redispatch), ("decode", decode))}
     kept = int((merged[0] >= 0).sum())
     b = data.element_size()
-    # partition encodes S*E*4 + S*M*b (each token row once per slot here: x2) + kept*M*b,
+    # algorithmic bytes: partition encodes S*E*4 + S*M*b (each token row once per slot here: x2) + kept*M*b,
     # merge 2*(kS)*8, redispatch kept*M*b + E*C*M*b, decode kept*M*b + S*M*b + kS*12
     alg = (S * E * 4 + S * M * b + kept * M * b) + 2 * (2 * S) * 8 + (kept * M * b + E * Cap * M * b) + \
           (kept * M * b + S * M * b + 2 * S * 12)
@@ -243,6 +243,20 @@ def bench_config4_partitioned(ops, lib, capi, data, logits, S, M, E, cf, iters):
             "frac_of_hbm_peak": round(alg / (total * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
             "note": "token rows are read once per slot (two passes) in this call pattern; "
                     "partition encodes write used rows only (zero_tail=False), redispatch zero-fills the merged tail"}
+
+
+def bench_pipeline(pkg, data, logits, S, M, E, cf, iters):
+    """Partitioned top-1 encode -> exchange (pack / unpack keyed by elements_per_expert) -> decode, 4 partitions,
+    issued on one stream and on two (exchange of partition i beside the encode of partition i+1)."""
+    layer = pkg.pipeline.PartitionedMoeLayer(S, M, E, 4, cf, dtype=data.dtype, gate_is_logits=True)
+    layer.run_serial(data, logits)
+    layer.run(data, logits)
+    t_serial = event_ms(lambda: layer.run_serial(data, logits), iters)
+    t_piped = event_ms(lambda: layer.run(data, logits), iters)
+    return {"workload": "4 partitions, top-1, S=%d M=%d E=%d C=%d" % (S, M, E, layer.C),
+            "ms_one_stream": round(t_serial, 4), "ms_two_streams": round(t_piped, 4),
+            "note": "every stage is HBM-bound on one GPU, so the streams share one memory system; the pattern "
+                    "pays when the exchange is a real all-to-all over xGMI"}
 
 
 def bench_backward(ops, data, outs, dec, S, M, E, Cap, K, kept, iters):
@@ -433,6 +447,7 @@ def main():
     del dec, outs
     torch.cuda.empty_cache()
     result["config4_partitioned"] = bench_config4_partitioned(ops, lib, capi, data, logits, S, M, E, cf, max(5, n // 2))
+    result["pipeline"] = bench_pipeline(pkg, data, logits, S, M, E, cf, max(5, n // 2))
     del data
     torch.cuda.empty_cache()
     if not args.no_lans:

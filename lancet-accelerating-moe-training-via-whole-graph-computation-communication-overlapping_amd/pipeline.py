@@ -1,0 +1,105 @@
+"""A partitioned MoE dispatch pipeline over two HIP streams: the call pattern Lancet's partition pass
+emits for one MoE layer (src/pass/dist_optimization/partition_exprs.cc:1709-1795), on one GPU.
+
+The token batch is cut into P partitions.  Partition i is encoded with the used capacity of partition
+i-1 chained in and capacity_factor x P (`:1750-1762`), scheduled at pipeline index i (`:1775`); its
+exchange then overlaps the encode of partition i+1.  With one GPU there is no all-to-all, so the
+exchange stage does what the all-to-allv does to the buffer on either side of the wire: the rows each
+expert uses are packed back to back, keyed by elements_per_expert (the send counts,
+src/op/dialect/nccl/nccl.cc:373-421), and unpacked into a zero-filled [E, C, M] receive buffer.  The
+expert computation is the identity.  Partition i is then decoded from its own receive buffer.
+
+Streams carry the default priority.  Every buffer is allocated once, in the constructor; `run` only
+launches kernels and records events, so it can be called in a loop.
+"""
+import torch
+
+from . import ops
+
+
+class PartitionedMoeLayer:
+    def __init__(self, S, M, E, n_partitions, capacity_factor=1.0, dtype=torch.float32, gate_is_logits=False,
+                 device="cuda"):
+        if S % n_partitions != 0:
+            raise ValueError("the token count must divide into n_partitions")
+        self.S, self.M, self.E, self.P = S, M, E, n_partitions
+        self.Sp = S // n_partitions
+        self.cf = float(capacity_factor) * n_partitions   # partition_exprs.cc:1754-1760
+        self.gate_is_logits = gate_is_logits
+        self.C = ops.moe_capacity(self.Sp, E, self.cf)
+        dev = torch.device(device)
+        P, Sp, C = self.P, self.Sp, self.C
+        self.enc = [(torch.empty(Sp, dtype=torch.float32, device=dev),
+                     torch.empty((2, Sp), dtype=torch.int32, device=dev),
+                     torch.empty(E, dtype=torch.int32, device=dev),
+                     torch.empty(E, dtype=torch.int64, device=dev),
+                     torch.empty((E, C, M), dtype=dtype, device=dev)) for _ in range(P)]
+        # one scan workspace per partition: encodes of neighbouring partitions never share one
+        self.ws = [torch.empty(ops.moe_encode_workspace_bytes(Sp, E, 1), dtype=torch.uint8, device=dev)
+                   for _ in range(P)]
+        self.wire = [torch.empty(E * C * M, dtype=dtype, device=dev) for _ in range(P)]
+        self.recv = [torch.empty((E, C, M), dtype=dtype, device=dev) for _ in range(P)]
+        self.out = torch.empty((S, M), dtype=dtype, device=dev)
+        self.zero_used = torch.zeros(E, dtype=torch.int32, device=dev)
+        self.compute = torch.cuda.Stream(device=dev)
+        self.exchange = torch.cuda.Stream(device=dev)
+        self.encoded = [torch.cuda.Event() for _ in range(P)]
+        self.received = [torch.cuda.Event() for _ in range(P)]
+
+    # ---- the three stages of one partition ----------------------------------------------------
+    def _encode(self, i, data, gate):
+        sl = slice(i * self.Sp, (i + 1) * self.Sp)
+        used = self.zero_used if i == 0 else self.enc[i - 1][2]
+        # the send buffer only feeds the packing copy, which reads the used rows: no tail zero-fill
+        ops.moe_encode(data[sl], gate[sl], used, self.cf, gate_is_logits=self.gate_is_logits, zero_tail=False,
+                       workspace=self.ws[i], out=self.enc[i])
+
+    def _exchange(self, i):
+        _, _, _, elems, disp = self.enc[i]
+        ops.memcpy_sparse_to_cont_3d(disp, self.wire[i], elems, axis=0)
+        ops.memcpy_cont_to_sparse_3d(self.wire[i], self.recv[i], elems, axis=0, zero_tail=True)
+
+    def _decode(self, i):
+        gates_s, indloc = self.enc[i][0], self.enc[i][1]
+        ops.moe_decode(self.recv[i], gates_s, indloc, out=self.out[i * self.Sp:(i + 1) * self.Sp])
+
+    # ---- schedules ----------------------------------------------------------------------------
+    def run_serial(self, data, gate):
+        """Every stage of every partition on the current stream, in pipeline order."""
+        for i in range(self.P):
+            self._encode(i, data, gate)
+            self._exchange(i)
+            self._decode(i)
+        return self.out
+
+    def run(self, data, gate):
+        """Encodes and decodes on one stream, exchanges on another: the exchange of partition i runs beside
+        the encode of partition i+1, the decode of partition i after its exchange.  Returns the output;
+        the caller's current stream waits for the pipeline before it may use it."""
+        cur = torch.cuda.current_stream()
+        start = torch.cuda.Event()
+        start.record(cur)
+        self.compute.wait_event(start)
+        self.exchange.wait_event(start)
+        for i in range(self.P):
+            with torch.cuda.stream(self.compute):
+                self._encode(i, data, gate)
+                self.encoded[i].record(self.compute)
+                if i > 0:
+                    self.compute.wait_event(self.received[i - 1])
+                    self._decode(i - 1)
+            with torch.cuda.stream(self.exchange):
+                self.exchange.wait_event(self.encoded[i])
+                self._exchange(i)
+                self.received[i].record(self.exchange)
+        with torch.cuda.stream(self.compute):
+            self.compute.wait_event(self.received[self.P - 1])
+            self._decode(self.P - 1)
+            done = torch.cuda.Event()
+            done.record(self.compute)
+        cur.wait_event(done)
+        return self.out
+
+    def kept_masks(self):
+        """indices_locations of every partition, the input moe_merge_masks takes."""
+        return [e[1] for e in self.enc]

@@ -1,0 +1,850 @@
+// Fused multi-tensor LANS step.  The reference makes six sweeps over the optimizer state
+// (src/op/dialect/cuda/kernels/multi_tensor_lans.cu:401-450: l2norm(g), l2norm(p), stage 1,
+// l2norm(u_m), l2norm(u_g), stage 2, 68 B/param of traffic).  Here the step has three phases
+//   phase 1  reads g, p            -> per-chunk sums of g^2 and p^2
+//   phase 2  reads g, p, m, v      -> writes m, v; per-chunk sums of u_m^2 and u_g^2
+//   phase 3  reads g, p, m, v      -> recomputes u_m, u_g (never stored) and writes p
+// and two schedules:
+//   * sweeps (default): three plain launches + two tiny per-tensor reductions.  Real HBM traffic
+//     is 52 B/param (g, p read three times, m, v twice) and each sweep streams at the rate a plain
+//     copy reaches on this chip.
+//   * resident (opt-in): ONE persistent kernel in which a workgroup takes a chunk through all three
+//     phases and keeps it on chip in between (g, then u_m and u_g, in registers; p in LDS), so every
+//     array is read once and written once: 28 B/param.  Between phases the workgroups of a tensor
+//     exchange chunk partials as self-validating 64-bit words (step epoch in the high half, fp32 sum
+//     in the low half, one agent-scope atomic store each); the workgroup that arrives last at a
+//     per-tensor counter sums them in a fixed order and publishes the norm the same way.  Nothing
+//     else crosses workgroups, so no fences are needed.  Chunks are handed out in list order by a
+//     ticket; a workgroup only ever waits for chunks of its own tensor, so the kernel drains as long
+//     as the chunks of one tensor all fit on the chip at once, which set_schedule checks (the limit
+//     is the register file: about 4M parameters per tensor on 256 CUs).  Waits are bounded.
+// Work is cut into fixed-size chunks described by device-resident tables built once per
+// parameter set, instead of kernel arguments re-packed for every launch
+// (multi_tensor_apply.cuh:39-92).  Chunk partials are combined in a fixed order in double
+// precision, so each schedule is deterministic (the two differ in the last bits: a chunk's own sum is
+// accumulated in a different order).
+#include "launchers.hpp"
+#include "common.hpp"
+#include "../../include/lancet_hip.h"
+#include <algorithm>
+#include <new>
+#include <vector>
+
+namespace lancet {
+
+constexpr int kLansThreads = 256;
+constexpr int kLansChunk = 8192;  // elements per task: 8 float4 per thread and array
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+struct LansTables {
+  const float* const* g;  // [T] device pointers
+  float* const* p;
+  float* const* m;
+  float* const* v;
+  const int64_t* numel;        // [T]
+  const int32_t* chunk_tensor; // [nchunks]
+  const int32_t* tensor_first; // [T+1] first chunk of each tensor
+  float* partial;              // [2][nchunks]      (sweeps schedule)
+  uint64_t* part_word;         // [4][nchunks]      (resident schedule: epoch | fp32 sum of squares)
+  uint64_t* norm_word;         // [4][T]            (resident schedule: epoch | fp32 norm)
+  uint32_t* ticket;            // [1] next task; [1] error flag; [2][T] arrivals (resident schedule)
+  float* norms;                // [4][T]: g, p, u_m, u_g
+  float* consts;               // [2]: bias_correction1, bias_correction2
+  int T;
+  int nchunks;
+};
+
+struct LansScalars {
+  float lr, beta1, beta2, beta3, eps, wd;
+  int mode, normalize_grad, bias_correction;
+  int step_host;
+  const float* step_dev;
+  uint32_t epoch;
+  uint32_t spin_limit;
+};
+
+__device__ __forceinline__ float block_sum(float v, float* s_red) {
+  v = wave_sum(v);
+  const int w = threadIdx.x / kWave;
+  if (lane_id() == 0) s_red[w] = v;
+  __syncthreads();
+  float r = 0.f;
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int k = 0; k < kLansThreads / kWave; ++k) r += s_red[k];
+  }
+  __syncthreads();
+  return r;  // valid on thread 0
+}
+
+struct ChunkView {
+  int tensor;
+  int64_t begin;  // first element of the chunk inside the tensor
+  int n;          // elements in the chunk
+};
+
+__device__ __forceinline__ ChunkView chunk_view(const LansTables& t, int chunk) {
+  ChunkView c;
+  c.tensor = t.chunk_tensor[chunk];
+  c.begin = static_cast<int64_t>(chunk - t.tensor_first[c.tensor]) * kLansChunk;
+  const int64_t left = t.numel[c.tensor] - c.begin;
+  c.n = static_cast<int>(left < kLansChunk ? left : kLansChunk);
+  return c;
+}
+
+__device__ __forceinline__ bool vec_ok(const void* a, const void* b, const void* c, const void* d) {
+  return ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) |
+           reinterpret_cast<uintptr_t>(c) | reinterpret_cast<uintptr_t>(d)) & 15u) == 0;
+}
+
+// ---- elementwise math, in the reference's operation order (multi_tensor_lans.cu:283-307) ----
+struct LansElem {
+  float gnorm_eps;  // ||g|| + eps
+  bool normalize;   // normalize_grad && ||g|| != 0
+  float beta1, beta2, beta3, one_minus_beta2, bc1, bc2, eps, wd;
+  int mode;
+
+  __device__ __forceinline__ float scaled_grad(float g, float p) const {
+#pragma clang fp contract(off)
+    float sg = g;
+    if (normalize) sg = sg / gnorm_eps;
+    if (mode == 0) sg = sg + wd * p;
+    return sg;
+  }
+  __device__ __forceinline__ void moments(float sg, float& m, float& v) const {
+#pragma clang fp contract(off)
+    m = m * beta1 + beta3 * sg;
+    v = v * beta2 + one_minus_beta2 * sg * sg;
+  }
+  __device__ __forceinline__ void updates(float sg, float p, float m, float v, float& um, float& ug) const {
+#pragma clang fp contract(off)
+    const float denom = sqrtf(v / bc2) + eps;
+    um = (m / bc1) / denom;
+    ug = sg / denom;
+    if (mode != 0) {
+      const float sp = wd * p;
+      um = um + sp;
+      ug = ug + sp;
+    }
+  }
+};
+
+__device__ __forceinline__ LansElem make_elem(const LansScalars& sc, float gn, float bc1, float bc2) {
+  LansElem e;
+  e.gnorm_eps = gn + sc.eps;
+  e.normalize = sc.normalize_grad && gn != 0.f;
+  e.beta1 = sc.beta1;
+  e.beta2 = sc.beta2;
+  e.beta3 = sc.beta3;
+  e.one_minus_beta2 = 1.f - sc.beta2;
+  e.bc1 = bc1;
+  e.bc2 = bc2;
+  e.eps = sc.eps;
+  e.wd = sc.wd;
+  e.mode = sc.mode;
+  return e;
+}
+
+// bias corrections 1 - beta^step (src/op/dialect/cuda/lans.cc:108-113), from a host step or
+// from the fp32 step scalar in device memory (no host synchronisation, unlike lans.cc:102-107)
+__device__ __forceinline__ void bias_corrections(const LansScalars& sc, float& bc1, float& bc2) {
+  int step = sc.step_host;
+  if (sc.step_dev) step = static_cast<int>(*sc.step_dev);
+  bc1 = 1.f;
+  bc2 = 1.f;
+  if (sc.bias_correction) {
+    bc1 = static_cast<float>(1.0 - pow(static_cast<double>(sc.beta1), step));
+    bc2 = static_cast<float>(1.0 - pow(static_cast<double>(sc.beta2), step));
+  }
+}
+
+// ---- the three phases on one chunk, executed by one workgroup ------------------------------
+// phase 1: sums of squares of g and p (L2NormFunctor, multi_tensor_lans.cu:95-167); valid on thread 0
+__device__ __forceinline__ void chunk_norm_gp(const LansTables& t, const ChunkView& c, float* s_red,
+                                              float& sum_g, float& sum_p) {
+  const float* g = t.g[c.tensor] + c.begin;
+  const float* p = t.p[c.tensor] + c.begin;
+  float ag = 0.f, ap = 0.f;
+  int scalar_from = 0;
+  if (vec_ok(g, p, g, p)) {
+    const int nv = c.n / 4;
+    const f32x4* g4 = reinterpret_cast<const f32x4*>(g);
+    const f32x4* p4 = reinterpret_cast<const f32x4*>(p);
+#pragma unroll 4
+    for (int i = threadIdx.x; i < nv; i += kLansThreads) {
+      const f32x4 x = g4[i], y = p4[i];
+      ag += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+      ap += y.x * y.x + y.y * y.y + y.z * y.z + y.w * y.w;
+    }
+    scalar_from = nv * 4;
+  }
+  for (int i = scalar_from + threadIdx.x; i < c.n; i += kLansThreads) {
+    ag += g[i] * g[i];
+    ap += p[i] * p[i];
+  }
+  sum_g = block_sum(ag, s_red);
+  sum_p = block_sum(ap, s_red);
+}
+
+// phase 2: moments + sums of squares of the two updates (LANSStage1Functor :207-322 and the two
+// l2norm sweeps after it, :434-441); sums valid on thread 0
+__device__ __forceinline__ void chunk_moments(const LansTables& t, const ChunkView& c, const LansElem& el,
+                                              float* s_red, float& sum_um, float& sum_ug) {
+  const float* g = t.g[c.tensor] + c.begin;
+  const float* p = t.p[c.tensor] + c.begin;
+  float* m = t.m[c.tensor] + c.begin;
+  float* v = t.v[c.tensor] + c.begin;
+  float am = 0.f, ag = 0.f;
+  int scalar_from = 0;
+  if (vec_ok(g, p, m, v)) {
+    const int nv = c.n / 4;
+    const f32x4* g4 = reinterpret_cast<const f32x4*>(g);
+    const f32x4* p4 = reinterpret_cast<const f32x4*>(p);
+    f32x4* m4 = reinterpret_cast<f32x4*>(m);
+    f32x4* v4 = reinterpret_cast<f32x4*>(v);
+#pragma unroll 2
+    for (int i = threadIdx.x; i < nv; i += kLansThreads) {
+      const f32x4 xg = g4[i], xp = p4[i];
+      f32x4 xm = m4[i], xv = v4[i];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const float sg = el.scaled_grad(xg[k], xp[k]);
+        float mm = xm[k], vv = xv[k], um, ug;
+        el.moments(sg, mm, vv);
+        el.updates(sg, xp[k], mm, vv, um, ug);
+        xm[k] = mm;
+        xv[k] = vv;
+        am += um * um;
+        ag += ug * ug;
+      }
+      m4[i] = xm;
+      v4[i] = xv;
+    }
+    scalar_from = nv * 4;
+  }
+  for (int i = scalar_from + threadIdx.x; i < c.n; i += kLansThreads) {
+    const float sg = el.scaled_grad(g[i], p[i]);
+    float mm = m[i], vv = v[i], um, ug;
+    el.moments(sg, mm, vv);
+    el.updates(sg, p[i], mm, vv, um, ug);
+    m[i] = mm;
+    v[i] = vv;
+    am += um * um;
+    ag += ug * ug;
+  }
+  sum_um = block_sum(am, s_red);
+  sum_ug = block_sum(ag, s_red);
+}
+
+// phase 3: trust ratios and parameter update (LANSStage2Functor :326-399)
+__device__ __forceinline__ void chunk_update(const LansTables& t, const ChunkView& c, const LansElem& el,
+                                             const LansScalars& sc, float pn, float umn, float ugn) {
+  float ratio_m = (umn != 0.f && pn != 0.f) ? sc.lr * (pn / umn) : sc.lr;
+  float ratio_g = (ugn != 0.f && pn != 0.f) ? sc.lr * (pn / ugn) : sc.lr;
+  ratio_m *= sc.beta1;
+  ratio_g *= sc.beta3;
+  const float* g = t.g[c.tensor] + c.begin;
+  float* p = t.p[c.tensor] + c.begin;
+  const float* m = t.m[c.tensor] + c.begin;
+  const float* v = t.v[c.tensor] + c.begin;
+  int scalar_from = 0;
+  if (vec_ok(g, p, m, v)) {
+    const int nv = c.n / 4;
+    const f32x4* g4 = reinterpret_cast<const f32x4*>(g);
+    f32x4* p4 = reinterpret_cast<f32x4*>(p);
+    const f32x4* m4 = reinterpret_cast<const f32x4*>(m);
+    const f32x4* v4 = reinterpret_cast<const f32x4*>(v);
+#pragma unroll 2
+    for (int i = threadIdx.x; i < nv; i += kLansThreads) {
+      const f32x4 xg = g4[i], xm = m4[i], xv = v4[i];
+      f32x4 xp = p4[i];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+#pragma clang fp contract(off)
+        const float sg = el.scaled_grad(xg[k], xp[k]);
+        float um, ug;
+        el.updates(sg, xp[k], xm[k], xv[k], um, ug);
+        xp[k] = xp[k] - (ratio_m * um) - (ratio_g * ug);
+      }
+      p4[i] = xp;
+    }
+    scalar_from = nv * 4;
+  }
+  for (int i = scalar_from + threadIdx.x; i < c.n; i += kLansThreads) {
+#pragma clang fp contract(off)
+    const float sg = el.scaled_grad(g[i], p[i]);
+    float um, ug;
+    el.updates(sg, p[i], m[i], v[i], um, ug);
+    p[i] = p[i] - (ratio_m * um) - (ratio_g * ug);
+  }
+}
+
+// sqrt of the sum of a tensor's chunk partials: one wave, lane-strided double sums, xor tree
+// (fixed order, so every caller gets the same bits).  get(c) returns the partial of chunk c.
+template <typename Get>
+__device__ __forceinline__ float wave_norm(int lo, int hi, Get get) {
+  double acc = 0.0;
+  for (int c = lo + lane_id(); c < hi; c += kWave) acc += static_cast<double>(get(c));
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, kWave);
+  return static_cast<float>(sqrt(acc));
+}
+
+// =======================================================================================
+// schedule "sweeps": three launches + two per-tensor reductions
+// =======================================================================================
+__global__ void lans_prepare_kernel(LansTables t, LansScalars sc) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) bias_corrections(sc, t.consts[0], t.consts[1]);
+}
+
+__global__ __launch_bounds__(kLansThreads) void lans_norm_gp_kernel(LansTables t) {
+  __shared__ float s_red[kLansThreads / kWave];
+  const ChunkView c = chunk_view(t, blockIdx.x);
+  float sg, sp;
+  chunk_norm_gp(t, c, s_red, sg, sp);
+  if (threadIdx.x == 0) {
+    t.partial[blockIdx.x] = sg;
+    t.partial[t.nchunks + blockIdx.x] = sp;
+  }
+}
+
+// per-tensor sqrt(sum of chunk partials) (cleanup, multi_tensor_lans.cu:169-185)
+__global__ __launch_bounds__(kLansThreads) void lans_reduce_kernel(LansTables t, int first_norm) {
+  const int tensor = blockIdx.x * (kLansThreads / kWave) + threadIdx.x / kWave;
+  if (tensor >= t.T) return;
+  const int lo = t.tensor_first[tensor], hi = t.tensor_first[tensor + 1];
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    const float* part = t.partial + static_cast<size_t>(k) * t.nchunks;
+    const float n = wave_norm(lo, hi, [&](int c) { return part[c]; });
+    if (lane_id() == 0) t.norms[(first_norm + k) * t.T + tensor] = n;
+  }
+}
+
+__global__ __launch_bounds__(kLansThreads) void lans_moments_kernel(LansTables t, LansScalars sc) {
+  __shared__ float s_red[kLansThreads / kWave];
+  const ChunkView c = chunk_view(t, blockIdx.x);
+  const LansElem el = make_elem(sc, t.norms[c.tensor], t.consts[0], t.consts[1]);
+  float sm, sg;
+  chunk_moments(t, c, el, s_red, sm, sg);
+  if (threadIdx.x == 0) {
+    t.partial[blockIdx.x] = sm;
+    t.partial[t.nchunks + blockIdx.x] = sg;
+  }
+}
+
+__global__ __launch_bounds__(kLansThreads) void lans_update_kernel(LansTables t, LansScalars sc) {
+  const ChunkView c = chunk_view(t, blockIdx.x);
+  const LansElem el = make_elem(sc, t.norms[c.tensor], t.consts[0], t.consts[1]);
+  chunk_update(t, c, el, sc, t.norms[1 * t.T + c.tensor], t.norms[2 * t.T + c.tensor], t.norms[3 * t.T + c.tensor]);
+}
+
+// =======================================================================================
+// words published between workgroups: step epoch in the high half, fp32 value in the low half
+// =======================================================================================
+__device__ __forceinline__ uint64_t ld_word(const uint64_t* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_word(uint64_t* p, uint32_t epoch, float v) {
+  __hip_atomic_store(p, (static_cast<uint64_t>(epoch) << 32) | __float_as_uint(v), __ATOMIC_RELAXED,
+                     __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// =======================================================================================
+// schedule "resident": one persistent kernel; a workgroup keeps its chunk in registers across
+// the two per-tensor reductions, so every array is read once and written once (28 B/param)
+// =======================================================================================
+constexpr int kVecPerThread = kLansChunk / 4 / kLansThreads;  // float4 per thread and array
+
+__device__ __forceinline__ f32x4 ld4(const float* a, int e) { return *reinterpret_cast<const f32x4*>(a + e); }
+__device__ __forceinline__ void st4(float* a, int e, f32x4 x) { *reinterpret_cast<f32x4*>(a + e) = x; }
+
+constexpr int kMaxResidentChunks = 512;  // chunks of one tensor the resident schedule can gather
+
+struct ResidentShared {
+  f32x4 p[kVecPerThread][kLansThreads];  // the chunk's parameters, one private slot per thread and float4
+  float part[2][kMaxResidentChunks];     // gathered chunk partials of the tensor
+  float red[kLansThreads / kWave];
+  float norm[4];
+  int chunk;
+  int last;
+};
+
+__device__ __forceinline__ uint64_t wait_word(const LansTables& t, const LansScalars& sc, const uint64_t* src) {
+  uint64_t x = ld_word(src);
+  uint32_t spins = 0;
+  while (static_cast<uint32_t>(x >> 32) != sc.epoch) {
+    if (++spins > sc.spin_limit) {  // bounded: flag the plan, carry on
+      st_agent(t.ticket + 1, 1u);
+      break;
+    }
+    __builtin_amdgcn_s_sleep(2);
+    x = ld_word(src);
+  }
+  return x;
+}
+
+// Norms `first` and `first`+1 of the tensor from the partials its workgroups publish (this one has
+// published its own, a0 and a1, just before).  The workgroup that arrives last (a per-tensor counter,
+// cleared by the host before the step) gathers the partials into LDS, sums them in the fixed order of
+// wave_norm and publishes the two norms as self-validating words; every other workgroup waits for those
+// two words only.  Waits are bounded.
+__device__ __forceinline__ void resident_norms(const LansTables& t, const LansScalars& sc, int first, int tensor,
+                                               float a0, float a1, ResidentShared& sh) {
+  const int lo = t.tensor_first[tensor];
+  const int nc = t.tensor_first[tensor + 1] - lo;
+  const int w = threadIdx.x / kWave;
+  if (nc == 1) {
+    if (threadIdx.x == 0) {
+      sh.part[0][0] = a0;
+      sh.part[1][0] = a1;
+    }
+    __syncthreads();
+  } else {
+    if (threadIdx.x == 0) {
+      uint32_t* arrive = t.ticket + 2 + static_cast<size_t>(first / 2) * t.T + tensor;
+      const uint32_t old = __hip_atomic_fetch_add(arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      sh.last = old == static_cast<uint32_t>(nc - 1);
+    }
+    __syncthreads();
+    if (!sh.last) {
+      if (w < 2 && lane_id() == 0) {
+        const uint64_t x = wait_word(t, sc, t.norm_word + static_cast<size_t>(first + w) * t.T + tensor);
+        sh.norm[first + w] = __uint_as_float(static_cast<uint32_t>(x));
+      }
+      __syncthreads();
+      return;
+    }
+    for (int idx = threadIdx.x; idx < 2 * nc; idx += kLansThreads) {
+      const int which = idx >= nc ? 1 : 0;
+      const uint64_t x = wait_word(t, sc, t.part_word + static_cast<size_t>(first + which) * t.nchunks + lo + (idx - which * nc));
+      sh.part[which][idx - which * nc] = __uint_as_float(static_cast<uint32_t>(x));
+    }
+    __syncthreads();
+  }
+  if (w < 2) {
+    const float n = wave_norm(0, nc, [&](int c) { return sh.part[w][c]; });
+    if (lane_id() == 0) {
+      sh.norm[first + w] = n;
+      if (nc > 1) st_word(t.norm_word + static_cast<size_t>(first + w) * t.T + tensor, sc.epoch, n);
+    }
+  }
+  __syncthreads();
+}
+
+// One whole chunk of 16-byte aligned arrays through the three phases, every access an unconditional
+// float4.  g and then the updates u_m, u_g stay in registers, p in LDS: each array is read once and
+// written once.
+// threadIdx.x behind an empty asm: what is derived from it (addresses of this phase) is computed where it
+// is used instead of once for the whole kernel, which would keep it in registers across every phase
+__device__ __forceinline__ int opaque_tid() {
+  int t = threadIdx.x;
+  asm volatile("" : "+v"(t));
+  return t;
+}
+
+__device__ __forceinline__ void resident_chunk(const LansTables& t, const LansScalars& sc, const ChunkView& c, int chunk,
+                                               float bc1, float bc2, ResidentShared& sh) {
+  const float* g = t.g[c.tensor] + c.begin;
+  float* p = t.p[c.tensor] + c.begin;
+  float* m = t.m[c.tensor] + c.begin;
+  float* v = t.v[c.tensor] + c.begin;
+  f32x4 xg[kVecPerThread], xu[kVecPerThread];
+  // phase 1
+  float a0 = 0.f, a1 = 0.f;
+  int tid = opaque_tid();
+#pragma unroll
+  for (int k = 0; k < kVecPerThread; ++k) {
+    const int e = 4 * (tid + k * kLansThreads);
+    xg[k] = ld4(g, e);
+    const f32x4 xp = ld4(p, e);
+    sh.p[k][tid] = xp;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      a0 += xg[k][j] * xg[k][j];
+      a1 += xp[j] * xp[j];
+    }
+  }
+  a0 = block_sum(a0, sh.red);
+  a1 = block_sum(a1, sh.red);
+  if (threadIdx.x == 0) {
+    st_word(t.part_word + chunk, sc.epoch, a0);
+    st_word(t.part_word + t.nchunks + chunk, sc.epoch, a1);
+  }
+  resident_norms(t, sc, 0, c.tensor, a0, a1, sh);
+  // phase 2: m, v get their final values; u_g takes the registers of g
+  const LansElem el = make_elem(sc, sh.norm[0], bc1, bc2);
+  a0 = 0.f, a1 = 0.f;
+  tid = opaque_tid();
+#pragma unroll
+  for (int k = 0; k < kVecPerThread; ++k) {
+    const int e = 4 * (tid + k * kLansThreads);
+    f32x4 xm = ld4(m, e), xv = ld4(v, e);
+    const f32x4 xp = sh.p[k][tid];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float sg = el.scaled_grad(xg[k][j], xp[j]);
+      float mm = xm[j], vv = xv[j], u0, u1;
+      el.moments(sg, mm, vv);
+      el.updates(sg, xp[j], mm, vv, u0, u1);
+      xm[j] = mm;
+      xv[j] = vv;
+      xu[k][j] = u0;
+      xg[k][j] = u1;
+      a0 += u0 * u0;
+      a1 += u1 * u1;
+    }
+    st4(m, e, xm);
+    st4(v, e, xv);
+  }
+  a0 = block_sum(a0, sh.red);
+  a1 = block_sum(a1, sh.red);
+  if (threadIdx.x == 0) {
+    st_word(t.part_word + 2 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a0);
+    st_word(t.part_word + 3 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a1);
+  }
+  resident_norms(t, sc, 2, c.tensor, a0, a1, sh);
+  if (threadIdx.x == 0 && chunk == t.tensor_first[c.tensor]) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) t.norms[k * t.T + c.tensor] = sh.norm[k];
+  }
+  // phase 3
+  const float pn = sh.norm[1], umn = sh.norm[2], ugn = sh.norm[3];
+  float ratio_m = (umn != 0.f && pn != 0.f) ? sc.lr * (pn / umn) : sc.lr;
+  float ratio_g = (ugn != 0.f && pn != 0.f) ? sc.lr * (pn / ugn) : sc.lr;
+  ratio_m *= sc.beta1;
+  ratio_g *= sc.beta3;
+  tid = opaque_tid();
+#pragma unroll
+  for (int k = 0; k < kVecPerThread; ++k) {
+    const int e = 4 * (tid + k * kLansThreads);
+    f32x4 xp = sh.p[k][tid];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma clang fp contract(off)
+      xp[j] = xp[j] - (ratio_m * xu[k][j]) - (ratio_g * xg[k][j]);
+    }
+    st4(p, e, xp);
+  }
+}
+
+// A partial or unaligned chunk through the same three phases with the streaming chunk functions of the
+// sweeps (nothing held in registers; m and v written in phase 2 are read back by the thread that wrote
+// them).  At most one chunk per tensor takes this path when arrays are aligned.
+__device__ __forceinline__ void resident_chunk_streamed(const LansTables& t, const LansScalars& sc, const ChunkView& c,
+                                                        int chunk, float bc1, float bc2, ResidentShared& sh) {
+  float a0, a1;
+  chunk_norm_gp(t, c, sh.red, a0, a1);
+  if (threadIdx.x == 0) {
+    st_word(t.part_word + chunk, sc.epoch, a0);
+    st_word(t.part_word + t.nchunks + chunk, sc.epoch, a1);
+  }
+  resident_norms(t, sc, 0, c.tensor, a0, a1, sh);
+  const LansElem el = make_elem(sc, sh.norm[0], bc1, bc2);
+  chunk_moments(t, c, el, sh.red, a0, a1);
+  if (threadIdx.x == 0) {
+    st_word(t.part_word + 2 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a0);
+    st_word(t.part_word + 3 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a1);
+  }
+  resident_norms(t, sc, 2, c.tensor, a0, a1, sh);
+  if (threadIdx.x == 0 && chunk == t.tensor_first[c.tensor]) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) t.norms[k * t.T + c.tensor] = sh.norm[k];
+  }
+  chunk_update(t, c, el, sc, sh.norm[1], sh.norm[2], sh.norm[3]);
+}
+
+// WAVES = waves per SIMD the kernel is compiled for, i.e. workgroups per CU: 3 keeps everything in
+// registers; 4 holds two of the largest supported tensors at once (1024 chunks on 256 CUs) at the price
+// of some register spills, which pays when single tensors fill half the chip.
+template <int WAVES>
+__global__ __launch_bounds__(kLansThreads, WAVES) void lans_resident_kernel(LansTables t, LansScalars sc) {
+  __shared__ ResidentShared sh;
+  float bc1, bc2;
+  bias_corrections(sc, bc1, bc2);
+  while (true) {
+    __syncthreads();  // shared words of the previous chunk are no longer read
+    if (threadIdx.x == 0) sh.chunk = static_cast<int>(atomicAdd(t.ticket, 1u));
+    __syncthreads();
+    const int chunk = sh.chunk;
+    if (chunk >= t.nchunks) break;  // every workgroup reaches this: chunks are finite
+    const ChunkView c = chunk_view(t, chunk);
+    const bool full = c.n == kLansChunk &&
+                      vec_ok(t.g[c.tensor], t.p[c.tensor], t.m[c.tensor], t.v[c.tensor]);
+    if (full) resident_chunk(t, sc, c, chunk, bc1, bc2, sh);
+    else resident_chunk_streamed(t, sc, c, chunk, bc1, bc2, sh);
+  }
+}
+
+}  // namespace lancet
+
+// ---------------------------------------------------------------------------------------
+// plan object and C entry points
+// ---------------------------------------------------------------------------------------
+using namespace lancet;
+
+struct lancet_lans_plan {
+  uint32_t magic;
+  int device;
+  int T;
+  int nchunks;
+  std::vector<int64_t> numels;
+  std::vector<const void*> shadow;  // last uploaded 4T pointers
+  void* dev_block;                  // one allocation holding every table
+  void** h_ptrs;                    // pinned staging for the pointer tables
+  hipEvent_t upload_done;
+  bool upload_pending;
+  LansTables tables;
+  int schedule;           // LANCET_LANS_SWEEPS or LANCET_LANS_RESIDENT
+  int resident_waves;     // kernel variant of the resident schedule (workgroups per CU)
+  int resident_grid;      // workgroups of that variant the device runs at once
+  int max_tensor_chunks;  // chunks of the largest tensor
+  uint32_t epoch;         // step counter that tags the words of the resident schedule
+  size_t words_offset; // part_word + norm_word inside dev_block
+  size_t words_bytes;
+};
+
+static constexpr uint32_t kPlanMagic = 0x4c414e53u;  // "LANS"
+
+static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+static void chunk_tables(const int64_t* numels, int T, std::vector<int32_t>& ctensor, std::vector<int32_t>& first) {
+  first.assign(T + 1, 0);
+  ctensor.clear();
+  int c = 0;
+  for (int i = 0; i < T; ++i) {
+    first[i] = c;
+    const int k = static_cast<int>((numels[i] + kLansChunk - 1) / kLansChunk);
+    for (int j = 0; j < k; ++j) ctensor.push_back(i);
+    c += k;
+  }
+  first[T] = c;
+}
+
+// Host-only view of the chunk -> tensor map a plan builds for `numels` (no device needed).
+extern "C" int64_t lancet_lans_debug_chunk_table(const int64_t* numels, int T, int32_t* chunk_tensor_out,
+                                                 int64_t capacity) {
+  if (!numels || T <= 0) return -1;
+  std::vector<int32_t> ctensor, first;
+  chunk_tables(numels, T, ctensor, first);
+  for (int64_t i = 0; i < capacity && i < static_cast<int64_t>(ctensor.size()); ++i)
+    if (chunk_tensor_out) chunk_tensor_out[i] = ctensor[i];
+  return static_cast<int64_t>(ctensor.size());
+}
+
+extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans_plan_t* out) {
+  if (!numels || !out) return LANCET_ERR_NULL;
+  if (T <= 0) return LANCET_ERR_SHAPE;
+  int64_t nchunks64 = 0;
+  for (int i = 0; i < T; ++i) {
+    if (numels[i] < 0) return LANCET_ERR_SHAPE;
+    nchunks64 += (numels[i] + kLansChunk - 1) / kLansChunk;
+  }
+  if (nchunks64 > 0x7fffffff) return LANCET_ERR_SHAPE;
+  lancet_lans_plan* pl = new (std::nothrow) lancet_lans_plan();
+  if (!pl) return static_cast<int>(hipErrorOutOfMemory);
+  pl->magic = kPlanMagic;
+  pl->T = T;
+  pl->nchunks = static_cast<int>(nchunks64);
+  pl->numels.assign(numels, numels + T);
+  pl->shadow.assign(4 * static_cast<size_t>(T), nullptr);
+  pl->dev_block = nullptr;
+  pl->h_ptrs = nullptr;
+  pl->upload_done = nullptr;
+  pl->upload_pending = false;
+  hipError_t err = hipGetDevice(&pl->device);
+  // device block layout
+  const size_t n = static_cast<size_t>(pl->nchunks);
+  size_t off = 0;
+  const size_t o_ptrs = off;      off = align_up(off + 4 * T * sizeof(void*), 256);
+  const size_t o_numel = off;     off = align_up(off + T * sizeof(int64_t), 256);
+  const size_t o_ctensor = off;   off = align_up(off + (n ? n : 1) * sizeof(int32_t), 256);
+  const size_t o_first = off;     off = align_up(off + (T + 1) * sizeof(int32_t), 256);
+  const size_t o_partial = off;   off = align_up(off + 2 * (n ? n : 1) * sizeof(float), 256);
+  const size_t o_norms = off;     off = align_up(off + 4 * T * sizeof(float), 256);
+  const size_t o_consts = off;    off = align_up(off + 2 * sizeof(float), 256);
+  const size_t o_words = off;     off = align_up(off + 4 * ((n ? n : 1) + T) * sizeof(uint64_t), 256);
+  const size_t o_ticket = off;    off = align_up(off + (2 + 2 * static_cast<size_t>(T)) * sizeof(uint32_t), 256);
+  pl->schedule = LANCET_LANS_SWEEPS;
+  pl->epoch = 0;
+  pl->words_offset = o_words;
+  pl->words_bytes = 4 * ((n ? n : 1) + T) * sizeof(uint64_t);
+  int cus = 256;
+  if (err == hipSuccess) err = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, pl->device);
+  pl->resident_grid = 0;
+  pl->max_tensor_chunks = 0;
+  for (int i = 0; i < T; ++i)
+    pl->max_tensor_chunks = std::max<int>(pl->max_tensor_chunks, static_cast<int>((numels[i] + kLansChunk - 1) / kLansChunk));
+  if (err == hipSuccess) {
+    // the variant with more workgroups per CU only when one tensor would take more than half the chip
+    int per_cu3 = 0, per_cu4 = 0;
+    err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu3, lans_resident_kernel<3>, kLansThreads, 0);
+    if (err == hipSuccess)
+      err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu4, lans_resident_kernel<4>, kLansThreads, 0);
+    const bool wide = 2 * pl->max_tensor_chunks > per_cu3 * cus;
+    pl->resident_waves = wide ? 4 : 3;
+    pl->resident_grid = (wide ? per_cu4 : per_cu3) * cus;
+  }
+  if (err == hipSuccess) err = hipMalloc(&pl->dev_block, off);
+  if (err == hipSuccess) err = hipHostMalloc(reinterpret_cast<void**>(&pl->h_ptrs), 4 * T * sizeof(void*), hipHostMallocDefault);
+  if (err == hipSuccess) err = hipEventCreateWithFlags(&pl->upload_done, hipEventDisableTiming);
+  if (err == hipSuccess) {
+    std::vector<int32_t> ctensor, first;
+    chunk_tables(numels, T, ctensor, first);
+    char* base = static_cast<char*>(pl->dev_block);
+    err = hipMemcpy(base + o_numel, numels, T * sizeof(int64_t), hipMemcpyHostToDevice);
+    if (err == hipSuccess && n) err = hipMemcpy(base + o_ctensor, ctensor.data(), n * sizeof(int32_t), hipMemcpyHostToDevice);
+    if (err == hipSuccess) err = hipMemcpy(base + o_first, first.data(), (T + 1) * sizeof(int32_t), hipMemcpyHostToDevice);
+    if (err == hipSuccess) err = hipMemset(base + o_norms, 0, 4 * T * sizeof(float));
+    if (err == hipSuccess) err = hipMemset(base + o_words, 0, pl->words_bytes);
+    LansTables& t = pl->tables;
+    t.part_word = reinterpret_cast<uint64_t*>(base + o_words);
+    t.norm_word = t.part_word + 4 * (n ? n : 1);
+    t.ticket = reinterpret_cast<uint32_t*>(base + o_ticket);
+    void** dptrs = reinterpret_cast<void**>(base + o_ptrs);
+    t.g = reinterpret_cast<const float* const*>(dptrs);
+    t.p = reinterpret_cast<float* const*>(dptrs + T);
+    t.m = reinterpret_cast<float* const*>(dptrs + 2 * T);
+    t.v = reinterpret_cast<float* const*>(dptrs + 3 * T);
+    t.numel = reinterpret_cast<const int64_t*>(base + o_numel);
+    t.chunk_tensor = reinterpret_cast<const int32_t*>(base + o_ctensor);
+    t.tensor_first = reinterpret_cast<const int32_t*>(base + o_first);
+    t.partial = reinterpret_cast<float*>(base + o_partial);
+    t.norms = reinterpret_cast<float*>(base + o_norms);
+    t.consts = reinterpret_cast<float*>(base + o_consts);
+    t.T = T;
+    t.nchunks = pl->nchunks;
+  }
+  if (err != hipSuccess) {
+    lancet_lans_plan_destroy(pl);
+    return static_cast<int>(err);
+  }
+  *out = pl;
+  return LANCET_OK;
+}
+
+extern "C" int lancet_lans_plan_destroy(lancet_lans_plan_t pl) {
+  if (!pl || pl->magic != kPlanMagic) return LANCET_ERR_PLAN;
+  if (pl->upload_done) {
+    if (pl->upload_pending) (void)hipEventSynchronize(pl->upload_done);
+    (void)hipEventDestroy(pl->upload_done);
+  }
+  if (pl->h_ptrs) (void)hipHostFree(pl->h_ptrs);
+  if (pl->dev_block) (void)hipFree(pl->dev_block);
+  pl->magic = 0;
+  delete pl;
+  return LANCET_OK;
+}
+
+extern "C" int lancet_lans_plan_norms(lancet_lans_plan_t pl, float* norms, lancet_stream_t stream) {
+  if (!pl || pl->magic != kPlanMagic) return LANCET_ERR_PLAN;
+  if (!norms) return LANCET_ERR_NULL;
+  return static_cast<int>(hipMemcpyAsync(norms, pl->tables.norms, 4 * static_cast<size_t>(pl->T) * sizeof(float),
+                                         hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream)));
+}
+
+extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, float* const* p,
+                                float* const* m, float* const* v, int step_host,
+                                const float* step_dev, const lancet_lans_hyper* h,
+                                lancet_stream_t stream) {
+  if (!pl || pl->magic != kPlanMagic) return LANCET_ERR_PLAN;
+  if (!g || !p || !m || !v || !h) return LANCET_ERR_NULL;
+  if (!step_dev && step_host < 1) return LANCET_ERR_SHAPE;
+  if (h->mode != 0 && h->mode != 1) return LANCET_ERR_SHAPE;
+  const int T = pl->T;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  bool changed = false;
+  for (int i = 0; i < T; ++i) {
+    if (pl->numels[i] > 0 && (!g[i] || !p[i] || !m[i] || !v[i])) return LANCET_ERR_NULL;
+    if ((reinterpret_cast<uintptr_t>(g[i]) | reinterpret_cast<uintptr_t>(p[i]) |
+         reinterpret_cast<uintptr_t>(m[i]) | reinterpret_cast<uintptr_t>(v[i])) & 3u)
+      return LANCET_ERR_ALIGN;
+    changed = changed || pl->shadow[i] != g[i] || pl->shadow[T + i] != p[i] ||
+              pl->shadow[2 * T + i] != m[i] || pl->shadow[3 * T + i] != v[i];
+  }
+  hipError_t err = hipSuccess;
+  if (changed) {
+    // the pinned staging buffer may still be the source of the previous upload
+    if (pl->upload_pending) {
+      err = hipEventSynchronize(pl->upload_done);
+      if (err != hipSuccess) return static_cast<int>(err);
+    }
+    for (int i = 0; i < T; ++i) {
+      pl->shadow[i] = pl->h_ptrs[i] = const_cast<float*>(g[i]);
+      pl->shadow[T + i] = pl->h_ptrs[T + i] = p[i];
+      pl->shadow[2 * T + i] = pl->h_ptrs[2 * T + i] = m[i];
+      pl->shadow[3 * T + i] = pl->h_ptrs[3 * T + i] = v[i];
+    }
+    err = hipMemcpyAsync(pl->dev_block, pl->h_ptrs,
+                         4 * static_cast<size_t>(T) * sizeof(void*), hipMemcpyHostToDevice, st);
+    if (err == hipSuccess) err = hipEventRecord(pl->upload_done, st);
+    if (err != hipSuccess) return static_cast<int>(err);
+    pl->upload_pending = true;
+  }
+  if (pl->nchunks == 0) return LANCET_OK;
+  LansScalars sc;
+  sc.lr = h->learning_rate;
+  sc.beta1 = h->beta1;
+  sc.beta2 = h->beta2;
+  sc.beta3 = h->grad_averaging ? 1.f - h->beta1 : 1.f;
+  sc.eps = h->eps;
+  sc.wd = h->weight_decay;
+  sc.mode = h->mode;
+  sc.normalize_grad = h->normalize_grad;
+  sc.bias_correction = h->bias_correction;
+  sc.step_host = step_host;
+  sc.step_dev = step_dev;
+  const LansTables& t = pl->tables;
+  sc.spin_limit = current_spin_limit();
+  if (pl->schedule == LANCET_LANS_RESIDENT) {
+    if (++pl->epoch == 0) {
+      err = hipMemsetAsync(static_cast<char*>(pl->dev_block) + pl->words_offset, 0, pl->words_bytes, st);
+      if (err != hipSuccess) return static_cast<int>(err);
+      pl->epoch = 1;
+    }
+    sc.epoch = pl->epoch;
+    err = run_fill_u32(t.ticket, 2 + 2 * static_cast<size_t>(T), 0u, st);
+    if (err != hipSuccess) return static_cast<int>(err);
+    const int grid = std::min(pl->resident_grid, t.nchunks);
+    if (pl->resident_waves == 4) lans_resident_kernel<4><<<grid, kLansThreads, 0, st>>>(t, sc);
+    else lans_resident_kernel<3><<<grid, kLansThreads, 0, st>>>(t, sc);
+    return static_cast<int>(hipGetLastError());
+  }
+  sc.epoch = 0;
+  const int rblocks = (T + kLansThreads / kWave - 1) / (kLansThreads / kWave);
+  lans_prepare_kernel<<<1, 64, 0, st>>>(t, sc);
+  lans_norm_gp_kernel<<<t.nchunks, kLansThreads, 0, st>>>(t);
+  lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 0);
+  lans_moments_kernel<<<t.nchunks, kLansThreads, 0, st>>>(t, sc);
+  lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 2);
+  lans_update_kernel<<<t.nchunks, kLansThreads, 0, st>>>(t, sc);
+  return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int lancet_lans_plan_set_schedule(lancet_lans_plan_t pl, int schedule) {
+  if (!pl || pl->magic != kPlanMagic) return LANCET_ERR_PLAN;
+  if (schedule != LANCET_LANS_SWEEPS && schedule != LANCET_LANS_RESIDENT) return LANCET_ERR_SHAPE;
+  // a tensor's chunks must all be held by running workgroups at once
+  if (schedule == LANCET_LANS_RESIDENT && pl->max_tensor_chunks > std::min(pl->resident_grid, kMaxResidentChunks))
+    return LANCET_ERR_SHAPE;
+  pl->schedule = schedule;
+  return LANCET_OK;
+}
+
+extern "C" int lancet_lans_plan_resident_capacity(lancet_lans_plan_t pl, int* workgroups, int* max_tensor_chunks) {
+  if (!pl || pl->magic != kPlanMagic) return LANCET_ERR_PLAN;
+  if (workgroups) *workgroups = std::min(pl->resident_grid, kMaxResidentChunks);
+  if (max_tensor_chunks) *max_tensor_chunks = pl->max_tensor_chunks;
+  return LANCET_OK;
+}
+
+extern "C" int lancet_lans_plan_error(lancet_lans_plan_t pl, lancet_stream_t stream, int* error_out) {
+  if (!pl || pl->magic != kPlanMagic) return LANCET_ERR_PLAN;
+  if (!error_out) return LANCET_ERR_NULL;
+  uint32_t word = 0;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipError_t e = hipMemcpyAsync(&word, pl->tables.ticket + 1, sizeof(word), hipMemcpyDeviceToHost, st);
+  if (e == hipSuccess) e = hipStreamSynchronize(st);
+  *error_out = static_cast<int>(word);
+  return static_cast<int>(e);
+}

@@ -38,6 +38,16 @@ __device__ __forceinline__ void st_release_agent(uint32_t* p, uint32_t v) {
   __hip_atomic_store(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// ---- pointers known to be device global memory ------------------------------------------
+// A pointer read from a table in memory, or picked at run time among several, is a generic (flat)
+// pointer to the compiler: flat loads and stores need a 64-bit address in vector registers each.
+// Typed as global memory they take a scalar base plus a 32-bit offset.
+#define LANCET_GLOBAL __attribute__((address_space(1)))
+template <typename T>
+__device__ __forceinline__ LANCET_GLOBAL T* as_global(T* p) {
+  return (LANCET_GLOBAL T*)p;
+}
+
 // ---- 16-byte streaming row moves ---------------------------------------------------
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 

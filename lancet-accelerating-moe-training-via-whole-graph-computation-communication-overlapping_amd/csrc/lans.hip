@@ -92,9 +92,9 @@ __device__ __forceinline__ ChunkView chunk_view(const LansTables& t, int chunk) 
   return c;
 }
 
-__device__ __forceinline__ bool vec_ok(const void* a, const void* b, const void* c, const void* d) {
-  return ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) |
-           reinterpret_cast<uintptr_t>(c) | reinterpret_cast<uintptr_t>(d)) & 15u) == 0;
+template <typename A, typename B, typename C, typename D>
+__device__ __forceinline__ bool vec_ok(A a, B b, C c, D d) {
+  return (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)d) & 15u) == 0;
 }
 
 // ---- elementwise math, in the reference's operation order (multi_tensor_lans.cu:283-307) ----
@@ -162,14 +162,14 @@ __device__ __forceinline__ void bias_corrections(const LansScalars& sc, float& b
 // phase 1: sums of squares of g and p (L2NormFunctor, multi_tensor_lans.cu:95-167); valid on thread 0
 __device__ __forceinline__ void chunk_norm_gp(const LansTables& t, const ChunkView& c, float* s_red,
                                               float& sum_g, float& sum_p) {
-  const float* g = t.g[c.tensor] + c.begin;
-  const float* p = t.p[c.tensor] + c.begin;
+  const LANCET_GLOBAL float* g = as_global(t.g[c.tensor] + c.begin);
+  const LANCET_GLOBAL float* p = as_global(t.p[c.tensor] + c.begin);
   float ag = 0.f, ap = 0.f;
   int scalar_from = 0;
   if (vec_ok(g, p, g, p)) {
     const int nv = c.n / 4;
-    const f32x4* g4 = reinterpret_cast<const f32x4*>(g);
-    const f32x4* p4 = reinterpret_cast<const f32x4*>(p);
+    const LANCET_GLOBAL f32x4* g4 = (const LANCET_GLOBAL f32x4*)g;
+    const LANCET_GLOBAL f32x4* p4 = (const LANCET_GLOBAL f32x4*)p;
 #pragma unroll 4
     for (int i = threadIdx.x; i < nv; i += kLansThreads) {
       const f32x4 x = g4[i], y = p4[i];
@@ -190,18 +190,18 @@ __device__ __forceinline__ void chunk_norm_gp(const LansTables& t, const ChunkVi
 // l2norm sweeps after it, :434-441); sums valid on thread 0
 __device__ __forceinline__ void chunk_moments(const LansTables& t, const ChunkView& c, const LansElem& el,
                                               float* s_red, float& sum_um, float& sum_ug) {
-  const float* g = t.g[c.tensor] + c.begin;
-  const float* p = t.p[c.tensor] + c.begin;
-  float* m = t.m[c.tensor] + c.begin;
-  float* v = t.v[c.tensor] + c.begin;
+  const LANCET_GLOBAL float* g = as_global(t.g[c.tensor] + c.begin);
+  const LANCET_GLOBAL float* p = as_global(t.p[c.tensor] + c.begin);
+  LANCET_GLOBAL float* m = as_global(t.m[c.tensor] + c.begin);
+  LANCET_GLOBAL float* v = as_global(t.v[c.tensor] + c.begin);
   float am = 0.f, ag = 0.f;
   int scalar_from = 0;
   if (vec_ok(g, p, m, v)) {
     const int nv = c.n / 4;
-    const f32x4* g4 = reinterpret_cast<const f32x4*>(g);
-    const f32x4* p4 = reinterpret_cast<const f32x4*>(p);
-    f32x4* m4 = reinterpret_cast<f32x4*>(m);
-    f32x4* v4 = reinterpret_cast<f32x4*>(v);
+    const LANCET_GLOBAL f32x4* g4 = (const LANCET_GLOBAL f32x4*)g;
+    const LANCET_GLOBAL f32x4* p4 = (const LANCET_GLOBAL f32x4*)p;
+    LANCET_GLOBAL f32x4* m4 = (LANCET_GLOBAL f32x4*)m;
+    LANCET_GLOBAL f32x4* v4 = (LANCET_GLOBAL f32x4*)v;
 #pragma unroll 2
     for (int i = threadIdx.x; i < nv; i += kLansThreads) {
       const f32x4 xg = g4[i], xp = p4[i];
@@ -243,17 +243,17 @@ __device__ __forceinline__ void chunk_update(const LansTables& t, const ChunkVie
   float ratio_g = (ugn != 0.f && pn != 0.f) ? sc.lr * (pn / ugn) : sc.lr;
   ratio_m *= sc.beta1;
   ratio_g *= sc.beta3;
-  const float* g = t.g[c.tensor] + c.begin;
-  float* p = t.p[c.tensor] + c.begin;
-  const float* m = t.m[c.tensor] + c.begin;
-  const float* v = t.v[c.tensor] + c.begin;
+  const LANCET_GLOBAL float* g = as_global(t.g[c.tensor] + c.begin);
+  LANCET_GLOBAL float* p = as_global(t.p[c.tensor] + c.begin);
+  const LANCET_GLOBAL float* m = as_global(t.m[c.tensor] + c.begin);
+  const LANCET_GLOBAL float* v = as_global(t.v[c.tensor] + c.begin);
   int scalar_from = 0;
   if (vec_ok(g, p, m, v)) {
     const int nv = c.n / 4;
-    const f32x4* g4 = reinterpret_cast<const f32x4*>(g);
-    f32x4* p4 = reinterpret_cast<f32x4*>(p);
-    const f32x4* m4 = reinterpret_cast<const f32x4*>(m);
-    const f32x4* v4 = reinterpret_cast<const f32x4*>(v);
+    const LANCET_GLOBAL f32x4* g4 = (const LANCET_GLOBAL f32x4*)g;
+    LANCET_GLOBAL f32x4* p4 = (LANCET_GLOBAL f32x4*)p;
+    const LANCET_GLOBAL f32x4* m4 = (const LANCET_GLOBAL f32x4*)m;
+    const LANCET_GLOBAL f32x4* v4 = (const LANCET_GLOBAL f32x4*)v;
 #pragma unroll 2
     for (int i = threadIdx.x; i < nv; i += kLansThreads) {
       const f32x4 xg = g4[i], xm = m4[i], xv = v4[i];
@@ -356,8 +356,8 @@ __device__ __forceinline__ void st_word(uint64_t* p, uint32_t epoch, float v) {
 // =======================================================================================
 constexpr int kVecPerThread = kLansChunk / 4 / kLansThreads;  // float4 per thread and array
 
-__device__ __forceinline__ f32x4 ld4(const float* a, int e) { return *reinterpret_cast<const f32x4*>(a + e); }
-__device__ __forceinline__ void st4(float* a, int e, f32x4 x) { *reinterpret_cast<f32x4*>(a + e) = x; }
+__device__ __forceinline__ f32x4 ld4(const LANCET_GLOBAL float* a, int e) { return *(const LANCET_GLOBAL f32x4*)(a + e); }
+__device__ __forceinline__ void st4(LANCET_GLOBAL float* a, int e, f32x4 x) { *(LANCET_GLOBAL f32x4*)(a + e) = x; }
 
 constexpr int kMaxResidentChunks = 512;  // chunks of one tensor the resident schedule can gather
 
@@ -437,16 +437,20 @@ __device__ __forceinline__ void resident_norms(const LansTables& t, const LansSc
 // written once.
 __device__ __forceinline__ void resident_chunk(const LansTables& t, const LansScalars& sc, const ChunkView& c, int chunk,
                                                float bc1, float bc2, ResidentShared& sh) {
-  const float* g = t.g[c.tensor] + c.begin;
-  float* p = t.p[c.tensor] + c.begin;
-  float* m = t.m[c.tensor] + c.begin;
-  float* v = t.v[c.tensor] + c.begin;
+  const LANCET_GLOBAL float* g = as_global(t.g[c.tensor] + c.begin);
+  LANCET_GLOBAL float* p = as_global(t.p[c.tensor] + c.begin);
+  LANCET_GLOBAL float* m = as_global(t.m[c.tensor] + c.begin);
+  LANCET_GLOBAL float* v = as_global(t.v[c.tensor] + c.begin);
   f32x4 xg[kVecPerThread], xu[kVecPerThread];
+  // a wave owns 2048 consecutive elements: float4 k of lane l is element 4 * (64 k + l) of them, so one
+  // load instruction of a wave covers 1 KB of consecutive memory and the eight of a thread differ by
+  // constant offsets
+  const int e0 = (threadIdx.x / kWave) * (kLansChunk / kWavesPerTile) + 4 * lane_id();
   // phase 1
   float a0 = 0.f, a1 = 0.f;
 #pragma unroll
   for (int k = 0; k < kVecPerThread; ++k) {
-    const int e = 4 * (threadIdx.x + k * kLansThreads);
+    const int e = e0 + k * (4 * kWave);
     xg[k] = ld4(g, e);
     const f32x4 xp = ld4(p, e);
     sh.p[k][threadIdx.x] = xp;
@@ -468,7 +472,7 @@ __device__ __forceinline__ void resident_chunk(const LansTables& t, const LansSc
   a0 = 0.f, a1 = 0.f;
 #pragma unroll
   for (int k = 0; k < kVecPerThread; ++k) {
-    const int e = 4 * (threadIdx.x + k * kLansThreads);
+    const int e = e0 + k * (4 * kWave);
     f32x4 xm = ld4(m, e), xv = ld4(v, e);
     const f32x4 xp = sh.p[k][threadIdx.x];
 #pragma unroll
@@ -506,7 +510,7 @@ __device__ __forceinline__ void resident_chunk(const LansTables& t, const LansSc
   ratio_g *= sc.beta3;
 #pragma unroll
   for (int k = 0; k < kVecPerThread; ++k) {
-    const int e = 4 * (threadIdx.x + k * kLansThreads);
+    const int e = e0 + k * (4 * kWave);
     f32x4 xp = sh.p[k][threadIdx.x];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -555,7 +559,8 @@ __global__ __launch_bounds__(kLansThreads, WAVES) void lans_resident_kernel(Lans
     __syncthreads();  // shared words of the previous chunk are no longer read
     if (threadIdx.x == 0) sh.chunk = static_cast<int>(atomicAdd(t.ticket, 1u));
     __syncthreads();
-    const int chunk = sh.chunk;
+    // one value for the whole workgroup, and known to be: pointers and sizes derived from it stay scalar
+    const int chunk = __builtin_amdgcn_readfirstlane(sh.chunk);
     if (chunk >= t.nchunks) break;  // every workgroup reaches this: chunks are finite
     const ChunkView c = chunk_view(t, chunk);
     const bool full = c.n == kLansChunk &&

@@ -17,6 +17,8 @@ __device__ __forceinline__ V ldv(const V* p) { return __builtin_nontemporal_load
 template <typename V>
 __device__ __forceinline__ void stv(V* p, V v) { __builtin_nontemporal_store(v, p); }
 template <typename V>
+__device__ __forceinline__ void stv(LANCET_GLOBAL V* p, V v) { __builtin_nontemporal_store(v, p); }
+template <typename V>
 __device__ __forceinline__ V zero_v() { return V(0); }
 template <>
 __device__ __forceinline__ u32x4 zero_v<u32x4>() { return u32x4{0u, 0u, 0u, 0u}; }
@@ -48,7 +50,8 @@ __global__ __launch_bounds__(kTile) void scatter_rows_kernel(ScatterArgs<V> a) {
   if (static_cast<int>(blockIdx.x) < a.token_blocks) {
     const int s = blockIdx.x * kRowsPerBlock + w;
     if (s >= a.S) return;
-    V* dst[K];
+    // destinations picked at run time: typed as global memory so the stores are not flat
+    LANCET_GLOBAL V* dst[K];
     int nd = 0;
 #pragma unroll
     for (int j = 0; j < K; ++j) {
@@ -56,8 +59,8 @@ __global__ __launch_bounds__(kTile) void scatter_rows_kernel(ScatterArgs<V> a) {
       const int l = a.loc[static_cast<size_t>(j) * a.S + s];
       bool ok = e >= 0 && e < a.E && l >= 0 && l < a.C;
       if (ok && a.avail_used) ok = l < a.C - a.avail_used[e];
-      dst[j] = nullptr;
-      if (ok) dst[nd++] = a.out + (static_cast<size_t>(e) * a.C + l) * a.row_vecs;
+      dst[j] = as_global(a.out);
+      if (ok) dst[nd++] = as_global(a.out + (static_cast<size_t>(e) * a.C + l) * a.row_vecs);
     }
     if (nd == 0) return;
     const V* src = a.data + static_cast<size_t>(s) * a.row_vecs;

@@ -8,6 +8,7 @@ gate_is_logits, workspace, out).  torch supplies device memory and the current
 stream; all computation is done by the HIP kernels behind the C ABI.
 """
 import ctypes as C
+import os
 
 import torch
 
@@ -454,6 +455,11 @@ def lans(tensor_list, step, learning_rate, beta1, beta2, eps, bias_correction, w
     plan = _PLANS.get(key)
     if plan is None:
         plan = _PLANS[key] = LansPlan(key[0])
+        if os.environ.get("LANCET_LANS_SCHEDULE") == "resident":
+            try:
+                plan.set_schedule(capi.LANS_RESIDENT)
+            except RuntimeError:      # a tensor too large for it: the three sweeps stay
+                pass
     hyper = capi.LansHyper(float(learning_rate), float(beta1), float(beta2), float(eps), int(bias_correction),
                            float(weight_decay), int(grad_averaging), int(mode), int(bool(normalize_grad)))
     if torch.is_tensor(step):

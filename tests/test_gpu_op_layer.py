@@ -55,8 +55,11 @@ def test_bpr_merge_redispatch_through_the_op_layer(pkg, ex):
     np.testing.assert_array_equal(to_np(red), mo.moe_redispatch(o_bufs, o_ils))
 
 
-def test_lans_through_the_op_layer_with_cached_openv(pkg, ex):
-    shapes = [(128, 64), (33,), (5000,)]
+@pytest.mark.parametrize("schedule", ["sweeps", "resident"])
+def test_lans_through_the_op_layer_with_cached_openv(pkg, ex, monkeypatch, schedule):
+    # the OpEnv reads LANCET_LANS_SCHEDULE when it is built
+    monkeypatch.setenv("LANCET_LANS_SCHEDULE", schedule)
+    shapes = [(128, 64), (33,), (5000,), (3, 8192)]
     rng = np.random.default_rng(0)
     p = [rng.normal(0, 0.02, s).astype(np.float32) for s in shapes]
     m = [np.zeros(s, np.float32) for s in shapes]

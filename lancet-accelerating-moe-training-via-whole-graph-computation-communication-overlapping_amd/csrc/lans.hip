@@ -97,6 +97,12 @@ __device__ __forceinline__ bool vec_ok(A a, B b, C c, D d) {
   return (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)d) & 15u) == 0;
 }
 
+// A value every lane holds alike, moved to a scalar register: it then costs no vector register
+// for as long as it lives.
+__device__ __forceinline__ float uniform(float x) {
+  return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(x)));
+}
+
 // ---- elementwise math, in the reference's operation order (multi_tensor_lans.cu:283-307) ----
 struct LansElem {
   float gnorm_eps;  // ||g|| + eps
@@ -131,14 +137,14 @@ struct LansElem {
 
 __device__ __forceinline__ LansElem make_elem(const LansScalars& sc, float gn, float bc1, float bc2) {
   LansElem e;
-  e.gnorm_eps = gn + sc.eps;
-  e.normalize = sc.normalize_grad && gn != 0.f;
+  e.gnorm_eps = uniform(gn + sc.eps);
+  e.normalize = sc.normalize_grad && uniform(gn) != 0.f;
   e.beta1 = sc.beta1;
   e.beta2 = sc.beta2;
   e.beta3 = sc.beta3;
-  e.one_minus_beta2 = 1.f - sc.beta2;
-  e.bc1 = bc1;
-  e.bc2 = bc2;
+  e.one_minus_beta2 = uniform(1.f - sc.beta2);
+  e.bc1 = uniform(bc1);
+  e.bc2 = uniform(bc2);
   e.eps = sc.eps;
   e.wd = sc.wd;
   e.mode = sc.mode;
@@ -503,11 +509,11 @@ __device__ __forceinline__ void resident_chunk(const LansTables& t, const LansSc
     for (int k = 0; k < 4; ++k) t.norms[k * t.T + c.tensor] = sh.norm[k];
   }
   // phase 3
-  const float pn = sh.norm[1], umn = sh.norm[2], ugn = sh.norm[3];
+  const float pn = uniform(sh.norm[1]), umn = uniform(sh.norm[2]), ugn = uniform(sh.norm[3]);
   float ratio_m = (umn != 0.f && pn != 0.f) ? sc.lr * (pn / umn) : sc.lr;
   float ratio_g = (ugn != 0.f && pn != 0.f) ? sc.lr * (pn / ugn) : sc.lr;
-  ratio_m *= sc.beta1;
-  ratio_g *= sc.beta3;
+  ratio_m = uniform(ratio_m * sc.beta1);
+  ratio_g = uniform(ratio_g * sc.beta3);
 #pragma unroll
   for (int k = 0; k < kVecPerThread; ++k) {
     const int e = e0 + k * (4 * kWave);

@@ -113,7 +113,9 @@ def bench_lans(ops, capi, steps, warmup, scale, only_schedule=None):
     return {"tensors": len(shapes), "params": total, "ms_per_step": round(ms, 4), "schedule": best,
             "ms_per_step_by_schedule": {k: round(v, 4) for k, v in timed.items()},
             "algorithmic_GBps": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
-            "bytes_per_param_algorithmic": 28, "bytes_per_param_traffic": {"sweeps": 52, "resident": 28},
+            "bytes_per_param_algorithmic": 28,
+            # HBM bytes per parameter measured with rocprofv3 --pmc (profiles/scatter_decode_lans_hbm_traffic.md)
+            "bytes_per_param_traffic_measured": {"sweeps": 52.0, "resident": 39.1},
             "steps": steps}
 
 

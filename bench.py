@@ -3,7 +3,10 @@
 A "step" is one pass of the hot path over one batch of synthetic input: raf.op.moe_encode
 (routing + scatter) followed by raf.op.moe_decode at the headline shape of BASELINE.json
 (S=65536 tokens, M=4096 bf16, E=32 experts, top-2, capacity factor 1.25 -> C=5120), inputs
-resident in HBM.  Prints ONE JSON line (see README / DESIGN.md for the fields).
+resident in HBM.  Prints ONE JSON line: metric / value / unit (tokens per second of encode + decode),
+`roofline` (the scatter kernel against 8 TB/s of HBM, timed with HIP events), `ops`, `backward`,
+`config4_partitioned`, `pipeline`, `lans` (per-phase and side workloads) and `cpu_baseline` (the C/OpenMP
+restatement of the reference's algorithm timed on this host).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-lans] [--no-cpu]
 """
@@ -114,7 +117,7 @@ def bench_lans(ops, capi, steps, warmup, scale, only_schedule=None):
             "ms_per_step_by_schedule": {k: round(v, 4) for k, v in timed.items()},
             "algorithmic_GBps": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
             "bytes_per_param_algorithmic": 28,
-            # HBM bytes per parameter measured with rocprofv3 --pmc (profiles/scatter_decode_lans_hbm_traffic.md)
+            # HBM bytes per parameter measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this workload
             "bytes_per_param_traffic_measured": {"sweeps": 52.0, "resident": 39.1},
             "steps": steps}
 

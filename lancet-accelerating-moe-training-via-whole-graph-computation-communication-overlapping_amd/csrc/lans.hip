@@ -487,6 +487,9 @@ __device__ __forceinline__ void resident_chunk(const LansTables& t, const LansSc
       float mm = xm[j], vv = xv[j], u0, u1;
       el.moments(sg, mm, vv);
       el.updates(sg, xp[j], mm, vv, u0, u1);
+      // the two updates are final here: nothing of their computation may be left for phase 3 (the
+      // compiler otherwise carries a third value per element, wd * p, across the wait)
+      asm volatile("" : "+v"(u0), "+v"(u1));
       xm[j] = mm;
       xv[j] = vv;
       xu[k][j] = u0;
@@ -553,11 +556,11 @@ __device__ __forceinline__ void resident_chunk_streamed(const LansTables& t, con
   chunk_update(t, c, el, sc, sh.norm[1], sh.norm[2], sh.norm[3]);
 }
 
-// WAVES = waves per SIMD the kernel is compiled for, i.e. workgroups per CU: 3 keeps everything in
-// registers; 4 holds two of the largest supported tensors at once (1024 chunks on 256 CUs) at the price
-// of some register spills, which pays when single tensors fill half the chip.
-template <int WAVES>
-__global__ __launch_bounds__(kLansThreads, WAVES) void lans_resident_kernel(LansTables t, LansScalars sc) {
+// Compiled for four waves per SIMD (128 registers per lane), i.e. four workgroups per CU, which is also
+// what the 36 KB of LDS per workgroup allows: 1024 chunks on 256 CUs, two of the largest supported
+// tensors at once, so that memory stays busy while the workgroups of one tensor wait.
+constexpr int kResidentWavesPerSimd = 4;
+__global__ __launch_bounds__(kLansThreads, kResidentWavesPerSimd) void lans_resident_kernel(LansTables t, LansScalars sc) {
   __shared__ ResidentShared sh;
   float bc1, bc2;
   bias_corrections(sc, bc1, bc2);
@@ -596,8 +599,7 @@ struct lancet_lans_plan {
   bool upload_pending;
   LansTables tables;
   int schedule;           // LANCET_LANS_SWEEPS or LANCET_LANS_RESIDENT
-  int resident_waves;     // kernel variant of the resident schedule (workgroups per CU)
-  int resident_grid;      // workgroups of that variant the device runs at once
+  int resident_grid;      // workgroups of the resident schedule the device runs at once
   int max_tensor_chunks;  // chunks of the largest tensor
   uint32_t epoch;         // step counter that tags the words of the resident schedule
   size_t words_offset; // part_word + norm_word inside dev_block
@@ -676,14 +678,9 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
   for (int i = 0; i < T; ++i)
     pl->max_tensor_chunks = std::max<int>(pl->max_tensor_chunks, static_cast<int>((numels[i] + kLansChunk - 1) / kLansChunk));
   if (err == hipSuccess) {
-    // the variant with more workgroups per CU only when one tensor would take more than half the chip
-    int per_cu3 = 0, per_cu4 = 0;
-    err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu3, lans_resident_kernel<3>, kLansThreads, 0);
-    if (err == hipSuccess)
-      err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu4, lans_resident_kernel<4>, kLansThreads, 0);
-    const bool wide = 2 * pl->max_tensor_chunks > per_cu3 * cus;
-    pl->resident_waves = wide ? 4 : 3;
-    pl->resident_grid = (wide ? per_cu4 : per_cu3) * cus;
+    int per_cu = 0;
+    err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lans_resident_kernel, kLansThreads, 0);
+    pl->resident_grid = per_cu * cus;
   }
   if (err == hipSuccess) err = hipMalloc(&pl->dev_block, off);
   if (err == hipSuccess) err = hipHostMalloc(reinterpret_cast<void**>(&pl->h_ptrs), 4 * T * sizeof(void*), hipHostMallocDefault);
@@ -806,8 +803,7 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
     err = run_fill_u32(t.ticket, 2 + 2 * static_cast<size_t>(T), 0u, st);
     if (err != hipSuccess) return static_cast<int>(err);
     const int grid = std::min(pl->resident_grid, t.nchunks);
-    if (pl->resident_waves == 4) lans_resident_kernel<4><<<grid, kLansThreads, 0, st>>>(t, sc);
-    else lans_resident_kernel<3><<<grid, kLansThreads, 0, st>>>(t, sc);
+    lans_resident_kernel<<<grid, kLansThreads, 0, st>>>(t, sc);
     return static_cast<int>(hipGetLastError());
   }
   sc.epoch = 0;

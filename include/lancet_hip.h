@@ -268,14 +268,15 @@ int lancet_lans_step(lancet_lans_plan_t plan, const float* const* g, float* cons
                      const lancet_lans_hyper* hyper, lancet_stream_t stream);
 /* Schedules of the step.  LANCET_LANS_SWEEPS (default): three whole-state sweeps with two per-tensor
  * reductions between them (52 B/param of traffic).  LANCET_LANS_RESIDENT: one persistent kernel that keeps
- * each chunk on chip across the two reductions (28 B/param); every tensor must fit on the chip at once
- * (lancet_lans_plan_resident_capacity), else set_schedule returns LANCET_ERR_SHAPE and the plan keeps its
- * schedule.  Each schedule is deterministic; the two agree to fp32 rounding of the per-chunk sums. */
+ * each chunk on chip across the two reductions (28 B/param) for the tensors that fit on the chip at once
+ * (lancet_lans_plan_resident_capacity) and the three sweeps, in the same step, for the larger ones; a plan
+ * with no tensor that fits gets LANCET_ERR_SHAPE from set_schedule and keeps its schedule.  Each schedule is deterministic; the two agree to fp32 rounding of the per-chunk sums. */
 #define LANCET_LANS_SWEEPS 0
 #define LANCET_LANS_RESIDENT 1
 int lancet_lans_plan_set_schedule(lancet_lans_plan_t plan, int schedule);
-/* workgroups: chunks (of 8192 parameters) the resident schedule holds at once on this device = the
- * largest tensor it accepts; max_tensor_chunks: chunks of the plan's largest tensor.  Either may be NULL. */
+/* workgroups: chunks (of 8192 parameters) of the largest tensor the resident kernel takes on this device
+ * (larger tensors of the plan go through the sweeps); max_tensor_chunks: chunks of the plan's largest
+ * tensor.  Either may be NULL. */
 int lancet_lans_plan_resident_capacity(lancet_lans_plan_t plan, int* workgroups, int* max_tensor_chunks);
 /* Reads (synchronously) the plan's error word: 1 when a bounded wait of the resident schedule
  * gave up (results of that step are undefined). */
@@ -286,9 +287,13 @@ int lancet_lans_plan_error(lancet_lans_plan_t plan, lancet_stream_t stream, int*
  * norms4xT, a device buffer of 4*T floats, asynchronously on `stream`. */
 int lancet_lans_plan_norms(lancet_lans_plan_t plan, float* norms4xT, lancet_stream_t stream);
 
-/* Host-only view of what a plan builds for `numels` (no device needed): the chunk -> tensor map.
- * Returns the number of chunks; fills at most `capacity` entries (chunk_tensor_out may be NULL). */
-int64_t lancet_lans_debug_chunk_table(const int64_t* numels, int T, int32_t* chunk_tensor_out, int64_t capacity);
+/* Host-only view of what a plan builds for `numels` when the resident kernel takes tensors of up to
+ * resident_limit chunks (no device needed): for every chunk, in the order the kernel hands them out, the
+ * position of its tensor in the caller's list; *n_resident_chunks = how many the resident kernel hands out
+ * (the rest go through the sweeps).  Returns the number of chunks; fills at most `capacity` entries
+ * (either output may be NULL). */
+int64_t lancet_lans_debug_chunk_table(const int64_t* numels, int T, int resident_limit, int32_t* chunk_tensor_out,
+                                      int64_t capacity, int64_t* n_resident_chunks);
 
 /* Test hook: number of polls a workgroup of the position scan waits for a predecessor
  * before it gives up, flags the workspace and finishes with undefined results

@@ -77,7 +77,7 @@ SIGNATURES = {
     "lancet_lans_plan_norms": (_int, [_vp, _vp, _vp]),
     "lancet_lans_plan_set_schedule": (_int, [_vp, _int]),
     "lancet_lans_plan_error": (_int, [_vp, _vp, C.POINTER(_int)]),
-    "lancet_lans_debug_chunk_table": (_i64, [C.POINTER(_i64), _int, _vp, _i64]),
+    "lancet_lans_debug_chunk_table": (_i64, [C.POINTER(_i64), _int, _int, _vp, _i64, C.POINTER(_i64)]),
     "lancet_lans_plan_resident_capacity": (_int, [_vp, C.POINTER(_int), C.POINTER(_int)]),
     "lancet_debug_set_spin_limit": (None, [_u32]),
     "lancet_scan_workspace_error": (_int, [_vp, _vp, C.POINTER(_int)]),

@@ -50,8 +50,10 @@ struct LansTables {
   uint32_t* ticket;            // [1] next task; [1] error flag; [2][T] arrivals (resident schedule)
   float* norms;                // [4][T]: g, p, u_m, u_g
   float* consts;               // [2]: bias_correction1, bias_correction2
+  const int32_t* order;        // [T] position in the caller's lists of the plan's i-th tensor
   int T;
   int nchunks;
+  int nres;                    // chunks [0, nres) belong to tensors the resident schedule can hold
 };
 
 struct LansScalars {
@@ -303,20 +305,23 @@ __global__ void lans_prepare_kernel(LansTables t, LansScalars sc) {
   if (threadIdx.x == 0 && blockIdx.x == 0) bias_corrections(sc, t.consts[0], t.consts[1]);
 }
 
-__global__ __launch_bounds__(kLansThreads) void lans_norm_gp_kernel(LansTables t) {
+// The sweeps cover chunks [chunk_base, nchunks) and tensors [tensor_base, T): everything, or what the
+// resident kernel left (tensors too large for it).
+__global__ __launch_bounds__(kLansThreads) void lans_norm_gp_kernel(LansTables t, int chunk_base) {
   __shared__ float s_red[kLansThreads / kWave];
-  const ChunkView c = chunk_view(t, blockIdx.x);
+  const int chunk = chunk_base + blockIdx.x;
+  const ChunkView c = chunk_view(t, chunk);
   float sg, sp;
   chunk_norm_gp(t, c, s_red, sg, sp);
   if (threadIdx.x == 0) {
-    t.partial[blockIdx.x] = sg;
-    t.partial[t.nchunks + blockIdx.x] = sp;
+    t.partial[chunk] = sg;
+    t.partial[t.nchunks + chunk] = sp;
   }
 }
 
 // per-tensor sqrt(sum of chunk partials) (cleanup, multi_tensor_lans.cu:169-185)
-__global__ __launch_bounds__(kLansThreads) void lans_reduce_kernel(LansTables t, int first_norm) {
-  const int tensor = blockIdx.x * (kLansThreads / kWave) + threadIdx.x / kWave;
+__global__ __launch_bounds__(kLansThreads) void lans_reduce_kernel(LansTables t, int first_norm, int tensor_base) {
+  const int tensor = tensor_base + blockIdx.x * (kLansThreads / kWave) + threadIdx.x / kWave;
   if (tensor >= t.T) return;
   const int lo = t.tensor_first[tensor], hi = t.tensor_first[tensor + 1];
 #pragma unroll
@@ -327,22 +332,31 @@ __global__ __launch_bounds__(kLansThreads) void lans_reduce_kernel(LansTables t,
   }
 }
 
-__global__ __launch_bounds__(kLansThreads) void lans_moments_kernel(LansTables t, LansScalars sc) {
+__global__ __launch_bounds__(kLansThreads) void lans_moments_kernel(LansTables t, LansScalars sc, int chunk_base) {
   __shared__ float s_red[kLansThreads / kWave];
-  const ChunkView c = chunk_view(t, blockIdx.x);
+  const int chunk = chunk_base + blockIdx.x;
+  const ChunkView c = chunk_view(t, chunk);
   const LansElem el = make_elem(sc, t.norms[c.tensor], t.consts[0], t.consts[1]);
   float sm, sg;
   chunk_moments(t, c, el, s_red, sm, sg);
   if (threadIdx.x == 0) {
-    t.partial[blockIdx.x] = sm;
-    t.partial[t.nchunks + blockIdx.x] = sg;
+    t.partial[chunk] = sm;
+    t.partial[t.nchunks + chunk] = sg;
   }
 }
 
-__global__ __launch_bounds__(kLansThreads) void lans_update_kernel(LansTables t, LansScalars sc) {
-  const ChunkView c = chunk_view(t, blockIdx.x);
+__global__ __launch_bounds__(kLansThreads) void lans_update_kernel(LansTables t, LansScalars sc, int chunk_base) {
+  const ChunkView c = chunk_view(t, chunk_base + blockIdx.x);
   const LansElem el = make_elem(sc, t.norms[c.tensor], t.consts[0], t.consts[1]);
   chunk_update(t, c, el, sc, t.norms[1 * t.T + c.tensor], t.norms[2 * t.T + c.tensor], t.norms[3 * t.T + c.tensor]);
+}
+
+// norms live in the plan's tensor order; callers get them in the order of their lists
+__global__ void lans_gather_norms_kernel(LansTables t, float* dst) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= t.T) return;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) dst[k * t.T + t.order[i]] = t.norms[k * t.T + i];
 }
 
 // =======================================================================================
@@ -570,7 +584,7 @@ __global__ __launch_bounds__(kLansThreads, kResidentWavesPerSimd) void lans_resi
     __syncthreads();
     // one value for the whole workgroup, and known to be: pointers and sizes derived from it stay scalar
     const int chunk = __builtin_amdgcn_readfirstlane(sh.chunk);
-    if (chunk >= t.nchunks) break;  // every workgroup reaches this: chunks are finite
+    if (chunk >= t.nres) break;  // every workgroup reaches this: chunks are finite
     const ChunkView c = chunk_view(t, chunk);
     const bool full = c.n == kLansChunk &&
                       vec_ok(t.g[c.tensor], t.p[c.tensor], t.m[c.tensor], t.v[c.tensor]);
@@ -601,6 +615,10 @@ struct lancet_lans_plan {
   int schedule;           // LANCET_LANS_SWEEPS or LANCET_LANS_RESIDENT
   int resident_grid;      // workgroups of the resident schedule the device runs at once
   int max_tensor_chunks;  // chunks of the largest tensor
+  int resident_limit;     // chunks of the largest tensor the resident schedule holds on this device
+  int n_res_tensors;      // tensors within that limit: the first ones in the plan's own order
+  int n_res_chunks;
+  std::vector<int32_t> order;  // plan position -> position in the caller's lists
   uint32_t epoch;         // step counter that tags the words of the resident schedule
   size_t words_offset; // part_word + norm_word inside dev_block
   size_t words_bytes;
@@ -623,14 +641,35 @@ static void chunk_tables(const int64_t* numels, int T, std::vector<int32_t>& cte
   first[T] = c;
 }
 
-// Host-only view of the chunk -> tensor map a plan builds for `numels` (no device needed).
-extern "C" int64_t lancet_lans_debug_chunk_table(const int64_t* numels, int T, int32_t* chunk_tensor_out,
-                                                 int64_t capacity) {
+// The plan's own tensor order: tensors of at most `limit` chunks first (the resident schedule takes
+// those), the larger ones after them (they go through the sweeps), list order kept inside each group.
+static int tensor_order(const int64_t* numels, int T, int limit, std::vector<int32_t>& order) {
+  order.clear();
+  for (int pass = 0; pass < 2; ++pass)
+    for (int i = 0; i < T; ++i) {
+      const bool fits = (numels[i] + kLansChunk - 1) / kLansChunk <= limit;
+      if (fits == (pass == 0)) order.push_back(i);
+    }
+  int n_fit = 0;
+  for (int i = 0; i < T; ++i) n_fit += (numels[i] + kLansChunk - 1) / kLansChunk <= limit;
+  return n_fit;
+}
+
+// Host-only view of what a plan builds for `numels` when the resident schedule holds tensors of up to
+// `resident_limit` chunks (no device needed): for every chunk, in ticket order, the position of its
+// tensor in the caller's list; *n_resident_chunks = chunks the resident kernel hands out.
+extern "C" int64_t lancet_lans_debug_chunk_table(const int64_t* numels, int T, int resident_limit,
+                                                 int32_t* chunk_tensor_out, int64_t capacity,
+                                                 int64_t* n_resident_chunks) {
   if (!numels || T <= 0) return -1;
-  std::vector<int32_t> ctensor, first;
-  chunk_tables(numels, T, ctensor, first);
+  std::vector<int32_t> order, ctensor, first;
+  const int n_fit = tensor_order(numels, T, resident_limit, order);
+  std::vector<int64_t> perm(T);
+  for (int i = 0; i < T; ++i) perm[i] = numels[order[i]];
+  chunk_tables(perm.data(), T, ctensor, first);
   for (int64_t i = 0; i < capacity && i < static_cast<int64_t>(ctensor.size()); ++i)
-    if (chunk_tensor_out) chunk_tensor_out[i] = ctensor[i];
+    if (chunk_tensor_out) chunk_tensor_out[i] = order[ctensor[i]];
+  if (n_resident_chunks) *n_resident_chunks = first[n_fit];
   return static_cast<int64_t>(ctensor.size());
 }
 
@@ -667,6 +706,7 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
   const size_t o_consts = off;    off = align_up(off + 2 * sizeof(float), 256);
   const size_t o_words = off;     off = align_up(off + 4 * ((n ? n : 1) + T) * sizeof(uint64_t), 256);
   const size_t o_ticket = off;    off = align_up(off + (2 + 2 * static_cast<size_t>(T)) * sizeof(uint32_t), 256);
+  const size_t o_order = off;     off = align_up(off + T * sizeof(int32_t), 256);
   pl->schedule = LANCET_LANS_SWEEPS;
   pl->epoch = 0;
   pl->words_offset = o_words;
@@ -682,18 +722,25 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
     err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lans_resident_kernel, kLansThreads, 0);
     pl->resident_grid = per_cu * cus;
   }
+  pl->resident_limit = std::min(pl->resident_grid, kMaxResidentChunks);
+  pl->n_res_tensors = tensor_order(numels, T, pl->resident_limit, pl->order);
   if (err == hipSuccess) err = hipMalloc(&pl->dev_block, off);
   if (err == hipSuccess) err = hipHostMalloc(reinterpret_cast<void**>(&pl->h_ptrs), 4 * T * sizeof(void*), hipHostMallocDefault);
   if (err == hipSuccess) err = hipEventCreateWithFlags(&pl->upload_done, hipEventDisableTiming);
   if (err == hipSuccess) {
     std::vector<int32_t> ctensor, first;
-    chunk_tables(numels, T, ctensor, first);
+    std::vector<int64_t> perm(T);
+    for (int i = 0; i < T; ++i) perm[i] = numels[pl->order[i]];
+    chunk_tables(perm.data(), T, ctensor, first);
+    pl->n_res_chunks = first[pl->n_res_tensors];
     char* base = static_cast<char*>(pl->dev_block);
-    err = hipMemcpy(base + o_numel, numels, T * sizeof(int64_t), hipMemcpyHostToDevice);
+    err = hipMemcpy(base + o_numel, perm.data(), T * sizeof(int64_t), hipMemcpyHostToDevice);
+    if (err == hipSuccess) err = hipMemcpy(base + o_order, pl->order.data(), T * sizeof(int32_t), hipMemcpyHostToDevice);
     if (err == hipSuccess && n) err = hipMemcpy(base + o_ctensor, ctensor.data(), n * sizeof(int32_t), hipMemcpyHostToDevice);
     if (err == hipSuccess) err = hipMemcpy(base + o_first, first.data(), (T + 1) * sizeof(int32_t), hipMemcpyHostToDevice);
     if (err == hipSuccess) err = hipMemset(base + o_norms, 0, 4 * T * sizeof(float));
     if (err == hipSuccess) err = hipMemset(base + o_words, 0, pl->words_bytes);
+    if (err == hipSuccess) err = hipMemset(base + o_ticket, 0, (2 + 2 * static_cast<size_t>(T)) * sizeof(uint32_t));
     LansTables& t = pl->tables;
     t.part_word = reinterpret_cast<uint64_t*>(base + o_words);
     t.norm_word = t.part_word + 4 * (n ? n : 1);
@@ -709,8 +756,10 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
     t.partial = reinterpret_cast<float*>(base + o_partial);
     t.norms = reinterpret_cast<float*>(base + o_norms);
     t.consts = reinterpret_cast<float*>(base + o_consts);
+    t.order = reinterpret_cast<const int32_t*>(base + o_order);
     t.T = T;
     t.nchunks = pl->nchunks;
+    t.nres = pl->n_res_chunks;
   }
   if (err != hipSuccess) {
     lancet_lans_plan_destroy(pl);
@@ -736,8 +785,8 @@ extern "C" int lancet_lans_plan_destroy(lancet_lans_plan_t pl) {
 extern "C" int lancet_lans_plan_norms(lancet_lans_plan_t pl, float* norms, lancet_stream_t stream) {
   if (!pl || pl->magic != kPlanMagic) return LANCET_ERR_PLAN;
   if (!norms) return LANCET_ERR_NULL;
-  return static_cast<int>(hipMemcpyAsync(norms, pl->tables.norms, 4 * static_cast<size_t>(pl->T) * sizeof(float),
-                                         hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream)));
+  lans_gather_norms_kernel<<<(pl->T + 255) / 256, 256, 0, static_cast<hipStream_t>(stream)>>>(pl->tables, norms);
+  return static_cast<int>(hipGetLastError());
 }
 
 extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, float* const* p,
@@ -767,10 +816,15 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
       if (err != hipSuccess) return static_cast<int>(err);
     }
     for (int i = 0; i < T; ++i) {
-      pl->shadow[i] = pl->h_ptrs[i] = const_cast<float*>(g[i]);
-      pl->shadow[T + i] = pl->h_ptrs[T + i] = p[i];
-      pl->shadow[2 * T + i] = pl->h_ptrs[2 * T + i] = m[i];
-      pl->shadow[3 * T + i] = pl->h_ptrs[3 * T + i] = v[i];
+      pl->shadow[i] = const_cast<float*>(g[i]);
+      pl->shadow[T + i] = p[i];
+      pl->shadow[2 * T + i] = m[i];
+      pl->shadow[3 * T + i] = v[i];
+      const int u = pl->order[i];  // the plan's i-th tensor is the caller's u-th
+      pl->h_ptrs[i] = const_cast<float*>(g[u]);
+      pl->h_ptrs[T + i] = p[u];
+      pl->h_ptrs[2 * T + i] = m[u];
+      pl->h_ptrs[3 * T + i] = v[u];
     }
     err = hipMemcpyAsync(pl->dev_block, pl->h_ptrs,
                          4 * static_cast<size_t>(T) * sizeof(void*), hipMemcpyHostToDevice, st);
@@ -793,8 +847,12 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
   sc.step_dev = step_dev;
   const LansTables& t = pl->tables;
   sc.spin_limit = current_spin_limit();
-  if (pl->schedule == LANCET_LANS_RESIDENT) {
-    if (++pl->epoch == 0) {
+  // chunks [0, chunk_base) and tensors [0, tensor_base) go through the resident kernel, the rest
+  // (everything, under the sweeps schedule) through the three sweeps
+  int chunk_base = 0, tensor_base = 0;
+  sc.epoch = 0;
+  if (pl->schedule == LANCET_LANS_RESIDENT && pl->n_res_chunks > 0) {
+    if (++pl->epoch == 0) {  // tag wrapped: forget every word of earlier steps
       err = hipMemsetAsync(static_cast<char*>(pl->dev_block) + pl->words_offset, 0, pl->words_bytes, st);
       if (err != hipSuccess) return static_cast<int>(err);
       pl->epoch = 1;
@@ -802,34 +860,38 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
     sc.epoch = pl->epoch;
     err = run_fill_u32(t.ticket, 2 + 2 * static_cast<size_t>(T), 0u, st);
     if (err != hipSuccess) return static_cast<int>(err);
-    const int grid = std::min(pl->resident_grid, t.nchunks);
+    const int grid = std::min(pl->resident_grid, pl->n_res_chunks);
     lans_resident_kernel<<<grid, kLansThreads, 0, st>>>(t, sc);
-    return static_cast<int>(hipGetLastError());
+    chunk_base = pl->n_res_chunks;
+    tensor_base = pl->n_res_tensors;
   }
-  sc.epoch = 0;
-  const int rblocks = (T + kLansThreads / kWave - 1) / (kLansThreads / kWave);
-  lans_prepare_kernel<<<1, 64, 0, st>>>(t, sc);
-  lans_norm_gp_kernel<<<t.nchunks, kLansThreads, 0, st>>>(t);
-  lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 0);
-  lans_moments_kernel<<<t.nchunks, kLansThreads, 0, st>>>(t, sc);
-  lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 2);
-  lans_update_kernel<<<t.nchunks, kLansThreads, 0, st>>>(t, sc);
+  const int nsweep = t.nchunks - chunk_base;
+  if (nsweep > 0) {
+    const int per_block = kLansThreads / kWave;
+    const int rblocks = (T - tensor_base + per_block - 1) / per_block;
+    lans_prepare_kernel<<<1, 64, 0, st>>>(t, sc);
+    lans_norm_gp_kernel<<<nsweep, kLansThreads, 0, st>>>(t, chunk_base);
+    lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 0, tensor_base);
+    lans_moments_kernel<<<nsweep, kLansThreads, 0, st>>>(t, sc, chunk_base);
+    lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 2, tensor_base);
+    lans_update_kernel<<<nsweep, kLansThreads, 0, st>>>(t, sc, chunk_base);
+  }
   return static_cast<int>(hipGetLastError());
 }
 
 extern "C" int lancet_lans_plan_set_schedule(lancet_lans_plan_t pl, int schedule) {
   if (!pl || pl->magic != kPlanMagic) return LANCET_ERR_PLAN;
   if (schedule != LANCET_LANS_SWEEPS && schedule != LANCET_LANS_RESIDENT) return LANCET_ERR_SHAPE;
-  // a tensor's chunks must all be held by running workgroups at once
-  if (schedule == LANCET_LANS_RESIDENT && pl->max_tensor_chunks > std::min(pl->resident_grid, kMaxResidentChunks))
-    return LANCET_ERR_SHAPE;
+  // a tensor's chunks must all be held by running workgroups at once; tensors too large for that go
+  // through the sweeps inside the same step, and a plan made only of such tensors has no use for the kernel
+  if (schedule == LANCET_LANS_RESIDENT && pl->n_res_chunks == 0 && pl->nchunks > 0) return LANCET_ERR_SHAPE;
   pl->schedule = schedule;
   return LANCET_OK;
 }
 
 extern "C" int lancet_lans_plan_resident_capacity(lancet_lans_plan_t pl, int* workgroups, int* max_tensor_chunks) {
   if (!pl || pl->magic != kPlanMagic) return LANCET_ERR_PLAN;
-  if (workgroups) *workgroups = std::min(pl->resident_grid, kMaxResidentChunks);
+  if (workgroups) *workgroups = pl->resident_limit;
   if (max_tensor_chunks) *max_tensor_chunks = pl->max_tensor_chunks;
   return LANCET_OK;
 }

@@ -182,13 +182,16 @@ def test_op_layer_errors_are_reported_not_fatal(pkg):
 
 
 # ----------------------------------------------------------------------------- LANS task queue
-def _chunk_table(pkg, numels):
+def _chunk_table(pkg, numels, limit=1 << 30):
+    """(tensor of every chunk in ticket order, chunks the resident kernel hands out)."""
     lib = pkg.capi.load()
     arr = (C.c_int64 * len(numels))(*numels)
-    n = lib.lancet_lans_debug_chunk_table(arr, len(numels), None, 0)
+    n = lib.lancet_lans_debug_chunk_table(arr, len(numels), limit, None, 0, None)
     ctensor = np.empty(max(n, 1), np.int32)
-    assert lib.lancet_lans_debug_chunk_table(arr, len(numels), ctensor.ctypes.data_as(C.c_void_p), n) == n
-    return ctensor[:n]
+    nres = C.c_int64(-1)
+    assert lib.lancet_lans_debug_chunk_table(arr, len(numels), limit, ctensor.ctypes.data_as(C.c_void_p), n,
+                                             C.byref(nres)) == n
+    return ctensor[:n], nres.value
 
 
 def _simulate_resident(ctensor, workers, rng):
@@ -241,11 +244,27 @@ def test_lans_resident_schedule_drains(pkg, case):
         numels = [int(x) for x in rng.integers(0, 600_000, 60)] + [0, 1, 8192, 8193]
     else:
         numels = [1, 2, 3]
-    ctensor = _chunk_table(pkg, numels)
-    assert len(ctensor) == sum((n + 8191) // 8192 for n in numels)
+    ctensor, nres = _chunk_table(pkg, numels)
+    assert len(ctensor) == nres == sum((n + 8191) // 8192 for n in numels)
     assert (np.diff(ctensor) >= 0).all()                       # chunks of a tensor are consecutive tickets
     largest = int(np.bincount(ctensor).max())
     for workers in (largest, largest + 3, 4 * largest):
         assert _simulate_resident(ctensor, workers, rng)
     if largest > 1:
         assert not _simulate_resident(ctensor, largest - 1, rng)
+
+
+def test_lans_plan_orders_tensors_that_do_not_fit_last(pkg):
+    """Tensors with more chunks than the resident kernel holds come after all the others in the plan's
+    ticket order and are left to the sweeps; every chunk of every tensor appears exactly once."""
+    numels = [100, 5 * 8192, 8192 * 40 + 1, 3, 8192 * 41, 8192 * 40, 0, 7 * 8192]
+    limit = 40
+    ctensor, nres = _chunk_table(pkg, numels, limit)
+    chunks = [(n + 8191) // 8192 for n in numels]
+    assert len(ctensor) == sum(chunks)
+    np.testing.assert_array_equal(np.bincount(ctensor, minlength=len(numels)), chunks)
+    fits = [i for i, c in enumerate(chunks) if c <= limit]
+    assert nres == sum(chunks[i] for i in fits)
+    assert set(ctensor[:nres]) == {i for i in fits if chunks[i] > 0}
+    assert list(dict.fromkeys(ctensor[nres:])) == [2, 4]        # list order is kept inside each group
+    assert _simulate_resident(ctensor[:nres], limit, np.random.default_rng(1))

@@ -180,14 +180,41 @@ def test_lans_resident_schedule_against_oracle(pkg):
     plan.close()
 
 
-def test_lans_resident_schedule_rejects_a_tensor_that_does_not_fit(pkg):
+def test_lans_resident_schedule_with_tensors_that_do_not_fit(pkg):
+    """Tensors with more chunks than the chip holds at once go through the sweeps inside the same step; the
+    caller sees one step, norms in the order of its lists, and the same values as the pure sweeps schedule."""
     capi = pkg.capi
-    plan = pkg.ops.LansPlan([1024, 1024])
-    workgroups, largest = plan.resident_capacity()
-    plan.close()
-    assert largest == 1 and workgroups >= 256
-    big = pkg.ops.LansPlan([(workgroups + 1) * 8192])       # no memory is touched by creating a plan
-    assert big.resident_capacity()[1] == workgroups + 1
+    probe = pkg.ops.LansPlan([1024, 1024])
+    limit, largest = probe.resident_capacity()
+    probe.close()
+    assert largest == 1 and limit >= 256
+    big = (limit + 1) * 8192
+    numels = [1024, big, 70000, big + 3 * 8192 + 5, 8192]
+    results = []
+    for schedule in (capi.LANS_SWEEPS, capi.LANS_RESIDENT):
+        gen = torch.Generator(device="cuda").manual_seed(11)
+        total = sum(numels)
+        flat = [torch.empty(total, device="cuda").normal_(0, s, generator=gen) for s in (1e-3, 0.02)]
+        flat += [torch.zeros(total, device="cuda") for _ in range(2)]
+        views = [list(torch.split(t, numels)) for t in flat]
+        plan = pkg.ops.LansPlan(numels, schedule=schedule)
+        assert plan.resident_capacity() == (limit, limit + 5)
+        hyper = capi.LansHyper(1e-3, 0.9, 0.999, 1e-6, 1, 0.01, 1, 1, 1)
+        for step in (1, 2):
+            plan.step(*views, step, hyper)
+        torch.cuda.synchronize()
+        assert plan.error() == 0
+        results.append((flat, plan.norms()))
+        plan.close()
+    for name, a, b in zip("gpmv", results[0][0], results[1][0]):
+        assert (a - b).abs().max().item() <= 2e-6 * a.abs().max().item(), name
+    torch.testing.assert_close(results[0][1], results[1][1], rtol=2e-6, atol=0)
+    # the two large tensors took the same kernels under both schedules: the same bits
+    off = np.cumsum([0] + numels)
+    for i in (1, 3):
+        assert torch.equal(results[0][0][1][off[i]:off[i + 1]], results[1][0][1][off[i]:off[i + 1]])
+    # a plan made only of tensors that do not fit has no use for the resident kernel
+    only_big = pkg.ops.LansPlan([big])                       # no memory is touched by creating a plan
     with pytest.raises(RuntimeError):
-        big.set_schedule(capi.LANS_RESIDENT)
-    big.close()
+        only_big.set_schedule(capi.LANS_RESIDENT)
+    only_big.close()

@@ -14,10 +14,12 @@
 //     exchange chunk partials as self-validating 64-bit words (step epoch in the high half, fp32 sum
 //     in the low half, one agent-scope atomic store each); the workgroup that arrives last at a
 //     per-tensor counter sums them in a fixed order and publishes the norm the same way.  Nothing
-//     else crosses workgroups, so no fences are needed.  Chunks are handed out in list order by a
+//     else crosses workgroups, so no fences are needed.  Chunks are handed out in order by a
 //     ticket; a workgroup only ever waits for chunks of its own tensor, so the kernel drains as long
-//     as the chunks of one tensor all fit on the chip at once, which set_schedule checks (the limit
-//     is the register file: about 4M parameters per tensor on 256 CUs).  Waits are bounded.
+//     as the chunks of one tensor all fit on the chip at once (the limit is the register file: about
+//     4M parameters per tensor on 256 CUs).  The plan orders its tensors so that those within the
+//     limit come first; the kernel takes them, and larger tensors go through the sweeps in the same
+//     step.  Waits are bounded.
 // Work is cut into fixed-size chunks described by device-resident tables built once per
 // parameter set, instead of kernel arguments re-packed for every launch
 // (multi_tensor_apply.cuh:39-92).  Chunk partials are combined in a fixed order in double

@@ -264,6 +264,66 @@ def bench_pipeline(pkg, data, logits, S, M, E, cf, iters):
                     "pays when the exchange is a real all-to-all over xGMI"}
 
 
+def bench_other_configs(ops, iters):
+    """BASELINE configs 1-3 (parity-test cases) timed for reference: encode + decode per pass; config 1 also
+    replayed from a captured graph, which removes the launch gaps that dominate at that size."""
+    import numpy as np
+    import torch
+    out = {}
+
+    def run(name, S, M, E, cf, k, dtype, bpr=False, zipf=False, scale=1.0, graph=False):
+        rng = np.random.default_rng(0)
+        data = torch.from_numpy(rng.standard_normal((S, M), dtype=np.float32)).cuda().to(dtype)
+        logits = rng.standard_normal((S, E), dtype=np.float32) * np.float32(scale)
+        if zipf:
+            r = np.arange(1, E + 1, dtype=np.float64)
+            bias = 3.0 * (r ** -1.2 - E ** -1.2) / (1.0 - E ** -1.2)
+            logits = logits + bias[rng.permutation(E)].astype(np.float32)[None, :]
+        gate = torch.from_numpy(logits.astype(np.float32)).cuda()
+        if bpr:
+            gate = torch.softmax(gate, dim=1)
+        Cap = ops.moe_capacity(S, E, cf * k)
+        bufs = (torch.empty(k * S, device="cuda"), torch.empty((2, k * S), dtype=torch.int32, device="cuda"),
+                torch.empty(E, dtype=torch.int32, device="cuda"), torch.empty(E, dtype=torch.int64, device="cuda"),
+                torch.empty((E, Cap, M), dtype=dtype, device="cuda"))
+        ws = torch.empty(max(ops.moe_encode_workspace_bytes(S, E, k), ops.moe_encode_bpr_workspace_bytes(S, E, 1)),
+                         dtype=torch.uint8, device="cuda")
+        dec = torch.empty((S, M), dtype=dtype, device="cuda")
+
+        def step():
+            if bpr:
+                ops.moe_encode_batch_prioritized(data, gate, 1, 0, cf, workspace=ws, out=bufs)
+            else:
+                ops.moe_encode(data, gate, None, cf, top_k=k, gate_is_logits=True, workspace=ws, out=bufs)
+            ops.moe_decode(bufs[4], bufs[0], bufs[1], top_k=k, out=dec)
+
+        step()
+        ms = event_ms(step, iters)
+        kept = int((bufs[1][0] >= 0).sum())
+        b = data.element_size()
+        alg = (S * E * 4 + S * M * b + E * Cap * M * b + k * S * 12 + E * 12) + (kept * M * b + S * M * b + k * S * 12)
+        rec = {"ms": round(ms, 4), "tokens_per_s": round(S / (ms * 1e-3), 1), "kept_slots": kept, "slots": k * S,
+               "algorithmic_bytes": alg, "frac_of_hbm_peak": round(alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+        if graph:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                step()
+            torch.cuda.current_stream().wait_stream(side)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                step()
+            g.replay()
+            rec["ms_graph_replay"] = round(event_ms(g.replay, iters), 4)
+        out[name] = rec
+
+    run("config1_top1_fp32", 4096, 768, 8, 1.25, 1, torch.float32, graph=True)
+    run("config2_top2_fp32", 16384, 1024, 16, 1.0, 2, torch.float32, zipf=True)
+    run("config2_top2_bf16", 16384, 1024, 16, 1.0, 2, torch.bfloat16, zipf=True)
+    run("config3_bpr_bf16", 32768, 2048, 64, 1.25, 1, torch.bfloat16, bpr=True, scale=2.0)
+    return out
+
+
 def bench_backward(ops, data, outs, dec, S, M, E, Cap, K, kept, iters):
     """The four backward ops at the headline shape (dy buffers reuse forward tensors as values)."""
     import torch
@@ -453,6 +513,7 @@ def main():
     torch.cuda.empty_cache()
     result["config4_partitioned"] = bench_config4_partitioned(ops, lib, capi, data, logits, S, M, E, cf, max(5, n // 2))
     result["pipeline"] = bench_pipeline(pkg, data, logits, S, M, E, cf, max(5, n // 2))
+    result["other_configs"] = bench_other_configs(ops, max(10, n))
     del data
     torch.cuda.empty_cache()
     if not args.no_lans:

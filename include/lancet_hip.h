@@ -246,7 +246,10 @@ int lancet_moe_redispatch(const void* const* data, const int32_t* const* indices
  * g/p/m/v are HOST arrays of T device pointers to fp32 tensors (the four quarters of the
  * reference's tensor_list).  p, m, v are updated in place; g is not modified.
  * step: pass step_host >= 1, or a device pointer step_dev to the fp32 step scalar the
- * reference passes (read on the device; no host synchronisation). */
+ * reference passes (read on the device; no host synchronisation).
+ * A plan's steps share its partial sums and control words: issue them on one stream, or order
+ * them yourself; two steps of one plan that overlap on the device race.  Plans are independent
+ * of each other. */
 typedef struct lancet_lans_plan* lancet_lans_plan_t;
 
 typedef struct lancet_lans_hyper {

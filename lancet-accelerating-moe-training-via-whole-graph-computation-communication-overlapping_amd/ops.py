@@ -108,6 +108,46 @@ def moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_
     return gates_s, indloc, used_out, elems.view(torch.uint64) if elems.dtype == torch.int64 else elems, disp
 
 
+def moe_route(gate, used_capacity, M, capacity_factor=1.0, top_k=1, gate_is_logits=False, workspace=None, out=None):
+    """The routing half of moe_encode (selection + position scan, src/op/dialect/cuda/moe.cc:366-380), so that
+    a caller can run it ahead of, or beside, the row movement of another partition.  M only scales
+    elements_per_expert.  Returns (gates_s, indices_locations, used_capacity, elements_per_expert)."""
+    lib = capi.load()
+    _dev(gate, "gate")
+    _need(gate.dim() == 2 and gate.dtype == torch.float32, "gate must be 2-D float32")
+    S, E = gate.shape
+    _need(top_k in (1, 2), "top_k must be 1 or 2")
+    Cap = moe_capacity(S, E, float(capacity_factor) * (2.0 if top_k == 2 else 1.0))
+    dev = gate.device
+    if out is None:
+        out = (torch.empty(top_k * S, dtype=torch.float32, device=dev),
+               torch.empty((2, top_k * S), dtype=torch.int32, device=dev),
+               torch.empty(E, dtype=torch.int32, device=dev), torch.empty(E, dtype=torch.int64, device=dev))
+    gates_s, indloc, used_out, elems = out[:4]
+    ws = _workspace(moe_encode_workspace_bytes(S, E, top_k), dev, workspace)
+    st = lib.lancet_moe_route(_p(gate), _p(used_capacity), S, int(M), E, Cap, top_k, _flags(gate_is_logits, True),
+                              _p(gates_s), _p(indloc), _p(used_out), _p(elems), _p(ws), ws.numel(), _stream())
+    capi.check(st, "lancet_moe_route")
+    return gates_s, indloc, used_out, elems
+
+
+def moe_scatter(data, indices_locations, used_in, used_out, n_experts, capacity, top_k=1, zero_tail=True, out=None):
+    """The row-movement half of moe_encode (launch_encode_forward, moe.cc:381-395) on routing produced by
+    moe_route: returns dispatched [E, C, M]."""
+    lib = capi.load()
+    _dev(data, "data")
+    _need(data.dim() == 2, "Expected input data to be 2D.")
+    S = _check_indloc(indices_locations, top_k)
+    _need(S == data.shape[0], "indices_locations and data disagree on the token count")
+    M = data.shape[1]
+    if out is None:
+        out = torch.empty((n_experts, capacity, M), dtype=data.dtype, device=data.device)
+    st = lib.lancet_moe_scatter(_p(data), _p(indices_locations), _p(used_in), _p(used_out), S, M, int(n_experts),
+                                int(capacity), top_k, _dtype_code(data), _flags(False, zero_tail), _p(out), _stream())
+    capi.check(st, "lancet_moe_scatter")
+    return out
+
+
 def moe_encode_bpr_workspace_bytes(S0, E, n_partitions=1):
     return int(capi.load().lancet_moe_encode_bpr_workspace_bytes(int(S0), int(E), int(n_partitions)))
 

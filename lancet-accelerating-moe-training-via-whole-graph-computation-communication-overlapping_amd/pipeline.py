@@ -1,9 +1,11 @@
-"""A partitioned MoE dispatch pipeline over two HIP streams: the call pattern Lancet's partition pass
+"""A partitioned MoE dispatch pipeline over three HIP streams (routing, row movement, exchange): the call pattern Lancet's partition pass
 emits for one MoE layer (src/pass/dist_optimization/partition_exprs.cc:1709-1795), on one GPU.
 
 The token batch is cut into P partitions.  Partition i is encoded with the used capacity of partition
 i-1 chained in and capacity_factor x P (`:1750-1762`), scheduled at pipeline index i (`:1775`); its
-exchange then overlaps the encode of partition i+1.  With one GPU there is no all-to-all, so the
+exchange then overlaps the encode of partition i+1.  The chain only links the routing halves of the
+encodes (selection + position scan: small, latency-bound kernels), so those run ahead on a stream of
+their own while the row movement of earlier partitions streams.  With one GPU there is no all-to-all, so the
 exchange stage does what the all-to-allv does to the buffer on either side of the wire: the rows each
 expert uses are packed back to back, keyed by elements_per_expert (the send counts,
 src/op/dialect/nccl/nccl.cc:373-421), and unpacked into a zero-filled [E, C, M] receive buffer.  The
@@ -41,8 +43,10 @@ class PartitionedMoeLayer:
         self.recv = [torch.empty((E, C, M), dtype=dtype, device=dev) for _ in range(P)]
         self.out = torch.empty((S, M), dtype=dtype, device=dev)
         self.zero_used = torch.zeros(E, dtype=torch.int32, device=dev)
+        self.routing = torch.cuda.Stream(device=dev)
         self.compute = torch.cuda.Stream(device=dev)
         self.exchange = torch.cuda.Stream(device=dev)
+        self.routed = [torch.cuda.Event() for _ in range(P)]
         self.encoded = [torch.cuda.Event() for _ in range(P)]
         self.received = [torch.cuda.Event() for _ in range(P)]
 
@@ -53,6 +57,18 @@ class PartitionedMoeLayer:
         # the send buffer only feeds the packing copy, which reads the used rows: no tail zero-fill
         ops.moe_encode(data[sl], gate[sl], used, self.cf, gate_is_logits=self.gate_is_logits, zero_tail=False,
                        workspace=self.ws[i], out=self.enc[i])
+
+    def _route(self, i, gate):
+        sl = slice(i * self.Sp, (i + 1) * self.Sp)
+        used = self.zero_used if i == 0 else self.enc[i - 1][2]
+        ops.moe_route(gate[sl], used, self.M, self.cf, gate_is_logits=self.gate_is_logits, workspace=self.ws[i],
+                      out=self.enc[i])
+
+    def _scatter(self, i, data):
+        sl = slice(i * self.Sp, (i + 1) * self.Sp)
+        used = self.zero_used if i == 0 else self.enc[i - 1][2]
+        ops.moe_scatter(data[sl], self.enc[i][1], used, self.enc[i][2], self.E, self.C, zero_tail=False,
+                        out=self.enc[i][4])
 
     def _exchange(self, i):
         _, _, _, elems, disp = self.enc[i]
@@ -73,17 +89,23 @@ class PartitionedMoeLayer:
         return self.out
 
     def run(self, data, gate):
-        """Encodes and decodes on one stream, exchanges on another: the exchange of partition i runs beside
-        the encode of partition i+1, the decode of partition i after its exchange.  Returns the output;
-        the caller's current stream waits for the pipeline before it may use it."""
+        """Routing of all partitions on one stream, row movement (scatter, decode) on a second, exchanges on
+        a third: the exchange of partition i runs beside the scatter of partition i+1, the decode of
+        partition i after its exchange.  Returns the output; the caller's current stream waits for the
+        pipeline before it may use it."""
         cur = torch.cuda.current_stream()
         start = torch.cuda.Event()
         start.record(cur)
-        self.compute.wait_event(start)
-        self.exchange.wait_event(start)
+        for s in (self.routing, self.compute, self.exchange):
+            s.wait_event(start)
+        with torch.cuda.stream(self.routing):
+            for i in range(self.P):
+                self._route(i, gate)
+                self.routed[i].record(self.routing)
         for i in range(self.P):
             with torch.cuda.stream(self.compute):
-                self._encode(i, data, gate)
+                self.compute.wait_event(self.routed[i])
+                self._scatter(i, data)
                 self.encoded[i].record(self.compute)
                 if i > 0:
                     self.compute.wait_event(self.received[i - 1])

@@ -452,3 +452,23 @@ def test_sparse_packed_copies_scale_and_encode_counts(pkg):
     got_h = ops.memcpy_sparse_to_cont_3d(rows_to_torch(disp16, "bf16"), rows_to_torch(np.zeros(kept * M, disp16.dtype), "bf16"),
                                          elems, shrink_element_size_by=2)
     np.testing.assert_array_equal(to_np(got_h), want_h)
+
+
+# ----------------------------------------------------------------------------- route / scatter halves
+@pytest.mark.parametrize("k,dt", [(1, "f32"), (2, "bf16"), (1, "f16")])
+def test_route_then_scatter_equals_encode(pkg, k, dt):
+    """lancet_moe_route + lancet_moe_scatter (the two halves of MoeEncode::Execute, moe.cc:366-380 and
+    :381-395) give what moe_encode gives, with used capacity carried in."""
+    ops = pkg.ops
+    S, M, E, cf = 1500, 48, 12, 0.75
+    data, logits = make_inputs(5 + k, S, M, E, zipf_bias=True)
+    Cap = ops.moe_capacity(S, E, cf * k)
+    used0 = np.zeros(E, np.int32) if k == 2 else np.random.default_rng(1).integers(0, Cap // 2, E).astype(np.int32)
+    d_data, d_gate, d_used = rows_to_torch(data, dt), dev(logits), dev(used0)
+    whole = ops.moe_encode(d_data, d_gate, d_used, cf, top_k=k, gate_is_logits=True)
+    gates_s, indloc, used_out, elems = ops.moe_route(d_gate, d_used, M, cf, top_k=k, gate_is_logits=True)
+    disp = ops.moe_scatter(d_data, indloc, d_used, used_out, E, Cap, top_k=k)
+    for a, b in zip(whole, (gates_s, indloc, used_out, elems, disp)):
+        assert torch.equal(a.view(torch.int64) if a.dtype == torch.uint64 else a,
+                           b.view(torch.int64) if b.dtype in (torch.uint64,) else b)
+    assert (to_np(indloc)[0] < 0).any()

@@ -218,3 +218,43 @@ def test_lans_resident_schedule_with_tensors_that_do_not_fit(pkg):
     with pytest.raises(RuntimeError):
         only_big.set_schedule(capi.LANS_RESIDENT)
     only_big.close()
+
+
+def test_lans_resident_schedule_beside_other_work(pkg):
+    """The resident kernel's workgroups wait for one another, so they must all get onto the chip: with
+    another stream keeping compute units busy they get there as that work retires, the waits stay within
+    their bound (error word 0) and the result is the one an idle GPU gives."""
+    capi = pkg.capi
+    numels = [4 << 20, 1 << 20, 4 << 20, 1024, 3 << 20]
+    hyper = capi.LansHyper(1e-3, 0.9, 0.999, 1e-6, 1, 0.01, 1, 1, 1)
+
+    def state():
+        gen = torch.Generator(device="cuda").manual_seed(3)
+        total = sum(numels)
+        flat = [torch.empty(total, device="cuda").normal_(0, s, generator=gen) for s in (1e-3, 0.02)]
+        flat += [torch.zeros(total, device="cuda") for _ in range(2)]
+        return flat, [list(torch.split(t, numels)) for t in flat]
+
+    flat_a, views_a = state()
+    plan = pkg.ops.LansPlan(numels, schedule=capi.LANS_RESIDENT)
+    for step in (1, 2, 3):
+        plan.step(*views_a, step, hyper)
+    torch.cuda.synchronize()
+    assert plan.error() == 0
+
+    flat_b, views_b = state()
+    side = torch.cuda.Stream()
+    x = torch.randn(64 << 20, device="cuda")
+    y = torch.empty_like(x)
+    torch.cuda.synchronize()
+    for step in (1, 2, 3):
+        with torch.cuda.stream(side):
+            for _ in range(6):                      # streaming work that occupies every compute unit
+                torch.mul(x, 1.0001, out=y)
+                torch.add(y, 1.0, out=x)
+        plan.step(*views_b, step, hyper)
+    torch.cuda.synchronize()
+    assert plan.error() == 0
+    for a, b in zip(flat_a, flat_b):
+        assert torch.equal(a, b)
+    plan.close()

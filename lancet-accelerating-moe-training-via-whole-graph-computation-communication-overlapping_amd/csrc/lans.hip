@@ -8,18 +8,19 @@
 //   * sweeps (default): three plain launches + two tiny per-tensor reductions.  Real HBM traffic
 //     is 52 B/param (g, p read three times, m, v twice) and each sweep streams at the rate a plain
 //     copy reaches on this chip.
-//   * resident (opt-in): ONE persistent kernel in which a workgroup takes a chunk through all three
-//     phases and keeps it on chip in between (g, then u_m and u_g, in registers; p in LDS), so every
-//     array is read once and written once: 28 B/param.  Between phases the workgroups of a tensor
-//     exchange chunk partials as self-validating 64-bit words (step epoch in the high half, fp32 sum
-//     in the low half, one agent-scope atomic store each); the workgroup that arrives last at a
-//     per-tensor counter sums them in a fixed order and publishes the norm the same way.  Nothing
-//     else crosses workgroups, so no fences are needed.  Chunks are handed out in order by a
-//     ticket; a workgroup only ever waits for chunks of its own tensor, so the kernel drains as long
-//     as the chunks of one tensor all fit on the chip at once (the limit is the register file: about
-//     4M parameters per tensor on 256 CUs).  The plan orders its tensors so that those within the
-//     limit come first; the kernel takes them, and larger tensors go through the sweeps in the same
-//     step.  Waits are bounded.
+//   * resident (opt-in): a sweep over g alone for ||g|| (4 B/param), then ONE persistent kernel in
+//     which a workgroup takes a chunk through phases 2 and 3 and keeps it on chip in between (u_m and
+//     u_g in registers, p in LDS), so every array is read once and written once: 32 B/param with the
+//     sweep.  Before phase 3 the workgroups of a tensor exchange three chunk partials (p^2, u_m^2,
+//     u_g^2) as self-validating 64-bit words (step epoch in the high half, fp32 sum in the low half,
+//     one agent-scope atomic store each); the workgroup that arrives last at a per-tensor counter
+//     sums them in a fixed order and publishes the norms the same way.  Nothing else crosses
+//     workgroups, so no fences are needed.  Chunks are handed out in order by a ticket; a workgroup
+//     only ever waits for chunks of its own tensor, so the kernel drains as long as the chunks of one
+//     tensor all fit on the chip at once (the limit is the register file: about 4M parameters per
+//     tensor on 256 CUs).  The plan orders its tensors so that those within the limit come first;
+//     the kernel takes them, and larger tensors go through the sweeps in the same step.  Waits are
+//     bounded.
 // Work is cut into fixed-size chunks described by device-resident tables built once per
 // parameter set, instead of kernel arguments re-packed for every launch
 // (multi_tensor_apply.cuh:39-92).  Chunk partials are combined in a fixed order in double
@@ -49,7 +50,7 @@ struct LansTables {
   float* partial;              // [2][nchunks]      (sweeps schedule)
   uint64_t* part_word;         // [4][nchunks]      (resident schedule: epoch | fp32 sum of squares)
   uint64_t* norm_word;         // [4][T]            (resident schedule: epoch | fp32 norm)
-  uint32_t* ticket;            // [1] next task; [1] error flag; [2][T] arrivals (resident schedule)
+  uint32_t* ticket;            // [1] next task; [1] error flag; [T] arrivals (resident schedule)
   float* norms;                // [4][T]: g, p, u_m, u_g
   float* consts;               // [2]: bias_correction1, bias_correction2
   const int32_t* order;        // [T] position in the caller's lists of the plan's i-th tensor
@@ -321,13 +322,35 @@ __global__ __launch_bounds__(kLansThreads) void lans_norm_gp_kernel(LansTables t
   }
 }
 
+// Sum g^2 alone, chunks [0, nchunks_g): ahead of the resident kernel in its one-wait form
+__global__ __launch_bounds__(kLansThreads) void lans_norm_g_kernel(LansTables t) {
+  __shared__ float s_red[kLansThreads / kWave];
+  const ChunkView c = chunk_view(t, blockIdx.x);
+  const LANCET_GLOBAL float* g = as_global(t.g[c.tensor] + c.begin);
+  float ag = 0.f;
+  int scalar_from = 0;
+  if (vec_ok(g, g, g, g)) {
+    const int nv = c.n / 4;
+    const LANCET_GLOBAL f32x4* g4 = (const LANCET_GLOBAL f32x4*)g;
+#pragma unroll 8
+    for (int i = threadIdx.x; i < nv; i += kLansThreads) {
+      const f32x4 x = g4[i];
+      ag += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+    }
+    scalar_from = nv * 4;
+  }
+  for (int i = scalar_from + threadIdx.x; i < c.n; i += kLansThreads) ag += g[i] * g[i];
+  ag = block_sum(ag, s_red);
+  if (threadIdx.x == 0) t.partial[blockIdx.x] = ag;
+}
+
 // per-tensor sqrt(sum of chunk partials) (cleanup, multi_tensor_lans.cu:169-185)
-__global__ __launch_bounds__(kLansThreads) void lans_reduce_kernel(LansTables t, int first_norm, int tensor_base) {
+__global__ __launch_bounds__(kLansThreads) void lans_reduce_kernel(LansTables t, int first_norm, int tensor_base,
+                                                                   int tensor_end, int count) {
   const int tensor = tensor_base + blockIdx.x * (kLansThreads / kWave) + threadIdx.x / kWave;
-  if (tensor >= t.T) return;
+  if (tensor >= tensor_end) return;
   const int lo = t.tensor_first[tensor], hi = t.tensor_first[tensor + 1];
-#pragma unroll
-  for (int k = 0; k < 2; ++k) {
+  for (int k = 0; k < count; ++k) {
     const float* part = t.partial + static_cast<size_t>(k) * t.nchunks;
     const float n = wave_norm(lo, hi, [&](int c) { return part[c]; });
     if (lane_id() == 0) t.norms[(first_norm + k) * t.T + tensor] = n;
@@ -385,7 +408,7 @@ constexpr int kMaxResidentChunks = 512;  // chunks of one tensor the resident sc
 
 struct ResidentShared {
   f32x4 p[kVecPerThread][kLansThreads];  // the chunk's parameters, one private slot per thread and float4
-  float part[2][kMaxResidentChunks];     // gathered chunk partials of the tensor
+  float part[3][kMaxResidentChunks];     // gathered chunk partials of the tensor
   float red[kLansThreads / kWave];
   float norm[4];
   int chunk;
@@ -406,45 +429,46 @@ __device__ __forceinline__ uint64_t wait_word(const LansTables& t, const LansSca
   return x;
 }
 
-// Norms `first` and `first`+1 of the tensor from the partials its workgroups publish (this one has
-// published its own, a0 and a1, just before).  The workgroup that arrives last (a per-tensor counter,
-// cleared by the host before the step) gathers the partials into LDS, sums them in the fixed order of
-// wave_norm and publishes the two norms as self-validating words; every other workgroup waits for those
-// two words only.  Waits are bounded.
+// Norms first .. first+N-1 of the tensor from the partials its workgroups publish (this one has
+// published its own, a[], just before).  The workgroup that arrives last (a per-tensor counter, cleared
+// by the host before the step) gathers the partials into LDS, sums them in the fixed order of
+// wave_norm and publishes the norms as self-validating words; every other workgroup waits for those
+// words only.  Waits are bounded.
+template <int N>
 __device__ __forceinline__ void resident_norms(const LansTables& t, const LansScalars& sc, int first, int tensor,
-                                               float a0, float a1, ResidentShared& sh) {
+                                               const float (&a)[N], ResidentShared& sh) {
   const int lo = t.tensor_first[tensor];
   const int nc = t.tensor_first[tensor + 1] - lo;
   const int w = threadIdx.x / kWave;
   if (nc == 1) {
     if (threadIdx.x == 0) {
-      sh.part[0][0] = a0;
-      sh.part[1][0] = a1;
+#pragma unroll
+      for (int k = 0; k < N; ++k) sh.part[k][0] = a[k];
     }
     __syncthreads();
   } else {
     if (threadIdx.x == 0) {
-      uint32_t* arrive = t.ticket + 2 + static_cast<size_t>(first / 2) * t.T + tensor;
+      uint32_t* arrive = t.ticket + 2 + tensor;
       const uint32_t old = __hip_atomic_fetch_add(arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       sh.last = old == static_cast<uint32_t>(nc - 1);
     }
     __syncthreads();
     if (!sh.last) {
-      if (w < 2 && lane_id() == 0) {
+      if (w < N && lane_id() == 0) {
         const uint64_t x = wait_word(t, sc, t.norm_word + static_cast<size_t>(first + w) * t.T + tensor);
         sh.norm[first + w] = __uint_as_float(static_cast<uint32_t>(x));
       }
       __syncthreads();
       return;
     }
-    for (int idx = threadIdx.x; idx < 2 * nc; idx += kLansThreads) {
-      const int which = idx >= nc ? 1 : 0;
+    for (int idx = threadIdx.x; idx < N * nc; idx += kLansThreads) {
+      const int which = idx / nc;
       const uint64_t x = wait_word(t, sc, t.part_word + static_cast<size_t>(first + which) * t.nchunks + lo + (idx - which * nc));
       sh.part[which][idx - which * nc] = __uint_as_float(static_cast<uint32_t>(x));
     }
     __syncthreads();
   }
-  if (w < 2) {
+  if (w < N) {
     const float n = wave_norm(0, nc, [&](int c) { return sh.part[w][c]; });
     if (lane_id() == 0) {
       sh.norm[first + w] = n;
@@ -454,80 +478,64 @@ __device__ __forceinline__ void resident_norms(const LansTables& t, const LansSc
   __syncthreads();
 }
 
-// One whole chunk of 16-byte aligned arrays through the three phases, every access an unconditional
-// float4.  g and then the updates u_m, u_g stay in registers, p in LDS: each array is read once and
-// written once.
-__device__ __forceinline__ void resident_chunk(const LansTables& t, const LansScalars& sc, const ChunkView& c, int chunk,
-                                               float bc1, float bc2, ResidentShared& sh) {
+// One whole chunk of 16-byte aligned arrays, every access an unconditional float4.  ||g|| of the tensor is
+// already in t.norms (a sweep over g alone ran first), so one pass loads everything, writes m and v and
+// leaves u_m, u_g in registers and p in LDS; Sum p^2 joins the two update sums at the single wait, after
+// which p is written: every array is read once and written once, g twice.
+__device__ __forceinline__ void resident_chunk(const LansTables& t, const LansScalars& sc, const ChunkView& c,
+                                                       int chunk, float bc1, float bc2, ResidentShared& sh) {
   const LANCET_GLOBAL float* g = as_global(t.g[c.tensor] + c.begin);
   LANCET_GLOBAL float* p = as_global(t.p[c.tensor] + c.begin);
   LANCET_GLOBAL float* m = as_global(t.m[c.tensor] + c.begin);
   LANCET_GLOBAL float* v = as_global(t.v[c.tensor] + c.begin);
-  f32x4 xg[kVecPerThread], xu[kVecPerThread];
+  f32x4 xg[kVecPerThread], xu[kVecPerThread];  // u_g and u_m of the thread's eight float4
   // a wave owns 2048 consecutive elements: float4 k of lane l is element 4 * (64 k + l) of them, so one
-  // load instruction of a wave covers 1 KB of consecutive memory and the eight of a thread differ by
-  // constant offsets
+  // load instruction of a wave covers 1 KB of consecutive memory
   const int e0 = (threadIdx.x / kWave) * (kLansChunk / kWavesPerTile) + 4 * lane_id();
-  // phase 1
-  float a0 = 0.f, a1 = 0.f;
+  const LansElem el = make_elem(sc, t.norms[c.tensor], bc1, bc2);
+  float a0 = 0.f, a1 = 0.f, a2 = 0.f;
 #pragma unroll
   for (int k = 0; k < kVecPerThread; ++k) {
     const int e = e0 + k * (4 * kWave);
-    xg[k] = ld4(g, e);
-    const f32x4 xp = ld4(p, e);
+    const f32x4 g4 = ld4(g, e), xp = ld4(p, e);
+    f32x4 xm = ld4(m, e), xv = ld4(v, e);
     sh.p[k][threadIdx.x] = xp;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      a0 += xg[k][j] * xg[k][j];
-      a1 += xp[j] * xp[j];
-    }
-  }
-  a0 = block_sum(a0, sh.red);
-  a1 = block_sum(a1, sh.red);
-  if (threadIdx.x == 0) {
-    st_word(t.part_word + chunk, sc.epoch, a0);
-    st_word(t.part_word + t.nchunks + chunk, sc.epoch, a1);
-  }
-  resident_norms(t, sc, 0, c.tensor, a0, a1, sh);
-  // phase 2: m, v get their final values; u_g takes the registers of g
-  const LansElem el = make_elem(sc, sh.norm[0], bc1, bc2);
-  a0 = 0.f, a1 = 0.f;
-#pragma unroll
-  for (int k = 0; k < kVecPerThread; ++k) {
-    const int e = e0 + k * (4 * kWave);
-    f32x4 xm = ld4(m, e), xv = ld4(v, e);
-    const f32x4 xp = sh.p[k][threadIdx.x];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float sg = el.scaled_grad(xg[k][j], xp[j]);
+      const float sg = el.scaled_grad(g4[j], xp[j]);
       float mm = xm[j], vv = xv[j], u0, u1;
       el.moments(sg, mm, vv);
       el.updates(sg, xp[j], mm, vv, u0, u1);
-      // the two updates are final here: nothing of their computation may be left for phase 3 (the
-      // compiler otherwise carries a third value per element, wd * p, across the wait)
+      // the two updates are final here: nothing of their computation may be left for after the wait (the
+      // compiler otherwise carries a third value per element, wd * p, across it and spills)
       asm volatile("" : "+v"(u0), "+v"(u1));
       xm[j] = mm;
       xv[j] = vv;
       xu[k][j] = u0;
       xg[k][j] = u1;
-      a0 += u0 * u0;
-      a1 += u1 * u1;
+      a0 += xp[j] * xp[j];
+      a1 += u0 * u0;
+      a2 += u1 * u1;
     }
     st4(m, e, xm);
     st4(v, e, xv);
   }
   a0 = block_sum(a0, sh.red);
   a1 = block_sum(a1, sh.red);
+  a2 = block_sum(a2, sh.red);
   if (threadIdx.x == 0) {
-    st_word(t.part_word + 2 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a0);
-    st_word(t.part_word + 3 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a1);
+    st_word(t.part_word + 1 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a0);
+    st_word(t.part_word + 2 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a1);
+    st_word(t.part_word + 3 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a2);
   }
-  resident_norms(t, sc, 2, c.tensor, a0, a1, sh);
+  {
+    const float a[3] = {a0, a1, a2};
+    resident_norms<3>(t, sc, 1, c.tensor, a, sh);
+  }
   if (threadIdx.x == 0 && chunk == t.tensor_first[c.tensor]) {
 #pragma unroll
-    for (int k = 0; k < 4; ++k) t.norms[k * t.T + c.tensor] = sh.norm[k];
+    for (int k = 1; k < 4; ++k) t.norms[k * t.T + c.tensor] = sh.norm[k];
   }
-  // phase 3
   const float pn = uniform(sh.norm[1]), umn = uniform(sh.norm[2]), ugn = uniform(sh.norm[3]);
   float ratio_m = (umn != 0.f && pn != 0.f) ? sc.lr * (pn / umn) : sc.lr;
   float ratio_g = (ugn != 0.f && pn != 0.f) ? sc.lr * (pn / ugn) : sc.lr;
@@ -546,28 +554,25 @@ __device__ __forceinline__ void resident_chunk(const LansTables& t, const LansSc
   }
 }
 
-// A partial or unaligned chunk through the same three phases with the streaming chunk functions of the
-// sweeps (nothing held in registers; m and v written in phase 2 are read back by the thread that wrote
-// them).  At most one chunk per tensor takes this path when arrays are aligned.
+// A partial or unaligned chunk through the same protocol with the streaming chunk functions of the
+// sweeps (nothing held in registers; m and v written before the wait are read back after it by the thread
+// that wrote them).  At most one chunk per tensor takes this path when arrays are aligned.
 __device__ __forceinline__ void resident_chunk_streamed(const LansTables& t, const LansScalars& sc, const ChunkView& c,
                                                         int chunk, float bc1, float bc2, ResidentShared& sh) {
-  float a0, a1;
-  chunk_norm_gp(t, c, sh.red, a0, a1);
+  float sum_g, a0, a1, a2;
+  chunk_norm_gp(t, c, sh.red, sum_g, a0);
+  const LansElem el = make_elem(sc, t.norms[c.tensor], bc1, bc2);
+  chunk_moments(t, c, el, sh.red, a1, a2);
   if (threadIdx.x == 0) {
-    st_word(t.part_word + chunk, sc.epoch, a0);
-    st_word(t.part_word + t.nchunks + chunk, sc.epoch, a1);
+    st_word(t.part_word + 1 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a0);
+    st_word(t.part_word + 2 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a1);
+    st_word(t.part_word + 3 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a2);
   }
-  resident_norms(t, sc, 0, c.tensor, a0, a1, sh);
-  const LansElem el = make_elem(sc, sh.norm[0], bc1, bc2);
-  chunk_moments(t, c, el, sh.red, a0, a1);
-  if (threadIdx.x == 0) {
-    st_word(t.part_word + 2 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a0);
-    st_word(t.part_word + 3 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a1);
-  }
-  resident_norms(t, sc, 2, c.tensor, a0, a1, sh);
+  const float a[3] = {a0, a1, a2};
+  resident_norms<3>(t, sc, 1, c.tensor, a, sh);
   if (threadIdx.x == 0 && chunk == t.tensor_first[c.tensor]) {
 #pragma unroll
-    for (int k = 0; k < 4; ++k) t.norms[k * t.T + c.tensor] = sh.norm[k];
+    for (int k = 1; k < 4; ++k) t.norms[k * t.T + c.tensor] = sh.norm[k];
   }
   chunk_update(t, c, el, sc, sh.norm[1], sh.norm[2], sh.norm[3]);
 }
@@ -707,7 +712,7 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
   const size_t o_norms = off;     off = align_up(off + 4 * T * sizeof(float), 256);
   const size_t o_consts = off;    off = align_up(off + 2 * sizeof(float), 256);
   const size_t o_words = off;     off = align_up(off + 4 * ((n ? n : 1) + T) * sizeof(uint64_t), 256);
-  const size_t o_ticket = off;    off = align_up(off + (2 + 2 * static_cast<size_t>(T)) * sizeof(uint32_t), 256);
+  const size_t o_ticket = off;    off = align_up(off + (2 + static_cast<size_t>(T)) * sizeof(uint32_t), 256);
   const size_t o_order = off;     off = align_up(off + T * sizeof(int32_t), 256);
   pl->schedule = LANCET_LANS_SWEEPS;
   pl->epoch = 0;
@@ -742,7 +747,7 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
     if (err == hipSuccess) err = hipMemcpy(base + o_first, first.data(), (T + 1) * sizeof(int32_t), hipMemcpyHostToDevice);
     if (err == hipSuccess) err = hipMemset(base + o_norms, 0, 4 * T * sizeof(float));
     if (err == hipSuccess) err = hipMemset(base + o_words, 0, pl->words_bytes);
-    if (err == hipSuccess) err = hipMemset(base + o_ticket, 0, (2 + 2 * static_cast<size_t>(T)) * sizeof(uint32_t));
+    if (err == hipSuccess) err = hipMemset(base + o_ticket, 0, (2 + static_cast<size_t>(T)) * sizeof(uint32_t));
     LansTables& t = pl->tables;
     t.part_word = reinterpret_cast<uint64_t*>(base + o_words);
     t.norm_word = t.part_word + 4 * (n ? n : 1);
@@ -860,9 +865,12 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
       pl->epoch = 1;
     }
     sc.epoch = pl->epoch;
-    err = run_fill_u32(t.ticket, 2 + 2 * static_cast<size_t>(T), 0u, st);
+    err = run_fill_u32(t.ticket, 2 + static_cast<size_t>(T), 0u, st);
     if (err != hipSuccess) return static_cast<int>(err);
     const int grid = std::min(pl->resident_grid, pl->n_res_chunks);
+    const int per_block = kLansThreads / kWave;
+    lans_norm_g_kernel<<<pl->n_res_chunks, kLansThreads, 0, st>>>(t);
+    lans_reduce_kernel<<<(pl->n_res_tensors + per_block - 1) / per_block, kLansThreads, 0, st>>>(t, 0, 0, pl->n_res_tensors, 1);
     lans_resident_kernel<<<grid, kLansThreads, 0, st>>>(t, sc);
     chunk_base = pl->n_res_chunks;
     tensor_base = pl->n_res_tensors;
@@ -873,9 +881,9 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
     const int rblocks = (T - tensor_base + per_block - 1) / per_block;
     lans_prepare_kernel<<<1, 64, 0, st>>>(t, sc);
     lans_norm_gp_kernel<<<nsweep, kLansThreads, 0, st>>>(t, chunk_base);
-    lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 0, tensor_base);
+    lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 0, tensor_base, T, 2);
     lans_moments_kernel<<<nsweep, kLansThreads, 0, st>>>(t, sc, chunk_base);
-    lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 2, tensor_base);
+    lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 2, tensor_base, T, 2);
     lans_update_kernel<<<nsweep, kLansThreads, 0, st>>>(t, sc, chunk_base);
   }
   return static_cast<int>(hipGetLastError());

@@ -195,17 +195,16 @@ def _chunk_table(pkg, numels, limit=1 << 30):
 
 
 def _simulate_resident(ctensor, workers, rng):
-    """The resident LANS schedule as a state machine: `workers` workgroups take chunks in list order from a
-    ticket; a workgroup publishes its phase-1 partial when it takes the chunk, moves to phase 2 once every
-    chunk of the tensor has published phase 1, publishes phase 2, and finishes once every chunk of the tensor
-    has published phase 2.  Workgroups are advanced in random order.  Returns True when every chunk finishes,
-    False when no workgroup can move."""
+    """The resident LANS kernel as a state machine: `workers` workgroups take chunks in ticket order; a
+    workgroup publishes its chunk's partial sums once it has taken the chunk (nothing it needs for that comes
+    from another workgroup) and finishes, freeing itself for the next ticket, once every chunk of the tensor
+    has published.  Workgroups are advanced in random order.  Returns True when every chunk finishes, False
+    when no workgroup can move."""
     n = len(ctensor)
     size = np.bincount(ctensor, minlength=int(ctensor.max()) + 1 if n else 1)
-    pub1 = np.zeros_like(size)
-    pub2 = np.zeros_like(size)
+    published = np.zeros_like(size)
     ticket, done = 0, 0
-    held = [None] * workers          # (tensor, phase) of the chunk a workgroup holds
+    held = [None] * workers          # tensor of the chunk a workgroup holds
     while done < n:
         moved = False
         for w in rng.permutation(workers):
@@ -213,19 +212,13 @@ def _simulate_resident(ctensor, workers, rng):
                 if ticket < n:
                     t = int(ctensor[ticket])
                     ticket += 1
-                    pub1[t] += 1
-                    held[w] = (t, 1)
+                    published[t] += 1
+                    held[w] = t
                     moved = True
-            else:
-                t, ph = held[w]
-                if ph == 1 and pub1[t] == size[t]:
-                    pub2[t] += 1
-                    held[w] = (t, 2)
-                    moved = True
-                elif ph == 2 and pub2[t] == size[t]:
-                    held[w] = None
-                    done += 1
-                    moved = True
+            elif published[held[w]] == size[held[w]]:
+                held[w] = None
+                done += 1
+                moved = True
         if not moved:
             return False
     return True

@@ -3,7 +3,7 @@
  * the MoE token-dispatch path and the fused LANS step.
  *
  * Every entry point replaces one piece of the reference's native launcher surface
- * (src/op/dialect/cuda/kernels/kernel_util.cuh:25-66) or of the OpEnv that drives it
+ * (src/op/dialect/cuda/kernels/kernel_util.cuh:25-79) or of the OpEnv that drives it
  * (src/op/dialect/cuda/moe.cc, src/op/dialect/cuda/lans.cc); the citation on each
  * declaration names the piece.  Conventions:
  *

@@ -48,7 +48,7 @@ extern "C" {
 #define LANCET_ERR_ALIGN (-5)     /* a pointer is not aligned to its element type */
 #define LANCET_ERR_TOPK (-6)      /* top_k not 1 or 2, or top_k = 2 with fewer than 2 experts */
 #define LANCET_ERR_PARTITION (-7) /* bad n_partitions / partition_id */
-#define LANCET_ERR_PLAN (-8)      /* invalid LANS plan handle */
+#define LANCET_ERR_PLAN (-8)      /* invalid LANS plan handle, or a plan of another device than the current one */
 
 /* limits */
 #define LANCET_MAX_EXPERTS 512

@@ -804,6 +804,8 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
   if (!g || !p || !m || !v || !h) return LANCET_ERR_NULL;
   if (!step_dev && step_host < 1) return LANCET_ERR_SHAPE;
   if (h->mode != 0 && h->mode != 1) return LANCET_ERR_SHAPE;
+  int current = -1;
+  if (hipGetDevice(&current) != hipSuccess || current != pl->device) return LANCET_ERR_PLAN;  // tables live on pl->device
   const int T = pl->T;
   hipStream_t st = static_cast<hipStream_t>(stream);
   bool changed = false;

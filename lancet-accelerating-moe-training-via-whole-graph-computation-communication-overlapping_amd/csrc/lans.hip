@@ -322,7 +322,7 @@ __global__ __launch_bounds__(kLansThreads) void lans_norm_gp_kernel(LansTables t
   }
 }
 
-// Sum g^2 alone, chunks [0, nchunks_g): ahead of the resident kernel in its one-wait form
+// Sum g^2 alone over the chunks the resident kernel will take: it needs ||g|| when it starts a chunk
 __global__ __launch_bounds__(kLansThreads) void lans_norm_g_kernel(LansTables t) {
   __shared__ float s_red[kLansThreads / kWave];
   const ChunkView c = chunk_view(t, blockIdx.x);
@@ -396,8 +396,8 @@ __device__ __forceinline__ void st_word(uint64_t* p, uint32_t epoch, float v) {
 }
 
 // =======================================================================================
-// schedule "resident": one persistent kernel; a workgroup keeps its chunk in registers across
-// the two per-tensor reductions, so every array is read once and written once (28 B/param)
+// schedule "resident": a sweep over g, then one persistent kernel in which a workgroup keeps its
+// chunk on chip between moments and update, so every array is read once and written once, g twice
 // =======================================================================================
 constexpr int kVecPerThread = kLansChunk / 4 / kLansThreads;  // float4 per thread and array
 

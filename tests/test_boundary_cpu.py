@@ -261,3 +261,16 @@ def test_lans_plan_orders_tensors_that_do_not_fit_last(pkg):
     assert set(ctensor[:nres]) == {i for i in fits if chunks[i] > 0}
     assert list(dict.fromkeys(ctensor[nres:])) == [2, 4]        # list order is kept inside each group
     assert _simulate_resident(ctensor[:nres], limit, np.random.default_rng(1))
+
+
+def test_missing_library_is_an_error_not_a_fallback(pkg, monkeypatch, tmp_path):
+    """Without the built library every operator raises; nothing routes to a CPU implementation."""
+    capi = pkg.capi
+    monkeypatch.setattr(capi, "_lib", None)
+    monkeypatch.setattr(capi, "LIB_PATH", str(tmp_path / "liblancet_hip.so"))
+    with pytest.raises(RuntimeError, match="not built"):
+        capi.load()
+    with pytest.raises(RuntimeError, match="not built"):
+        pkg.ops.moe_capacity(16, 4, 1.0)
+    src = open(os.path.join(os.path.dirname(capi.__file__), "ops.py")).read()
+    assert "oracle" not in src and "numpy" not in src          # the operator layer never imports the checker

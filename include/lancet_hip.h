@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define LANCET_ABI_VERSION 1
+#define LANCET_ABI_VERSION 2
 
 /* element type of token rows */
 #define LANCET_F32 0
@@ -78,9 +78,12 @@ int64_t lancet_moe_capacity(int64_t S, int64_t E, float capacity_factor);
  * with slot 1's expert masked), and gate[s, idx] or its softmax probability.
  * Replaces: the three TVM-compiled micro-kernels argmax / one_hot / multiply+sum that
  * MoeEncode runs first (src/op/dialect/cuda/moe.cc:177-250, executed :366-371) and, with
- * LANCET_GATE_IS_LOGITS, the softmax in front of the op (models/benchmark/pytorch/utils.py:565-573). */
-int lancet_gate_topk(const float* gate, int64_t S, int64_t E, int top_k, unsigned flags,
-                     int32_t* idx, float* val, lancet_stream_t stream);
+ * LANCET_GATE_IS_LOGITS, the softmax in front of the op (models/benchmark/pytorch/utils.py:565-573).
+ * gate2_noise (top_k = 2 only, may be NULL): [S,E] values added to `gate` for the second choice alone,
+ * the first choice masked out - the Gumbel noise of docker/resources/sharded_moe.py:275-278, drawn by
+ * the caller; val is always read from `gate` itself. */
+int lancet_gate_topk(const float* gate, const float* gate2_noise, int64_t S, int64_t E, int top_k,
+                     unsigned flags, int32_t* idx, float* val, lancet_stream_t stream);
 
 /* ---- launcher level ----------------------------------------------------------------
  * Replaces launch_gen_location (kernel_util.cuh:60; tutel_moe_dispatch.cu:164-212,548-553).
@@ -107,9 +110,9 @@ int lancet_launch_encode_forward(const int32_t* indices, const int32_t* location
  * (docker/resources/sharded_moe.py:253-324, no noise): outputs are slot-major
  * (gates_s[2S], indices_locations[2, 2S]) in the layout moe_merge_masks produces for the two
  * chained top-1 encodes it is equivalent to, and gates_s holds the normalised combine weights.
- * used_in may be NULL (= zeros). */
+ * used_in may be NULL (= zeros); gate2_noise as in lancet_gate_topk, NULL = none. */
 size_t lancet_moe_encode_workspace_bytes(int64_t S, int64_t E, int top_k);
-int lancet_moe_encode(const void* data, const float* gate, const int32_t* used_in,
+int lancet_moe_encode(const void* data, const float* gate, const float* gate2_noise, const int32_t* used_in,
                       int64_t S, int64_t M, int64_t E, int64_t C, int top_k, int dtype,
                       unsigned flags, float* gates_s, int32_t* indices_locations,
                       int32_t* used_out, uint64_t* elements_per_expert, void* dispatched,
@@ -123,8 +126,8 @@ int lancet_moe_encode(const void* data, const float* gate, const int32_t* used_i
  *                        except the buffer;
  *   lancet_moe_scatter = launch_encode_forward (moe.cc:381-395) on routing produced by
  *                        lancet_moe_route; zero-fills the rows past used_out - used_in. */
-int lancet_moe_route(const float* gate, const int32_t* used_in, int64_t S, int64_t M, int64_t E,
-                     int64_t C, int top_k, unsigned flags, float* gates_s,
+int lancet_moe_route(const float* gate, const float* gate2_noise, const int32_t* used_in, int64_t S, int64_t M,
+                     int64_t E, int64_t C, int top_k, unsigned flags, float* gates_s,
                      int32_t* indices_locations, int32_t* used_out, uint64_t* elements_per_expert,
                      void* workspace, size_t workspace_bytes, lancet_stream_t stream);
 int lancet_moe_scatter(const void* data, const int32_t* indices_locations, const int32_t* used_in,

@@ -12,6 +12,7 @@ LIB_PATH = os.path.join(HERE, "lib", "liblancet_hip.so")
 F32, BF16, F16 = 0, 1, 2
 GATE_IS_LOGITS = 1
 NO_TAIL_ZERO = 2
+ABI_VERSION = 2
 ZERO_TAIL = 4
 LANS_SWEEPS, LANS_RESIDENT = 0, 1
 MAX_EXPERTS = 512
@@ -40,14 +41,14 @@ SIGNATURES = {
     "lancet_abi_version": (_int, []),
     "lancet_status_string": (C.c_char_p, [_int]),
     "lancet_moe_capacity": (_i64, [_i64, _i64, _f32]),
-    "lancet_gate_topk": (_int, [_vp, _i64, _i64, _int, _u32, _vp, _vp, _vp]),
+    "lancet_gate_topk": (_int, [_vp, _vp, _i64, _i64, _int, _u32, _vp, _vp, _vp]),
     "lancet_gen_location_workspace_bytes": (_sz, [_i64, _i64]),
     "lancet_launch_gen_location": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _sz, _vp]),
     "lancet_launch_encode_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "lancet_moe_encode_workspace_bytes": (_sz, [_i64, _i64, _int]),
-    "lancet_moe_encode": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _u32,
+    "lancet_moe_encode": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _u32,
                                  _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
-    "lancet_moe_route": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _u32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "lancet_moe_route": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _u32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "lancet_moe_scatter": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _u32, _vp, _vp]),
     "lancet_moe_encode_bpr_workspace_bytes": (_sz, [_i64, _i64, _int]),
     "lancet_moe_encode_bpr": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _u32,
@@ -101,8 +102,8 @@ def load():
         fn.restype = res
         fn.argtypes = args
     got = lib.lancet_abi_version()
-    if got != 1:
-        raise RuntimeError("liblancet_hip.so has ABI version %d, expected 1" % got)
+    if got != ABI_VERSION:
+        raise RuntimeError("liblancet_hip.so has ABI version %d, expected %d" % (got, ABI_VERSION))
     _lib = lib
     return lib
 

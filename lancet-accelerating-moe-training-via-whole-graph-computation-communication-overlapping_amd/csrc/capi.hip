@@ -78,14 +78,16 @@ extern "C" int lancet_scan_workspace_error(const void* workspace, lancet_stream_
 }
 
 // ---- routing front end ---------------------------------------------------------------
-extern "C" int lancet_gate_topk(const float* gate, int64_t S, int64_t E, int top_k, unsigned flags,
-                                int32_t* idx, float* val, lancet_stream_t stream) {
+extern "C" int lancet_gate_topk(const float* gate, const float* gate2_noise, int64_t S, int64_t E, int top_k,
+                                unsigned flags, int32_t* idx, float* val, lancet_stream_t stream) {
   if (!gate || !idx || !val) return LANCET_ERR_NULL;
   if (int r = check_dims(S, 0, E, 0)) return r;
   if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
   if (top_k == 2 && E < 2) return LANCET_ERR_TOPK;
-  if (misaligned(gate, 4) || misaligned(idx, 4) || misaligned(val, 4)) return LANCET_ERR_ALIGN;
-  return rc(run_gate_topk(gate, static_cast<int>(S), static_cast<int>(E), top_k,
+  if (gate2_noise && top_k != 2) return LANCET_ERR_TOPK;  // the noise only exists for the second choice
+  if (misaligned(gate, 4) || misaligned(gate2_noise, 4) || misaligned(idx, 4) || misaligned(val, 4))
+    return LANCET_ERR_ALIGN;
+  return rc(run_gate_topk(gate, gate2_noise, static_cast<int>(S), static_cast<int>(E), top_k,
                           (flags & LANCET_GATE_IS_LOGITS) != 0, idx, val, S_(stream)));
 }
 
@@ -105,7 +107,7 @@ extern "C" int lancet_launch_gen_location(int32_t* indices, const int32_t* in_ca
   if (misaligned(indices, 4) || misaligned(locations, 4) || misaligned(out_capused, 4) ||
       misaligned(out_elements_per_expert, 8) || misaligned(workspace, 4) || misaligned(in_capused, 4))
     return LANCET_ERR_ALIGN;
-  return rc(run_route_scan(nullptr, indices, in_capused, static_cast<int>(S), static_cast<int>(E),
+  return rc(run_route_scan(nullptr, nullptr, indices, in_capused, static_cast<int>(S), static_cast<int>(E),
                            static_cast<int>(C), static_cast<int>(M), 1, false, nullptr, indices, locations,
                            out_capused, out_elements_per_expert, workspace, S_(stream)));
 }
@@ -135,8 +137,8 @@ extern "C" size_t lancet_moe_encode_workspace_bytes(int64_t S, int64_t E, int to
   return scan_workspace_bytes(S, E, top_k);
 }
 
-extern "C" int lancet_moe_route(const float* gate, const int32_t* used_in, int64_t S, int64_t M, int64_t E,
-                                int64_t C, int top_k, unsigned flags, float* gates_s,
+extern "C" int lancet_moe_route(const float* gate, const float* gate2_noise, const int32_t* used_in, int64_t S,
+                                int64_t M, int64_t E, int64_t C, int top_k, unsigned flags, float* gates_s,
                                 int32_t* indices_locations, int32_t* used_out, uint64_t* elements_per_expert,
                                 void* workspace, size_t workspace_bytes, lancet_stream_t stream) {
   if (((!gate || !gates_s || !indices_locations) && S > 0) || !used_out || !elements_per_expert)
@@ -144,12 +146,13 @@ extern "C" int lancet_moe_route(const float* gate, const int32_t* used_in, int64
   if (int r = check_dims(S, M, E, C)) return r;
   if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
   if (top_k == 2 && E < 2) return LANCET_ERR_TOPK;
+  if (gate2_noise && top_k != 2) return LANCET_ERR_TOPK;
   if (!workspace || workspace_bytes < lancet_moe_encode_workspace_bytes(S, E, top_k)) return LANCET_ERR_WORKSPACE;
-  if (misaligned(gate, 4) || misaligned(gates_s, 4) || misaligned(indices_locations, 4) || misaligned(used_in, 4) ||
+  if (misaligned(gate, 4) || misaligned(gate2_noise, 4) || misaligned(gates_s, 4) || misaligned(indices_locations, 4) || misaligned(used_in, 4) ||
       misaligned(used_out, 4) || misaligned(elements_per_expert, 8) || misaligned(workspace, 4))
     return LANCET_ERR_ALIGN;
   const int s = static_cast<int>(S);
-  return rc(run_route_scan(gate, nullptr, used_in, s, static_cast<int>(E), static_cast<int>(C),
+  return rc(run_route_scan(gate, gate2_noise, nullptr, used_in, s, static_cast<int>(E), static_cast<int>(C),
                            static_cast<int>(M), top_k, (flags & LANCET_GATE_IS_LOGITS) != 0, gates_s,
                            indices_locations, indices_locations + static_cast<size_t>(top_k) * s, used_out,
                            elements_per_expert, workspace, S_(stream)));
@@ -174,8 +177,9 @@ extern "C" int lancet_moe_scatter(const void* data, const int32_t* indices_locat
                              static_cast<int>(E), static_cast<int>(C), top_k, eb, S_(stream)));
 }
 
-extern "C" int lancet_moe_encode(const void* data, const float* gate, const int32_t* used_in, int64_t S,
-                                 int64_t M, int64_t E, int64_t C, int top_k, int dtype, unsigned flags,
+extern "C" int lancet_moe_encode(const void* data, const float* gate, const float* gate2_noise,
+                                 const int32_t* used_in, int64_t S, int64_t M, int64_t E, int64_t C, int top_k,
+                                 int dtype, unsigned flags,
                                  float* gates_s, int32_t* indices_locations, int32_t* used_out,
                                  uint64_t* elements_per_expert, void* dispatched, void* workspace,
                                  size_t workspace_bytes, lancet_stream_t stream) {
@@ -184,7 +188,7 @@ extern "C" int lancet_moe_encode(const void* data, const float* gate, const int3
   const int eb = elem_bytes(dtype);
   if (!eb) return LANCET_ERR_DTYPE;
   if (misaligned(data, eb) || misaligned(dispatched, eb)) return LANCET_ERR_ALIGN;
-  if (int r = lancet_moe_route(gate, used_in, S, M, E, C, top_k, flags, gates_s, indices_locations, used_out,
+  if (int r = lancet_moe_route(gate, gate2_noise, used_in, S, M, E, C, top_k, flags, gates_s, indices_locations, used_out,
                                elements_per_expert, workspace, workspace_bytes, stream))
     return r;
   return lancet_moe_scatter(data, indices_locations, used_in, used_out, S, M, E, C, top_k, dtype, flags, dispatched,

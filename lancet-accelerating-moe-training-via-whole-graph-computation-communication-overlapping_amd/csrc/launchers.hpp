@@ -18,11 +18,12 @@ uint32_t current_spin_limit();
 void set_spin_limit(uint32_t limit);
 
 hipError_t run_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t st);
-hipError_t run_gate_topk(const float* gate, int S, int E, int K, bool is_logits, int32_t* idx,
+// noise (top-2 only, may be null): [S,E] values added to the row for the second choice
+hipError_t run_gate_topk(const float* gate, const float* noise, int S, int E, int K, bool is_logits, int32_t* idx,
                          float* val, hipStream_t st);
 // gate-driven (idx_in == nullptr) or index-driven (gate == nullptr, K == 1) routing + scan.
 // idx_out/loc_out are [K*S] each.
-hipError_t run_route_scan(const float* gate, const int32_t* idx_in, const int32_t* used_in, int S,
+hipError_t run_route_scan(const float* gate, const float* noise, const int32_t* idx_in, const int32_t* used_in, int S,
                           int E, int C, int M, int K, bool is_logits, float* gates_s,
                           int32_t* idx_out, int32_t* loc_out, int32_t* used_out,
                           uint64_t* elems_out, void* ws, hipStream_t st);

@@ -39,8 +39,11 @@ struct Routed {
   float p0, p1;
 };
 
+// noise (K = 2 only, may be null): values added to the row for the second choice alone, the first
+// choice masked out (docker/resources/sharded_moe.py:275-278); gate values always come from the row.
 template <int K>
-__device__ __forceinline__ Routed route_token(const float* __restrict__ row, int E, bool is_logits) {
+__device__ __forceinline__ Routed route_token(const float* __restrict__ row, const float* __restrict__ noise, int E,
+                                              bool is_logits) {
   typedef float f32x4 __attribute__((ext_vector_type(4)));
   TopState t = {0.f, 0.f, -1, -1};
   const bool vec = ((E & 3) == 0) && ((reinterpret_cast<uintptr_t>(row) & 15u) == 0);
@@ -55,6 +58,19 @@ __device__ __forceinline__ Routed route_token(const float* __restrict__ row, int
     }
   } else {
     for (int j = 0; j < E; ++j) t = consider<K>(t, row[j], j);
+  }
+  if (K == 2 && noise) {
+    // second choice again, on row + noise: first max over the experts other than the first choice
+    float best = 0.f;
+    t.i2 = -1;
+    for (int j = 0; j < E; ++j) {
+      const float x = row[j];
+      const float y = x + noise[j];
+      const bool take = (j != t.i1) & ((t.i2 < 0) | (y > best));
+      best = take ? y : best;
+      t.v2 = take ? x : t.v2;
+      t.i2 = take ? j : t.i2;
+    }
   }
   float sum = 1.f;
   if (is_logits) {
@@ -82,6 +98,7 @@ __device__ __forceinline__ Routed route_token(const float* __restrict__ row, int
 
 struct RouteArgs {
   const float* gate;      // [S,E] (NULL when idx_in is given)
+  const float* noise;     // [S,E] or NULL: added for the second choice (K = 2)
   const int32_t* idx_in;  // launcher-level entry: expert per token already chosen (may alias idx_out)
   const int32_t* used_in; // [E] or NULL (= zeros)
   float* gates_s;         // [K*S] (NULL when idx_in is given)
@@ -123,7 +140,9 @@ __global__ __launch_bounds__(kTile) void route_scan_kernel(RouteArgs a) {
       const int x = a.idx_in[s];
       e[0] = (x >= 0 && x < a.E) ? x : -1;
     } else {
-      const Routed r = route_token<K>(a.gate + static_cast<size_t>(s) * a.E, a.E, a.is_logits != 0);
+      const Routed r = route_token<K>(a.gate + static_cast<size_t>(s) * a.E,
+                                      a.noise ? a.noise + static_cast<size_t>(s) * a.E : nullptr, a.E,
+                                      a.is_logits != 0);
       e[0] = r.e0;
       p[0] = r.p0;
       if (K == 2) {
@@ -213,11 +232,12 @@ __global__ __launch_bounds__(kTile) void finalize_top2_kernel(RouteArgs a) {
 
 // Selection only (no scan).
 template <int K>
-__global__ __launch_bounds__(kTile) void gate_topk_kernel(const float* gate, int S, int E, int is_logits,
-                                                          int32_t* idx, float* val) {
+__global__ __launch_bounds__(kTile) void gate_topk_kernel(const float* gate, const float* noise, int S, int E,
+                                                          int is_logits, int32_t* idx, float* val) {
   const int s = blockIdx.x * kTile + threadIdx.x;
   if (s >= S) return;
-  const Routed r = route_token<K>(gate + static_cast<size_t>(s) * E, E, is_logits != 0);
+  const Routed r = route_token<K>(gate + static_cast<size_t>(s) * E, noise ? noise + static_cast<size_t>(s) * E : nullptr,
+                                  E, is_logits != 0);
   idx[s] = r.e0;
   val[s] = r.p0;
   if (K == 2) {
@@ -440,21 +460,22 @@ hipError_t run_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t st) {
   return hipGetLastError();
 }
 
-hipError_t run_gate_topk(const float* gate, int S, int E, int K, bool is_logits, int32_t* idx,
+hipError_t run_gate_topk(const float* gate, const float* noise, int S, int E, int K, bool is_logits, int32_t* idx,
                          float* val, hipStream_t st) {
   if (S == 0) return hipSuccess;
   const int blocks = (S + kTile - 1) / kTile;
-  if (K == 1) gate_topk_kernel<1><<<blocks, kTile, 0, st>>>(gate, S, E, is_logits, idx, val);
-  else gate_topk_kernel<2><<<blocks, kTile, 0, st>>>(gate, S, E, is_logits, idx, val);
+  if (K == 1) gate_topk_kernel<1><<<blocks, kTile, 0, st>>>(gate, nullptr, S, E, is_logits, idx, val);
+  else gate_topk_kernel<2><<<blocks, kTile, 0, st>>>(gate, noise, S, E, is_logits, idx, val);
   return hipGetLastError();
 }
 
-hipError_t run_route_scan(const float* gate, const int32_t* idx_in, const int32_t* used_in, int S,
+hipError_t run_route_scan(const float* gate, const float* noise, const int32_t* idx_in, const int32_t* used_in, int S,
                           int E, int C, int M, int K, bool is_logits, float* gates_s,
                           int32_t* idx_out, int32_t* loc_out, int32_t* used_out,
                           uint64_t* elems_out, void* ws, hipStream_t st) {
   RouteArgs a;
   a.gate = gate;
+  a.noise = K == 2 ? noise : nullptr;
   a.idx_in = idx_in;
   a.used_in = used_in;
   a.gates_s = gates_s;
@@ -514,7 +535,7 @@ hipError_t run_bpr_route(const float* gate, int S0, int E, int C, int M, int n_p
   a.spin_limit = current_spin_limit();
   hipError_t err = run_fill_u32(static_cast<uint32_t*>(ws), scan_ws_words(a.ntiles, 2 * E), 0u, st);
   if (err != hipSuccess) return err;
-  err = run_gate_topk(gate, S0, E, 1, is_logits, idx0, prio, st);
+  err = run_gate_topk(gate, nullptr, S0, E, 1, is_logits, idx0, prio, st);
   if (err != hipSuccess) return err;
   bpr_select_kernel<<<E, kSelectThreads, 0, st>>>(a);
   err = hipGetLastError();

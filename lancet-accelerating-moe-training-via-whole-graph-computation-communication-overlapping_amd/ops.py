@@ -71,19 +71,30 @@ def _flags(gate_is_logits, zero_tail):
     return (capi.GATE_IS_LOGITS if gate_is_logits else 0) | (0 if zero_tail else capi.NO_TAIL_ZERO)
 
 
+def _check_noise(gate2_noise, gate, top_k):
+    if gate2_noise is None:
+        return
+    _dev(gate2_noise, "gate2_noise")
+    _need(top_k == 2, "gate2_noise only exists for the second choice (top_k = 2)")
+    _need(gate2_noise.shape == gate.shape and gate2_noise.dtype == torch.float32, "gate2_noise must be float32 [S, E]")
+
+
 def moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_logits=False,
-               zero_tail=True, workspace=None, out=None):
+               zero_tail=True, gate2_noise=None, workspace=None, out=None):
     """raf.op.moe_encode(data, gate, used_capacity, capacity_factor=1.0).
 
     Returns (gates_s [k*S] f32, indices_locations [2, k*S] i32, used_capacity [E] i32,
     elements_per_expert [E] u64, dispatched [E, C, M]).  With top_k = 2 the capacity follows
-    GShard: capacity_factor is doubled before the reference formula is applied.  zero_tail=False
+    GShard: capacity_factor is doubled before the reference formula is applied; gate2_noise [S, E], if
+    given, is added to the gate for the second choice alone (the Gumbel noise of
+    docker/resources/sharded_moe.py:275, drawn by the caller).  zero_tail=False
     leaves rows past the used capacity unwritten (partition buffers that only feed moe_redispatch)."""
     lib = capi.load()
     dt = _check_encode_inputs(data, gate)
     S, M = data.shape
     E = gate.shape[1]
     _need(top_k in (1, 2), "top_k must be 1 or 2")
+    _check_noise(gate2_noise, gate, top_k)
     cf = float(capacity_factor) * (2.0 if top_k == 2 else 1.0)
     Cap = moe_capacity(S, E, cf)
     if used_capacity is not None:
@@ -101,14 +112,15 @@ def moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_
         gates_s, indloc, used_out, elems, disp = out
     ws_bytes = moe_encode_workspace_bytes(S, E, top_k)
     ws = _workspace(ws_bytes, dev, workspace)
-    st = lib.lancet_moe_encode(_p(data), _p(gate), _p(used_capacity), S, M, E, Cap, top_k, dt,
+    st = lib.lancet_moe_encode(_p(data), _p(gate), _p(gate2_noise), _p(used_capacity), S, M, E, Cap, top_k, dt,
                                _flags(gate_is_logits, zero_tail), _p(gates_s), _p(indloc),
                                _p(used_out), _p(elems), _p(disp), _p(ws), ws.numel(), _stream())
     capi.check(st, "lancet_moe_encode")
     return gates_s, indloc, used_out, elems.view(torch.uint64) if elems.dtype == torch.int64 else elems, disp
 
 
-def moe_route(gate, used_capacity, M, capacity_factor=1.0, top_k=1, gate_is_logits=False, workspace=None, out=None):
+def moe_route(gate, used_capacity, M, capacity_factor=1.0, top_k=1, gate_is_logits=False, gate2_noise=None,
+              workspace=None, out=None):
     """The routing half of moe_encode (selection + position scan, src/op/dialect/cuda/moe.cc:366-380), so that
     a caller can run it ahead of, or beside, the row movement of another partition.  M only scales
     elements_per_expert.  Returns (gates_s, indices_locations, used_capacity, elements_per_expert)."""
@@ -117,6 +129,7 @@ def moe_route(gate, used_capacity, M, capacity_factor=1.0, top_k=1, gate_is_logi
     _need(gate.dim() == 2 and gate.dtype == torch.float32, "gate must be 2-D float32")
     S, E = gate.shape
     _need(top_k in (1, 2), "top_k must be 1 or 2")
+    _check_noise(gate2_noise, gate, top_k)
     Cap = moe_capacity(S, E, float(capacity_factor) * (2.0 if top_k == 2 else 1.0))
     dev = gate.device
     if out is None:
@@ -125,7 +138,7 @@ def moe_route(gate, used_capacity, M, capacity_factor=1.0, top_k=1, gate_is_logi
                torch.empty(E, dtype=torch.int32, device=dev), torch.empty(E, dtype=torch.int64, device=dev))
     gates_s, indloc, used_out, elems = out[:4]
     ws = _workspace(moe_encode_workspace_bytes(S, E, top_k), dev, workspace)
-    st = lib.lancet_moe_route(_p(gate), _p(used_capacity), S, int(M), E, Cap, top_k, _flags(gate_is_logits, True),
+    st = lib.lancet_moe_route(_p(gate), _p(gate2_noise), _p(used_capacity), S, int(M), E, Cap, top_k, _flags(gate_is_logits, True),
                               _p(gates_s), _p(indloc), _p(used_out), _p(elems), _p(ws), ws.numel(), _stream())
     capi.check(st, "lancet_moe_route")
     return gates_s, indloc, used_out, elems

@@ -122,17 +122,31 @@ class MoeEncode : public OpEnv {
     ws_bytes_ = lancet_moe_encode_workspace_bytes(shape_.S, shape_.E, top_k_);
     RequestWorkspace(&ws_, device_id_, static_cast<int64_t>(ws_bytes_));
     this->arg_indices = {0, 1, 2};  // data, gate, used_capacity
+    // trailing extension: gate2_noise [S, E] for the second choice of top_k = 2
+    has_noise_ = cv.args.size() > 7 && cv.args[7].kind == Value::kTensor;
+    if (has_noise_) {
+      const Tensor& noise = cv.args[7].AsTensor();
+      RAF_CHECK(top_k_ == 2, "gate2_noise only exists for the second choice (top_k = 2)");
+      RAF_CHECK(noise.shape == cv.args[1].AsTensor().shape && noise.dtype.code == DTypeCode::kFloat && noise.dtype.bits == 32,
+                "gate2_noise must be float32 [S, E]");
+      this->arg_indices.push_back(7);
+    }
   }
 
-  void Execute(const CallValues& cv) override { Execute({cv.args[0], cv.args[1], cv.args[2]}, cv.out); }
+  void Execute(const CallValues& cv) override {
+    std::vector<Value> inputs = {cv.args[0], cv.args[1], cv.args[2]};
+    if (has_noise_) inputs.push_back(cv.args[7]);
+    Execute(inputs, cv.out);
+  }
 
   void Execute(const std::vector<Value>& inputs, Value output) override {
     const Tensor& data = inputs[0].AsTensor();
     const Tensor& gate = inputs[1].AsTensor();
     const Tensor& used = inputs[2].AsTensor();
+    const float* noise = has_noise_ ? static_cast<const float*>(inputs[3].AsTensor().data) : nullptr;
     const auto& out = output.AsTuple();
     RAF_CHECK(out.size() == 5, "Expected output to be a 5-Tuple");
-    CheckStatus(lancet_moe_encode(data.data, static_cast<const float*>(gate.data),
+    CheckStatus(lancet_moe_encode(data.data, static_cast<const float*>(gate.data), noise,
                                   static_cast<const int32_t*>(used.data), shape_.S, shape_.M, shape_.E, shape_.C,
                                   top_k_, dtype_, flags_, static_cast<float*>(out[0].AsTensor().data),
                                   static_cast<int32_t*>(out[1].AsTensor().data),
@@ -149,6 +163,7 @@ class MoeEncode : public OpEnv {
   EncodeShape shape_;
   int top_k_, dtype_, device_id_;
   unsigned flags_;
+  bool has_noise_ = false;
   void* ws_ = nullptr;
   size_t ws_bytes_ = 0;
 };

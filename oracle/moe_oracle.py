@@ -63,12 +63,13 @@ def softmax_rows(logits):
 # --------------------------------------------------------------------------
 # A1 / A2 front end: top-1 / top-2 selection on the array the op is given
 # --------------------------------------------------------------------------
-def select_topk(gate, k=1, gate_is_logits=False):
+def select_topk(gate, k=1, gate_is_logits=False, gate2_noise=None):
     """Returns (idx [k,S] int32, val [k,S] fp32).
 
     idx[0] = argmax_e gate[s,e] (first max; src/op/dialect/cuda/moe.cc:177-195,
     tests/python/op/cuda/test_cuda_moe.py:115).  idx[1] = argmax with idx[0]
-    masked to -inf (docker/resources/sharded_moe.py:275-278, noise dropped).
+    masked to -inf (docker/resources/sharded_moe.py:275-278); gate2_noise [S,E], if given,
+    is added (fp32) to the array for that second choice alone, as the Gumbel noise of :275 is.
     val = gate[s, idx] (moe.cc:232-250: sum_e gate*onehot), or the softmax
     probability of that expert when the array holds logits."""
     g = np.asarray(gate, dtype=np.float32)
@@ -82,7 +83,7 @@ def select_topk(gate, k=1, gate_is_logits=False):
     val[0] = prob[rows, i1]
     if k == 2:
         assert E >= 2
-        masked = g.copy()
+        masked = g.copy() if gate2_noise is None else (g + np.asarray(gate2_noise, dtype=np.float32)).astype(np.float32)
         masked[rows, i1] = -np.inf
         # argmax of a row that is all -inf apart from i1 must not return i1
         i2 = np.argmax(masked, axis=1).astype(np.int32)
@@ -280,7 +281,7 @@ def moe_decode(expert_out, gates_s, indloc, k=1, round_fn=None):
 # A.6: top-2 extension (docker/resources/sharded_moe.py:253-324, no Gumbel noise)
 # --------------------------------------------------------------------------
 def moe_encode_top2(data, gate, used_in, capacity_factor=1.0, gate_is_logits=False,
-                    C=None, fast_scatter=False):
+                    C=None, fast_scatter=False, gate2_noise=None):
     """GShard top-2 expressed as two chained reference top-1 encodes, merged:
     slot 1 with used_in, slot 2 with used_out(slot 1); merged layout is what
     moe_merge_masks/moe_redispatch give for the two calls.  Capacity follows the
@@ -292,7 +293,7 @@ def moe_encode_top2(data, gate, used_in, capacity_factor=1.0, gate_is_logits=Fal
     E = gate.shape[1]
     if C is None:
         C = capacity(S, E, 2.0 * capacity_factor)
-    sel, val = select_topk(gate, 2, gate_is_logits)
+    sel, val = select_topk(gate, 2, gate_is_logits, gate2_noise)
     used_in = np.asarray(used_in, dtype=np.int32)
     i1, l1, used1, _ = gen_location(sel[0], used_in, C, M, E)
     i2, l2, used2, _ = gen_location(sel[1], used1, C, M, E)

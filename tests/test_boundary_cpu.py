@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol(pkg):
     for n in names:
         assert hasattr(lib, n), "liblancet_hip.so does not export %s" % n
     assert sorted(pkg.capi.SIGNATURES) == names, "capi.SIGNATURES and the header disagree"
-    assert lib.lancet_abi_version() == 1
+    assert lib.lancet_abi_version() == pkg.capi.ABI_VERSION == 2
 
 
 def test_capacity_formula(pkg):
@@ -39,22 +39,24 @@ def test_workspace_sizes_and_argument_rejection(pkg):
     assert lib.lancet_moe_encode_workspace_bytes(0, 4, 1) == (2 + 1 * 4) * 4
     assert lib.lancet_moe_encode_workspace_bytes(10, 0, 1) == 0
     one = C.c_void_p(16)  # never dereferenced: every call below is rejected before any launch
-    st = lib.lancet_moe_encode(one, one, None, 8, 4, 2, 4, 1, 99, 0, one, one, one, one, one, one, 1 << 20, None)
+    st = lib.lancet_moe_encode(one, one, None, None, 8, 4, 2, 4, 1, 99, 0, one, one, one, one, one, one, 1 << 20, None)
     assert st == capi.ERR_DTYPE
-    st = lib.lancet_moe_encode(one, one, None, 8, 4, 2, 4, 3, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
+    st = lib.lancet_moe_encode(one, one, None, None, 8, 4, 2, 4, 3, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
     assert st == capi.ERR_TOPK
-    st = lib.lancet_moe_encode(one, one, None, 8, 4, 1, 4, 2, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
+    st = lib.lancet_moe_encode(one, one, None, None, 8, 4, 1, 4, 2, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
     assert st == capi.ERR_TOPK                      # top-2 needs two experts
-    st = lib.lancet_moe_encode(one, one, None, 8, 4, 2, 4, 1, capi.F32, 0, one, one, one, one, one, one, 8, None)
+    st = lib.lancet_moe_encode(one, one, None, None, 8, 4, 2, 4, 1, capi.F32, 0, one, one, one, one, one, one, 8, None)
     assert st == capi.ERR_WORKSPACE
-    st = lib.lancet_moe_encode(one, one, None, 8, 4, 2, 4, 1, capi.F32, 0, one, None, one, one, one, one, 1 << 20, None)
+    st = lib.lancet_moe_encode(one, one, None, None, 8, 4, 2, 4, 1, capi.F32, 0, one, None, one, one, one, one, 1 << 20, None)
     assert st == capi.ERR_NULL
-    st = lib.lancet_moe_encode(one, one, None, -1, 4, 2, 4, 1, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
+    st = lib.lancet_moe_encode(one, one, None, None, -1, 4, 2, 4, 1, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
     assert st == capi.ERR_SHAPE
-    st = lib.lancet_moe_encode(one, one, None, 8, 4, 1000, 4, 1, capi.F32, 0, one, one, one, one, one, one, 1 << 30, None)
+    st = lib.lancet_moe_encode(one, one, None, None, 8, 4, 1000, 4, 1, capi.F32, 0, one, one, one, one, one, one, 1 << 30, None)
     assert st == capi.ERR_SHAPE                     # more experts than LANCET_MAX_EXPERTS
-    st = lib.lancet_moe_encode(C.c_void_p(18), one, None, 8, 4, 2, 4, 1, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
+    st = lib.lancet_moe_encode(C.c_void_p(18), one, None, None, 8, 4, 2, 4, 1, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
     assert st == capi.ERR_ALIGN
+    st = lib.lancet_moe_encode(one, one, one, None, 8, 4, 2, 4, 1, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
+    assert st == capi.ERR_TOPK                      # noise for a second choice that does not exist
     st = lib.lancet_moe_encode_bpr(one, one, 8, 4, 2, 4, 2, 2, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
     assert st == capi.ERR_PARTITION
     ptrs = capi.ptr_array([16] * 70)

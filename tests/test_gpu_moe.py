@@ -472,3 +472,32 @@ def test_route_then_scatter_equals_encode(pkg, k, dt):
         assert torch.equal(a.view(torch.int64) if a.dtype == torch.uint64 else a,
                            b.view(torch.int64) if b.dtype in (torch.uint64,) else b)
     assert (to_np(indloc)[0] < 0).any()
+
+
+# ----------------------------------------------------------------------------- top-2 with second-choice noise
+@pytest.mark.parametrize("dt,is_logits", [("f32", True), ("bf16", True), ("f32", False)])
+def test_encode_top2_with_second_choice_noise(pkg, dt, is_logits):
+    """gate2_noise stands for the Gumbel sample GShard adds before the second argmax
+    (docker/resources/sharded_moe.py:275-278): it moves second choices, never the first, and gate values
+    still come from the un-noised gate.  Through the op function, the routing half alone and the op layer."""
+    ops = pkg.ops
+    S, M, E, cf = 1800, 32, 10, 0.8
+    data, logits = make_inputs(77, S, M, E, zipf_bias=True)
+    gate = logits if is_logits else mo.softmax_rows(logits)
+    noise = np.random.default_rng(8).gumbel(size=(S, E)).astype(np.float32) * np.float32(1.0 if is_logits else 0.05)
+    x = rows_as_oracle(data, dt)
+    used0 = np.zeros(E, np.int32)
+    want = mo.moe_encode_top2(x, gate, used0, cf, gate_is_logits=is_logits, fast_scatter=True, gate2_noise=noise)
+    plain = mo.moe_encode_top2(x, gate, used0, cf, gate_is_logits=is_logits, fast_scatter=True)
+    assert (want[1][0, S:] != plain[1][0, S:]).any()
+    d_x, d_gate, d_noise, d_used = rows_to_torch(data, dt), dev(gate), dev(noise), dev(used0)
+    got = ops.moe_encode(d_x, d_gate, d_used, cf, top_k=2, gate_is_logits=is_logits, gate2_noise=d_noise)
+    check_encode(got, want, gate_exact=not is_logits)
+    routed = ops.moe_route(d_gate, d_used, M, cf, top_k=2, gate_is_logits=is_logits, gate2_noise=d_noise)
+    np.testing.assert_array_equal(to_np(routed[1]), want[1])
+    ex = pkg.raf_executor.Executor()
+    outs = ex("raf.op.moe_encode", d_x, d_gate, d_used, cf, 2, int(is_logits), 1, d_noise)
+    np.testing.assert_array_equal(to_np(outs[1]), want[1])
+    np.testing.assert_array_equal(to_np(outs[4]), want[4])
+    with pytest.raises(ValueError):
+        ops.moe_encode(d_x, d_gate, d_used, cf, top_k=1, gate2_noise=d_noise)

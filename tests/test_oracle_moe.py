@@ -208,13 +208,15 @@ def test_bpr_bruteforce(S0, E, P, cf, ties):
 
 
 # ---------------------------------------------------------------- top-2 (A.6) vs dense GShard form
-def dense_top2(logits, data, C):
-    """docker/resources/sharded_moe.py:253-324 written with dense masks, no noise."""
+def dense_top2(logits, data, C, noise=None):
+    """docker/resources/sharded_moe.py:253-324 written with dense masks; `noise` stands for the Gumbel
+    sample of :275 (logits_w_noise = logits + noise, used for the second choice only)."""
     S, E = logits.shape
     gates = sp_softmax(logits.astype(np.float64), axis=1)
     i1 = np.argmax(gates, axis=1)
     mask1 = np.eye(E, dtype=np.int64)[i1]
-    except1 = np.where(mask1.astype(bool), -np.inf, logits.astype(np.float64))
+    w_noise = logits if noise is None else (logits + noise).astype(np.float32)
+    except1 = np.where(mask1.astype(bool), -np.inf, w_noise.astype(np.float64))
     i2 = np.argmax(except1, axis=1)
     mask2 = np.eye(E, dtype=np.int64)[i2]
     loc1 = np.cumsum(mask1, axis=0) - 1
@@ -237,16 +239,21 @@ def dense_top2(logits, data, C):
     return cw, disp
 
 
+@pytest.mark.parametrize("noisy", [False, True])
 @pytest.mark.parametrize("S,E,cf,seed", [(48, 4, 1.0, 0), (64, 8, 0.5, 1), (40, 3, 2.0, 2)])
-def test_top2_matches_dense_gshard(S, E, cf, seed):
+def test_top2_matches_dense_gshard(S, E, cf, seed, noisy):
     M = 5
     data, logits = rng_case(seed, S, M, E)
     logits[:, 0] += 1.5   # a hot expert so that slot 1 and slot 2 both overflow
+    noise = np.random.default_rng(seed + 50).gumbel(size=(S, E)).astype(np.float32) if noisy else None
     C = int(np.ceil(2 * S / E * cf))
     assert C == mo.capacity(S, E, 2 * cf) or (2 * S / E * cf) != int(2 * S / E * cf)
     gates, il, used, elems, disp = mo.moe_encode_top2(data, logits, np.zeros(E, np.int32), cf,
-                                                      gate_is_logits=True, C=C)
-    cw, ddisp = dense_top2(logits, data, C)
+                                                      gate_is_logits=True, C=C, gate2_noise=noise)
+    cw, ddisp = dense_top2(logits, data, C, noise)
+    if noisy:   # the noise changes second choices, or the case pins nothing
+        plain = mo.select_topk(logits, 2, True)[0][1]
+        assert (mo.select_topk(logits, 2, True, noise)[0][1] != plain).any()
     mine = np.zeros((S, E, C))
     for j in range(2):
         for s in range(S):

@@ -235,6 +235,23 @@ def bench_config4_partitioned(ops, lib, capi, data, logits, S, M, E, cf, iters):
 
     t = {name: event_ms(fn, iters) for name, fn in (("encode_x8", encodes), ("merge_masks", merge),
                                                      ("redispatch", redispatch), ("decode", decode))}
+
+    # the same eight encodes writing straight into one shared buffer (rows behind those of the earlier
+    # calls, the last call zero-fills what is left): no redispatch pass
+    shared_outs = [o[:4] + (red,) for o in outs]
+
+    def encodes_shared():
+        used = zero
+        for i in range(2 * P):
+            ops.moe_encode(parts[i], gates[i], used, 2 * cf * P, zero_tail=(i == 2 * P - 1), rows_at_used=True,
+                           workspace=ws, out=shared_outs[i])
+            used = outs[i][2]
+
+    want_red = red.clone()
+    encodes_shared()
+    if not torch.equal(red, want_red):
+        raise RuntimeError("shared-buffer encodes differ from moe_redispatch")
+    t_shared = event_ms(encodes_shared, iters)
     kept = int((merged[0] >= 0).sum())
     b = data.element_size()
     # algorithmic bytes: partition encodes S*E*4 + S*M*b (each token row once per slot here: x2) + kept*M*b,
@@ -242,10 +259,19 @@ def bench_config4_partitioned(ops, lib, capi, data, logits, S, M, E, cf, iters):
     alg = (S * E * 4 + S * M * b + kept * M * b) + 2 * (2 * S) * 8 + (kept * M * b + E * Cap * M * b) + \
           (kept * M * b + S * M * b + 2 * S * 12)
     total = sum(t.values())
+    total_shared = t_shared + t["merge_masks"] + t["decode"]
+    alg_shared = (S * E * 4 + 2 * S * M * b + E * Cap * M * b) + 2 * (2 * S) * 8 + (kept * M * b + S * M * b + 2 * S * 12)
     return {"workload": "4 partitions x 2 slots -> merge_masks -> redispatch -> decode, S=%d M=%d E=%d C=%d" % (S, M, E, Cap),
             "ms": {k: round(v, 4) for k, v in t.items()}, "ms_total": round(total, 4),
             "tokens_per_s": round(S / (total * 1e-3), 1), "algorithmic_bytes": alg,
             "frac_of_hbm_peak": round(alg / (total * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "shared_buffer": {"what": "the eight encodes write into one [E,C,M] buffer at their final rows "
+                                      "(LANCET_ROWS_AT_USED), no redispatch pass; the buffer is verified equal",
+                              "ms": {"encode_x8": round(t_shared, 4), "merge_masks": round(t["merge_masks"], 4),
+                                     "decode": round(t["decode"], 4)},
+                              "ms_total": round(total_shared, 4), "tokens_per_s": round(S / (total_shared * 1e-3), 1),
+                              "algorithmic_bytes": alg_shared,
+                              "frac_of_hbm_peak": round(alg_shared / (total_shared * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
             "note": "token rows are read once per slot (two passes) in this call pattern; "
                     "partition encodes write used rows only (zero_tail=False), redispatch zero-fills the merged tail"}
 

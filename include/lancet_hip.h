@@ -63,6 +63,13 @@ extern "C" {
  * (tutel_moe_dispatch.cu:466), is spent on. */
 #define LANCET_NO_TAIL_ZERO 2u
 #define LANCET_ZERO_TAIL 4u /* lancet_memcpy_cont_to_sparse_3d: clear what the copy leaves untouched */
+/* lancet_moe_encode / lancet_moe_scatter: write the rows of expert e from row used_in[e] on instead of
+ * row 0, i.e. behind the rows that the calls chained before this one (through used_capacity) wrote into
+ * the same buffer; the zero-fill, if any, then covers rows [used_out[e], C).  Chained partition encodes
+ * that share one buffer this way leave it as moe_redispatch would build it from separate buffers
+ * (reference: redispatch_kernel, tutel_moe_dispatch.cu:365-408), without that second pass over the rows.
+ * indices_locations are unchanged (locations stay relative to the call, as moe_merge_masks expects). */
+#define LANCET_ROWS_AT_USED 8u
 
 typedef void* lancet_stream_t;
 

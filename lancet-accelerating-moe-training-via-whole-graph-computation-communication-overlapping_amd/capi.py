@@ -14,6 +14,7 @@ GATE_IS_LOGITS = 1
 NO_TAIL_ZERO = 2
 ABI_VERSION = 2
 ZERO_TAIL = 4
+ROWS_AT_USED = 8
 LANS_SWEEPS, LANS_RESIDENT = 0, 1
 MAX_EXPERTS = 512
 MAX_PARTITIONS = 64

@@ -126,7 +126,7 @@ extern "C" int lancet_launch_encode_forward(const int32_t* indices, const int32_
   // buffer is cleared first, as the reference launcher does
   hipError_t e = run_zero_bytes(dispatched, static_cast<size_t>(E) * C * M * eb, S_(stream));
   if (e != hipSuccess) return rc(e);
-  return rc(run_scatter_rows(data, dispatched, indices, locations, capused, nullptr, nullptr,
+  return rc(run_scatter_rows(data, dispatched, indices, locations, capused, nullptr, nullptr, nullptr,
                              static_cast<int>(S), static_cast<int>(M), static_cast<int>(E),
                              static_cast<int>(C), 1, eb, S_(stream)));
 }
@@ -172,8 +172,11 @@ extern "C" int lancet_moe_scatter(const void* data, const int32_t* indices_locat
     return LANCET_ERR_ALIGN;
   const int s = static_cast<int>(S);
   const bool tail = !(flags & LANCET_NO_TAIL_ZERO);
+  // rows of this call start at row 0 of every expert, or behind the rows earlier calls used
+  const bool at_used = (flags & LANCET_ROWS_AT_USED) != 0 && used_in != nullptr;
   return rc(run_scatter_rows(data, dispatched, indices_locations, indices_locations + static_cast<size_t>(top_k) * s,
-                             nullptr, tail ? used_in : nullptr, tail ? used_out : nullptr, s, static_cast<int>(M),
+                             nullptr, at_used ? used_in : nullptr, (tail && !at_used) ? used_in : nullptr,
+                             tail ? used_out : nullptr, s, static_cast<int>(M),
                              static_cast<int>(E), static_cast<int>(C), top_k, eb, S_(stream)));
 }
 
@@ -229,7 +232,7 @@ extern "C" int lancet_moe_encode_bpr(const void* data, const float* gate, int64_
                                loc, used_out, elements_per_expert, workspace, S_(stream));
   if (e != hipSuccess) return rc(e);
   const char* part = static_cast<const char*>(data) + static_cast<size_t>(partition_id) * s * M * eb;
-  return rc(run_scatter_rows(part, dispatched, idx, loc, nullptr, nullptr,
+  return rc(run_scatter_rows(part, dispatched, idx, loc, nullptr, nullptr, nullptr,
                              (flags & LANCET_NO_TAIL_ZERO) ? nullptr : used_out, s, static_cast<int>(M),
                              static_cast<int>(E), static_cast<int>(C), 1, eb, S_(stream)));
 }

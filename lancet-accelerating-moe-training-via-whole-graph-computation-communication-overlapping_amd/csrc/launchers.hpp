@@ -35,11 +35,13 @@ hipError_t run_top2_normalize(const float* raw, const int32_t* idx, int S, float
 
 // ---- row movers (moe_rows.hip) ------------------------------------------------------
 // Scatter of token rows into [E,C,M].  avail_used (may be null): only rows with
-// loc < C - avail_used[idx] are written (the reference's capused test).  When rows_hi is
+// loc < C - avail_used[idx] are written (the reference's capused test).  row_base (may be null):
+// location l of expert e goes to row row_base[e] + l instead of row l.  When rows_hi is
 // non-null the launch also zero-fills rows [rows_hi[e] - rows_lo[e], C) of every expert
 // (rows_lo may be null = zeros); otherwise the caller has cleared the buffer.
 hipError_t run_scatter_rows(const void* data, void* out, const int32_t* idx, const int32_t* loc,
-                            const int32_t* avail_used, const int32_t* rows_lo, const int32_t* rows_hi,
+                            const int32_t* avail_used, const int32_t* row_base, const int32_t* rows_lo,
+                            const int32_t* rows_hi,
                             int S, int M, int E, int C, int K, int elem_bytes, hipStream_t st);
 hipError_t run_zero_bytes(void* p, size_t nbytes, hipStream_t st);
 hipError_t run_decode_rows(const void* expert_out, const float* gates, const int32_t* idx,

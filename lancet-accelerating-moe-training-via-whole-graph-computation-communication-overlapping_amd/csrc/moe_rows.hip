@@ -35,6 +35,7 @@ struct ScatterArgs {
   const int32_t* idx;         // [K*S]
   const int32_t* loc;         // [K*S]
   const int32_t* avail_used;  // [E] or null
+  const int32_t* row_base;    // [E] or null: row of expert e that location 0 maps to
   const int32_t* rows_lo;     // [E] or null
   const int32_t* rows_hi;     // [E] or null (no tail fill)
   int S, E, C, K;
@@ -56,10 +57,14 @@ __global__ __launch_bounds__(kTile) void scatter_rows_kernel(ScatterArgs<V> a) {
 #pragma unroll
     for (int j = 0; j < K; ++j) {
       const int e = a.idx[static_cast<size_t>(j) * a.S + s];
-      const int l = a.loc[static_cast<size_t>(j) * a.S + s];
+      int l = a.loc[static_cast<size_t>(j) * a.S + s];
       bool ok = e >= 0 && e < a.E && l >= 0 && l < a.C;
       if (ok && a.avail_used) ok = l < a.C - a.avail_used[e];
       dst[j] = as_global(a.out);
+      if (ok && a.row_base) {
+        l += a.row_base[e];
+        ok = l < a.C;
+      }
       if (ok) dst[nd++] = as_global(a.out + (static_cast<size_t>(e) * a.C + l) * a.row_vecs);
     }
     if (nd == 0) return;
@@ -541,7 +546,7 @@ static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t
 
 template <typename V>
 static hipError_t scatter_launch(const void* data, void* out, const int32_t* idx, const int32_t* loc,
-                                 const int32_t* avail_used, const int32_t* rows_lo,
+                                 const int32_t* avail_used, const int32_t* row_base, const int32_t* rows_lo,
                                  const int32_t* rows_hi, int S, int E, int C, int K, int row_vecs,
                                  hipStream_t st) {
   ScatterArgs<V> a;
@@ -550,6 +555,7 @@ static hipError_t scatter_launch(const void* data, void* out, const int32_t* idx
   a.idx = idx;
   a.loc = loc;
   a.avail_used = avail_used;
+  a.row_base = row_base;
   a.rows_lo = rows_lo;
   a.rows_hi = rows_hi;
   a.S = S;
@@ -567,16 +573,17 @@ static hipError_t scatter_launch(const void* data, void* out, const int32_t* idx
 }
 
 hipError_t run_scatter_rows(const void* data, void* out, const int32_t* idx, const int32_t* loc,
-                            const int32_t* avail_used, const int32_t* rows_lo, const int32_t* rows_hi,
+                            const int32_t* avail_used, const int32_t* row_base, const int32_t* rows_lo,
+                            const int32_t* rows_hi,
                             int S, int M, int E, int C, int K, int elem_bytes, hipStream_t st) {
   const size_t row_bytes = static_cast<size_t>(M) * elem_bytes;
   if (row_bytes == 0) return hipSuccess;
   if (row_bytes % 16 == 0 && aligned16(data) && aligned16(out))
-    return scatter_launch<u32x4>(data, out, idx, loc, avail_used, rows_lo, rows_hi, S, E, C, K,
+    return scatter_launch<u32x4>(data, out, idx, loc, avail_used, row_base, rows_lo, rows_hi, S, E, C, K,
                                  static_cast<int>(row_bytes / 16), st);
   if (elem_bytes == 4)
-    return scatter_launch<uint32_t>(data, out, idx, loc, avail_used, rows_lo, rows_hi, S, E, C, K, M, st);
-  return scatter_launch<uint16_t>(data, out, idx, loc, avail_used, rows_lo, rows_hi, S, E, C, K, M, st);
+    return scatter_launch<uint32_t>(data, out, idx, loc, avail_used, row_base, rows_lo, rows_hi, S, E, C, K, M, st);
+  return scatter_launch<uint16_t>(data, out, idx, loc, avail_used, row_base, rows_lo, rows_hi, S, E, C, K, M, st);
 }
 
 hipError_t run_zero_bytes(void* p, size_t nbytes, hipStream_t st) {

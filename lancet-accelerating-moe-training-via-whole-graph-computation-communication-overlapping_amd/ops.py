@@ -67,8 +67,9 @@ def moe_encode_workspace_bytes(S, E, top_k=1):
     return int(capi.load().lancet_moe_encode_workspace_bytes(int(S), int(E), int(top_k)))
 
 
-def _flags(gate_is_logits, zero_tail):
-    return (capi.GATE_IS_LOGITS if gate_is_logits else 0) | (0 if zero_tail else capi.NO_TAIL_ZERO)
+def _flags(gate_is_logits, zero_tail, rows_at_used=False):
+    return ((capi.GATE_IS_LOGITS if gate_is_logits else 0) | (0 if zero_tail else capi.NO_TAIL_ZERO) |
+            (capi.ROWS_AT_USED if rows_at_used else 0))
 
 
 def _check_noise(gate2_noise, gate, top_k):
@@ -80,14 +81,16 @@ def _check_noise(gate2_noise, gate, top_k):
 
 
 def moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_logits=False,
-               zero_tail=True, gate2_noise=None, workspace=None, out=None):
+               zero_tail=True, gate2_noise=None, rows_at_used=False, workspace=None, out=None):
     """raf.op.moe_encode(data, gate, used_capacity, capacity_factor=1.0).
 
     Returns (gates_s [k*S] f32, indices_locations [2, k*S] i32, used_capacity [E] i32,
     elements_per_expert [E] u64, dispatched [E, C, M]).  With top_k = 2 the capacity follows
     GShard: capacity_factor is doubled before the reference formula is applied; gate2_noise [S, E], if
     given, is added to the gate for the second choice alone (the Gumbel noise of
-    docker/resources/sharded_moe.py:275, drawn by the caller).  zero_tail=False
+    docker/resources/sharded_moe.py:275, drawn by the caller).  rows_at_used=True writes the rows of expert e
+    from row used_capacity[e] on: chained partition encodes that pass the same `dispatched` buffer (out=) fill
+    it the way moe_redispatch would, the last one with zero_tail=True, the others without.  zero_tail=False
     leaves rows past the used capacity unwritten (partition buffers that only feed moe_redispatch)."""
     lib = capi.load()
     dt = _check_encode_inputs(data, gate)
@@ -113,7 +116,7 @@ def moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_
     ws_bytes = moe_encode_workspace_bytes(S, E, top_k)
     ws = _workspace(ws_bytes, dev, workspace)
     st = lib.lancet_moe_encode(_p(data), _p(gate), _p(gate2_noise), _p(used_capacity), S, M, E, Cap, top_k, dt,
-                               _flags(gate_is_logits, zero_tail), _p(gates_s), _p(indloc),
+                               _flags(gate_is_logits, zero_tail, rows_at_used), _p(gates_s), _p(indloc),
                                _p(used_out), _p(elems), _p(disp), _p(ws), ws.numel(), _stream())
     capi.check(st, "lancet_moe_encode")
     return gates_s, indloc, used_out, elems.view(torch.uint64) if elems.dtype == torch.int64 else elems, disp
@@ -144,7 +147,8 @@ def moe_route(gate, used_capacity, M, capacity_factor=1.0, top_k=1, gate_is_logi
     return gates_s, indloc, used_out, elems
 
 
-def moe_scatter(data, indices_locations, used_in, used_out, n_experts, capacity, top_k=1, zero_tail=True, out=None):
+def moe_scatter(data, indices_locations, used_in, used_out, n_experts, capacity, top_k=1, zero_tail=True,
+                rows_at_used=False, out=None):
     """The row-movement half of moe_encode (launch_encode_forward, moe.cc:381-395) on routing produced by
     moe_route: returns dispatched [E, C, M]."""
     lib = capi.load()
@@ -156,7 +160,8 @@ def moe_scatter(data, indices_locations, used_in, used_out, n_experts, capacity,
     if out is None:
         out = torch.empty((n_experts, capacity, M), dtype=data.dtype, device=data.device)
     st = lib.lancet_moe_scatter(_p(data), _p(indices_locations), _p(used_in), _p(used_out), S, M, int(n_experts),
-                                int(capacity), top_k, _dtype_code(data), _flags(False, zero_tail), _p(out), _stream())
+                                int(capacity), top_k, _dtype_code(data), _flags(False, zero_tail, rows_at_used), _p(out),
+                                _stream())
     capi.check(st, "lancet_moe_scatter")
     return out
 

@@ -501,3 +501,39 @@ def test_encode_top2_with_second_choice_noise(pkg, dt, is_logits):
     np.testing.assert_array_equal(to_np(outs[4]), want[4])
     with pytest.raises(ValueError):
         ops.moe_encode(d_x, d_gate, d_used, cf, top_k=1, gate2_noise=d_noise)
+
+
+# ----------------------------------------------------------------------------- partition encodes into one buffer
+@pytest.mark.parametrize("P,E,S0,M,dt", [(4, 8, 2048, 64, "f32"), (3, 5, 999, 24, "bf16"), (2, 2, 512, 8, "f32")])
+def test_chained_encodes_into_one_buffer_equal_redispatch(pkg, P, E, S0, M, dt):
+    """LANCET_ROWS_AT_USED: partition encodes chained through used_capacity write their rows behind those of
+    the earlier partitions, all into one [E, C, M] buffer, the last one zero-filling what is left.  The
+    buffer is bit for bit what moe_redispatch builds from separate partition buffers
+    (tests/python/op/cuda/test_cuda_moe.py:384-471 protocol), and also what one encode of the whole batch gives."""
+    ops = pkg.ops
+    S = S0 // P
+    S0 = S * P
+    cf = 0.75
+    data, logits = make_inputs(P + E, S0, M, E, zipf_bias=True)
+    gate = mo.softmax_rows(logits)
+    d_data, d_gate = rows_to_torch(data, dt), dev(gate)
+    Cap = ops.moe_capacity(S, E, cf * P)
+    shared = torch.full((E, Cap, M), 7.0, dtype=d_data.dtype, device="cuda")   # stale contents must not survive
+    used = torch.zeros(E, dtype=torch.int32, device="cuda")
+    ils, bufs = [], []
+    for p in range(P):
+        sl = slice(p * S, (p + 1) * S)
+        sep = ops.moe_encode(d_data[sl], d_gate[sl], used, cf * P)
+        outs = (torch.empty(S, device="cuda"), torch.empty((2, S), dtype=torch.int32, device="cuda"),
+                torch.empty(E, dtype=torch.int32, device="cuda"), torch.empty(E, dtype=torch.int64, device="cuda"), shared)
+        one = ops.moe_encode(d_data[sl], d_gate[sl], used, cf * P, zero_tail=(p == P - 1), rows_at_used=True, out=outs)
+        assert torch.equal(one[1], sep[1]) and torch.equal(one[2], sep[2])       # routing outputs are unchanged
+        ils.append(sep[1])
+        bufs.append(sep[4])
+        used = sep[2]
+    want = ops.moe_redispatch(bufs, ils)
+    assert torch.equal(shared, want)
+    assert (to_np(torch.stack(ils))[:, 0] < 0).any()                             # the case drops tokens
+    if ops.moe_capacity(S0, E, cf) == Cap:
+        whole = ops.moe_encode(d_data, d_gate, torch.zeros(E, dtype=torch.int32, device="cuda"), cf)
+        assert torch.equal(shared, whole[4])

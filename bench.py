@@ -118,7 +118,7 @@ def bench_lans(ops, capi, steps, warmup, scale, only_schedule=None):
             "algorithmic_GBps": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
             "bytes_per_param_algorithmic": 28,
             # HBM bytes per parameter measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this workload
-            "bytes_per_param_traffic_measured": {"sweeps": 52.0, "resident": 32.0},
+            "bytes_per_param_traffic_measured": {"sweeps": 48.0, "resident": 32.0},
             "steps": steps}
 
 

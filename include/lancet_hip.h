@@ -280,7 +280,7 @@ int lancet_lans_step(lancet_lans_plan_t plan, const float* const* g, float* cons
                      float* const* m, float* const* v, int step_host, const float* step_dev,
                      const lancet_lans_hyper* hyper, lancet_stream_t stream);
 /* Schedules of the step.  LANCET_LANS_SWEEPS (default): three whole-state sweeps with two per-tensor
- * reductions between them (52 B/param of traffic).  LANCET_LANS_RESIDENT: one persistent kernel that keeps
+ * reductions between them (48 B/param of traffic).  LANCET_LANS_RESIDENT: one persistent kernel that keeps
  * each chunk on chip between moments and update, after a sweep over g for its norm (32 B/param), for the tensors that fit on the chip at once
  * (lancet_lans_plan_resident_capacity) and the three sweeps, in the same step, for the larger ones; a plan
  * with no tensor that fits gets LANCET_ERR_SHAPE from set_schedule and keeps its schedule.  Each schedule is deterministic; the two agree to fp32 rounding of the per-chunk sums. */

@@ -1,12 +1,12 @@
 // Fused multi-tensor LANS step.  The reference makes six sweeps over the optimizer state
 // (src/op/dialect/cuda/kernels/multi_tensor_lans.cu:401-450: l2norm(g), l2norm(p), stage 1,
 // l2norm(u_m), l2norm(u_g), stage 2, 68 B/param of traffic).  Here the step has three phases
-//   phase 1  reads g, p            -> per-chunk sums of g^2 and p^2
-//   phase 2  reads g, p, m, v      -> writes m, v; per-chunk sums of u_m^2 and u_g^2
+//   phase 1  reads g               -> per-chunk sums of g^2
+//   phase 2  reads g, p, m, v      -> writes m, v; per-chunk sums of p^2, u_m^2 and u_g^2
 //   phase 3  reads g, p, m, v      -> recomputes u_m, u_g (never stored) and writes p
 // and two schedules:
 //   * sweeps (default): three plain launches + two tiny per-tensor reductions.  Real HBM traffic
-//     is 52 B/param (g, p read three times, m, v twice) and each sweep streams at the rate a plain
+//     is 48 B/param (g read three times, p, m, v twice) and each sweep streams at the rate a plain
 //     copy reaches on this chip.
 //   * resident (opt-in): a sweep over g alone for ||g|| (4 B/param), then ONE persistent kernel in
 //     which a workgroup takes a chunk through phases 2 and 3 and keeps it on chip in between (u_m and
@@ -47,7 +47,7 @@ struct LansTables {
   const int64_t* numel;        // [T]
   const int32_t* chunk_tensor; // [nchunks]
   const int32_t* tensor_first; // [T+1] first chunk of each tensor
-  float* partial;              // [2][nchunks]      (sweeps schedule)
+  float* partial;              // [3][nchunks]      (sweeps)
   uint64_t* part_word;         // [4][nchunks]      (resident schedule: epoch | fp32 sum of squares)
   uint64_t* norm_word;         // [4][T]            (resident schedule: epoch | fp32 norm)
   uint32_t* ticket;            // [1] next task; [1] error flag; [T] arrivals (resident schedule)
@@ -170,42 +170,35 @@ __device__ __forceinline__ void bias_corrections(const LansScalars& sc, float& b
 }
 
 // ---- the three phases on one chunk, executed by one workgroup ------------------------------
-// phase 1: sums of squares of g and p (L2NormFunctor, multi_tensor_lans.cu:95-167); valid on thread 0
-__device__ __forceinline__ void chunk_norm_gp(const LansTables& t, const ChunkView& c, float* s_red,
-                                              float& sum_g, float& sum_p) {
+// phase 1: sum of squares of g (L2NormFunctor, multi_tensor_lans.cu:95-167); valid on thread 0.
+// (The sum of squares of p is not needed before phase 3 and is taken in phase 2, which reads p anyway.)
+__device__ __forceinline__ float chunk_norm_g(const LansTables& t, const ChunkView& c, float* s_red) {
   const LANCET_GLOBAL float* g = as_global(t.g[c.tensor] + c.begin);
-  const LANCET_GLOBAL float* p = as_global(t.p[c.tensor] + c.begin);
-  float ag = 0.f, ap = 0.f;
+  float ag = 0.f;
   int scalar_from = 0;
-  if (vec_ok(g, p, g, p)) {
+  if (vec_ok(g, g, g, g)) {
     const int nv = c.n / 4;
     const LANCET_GLOBAL f32x4* g4 = (const LANCET_GLOBAL f32x4*)g;
-    const LANCET_GLOBAL f32x4* p4 = (const LANCET_GLOBAL f32x4*)p;
-#pragma unroll 4
+#pragma unroll 8
     for (int i = threadIdx.x; i < nv; i += kLansThreads) {
-      const f32x4 x = g4[i], y = p4[i];
+      const f32x4 x = g4[i];
       ag += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
-      ap += y.x * y.x + y.y * y.y + y.z * y.z + y.w * y.w;
     }
     scalar_from = nv * 4;
   }
-  for (int i = scalar_from + threadIdx.x; i < c.n; i += kLansThreads) {
-    ag += g[i] * g[i];
-    ap += p[i] * p[i];
-  }
-  sum_g = block_sum(ag, s_red);
-  sum_p = block_sum(ap, s_red);
+  for (int i = scalar_from + threadIdx.x; i < c.n; i += kLansThreads) ag += g[i] * g[i];
+  return block_sum(ag, s_red);
 }
 
-// phase 2: moments + sums of squares of the two updates (LANSStage1Functor :207-322 and the two
-// l2norm sweeps after it, :434-441); sums valid on thread 0
+// phase 2: moments + sums of squares of p and of the two updates (LANSStage1Functor :207-322 and the
+// l2norm sweeps around it, :428-441); sums valid on thread 0
 __device__ __forceinline__ void chunk_moments(const LansTables& t, const ChunkView& c, const LansElem& el,
-                                              float* s_red, float& sum_um, float& sum_ug) {
+                                              float* s_red, float& sum_p, float& sum_um, float& sum_ug) {
   const LANCET_GLOBAL float* g = as_global(t.g[c.tensor] + c.begin);
   const LANCET_GLOBAL float* p = as_global(t.p[c.tensor] + c.begin);
   LANCET_GLOBAL float* m = as_global(t.m[c.tensor] + c.begin);
   LANCET_GLOBAL float* v = as_global(t.v[c.tensor] + c.begin);
-  float am = 0.f, ag = 0.f;
+  float ap = 0.f, am = 0.f, ag = 0.f;
   int scalar_from = 0;
   if (vec_ok(g, p, m, v)) {
     const int nv = c.n / 4;
@@ -225,6 +218,7 @@ __device__ __forceinline__ void chunk_moments(const LansTables& t, const ChunkVi
         el.updates(sg, xp[k], mm, vv, um, ug);
         xm[k] = mm;
         xv[k] = vv;
+        ap += xp[k] * xp[k];
         am += um * um;
         ag += ug * ug;
       }
@@ -240,9 +234,11 @@ __device__ __forceinline__ void chunk_moments(const LansTables& t, const ChunkVi
     el.updates(sg, p[i], mm, vv, um, ug);
     m[i] = mm;
     v[i] = vv;
+    ap += p[i] * p[i];
     am += um * um;
     ag += ug * ug;
   }
+  sum_p = block_sum(ap, s_red);
   sum_um = block_sum(am, s_red);
   sum_ug = block_sum(ag, s_red);
 }
@@ -308,40 +304,13 @@ __global__ void lans_prepare_kernel(LansTables t, LansScalars sc) {
   if (threadIdx.x == 0 && blockIdx.x == 0) bias_corrections(sc, t.consts[0], t.consts[1]);
 }
 
-// The sweeps cover chunks [chunk_base, nchunks) and tensors [tensor_base, T): everything, or what the
-// resident kernel left (tensors too large for it).
-__global__ __launch_bounds__(kLansThreads) void lans_norm_gp_kernel(LansTables t, int chunk_base) {
+// The sweeps cover chunks [chunk_base, chunk_base + gridDim.x): all of them, or the ones the resident
+// kernel takes (first sweep only), or the ones it leaves (tensors too large for it).
+__global__ __launch_bounds__(kLansThreads) void lans_norm_g_kernel(LansTables t, int chunk_base) {
   __shared__ float s_red[kLansThreads / kWave];
   const int chunk = chunk_base + blockIdx.x;
-  const ChunkView c = chunk_view(t, chunk);
-  float sg, sp;
-  chunk_norm_gp(t, c, s_red, sg, sp);
-  if (threadIdx.x == 0) {
-    t.partial[chunk] = sg;
-    t.partial[t.nchunks + chunk] = sp;
-  }
-}
-
-// Sum g^2 alone over the chunks the resident kernel will take: it needs ||g|| when it starts a chunk
-__global__ __launch_bounds__(kLansThreads) void lans_norm_g_kernel(LansTables t) {
-  __shared__ float s_red[kLansThreads / kWave];
-  const ChunkView c = chunk_view(t, blockIdx.x);
-  const LANCET_GLOBAL float* g = as_global(t.g[c.tensor] + c.begin);
-  float ag = 0.f;
-  int scalar_from = 0;
-  if (vec_ok(g, g, g, g)) {
-    const int nv = c.n / 4;
-    const LANCET_GLOBAL f32x4* g4 = (const LANCET_GLOBAL f32x4*)g;
-#pragma unroll 8
-    for (int i = threadIdx.x; i < nv; i += kLansThreads) {
-      const f32x4 x = g4[i];
-      ag += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
-    }
-    scalar_from = nv * 4;
-  }
-  for (int i = scalar_from + threadIdx.x; i < c.n; i += kLansThreads) ag += g[i] * g[i];
-  ag = block_sum(ag, s_red);
-  if (threadIdx.x == 0) t.partial[blockIdx.x] = ag;
+  const float sg = chunk_norm_g(t, chunk_view(t, chunk), s_red);
+  if (threadIdx.x == 0) t.partial[chunk] = sg;
 }
 
 // per-tensor sqrt(sum of chunk partials) (cleanup, multi_tensor_lans.cu:169-185)
@@ -362,11 +331,12 @@ __global__ __launch_bounds__(kLansThreads) void lans_moments_kernel(LansTables t
   const int chunk = chunk_base + blockIdx.x;
   const ChunkView c = chunk_view(t, chunk);
   const LansElem el = make_elem(sc, t.norms[c.tensor], t.consts[0], t.consts[1]);
-  float sm, sg;
-  chunk_moments(t, c, el, s_red, sm, sg);
+  float sp, sm, sg;
+  chunk_moments(t, c, el, s_red, sp, sm, sg);
   if (threadIdx.x == 0) {
-    t.partial[chunk] = sm;
-    t.partial[t.nchunks + chunk] = sg;
+    t.partial[chunk] = sp;
+    t.partial[t.nchunks + chunk] = sm;
+    t.partial[2 * static_cast<size_t>(t.nchunks) + chunk] = sg;
   }
 }
 
@@ -559,10 +529,9 @@ __device__ __forceinline__ void resident_chunk(const LansTables& t, const LansSc
 // that wrote them).  At most one chunk per tensor takes this path when arrays are aligned.
 __device__ __forceinline__ void resident_chunk_streamed(const LansTables& t, const LansScalars& sc, const ChunkView& c,
                                                         int chunk, float bc1, float bc2, ResidentShared& sh) {
-  float sum_g, a0, a1, a2;
-  chunk_norm_gp(t, c, sh.red, sum_g, a0);
+  float a0, a1, a2;
   const LansElem el = make_elem(sc, t.norms[c.tensor], bc1, bc2);
-  chunk_moments(t, c, el, sh.red, a1, a2);
+  chunk_moments(t, c, el, sh.red, a0, a1, a2);
   if (threadIdx.x == 0) {
     st_word(t.part_word + 1 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a0);
     st_word(t.part_word + 2 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a1);
@@ -708,7 +677,7 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
   const size_t o_numel = off;     off = align_up(off + T * sizeof(int64_t), 256);
   const size_t o_ctensor = off;   off = align_up(off + (n ? n : 1) * sizeof(int32_t), 256);
   const size_t o_first = off;     off = align_up(off + (T + 1) * sizeof(int32_t), 256);
-  const size_t o_partial = off;   off = align_up(off + 2 * (n ? n : 1) * sizeof(float), 256);
+  const size_t o_partial = off;   off = align_up(off + 3 * (n ? n : 1) * sizeof(float), 256);
   const size_t o_norms = off;     off = align_up(off + 4 * T * sizeof(float), 256);
   const size_t o_consts = off;    off = align_up(off + 2 * sizeof(float), 256);
   const size_t o_words = off;     off = align_up(off + 4 * ((n ? n : 1) + T) * sizeof(uint64_t), 256);
@@ -871,7 +840,7 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
     if (err != hipSuccess) return static_cast<int>(err);
     const int grid = std::min(pl->resident_grid, pl->n_res_chunks);
     const int per_block = kLansThreads / kWave;
-    lans_norm_g_kernel<<<pl->n_res_chunks, kLansThreads, 0, st>>>(t);
+    lans_norm_g_kernel<<<pl->n_res_chunks, kLansThreads, 0, st>>>(t, 0);
     lans_reduce_kernel<<<(pl->n_res_tensors + per_block - 1) / per_block, kLansThreads, 0, st>>>(t, 0, 0, pl->n_res_tensors, 1);
     lans_resident_kernel<<<grid, kLansThreads, 0, st>>>(t, sc);
     chunk_base = pl->n_res_chunks;
@@ -882,10 +851,10 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
     const int per_block = kLansThreads / kWave;
     const int rblocks = (T - tensor_base + per_block - 1) / per_block;
     lans_prepare_kernel<<<1, 64, 0, st>>>(t, sc);
-    lans_norm_gp_kernel<<<nsweep, kLansThreads, 0, st>>>(t, chunk_base);
-    lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 0, tensor_base, T, 2);
+    lans_norm_g_kernel<<<nsweep, kLansThreads, 0, st>>>(t, chunk_base);
+    lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 0, tensor_base, T, 1);
     lans_moments_kernel<<<nsweep, kLansThreads, 0, st>>>(t, sc, chunk_base);
-    lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 2, tensor_base, T, 2);
+    lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 1, tensor_base, T, 3);
     lans_update_kernel<<<nsweep, kLansThreads, 0, st>>>(t, sc, chunk_base);
   }
   return static_cast<int>(hipGetLastError());

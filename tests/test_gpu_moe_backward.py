@@ -96,3 +96,73 @@ def test_backward_matches_autograd_through_forward_ops(pkg):
     (yr * Y.double()).sum().backward()
     torch.testing.assert_close(d_x.double(), xr.grad, rtol=1e-5, atol=1e-6)
     torch.testing.assert_close(d_gate.double(), gr.grad, rtol=1e-5, atol=1e-5)
+
+
+def _dense_layer(x, logits, W, il, C):
+    """The MoE layer in DeepSpeed's einsum form (docker/resources/sharded_moe.py:315-322 and the
+    'sec,sm->ecm' / 'sec,ecm->sm' products of MOELayer.forward), fp64, with the routing decisions
+    (expert, location of every kept token) taken as constants."""
+    S, E = logits.shape
+    gate = torch.softmax(logits, dim=1)
+    idx, loc = il[0].long(), il[1].long()
+    kept = idx >= 0
+    mask = torch.zeros((S, E, C), dtype=torch.float64, device=x.device)
+    mask[torch.arange(S, device=x.device)[kept], idx[kept], loc[kept]] = 1.0
+    gates_s = (gate * mask.sum(2)).sum(1)
+    disp = torch.einsum("sec,sm->ecm", mask, x)
+    expert_out = torch.tanh(torch.bmm(disp, W))
+    return torch.einsum("sec,ecm->sm", mask * gates_s[:, None, None], expert_out)
+
+
+@pytest.mark.parametrize("bpr", [False, True])
+def test_autograd_wiring_of_a_whole_layer(pkg, bpr):
+    """softmax -> moe_encode -> per-expert matmul + tanh -> moe_decode, differentiated by torch.autograd through
+    the gradient rules of src/op/grad/moe.cc, against the dense einsum form of the same layer in fp64."""
+    grad = pkg.grad
+    S, M, E = 384, 32, 6
+    data, logits_np = make_inputs(21, S, M, E, zipf_bias=True)
+    rng = np.random.default_rng(3)
+    W0 = dev((rng.standard_normal((E, M, M)) / np.sqrt(M)).astype(np.float32))
+    Y = dev(rng.standard_normal((S, M)).astype(np.float32))
+    x = dev(data).requires_grad_(True)
+    logits = dev(logits_np).requires_grad_(True)
+    W = W0.clone().requires_grad_(True)
+    gate = torch.softmax(logits, dim=1)
+    if bpr:
+        gates_s, il, used, elems, disp = grad.moe_encode_batch_prioritized(x, gate, 1, 0, 0.75)
+    else:
+        gates_s, il, used, elems, disp = grad.moe_encode(x, gate, None, 0.75)
+    assert not il.requires_grad and disp.requires_grad and gates_s.requires_grad
+    assert bool((il[0] < 0).any())                                   # some tokens are dropped
+    out = grad.moe_decode(torch.tanh(torch.bmm(disp, W)), gates_s, il)
+    (out * Y).sum().backward()
+
+    xr = x.detach().double().requires_grad_(True)
+    lr = logits.detach().double().requires_grad_(True)
+    Wr = W0.double().requires_grad_(True)
+    ref = _dense_layer(xr, lr, Wr, il, disp.shape[1])
+    torch.testing.assert_close(out.detach().double(), ref.detach(), rtol=1e-5, atol=1e-5)
+    (ref * Y.double()).sum().backward()
+    torch.testing.assert_close(x.grad.double(), xr.grad, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(logits.grad.double(), lr.grad, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(W.grad.double(), Wr.grad, rtol=1e-4, atol=1e-5)
+
+
+def test_autograd_wiring_of_a_prioritized_partition(pkg):
+    """moe_encode_batch_prioritized sees the whole batch and encodes one partition: the tokens of the other
+    partitions get zero gradient, the partition's own tokens the gradient of the plain rule."""
+    grad, ops = pkg.grad, pkg.ops
+    S0, M, E, P, pid = 512, 16, 4, 4, 2
+    data, logits_np = make_inputs(8, S0, M, E)
+    x = dev(data).requires_grad_(True)
+    gate = dev(mo.softmax_rows(logits_np)).requires_grad_(True)
+    gates_s, il, used, elems, disp = grad.moe_encode_batch_prioritized(x, gate, P, pid, 0.5)
+    wd, wg = torch.randn_like(disp), torch.randn_like(gates_s)
+    ((disp * wd).sum() + (gates_s * wg).sum()).backward()
+    S = S0 // P
+    own = slice(pid * S, (pid + 1) * S)
+    assert torch.equal(x.grad[own], ops.moe_encode_dx(wd, il))
+    assert torch.equal(gate.grad[own], ops.moe_encode_dg(wg, il, E))
+    rest = torch.ones(S0, dtype=torch.bool, device="cuda")
+    rest[own] = False
+    assert not bool(x.grad[rest].any()) and not bool(gate.grad[rest].any())

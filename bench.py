@@ -252,6 +252,32 @@ def bench_config4_partitioned(ops, lib, capi, data, logits, S, M, E, cf, iters):
     if not torch.equal(red, want_red):
         raise RuntimeError("shared-buffer encodes differ from moe_redispatch")
     t_shared = event_ms(encodes_shared, iters)
+
+    # the whole sequences in one timed region, launched op by op and replayed from a captured graph (no host
+    # work between launches: what a compiled caller sees)
+    def sequence():
+        encodes(), merge(), redispatch(), decode()
+
+    def sequence_shared():
+        encodes_shared(), merge(), decode()
+
+    def graph_ms(fn):
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fn()
+        torch.cuda.current_stream().wait_stream(side)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            fn()
+        g.replay()
+        return event_ms(g.replay, iters)
+
+    seq = {"ms_sequence": round(event_ms(sequence, iters), 4), "ms_graph_replay": round(graph_ms(sequence), 4)}
+    seq_shared = {"ms_sequence": round(event_ms(sequence_shared, iters), 4),
+                  "ms_graph_replay": round(graph_ms(sequence_shared), 4)}
+    if not torch.equal(red, want_red):
+        raise RuntimeError("graph replay of the shared-buffer encodes differs from moe_redispatch")
     kept = int((merged[0] >= 0).sum())
     b = data.element_size()
     # algorithmic bytes: partition encodes S*E*4 + S*M*b (each token row once per slot here: x2) + kept*M*b,
@@ -265,12 +291,15 @@ def bench_config4_partitioned(ops, lib, capi, data, logits, S, M, E, cf, iters):
             "ms": {k: round(v, 4) for k, v in t.items()}, "ms_total": round(total, 4),
             "tokens_per_s": round(S / (total * 1e-3), 1), "algorithmic_bytes": alg,
             "frac_of_hbm_peak": round(alg / (total * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "whole_sequence": dict(seq, frac_of_hbm_peak_graph=round(alg / (seq["ms_graph_replay"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)),
             "shared_buffer": {"what": "the eight encodes write into one [E,C,M] buffer at their final rows "
                                       "(LANCET_ROWS_AT_USED), no redispatch pass; the buffer is verified equal",
                               "ms": {"encode_x8": round(t_shared, 4), "merge_masks": round(t["merge_masks"], 4),
                                      "decode": round(t["decode"], 4)},
                               "ms_total": round(total_shared, 4), "tokens_per_s": round(S / (total_shared * 1e-3), 1),
                               "algorithmic_bytes": alg_shared,
+                              "whole_sequence": dict(seq_shared, frac_of_hbm_peak_graph=round(
+                                  alg_shared / (seq_shared["ms_graph_replay"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)),
                               "frac_of_hbm_peak": round(alg_shared / (total_shared * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
             "note": "token rows are read once per slot (two passes) in this call pattern; "
                     "partition encodes write used rows only (zero_tail=False), redispatch zero-fills the merged tail"}

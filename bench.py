@@ -278,6 +278,35 @@ def bench_config4_partitioned(ops, lib, capi, data, logits, S, M, E, cf, iters):
                   "ms_graph_replay": round(graph_ms(sequence_shared), 4)}
     if not torch.equal(red, want_red):
         raise RuntimeError("graph replay of the shared-buffer encodes differs from moe_redispatch")
+    # the same partitions with the batch routed once: one top-2 routing call over all S tokens (the gate is
+    # all it needs), then one scatter per partition straight to the final rows (each token row read once for
+    # both slots) and one decode per partition; no merge_masks, no redispatch
+    r_g = torch.empty(2 * S, device="cuda")
+    r_il = torch.empty((2, 2 * S), dtype=torch.int32, device="cuda")
+    r_used = torch.empty(E, dtype=torch.int32, device="cuda")
+    r_elems = torch.empty(E, dtype=torch.int64, device="cuda")
+    r_ws = torch.empty(ops.moe_encode_workspace_bytes(S, E, 2), dtype=torch.uint8, device="cuda")
+    r_buf = torch.full_like(red, 9.0)
+    r_dec = torch.empty_like(dec)
+
+    def routed_once():
+        ops.moe_route(logits, None, M, cf, top_k=2, gate_is_logits=True, workspace=r_ws, out=(r_g, r_il, r_used, r_elems))
+        for pi in range(P):
+            ops.moe_scatter_tokens(data[pi * Sp:(pi + 1) * Sp], r_il, None, r_used, pi * Sp, E, Cap, top_k=2,
+                                   zero_tail=(pi == P - 1), out=r_buf)
+        for pi in range(P):
+            ops.moe_decode_tokens(r_buf, r_g, r_il, pi * Sp, Sp, top_k=2, out=r_dec[pi * Sp:(pi + 1) * Sp])
+
+    routed_once()
+    if not torch.equal(r_buf, want_red):
+        raise RuntimeError("partition scatters of the once-routed batch differ from moe_redispatch")
+    if not torch.equal(r_il[0], merged[0]) or not torch.equal(r_il[1][merged[0] >= 0], merged[1][merged[0] >= 0]):
+        raise RuntimeError("whole-batch routing differs from the merged partition masks")
+    decode()
+    if not torch.equal(r_dec, dec):
+        raise RuntimeError("partition decodes of the once-routed batch differ from moe_decode")
+    seq_routed = {"ms_sequence": round(event_ms(routed_once, iters), 4), "ms_graph_replay": round(graph_ms(routed_once), 4)}
+
     kept = int((merged[0] >= 0).sum())
     b = data.element_size()
     # algorithmic bytes: partition encodes S*E*4 + S*M*b (each token row once per slot here: x2) + kept*M*b,
@@ -301,6 +330,14 @@ def bench_config4_partitioned(ops, lib, capi, data, logits, S, M, E, cf, iters):
                               "whole_sequence": dict(seq_shared, frac_of_hbm_peak_graph=round(
                                   alg_shared / (seq_shared["ms_graph_replay"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)),
                               "frac_of_hbm_peak": round(alg_shared / (total_shared * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
+            "routed_once": dict(seq_routed, what="one top-2 routing call over the whole batch, then one scatter and one "
+                                "decode per partition on token ranges of that routing (lancet_moe_scatter_tokens / "
+                                "_decode_tokens): rows go straight to their final places, each token row is read once; "
+                                "buffer, mask and output verified equal to the merged / redispatched ones",
+                                tokens_per_s=round(S / (seq_routed["ms_sequence"] * 1e-3), 1),
+                                algorithmic_bytes=alg_shared - S * M * b - 2 * (2 * S) * 8,
+                                frac_of_hbm_peak=round((alg_shared - S * M * b - 2 * (2 * S) * 8) /
+                                                       (seq_routed["ms_sequence"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)),
             "note": "token rows are read once per slot (two passes) in this call pattern; "
                     "partition encodes write used rows only (zero_tail=False), redispatch zero-fills the merged tail"}
 

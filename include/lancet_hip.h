@@ -162,6 +162,29 @@ int lancet_moe_decode(const void* expert_out, const float* gates_s,
                       const int32_t* indices_locations, int64_t S, int64_t M, int64_t E,
                       int64_t C, int top_k, int dtype, void* out, lancet_stream_t stream);
 
+/* ---- token ranges of a whole-batch mask -------------------------------------------------
+ * The partition pass cuts the token batch so that the exchange of one partition overlaps the work on
+ * another (src/pass/dist_optimization/partition_exprs.cc:1709-1795) and chains the partitions' encodes
+ * through used_capacity; the chained encodes, merged by moe_merge_masks, are by construction the routing
+ * of the whole batch (tests/python/op/cuda/test_cuda_moe.py:384-471).  Routing only needs the [S, E] gate,
+ * so a caller that has the gate of the whole batch routes once (lancet_moe_route, S = S_total) and then
+ * moves rows partition by partition with these two calls: tokens [token_first, token_first + n_tokens)
+ * of the whole-batch indices_locations [2, top_k * S_total] (and gates_s [top_k * S_total]).  data and
+ * out hold the rows of those tokens only ([n_tokens, M]); dispatched / expert_out is the whole [E, C, M]
+ * buffer, rows at their final places, so no moe_merge_masks / moe_redispatch pass is needed and each
+ * token row is read once also for top_k = 2.  lancet_moe_scatter_tokens zero-fills the rows
+ * past used_out - used_in (used_in, used_out as given to and returned by the routing call; used_in NULL =
+ * zeros) unless LANCET_NO_TAIL_ZERO is set: one call of the sequence should do it; both may be NULL with
+ * that flag.  The partitions' scatters together give bit for bit the buffer of one
+ * lancet_moe_encode over the batch. */
+int lancet_moe_scatter_tokens(const void* data, const int32_t* indices_locations, const int32_t* used_in,
+                              const int32_t* used_out, int64_t S_total, int64_t token_first, int64_t n_tokens, int64_t M, int64_t E,
+                              int64_t C, int top_k, int dtype, unsigned flags, void* dispatched,
+                              lancet_stream_t stream);
+int lancet_moe_decode_tokens(const void* expert_out, const float* gates_s, const int32_t* indices_locations,
+                             int64_t S_total, int64_t token_first, int64_t n_tokens, int64_t M, int64_t E,
+                             int64_t C, int top_k, int dtype, void* out, lancet_stream_t stream);
+
 /* ---- raf.op.moe_redispatch_expert_input ------------------------------------------------
  * Replaces MoeRedispatchExpertInput::Execute / launch_redispatch_expert_input (moe.cc:945-1073;
  * kernel_util.cuh:55; tutel_moe_dispatch.cu:436-456,586-598): merge, for one local expert, of the

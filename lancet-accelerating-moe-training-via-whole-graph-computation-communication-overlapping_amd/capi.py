@@ -54,6 +54,8 @@ SIGNATURES = {
     "lancet_moe_encode_bpr_workspace_bytes": (_sz, [_i64, _i64, _int]),
     "lancet_moe_encode_bpr": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _u32,
                                      _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "lancet_moe_scatter_tokens": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _u32, _vp, _vp]),
+    "lancet_moe_decode_tokens": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp]),
     "lancet_moe_decode": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp]),
     "lancet_moe_redispatch_expert_input": (_int, [C.POINTER(_vp), C.POINTER(_vp), _int, _int, _int, _i64, _i64, _i64,
                                                   _int, _int, _vp, _vp]),

@@ -198,6 +198,59 @@ extern "C" int lancet_moe_encode(const void* data, const float* gate, const floa
                             stream);
 }
 
+// ---- token ranges of a whole-batch mask ------------------------------------------------
+namespace {
+int check_range(int64_t S_total, int64_t token_first, int64_t n_tokens) {
+  if (S_total < 0 || S_total > 0x3fffffff || token_first < 0 || n_tokens < 0 || token_first > S_total ||
+      n_tokens > S_total - token_first)
+    return LANCET_ERR_SHAPE;
+  return LANCET_OK;
+}
+}  // namespace
+
+extern "C" int lancet_moe_scatter_tokens(const void* data, const int32_t* indices_locations, const int32_t* used_in,
+                                         const int32_t* used_out, int64_t S_total, int64_t token_first, int64_t n_tokens, int64_t M, int64_t E,
+                                         int64_t C, int top_k, int dtype, unsigned flags, void* dispatched,
+                                         lancet_stream_t stream) {
+  const bool tail = !(flags & LANCET_NO_TAIL_ZERO);
+  if ((!data && n_tokens > 0 && M > 0) || (!indices_locations && n_tokens > 0) || (tail && !used_out) ||
+      (!dispatched && C > 0 && M > 0))
+    return LANCET_ERR_NULL;
+  const int eb = elem_bytes(dtype);
+  if (!eb) return LANCET_ERR_DTYPE;
+  if (int r = check_dims(S_total, M, E, C)) return r;
+  if (int r = check_range(S_total, token_first, n_tokens)) return r;
+  if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
+  if (misaligned(data, eb) || misaligned(dispatched, eb) || misaligned(indices_locations, 4) ||
+      misaligned(used_in, 4) || misaligned(used_out, 4))
+    return LANCET_ERR_ALIGN;
+  const size_t st = static_cast<size_t>(S_total);
+  return rc(run_scatter_rows(data, dispatched, indices_locations + token_first,
+                             indices_locations + static_cast<size_t>(top_k) * st + token_first, nullptr, nullptr,
+                             tail ? used_in : nullptr, tail ? used_out : nullptr, static_cast<int>(n_tokens), static_cast<int>(M),
+                             static_cast<int>(E), static_cast<int>(C), top_k, eb, S_(stream), static_cast<int>(S_total)));
+}
+
+extern "C" int lancet_moe_decode_tokens(const void* expert_out, const float* gates_s, const int32_t* indices_locations,
+                                        int64_t S_total, int64_t token_first, int64_t n_tokens, int64_t M, int64_t E,
+                                        int64_t C, int top_k, int dtype, void* out, lancet_stream_t stream) {
+  if ((!expert_out && C > 0 && M > 0) || ((!gates_s || !indices_locations) && n_tokens > 0) ||
+      (!out && n_tokens > 0 && M > 0))
+    return LANCET_ERR_NULL;
+  const int eb = elem_bytes(dtype);
+  if (!eb) return LANCET_ERR_DTYPE;
+  if (int r = check_dims(S_total, M, E, C)) return r;
+  if (int r = check_range(S_total, token_first, n_tokens)) return r;
+  if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
+  if (misaligned(expert_out, eb) || misaligned(out, eb) || misaligned(gates_s, 4) || misaligned(indices_locations, 4))
+    return LANCET_ERR_ALIGN;
+  const size_t st = static_cast<size_t>(S_total);
+  return rc(run_decode_rows(expert_out, gates_s + token_first, indices_locations + token_first,
+                            indices_locations + static_cast<size_t>(top_k) * st + token_first, out,
+                            static_cast<int>(n_tokens), static_cast<int>(M), static_cast<int>(E), static_cast<int>(C),
+                            top_k, dtype, S_(stream), static_cast<int>(S_total)));
+}
+
 // ---- raf.op.moe_encode_batch_prioritized ----------------------------------------------
 extern "C" size_t lancet_moe_encode_bpr_workspace_bytes(int64_t S0, int64_t E, int n_partitions) {
   if (S0 < 0 || E < 1 || n_partitions < 1) return 0;

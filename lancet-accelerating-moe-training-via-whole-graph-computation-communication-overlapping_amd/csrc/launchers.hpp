@@ -38,15 +38,18 @@ hipError_t run_top2_normalize(const float* raw, const int32_t* idx, int S, float
 // loc < C - avail_used[idx] are written (the reference's capused test).  row_base (may be null):
 // location l of expert e goes to row row_base[e] + l instead of row l.  When rows_hi is
 // non-null the launch also zero-fills rows [rows_hi[e] - rows_lo[e], C) of every expert
-// (rows_lo may be null = zeros); otherwise the caller has cleared the buffer.
+// (rows_lo may be null = zeros); otherwise the caller has cleared the buffer.  slot_stride: distance
+// between the K slots of one token in idx / loc (and gates, for decode); negative = S.  A call that
+// moves a token range of a larger mask passes pointers to the range's first token and the mask's
+// token count here.
 hipError_t run_scatter_rows(const void* data, void* out, const int32_t* idx, const int32_t* loc,
                             const int32_t* avail_used, const int32_t* row_base, const int32_t* rows_lo,
                             const int32_t* rows_hi,
-                            int S, int M, int E, int C, int K, int elem_bytes, hipStream_t st);
+                            int S, int M, int E, int C, int K, int elem_bytes, hipStream_t st, int slot_stride = -1);
 hipError_t run_zero_bytes(void* p, size_t nbytes, hipStream_t st);
 hipError_t run_decode_rows(const void* expert_out, const float* gates, const int32_t* idx,
                            const int32_t* loc, void* out, int S, int M, int E, int C, int K,
-                           int dtype, hipStream_t st);
+                           int dtype, hipStream_t st, int slot_stride = -1);
 
 // backward (gates == nullptr in run_decode_rows gives moe_encode_dx)
 hipError_t run_encode_dg(const float* dy, const int32_t* idx, int S, int E, int K, float* grad_gates, hipStream_t st);

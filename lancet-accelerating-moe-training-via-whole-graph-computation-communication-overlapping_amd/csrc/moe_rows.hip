@@ -39,6 +39,8 @@ struct ScatterArgs {
   const int32_t* rows_lo;     // [E] or null
   const int32_t* rows_hi;     // [E] or null (no tail fill)
   int S, E, C, K;
+  int slot_stride;            // distance between the slots of one token in idx / loc (S, or the whole batch's
+                              // token count when this call moves a token range of a larger mask)
   int row_vecs;               // granules per row
   int token_blocks;
   int tail_chunks;            // tail workgroups per expert
@@ -56,8 +58,8 @@ __global__ __launch_bounds__(kTile) void scatter_rows_kernel(ScatterArgs<V> a) {
     int nd = 0;
 #pragma unroll
     for (int j = 0; j < K; ++j) {
-      const int e = a.idx[static_cast<size_t>(j) * a.S + s];
-      int l = a.loc[static_cast<size_t>(j) * a.S + s];
+      const int e = a.idx[static_cast<size_t>(j) * a.slot_stride + s];
+      int l = a.loc[static_cast<size_t>(j) * a.slot_stride + s];
       bool ok = e >= 0 && e < a.E && l >= 0 && l < a.C;
       if (ok && a.avail_used) ok = l < a.C - a.avail_used[e];
       dst[j] = as_global(a.out);
@@ -184,6 +186,7 @@ struct DecodeArgs {
   const int32_t* loc;    // [K*S]
   void* out;             // [S, M]
   int S, M, E, C;
+  int slot_stride;       // distance between the slots of one token in gates / idx / loc
 };
 
 template <int DT, int K, bool VEC>
@@ -199,10 +202,10 @@ __global__ __launch_bounds__(kTile) void decode_rows_kernel(DecodeArgs a) {
   bool any = false;
 #pragma unroll
   for (int j = 0; j < K; ++j) {
-    const int e = a.idx[static_cast<size_t>(j) * a.S + s];
-    const int l = a.loc[static_cast<size_t>(j) * a.S + s];
+    const int e = a.idx[static_cast<size_t>(j) * a.slot_stride + s];
+    const int l = a.loc[static_cast<size_t>(j) * a.slot_stride + s];
     ok[j] = e >= 0 && e < a.E && l >= 0 && l < a.C;
-    g[j] = ok[j] ? (a.gates ? a.gates[static_cast<size_t>(j) * a.S + s] : 1.f) : 0.f;
+    g[j] = ok[j] ? (a.gates ? a.gates[static_cast<size_t>(j) * a.slot_stride + s] : 1.f) : 0.f;
     row[j] = ok[j] ? (static_cast<size_t>(e) * a.C + l) : 0;
     any = any || ok[j];
   }
@@ -548,7 +551,7 @@ template <typename V>
 static hipError_t scatter_launch(const void* data, void* out, const int32_t* idx, const int32_t* loc,
                                  const int32_t* avail_used, const int32_t* row_base, const int32_t* rows_lo,
                                  const int32_t* rows_hi, int S, int E, int C, int K, int row_vecs,
-                                 hipStream_t st) {
+                                 int slot_stride, hipStream_t st) {
   ScatterArgs<V> a;
   a.data = static_cast<const V*>(data);
   a.out = static_cast<V*>(out);
@@ -562,6 +565,7 @@ static hipError_t scatter_launch(const void* data, void* out, const int32_t* idx
   a.E = E;
   a.C = C;
   a.K = K;
+  a.slot_stride = slot_stride;
   a.row_vecs = row_vecs;
   a.token_blocks = (S + kRowsPerBlock - 1) / kRowsPerBlock;
   a.tail_chunks = rows_hi ? (C + kTailRows - 1) / kTailRows : 0;
@@ -575,15 +579,16 @@ static hipError_t scatter_launch(const void* data, void* out, const int32_t* idx
 hipError_t run_scatter_rows(const void* data, void* out, const int32_t* idx, const int32_t* loc,
                             const int32_t* avail_used, const int32_t* row_base, const int32_t* rows_lo,
                             const int32_t* rows_hi,
-                            int S, int M, int E, int C, int K, int elem_bytes, hipStream_t st) {
+                            int S, int M, int E, int C, int K, int elem_bytes, hipStream_t st, int slot_stride) {
   const size_t row_bytes = static_cast<size_t>(M) * elem_bytes;
   if (row_bytes == 0) return hipSuccess;
+  const int ss = slot_stride < 0 ? S : slot_stride;
   if (row_bytes % 16 == 0 && aligned16(data) && aligned16(out))
     return scatter_launch<u32x4>(data, out, idx, loc, avail_used, row_base, rows_lo, rows_hi, S, E, C, K,
-                                 static_cast<int>(row_bytes / 16), st);
+                                 static_cast<int>(row_bytes / 16), ss, st);
   if (elem_bytes == 4)
-    return scatter_launch<uint32_t>(data, out, idx, loc, avail_used, row_base, rows_lo, rows_hi, S, E, C, K, M, st);
-  return scatter_launch<uint16_t>(data, out, idx, loc, avail_used, row_base, rows_lo, rows_hi, S, E, C, K, M, st);
+    return scatter_launch<uint32_t>(data, out, idx, loc, avail_used, row_base, rows_lo, rows_hi, S, E, C, K, M, ss, st);
+  return scatter_launch<uint16_t>(data, out, idx, loc, avail_used, row_base, rows_lo, rows_hi, S, E, C, K, M, ss, st);
 }
 
 hipError_t run_zero_bytes(void* p, size_t nbytes, hipStream_t st) {
@@ -622,7 +627,7 @@ static hipError_t decode_launch(const DecodeArgs& a, int K, bool vec, hipStream_
 
 hipError_t run_decode_rows(const void* expert_out, const float* gates, const int32_t* idx,
                            const int32_t* loc, void* out, int S, int M, int E, int C, int K,
-                           int dtype, hipStream_t st) {
+                           int dtype, hipStream_t st, int slot_stride) {
   DecodeArgs a;
   a.expert_out = expert_out;
   a.gates = gates;
@@ -633,6 +638,7 @@ hipError_t run_decode_rows(const void* expert_out, const float* gates, const int
   a.M = M;
   a.E = E;
   a.C = C;
+  a.slot_stride = slot_stride < 0 ? S : slot_stride;
   const int per_vec = (dtype == LANCET_F32) ? 4 : 8;
   const bool vec = (M % per_vec == 0) && aligned16(expert_out) && aligned16(out);
   switch (dtype) {

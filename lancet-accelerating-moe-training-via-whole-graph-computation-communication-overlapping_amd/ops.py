@@ -166,6 +166,47 @@ def moe_scatter(data, indices_locations, used_in, used_out, n_experts, capacity,
     return out
 
 
+def moe_scatter_tokens(data, indices_locations, used_in, used_out, token_first, n_experts, capacity, top_k=1,
+                       zero_tail=True, out=None):
+    """Row movement of tokens [token_first, token_first + len(data)) of a whole-batch routing
+    (moe_route over all S_total tokens): data holds the rows of those tokens, `out` is the whole [E, C, M]
+    buffer and the rows go to their final places.  The calls of all token ranges together give the buffer of
+    one moe_encode over the batch; one of them passes zero_tail=True, the others False.  used_in / used_out are
+    what the routing call took and returned (used_in None = zeros)."""
+    lib = capi.load()
+    _dev(data, "data")
+    _need(data.dim() == 2, "Expected input data to be 2D.")
+    S_total = _check_indloc(indices_locations, top_k)
+    n, M = data.shape
+    _need(0 <= token_first and token_first + n <= S_total, "token range outside the routed batch")
+    if out is None:
+        out = torch.empty((n_experts, capacity, M), dtype=data.dtype, device=data.device)
+    st = lib.lancet_moe_scatter_tokens(_p(data), _p(indices_locations), _p(used_in), _p(used_out), S_total, int(token_first), n, M,
+                                       int(n_experts), int(capacity), top_k, _dtype_code(data),
+                                       _flags(False, zero_tail), _p(out), _stream())
+    capi.check(st, "lancet_moe_scatter_tokens")
+    return out
+
+
+def moe_decode_tokens(data, gate, indices_locations, token_first, n_tokens, top_k=1, out=None):
+    """moe_decode of tokens [token_first, token_first + n_tokens) of a whole-batch routing: gate [k*S_total] and
+    indices_locations [2, k*S_total] cover the batch, the result is [n_tokens, M]."""
+    lib = capi.load()
+    _dev(data, "data"), _dev(gate, "gate")
+    _need(data.dim() == 3, "Expected input data to be 3D.")
+    _need(gate.dim() == 1 and gate.dtype == torch.float32, "gate must be 1-D float32")
+    S_total = _check_indloc(indices_locations, top_k)
+    _need(gate.shape[0] == top_k * S_total, "gate and indices_locations disagree on the token count")
+    _need(0 <= token_first and 0 <= n_tokens and token_first + n_tokens <= S_total, "token range outside the routed batch")
+    E, Cap, M = data.shape
+    if out is None:
+        out = torch.empty((n_tokens, M), dtype=data.dtype, device=data.device)
+    st = lib.lancet_moe_decode_tokens(_p(data), _p(gate), _p(indices_locations), S_total, int(token_first),
+                                      int(n_tokens), M, E, Cap, top_k, _dtype_code(data), _p(out), _stream())
+    capi.check(st, "lancet_moe_decode_tokens")
+    return out
+
+
 def moe_encode_bpr_workspace_bytes(S0, E, n_partitions=1):
     return int(capi.load().lancet_moe_encode_bpr_workspace_bytes(int(S0), int(E), int(n_partitions)))
 

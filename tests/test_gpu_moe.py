@@ -537,3 +537,42 @@ def test_chained_encodes_into_one_buffer_equal_redispatch(pkg, P, E, S0, M, dt):
     if ops.moe_capacity(S0, E, cf) == Cap:
         whole = ops.moe_encode(d_data, d_gate, torch.zeros(E, dtype=torch.int32, device="cuda"), cf)
         assert torch.equal(shared, whole[4])
+
+
+# ----------------------------------------------------------------------------- token ranges of a whole-batch routing
+@pytest.mark.parametrize("k,dt,P,S,M,E", [(2, "bf16", 4, 2048, 64, 8), (1, "f32", 3, 999, 24, 5), (2, "f32", 2, 512, 5, 4),
+                                          (2, "f16", 5, 1000, 40, 16)])
+@pytest.mark.parametrize("with_used_in", [False, True])
+def test_token_range_scatter_and_decode_equal_the_whole_batch(pkg, k, dt, P, S, M, E, with_used_in):
+    """Route the whole batch once, then move rows range by range (lancet_moe_scatter_tokens /
+    lancet_moe_decode_tokens): the buffer is bit for bit the one moe_encode builds for the batch (itself checked
+    against the oracle), stale contents of the shared buffer do not survive, and the ranges' decodes are the
+    rows of the whole-batch decode."""
+    ops = pkg.ops
+    cf = 0.75
+    data, logits = make_inputs(S + k, S, M, E, zipf_bias=True)
+    gate = mo.softmax_rows(logits)
+    d_data, d_gate = rows_to_torch(data, dt), dev(gate)
+    used_in = dev(np.arange(E, dtype=np.int32) % 3) if with_used_in else None
+    g, il, used, elems, disp = ops.moe_encode(d_data, d_gate, used_in, cf, top_k=k)
+    want_rows = mo.moe_encode_top2 if k == 2 else mo.moe_encode
+    ref = want_rows(rows_as_oracle(data, dt), gate, to_np(used_in) if with_used_in else np.zeros(E, np.int32), cf)
+    np.testing.assert_array_equal(to_np(disp), ref[4])
+    assert (to_np(il)[0] < 0).any()
+    C = disp.shape[1]
+    shared = torch.full_like(disp, 5.0)
+    bounds = [S * p // P for p in range(P + 1)]
+    bounds[1] += 1                                   # ranges of unequal length, one of them odd
+    for p in range(P):
+        lo, hi = bounds[p], bounds[p + 1]
+        ops.moe_scatter_tokens(d_data[lo:hi], il, used_in, used, lo, E, C, top_k=k, zero_tail=(p == 1), out=shared)
+    assert torch.equal(shared, disp)
+    whole = ops.moe_decode(disp, g, il, top_k=k)
+    for p in range(P):
+        lo, hi = bounds[p], bounds[p + 1]
+        part = ops.moe_decode_tokens(shared, g, il, lo, hi - lo, top_k=k)
+        assert torch.equal(part, whole[lo:hi])
+    empty = ops.moe_decode_tokens(shared, g, il, S, 0, top_k=k)
+    assert empty.shape == (0, M)
+    with pytest.raises(ValueError):
+        ops.moe_decode_tokens(shared, g, il, S - 1, 2, top_k=k)

@@ -302,6 +302,10 @@ int lancet_lans_plan_destroy(lancet_lans_plan_t plan);
 int lancet_lans_step(lancet_lans_plan_t plan, const float* const* g, float* const* p,
                      float* const* m, float* const* v, int step_host, const float* step_dev,
                      const lancet_lans_hyper* hyper, lancet_stream_t stream);
+/* A step may be recorded into a HIP graph (either schedule): with step_dev the step number is read on the
+ * device, and everything else that changes from step to step lives in the plan's device memory, so each
+ * replay is a new step.  The pointer tables are uploaded (one host-to-device copy) by the first call that
+ * sees a new set of pointers: make that call once before recording. */
 /* Schedules of the step.  LANCET_LANS_SWEEPS (default): three whole-state sweeps with two per-tensor
  * reductions between them (48 B/param of traffic).  LANCET_LANS_RESIDENT: one persistent kernel that keeps
  * each chunk on chip between moments and update, after a sweep over g for its norm (32 B/param), for the tensors that fit on the chip at once

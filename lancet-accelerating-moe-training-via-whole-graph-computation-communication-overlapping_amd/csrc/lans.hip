@@ -50,7 +50,7 @@ struct LansTables {
   float* partial;              // [3][nchunks]      (sweeps)
   uint64_t* part_word;         // [4][nchunks]      (resident schedule: epoch | fp32 sum of squares)
   uint64_t* norm_word;         // [4][T]            (resident schedule: epoch | fp32 norm)
-  uint32_t* ticket;            // [1] next task; [1] error flag; [T] arrivals (resident schedule)
+  uint32_t* ticket;            // [1] next task; [1] error flag; [T] arrivals; [1] step epoch (resident schedule)
   float* norms;                // [4][T]: g, p, u_m, u_g
   float* consts;               // [2]: bias_correction1, bias_correction2
   const int32_t* order;        // [T] position in the caller's lists of the plan's i-th tensor
@@ -64,7 +64,7 @@ struct LansScalars {
   int mode, normalize_grad, bias_correction;
   int step_host;
   const float* step_dev;
-  uint32_t epoch;
+  uint32_t epoch;              // filled in on the device (the word behind the arrival counters)
   uint32_t spin_limit;
 };
 
@@ -550,8 +550,26 @@ __device__ __forceinline__ void resident_chunk_streamed(const LansTables& t, con
 // what the 36 KB of LDS per workgroup allows: 1024 chunks on 256 CUs, two of the largest supported
 // tensors at once, so that memory stays busy while the workgroups of one tensor wait.
 constexpr int kResidentWavesPerSimd = 4;
+
+// Start of a resident step: clears the ticket, the error flag and the arrival counters and moves the
+// step epoch on.  The epoch lives on the device so that a step recorded in a graph tags every replay
+// differently; when it wraps (2^32 steps) every word of earlier steps is forgotten.
+__global__ __launch_bounds__(kLansThreads) void lans_begin_kernel(LansTables t, size_t nwords) {
+  const size_t i = blockIdx.x * static_cast<size_t>(kLansThreads) + threadIdx.x;
+  if (i < 2 + static_cast<size_t>(t.T)) t.ticket[i] = 0u;
+  if (blockIdx.x == 0) {
+    uint32_t* ep = t.ticket + 2 + t.T;
+    const uint32_t e = *ep + 1u;
+    if (e == 0u)
+      for (size_t k = threadIdx.x; k < nwords; k += kLansThreads) t.part_word[k] = 0;  // norm words follow
+    __syncthreads();
+    if (threadIdx.x == 0) *ep = e == 0u ? 1u : e;
+  }
+}
+
 __global__ __launch_bounds__(kLansThreads, kResidentWavesPerSimd) void lans_resident_kernel(LansTables t, LansScalars sc) {
   __shared__ ResidentShared sh;
+  sc.epoch = __builtin_amdgcn_readfirstlane(t.ticket[2 + t.T]);
   float bc1, bc2;
   bias_corrections(sc, bc1, bc2);
   while (true) {
@@ -595,7 +613,6 @@ struct lancet_lans_plan {
   int n_res_tensors;      // tensors within that limit: the first ones in the plan's own order
   int n_res_chunks;
   std::vector<int32_t> order;  // plan position -> position in the caller's lists
-  uint32_t epoch;         // step counter that tags the words of the resident schedule
   size_t words_offset; // part_word + norm_word inside dev_block
   size_t words_bytes;
 };
@@ -681,10 +698,9 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
   const size_t o_norms = off;     off = align_up(off + 4 * T * sizeof(float), 256);
   const size_t o_consts = off;    off = align_up(off + 2 * sizeof(float), 256);
   const size_t o_words = off;     off = align_up(off + 4 * ((n ? n : 1) + T) * sizeof(uint64_t), 256);
-  const size_t o_ticket = off;    off = align_up(off + (2 + static_cast<size_t>(T)) * sizeof(uint32_t), 256);
+  const size_t o_ticket = off;    off = align_up(off + (3 + static_cast<size_t>(T)) * sizeof(uint32_t), 256);
   const size_t o_order = off;     off = align_up(off + T * sizeof(int32_t), 256);
   pl->schedule = LANCET_LANS_SWEEPS;
-  pl->epoch = 0;
   pl->words_offset = o_words;
   pl->words_bytes = 4 * ((n ? n : 1) + T) * sizeof(uint64_t);
   int cus = 256;
@@ -716,7 +732,7 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
     if (err == hipSuccess) err = hipMemcpy(base + o_first, first.data(), (T + 1) * sizeof(int32_t), hipMemcpyHostToDevice);
     if (err == hipSuccess) err = hipMemset(base + o_norms, 0, 4 * T * sizeof(float));
     if (err == hipSuccess) err = hipMemset(base + o_words, 0, pl->words_bytes);
-    if (err == hipSuccess) err = hipMemset(base + o_ticket, 0, (2 + static_cast<size_t>(T)) * sizeof(uint32_t));
+    if (err == hipSuccess) err = hipMemset(base + o_ticket, 0, (3 + static_cast<size_t>(T)) * sizeof(uint32_t));
     LansTables& t = pl->tables;
     t.part_word = reinterpret_cast<uint64_t*>(base + o_words);
     t.norm_word = t.part_word + 4 * (n ? n : 1);
@@ -830,14 +846,8 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
   int chunk_base = 0, tensor_base = 0;
   sc.epoch = 0;
   if (pl->schedule == LANCET_LANS_RESIDENT && pl->n_res_chunks > 0) {
-    if (++pl->epoch == 0) {  // tag wrapped: forget every word of earlier steps
-      err = hipMemsetAsync(static_cast<char*>(pl->dev_block) + pl->words_offset, 0, pl->words_bytes, st);
-      if (err != hipSuccess) return static_cast<int>(err);
-      pl->epoch = 1;
-    }
-    sc.epoch = pl->epoch;
-    err = run_fill_u32(t.ticket, 2 + static_cast<size_t>(T), 0u, st);
-    if (err != hipSuccess) return static_cast<int>(err);
+    const unsigned begin_blocks = static_cast<unsigned>((2 + static_cast<size_t>(T) + kLansThreads - 1) / kLansThreads);
+    lans_begin_kernel<<<begin_blocks, kLansThreads, 0, st>>>(t, pl->words_bytes / sizeof(uint64_t));
     const int grid = std::min(pl->resident_grid, pl->n_res_chunks);
     const int per_block = kLansThreads / kWave;
     lans_norm_g_kernel<<<pl->n_res_chunks, kLansThreads, 0, st>>>(t, 0);

@@ -276,3 +276,20 @@ def test_missing_library_is_an_error_not_a_fallback(pkg, monkeypatch, tmp_path):
         pkg.ops.moe_capacity(16, 4, 1.0)
     src = open(os.path.join(os.path.dirname(capi.__file__), "ops.py")).read()
     assert "oracle" not in src and "numpy" not in src          # the operator layer never imports the checker
+
+
+def test_header_is_plain_c_and_the_c_client_links():
+    """include/lancet_hip.h must compile as C99 and as C++11 on its own; the C client under tests/c_client
+    builds against the in-tree library with gcc (it runs in the GPU tests)."""
+    import shutil
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    hdr = os.path.join(root, "include", "lancet_hip.h")
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-x", "c", hdr], check=True)
+    subprocess.run(["g++", "-std=c++11", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-x", "c++", hdr],
+                   check=True)
+    if not os.path.isdir("/opt/rocm/include"):
+        pytest.skip("HIP runtime headers are not installed")
+    build_dir = os.path.join(root, "tests", "c_client")
+    subprocess.run(["make", "-C", build_dir, "-B"], check=True, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
+    assert os.path.exists(os.path.join(build_dir, "lancet_client")) and shutil.which("gcc")

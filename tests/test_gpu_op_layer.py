@@ -86,3 +86,15 @@ def test_executor_reports_op_errors(pkg, ex):
            torch.zeros(2, dtype=torch.int32, device="cuda"), 1.0)
     with pytest.raises(pkg.raf_executor.RafError, match="float32"):
         ex("raf.op.lans", [torch.zeros(4, device="cuda", dtype=torch.float16)] * 4, 1, 1e-3, 0.9, 0.999, 1e-6, 1, 0.01, 1, 1, True)
+
+
+def test_plain_c_client_of_the_c_abi():
+    """tests/c_client/lancet_client.c: a C99 program that links the library and the HIP runtime only (no
+    Python, no torch) and checks encode + decode on a hand-computed case."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "c_client", "lancet_client")
+    assert os.path.exists(exe), "run __graft_entry__.build() (or make -C tests/c_client) first"
+    proc = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=100)
+    assert proc.returncode == 0, proc.stdout
+    assert "match the hand-computed case" in proc.stdout

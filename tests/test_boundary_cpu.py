@@ -68,6 +68,16 @@ def test_workspace_sizes_and_argument_rejection(pkg):
     assert lib.lancet_memcpy_cont_to_sparse_3d(one, None, one, 8, 1, 0, 0, 4, 4, 4, 64, 1, 1, capi.F32, 0, None) == capi.ERR_NULL
     assert lib.lancet_memcpy_cont_to_sparse_3d(one, one, C.c_void_p(12), 8, 1, 0, 1, 4, 4, 4, 64, 1, 1, capi.BF16, 0, None) == capi.ERR_ALIGN
     assert lib.lancet_memcpy_cont_to_sparse_3d(one, one, one, 8, 1, 0, 1, 4, 0, 4, 64, 1, 1, capi.BF16, 0, None) == capi.OK
+    # token ranges of a whole-batch routing: the range must lie inside the batch
+    sc, dc = lib.lancet_moe_scatter_tokens, lib.lancet_moe_decode_tokens
+    assert sc(one, one, None, one, 64, 60, 8, 4, 2, 4, 1, capi.F32, 0, one, None) == capi.ERR_SHAPE
+    assert sc(one, one, None, one, 64, -1, 8, 4, 2, 4, 1, capi.F32, 0, one, None) == capi.ERR_SHAPE
+    assert sc(one, one, None, None, 64, 0, 8, 4, 2, 4, 1, capi.F32, 0, one, None) == capi.ERR_NULL   # tail fill needs used_out
+    assert sc(one, one, None, one, 64, 0, 8, 4, 2, 4, 3, capi.F32, 0, one, None) == capi.ERR_TOPK
+    assert sc(one, one, None, one, 64, 0, 8, 4, 2, 4, 1, 7, 0, one, None) == capi.ERR_DTYPE
+    assert dc(one, one, one, 64, 57, 8, 4, 2, 4, 1, capi.F32, one, None) == capi.ERR_SHAPE
+    assert dc(one, None, one, 64, 0, 8, 4, 2, 4, 1, capi.F32, one, None) == capi.ERR_NULL
+    assert dc(one, one, one, 64, 0, 8, 4, 2, 4, 1, capi.F32, C.c_void_p(6), None) == capi.ERR_ALIGN
     assert lib.lancet_lans_plan_destroy(None) == capi.ERR_PLAN
     assert "workspace" in capi.status_string(capi.ERR_WORKSPACE)
 

@@ -576,3 +576,53 @@ def test_token_range_scatter_and_decode_equal_the_whole_batch(pkg, k, dt, P, S, 
     assert empty.shape == (0, M)
     with pytest.raises(ValueError):
         ops.moe_decode_tokens(shared, g, il, S - 1, 2, top_k=k)
+
+
+# ----------------------------------------------------------------------------- non-finite gates
+@pytest.mark.parametrize("mode", ["top1", "top2", "bpr"])
+@pytest.mark.parametrize("is_logits", [False, True])
+def test_non_finite_gates_keep_the_outputs_well_formed(pkg, mode, is_logits):
+    """NaN and infinities in the gate: which expert such a token goes to is not pinned by anything the
+    reference holds, but the outputs must stay well formed: experts in range, kept locations below the
+    capacity and distinct per expert, counts consistent, rows copied bit for bit, no bounded wait tripped;
+    tokens whose row is finite route exactly as in a batch without the bad rows' values."""
+    ops = pkg.ops
+    S, M, E, cf = 3000, 16, 8, 0.6
+    data, logits = make_inputs(77, S, M, E)
+    rng = np.random.default_rng(5)
+    bad = rng.random(S) < 0.2
+    vals = np.array([np.nan, np.inf, -np.inf], np.float32)
+    poisoned = logits.copy()
+    for s in np.nonzero(bad)[0]:
+        k = rng.integers(1, E + 1)
+        poisoned[s, rng.choice(E, k, replace=False)] = vals[rng.integers(0, 3, k)]
+    d_data = dev(data)
+    if mode == "bpr":
+        g, il, used, elems, disp = ops.moe_encode_batch_prioritized(d_data, dev(poisoned), 1, 0, cf, gate_is_logits=is_logits)
+        k = 1
+    else:
+        k = 2 if mode == "top2" else 1
+        g, il, used, elems, disp = ops.moe_encode(d_data, dev(poisoned), None, cf, top_k=k, gate_is_logits=is_logits)
+    torch.cuda.synchronize()
+    il, used, elems, disp = to_np(il), to_np(used), to_np(elems), to_np(disp)
+    C = disp.shape[1]
+    idx, loc = il[0], il[1]
+    assert idx.min() >= -1 and idx.max() < E
+    kept = idx >= 0
+    assert (loc[kept] >= 0).all() and (loc[kept] < C).all()
+    slots = idx[kept].astype(np.int64) * C + loc[kept]
+    assert np.unique(slots).size == slots.size
+    counts = np.bincount(idx[kept], minlength=E)
+    np.testing.assert_array_equal(counts, used)
+    np.testing.assert_array_equal(elems, used.astype(np.uint64) * M)
+    for e in range(E):                                  # locations of an expert are exactly 0 .. used-1
+        assert set(loc[kept & (idx == e)]) == set(range(used[e]))
+    tok = np.tile(np.arange(S), k)
+    np.testing.assert_array_equal(disp[idx[kept], loc[kept]], data[tok[kept]])
+    assert not disp.reshape(E * C, M)[np.setdiff1d(np.arange(E * C), slots)].any()
+    if mode != "bpr":
+        # first choices of the finite rows are the oracle's (later tokens' locations may differ: bad rows count)
+        sel, _ = mo.select_topk(logits, k, gate_is_logits=is_logits)
+        first = idx[:S]
+        good = ~bad & (first >= 0)
+        np.testing.assert_array_equal(first[good], sel[0][good])

@@ -154,3 +154,71 @@ def test_config4_lancet_forward_pipeline_bf16(pkg):
     i2, l2, u2, _ = mo.gen_location(osel[1], u1, 5120, M, E)
     np.testing.assert_array_equal(to_np(merged), mo.moe_merge_masks([np.stack([i1, l1]), np.stack([i2, l2])], E))
     check_buffer_properties(data, merged, used, red, 2)
+
+
+# ----------------------------------------------------------------------------- config 5: LANS at full size
+def _config5_shapes():
+    """24 layers x {4 x [1024,1024], 8 x [1024]}, every second layer 32 expert matrices ([1024,4096] and
+    [4096,1024] x 16 experts), final norm 2 x [1024]: 674 tensors, 1,711,474,688 parameters."""
+    shapes = []
+    for layer in range(24):
+        shapes += [(1024, 1024)] * 4 + [(1024,)] * 8
+        if layer % 2 == 1:
+            shapes += [(1024, 4096), (4096, 1024)] * 16
+    return shapes + [(1024,)] * 2
+
+
+def test_config5_lans_full_size(pkg):
+    """All 674 tensors stepped 10 times by both schedules.  The oracle follows a sample of the tensors (one of
+    every shape, at the list's ends and in its middle: a step is independent per tensor) through the same 10
+    steps: parameters within 1e-6 of max|p| (m, v 1e-5).  Over the whole list: the norms the plan reports
+    against torch's fp64 norms of the same arrays, and the two schedules against each other (2e-6)."""
+    import importlib
+    lo = importlib.import_module("oracle.lans_oracle")
+    ops, capi = pkg.ops, pkg.capi
+    free, _ = torch.cuda.mem_get_info()
+    if free < 80 << 30:
+        pytest.skip("needs 80 GiB of free device memory")
+    shapes = _config5_shapes()
+    numels = [int(np.prod(s)) for s in shapes]
+    assert len(shapes) == 674 and sum(numels) == 1711474688
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    p0 = [torch.randn(s, generator=gen, device="cuda") * 0.02 for s in shapes]
+    state = {}
+    for name, sched in (("sweeps", capi.LANS_SWEEPS), ("resident", capi.LANS_RESIDENT)):
+        state[name] = ([x.clone() for x in p0], [torch.zeros_like(x) for x in p0], [torch.zeros_like(x) for x in p0],
+                       ops.LansPlan(numels, schedule=sched))
+    sample = [0, 4, 12, 16, 24, 25, 300, 341, 672, 673]              # matrices, vectors, both expert shapes, the ends
+    assert {shapes[i] for i in sample} == set(shapes)
+    ref_p = [to_np(p0[i]) for i in sample]
+    ref_m = [np.zeros(shapes[i], np.float32) for i in sample]
+    ref_v = [np.zeros(shapes[i], np.float32) for i in sample]
+    hyper = capi.LansHyper(1e-3, 0.9, 0.999, 1e-6, 1, 0.01, 1, 1, 1)
+    g = [torch.empty_like(x) for x in p0]
+    for step in range(1, 11):
+        for x in g:
+            x.normal_(0.0, 1e-3, generator=gen)
+        for name in ("sweeps", "resident"):
+            p, m, v, plan = state[name]
+            plan.step(g, p, m, v, step, hyper)
+        lo.lans_step([to_np(g[i]) for i in sample], ref_p, ref_m, ref_v, step)
+        if step in (1, 10):
+            p, m, v, plan = state["sweeps"]
+            norms = to_np(plan.norms())
+            want_g = torch.stack([torch.linalg.vector_norm(x.double()) for x in g]).cpu().numpy()
+            np.testing.assert_allclose(norms[0], want_g, rtol=2e-6)
+    torch.cuda.synchronize()
+    for name in ("sweeps", "resident"):
+        p, m, v, plan = state[name]
+        assert plan.error() == 0
+        for k, i in enumerate(sample):
+            for got, want, tol, what in ((p[i], ref_p[k], 1e-6, "p"), (m[i], ref_m[k], 1e-5, "m"), (v[i], ref_v[k], 1e-5, "v")):
+                err = np.abs(to_np(got).astype(np.float64) - want).max()
+                assert err <= tol * np.abs(want).max(), "%s %s[%d]: %.3e" % (name, what, i, err)
+    ps, pr = state["sweeps"][0], state["resident"][0]
+    for i in range(len(shapes)):
+        scale = float(ps[i].abs().max())
+        assert float((ps[i] - pr[i]).abs().max()) <= 2e-6 * scale, i
+        assert bool((ps[i] != p0[i]).any())                         # every tensor was stepped
+    for name in ("sweeps", "resident"):
+        state[name][3].close()

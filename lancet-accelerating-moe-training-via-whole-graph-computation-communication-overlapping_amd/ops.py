@@ -582,6 +582,17 @@ class LansStepper:
                       int(mode), bool(normalize_grad))
         self._step = 1
 
-    def step(self, grads):
-        lans(list(grads) + self.params + self.m + self.v, self._step, *self.hyper)
+    def step(self, grads=None):
+        """grads: one gradient per parameter, None for a parameter without one (it is left out of the step, as
+        python/raf/optim/lans.py:82-84 leaves out parameters whose .grad is None); default: the parameters' .grad."""
+        if grads is None:
+            grads = [p.grad for p in self.params]
+        grads = list(grads)
+        _need(len(grads) == len(self.params), "one gradient (or None) per parameter")
+        live = [i for i, g in enumerate(grads) if g is not None]
+        if live:
+            pick = lambda lst: [lst[i] for i in live]
+            # the update writes the parameters in place, outside autograd
+            lans(pick(grads) + [p.detach() for p in pick(self.params)] + pick(self.m) + pick(self.v), self._step,
+                 *self.hyper)
         self._step += 1

@@ -258,3 +258,36 @@ def test_lans_resident_schedule_beside_other_work(pkg):
     for a, b in zip(flat_a, flat_b):
         assert torch.equal(a, b)
     plan.close()
+
+
+def test_stepper_trains_a_small_model_like_the_reference_optimizer(pkg):
+    """LansStepper is the counterpart of raf.optim.lans.LANS (python/raf/optim/lans.py:44-103): it owns m, v and the
+    step counter, takes the parameters' .grad, and leaves out parameters without a gradient.  Five training
+    steps of a two-layer model against the oracle fed with the same gradients."""
+    torch.manual_seed(0)
+    w1 = (torch.randn(64, 32, device="cuda") * 0.1).requires_grad_(True)
+    b1 = torch.zeros(32, device="cuda", requires_grad=True)
+    w2 = (torch.randn(32, 8, device="cuda") * 0.1).requires_grad_(True)
+    unused = torch.ones(5, device="cuda", requires_grad=True)          # never reached by the loss: .grad stays None
+    params = [w1, b1, w2, unused]
+    opt = pkg.ops.LansStepper(params, lr=2e-3, weight_decay=0.05)
+    ref_p = [to_np(p.detach()) for p in params[:3]]
+    ref_m = [np.zeros_like(a) for a in ref_p]
+    ref_v = [np.zeros_like(a) for a in ref_p]
+    x = torch.randn(128, 64, device="cuda")
+    y = torch.randn(128, 8, device="cuda")
+    losses = []
+    for step in range(1, 6):
+        for p in params:
+            p.grad = None
+        loss = ((torch.tanh(x @ w1 + b1) @ w2 - y) ** 2).mean()
+        loss.backward()
+        losses.append(float(loss.detach()))
+        lo.lans_step([to_np(p.grad) for p in params[:3]], ref_p, ref_m, ref_v, step, lr=2e-3, weight_decay=0.05)
+        opt.step()
+    assert losses[-1] < losses[0]
+    for p, want in zip(params[:3], ref_p):
+        assert_close_scaled(to_np(p.detach()), want, 5e-6, "parameter")   # gradients feed back: errors compound
+    np.testing.assert_array_equal(to_np(unused.detach()), np.ones(5, np.float32))
+    with pytest.raises(ValueError):
+        opt.step([None])

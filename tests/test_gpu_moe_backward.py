@@ -4,6 +4,8 @@ oracle (itself pinned against torch autograd in tests/test_oracle_moe.py).
 Bar: encode_dx, encode_dg and fp32 decode_dx are copies or single fp32 products -> bit-exact;
 16-bit decode_dx within 1 ulp; decode_dg is a length-M dot product summed in a different order than
 the oracle's fp64 sum -> 1e-5 of sum|a_i*b_i|."""
+import copy
+
 import numpy as np
 import pytest
 import torch
@@ -166,3 +168,52 @@ def test_autograd_wiring_of_a_prioritized_partition(pkg):
     rest = torch.ones(S0, dtype=torch.bool, device="cuda")
     rest[own] = False
     assert not bool(x.grad[rest].any()) and not bool(gate.grad[rest].any())
+
+
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+def test_moe_layer_module_against_a_dense_layer(pkg, dt):
+    """Gate / Experts / MOELayerImpl (the reference's layer, models/benchmark/pytorch/utils.py:529-634) on the HIP
+    operators: output and all parameter gradients against the same layer written densely with one-hot masks in
+    torch (the form of the reference's FakeMoeEncodeOp / FakeMoeDecodeOp, :349-370,454-462), in fp64."""
+    ml = pkg.moe_layer
+    torch.manual_seed(3)
+    B, L, M, E, H = 4, 96, 32, 4, 48
+    expert = torch.nn.Sequential(torch.nn.Linear(M, H), torch.nn.GELU(), torch.nn.Linear(H, M))
+    layer = ml.MOELayerImpl(ml.Gate(M, E), ml.Experts(expert, 1, M, E), 1, E, capacity_factor=0.75).cuda()
+    for i, e in enumerate(layer.experts.experts):            # the copies start equal: make the experts differ
+        for p in e.parameters():
+            p.data.add_(0.05 * (i + 1) * torch.randn_like(p))
+    layer = layer.to(dt)
+    x = torch.randn(B, L, M, device="cuda").to(dt).requires_grad_(True)
+    Y = torch.randn(B, L, M, device="cuda")
+    out = layer(x)
+    assert out.shape == x.shape and out.dtype == dt
+    (out.float() * Y).sum().backward()
+
+    # dense fp64 layer with the same parameters and the same routing decisions
+    ref = copy.deepcopy(layer).double()
+    xr = x.detach().double().requires_grad_(True)
+    flat = xr.reshape(-1, M)
+    gate = torch.softmax(ref.gate.wg(flat), dim=1)
+    S = flat.shape[0]
+    C = pkg.ops.moe_capacity(S, E, 0.75)
+    with torch.no_grad():
+        _, il, _, _, _ = pkg.ops.moe_encode(x.detach().reshape(-1, M).contiguous(), layer.gate(x.detach().reshape(-1, M)), None, 0.75)
+    idx, loc = il[0].long(), il[1].long()
+    kept = idx >= 0
+    assert bool((~kept).any())
+    mask = torch.zeros((S, E, C), dtype=torch.float64, device="cuda")
+    mask[torch.arange(S, device="cuda")[kept], idx[kept], loc[kept]] = 1.0
+    gates_s = (gate * mask.sum(2)).sum(1)
+    disp = torch.einsum("sec,sm->ecm", mask, flat)
+    eo = torch.stack([ref.experts.experts[e](disp[e]) for e in range(E)])
+    want = torch.einsum("sec,ecm->sm", mask * gates_s[:, None, None], eo).reshape(B, L, M)
+    (want * Y.double()).sum().backward()
+    tol = dict(rtol=1e-4, atol=1e-5) if dt == torch.float32 else dict(rtol=5e-2, atol=5e-2)
+    torch.testing.assert_close(out.detach().double(), want.detach(), **tol)
+    torch.testing.assert_close(x.grad.double(), xr.grad, **tol)
+    for (n, a), (_, b) in zip(layer.named_parameters(), ref.named_parameters()):
+        assert a.grad is not None, n
+        scale = float(b.grad.abs().max())
+        err = float((a.grad.double() - b.grad).abs().max())
+        assert err <= (1e-4 if dt == torch.float32 else 5e-2) * max(scale, 1e-6), (n, err, scale)

@@ -61,6 +61,24 @@ def event_ms(fn, iters):
     return start.elapsed_time(stop) / iters
 
 
+def hbm_probe(iters):
+    """What plain streaming kernels reach on this device, measured beside the row movers: a device-to-device
+    copy (half reads, half writes) and a fill (writes only) of 1 GiB, torch's own kernels.  The row movers'
+    fractions of the 8 TB/s peak are to be read against these."""
+    import torch
+    n = 1 << 30
+    src = torch.zeros(n, dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(src)
+    dst.copy_(src), dst.zero_()
+    ms_copy = event_ms(lambda: dst.copy_(src), iters)
+    ms_fill = event_ms(lambda: dst.zero_(), iters)
+    out = {"bytes": n, "copy_GBps": round(2 * n / ms_copy / 1e6, 1), "fill_GBps": round(n / ms_fill / 1e6, 1),
+           "copy_frac_of_peak": round(2 * n / ms_copy / 1e6 / HBM_PEAK_GBS, 4),
+           "fill_frac_of_peak": round(n / ms_fill / 1e6 / HBM_PEAK_GBS, 4)}
+    del src, dst
+    return out
+
+
 def lans_shapes(scale=1.0):
     """BASELINE config 5: 24 layers x {4 x [1024,1024], 4 x [1024] biases, 4 x [1024] norms},
     12 MoE layers x 16 experts x {[1024,4096],[4096,1024]}, final norm 2 x [1024]:
@@ -602,6 +620,7 @@ def main():
             "encode_plus_decode_frac": round(gbs(enc_bytes + dec_bytes, ms_enc + ms_dec) / HBM_PEAK_GBS, 4),
         },
     }
+    result["hbm_probe"] = hbm_probe(n)
     result["backward"] = bench_backward(ops, data, outs, dec, S, M, E, Cap, K, kept, n)
     del dec, outs
     torch.cuda.empty_cache()

@@ -8,7 +8,7 @@
 
 namespace lancet {
 
-constexpr int kRowsPerBlock = kTile / kWave;  // one wave per row
+constexpr int kRowsPerBlock = kTile / kWave;  // waves per workgroup; a wave moves a row or a share of one
 constexpr int kTailRows = 16;                 // rows zero-filled by one tail workgroup
 
 // Access granule: 16 bytes when the row size and the pointers allow, else one element.
@@ -42,6 +42,7 @@ struct ScatterArgs {
   int slot_stride;            // distance between the slots of one token in idx / loc (S, or the whole batch's
                               // token count when this call moves a token range of a larger mask)
   int row_vecs;               // granules per row
+  int waves_per_row;          // waves that share one token row
   int token_blocks;
   int tail_chunks;            // tail workgroups per expert
 };
@@ -51,7 +52,12 @@ __global__ __launch_bounds__(kTile) void scatter_rows_kernel(ScatterArgs<V> a) {
   const int w = threadIdx.x / kWave;
   const int lane = threadIdx.x & (kWave - 1);
   if (static_cast<int>(blockIdx.x) < a.token_blocks) {
-    const int s = blockIdx.x * kRowsPerBlock + w;
+    // waves_per_row waves share a token row, each moving every waves_per_row-th run of 64 granules: short
+    // waves in row order keep the chip-wide write stream close to address order, which the memory system
+    // rewards (one granule per lane streams ~8 % faster than a wave walking a whole 8 KB row)
+    const long gw = static_cast<long>(blockIdx.x) * kRowsPerBlock + w;
+    const int s = static_cast<int>(gw / a.waves_per_row);
+    const int part = static_cast<int>(gw - static_cast<long>(s) * a.waves_per_row);
     if (s >= a.S) return;
     // destinations picked at run time: typed as global memory so the stores are not flat
     LANCET_GLOBAL V* dst[K];
@@ -71,21 +77,19 @@ __global__ __launch_bounds__(kTile) void scatter_rows_kernel(ScatterArgs<V> a) {
     }
     if (nd == 0) return;
     const V* src = a.data + static_cast<size_t>(s) * a.row_vecs;
-    int v = lane;
-    for (; v + 3 * kWave < a.row_vecs; v += 4 * kWave) {
-      const V x0 = ldv(src + v), x1 = ldv(src + v + kWave), x2 = ldv(src + v + 2 * kWave),
-              x3 = ldv(src + v + 3 * kWave);
+    const int step = a.waves_per_row * kWave;
+    int v = part * kWave + lane;
+    for (; v + step < a.row_vecs; v += 2 * step) {
+      const V x0 = ldv(src + v), x1 = ldv(src + v + step);
 #pragma unroll
       for (int j = 0; j < K; ++j) {
         if (j < nd) {
           stv(dst[j] + v, x0);
-          stv(dst[j] + v + kWave, x1);
-          stv(dst[j] + v + 2 * kWave, x2);
-          stv(dst[j] + v + 3 * kWave, x3);
+          stv(dst[j] + v + step, x1);
         }
       }
     }
-    for (; v < a.row_vecs; v += kWave) {
+    if (v < a.row_vecs) {
       const V x = ldv(src + v);
 #pragma unroll
       for (int j = 0; j < K; ++j)
@@ -187,6 +191,7 @@ struct DecodeArgs {
   void* out;             // [S, M]
   int S, M, E, C;
   int slot_stride;       // distance between the slots of one token in gates / idx / loc
+  int waves_per_row;     // waves that share one token row (each takes every waves_per_row-th run of 64 granules)
 };
 
 template <int DT, int K, bool VEC>
@@ -194,8 +199,11 @@ __global__ __launch_bounds__(kTile) void decode_rows_kernel(DecodeArgs a) {
   typedef Codec<DT> Cd;
   const int w = threadIdx.x / kWave;
   const int lane = threadIdx.x & (kWave - 1);
-  const int s = blockIdx.x * kRowsPerBlock + w;
+  const long gw = static_cast<long>(blockIdx.x) * kRowsPerBlock + w;
+  const int s = static_cast<int>(gw / a.waves_per_row);
+  const int part = static_cast<int>(gw - static_cast<long>(s) * a.waves_per_row);
   if (s >= a.S) return;
+  const int step = a.waves_per_row * kWave;
   float g[K];
   size_t row[K];
   bool ok[K];
@@ -214,22 +222,22 @@ __global__ __launch_bounds__(kTile) void decode_rows_kernel(DecodeArgs a) {
     u32x4* dst = static_cast<u32x4*>(a.out) + static_cast<size_t>(s) * row_vecs;
     const u32x4* base = static_cast<const u32x4*>(a.expert_out);
     const u32x4 z = {0u, 0u, 0u, 0u};
+    int v = part * kWave + lane;
     if (!any) {
-      for (int v = lane; v < row_vecs; v += kWave) st_stream(dst + v, z);
+      for (; v < row_vecs; v += step) st_stream(dst + v, z);
       return;
     }
-    int v = lane;
-    for (; v + kWave < row_vecs; v += 2 * kWave) {  // two granules in flight per slot
+    for (; v + step < row_vecs; v += 2 * step) {  // two granules in flight per slot
       u32x4 xa[K], xb[K];
 #pragma unroll
       for (int j = 0; j < K; ++j) {
         xa[j] = ok[j] ? ld_stream(base + row[j] * row_vecs + v) : z;
-        xb[j] = ok[j] ? ld_stream(base + row[j] * row_vecs + v + kWave) : z;
+        xb[j] = ok[j] ? ld_stream(base + row[j] * row_vecs + v + step) : z;
       }
       st_stream(dst + v, combine_vec<DT, K>(xa, g));
-      st_stream(dst + v + kWave, combine_vec<DT, K>(xb, g));
+      st_stream(dst + v + step, combine_vec<DT, K>(xb, g));
     }
-    for (; v < row_vecs; v += kWave) {
+    if (v < row_vecs) {
       u32x4 xa[K];
 #pragma unroll
       for (int j = 0; j < K; ++j) xa[j] = ok[j] ? ld_stream(base + row[j] * row_vecs + v) : z;
@@ -239,7 +247,7 @@ __global__ __launch_bounds__(kTile) void decode_rows_kernel(DecodeArgs a) {
     typedef typename Cd::S St;
     St* dst = static_cast<St*>(a.out) + static_cast<size_t>(s) * a.M;
     const St* base = static_cast<const St*>(a.expert_out);
-    for (int i = lane; i < a.M; i += kWave) {
+    for (int i = part * kWave + lane; i < a.M; i += step) {
 #pragma clang fp contract(off)
       float acc = ok[0] ? mul_rn(g[0], Cd::get(base[row[0] * a.M + i])) : 0.f;
       if (K == 2) acc = add_rn(acc, ok[1] ? mul_rn(g[1], Cd::get(base[row[1] * a.M + i])) : 0.f);
@@ -547,6 +555,13 @@ __global__ __launch_bounds__(kTile) void decode_dg_kernel(const void* dy, const 
 // ---------------------------------------------------------------------------------------
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Waves that share one row of `units` granules: one granule per lane where the grid allows it, at most 16.
+static inline int split_waves(long units, long rows) {
+  long wpr = std::min<long>(std::max<long>((units + kWave - 1) / kWave, 1), 16);
+  while (wpr > 1 && (rows * wpr + kRowsPerBlock - 1) / kRowsPerBlock > 0x3fffffffL) wpr /= 2;
+  return static_cast<int>(wpr);
+}
+
 template <typename V>
 static hipError_t scatter_launch(const void* data, void* out, const int32_t* idx, const int32_t* loc,
                                  const int32_t* avail_used, const int32_t* row_base, const int32_t* rows_lo,
@@ -567,7 +582,9 @@ static hipError_t scatter_launch(const void* data, void* out, const int32_t* idx
   a.K = K;
   a.slot_stride = slot_stride;
   a.row_vecs = row_vecs;
-  a.token_blocks = (S + kRowsPerBlock - 1) / kRowsPerBlock;
+  const long wpr = split_waves(row_vecs, S);
+  a.waves_per_row = static_cast<int>(wpr);
+  a.token_blocks = static_cast<int>((static_cast<long>(S) * wpr + kRowsPerBlock - 1) / kRowsPerBlock);
   a.tail_chunks = rows_hi ? (C + kTailRows - 1) / kTailRows : 0;
   const long blocks = static_cast<long>(a.token_blocks) + static_cast<long>(a.tail_chunks) * E;
   if (blocks == 0) return hipSuccess;
@@ -612,9 +629,11 @@ hipError_t run_zero_bytes(void* p, size_t nbytes, hipStream_t st) {
 }
 
 template <int DT>
-static hipError_t decode_launch(const DecodeArgs& a, int K, bool vec, hipStream_t st) {
-  const int blocks = (a.S + kRowsPerBlock - 1) / kRowsPerBlock;
-  if (blocks == 0 || a.M == 0) return hipSuccess;
+static hipError_t decode_launch(DecodeArgs a, int K, bool vec, hipStream_t st) {
+  if (a.S == 0 || a.M == 0) return hipSuccess;
+  const long wpr = split_waves(vec ? a.M / Codec<DT>::kPerVec : a.M, a.S);
+  a.waves_per_row = static_cast<int>(wpr);
+  const unsigned blocks = static_cast<unsigned>((static_cast<long>(a.S) * wpr + kRowsPerBlock - 1) / kRowsPerBlock);
   if (K == 1) {
     if (vec) decode_rows_kernel<DT, 1, true><<<blocks, kTile, 0, st>>>(a);
     else decode_rows_kernel<DT, 1, false><<<blocks, kTile, 0, st>>>(a);

@@ -169,6 +169,11 @@ __device__ __forceinline__ void bias_corrections(const LansScalars& sc, float& b
   }
 }
 
+// Streaming accesses: every array is touched once per sweep and is far larger than the caches; non-temporal
+// loads and stores stream measurably faster here than plain ones.
+__device__ __forceinline__ f32x4 ldn(const LANCET_GLOBAL f32x4* p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ void stn(LANCET_GLOBAL f32x4* p, f32x4 x) { __builtin_nontemporal_store(x, p); }
+
 // ---- the three phases on one chunk, executed by one workgroup ------------------------------
 // phase 1: sum of squares of g (L2NormFunctor, multi_tensor_lans.cu:95-167); valid on thread 0.
 // (The sum of squares of p is not needed before phase 3 and is taken in phase 2, which reads p anyway.)
@@ -181,7 +186,7 @@ __device__ __forceinline__ float chunk_norm_g(const LansTables& t, const ChunkVi
     const LANCET_GLOBAL f32x4* g4 = (const LANCET_GLOBAL f32x4*)g;
 #pragma unroll 8
     for (int i = threadIdx.x; i < nv; i += kLansThreads) {
-      const f32x4 x = g4[i];
+      const f32x4 x = ldn(g4 + i);
       ag += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
     }
     scalar_from = nv * 4;
@@ -208,8 +213,8 @@ __device__ __forceinline__ void chunk_moments(const LansTables& t, const ChunkVi
     LANCET_GLOBAL f32x4* v4 = (LANCET_GLOBAL f32x4*)v;
 #pragma unroll 2
     for (int i = threadIdx.x; i < nv; i += kLansThreads) {
-      const f32x4 xg = g4[i], xp = p4[i];
-      f32x4 xm = m4[i], xv = v4[i];
+      const f32x4 xg = ldn(g4 + i), xp = ldn(p4 + i);
+      f32x4 xm = ldn(m4 + i), xv = ldn(v4 + i);
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         const float sg = el.scaled_grad(xg[k], xp[k]);
@@ -222,8 +227,8 @@ __device__ __forceinline__ void chunk_moments(const LansTables& t, const ChunkVi
         am += um * um;
         ag += ug * ug;
       }
-      m4[i] = xm;
-      v4[i] = xv;
+      stn(m4 + i, xm);
+      stn(v4 + i, xv);
     }
     scalar_from = nv * 4;
   }
@@ -263,8 +268,8 @@ __device__ __forceinline__ void chunk_update(const LansTables& t, const ChunkVie
     const LANCET_GLOBAL f32x4* v4 = (const LANCET_GLOBAL f32x4*)v;
 #pragma unroll 2
     for (int i = threadIdx.x; i < nv; i += kLansThreads) {
-      const f32x4 xg = g4[i], xm = m4[i], xv = v4[i];
-      f32x4 xp = p4[i];
+      const f32x4 xg = ldn(g4 + i), xm = ldn(m4 + i), xv = ldn(v4 + i);
+      f32x4 xp = ldn(p4 + i);
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
 #pragma clang fp contract(off)
@@ -273,7 +278,7 @@ __device__ __forceinline__ void chunk_update(const LansTables& t, const ChunkVie
         el.updates(sg, xp[k], xm[k], xv[k], um, ug);
         xp[k] = xp[k] - (ratio_m * um) - (ratio_g * ug);
       }
-      p4[i] = xp;
+      stn(p4 + i, xp);
     }
     scalar_from = nv * 4;
   }
@@ -371,8 +376,8 @@ __device__ __forceinline__ void st_word(uint64_t* p, uint32_t epoch, float v) {
 // =======================================================================================
 constexpr int kVecPerThread = kLansChunk / 4 / kLansThreads;  // float4 per thread and array
 
-__device__ __forceinline__ f32x4 ld4(const LANCET_GLOBAL float* a, int e) { return *(const LANCET_GLOBAL f32x4*)(a + e); }
-__device__ __forceinline__ void st4(LANCET_GLOBAL float* a, int e, f32x4 x) { *(LANCET_GLOBAL f32x4*)(a + e) = x; }
+__device__ __forceinline__ f32x4 ld4(const LANCET_GLOBAL float* a, int e) { return ldn((const LANCET_GLOBAL f32x4*)(a + e)); }
+__device__ __forceinline__ void st4(LANCET_GLOBAL float* a, int e, f32x4 x) { stn((LANCET_GLOBAL f32x4*)(a + e), x); }
 
 constexpr int kMaxResidentChunks = 512;  // chunks of one tensor the resident schedule can gather
 

@@ -622,7 +622,8 @@ hipError_t run_zero_bytes(void* p, size_t nbytes, hipStream_t st) {
   const size_t nvec = nbytes / 16;
   const size_t ntail = nbytes - nvec * 16;
   if (nvec || ntail) {
-    const int blocks = static_cast<int>(std::min<size_t>((nvec + 255) / 256 + 1, 8192));
+    // one granule per thread up to 2^22 workgroups (16 GiB), a loop beyond that
+    const int blocks = static_cast<int>(std::min<size_t>((nvec + 255) / 256 + 1, size_t(1) << 22));
     zero_bytes_kernel<<<blocks, 256, 0, st>>>(reinterpret_cast<u32x4*>(b), nvec, b + nvec * 16, ntail);
   }
   return hipGetLastError();

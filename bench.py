@@ -61,20 +61,29 @@ def event_ms(fn, iters):
     return start.elapsed_time(stop) / iters
 
 
-def hbm_probe(iters):
-    """What plain streaming kernels reach on this device, measured beside the row movers: a device-to-device
-    copy (half reads, half writes) and a fill (writes only) of 1 GiB, torch's own kernels.  The row movers'
-    fractions of the 8 TB/s peak are to be read against these."""
+def hbm_probe(lib, iters):
+    """What plain streaming kernels reach on this device, measured beside the row movers, over 1 GiB: the
+    library's own probe kernels (lancet_debug_stream: one 16-byte non-temporal access per thread, workgroups in
+    address order, the shape that streams fastest here) and torch's copy_ / zero_ for comparison.  The row
+    movers' fractions of the 8 TB/s peak are to be read against these."""
+    import ctypes as C
     import torch
     n = 1 << 30
     src = torch.zeros(n, dtype=torch.uint8, device="cuda")
     dst = torch.empty_like(src)
+    p = lambda t: C.c_void_p(t.data_ptr())
+
+    def run(kind):
+        assert lib.lancet_debug_stream(kind, p(dst), p(src), n, None) == 0
+
+    out = {"bytes": n}
+    for name, kind, nbytes in (("read_GBps", 0, n), ("fill_GBps", 1, n), ("copy_GBps", 2, 2 * n)):
+        run(kind)
+        out[name] = round(nbytes / event_ms(lambda: run(kind), iters) / 1e6, 1)
     dst.copy_(src), dst.zero_()
-    ms_copy = event_ms(lambda: dst.copy_(src), iters)
-    ms_fill = event_ms(lambda: dst.zero_(), iters)
-    out = {"bytes": n, "copy_GBps": round(2 * n / ms_copy / 1e6, 1), "fill_GBps": round(n / ms_fill / 1e6, 1),
-           "copy_frac_of_peak": round(2 * n / ms_copy / 1e6 / HBM_PEAK_GBS, 4),
-           "fill_frac_of_peak": round(n / ms_fill / 1e6 / HBM_PEAK_GBS, 4)}
+    out["torch_copy_GBps"] = round(2 * n / event_ms(lambda: dst.copy_(src), iters) / 1e6, 1)
+    out["torch_fill_GBps"] = round(n / event_ms(lambda: dst.zero_(), iters) / 1e6, 1)
+    out["copy_frac_of_peak"] = round(out["copy_GBps"] / HBM_PEAK_GBS, 4)
     del src, dst
     return out
 
@@ -620,7 +629,7 @@ def main():
             "encode_plus_decode_frac": round(gbs(enc_bytes + dec_bytes, ms_enc + ms_dec) / HBM_PEAK_GBS, 4),
         },
     }
-    result["hbm_probe"] = hbm_probe(n)
+    result["hbm_probe"] = hbm_probe(lib, n)
     result["backward"] = bench_backward(ops, data, outs, dec, S, M, E, Cap, K, kept, n)
     del dec, outs
     torch.cuda.empty_cache()

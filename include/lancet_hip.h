@@ -339,6 +339,12 @@ int64_t lancet_lans_debug_chunk_table(const int64_t* numels, int T, int resident
  * before it gives up, flags the workspace and finishes with undefined results
  * (0 restores the default).  Lets a host test exercise the bounded wait without hanging. */
 void lancet_debug_set_spin_limit(unsigned limit);
+/* Measurement aid (no counterpart in the reference): one plain streaming kernel over `bytes` bytes (a multiple
+ * of 4096), one 16-byte non-temporal access per thread, workgroups in address order: the launch shape that
+ * streams fastest on this device.  kind 0 reads src, 1 fills dst with zeros, 2 copies src to dst.  bench.py
+ * times these beside the row movers so that their fractions of the peak can be read against what the
+ * memory system delivers to the simplest possible kernel. */
+int lancet_debug_stream(int kind, void* dst, const void* src, size_t bytes, lancet_stream_t stream);
 /* Reads (synchronously) the error word a scan workspace carries: 0 = ok, 1 = a wait gave up. */
 int lancet_scan_workspace_error(const void* workspace, lancet_stream_t stream, int* error_out);
 

@@ -56,6 +56,7 @@ SIGNATURES = {
                                      _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "lancet_moe_scatter_tokens": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _u32, _vp, _vp]),
     "lancet_moe_decode_tokens": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp]),
+    "lancet_debug_stream": (_int, [_int, _vp, _vp, _sz, _vp]),
     "lancet_moe_decode": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp]),
     "lancet_moe_redispatch_expert_input": (_int, [C.POINTER(_vp), C.POINTER(_vp), _int, _int, _int, _i64, _i64, _i64,
                                                   _int, _int, _vp, _vp]),

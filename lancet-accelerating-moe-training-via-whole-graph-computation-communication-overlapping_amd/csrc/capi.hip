@@ -1,6 +1,7 @@
 // C ABI of the MoE dispatch path: argument validation, then kernel launches on the caller's
 // stream.  Nothing here allocates, synchronises or keeps state between calls.
 #include "../../include/lancet_hip.h"
+#include "common.hpp"
 #include "launchers.hpp"
 
 using namespace lancet;
@@ -75,6 +76,38 @@ extern "C" int lancet_scan_workspace_error(const void* workspace, lancet_stream_
   if (e == hipSuccess) e = hipStreamSynchronize(S_(stream));
   *error_out = static_cast<int>(word);
   return rc(e);
+}
+
+// ---- plain streaming kernels (measurement aid) -------------------------------------------
+namespace {
+template <int KIND>
+__global__ __launch_bounds__(256) void stream_kernel(u32x4* __restrict__ dst, const u32x4* __restrict__ src) {
+  const size_t i = blockIdx.x * static_cast<size_t>(256) + threadIdx.x;
+  if (KIND == 0) {
+    const u32x4 x = ld_stream(src + i);
+    if ((x.x ^ x.y ^ x.z ^ x.w) == 0x5eedf00du && dst) st_stream(dst, x);  // keeps the load alive; practically never taken
+  } else if (KIND == 1) {
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    st_stream(dst + i, z);
+  } else {
+    st_stream(dst + i, ld_stream(src + i));
+  }
+}
+}  // namespace
+
+extern "C" int lancet_debug_stream(int kind, void* dst, const void* src, size_t bytes, lancet_stream_t stream) {
+  if (kind < 0 || kind > 2) return LANCET_ERR_SHAPE;
+  if (bytes % 4096 != 0 || bytes / 4096 > 0x7fffffffu) return LANCET_ERR_SHAPE;
+  if ((kind != 1 && !src) || (kind != 0 && !dst)) return LANCET_ERR_NULL;
+  if (misaligned(dst, 16) || misaligned(src, 16)) return LANCET_ERR_ALIGN;
+  if (bytes == 0) return LANCET_OK;
+  const unsigned blocks = static_cast<unsigned>(bytes / 4096);
+  u32x4* d = static_cast<u32x4*>(dst);
+  const u32x4* s = static_cast<const u32x4*>(src);
+  if (kind == 0) stream_kernel<0><<<blocks, 256, 0, S_(stream)>>>(d, s);
+  else if (kind == 1) stream_kernel<1><<<blocks, 256, 0, S_(stream)>>>(d, s);
+  else stream_kernel<2><<<blocks, 256, 0, S_(stream)>>>(d, s);
+  return rc(hipGetLastError());
 }
 
 // ---- routing front end ---------------------------------------------------------------

@@ -626,3 +626,20 @@ def test_non_finite_gates_keep_the_outputs_well_formed(pkg, mode, is_logits):
         first = idx[:S]
         good = ~bad & (first >= 0)
         np.testing.assert_array_equal(first[good], sel[0][good])
+
+
+def test_streaming_probe_kernels(pkg, lib):
+    """lancet_debug_stream (the plain read / fill / copy kernels bench.py times beside the row movers)."""
+    import ctypes as C
+    n = 3 * 4096
+    src = torch.randint(0, 255, (n,), dtype=torch.uint8, device="cuda")
+    dst = torch.full((n + 4096,), 7, dtype=torch.uint8, device="cuda")
+    p = lambda t: C.c_void_p(t.data_ptr())
+    assert lib.lancet_debug_stream(2, p(dst), p(src), n, None) == 0
+    assert torch.equal(dst[:n], src) and bool((dst[n:] == 7).all())
+    assert lib.lancet_debug_stream(1, p(dst), None, 4096, None) == 0
+    assert not bool(dst[:4096].any()) and torch.equal(dst[4096:n], src[4096:])
+    assert lib.lancet_debug_stream(0, None, p(src), n, None) == 0
+    assert lib.lancet_debug_stream(2, p(dst), p(src), 100, None) == pkg.capi.ERR_SHAPE
+    assert lib.lancet_debug_stream(2, None, p(src), n, None) == pkg.capi.ERR_NULL
+    torch.cuda.synchronize()

@@ -42,7 +42,7 @@ struct ScatterArgs {
   int slot_stride;            // distance between the slots of one token in idx / loc (S, or the whole batch's
                               // token count when this call moves a token range of a larger mask)
   int row_vecs;               // granules per row
-  int waves_per_row;          // waves that share one token row
+  int wpr_shift;              // 2^wpr_shift waves share one token row
   int token_blocks;
   int tail_chunks;            // tail workgroups per expert
 };
@@ -52,12 +52,12 @@ __global__ __launch_bounds__(kTile) void scatter_rows_kernel(ScatterArgs<V> a) {
   const int w = threadIdx.x / kWave;
   const int lane = threadIdx.x & (kWave - 1);
   if (static_cast<int>(blockIdx.x) < a.token_blocks) {
-    // waves_per_row waves share a token row, each moving every waves_per_row-th run of 64 granules: short
+    // 2^wpr_shift waves share a token row, each moving every 2^wpr_shift-th run of 64 granules: short
     // waves in row order keep the chip-wide write stream close to address order, which the memory system
     // rewards (one granule per lane streams ~8 % faster than a wave walking a whole 8 KB row)
-    const long gw = static_cast<long>(blockIdx.x) * kRowsPerBlock + w;
-    const int s = static_cast<int>(gw / a.waves_per_row);
-    const int part = static_cast<int>(gw - static_cast<long>(s) * a.waves_per_row);
+    const uint32_t gw = blockIdx.x * static_cast<uint32_t>(kRowsPerBlock) + w;  // below 2^32: the launcher sees to it
+    const int s = static_cast<int>(gw >> a.wpr_shift);
+    const int part = static_cast<int>(gw & ((1u << a.wpr_shift) - 1u));
     if (s >= a.S) return;
     // destinations picked at run time: typed as global memory so the stores are not flat
     LANCET_GLOBAL V* dst[K];
@@ -77,7 +77,7 @@ __global__ __launch_bounds__(kTile) void scatter_rows_kernel(ScatterArgs<V> a) {
     }
     if (nd == 0) return;
     const V* src = a.data + static_cast<size_t>(s) * a.row_vecs;
-    const int step = a.waves_per_row * kWave;
+    const int step = kWave << a.wpr_shift;
     int v = part * kWave + lane;
     for (; v + step < a.row_vecs; v += 2 * step) {
       const V x0 = ldv(src + v), x1 = ldv(src + v + step);
@@ -191,7 +191,7 @@ struct DecodeArgs {
   void* out;             // [S, M]
   int S, M, E, C;
   int slot_stride;       // distance between the slots of one token in gates / idx / loc
-  int waves_per_row;     // waves that share one token row (each takes every waves_per_row-th run of 64 granules)
+  int wpr_shift;         // 2^wpr_shift waves share one token row (each takes every 2^wpr_shift-th run of 64 granules)
 };
 
 template <int DT, int K, bool VEC>
@@ -199,11 +199,11 @@ __global__ __launch_bounds__(kTile) void decode_rows_kernel(DecodeArgs a) {
   typedef Codec<DT> Cd;
   const int w = threadIdx.x / kWave;
   const int lane = threadIdx.x & (kWave - 1);
-  const long gw = static_cast<long>(blockIdx.x) * kRowsPerBlock + w;
-  const int s = static_cast<int>(gw / a.waves_per_row);
-  const int part = static_cast<int>(gw - static_cast<long>(s) * a.waves_per_row);
+  const uint32_t gw = blockIdx.x * static_cast<uint32_t>(kRowsPerBlock) + w;
+  const int s = static_cast<int>(gw >> a.wpr_shift);
+  const int part = static_cast<int>(gw & ((1u << a.wpr_shift) - 1u));
   if (s >= a.S) return;
-  const int step = a.waves_per_row * kWave;
+  const int step = kWave << a.wpr_shift;
   float g[K];
   size_t row[K];
   bool ok[K];
@@ -555,14 +555,17 @@ __global__ __launch_bounds__(kTile) void decode_dg_kernel(const void* dy, const 
 // ---------------------------------------------------------------------------------------
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// Waves that share one row of `units` granules: per_lane granules per lane where the grid allows it, at
-// most 16 waves.  Measured at 8 KB rows: the scatter is fastest with one granule per lane (8 waves a row),
-// the gather-combine with two (4 waves a row).
+// log2 of the number of waves that share one row of `units` granules: a power of two (the kernels split the wave
+// index with a shift), per_lane granules per lane where the grid allows it, at most 16 waves.  Measured at 8 KB
+// rows: the scatter is fastest with one granule per lane (8 waves a row), the gather-combine with two (4 waves).
 static inline int split_waves(long units, long rows, int per_lane = 1) {
   const long span = static_cast<long>(kWave) * per_lane;
-  long wpr = std::min<long>(std::max<long>((units + span - 1) / span, 1), 16);
-  while (wpr > 1 && (rows * wpr + kRowsPerBlock - 1) / kRowsPerBlock > 0x3fffffffL) wpr /= 2;
-  return static_cast<int>(wpr);
+  const long want = std::max<long>((units + span - 1) / span, 1);
+  int shift = 0;
+  while (shift < 4 && (1L << shift) < want) ++shift;
+  // the grid stays below 2^30 workgroups and the wave index below 2^32
+  while (shift > 0 && ((rows << shift) + kRowsPerBlock - 1) / kRowsPerBlock > 0x3fffffffL) --shift;
+  return shift;
 }
 
 template <typename V>
@@ -585,9 +588,8 @@ static hipError_t scatter_launch(const void* data, void* out, const int32_t* idx
   a.K = K;
   a.slot_stride = slot_stride;
   a.row_vecs = row_vecs;
-  const long wpr = split_waves(row_vecs, S);
-  a.waves_per_row = static_cast<int>(wpr);
-  a.token_blocks = static_cast<int>((static_cast<long>(S) * wpr + kRowsPerBlock - 1) / kRowsPerBlock);
+  a.wpr_shift = split_waves(row_vecs, S);
+  a.token_blocks = static_cast<int>(((static_cast<long>(S) << a.wpr_shift) + kRowsPerBlock - 1) / kRowsPerBlock);
   a.tail_chunks = rows_hi ? (C + kTailRows - 1) / kTailRows : 0;
   const long blocks = static_cast<long>(a.token_blocks) + static_cast<long>(a.tail_chunks) * E;
   if (blocks == 0) return hipSuccess;
@@ -635,9 +637,8 @@ hipError_t run_zero_bytes(void* p, size_t nbytes, hipStream_t st) {
 template <int DT>
 static hipError_t decode_launch(DecodeArgs a, int K, bool vec, hipStream_t st) {
   if (a.S == 0 || a.M == 0) return hipSuccess;
-  const long wpr = split_waves(vec ? a.M / Codec<DT>::kPerVec : a.M, a.S, 2);
-  a.waves_per_row = static_cast<int>(wpr);
-  const unsigned blocks = static_cast<unsigned>((static_cast<long>(a.S) * wpr + kRowsPerBlock - 1) / kRowsPerBlock);
+  a.wpr_shift = split_waves(vec ? a.M / Codec<DT>::kPerVec : a.M, a.S, 2);
+  const unsigned blocks = static_cast<unsigned>(((static_cast<long>(a.S) << a.wpr_shift) + kRowsPerBlock - 1) / kRowsPerBlock);
   if (K == 1) {
     if (vec) decode_rows_kernel<DT, 1, true><<<blocks, kTile, 0, st>>>(a);
     else decode_rows_kernel<DT, 1, false><<<blocks, kTile, 0, st>>>(a);

@@ -643,3 +643,34 @@ def test_streaming_probe_kernels(pkg, lib):
     assert lib.lancet_debug_stream(2, p(dst), p(src), 100, None) == pkg.capi.ERR_SHAPE
     assert lib.lancet_debug_stream(2, None, p(src), n, None) == pkg.capi.ERR_NULL
     torch.cuda.synchronize()
+
+
+# ----------------------------------------------------------------------------- rows split over several waves
+@pytest.mark.parametrize("M", [252, 256, 260, 508, 516, 1001, 1024, 1028, 2050, 4104, 8200, 16392, 33000])
+@pytest.mark.parametrize("dt,k", [("f32", 1), ("bf16", 2), ("f16", 1), ("f32", 2)])
+def test_rows_of_every_split(pkg, M, dt, k):
+    """The row movers hand a row to 1, 2, 4, 8 or 16 waves by its length (one or two 16-byte granules per lane,
+    further granules in a loop).  Row lengths around every switch point, rows that are not a multiple of the
+    granule (element-wise path) and rows longer than one pass of 16 waves, against the oracle."""
+    ops = pkg.ops
+    S, E, cf = 150, 4, 0.8
+    data, logits = make_inputs(M + k, S, M, E, zipf_bias=True)
+    gate = mo.softmax_rows(logits)
+    rows = rows_as_oracle(data, dt)
+    used0 = np.zeros(E, np.int32)
+    want = (mo.moe_encode_top2 if k == 2 else mo.moe_encode)(rows, gate, used0, cf, fast_scatter=True)
+    got = ops.moe_encode(rows_to_torch(data, dt), dev(gate), None, cf, top_k=k)
+    check_encode(got, want, gate_exact=True)
+    assert (want[1][0] < 0).any()
+
+    def same(got_t, want32):
+        if dt == "f32":
+            np.testing.assert_array_equal(to_np(got_t), want32)
+            return
+        tdt = torch.bfloat16 if dt == "bf16" else torch.float16
+        a = got_t.cpu().view(torch.int16).to(torch.int32)
+        b = torch.from_numpy(want32).to(tdt).view(torch.int16).to(torch.int32)
+        assert int((a - b).abs().max()) <= 1                 # one rounding of the same fp32 value on both sides
+
+    same(ops.moe_decode(got[4], got[0], got[1], top_k=k), mo.moe_decode(want[4], want[0], want[1], k=k))
+    same(ops.moe_encode_dx(got[4], got[1], top_k=k), mo.moe_encode_dx(want[4], want[1], k))

@@ -43,3 +43,40 @@ def test_pipeline_equals_unpartitioned_ops(pkg, dt, S, M, E, P, cf):
     want = mo.moe_decode(to_np(disp), to_np(gates_s), to_np(indloc),
                          round_fn=None if dt == "f32" else mo.round_to_bf16)
     np.testing.assert_array_equal(to_np(piped), want)
+
+
+def test_concurrent_calls_on_separate_streams_share_no_state(pkg):
+    """Eight encode + decode pairs issued on eight streams at once, each with its own workspace and outputs
+    (the library keeps no state between calls), repeated a few times: every result equals the one the same
+    call gives when it runs alone."""
+    import numpy as np
+    from tests.gpu_util import dev, make_inputs
+    ops = pkg.ops
+    S, M, E, cf = 8192, 512, 16, 0.9
+    jobs = []
+    for i in range(8):
+        k = 1 + i % 2
+        data, logits = make_inputs(40 + i, S, M, E, zipf_bias=bool(i & 2))
+        d_data = dev(data).to(torch.bfloat16 if i % 3 else torch.float32)
+        d_logits = dev(logits)
+        alone = ops.moe_encode(d_data, d_logits, None, cf, top_k=k, gate_is_logits=True)
+        alone_out = ops.moe_decode(alone[4], alone[0], alone[1], top_k=k)
+        outs = tuple(torch.empty_like(t) if t.dtype != torch.uint64 else torch.empty(t.shape, dtype=torch.int64, device="cuda")
+                     for t in alone)
+        ws = torch.empty(ops.moe_encode_workspace_bytes(S, E, k), dtype=torch.uint8, device="cuda")
+        jobs.append((k, d_data, d_logits, alone, alone_out, outs, ws, torch.empty_like(alone_out), torch.cuda.Stream()))
+    torch.cuda.synchronize()
+    for _ in range(3):
+        for k, d_data, d_logits, _, _, outs, ws, dec, stream in jobs:
+            with torch.cuda.stream(stream):
+                ops.moe_encode(d_data, d_logits, None, cf, top_k=k, gate_is_logits=True, workspace=ws, out=outs)
+                ops.moe_decode(outs[4], outs[0], outs[1], top_k=k, out=dec)
+        torch.cuda.synchronize()
+        for k, _, _, alone, alone_out, outs, ws, dec, _ in jobs:
+            for a, b in zip(alone, outs):
+                assert torch.equal(a.view(torch.int64) if a.dtype == torch.uint64 else a, b)
+            assert torch.equal(alone_out, dec)
+            for t in outs:
+                t.zero_()
+            dec.zero_()
+        torch.cuda.synchronize()            # the clears run on the default stream

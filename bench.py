@@ -469,6 +469,28 @@ def bench_backward(ops, data, outs, dec, S, M, E, Cap, K, kept, iters):
     return res
 
 
+def bench_expert_input(ops, M, iters):
+    """moe_redispatch_expert_input at the shape one of 8 expert-parallel ranks would see for BASELINE config 4:
+    G = 8 source ranks, 4 local experts, capacity 5120, 4 token partitions, bf16 rows; every partition brings
+    about a quarter of the rows of each source rank.  Algorithmic bytes: received rows read once, the whole
+    [C, G, M] output written once (rows past the received ones are zero-filled)."""
+    import torch
+    P, G, LE, Cap = 4, 8, 4, 5120
+    gen = torch.Generator(device="cuda").manual_seed(9)
+    data = [torch.empty((Cap, G, M), device="cuda", dtype=torch.bfloat16).normal_(0, 1, generator=gen) for _ in range(P)]
+    rows = torch.randint(Cap // P - 200, Cap // P, (P, G * LE), generator=gen, device="cuda")
+    cnts = [(rows[p] * M).to(torch.int64) for p in range(P)]
+    out = torch.empty((Cap, G, M), device="cuda", dtype=torch.bfloat16)
+    fn = lambda: ops.moe_redispatch_expert_input(data, cnts, 1, LE, out=out)
+    fn()
+    ms = event_ms(fn, iters)
+    received = int(rows.view(P, G, LE)[:, :, 1].sum())
+    nbytes = received * M * 2 + Cap * G * M * 2
+    return {"workload": "P=%d G=%d LE=%d C=%d M=%d bf16, local expert 1" % (P, G, LE, Cap, M), "ms": round(ms, 4),
+            "received_rows": received, "algorithmic_bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1),
+            "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+
+
 def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -634,6 +656,7 @@ def main():
     del dec, outs
     torch.cuda.empty_cache()
     result["config4_partitioned"] = bench_config4_partitioned(ops, lib, capi, data, logits, S, M, E, cf, max(5, n // 2))
+    result["expert_input_merge"] = bench_expert_input(ops, M, max(10, n))
     result["pipeline"] = bench_pipeline(pkg, data, logits, S, M, E, cf, max(5, n // 2))
     result["other_configs"] = bench_other_configs(ops, max(10, n))
     del data

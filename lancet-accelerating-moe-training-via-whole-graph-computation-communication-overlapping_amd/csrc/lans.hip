@@ -47,7 +47,7 @@ struct LansTables {
   const int64_t* numel;        // [T]
   const int32_t* chunk_tensor; // [nchunks]
   const int32_t* tensor_first; // [T+1] first chunk of each tensor
-  float* partial;              // [3][nchunks]      (sweeps)
+  float* partial;              // [3][nchunks * kSweepSplit]  (sweeps: one sum per slice)
   uint64_t* part_word;         // [4][nchunks]      (resident schedule: epoch | fp32 sum of squares)
   uint64_t* norm_word;         // [4][T]            (resident schedule: epoch | fp32 norm)
   uint32_t* ticket;            // [1] next task; [1] error flag; [T] arrivals; [1] step epoch (resident schedule)
@@ -309,44 +309,69 @@ __global__ void lans_prepare_kernel(LansTables t, LansScalars sc) {
   if (threadIdx.x == 0 && blockIdx.x == 0) bias_corrections(sc, t.consts[0], t.consts[1]);
 }
 
-// The sweeps cover chunks [chunk_base, chunk_base + gridDim.x): all of them, or the ones the resident
+// The sweeps hand every chunk to kSweepSplit workgroups (a slice of kLansChunk / kSweepSplit elements each:
+// one float4 per thread and array).  Short workgroups in address order stream a few percent faster than
+// workgroups that loop over a whole chunk; the chunk stays the unit of the tables and of the resident kernel.
+#ifndef LANCET_SWEEP_SPLIT
+#define LANCET_SWEEP_SPLIT 8
+#endif
+constexpr int kSweepSplit = LANCET_SWEEP_SPLIT;
+constexpr int kSweepSlice = kLansChunk / kSweepSplit;
+
+// slice blockIdx.x % kSweepSplit of chunk chunk_base + blockIdx.x / kSweepSplit (n may be 0: past the tensor's end)
+__device__ __forceinline__ ChunkView slice_view(const LansTables& t, int chunk_base, int& slot) {
+  const int chunk = chunk_base + static_cast<int>(blockIdx.x / kSweepSplit);
+  const int sub = static_cast<int>(blockIdx.x % kSweepSplit);
+  slot = chunk * kSweepSplit + sub;
+  ChunkView c = chunk_view(t, chunk);
+  const int first = sub * kSweepSlice;
+  c.begin += first;
+  c.n = c.n > first ? (c.n - first < kSweepSlice ? c.n - first : kSweepSlice) : 0;
+  return c;
+}
+
+// The sweep over g covers chunks [chunk_base, chunk_base + gridDim.x), the other two
+// [chunk_base, chunk_base + gridDim.x / kSweepSplit): all of them, or the ones the resident
 // kernel takes (first sweep only), or the ones it leaves (tensors too large for it).
 __global__ __launch_bounds__(kLansThreads) void lans_norm_g_kernel(LansTables t, int chunk_base) {
   __shared__ float s_red[kLansThreads / kWave];
-  const int chunk = chunk_base + blockIdx.x;
+  const int chunk = chunk_base + blockIdx.x;  // a whole chunk per workgroup: this sweep only reads, and splitting it costs more in reductions than it gains
   const float sg = chunk_norm_g(t, chunk_view(t, chunk), s_red);
   if (threadIdx.x == 0) t.partial[chunk] = sg;
 }
 
 // per-tensor sqrt(sum of chunk partials) (cleanup, multi_tensor_lans.cu:169-185)
+// split: partial sums per chunk (1 after the sweep over g, kSweepSplit after the moments sweep)
 __global__ __launch_bounds__(kLansThreads) void lans_reduce_kernel(LansTables t, int first_norm, int tensor_base,
-                                                                   int tensor_end, int count) {
+                                                                   int tensor_end, int count, int split) {
   const int tensor = tensor_base + blockIdx.x * (kLansThreads / kWave) + threadIdx.x / kWave;
   if (tensor >= tensor_end) return;
   const int lo = t.tensor_first[tensor], hi = t.tensor_first[tensor + 1];
   for (int k = 0; k < count; ++k) {
-    const float* part = t.partial + static_cast<size_t>(k) * t.nchunks;
-    const float n = wave_norm(lo, hi, [&](int c) { return part[c]; });
+    const float* part = t.partial + static_cast<size_t>(k) * t.nchunks * split;
+    const float n = wave_norm(lo * split, hi * split, [&](int c) { return part[c]; });
     if (lane_id() == 0) t.norms[(first_norm + k) * t.T + tensor] = n;
   }
 }
 
 __global__ __launch_bounds__(kLansThreads) void lans_moments_kernel(LansTables t, LansScalars sc, int chunk_base) {
   __shared__ float s_red[kLansThreads / kWave];
-  const int chunk = chunk_base + blockIdx.x;
-  const ChunkView c = chunk_view(t, chunk);
+  int slot;
+  const ChunkView c = slice_view(t, chunk_base, slot);
   const LansElem el = make_elem(sc, t.norms[c.tensor], t.consts[0], t.consts[1]);
   float sp, sm, sg;
   chunk_moments(t, c, el, s_red, sp, sm, sg);
   if (threadIdx.x == 0) {
-    t.partial[chunk] = sp;
-    t.partial[t.nchunks + chunk] = sm;
-    t.partial[2 * static_cast<size_t>(t.nchunks) + chunk] = sg;
+    const size_t row = static_cast<size_t>(t.nchunks) * kSweepSplit;
+    t.partial[slot] = sp;
+    t.partial[row + slot] = sm;
+    t.partial[2 * row + slot] = sg;
   }
 }
 
 __global__ __launch_bounds__(kLansThreads) void lans_update_kernel(LansTables t, LansScalars sc, int chunk_base) {
-  const ChunkView c = chunk_view(t, chunk_base + blockIdx.x);
+  int slot;
+  const ChunkView c = slice_view(t, chunk_base, slot);
   const LansElem el = make_elem(sc, t.norms[c.tensor], t.consts[0], t.consts[1]);
   chunk_update(t, c, el, sc, t.norms[1 * t.T + c.tensor], t.norms[2 * t.T + c.tensor], t.norms[3 * t.T + c.tensor]);
 }
@@ -679,7 +704,7 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
     if (numels[i] < 0) return LANCET_ERR_SHAPE;
     nchunks64 += (numels[i] + kLansChunk - 1) / kLansChunk;
   }
-  if (nchunks64 > 0x7fffffff) return LANCET_ERR_SHAPE;
+  if (nchunks64 * kSweepSplit > 0x7fffffff) return LANCET_ERR_SHAPE;  // slices index the partial sums and the grids
   lancet_lans_plan* pl = new (std::nothrow) lancet_lans_plan();
   if (!pl) return static_cast<int>(hipErrorOutOfMemory);
   pl->magic = kPlanMagic;
@@ -699,7 +724,7 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
   const size_t o_numel = off;     off = align_up(off + T * sizeof(int64_t), 256);
   const size_t o_ctensor = off;   off = align_up(off + (n ? n : 1) * sizeof(int32_t), 256);
   const size_t o_first = off;     off = align_up(off + (T + 1) * sizeof(int32_t), 256);
-  const size_t o_partial = off;   off = align_up(off + 3 * (n ? n : 1) * sizeof(float), 256);
+  const size_t o_partial = off;   off = align_up(off + 3 * (n ? n : 1) * kSweepSplit * sizeof(float), 256);
   const size_t o_norms = off;     off = align_up(off + 4 * T * sizeof(float), 256);
   const size_t o_consts = off;    off = align_up(off + 2 * sizeof(float), 256);
   const size_t o_words = off;     off = align_up(off + 4 * ((n ? n : 1) + T) * sizeof(uint64_t), 256);
@@ -856,7 +881,7 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
     const int grid = std::min(pl->resident_grid, pl->n_res_chunks);
     const int per_block = kLansThreads / kWave;
     lans_norm_g_kernel<<<pl->n_res_chunks, kLansThreads, 0, st>>>(t, 0);
-    lans_reduce_kernel<<<(pl->n_res_tensors + per_block - 1) / per_block, kLansThreads, 0, st>>>(t, 0, 0, pl->n_res_tensors, 1);
+    lans_reduce_kernel<<<(pl->n_res_tensors + per_block - 1) / per_block, kLansThreads, 0, st>>>(t, 0, 0, pl->n_res_tensors, 1, 1);
     lans_resident_kernel<<<grid, kLansThreads, 0, st>>>(t, sc);
     chunk_base = pl->n_res_chunks;
     tensor_base = pl->n_res_tensors;
@@ -867,10 +892,10 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
     const int rblocks = (T - tensor_base + per_block - 1) / per_block;
     lans_prepare_kernel<<<1, 64, 0, st>>>(t, sc);
     lans_norm_g_kernel<<<nsweep, kLansThreads, 0, st>>>(t, chunk_base);
-    lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 0, tensor_base, T, 1);
-    lans_moments_kernel<<<nsweep, kLansThreads, 0, st>>>(t, sc, chunk_base);
-    lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 1, tensor_base, T, 3);
-    lans_update_kernel<<<nsweep, kLansThreads, 0, st>>>(t, sc, chunk_base);
+    lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 0, tensor_base, T, 1, 1);
+    lans_moments_kernel<<<nsweep * kSweepSplit, kLansThreads, 0, st>>>(t, sc, chunk_base);
+    lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 1, tensor_base, T, 3, kSweepSplit);
+    lans_update_kernel<<<nsweep * kSweepSplit, kLansThreads, 0, st>>>(t, sc, chunk_base);
   }
   return static_cast<int>(hipGetLastError());
 }

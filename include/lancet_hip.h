@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define LANCET_ABI_VERSION 2
+#define LANCET_ABI_VERSION 3
 
 /* element type of token rows */
 #define LANCET_F32 0

@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol(pkg):
     for n in names:
         assert hasattr(lib, n), "liblancet_hip.so does not export %s" % n
     assert sorted(pkg.capi.SIGNATURES) == names, "capi.SIGNATURES and the header disagree"
-    assert lib.lancet_abi_version() == pkg.capi.ABI_VERSION == 2
+    assert lib.lancet_abi_version() == pkg.capi.ABI_VERSION == 3
 
 
 def test_capacity_formula(pkg):

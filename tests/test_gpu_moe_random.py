@@ -77,3 +77,26 @@ def test_encode_bpr_random(pkg, seed):
         np.testing.assert_array_equal(to_np(elems), want[3])
         np.testing.assert_array_equal(to_np(g), want[0])
         np.testing.assert_array_equal(to_np(disp), want[4])
+
+
+@pytest.mark.parametrize("S,E,k,cf,skew", [(300001, 512, 2, 1.0, 3.0), (262144, 2, 2, 0.3, 0.0), (100000, 100, 1, 2.5, 1.0),
+                                           (65536, 256, 2, 0.3, 3.0), (300001, 3, 1, 1.0, 0.0), (262144, 64, 1, 0.3, 3.0)])
+def test_routing_over_many_tiles(pkg, S, E, k, cf, skew):
+    """Long batches: more than a thousand scan tiles, look-back windows of a couple of rows (E = 512, top-2) up
+    to hundreds, a crowded expert, chained used capacity; every output against the oracle (M = 4 keeps the
+    oracle's row movement small)."""
+    rng = np.random.default_rng(S + E + k)
+    M = 4
+    logits = rng.standard_normal((S, E), dtype=np.float32)
+    logits[:, rng.integers(E)] += np.float32(skew)
+    data = rng.standard_normal((S, M), dtype=np.float32)
+    used0 = np.zeros(E, np.int32)
+    if k == 1:
+        used0 = rng.integers(0, max(mo.capacity(S, E, cf), 1) + 1, E).astype(np.int32)
+    want = (mo.moe_encode_top2 if k == 2 else mo.moe_encode)(data, logits, used0, cf, gate_is_logits=True, fast_scatter=True)
+    got = pkg.ops.moe_encode(dev(data), dev(logits), dev(used0), cf, top_k=k, gate_is_logits=True)
+    np.testing.assert_array_equal(to_np(got[1]), want[1])
+    np.testing.assert_array_equal(to_np(got[2]), want[2])
+    np.testing.assert_array_equal(to_np(got[3]), want[3])
+    np.testing.assert_allclose(to_np(got[0]), want[0], rtol=1e-5, atol=0)
+    np.testing.assert_array_equal(to_np(got[4]), want[4])

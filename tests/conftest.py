@@ -16,8 +16,14 @@ def pytest_configure(config):
 
 
 def load_pkg():
-    """The package directory name is not a Python identifier; importlib takes it as is."""
-    return importlib.import_module(PKG_NAME)
+    """The package directory name is not a Python identifier; importlib takes it as is.  The native libraries
+    are normally built beforehand (__graft_entry__.build()); a checkout in which nothing is built yet gets
+    them built once here, so that the tests can load them (the package itself never builds or falls back)."""
+    pkg = importlib.import_module(PKG_NAME)
+    ops_lib = os.path.join(os.path.dirname(pkg.capi.LIB_PATH), "liblancet_raf_ops.so")
+    if not os.path.exists(pkg.capi.LIB_PATH) or not os.path.exists(ops_lib):
+        importlib.import_module(PKG_NAME + ".build").build_all()
+    return pkg
 
 
 @pytest.fixture(scope="session")

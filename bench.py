@@ -376,10 +376,13 @@ def bench_pipeline(pkg, data, logits, S, M, E, cf, iters):
     layer = pkg.pipeline.PartitionedMoeLayer(S, M, E, 4, cf, dtype=data.dtype, gate_is_logits=True)
     layer.run_serial(data, logits)
     layer.run(data, logits)
+    layer.run_routed_once(data, logits)
     t_serial = event_ms(lambda: layer.run_serial(data, logits), iters)
     t_piped = event_ms(lambda: layer.run(data, logits), iters)
+    t_once = event_ms(lambda: layer.run_routed_once(data, logits), iters)
     return {"workload": "4 partitions, top-1, S=%d M=%d E=%d C=%d" % (S, M, E, layer.C),
             "ms_one_stream": round(t_serial, 4), "ms_three_streams": round(t_piped, 4),
+            "ms_routed_once_three_streams": round(t_once, 4),
             "note": "every stage but routing is HBM-bound on one GPU, so the streams share one memory system and "
                     "the event hops cost more than the overlap returns; the pattern pays when the exchange is a real "
                     "all-to-all over xGMI"}

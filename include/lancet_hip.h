@@ -217,6 +217,30 @@ int lancet_memcpy_cont_to_sparse_3d(const void* src, void* dst, const uint64_t* 
                                     int scale_element_size_by, int shrink_element_size_by, int dtype,
                                     unsigned flags, lancet_stream_t stream);
 
+/* The same copies on row ranges (no counterpart in the reference): block b's valid elements are
+ * [starts_per_dim[b*stride + offset], + nelements_per_dim[b*stride + offset]) instead of the block's first ones.
+ * For a buffer that several token partitions share (lancet_moe_scatter_tokens): what one partition owns is, per
+ * expert, a run of rows behind those of the partitions before it, and these copies pack that run for the
+ * partition's exchange and unpack what comes back.  Nothing outside the ranges is touched. */
+int lancet_memcpy_sparse_ranges_to_cont_3d(const void* src, void* dst, const uint64_t* nelements_per_dim,
+                                           const uint64_t* starts_per_dim, int64_t n_counts, int nelements_stride,
+                                           int nelements_offset, int axis, int64_t dim0, int64_t dim1, int64_t dim2,
+                                           int64_t dst_elems, int dtype, lancet_stream_t stream);
+int lancet_memcpy_cont_to_sparse_ranges_3d(const void* src, void* dst, const uint64_t* nelements_per_dim,
+                                           const uint64_t* starts_per_dim, int64_t n_counts, int nelements_stride,
+                                           int nelements_offset, int axis, int64_t dim0, int64_t dim1, int64_t dim2,
+                                           int64_t src_elems, int dtype, lancet_stream_t stream);
+/* Row ranges of n_partitions equal token partitions inside a whole-batch routing (indices_locations
+ * [2, top_k * S_total] of lancet_moe_route over all tokens): starts and counts are [top_k * n_partitions, E]
+ * uint64 in ELEMENTS (rows x M), rows ordered slot-major, then partition, which is the order in which the rows
+ * follow each other inside every expert (the capacity order moe_merge_masks uses, moe.cc:772-802).
+ * counts[j*P + p][e] = M x kept tokens of partition p whose slot j went to expert e; starts = the sum of the counts
+ * before it.  counts rows are what elements_per_expert would be for the partition's own encode. */
+size_t lancet_moe_partition_ranges_workspace_bytes(int top_k, int n_partitions, int64_t E);
+int lancet_moe_partition_ranges(const int32_t* indices_locations, int64_t S_total, int top_k, int n_partitions,
+                                int64_t E, int64_t M, uint64_t* starts, uint64_t* counts, void* workspace,
+                                size_t workspace_bytes, lancet_stream_t stream);
+
 /* ---- backward ops (raf.op.moe_encode_dx / _dg, raf.op.moe_decode_dx / _dg) ------------------
  * Gradients wired by src/op/grad/moe.cc:30-93.  Gate-side gradients are fp32 like gates_s; top_k = 2
  * takes the slot-major layout of the forward ops.

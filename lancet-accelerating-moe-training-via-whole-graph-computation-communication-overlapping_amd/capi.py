@@ -56,6 +56,10 @@ SIGNATURES = {
                                      _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "lancet_moe_scatter_tokens": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _u32, _vp, _vp]),
     "lancet_moe_decode_tokens": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp]),
+    "lancet_memcpy_sparse_ranges_to_cont_3d": (_int, [_vp, _vp, _vp, _vp, _i64, _int, _int, _int, _i64, _i64, _i64, _i64, _int, _vp]),
+    "lancet_memcpy_cont_to_sparse_ranges_3d": (_int, [_vp, _vp, _vp, _vp, _i64, _int, _int, _int, _i64, _i64, _i64, _i64, _int, _vp]),
+    "lancet_moe_partition_ranges_workspace_bytes": (_sz, [_int, _int, _i64]),
+    "lancet_moe_partition_ranges": (_int, [_vp, _i64, _int, _int, _i64, _i64, _vp, _vp, _vp, _sz, _vp]),
     "lancet_debug_stream": (_int, [_int, _vp, _vp, _sz, _vp]),
     "lancet_moe_decode": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp]),
     "lancet_moe_redispatch_expert_input": (_int, [C.POINTER(_vp), C.POINTER(_vp), _int, _int, _int, _i64, _i64, _i64,

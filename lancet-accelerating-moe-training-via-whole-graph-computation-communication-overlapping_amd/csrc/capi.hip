@@ -366,7 +366,7 @@ extern "C" int lancet_moe_redispatch_expert_input(const void* const* data, const
 
 // ---- sparse <-> packed copies ---------------------------------------------------------------
 namespace {
-int sparse_copy(const void* src, void* dst, const uint64_t* counts, int64_t n_counts, int stride, int offset, int axis,
+int sparse_copy(const void* src, void* dst, const uint64_t* counts, const uint64_t* starts, int64_t n_counts, int stride, int offset, int axis,
                 int64_t dim0, int64_t dim1, int64_t dim2, int64_t cont_elems, int scale, int shrink, int dtype,
                 unsigned flags, bool to_cont, lancet_stream_t stream) {
   const int eb = elem_bytes(dtype);
@@ -382,8 +382,8 @@ int sparse_copy(const void* src, void* dst, const uint64_t* counts, int64_t n_co
   if (nblocks == 0 || other * dim2 == 0) return LANCET_OK;
   if (!src || !dst || !counts) return LANCET_ERR_NULL;
   if ((nblocks - 1) * stride + offset >= n_counts) return LANCET_ERR_SHAPE;
-  if (misaligned(src, eb) || misaligned(dst, eb) || misaligned(counts, 8)) return LANCET_ERR_ALIGN;
-  return rc(run_sparse_copy_3d(src, dst, counts, stride, offset, axis, static_cast<int>(dim0), static_cast<int>(dim1),
+  if (misaligned(src, eb) || misaligned(dst, eb) || misaligned(counts, 8) || misaligned(starts, 8)) return LANCET_ERR_ALIGN;
+  return rc(run_sparse_copy_3d(src, dst, counts, starts, stride, offset, axis, static_cast<int>(dim0), static_cast<int>(dim1),
                                static_cast<int>(dim2), static_cast<uint64_t>(cont_elems), static_cast<uint64_t>(scale),
                                static_cast<uint64_t>(shrink), to_cont, (flags & LANCET_ZERO_TAIL) != 0, eb, S_(stream)));
 }
@@ -394,7 +394,7 @@ extern "C" int lancet_memcpy_sparse_to_cont_3d(const void* src, void* dst, const
                                                int64_t dim0, int64_t dim1, int64_t dim2, int64_t dst_elems,
                                                int scale_element_size_by, int shrink_element_size_by, int dtype,
                                                lancet_stream_t stream) {
-  return sparse_copy(src, dst, nelements_per_dim, n_counts, nelements_stride, nelements_offset, axis, dim0, dim1, dim2,
+  return sparse_copy(src, dst, nelements_per_dim, nullptr, n_counts, nelements_stride, nelements_offset, axis, dim0, dim1, dim2,
                      dst_elems, scale_element_size_by, shrink_element_size_by, dtype, 0u, true, stream);
 }
 
@@ -403,8 +403,75 @@ extern "C" int lancet_memcpy_cont_to_sparse_3d(const void* src, void* dst, const
                                                int64_t dim0, int64_t dim1, int64_t dim2, int64_t src_elems,
                                                int scale_element_size_by, int shrink_element_size_by, int dtype,
                                                unsigned flags, lancet_stream_t stream) {
-  return sparse_copy(src, dst, nelements_per_dim, n_counts, nelements_stride, nelements_offset, axis, dim0, dim1, dim2,
+  return sparse_copy(src, dst, nelements_per_dim, nullptr, n_counts, nelements_stride, nelements_offset, axis, dim0, dim1, dim2,
                      src_elems, scale_element_size_by, shrink_element_size_by, dtype, flags, false, stream);
+}
+
+extern "C" int lancet_memcpy_sparse_ranges_to_cont_3d(const void* src, void* dst, const uint64_t* nelements_per_dim,
+                                                      const uint64_t* starts_per_dim, int64_t n_counts,
+                                                      int nelements_stride, int nelements_offset, int axis, int64_t dim0,
+                                                      int64_t dim1, int64_t dim2, int64_t dst_elems, int dtype,
+                                                      lancet_stream_t stream) {
+  if (!starts_per_dim && dim0 > 0 && dim1 > 0 && dim2 > 0) return LANCET_ERR_NULL;
+  return sparse_copy(src, dst, nelements_per_dim, starts_per_dim, n_counts, nelements_stride, nelements_offset, axis, dim0,
+                     dim1, dim2, dst_elems, 1, 1, dtype, 0u, true, stream);
+}
+
+extern "C" int lancet_memcpy_cont_to_sparse_ranges_3d(const void* src, void* dst, const uint64_t* nelements_per_dim,
+                                                      const uint64_t* starts_per_dim, int64_t n_counts,
+                                                      int nelements_stride, int nelements_offset, int axis, int64_t dim0,
+                                                      int64_t dim1, int64_t dim2, int64_t src_elems, int dtype,
+                                                      lancet_stream_t stream) {
+  if (!starts_per_dim && dim0 > 0 && dim1 > 0 && dim2 > 0) return LANCET_ERR_NULL;
+  return sparse_copy(src, dst, nelements_per_dim, starts_per_dim, n_counts, nelements_stride, nelements_offset, axis, dim0,
+                     dim1, dim2, src_elems, 1, 1, dtype, 0u, false, stream);
+}
+
+// ---- row ranges of token partitions inside a whole-batch routing --------------------------------
+namespace {
+__global__ __launch_bounds__(256) void partition_ranges_kernel(const uint32_t* __restrict__ counts, int Q, int E, int64_t M,
+                                                               uint64_t* __restrict__ starts, uint64_t* __restrict__ cnts) {
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= E) return;
+  uint64_t run = 0;
+  for (int q = 0; q < Q; ++q) {  // capacity order: slot-major, then partition
+    const uint64_t k = counts[static_cast<size_t>(q) * E + e];
+    starts[static_cast<size_t>(q) * E + e] = run * static_cast<uint64_t>(M);
+    cnts[static_cast<size_t>(q) * E + e] = k * static_cast<uint64_t>(M);
+    run += k;
+  }
+}
+}  // namespace
+
+extern "C" size_t lancet_moe_partition_ranges_workspace_bytes(int top_k, int n_partitions, int64_t E) {
+  if (top_k < 1 || top_k > 2 || n_partitions < 1 || E < 1) return 0;
+  return static_cast<size_t>(top_k) * n_partitions * E * sizeof(uint32_t);
+}
+
+extern "C" int lancet_moe_partition_ranges(const int32_t* indices_locations, int64_t S_total, int top_k, int n_partitions,
+                                           int64_t E, int64_t M, uint64_t* starts, uint64_t* counts, void* workspace,
+                                           size_t workspace_bytes, lancet_stream_t stream) {
+  if ((!indices_locations && S_total > 0) || !starts || !counts) return LANCET_ERR_NULL;
+  if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
+  if (int r = check_dims(S_total, M, E, 0)) return r;
+  if (n_partitions < 1 || top_k * n_partitions > LANCET_MAX_PARTITIONS || S_total % n_partitions != 0)
+    return LANCET_ERR_PARTITION;
+  if (!workspace || workspace_bytes < lancet_moe_partition_ranges_workspace_bytes(top_k, n_partitions, E))
+    return LANCET_ERR_WORKSPACE;
+  if (misaligned(indices_locations, 4) || misaligned(starts, 8) || misaligned(counts, 8) || misaligned(workspace, 4))
+    return LANCET_ERR_ALIGN;
+  const int Q = top_k * n_partitions;
+  const int64_t Sp = S_total / n_partitions;
+  PtrTable t;
+  for (int q = 0; q < kMaxPartitions; ++q) t.p[q] = nullptr;
+  for (int j = 0; j < top_k; ++j)
+    for (int p = 0; p < n_partitions; ++p) t.p[j * n_partitions + p] = indices_locations + j * S_total + p * Sp;
+  uint32_t* hist = static_cast<uint32_t*>(workspace);
+  hipError_t e = run_count_experts(t, Q, static_cast<int>(Sp), static_cast<int>(E), hist, S_(stream));
+  if (e != hipSuccess) return rc(e);
+  partition_ranges_kernel<<<static_cast<unsigned>((E + 255) / 256), 256, 0, S_(stream)>>>(hist, Q, static_cast<int>(E), M,
+                                                                                         starts, counts);
+  return rc(hipGetLastError());
 }
 
 // ---- backward ops -------------------------------------------------------------------

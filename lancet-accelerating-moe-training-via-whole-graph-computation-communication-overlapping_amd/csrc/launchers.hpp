@@ -75,8 +75,9 @@ hipError_t run_redispatch_expert_input(const PtrTable& bufs, const void* const* 
 
 // ---- sparse <-> packed copies (sparse_copy.hip) -----------------------------------------
 // counts[b*stride + offset] elements of block b along `axis` (0 or 1) of a [dim0, dim1, dim2] buffer;
-// cont_cap = elements the packed stream holds.  to_cont: buffer -> stream.
-hipError_t run_sparse_copy_3d(const void* src, void* dst, const uint64_t* counts, int stride, int offset, int axis,
+// cont_cap = elements the packed stream holds.  to_cont: buffer -> stream.  starts (may be null = zeros): first
+// element of block b that takes part, read like the counts.
+hipError_t run_sparse_copy_3d(const void* src, void* dst, const uint64_t* counts, const uint64_t* starts, int stride, int offset, int axis,
                               int dim0, int dim1, int dim2, uint64_t cont_cap, uint64_t scale, uint64_t shrink,
                               bool to_cont, bool zero_tail, int elem_bytes, hipStream_t st);
 

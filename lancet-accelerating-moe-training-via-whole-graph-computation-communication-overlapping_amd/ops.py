@@ -473,6 +473,55 @@ def memcpy_cont_to_sparse_3d(src, dst, nelements_per_dim, nelements_stride=1, ne
     return dst
 
 
+def memcpy_sparse_ranges_to_cont_3d(src, dst, nelements_per_dim, starts_per_dim, nelements_stride=1, nelements_offset=0,
+                                    axis=0):
+    """memcpy_sparse_to_cont_3d on row ranges: block b contributes its elements [start_b, start_b + n_b) (both
+    arrays indexed b*stride + offset).  Packs what one token partition owns inside a shared buffer."""
+    lib = capi.load()
+    (d0, d1, d2), n_dst, n_cnt = _sparse_copy_args(src, dst, nelements_per_dim, nelements_stride, nelements_offset, axis)
+    _dev(starts_per_dim, "starts_per_dim")
+    _need(starts_per_dim.dtype == nelements_per_dim.dtype and starts_per_dim.numel() == n_cnt and
+          starts_per_dim.is_contiguous(), "starts_per_dim must match nelements_per_dim")
+    st = lib.lancet_memcpy_sparse_ranges_to_cont_3d(_p(src), _p(dst), _p(nelements_per_dim), _p(starts_per_dim), n_cnt,
+                                                    int(nelements_stride), int(nelements_offset), int(axis), d0, d1, d2,
+                                                    n_dst, _dtype_code(src), _stream())
+    capi.check(st, "lancet_memcpy_sparse_ranges_to_cont_3d")
+    return dst
+
+
+def memcpy_cont_to_sparse_ranges_3d(src, dst, nelements_per_dim, starts_per_dim, nelements_stride=1, nelements_offset=0,
+                                    axis=0):
+    """The inverse of memcpy_sparse_ranges_to_cont_3d: only the ranges are written."""
+    lib = capi.load()
+    (d0, d1, d2), n_src, n_cnt = _sparse_copy_args(dst, src, nelements_per_dim, nelements_stride, nelements_offset, axis)
+    _dev(starts_per_dim, "starts_per_dim")
+    _need(starts_per_dim.dtype == nelements_per_dim.dtype and starts_per_dim.numel() == n_cnt and
+          starts_per_dim.is_contiguous(), "starts_per_dim must match nelements_per_dim")
+    st = lib.lancet_memcpy_cont_to_sparse_ranges_3d(_p(src), _p(dst), _p(nelements_per_dim), _p(starts_per_dim), n_cnt,
+                                                    int(nelements_stride), int(nelements_offset), int(axis), d0, d1, d2,
+                                                    n_src, _dtype_code(dst), _stream())
+    capi.check(st, "lancet_memcpy_cont_to_sparse_ranges_3d")
+    return dst
+
+
+def moe_partition_ranges(indices_locations, n_partitions, n_experts, M, top_k=1, workspace=None, out=None):
+    """Row ranges of n_partitions equal token partitions inside a whole-batch routing: returns (starts, counts), each
+    int64 [top_k * n_partitions, E] in elements (rows x M), rows ordered slot-major then partition."""
+    lib = capi.load()
+    S_total = _check_indloc(indices_locations, top_k)
+    _need(n_partitions >= 1 and S_total % n_partitions == 0, "the token count must divide into n_partitions")
+    Q = top_k * int(n_partitions)
+    dev = indices_locations.device
+    if out is None:
+        out = (torch.empty((Q, n_experts), dtype=torch.int64, device=dev), torch.empty((Q, n_experts), dtype=torch.int64, device=dev))
+    starts, counts = out
+    ws = _workspace(lib.lancet_moe_partition_ranges_workspace_bytes(top_k, int(n_partitions), int(n_experts)), dev, workspace)
+    st = lib.lancet_moe_partition_ranges(_p(indices_locations), S_total, top_k, int(n_partitions), int(n_experts), int(M),
+                                         _p(starts), _p(counts), _p(ws), ws.numel(), _stream())
+    capi.check(st, "lancet_moe_partition_ranges")
+    return starts, counts
+
+
 # ------------------------------------------------------------------------------------ LANS
 class LansPlan:
     """Owns the native plan of one parameter set (what the reference's LansImpl constructor

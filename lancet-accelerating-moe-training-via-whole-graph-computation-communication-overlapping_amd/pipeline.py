@@ -46,6 +46,18 @@ class PartitionedMoeLayer:
         self.routing = torch.cuda.Stream(device=dev)
         self.compute = torch.cuda.Stream(device=dev)
         self.exchange = torch.cuda.Stream(device=dev)
+        # the same layer with the batch routed once (run_routed_once): one send and one receive buffer that the
+        # partitions share, each owning a run of rows per expert
+        self.Ct = ops.moe_capacity(S, E, float(capacity_factor))
+        self.whole = (torch.empty(S, dtype=torch.float32, device=dev), torch.empty((2, S), dtype=torch.int32, device=dev),
+                      torch.empty(E, dtype=torch.int32, device=dev), torch.empty(E, dtype=torch.int64, device=dev))
+        self.whole_ws = torch.empty(ops.moe_encode_workspace_bytes(S, E, 1), dtype=torch.uint8, device=dev)
+        self.ranges = (torch.empty((P, E), dtype=torch.int64, device=dev), torch.empty((P, E), dtype=torch.int64, device=dev))
+        self.ranges_ws = torch.empty(max(4, P * E * 4), dtype=torch.uint8, device=dev)
+        self.send = torch.empty((E, self.Ct, M), dtype=dtype, device=dev)
+        self.recv_all = torch.empty((E, self.Ct, M), dtype=dtype, device=dev)
+        self.no_rows = torch.empty((0, M), dtype=dtype, device=dev)
+        self.routed_all = torch.cuda.Event()
         self.routed = [torch.cuda.Event() for _ in range(P)]
         self.encoded = [torch.cuda.Event() for _ in range(P)]
         self.received = [torch.cuda.Event() for _ in range(P)]
@@ -117,6 +129,50 @@ class PartitionedMoeLayer:
         with torch.cuda.stream(self.compute):
             self.compute.wait_event(self.received[self.P - 1])
             self._decode(self.P - 1)
+            done = torch.cuda.Event()
+            done.record(self.compute)
+        cur.wait_event(done)
+        return self.out
+
+    def run_routed_once(self, data, gate):
+        """The partitions as token ranges of ONE routing of the whole batch (the chained partition encodes, merged,
+        are that routing): routing and the partitions' row ranges first, then per partition the scatter of its tokens
+        into the shared send buffer, the exchange of the rows it owns there (packed and unpacked at its ranges) and
+        the decode of its tokens from the shared receive buffer.  Same streams as `run`; the output equals
+        moe_decode(moe_encode(whole batch))."""
+        cur = torch.cuda.current_stream()
+        start = torch.cuda.Event()
+        start.record(cur)
+        for s in (self.routing, self.compute, self.exchange):
+            s.wait_event(start)
+        g, il, used, _ = self.whole
+        starts, counts = self.ranges
+        with torch.cuda.stream(self.routing):
+            ops.moe_route(gate, None, self.M, self.cf / self.P, gate_is_logits=self.gate_is_logits,
+                          workspace=self.whole_ws, out=self.whole)
+            ops.moe_partition_ranges(il, self.P, self.E, self.M, workspace=self.ranges_ws, out=self.ranges)
+            # rows of the receive buffer no partition owns: cleared once (a scatter of no tokens is only the tail fill)
+            ops.moe_scatter_tokens(self.no_rows, il, None, used, 0, self.E, self.Ct, zero_tail=True, out=self.recv_all)
+            self.routed_all.record(self.routing)
+        self.compute.wait_event(self.routed_all)
+        self.exchange.wait_event(self.routed_all)
+        for i in range(self.P):
+            sl = slice(i * self.Sp, (i + 1) * self.Sp)
+            with torch.cuda.stream(self.compute):
+                ops.moe_scatter_tokens(data[sl], il, None, used, i * self.Sp, self.E, self.Ct, zero_tail=False, out=self.send)
+                self.encoded[i].record(self.compute)
+                if i > 0:
+                    self.compute.wait_event(self.received[i - 1])
+                    ops.moe_decode_tokens(self.recv_all, g, il, (i - 1) * self.Sp, self.Sp,
+                                          out=self.out[(i - 1) * self.Sp:i * self.Sp])
+            with torch.cuda.stream(self.exchange):
+                self.exchange.wait_event(self.encoded[i])
+                ops.memcpy_sparse_ranges_to_cont_3d(self.send, self.wire[i], counts[i], starts[i], axis=0)
+                ops.memcpy_cont_to_sparse_ranges_3d(self.wire[i], self.recv_all, counts[i], starts[i], axis=0)
+                self.received[i].record(self.exchange)
+        with torch.cuda.stream(self.compute):
+            self.compute.wait_event(self.received[self.P - 1])
+            ops.moe_decode_tokens(self.recv_all, g, il, (self.P - 1) * self.Sp, self.Sp, out=self.out[(self.P - 1) * self.Sp:])
             done = torch.cuda.Event()
             done.record(self.compute)
         cur.wait_event(done)

@@ -465,3 +465,58 @@ def memcpy_cont_to_sparse_3d(src, dst, nelements_per_dim, stride=1, offset=0, ax
         else:
             out[:, b, :] = blk.reshape(out.shape[0], out.shape[2])
     return out
+
+
+
+# --------------------------------------------------------------------------
+# Row ranges of token partitions inside a whole-batch routing, and the sparse copies on ranges.  No counterpart in
+# the reference; pinned in tests/test_oracle_moe.py by the identity they exist for: packing the ranges of
+# partition p out of the whole-batch buffer gives what packing partition p's own chained encode gives
+# (tests/python/op/cuda/test_cuda_moe.py:384-471 protocol + sparse_memcpy.cu semantics).
+# --------------------------------------------------------------------------
+def moe_partition_ranges(indloc, n_partitions, n_experts, M, k=1):
+    """(starts, counts) uint64 [k*P, E] in elements: counts[j*P+p][e] = M * #kept tokens of partition p with slot-j
+    expert e; starts = running sum over the rows before (slot-major, then partition: the capacity order)."""
+    S = indloc.shape[1] // k
+    Sp = S // n_partitions
+    Q = k * n_partitions
+    counts = np.zeros((Q, n_experts), np.uint64)
+    for j in range(k):
+        for p in range(n_partitions):
+            idx = indloc[0, j * S + p * Sp: j * S + (p + 1) * Sp]
+            kept = idx[(idx >= 0) & (idx < n_experts)]
+            counts[j * n_partitions + p] = np.bincount(kept, minlength=n_experts).astype(np.uint64) * np.uint64(M)
+    starts = np.zeros_like(counts)
+    starts[1:] = np.cumsum(counts, axis=0, dtype=np.uint64)[:-1]
+    return starts, counts
+
+
+def memcpy_sparse_ranges_to_cont_3d(src, dst, counts, starts, axis=0):
+    """Packs elements [start_b, start_b + n_b) of every block b (stream order of the block) into dst."""
+    out = np.array(dst, copy=True).reshape(-1)
+    off = 0
+    for b in range(src.shape[axis]):
+        blk = _sparse_block_view(src, axis, b)
+        s0 = min(int(starts[b]), blk.size)
+        n = max(0, min(int(counts[b]), blk.size - s0, out.size - off))
+        out[off:off + n] = blk[s0:s0 + n]
+        off += int(counts[b])
+    return out
+
+
+def memcpy_cont_to_sparse_ranges_3d(src, dst, counts, starts, axis=0):
+    """The inverse: only the ranges of dst are written."""
+    out = np.array(dst, copy=True)
+    flat = np.asarray(src).reshape(-1)
+    off = 0
+    for b in range(out.shape[axis]):
+        blk = np.array(_sparse_block_view(out, axis, b), copy=True)
+        s0 = min(int(starts[b]), blk.size)
+        n = max(0, min(int(counts[b]), blk.size - s0, flat.size - off))
+        blk[s0:s0 + n] = flat[off:off + n]
+        if axis == 0:
+            out[b] = blk.reshape(out.shape[1], out.shape[2])
+        else:
+            out[:, b, :] = blk.reshape(out.shape[0], out.shape[2])
+        off += int(counts[b])
+    return out

@@ -78,6 +78,18 @@ def test_workspace_sizes_and_argument_rejection(pkg):
     assert dc(one, one, one, 64, 57, 8, 4, 2, 4, 1, capi.F32, one, None) == capi.ERR_SHAPE
     assert dc(one, None, one, 64, 0, 8, 4, 2, 4, 1, capi.F32, one, None) == capi.ERR_NULL
     assert dc(one, one, one, 64, 0, 8, 4, 2, 4, 1, capi.F32, C.c_void_p(6), None) == capi.ERR_ALIGN
+    # row ranges of token partitions
+    pr = lib.lancet_moe_partition_ranges
+    assert lib.lancet_moe_partition_ranges_workspace_bytes(2, 4, 8) == 2 * 4 * 8 * 4
+    assert pr(one, 64, 1, 3, 8, 4, one, one, one, 1 << 20, None) == capi.ERR_PARTITION      # 64 tokens, 3 partitions
+    assert pr(one, 64, 2, 40, 8, 4, one, one, one, 1 << 20, None) == capi.ERR_PARTITION     # 2 x 40 > LANCET_MAX_PARTITIONS
+    assert pr(one, 64, 3, 4, 8, 4, one, one, one, 1 << 20, None) == capi.ERR_TOPK
+    assert pr(one, 64, 1, 4, 8, 4, one, one, one, 8, None) == capi.ERR_WORKSPACE
+    assert pr(one, 64, 1, 4, 8, 4, None, one, one, 1 << 20, None) == capi.ERR_NULL
+    rc_ = lib.lancet_memcpy_sparse_ranges_to_cont_3d
+    assert rc_(one, one, one, None, 8, 1, 0, 0, 4, 4, 4, 64, capi.F32, None) == capi.ERR_NULL       # ranges need starts
+    assert rc_(one, one, one, C.c_void_p(20), 8, 1, 0, 0, 4, 4, 4, 64, capi.F32, None) == capi.ERR_ALIGN
+    assert lib.lancet_memcpy_cont_to_sparse_ranges_3d(one, one, one, one, 8, 1, 0, 2, 4, 4, 4, 64, capi.F32, None) == capi.ERR_SHAPE
     assert lib.lancet_lans_plan_destroy(None) == capi.ERR_PLAN
     assert "workspace" in capi.status_string(capi.ERR_WORKSPACE)
 

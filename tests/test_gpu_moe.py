@@ -674,3 +674,61 @@ def test_rows_of_every_split(pkg, M, dt, k):
 
     same(ops.moe_decode(got[4], got[0], got[1], top_k=k), mo.moe_decode(want[4], want[0], want[1], k=k))
     same(ops.moe_encode_dx(got[4], got[1], top_k=k), mo.moe_encode_dx(want[4], want[1], k))
+
+
+# ----------------------------------------------------------------------------- row ranges of token partitions
+@pytest.mark.parametrize("k,dt,P,S,M,E", [(1, "f32", 4, 2048, 64, 8), (2, "bf16", 4, 2048, 64, 8), (2, "f32", 3, 999, 5, 5),
+                                          (1, "f16", 2, 512, 24, 16), (2, "bf16", 8, 4096, 40, 32)])
+def test_partition_ranges_and_range_copies(pkg, k, dt, P, S, M, E):
+    """lancet_moe_partition_ranges and the sparse copies on ranges against the oracle, and the round trip they are
+    for: every partition's rows packed out of the shared buffer and unpacked into an empty one rebuild the buffer."""
+    ops = pkg.ops
+    S -= S % P
+    cf = 0.7
+    data, logits = make_inputs(S + 3 * k, S, M, E, zipf_bias=True)
+    gate = mo.softmax_rows(logits)
+    rows = rows_as_oracle(data, dt)
+    want = (mo.moe_encode_top2 if k == 2 else mo.moe_encode)(rows, gate, np.zeros(E, np.int32), cf, fast_scatter=True)
+    g, il, used, elems, disp = ops.moe_encode(rows_to_torch(data, dt), dev(gate), None, cf, top_k=k)
+    np.testing.assert_array_equal(to_np(il), want[1])
+    w_starts, w_counts = mo.moe_partition_ranges(want[1], P, E, M, k=k)
+    starts, counts = ops.moe_partition_ranges(il, P, E, M, top_k=k)
+    np.testing.assert_array_equal(to_np(starts).astype(np.uint64), w_starts)
+    np.testing.assert_array_equal(to_np(counts).astype(np.uint64), w_counts)
+    rebuilt = torch.zeros_like(disp)
+    for q in range(k * P):
+        total = int(w_counts[q].sum())
+        wire = torch.full((total + 3,), 5.0, dtype=disp.dtype, device="cuda")
+        ops.memcpy_sparse_ranges_to_cont_3d(disp, wire, counts[q], starts[q], axis=0)
+        ref = mo.memcpy_sparse_ranges_to_cont_3d(want[4], np.full(total + 3, 5.0, np.float32), w_counts[q], w_starts[q])
+        np.testing.assert_array_equal(to_np(wire), ref)
+        ops.memcpy_cont_to_sparse_ranges_3d(wire, rebuilt, counts[q], starts[q], axis=0)
+    assert torch.equal(rebuilt, disp)
+    # the ranges of one (slot, partition) as a strided view of the whole table, the way a caller picks a row
+    q = k * P - 1
+    wire = torch.zeros(int(w_counts[q].sum()), dtype=disp.dtype, device="cuda")
+    ops.memcpy_sparse_ranges_to_cont_3d(disp, wire, counts, starts, nelements_stride=1, nelements_offset=q * E, axis=0)
+    ref = mo.memcpy_sparse_ranges_to_cont_3d(want[4], np.zeros(wire.numel(), np.float32), w_counts[q], w_starts[q])
+    np.testing.assert_array_equal(to_np(wire), ref)
+
+
+def test_range_copies_along_axis_1(pkg):
+    ops = pkg.ops
+    rng = np.random.default_rng(2)
+    d0, d1, d2 = 6, 5, 24
+    buf = rng.standard_normal((d0, d1, d2)).astype(np.float32)
+    starts = np.array([0, 24, 48, 5, 143], np.uint64)         # whole rows, a row, an odd start, the last element
+    counts = np.array([48, 24, 96, 11, 1], np.uint64)
+    total = int(counts.sum())
+    wire = ops.memcpy_sparse_ranges_to_cont_3d(dev(buf), torch.zeros(total, device="cuda"), dev(counts.astype(np.int64)),
+                                               dev(starts.astype(np.int64)), axis=1)
+    np.testing.assert_array_equal(to_np(wire), mo.memcpy_sparse_ranges_to_cont_3d(buf, np.zeros(total, np.float32), counts, starts, axis=1))
+    back = ops.memcpy_cont_to_sparse_ranges_3d(wire, torch.full((d0, d1, d2), 9.0, device="cuda"), dev(counts.astype(np.int64)),
+                                               dev(starts.astype(np.int64)), axis=1)
+    np.testing.assert_array_equal(to_np(back), mo.memcpy_cont_to_sparse_ranges_3d(to_np(wire), np.full((d0, d1, d2), 9.0, np.float32),
+                                                                                 counts, starts, axis=1))
+    # a range that would leave its block is clipped
+    starts[2], counts[2] = 100, 1000
+    wire2 = ops.memcpy_sparse_ranges_to_cont_3d(dev(buf), torch.zeros(2000, device="cuda"), dev(counts.astype(np.int64)),
+                                                dev(starts.astype(np.int64)), axis=1)
+    np.testing.assert_array_equal(to_np(wire2), mo.memcpy_sparse_ranges_to_cont_3d(buf, np.zeros(2000, np.float32), counts, starts, axis=1))

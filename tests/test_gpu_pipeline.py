@@ -39,6 +39,13 @@ def test_pipeline_equals_unpartitioned_ops(pkg, dt, S, M, E, P, cf):
     kept_whole = to_np(indloc)[0] >= 0
     np.testing.assert_array_equal(to_np(merged)[0] >= 0, kept_whole)
     assert 0 < kept_whole.sum() < S                      # the case drops tokens
+    # the same partitions as token ranges of one whole-batch routing, exchanged at their row ranges
+    layer.out.fill_(3.0), layer.send.fill_(4.0), layer.recv_all.fill_(5.0)
+    once = layer.run_routed_once(d_x, d_gate).clone()
+    assert torch.equal(once, whole)
+    assert torch.equal(layer.recv_all, disp) and torch.equal(layer.whole[1], indloc)
+    layer.run_routed_once(rows_to_torch(x2, dt), d_gate)
+    assert torch.equal(layer.run_routed_once(d_x, d_gate), whole)
     # and the oracle agrees on the decode of the kept tokens
     want = mo.moe_decode(to_np(disp), to_np(gates_s), to_np(indloc),
                          round_fn=None if dt == "f32" else mo.round_to_bf16)

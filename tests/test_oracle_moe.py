@@ -442,3 +442,60 @@ def test_sparse_copy_packs_encode_output():
     want = np.concatenate([disp[e, :used[e]].reshape(-1) for e in range(E)])
     np.testing.assert_array_equal(packed, want)
     np.testing.assert_array_equal(mo.memcpy_cont_to_sparse_3d(packed, np.zeros_like(disp), elems), disp)
+
+
+# ---------------------------------------------------------------- row ranges of partitions inside a whole-batch routing
+@pytest.mark.parametrize("P,E", [(2, 2), (4, 8), (4, 3)])
+def test_partition_ranges_pack_what_the_chained_partition_encodes_pack(P, E):
+    """The ranges exist for one identity: what partition p owns inside the buffer of the whole-batch encode is what
+    partition p's own chained encode (tests/python/op/cuda/test_cuda_moe.py:384-471 protocol) holds in its first
+    rows, so packing either way gives the same stream, counts = the chained encode's elements_per_expert, and
+    unpacking every partition's stream at its ranges rebuilds the whole buffer."""
+    S0, M = 264, 6
+    S0 -= S0 % (P * E)
+    data, gate = rng_case(11 + P, S0, M, E)
+    gate[:, 0] += 0.4                       # a crowded expert: the chain drops tokens
+    S = S0 // P
+    zero = np.zeros(E, np.int32)
+    _, wil, wused, _, wdisp = mo.moe_encode(data, gate, zero, 0.75)
+    starts, counts = mo.moe_partition_ranges(wil, P, E, M)
+    assert (wil[0] < 0).any()
+    used = zero
+    rebuilt = np.zeros_like(wdisp)
+    for p in range(P):
+        sl = slice(p * S, (p + 1) * S)
+        _, il, used, elems, disp = mo.moe_encode(data[sl], gate[sl], used, 0.75 * P)
+        assert disp.shape == wdisp.shape
+        np.testing.assert_array_equal(counts[p], elems)
+        total = int(elems.sum())
+        own = mo.memcpy_sparse_to_cont_3d(disp, np.full(total, 7, disp.dtype), elems)
+        ranged = mo.memcpy_sparse_ranges_to_cont_3d(wdisp, np.full(total, 9, wdisp.dtype), counts[p], starts[p])
+        np.testing.assert_array_equal(ranged, own)
+        rebuilt = mo.memcpy_cont_to_sparse_ranges_3d(ranged, rebuilt, counts[p], starts[p])
+    np.testing.assert_array_equal(used, wused)
+    np.testing.assert_array_equal(rebuilt, wdisp)
+    # the ranges tile the used rows of every expert without gaps or overlap
+    np.testing.assert_array_equal(starts[0], np.zeros(E, np.uint64))
+    np.testing.assert_array_equal(starts[1:], (starts + counts)[:-1])
+    np.testing.assert_array_equal((starts + counts)[-1], wused.astype(np.uint64) * np.uint64(M))
+
+
+def test_partition_ranges_of_a_top2_routing_hold_the_partitions_tokens_in_order():
+    """top-2: rows of expert e follow each other slot-major, then by partition, then by token
+    (docker/resources/sharded_moe.py:282-295: second choices are placed behind all first choices).  Every range
+    must hold exactly the rows of the kept tokens of its (slot, partition, expert), in token order."""
+    S0, M, E, P = 240, 5, 4, 3
+    data, gate = rng_case(3, S0, M, E)
+    _, il, used, _, disp = mo.moe_encode_top2(data, gate, np.zeros(E, np.int32), 0.6)
+    starts, counts = mo.moe_partition_ranges(il, P, E, M, k=2)
+    S = S0 // P
+    assert (il[0] < 0).any()
+    for j in range(2):
+        for p in range(P):
+            for e in range(E):
+                toks = [s for s in range(p * S, (p + 1) * S) if il[0, j * S0 + s] == e]
+                r0 = int(starts[j * P + p, e]) // M
+                assert int(counts[j * P + p, e]) == len(toks) * M
+                np.testing.assert_array_equal(disp[e, r0:r0 + len(toks)], data[toks])
+                assert [int(il[1, j * S0 + s]) for s in toks] == list(range(r0, r0 + len(toks)))
+    np.testing.assert_array_equal((starts + counts)[-1], used.astype(np.uint64) * np.uint64(M))

@@ -11,6 +11,11 @@ expert uses are packed back to back, keyed by elements_per_expert (the send coun
 src/op/dialect/nccl/nccl.cc:373-421), and unpacked into a zero-filled [E, C, M] receive buffer.  The
 expert computation is the identity.  Partition i is then decoded from its own receive buffer.
 
+`run_routed_once` is the same layer with the partitions taken as token ranges of ONE routing of the whole batch
+(the chained partition encodes, merged, are that routing): one send and one receive buffer shared by the
+partitions, every partition scattering, exchanging (at the row ranges it owns) and decoding its own tokens.  It
+moves each row once per stage and needs no per-partition buffers.
+
 Streams carry the default priority.  Every buffer is allocated once, in the constructor; `run` only
 launches kernels and records events, so it can be called in a loop.
 """

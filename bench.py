@@ -208,7 +208,7 @@ def cpu_baseline_lans(hyper_steps=2):
             "kind": "port", "sample": "C/OpenMP restatement, one MoE layer's 32 expert tensors"}
 
 
-def bench_config4_partitioned(ops, lib, capi, data, logits, S, M, E, cf, iters):
+def bench_config4_partitioned(pkg, ops, lib, capi, data, logits, S, M, E, cf, iters):
     """BASELINE config 4 as configured: 4 token partitions x 2 slots encoded in capacity order
     (s1p0..s1p3, s2p0..s2p3) with chained used capacity, moe_merge_masks, moe_redispatch, moe_decode.
     Per-slot gate arrays are prepared outside the timed region."""
@@ -333,6 +333,15 @@ def bench_config4_partitioned(ops, lib, capi, data, logits, S, M, E, cf, iters):
     if not torch.equal(r_dec, dec):
         raise RuntimeError("partition decodes of the once-routed batch differ from moe_decode")
     seq_routed = {"ms_sequence": round(event_ms(routed_once, iters), 4), "ms_graph_replay": round(graph_ms(routed_once), 4)}
+
+    # ... and with the exchange staged as well: every partition packs the rows it owns in the shared send buffer
+    # (one range per slot and expert) and unpacks them into the shared receive buffer its decode reads
+    once = pkg.pipeline.RoutedOnceMoeLayer(S, M, E, P, cf, top_k=2, dtype=data.dtype, gate_is_logits=True)
+    once.run(data, logits)
+    if not torch.equal(once.recv, want_red) or not torch.equal(once.out, dec):
+        raise RuntimeError("routed-once pipeline with exchange differs from the merged / redispatched result")
+    seq_routed["ms_with_exchange_three_streams"] = round(event_ms(lambda: once.run(data, logits), iters), 4)
+    del once
 
     kept = int((merged[0] >= 0).sum())
     b = data.element_size()
@@ -658,7 +667,7 @@ def main():
     result["backward"] = bench_backward(ops, data, outs, dec, S, M, E, Cap, K, kept, n)
     del dec, outs
     torch.cuda.empty_cache()
-    result["config4_partitioned"] = bench_config4_partitioned(ops, lib, capi, data, logits, S, M, E, cf, max(5, n // 2))
+    result["config4_partitioned"] = bench_config4_partitioned(pkg, ops, lib, capi, data, logits, S, M, E, cf, max(5, n // 2))
     result["expert_input_merge"] = bench_expert_input(ops, M, max(10, n))
     result["pipeline"] = bench_pipeline(pkg, data, logits, S, M, E, cf, max(5, n // 2))
     result["other_configs"] = bench_other_configs(ops, max(10, n))

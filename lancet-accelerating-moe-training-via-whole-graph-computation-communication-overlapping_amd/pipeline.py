@@ -51,18 +51,8 @@ class PartitionedMoeLayer:
         self.routing = torch.cuda.Stream(device=dev)
         self.compute = torch.cuda.Stream(device=dev)
         self.exchange = torch.cuda.Stream(device=dev)
-        # the same layer with the batch routed once (run_routed_once): one send and one receive buffer that the
-        # partitions share, each owning a run of rows per expert
-        self.Ct = ops.moe_capacity(S, E, float(capacity_factor))
-        self.whole = (torch.empty(S, dtype=torch.float32, device=dev), torch.empty((2, S), dtype=torch.int32, device=dev),
-                      torch.empty(E, dtype=torch.int32, device=dev), torch.empty(E, dtype=torch.int64, device=dev))
-        self.whole_ws = torch.empty(ops.moe_encode_workspace_bytes(S, E, 1), dtype=torch.uint8, device=dev)
-        self.ranges = (torch.empty((P, E), dtype=torch.int64, device=dev), torch.empty((P, E), dtype=torch.int64, device=dev))
-        self.ranges_ws = torch.empty(max(4, P * E * 4), dtype=torch.uint8, device=dev)
-        self.send = torch.empty((E, self.Ct, M), dtype=dtype, device=dev)
-        self.recv_all = torch.empty((E, self.Ct, M), dtype=dtype, device=dev)
-        self.no_rows = torch.empty((0, M), dtype=dtype, device=dev)
-        self.routed_all = torch.cuda.Event()
+        self.once = RoutedOnceMoeLayer(S, M, E, n_partitions, capacity_factor, 1, dtype, gate_is_logits, device,
+                                       streams=(self.routing, self.compute, self.exchange))
         self.routed = [torch.cuda.Event() for _ in range(P)]
         self.encoded = [torch.cuda.Event() for _ in range(P)]
         self.received = [torch.cuda.Event() for _ in range(P)]
@@ -140,11 +130,53 @@ class PartitionedMoeLayer:
         return self.out
 
     def run_routed_once(self, data, gate):
-        """The partitions as token ranges of ONE routing of the whole batch (the chained partition encodes, merged,
-        are that routing): routing and the partitions' row ranges first, then per partition the scatter of its tokens
-        into the shared send buffer, the exchange of the rows it owns there (packed and unpacked at its ranges) and
-        the decode of its tokens from the shared receive buffer.  Same streams as `run`; the output equals
-        moe_decode(moe_encode(whole batch))."""
+        """The same partitions as token ranges of one routing of the whole batch: see RoutedOnceMoeLayer."""
+        return self.once.run(data, gate)
+
+    def kept_masks(self):
+        """indices_locations of every partition, the input moe_merge_masks takes."""
+        return [e[1] for e in self.enc]
+
+
+class RoutedOnceMoeLayer:
+    """The partitioned layer with the partitions taken as token ranges of ONE routing of the whole batch (the chained
+    partition encodes, merged, are that routing; for top-2 in GShard's capacity order: all first choices, then all
+    second choices).  Routing and the partitions' row ranges come first; then, per partition, the scatter of its
+    tokens into the shared send buffer (each token row read once, also for top-2), the exchange of the rows it owns
+    there (packed and unpacked at its ranges, one range per slot and expert) and the decode of its tokens from the
+    shared receive buffer.  The output equals moe_decode(moe_encode(whole batch)); no buffer is per partition but
+    the packed streams."""
+
+    def __init__(self, S, M, E, n_partitions, capacity_factor=1.0, top_k=1, dtype=torch.float32, gate_is_logits=False,
+                 device="cuda", streams=None):
+        if S % n_partitions != 0:
+            raise ValueError("the token count must divide into n_partitions")
+        self.S, self.M, self.E, self.P, self.K = S, M, E, n_partitions, top_k
+        self.Sp = S // n_partitions
+        self.cf = float(capacity_factor)
+        self.gate_is_logits = gate_is_logits
+        self.C = ops.moe_capacity(S, E, self.cf * (2.0 if top_k == 2 else 1.0))
+        dev = torch.device(device)
+        P, K, Sp = n_partitions, top_k, self.Sp
+        self.whole = (torch.empty(K * S, dtype=torch.float32, device=dev), torch.empty((2, K * S), dtype=torch.int32, device=dev),
+                      torch.empty(E, dtype=torch.int32, device=dev), torch.empty(E, dtype=torch.int64, device=dev))
+        self.whole_ws = torch.empty(ops.moe_encode_workspace_bytes(S, E, K), dtype=torch.uint8, device=dev)
+        self.ranges = (torch.empty((K * P, E), dtype=torch.int64, device=dev),
+                       torch.empty((K * P, E), dtype=torch.int64, device=dev))
+        self.ranges_ws = torch.empty(max(4, K * P * E * 4), dtype=torch.uint8, device=dev)
+        self.send = torch.empty((E, self.C, M), dtype=dtype, device=dev)
+        self.recv = torch.empty((E, self.C, M), dtype=dtype, device=dev)
+        # packed streams: one per partition and slot (a partition sends at most Sp rows per slot)
+        self.wire = [[torch.empty(Sp * M, dtype=dtype, device=dev) for _ in range(K)] for _ in range(P)]
+        self.out = torch.empty((S, M), dtype=dtype, device=dev)
+        self.no_rows = torch.empty((0, M), dtype=dtype, device=dev)
+        self.routing, self.compute, self.exchange = streams or tuple(torch.cuda.Stream(device=dev) for _ in range(3))
+        self.routed = torch.cuda.Event()
+        self.scattered = [torch.cuda.Event() for _ in range(P)]
+        self.received = [torch.cuda.Event() for _ in range(P)]
+
+    def run(self, data, gate):
+        P, K, Sp, E, C = self.P, self.K, self.Sp, self.E, self.C
         cur = torch.cuda.current_stream()
         start = torch.cuda.Event()
         start.record(cur)
@@ -153,36 +185,37 @@ class PartitionedMoeLayer:
         g, il, used, _ = self.whole
         starts, counts = self.ranges
         with torch.cuda.stream(self.routing):
-            ops.moe_route(gate, None, self.M, self.cf / self.P, gate_is_logits=self.gate_is_logits,
+            ops.moe_route(gate, None, self.M, self.cf, top_k=K, gate_is_logits=self.gate_is_logits,
                           workspace=self.whole_ws, out=self.whole)
-            ops.moe_partition_ranges(il, self.P, self.E, self.M, workspace=self.ranges_ws, out=self.ranges)
+            ops.moe_partition_ranges(il, P, E, self.M, top_k=K, workspace=self.ranges_ws, out=self.ranges)
             # rows of the receive buffer no partition owns: cleared once (a scatter of no tokens is only the tail fill)
-            ops.moe_scatter_tokens(self.no_rows, il, None, used, 0, self.E, self.Ct, zero_tail=True, out=self.recv_all)
-            self.routed_all.record(self.routing)
-        self.compute.wait_event(self.routed_all)
-        self.exchange.wait_event(self.routed_all)
-        for i in range(self.P):
-            sl = slice(i * self.Sp, (i + 1) * self.Sp)
+            ops.moe_scatter_tokens(self.no_rows, il, None, used, 0, E, C, top_k=K, zero_tail=True, out=self.recv)
+            self.routed.record(self.routing)
+        self.compute.wait_event(self.routed)
+        self.exchange.wait_event(self.routed)
+
+        def decode(i):
+            ops.moe_decode_tokens(self.recv, g, il, i * Sp, Sp, top_k=K, out=self.out[i * Sp:(i + 1) * Sp])
+
+        for i in range(P):
             with torch.cuda.stream(self.compute):
-                ops.moe_scatter_tokens(data[sl], il, None, used, i * self.Sp, self.E, self.Ct, zero_tail=False, out=self.send)
-                self.encoded[i].record(self.compute)
+                ops.moe_scatter_tokens(data[i * Sp:(i + 1) * Sp], il, None, used, i * Sp, E, C, top_k=K, zero_tail=False,
+                                       out=self.send)
+                self.scattered[i].record(self.compute)
                 if i > 0:
                     self.compute.wait_event(self.received[i - 1])
-                    ops.moe_decode_tokens(self.recv_all, g, il, (i - 1) * self.Sp, self.Sp,
-                                          out=self.out[(i - 1) * self.Sp:i * self.Sp])
+                    decode(i - 1)
             with torch.cuda.stream(self.exchange):
-                self.exchange.wait_event(self.encoded[i])
-                ops.memcpy_sparse_ranges_to_cont_3d(self.send, self.wire[i], counts[i], starts[i], axis=0)
-                ops.memcpy_cont_to_sparse_ranges_3d(self.wire[i], self.recv_all, counts[i], starts[i], axis=0)
+                self.exchange.wait_event(self.scattered[i])
+                for j in range(K):
+                    q = j * P + i
+                    ops.memcpy_sparse_ranges_to_cont_3d(self.send, self.wire[i][j], counts[q], starts[q], axis=0)
+                    ops.memcpy_cont_to_sparse_ranges_3d(self.wire[i][j], self.recv, counts[q], starts[q], axis=0)
                 self.received[i].record(self.exchange)
         with torch.cuda.stream(self.compute):
-            self.compute.wait_event(self.received[self.P - 1])
-            ops.moe_decode_tokens(self.recv_all, g, il, (self.P - 1) * self.Sp, self.Sp, out=self.out[(self.P - 1) * self.Sp:])
+            self.compute.wait_event(self.received[P - 1])
+            decode(P - 1)
             done = torch.cuda.Event()
             done.record(self.compute)
         cur.wait_event(done)
         return self.out
-
-    def kept_masks(self):
-        """indices_locations of every partition, the input moe_merge_masks takes."""
-        return [e[1] for e in self.enc]

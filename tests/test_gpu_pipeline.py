@@ -40,10 +40,10 @@ def test_pipeline_equals_unpartitioned_ops(pkg, dt, S, M, E, P, cf):
     np.testing.assert_array_equal(to_np(merged)[0] >= 0, kept_whole)
     assert 0 < kept_whole.sum() < S                      # the case drops tokens
     # the same partitions as token ranges of one whole-batch routing, exchanged at their row ranges
-    layer.out.fill_(3.0), layer.send.fill_(4.0), layer.recv_all.fill_(5.0)
+    layer.out.fill_(3.0), layer.once.send.fill_(4.0), layer.once.recv.fill_(5.0), layer.once.out.fill_(6.0)
     once = layer.run_routed_once(d_x, d_gate).clone()
     assert torch.equal(once, whole)
-    assert torch.equal(layer.recv_all, disp) and torch.equal(layer.whole[1], indloc)
+    assert torch.equal(layer.once.recv, disp) and torch.equal(layer.once.whole[1], indloc)
     layer.run_routed_once(rows_to_torch(x2, dt), d_gate)
     assert torch.equal(layer.run_routed_once(d_x, d_gate), whole)
     # and the oracle agrees on the decode of the kept tokens
@@ -87,3 +87,25 @@ def test_concurrent_calls_on_separate_streams_share_no_state(pkg):
                 t.zero_()
             dec.zero_()
         torch.cuda.synchronize()            # the clears run on the default stream
+
+
+@pytest.mark.parametrize("dt,S,M,E,P,cf", [("bf16", 8192, 256, 16, 4, 0.6), ("f32", 3000, 40, 6, 3, 1.0), ("f16", 4096, 64, 32, 8, 0.4)])
+def test_routed_once_pipeline_top2_equals_unpartitioned_ops(pkg, dt, S, M, E, P, cf):
+    """RoutedOnceMoeLayer with top-2 routing: one routing of the batch, per partition a scatter of its tokens (both
+    slots), the exchange of the rows it owns (one range per slot and expert) and a decode, against moe_encode +
+    moe_decode over the whole batch, twice over the same buffers."""
+    ops = pkg.ops
+    rng = np.random.default_rng(S + P)
+    x = rows_as_oracle(rng.standard_normal((S, M), dtype=np.float32), dt)
+    logits = rng.standard_normal((S, E), dtype=np.float32) * 2
+    d_x, d_gate = rows_to_torch(x, dt), dev(logits)
+    layer = pkg.pipeline.RoutedOnceMoeLayer(S, M, E, P, cf, top_k=2, dtype=d_x.dtype, gate_is_logits=True)
+    layer.send.fill_(4.0), layer.recv.fill_(5.0), layer.out.fill_(6.0)
+    got = layer.run(d_x, d_gate).clone()
+    gates_s, indloc, used, elems, disp = ops.moe_encode(d_x, d_gate, None, cf, top_k=2, gate_is_logits=True)
+    whole = ops.moe_decode(disp, gates_s, indloc, top_k=2)
+    assert torch.equal(got, whole) and torch.equal(layer.recv, disp)
+    assert bool((indloc[0] < 0).any())
+    x2 = rows_as_oracle(rng.standard_normal((S, M), dtype=np.float32), dt)
+    layer.run(rows_to_torch(x2, dt), d_gate)
+    assert torch.equal(layer.run(d_x, d_gate), whole)

@@ -49,6 +49,7 @@ extern "C" {
 #define LANCET_ERR_TOPK (-6)      /* top_k not 1 or 2, or top_k = 2 with fewer than 2 experts */
 #define LANCET_ERR_PARTITION (-7) /* bad n_partitions / partition_id */
 #define LANCET_ERR_PLAN (-8)      /* invalid LANS plan handle, or a plan of another device than the current one */
+#define LANCET_ERR_SCRATCH (-9)   /* lancet_moe_encode_noalloc: the sizes need more than LANCET_NOALLOC_SCRATCH_BYTES */
 
 /* limits */
 #define LANCET_MAX_EXPERTS 512
@@ -124,6 +125,24 @@ int lancet_moe_encode(const void* data, const float* gate, const float* gate2_no
                       unsigned flags, float* gates_s, int32_t* indices_locations,
                       int32_t* used_out, uint64_t* elements_per_expert, void* dispatched,
                       void* workspace, size_t workspace_bytes, lancet_stream_t stream);
+
+/* lancet_moe_encode without the workspace argument, for callers that cannot allocate device memory: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  (No counterpart in the
+ * reference, whose executor allocates a workspace before every Execute, src/impl/vm/vm.cc:1260-1266.)
+ * The scan's scratch (ticket, error word, descriptor table) lives in a static device array of
+ * LANCET_NOALLOC_SCRATCH_BYTES that each GPU holds until the process ends; sizes whose
+ * lancet_moe_encode_workspace_bytes(S, E, top_k) exceeds it are rejected with LANCET_ERR_SCRATCH
+ * (1 MiB covers S * top_k * E <= 67 million, e.g. S = 65536, E = 512, top_k = 2).  The call allocates
+ * nothing and launches the same kernels as lancet_moe_encode, with identical results.  All calls on one
+ * GPU share the array: calls that overlap on one GPU race, so issue them on one stream or order them
+ * yourself.  The first call on a device looks the array's address up (no launch, no allocation); make that
+ * call once before recording a graph. */
+#define LANCET_NOALLOC_SCRATCH_BYTES (1u << 20)
+int lancet_moe_encode_noalloc(const void* data, const float* gate, const float* gate2_noise,
+                              const int32_t* used_in, int64_t S, int64_t M, int64_t E, int64_t C, int top_k,
+                              int dtype, unsigned flags, float* gates_s, int32_t* indices_locations,
+                              int32_t* used_out, uint64_t* elements_per_expert, void* dispatched,
+                              lancet_stream_t stream);
 
 /* The two phases of lancet_moe_encode as separate calls, for callers that overlap the routing of
  * one token partition with the row movement of another (Lancet's forward pipelining,

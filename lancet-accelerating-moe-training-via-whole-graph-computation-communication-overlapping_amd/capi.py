@@ -20,7 +20,8 @@ MAX_EXPERTS = 512
 MAX_PARTITIONS = 64
 
 OK = 0
-ERR_NULL, ERR_SHAPE, ERR_DTYPE, ERR_WORKSPACE, ERR_ALIGN, ERR_TOPK, ERR_PARTITION, ERR_PLAN = range(-1, -9, -1)
+ERR_NULL, ERR_SHAPE, ERR_DTYPE, ERR_WORKSPACE, ERR_ALIGN, ERR_TOPK, ERR_PARTITION, ERR_PLAN, ERR_SCRATCH = range(-1, -10, -1)
+NOALLOC_SCRATCH_BYTES = 1 << 20
 
 
 class LansHyper(C.Structure):
@@ -49,6 +50,8 @@ SIGNATURES = {
     "lancet_moe_encode_workspace_bytes": (_sz, [_i64, _i64, _int]),
     "lancet_moe_encode": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _u32,
                                  _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "lancet_moe_encode_noalloc": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _u32,
+                                         _vp, _vp, _vp, _vp, _vp, _vp]),
     "lancet_moe_route": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _u32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "lancet_moe_scatter": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _u32, _vp, _vp]),
     "lancet_moe_encode_bpr_workspace_bytes": (_sz, [_i64, _i64, _int]),

@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define LANCET_ABI_VERSION 3
+#define LANCET_ABI_VERSION 4
 
 /* element type of token rows */
 #define LANCET_F32 0
@@ -50,6 +50,7 @@ extern "C" {
 #define LANCET_ERR_PARTITION (-7) /* bad n_partitions / partition_id */
 #define LANCET_ERR_PLAN (-8)      /* invalid LANS plan handle, or a plan of another device than the current one */
 #define LANCET_ERR_SCRATCH (-9)   /* lancet_moe_encode_noalloc: the sizes need more than LANCET_NOALLOC_SCRATCH_BYTES */
+#define LANCET_ERR_STALLED (-10)  /* lancet_lans_step: an earlier step of the plan gave up a wait; call lancet_lans_plan_error */
 
 /* limits */
 #define LANCET_MAX_EXPERTS 512
@@ -323,6 +324,9 @@ int lancet_moe_redispatch(const void* const* data, const int32_t* const* indices
  * reference's tensor_list).  p, m, v are updated in place; g is not modified.
  * step: pass step_host >= 1, or a device pointer step_dev to the fp32 step scalar the
  * reference passes (read on the device; no host synchronisation).
+ * grad_norms: NULL, or a device array of T floats holding ||g_i||_2 in the order of the lists, for a caller
+ * that already has them (per-tensor norms from gradient clipping): the step then skips its own pass over g
+ * for them (the first l2norm sweep of multi_tensor_lans.cu:412-418).
  * A plan's steps share its partial sums and control words: issue them on one stream, or order
  * them yourself; two steps of one plan that overlap on the device race.  Plans are independent
  * of each other. */
@@ -344,16 +348,27 @@ int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans_plan_t* pl
 int lancet_lans_plan_destroy(lancet_lans_plan_t plan);
 int lancet_lans_step(lancet_lans_plan_t plan, const float* const* g, float* const* p,
                      float* const* m, float* const* v, int step_host, const float* step_dev,
-                     const lancet_lans_hyper* hyper, lancet_stream_t stream);
+                     const lancet_lans_hyper* hyper, const float* grad_norms, lancet_stream_t stream);
 /* A step may be recorded into a HIP graph (either schedule): with step_dev the step number is read on the
  * device, and everything else that changes from step to step lives in the plan's device memory, so each
  * replay is a new step.  The pointer tables are uploaded (one host-to-device copy) by the first call that
  * sees a new set of pointers: make that call once before recording. */
-/* Schedules of the step.  LANCET_LANS_SWEEPS (default): three whole-state sweeps with two per-tensor
- * reductions between them (48 B/param of traffic).  LANCET_LANS_RESIDENT: one persistent kernel that keeps
- * each chunk on chip between moments and update, after a sweep over g for its norm (32 B/param), for the tensors that fit on the chip at once
- * (lancet_lans_plan_resident_capacity) and the three sweeps, in the same step, for the larger ones; a plan
- * with no tensor that fits gets LANCET_ERR_SHAPE from set_schedule and keeps its schedule.  Each schedule is deterministic; the two agree to fp32 rounding of the per-chunk sums. */
+/* Schedules of the step.
+ * LANCET_LANS_SWEEPS (default): three whole-state sweeps with two per-tensor reductions between them
+ * (48 B/param of traffic).  No workgroup waits for another.
+ * LANCET_LANS_RESIDENT: one persistent kernel that reads and writes every array once (28 B/param): each
+ * workgroup runs a three-stage pipeline over chunks of 8192 parameters and keeps a chunk on chip between the
+ * stages, for the tensors of at most lancet_lans_plan_resident_capacity() chunks; larger tensors of the plan
+ * take the three sweeps in the same step, and a plan with no tensor that fits gets LANCET_ERR_SHAPE from
+ * set_schedule and keeps its schedule.  Contract of this schedule: its workgroups wait for one another (for
+ * chunks of the same tensor only), so at least half of them must be running on the device at the same time.
+ * The grid is sized to what an otherwise idle device runs at once; other kernels on the device delay the
+ * step until enough of its workgroups have started, and only something that keeps the device occupied
+ * without end (e.g. another kernel that itself waits for this step) can stall it.  Every wait is bounded:
+ * a wait that gives up leaves the parameters of the tensors concerned unwritten (their m and v may already
+ * hold the new moments), sets the plan's sticky error, and the NEXT lancet_lans_step on the plan returns
+ * LANCET_ERR_STALLED without launching anything, until lancet_lans_plan_error has been called.
+ * Each schedule is deterministic; the two agree to fp32 rounding of the per-chunk sums. */
 #define LANCET_LANS_SWEEPS 0
 #define LANCET_LANS_RESIDENT 1
 int lancet_lans_plan_set_schedule(lancet_lans_plan_t plan, int schedule);
@@ -361,8 +376,8 @@ int lancet_lans_plan_set_schedule(lancet_lans_plan_t plan, int schedule);
  * (larger tensors of the plan go through the sweeps); max_tensor_chunks: chunks of the plan's largest
  * tensor.  Either may be NULL. */
 int lancet_lans_plan_resident_capacity(lancet_lans_plan_t plan, int* workgroups, int* max_tensor_chunks);
-/* Reads (synchronously) the plan's error word: 1 when a bounded wait of the resident schedule
- * gave up (results of that step are undefined). */
+/* Reads (synchronising `stream`) and clears the plan's sticky error: 1 when a bounded wait of the resident
+ * schedule gave up in any step since the last call. */
 int lancet_lans_plan_error(lancet_lans_plan_t plan, lancet_stream_t stream, int* error_out);
 
 /* Copies the four per-tensor norm vectors of the last step (||g||, ||p||, ||u_m||, ||u_g||;
@@ -370,24 +385,6 @@ int lancet_lans_plan_error(lancet_lans_plan_t plan, lancet_stream_t stream, int*
  * norms4xT, a device buffer of 4*T floats, asynchronously on `stream`. */
 int lancet_lans_plan_norms(lancet_lans_plan_t plan, float* norms4xT, lancet_stream_t stream);
 
-/* Host-only view of what a plan builds for `numels` when the resident kernel takes tensors of up to
- * resident_limit chunks (no device needed): for every chunk, in the order the kernel hands them out, the
- * position of its tensor in the caller's list; *n_resident_chunks = how many the resident kernel hands out
- * (the rest go through the sweeps).  Returns the number of chunks; fills at most `capacity` entries
- * (either output may be NULL). */
-int64_t lancet_lans_debug_chunk_table(const int64_t* numels, int T, int resident_limit, int32_t* chunk_tensor_out,
-                                      int64_t capacity, int64_t* n_resident_chunks);
-
-/* Test hook: number of polls a workgroup of the position scan waits for a predecessor
- * before it gives up, flags the workspace and finishes with undefined results
- * (0 restores the default).  Lets a host test exercise the bounded wait without hanging. */
-void lancet_debug_set_spin_limit(unsigned limit);
-/* Measurement aid (no counterpart in the reference): one plain streaming kernel over `bytes` bytes (a multiple
- * of 4096), one 16-byte non-temporal access per thread, workgroups in address order: the launch shape that
- * streams fastest on this device.  kind 0 reads src, 1 fills dst with zeros, 2 copies src to dst.  bench.py
- * times these beside the row movers so that their fractions of the peak can be read against what the
- * memory system delivers to the simplest possible kernel. */
-int lancet_debug_stream(int kind, void* dst, const void* src, size_t bytes, lancet_stream_t stream);
 /* Reads (synchronously) the error word a scan workspace carries: 0 = ok, 1 = a wait gave up. */
 int lancet_scan_workspace_error(const void* workspace, lancet_stream_t stream, int* error_out);
 

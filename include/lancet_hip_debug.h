@@ -1,0 +1,42 @@
+/*
+ * lancet_hip_debug.h - test and measurement hooks of liblancet_hip.so.  Not part of the operator surface:
+ * nothing here replaces a piece of the reference, and a product build may leave these symbols out.
+ */
+#ifndef LANCET_HIP_DEBUG_H_
+#define LANCET_HIP_DEBUG_H_
+
+#include "lancet_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Host-only view of what a LANS plan builds for `numels` when the resident kernel takes tensors of up to
+ * resident_limit chunks and runs `round` workgroups (no device needed): for every chunk slot, in the order the
+ * kernel hands them out, the position of its tensor in the caller's list, or -1 for a padding slot (a tensor
+ * that does not fit into what is left of a round of `round` slots starts the next round);
+ * *n_resident_chunks = slots the resident kernel hands out (the rest go through the sweeps).  Returns the
+ * number of slots; fills at most `capacity` entries (either output may be NULL). */
+int64_t lancet_lans_debug_chunk_table(const int64_t* numels, int T, int resident_limit, int round,
+                                      int32_t* chunk_tensor_out, int64_t capacity, int64_t* n_resident_chunks);
+
+/* Test hook of one plan: spin_limit = polls a workgroup of the resident schedule waits for a word before it
+ * gives up (0 restores the default); flags bit 0: the workgroup that sums a tensor's partials withholds the
+ * norms, so that every wait for them runs into the limit.  Lets a host test exercise the bounded waits and the
+ * error path while every kernel still exits normally. */
+int lancet_lans_plan_debug(lancet_lans_plan_t plan, unsigned spin_limit, unsigned flags);
+
+/* Test hook: number of polls a workgroup of the position scan waits for a predecessor
+ * before it gives up, flags the workspace and finishes with undefined results
+ * (0 restores the default).  Lets a host test exercise the bounded wait without hanging. */
+void lancet_debug_set_spin_limit(unsigned limit);
+/* Measurement aid (no counterpart in the reference): one plain streaming kernel over `bytes` bytes (a multiple
+ * of 4096), one 16-byte non-temporal access per thread, workgroups in address order: the launch shape that
+ * streams fastest on this device.  kind 0 reads src, 1 fills dst with zeros, 2 copies src to dst.  bench.py
+ * times these beside the row movers so that their fractions of the peak can be read against what the
+ * memory system delivers to the simplest possible kernel. */
+int lancet_debug_stream(int kind, void* dst, const void* src, size_t bytes, lancet_stream_t stream);
+#ifdef __cplusplus
+}
+#endif
+#endif /* LANCET_HIP_DEBUG_H_ */

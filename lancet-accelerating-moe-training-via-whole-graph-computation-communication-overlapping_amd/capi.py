@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(HERE, "lib", "liblancet_hip.so")
 F32, BF16, F16 = 0, 1, 2
 GATE_IS_LOGITS = 1
 NO_TAIL_ZERO = 2
-ABI_VERSION = 3
+ABI_VERSION = 4
 ZERO_TAIL = 4
 ROWS_AT_USED = 8
 LANS_SWEEPS, LANS_RESIDENT = 0, 1
@@ -20,7 +20,8 @@ MAX_EXPERTS = 512
 MAX_PARTITIONS = 64
 
 OK = 0
-ERR_NULL, ERR_SHAPE, ERR_DTYPE, ERR_WORKSPACE, ERR_ALIGN, ERR_TOPK, ERR_PARTITION, ERR_PLAN, ERR_SCRATCH = range(-1, -10, -1)
+(ERR_NULL, ERR_SHAPE, ERR_DTYPE, ERR_WORKSPACE, ERR_ALIGN, ERR_TOPK, ERR_PARTITION, ERR_PLAN, ERR_SCRATCH,
+ ERR_STALLED) = range(-1, -11, -1)
 NOALLOC_SCRATCH_BYTES = 1 << 20
 
 
@@ -85,11 +86,12 @@ SIGNATURES = {
     "lancet_lans_plan_create": (_int, [C.POINTER(_i64), _int, C.POINTER(_vp)]),
     "lancet_lans_plan_destroy": (_int, [_vp]),
     "lancet_lans_step": (_int, [_vp, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),
-                                _int, _vp, C.POINTER(LansHyper), _vp]),
+                                _int, _vp, C.POINTER(LansHyper), _vp, _vp]),
     "lancet_lans_plan_norms": (_int, [_vp, _vp, _vp]),
     "lancet_lans_plan_set_schedule": (_int, [_vp, _int]),
     "lancet_lans_plan_error": (_int, [_vp, _vp, C.POINTER(_int)]),
-    "lancet_lans_debug_chunk_table": (_i64, [C.POINTER(_i64), _int, _int, _vp, _i64, C.POINTER(_i64)]),
+    "lancet_lans_debug_chunk_table": (_i64, [C.POINTER(_i64), _int, _int, _int, _vp, _i64, C.POINTER(_i64)]),
+    "lancet_lans_plan_debug": (_int, [_vp, _u32, _u32]),
     "lancet_lans_plan_resident_capacity": (_int, [_vp, C.POINTER(_int), C.POINTER(_int)]),
     "lancet_debug_set_spin_limit": (None, [_u32]),
     "lancet_scan_workspace_error": (_int, [_vp, _vp, C.POINTER(_int)]),

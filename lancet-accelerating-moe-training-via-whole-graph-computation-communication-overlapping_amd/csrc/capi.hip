@@ -1,6 +1,6 @@
 // C ABI of the MoE dispatch path: argument validation, then kernel launches on the caller's
 // stream.  Nothing here allocates, synchronises or keeps state between calls.
-#include "../../include/lancet_hip.h"
+#include "../../include/lancet_hip_debug.h"
 #include "common.hpp"
 #include "launchers.hpp"
 
@@ -56,6 +56,7 @@ extern "C" const char* lancet_status_string(int status) {
     case LANCET_ERR_TOPK: return "top_k must be 1 or 2 (2 needs at least two experts)";
     case LANCET_ERR_PARTITION: return "bad n_partitions / partition_id";
     case LANCET_ERR_PLAN: return "invalid LANS plan";
+    case LANCET_ERR_STALLED: return "an earlier LANS step of this plan gave up a wait (call lancet_lans_plan_error)";
     case LANCET_ERR_SCRATCH: return "sizes exceed the static scratch of the allocation-free entry point";
     default: return status > 0 ? hipGetErrorString(static_cast<hipError_t>(status)) : "unknown status";
   }

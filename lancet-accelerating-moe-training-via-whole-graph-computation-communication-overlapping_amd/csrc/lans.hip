@@ -1,26 +1,30 @@
 // Fused multi-tensor LANS step.  The reference makes six sweeps over the optimizer state
 // (src/op/dialect/cuda/kernels/multi_tensor_lans.cu:401-450: l2norm(g), l2norm(p), stage 1,
 // l2norm(u_m), l2norm(u_g), stage 2, 68 B/param of traffic).  Here the step has three phases
-//   phase 1  reads g               -> per-chunk sums of g^2
-//   phase 2  reads g, p, m, v      -> writes m, v; per-chunk sums of p^2, u_m^2 and u_g^2
-//   phase 3  reads g, p, m, v      -> recomputes u_m, u_g (never stored) and writes p
+//   phase N  reads g               -> per-chunk sums of g^2
+//   phase M  reads g, p, m, v      -> writes m, v; per-chunk sums of p^2, u_m^2 and u_g^2
+//   phase U  reads g, p, m, v      -> recomputes u_m, u_g (never stored) and writes p
 // and two schedules:
 //   * sweeps (default): three plain launches + two tiny per-tensor reductions.  Real HBM traffic
-//     is 48 B/param (g read three times, p, m, v twice) and each sweep streams at the rate a plain
-//     copy reaches on this chip.
-//   * resident (opt-in): a sweep over g alone for ||g|| (4 B/param), then ONE persistent kernel in
-//     which a workgroup takes a chunk through phases 2 and 3 and keeps it on chip in between (u_m and
-//     u_g in registers, p in LDS), so every array is read once and written once: 32 B/param with the
-//     sweep.  Before phase 3 the workgroups of a tensor exchange three chunk partials (p^2, u_m^2,
-//     u_g^2) as self-validating 64-bit words (step epoch in the high half, fp32 sum in the low half,
-//     one agent-scope atomic store each); the workgroup that arrives last at a per-tensor counter
+//     is 48 B/param (g read three times, p, m, v twice).
+//   * resident (opt-in): ONE persistent kernel in which every array is read once and written once
+//     (28 B/param).  A workgroup runs a three-stage software pipeline over the chunks it draws from a
+//     ticket: stage N loads g of a chunk into registers and publishes its sum of squares; stage M, one
+//     iteration later, loads p, m, v of that chunk, writes m and v and keeps u_m, u_g in registers and p
+//     in LDS; stage U, another iteration later, writes p.  Between the stages of one chunk the workgroup
+//     works on its other two chunks, so the per-tensor norms a stage needs (||g|| for M; ||p||, ||u_m||,
+//     ||u_g|| for U) have normally been published long before it asks for them.  Workgroups exchange
+//     chunk partials as self-validating 64-bit words (step epoch in the high half, fp32 sum in the low
+//     half, one agent-scope atomic store each); the workgroup that arrives last at a per-tensor counter
 //     sums them in a fixed order and publishes the norms the same way.  Nothing else crosses
-//     workgroups, so no fences are needed.  Chunks are handed out in order by a ticket; a workgroup
-//     only ever waits for chunks of its own tensor, so the kernel drains as long as the chunks of one
-//     tensor all fit on the chip at once (the limit is the register file: about 4M parameters per
-//     tensor on 256 CUs).  The plan orders its tensors so that those within the limit come first;
-//     the kernel takes them, and larger tensors go through the sweeps in the same step.  Waits are
-//     bounded.
+//     workgroups, so no fences are needed.  The plan packs tensors into rounds of as many chunks as the
+//     device runs workgroups (padding a round rather than splitting a tensor over two), so that all
+//     chunks of a tensor are drawn in the same pipeline iteration.  A workgroup waits only for chunks of
+//     tensors it holds, chunks are drawn in order, and a workgroup holds at most two chunks that have not
+//     passed stage M: the kernel drains as long as half as many workgroups as the largest tensor has
+//     chunks are running.  Larger tensors go through the sweeps in the same step.  Waits are bounded; a
+//     wait that gives up poisons what it would have fed, so that no parameter is written from an unknown
+//     norm, and raises a sticky error the next step reports.
 // Work is cut into fixed-size chunks described by device-resident tables built once per
 // parameter set, instead of kernel arguments re-packed for every launch
 // (multi_tensor_apply.cuh:39-92).  Chunk partials are combined in a fixed order in double
@@ -28,7 +32,7 @@
 // accumulated in a different order).
 #include "launchers.hpp"
 #include "common.hpp"
-#include "../../include/lancet_hip.h"
+#include "../../include/lancet_hip_debug.h"
 #include <algorithm>
 #include <new>
 #include <vector>
@@ -39,24 +43,33 @@ constexpr int kLansThreads = 256;
 constexpr int kLansChunk = 8192;  // elements per task: 8 float4 per thread and array
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+// control words of a plan (uint32): [0] next ticket of the resident kernel, [1] error (sticky: only
+// lancet_lans_plan_error clears it), [2] step epoch, [3] unused, then T arrival counters of stage N
+// and T of stage M
+constexpr int kCtlTicket = 0, kCtlError = 1, kCtlEpoch = 2, kCtlArrive = 4;
+
 struct LansTables {
   const float* const* g;  // [T] device pointers
   float* const* p;
   float* const* m;
   float* const* v;
   const int64_t* numel;        // [T]
-  const int32_t* chunk_tensor; // [nchunks]
-  const int32_t* tensor_first; // [T+1] first chunk of each tensor
+  const int32_t* chunk_tensor; // [nchunks] tensor of a chunk slot, -1 = padding slot of a round
+  const int32_t* tensor_first; // [T] first chunk slot of each tensor (its chunks are consecutive)
+  const int32_t* tensor_chunks;// [T] chunks of each tensor
   float* partial;              // [3][nchunks * kSweepSplit]  (sweeps: one sum per slice)
-  uint64_t* part_word;         // [4][nchunks]      (resident schedule: epoch | fp32 sum of squares)
-  uint64_t* norm_word;         // [4][T]            (resident schedule: epoch | fp32 norm)
-  uint32_t* ticket;            // [1] next task; [1] error flag; [T] arrivals; [1] step epoch (resident schedule)
+  uint64_t* part_word;         // [4][nchunks]      (resident schedule: tag | fp32 sum of squares)
+  uint64_t* norm_word;         // [4][T]            (resident schedule: tag | fp32 norm)
+  uint32_t* ctl;               // control words, see kCtl*
+  uint32_t* host_status;       // device view of a pinned host word: set with the error word, read by the next step
   float* norms;                // [4][T]: g, p, u_m, u_g
   float* consts;               // [2]: bias_correction1, bias_correction2
   const int32_t* order;        // [T] position in the caller's lists of the plan's i-th tensor
+  const float* grad_norms;     // [T] ||g|| per tensor in the caller's order, or null: computed by the step
   int T;
-  int nchunks;
-  int nres;                    // chunks [0, nres) belong to tensors the resident schedule can hold
+  int nchunks;                 // chunk slots, padding included
+  int nres;                    // slots [0, nres) are handed out by the resident kernel
+  uint32_t debug_flags;        // bit 0: the last arriver withholds the norms (exercises the bounded waits)
 };
 
 struct LansScalars {
@@ -64,7 +77,7 @@ struct LansScalars {
   int mode, normalize_grad, bias_correction;
   int step_host;
   const float* step_dev;
-  uint32_t epoch;              // filled in on the device (the word behind the arrival counters)
+  uint32_t epoch;              // filled in on the device
   uint32_t spin_limit;
 };
 
@@ -83,7 +96,7 @@ __device__ __forceinline__ float block_sum(float v, float* s_red) {
 }
 
 struct ChunkView {
-  int tensor;
+  int tensor;     // -1: a padding slot
   int64_t begin;  // first element of the chunk inside the tensor
   int n;          // elements in the chunk
 };
@@ -91,9 +104,13 @@ struct ChunkView {
 __device__ __forceinline__ ChunkView chunk_view(const LansTables& t, int chunk) {
   ChunkView c;
   c.tensor = t.chunk_tensor[chunk];
-  c.begin = static_cast<int64_t>(chunk - t.tensor_first[c.tensor]) * kLansChunk;
-  const int64_t left = t.numel[c.tensor] - c.begin;
-  c.n = static_cast<int>(left < kLansChunk ? left : kLansChunk);
+  c.begin = 0;
+  c.n = 0;
+  if (c.tensor >= 0) {
+    c.begin = static_cast<int64_t>(chunk - t.tensor_first[c.tensor]) * kLansChunk;
+    const int64_t left = t.numel[c.tensor] - c.begin;
+    c.n = static_cast<int>(left < kLansChunk ? left : kLansChunk);
+  }
   return c;
 }
 
@@ -109,16 +126,21 @@ __device__ __forceinline__ float uniform(float x) {
 }
 
 // ---- elementwise math, in the reference's operation order (multi_tensor_lans.cu:283-307) ----
+// Divisions by a value the whole tensor shares (||g|| + eps, the two bias corrections) are multiplications
+// by its correctly rounded reciprocal, and the two quotients over the same per-element denominator share one
+// correctly rounded reciprocal: one division and one square root per element instead of five and one.  Each
+// such product is within 1.5 ulp of the quotient the reference forms (0.5 ulp), far inside the 1e-6 the
+// parameters are held to; a step is bound by memory only as long as the arithmetic stays this small.
 struct LansElem {
-  float gnorm_eps;  // ||g|| + eps
-  bool normalize;   // normalize_grad && ||g|| != 0
-  float beta1, beta2, beta3, one_minus_beta2, bc1, bc2, eps, wd;
+  float inv_gnorm_eps;  // 1 / (||g|| + eps)
+  bool normalize;       // normalize_grad && ||g|| != 0
+  float beta1, beta2, beta3, one_minus_beta2, inv_bc1, inv_bc2, eps, wd;
   int mode;
 
   __device__ __forceinline__ float scaled_grad(float g, float p) const {
 #pragma clang fp contract(off)
     float sg = g;
-    if (normalize) sg = sg / gnorm_eps;
+    if (normalize) sg = sg * inv_gnorm_eps;
     if (mode == 0) sg = sg + wd * p;
     return sg;
   }
@@ -129,9 +151,10 @@ struct LansElem {
   }
   __device__ __forceinline__ void updates(float sg, float p, float m, float v, float& um, float& ug) const {
 #pragma clang fp contract(off)
-    const float denom = sqrtf(v / bc2) + eps;
-    um = (m / bc1) / denom;
-    ug = sg / denom;
+    const float denom = sqrtf(v * inv_bc2) + eps;
+    const float r = 1.f / denom;
+    um = (m * inv_bc1) * r;
+    ug = sg * r;
     if (mode != 0) {
       const float sp = wd * p;
       um = um + sp;
@@ -142,14 +165,14 @@ struct LansElem {
 
 __device__ __forceinline__ LansElem make_elem(const LansScalars& sc, float gn, float bc1, float bc2) {
   LansElem e;
-  e.gnorm_eps = uniform(gn + sc.eps);
+  e.inv_gnorm_eps = uniform(1.f / (gn + sc.eps));
   e.normalize = sc.normalize_grad && uniform(gn) != 0.f;
   e.beta1 = sc.beta1;
   e.beta2 = sc.beta2;
   e.beta3 = sc.beta3;
   e.one_minus_beta2 = uniform(1.f - sc.beta2);
-  e.bc1 = uniform(bc1);
-  e.bc2 = uniform(bc2);
+  e.inv_bc1 = uniform(1.f / bc1);
+  e.inv_bc2 = uniform(1.f / bc2);
   e.eps = sc.eps;
   e.wd = sc.wd;
   e.mode = sc.mode;
@@ -336,7 +359,9 @@ __device__ __forceinline__ ChunkView slice_view(const LansTables& t, int chunk_b
 __global__ __launch_bounds__(kLansThreads) void lans_norm_g_kernel(LansTables t, int chunk_base) {
   __shared__ float s_red[kLansThreads / kWave];
   const int chunk = chunk_base + blockIdx.x;  // a whole chunk per workgroup: this sweep only reads, and splitting it costs more in reductions than it gains
-  const float sg = chunk_norm_g(t, chunk_view(t, chunk), s_red);
+  const ChunkView c = chunk_view(t, chunk);
+  if (c.tensor < 0) return;  // padding slot (uniform over the workgroup)
+  const float sg = chunk_norm_g(t, c, s_red);
   if (threadIdx.x == 0) t.partial[chunk] = sg;
 }
 
@@ -346,7 +371,7 @@ __global__ __launch_bounds__(kLansThreads) void lans_reduce_kernel(LansTables t,
                                                                    int tensor_end, int count, int split) {
   const int tensor = tensor_base + blockIdx.x * (kLansThreads / kWave) + threadIdx.x / kWave;
   if (tensor >= tensor_end) return;
-  const int lo = t.tensor_first[tensor], hi = t.tensor_first[tensor + 1];
+  const int lo = t.tensor_first[tensor], hi = lo + t.tensor_chunks[tensor];
   for (int k = 0; k < count; ++k) {
     const float* part = t.partial + static_cast<size_t>(k) * t.nchunks * split;
     const float n = wave_norm(lo * split, hi * split, [&](int c) { return part[c]; });
@@ -358,6 +383,7 @@ __global__ __launch_bounds__(kLansThreads) void lans_moments_kernel(LansTables t
   __shared__ float s_red[kLansThreads / kWave];
   int slot;
   const ChunkView c = slice_view(t, chunk_base, slot);
+  if (c.tensor < 0) return;  // padding slot (uniform over the workgroup)
   const LansElem el = make_elem(sc, t.norms[c.tensor], t.consts[0], t.consts[1]);
   float sp, sm, sg;
   chunk_moments(t, c, el, s_red, sp, sm, sg);
@@ -372,8 +398,15 @@ __global__ __launch_bounds__(kLansThreads) void lans_moments_kernel(LansTables t
 __global__ __launch_bounds__(kLansThreads) void lans_update_kernel(LansTables t, LansScalars sc, int chunk_base) {
   int slot;
   const ChunkView c = slice_view(t, chunk_base, slot);
+  if (c.tensor < 0) return;
   const LansElem el = make_elem(sc, t.norms[c.tensor], t.consts[0], t.consts[1]);
   chunk_update(t, c, el, sc, t.norms[1 * t.T + c.tensor], t.norms[2 * t.T + c.tensor], t.norms[3 * t.T + c.tensor]);
+}
+
+// ||g|| per tensor supplied by the caller (in the order of its lists) instead of the sweep over g
+__global__ void lans_take_grad_norms_kernel(LansTables t) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < t.T) t.norms[i] = t.grad_norms[t.order[i]];
 }
 
 // norms live in the plan's tensor order; callers get them in the order of their lists
@@ -385,211 +418,611 @@ __global__ void lans_gather_norms_kernel(LansTables t, float* dst) {
 }
 
 // =======================================================================================
-// words published between workgroups: step epoch in the high half, fp32 value in the low half
+// words published between workgroups: a tag in the high half (bit 31: poisoned, bits 0..30: the
+// step epoch), an fp32 value in the low half
 // =======================================================================================
+constexpr uint32_t kPoison = 0x80000000u;
+
 __device__ __forceinline__ uint64_t ld_word(const uint64_t* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ void st_word(uint64_t* p, uint32_t epoch, float v) {
-  __hip_atomic_store(p, (static_cast<uint64_t>(epoch) << 32) | __float_as_uint(v), __ATOMIC_RELAXED,
+__device__ __forceinline__ void st_word(uint64_t* p, uint32_t tag, float v) {
+  __hip_atomic_store(p, (static_cast<uint64_t>(tag) << 32) | __float_as_uint(v), __ATOMIC_RELAXED,
                      __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// =======================================================================================
-// schedule "resident": a sweep over g, then one persistent kernel in which a workgroup keeps its
-// chunk on chip between moments and update, so every array is read once and written once, g twice
-// =======================================================================================
-constexpr int kVecPerThread = kLansChunk / 4 / kLansThreads;  // float4 per thread and array
+// sticky: the device word for lancet_lans_plan_error, the pinned host word for the next lancet_lans_step
+__device__ __forceinline__ void flag_error(const LansTables& t) {
+  st_agent(t.ctl + kCtlError, 1u);
+  __hip_atomic_store(t.host_status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
 
-__device__ __forceinline__ f32x4 ld4(const LANCET_GLOBAL float* a, int e) { return ldn((const LANCET_GLOBAL f32x4*)(a + e)); }
-__device__ __forceinline__ void st4(LANCET_GLOBAL float* a, int e, f32x4 x) { stn((LANCET_GLOBAL f32x4*)(a + e), x); }
-
-constexpr int kMaxResidentChunks = 512;  // chunks of one tensor the resident schedule can gather
-
-struct ResidentShared {
-  f32x4 p[kVecPerThread][kLansThreads];  // the chunk's parameters, one private slot per thread and float4
-  float part[3][kMaxResidentChunks];     // gathered chunk partials of the tensor
-  float red[kLansThreads / kWave];
-  float norm[4];
-  int chunk;
-  int last;
+struct Waited {
+  float value;
+  bool bad;  // the wait gave up, or the word was published poisoned
 };
 
-__device__ __forceinline__ uint64_t wait_word(const LansTables& t, const LansScalars& sc, const uint64_t* src) {
+__device__ __forceinline__ Waited wait_word(const LansTables& t, const LansScalars& sc, const uint64_t* src) {
+#ifdef LANCET_LANS_PROBE
+  return Waited{1.f, false};
+#endif
   uint64_t x = ld_word(src);
   uint32_t spins = 0;
-  while (static_cast<uint32_t>(x >> 32) != sc.epoch) {
-    if (++spins > sc.spin_limit) {  // bounded: flag the plan, carry on
-      st_agent(t.ticket + 1, 1u);
-      break;
+  while ((static_cast<uint32_t>(x >> 32) & ~kPoison) != sc.epoch) {
+    // bounded; and once any wait of the plan has given up the others stop early, so that a stalled step
+    // ends after about one bound, not one per chunk
+    if (++spins > sc.spin_limit || ((spins & 63u) == 0u && ld_agent(t.ctl + kCtlError) != 0u)) {
+      flag_error(t);
+      return Waited{0.f, true};
     }
     __builtin_amdgcn_s_sleep(2);
     x = ld_word(src);
   }
-  return x;
+#ifdef LANCET_LANS_TIMING
+  if (spins) atomicAdd(t.ctl + 3, spins);
+#endif
+  return Waited{__uint_as_float(static_cast<uint32_t>(x)), (static_cast<uint32_t>(x >> 32) & kPoison) != 0};
 }
 
-// Norms first .. first+N-1 of the tensor from the partials its workgroups publish (this one has
-// published its own, a[], just before).  The workgroup that arrives last (a per-tensor counter, cleared
-// by the host before the step) gathers the partials into LDS, sums them in the fixed order of
-// wave_norm and publishes the norms as self-validating words; every other workgroup waits for those
-// words only.  Waits are bounded.
-template <int N>
-__device__ __forceinline__ void resident_norms(const LansTables& t, const LansScalars& sc, int first, int tensor,
-                                               const float (&a)[N], ResidentShared& sh) {
-  const int lo = t.tensor_first[tensor];
-  const int nc = t.tensor_first[tensor + 1] - lo;
-  const int w = threadIdx.x / kWave;
-  if (nc == 1) {
-    if (threadIdx.x == 0) {
+// =======================================================================================
+// schedule "resident": one persistent kernel, a three-stage software pipeline per workgroup
+// =======================================================================================
+constexpr int kVecPerThread = kLansChunk / 4 / kLansThreads;  // float4 per thread and array
+
+// Workgroup barrier that orders LDS accesses only.  __syncthreads() also waits for every global load and
+// store the wave has in flight, which would drain the streams of this kernel several times per chunk; all
+// that crosses the waves of a workgroup here is in LDS (global words other workgroups read are atomics).
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+__device__ __forceinline__ float block_sum_lds(float v, float* s_red) {
+  v = wave_sum(v);
+  if (lane_id() == 0) s_red[threadIdx.x / kWave] = v;
+  lds_barrier();
+  float r = 0.f;
+  if (threadIdx.x == 0) {
 #pragma unroll
-      for (int k = 0; k < N; ++k) sh.part[k][0] = a[k];
-    }
-    __syncthreads();
-  } else {
-    if (threadIdx.x == 0) {
-      uint32_t* arrive = t.ticket + 2 + tensor;
-      const uint32_t old = __hip_atomic_fetch_add(arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      sh.last = old == static_cast<uint32_t>(nc - 1);
-    }
-    __syncthreads();
-    if (!sh.last) {
-      if (w < N && lane_id() == 0) {
-        const uint64_t x = wait_word(t, sc, t.norm_word + static_cast<size_t>(first + w) * t.T + tensor);
-        sh.norm[first + w] = __uint_as_float(static_cast<uint32_t>(x));
-      }
-      __syncthreads();
-      return;
-    }
-    for (int idx = threadIdx.x; idx < N * nc; idx += kLansThreads) {
-      const int which = idx / nc;
-      const uint64_t x = wait_word(t, sc, t.part_word + static_cast<size_t>(first + which) * t.nchunks + lo + (idx - which * nc));
-      sh.part[which][idx - which * nc] = __uint_as_float(static_cast<uint32_t>(x));
-    }
-    __syncthreads();
+    for (int k = 0; k < kLansThreads / kWave; ++k) r += s_red[k];
   }
-  if (w < N) {
-    const float n = wave_norm(0, nc, [&](int c) { return sh.part[w][c]; });
-    if (lane_id() == 0) {
-      sh.norm[first + w] = n;
-      if (nc > 1) st_word(t.norm_word + static_cast<size_t>(first + w) * t.T + tensor, sc.epoch, n);
-    }
+  return r;  // valid on thread 0; s_red is free again after the caller's next barrier
+}
+#ifndef LANCET_LANS_ALIGN
+#define LANCET_LANS_ALIGN 1
+#endif
+#ifndef LANCET_LANS_SCHED_K
+#define LANCET_LANS_SCHED_K 0
+#endif
+constexpr int kMaxResidentChunks = 512;  // chunks of one tensor whose partials one workgroup sums
+constexpr uint32_t kPayPolls = 32;       // polls of a tensor's arrival counter at the end of stage N (tens of microseconds)
+
+struct PipeShared {
+  f32x4 p[2][kVecPerThread][kLansThreads];  // parameters of the two chunks between stages M and U, one private slot per thread and float4
+  float part[3][kMaxResidentChunks];        // gathered chunk partials of a tensor
+  float red[3][kLansThreads / kWave];
+  float norm[4];
+  int chunk;
+  int mode;
+  int bad, gather_bad;
+};
+
+// a chunk a workgroup holds between stages; every field is uniform over the workgroup
+struct Slot {
+  int chunk;   // -1: empty (the ticket ran out)
+  int tensor;  // -1: padding slot, nothing to do
+  int n;       // elements
+  int full;    // whole chunk of 16-byte aligned arrays: plain global accesses
+  int dead;    // stage M was skipped (||g|| never came): the parameters stay as they are
+  int lo, nc;  // first chunk slot and number of chunks of the tensor
+  int owes;    // bit k: this workgroup has to sum norm k of the tensor (see pay_norm)
+  int64_t begin;
+  __device__ __forceinline__ bool real() const { return chunk >= 0 && tensor >= 0; }
+};
+
+// What thread 0 of a workgroup has in flight towards other workgroups.  Every remote access of the
+// pipeline (ticket, arrival counters, norm words) is issued one stage before its result is looked at, so
+// that its latency passes while the workgroup streams; only a word that is still missing then is polled.
+struct Control {
+  uint32_t ticket;     // drawn at the start of a pass for its stage N
+  uint64_t g_word[1];  // ||g|| word of s2's tensor (s1's in the next pass), read in front of stage N's loads
+  uint64_t u_word[3];  // norm words of s0's tensor, read in front of stage N's loads
+#ifdef LANCET_LANS_TIMING
+  long long acc[8];
+  long long seg[8];
+  long long last;
+  long long pass_begin;
+#endif
+};
+
+// A partial chunk at the end of a tensor, and a tensor that is only 4-byte aligned, go through buffer
+// instructions: the descriptor carries the chunk's size in bytes, and the hardware checks every dword of an
+// access against it (out-of-range reads give zeros, which add nothing to any sum, out-of-range writes are
+// dropped), so they take the same 16-byte accesses as everything else, without a predicate per element.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t chunk_rsrc(const float* base, int n) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, n * 4, 0x00020000);  // raw buffer of 32-bit words
+}
+// one array of a chunk: a plain pointer for whole chunks of 16-byte aligned arrays (global loads stream
+// faster than buffer loads here), a checked buffer otherwise
+template <bool FULL>
+struct ChunkArray {
+  LANCET_GLOBAL float* ptr;
+  __amdgpu_buffer_rsrc_t rsrc;
+  __device__ __forceinline__ ChunkArray(const float* base, int n) {
+    if (FULL) ptr = as_global(const_cast<float*>(base));
+    else rsrc = chunk_rsrc(base, n);
   }
-  __syncthreads();
+  __device__ __forceinline__ f32x4 load(int e) const {
+    if (FULL) return __builtin_nontemporal_load((const LANCET_GLOBAL f32x4*)(ptr + e));
+    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, e * 4, 0, 2));
+  }
+  __device__ __forceinline__ void store(int e, f32x4 x) const {
+    if (FULL) __builtin_nontemporal_store(x, (LANCET_GLOBAL f32x4*)(ptr + e));
+    else __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, x), rsrc, e * 4, 0, 2);
+  }
+};
+
+// a wave owns 2048 consecutive elements of the chunk: float4 k of lane l is element 4 * (64 k + l) of them,
+// so one load instruction of a wave covers 1 KB of consecutive memory
+__device__ __forceinline__ int chunk_elem(int k) {
+  return (threadIdx.x / kWave) * (kLansChunk / kWavesPerTile) + 4 * lane_id() + k * (4 * kWave);
 }
 
-// One whole chunk of 16-byte aligned arrays, every access an unconditional float4.  ||g|| of the tensor is
-// already in t.norms (a sweep over g alone ran first), so one pass loads everything, writes m and v and
-// leaves u_m, u_g in registers and p in LDS; Sum p^2 joins the two update sums at the single wait, after
-// which p is written: every array is read once and written once, g twice.
-__device__ __forceinline__ void resident_chunk(const LansTables& t, const LansScalars& sc, const ChunkView& c,
-                                                       int chunk, float bc1, float bc2, ResidentShared& sh) {
-  const LANCET_GLOBAL float* g = as_global(t.g[c.tensor] + c.begin);
-  LANCET_GLOBAL float* p = as_global(t.p[c.tensor] + c.begin);
-  LANCET_GLOBAL float* m = as_global(t.m[c.tensor] + c.begin);
-  LANCET_GLOBAL float* v = as_global(t.v[c.tensor] + c.begin);
-  f32x4 xg[kVecPerThread], xu[kVecPerThread];  // u_g and u_m of the thread's eight float4
-  // a wave owns 2048 consecutive elements: float4 k of lane l is element 4 * (64 k + l) of them, so one
-  // load instruction of a wave covers 1 KB of consecutive memory
-  const int e0 = (threadIdx.x / kWave) * (kLansChunk / kWavesPerTile) + 4 * lane_id();
-  const LansElem el = make_elem(sc, t.norms[c.tensor], bc1, bc2);
-  float a0 = 0.f, a1 = 0.f, a2 = 0.f;
+#ifdef LANCET_LANS_TIMING
+__device__ unsigned long long g_misses, g_spins;
+__device__ unsigned g_most = 0, g_fewest = 0xffffffffu;
+__device__ long long g_wait[1024];
+__device__ unsigned g_hist[64];
+__device__ unsigned long long g_seg[2][8];
+__device__ unsigned g_modes[1024][3];
+#endif
+// A word read ahead: taken as it is when it carries this step's tag, polled for otherwise.
+__device__ __forceinline__ Waited resolve_word(const LansTables& t, const LansScalars& sc, uint64_t ahead, const uint64_t* src) {
+#ifdef LANCET_LANS_PROBE
+  return Waited{1.f, false};
+#endif
+  if ((static_cast<uint32_t>(ahead >> 32) & ~kPoison) == sc.epoch)
+    return Waited{__uint_as_float(static_cast<uint32_t>(ahead)), (static_cast<uint32_t>(ahead >> 32) & kPoison) != 0};
+#ifdef LANCET_LANS_TIMING
+  atomicAdd(&g_misses, 1ull);
+#endif
+  return wait_word(t, sc, src);
+}
+
+// Thread 0: publishes the N chunk sums a[] of slot s as words first .. first+N-1 and counts the chunk in at
+// the tensor's arrival counter (nothing comes back: no round trip).
+template <int N>
+__device__ __forceinline__ void publish(const LansTables& t, const LansScalars& sc, int first, const Slot& s,
+                                        const float (&a)[N], bool poison, uint32_t* arrive) {
+#ifdef LANCET_LANS_PROBE
+  return;
+#endif
+  if (t.debug_flags & 1u) return;  // test hook: nothing is ever published, every wait runs into its bound
+  const uint32_t tag = sc.epoch | (poison ? kPoison : 0u);
+#pragma unroll
+  for (int k = 0; k < N; ++k) st_word(t.part_word + static_cast<size_t>(first + k) * t.nchunks + s.chunk, tag, a[k]);
+  (void)__hip_atomic_fetch_add(arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Who sums a tensor's partials.  Norm 0 (||g||) is summed by the workgroup that drew the tensor's first chunk,
+// norms 1, 2, 3 (||p||, ||u_m||, ||u_g||) by those that drew its first, second and third (chunk lo + (k - 1) %
+// nc).  Chunks are drawn in order, so these are workgroups that were ahead of the others when the tensor's
+// round began: they have the time, and the workgroup that arrives last, which everyone else is waiting for, is
+// spared (summing there would make it later still, tensor after tensor).  One norm is 512 words at most, two
+// loads per thread.  A workgroup pays what it owes at the end of stage N of the pass in which the tensor went
+// through the stage in question: it waits there, for a bounded short while, for the tensor's arrival counter
+// to fill up, which is normally long before anybody asks for the norm.  What is still owed then is paid when
+// the workgroup needs the norm itself.
+
+// norm `kind` of slot s's tensor: true when it has been formed and published (sh.norm[kind] holds it)
+__device__ __forceinline__ bool pay_norm(const LansTables& t, const LansScalars& sc, int kind, const Slot& s,
+                                         uint32_t max_polls, PipeShared& sh) {
+#ifdef LANCET_LANS_PROBE
+  return true;
+#endif
+  const uint32_t* arrive = t.ctl + kCtlArrive + (kind == 0 ? 0 : t.T) + s.tensor;
+  if (threadIdx.x == 0) {
+    uint32_t polls = 0;
+    bool full;
+    while (!(full = ld_agent(arrive) >= static_cast<uint32_t>(s.nc)) && ++polls <= max_polls) {
+      if ((polls & 63u) == 0u && ld_agent(t.ctl + kCtlError) != 0u) break;
+      __builtin_amdgcn_s_sleep(2);
+    }
+    sh.mode = full;
+    sh.gather_bad = 0;
+  }
+  lds_barrier();
+  if (__builtin_amdgcn_readfirstlane(sh.mode) == 0) return false;
+  // the partials (each a self-validating word: an arrival can be seen before the words it follows), every
+  // thread's loads in flight together
+  constexpr int kPerThread = kMaxResidentChunks / kLansThreads;
+  const uint64_t* words = t.part_word + static_cast<size_t>(kind) * t.nchunks + s.lo;
+  uint64_t word[kPerThread];
+#pragma unroll
+  for (int i = 0; i < kPerThread; ++i) {
+    const int c = threadIdx.x + i * kLansThreads;
+    word[i] = c < s.nc ? ld_word(words + c) : 0;
+  }
+#pragma unroll
+  for (int i = 0; i < kPerThread; ++i) {
+    const int c = threadIdx.x + i * kLansThreads;
+    if (c < s.nc) {
+      const Waited w = resolve_word(t, sc, word[i], words + c);
+      sh.part[0][c] = w.value;
+      if (w.bad) sh.gather_bad = 1;  // a poisoned or missing partial poisons the norm
+    }
+  }
+  lds_barrier();
+  if (threadIdx.x < kWave) {
+    const float n = wave_norm(0, s.nc, [&](int c) { return sh.part[0][c]; });  // fixed order: the same bits every time
+    if (lane_id() == 0) {
+      sh.norm[kind] = n;
+      t.norms[kind * t.T + s.tensor] = n;
+      st_word(t.norm_word + static_cast<size_t>(kind) * t.T + s.tensor, sc.epoch | (sh.gather_bad ? kPoison : 0u), n);
+    }
+  }
+  lds_barrier();
+  return true;
+}
+
+// pays the norms of `kinds` (a bit mask) that slot s still owes
+__device__ __forceinline__ void pay_norms(const LansTables& t, const LansScalars& sc, Slot& s, int kinds,
+                                          uint32_t max_polls, PipeShared& sh) {
+#pragma unroll
+  for (int kind = 0; kind < 4; ++kind)
+    if ((s.owes & kinds & (1 << kind)) && pay_norm(t, sc, kind, s, max_polls, sh)) s.owes &= ~(1 << kind);
+}
+
+// Norms first .. first+N-1 of slot s's tensor into sh.norm; `ahead` are the norm words as thread 0 read them
+// ahead: when they carry this step's tag that is all.  Otherwise thread 0 polls for them (bounded).  Returns
+// true when the norms are unknown (a wait gave up, or a chunk was poisoned).  Called by the whole workgroup.
+template <int N>
+__device__ __forceinline__ bool acquire_norms(const LansTables& t, const LansScalars& sc, int first, Slot& s,
+                                              const uint64_t (&ahead)[N], PipeShared& sh) {
+#ifdef LANCET_LANS_PROBE
+  if (threadIdx.x == 0) for (int k = 0; k < N; ++k) sh.norm[first + k] = 1.f;
+  lds_barrier();
+  return false;
+#endif
+  const int kinds = ((1 << N) - 1) << first;
+  const bool owed = (s.owes & kinds) != 0;
+  if (owed) pay_norms(t, sc, s, kinds, sc.spin_limit, sh);  // nobody else will form them
+  if (threadIdx.x == 0) {
+#ifdef LANCET_LANS_TIMING
+    const long long t_in = clock64();
+#endif
+    uint64_t w[N];
+#pragma unroll
+    for (int k = 0; k < N; ++k) w[k] = owed ? 0 : ahead[k];
+    bool gave_up = false;
+    uint32_t spins = 0;
+    while (true) {
+      bool have = true;
+#pragma unroll
+      for (int k = 0; k < N; ++k) have = have && (static_cast<uint32_t>(w[k] >> 32) & ~kPoison) == sc.epoch;
+      if (have) break;
+      // bounded; and once any wait of the plan has given up the others stop early, so that a stalled step
+      // ends after about one bound, not one per chunk
+      if (++spins > sc.spin_limit || ((spins & 63u) == 0u && ld_agent(t.ctl + kCtlError) != 0u)) { gave_up = true; break; }
+      if (spins > 1) __builtin_amdgcn_s_sleep(2);
+#pragma unroll
+      for (int k = 0; k < N; ++k) w[k] = ld_word(t.norm_word + static_cast<size_t>(first + k) * t.T + s.tensor);
+    }
+    int bad = gave_up;
+    if (gave_up) flag_error(t);
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+      sh.norm[first + k] = __uint_as_float(static_cast<uint32_t>(w[k]));
+      bad |= (static_cast<uint32_t>(w[k] >> 32) & kPoison) != 0;
+    }
+    sh.bad = bad;
+#ifdef LANCET_LANS_TIMING
+    g_wait[blockIdx.x] += clock64() - t_in;
+    g_modes[blockIdx.x][spins == 0 ? 0 : 1] += 1;
+#endif
+  }
+  lds_barrier();
+  return __builtin_amdgcn_readfirstlane(sh.bad) != 0;
+}
+
+template <bool FULL>
+__device__ __forceinline__ float load_g(const LansTables& t, const Slot& s, f32x4 (&g)[kVecPerThread]) {
+  const ChunkArray<FULL> src(t.g[s.tensor] + s.begin, s.n);
+  float a = 0.f;
 #pragma unroll
   for (int k = 0; k < kVecPerThread; ++k) {
-    const int e = e0 + k * (4 * kWave);
-    const f32x4 g4 = ld4(g, e), xp = ld4(p, e);
-    f32x4 xm = ld4(m, e), xv = ld4(v, e);
-    sh.p[k][threadIdx.x] = xp;
+    g[k] = src.load(chunk_elem(k));
+    a += g[k].x * g[k].x + g[k].y * g[k].y + g[k].z * g[k].z + g[k].w * g[k].w;
+  }
+  return a;
+}
+
+// Moments and the two updates (LANSStage1Functor, multi_tensor_lans.cu:207-322, and the l2norm sweeps
+// around it, :428-441) of a chunk whose g sits in registers.  m and v are written; u_m, u_g stay in
+// registers and p in LDS for stage U.  The loads of float4 k+1 are issued before the stores of float4 k:
+// memory operations of a wave complete in order, so a load behind a store would wait for it.
+template <bool FULL, int PAR>
+__device__ __forceinline__ void moments_chunk(const LansTables& t, const Slot& s, const LansElem& el,
+                                              const f32x4 (&g)[kVecPerThread], f32x4 (&um)[kVecPerThread],
+                                              f32x4 (&ug)[kVecPerThread], PipeShared& sh, float (&a)[3]) {
+  const ChunkArray<FULL> p(t.p[s.tensor] + s.begin, s.n), m(t.m[s.tensor] + s.begin, s.n), v(t.v[s.tensor] + s.begin, s.n);
+  float a0 = 0.f, a1 = 0.f, a2 = 0.f;
+  f32x4 np = p.load(chunk_elem(0));
+  f32x4 nm = m.load(chunk_elem(0)), nv = v.load(chunk_elem(0));
+#pragma unroll
+  for (int k = 0; k < kVecPerThread; ++k) {
+    const int e = chunk_elem(k);
+    const f32x4 xp = np;
+    f32x4 xm = nm, xv = nv;
+    if (k + 1 < kVecPerThread) {
+      np = p.load(chunk_elem(k + 1));
+      nm = m.load(chunk_elem(k + 1));
+      nv = v.load(chunk_elem(k + 1));
+    }
+#if LANCET_LANS_SCHED_K
+    __builtin_amdgcn_sched_barrier(0);  // keeps the loads above the stores below
+#endif
+    sh.p[PAR][k][threadIdx.x] = xp;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const float sg = el.scaled_grad(g4[j], xp[j]);
+      const float sg = el.scaled_grad(g[k][j], xp[j]);
       float mm = xm[j], vv = xv[j], u0, u1;
       el.moments(sg, mm, vv);
       el.updates(sg, xp[j], mm, vv, u0, u1);
-      // the two updates are final here: nothing of their computation may be left for after the wait (the
-      // compiler otherwise carries a third value per element, wd * p, across it and spills)
+      // the two updates are final here: nothing of their computation may be left for stage U (the
+      // compiler otherwise carries a third value per element, wd * p, across the stages and spills)
       asm volatile("" : "+v"(u0), "+v"(u1));
       xm[j] = mm;
       xv[j] = vv;
-      xu[k][j] = u0;
-      xg[k][j] = u1;
+      um[k][j] = u0;
+      ug[k][j] = u1;
       a0 += xp[j] * xp[j];
       a1 += u0 * u0;
       a2 += u1 * u1;
     }
-    st4(m, e, xm);
-    st4(v, e, xv);
+    m.store(e, xm);
+    v.store(e, xv);
   }
-  a0 = block_sum(a0, sh.red);
-  a1 = block_sum(a1, sh.red);
-  a2 = block_sum(a2, sh.red);
-  if (threadIdx.x == 0) {
-    st_word(t.part_word + 1 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a0);
-    st_word(t.part_word + 2 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a1);
-    st_word(t.part_word + 3 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a2);
-  }
-  {
-    const float a[3] = {a0, a1, a2};
-    resident_norms<3>(t, sc, 1, c.tensor, a, sh);
-  }
-  if (threadIdx.x == 0 && chunk == t.tensor_first[c.tensor]) {
-#pragma unroll
-    for (int k = 1; k < 4; ++k) t.norms[k * t.T + c.tensor] = sh.norm[k];
-  }
-  const float pn = uniform(sh.norm[1]), umn = uniform(sh.norm[2]), ugn = uniform(sh.norm[3]);
-  float ratio_m = (umn != 0.f && pn != 0.f) ? sc.lr * (pn / umn) : sc.lr;
-  float ratio_g = (ugn != 0.f && pn != 0.f) ? sc.lr * (pn / ugn) : sc.lr;
-  ratio_m = uniform(ratio_m * sc.beta1);
-  ratio_g = uniform(ratio_g * sc.beta3);
-#pragma unroll
-  for (int k = 0; k < kVecPerThread; ++k) {
-    const int e = e0 + k * (4 * kWave);
-    f32x4 xp = sh.p[k][threadIdx.x];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-#pragma clang fp contract(off)
-      xp[j] = xp[j] - (ratio_m * xu[k][j]) - (ratio_g * xg[k][j]);
+  a[0] = a0;
+  a[1] = a1;
+  a[2] = a2;
+}
+
+#ifdef LANCET_LANS_TIMING
+#define EVT(slot, e) do { if (threadIdx.x == 0 && (slot).real() && (slot).tensor == 100) reinterpret_cast<long long*>(t.partial)[blockIdx.x * 8 + (e)] = wall_clock64(); } while (0)
+#define EVT1(slot, e) do { if (threadIdx.x == 0 && (slot).tensor == 100) reinterpret_cast<long long*>(t.partial)[512 * 8 + (e)] = wall_clock64(); } while (0)
+#else
+#define EVT(slot, e) do { } while (0)
+#define EVT1(slot, e) do { } while (0)
+#endif
+#ifdef LANCET_LANS_TIMING
+#define TSTAMP(i) do { if (threadIdx.x == 0) { const long long now_ = clock64(); ctl.acc[i] += now_ - ctl.last; ctl.seg[i] = now_ - ctl.last; ctl.last = now_; } } while (0)
+#else
+#define TSTAMP(i) do { } while (0)
+#endif
+
+// One pass of the pipeline: stage M on s1 (its g in `g`; its updates go to um_new / ug_new, its parameters to
+// sh.p[PAR]), stage N on a newly drawn slot, whose g goes into `g`, which stage M has just used up, stage U
+// on s0 (updates in um_old / ug_old, parameters in sh.p[PAR ^ 1]); then the slots move up.  Consecutive
+// passes alternate between the two g arrays and between the two parities.
+//
+// Memory operations of a wave complete in order, and under load a round trip takes microseconds: a value
+// that comes from memory is free when it is asked for before a stage's loads and looked at after them, and
+// costs a drain of the wave's stores when it is looked at behind them.  So thread 0 draws the ticket and
+// reads the norm words ahead, at the two places of a pass where its wave has nothing in flight (the start of
+// the pass, and before the loads of stage N), and looks at what the arrival counters returned one stage
+// later.  A workgroup that arrived last owes the tensor its norms and always pays before it waits itself
+// (it may hold two chunks of the tensor).  Returns false when the workgroup holds nothing any more.
+template <int PAR>
+__device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansScalars& sc, float bc1, float bc2,
+                                              Slot& s0, Slot& s1, Slot& s2, Control& ctl,
+                                              f32x4 (&g)[kVecPerThread],
+                                              f32x4 (&um_new)[kVecPerThread], f32x4 (&ug_new)[kVecPerThread],
+                                              const f32x4 (&um_old)[kVecPerThread], const f32x4 (&ug_old)[kVecPerThread],
+                                              PipeShared& sh, bool align = false) {
+  const bool own_norms = t.grad_norms == nullptr;
+  // ---- start of the pass ---------------------------------------------------------------------------------
+  lds_barrier();
+  bool bad = false;
+  if (s1.real()) {
+    if (own_norms) {
+      bad = acquire_norms<1>(t, sc, 0, s1, ctl.g_word, sh);
+    } else {
+      if (threadIdx.x == 0) sh.norm[0] = t.norms[s1.tensor];  // copied from the caller's array before this kernel
+      lds_barrier();
     }
-    st4(p, e, xp);
   }
-}
-
-// A partial or unaligned chunk through the same protocol with the streaming chunk functions of the
-// sweeps (nothing held in registers; m and v written before the wait are read back after it by the thread
-// that wrote them).  At most one chunk per tensor takes this path when arrays are aligned.
-__device__ __forceinline__ void resident_chunk_streamed(const LansTables& t, const LansScalars& sc, const ChunkView& c,
-                                                        int chunk, float bc1, float bc2, ResidentShared& sh) {
-  float a0, a1, a2;
-  const LansElem el = make_elem(sc, t.norms[c.tensor], bc1, bc2);
-  chunk_moments(t, c, el, sh.red, a0, a1, a2);
   if (threadIdx.x == 0) {
-    st_word(t.part_word + 1 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a0);
-    st_word(t.part_word + 2 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a1);
-    st_word(t.part_word + 3 * static_cast<size_t>(t.nchunks) + chunk, sc.epoch, a2);
+    // The plan lays a tensor's chunks out inside one round of as many slots as there are workgroups, so that
+    // they are all drawn in the same pass and pass through the stages together.  That holds as long as every
+    // workgroup has made its k-th draw before any makes its (k+1)-th, which the waits see to from the third
+    // pass on; before its second draw a workgroup gives the others a moment to make their first (bounded: a
+    // few microseconds, whether or not they all come).
+    if (align) {
+      const uint32_t everyone = min(static_cast<uint32_t>(gridDim.x), static_cast<uint32_t>(t.nres));
+      for (int spins = 0; spins < 256 && ld_agent(t.ctl + kCtlTicket) < everyone; ++spins) __builtin_amdgcn_s_sleep(8);
+    }
+    // The ticket of this pass's stage N.  Drawn behind the wait for ||g|| of s1's tensor: every chunk of that
+    // tensor has been drawn by now, so the new slot cannot be a third chunk of it in this workgroup's hands.
+    ctl.ticket = atomicAdd(t.ctl + kCtlTicket, 1u);
   }
-  const float a[3] = {a0, a1, a2};
-  resident_norms<3>(t, sc, 1, c.tensor, a, sh);
-  if (threadIdx.x == 0 && chunk == t.tensor_first[c.tensor]) {
+  EVT(s1, 1);
+  TSTAMP(0);
+  // ---- stage M on s1 ---------------------------------------------------------------------------------------
+  if (s1.real()) {
+    float a[3] = {0.f, 0.f, 0.f};
+    if (!bad) {
+      const LansElem el = make_elem(sc, sh.norm[0], bc1, bc2);
+      if (s1.full) moments_chunk<true, PAR>(t, s1, el, g, um_new, ug_new, sh, a);
+      else moments_chunk<false, PAR>(t, s1, el, g, um_new, ug_new, sh, a);
+    } else {
+      s1.dead = 1;  // ||g|| is unknown: the chunk is left as it is, and so will its tensor's parameters be
+    }
+    TSTAMP(1);
 #pragma unroll
-    for (int k = 1; k < 4; ++k) t.norms[k * t.T + c.tensor] = sh.norm[k];
+    for (int k = 0; k < 3; ++k) a[k] = wave_sum(a[k]);
+    if (lane_id() == 0) {
+#pragma unroll
+      for (int k = 0; k < 3; ++k) sh.red[k][threadIdx.x / kWave] = a[k];
+    }
+    lds_barrier();
+    if (threadIdx.x == 0) {
+#pragma unroll
+      for (int k = 0; k < 3; ++k) {
+        float r = 0.f;
+#pragma unroll
+        for (int w = 0; w < kLansThreads / kWave; ++w) r += sh.red[k][w];
+        a[k] = r;
+      }
+      publish<3>(t, sc, 1, s1, a, bad, t.ctl + kCtlArrive + t.T + s1.tensor);
+    }
+    EVT(s1, 2);
   }
-  chunk_update(t, c, el, sc, sh.norm[1], sh.norm[2], sh.norm[3]);
+  TSTAMP(2);
+  EVT(s0, 7);
+  EVT(s2, 6);
+  // ---- stage N on a new slot -------------------------------------------------------------------------------
+  Slot s3;
+  if (threadIdx.x == 0) {
+    // read ahead, in front of the loads of g: the norms stage U needs (s0's tensor) and ||g|| for the next
+    // pass's stage M (s2's tensor)
+    if (s0.real()) {
+#pragma unroll
+      for (int k = 0; k < 3; ++k) ctl.u_word[k] = ld_word(t.norm_word + static_cast<size_t>(1 + k) * t.T + s0.tensor);
+    }
+    if (s2.real() && own_norms) ctl.g_word[0] = ld_word(t.norm_word + s2.tensor);
+    sh.chunk = static_cast<int>(ctl.ticket);
+  }
+  lds_barrier();
+  {
+    // one value for the whole workgroup, and known to be: pointers and sizes derived from it stay scalar
+    const int chunk = __builtin_amdgcn_readfirstlane(sh.chunk);
+    s3.chunk = (chunk >= 0 && chunk < t.nres) ? chunk : -1;
+    s3.tensor = -1;
+    s3.dead = 0;
+    s3.owes = 0;
+    if (s3.chunk >= 0) {
+      const ChunkView c = chunk_view(t, s3.chunk);
+      s3.tensor = c.tensor;
+      if (c.tensor >= 0) {
+        s3.n = c.n;
+        s3.begin = c.begin;
+        s3.lo = t.tensor_first[c.tensor];
+        s3.nc = t.tensor_chunks[c.tensor];
+        const int at = s3.chunk - s3.lo;
+        s3.owes = (own_norms && at == 0 ? 1 : 0) | (at == 0 ? 2 : 0) | (at == 1 % s3.nc ? 4 : 0) | (at == 2 % s3.nc ? 8 : 0);
+        s3.full = c.n == kLansChunk && vec_ok(t.g[c.tensor], t.p[c.tensor], t.m[c.tensor], t.v[c.tensor]);
+      }
+    }
+  }
+  TSTAMP(3);
+  if (s3.real()) {
+    // g of the chunk into registers, its sum of squares published (L2NormFunctor, multi_tensor_lans.cu:95-167)
+    float a = s3.full ? load_g<true>(t, s3, g) : load_g<false>(t, s3, g);
+    if (own_norms) {
+      a = block_sum_lds(a, sh.red[0]);
+      if (threadIdx.x == 0) {
+        const float sums[1] = {a};
+        publish<1>(t, sc, 0, s3, sums, false, t.ctl + kCtlArrive + s3.tensor);
+      }
+    }
+    EVT(s3, 0);
+  }
+  TSTAMP(4);
+#ifdef LANCET_LANS_TIMING
+  if (threadIdx.x == 0 && s3.real()) ctl.acc[7] += 1;
+#endif
+  // ---- stage U on s0 ---------------------------------------------------------------------------------------
+  // Trust ratios and the parameter update (LANSStage2Functor, multi_tensor_lans.cu:326-399) from the updates
+  // in registers and the parameters in LDS.  Nothing is written unless all three norms are known.
+  bool bad_u = true;
+  // first what this workgroup owes others: ||g|| of s3's tensor, which has just been through stage N, and
+  // the three norms of s1's, through stage M earlier in this pass
+  if (s3.real()) pay_norms(t, sc, s3, 1, kPayPolls, sh);
+  if (s1.real()) pay_norms(t, sc, s1, 14, kPayPolls, sh);
+  if (s0.real()) bad_u = acquire_norms<3>(t, sc, 1, s0, ctl.u_word, sh) || s0.dead != 0;
+  EVT(s0, 3);
+  TSTAMP(5);
+  if (s0.real() && !bad_u) {
+    const float pn = uniform(sh.norm[1]), umn = uniform(sh.norm[2]), ugn = uniform(sh.norm[3]);
+    float ratio_m = (umn != 0.f && pn != 0.f) ? sc.lr * (pn / umn) : sc.lr;
+    float ratio_g = (ugn != 0.f && pn != 0.f) ? sc.lr * (pn / ugn) : sc.lr;
+    ratio_m = uniform(ratio_m * sc.beta1);
+    ratio_g = uniform(ratio_g * sc.beta3);
+    const ChunkArray<true> p_full(t.p[s0.tensor] + s0.begin, s0.n);
+    const ChunkArray<false> p_part(t.p[s0.tensor] + s0.begin, s0.n);
+#pragma unroll
+    for (int k = 0; k < kVecPerThread; ++k) {
+      f32x4 xp = sh.p[PAR ^ 1][k][threadIdx.x];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma clang fp contract(off)
+        xp[j] = xp[j] - (ratio_m * um_old[k][j]) - (ratio_g * ug_old[k][j]);
+      }
+      if (s0.full) p_full.store(chunk_elem(k), xp);
+      else p_part.store(chunk_elem(k), xp);
+    }
+  }
+  TSTAMP(6);
+#ifdef LANCET_LANS_TIMING
+  if (threadIdx.x == 0) {
+    const long long now = wall_clock64();
+    if (ctl.pass_begin && s1.real()) {
+      long long d = (now - ctl.pass_begin) / 200;
+      atomicAdd(&g_hist[d > 63 ? 63 : (int)d], 1u);
+      const int slow = d >= 16;
+      for (int i = 0; i < 7; ++i) atomicAdd(&g_seg[slow][i], (unsigned long long)ctl.seg[i]);
+      atomicAdd(&g_seg[slow][7], 1ull);
+    }
+    ctl.pass_begin = now;
+  }
+#endif
+  // ---- the slots move up ------------------------------------------------------------------------------------
+  s0 = s1;
+  s1 = s2;
+  s2 = s3;
+  return s0.chunk >= 0 || s1.chunk >= 0 || s2.chunk >= 0;
 }
 
-// Compiled for four waves per SIMD (128 registers per lane), i.e. four workgroups per CU, which is also
-// what the 36 KB of LDS per workgroup allows: 1024 chunks on 256 CUs, two of the largest supported
-// tensors at once, so that memory stays busy while the workgroups of one tensor wait.
-constexpr int kResidentWavesPerSimd = 4;
+// Two workgroups per CU (two waves per SIMD, 256 registers per lane): a workgroup holds g of two chunks,
+// u_m and u_g of two more (one of them being filled from the first g) and 64 KB of parameters in LDS.
+constexpr int kResidentWavesPerSimd = 2;
 
-// Start of a resident step: clears the ticket, the error flag and the arrival counters and moves the
-// step epoch on.  The epoch lives on the device so that a step recorded in a graph tags every replay
-// differently; when it wraps (2^32 steps) every word of earlier steps is forgotten.
+// Start of a resident step: clears the ticket and the arrival counters and moves the step epoch on.  The
+// epoch lives on the device so that a step recorded in a graph tags every replay differently; when it
+// wraps (2^31 steps) every word of earlier steps is forgotten.  The error word is left alone.
 __global__ __launch_bounds__(kLansThreads) void lans_begin_kernel(LansTables t, size_t nwords) {
+#ifdef LANCET_LANS_TIMING
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    const long long* d = reinterpret_cast<const long long*>(t.partial);
+    const char* names[8] = {"N published", "G resolved (M starts)", "M published", "U norms resolved", "", "", "G word read ahead", "U words read ahead"};
+    long long base = d[0];
+    for (int w = 0; w < 512; ++w) if (d[w * 8] && d[w * 8] < base) base = d[w * 8];
+    for (int e = 0; e < 8; ++e) {
+      if (e == 4 || e == 5) continue;
+      long long lo = 1ll << 62, hi = 0, sum = 0; int n = 0;
+      for (int w = 0; w < 512; ++w) { const long long x = d[w * 8 + e]; if (!x) continue; lo = x < lo ? x : lo; hi = x > hi ? x : hi; sum += x; ++n; }
+      if (n) printf("tensor 100 event %d n %d min %d avg %d max %d (x10ns)\n", e, n, (int)(lo - base), (int)(sum / n - base), (int)(hi - base));
+    }
+    for (int b = 0; b < 64; b += 8)
+      printf("pass duration histogram, 2 us bins from %d us: %u %u %u %u %u %u %u %u\n", 2 * b, g_hist[b], g_hist[b + 1], g_hist[b + 2], g_hist[b + 3], g_hist[b + 4], g_hist[b + 5], g_hist[b + 6], g_hist[b + 7]);
+    for (int b = 0; b < 64; ++b) g_hist[b] = 0;
+    for (int k = 0; k < 2; ++k) {
+      const unsigned long long n = g_seg[k][7] ? g_seg[k][7] : 1;
+      printf("%s passes %llu: avg cycles start %llu M %llu sumpub %llu draw %llu N %llu pay+preU %llu U %llu\n", k ? "slow (>=32us)" : "fast", g_seg[k][7],
+             g_seg[k][0] / n, g_seg[k][1] / n, g_seg[k][2] / n, g_seg[k][3] / n, g_seg[k][4] / n, g_seg[k][5] / n, g_seg[k][6] / n);
+      for (int i = 0; i < 8; ++i) g_seg[k][i] = 0;
+    }
+    long long wlo = 1ll << 62, whi = 0, wsum = 0; int ilo = 0, ihi = 0;
+    for (int w = 0; w < 512; ++w) { if (g_wait[w] < wlo) { wlo = g_wait[w]; ilo = w; } if (g_wait[w] > whi) { whi = g_wait[w]; ihi = w; } wsum += g_wait[w]; }
+    printf("cycles in acquire per wg (cumulative): min %lld (wg %d) avg %lld max %lld (wg %d)\n", wlo, ilo, wsum / 512, whi, ihi);
+    printf("wg %d: hits %u polled-then-words %u polled-then-summed %u;  wg %d: %u %u %u\n", ilo, g_modes[ilo][0], g_modes[ilo][1], g_modes[ilo][2], ihi, g_modes[ihi][0], g_modes[ihi][1], g_modes[ihi][2]);
+  }
+#endif
   const size_t i = blockIdx.x * static_cast<size_t>(kLansThreads) + threadIdx.x;
-  if (i < 2 + static_cast<size_t>(t.T)) t.ticket[i] = 0u;
+  if (i < 2 * static_cast<size_t>(t.T)) t.ctl[kCtlArrive + i] = 0u;
+  if (i == 0) t.ctl[kCtlTicket] = 0u;
   if (blockIdx.x == 0) {
-    uint32_t* ep = t.ticket + 2 + t.T;
-    const uint32_t e = *ep + 1u;
+    uint32_t* ep = t.ctl + kCtlEpoch;
+    const uint32_t e = (*ep + 1u) & ~kPoison;
     if (e == 0u)
       for (size_t k = threadIdx.x; k < nwords; k += kLansThreads) t.part_word[k] = 0;  // norm words follow
     __syncthreads();
@@ -598,23 +1031,48 @@ __global__ __launch_bounds__(kLansThreads) void lans_begin_kernel(LansTables t, 
 }
 
 __global__ __launch_bounds__(kLansThreads, kResidentWavesPerSimd) void lans_resident_kernel(LansTables t, LansScalars sc) {
-  __shared__ ResidentShared sh;
-  sc.epoch = __builtin_amdgcn_readfirstlane(t.ticket[2 + t.T]);
+  __shared__ PipeShared sh;
+  sc.epoch = __builtin_amdgcn_readfirstlane(t.ctl[kCtlEpoch]);
   float bc1, bc2;
   bias_corrections(sc, bc1, bc2);
-  while (true) {
-    __syncthreads();  // shared words of the previous chunk are no longer read
-    if (threadIdx.x == 0) sh.chunk = static_cast<int>(atomicAdd(t.ticket, 1u));
-    __syncthreads();
-    // one value for the whole workgroup, and known to be: pointers and sizes derived from it stay scalar
-    const int chunk = __builtin_amdgcn_readfirstlane(sh.chunk);
-    if (chunk >= t.nres) break;  // every workgroup reaches this: chunks are finite
-    const ChunkView c = chunk_view(t, chunk);
-    const bool full = c.n == kLansChunk &&
-                      vec_ok(t.g[c.tensor], t.p[c.tensor], t.m[c.tensor], t.v[c.tensor]);
-    if (full) resident_chunk(t, sc, c, chunk, bc1, bc2, sh);
-    else resident_chunk_streamed(t, sc, c, chunk, bc1, bc2, sh);
+  bc1 = uniform(bc1);
+  bc2 = uniform(bc2);
+  // s0: between stages M and U; s1, s2: between stages N and M, s1 the older.  Register arrays rotate with
+  // the slots: g of s1 / s2 alternates between ga and gb, the updates between parity 0 and 1.
+  f32x4 ga[kVecPerThread], gb[kVecPerThread];
+  f32x4 um0[kVecPerThread], ug0[kVecPerThread], um1[kVecPerThread], ug1[kVecPerThread];
+  Slot s0, s1, s2;
+  s0.chunk = s1.chunk = s2.chunk = -1;
+  s0.tensor = s1.tensor = s2.tensor = -1;
+  s0.dead = s1.dead = s2.dead = 0;
+  s0.owes = s1.owes = s2.owes = 0;
+  Control ctl;
+  ctl.ticket = 0u;
+  ctl.g_word[0] = 0;
+  ctl.u_word[0] = ctl.u_word[1] = ctl.u_word[2] = 0;
+#ifdef LANCET_LANS_TIMING
+  for (int i = 0; i < 8; ++i) ctl.acc[i] = 0;
+  ctl.pass_begin = 0;
+  ctl.last = clock64();
+  const long long t_begin = ctl.last;
+#endif
+  // the first two passes find empty slots (their stages M and U have nothing to do) and fill the pipeline;
+  // every pass draws a ticket, tickets run out, and every wait is bounded: all workgroups leave
+  bool more = pipeline_pass<0>(t, sc, bc1, bc2, s0, s1, s2, ctl, ga, um0, ug0, um1, ug1, sh) &&
+              pipeline_pass<1>(t, sc, bc1, bc2, s0, s1, s2, ctl, gb, um1, ug1, um0, ug0, sh, LANCET_LANS_ALIGN != 0);
+  while (more) {
+    if (!pipeline_pass<0>(t, sc, bc1, bc2, s0, s1, s2, ctl, ga, um0, ug0, um1, ug1, sh)) break;
+    if (!pipeline_pass<1>(t, sc, bc1, bc2, s0, s1, s2, ctl, gb, um1, ug1, um0, ug0, sh)) break;
   }
+#ifdef LANCET_LANS_TIMING
+  if (threadIdx.x == 0 && (blockIdx.x % 128) == 5)
+    printf("misses(all wgs so far) %llu spins(all wgs so far) %u\n", g_misses, t.ctl[3]);
+  if (threadIdx.x == 0) atomicMax(&g_most, (unsigned)ctl.acc[7]), atomicMin(&g_fewest, (unsigned)ctl.acc[7]);
+  if (threadIdx.x == 0 && (blockIdx.x % 128) == 5) printf("chunks of this wg %lld; fewest/most over wgs that have finished: %u %u\n", ctl.acc[7], g_fewest, g_most);
+  if (threadIdx.x == 0 && (blockIdx.x % 128) == 5)
+    printf("wg %3d total %lld: start %lld M %lld sumpub %lld draw %lld N %lld preU %lld U %lld\n", blockIdx.x,
+           clock64() - t_begin, ctl.acc[0], ctl.acc[1], ctl.acc[2], ctl.acc[3], ctl.acc[4], ctl.acc[5], ctl.acc[6]);
+#endif
 }
 
 }  // namespace lancet
@@ -628,72 +1086,84 @@ struct lancet_lans_plan {
   uint32_t magic;
   int device;
   int T;
-  int nchunks;
+  int nchunks;                      // chunk slots, padding included
   std::vector<int64_t> numels;
   std::vector<const void*> shadow;  // last uploaded 4T pointers
   void* dev_block;                  // one allocation holding every table
   void** h_ptrs;                    // pinned staging for the pointer tables
+  uint32_t* h_status;               // pinned word the resident kernel sets with its error word
   hipEvent_t upload_done;
   bool upload_pending;
   LansTables tables;
   int schedule;           // LANCET_LANS_SWEEPS or LANCET_LANS_RESIDENT
   int resident_grid;      // workgroups of the resident schedule the device runs at once
   int max_tensor_chunks;  // chunks of the largest tensor
-  int resident_limit;     // chunks of the largest tensor the resident schedule holds on this device
+  int resident_limit;     // chunks of the largest tensor the resident schedule takes on this device
   int n_res_tensors;      // tensors within that limit: the first ones in the plan's own order
-  int n_res_chunks;
+  int n_res_chunks;       // chunk slots the resident kernel hands out (padding included)
   std::vector<int32_t> order;  // plan position -> position in the caller's lists
-  size_t words_offset; // part_word + norm_word inside dev_block
   size_t words_bytes;
+  uint32_t spin_limit;
 };
 
 static constexpr uint32_t kPlanMagic = 0x4c414e53u;  // "LANS"
+static constexpr uint32_t kDefaultSpinLimit = 1u << 20;  // about a second of polling; a healthy wait is microseconds
 
 static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+static inline int chunks_of(int64_t numel) { return static_cast<int>((numel + kLansChunk - 1) / kLansChunk); }
 
-static void chunk_tables(const int64_t* numels, int T, std::vector<int32_t>& ctensor, std::vector<int32_t>& first) {
-  first.assign(T + 1, 0);
-  ctensor.clear();
-  int c = 0;
+// The plan's own tensor order and chunk slots.  Tensors of at most `limit` chunks come first, largest first
+// (list order among equals), packed into rounds of `round` slots: a tensor that does not fit into what is
+// left of a round starts the next one and the rest of the round is padding (chunk_tensor -1), so that all
+// chunks of a tensor are drawn in the same pass of the resident kernel's workgroups.  Larger tensors follow
+// in list order, without padding: they go through the sweeps.  first[i] / ctensor are in plan order.
+struct ChunkLayout {
+  std::vector<int32_t> order, ctensor, first, count;
+  int n_fit = 0;       // tensors the resident kernel takes
+  int n_res_slots = 0; // slots it hands out
+};
+
+static ChunkLayout chunk_layout(const int64_t* numels, int T, int limit, int round) {
+  ChunkLayout L;
+  std::vector<int32_t> fit, big;
+  for (int i = 0; i < T; ++i) (chunks_of(numels[i]) <= limit ? fit : big).push_back(i);
+  std::stable_sort(fit.begin(), fit.end(), [&](int a, int b) { return chunks_of(numels[a]) > chunks_of(numels[b]); });
+  L.n_fit = static_cast<int>(fit.size());
+  L.order = fit;
+  L.order.insert(L.order.end(), big.begin(), big.end());
+  L.first.assign(T, 0);
+  L.count.assign(T, 0);
+  if (round < 1) round = 1;
   for (int i = 0; i < T; ++i) {
-    first[i] = c;
-    const int k = static_cast<int>((numels[i] + kLansChunk - 1) / kLansChunk);
-    for (int j = 0; j < k; ++j) ctensor.push_back(i);
-    c += k;
-  }
-  first[T] = c;
-}
-
-// The plan's own tensor order: tensors of at most `limit` chunks first (the resident schedule takes
-// those), the larger ones after them (they go through the sweeps), list order kept inside each group.
-static int tensor_order(const int64_t* numels, int T, int limit, std::vector<int32_t>& order) {
-  order.clear();
-  for (int pass = 0; pass < 2; ++pass)
-    for (int i = 0; i < T; ++i) {
-      const bool fits = (numels[i] + kLansChunk - 1) / kLansChunk <= limit;
-      if (fits == (pass == 0)) order.push_back(i);
+    const int k = chunks_of(numels[L.order[i]]);
+    if (i < L.n_fit && k <= round) {
+      const int used = static_cast<int>(L.ctensor.size()) % round;
+      if (used + k > round) L.ctensor.insert(L.ctensor.end(), round - used, -1);
     }
-  int n_fit = 0;
-  for (int i = 0; i < T; ++i) n_fit += (numels[i] + kLansChunk - 1) / kLansChunk <= limit;
-  return n_fit;
+    if (i == L.n_fit) L.n_res_slots = static_cast<int>(L.ctensor.size());
+    L.first[i] = static_cast<int32_t>(L.ctensor.size());
+    L.count[i] = k;
+    L.ctensor.insert(L.ctensor.end(), k, i);
+  }
+  if (L.n_fit == T) L.n_res_slots = static_cast<int>(L.ctensor.size());
+  return L;
 }
 
-// Host-only view of what a plan builds for `numels` when the resident schedule holds tensors of up to
-// `resident_limit` chunks (no device needed): for every chunk, in ticket order, the position of its
-// tensor in the caller's list; *n_resident_chunks = chunks the resident kernel hands out.
-extern "C" int64_t lancet_lans_debug_chunk_table(const int64_t* numels, int T, int resident_limit,
+// Host-only view of what a plan builds for `numels` when the resident kernel takes tensors of up to
+// `resident_limit` chunks and runs `round` workgroups (no device needed): for every chunk slot, in ticket
+// order, the position of its tensor in the caller's list (-1: padding); *n_resident_chunks = slots the
+// resident kernel hands out.
+extern "C" int64_t lancet_lans_debug_chunk_table(const int64_t* numels, int T, int resident_limit, int round,
                                                  int32_t* chunk_tensor_out, int64_t capacity,
                                                  int64_t* n_resident_chunks) {
   if (!numels || T <= 0) return -1;
-  std::vector<int32_t> order, ctensor, first;
-  const int n_fit = tensor_order(numels, T, resident_limit, order);
-  std::vector<int64_t> perm(T);
-  for (int i = 0; i < T; ++i) perm[i] = numels[order[i]];
-  chunk_tables(perm.data(), T, ctensor, first);
-  for (int64_t i = 0; i < capacity && i < static_cast<int64_t>(ctensor.size()); ++i)
-    if (chunk_tensor_out) chunk_tensor_out[i] = order[ctensor[i]];
-  if (n_resident_chunks) *n_resident_chunks = first[n_fit];
-  return static_cast<int64_t>(ctensor.size());
+  for (int i = 0; i < T; ++i)
+    if (numels[i] < 0) return -1;
+  const ChunkLayout L = chunk_layout(numels, T, resident_limit, round);
+  for (int64_t i = 0; i < capacity && i < static_cast<int64_t>(L.ctensor.size()); ++i)
+    if (chunk_tensor_out) chunk_tensor_out[i] = L.ctensor[i] < 0 ? -1 : L.order[L.ctensor[i]];
+  if (n_resident_chunks) *n_resident_chunks = L.n_res_slots;
+  return static_cast<int64_t>(L.ctensor.size());
 }
 
 extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans_plan_t* out) {
@@ -702,71 +1172,81 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
   int64_t nchunks64 = 0;
   for (int i = 0; i < T; ++i) {
     if (numels[i] < 0) return LANCET_ERR_SHAPE;
-    nchunks64 += (numels[i] + kLansChunk - 1) / kLansChunk;
+    nchunks64 += chunks_of(numels[i]);
   }
-  if (nchunks64 * kSweepSplit > 0x7fffffff) return LANCET_ERR_SHAPE;  // slices index the partial sums and the grids
+  // slices index the partial sums and the grids; padding at most doubles the slots
+  if (2 * nchunks64 * kSweepSplit > 0x7fffffff) return LANCET_ERR_SHAPE;
   lancet_lans_plan* pl = new (std::nothrow) lancet_lans_plan();
   if (!pl) return static_cast<int>(hipErrorOutOfMemory);
   pl->magic = kPlanMagic;
   pl->T = T;
-  pl->nchunks = static_cast<int>(nchunks64);
   pl->numels.assign(numels, numels + T);
   pl->shadow.assign(4 * static_cast<size_t>(T), nullptr);
   pl->dev_block = nullptr;
   pl->h_ptrs = nullptr;
+  pl->h_status = nullptr;
   pl->upload_done = nullptr;
   pl->upload_pending = false;
-  hipError_t err = hipGetDevice(&pl->device);
-  // device block layout
-  const size_t n = static_cast<size_t>(pl->nchunks);
-  size_t off = 0;
-  const size_t o_ptrs = off;      off = align_up(off + 4 * T * sizeof(void*), 256);
-  const size_t o_numel = off;     off = align_up(off + T * sizeof(int64_t), 256);
-  const size_t o_ctensor = off;   off = align_up(off + (n ? n : 1) * sizeof(int32_t), 256);
-  const size_t o_first = off;     off = align_up(off + (T + 1) * sizeof(int32_t), 256);
-  const size_t o_partial = off;   off = align_up(off + 3 * (n ? n : 1) * kSweepSplit * sizeof(float), 256);
-  const size_t o_norms = off;     off = align_up(off + 4 * T * sizeof(float), 256);
-  const size_t o_consts = off;    off = align_up(off + 2 * sizeof(float), 256);
-  const size_t o_words = off;     off = align_up(off + 4 * ((n ? n : 1) + T) * sizeof(uint64_t), 256);
-  const size_t o_ticket = off;    off = align_up(off + (3 + static_cast<size_t>(T)) * sizeof(uint32_t), 256);
-  const size_t o_order = off;     off = align_up(off + T * sizeof(int32_t), 256);
+  pl->spin_limit = kDefaultSpinLimit;
   pl->schedule = LANCET_LANS_SWEEPS;
-  pl->words_offset = o_words;
-  pl->words_bytes = 4 * ((n ? n : 1) + T) * sizeof(uint64_t);
+  hipError_t err = hipGetDevice(&pl->device);
   int cus = 256;
   if (err == hipSuccess) err = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, pl->device);
   pl->resident_grid = 0;
   pl->max_tensor_chunks = 0;
-  for (int i = 0; i < T; ++i)
-    pl->max_tensor_chunks = std::max<int>(pl->max_tensor_chunks, static_cast<int>((numels[i] + kLansChunk - 1) / kLansChunk));
+  for (int i = 0; i < T; ++i) pl->max_tensor_chunks = std::max(pl->max_tensor_chunks, chunks_of(numels[i]));
   if (err == hipSuccess) {
     int per_cu = 0;
     err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lans_resident_kernel, kLansThreads, 0);
     pl->resident_grid = per_cu * cus;
   }
+  // a tensor's chunks fit one round, so the kernel drains with half of its workgroups on the chip
   pl->resident_limit = std::min(pl->resident_grid, kMaxResidentChunks);
-  pl->n_res_tensors = tensor_order(numels, T, pl->resident_limit, pl->order);
+  const ChunkLayout L = chunk_layout(numels, T, pl->resident_limit, pl->resident_grid);
+  pl->order = L.order;
+  pl->n_res_tensors = L.n_fit;
+  pl->n_res_chunks = L.n_res_slots;
+  pl->nchunks = static_cast<int>(L.ctensor.size());
+  // device block layout
+  const size_t n = static_cast<size_t>(pl->nchunks);
+  const size_t n1 = n ? n : 1;
+  size_t off = 0;
+  const size_t o_ptrs = off;      off = align_up(off + 4 * T * sizeof(void*), 256);
+  const size_t o_numel = off;     off = align_up(off + T * sizeof(int64_t), 256);
+  const size_t o_ctensor = off;   off = align_up(off + n1 * sizeof(int32_t), 256);
+  const size_t o_first = off;     off = align_up(off + T * sizeof(int32_t), 256);
+  const size_t o_count = off;     off = align_up(off + T * sizeof(int32_t), 256);
+  const size_t o_partial = off;   off = align_up(off + 3 * n1 * kSweepSplit * sizeof(float), 256);
+  const size_t o_norms = off;     off = align_up(off + 4 * T * sizeof(float), 256);
+  const size_t o_consts = off;    off = align_up(off + 2 * sizeof(float), 256);
+  const size_t o_words = off;     off = align_up(off + 4 * (n1 + T) * sizeof(uint64_t), 256);
+  const size_t n_ctl = kCtlArrive + 2 * static_cast<size_t>(T);
+  const size_t o_ctl = off;       off = align_up(off + n_ctl * sizeof(uint32_t), 256);
+  const size_t o_order = off;     off = align_up(off + T * sizeof(int32_t), 256);
+  pl->words_bytes = 4 * (n1 + T) * sizeof(uint64_t);
   if (err == hipSuccess) err = hipMalloc(&pl->dev_block, off);
   if (err == hipSuccess) err = hipHostMalloc(reinterpret_cast<void**>(&pl->h_ptrs), 4 * T * sizeof(void*), hipHostMallocDefault);
+  if (err == hipSuccess) err = hipHostMalloc(reinterpret_cast<void**>(&pl->h_status), 64, hipHostMallocDefault);
   if (err == hipSuccess) err = hipEventCreateWithFlags(&pl->upload_done, hipEventDisableTiming);
   if (err == hipSuccess) {
-    std::vector<int32_t> ctensor, first;
+    *pl->h_status = 0u;
     std::vector<int64_t> perm(T);
     for (int i = 0; i < T; ++i) perm[i] = numels[pl->order[i]];
-    chunk_tables(perm.data(), T, ctensor, first);
-    pl->n_res_chunks = first[pl->n_res_tensors];
     char* base = static_cast<char*>(pl->dev_block);
     err = hipMemcpy(base + o_numel, perm.data(), T * sizeof(int64_t), hipMemcpyHostToDevice);
     if (err == hipSuccess) err = hipMemcpy(base + o_order, pl->order.data(), T * sizeof(int32_t), hipMemcpyHostToDevice);
-    if (err == hipSuccess && n) err = hipMemcpy(base + o_ctensor, ctensor.data(), n * sizeof(int32_t), hipMemcpyHostToDevice);
-    if (err == hipSuccess) err = hipMemcpy(base + o_first, first.data(), (T + 1) * sizeof(int32_t), hipMemcpyHostToDevice);
+    if (err == hipSuccess && n) err = hipMemcpy(base + o_ctensor, L.ctensor.data(), n * sizeof(int32_t), hipMemcpyHostToDevice);
+    if (err == hipSuccess) err = hipMemcpy(base + o_first, L.first.data(), T * sizeof(int32_t), hipMemcpyHostToDevice);
+    if (err == hipSuccess) err = hipMemcpy(base + o_count, L.count.data(), T * sizeof(int32_t), hipMemcpyHostToDevice);
     if (err == hipSuccess) err = hipMemset(base + o_norms, 0, 4 * T * sizeof(float));
     if (err == hipSuccess) err = hipMemset(base + o_words, 0, pl->words_bytes);
-    if (err == hipSuccess) err = hipMemset(base + o_ticket, 0, (3 + static_cast<size_t>(T)) * sizeof(uint32_t));
+    if (err == hipSuccess) err = hipMemset(base + o_ctl, 0, n_ctl * sizeof(uint32_t));
     LansTables& t = pl->tables;
     t.part_word = reinterpret_cast<uint64_t*>(base + o_words);
-    t.norm_word = t.part_word + 4 * (n ? n : 1);
-    t.ticket = reinterpret_cast<uint32_t*>(base + o_ticket);
+    t.norm_word = t.part_word + 4 * n1;
+    t.ctl = reinterpret_cast<uint32_t*>(base + o_ctl);
+    t.host_status = nullptr;
+    if (err == hipSuccess) err = hipHostGetDevicePointer(reinterpret_cast<void**>(&t.host_status), pl->h_status, 0);
     void** dptrs = reinterpret_cast<void**>(base + o_ptrs);
     t.g = reinterpret_cast<const float* const*>(dptrs);
     t.p = reinterpret_cast<float* const*>(dptrs + T);
@@ -775,13 +1255,16 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
     t.numel = reinterpret_cast<const int64_t*>(base + o_numel);
     t.chunk_tensor = reinterpret_cast<const int32_t*>(base + o_ctensor);
     t.tensor_first = reinterpret_cast<const int32_t*>(base + o_first);
+    t.tensor_chunks = reinterpret_cast<const int32_t*>(base + o_count);
     t.partial = reinterpret_cast<float*>(base + o_partial);
     t.norms = reinterpret_cast<float*>(base + o_norms);
     t.consts = reinterpret_cast<float*>(base + o_consts);
     t.order = reinterpret_cast<const int32_t*>(base + o_order);
+    t.grad_norms = nullptr;
     t.T = T;
     t.nchunks = pl->nchunks;
     t.nres = pl->n_res_chunks;
+    t.debug_flags = 0u;
   }
   if (err != hipSuccess) {
     lancet_lans_plan_destroy(pl);
@@ -798,6 +1281,7 @@ extern "C" int lancet_lans_plan_destroy(lancet_lans_plan_t pl) {
     (void)hipEventDestroy(pl->upload_done);
   }
   if (pl->h_ptrs) (void)hipHostFree(pl->h_ptrs);
+  if (pl->h_status) (void)hipHostFree(pl->h_status);
   if (pl->dev_block) (void)hipFree(pl->dev_block);
   pl->magic = 0;
   delete pl;
@@ -814,13 +1298,17 @@ extern "C" int lancet_lans_plan_norms(lancet_lans_plan_t pl, float* norms, lance
 extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, float* const* p,
                                 float* const* m, float* const* v, int step_host,
                                 const float* step_dev, const lancet_lans_hyper* h,
-                                lancet_stream_t stream) {
+                                const float* grad_norms, lancet_stream_t stream) {
   if (!pl || pl->magic != kPlanMagic) return LANCET_ERR_PLAN;
   if (!g || !p || !m || !v || !h) return LANCET_ERR_NULL;
   if (!step_dev && step_host < 1) return LANCET_ERR_SHAPE;
   if (h->mode != 0 && h->mode != 1) return LANCET_ERR_SHAPE;
   int current = -1;
   if (hipGetDevice(&current) != hipSuccess || current != pl->device) return LANCET_ERR_PLAN;  // tables live on pl->device
+  // an earlier step of this plan gave up a wait: nothing more is launched until lancet_lans_plan_error
+  // has been called (the word is written by the device; reading it needs no synchronisation)
+  if (__atomic_load_n(pl->h_status, __ATOMIC_RELAXED) != 0u) return LANCET_ERR_STALLED;
+  if (reinterpret_cast<uintptr_t>(grad_norms) & 3u) return LANCET_ERR_ALIGN;
   const int T = pl->T;
   hipStream_t st = static_cast<hipStream_t>(stream);
   bool changed = false;
@@ -869,19 +1357,18 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
   sc.bias_correction = h->bias_correction;
   sc.step_host = step_host;
   sc.step_dev = step_dev;
-  const LansTables& t = pl->tables;
-  sc.spin_limit = current_spin_limit();
-  // chunks [0, chunk_base) and tensors [0, tensor_base) go through the resident kernel, the rest
+  LansTables t = pl->tables;
+  t.grad_norms = grad_norms;
+  sc.spin_limit = pl->spin_limit;
+  sc.epoch = 0;
+  if (grad_norms) lans_take_grad_norms_kernel<<<(T + 255) / 256, 256, 0, st>>>(t);
+  // slots [0, chunk_base) and tensors [0, tensor_base) go through the resident kernel, the rest
   // (everything, under the sweeps schedule) through the three sweeps
   int chunk_base = 0, tensor_base = 0;
-  sc.epoch = 0;
   if (pl->schedule == LANCET_LANS_RESIDENT && pl->n_res_chunks > 0) {
-    const unsigned begin_blocks = static_cast<unsigned>((2 + static_cast<size_t>(T) + kLansThreads - 1) / kLansThreads);
+    const unsigned begin_blocks = static_cast<unsigned>((2 * static_cast<size_t>(T) + kLansThreads - 1) / kLansThreads);
     lans_begin_kernel<<<begin_blocks, kLansThreads, 0, st>>>(t, pl->words_bytes / sizeof(uint64_t));
     const int grid = std::min(pl->resident_grid, pl->n_res_chunks);
-    const int per_block = kLansThreads / kWave;
-    lans_norm_g_kernel<<<pl->n_res_chunks, kLansThreads, 0, st>>>(t, 0);
-    lans_reduce_kernel<<<(pl->n_res_tensors + per_block - 1) / per_block, kLansThreads, 0, st>>>(t, 0, 0, pl->n_res_tensors, 1, 1);
     lans_resident_kernel<<<grid, kLansThreads, 0, st>>>(t, sc);
     chunk_base = pl->n_res_chunks;
     tensor_base = pl->n_res_tensors;
@@ -891,8 +1378,10 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
     const int per_block = kLansThreads / kWave;
     const int rblocks = (T - tensor_base + per_block - 1) / per_block;
     lans_prepare_kernel<<<1, 64, 0, st>>>(t, sc);
-    lans_norm_g_kernel<<<nsweep, kLansThreads, 0, st>>>(t, chunk_base);
-    lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 0, tensor_base, T, 1, 1);
+    if (!grad_norms) {
+      lans_norm_g_kernel<<<nsweep, kLansThreads, 0, st>>>(t, chunk_base);
+      lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 0, tensor_base, T, 1, 1);
+    }
     lans_moments_kernel<<<nsweep * kSweepSplit, kLansThreads, 0, st>>>(t, sc, chunk_base);
     lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 1, tensor_base, T, 3, kSweepSplit);
     lans_update_kernel<<<nsweep * kSweepSplit, kLansThreads, 0, st>>>(t, sc, chunk_base);
@@ -903,8 +1392,8 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
 extern "C" int lancet_lans_plan_set_schedule(lancet_lans_plan_t pl, int schedule) {
   if (!pl || pl->magic != kPlanMagic) return LANCET_ERR_PLAN;
   if (schedule != LANCET_LANS_SWEEPS && schedule != LANCET_LANS_RESIDENT) return LANCET_ERR_SHAPE;
-  // a tensor's chunks must all be held by running workgroups at once; tensors too large for that go
-  // through the sweeps inside the same step, and a plan made only of such tensors has no use for the kernel
+  // tensors too large for the resident kernel go through the sweeps inside the same step; a plan made only
+  // of such tensors has no use for the kernel
   if (schedule == LANCET_LANS_RESIDENT && pl->n_res_chunks == 0 && pl->nchunks > 0) return LANCET_ERR_SHAPE;
   pl->schedule = schedule;
   return LANCET_OK;
@@ -922,8 +1411,22 @@ extern "C" int lancet_lans_plan_error(lancet_lans_plan_t pl, lancet_stream_t str
   if (!error_out) return LANCET_ERR_NULL;
   uint32_t word = 0;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  hipError_t e = hipMemcpyAsync(&word, pl->tables.ticket + 1, sizeof(word), hipMemcpyDeviceToHost, st);
+  hipError_t e = hipMemcpyAsync(&word, pl->tables.ctl + kCtlError, sizeof(word), hipMemcpyDeviceToHost, st);
   if (e == hipSuccess) e = hipStreamSynchronize(st);
+  // the reader, and only the reader, clears the error (the steps on `stream` have finished)
+  if (e == hipSuccess && (word != 0u || __atomic_load_n(pl->h_status, __ATOMIC_RELAXED) != 0u)) {
+    word = 1u;
+    e = hipMemsetAsync(pl->tables.ctl + kCtlError, 0, sizeof(uint32_t), st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    __atomic_store_n(pl->h_status, 0u, __ATOMIC_RELAXED);
+  }
   *error_out = static_cast<int>(word);
   return static_cast<int>(e);
+}
+
+extern "C" int lancet_lans_plan_debug(lancet_lans_plan_t pl, unsigned spin_limit, unsigned flags) {
+  if (!pl || pl->magic != kPlanMagic) return LANCET_ERR_PLAN;
+  pl->spin_limit = spin_limit ? spin_limit : kDefaultSpinLimit;
+  pl->tables.debug_flags = flags;
+  return LANCET_OK;
 }

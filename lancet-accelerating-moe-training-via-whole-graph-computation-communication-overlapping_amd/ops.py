@@ -550,9 +550,14 @@ class LansPlan:
         return wg.value, mx.value
 
     def error(self):
+        """Reads and clears the plan's sticky error (synchronises the current stream)."""
         err = C.c_int(-1)
         capi.check(self._lib.lancet_lans_plan_error(self._h, _stream(), C.byref(err)), "lancet_lans_plan_error")
         return err.value
+
+    def debug(self, spin_limit=0, flags=0):
+        """Test hook (include/lancet_hip_debug.h): bound of the resident schedule's waits, bit 0 = withhold norms."""
+        capi.check(self._lib.lancet_lans_plan_debug(self._h, int(spin_limit), int(flags)), "lancet_lans_plan_debug")
 
     def close(self):
         if self._h is not None:
@@ -565,8 +570,14 @@ class LansPlan:
         except Exception:
             pass
 
-    def step(self, g, p, m, v, step, hyper, step_dev=None):
+    def step(self, g, p, m, v, step, hyper, step_dev=None, grad_norms=None):
+        """One LANS step.  grad_norms: optional float32 GPU tensor [T] of ||g_i|| in list order (skips the
+        step's own pass over g).  Raises LancetError(ERR_STALLED) when an earlier step of the resident
+        schedule gave up a wait, until error() has been read."""
         T = len(self.numels)
+        if grad_norms is not None:
+            _need(grad_norms.is_cuda and grad_norms.dtype == torch.float32 and grad_norms.numel() == T and
+                  grad_norms.is_contiguous(), "grad_norms must be a contiguous float32 GPU tensor of T values")
         _need(len(g) == len(p) == len(m) == len(v) == T, "tensor lists must have one entry per planned tensor")
         for lst in (g, p, m, v):
             for t, n in zip(lst, self.numels):
@@ -574,7 +585,7 @@ class LansPlan:
                       "LANS tensors must be contiguous float32 GPU tensors of the planned sizes")
         arrs = [capi.ptr_array([t.data_ptr() for t in lst]) for lst in (g, p, m, v)]
         st = self._lib.lancet_lans_step(self._h, arrs[0], arrs[1], arrs[2], arrs[3], int(step),
-                                        _p(step_dev), C.byref(hyper), _stream())
+                                        _p(step_dev), C.byref(hyper), _p(grad_norms), _stream())
         capi.check(st, "lancet_lans_step")
 
     def norms(self):

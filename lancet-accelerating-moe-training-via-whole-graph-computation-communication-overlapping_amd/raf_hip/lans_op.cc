@@ -86,7 +86,7 @@ class LansImpl : public OpEnv {
       step_host = static_cast<int>(inputs[1].AsInt());
     }
     int st = lancet_lans_step(plan_, ptrs.data(), ptrs.data() + n, ptrs.data() + 2 * n, ptrs.data() + 3 * n,
-                              step_host, step_dev, &hyper_, GetStream(device_id_));
+                              step_host, step_dev, &hyper_, /*grad_norms=*/nullptr, GetStream(device_id_));
     if (st != LANCET_OK)
       throw Error(std::string("lancet_lans_step failed: ") + lancet_status_string(st) + " (status " + std::to_string(st) + ")");
   }

@@ -11,8 +11,8 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def header_symbols():
-    text = open(os.path.join(ROOT, "include", "lancet_hip.h")).read()
+def header_symbols(name="lancet_hip.h"):
+    text = open(os.path.join(ROOT, "include", name)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(lancet_[a-z0-9_]+)\s*\(", text)))
 
@@ -20,11 +20,14 @@ def header_symbols():
 def test_library_exports_every_declared_symbol(pkg):
     lib = pkg.capi.load()
     names = header_symbols()
+    hooks = header_symbols("lancet_hip_debug.h")
     assert len(names) >= 25
-    for n in names:
+    for n in names + hooks:
         assert hasattr(lib, n), "liblancet_hip.so does not export %s" % n
-    assert sorted(pkg.capi.SIGNATURES) == names, "capi.SIGNATURES and the header disagree"
-    assert lib.lancet_abi_version() == pkg.capi.ABI_VERSION == 3
+    assert sorted(pkg.capi.SIGNATURES) == sorted(names + hooks), "capi.SIGNATURES and the headers disagree"
+    assert lib.lancet_abi_version() == pkg.capi.ABI_VERSION == 4
+    # test and measurement hooks live in their own header; the operator surface declares none
+    assert not [n for n in names if "debug" in n] and all("debug" in n for n in hooks)
 
 
 def test_capacity_formula(pkg):
@@ -206,53 +209,102 @@ def test_op_layer_errors_are_reported_not_fatal(pkg):
 
 
 # ----------------------------------------------------------------------------- LANS task queue
-def _chunk_table(pkg, numels, limit=1 << 30):
-    """(tensor of every chunk in ticket order, chunks the resident kernel hands out)."""
+def _chunk_table(pkg, numels, limit=1 << 30, round_=1 << 30):
+    """(tensor of every chunk slot in ticket order, -1 = padding; slots the resident kernel hands out)."""
     lib = pkg.capi.load()
     arr = (C.c_int64 * len(numels))(*numels)
-    n = lib.lancet_lans_debug_chunk_table(arr, len(numels), limit, None, 0, None)
+    n = lib.lancet_lans_debug_chunk_table(arr, len(numels), limit, round_, None, 0, None)
     ctensor = np.empty(max(n, 1), np.int32)
     nres = C.c_int64(-1)
-    assert lib.lancet_lans_debug_chunk_table(arr, len(numels), limit, ctensor.ctypes.data_as(C.c_void_p), n,
+    assert lib.lancet_lans_debug_chunk_table(arr, len(numels), limit, round_, ctensor.ctypes.data_as(C.c_void_p), n,
                                              C.byref(nres)) == n
     return ctensor[:n], nres.value
 
 
-def _simulate_resident(ctensor, workers, rng):
-    """The resident LANS kernel as a state machine: `workers` workgroups take chunks in ticket order; a
-    workgroup publishes its chunk's partial sums once it has taken the chunk (nothing it needs for that comes
-    from another workgroup) and finishes, freeing itself for the next ticket, once every chunk of the tensor
-    has published.  Workgroups are advanced in random order.  Returns True when every chunk finishes, False
-    when no workgroup can move."""
+def _simulate_resident(ctensor, workers, rng, pay_before_waiting=True):
+    """The resident LANS kernel as a state machine.  Every workgroup runs passes of
+        [N duty] M(s1) [M duty if s0 and s1 share a tensor] U(s0) rotate [M duty] N(new s2)
+    on the chunk slots it draws in ticket order (the first two passes find s0 and s1 empty).  Stage N draws a
+    slot and counts it in at its tensor; the workgroup whose arrival completes a tensor owes it the norm and
+    pays at the next duty point of its own program.  Stage M of a slot needs the norm of stage N of its tensor,
+    stage U the norm of stage M.  Padding slots (-1) pass every stage at once.  Workgroups are advanced in
+    random order.  Returns True when every chunk has been through U, False when no workgroup can move.
+    pay_before_waiting=False moves the duties behind the waits (a workgroup that holds two chunks of a tensor
+    then waits for a norm it owes itself)."""
     n = len(ctensor)
-    size = np.bincount(ctensor, minlength=int(ctensor.max()) + 1 if n else 1)
-    published = np.zeros_like(size)
-    ticket, done = 0, 0
-    held = [None] * workers          # tensor of the chunk a workgroup holds
-    while done < n:
+    real = ctensor[ctensor >= 0]
+    size = np.bincount(real, minlength=int(real.max()) + 1 if len(real) else 1)
+    arrived = [np.zeros_like(size), np.zeros_like(size)]     # stage N, stage M
+    ready = [np.zeros(len(size), bool), np.zeros(len(size), bool)]
+    state = {"ticket": 0, "done": 0}
+
+    class WG:
+        def __init__(self):
+            self.s = [None, None, None]
+            self.owes = [None, None]       # tensor whose stage-N / stage-M norm this workgroup has to form
+            self.pc = 0
+
+    def is_real(x):
+        return x is not None and x >= 0
+
+    def arrive(w, stage, tensor):
+        arrived[stage][tensor] += 1
+        if arrived[stage][tensor] == size[tensor]:
+            w.owes[stage] = tensor
+
+    def pay(w, stage):
+        if w.owes[stage] is not None:
+            ready[stage][w.owes[stage]] = True
+            w.owes[stage] = None
+
+    wgs = [WG() for _ in range(workers)]
+    live = set(range(workers))
+    while live:
         moved = False
-        for w in rng.permutation(workers):
-            if held[w] is None:
-                if ticket < n:
-                    t = int(ctensor[ticket])
-                    ticket += 1
-                    published[t] += 1
-                    held[w] = t
+        for i in rng.permutation(sorted(live)):
+            w = wgs[i]
+            s0, s1, s2 = w.s
+            if w.pc == 0:                                   # stage M on s1
+                if pay_before_waiting:
+                    pay(w, 0)
+                if not is_real(s1) or ready[0][s1]:
+                    pay(w, 0)
+                    if is_real(s1):
+                        arrive(w, 1, s1)
+                    w.pc = 1
                     moved = True
-            elif published[held[w]] == size[held[w]]:
-                held[w] = None
-                done += 1
+            elif w.pc == 1:                                 # stage U on s0
+                if pay_before_waiting and is_real(s0) and s0 == s1:
+                    pay(w, 1)
+                if not is_real(s0) or ready[1][s0]:
+                    if is_real(s0):
+                        state["done"] += 1
+                    w.pc = 2
+                    moved = True
+            else:                                           # the slots move up, stage N draws a slot
+                pay(w, 1)
+                drawn = None
+                if state["ticket"] < n:
+                    drawn = int(ctensor[state["ticket"]])
+                    state["ticket"] += 1
+                    if drawn >= 0:
+                        arrive(w, 0, drawn)
+                w.s = [s1, s2, drawn]
+                w.pc = 0
                 moved = True
+                if all(x is None for x in w.s):
+                    pay(w, 0)
+                    live.discard(i)
         if not moved:
             return False
-    return True
+    return state["done"] == len(real)
 
 
 @pytest.mark.parametrize("case", ["config5", "random", "tiny"])
 def test_lans_resident_schedule_drains(pkg, case):
-    """A workgroup of the resident schedule waits only for chunks of its own tensor, and chunks are handed
-    out in list order, so the kernel drains whenever the workgroups on the chip are at least as many as the
-    chunks of the largest tensor (what lancet_lans_plan_set_schedule checks) and can stall with fewer."""
+    """A workgroup of the resident schedule waits only for chunks of tensors it holds, slots are handed out in
+    order, and a workgroup holds at most two slots that have not passed stage M: the kernel drains whenever the
+    running workgroups are at least half the chunks of the largest tensor, and stalls with fewer."""
     import bench
     rng = np.random.default_rng(0)
     if case == "config5":
@@ -261,30 +313,47 @@ def test_lans_resident_schedule_drains(pkg, case):
         numels = [int(x) for x in rng.integers(0, 600_000, 60)] + [0, 1, 8192, 8193]
     else:
         numels = [1, 2, 3]
-    ctensor, nres = _chunk_table(pkg, numels)
-    assert len(ctensor) == nres == sum((n + 8191) // 8192 for n in numels)
-    assert (np.diff(ctensor) >= 0).all()                       # chunks of a tensor are consecutive tickets
-    largest = int(np.bincount(ctensor).max())
-    for workers in (largest, largest + 3, 4 * largest):
-        assert _simulate_resident(ctensor, workers, rng)
-    if largest > 1:
-        assert not _simulate_resident(ctensor, largest - 1, rng)
+    chunks = [(x + 8191) // 8192 for x in numels]
+    largest = max(chunks)
+    for round_ in (largest, largest + 3, 4 * largest):
+        ctensor, nres = _chunk_table(pkg, numels, largest, round_)
+        assert len(ctensor) == nres
+        real = ctensor[ctensor >= 0]
+        np.testing.assert_array_equal(np.bincount(real, minlength=len(numels)), chunks)   # every chunk exactly once
+        assert (np.diff(np.flatnonzero(np.diff(real) != 0)) > 0).all()
+        for i in set(real.tolist()):                      # chunks of a tensor are consecutive slots of ONE round
+            where = np.flatnonzero(ctensor == i)
+            assert where[-1] - where[0] + 1 == len(where) and where[0] // round_ == where[-1] // round_
+        sizes = [chunks[i] for i in dict.fromkeys(real.tolist())]
+        assert sizes == sorted(sizes, reverse=True)       # largest tensors first
+        for workers in ((largest + 1) // 2, round_, round_ + 5):
+            assert _simulate_resident(ctensor, workers, rng)
+    if largest > 2:
+        ctensor, _ = _chunk_table(pkg, numels, largest, largest)
+        assert not _simulate_resident(ctensor, (largest + 1) // 2 - 1, rng)
+        # a workgroup that held two chunks of one tensor would wait for a norm it owes itself
+        assert not _simulate_resident(ctensor, (largest + 1) // 2, rng, pay_before_waiting=False)
 
 
 def test_lans_plan_orders_tensors_that_do_not_fit_last(pkg):
-    """Tensors with more chunks than the resident kernel holds come after all the others in the plan's
-    ticket order and are left to the sweeps; every chunk of every tensor appears exactly once."""
+    """Tensors with more chunks than the resident kernel takes come after all the others in the plan's
+    slot order, without padding, and are left to the sweeps; every chunk of every tensor appears exactly once."""
     numels = [100, 5 * 8192, 8192 * 40 + 1, 3, 8192 * 41, 8192 * 40, 0, 7 * 8192]
     limit = 40
-    ctensor, nres = _chunk_table(pkg, numels, limit)
+    ctensor, nres = _chunk_table(pkg, numels, limit, limit)
     chunks = [(n + 8191) // 8192 for n in numels]
-    assert len(ctensor) == sum(chunks)
-    np.testing.assert_array_equal(np.bincount(ctensor, minlength=len(numels)), chunks)
+    real = ctensor[ctensor >= 0]
+    np.testing.assert_array_equal(np.bincount(real, minlength=len(numels)), chunks)
     fits = [i for i, c in enumerate(chunks) if c <= limit]
-    assert nres == sum(chunks[i] for i in fits)
-    assert set(ctensor[:nres]) == {i for i in fits if chunks[i] > 0}
-    assert list(dict.fromkeys(ctensor[nres:])) == [2, 4]        # list order is kept inside each group
+    assert set(ctensor[:nres]) - {-1} == {i for i in fits if chunks[i] > 0}
+    # rounds of 40 slots: [tensor 5 (40)] [tensor 7 (7), tensor 1 (5), tensors 0 and 3 (1 each)]: no padding needed
+    assert nres == sum(chunks[i] for i in fits) and (ctensor[:nres] >= 0).all()
+    assert list(dict.fromkeys(ctensor[:nres])) == [5, 7, 1, 0, 3]
+    assert list(dict.fromkeys(ctensor[nres:])) == [2, 4] and (ctensor[nres:] >= 0).all()   # list order, no padding
     assert _simulate_resident(ctensor[:nres], limit, np.random.default_rng(1))
+    # a tensor that does not fit into what is left of a round starts the next one
+    ctensor, nres = _chunk_table(pkg, [3 * 8192, 3 * 8192, 3 * 8192], 4, 4)
+    assert ctensor.tolist() == [0, 0, 0, -1, 1, 1, 1, -1, 2, 2, 2] and nres == 11
 
 
 def test_missing_library_is_an_error_not_a_fallback(pkg, monkeypatch, tmp_path):

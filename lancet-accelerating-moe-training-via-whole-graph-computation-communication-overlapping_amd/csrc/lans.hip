@@ -40,13 +40,15 @@
 namespace lancet {
 
 constexpr int kLansThreads = 256;
-constexpr int kLansChunk = 8192;  // elements per task: 8 float4 per thread and array
+#ifndef LANCET_LANS_CHUNK
+#define LANCET_LANS_CHUNK 8192
+#endif
+constexpr int kLansChunk = LANCET_LANS_CHUNK;  // elements per task: kLansChunk / 1024 float4 per thread and array
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // control words of a plan (uint32): [0] next ticket of the resident kernel, [1] error (sticky: only
-// lancet_lans_plan_error clears it), [2] step epoch, [3] unused, then T arrival counters of stage N
-// and T of stage M
-constexpr int kCtlTicket = 0, kCtlError = 1, kCtlEpoch = 2, kCtlArrive = 4;
+// lancet_lans_plan_error clears it), [2] step epoch, [3] unused
+constexpr int kCtlTicket = 0, kCtlError = 1, kCtlEpoch = 2, kCtlWords = 4;
 
 struct LansTables {
   const float* const* g;  // [T] device pointers
@@ -336,7 +338,7 @@ __global__ void lans_prepare_kernel(LansTables t, LansScalars sc) {
 // one float4 per thread and array).  Short workgroups in address order stream a few percent faster than
 // workgroups that loop over a whole chunk; the chunk stays the unit of the tables and of the resident kernel.
 #ifndef LANCET_SWEEP_SPLIT
-#define LANCET_SWEEP_SPLIT 8
+#define LANCET_SWEEP_SPLIT (LANCET_LANS_CHUNK / 1024)
 #endif
 constexpr int kSweepSplit = LANCET_SWEEP_SPLIT;
 constexpr int kSweepSlice = kLansChunk / kSweepSplit;
@@ -437,37 +439,34 @@ __device__ __forceinline__ void flag_error(const LansTables& t) {
   __hip_atomic_store(t.host_status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
-struct Waited {
-  float value;
-  bool bad;  // the wait gave up, or the word was published poisoned
-};
+__device__ __forceinline__ bool word_is_current(uint64_t x, uint32_t epoch) {
+  return (static_cast<uint32_t>(x >> 32) & ~kPoison) == epoch;
+}
+__device__ __forceinline__ bool word_is_poisoned(uint64_t x) { return (static_cast<uint32_t>(x >> 32) & kPoison) != 0; }
 
-__device__ __forceinline__ Waited wait_word(const LansTables& t, const LansScalars& sc, const uint64_t* src) {
-#ifdef LANCET_LANS_PROBE
-  return Waited{1.f, false};
-#endif
+// Polls for a word of this step.  Bounded; and once any wait of the plan has given up the others stop early,
+// so that a stalled step ends after about one bound, not one per chunk.  Returns 0 (no tag) when it gives up.
+__device__ __forceinline__ uint64_t wait_word(const LansTables& t, const LansScalars& sc, const uint64_t* src) {
   uint64_t x = ld_word(src);
   uint32_t spins = 0;
-  while ((static_cast<uint32_t>(x >> 32) & ~kPoison) != sc.epoch) {
-    // bounded; and once any wait of the plan has given up the others stop early, so that a stalled step
-    // ends after about one bound, not one per chunk
+  while (!word_is_current(x, sc.epoch)) {
     if (++spins > sc.spin_limit || ((spins & 63u) == 0u && ld_agent(t.ctl + kCtlError) != 0u)) {
       flag_error(t);
-      return Waited{0.f, true};
+      return 0;
     }
     __builtin_amdgcn_s_sleep(2);
     x = ld_word(src);
   }
-#ifdef LANCET_LANS_TIMING
-  if (spins) atomicAdd(t.ctl + 3, spins);
-#endif
-  return Waited{__uint_as_float(static_cast<uint32_t>(x)), (static_cast<uint32_t>(x >> 32) & kPoison) != 0};
+  return x;
 }
 
 // =======================================================================================
 // schedule "resident": one persistent kernel, a three-stage software pipeline per workgroup
 // =======================================================================================
 constexpr int kVecPerThread = kLansChunk / 4 / kLansThreads;  // float4 per thread and array
+#ifndef LANCET_LANS_ALIGN
+#define LANCET_LANS_ALIGN 1
+#endif
 
 // Workgroup barrier that orders LDS accesses only.  __syncthreads() also waits for every global load and
 // store the wave has in flight, which would drain the streams of this kernel several times per chunk; all
@@ -485,113 +484,53 @@ __device__ __forceinline__ float block_sum_lds(float v, float* s_red) {
   }
   return r;  // valid on thread 0; s_red is free again after the caller's next barrier
 }
-#ifndef LANCET_LANS_ALIGN
-#define LANCET_LANS_ALIGN 1
-#endif
-#ifndef LANCET_LANS_SCHED_K
-#define LANCET_LANS_SCHED_K 0
-#endif
-constexpr int kMaxResidentChunks = 512;  // chunks of one tensor whose partials one workgroup sums
-constexpr uint32_t kPayPolls = 32;       // polls of a tensor's arrival counter at the end of stage N (tens of microseconds)
+
+constexpr int kMaxResidentChunks = 4 * 1024 * 1024 / kLansChunk;      // chunks of the largest tensor the kernel takes (4M parameters)
+constexpr int kGatherPerThread = kMaxResidentChunks / kLansThreads;  // partials of one norm a thread reads
+static_assert(kLansThreads / kWave == 4, "one wave per norm");
 
 struct PipeShared {
   f32x4 p[2][kVecPerThread][kLansThreads];  // parameters of the two chunks between stages M and U, one private slot per thread and float4
-  float part[3][kMaxResidentChunks];        // gathered chunk partials of a tensor
+  float part[4][kMaxResidentChunks];        // chunk partials: [0] of s2's tensor (g^2), [1..3] of s0's (p^2, u_m^2, u_g^2)
   float red[3][kLansThreads / kWave];
-  float norm[4];
+  float norm[4];   // [1..3]: the norms stage U of this pass needs
+  float g_next;    // ||g|| of s2's tensor: for stage M of the next pass
+  int g_next_bad;  // ... is unknown
+  int u_bad;       // a norm of s0's tensor is unknown
+  int retry;       // a sum read ahead was not there yet
   int chunk;
-  int mode;
-  int bad, gather_bad;
 };
 
 // a chunk a workgroup holds between stages; every field is uniform over the workgroup
 struct Slot {
   int chunk;   // -1: empty (the ticket ran out)
   int tensor;  // -1: padding slot, nothing to do
-  int n;       // elements
-  int full;    // whole chunk of 16-byte aligned arrays: plain global accesses
-  int dead;    // stage M was skipped (||g|| never came): the parameters stay as they are
+  int dead;    // stage M was skipped (||g|| unknown): the parameters stay as they are
   int lo, nc;  // first chunk slot and number of chunks of the tensor
-  int owes;    // bit k: this workgroup has to sum norm k of the tensor (see pay_norm)
   int64_t begin;
   __device__ __forceinline__ bool real() const { return chunk >= 0 && tensor >= 0; }
 };
 
-// What thread 0 of a workgroup has in flight towards other workgroups.  Every remote access of the
-// pipeline (ticket, arrival counters, norm words) is issued one stage before its result is looked at, so
-// that its latency passes while the workgroup streams; only a word that is still missing then is polled.
-struct Control {
-  uint32_t ticket;     // drawn at the start of a pass for its stage N
-  uint64_t g_word[1];  // ||g|| word of s2's tensor (s1's in the next pass), read in front of stage N's loads
-  uint64_t u_word[3];  // norm words of s0's tensor, read in front of stage N's loads
-#ifdef LANCET_LANS_TIMING
-  long long acc[8];
-  long long seg[8];
-  long long last;
-  long long pass_begin;
-#endif
-};
-
-// A partial chunk at the end of a tensor, and a tensor that is only 4-byte aligned, go through buffer
-// instructions: the descriptor carries the chunk's size in bytes, and the hardware checks every dword of an
-// access against it (out-of-range reads give zeros, which add nothing to any sum, out-of-range writes are
-// dropped), so they take the same 16-byte accesses as everything else, without a predicate per element.
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t chunk_rsrc(const float* base, int n) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, n * 4, 0x00020000);  // raw buffer of 32-bit words
+// The resident kernel only takes whole chunks of 16-byte aligned arrays (the plan leaves tensors that are not a
+// multiple of the chunk to the sweeps; a step whose pointers are not aligned runs as sweeps altogether): every
+// access is an unconditional, non-temporal float4.
+__device__ __forceinline__ f32x4 ld_chunk4(const LANCET_GLOBAL float* a, int e) {
+  return __builtin_nontemporal_load((const LANCET_GLOBAL f32x4*)(a + e));
 }
-// one array of a chunk: a plain pointer for whole chunks of 16-byte aligned arrays (global loads stream
-// faster than buffer loads here), a checked buffer otherwise
-template <bool FULL>
-struct ChunkArray {
-  LANCET_GLOBAL float* ptr;
-  __amdgpu_buffer_rsrc_t rsrc;
-  __device__ __forceinline__ ChunkArray(const float* base, int n) {
-    if (FULL) ptr = as_global(const_cast<float*>(base));
-    else rsrc = chunk_rsrc(base, n);
-  }
-  __device__ __forceinline__ f32x4 load(int e) const {
-    if (FULL) return __builtin_nontemporal_load((const LANCET_GLOBAL f32x4*)(ptr + e));
-    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, e * 4, 0, 2));
-  }
-  __device__ __forceinline__ void store(int e, f32x4 x) const {
-    if (FULL) __builtin_nontemporal_store(x, (LANCET_GLOBAL f32x4*)(ptr + e));
-    else __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, x), rsrc, e * 4, 0, 2);
-  }
-};
+__device__ __forceinline__ void st_chunk4(LANCET_GLOBAL float* a, int e, f32x4 x) {
+  __builtin_nontemporal_store(x, (LANCET_GLOBAL f32x4*)(a + e));
+}
 
-// a wave owns 2048 consecutive elements of the chunk: float4 k of lane l is element 4 * (64 k + l) of them,
-// so one load instruction of a wave covers 1 KB of consecutive memory
+// a wave owns a quarter of the chunk: float4 k of lane l is element 4 * (64 k + l) of it, so one load
+// instruction of a wave covers 1 KB of consecutive memory
 __device__ __forceinline__ int chunk_elem(int k) {
   return (threadIdx.x / kWave) * (kLansChunk / kWavesPerTile) + 4 * lane_id() + k * (4 * kWave);
 }
 
-#ifdef LANCET_LANS_TIMING
-__device__ unsigned long long g_misses, g_spins;
-__device__ unsigned g_most = 0, g_fewest = 0xffffffffu;
-__device__ long long g_wait[1024];
-__device__ unsigned g_hist[64];
-__device__ unsigned long long g_seg[2][8];
-__device__ unsigned g_modes[1024][3];
-#endif
-// A word read ahead: taken as it is when it carries this step's tag, polled for otherwise.
-__device__ __forceinline__ Waited resolve_word(const LansTables& t, const LansScalars& sc, uint64_t ahead, const uint64_t* src) {
-#ifdef LANCET_LANS_PROBE
-  return Waited{1.f, false};
-#endif
-  if ((static_cast<uint32_t>(ahead >> 32) & ~kPoison) == sc.epoch)
-    return Waited{__uint_as_float(static_cast<uint32_t>(ahead)), (static_cast<uint32_t>(ahead >> 32) & kPoison) != 0};
-#ifdef LANCET_LANS_TIMING
-  atomicAdd(&g_misses, 1ull);
-#endif
-  return wait_word(t, sc, src);
-}
-
-// Thread 0: publishes the N chunk sums a[] of slot s as words first .. first+N-1 and counts the chunk in at
-// the tensor's arrival counter (nothing comes back: no round trip).
+// Thread 0: publishes the N chunk sums a[] of slot s as words first .. first+N-1 (fire and forget).
 template <int N>
 __device__ __forceinline__ void publish(const LansTables& t, const LansScalars& sc, int first, const Slot& s,
-                                        const float (&a)[N], bool poison, uint32_t* arrive) {
+                                        const float (&a)[N], bool poison) {
 #ifdef LANCET_LANS_PROBE
   return;
 #endif
@@ -599,137 +538,50 @@ __device__ __forceinline__ void publish(const LansTables& t, const LansScalars& 
   const uint32_t tag = sc.epoch | (poison ? kPoison : 0u);
 #pragma unroll
   for (int k = 0; k < N; ++k) st_word(t.part_word + static_cast<size_t>(first + k) * t.nchunks + s.chunk, tag, a[k]);
-  (void)__hip_atomic_fetch_add(arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Who sums a tensor's partials.  Norm 0 (||g||) is summed by the workgroup that drew the tensor's first chunk,
-// norms 1, 2, 3 (||p||, ||u_m||, ||u_g||) by those that drew its first, second and third (chunk lo + (k - 1) %
-// nc).  Chunks are drawn in order, so these are workgroups that were ahead of the others when the tensor's
-// round began: they have the time, and the workgroup that arrives last, which everyone else is waiting for, is
-// spared (summing there would make it later still, tensor after tensor).  One norm is 512 words at most, two
-// loads per thread.  A workgroup pays what it owes at the end of stage N of the pass in which the tensor went
-// through the stage in question: it waits there, for a bounded short while, for the tensor's arrival counter
-// to fill up, which is normally long before anybody asks for the norm.  What is still owed then is paid when
-// the workgroup needs the norm itself.
-
-// norm `kind` of slot s's tensor: true when it has been formed and published (sh.norm[kind] holds it)
-__device__ __forceinline__ bool pay_norm(const LansTables& t, const LansScalars& sc, int kind, const Slot& s,
-                                         uint32_t max_polls, PipeShared& sh) {
-#ifdef LANCET_LANS_PROBE
-  return true;
-#endif
-  const uint32_t* arrive = t.ctl + kCtlArrive + (kind == 0 ? 0 : t.T) + s.tensor;
-  if (threadIdx.x == 0) {
-    uint32_t polls = 0;
-    bool full;
-    while (!(full = ld_agent(arrive) >= static_cast<uint32_t>(s.nc)) && ++polls <= max_polls) {
-      if ((polls & 63u) == 0u && ld_agent(t.ctl + kCtlError) != 0u) break;
-      __builtin_amdgcn_s_sleep(2);
-    }
-    sh.mode = full;
-    sh.gather_bad = 0;
-  }
-  lds_barrier();
-  if (__builtin_amdgcn_readfirstlane(sh.mode) == 0) return false;
-  // the partials (each a self-validating word: an arrival can be seen before the words it follows), every
-  // thread's loads in flight together
-  constexpr int kPerThread = kMaxResidentChunks / kLansThreads;
-  const uint64_t* words = t.part_word + static_cast<size_t>(kind) * t.nchunks + s.lo;
-  uint64_t word[kPerThread];
+// the partials of one norm of slot s's tensor as this thread reads them (issued, not yet looked at)
+__device__ __forceinline__ void gather_issue(const LansTables& t, int kind, const Slot& s, uint64_t (&word)[kGatherPerThread]) {
+  const uint64_t* src = t.part_word + static_cast<size_t>(kind) * t.nchunks + s.lo;
 #pragma unroll
-  for (int i = 0; i < kPerThread; ++i) {
+  for (int i = 0; i < kGatherPerThread; ++i) {
     const int c = threadIdx.x + i * kLansThreads;
-    word[i] = c < s.nc ? ld_word(words + c) : 0;
+    word[i] = c < s.nc ? ld_word(src + c) : 0;
   }
+}
+// ... looked at: values into LDS.  Straight-line: a word that is not there yet (or is poisoned) only raises
+// a flag; gather_again fetches those.
+__device__ __forceinline__ void gather_take(const LansScalars& sc, const Slot& s, const uint64_t (&word)[kGatherPerThread],
+                                            float* part, bool& retry) {
 #pragma unroll
-  for (int i = 0; i < kPerThread; ++i) {
+  for (int i = 0; i < kGatherPerThread; ++i) {
     const int c = threadIdx.x + i * kLansThreads;
     if (c < s.nc) {
-      const Waited w = resolve_word(t, sc, word[i], words + c);
-      sh.part[0][c] = w.value;
-      if (w.bad) sh.gather_bad = 1;  // a poisoned or missing partial poisons the norm
+      part[c] = __uint_as_float(static_cast<uint32_t>(word[i]));
+      retry = retry || !word_is_current(word[i], sc.epoch) || word_is_poisoned(word[i]);
     }
   }
-  lds_barrier();
-  if (threadIdx.x < kWave) {
-    const float n = wave_norm(0, s.nc, [&](int c) { return sh.part[0][c]; });  // fixed order: the same bits every time
-    if (lane_id() == 0) {
-      sh.norm[kind] = n;
-      t.norms[kind * t.T + s.tensor] = n;
-      st_word(t.norm_word + static_cast<size_t>(kind) * t.T + s.tensor, sc.epoch | (sh.gather_bad ? kPoison : 0u), n);
-    }
+}
+// The same partials again, polled for one by one (rare: a workgroup that is ahead of the one that publishes);
+// true when one stays missing (its wait gave up) or is poisoned.
+__device__ __forceinline__ bool gather_again(const LansTables& t, const LansScalars& sc, int kind, const Slot& s, float* part) {
+  const uint64_t* src = t.part_word + static_cast<size_t>(kind) * t.nchunks + s.lo;
+  bool bad = false;
+#pragma unroll 1
+  for (int c = threadIdx.x; c < s.nc; c += kLansThreads) {
+    const uint64_t x = wait_word(t, sc, src + c);
+    part[c] = __uint_as_float(static_cast<uint32_t>(x));
+    bad = bad || !word_is_current(x, sc.epoch) || word_is_poisoned(x);
   }
-  lds_barrier();
-  return true;
+  return bad;
 }
 
-// pays the norms of `kinds` (a bit mask) that slot s still owes
-__device__ __forceinline__ void pay_norms(const LansTables& t, const LansScalars& sc, Slot& s, int kinds,
-                                          uint32_t max_polls, PipeShared& sh) {
-#pragma unroll
-  for (int kind = 0; kind < 4; ++kind)
-    if ((s.owes & kinds & (1 << kind)) && pay_norm(t, sc, kind, s, max_polls, sh)) s.owes &= ~(1 << kind);
-}
-
-// Norms first .. first+N-1 of slot s's tensor into sh.norm; `ahead` are the norm words as thread 0 read them
-// ahead: when they carry this step's tag that is all.  Otherwise thread 0 polls for them (bounded).  Returns
-// true when the norms are unknown (a wait gave up, or a chunk was poisoned).  Called by the whole workgroup.
-template <int N>
-__device__ __forceinline__ bool acquire_norms(const LansTables& t, const LansScalars& sc, int first, Slot& s,
-                                              const uint64_t (&ahead)[N], PipeShared& sh) {
-#ifdef LANCET_LANS_PROBE
-  if (threadIdx.x == 0) for (int k = 0; k < N; ++k) sh.norm[first + k] = 1.f;
-  lds_barrier();
-  return false;
-#endif
-  const int kinds = ((1 << N) - 1) << first;
-  const bool owed = (s.owes & kinds) != 0;
-  if (owed) pay_norms(t, sc, s, kinds, sc.spin_limit, sh);  // nobody else will form them
-  if (threadIdx.x == 0) {
-#ifdef LANCET_LANS_TIMING
-    const long long t_in = clock64();
-#endif
-    uint64_t w[N];
-#pragma unroll
-    for (int k = 0; k < N; ++k) w[k] = owed ? 0 : ahead[k];
-    bool gave_up = false;
-    uint32_t spins = 0;
-    while (true) {
-      bool have = true;
-#pragma unroll
-      for (int k = 0; k < N; ++k) have = have && (static_cast<uint32_t>(w[k] >> 32) & ~kPoison) == sc.epoch;
-      if (have) break;
-      // bounded; and once any wait of the plan has given up the others stop early, so that a stalled step
-      // ends after about one bound, not one per chunk
-      if (++spins > sc.spin_limit || ((spins & 63u) == 0u && ld_agent(t.ctl + kCtlError) != 0u)) { gave_up = true; break; }
-      if (spins > 1) __builtin_amdgcn_s_sleep(2);
-#pragma unroll
-      for (int k = 0; k < N; ++k) w[k] = ld_word(t.norm_word + static_cast<size_t>(first + k) * t.T + s.tensor);
-    }
-    int bad = gave_up;
-    if (gave_up) flag_error(t);
-#pragma unroll
-    for (int k = 0; k < N; ++k) {
-      sh.norm[first + k] = __uint_as_float(static_cast<uint32_t>(w[k]));
-      bad |= (static_cast<uint32_t>(w[k] >> 32) & kPoison) != 0;
-    }
-    sh.bad = bad;
-#ifdef LANCET_LANS_TIMING
-    g_wait[blockIdx.x] += clock64() - t_in;
-    g_modes[blockIdx.x][spins == 0 ? 0 : 1] += 1;
-#endif
-  }
-  lds_barrier();
-  return __builtin_amdgcn_readfirstlane(sh.bad) != 0;
-}
-
-template <bool FULL>
 __device__ __forceinline__ float load_g(const LansTables& t, const Slot& s, f32x4 (&g)[kVecPerThread]) {
-  const ChunkArray<FULL> src(t.g[s.tensor] + s.begin, s.n);
+  const LANCET_GLOBAL float* src = as_global(t.g[s.tensor] + s.begin);
   float a = 0.f;
 #pragma unroll
   for (int k = 0; k < kVecPerThread; ++k) {
-    g[k] = src.load(chunk_elem(k));
+    g[k] = ld_chunk4(src, chunk_elem(k));
     a += g[k].x * g[k].x + g[k].y * g[k].y + g[k].z * g[k].z + g[k].w * g[k].w;
   }
   return a;
@@ -739,27 +591,29 @@ __device__ __forceinline__ float load_g(const LansTables& t, const Slot& s, f32x
 // around it, :428-441) of a chunk whose g sits in registers.  m and v are written; u_m, u_g stay in
 // registers and p in LDS for stage U.  The loads of float4 k+1 are issued before the stores of float4 k:
 // memory operations of a wave complete in order, so a load behind a store would wait for it.
-template <bool FULL, int PAR>
+template <int PAR>
 __device__ __forceinline__ void moments_chunk(const LansTables& t, const Slot& s, const LansElem& el,
                                               const f32x4 (&g)[kVecPerThread], f32x4 (&um)[kVecPerThread],
-                                              f32x4 (&ug)[kVecPerThread], PipeShared& sh, float (&a)[3]) {
-  const ChunkArray<FULL> p(t.p[s.tensor] + s.begin, s.n), m(t.m[s.tensor] + s.begin, s.n), v(t.v[s.tensor] + s.begin, s.n);
+                                              f32x4 (&ug)[kVecPerThread], PipeShared& sh, float (&a)[3], uint32_t ticket) {
+  const LANCET_GLOBAL float* p = as_global(t.p[s.tensor] + s.begin);
+  LANCET_GLOBAL float* m = as_global(t.m[s.tensor] + s.begin);
+  LANCET_GLOBAL float* v = as_global(t.v[s.tensor] + s.begin);
   float a0 = 0.f, a1 = 0.f, a2 = 0.f;
-  f32x4 np = p.load(chunk_elem(0));
-  f32x4 nm = m.load(chunk_elem(0)), nv = v.load(chunk_elem(0));
+  f32x4 np = ld_chunk4(p, chunk_elem(0));
+  f32x4 nm = ld_chunk4(m, chunk_elem(0)), nv = ld_chunk4(v, chunk_elem(0));
+  // the ticket drawn at the start of the pass is looked at here, behind three loads and in front of every
+  // store of the stage: looked at behind the stores it would cost their completion
+  if (threadIdx.x == 0) sh.chunk = static_cast<int>(ticket);
 #pragma unroll
   for (int k = 0; k < kVecPerThread; ++k) {
     const int e = chunk_elem(k);
     const f32x4 xp = np;
     f32x4 xm = nm, xv = nv;
     if (k + 1 < kVecPerThread) {
-      np = p.load(chunk_elem(k + 1));
-      nm = m.load(chunk_elem(k + 1));
-      nv = v.load(chunk_elem(k + 1));
+      np = ld_chunk4(p, chunk_elem(k + 1));
+      nm = ld_chunk4(m, chunk_elem(k + 1));
+      nv = ld_chunk4(v, chunk_elem(k + 1));
     }
-#if LANCET_LANS_SCHED_K
-    __builtin_amdgcn_sched_barrier(0);  // keeps the loads above the stores below
-#endif
     sh.p[PAR][k][threadIdx.x] = xp;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -778,56 +632,52 @@ __device__ __forceinline__ void moments_chunk(const LansTables& t, const Slot& s
       a1 += u0 * u0;
       a2 += u1 * u1;
     }
-    m.store(e, xm);
-    v.store(e, xv);
+    st_chunk4(m, e, xm);
+    st_chunk4(v, e, xv);
   }
   a[0] = a0;
   a[1] = a1;
   a[2] = a2;
 }
 
-#ifdef LANCET_LANS_TIMING
-#define EVT(slot, e) do { if (threadIdx.x == 0 && (slot).real() && (slot).tensor == 100) reinterpret_cast<long long*>(t.partial)[blockIdx.x * 8 + (e)] = wall_clock64(); } while (0)
-#define EVT1(slot, e) do { if (threadIdx.x == 0 && (slot).tensor == 100) reinterpret_cast<long long*>(t.partial)[512 * 8 + (e)] = wall_clock64(); } while (0)
-#else
-#define EVT(slot, e) do { } while (0)
-#define EVT1(slot, e) do { } while (0)
-#endif
-#ifdef LANCET_LANS_TIMING
-#define TSTAMP(i) do { if (threadIdx.x == 0) { const long long now_ = clock64(); ctl.acc[i] += now_ - ctl.last; ctl.seg[i] = now_ - ctl.last; ctl.last = now_; } } while (0)
-#else
-#define TSTAMP(i) do { } while (0)
-#endif
-
 // One pass of the pipeline: stage M on s1 (its g in `g`; its updates go to um_new / ug_new, its parameters to
 // sh.p[PAR]), stage N on a newly drawn slot, whose g goes into `g`, which stage M has just used up, stage U
 // on s0 (updates in um_old / ug_old, parameters in sh.p[PAR ^ 1]); then the slots move up.  Consecutive
 // passes alternate between the two g arrays and between the two parities.
 //
+// Norms.  Every workgroup publishes the sums of its chunks (one word for stage N, three for stage M) and
+// every workgroup forms the norms it needs itself, from the published sums of all the tensor's chunks, in
+// the fixed order of wave_norm: they all get the same bits, nobody waits for a workgroup in charge, and the
+// workgroup that is behind the others has no more to do than they.  A tensor has at most
+// kMaxResidentChunks chunks: kGatherPerThread words per thread and norm.
+//
 // Memory operations of a wave complete in order, and under load a round trip takes microseconds: a value
 // that comes from memory is free when it is asked for before a stage's loads and looked at after them, and
-// costs a drain of the wave's stores when it is looked at behind them.  So thread 0 draws the ticket and
-// reads the norm words ahead, at the two places of a pass where its wave has nothing in flight (the start of
-// the pass, and before the loads of stage N), and looks at what the arrival counters returned one stage
-// later.  A workgroup that arrived last owes the tensor its norms and always pays before it waits itself
-// (it may hold two chunks of the tensor).  Returns false when the workgroup holds nothing any more.
+// costs a drain of the wave's stores when it is looked at behind them.  So the ticket is drawn at the start
+// of the pass and looked at behind the first loads of stage M, and the sums of other workgroups are read in
+// front of the loads of stage N and looked at behind them: those of s0's tensor, whose stage M was a pass
+// ago, for the stage U that follows, and those of s2's, whose stage N was a pass ago, for stage M of the
+// next pass (the norm is carried there in LDS; a register carried over would be looked at behind stage U's
+// stores).  Only a sum that is still missing then is polled for.  Returns false when the workgroup holds
+// nothing any more.
 template <int PAR>
 __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansScalars& sc, float bc1, float bc2,
-                                              Slot& s0, Slot& s1, Slot& s2, Control& ctl,
+                                              Slot& s0, Slot& s1, Slot& s2, uint32_t& ticket,
                                               f32x4 (&g)[kVecPerThread],
                                               f32x4 (&um_new)[kVecPerThread], f32x4 (&ug_new)[kVecPerThread],
                                               const f32x4 (&um_old)[kVecPerThread], const f32x4 (&ug_old)[kVecPerThread],
-                                              PipeShared& sh, bool align = false) {
+                                              PipeShared& sh, bool align) {
   const bool own_norms = t.grad_norms == nullptr;
   // ---- start of the pass ---------------------------------------------------------------------------------
   lds_barrier();
+  float g_norm = 0.f;
   bool bad = false;
   if (s1.real()) {
     if (own_norms) {
-      bad = acquire_norms<1>(t, sc, 0, s1, ctl.g_word, sh);
+      g_norm = sh.g_next;  // formed at the end of the pass before
+      bad = __builtin_amdgcn_readfirstlane(sh.g_next_bad) != 0;
     } else {
-      if (threadIdx.x == 0) sh.norm[0] = t.norms[s1.tensor];  // copied from the caller's array before this kernel
-      lds_barrier();
+      g_norm = t.norms[s1.tensor];  // copied from the caller's array before this kernel
     }
   }
   if (threadIdx.x == 0) {
@@ -840,23 +690,18 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
       const uint32_t everyone = min(static_cast<uint32_t>(gridDim.x), static_cast<uint32_t>(t.nres));
       for (int spins = 0; spins < 256 && ld_agent(t.ctl + kCtlTicket) < everyone; ++spins) __builtin_amdgcn_s_sleep(8);
     }
-    // The ticket of this pass's stage N.  Drawn behind the wait for ||g|| of s1's tensor: every chunk of that
-    // tensor has been drawn by now, so the new slot cannot be a third chunk of it in this workgroup's hands.
-    ctl.ticket = atomicAdd(t.ctl + kCtlTicket, 1u);
+    ticket = atomicAdd(t.ctl + kCtlTicket, 1u);  // for this pass's stage N
   }
-  EVT(s1, 1);
-  TSTAMP(0);
   // ---- stage M on s1 ---------------------------------------------------------------------------------------
   if (s1.real()) {
     float a[3] = {0.f, 0.f, 0.f};
     if (!bad) {
-      const LansElem el = make_elem(sc, sh.norm[0], bc1, bc2);
-      if (s1.full) moments_chunk<true, PAR>(t, s1, el, g, um_new, ug_new, sh, a);
-      else moments_chunk<false, PAR>(t, s1, el, g, um_new, ug_new, sh, a);
+      const LansElem el = make_elem(sc, g_norm, bc1, bc2);
+      moments_chunk<PAR>(t, s1, el, g, um_new, ug_new, sh, a, ticket);
     } else {
+      if (threadIdx.x == 0) sh.chunk = static_cast<int>(ticket);
       s1.dead = 1;  // ||g|| is unknown: the chunk is left as it is, and so will its tensor's parameters be
     }
-    TSTAMP(1);
 #pragma unroll
     for (int k = 0; k < 3; ++k) a[k] = wave_sum(a[k]);
     if (lane_id() == 0) {
@@ -872,83 +717,113 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
         for (int w = 0; w < kLansThreads / kWave; ++w) r += sh.red[k][w];
         a[k] = r;
       }
-      publish<3>(t, sc, 1, s1, a, bad, t.ctl + kCtlArrive + t.T + s1.tensor);
+      publish<3>(t, sc, 1, s1, a, bad);
     }
-    EVT(s1, 2);
+  } else if (threadIdx.x == 0) {
+    sh.chunk = static_cast<int>(ticket);
   }
-  TSTAMP(2);
-  EVT(s0, 7);
-  EVT(s2, 6);
   // ---- stage N on a new slot -------------------------------------------------------------------------------
-  Slot s3;
-  if (threadIdx.x == 0) {
-    // read ahead, in front of the loads of g: the norms stage U needs (s0's tensor) and ||g|| for the next
-    // pass's stage M (s2's tensor)
-    if (s0.real()) {
+  // in front of the loads of g: the sums other workgroups have published
+  uint64_t words_g[kGatherPerThread], words_u[3][kGatherPerThread];
+  const bool need_u = s0.real();
+  const bool need_g = s2.real() && own_norms;
+#ifndef LANCET_LANS_PROBE
+  if (need_u) {
 #pragma unroll
-      for (int k = 0; k < 3; ++k) ctl.u_word[k] = ld_word(t.norm_word + static_cast<size_t>(1 + k) * t.T + s0.tensor);
-    }
-    if (s2.real() && own_norms) ctl.g_word[0] = ld_word(t.norm_word + s2.tensor);
-    sh.chunk = static_cast<int>(ctl.ticket);
+    for (int k = 0; k < 3; ++k) gather_issue(t, 1 + k, s0, words_u[k]);
+  }
+  if (need_g) gather_issue(t, 0, s2, words_g);
+#endif
+  if (threadIdx.x == 0) {
+    sh.u_bad = 0;
+    sh.g_next_bad = 0;
+    sh.retry = 0;
   }
   lds_barrier();
+  Slot s3;
   {
     // one value for the whole workgroup, and known to be: pointers and sizes derived from it stay scalar
     const int chunk = __builtin_amdgcn_readfirstlane(sh.chunk);
     s3.chunk = (chunk >= 0 && chunk < t.nres) ? chunk : -1;
     s3.tensor = -1;
     s3.dead = 0;
-    s3.owes = 0;
     if (s3.chunk >= 0) {
       const ChunkView c = chunk_view(t, s3.chunk);
       s3.tensor = c.tensor;
       if (c.tensor >= 0) {
-        s3.n = c.n;
         s3.begin = c.begin;
         s3.lo = t.tensor_first[c.tensor];
         s3.nc = t.tensor_chunks[c.tensor];
-        const int at = s3.chunk - s3.lo;
-        s3.owes = (own_norms && at == 0 ? 1 : 0) | (at == 0 ? 2 : 0) | (at == 1 % s3.nc ? 4 : 0) | (at == 2 % s3.nc ? 8 : 0);
-        s3.full = c.n == kLansChunk && vec_ok(t.g[c.tensor], t.p[c.tensor], t.m[c.tensor], t.v[c.tensor]);
       }
     }
   }
-  TSTAMP(3);
   if (s3.real()) {
     // g of the chunk into registers, its sum of squares published (L2NormFunctor, multi_tensor_lans.cu:95-167)
-    float a = s3.full ? load_g<true>(t, s3, g) : load_g<false>(t, s3, g);
+    float a = load_g(t, s3, g);
     if (own_norms) {
       a = block_sum_lds(a, sh.red[0]);
       if (threadIdx.x == 0) {
         const float sums[1] = {a};
-        publish<1>(t, sc, 0, s3, sums, false, t.ctl + kCtlArrive + s3.tensor);
+        publish<1>(t, sc, 0, s3, sums, false);
       }
     }
-    EVT(s3, 0);
   }
-  TSTAMP(4);
-#ifdef LANCET_LANS_TIMING
-  if (threadIdx.x == 0 && s3.real()) ctl.acc[7] += 1;
+  // ---- the norms ---------------------------------------------------------------------------------------------
+#ifdef LANCET_LANS_PROBE
+  if (threadIdx.x == 0) sh.norm[1] = sh.norm[2] = sh.norm[3] = sh.g_next = 1.f;
+  lds_barrier();
+#else
+  {
+    bool retry = false;
+    if (need_u) {
+#pragma unroll
+      for (int k = 0; k < 3; ++k) gather_take(sc, s0, words_u[k], sh.part[1 + k], retry);
+    }
+    if (need_g) gather_take(sc, s2, words_g, sh.part[0], retry);
+    if (retry) sh.retry = 1;
+  }
+  lds_barrier();
+  if (__builtin_amdgcn_readfirstlane(sh.retry) != 0) {
+    // something was not there yet (or is poisoned): everything again, with patience
+    if (need_u) {
+      bool missing = false;
+#pragma unroll 1
+      for (int k = 1; k < 4; ++k) missing = gather_again(t, sc, k, s0, sh.part[k]) || missing;
+      if (missing) sh.u_bad = 1;
+    }
+    if (need_g && gather_again(t, sc, 0, s2, sh.part[0])) sh.g_next_bad = 1;
+    lds_barrier();
+  }
+  {
+    const int w = threadIdx.x / kWave;  // wave w sums norm w: the same fixed order in every workgroup
+    if (w == 0) {
+      if (need_g) {
+        const float n = wave_norm(0, s2.nc, [&](int c) { return sh.part[0][c]; });
+        if (lane_id() == 0) {
+          sh.g_next = n;
+          if (s2.chunk == s2.lo) t.norms[s2.tensor] = n;  // for lancet_lans_plan_norms
+        }
+      }
+    } else if (need_u) {
+      const float n = wave_norm(0, s0.nc, [&](int c) { return sh.part[w][c]; });
+      if (lane_id() == 0) {
+        sh.norm[w] = n;
+        if (s0.chunk == s0.lo) t.norms[w * t.T + s0.tensor] = n;
+      }
+    }
+  }
+  lds_barrier();
 #endif
   // ---- stage U on s0 ---------------------------------------------------------------------------------------
   // Trust ratios and the parameter update (LANSStage2Functor, multi_tensor_lans.cu:326-399) from the updates
   // in registers and the parameters in LDS.  Nothing is written unless all three norms are known.
-  bool bad_u = true;
-  // first what this workgroup owes others: ||g|| of s3's tensor, which has just been through stage N, and
-  // the three norms of s1's, through stage M earlier in this pass
-  if (s3.real()) pay_norms(t, sc, s3, 1, kPayPolls, sh);
-  if (s1.real()) pay_norms(t, sc, s1, 14, kPayPolls, sh);
-  if (s0.real()) bad_u = acquire_norms<3>(t, sc, 1, s0, ctl.u_word, sh) || s0.dead != 0;
-  EVT(s0, 3);
-  TSTAMP(5);
-  if (s0.real() && !bad_u) {
+  if (need_u && !s0.dead && __builtin_amdgcn_readfirstlane(sh.u_bad) == 0) {
     const float pn = uniform(sh.norm[1]), umn = uniform(sh.norm[2]), ugn = uniform(sh.norm[3]);
     float ratio_m = (umn != 0.f && pn != 0.f) ? sc.lr * (pn / umn) : sc.lr;
     float ratio_g = (ugn != 0.f && pn != 0.f) ? sc.lr * (pn / ugn) : sc.lr;
     ratio_m = uniform(ratio_m * sc.beta1);
     ratio_g = uniform(ratio_g * sc.beta3);
-    const ChunkArray<true> p_full(t.p[s0.tensor] + s0.begin, s0.n);
-    const ChunkArray<false> p_part(t.p[s0.tensor] + s0.begin, s0.n);
+    LANCET_GLOBAL float* p = as_global(t.p[s0.tensor] + s0.begin);
 #pragma unroll
     for (int k = 0; k < kVecPerThread; ++k) {
       f32x4 xp = sh.p[PAR ^ 1][k][threadIdx.x];
@@ -957,24 +832,9 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
 #pragma clang fp contract(off)
         xp[j] = xp[j] - (ratio_m * um_old[k][j]) - (ratio_g * ug_old[k][j]);
       }
-      if (s0.full) p_full.store(chunk_elem(k), xp);
-      else p_part.store(chunk_elem(k), xp);
+      st_chunk4(p, chunk_elem(k), xp);
     }
   }
-  TSTAMP(6);
-#ifdef LANCET_LANS_TIMING
-  if (threadIdx.x == 0) {
-    const long long now = wall_clock64();
-    if (ctl.pass_begin && s1.real()) {
-      long long d = (now - ctl.pass_begin) / 200;
-      atomicAdd(&g_hist[d > 63 ? 63 : (int)d], 1u);
-      const int slow = d >= 16;
-      for (int i = 0; i < 7; ++i) atomicAdd(&g_seg[slow][i], (unsigned long long)ctl.seg[i]);
-      atomicAdd(&g_seg[slow][7], 1ull);
-    }
-    ctl.pass_begin = now;
-  }
-#endif
   // ---- the slots move up ------------------------------------------------------------------------------------
   s0 = s1;
   s1 = s2;
@@ -982,51 +842,26 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
   return s0.chunk >= 0 || s1.chunk >= 0 || s2.chunk >= 0;
 }
 
-// Two workgroups per CU (two waves per SIMD, 256 registers per lane): a workgroup holds g of two chunks,
-// u_m and u_g of two more (one of them being filled from the first g) and 64 KB of parameters in LDS.
-constexpr int kResidentWavesPerSimd = 2;
-
-// Start of a resident step: clears the ticket and the arrival counters and moves the step epoch on.  The
-// epoch lives on the device so that a step recorded in a graph tags every replay differently; when it
-// wraps (2^31 steps) every word of earlier steps is forgotten.  The error word is left alone.
-__global__ __launch_bounds__(kLansThreads) void lans_begin_kernel(LansTables t, size_t nwords) {
-#ifdef LANCET_LANS_TIMING
-  if (blockIdx.x == 0 && threadIdx.x == 0) {
-    const long long* d = reinterpret_cast<const long long*>(t.partial);
-    const char* names[8] = {"N published", "G resolved (M starts)", "M published", "U norms resolved", "", "", "G word read ahead", "U words read ahead"};
-    long long base = d[0];
-    for (int w = 0; w < 512; ++w) if (d[w * 8] && d[w * 8] < base) base = d[w * 8];
-    for (int e = 0; e < 8; ++e) {
-      if (e == 4 || e == 5) continue;
-      long long lo = 1ll << 62, hi = 0, sum = 0; int n = 0;
-      for (int w = 0; w < 512; ++w) { const long long x = d[w * 8 + e]; if (!x) continue; lo = x < lo ? x : lo; hi = x > hi ? x : hi; sum += x; ++n; }
-      if (n) printf("tensor 100 event %d n %d min %d avg %d max %d (x10ns)\n", e, n, (int)(lo - base), (int)(sum / n - base), (int)(hi - base));
-    }
-    for (int b = 0; b < 64; b += 8)
-      printf("pass duration histogram, 2 us bins from %d us: %u %u %u %u %u %u %u %u\n", 2 * b, g_hist[b], g_hist[b + 1], g_hist[b + 2], g_hist[b + 3], g_hist[b + 4], g_hist[b + 5], g_hist[b + 6], g_hist[b + 7]);
-    for (int b = 0; b < 64; ++b) g_hist[b] = 0;
-    for (int k = 0; k < 2; ++k) {
-      const unsigned long long n = g_seg[k][7] ? g_seg[k][7] : 1;
-      printf("%s passes %llu: avg cycles start %llu M %llu sumpub %llu draw %llu N %llu pay+preU %llu U %llu\n", k ? "slow (>=32us)" : "fast", g_seg[k][7],
-             g_seg[k][0] / n, g_seg[k][1] / n, g_seg[k][2] / n, g_seg[k][3] / n, g_seg[k][4] / n, g_seg[k][5] / n, g_seg[k][6] / n);
-      for (int i = 0; i < 8; ++i) g_seg[k][i] = 0;
-    }
-    long long wlo = 1ll << 62, whi = 0, wsum = 0; int ilo = 0, ihi = 0;
-    for (int w = 0; w < 512; ++w) { if (g_wait[w] < wlo) { wlo = g_wait[w]; ilo = w; } if (g_wait[w] > whi) { whi = g_wait[w]; ihi = w; } wsum += g_wait[w]; }
-    printf("cycles in acquire per wg (cumulative): min %lld (wg %d) avg %lld max %lld (wg %d)\n", wlo, ilo, wsum / 512, whi, ihi);
-    printf("wg %d: hits %u polled-then-words %u polled-then-summed %u;  wg %d: %u %u %u\n", ilo, g_modes[ilo][0], g_modes[ilo][1], g_modes[ilo][2], ihi, g_modes[ihi][0], g_modes[ihi][1], g_modes[ihi][2]);
-  }
+#ifndef LANCET_LANS_WAVES
+#define LANCET_LANS_WAVES 2
 #endif
-  const size_t i = blockIdx.x * static_cast<size_t>(kLansThreads) + threadIdx.x;
-  if (i < 2 * static_cast<size_t>(t.T)) t.ctl[kCtlArrive + i] = 0u;
-  if (i == 0) t.ctl[kCtlTicket] = 0u;
-  if (blockIdx.x == 0) {
-    uint32_t* ep = t.ctl + kCtlEpoch;
-    const uint32_t e = (*ep + 1u) & ~kPoison;
-    if (e == 0u)
-      for (size_t k = threadIdx.x; k < nwords; k += kLansThreads) t.part_word[k] = 0;  // norm words follow
-    __syncthreads();
-    if (threadIdx.x == 0) *ep = e == 0u ? 1u : e;
+// Workgroups per CU = waves per SIMD: with two, a wave has 256 registers for g of two chunks, u_m and u_g of
+// two more (one of them being filled from the first g) and the sums read ahead, and a workgroup 64 KB of
+// LDS for parameters.
+constexpr int kResidentWavesPerSimd = LANCET_LANS_WAVES;
+
+// Start of a resident step: clears the ticket and moves the step epoch on.  The epoch lives on the device so
+// that a step recorded in a graph tags every replay differently; when it wraps (2^31 steps) every word of
+// earlier steps is forgotten.  The error word is left alone.
+__global__ __launch_bounds__(kLansThreads) void lans_begin_kernel(LansTables t, size_t nwords) {
+  uint32_t* ep = t.ctl + kCtlEpoch;
+  const uint32_t e = (*ep + 1u) & ~kPoison;
+  if (e == 0u)
+    for (size_t k = threadIdx.x; k < nwords; k += kLansThreads) t.part_word[k] = 0;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    *ep = e == 0u ? 1u : e;
+    t.ctl[kCtlTicket] = 0u;
   }
 }
 
@@ -1045,34 +880,17 @@ __global__ __launch_bounds__(kLansThreads, kResidentWavesPerSimd) void lans_resi
   s0.chunk = s1.chunk = s2.chunk = -1;
   s0.tensor = s1.tensor = s2.tensor = -1;
   s0.dead = s1.dead = s2.dead = 0;
-  s0.owes = s1.owes = s2.owes = 0;
-  Control ctl;
-  ctl.ticket = 0u;
-  ctl.g_word[0] = 0;
-  ctl.u_word[0] = ctl.u_word[1] = ctl.u_word[2] = 0;
-#ifdef LANCET_LANS_TIMING
-  for (int i = 0; i < 8; ++i) ctl.acc[i] = 0;
-  ctl.pass_begin = 0;
-  ctl.last = clock64();
-  const long long t_begin = ctl.last;
-#endif
+  if (threadIdx.x == 0) {
+    sh.g_next = 0.f;
+    sh.g_next_bad = 0;
+  }
+  uint32_t ticket = 0u;  // thread 0
   // the first two passes find empty slots (their stages M and U have nothing to do) and fill the pipeline;
   // every pass draws a ticket, tickets run out, and every wait is bounded: all workgroups leave
-  bool more = pipeline_pass<0>(t, sc, bc1, bc2, s0, s1, s2, ctl, ga, um0, ug0, um1, ug1, sh) &&
-              pipeline_pass<1>(t, sc, bc1, bc2, s0, s1, s2, ctl, gb, um1, ug1, um0, ug0, sh, LANCET_LANS_ALIGN != 0);
-  while (more) {
-    if (!pipeline_pass<0>(t, sc, bc1, bc2, s0, s1, s2, ctl, ga, um0, ug0, um1, ug1, sh)) break;
-    if (!pipeline_pass<1>(t, sc, bc1, bc2, s0, s1, s2, ctl, gb, um1, ug1, um0, ug0, sh)) break;
+  for (int pair = 0;; ++pair) {
+    if (!pipeline_pass<0>(t, sc, bc1, bc2, s0, s1, s2, ticket, ga, um0, ug0, um1, ug1, sh, false)) break;
+    if (!pipeline_pass<1>(t, sc, bc1, bc2, s0, s1, s2, ticket, gb, um1, ug1, um0, ug0, sh, pair == 0 && LANCET_LANS_ALIGN != 0)) break;
   }
-#ifdef LANCET_LANS_TIMING
-  if (threadIdx.x == 0 && (blockIdx.x % 128) == 5)
-    printf("misses(all wgs so far) %llu spins(all wgs so far) %u\n", g_misses, t.ctl[3]);
-  if (threadIdx.x == 0) atomicMax(&g_most, (unsigned)ctl.acc[7]), atomicMin(&g_fewest, (unsigned)ctl.acc[7]);
-  if (threadIdx.x == 0 && (blockIdx.x % 128) == 5) printf("chunks of this wg %lld; fewest/most over wgs that have finished: %u %u\n", ctl.acc[7], g_fewest, g_most);
-  if (threadIdx.x == 0 && (blockIdx.x % 128) == 5)
-    printf("wg %3d total %lld: start %lld M %lld sumpub %lld draw %lld N %lld preU %lld U %lld\n", blockIdx.x,
-           clock64() - t_begin, ctl.acc[0], ctl.acc[1], ctl.acc[2], ctl.acc[3], ctl.acc[4], ctl.acc[5], ctl.acc[6]);
-#endif
 }
 
 }  // namespace lancet
@@ -1112,11 +930,11 @@ static constexpr uint32_t kDefaultSpinLimit = 1u << 20;  // about a second of po
 static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 static inline int chunks_of(int64_t numel) { return static_cast<int>((numel + kLansChunk - 1) / kLansChunk); }
 
-// The plan's own tensor order and chunk slots.  Tensors of at most `limit` chunks come first, largest first
+// The plan's own tensor order and chunk slots.  Tensors of at most `limit` whole chunks come first, largest first
 // (list order among equals), packed into rounds of `round` slots: a tensor that does not fit into what is
 // left of a round starts the next one and the rest of the round is padding (chunk_tensor -1), so that all
-// chunks of a tensor are drawn in the same pass of the resident kernel's workgroups.  Larger tensors follow
-// in list order, without padding: they go through the sweeps.  first[i] / ctensor are in plan order.
+// chunks of a tensor are drawn in the same pass of the resident kernel's workgroups.  The other tensors (larger,
+// or not a multiple of the chunk) follow in list order, without padding: they go through the sweeps.  first[i] / ctensor are in plan order.
 struct ChunkLayout {
   std::vector<int32_t> order, ctensor, first, count;
   int n_fit = 0;       // tensors the resident kernel takes
@@ -1126,7 +944,9 @@ struct ChunkLayout {
 static ChunkLayout chunk_layout(const int64_t* numels, int T, int limit, int round) {
   ChunkLayout L;
   std::vector<int32_t> fit, big;
-  for (int i = 0; i < T; ++i) (chunks_of(numels[i]) <= limit ? fit : big).push_back(i);
+  // the resident kernel takes whole chunks only
+  for (int i = 0; i < T; ++i)
+    ((chunks_of(numels[i]) <= limit && numels[i] % kLansChunk == 0) ? fit : big).push_back(i);
   std::stable_sort(fit.begin(), fit.end(), [&](int a, int b) { return chunks_of(numels[a]) > chunks_of(numels[b]); });
   L.n_fit = static_cast<int>(fit.size());
   L.order = fit;
@@ -1201,6 +1021,7 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
     pl->resident_grid = per_cu * cus;
   }
   // a tensor's chunks fit one round, so the kernel drains with half of its workgroups on the chip
+  // a tensor's chunks fit one round: they are all drawn in one pass
   pl->resident_limit = std::min(pl->resident_grid, kMaxResidentChunks);
   const ChunkLayout L = chunk_layout(numels, T, pl->resident_limit, pl->resident_grid);
   pl->order = L.order;
@@ -1220,7 +1041,7 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
   const size_t o_norms = off;     off = align_up(off + 4 * T * sizeof(float), 256);
   const size_t o_consts = off;    off = align_up(off + 2 * sizeof(float), 256);
   const size_t o_words = off;     off = align_up(off + 4 * (n1 + T) * sizeof(uint64_t), 256);
-  const size_t n_ctl = kCtlArrive + 2 * static_cast<size_t>(T);
+  const size_t n_ctl = kCtlWords;
   const size_t o_ctl = off;       off = align_up(off + n_ctl * sizeof(uint32_t), 256);
   const size_t o_order = off;     off = align_up(off + T * sizeof(int32_t), 256);
   pl->words_bytes = 4 * (n1 + T) * sizeof(uint64_t);
@@ -1312,11 +1133,13 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
   const int T = pl->T;
   hipStream_t st = static_cast<hipStream_t>(stream);
   bool changed = false;
+  bool aligned16 = true;  // the resident kernel moves float4s: a step with a tensor that is not 16-byte aligned runs as sweeps
   for (int i = 0; i < T; ++i) {
     if (pl->numels[i] > 0 && (!g[i] || !p[i] || !m[i] || !v[i])) return LANCET_ERR_NULL;
-    if ((reinterpret_cast<uintptr_t>(g[i]) | reinterpret_cast<uintptr_t>(p[i]) |
-         reinterpret_cast<uintptr_t>(m[i]) | reinterpret_cast<uintptr_t>(v[i])) & 3u)
-      return LANCET_ERR_ALIGN;
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(g[i]) | reinterpret_cast<uintptr_t>(p[i]) |
+                           reinterpret_cast<uintptr_t>(m[i]) | reinterpret_cast<uintptr_t>(v[i]);
+    if (bits & 3u) return LANCET_ERR_ALIGN;
+    aligned16 = aligned16 && (bits & 15u) == 0;
     changed = changed || pl->shadow[i] != g[i] || pl->shadow[T + i] != p[i] ||
               pl->shadow[2 * T + i] != m[i] || pl->shadow[3 * T + i] != v[i];
   }
@@ -1365,9 +1188,8 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
   // slots [0, chunk_base) and tensors [0, tensor_base) go through the resident kernel, the rest
   // (everything, under the sweeps schedule) through the three sweeps
   int chunk_base = 0, tensor_base = 0;
-  if (pl->schedule == LANCET_LANS_RESIDENT && pl->n_res_chunks > 0) {
-    const unsigned begin_blocks = static_cast<unsigned>((2 * static_cast<size_t>(T) + kLansThreads - 1) / kLansThreads);
-    lans_begin_kernel<<<begin_blocks, kLansThreads, 0, st>>>(t, pl->words_bytes / sizeof(uint64_t));
+  if (pl->schedule == LANCET_LANS_RESIDENT && pl->n_res_chunks > 0 && aligned16) {
+    lans_begin_kernel<<<1, kLansThreads, 0, st>>>(t, pl->words_bytes / sizeof(uint64_t));
     const int grid = std::min(pl->resident_grid, pl->n_res_chunks);
     lans_resident_kernel<<<grid, kLansThreads, 0, st>>>(t, sc);
     chunk_base = pl->n_res_chunks;

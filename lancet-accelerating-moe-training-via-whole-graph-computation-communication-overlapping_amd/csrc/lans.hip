@@ -467,6 +467,18 @@ constexpr int kVecPerThread = kLansChunk / 4 / kLansThreads;  // float4 per thre
 #ifndef LANCET_LANS_ALIGN
 #define LANCET_LANS_ALIGN 1
 #endif
+#ifndef LANCET_LANS_SB
+#define LANCET_LANS_SB 0
+#endif
+#ifndef LANCET_LANS_PREFETCH
+#define LANCET_LANS_PREFETCH 1
+#endif
+constexpr int kPrefetch = LANCET_LANS_PREFETCH;
+__device__ __forceinline__ void stage_fence() {
+#if LANCET_LANS_SB & 4
+  __builtin_amdgcn_sched_barrier(0);
+#endif
+}
 
 // Workgroup barrier that orders LDS accesses only.  __syncthreads() also waits for every global load and
 // store the wave has in flight, which would drain the streams of this kernel several times per chunk; all
@@ -599,21 +611,30 @@ __device__ __forceinline__ void moments_chunk(const LansTables& t, const Slot& s
   LANCET_GLOBAL float* m = as_global(t.m[s.tensor] + s.begin);
   LANCET_GLOBAL float* v = as_global(t.v[s.tensor] + s.begin);
   float a0 = 0.f, a1 = 0.f, a2 = 0.f;
-  f32x4 np = ld_chunk4(p, chunk_elem(0));
-  f32x4 nm = ld_chunk4(m, chunk_elem(0)), nv = ld_chunk4(v, chunk_elem(0));
-  // the ticket drawn at the start of the pass is looked at here, behind three loads and in front of every
+  // kPrefetch float4 of each array are in flight ahead of the one being worked on
+  f32x4 np[kPrefetch], nm[kPrefetch], nv[kPrefetch];
+#pragma unroll
+  for (int d = 0; d < kPrefetch; ++d) {
+    np[d] = ld_chunk4(p, chunk_elem(d));
+    nm[d] = ld_chunk4(m, chunk_elem(d));
+    nv[d] = ld_chunk4(v, chunk_elem(d));
+  }
+  // the ticket drawn at the start of the pass is looked at here, behind the first loads and in front of every
   // store of the stage: looked at behind the stores it would cost their completion
   if (threadIdx.x == 0) sh.chunk = static_cast<int>(ticket);
 #pragma unroll
   for (int k = 0; k < kVecPerThread; ++k) {
     const int e = chunk_elem(k);
-    const f32x4 xp = np;
-    f32x4 xm = nm, xv = nv;
-    if (k + 1 < kVecPerThread) {
-      np = ld_chunk4(p, chunk_elem(k + 1));
-      nm = ld_chunk4(m, chunk_elem(k + 1));
-      nv = ld_chunk4(v, chunk_elem(k + 1));
+    const f32x4 xp = np[k % kPrefetch];
+    f32x4 xm = nm[k % kPrefetch], xv = nv[k % kPrefetch];
+    if (k + kPrefetch < kVecPerThread) {
+      np[k % kPrefetch] = ld_chunk4(p, chunk_elem(k + kPrefetch));
+      nm[k % kPrefetch] = ld_chunk4(m, chunk_elem(k + kPrefetch));
+      nv[k % kPrefetch] = ld_chunk4(v, chunk_elem(k + kPrefetch));
     }
+#if LANCET_LANS_SB & 1
+    __builtin_amdgcn_sched_barrier(0);
+#endif
     sh.p[PAR][k][threadIdx.x] = xp;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -634,10 +655,20 @@ __device__ __forceinline__ void moments_chunk(const LansTables& t, const Slot& s
     }
     st_chunk4(m, e, xm);
     st_chunk4(v, e, xv);
+#if LANCET_LANS_SB & 2
+    __builtin_amdgcn_sched_barrier(0);
+#endif
   }
   a[0] = a0;
   a[1] = a1;
   a[2] = a2;
+}
+
+// Gives register arrays a value on the paths that do not fill them.  Without it the value they held before
+// would count as still needed there, and with it the registers, all through the stage in front.
+__device__ __forceinline__ void forget(f32x4 (&a)[kVecPerThread], f32x4 (&b)[kVecPerThread]) {
+#pragma unroll
+  for (int k = 0; k < kVecPerThread; ++k) a[k] = b[k] = f32x4{0.f, 0.f, 0.f, 0.f};
 }
 
 // One pass of the pipeline: stage M on s1 (its g in `g`; its updates go to um_new / ug_new, its parameters to
@@ -701,6 +732,7 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
     } else {
       if (threadIdx.x == 0) sh.chunk = static_cast<int>(ticket);
       s1.dead = 1;  // ||g|| is unknown: the chunk is left as it is, and so will its tensor's parameters be
+      forget(um_new, ug_new);
     }
 #pragma unroll
     for (int k = 0; k < 3; ++k) a[k] = wave_sum(a[k]);
@@ -719,9 +751,11 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
       }
       publish<3>(t, sc, 1, s1, a, bad);
     }
-  } else if (threadIdx.x == 0) {
-    sh.chunk = static_cast<int>(ticket);
+  } else {
+    if (threadIdx.x == 0) sh.chunk = static_cast<int>(ticket);
+    forget(um_new, ug_new);
   }
+  stage_fence();
   // ---- stage N on a new slot -------------------------------------------------------------------------------
   // in front of the loads of g: the sums other workgroups have published
   uint64_t words_g[kGatherPerThread], words_u[3][kGatherPerThread];
@@ -768,6 +802,7 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
       }
     }
   }
+  stage_fence();
   // ---- the norms ---------------------------------------------------------------------------------------------
 #ifdef LANCET_LANS_PROBE
   if (threadIdx.x == 0) sh.norm[1] = sh.norm[2] = sh.norm[3] = sh.g_next = 1.f;
@@ -814,6 +849,7 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
   }
   lds_barrier();
 #endif
+  stage_fence();
   // ---- stage U on s0 ---------------------------------------------------------------------------------------
   // Trust ratios and the parameter update (LANSStage2Functor, multi_tensor_lans.cu:326-399) from the updates
   // in registers and the parameters in LDS.  Nothing is written unless all three norms are known.
@@ -835,6 +871,7 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
       st_chunk4(p, chunk_elem(k), xp);
     }
   }
+  stage_fence();
   // ---- the slots move up ------------------------------------------------------------------------------------
   s0 = s1;
   s1 = s2;

@@ -444,22 +444,6 @@ __device__ __forceinline__ bool word_is_current(uint64_t x, uint32_t epoch) {
 }
 __device__ __forceinline__ bool word_is_poisoned(uint64_t x) { return (static_cast<uint32_t>(x >> 32) & kPoison) != 0; }
 
-// Polls for a word of this step.  Bounded; and once any wait of the plan has given up the others stop early,
-// so that a stalled step ends after about one bound, not one per chunk.  Returns 0 (no tag) when it gives up.
-__device__ __forceinline__ uint64_t wait_word(const LansTables& t, const LansScalars& sc, const uint64_t* src) {
-  uint64_t x = ld_word(src);
-  uint32_t spins = 0;
-  while (!word_is_current(x, sc.epoch)) {
-    if (++spins > sc.spin_limit || ((spins & 63u) == 0u && ld_agent(t.ctl + kCtlError) != 0u)) {
-      flag_error(t);
-      return 0;
-    }
-    __builtin_amdgcn_s_sleep(2);
-    x = ld_word(src);
-  }
-  return x;
-}
-
 // =======================================================================================
 // schedule "resident": one persistent kernel, a three-stage software pipeline per workgroup
 // =======================================================================================
@@ -474,6 +458,8 @@ constexpr int kVecPerThread = kLansChunk / 4 / kLansThreads;  // float4 per thre
 #define LANCET_LANS_PREFETCH 1
 #endif
 constexpr int kPrefetch = LANCET_LANS_PREFETCH;
+#define LIKELY(x) __builtin_expect(!!(x), 1)
+#define UNLIKELY(x) __builtin_expect(!!(x), 0)
 __device__ __forceinline__ void stage_fence() {
 #if LANCET_LANS_SB & 4
   __builtin_amdgcn_sched_barrier(0);
@@ -509,7 +495,8 @@ struct PipeShared {
   float g_next;    // ||g|| of s2's tensor: for stage M of the next pass
   int g_next_bad;  // ... is unknown
   int u_bad;       // a norm of s0's tensor is unknown
-  int retry;       // a sum read ahead was not there yet
+  int retry_u, retry_g;  // a sum read ahead was not there yet
+  int give_up;           // ... and never came (sticky for the rest of the kernel)
   int chunk;
 };
 
@@ -526,17 +513,27 @@ struct Slot {
 // The resident kernel only takes whole chunks of 16-byte aligned arrays (the plan leaves tensors that are not a
 // multiple of the chunk to the sweeps; a step whose pointers are not aligned runs as sweeps altogether): every
 // access is an unconditional, non-temporal float4.
-__device__ __forceinline__ f32x4 ld_chunk4(const LANCET_GLOBAL float* a, int e) {
-  return __builtin_nontemporal_load((const LANCET_GLOBAL f32x4*)(a + e));
-}
-__device__ __forceinline__ void st_chunk4(LANCET_GLOBAL float* a, int e, f32x4 x) {
-  __builtin_nontemporal_store(x, (LANCET_GLOBAL f32x4*)(a + e));
+// A table entry (tensor pointers, chunk tables) read as constant memory: nothing writes the tables while a
+// kernel runs, and said this way the read goes through the scalar unit and its result stays in scalar
+// registers.  A plain read behind the kernel's own stores has to assume they changed the table, takes the
+// vector unit, and every pointer it yields costs two vector registers for as long as it lives.
+template <typename T>
+__device__ __forceinline__ T ld_table(const T* p) {
+  return *(const __attribute__((address_space(4))) T*)(p);
 }
 
-// a wave owns a quarter of the chunk: float4 k of lane l is element 4 * (64 k + l) of it, so one load
-// instruction of a wave covers 1 KB of consecutive memory
-__device__ __forceinline__ int chunk_elem(int k) {
-  return (threadIdx.x / kWave) * (kLansChunk / kWavesPerTile) + 4 * lane_id() + k * (4 * kWave);
+// float4 k of a thread: the wave's quarter of the chunk starts lane_offset() elements into it, float4 k lies
+// k * 256 elements further on (one load instruction of a wave covers 1 KB of consecutive memory).  The
+// address is a uniform 64-bit base plus an unsigned 32-bit offset per lane, the form that takes its base
+// from scalar registers and one vector register for the offset.
+__device__ __forceinline__ uint32_t lane_offset() {
+  return static_cast<uint32_t>((threadIdx.x / kWave) * (kLansChunk / kWavesPerTile) + 4 * lane_id());
+}
+__device__ __forceinline__ f32x4 ld_chunk4(const LANCET_GLOBAL float* a, int k) {
+  return __builtin_nontemporal_load((const LANCET_GLOBAL f32x4*)(a + k * (4 * kWave) + lane_offset()));
+}
+__device__ __forceinline__ void st_chunk4(LANCET_GLOBAL float* a, int k, f32x4 x) {
+  __builtin_nontemporal_store(x, (LANCET_GLOBAL f32x4*)(a + k * (4 * kWave) + lane_offset()));
 }
 
 // Thread 0: publishes the N chunk sums a[] of slot s as words first .. first+N-1 (fire and forget).
@@ -561,39 +558,27 @@ __device__ __forceinline__ void gather_issue(const LansTables& t, int kind, cons
     word[i] = c < s.nc ? ld_word(src + c) : 0;
   }
 }
-// ... looked at: values into LDS.  Straight-line: a word that is not there yet (or is poisoned) only raises
-// a flag; gather_again fetches those.
+// ... looked at: values into LDS; says whether a word is not of this step yet, or is poisoned
 __device__ __forceinline__ void gather_take(const LansScalars& sc, const Slot& s, const uint64_t (&word)[kGatherPerThread],
-                                            float* part, bool& retry) {
+                                            float* part, bool& missing, bool& poisoned) {
 #pragma unroll
   for (int i = 0; i < kGatherPerThread; ++i) {
     const int c = threadIdx.x + i * kLansThreads;
     if (c < s.nc) {
       part[c] = __uint_as_float(static_cast<uint32_t>(word[i]));
-      retry = retry || !word_is_current(word[i], sc.epoch) || word_is_poisoned(word[i]);
+      const bool there = word_is_current(word[i], sc.epoch);
+      missing = missing || !there;
+      poisoned = poisoned || (there && word_is_poisoned(word[i]));
     }
   }
 }
-// The same partials again, polled for one by one (rare: a workgroup that is ahead of the one that publishes);
-// true when one stays missing (its wait gave up) or is poisoned.
-__device__ __forceinline__ bool gather_again(const LansTables& t, const LansScalars& sc, int kind, const Slot& s, float* part) {
-  const uint64_t* src = t.part_word + static_cast<size_t>(kind) * t.nchunks + s.lo;
-  bool bad = false;
-#pragma unroll 1
-  for (int c = threadIdx.x; c < s.nc; c += kLansThreads) {
-    const uint64_t x = wait_word(t, sc, src + c);
-    part[c] = __uint_as_float(static_cast<uint32_t>(x));
-    bad = bad || !word_is_current(x, sc.epoch) || word_is_poisoned(x);
-  }
-  return bad;
-}
 
 __device__ __forceinline__ float load_g(const LansTables& t, const Slot& s, f32x4 (&g)[kVecPerThread]) {
-  const LANCET_GLOBAL float* src = as_global(t.g[s.tensor] + s.begin);
+  const LANCET_GLOBAL float* src = as_global(ld_table(t.g + s.tensor) + s.begin);
   float a = 0.f;
 #pragma unroll
   for (int k = 0; k < kVecPerThread; ++k) {
-    g[k] = ld_chunk4(src, chunk_elem(k));
+    g[k] = ld_chunk4(src, k);
     a += g[k].x * g[k].x + g[k].y * g[k].y + g[k].z * g[k].z + g[k].w * g[k].w;
   }
   return a;
@@ -607,30 +592,29 @@ template <int PAR>
 __device__ __forceinline__ void moments_chunk(const LansTables& t, const Slot& s, const LansElem& el,
                                               const f32x4 (&g)[kVecPerThread], f32x4 (&um)[kVecPerThread],
                                               f32x4 (&ug)[kVecPerThread], PipeShared& sh, float (&a)[3], uint32_t ticket) {
-  const LANCET_GLOBAL float* p = as_global(t.p[s.tensor] + s.begin);
-  LANCET_GLOBAL float* m = as_global(t.m[s.tensor] + s.begin);
-  LANCET_GLOBAL float* v = as_global(t.v[s.tensor] + s.begin);
+  const LANCET_GLOBAL float* p = as_global(ld_table(t.p + s.tensor) + s.begin);
+  LANCET_GLOBAL float* m = as_global(ld_table(t.m + s.tensor) + s.begin);
+  LANCET_GLOBAL float* v = as_global(ld_table(t.v + s.tensor) + s.begin);
   float a0 = 0.f, a1 = 0.f, a2 = 0.f;
   // kPrefetch float4 of each array are in flight ahead of the one being worked on
   f32x4 np[kPrefetch], nm[kPrefetch], nv[kPrefetch];
 #pragma unroll
   for (int d = 0; d < kPrefetch; ++d) {
-    np[d] = ld_chunk4(p, chunk_elem(d));
-    nm[d] = ld_chunk4(m, chunk_elem(d));
-    nv[d] = ld_chunk4(v, chunk_elem(d));
+    np[d] = ld_chunk4(p, d);
+    nm[d] = ld_chunk4(m, d);
+    nv[d] = ld_chunk4(v, d);
   }
   // the ticket drawn at the start of the pass is looked at here, behind the first loads and in front of every
   // store of the stage: looked at behind the stores it would cost their completion
   if (threadIdx.x == 0) sh.chunk = static_cast<int>(ticket);
 #pragma unroll
   for (int k = 0; k < kVecPerThread; ++k) {
-    const int e = chunk_elem(k);
     const f32x4 xp = np[k % kPrefetch];
     f32x4 xm = nm[k % kPrefetch], xv = nv[k % kPrefetch];
     if (k + kPrefetch < kVecPerThread) {
-      np[k % kPrefetch] = ld_chunk4(p, chunk_elem(k + kPrefetch));
-      nm[k % kPrefetch] = ld_chunk4(m, chunk_elem(k + kPrefetch));
-      nv[k % kPrefetch] = ld_chunk4(v, chunk_elem(k + kPrefetch));
+      np[k % kPrefetch] = ld_chunk4(p, k + kPrefetch);
+      nm[k % kPrefetch] = ld_chunk4(m, k + kPrefetch);
+      nv[k % kPrefetch] = ld_chunk4(v, k + kPrefetch);
     }
 #if LANCET_LANS_SB & 1
     __builtin_amdgcn_sched_barrier(0);
@@ -653,8 +637,8 @@ __device__ __forceinline__ void moments_chunk(const LansTables& t, const Slot& s
       a1 += u0 * u0;
       a2 += u1 * u1;
     }
-    st_chunk4(m, e, xm);
-    st_chunk4(v, e, xv);
+    st_chunk4(m, k, xm);
+    st_chunk4(v, k, xv);
 #if LANCET_LANS_SB & 2
     __builtin_amdgcn_sched_barrier(0);
 #endif
@@ -693,7 +677,7 @@ __device__ __forceinline__ void forget(f32x4 (&a)[kVecPerThread], f32x4 (&b)[kVe
 // nothing any more.
 template <int PAR>
 __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansScalars& sc, float bc1, float bc2,
-                                              Slot& s0, Slot& s1, Slot& s2, uint32_t& ticket,
+                                              Slot& s0, Slot& s1, Slot& s2,
                                               f32x4 (&g)[kVecPerThread],
                                               f32x4 (&um_new)[kVecPerThread], f32x4 (&ug_new)[kVecPerThread],
                                               const f32x4 (&um_old)[kVecPerThread], const f32x4 (&ug_old)[kVecPerThread],
@@ -703,7 +687,7 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
   lds_barrier();
   float g_norm = 0.f;
   bool bad = false;
-  if (s1.real()) {
+  if (LIKELY(s1.real())) {
     if (own_norms) {
       g_norm = sh.g_next;  // formed at the end of the pass before
       bad = __builtin_amdgcn_readfirstlane(sh.g_next_bad) != 0;
@@ -711,22 +695,23 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
       g_norm = t.norms[s1.tensor];  // copied from the caller's array before this kernel
     }
   }
+  uint32_t ticket = 0u;  // thread 0: for this pass's stage N
   if (threadIdx.x == 0) {
     // The plan lays a tensor's chunks out inside one round of as many slots as there are workgroups, so that
     // they are all drawn in the same pass and pass through the stages together.  That holds as long as every
     // workgroup has made its k-th draw before any makes its (k+1)-th, which the waits see to from the third
     // pass on; before its second draw a workgroup gives the others a moment to make their first (bounded: a
     // few microseconds, whether or not they all come).
-    if (align) {
+    if (UNLIKELY(align)) {
       const uint32_t everyone = min(static_cast<uint32_t>(gridDim.x), static_cast<uint32_t>(t.nres));
       for (int spins = 0; spins < 256 && ld_agent(t.ctl + kCtlTicket) < everyone; ++spins) __builtin_amdgcn_s_sleep(8);
     }
-    ticket = atomicAdd(t.ctl + kCtlTicket, 1u);  // for this pass's stage N
+    ticket = atomicAdd(t.ctl + kCtlTicket, 1u);
   }
   // ---- stage M on s1 ---------------------------------------------------------------------------------------
-  if (s1.real()) {
+  if (LIKELY(s1.real())) {
     float a[3] = {0.f, 0.f, 0.f};
-    if (!bad) {
+    if (LIKELY(!bad)) {
       const LansElem el = make_elem(sc, g_norm, bc1, bc2);
       moments_chunk<PAR>(t, s1, el, g, um_new, ug_new, sh, a, ticket);
     } else {
@@ -762,16 +747,16 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
   const bool need_u = s0.real();
   const bool need_g = s2.real() && own_norms;
 #ifndef LANCET_LANS_PROBE
-  if (need_u) {
+  if (LIKELY(need_u)) {
 #pragma unroll
     for (int k = 0; k < 3; ++k) gather_issue(t, 1 + k, s0, words_u[k]);
   }
-  if (need_g) gather_issue(t, 0, s2, words_g);
+  if (LIKELY(need_g)) gather_issue(t, 0, s2, words_g);
 #endif
   if (threadIdx.x == 0) {
     sh.u_bad = 0;
     sh.g_next_bad = 0;
-    sh.retry = 0;
+    sh.retry_u = sh.retry_g = 0;
   }
   lds_barrier();
   Slot s3;
@@ -782,16 +767,15 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
     s3.tensor = -1;
     s3.dead = 0;
     if (s3.chunk >= 0) {
-      const ChunkView c = chunk_view(t, s3.chunk);
-      s3.tensor = c.tensor;
-      if (c.tensor >= 0) {
-        s3.begin = c.begin;
-        s3.lo = t.tensor_first[c.tensor];
-        s3.nc = t.tensor_chunks[c.tensor];
+      s3.tensor = ld_table(t.chunk_tensor + s3.chunk);
+      if (s3.tensor >= 0) {
+        s3.lo = ld_table(t.tensor_first + s3.tensor);
+        s3.nc = ld_table(t.tensor_chunks + s3.tensor);
+        s3.begin = static_cast<int64_t>(s3.chunk - s3.lo) * kLansChunk;
       }
     }
   }
-  if (s3.real()) {
+  if (LIKELY(s3.real())) {
     // g of the chunk into registers, its sum of squares published (L2NormFunctor, multi_tensor_lans.cu:95-167)
     float a = load_g(t, s3, g);
     if (own_norms) {
@@ -809,24 +793,57 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
   lds_barrier();
 #else
   {
-    bool retry = false;
-    if (need_u) {
+    bool miss_u = false, miss_g = false, poisoned_u = false, poisoned_g = false;
+    if (LIKELY(need_u)) {
 #pragma unroll
-      for (int k = 0; k < 3; ++k) gather_take(sc, s0, words_u[k], sh.part[1 + k], retry);
+      for (int k = 0; k < 3; ++k) gather_take(sc, s0, words_u[k], sh.part[1 + k], miss_u, poisoned_u);
     }
-    if (need_g) gather_take(sc, s2, words_g, sh.part[0], retry);
-    if (retry) sh.retry = 1;
+    if (LIKELY(need_g)) gather_take(sc, s2, words_g, sh.part[0], miss_g, poisoned_g);
+    if (UNLIKELY(poisoned_u)) sh.u_bad = 1;
+    if (UNLIKELY(poisoned_g)) sh.g_next_bad = 1;
+    if (UNLIKELY(miss_u)) sh.retry_u = 1;
+    if (UNLIKELY(miss_g)) sh.retry_g = 1;
   }
   lds_barrier();
-  if (__builtin_amdgcn_readfirstlane(sh.retry) != 0) {
-    // something was not there yet (or is poisoned): everything again, with patience
-    if (need_u) {
-      bool missing = false;
+  // A workgroup that is ahead of one it depends on gets here before that one has published: it reads
+  // everything again until it is all there.  Bounded; and once any wait of the plan has given up the
+  // others stop at their next look, so that a stalled step ends after about one bound, not one per chunk.
+  if (__builtin_expect(__builtin_amdgcn_readfirstlane(sh.retry_u | sh.retry_g) != 0, 0))
 #pragma unroll 1
-      for (int k = 1; k < 4; ++k) missing = gather_again(t, sc, k, s0, sh.part[k]) || missing;
-      if (missing) sh.u_bad = 1;
+  for (uint32_t spins = 1; __builtin_amdgcn_readfirstlane(sh.retry_u | sh.retry_g) != 0; ++spins) {
+#ifdef LANCET_LANS_DIAG
+    if (threadIdx.x == 0 && spins == 1) atomicAdd(t.ctl + 3, 1u);
+#endif
+    const bool again_u = __builtin_amdgcn_readfirstlane(sh.retry_u) != 0;
+    const bool again_g = __builtin_amdgcn_readfirstlane(sh.retry_g) != 0;
+    lds_barrier();  // everyone has seen the flags
+    if (threadIdx.x == 0) {
+      sh.retry_u = sh.retry_g = 0;
+      if (sh.give_up != 0 || spins > sc.spin_limit || ((spins & 15u) == 0u && ld_agent(t.ctl + kCtlError) != 0u)) {
+        flag_error(t);
+        if (again_u) sh.u_bad = 1;
+        if (again_g) sh.g_next_bad = 1;
+        sh.give_up = 1;
+      }
     }
-    if (need_g && gather_again(t, sc, 0, s2, sh.part[0])) sh.g_next_bad = 1;
+    lds_barrier();
+    if (__builtin_amdgcn_readfirstlane(sh.give_up) != 0) break;
+    __builtin_amdgcn_s_sleep(8);
+    bool miss_u = false, miss_g = false, poisoned_u = false, poisoned_g = false;
+    if (again_u) {
+#pragma unroll
+      for (int k = 0; k < 3; ++k) gather_issue(t, 1 + k, s0, words_u[k]);
+#pragma unroll
+      for (int k = 0; k < 3; ++k) gather_take(sc, s0, words_u[k], sh.part[1 + k], miss_u, poisoned_u);
+    }
+    if (again_g) {
+      gather_issue(t, 0, s2, words_g);
+      gather_take(sc, s2, words_g, sh.part[0], miss_g, poisoned_g);
+    }
+    if (poisoned_u) sh.u_bad = 1;
+    if (poisoned_g) sh.g_next_bad = 1;
+    if (miss_u) sh.retry_u = 1;
+    if (miss_g) sh.retry_g = 1;
     lds_barrier();
   }
   {
@@ -853,13 +870,13 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
   // ---- stage U on s0 ---------------------------------------------------------------------------------------
   // Trust ratios and the parameter update (LANSStage2Functor, multi_tensor_lans.cu:326-399) from the updates
   // in registers and the parameters in LDS.  Nothing is written unless all three norms are known.
-  if (need_u && !s0.dead && __builtin_amdgcn_readfirstlane(sh.u_bad) == 0) {
+  if (LIKELY(need_u && !s0.dead && __builtin_amdgcn_readfirstlane(sh.u_bad) == 0)) {
     const float pn = uniform(sh.norm[1]), umn = uniform(sh.norm[2]), ugn = uniform(sh.norm[3]);
     float ratio_m = (umn != 0.f && pn != 0.f) ? sc.lr * (pn / umn) : sc.lr;
     float ratio_g = (ugn != 0.f && pn != 0.f) ? sc.lr * (pn / ugn) : sc.lr;
     ratio_m = uniform(ratio_m * sc.beta1);
     ratio_g = uniform(ratio_g * sc.beta3);
-    LANCET_GLOBAL float* p = as_global(t.p[s0.tensor] + s0.begin);
+    LANCET_GLOBAL float* p = as_global(ld_table(t.p + s0.tensor) + s0.begin);
 #pragma unroll
     for (int k = 0; k < kVecPerThread; ++k) {
       f32x4 xp = sh.p[PAR ^ 1][k][threadIdx.x];
@@ -868,7 +885,7 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
 #pragma clang fp contract(off)
         xp[j] = xp[j] - (ratio_m * um_old[k][j]) - (ratio_g * ug_old[k][j]);
       }
-      st_chunk4(p, chunk_elem(k), xp);
+      st_chunk4(p, k, xp);
     }
   }
   stage_fence();
@@ -920,13 +937,13 @@ __global__ __launch_bounds__(kLansThreads, kResidentWavesPerSimd) void lans_resi
   if (threadIdx.x == 0) {
     sh.g_next = 0.f;
     sh.g_next_bad = 0;
+    sh.give_up = 0;
   }
-  uint32_t ticket = 0u;  // thread 0
   // the first two passes find empty slots (their stages M and U have nothing to do) and fill the pipeline;
   // every pass draws a ticket, tickets run out, and every wait is bounded: all workgroups leave
   for (int pair = 0;; ++pair) {
-    if (!pipeline_pass<0>(t, sc, bc1, bc2, s0, s1, s2, ticket, ga, um0, ug0, um1, ug1, sh, false)) break;
-    if (!pipeline_pass<1>(t, sc, bc1, bc2, s0, s1, s2, ticket, gb, um1, ug1, um0, ug0, sh, pair == 0 && LANCET_LANS_ALIGN != 0)) break;
+    if (!pipeline_pass<0>(t, sc, bc1, bc2, s0, s1, s2, ga, um0, ug0, um1, ug1, sh, false)) break;
+    if (!pipeline_pass<1>(t, sc, bc1, bc2, s0, s1, s2, gb, um1, ug1, um0, ug0, sh, pair == 0 && LANCET_LANS_ALIGN != 0)) break;
   }
 }
 
@@ -1270,6 +1287,13 @@ extern "C" int lancet_lans_plan_error(lancet_lans_plan_t pl, lancet_stream_t str
   if (!error_out) return LANCET_ERR_NULL;
   uint32_t word = 0;
   hipStream_t st = static_cast<hipStream_t>(stream);
+#ifdef LANCET_LANS_DIAG
+  {
+    uint32_t w[4];
+    (void)hipMemcpy(w, pl->tables.ctl, sizeof(w), hipMemcpyDeviceToHost);
+    fprintf(stderr, "[diag] retries %u (all steps so far), passes per step ~%d\n", w[3], pl->tables.nres);
+  }
+#endif
   hipError_t e = hipMemcpyAsync(&word, pl->tables.ctl + kCtlError, sizeof(word), hipMemcpyDeviceToHost, st);
   if (e == hipSuccess) e = hipStreamSynchronize(st);
   // the reader, and only the reader, clears the error (the steps on `stream` have finished)

@@ -48,7 +48,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // control words of a plan (uint32): [0] next ticket of the resident kernel, [1] error (sticky: only
 // lancet_lans_plan_error clears it), [2] step epoch, [3] unused
-constexpr int kCtlTicket = 0, kCtlError = 1, kCtlEpoch = 2, kCtlWords = 4;
+constexpr int kCtlTicket = 0, kCtlError = 1, kCtlEpoch = 2, kCtlWords = 8;
 
 struct LansTables {
   const float* const* g;  // [T] device pointers
@@ -71,6 +71,9 @@ struct LansTables {
   int T;
   int nchunks;                 // chunk slots, padding included
   int nres;                    // slots [0, nres) are handed out by the resident kernel
+#ifdef LANCET_LANS_TRACE
+  uint64_t* trace;             // 4 time stamps per chunk slot: draw, publish of stage M, look, ready
+#endif
   uint32_t debug_flags;        // bit 0: the last arriver withholds the norms (exercises the bounded waits)
 };
 
@@ -451,6 +454,12 @@ constexpr int kVecPerThread = kLansChunk / 4 / kLansThreads;  // float4 per thre
 #ifndef LANCET_LANS_ALIGN
 #define LANCET_LANS_ALIGN 1
 #endif
+#ifndef LANCET_LANS_PROBE
+#define LANCET_LANS_PROBE 0
+#endif
+#ifndef LANCET_LANS_POLL_SLEEP
+#define LANCET_LANS_POLL_SLEEP 16
+#endif
 #ifndef LANCET_LANS_SB
 #define LANCET_LANS_SB 0
 #endif
@@ -466,22 +475,21 @@ __device__ __forceinline__ void stage_fence() {
 #endif
 }
 
+// The thread's place in its workgroup, formed anew wherever it is needed: the wave's index is handed down in a
+// scalar register and the lane's number costs two instructions.  A value kept in a vector register from the
+// start of the kernel gets spilled in this code, and a reload that follows stores waits for all of them.
+__device__ __forceinline__ int fresh_lane() {
+  int l;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+  return l;
+}
+__device__ __forceinline__ int fresh_tid(int wave) { return wave * kWave + fresh_lane(); }
+__device__ __forceinline__ bool is_first(int wave) { return wave == 0 && fresh_lane() == 0; }
+
 // Workgroup barrier that orders LDS accesses only.  __syncthreads() also waits for every global load and
 // store the wave has in flight, which would drain the streams of this kernel several times per chunk; all
 // that crosses the waves of a workgroup here is in LDS (global words other workgroups read are atomics).
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-
-__device__ __forceinline__ float block_sum_lds(float v, float* s_red) {
-  v = wave_sum(v);
-  if (lane_id() == 0) s_red[threadIdx.x / kWave] = v;
-  lds_barrier();
-  float r = 0.f;
-  if (threadIdx.x == 0) {
-#pragma unroll
-    for (int k = 0; k < kLansThreads / kWave; ++k) r += s_red[k];
-  }
-  return r;  // valid on thread 0; s_red is free again after the caller's next barrier
-}
 
 constexpr int kMaxResidentChunks = 4 * 1024 * 1024 / kLansChunk;      // chunks of the largest tensor the kernel takes (4M parameters)
 constexpr int kGatherPerThread = kMaxResidentChunks / kLansThreads;  // partials of one norm a thread reads
@@ -495,9 +503,12 @@ struct PipeShared {
   float g_next;    // ||g|| of s2's tensor: for stage M of the next pass
   int g_next_bad;  // ... is unknown
   int u_bad;       // a norm of s0's tensor is unknown
-  int retry_u, retry_g;  // a sum read ahead was not there yet
+  int retry;             // a sum read ahead was not there yet
   int give_up;           // ... and never came (sticky for the rest of the kernel)
   int chunk;
+#ifdef LANCET_LANS_DIAG
+  int diag[2];
+#endif
 };
 
 // a chunk a workgroup holds between stages; every field is uniform over the workgroup
@@ -526,21 +537,32 @@ __device__ __forceinline__ T ld_table(const T* p) {
 // k * 256 elements further on (one load instruction of a wave covers 1 KB of consecutive memory).  The
 // address is a uniform 64-bit base plus an unsigned 32-bit offset per lane, the form that takes its base
 // from scalar registers and one vector register for the offset.
-__device__ __forceinline__ uint32_t lane_offset() {
-  return static_cast<uint32_t>((threadIdx.x / kWave) * (kLansChunk / kWavesPerTile) + 4 * lane_id());
+__device__ __forceinline__ uint32_t lane_offset(int wave) {
+  return static_cast<uint32_t>(wave * (kLansChunk / kWavesPerTile) + 4 * fresh_lane());
 }
-__device__ __forceinline__ f32x4 ld_chunk4(const LANCET_GLOBAL float* a, int k) {
-  return __builtin_nontemporal_load((const LANCET_GLOBAL f32x4*)(a + k * (4 * kWave) + lane_offset()));
+__device__ __forceinline__ f32x4 ld_chunk4(const LANCET_GLOBAL float* a, int k, int wave) {
+#if !defined(LANCET_LANS_NT) || (LANCET_LANS_NT & 1)
+  return __builtin_nontemporal_load((const LANCET_GLOBAL f32x4*)(a + k * (4 * kWave) + lane_offset(wave)));
+#else
+  return *(const LANCET_GLOBAL f32x4*)(a + k * (4 * kWave) + lane_offset(wave));
+#endif
 }
-__device__ __forceinline__ void st_chunk4(LANCET_GLOBAL float* a, int k, f32x4 x) {
-  __builtin_nontemporal_store(x, (LANCET_GLOBAL f32x4*)(a + k * (4 * kWave) + lane_offset()));
+#ifndef LANCET_LANS_NT
+#define LANCET_LANS_NT 3
+#endif
+__device__ __forceinline__ void st_chunk4(LANCET_GLOBAL float* a, int k, f32x4 x, int wave) {
+#if LANCET_LANS_NT & 2
+  __builtin_nontemporal_store(x, (LANCET_GLOBAL f32x4*)(a + k * (4 * kWave) + lane_offset(wave)));
+#else
+  *(LANCET_GLOBAL f32x4*)(a + k * (4 * kWave) + lane_offset(wave)) = x;
+#endif
 }
 
 // Thread 0: publishes the N chunk sums a[] of slot s as words first .. first+N-1 (fire and forget).
 template <int N>
 __device__ __forceinline__ void publish(const LansTables& t, const LansScalars& sc, int first, const Slot& s,
                                         const float (&a)[N], bool poison) {
-#ifdef LANCET_LANS_PROBE
+#if LANCET_LANS_PROBE == 1
   return;
 #endif
   if (t.debug_flags & 1u) return;  // test hook: nothing is ever published, every wait runs into its bound
@@ -550,38 +572,28 @@ __device__ __forceinline__ void publish(const LansTables& t, const LansScalars& 
 }
 
 // the partials of one norm of slot s's tensor as this thread reads them (issued, not yet looked at)
-__device__ __forceinline__ void gather_issue(const LansTables& t, int kind, const Slot& s, uint64_t (&word)[kGatherPerThread]) {
+__device__ __forceinline__ void gather_issue(const LansTables& t, int kind, const Slot& s, uint64_t (&word)[kGatherPerThread], int wave) {
   const uint64_t* src = t.part_word + static_cast<size_t>(kind) * t.nchunks + s.lo;
 #pragma unroll
   for (int i = 0; i < kGatherPerThread; ++i) {
-    const int c = threadIdx.x + i * kLansThreads;
+    const int c = fresh_tid(wave) + i * kLansThreads;
     word[i] = c < s.nc ? ld_word(src + c) : 0;
   }
 }
-// ... looked at: values into LDS; says whether a word is not of this step yet, or is poisoned
+// ... looked at: values into LDS.  Bit first_bit + i of `missing` is set for a word that is not of this step
+// yet; `poisoned` for one that is and carries the poison mark.
 __device__ __forceinline__ void gather_take(const LansScalars& sc, const Slot& s, const uint64_t (&word)[kGatherPerThread],
-                                            float* part, bool& missing, bool& poisoned) {
+                                            float* part, int first_bit, uint32_t& missing, bool& poisoned, int wave) {
 #pragma unroll
   for (int i = 0; i < kGatherPerThread; ++i) {
-    const int c = threadIdx.x + i * kLansThreads;
+    const int c = fresh_tid(wave) + i * kLansThreads;
     if (c < s.nc) {
       part[c] = __uint_as_float(static_cast<uint32_t>(word[i]));
       const bool there = word_is_current(word[i], sc.epoch);
-      missing = missing || !there;
+      if (!there) missing |= 1u << (first_bit + i);
       poisoned = poisoned || (there && word_is_poisoned(word[i]));
     }
   }
-}
-
-__device__ __forceinline__ float load_g(const LansTables& t, const Slot& s, f32x4 (&g)[kVecPerThread]) {
-  const LANCET_GLOBAL float* src = as_global(ld_table(t.g + s.tensor) + s.begin);
-  float a = 0.f;
-#pragma unroll
-  for (int k = 0; k < kVecPerThread; ++k) {
-    g[k] = ld_chunk4(src, k);
-    a += g[k].x * g[k].x + g[k].y * g[k].y + g[k].z * g[k].z + g[k].w * g[k].w;
-  }
-  return a;
 }
 
 // Moments and the two updates (LANSStage1Functor, multi_tensor_lans.cu:207-322, and the l2norm sweeps
@@ -591,7 +603,7 @@ __device__ __forceinline__ float load_g(const LansTables& t, const Slot& s, f32x
 template <int PAR>
 __device__ __forceinline__ void moments_chunk(const LansTables& t, const Slot& s, const LansElem& el,
                                               const f32x4 (&g)[kVecPerThread], f32x4 (&um)[kVecPerThread],
-                                              f32x4 (&ug)[kVecPerThread], PipeShared& sh, float (&a)[3], uint32_t ticket) {
+                                              f32x4 (&ug)[kVecPerThread], PipeShared& sh, float (&a)[3], uint32_t ticket, int wave) {
   const LANCET_GLOBAL float* p = as_global(ld_table(t.p + s.tensor) + s.begin);
   LANCET_GLOBAL float* m = as_global(ld_table(t.m + s.tensor) + s.begin);
   LANCET_GLOBAL float* v = as_global(ld_table(t.v + s.tensor) + s.begin);
@@ -600,26 +612,26 @@ __device__ __forceinline__ void moments_chunk(const LansTables& t, const Slot& s
   f32x4 np[kPrefetch], nm[kPrefetch], nv[kPrefetch];
 #pragma unroll
   for (int d = 0; d < kPrefetch; ++d) {
-    np[d] = ld_chunk4(p, d);
-    nm[d] = ld_chunk4(m, d);
-    nv[d] = ld_chunk4(v, d);
+    np[d] = ld_chunk4(p, d, wave);
+    nm[d] = ld_chunk4(m, d, wave);
+    nv[d] = ld_chunk4(v, d, wave);
   }
   // the ticket drawn at the start of the pass is looked at here, behind the first loads and in front of every
   // store of the stage: looked at behind the stores it would cost their completion
-  if (threadIdx.x == 0) sh.chunk = static_cast<int>(ticket);
+  if (is_first(wave)) sh.chunk = static_cast<int>(ticket);
 #pragma unroll
   for (int k = 0; k < kVecPerThread; ++k) {
     const f32x4 xp = np[k % kPrefetch];
     f32x4 xm = nm[k % kPrefetch], xv = nv[k % kPrefetch];
     if (k + kPrefetch < kVecPerThread) {
-      np[k % kPrefetch] = ld_chunk4(p, k + kPrefetch);
-      nm[k % kPrefetch] = ld_chunk4(m, k + kPrefetch);
-      nv[k % kPrefetch] = ld_chunk4(v, k + kPrefetch);
+      np[k % kPrefetch] = ld_chunk4(p, k + kPrefetch, wave);
+      nm[k % kPrefetch] = ld_chunk4(m, k + kPrefetch, wave);
+      nv[k % kPrefetch] = ld_chunk4(v, k + kPrefetch, wave);
     }
 #if LANCET_LANS_SB & 1
     __builtin_amdgcn_sched_barrier(0);
 #endif
-    sh.p[PAR][k][threadIdx.x] = xp;
+    sh.p[PAR][k][fresh_tid(wave)] = xp;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const float sg = el.scaled_grad(g[k][j], xp[j]);
@@ -637,8 +649,8 @@ __device__ __forceinline__ void moments_chunk(const LansTables& t, const Slot& s
       a1 += u0 * u0;
       a2 += u1 * u1;
     }
-    st_chunk4(m, k, xm);
-    st_chunk4(v, k, xv);
+    st_chunk4(m, k, xm, wave);
+    st_chunk4(v, k, xv, wave);
 #if LANCET_LANS_SB & 2
     __builtin_amdgcn_sched_barrier(0);
 #endif
@@ -646,6 +658,71 @@ __device__ __forceinline__ void moments_chunk(const LansTables& t, const Slot& s
   a[0] = a0;
   a[1] = a1;
   a[2] = a2;
+}
+
+// The slow path of a pass's gather: some of the sums this workgroup needs are not published yet.  Every
+// thread reads the words it misses again (bit kind * kGatherPerThread + i of `missing`: word i of its share of
+// that kind; lo_g / lo_u: first chunk slot of the tensor whose g sums / whose other sums are gathered) until
+// they are all there, or until the bound.  A function of its own on purpose: it runs rarely, is full of
+// loops, and inlined it misleads the register allocation of the straight-line code around it.
+__device__ __noinline__ void regather(const uint64_t* part_word, int nchunks, uint32_t* ctl, uint32_t* host_status,
+                                      uint32_t epoch, uint32_t spin_limit, int lo_g, int lo_u, uint32_t missing,
+                                      PipeShared* shp, int wave) {
+  PipeShared& sh = *shp;
+#pragma unroll 1
+  for (uint32_t spins = 1;; ++spins) {
+    lds_barrier();  // everyone has seen the flag
+    if (is_first(wave)) {
+      sh.retry = 0;
+      if (sh.give_up != 0 || spins > spin_limit || ((spins & 15u) == 0u && ld_agent(ctl + kCtlError) != 0u)) {
+        st_agent(ctl + kCtlError, 1u);
+        __hip_atomic_store(host_status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        sh.give_up = 1;
+      }
+    }
+    lds_barrier();
+    if (__builtin_amdgcn_readfirstlane(sh.give_up) != 0) {
+      if (missing >> kGatherPerThread) sh.u_bad = 1;
+      if (missing & ((1u << kGatherPerThread) - 1u)) sh.g_next_bad = 1;
+      lds_barrier();
+      return;
+    }
+    __builtin_amdgcn_s_sleep(LANCET_LANS_POLL_SLEEP);
+#pragma unroll 1
+    for (uint32_t left = missing; left != 0u; left &= left - 1u) {
+      const int bit = __builtin_ctz(left);
+      const int kind = bit / kGatherPerThread;
+      const int c = fresh_tid(wave) + (bit % kGatherPerThread) * kLansThreads;
+      const uint64_t x = ld_word(part_word + static_cast<size_t>(kind) * nchunks + (kind == 0 ? lo_g : lo_u) + c);
+      if (word_is_current(x, epoch)) {
+        missing &= ~(1u << bit);
+        sh.part[kind][c] = __uint_as_float(static_cast<uint32_t>(x));
+        if (word_is_poisoned(x)) {
+          if (kind == 0) sh.g_next_bad = 1; else sh.u_bad = 1;
+        }
+      }
+    }
+    if (missing != 0u) sh.retry = 1;
+    lds_barrier();
+    if (__builtin_amdgcn_readfirstlane(sh.retry) == 0) return;
+  }
+}
+
+// wave_norm over nc <= kMaxResidentChunks sums in LDS: the same additions in the same order (a sum that is not
+// there counts as +0, which changes no bit of a sum of squares), with all of a lane's reads issued at once.
+__device__ __forceinline__ float wave_norm_lds(const float* part, int nc) {
+  float x[kMaxResidentChunks / kWave];
+#pragma unroll
+  for (int i = 0; i < kMaxResidentChunks / kWave; ++i) {
+    const int c = fresh_lane() + i * kWave;
+    x[i] = c < nc ? part[c] : 0.f;
+  }
+  double acc = 0.0;
+#pragma unroll
+  for (int i = 0; i < kMaxResidentChunks / kWave; ++i) acc += static_cast<double>(x[i]);
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, kWave);
+  return static_cast<float>(sqrt(acc));
 }
 
 // Gives register arrays a value on the paths that do not fill them.  Without it the value they held before
@@ -681,7 +758,7 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
                                               f32x4 (&g)[kVecPerThread],
                                               f32x4 (&um_new)[kVecPerThread], f32x4 (&ug_new)[kVecPerThread],
                                               const f32x4 (&um_old)[kVecPerThread], const f32x4 (&ug_old)[kVecPerThread],
-                                              PipeShared& sh, bool align) {
+                                              PipeShared& sh, bool align, int wave) {
   const bool own_norms = t.grad_norms == nullptr;
   // ---- start of the pass ---------------------------------------------------------------------------------
   lds_barrier();
@@ -696,7 +773,10 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
     }
   }
   uint32_t ticket = 0u;  // thread 0: for this pass's stage N
-  if (threadIdx.x == 0) {
+#ifdef LANCET_LANS_TRACE
+  const uint64_t t_draw = wall_clock64();
+#endif
+  if (is_first(wave)) {
     // The plan lays a tensor's chunks out inside one round of as many slots as there are workgroups, so that
     // they are all drawn in the same pass and pass through the stages together.  That holds as long as every
     // workgroup has made its k-th draw before any makes its (k+1)-th, which the waits see to from the third
@@ -713,20 +793,20 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
     float a[3] = {0.f, 0.f, 0.f};
     if (LIKELY(!bad)) {
       const LansElem el = make_elem(sc, g_norm, bc1, bc2);
-      moments_chunk<PAR>(t, s1, el, g, um_new, ug_new, sh, a, ticket);
+      moments_chunk<PAR>(t, s1, el, g, um_new, ug_new, sh, a, ticket, wave);
     } else {
-      if (threadIdx.x == 0) sh.chunk = static_cast<int>(ticket);
+      if (is_first(wave)) sh.chunk = static_cast<int>(ticket);
       s1.dead = 1;  // ||g|| is unknown: the chunk is left as it is, and so will its tensor's parameters be
       forget(um_new, ug_new);
     }
 #pragma unroll
     for (int k = 0; k < 3; ++k) a[k] = wave_sum(a[k]);
-    if (lane_id() == 0) {
+    if (fresh_lane() == 0) {
 #pragma unroll
-      for (int k = 0; k < 3; ++k) sh.red[k][threadIdx.x / kWave] = a[k];
+      for (int k = 0; k < 3; ++k) sh.red[k][wave] = a[k];
     }
     lds_barrier();
-    if (threadIdx.x == 0) {
+    if (is_first(wave)) {
 #pragma unroll
       for (int k = 0; k < 3; ++k) {
         float r = 0.f;
@@ -735,28 +815,23 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
         a[k] = r;
       }
       publish<3>(t, sc, 1, s1, a, bad);
+#ifdef LANCET_LANS_TRACE
+      t.trace[4 * s1.chunk + 1] = wall_clock64();
+#endif
     }
   } else {
-    if (threadIdx.x == 0) sh.chunk = static_cast<int>(ticket);
+    if (is_first(wave)) sh.chunk = static_cast<int>(ticket);
     forget(um_new, ug_new);
   }
   stage_fence();
   // ---- stage N on a new slot -------------------------------------------------------------------------------
-  // in front of the loads of g: the sums other workgroups have published
   uint64_t words_g[kGatherPerThread], words_u[3][kGatherPerThread];
   const bool need_u = s0.real();
   const bool need_g = s2.real() && own_norms;
-#ifndef LANCET_LANS_PROBE
-  if (LIKELY(need_u)) {
-#pragma unroll
-    for (int k = 0; k < 3; ++k) gather_issue(t, 1 + k, s0, words_u[k]);
-  }
-  if (LIKELY(need_g)) gather_issue(t, 0, s2, words_g);
-#endif
-  if (threadIdx.x == 0) {
+  if (is_first(wave)) {
     sh.u_bad = 0;
     sh.g_next_bad = 0;
-    sh.retry_u = sh.retry_g = 0;
+    sh.retry = 0;
   }
   lds_barrier();
   Slot s3;
@@ -775,90 +850,99 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
       }
     }
   }
+#ifdef LANCET_LANS_TRACE
+  if (is_first(wave) && s3.real()) t.trace[4 * s3.chunk + 0] = t_draw;
+#endif
+  // g of the chunk into registers (L2NormFunctor, multi_tensor_lans.cu:95-167) and, right behind those loads,
+  // the sums other workgroups have published: read as late as possible, and still back before anything waits
+  // for them alone
   if (LIKELY(s3.real())) {
-    // g of the chunk into registers, its sum of squares published (L2NormFunctor, multi_tensor_lans.cu:95-167)
-    float a = load_g(t, s3, g);
-    if (own_norms) {
-      a = block_sum_lds(a, sh.red[0]);
-      if (threadIdx.x == 0) {
-        const float sums[1] = {a};
-        publish<1>(t, sc, 0, s3, sums, false);
-      }
-    }
+    const LANCET_GLOBAL float* src = as_global(ld_table(t.g + s3.tensor) + s3.begin);
+#pragma unroll
+    for (int k = 0; k < kVecPerThread; ++k) g[k] = ld_chunk4(src, k, wave);
+  }
+#if LANCET_LANS_PROBE != 1
+  if (LIKELY(need_u)) {
+#pragma unroll
+    for (int k = 0; k < 3; ++k) gather_issue(t, 1 + k, s0, words_u[k], wave);
+  }
+  if (LIKELY(need_g)) gather_issue(t, 0, s2, words_g, wave);
+#endif
+  if (LIKELY(s3.real())) {
+    float a = 0.f;
+#pragma unroll
+    for (int k = 0; k < kVecPerThread; ++k) a += g[k].x * g[k].x + g[k].y * g[k].y + g[k].z * g[k].z + g[k].w * g[k].w;
+    a = wave_sum(a);
+    if (fresh_lane() == 0) sh.red[0][wave] = a;
   }
   stage_fence();
   // ---- the norms ---------------------------------------------------------------------------------------------
-#ifdef LANCET_LANS_PROBE
-  if (threadIdx.x == 0) sh.norm[1] = sh.norm[2] = sh.norm[3] = sh.g_next = 1.f;
+#if LANCET_LANS_PROBE == 1
+  if (is_first(wave)) sh.norm[1] = sh.norm[2] = sh.norm[3] = sh.g_next = 1.f;
   lds_barrier();
 #else
+  // bit kind * kGatherPerThread + i: word i of this thread's share of that norm's sums is still missing
+  uint32_t missing = 0u;
   {
-    bool miss_u = false, miss_g = false, poisoned_u = false, poisoned_g = false;
+    bool poisoned_u = false, poisoned_g = false;
     if (LIKELY(need_u)) {
 #pragma unroll
-      for (int k = 0; k < 3; ++k) gather_take(sc, s0, words_u[k], sh.part[1 + k], miss_u, poisoned_u);
+      for (int k = 1; k < 4; ++k) gather_take(sc, s0, words_u[k - 1], sh.part[k], k * kGatherPerThread, missing, poisoned_u, wave);
     }
-    if (LIKELY(need_g)) gather_take(sc, s2, words_g, sh.part[0], miss_g, poisoned_g);
+    if (LIKELY(need_g)) gather_take(sc, s2, words_g, sh.part[0], 0, missing, poisoned_g, wave);
     if (UNLIKELY(poisoned_u)) sh.u_bad = 1;
     if (UNLIKELY(poisoned_g)) sh.g_next_bad = 1;
-    if (UNLIKELY(miss_u)) sh.retry_u = 1;
-    if (UNLIKELY(miss_g)) sh.retry_g = 1;
-  }
-  lds_barrier();
-  // A workgroup that is ahead of one it depends on gets here before that one has published: it reads
-  // everything again until it is all there.  Bounded; and once any wait of the plan has given up the
-  // others stop at their next look, so that a stalled step ends after about one bound, not one per chunk.
-  if (__builtin_expect(__builtin_amdgcn_readfirstlane(sh.retry_u | sh.retry_g) != 0, 0))
-#pragma unroll 1
-  for (uint32_t spins = 1; __builtin_amdgcn_readfirstlane(sh.retry_u | sh.retry_g) != 0; ++spins) {
-#ifdef LANCET_LANS_DIAG
-    if (threadIdx.x == 0 && spins == 1) atomicAdd(t.ctl + 3, 1u);
+#if LANCET_LANS_PROBE == 2
+    missing = 0u;  // timing experiment: nobody waits
 #endif
-    const bool again_u = __builtin_amdgcn_readfirstlane(sh.retry_u) != 0;
-    const bool again_g = __builtin_amdgcn_readfirstlane(sh.retry_g) != 0;
-    lds_barrier();  // everyone has seen the flags
-    if (threadIdx.x == 0) {
-      sh.retry_u = sh.retry_g = 0;
-      if (sh.give_up != 0 || spins > sc.spin_limit || ((spins & 15u) == 0u && ld_agent(t.ctl + kCtlError) != 0u)) {
-        flag_error(t);
-        if (again_u) sh.u_bad = 1;
-        if (again_g) sh.g_next_bad = 1;
-        sh.give_up = 1;
-      }
-    }
-    lds_barrier();
-    if (__builtin_amdgcn_readfirstlane(sh.give_up) != 0) break;
-    __builtin_amdgcn_s_sleep(8);
-    bool miss_u = false, miss_g = false, poisoned_u = false, poisoned_g = false;
-    if (again_u) {
-#pragma unroll
-      for (int k = 0; k < 3; ++k) gather_issue(t, 1 + k, s0, words_u[k]);
-#pragma unroll
-      for (int k = 0; k < 3; ++k) gather_take(sc, s0, words_u[k], sh.part[1 + k], miss_u, poisoned_u);
-    }
-    if (again_g) {
-      gather_issue(t, 0, s2, words_g);
-      gather_take(sc, s2, words_g, sh.part[0], miss_g, poisoned_g);
-    }
-    if (poisoned_u) sh.u_bad = 1;
-    if (poisoned_g) sh.g_next_bad = 1;
-    if (miss_u) sh.retry_u = 1;
-    if (miss_g) sh.retry_g = 1;
-    lds_barrier();
+    if (UNLIKELY(missing != 0u)) sh.retry = 1;
   }
+#ifdef LANCET_LANS_TRACE
+  if (is_first(wave) && need_u) t.trace[4 * s0.chunk + 2] = wall_clock64();
+#endif
+  lds_barrier();
+  if (is_first(wave) && s3.real() && own_norms) {
+    float r = 0.f;
+#pragma unroll
+    for (int w = 0; w < kLansThreads / kWave; ++w) r += sh.red[0][w];
+    const float sums[1] = {r};
+    publish<1>(t, sc, 0, s3, sums, false);
+  }
+  // A workgroup that is ahead of one it depends on gets here before that one has published.  Its threads
+  // read the words they miss again (only those: hundreds of workgroups wait like this at any time, and what
+  // they read while they wait competes with the one they wait for) until they are all there.  Bounded; and
+  // once any wait of the plan has given up the others stop at their next look, so that a stalled step ends
+  // after about one bound, not one per chunk.
+  if (UNLIKELY(__builtin_amdgcn_readfirstlane(sh.retry) != 0)) {
+#ifdef LANCET_LANS_DIAG
+    if (missing & ((1u << kGatherPerThread) - 1u)) sh.diag[0] = 1;
+    if (missing >> kGatherPerThread) sh.diag[1] = 1;
+    lds_barrier();
+    if (is_first(wave)) {
+      atomicAdd(t.ctl + 3, 1u);
+      if (sh.diag[0]) atomicAdd(t.ctl + 4, 1u);
+      if (sh.diag[1]) atomicAdd(t.ctl + 5, 1u);
+      sh.diag[0] = sh.diag[1] = 0;
+    }
+#endif
+    regather(t.part_word, t.nchunks, t.ctl, t.host_status, sc.epoch, sc.spin_limit, s2.lo, s0.lo, missing, &sh, wave);
+  }
+#ifdef LANCET_LANS_TRACE
+  if (is_first(wave) && need_u) t.trace[4 * s0.chunk + 3] = wall_clock64();
+#endif
   {
-    const int w = threadIdx.x / kWave;  // wave w sums norm w: the same fixed order in every workgroup
+    const int w = wave;  // wave w sums norm w: the same fixed order in every workgroup
     if (w == 0) {
       if (need_g) {
-        const float n = wave_norm(0, s2.nc, [&](int c) { return sh.part[0][c]; });
-        if (lane_id() == 0) {
+        const float n = wave_norm_lds(sh.part[0], s2.nc);
+        if (fresh_lane() == 0) {
           sh.g_next = n;
           if (s2.chunk == s2.lo) t.norms[s2.tensor] = n;  // for lancet_lans_plan_norms
         }
       }
     } else if (need_u) {
-      const float n = wave_norm(0, s0.nc, [&](int c) { return sh.part[w][c]; });
-      if (lane_id() == 0) {
+      const float n = wave_norm_lds(sh.part[w], s0.nc);
+      if (fresh_lane() == 0) {
         sh.norm[w] = n;
         if (s0.chunk == s0.lo) t.norms[w * t.T + s0.tensor] = n;
       }
@@ -879,13 +963,13 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
     LANCET_GLOBAL float* p = as_global(ld_table(t.p + s0.tensor) + s0.begin);
 #pragma unroll
     for (int k = 0; k < kVecPerThread; ++k) {
-      f32x4 xp = sh.p[PAR ^ 1][k][threadIdx.x];
+      f32x4 xp = sh.p[PAR ^ 1][k][fresh_tid(wave)];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
 #pragma clang fp contract(off)
         xp[j] = xp[j] - (ratio_m * um_old[k][j]) - (ratio_g * ug_old[k][j]);
       }
-      st_chunk4(p, k, xp);
+      st_chunk4(p, k, xp, wave);
     }
   }
   stage_fence();
@@ -896,6 +980,9 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
   return s0.chunk >= 0 || s1.chunk >= 0 || s2.chunk >= 0;
 }
 
+#ifndef LANCET_LANS_KATTR
+#define LANCET_LANS_KATTR
+#endif
 #ifndef LANCET_LANS_WAVES
 #define LANCET_LANS_WAVES 2
 #endif
@@ -919,8 +1006,9 @@ __global__ __launch_bounds__(kLansThreads) void lans_begin_kernel(LansTables t, 
   }
 }
 
-__global__ __launch_bounds__(kLansThreads, kResidentWavesPerSimd) void lans_resident_kernel(LansTables t, LansScalars sc) {
+__global__ __launch_bounds__(kLansThreads, kResidentWavesPerSimd) LANCET_LANS_KATTR void lans_resident_kernel(LansTables t, LansScalars sc) {
   __shared__ PipeShared sh;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x) / kWave;
   sc.epoch = __builtin_amdgcn_readfirstlane(t.ctl[kCtlEpoch]);
   float bc1, bc2;
   bias_corrections(sc, bc1, bc2);
@@ -938,12 +1026,15 @@ __global__ __launch_bounds__(kLansThreads, kResidentWavesPerSimd) void lans_resi
     sh.g_next = 0.f;
     sh.g_next_bad = 0;
     sh.give_up = 0;
+#ifdef LANCET_LANS_DIAG
+    sh.diag[0] = sh.diag[1] = 0;
+#endif
   }
   // the first two passes find empty slots (their stages M and U have nothing to do) and fill the pipeline;
   // every pass draws a ticket, tickets run out, and every wait is bounded: all workgroups leave
   for (int pair = 0;; ++pair) {
-    if (!pipeline_pass<0>(t, sc, bc1, bc2, s0, s1, s2, ga, um0, ug0, um1, ug1, sh, false)) break;
-    if (!pipeline_pass<1>(t, sc, bc1, bc2, s0, s1, s2, gb, um1, ug1, um0, ug0, sh, pair == 0 && LANCET_LANS_ALIGN != 0)) break;
+    if (!pipeline_pass<0>(t, sc, bc1, bc2, s0, s1, s2, ga, um0, ug0, um1, ug1, sh, false, wave)) break;
+    if (!pipeline_pass<1>(t, sc, bc1, bc2, s0, s1, s2, gb, um1, ug1, um0, ug0, sh, pair == 0 && LANCET_LANS_ALIGN != 0, wave)) break;
   }
 }
 
@@ -1140,6 +1231,9 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
     t.nchunks = pl->nchunks;
     t.nres = pl->n_res_chunks;
     t.debug_flags = 0u;
+#ifdef LANCET_LANS_TRACE
+    t.trace = nullptr;
+#endif
   }
   if (err != hipSuccess) {
     lancet_lans_plan_destroy(pl);
@@ -1234,6 +1328,12 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
   sc.bias_correction = h->bias_correction;
   sc.step_host = step_host;
   sc.step_dev = step_dev;
+#ifdef LANCET_LANS_TRACE
+  if (!pl->tables.trace) {
+    (void)hipMalloc(&pl->tables.trace, 4 * sizeof(uint64_t) * static_cast<size_t>(pl->tables.nres + 1));
+    (void)hipMemset(pl->tables.trace, 0, 4 * sizeof(uint64_t) * static_cast<size_t>(pl->tables.nres + 1));
+  }
+#endif
   LansTables t = pl->tables;
   t.grad_norms = grad_norms;
   sc.spin_limit = pl->spin_limit;
@@ -1287,11 +1387,27 @@ extern "C" int lancet_lans_plan_error(lancet_lans_plan_t pl, lancet_stream_t str
   if (!error_out) return LANCET_ERR_NULL;
   uint32_t word = 0;
   hipStream_t st = static_cast<hipStream_t>(stream);
+#ifdef LANCET_LANS_TRACE
+  if (const char* path = getenv("LANCET_TRACE_FILE")) {
+    (void)hipDeviceSynchronize();
+    const int n = pl->tables.nres;
+    std::vector<int32_t> ct(n);
+    std::vector<uint64_t> tr(4 * static_cast<size_t>(n));
+    (void)hipMemcpy(ct.data(), pl->tables.chunk_tensor, n * sizeof(int32_t), hipMemcpyDeviceToHost);
+    (void)hipMemcpy(tr.data(), pl->tables.trace, tr.size() * sizeof(uint64_t), hipMemcpyDeviceToHost);
+    if (FILE* f = fopen(path, "wb")) {
+      fwrite(&n, sizeof(n), 1, f);
+      fwrite(ct.data(), sizeof(int32_t), n, f);
+      fwrite(tr.data(), sizeof(uint64_t), tr.size(), f);
+      fclose(f);
+    }
+  }
+#endif
 #ifdef LANCET_LANS_DIAG
   {
-    uint32_t w[4];
+    uint32_t w[8];
     (void)hipMemcpy(w, pl->tables.ctl, sizeof(w), hipMemcpyDeviceToHost);
-    fprintf(stderr, "[diag] retries %u (all steps so far), passes per step ~%d\n", w[3], pl->tables.nres);
+    fprintf(stderr, "[diag] retries %u (g missing %u, u missing %u; all steps so far), passes per step ~%d\n", w[3], w[4], w[5], pl->tables.nres);
   }
 #endif
   hipError_t e = hipMemcpyAsync(&word, pl->tables.ctl + kCtlError, sizeof(word), hipMemcpyDeviceToHost, st);

@@ -48,7 +48,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // control words of a plan (uint32): [0] next ticket of the resident kernel, [1] error (sticky: only
 // lancet_lans_plan_error clears it), [2] step epoch, [3] unused
-constexpr int kCtlTicket = 0, kCtlError = 1, kCtlEpoch = 2, kCtlWords = 8;
+constexpr int kCtlTicket = 0, kCtlError = 1, kCtlEpoch = 2, kCtlWords = 4;
 
 struct LansTables {
   const float* const* g;  // [T] device pointers
@@ -71,9 +71,6 @@ struct LansTables {
   int T;
   int nchunks;                 // chunk slots, padding included
   int nres;                    // slots [0, nres) are handed out by the resident kernel
-#ifdef LANCET_LANS_TRACE
-  uint64_t* trace;             // 4 time stamps per chunk slot: draw, publish of stage M, look, ready
-#endif
   uint32_t debug_flags;        // bit 0: the last arriver withholds the norms (exercises the bounded waits)
 };
 
@@ -451,29 +448,9 @@ __device__ __forceinline__ bool word_is_poisoned(uint64_t x) { return (static_ca
 // schedule "resident": one persistent kernel, a three-stage software pipeline per workgroup
 // =======================================================================================
 constexpr int kVecPerThread = kLansChunk / 4 / kLansThreads;  // float4 per thread and array
-#ifndef LANCET_LANS_ALIGN
-#define LANCET_LANS_ALIGN 1
-#endif
-#ifndef LANCET_LANS_PROBE
-#define LANCET_LANS_PROBE 0
-#endif
-#ifndef LANCET_LANS_POLL_SLEEP
-#define LANCET_LANS_POLL_SLEEP 16
-#endif
-#ifndef LANCET_LANS_SB
-#define LANCET_LANS_SB 0
-#endif
-#ifndef LANCET_LANS_PREFETCH
-#define LANCET_LANS_PREFETCH 1
-#endif
-constexpr int kPrefetch = LANCET_LANS_PREFETCH;
+constexpr int kPrefetch = 3;  // float4 of each array stage M keeps in flight ahead of the one it works on
 #define LIKELY(x) __builtin_expect(!!(x), 1)
 #define UNLIKELY(x) __builtin_expect(!!(x), 0)
-__device__ __forceinline__ void stage_fence() {
-#if LANCET_LANS_SB & 4
-  __builtin_amdgcn_sched_barrier(0);
-#endif
-}
 
 // The thread's place in its workgroup, formed anew wherever it is needed: the wave's index is handed down in a
 // scalar register and the lane's number costs two instructions.  A value kept in a vector register from the
@@ -484,7 +461,7 @@ __device__ __forceinline__ int fresh_lane() {
   return l;
 }
 __device__ __forceinline__ int fresh_tid(int wave) { return wave * kWave + fresh_lane(); }
-__device__ __forceinline__ bool is_first(int wave) { return wave == 0 && fresh_lane() == 0; }
+__device__ __forceinline__ bool is_first(int wave) { return (fresh_lane() | wave) == 0; }  // thread 0, in one vector compare
 
 // Workgroup barrier that orders LDS accesses only.  __syncthreads() also waits for every global load and
 // store the wave has in flight, which would drain the streams of this kernel several times per chunk; all
@@ -506,9 +483,6 @@ struct PipeShared {
   int retry;             // a sum read ahead was not there yet
   int give_up;           // ... and never came (sticky for the rest of the kernel)
   int chunk;
-#ifdef LANCET_LANS_DIAG
-  int diag[2];
-#endif
 };
 
 // a chunk a workgroup holds between stages; every field is uniform over the workgroup
@@ -541,30 +515,16 @@ __device__ __forceinline__ uint32_t lane_offset(int wave) {
   return static_cast<uint32_t>(wave * (kLansChunk / kWavesPerTile) + 4 * fresh_lane());
 }
 __device__ __forceinline__ f32x4 ld_chunk4(const LANCET_GLOBAL float* a, int k, int wave) {
-#if !defined(LANCET_LANS_NT) || (LANCET_LANS_NT & 1)
   return __builtin_nontemporal_load((const LANCET_GLOBAL f32x4*)(a + k * (4 * kWave) + lane_offset(wave)));
-#else
-  return *(const LANCET_GLOBAL f32x4*)(a + k * (4 * kWave) + lane_offset(wave));
-#endif
 }
-#ifndef LANCET_LANS_NT
-#define LANCET_LANS_NT 3
-#endif
 __device__ __forceinline__ void st_chunk4(LANCET_GLOBAL float* a, int k, f32x4 x, int wave) {
-#if LANCET_LANS_NT & 2
   __builtin_nontemporal_store(x, (LANCET_GLOBAL f32x4*)(a + k * (4 * kWave) + lane_offset(wave)));
-#else
-  *(LANCET_GLOBAL f32x4*)(a + k * (4 * kWave) + lane_offset(wave)) = x;
-#endif
 }
 
 // Thread 0: publishes the N chunk sums a[] of slot s as words first .. first+N-1 (fire and forget).
 template <int N>
 __device__ __forceinline__ void publish(const LansTables& t, const LansScalars& sc, int first, const Slot& s,
                                         const float (&a)[N], bool poison) {
-#if LANCET_LANS_PROBE == 1
-  return;
-#endif
   if (t.debug_flags & 1u) return;  // test hook: nothing is ever published, every wait runs into its bound
   const uint32_t tag = sc.epoch | (poison ? kPoison : 0u);
 #pragma unroll
@@ -628,9 +588,6 @@ __device__ __forceinline__ void moments_chunk(const LansTables& t, const Slot& s
       nm[k % kPrefetch] = ld_chunk4(m, k + kPrefetch, wave);
       nv[k % kPrefetch] = ld_chunk4(v, k + kPrefetch, wave);
     }
-#if LANCET_LANS_SB & 1
-    __builtin_amdgcn_sched_barrier(0);
-#endif
     sh.p[PAR][k][fresh_tid(wave)] = xp;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -651,9 +608,9 @@ __device__ __forceinline__ void moments_chunk(const LansTables& t, const Slot& s
     }
     st_chunk4(m, k, xm, wave);
     st_chunk4(v, k, xv, wave);
-#if LANCET_LANS_SB & 2
-    __builtin_amdgcn_sched_barrier(0);
-#endif
+    // the sums are up to date here: left to itself the compiler keeps every p of the chunk in registers and
+    // adds the squares up at the end of the stage
+    asm volatile("" : "+v"(a0), "+v"(a1), "+v"(a2));
   }
   a[0] = a0;
   a[1] = a1;
@@ -687,7 +644,7 @@ __device__ __noinline__ void regather(const uint64_t* part_word, int nchunks, ui
       lds_barrier();
       return;
     }
-    __builtin_amdgcn_s_sleep(LANCET_LANS_POLL_SLEEP);
+    __builtin_amdgcn_s_sleep(16);
 #pragma unroll 1
     for (uint32_t left = missing; left != 0u; left &= left - 1u) {
       const int bit = __builtin_ctz(left);
@@ -758,7 +715,7 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
                                               f32x4 (&g)[kVecPerThread],
                                               f32x4 (&um_new)[kVecPerThread], f32x4 (&ug_new)[kVecPerThread],
                                               const f32x4 (&um_old)[kVecPerThread], const f32x4 (&ug_old)[kVecPerThread],
-                                              PipeShared& sh, bool align, int wave) {
+                                              PipeShared& sh, int wave) {
   const bool own_norms = t.grad_norms == nullptr;
   // ---- start of the pass ---------------------------------------------------------------------------------
   lds_barrier();
@@ -773,21 +730,7 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
     }
   }
   uint32_t ticket = 0u;  // thread 0: for this pass's stage N
-#ifdef LANCET_LANS_TRACE
-  const uint64_t t_draw = wall_clock64();
-#endif
-  if (is_first(wave)) {
-    // The plan lays a tensor's chunks out inside one round of as many slots as there are workgroups, so that
-    // they are all drawn in the same pass and pass through the stages together.  That holds as long as every
-    // workgroup has made its k-th draw before any makes its (k+1)-th, which the waits see to from the third
-    // pass on; before its second draw a workgroup gives the others a moment to make their first (bounded: a
-    // few microseconds, whether or not they all come).
-    if (UNLIKELY(align)) {
-      const uint32_t everyone = min(static_cast<uint32_t>(gridDim.x), static_cast<uint32_t>(t.nres));
-      for (int spins = 0; spins < 256 && ld_agent(t.ctl + kCtlTicket) < everyone; ++spins) __builtin_amdgcn_s_sleep(8);
-    }
-    ticket = atomicAdd(t.ctl + kCtlTicket, 1u);
-  }
+  if (is_first(wave)) ticket = atomicAdd(t.ctl + kCtlTicket, 1u);
   // ---- stage M on s1 ---------------------------------------------------------------------------------------
   if (LIKELY(s1.real())) {
     float a[3] = {0.f, 0.f, 0.f};
@@ -815,15 +758,11 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
         a[k] = r;
       }
       publish<3>(t, sc, 1, s1, a, bad);
-#ifdef LANCET_LANS_TRACE
-      t.trace[4 * s1.chunk + 1] = wall_clock64();
-#endif
     }
   } else {
     if (is_first(wave)) sh.chunk = static_cast<int>(ticket);
     forget(um_new, ug_new);
   }
-  stage_fence();
   // ---- stage N on a new slot -------------------------------------------------------------------------------
   uint64_t words_g[kGatherPerThread], words_u[3][kGatherPerThread];
   const bool need_u = s0.real();
@@ -850,9 +789,6 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
       }
     }
   }
-#ifdef LANCET_LANS_TRACE
-  if (is_first(wave) && s3.real()) t.trace[4 * s3.chunk + 0] = t_draw;
-#endif
   // g of the chunk into registers (L2NormFunctor, multi_tensor_lans.cu:95-167) and, right behind those loads,
   // the sums other workgroups have published: read as late as possible, and still back before anything waits
   // for them alone
@@ -861,13 +797,11 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
 #pragma unroll
     for (int k = 0; k < kVecPerThread; ++k) g[k] = ld_chunk4(src, k, wave);
   }
-#if LANCET_LANS_PROBE != 1
   if (LIKELY(need_u)) {
 #pragma unroll
     for (int k = 0; k < 3; ++k) gather_issue(t, 1 + k, s0, words_u[k], wave);
   }
   if (LIKELY(need_g)) gather_issue(t, 0, s2, words_g, wave);
-#endif
   if (LIKELY(s3.real())) {
     float a = 0.f;
 #pragma unroll
@@ -875,12 +809,7 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
     a = wave_sum(a);
     if (fresh_lane() == 0) sh.red[0][wave] = a;
   }
-  stage_fence();
   // ---- the norms ---------------------------------------------------------------------------------------------
-#if LANCET_LANS_PROBE == 1
-  if (is_first(wave)) sh.norm[1] = sh.norm[2] = sh.norm[3] = sh.g_next = 1.f;
-  lds_barrier();
-#else
   // bit kind * kGatherPerThread + i: word i of this thread's share of that norm's sums is still missing
   uint32_t missing = 0u;
   {
@@ -892,14 +821,8 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
     if (LIKELY(need_g)) gather_take(sc, s2, words_g, sh.part[0], 0, missing, poisoned_g, wave);
     if (UNLIKELY(poisoned_u)) sh.u_bad = 1;
     if (UNLIKELY(poisoned_g)) sh.g_next_bad = 1;
-#if LANCET_LANS_PROBE == 2
-    missing = 0u;  // timing experiment: nobody waits
-#endif
     if (UNLIKELY(missing != 0u)) sh.retry = 1;
   }
-#ifdef LANCET_LANS_TRACE
-  if (is_first(wave) && need_u) t.trace[4 * s0.chunk + 2] = wall_clock64();
-#endif
   lds_barrier();
   if (is_first(wave) && s3.real() && own_norms) {
     float r = 0.f;
@@ -914,22 +837,8 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
   // once any wait of the plan has given up the others stop at their next look, so that a stalled step ends
   // after about one bound, not one per chunk.
   if (UNLIKELY(__builtin_amdgcn_readfirstlane(sh.retry) != 0)) {
-#ifdef LANCET_LANS_DIAG
-    if (missing & ((1u << kGatherPerThread) - 1u)) sh.diag[0] = 1;
-    if (missing >> kGatherPerThread) sh.diag[1] = 1;
-    lds_barrier();
-    if (is_first(wave)) {
-      atomicAdd(t.ctl + 3, 1u);
-      if (sh.diag[0]) atomicAdd(t.ctl + 4, 1u);
-      if (sh.diag[1]) atomicAdd(t.ctl + 5, 1u);
-      sh.diag[0] = sh.diag[1] = 0;
-    }
-#endif
     regather(t.part_word, t.nchunks, t.ctl, t.host_status, sc.epoch, sc.spin_limit, s2.lo, s0.lo, missing, &sh, wave);
   }
-#ifdef LANCET_LANS_TRACE
-  if (is_first(wave) && need_u) t.trace[4 * s0.chunk + 3] = wall_clock64();
-#endif
   {
     const int w = wave;  // wave w sums norm w: the same fixed order in every workgroup
     if (w == 0) {
@@ -949,8 +858,6 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
     }
   }
   lds_barrier();
-#endif
-  stage_fence();
   // ---- stage U on s0 ---------------------------------------------------------------------------------------
   // Trust ratios and the parameter update (LANSStage2Functor, multi_tensor_lans.cu:326-399) from the updates
   // in registers and the parameters in LDS.  Nothing is written unless all three norms are known.
@@ -972,7 +879,6 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
       st_chunk4(p, k, xp, wave);
     }
   }
-  stage_fence();
   // ---- the slots move up ------------------------------------------------------------------------------------
   s0 = s1;
   s1 = s2;
@@ -980,21 +886,16 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
   return s0.chunk >= 0 || s1.chunk >= 0 || s2.chunk >= 0;
 }
 
-#ifndef LANCET_LANS_KATTR
-#define LANCET_LANS_KATTR
-#endif
-#ifndef LANCET_LANS_WAVES
-#define LANCET_LANS_WAVES 2
-#endif
 // Workgroups per CU = waves per SIMD: with two, a wave has 256 registers for g of two chunks, u_m and u_g of
 // two more (one of them being filled from the first g) and the sums read ahead, and a workgroup 64 KB of
 // LDS for parameters.
-constexpr int kResidentWavesPerSimd = LANCET_LANS_WAVES;
+constexpr int kResidentWavesPerSimd = 2;
 
-// Start of a resident step: clears the ticket and moves the step epoch on.  The epoch lives on the device so
+// Start of a resident step: clears the ticket, moves the step epoch on and forms the two bias corrections
+// (pow in double: kept out of the resident kernel, whose registers are all spoken for).  The epoch lives on the device so
 // that a step recorded in a graph tags every replay differently; when it wraps (2^31 steps) every word of
 // earlier steps is forgotten.  The error word is left alone.
-__global__ __launch_bounds__(kLansThreads) void lans_begin_kernel(LansTables t, size_t nwords) {
+__global__ __launch_bounds__(kLansThreads) void lans_begin_kernel(LansTables t, LansScalars sc, size_t nwords) {
   uint32_t* ep = t.ctl + kCtlEpoch;
   const uint32_t e = (*ep + 1u) & ~kPoison;
   if (e == 0u)
@@ -1003,17 +904,15 @@ __global__ __launch_bounds__(kLansThreads) void lans_begin_kernel(LansTables t, 
   if (threadIdx.x == 0) {
     *ep = e == 0u ? 1u : e;
     t.ctl[kCtlTicket] = 0u;
+    bias_corrections(sc, t.consts[0], t.consts[1]);
   }
 }
 
-__global__ __launch_bounds__(kLansThreads, kResidentWavesPerSimd) LANCET_LANS_KATTR void lans_resident_kernel(LansTables t, LansScalars sc) {
+__global__ __launch_bounds__(kLansThreads, kResidentWavesPerSimd) void lans_resident_kernel(LansTables t, LansScalars sc) {
   __shared__ PipeShared sh;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x) / kWave;
+  const int wave = static_cast<int>(static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(threadIdx.x)) / kWave);
   sc.epoch = __builtin_amdgcn_readfirstlane(t.ctl[kCtlEpoch]);
-  float bc1, bc2;
-  bias_corrections(sc, bc1, bc2);
-  bc1 = uniform(bc1);
-  bc2 = uniform(bc2);
+  const float bc1 = uniform(t.consts[0]), bc2 = uniform(t.consts[1]);  // lans_begin_kernel
   // s0: between stages M and U; s1, s2: between stages N and M, s1 the older.  Register arrays rotate with
   // the slots: g of s1 / s2 alternates between ga and gb, the updates between parity 0 and 1.
   f32x4 ga[kVecPerThread], gb[kVecPerThread];
@@ -1026,15 +925,12 @@ __global__ __launch_bounds__(kLansThreads, kResidentWavesPerSimd) LANCET_LANS_KA
     sh.g_next = 0.f;
     sh.g_next_bad = 0;
     sh.give_up = 0;
-#ifdef LANCET_LANS_DIAG
-    sh.diag[0] = sh.diag[1] = 0;
-#endif
   }
   // the first two passes find empty slots (their stages M and U have nothing to do) and fill the pipeline;
   // every pass draws a ticket, tickets run out, and every wait is bounded: all workgroups leave
-  for (int pair = 0;; ++pair) {
-    if (!pipeline_pass<0>(t, sc, bc1, bc2, s0, s1, s2, ga, um0, ug0, um1, ug1, sh, false, wave)) break;
-    if (!pipeline_pass<1>(t, sc, bc1, bc2, s0, s1, s2, gb, um1, ug1, um0, ug0, sh, pair == 0 && LANCET_LANS_ALIGN != 0, wave)) break;
+  for (;;) {
+    if (!pipeline_pass<0>(t, sc, bc1, bc2, s0, s1, s2, ga, um0, ug0, um1, ug1, sh, wave)) break;
+    if (!pipeline_pass<1>(t, sc, bc1, bc2, s0, s1, s2, gb, um1, ug1, um0, ug0, sh, wave)) break;
   }
 }
 
@@ -1231,9 +1127,6 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
     t.nchunks = pl->nchunks;
     t.nres = pl->n_res_chunks;
     t.debug_flags = 0u;
-#ifdef LANCET_LANS_TRACE
-    t.trace = nullptr;
-#endif
   }
   if (err != hipSuccess) {
     lancet_lans_plan_destroy(pl);
@@ -1328,12 +1221,6 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
   sc.bias_correction = h->bias_correction;
   sc.step_host = step_host;
   sc.step_dev = step_dev;
-#ifdef LANCET_LANS_TRACE
-  if (!pl->tables.trace) {
-    (void)hipMalloc(&pl->tables.trace, 4 * sizeof(uint64_t) * static_cast<size_t>(pl->tables.nres + 1));
-    (void)hipMemset(pl->tables.trace, 0, 4 * sizeof(uint64_t) * static_cast<size_t>(pl->tables.nres + 1));
-  }
-#endif
   LansTables t = pl->tables;
   t.grad_norms = grad_norms;
   sc.spin_limit = pl->spin_limit;
@@ -1343,7 +1230,7 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
   // (everything, under the sweeps schedule) through the three sweeps
   int chunk_base = 0, tensor_base = 0;
   if (pl->schedule == LANCET_LANS_RESIDENT && pl->n_res_chunks > 0 && aligned16) {
-    lans_begin_kernel<<<1, kLansThreads, 0, st>>>(t, pl->words_bytes / sizeof(uint64_t));
+    lans_begin_kernel<<<1, kLansThreads, 0, st>>>(t, sc, pl->words_bytes / sizeof(uint64_t));
     const int grid = std::min(pl->resident_grid, pl->n_res_chunks);
     lans_resident_kernel<<<grid, kLansThreads, 0, st>>>(t, sc);
     chunk_base = pl->n_res_chunks;
@@ -1353,7 +1240,7 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
   if (nsweep > 0) {
     const int per_block = kLansThreads / kWave;
     const int rblocks = (T - tensor_base + per_block - 1) / per_block;
-    lans_prepare_kernel<<<1, 64, 0, st>>>(t, sc);
+    if (chunk_base == 0) lans_prepare_kernel<<<1, 64, 0, st>>>(t, sc);  // the bias corrections
     if (!grad_norms) {
       lans_norm_g_kernel<<<nsweep, kLansThreads, 0, st>>>(t, chunk_base);
       lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 0, tensor_base, T, 1, 1);
@@ -1387,29 +1274,6 @@ extern "C" int lancet_lans_plan_error(lancet_lans_plan_t pl, lancet_stream_t str
   if (!error_out) return LANCET_ERR_NULL;
   uint32_t word = 0;
   hipStream_t st = static_cast<hipStream_t>(stream);
-#ifdef LANCET_LANS_TRACE
-  if (const char* path = getenv("LANCET_TRACE_FILE")) {
-    (void)hipDeviceSynchronize();
-    const int n = pl->tables.nres;
-    std::vector<int32_t> ct(n);
-    std::vector<uint64_t> tr(4 * static_cast<size_t>(n));
-    (void)hipMemcpy(ct.data(), pl->tables.chunk_tensor, n * sizeof(int32_t), hipMemcpyDeviceToHost);
-    (void)hipMemcpy(tr.data(), pl->tables.trace, tr.size() * sizeof(uint64_t), hipMemcpyDeviceToHost);
-    if (FILE* f = fopen(path, "wb")) {
-      fwrite(&n, sizeof(n), 1, f);
-      fwrite(ct.data(), sizeof(int32_t), n, f);
-      fwrite(tr.data(), sizeof(uint64_t), tr.size(), f);
-      fclose(f);
-    }
-  }
-#endif
-#ifdef LANCET_LANS_DIAG
-  {
-    uint32_t w[8];
-    (void)hipMemcpy(w, pl->tables.ctl, sizeof(w), hipMemcpyDeviceToHost);
-    fprintf(stderr, "[diag] retries %u (g missing %u, u missing %u; all steps so far), passes per step ~%d\n", w[3], w[4], w[5], pl->tables.nres);
-  }
-#endif
   hipError_t e = hipMemcpyAsync(&word, pl->tables.ctl + kCtlError, sizeof(word), hipMemcpyDeviceToHost, st);
   if (e == hipSuccess) e = hipStreamSynchronize(st);
   // the reader, and only the reader, clears the error (the steps on `stream` have finished)

@@ -354,27 +354,34 @@ int lancet_lans_step(lancet_lans_plan_t plan, const float* const* g, float* cons
  * replay is a new step.  The pointer tables are uploaded (one host-to-device copy) by the first call that
  * sees a new set of pointers: make that call once before recording. */
 /* Schedules of the step.
- * LANCET_LANS_SWEEPS (default): three whole-state sweeps with two per-tensor reductions between them
- * (48 B/param of traffic).  No workgroup waits for another.
- * LANCET_LANS_RESIDENT: one persistent kernel that reads and writes every array once (28 B/param): each
- * workgroup runs a three-stage pipeline over chunks of 8192 parameters and keeps a chunk on chip between the
- * stages, for the tensors of at most lancet_lans_plan_resident_capacity() chunks; larger tensors of the plan
- * take the three sweeps in the same step, and a plan with no tensor that fits gets LANCET_ERR_SHAPE from
- * set_schedule and keeps its schedule.  Contract of this schedule: its workgroups wait for one another (for
- * chunks of the same tensor only), so at least half of them must be running on the device at the same time.
- * The grid is sized to what an otherwise idle device runs at once; other kernels on the device delay the
- * step until enough of its workgroups have started, and only something that keeps the device occupied
- * without end (e.g. another kernel that itself waits for this step) can stall it.  Every wait is bounded:
- * a wait that gives up leaves the parameters of the tensors concerned unwritten (their m and v may already
- * hold the new moments), sets the plan's sticky error, and the NEXT lancet_lans_step on the plan returns
- * LANCET_ERR_STALLED without launching anything, until lancet_lans_plan_error has been called.
+ * LANCET_LANS_RESIDENT (what a new plan has when at least one tensor fits it): one persistent kernel that
+ * reads and writes every array once (28 B/param).  Each workgroup runs a three-stage pipeline over chunks of
+ * 8192 parameters (sum of g^2 / moments and the two updates / parameter write) and keeps a chunk on chip
+ * between the stages; it publishes the sums of its chunks and forms the norms it needs from the published
+ * sums of all the tensor's chunks.  The kernel takes the tensors that are whole multiples of 8192
+ * parameters and have at most lancet_lans_plan_resident_capacity() chunks; the other tensors of the plan
+ * take the three sweeps in the same step, and so does every tensor of a step in which an array of a tensor
+ * the kernel would take is not 16-byte aligned.
+ * Contract of this schedule: its workgroups wait for one another (for chunks of the same tensor only), so
+ * at least half of them must be running on the device at the same time.  The grid is sized to what an
+ * otherwise idle device runs at once; other kernels on the device delay the step until enough of its
+ * workgroups have started, and only something that keeps the device occupied without end (e.g. another
+ * kernel that itself waits for this step) can stall it.  Every wait is bounded: a wait that gives up leaves
+ * the parameters of the tensors concerned unwritten (their m and v may already hold the new moments), sets
+ * the plan's sticky error, and the NEXT lancet_lans_step on the plan returns LANCET_ERR_STALLED without
+ * launching anything, until lancet_lans_plan_error has been called.
+ * LANCET_LANS_SWEEPS: three whole-state sweeps with two per-tensor reductions between them (48 B/param of
+ * traffic).  No workgroup waits for another: the schedule for a device that is shared with kernels of
+ * unbounded duration.  set_schedule(LANCET_LANS_RESIDENT) on a plan with no tensor that fits returns
+ * LANCET_ERR_SHAPE and the plan keeps the sweeps.
  * Each schedule is deterministic; the two agree to fp32 rounding of the per-chunk sums. */
 #define LANCET_LANS_SWEEPS 0
 #define LANCET_LANS_RESIDENT 1
 int lancet_lans_plan_set_schedule(lancet_lans_plan_t plan, int schedule);
 /* workgroups: chunks (of 8192 parameters) of the largest tensor the resident kernel takes on this device
- * (larger tensors of the plan go through the sweeps); max_tensor_chunks: chunks of the plan's largest
- * tensor.  Either may be NULL. */
+ * (larger tensors of the plan go through the sweeps; 512 = 4M parameters on a device that runs 512 of the
+ * kernel's workgroups at once); max_tensor_chunks: chunks of the plan's largest tensor.  Either may be
+ * NULL. */
 int lancet_lans_plan_resident_capacity(lancet_lans_plan_t plan, int* workgroups, int* max_tensor_chunks);
 /* Reads (synchronising `stream`) and clears the plan's sticky error: 1 when a bounded wait of the resident
  * schedule gave up in any step since the last call. */

@@ -20,11 +20,16 @@ extern "C" {
 int64_t lancet_lans_debug_chunk_table(const int64_t* numels, int T, int resident_limit, int round,
                                       int32_t* chunk_tensor_out, int64_t capacity, int64_t* n_resident_chunks);
 
-/* Test hook of one plan: spin_limit = polls a workgroup of the resident schedule waits for a word before it
- * gives up (0 restores the default); flags bit 0: the workgroup that sums a tensor's partials withholds the
- * norms, so that every wait for them runs into the limit.  Lets a host test exercise the bounded waits and the
- * error path while every kernel still exits normally. */
+/* Test hook of one plan: spin_limit = times a workgroup of the resident schedule reads again the chunk sums it
+ * misses before it gives up (0 restores the default); flags bit 0: no workgroup publishes its chunk sums, so
+ * that every wait for them runs into the limit.  Lets a host test exercise the bounded waits and the error
+ * path while every kernel still exits normally. */
 int lancet_lans_plan_debug(lancet_lans_plan_t plan, unsigned spin_limit, unsigned flags);
+
+/* *slots = chunk slots the resident kernel handed out in the plan's last lancet_lans_step, 0 when that step
+ * went through the sweeps alone (schedule, no tensor that fits, or a resident tensor whose arrays were not
+ * 16-byte aligned).  Lets a test tell which kernels it has exercised. */
+int lancet_lans_plan_debug_last_resident(lancet_lans_plan_t plan, int* slots);
 
 /* Test hook: number of polls a workgroup of the position scan waits for a predecessor
  * before it gives up, flags the workspace and finishes with undefined results

@@ -92,6 +92,7 @@ SIGNATURES = {
     "lancet_lans_plan_error": (_int, [_vp, _vp, C.POINTER(_int)]),
     "lancet_lans_debug_chunk_table": (_i64, [C.POINTER(_i64), _int, _int, _int, _vp, _i64, C.POINTER(_i64)]),
     "lancet_lans_plan_debug": (_int, [_vp, _u32, _u32]),
+    "lancet_lans_plan_debug_last_resident": (_int, [_vp, C.POINTER(_int)]),
     "lancet_lans_plan_resident_capacity": (_int, [_vp, C.POINTER(_int), C.POINTER(_int)]),
     "lancet_debug_set_spin_limit": (None, [_u32]),
     "lancet_scan_workspace_error": (_int, [_vp, _vp, C.POINTER(_int)]),

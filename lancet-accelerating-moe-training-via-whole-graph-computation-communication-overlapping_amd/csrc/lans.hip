@@ -961,8 +961,10 @@ struct lancet_lans_plan {
   int n_res_tensors;      // tensors within that limit: the first ones in the plan's own order
   int n_res_chunks;       // chunk slots the resident kernel hands out (padding included)
   std::vector<int32_t> order;  // plan position -> position in the caller's lists
+  std::vector<char> is_resident;  // by position in the caller's lists: the resident kernel takes this tensor
   size_t words_bytes;
   uint32_t spin_limit;
+  int last_resident_slots;  // chunk slots the resident kernel of the last step handed out (0: it did not run)
 };
 
 static constexpr uint32_t kPlanMagic = 0x4c414e53u;  // "LANS"
@@ -1049,7 +1051,8 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
   pl->upload_done = nullptr;
   pl->upload_pending = false;
   pl->spin_limit = kDefaultSpinLimit;
-  pl->schedule = LANCET_LANS_SWEEPS;
+  pl->schedule = LANCET_LANS_SWEEPS;  // until the layout below says that the resident kernel has something to take
+  pl->last_resident_slots = 0;
   hipError_t err = hipGetDevice(&pl->device);
   int cus = 256;
   if (err == hipSuccess) err = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, pl->device);
@@ -1069,6 +1072,9 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
   pl->n_res_tensors = L.n_fit;
   pl->n_res_chunks = L.n_res_slots;
   pl->nchunks = static_cast<int>(L.ctensor.size());
+  if (pl->n_res_chunks > 0) pl->schedule = LANCET_LANS_RESIDENT;
+  pl->is_resident.assign(T, 0);
+  for (int k = 0; k < pl->n_res_tensors; ++k) pl->is_resident[pl->order[k]] = 1;
   // device block layout
   const size_t n = static_cast<size_t>(pl->nchunks);
   const size_t n1 = n ? n : 1;
@@ -1174,13 +1180,13 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
   const int T = pl->T;
   hipStream_t st = static_cast<hipStream_t>(stream);
   bool changed = false;
-  bool aligned16 = true;  // the resident kernel moves float4s: a step with a tensor that is not 16-byte aligned runs as sweeps
+  bool aligned16 = true;  // the resident kernel moves float4s: a step in which one of its tensors is not 16-byte aligned runs as sweeps
   for (int i = 0; i < T; ++i) {
     if (pl->numels[i] > 0 && (!g[i] || !p[i] || !m[i] || !v[i])) return LANCET_ERR_NULL;
     const uintptr_t bits = reinterpret_cast<uintptr_t>(g[i]) | reinterpret_cast<uintptr_t>(p[i]) |
                            reinterpret_cast<uintptr_t>(m[i]) | reinterpret_cast<uintptr_t>(v[i]);
     if (bits & 3u) return LANCET_ERR_ALIGN;
-    aligned16 = aligned16 && (bits & 15u) == 0;
+    aligned16 = aligned16 && (!pl->is_resident[i] || (bits & 15u) == 0);
     changed = changed || pl->shadow[i] != g[i] || pl->shadow[T + i] != p[i] ||
               pl->shadow[2 * T + i] != m[i] || pl->shadow[3 * T + i] != v[i];
   }
@@ -1229,12 +1235,14 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
   // slots [0, chunk_base) and tensors [0, tensor_base) go through the resident kernel, the rest
   // (everything, under the sweeps schedule) through the three sweeps
   int chunk_base = 0, tensor_base = 0;
+  pl->last_resident_slots = 0;
   if (pl->schedule == LANCET_LANS_RESIDENT && pl->n_res_chunks > 0 && aligned16) {
     lans_begin_kernel<<<1, kLansThreads, 0, st>>>(t, sc, pl->words_bytes / sizeof(uint64_t));
     const int grid = std::min(pl->resident_grid, pl->n_res_chunks);
     lans_resident_kernel<<<grid, kLansThreads, 0, st>>>(t, sc);
     chunk_base = pl->n_res_chunks;
     tensor_base = pl->n_res_tensors;
+    pl->last_resident_slots = chunk_base;
   }
   const int nsweep = t.nchunks - chunk_base;
   if (nsweep > 0) {
@@ -1285,6 +1293,13 @@ extern "C" int lancet_lans_plan_error(lancet_lans_plan_t pl, lancet_stream_t str
   }
   *error_out = static_cast<int>(word);
   return static_cast<int>(e);
+}
+
+extern "C" int lancet_lans_plan_debug_last_resident(lancet_lans_plan_t pl, int* slots) {
+  if (!pl || pl->magic != kPlanMagic) return LANCET_ERR_PLAN;
+  if (!slots) return LANCET_ERR_NULL;
+  *slots = pl->last_resident_slots;
+  return LANCET_OK;
 }
 
 extern "C" int lancet_lans_plan_debug(lancet_lans_plan_t pl, unsigned spin_limit, unsigned flags) {

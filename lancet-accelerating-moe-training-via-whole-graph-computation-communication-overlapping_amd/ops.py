@@ -539,7 +539,8 @@ class LansPlan:
             self.set_schedule(schedule)
 
     def set_schedule(self, schedule):
-        """capi.LANS_SWEEPS (default) or capi.LANS_RESIDENT (raises when a tensor is too large for it)."""
+        """capi.LANS_RESIDENT (what a new plan has when a tensor fits the resident kernel; raises on a plan
+        with no such tensor) or capi.LANS_SWEEPS (no workgroup waits for another)."""
         capi.check(self._lib.lancet_lans_plan_set_schedule(self._h, int(schedule)), "lancet_lans_plan_set_schedule")
 
     def resident_capacity(self):
@@ -556,8 +557,16 @@ class LansPlan:
         return err.value
 
     def debug(self, spin_limit=0, flags=0):
-        """Test hook (include/lancet_hip_debug.h): bound of the resident schedule's waits, bit 0 = withhold norms."""
+        """Test hook (include/lancet_hip_debug.h): bound of the resident schedule's waits, bit 0 = nothing
+        is published."""
         capi.check(self._lib.lancet_lans_plan_debug(self._h, int(spin_limit), int(flags)), "lancet_lans_plan_debug")
+
+    def last_resident_slots(self):
+        """Test hook: chunk slots the resident kernel took in the last step (0: sweeps only)."""
+        n = C.c_int(-1)
+        capi.check(self._lib.lancet_lans_plan_debug_last_resident(self._h, C.byref(n)),
+                   "lancet_lans_plan_debug_last_resident")
+        return n.value
 
     def close(self):
         if self._h is not None:
@@ -614,11 +623,9 @@ def lans(tensor_list, step, learning_rate, beta1, beta2, eps, bias_correction, w
     plan = _PLANS.get(key)
     if plan is None:
         plan = _PLANS[key] = LansPlan(key[0])
-        if os.environ.get("LANCET_LANS_SCHEDULE") == "resident":
-            try:
-                plan.set_schedule(capi.LANS_RESIDENT)
-            except RuntimeError:      # a tensor too large for it: the three sweeps stay
-                pass
+        # LANCET_LANS_SCHEDULE=sweeps: for a device this process shares with kernels of unbounded duration
+        if os.environ.get("LANCET_LANS_SCHEDULE") == "sweeps":
+            plan.set_schedule(capi.LANS_SWEEPS)
     hyper = capi.LansHyper(float(learning_rate), float(beta1), float(beta2), float(eps), int(bias_correction),
                            float(weight_decay), int(grad_averaging), int(mode), int(bool(normalize_grad)))
     if torch.is_tensor(step):

@@ -56,10 +56,10 @@ class LansImpl : public OpEnv {
     device_id_ = t0.device_id;
     int st = lancet_lans_plan_create(numels_.data(), param_group_n_, &plan_);
     if (st != LANCET_OK) throw Error(std::string("lancet_lans_plan_create failed: ") + lancet_status_string(st));
-    // LANCET_LANS_SCHEDULE=resident asks for the one-kernel schedule; a parameter set with a tensor too
-    // large for it keeps the three sweeps
+    // a new plan runs the one-kernel schedule for every tensor that fits it; LANCET_LANS_SCHEDULE=sweeps
+    // asks for the three sweeps (a device shared with kernels of unbounded duration)
     const char* schedule = std::getenv("LANCET_LANS_SCHEDULE");
-    if (schedule && std::strcmp(schedule, "resident") == 0) (void)lancet_lans_plan_set_schedule(plan_, LANCET_LANS_RESIDENT);
+    if (schedule && std::strcmp(schedule, "sweeps") == 0) (void)lancet_lans_plan_set_schedule(plan_, LANCET_LANS_SWEEPS);
     this->arg_indices = {0, 1};  // tensor_list, step
   }
 

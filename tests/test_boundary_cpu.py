@@ -221,41 +221,30 @@ def _chunk_table(pkg, numels, limit=1 << 30, round_=1 << 30):
     return ctensor[:n], nres.value
 
 
-def _simulate_resident(ctensor, workers, rng, pay_before_waiting=True):
+def _simulate_resident(ctensor, workers, rng, publish=True):
     """The resident LANS kernel as a state machine.  Every workgroup runs passes of
-        [N duty] M(s1) [M duty if s0 and s1 share a tensor] U(s0) rotate [M duty] N(new s2)
-    on the chunk slots it draws in ticket order (the first two passes find s0 and s1 empty).  Stage N draws a
-    slot and counts it in at its tensor; the workgroup whose arrival completes a tensor owes it the norm and
-    pays at the next duty point of its own program.  Stage M of a slot needs the norm of stage N of its tensor,
-    stage U the norm of stage M.  Padding slots (-1) pass every stage at once.  Workgroups are advanced in
-    random order.  Returns True when every chunk has been through U, False when no workgroup can move.
-    pay_before_waiting=False moves the duties behind the waits (a workgroup that holds two chunks of a tensor
-    then waits for a norm it owes itself)."""
+        draw a slot | M(s1), publish its three sums | N(drawn slot), publish its sum of g^2 |
+        wait for the M sums of every chunk of s0's tensor and the N sums of every chunk of s2's | U(s0) | rotate
+    on the chunk slots it draws in ticket order (s0 <- s1 <- s2 <- drawn; the first two passes find s0 and s1
+    empty).  Stage M of a slot needs no wait of its own: the norm of its tensor was formed at the wait of the
+    pass before, when the slot was s2.  Padding slots (-1) pass every stage at once.  Only `workers`
+    workgroups run (the others never get onto the chip and draw nothing); they are advanced in random
+    order.  Returns True when every chunk has been through U, False when no workgroup can move (on the
+    device: the bounded waits give up).  publish=False: the test hook that withholds every sum."""
     n = len(ctensor)
     real = ctensor[ctensor >= 0]
     size = np.bincount(real, minlength=int(real.max()) + 1 if len(real) else 1)
-    arrived = [np.zeros_like(size), np.zeros_like(size)]     # stage N, stage M
-    ready = [np.zeros(len(size), bool), np.zeros(len(size), bool)]
+    sums_n, sums_m = np.zeros_like(size), np.zeros_like(size)
     state = {"ticket": 0, "done": 0}
 
     class WG:
         def __init__(self):
             self.s = [None, None, None]
-            self.owes = [None, None]       # tensor whose stage-N / stage-M norm this workgroup has to form
-            self.pc = 0
+            self.drawn = None
+            self.waiting = False
 
     def is_real(x):
         return x is not None and x >= 0
-
-    def arrive(w, stage, tensor):
-        arrived[stage][tensor] += 1
-        if arrived[stage][tensor] == size[tensor]:
-            w.owes[stage] = tensor
-
-    def pay(w, stage):
-        if w.owes[stage] is not None:
-            ready[stage][w.owes[stage]] = True
-            w.owes[stage] = None
 
     wgs = [WG() for _ in range(workers)]
     live = set(range(workers))
@@ -264,36 +253,24 @@ def _simulate_resident(ctensor, workers, rng, pay_before_waiting=True):
         for i in rng.permutation(sorted(live)):
             w = wgs[i]
             s0, s1, s2 = w.s
-            if w.pc == 0:                                   # stage M on s1
-                if pay_before_waiting:
-                    pay(w, 0)
-                if not is_real(s1) or ready[0][s1]:
-                    pay(w, 0)
-                    if is_real(s1):
-                        arrive(w, 1, s1)
-                    w.pc = 1
-                    moved = True
-            elif w.pc == 1:                                 # stage U on s0
-                if pay_before_waiting and is_real(s0) and s0 == s1:
-                    pay(w, 1)
-                if not is_real(s0) or ready[1][s0]:
-                    if is_real(s0):
-                        state["done"] += 1
-                    w.pc = 2
-                    moved = True
-            else:                                           # the slots move up, stage N draws a slot
-                pay(w, 1)
-                drawn = None
+            if not w.waiting:                               # draw, stage M on s1, stage N on the drawn slot
+                w.drawn = None
                 if state["ticket"] < n:
-                    drawn = int(ctensor[state["ticket"]])
+                    w.drawn = int(ctensor[state["ticket"]])
                     state["ticket"] += 1
-                    if drawn >= 0:
-                        arrive(w, 0, drawn)
-                w.s = [s1, s2, drawn]
-                w.pc = 0
+                if publish and is_real(s1):
+                    sums_m[s1] += 1
+                if publish and is_real(w.drawn):
+                    sums_n[w.drawn] += 1
+                w.waiting = True
+                moved = True
+            elif (not is_real(s0) or sums_m[s0] == size[s0]) and (not is_real(s2) or sums_n[s2] == size[s2]):
+                if is_real(s0):                             # stage U on s0
+                    state["done"] += 1
+                w.s = [s1, s2, w.drawn]
+                w.waiting = False
                 moved = True
                 if all(x is None for x in w.s):
-                    pay(w, 0)
                     live.discard(i)
         if not moved:
             return False
@@ -303,53 +280,57 @@ def _simulate_resident(ctensor, workers, rng, pay_before_waiting=True):
 @pytest.mark.parametrize("case", ["config5", "random", "tiny"])
 def test_lans_resident_schedule_drains(pkg, case):
     """A workgroup of the resident schedule waits only for chunks of tensors it holds, slots are handed out in
-    order, and a workgroup holds at most two slots that have not passed stage M: the kernel drains whenever the
-    running workgroups are at least half the chunks of the largest tensor, and stalls with fewer."""
+    order, and a workgroup has drawn two slots by the time it first waits for one of them: the kernel drains
+    whenever the running workgroups are at least half the chunks of the largest tensor, and stalls with fewer
+    (and always when nothing is published)."""
     import bench
     rng = np.random.default_rng(0)
     if case == "config5":
         numels = [int(np.prod(s)) for s in bench.lans_shapes()][:40]
     elif case == "random":
-        numels = [int(x) for x in rng.integers(0, 600_000, 60)] + [0, 1, 8192, 8193]
+        numels = [int(x) * 8192 for x in rng.integers(0, 70, 60)] + [0, 1, 8192, 8193, 70 * 8192 - 1]
     else:
-        numels = [1, 2, 3]
+        numels = [8192, 2 * 8192, 3 * 8192]
     chunks = [(x + 8191) // 8192 for x in numels]
-    largest = max(chunks)
+    whole = [i for i, x in enumerate(numels) if x % 8192 == 0]
+    largest = max(chunks[i] for i in whole)
     for round_ in (largest, largest + 3, 4 * largest):
         ctensor, nres = _chunk_table(pkg, numels, largest, round_)
-        assert len(ctensor) == nres
         real = ctensor[ctensor >= 0]
         np.testing.assert_array_equal(np.bincount(real, minlength=len(numels)), chunks)   # every chunk exactly once
-        assert (np.diff(np.flatnonzero(np.diff(real) != 0)) > 0).all()
-        for i in set(real.tolist()):                      # chunks of a tensor are consecutive slots of ONE round
-            where = np.flatnonzero(ctensor == i)
+        res = ctensor[:nres]
+        # the kernel takes the tensors that are whole chunks (and fit); the others follow, without padding
+        assert set(res[res >= 0].tolist()) == {i for i in whole if chunks[i] > 0}
+        assert (ctensor[nres:] >= 0).all()
+        for i in set(res[res >= 0].tolist()):             # chunks of a tensor are consecutive slots of ONE round
+            where = np.flatnonzero(res == i)
             assert where[-1] - where[0] + 1 == len(where) and where[0] // round_ == where[-1] // round_
-        sizes = [chunks[i] for i in dict.fromkeys(real.tolist())]
+        sizes = [chunks[i] for i in dict.fromkeys(res[res >= 0].tolist())]
         assert sizes == sorted(sizes, reverse=True)       # largest tensors first
         for workers in ((largest + 1) // 2, round_, round_ + 5):
-            assert _simulate_resident(ctensor, workers, rng)
+            assert _simulate_resident(res, workers, rng)
+    ctensor, nres = _chunk_table(pkg, numels, largest, largest)
     if largest > 2:
-        ctensor, _ = _chunk_table(pkg, numels, largest, largest)
-        assert not _simulate_resident(ctensor, (largest + 1) // 2 - 1, rng)
-        # a workgroup that held two chunks of one tensor would wait for a norm it owes itself
-        assert not _simulate_resident(ctensor, (largest + 1) // 2, rng, pay_before_waiting=False)
+        assert not _simulate_resident(ctensor[:nres], (largest + 1) // 2 - 1, rng)
+    assert not _simulate_resident(ctensor[:nres], largest, rng, publish=False)
 
 
 def test_lans_plan_orders_tensors_that_do_not_fit_last(pkg):
-    """Tensors with more chunks than the resident kernel takes come after all the others in the plan's
-    slot order, without padding, and are left to the sweeps; every chunk of every tensor appears exactly once."""
-    numels = [100, 5 * 8192, 8192 * 40 + 1, 3, 8192 * 41, 8192 * 40, 0, 7 * 8192]
+    """Tensors with more chunks than the resident kernel takes, or that are not whole chunks, come after all
+    the others in the plan's slot order, without padding, and are left to the sweeps; every chunk of every
+    tensor appears exactly once."""
+    numels = [8192, 5 * 8192, 8192 * 40 + 1, 8192, 8192 * 41, 8192 * 40, 0, 7 * 8192, 100]
     limit = 40
     ctensor, nres = _chunk_table(pkg, numels, limit, limit)
     chunks = [(n + 8191) // 8192 for n in numels]
     real = ctensor[ctensor >= 0]
     np.testing.assert_array_equal(np.bincount(real, minlength=len(numels)), chunks)
-    fits = [i for i, c in enumerate(chunks) if c <= limit]
+    fits = [i for i, n in enumerate(numels) if n % 8192 == 0 and chunks[i] <= limit]
     assert set(ctensor[:nres]) - {-1} == {i for i in fits if chunks[i] > 0}
     # rounds of 40 slots: [tensor 5 (40)] [tensor 7 (7), tensor 1 (5), tensors 0 and 3 (1 each)]: no padding needed
     assert nres == sum(chunks[i] for i in fits) and (ctensor[:nres] >= 0).all()
     assert list(dict.fromkeys(ctensor[:nres])) == [5, 7, 1, 0, 3]
-    assert list(dict.fromkeys(ctensor[nres:])) == [2, 4] and (ctensor[nres:] >= 0).all()   # list order, no padding
+    assert list(dict.fromkeys(ctensor[nres:])) == [2, 4, 8] and (ctensor[nres:] >= 0).all()   # list order, no padding
     assert _simulate_resident(ctensor[:nres], limit, np.random.default_rng(1))
     # a tensor that does not fit into what is left of a round starts the next one
     ctensor, nres = _chunk_table(pkg, [3 * 8192, 3 * 8192, 3 * 8192], 4, 4)

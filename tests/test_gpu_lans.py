@@ -128,34 +128,109 @@ def test_lans_norms_and_plan_reuse(pkg):
     plan.close()
 
 
+def _fresh_state(numels, seed, offset=0):
+    """g, p, m, v as lists of separately allocated (so 16-byte aligned) tensors; with `offset`, every tensor is
+    a view that starts `offset` elements into its allocation."""
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    def alloc(n, std):
+        t = torch.zeros(n + offset, device="cuda")
+        if std:
+            t.normal_(0, std, generator=gen)
+        return t[offset:]
+    return [[alloc(n, std) for n in numels] for std in (1e-3, 0.02, 0, 0)]
+
+
 def test_lans_resident_schedule(pkg):
-    """The opt-in persistent-kernel schedule must terminate, leave its error word clear, be reproducible and
-    agree with the default three-sweep schedule to fp32 rounding of the per-chunk sums (whole and partial
-    chunks, tensors of one chunk and of many, an unaligned tensor)."""
+    """The persistent-kernel schedule must terminate, leave its error word clear, be reproducible and agree
+    with the three-sweep schedule to fp32 rounding of the per-chunk sums.  Tensors that are whole multiples
+    of the 8192-parameter chunk go through the kernel (one chunk, several, a quarter of a round, a whole round
+    of 512), the others through the sweeps of the same step."""
     capi = pkg.capi
-    numels = [1000, 70000, 5, 1 << 20, 3 * 8192, 8193, 1, (2 << 20) + 17, 1024, 1024, 4 << 20, 2 << 20]
+    numels = [1000, 65536, 5, 1 << 20, 3 * 8192, 8193, 1, (2 << 20) + 17, 8192, 8192, 4 << 20, 2 << 20, 8192 * 131]
+    resident_chunks = sum(n // 8192 for n in numels if n % 8192 == 0)
     results = []
-    for schedule in (capi.LANS_SWEEPS, capi.LANS_RESIDENT, capi.LANS_RESIDENT):
-        gen = torch.Generator(device="cuda").manual_seed(7)
-        total = sum(numels)
-        flat = [torch.empty(total, device="cuda").normal_(0, s, generator=gen) for s in (1e-3, 0.02)]
-        flat += [torch.zeros(total, device="cuda") for _ in range(2)]
-        views = [list(torch.split(t, numels)) for t in flat]
+    for schedule in (capi.LANS_SWEEPS, None, None):            # None: what a new plan has
+        state = _fresh_state(numels, 7)
         plan = pkg.ops.LansPlan(numels, schedule=schedule)
         hyper = capi.LansHyper(1e-3, 0.9, 0.999, 1e-6, 1, 0.01, 1, 1, 1)
         for step in (1, 2, 3):
-            plan.step(*views, step, hyper)
+            plan.step(*state, step, hyper)
         torch.cuda.synchronize()
         assert plan.error() == 0
-        results.append((flat, plan.norms()))
+        if schedule is None:                                    # padding included, so at least the chunks
+            assert plan.last_resident_slots() >= resident_chunks
+        else:
+            assert plan.last_resident_slots() == 0
+        results.append((state, plan.norms()))
         plan.close()
-    for a, b in zip(results[1][0], results[2][0]):          # run to run: the same bits
-        assert torch.equal(a, b)
+    for la, lb in zip(results[1][0], results[2][0]):          # run to run: the same bits
+        for a, b in zip(la, lb):
+            assert torch.equal(a, b)
     assert torch.equal(results[1][1], results[2][1])
-    for name, a, b in zip("gpmv", results[0][0], results[1][0]):
-        scale = a.abs().max().item()
-        assert (a - b).abs().max().item() <= 2e-6 * scale, name
+    for name, la, lb in zip("gpmv", results[0][0], results[1][0]):
+        for i, (a, b) in enumerate(zip(la, lb)):
+            scale = max(a.abs().max().item(), 1e-30)
+            assert (a - b).abs().max().item() <= 2e-6 * scale, (name, i)
     torch.testing.assert_close(results[0][1], results[1][1], rtol=2e-6, atol=0)
+
+
+def test_lans_resident_step_with_an_unaligned_tensor_runs_as_sweeps(pkg):
+    """The resident kernel moves float4s: a step in which an array of one of its tensors is not 16-byte
+    aligned goes through the sweeps instead, with the sweeps' bits."""
+    capi = pkg.capi
+    numels = [8192 * 4, 100, 8192]
+    hyper = capi.LansHyper(1e-3, 0.9, 0.999, 1e-6, 1, 0.01, 1, 1, 1)
+    out = []
+    for schedule, offset in ((capi.LANS_SWEEPS, 1), (capi.LANS_RESIDENT, 1), (capi.LANS_RESIDENT, 0)):
+        state = _fresh_state(numels, 9, offset)
+        plan = pkg.ops.LansPlan(numels, schedule=schedule)
+        plan.step(*state, 1, hyper)
+        plan.step(*state, 2, hyper)
+        torch.cuda.synchronize()
+        assert plan.error() == 0
+        out.append((state, plan.last_resident_slots()))
+        plan.close()
+    assert out[0][1] == 0 and out[1][1] == 0 and out[2][1] >= 5
+    for la, lb in zip(out[0][0], out[1][0]):
+        for a, b in zip(la, lb):
+            assert torch.equal(a, b)
+
+
+def test_lans_resident_give_up_is_fail_safe_and_sticky(pkg):
+    """With publication switched off (test hook) every wait of the resident kernel runs into its bound: the
+    kernel must still end, write no parameter, flag the plan; the next step must be refused until the error
+    has been read; after that the plan works again."""
+    capi = pkg.capi
+    numels = [1 << 20, 8192 * 3, 8192]
+    hyper = capi.LansHyper(1e-3, 0.9, 0.999, 1e-6, 1, 0.01, 1, 1, 1)
+    state = _fresh_state(numels, 13)
+    before = [[t.clone() for t in lst] for lst in state]
+    plan = pkg.ops.LansPlan(numels)
+    plan.debug(spin_limit=8, flags=1)
+    plan.step(*state, 1, hyper)
+    torch.cuda.synchronize()
+    # nothing was published, so no workgroup learned ||g||: stage M never ran, and nothing at all was written
+    for la, lb in zip(state, before):
+        for a, b in zip(la, lb):
+            assert torch.equal(a, b)
+    with pytest.raises(capi.LancetError) as info:          # refused on the host, nothing launched
+        plan.step(*state, 2, hyper)
+    assert info.value.status == capi.ERR_STALLED
+    assert plan.error() == 1                                # read ...
+    assert plan.error() == 0                                # ... and cleared
+    plan.debug(spin_limit=0, flags=0)
+    plan.step(*state, 1, hyper)
+    torch.cuda.synchronize()
+    assert plan.error() == 0
+    ref = [[t.clone() for t in lst] for lst in before]
+    other = pkg.ops.LansPlan(numels)
+    other.step(*ref, 1, hyper)
+    torch.cuda.synchronize()
+    for la, lb in zip(state, ref):
+        for a, b in zip(la, lb):
+            assert torch.equal(a, b)
+    plan.close()
+    other.close()
 
 
 def test_lans_resident_schedule_against_oracle(pkg):
@@ -173,6 +248,7 @@ def test_lans_resident_schedule_against_oracle(pkg):
         lo.lans_step(g, p, m, v, step)
         plan.step(dg, dp, dm, dv, step, hyper)
     assert plan.error() == 0
+    assert plan.last_resident_slots() >= 5                  # the (8192,) and (4, 8192) tensors
     for i in range(len(shapes)):
         assert_close_scaled(to_np(dp[i]), p[i], P_RTOL, "p[%d]" % i)
         assert_close_scaled(to_np(dm[i]), m[i], P_RTOL, "m[%d]" % i)
@@ -181,7 +257,7 @@ def test_lans_resident_schedule_against_oracle(pkg):
 
 
 def test_lans_resident_schedule_with_tensors_that_do_not_fit(pkg):
-    """Tensors with more chunks than the chip holds at once go through the sweeps inside the same step; the
+    """Tensors with more chunks than the kernel takes go through the sweeps inside the same step; the
     caller sees one step, norms in the order of its lists, and the same values as the pure sweeps schedule."""
     capi = pkg.capi
     probe = pkg.ops.LansPlan([1024, 1024])
@@ -189,31 +265,28 @@ def test_lans_resident_schedule_with_tensors_that_do_not_fit(pkg):
     probe.close()
     assert largest == 1 and limit >= 256
     big = (limit + 1) * 8192
-    numels = [1024, big, 70000, big + 3 * 8192 + 5, 8192]
+    numels = [1024, big, 65536, big + 3 * 8192 + 5, 8192]
     results = []
     for schedule in (capi.LANS_SWEEPS, capi.LANS_RESIDENT):
-        gen = torch.Generator(device="cuda").manual_seed(11)
-        total = sum(numels)
-        flat = [torch.empty(total, device="cuda").normal_(0, s, generator=gen) for s in (1e-3, 0.02)]
-        flat += [torch.zeros(total, device="cuda") for _ in range(2)]
-        views = [list(torch.split(t, numels)) for t in flat]
+        state = _fresh_state(numels, 11)
         plan = pkg.ops.LansPlan(numels, schedule=schedule)
         assert plan.resident_capacity() == (limit, limit + 5)
         hyper = capi.LansHyper(1e-3, 0.9, 0.999, 1e-6, 1, 0.01, 1, 1, 1)
         for step in (1, 2):
-            plan.step(*views, step, hyper)
+            plan.step(*state, step, hyper)
         torch.cuda.synchronize()
         assert plan.error() == 0
-        results.append((flat, plan.norms()))
+        assert plan.last_resident_slots() == (9 if schedule == capi.LANS_RESIDENT else 0)
+        results.append((state, plan.norms()))
         plan.close()
-    for name, a, b in zip("gpmv", results[0][0], results[1][0]):
-        assert (a - b).abs().max().item() <= 2e-6 * a.abs().max().item(), name
+    for name, la, lb in zip("gpmv", results[0][0], results[1][0]):
+        for i, (a, b) in enumerate(zip(la, lb)):
+            assert (a - b).abs().max().item() <= 2e-6 * max(a.abs().max().item(), 1e-30), (name, i)
     torch.testing.assert_close(results[0][1], results[1][1], rtol=2e-6, atol=0)
     # the two large tensors took the same kernels under both schedules: the same bits
-    off = np.cumsum([0] + numels)
     for i in (1, 3):
-        assert torch.equal(results[0][0][1][off[i]:off[i + 1]], results[1][0][1][off[i]:off[i + 1]])
-    # a plan made only of tensors that do not fit has no use for the resident kernel
+        assert torch.equal(results[0][0][1][i], results[1][0][1][i])
+    # a plan made only of tensors that do not fit has no use for the resident kernel and starts with the sweeps
     only_big = pkg.ops.LansPlan([big])                       # no memory is touched by creating a plan
     with pytest.raises(RuntimeError):
         only_big.set_schedule(capi.LANS_RESIDENT)
@@ -241,6 +314,7 @@ def test_lans_resident_schedule_beside_other_work(pkg):
         plan.step(*views_a, step, hyper)
     torch.cuda.synchronize()
     assert plan.error() == 0
+    assert plan.last_resident_slots() >= (12 << 20) // 8192
 
     flat_b, views_b = state()
     side = torch.cuda.Stream()

@@ -378,6 +378,8 @@ int lancet_lans_step(lancet_lans_plan_t plan, const float* const* g, float* cons
 #define LANCET_LANS_SWEEPS 0
 #define LANCET_LANS_RESIDENT 1
 int lancet_lans_plan_set_schedule(lancet_lans_plan_t plan, int schedule);
+/* *schedule = the schedule the plan's next step runs. */
+int lancet_lans_plan_schedule(lancet_lans_plan_t plan, int* schedule);
 /* workgroups: chunks (of 8192 parameters) of the largest tensor the resident kernel takes on this device
  * (larger tensors of the plan go through the sweeps; 512 = 4M parameters on a device that runs 512 of the
  * kernel's workgroups at once); max_tensor_chunks: chunks of the plan's largest tensor.  Either may be

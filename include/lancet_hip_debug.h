@@ -41,6 +41,11 @@ void lancet_debug_set_spin_limit(unsigned limit);
  * times these beside the row movers so that their fractions of the peak can be read against what the
  * memory system delivers to the simplest possible kernel. */
 int lancet_debug_stream(int kind, void* dst, const void* src, size_t bytes, lancet_stream_t stream);
+/* Measurement aid (no counterpart in the reference): the memory access pattern of an optimizer step and
+ * nothing else.  Reads g, p, m, v (n floats each, n a multiple of 1024, 16-byte aligned) and writes p, m, v,
+ * 28 bytes per element, with a few multiply-adds in between, one float4 per thread and array.  bench.py times
+ * it beside the LANS step: what the memory system delivers to a kernel that needs no norms. */
+int lancet_debug_stream_4r3w(const float* g, float* p, float* m, float* v, size_t n, lancet_stream_t stream);
 #ifdef __cplusplus
 }
 #endif

@@ -65,6 +65,7 @@ SIGNATURES = {
     "lancet_moe_partition_ranges_workspace_bytes": (_sz, [_int, _int, _i64]),
     "lancet_moe_partition_ranges": (_int, [_vp, _i64, _int, _int, _i64, _i64, _vp, _vp, _vp, _sz, _vp]),
     "lancet_debug_stream": (_int, [_int, _vp, _vp, _sz, _vp]),
+    "lancet_debug_stream_4r3w": (_int, [_vp, _vp, _vp, _vp, _sz, _vp]),
     "lancet_moe_decode": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp]),
     "lancet_moe_redispatch_expert_input": (_int, [C.POINTER(_vp), C.POINTER(_vp), _int, _int, _int, _i64, _i64, _i64,
                                                   _int, _int, _vp, _vp]),
@@ -88,6 +89,7 @@ SIGNATURES = {
     "lancet_lans_step": (_int, [_vp, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),
                                 _int, _vp, C.POINTER(LansHyper), _vp, _vp]),
     "lancet_lans_plan_norms": (_int, [_vp, _vp, _vp]),
+    "lancet_lans_plan_schedule": (_int, [_vp, C.POINTER(_int)]),
     "lancet_lans_plan_set_schedule": (_int, [_vp, _int]),
     "lancet_lans_plan_error": (_int, [_vp, _vp, C.POINTER(_int)]),
     "lancet_lans_debug_chunk_table": (_i64, [C.POINTER(_i64), _int, _int, _int, _vp, _i64, C.POINTER(_i64)]),

@@ -95,7 +95,33 @@ __global__ __launch_bounds__(256) void stream_kernel(u32x4* __restrict__ dst, co
     st_stream(dst + i, ld_stream(src + i));
   }
 }
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+// the access pattern of an optimizer step and nothing else: four arrays read, three of them written, one
+// float4 per thread and array, workgroups in address order
+__global__ __launch_bounds__(256) void stream_4r3w_kernel(const f32x4* __restrict__ g, f32x4* __restrict__ p,
+                                                          f32x4* __restrict__ m, f32x4* __restrict__ v) {
+  const size_t i = blockIdx.x * static_cast<size_t>(256) + threadIdx.x;
+  const f32x4 xg = __builtin_nontemporal_load(g + i);
+  f32x4 xp = __builtin_nontemporal_load(p + i), xm = __builtin_nontemporal_load(m + i), xv = __builtin_nontemporal_load(v + i);
+  xm = xm * 0.9f + xg * 0.1f;
+  xv = xv * 0.999f + xg * xg * 0.001f;
+  xp = xp - xm * 1e-3f;
+  __builtin_nontemporal_store(xm, m + i);
+  __builtin_nontemporal_store(xv, v + i);
+  __builtin_nontemporal_store(xp, p + i);
+}
 }  // namespace
+
+extern "C" int lancet_debug_stream_4r3w(const float* g, float* p, float* m, float* v, size_t n, lancet_stream_t stream) {
+  if (!g || !p || !m || !v) return LANCET_ERR_NULL;
+  if (n % 1024 != 0 || n / 1024 > 0x7fffffffu) return LANCET_ERR_SHAPE;
+  if (misaligned(g, 16) || misaligned(p, 16) || misaligned(m, 16) || misaligned(v, 16)) return LANCET_ERR_ALIGN;
+  if (n == 0) return LANCET_OK;
+  stream_4r3w_kernel<<<static_cast<unsigned>(n / 1024), 256, 0, S_(stream)>>>(
+      reinterpret_cast<const f32x4*>(g), reinterpret_cast<f32x4*>(p), reinterpret_cast<f32x4*>(m),
+      reinterpret_cast<f32x4*>(v));
+  return rc(hipGetLastError());
+}
 
 extern "C" int lancet_debug_stream(int kind, void* dst, const void* src, size_t bytes, lancet_stream_t stream) {
   if (kind < 0 || kind > 2) return LANCET_ERR_SHAPE;

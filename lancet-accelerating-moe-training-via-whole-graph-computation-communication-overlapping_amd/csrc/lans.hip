@@ -1270,6 +1270,13 @@ extern "C" int lancet_lans_plan_set_schedule(lancet_lans_plan_t pl, int schedule
   return LANCET_OK;
 }
 
+extern "C" int lancet_lans_plan_schedule(lancet_lans_plan_t pl, int* schedule) {
+  if (!pl || pl->magic != kPlanMagic) return LANCET_ERR_PLAN;
+  if (!schedule) return LANCET_ERR_NULL;
+  *schedule = pl->schedule;
+  return LANCET_OK;
+}
+
 extern "C" int lancet_lans_plan_resident_capacity(lancet_lans_plan_t pl, int* workgroups, int* max_tensor_chunks) {
   if (!pl || pl->magic != kPlanMagic) return LANCET_ERR_PLAN;
   if (workgroups) *workgroups = pl->resident_limit;

@@ -543,6 +543,12 @@ class LansPlan:
         with no such tensor) or capi.LANS_SWEEPS (no workgroup waits for another)."""
         capi.check(self._lib.lancet_lans_plan_set_schedule(self._h, int(schedule)), "lancet_lans_plan_set_schedule")
 
+    def schedule(self):
+        """The schedule the next step runs: capi.LANS_RESIDENT or capi.LANS_SWEEPS."""
+        n = C.c_int(-1)
+        capi.check(self._lib.lancet_lans_plan_schedule(self._h, C.byref(n)), "lancet_lans_plan_schedule")
+        return n.value
+
     def resident_capacity(self):
         """(chunks the resident schedule holds at once, chunks of this plan's largest tensor)."""
         wg, mx = C.c_int(0), C.c_int(0)

@@ -271,7 +271,7 @@ def bench_config4_partitioned(pkg, ops, lib, capi, data, logits, S, M, E, cf, it
     outs = [(torch.empty(Sp, device="cuda"), torch.empty((2, Sp), dtype=torch.int32, device="cuda"),
              torch.empty(E, dtype=torch.int32, device="cuda"), torch.empty(E, dtype=torch.int64, device="cuda"),
              torch.empty((E, Cap, M), dtype=data.dtype, device="cuda")) for _ in range(2 * P)]
-    ws = torch.empty(ops.moe_encode_workspace_bytes(Sp, E, 1), dtype=torch.uint8, device="cuda")
+    ws = ops.ScanWorkspace(ops.moe_encode_workspace_bytes(Sp, E, 1))
     zero = torch.zeros(E, dtype=torch.int32, device="cuda")
     merged = torch.empty((2, 2 * S), dtype=torch.int32, device="cuda")
     red = torch.empty((E, Cap, M), dtype=data.dtype, device="cuda")
@@ -351,7 +351,7 @@ def bench_config4_partitioned(pkg, ops, lib, capi, data, logits, S, M, E, cf, it
     r_il = torch.empty((2, 2 * S), dtype=torch.int32, device="cuda")
     r_used = torch.empty(E, dtype=torch.int32, device="cuda")
     r_elems = torch.empty(E, dtype=torch.int64, device="cuda")
-    r_ws = torch.empty(ops.moe_encode_workspace_bytes(S, E, 2), dtype=torch.uint8, device="cuda")
+    r_ws = ops.ScanWorkspace(ops.moe_encode_workspace_bytes(S, E, 2))
     r_buf = torch.full_like(red, 9.0)
     r_dec = torch.empty_like(dec)
 
@@ -458,8 +458,7 @@ def bench_other_configs(ops, iters):
         bufs = (torch.empty(k * S, device="cuda"), torch.empty((2, k * S), dtype=torch.int32, device="cuda"),
                 torch.empty(E, dtype=torch.int32, device="cuda"), torch.empty(E, dtype=torch.int64, device="cuda"),
                 torch.empty((E, Cap, M), dtype=dtype, device="cuda"))
-        ws = torch.empty(max(ops.moe_encode_workspace_bytes(S, E, k), ops.moe_encode_bpr_workspace_bytes(S, E, 1)),
-                         dtype=torch.uint8, device="cuda")
+        ws = ops.ScanWorkspace(max(ops.moe_encode_workspace_bytes(S, E, k), ops.moe_encode_bpr_workspace_bytes(S, E, 1)))
         dec = torch.empty((S, M), dtype=dtype, device="cuda")
 
         def step():
@@ -584,7 +583,7 @@ def main():
     outs = (torch.empty(K * S, device="cuda"), torch.empty((2, K * S), dtype=torch.int32, device="cuda"),
             torch.empty(E, dtype=torch.int32, device="cuda"), torch.empty(E, dtype=torch.int64, device="cuda"),
             torch.empty((E, Cap, M), dtype=torch.bfloat16, device="cuda"))
-    ws = torch.empty(ops.moe_encode_workspace_bytes(S, E, K), dtype=torch.uint8, device="cuda")
+    ws = ops.ScanWorkspace(ops.moe_encode_workspace_bytes(S, E, K))
     dec = torch.empty((S, M), dtype=torch.bfloat16, device="cuda")
 
     def encode():

@@ -13,7 +13,11 @@
  *     NULL = the default stream), is asynchronous with respect to the host and
  *     allocates nothing (the two lans_plan calls excepted, which own small tables);
  *   - outputs and workspaces are caller-owned; *_workspace_bytes() sizes the
- *     workspace, whose contents need not be initialised and are not preserved;
+ *     workspace.  Plain workspaces need no initialisation and are not preserved.  The
+ *     workspaces of the position scan (lancet_launch_gen_location, lancet_moe_encode,
+ *     lancet_moe_route, lancet_moe_encode_bpr) carry a few words of state from call to
+ *     call: set each up ONCE with lancet_scan_workspace_init after allocating it, let
+ *     nothing else write to it, and use it for one call at a time;
  *   - the return value is a status: 0 = ok, < 0 = rejected argument (nothing was
  *     launched), > 0 = a hipError_t from the runtime.  Nothing aborts the process
  *     (the reference CHECK/LOG(FATAL)s, src/common/cuda_utils.h:18-22).
@@ -32,7 +36,7 @@
 extern "C" {
 #endif
 
-#define LANCET_ABI_VERSION 4
+#define LANCET_ABI_VERSION 5
 
 /* element type of token rows */
 #define LANCET_F32 0
@@ -130,15 +134,15 @@ int lancet_moe_encode(const void* data, const float* gate, const float* gate2_no
 /* lancet_moe_encode without the workspace argument, for callers that cannot allocate device memory: code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  (No counterpart in the
  * reference, whose executor allocates a workspace before every Execute, src/impl/vm/vm.cc:1260-1266.)
- * The scan's scratch (ticket, error word, descriptor table) lives in a static device array of
+ * The scan's workspace (ticket, error word, descriptor table) lives in a static device array of
  * LANCET_NOALLOC_SCRATCH_BYTES that each GPU holds until the process ends; sizes whose
  * lancet_moe_encode_workspace_bytes(S, E, top_k) exceeds it are rejected with LANCET_ERR_SCRATCH
- * (1 MiB covers S * top_k * E <= 67 million, e.g. S = 65536, E = 512, top_k = 2).  The call allocates
+ * (it covers S * top_k * E <= 67 million, e.g. S = 65536, E = 512, top_k = 2).  The call allocates
  * nothing and launches the same kernels as lancet_moe_encode, with identical results.  All calls on one
  * GPU share the array: calls that overlap on one GPU race, so issue them on one stream or order them
- * yourself.  The first call on a device looks the array's address up (no launch, no allocation); make that
- * call once before recording a graph. */
-#define LANCET_NOALLOC_SCRATCH_BYTES (1u << 20)
+ * yourself.  The first call on a device looks the array's address up, sets the workspace up (one small
+ * launch on `stream`, no allocation) and waits for `stream`; make that call once before recording a graph. */
+#define LANCET_NOALLOC_SCRATCH_BYTES ((2u << 20) + 4096u)
 int lancet_moe_encode_noalloc(const void* data, const float* gate, const float* gate2_noise,
                               const int32_t* used_in, int64_t S, int64_t M, int64_t E, int64_t C, int top_k,
                               int dtype, unsigned flags, float* gates_s, int32_t* indices_locations,
@@ -394,8 +398,20 @@ int lancet_lans_plan_error(lancet_lans_plan_t plan, lancet_stream_t stream, int*
  * norms4xT, a device buffer of 4*T floats, asynchronously on `stream`. */
 int lancet_lans_plan_norms(lancet_lans_plan_t plan, float* norms4xT, lancet_stream_t stream);
 
-/* Reads (synchronously) the error word a scan workspace carries: 0 = ok, 1 = a wait gave up. */
-int lancet_scan_workspace_error(const void* workspace, lancet_stream_t stream, int* error_out);
+/* ---- workspaces of the position scan ---------------------------------------------------
+ * (No counterpart in the reference, whose scan kernel keeps no state: tutel_moe_dispatch.cu:164-212.)
+ * lancet_scan_workspace_init sets a workspace of workspace_bytes bytes (8-byte aligned, at least what the
+ * *_workspace_bytes() of the calls it will serve ask for) up, asynchronously on `stream`: once after
+ * allocation; every call that uses the workspace leaves it ready for the next, so that no call spends a
+ * launch on clearing it.  A call that is handed a workspace that is not set up launches nothing harmful:
+ * it sets every indices/locations entry and every used_out entry to -1 and the error word.
+ * Every wait inside the scan is bounded.  A wait that gives up sets the workspace's sticky error word,
+ * and the tokens whose positions depend on it get indices = locations = -1 and used_out = -1 (all of them,
+ * for top_k = 2): a consumer sees the failure in the outputs without a synchronisation.
+ * lancet_scan_workspace_error reads (synchronising `stream`) and clears the error word: *error_out = 1
+ * when any call on this workspace gave up a wait, or found it not set up, since the last read. */
+int lancet_scan_workspace_init(void* workspace, size_t workspace_bytes, lancet_stream_t stream);
+int lancet_scan_workspace_error(void* workspace, lancet_stream_t stream, int* error_out);
 
 #ifdef __cplusplus
 }

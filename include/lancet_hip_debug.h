@@ -31,10 +31,11 @@ int lancet_lans_plan_debug(lancet_lans_plan_t plan, unsigned spin_limit, unsigne
  * 16-byte aligned).  Lets a test tell which kernels it has exercised. */
 int lancet_lans_plan_debug_last_resident(lancet_lans_plan_t plan, int* slots);
 
-/* Test hook: number of polls a workgroup of the position scan waits for a predecessor
- * before it gives up, flags the workspace and finishes with undefined results
- * (0 restores the default).  Lets a host test exercise the bounded wait without hanging. */
-void lancet_debug_set_spin_limit(unsigned limit);
+/* Test hook: number of polls a workgroup of the position scan waits for a predecessor's word before it gives
+ * up (0 restores the default), kept in the workspace itself and read by every later call that uses it; set
+ * asynchronously on `stream`.  Lets a host test exercise the bounded wait while every kernel still exits
+ * normally. */
+int lancet_debug_scan_workspace_spin_limit(void* workspace, unsigned limit, lancet_stream_t stream);
 /* Measurement aid (no counterpart in the reference): one plain streaming kernel over `bytes` bytes (a multiple
  * of 4096), one 16-byte non-temporal access per thread, workgroups in address order: the launch shape that
  * streams fastest on this device.  kind 0 reads src, 1 fills dst with zeros, 2 copies src to dst.  bench.py

@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(HERE, "lib", "liblancet_hip.so")
 F32, BF16, F16 = 0, 1, 2
 GATE_IS_LOGITS = 1
 NO_TAIL_ZERO = 2
-ABI_VERSION = 4
+ABI_VERSION = 5
 ZERO_TAIL = 4
 ROWS_AT_USED = 8
 LANS_SWEEPS, LANS_RESIDENT = 0, 1
@@ -96,7 +96,8 @@ SIGNATURES = {
     "lancet_lans_plan_debug": (_int, [_vp, _u32, _u32]),
     "lancet_lans_plan_debug_last_resident": (_int, [_vp, C.POINTER(_int)]),
     "lancet_lans_plan_resident_capacity": (_int, [_vp, C.POINTER(_int), C.POINTER(_int)]),
-    "lancet_debug_set_spin_limit": (None, [_u32]),
+    "lancet_debug_scan_workspace_spin_limit": (_int, [_vp, _u32, _vp]),
+    "lancet_scan_workspace_init": (_int, [_vp, _sz, _vp]),
     "lancet_scan_workspace_error": (_int, [_vp, _vp, C.POINTER(_int)]),
 }
 

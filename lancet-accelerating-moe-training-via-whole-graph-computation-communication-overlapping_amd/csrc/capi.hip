@@ -68,16 +68,22 @@ extern "C" int64_t lancet_moe_capacity(int64_t S, int64_t E, float capacity_fact
   return static_cast<int64_t>(static_cast<int>(capacity_factor * static_cast<float>((S + E - 1) / E)));
 }
 
-extern "C" void lancet_debug_set_spin_limit(unsigned limit) { set_spin_limit(limit); }
+extern "C" int lancet_debug_scan_workspace_spin_limit(void* workspace, unsigned limit, lancet_stream_t stream) {
+  if (!workspace) return LANCET_ERR_NULL;
+  if (misaligned(workspace, 8)) return LANCET_ERR_ALIGN;
+  return rc(run_scan_ws_set_spin(workspace, limit, S_(stream)));
+}
 
-extern "C" int lancet_scan_workspace_error(const void* workspace, lancet_stream_t stream, int* error_out) {
+extern "C" int lancet_scan_workspace_init(void* workspace, size_t workspace_bytes, lancet_stream_t stream) {
+  if (!workspace) return LANCET_ERR_NULL;
+  if (misaligned(workspace, 8)) return LANCET_ERR_ALIGN;
+  if (workspace_bytes < scan_workspace_bytes(0, 1, 1)) return LANCET_ERR_WORKSPACE;
+  return rc(run_scan_ws_init(workspace, workspace_bytes, S_(stream)));
+}
+
+extern "C" int lancet_scan_workspace_error(void* workspace, lancet_stream_t stream, int* error_out) {
   if (!workspace || !error_out) return LANCET_ERR_NULL;
-  uint32_t word = 0;
-  hipError_t e = hipMemcpyAsync(&word, static_cast<const uint32_t*>(workspace) + 1, sizeof(word),
-                                hipMemcpyDeviceToHost, S_(stream));
-  if (e == hipSuccess) e = hipStreamSynchronize(S_(stream));
-  *error_out = static_cast<int>(word);
-  return rc(e);
+  return rc(run_scan_ws_take_error(workspace, error_out, S_(stream)));
 }
 
 // ---- plain streaming kernels (measurement aid) -------------------------------------------
@@ -166,7 +172,7 @@ extern "C" int lancet_launch_gen_location(int32_t* indices, const int32_t* in_ca
   if (int r = check_dims(S, M, E, C)) return r;
   if (!workspace || workspace_bytes < lancet_gen_location_workspace_bytes(S, E)) return LANCET_ERR_WORKSPACE;
   if (misaligned(indices, 4) || misaligned(locations, 4) || misaligned(out_capused, 4) ||
-      misaligned(out_elements_per_expert, 8) || misaligned(workspace, 4) || misaligned(in_capused, 4))
+      misaligned(out_elements_per_expert, 8) || misaligned(workspace, 8) || misaligned(in_capused, 4))
     return LANCET_ERR_ALIGN;
   return rc(run_route_scan(nullptr, nullptr, indices, in_capused, static_cast<int>(S), static_cast<int>(E),
                            static_cast<int>(C), static_cast<int>(M), 1, false, nullptr, indices, locations,
@@ -210,7 +216,7 @@ extern "C" int lancet_moe_route(const float* gate, const float* gate2_noise, con
   if (gate2_noise && top_k != 2) return LANCET_ERR_TOPK;
   if (!workspace || workspace_bytes < lancet_moe_encode_workspace_bytes(S, E, top_k)) return LANCET_ERR_WORKSPACE;
   if (misaligned(gate, 4) || misaligned(gate2_noise, 4) || misaligned(gates_s, 4) || misaligned(indices_locations, 4) || misaligned(used_in, 4) ||
-      misaligned(used_out, 4) || misaligned(elements_per_expert, 8) || misaligned(workspace, 4))
+      misaligned(used_out, 4) || misaligned(elements_per_expert, 8) || misaligned(workspace, 8))
     return LANCET_ERR_ALIGN;
   const int s = static_cast<int>(S);
   return rc(run_route_scan(gate, gate2_noise, nullptr, used_in, s, static_cast<int>(E), static_cast<int>(C),
@@ -335,7 +341,7 @@ extern "C" int lancet_moe_encode_bpr(const void* data, const float* gate, int64_
     return LANCET_ERR_WORKSPACE;
   if (misaligned(data, eb) || misaligned(dispatched, eb) || misaligned(gate, 4) || misaligned(gates_s, 4) ||
       misaligned(indices_locations, 4) || misaligned(used_out, 4) || misaligned(elements_per_expert, 8) ||
-      misaligned(workspace, 4))
+      misaligned(workspace, 8))
     return LANCET_ERR_ALIGN;
   const int s0 = static_cast<int>(S0);
   const int s = s0 / n_partitions;

@@ -14,8 +14,10 @@ constexpr int kMaxPartitions = 64;
 int64_t scan_num_tiles(int64_t S);
 size_t scan_workspace_bytes(int64_t S, int64_t E, int nsets);
 size_t bpr_workspace_bytes(int64_t S0, int64_t S, int64_t E);
-uint32_t current_spin_limit();
-void set_spin_limit(uint32_t limit);
+// one-time set-up of a scan workspace; its bound for waits; its sticky error word, read and cleared
+hipError_t run_scan_ws_init(void* ws, size_t nbytes, hipStream_t st);
+hipError_t run_scan_ws_set_spin(void* ws, uint32_t limit, hipStream_t st);
+hipError_t run_scan_ws_take_error(void* ws, int* error_out, hipStream_t st);
 
 hipError_t run_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t st);
 // noise (top-2 only, may be null): [S,E] values added to the row for the second choice

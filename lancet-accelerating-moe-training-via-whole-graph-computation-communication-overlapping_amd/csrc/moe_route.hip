@@ -110,7 +110,6 @@ struct RouteArgs {
   int S, E, C, M;
   int ntiles;
   int is_logits;
-  uint32_t spin_limit;
 };
 
 // K = 1: everything is final when the tile knows its prefix.
@@ -120,13 +119,29 @@ struct RouteArgs {
 template <int K>
 __global__ __launch_bounds__(kTile) void route_scan_kernel(RouteArgs a) {
   extern __shared__ uint32_t s_cnt[];
-  __shared__ uint32_t s_tile;
   const int tid = threadIdx.x;
-  if (tid == 0) s_tile = atomicAdd(a.ws.ticket, 1u);
-  __syncthreads();
-  const uint32_t tile = s_tile;
+  const TileStart me = tile_begin(a.ws, a.ntiles);
+  const uint32_t tile = me.tile;
   const int s = static_cast<int>(tile) * kTile + tid;
   const bool valid = s < a.S;
+  if (!me.ok) {
+    // no workspace to scan with: every token of this workgroup's range is marked, and so are the totals
+    if (valid) {
+#pragma unroll
+      for (int j = 0; j < K; ++j) {
+        a.idx_out[static_cast<size_t>(j) * a.S + s] = -1;
+        a.loc_out[static_cast<size_t>(j) * a.S + s] = -1;
+        if (a.gates_s) a.gates_s[static_cast<size_t>(j) * a.S + s] = 0.f;
+      }
+    }
+    if (blockIdx.x == 0) {
+      for (int c = tid; c < a.E; c += kTile) {
+        a.used_out[c] = -1;
+        a.elems_out[c] = 0;
+      }
+    }
+    return;
+  }
 
   int e[K];
   float p[K];
@@ -155,11 +170,14 @@ __global__ __launch_bounds__(kTile) void route_scan_kernel(RouteArgs a) {
   bool mem[K];
 #pragma unroll
   for (int j = 0; j < K; ++j) mem[j] = e[j] >= 0;
-  tile_scan<K>(e, mem, a.E, tile, a.ws, s_cnt, a.spin_limit, rank);
+  const bool poisoned = tile_scan<K>(e, mem, a.E, me, a.ws, s_cnt, rank);
 
   if (K == 1) {
     if (valid) {
-      if (e[0] >= 0) {
+      if (poisoned) {
+        a.idx_out[s] = -1;
+        a.loc_out[s] = -1;
+      } else if (e[0] >= 0) {
         const int used = a.used_in ? a.used_in[e[0]] : 0;
         const int r = static_cast<int>(rank[0]);
         a.loc_out[s] = r;
@@ -169,17 +187,6 @@ __global__ __launch_bounds__(kTile) void route_scan_kernel(RouteArgs a) {
         a.loc_out[s] = 0;
       }
       if (a.gates_s) a.gates_s[s] = p[0];
-    }
-    if (static_cast<int>(tile) == a.ntiles - 1) {
-      const uint32_t* s_agg = s_cnt + kWavesPerTile * a.E;
-      const uint32_t* s_base = s_agg + a.E;
-      for (int c = tid; c < a.E; c += kTile) {
-        const int64_t used = a.used_in ? a.used_in[c] : 0;
-        const int64_t total = static_cast<int64_t>(s_base[c]) + s_agg[c];
-        const int64_t uo = min(used + total, static_cast<int64_t>(a.C));
-        a.used_out[c] = static_cast<int32_t>(uo);
-        a.elems_out[c] = static_cast<uint64_t>((uo - used) * a.M);
-      }
     }
   } else {
     if (valid) {
@@ -191,6 +198,16 @@ __global__ __launch_bounds__(kTile) void route_scan_kernel(RouteArgs a) {
       }
     }
   }
+  // the tile that finishes last knows the totals and whether any tile was poisoned
+  const TileEnd te = tile_end(a.ws, me, a.ntiles, K * a.E, poisoned, s_cnt);
+  if (K == 1 && te.last) {
+    for (int c = tid; c < a.E; c += kTile) {
+      const int64_t used = a.used_in ? a.used_in[c] : 0;
+      const int64_t uo = min(used + static_cast<int64_t>(s_cnt[c]), static_cast<int64_t>(a.C));
+      a.used_out[c] = te.failed ? -1 : static_cast<int32_t>(uo);
+      a.elems_out[c] = te.failed ? 0 : static_cast<uint64_t>((uo - used) * a.M);
+    }
+  }
 }
 
 // Completes top-2 routing once all tiles are done: slot 1 is an ordinary top-1 encode with
@@ -199,33 +216,44 @@ __global__ __launch_bounds__(kTile) void route_scan_kernel(RouteArgs a) {
 // taken after the drop and normalised (docker/resources/sharded_moe.py:282-312).
 __global__ __launch_bounds__(kTile) void finalize_top2_kernel(RouteArgs a) {
   const int s = blockIdx.x * kTile + threadIdx.x;
-  // totals of both slots = the last tile's inclusive descriptors, [2][E]
-  const uint32_t* tot = a.ws.desc + static_cast<size_t>(a.ntiles - 1) * 2 * a.E;
+  // a workspace that is not set up: route_scan_kernel has marked every output already
+  if (ld_agent(a.ws.hdr + kWsMagic) != kWsMagicValue) return;
+  // totals of both slots [2][E] and the verdict of the scan, as its last tile left them in the header
+  const uint32_t* tot = a.ws.hdr + kWsTotals;
+  const bool poisoned = ld_agent(a.ws.hdr + kWsFailed) != 0u;
   if (s < a.S) {
-    const int e1 = a.idx_out[s], e2 = a.idx_out[a.S + s];
-    const int r1 = a.loc_out[s], r2 = a.loc_out[a.S + s];
-    const int u1 = a.used_in ? a.used_in[e1] : 0;
-    const int u2 = a.used_in ? a.used_in[e2] : 0;
-    const bool keep1 = r1 < a.C - u1;
-    const int64_t after1 = min(static_cast<int64_t>(u2) + (ld_agent(tot + e2) & kDescCountMask), static_cast<int64_t>(a.C));
-    const bool keep2 = r2 < a.C - after1;
-    a.idx_out[s] = keep1 ? e1 : -1;
-    a.loc_out[s] = keep1 ? r1 : -1;
-    a.idx_out[a.S + s] = keep2 ? e2 : -1;
-    a.loc_out[a.S + s] = keep2 ? r2 + static_cast<int>(after1 - u2) : -1;
-    const float g1 = keep1 ? a.gates_s[s] : 0.f;
-    const float g2 = keep2 ? a.gates_s[a.S + s] : 0.f;
-    const float den = fmaxf(g1 + g2, 1.1920929e-07f);
-    a.gates_s[s] = g1 / den;
-    a.gates_s[a.S + s] = g2 / den;
+    if (poisoned) {
+      a.idx_out[s] = a.idx_out[a.S + s] = -1;
+      a.loc_out[s] = a.loc_out[a.S + s] = -1;
+      a.gates_s[s] = a.gates_s[a.S + s] = 0.f;
+    } else {
+      const int e1 = a.idx_out[s], e2 = a.idx_out[a.S + s];
+      const int r1 = a.loc_out[s], r2 = a.loc_out[a.S + s];
+      const bool in1 = e1 >= 0 && e1 < a.E, in2 = e2 >= 0 && e2 < a.E;  // always, unless the scan left marks behind
+      const int u1 = (a.used_in && in1) ? a.used_in[e1] : 0;
+      const int u2 = (a.used_in && in2) ? a.used_in[e2] : 0;
+      const bool keep1 = in1 && r1 < a.C - u1;
+      const int64_t after1 = min(static_cast<int64_t>(u2) + (in2 ? tot[e2] : 0u),
+                                 static_cast<int64_t>(a.C));
+      const bool keep2 = in2 && r2 < a.C - after1;
+      a.idx_out[s] = keep1 ? e1 : -1;
+      a.loc_out[s] = keep1 ? r1 : -1;
+      a.idx_out[a.S + s] = keep2 ? e2 : -1;
+      a.loc_out[a.S + s] = keep2 ? r2 + static_cast<int>(after1 - u2) : -1;
+      const float g1 = keep1 ? a.gates_s[s] : 0.f;
+      const float g2 = keep2 ? a.gates_s[a.S + s] : 0.f;
+      const float den = fmaxf(g1 + g2, 1.1920929e-07f);
+      a.gates_s[s] = g1 / den;
+      a.gates_s[a.S + s] = g2 / den;
+    }
   }
   if (blockIdx.x == 0) {
     for (int c = threadIdx.x; c < a.E; c += kTile) {
       const int64_t used = a.used_in ? a.used_in[c] : 0;
-      const int64_t total = static_cast<int64_t>(ld_agent(tot + c) & kDescCountMask) + (ld_agent(tot + a.E + c) & kDescCountMask);
+      const int64_t total = static_cast<int64_t>(tot[c]) + tot[a.E + c];
       const int64_t uo = min(used + total, static_cast<int64_t>(a.C));
-      a.used_out[c] = static_cast<int32_t>(uo);
-      a.elems_out[c] = static_cast<uint64_t>((uo - used) * a.M);
+      a.used_out[c] = poisoned ? -1 : static_cast<int32_t>(uo);
+      a.elems_out[c] = poisoned ? 0 : static_cast<uint64_t>((uo - used) * a.M);
     }
   }
 }
@@ -282,12 +310,12 @@ __device__ __forceinline__ uint32_t order_key(float x) {
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
+// Everything the batch-prioritised routing keeps in the scan's workspace behind the descriptor table is a
+// 64-bit word tagged "not a descriptor" (foreign_word), the value in the low half: tok[s] also carries the
+// token's expert + 1 in the tag's low bits; par[0..2][e] = threshold, tie quota, ties before the partition.
 struct BprArgs {
-  const int32_t* idx0;   // [S0] expert per token
-  const float* prio;     // [S0] priority (gate value of the chosen expert)
-  uint32_t* thresh;      // [E]
-  int32_t* quota;        // [E]
-  int32_t* ties_before;  // [E]
+  uint64_t* tok;         // [S0] expert and priority (gate value of the chosen expert) per token
+  uint64_t* par;         // [3][E]
   int S0, S, E, C, M;
   int part_lo;           // first token of the partition
   int ntiles;
@@ -297,10 +325,21 @@ struct BprArgs {
   int32_t* used_out;     // [E]
   uint64_t* elems_out;   // [E]
   ScanWs ws;
-  uint32_t spin_limit;
 };
 
 constexpr int kSelectThreads = 1024;
+
+__device__ __forceinline__ int tok_expert(uint64_t w) { return static_cast<int>((w >> 32) & 0xffffu) - 1; }
+__device__ __forceinline__ float tok_prio(uint64_t w) { return __uint_as_float(static_cast<uint32_t>(w)); }
+__device__ __forceinline__ uint32_t par_value(const uint64_t* p) { return static_cast<uint32_t>(*p); }
+
+// first choice and its gate value (or softmax probability) of every token of the batch
+__global__ __launch_bounds__(kTile) void bpr_prepare_kernel(const float* gate, int S0, int E, int is_logits, uint64_t* tok) {
+  const int s = blockIdx.x * kTile + threadIdx.x;
+  if (s >= S0) return;
+  const Routed r = route_token<1>(gate + static_cast<size_t>(s) * E, nullptr, E, is_logits != 0);
+  tok[s] = foreign_word(static_cast<uint32_t>(r.e0 + 1), __float_as_uint(r.p0));
+}
 
 __global__ __launch_bounds__(kSelectThreads) void bpr_select_kernel(BprArgs a) {
   __shared__ uint32_t hist[256];
@@ -310,25 +349,25 @@ __global__ __launch_bounds__(kSelectThreads) void bpr_select_kernel(BprArgs a) {
   if (tid == 0) s_count = 0;
   __syncthreads();
   uint32_t local = 0;
-  for (int s = tid; s < a.S0; s += kSelectThreads) local += (a.idx0[s] == e);
+  for (int s = tid; s < a.S0; s += kSelectThreads) local += (tok_expert(a.tok[s]) == e);
   if (local) atomicAdd(&s_count, local);
   __syncthreads();
   const uint32_t count = s_count;
   if (a.C <= 0) {
     // nothing fits: no key is above the largest threshold and the tie quota is zero
     if (tid == 0) {
-      a.thresh[e] = 0xffffffffu;
-      a.quota[e] = 0;
-      a.ties_before[e] = 0;
+      a.par[e] = foreign_word(0u, 0xffffffffu);
+      a.par[a.E + e] = foreign_word(0u, 0u);
+      a.par[2 * a.E + e] = foreign_word(0u, 0u);
     }
     return;
   }
   if (count <= static_cast<uint32_t>(a.C)) {
     // everything fits: every key is above threshold 0 or ties with it under an unlimited quota
     if (tid == 0) {
-      a.thresh[e] = 0u;
-      a.quota[e] = 0x7fffffff;
-      a.ties_before[e] = 0;
+      a.par[e] = foreign_word(0u, 0u);
+      a.par[a.E + e] = foreign_word(0u, 0x7fffffffu);
+      a.par[2 * a.E + e] = foreign_word(0u, 0u);
     }
     return;
   }
@@ -342,8 +381,9 @@ __global__ __launch_bounds__(kSelectThreads) void bpr_select_kernel(BprArgs a) {
     __syncthreads();
     const uint32_t prefix = s_prefix;
     for (int s = tid; s < a.S0; s += kSelectThreads) {
-      if (a.idx0[s] != e) continue;
-      const uint32_t k = order_key(a.prio[s]);
+      const uint64_t t = a.tok[s];
+      if (tok_expert(t) != e) continue;
+      const uint32_t k = order_key(tok_prio(t));
       if (pass == 0 || (k >> (shift + 8)) == prefix) atomicAdd(&hist[(k >> shift) & 0xffu], 1u);
     }
     __syncthreads();
@@ -364,49 +404,63 @@ __global__ __launch_bounds__(kSelectThreads) void bpr_select_kernel(BprArgs a) {
   if (tid == 0) s_count = 0;
   __syncthreads();
   local = 0;
-  for (int s = tid; s < a.part_lo; s += kSelectThreads)
-    local += (a.idx0[s] == e && order_key(a.prio[s]) == thr);
+  for (int s = tid; s < a.part_lo; s += kSelectThreads) {
+    const uint64_t t = a.tok[s];
+    local += (tok_expert(t) == e && order_key(tok_prio(t)) == thr);
+  }
   if (local) atomicAdd(&s_count, local);
   __syncthreads();
   if (tid == 0) {
-    a.thresh[e] = thr;
-    a.quota[e] = static_cast<int32_t>(s_need);
-    a.ties_before[e] = static_cast<int32_t>(s_count);
+    a.par[e] = foreign_word(0u, thr);
+    a.par[a.E + e] = foreign_word(0u, s_need);
+    a.par[2 * a.E + e] = foreign_word(0u, s_count);
   }
 }
 
 __global__ __launch_bounds__(kTile) void bpr_scan_kernel(BprArgs a) {
   extern __shared__ uint32_t s_cnt[];
-  __shared__ uint32_t s_tile;
   const int tid = threadIdx.x;
-  if (tid == 0) s_tile = atomicAdd(a.ws.ticket, 1u);
-  __syncthreads();
-  const uint32_t tile = s_tile;
+  const TileStart me = tile_begin(a.ws, a.ntiles);
+  const uint32_t tile = me.tile;
   const int sl = static_cast<int>(tile) * kTile + tid;  // token inside the partition
   const bool valid = sl < a.S;
+  if (!me.ok) {
+    if (valid) {
+      a.idx_out[sl] = -1;
+      a.loc_out[sl] = -1;
+      a.gates_s[sl] = 0.f;
+    }
+    if (blockIdx.x == 0) {
+      for (int c = tid; c < a.E; c += kTile) {
+        a.used_out[c] = -1;
+        a.elems_out[c] = 0;
+      }
+    }
+    return;
+  }
   int cls[2] = {-1, -1};
   bool mem[2] = {false, false};
   float prio = 0.f;
   if (valid) {
-    const int s = a.part_lo + sl;
-    const int e = a.idx0[s];
-    prio = a.prio[s];
+    const uint64_t t = a.tok[a.part_lo + sl];
+    const int e = tok_expert(t);
+    prio = tok_prio(t);
     if (e >= 0 && e < a.E) {
       const uint32_t k = order_key(prio);
-      const uint32_t thr = a.thresh[e];
+      const uint32_t thr = par_value(a.par + e);
       cls[0] = cls[1] = e;
       mem[0] = k > thr;   // above the threshold: always stays
       mem[1] = k == thr;  // at the threshold: stays while the quota lasts
     }
   }
   uint32_t rank[2];
-  tile_scan<2>(cls, mem, a.E, tile, a.ws, s_cnt, a.spin_limit, rank);
+  const bool poisoned = tile_scan<2>(cls, mem, a.E, me, a.ws, s_cnt, rank);
   if (valid) {
     int idx = -1, loc = -1;
-    if (cls[0] >= 0) {
+    if (cls[0] >= 0 && !poisoned) {
       const int e = cls[0];
-      const int64_t q = a.quota[e];
-      const int64_t tb = a.ties_before[e];
+      const int64_t q = static_cast<int32_t>(par_value(a.par + a.E + e));
+      const int64_t tb = static_cast<int32_t>(par_value(a.par + 2 * a.E + e));
       const int64_t tie_rank = tb + rank[1];
       if (mem[0] || (mem[1] && tie_rank < q)) {
         idx = e;
@@ -417,18 +471,17 @@ __global__ __launch_bounds__(kTile) void bpr_scan_kernel(BprArgs a) {
     a.loc_out[sl] = loc;
     a.gates_s[sl] = prio;
   }
-  if (static_cast<int>(tile) == a.ntiles - 1) {
-    const uint32_t* s_agg = s_cnt + kWavesPerTile * 2 * a.E;
-    const uint32_t* s_base = s_agg + 2 * a.E;
+  const TileEnd te = tile_end(a.ws, me, a.ntiles, 2 * a.E, poisoned, s_cnt);
+  if (te.last) {
     for (int c = tid; c < a.E; c += kTile) {
-      const int64_t q = a.quota[c];
-      const int64_t tb = a.ties_before[c];
-      const int64_t above = static_cast<int64_t>(s_base[c]) + s_agg[c];
-      const int64_t ties = static_cast<int64_t>(s_base[a.E + c]) + s_agg[a.E + c];
+      const int64_t q = static_cast<int32_t>(par_value(a.par + a.E + c));
+      const int64_t tb = static_cast<int32_t>(par_value(a.par + 2 * a.E + c));
+      const int64_t above = s_cnt[c];
+      const int64_t ties = s_cnt[a.E + c];
       const int64_t kept = above + min(tb + ties, q) - min(tb, q);
       const int64_t uo = min(kept, static_cast<int64_t>(a.C));
-      a.used_out[c] = static_cast<int32_t>(uo);
-      a.elems_out[c] = static_cast<uint64_t>(uo * a.M);
+      a.used_out[c] = te.failed ? -1 : static_cast<int32_t>(uo);
+      a.elems_out[c] = te.failed ? 0 : static_cast<uint64_t>(uo * a.M);
     }
   }
 }
@@ -436,21 +489,39 @@ __global__ __launch_bounds__(kTile) void bpr_scan_kernel(BprArgs a) {
 // ---------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------
-static uint32_t g_spin_limit = 1u << 22;  // ~ seconds of polling; a healthy wait is microseconds
-
-uint32_t current_spin_limit() { return __atomic_load_n(&g_spin_limit, __ATOMIC_RELAXED); }
-void set_spin_limit(uint32_t limit) {
-  __atomic_store_n(&g_spin_limit, limit ? limit : (1u << 22), __ATOMIC_RELAXED);
-}
-
 int64_t scan_num_tiles(int64_t S) { return S > 0 ? (S + kTile - 1) / kTile : 1; }
 
 size_t scan_workspace_bytes(int64_t S, int64_t E, int nsets) {
-  return scan_ws_words(scan_num_tiles(S), nsets * E) * sizeof(uint32_t);
+  return scan_ws_bytes(scan_num_tiles(S), nsets * E);
 }
 
 size_t bpr_workspace_bytes(int64_t S0, int64_t S, int64_t E) {
-  return scan_workspace_bytes(S, E, 2) + (2 * static_cast<size_t>(S0) + 3 * static_cast<size_t>(E)) * 4;
+  return scan_workspace_bytes(S, E, 2) + (static_cast<size_t>(S0) + 3 * static_cast<size_t>(E)) * 8;
+}
+
+hipError_t run_scan_ws_init(void* ws, size_t nbytes, hipStream_t st) {
+  const size_t nwords = nbytes / sizeof(uint32_t);
+  if (nwords < kScanHeaderWords) return hipErrorInvalidValue;
+  const int blocks = static_cast<int>(std::min<size_t>((nwords + 255) / 256, 1024));
+  scan_ws_init_kernel<<<blocks, 256, 0, st>>>(static_cast<uint32_t*>(ws), nwords);
+  return hipGetLastError();
+}
+
+hipError_t run_scan_ws_set_spin(void* ws, uint32_t limit, hipStream_t st) {
+  return run_fill_u32(static_cast<uint32_t*>(ws) + kWsSpin, 1, limit, st);
+}
+
+hipError_t run_scan_ws_take_error(void* ws, int* error_out, hipStream_t st) {
+  uint32_t word = 0;
+  uint32_t* err = static_cast<uint32_t*>(ws) + kWsError;
+  hipError_t e = hipMemcpyAsync(&word, err, sizeof(word), hipMemcpyDeviceToHost, st);
+  if (e == hipSuccess) e = hipStreamSynchronize(st);
+  if (e == hipSuccess && word != 0u) {  // the reader, and only the reader, clears it
+    e = run_fill_u32(err, 1, 0u, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+  }
+  *error_out = word != 0u;
+  return e;
 }
 
 hipError_t run_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t st) {
@@ -489,10 +560,8 @@ hipError_t run_route_scan(const float* gate, const float* noise, const int32_t* 
   a.M = M;
   a.ntiles = static_cast<int>(scan_num_tiles(S));
   a.is_logits = is_logits;
-  a.spin_limit = current_spin_limit();
   a.ws = scan_ws_view(ws);
-  hipError_t err = run_fill_u32(static_cast<uint32_t*>(ws), scan_ws_words(a.ntiles, K * E), 0u, st);
-  if (err != hipSuccess) return err;
+  hipError_t err = hipSuccess;
   const size_t lds = scan_lds_bytes(K * E);
   if (K == 1) {
     route_scan_kernel<1><<<a.ntiles, kTile, lds, st>>>(a);
@@ -519,24 +588,19 @@ hipError_t run_bpr_route(const float* gate, int S0, int E, int C, int M, int n_p
   a.part_lo = partition_id * S;
   a.ntiles = static_cast<int>(scan_num_tiles(S));
   a.ws = scan_ws_view(ws);
-  uint32_t* extra = static_cast<uint32_t*>(ws) + scan_ws_words(a.ntiles, 2 * E);
-  int32_t* idx0 = reinterpret_cast<int32_t*>(extra);
-  float* prio = reinterpret_cast<float*>(extra + S0);
-  a.idx0 = idx0;
-  a.prio = prio;
-  a.thresh = extra + 2 * static_cast<size_t>(S0);
-  a.quota = reinterpret_cast<int32_t*>(a.thresh + E);
-  a.ties_before = a.quota + E;
+  a.tok = reinterpret_cast<uint64_t*>(static_cast<char*>(ws) + scan_ws_bytes(a.ntiles, 2 * E));
+  a.par = a.tok + S0;
   a.gates_s = gates_s;
   a.idx_out = idx_out;
   a.loc_out = loc_out;
   a.used_out = used_out;
   a.elems_out = elems_out;
-  a.spin_limit = current_spin_limit();
-  hipError_t err = run_fill_u32(static_cast<uint32_t*>(ws), scan_ws_words(a.ntiles, 2 * E), 0u, st);
-  if (err != hipSuccess) return err;
-  err = run_gate_topk(gate, nullptr, S0, E, 1, is_logits, idx0, prio, st);
-  if (err != hipSuccess) return err;
+  hipError_t err = hipSuccess;
+  if (S0 > 0) {
+    bpr_prepare_kernel<<<(S0 + kTile - 1) / kTile, kTile, 0, st>>>(gate, S0, E, is_logits, a.tok);
+    err = hipGetLastError();
+    if (err != hipSuccess) return err;
+  }
   bpr_select_kernel<<<E, kSelectThreads, 0, st>>>(a);
   err = hipGetLastError();
   if (err != hipSuccess) return err;

@@ -4,16 +4,27 @@
 //                    id; rank inside the wave = popcount of the peer mask below the lane;
 //   2. tile level  - per-wave counts in LDS, exclusive scan over the waves of the tile;
 //   3. across tiles - decoupled look-back over a [tiles][counters] descriptor table.  Every
-//                    descriptor is ONE 32-bit word: 2 status bits (1 = the tile's own count,
-//                    2 = inclusive prefix over all tiles up to it) above a 30-bit count, so a
-//                    word is self-validating and no fence separates "data" from "flag".  A
-//                    tile publishes its counts, then reads the words of its predecessors, a
-//                    window of rows at a time, all (row, counter) pairs in parallel, and stops
-//                    per counter at the nearest row that already holds an inclusive prefix.
+//                    descriptor is ONE 64-bit word: the launch epoch (30 bits, plus a poison
+//                    bit and a "not a descriptor" bit) in the high half; 2 status bits (1 = the tile's own count,
+//                    2 = inclusive prefix over all tiles up to it) above a 30-bit count in the
+//                    low half.  A word is self-validating: no fence separates "data" from
+//                    "flag", and a word of an earlier launch is simply not there yet, so
+//                    nothing clears the table between launches.  A tile publishes its counts,
+//                    then reads the words of its predecessors, a window of rows at a time, all
+//                    (row, counter) pairs in parallel, and stops per counter at the nearest row
+//                    that already holds an inclusive prefix.
 // Tiles are numbered by an atomic ticket, so a tile only ever waits for tiles that are
 // already running, and it only waits for their own counts, never for their prefixes: the
 // look-back is one round of parallel loads, not a serial chain.  Descriptor words are read
 // and written with agent-scope atomics (the eight XCDs of the chip have private L2 caches).
+//
+// The workspace carries its state from launch to launch (ticket, epoch): it is set up once
+// (scan_ws_init_kernel), every launch leaves it ready for the next (the tile that finishes
+// last resets the ticket and moves the epoch on), and a launch that finds no set-up workspace
+// flags it, marks its outputs and touches nothing else.  Every wait is bounded; a tile whose
+// wait gives up sets the workspace's sticky error word and poisons what it publishes, every
+// tile that builds on a poisoned word is poisoned too, and poisoned tiles write -1 for their
+// tokens: a consumer sees the failure in the outputs, without a synchronisation.
 //
 // Replaces the per-expert serial Blelloch scan of the reference
 // (src/op/dialect/cuda/kernels/tutel_moe_dispatch.cu:164-212: grid = E blocks, each
@@ -23,30 +34,178 @@
 
 namespace lancet {
 
-// Views into the caller's workspace (all uint32 words).
+// Header words of the workspace (uint32), followed by the descriptor table (uint64).
+enum : uint32_t {
+  kWsTicket = 0,  // next tile number; 0 between launches
+  kWsError = 1,   // sticky: a bounded wait gave up, or a launch found the workspace not set up
+  kWsEpoch = 2,   // tag of the running launch's descriptor words (1 .. 2^30-1)
+  kWsDone = 3,    // tiles of the running launch that have finished (and kDoneFailed); 0 between launches
+  kWsSpin = 4,    // polls a tile waits for a predecessor's word before it gives up (0: the default)
+  kWsMagic = 5,   // kWsMagicValue once the workspace is set up
+  kWsExtent = 6,  // largest number of descriptor words a launch has used
+  kWsFailed = 7,  // verdict of the last launch: 1 = a tile was poisoned (its outputs carry marks)
+  kWsTotals = 8,  // totals per counter of the last launch, kMaxScanCounters words
+  kScanHeaderWords = 8 + 1024
+};
+constexpr int kMaxScanCounters = 1024;        // 2 counter sets x 512 experts
+constexpr uint32_t kDoneFailed = 0x80000000u;  // in kWsDone: a tile that has finished was poisoned
+constexpr uint32_t kWsMagicValue = 0x4c53434eu;  // "LSCN"
+constexpr uint32_t kDefaultScanSpin = 1u << 22;  // ~ seconds of polling; a healthy wait is microseconds
+
 struct ScanWs {
-  uint32_t* ticket;  // [1]  next tile number
-  uint32_t* error;   // [1]  set to 1 when a bounded wait gave up
-  uint32_t* desc;    // [T][NC] descriptor words, zero before the launch
+  uint32_t* hdr;   // [kScanHeaderWords]
+  uint64_t* desc;  // [T][NC] descriptor words
 };
 
-constexpr uint32_t kScanHeaderWords = 2;  // ticket, error
 constexpr uint32_t kDescCountMask = 0x3fffffffu;
 constexpr uint32_t kDescAggregate = 1u << 30;
 constexpr uint32_t kDescInclusive = 2u << 30;
+constexpr uint32_t kDescPoison = 0x80000000u;   // in the high (epoch) half
+// Also in the high half: the word is no descriptor.  Callers that keep other data in a scan workspace (the
+// batch-prioritised routing does) store it as 64-bit words with this bit set, so that whatever a later launch
+// finds where it expects a descriptor is either a descriptor, tagged with its launch's epoch, or a word that
+// no epoch matches: launches of any shapes and kinds can share one workspace.
+constexpr uint32_t kDescForeign = 0x40000000u;
+constexpr uint32_t kEpochMask = 0x3fffffffu;
 
-// words that must be zero when the kernel starts
-__host__ __device__ inline size_t scan_ws_words(int64_t ntiles, int64_t ncounters) {
-  return kScanHeaderWords + static_cast<size_t>(ntiles) * static_cast<size_t>(ncounters);
+__host__ __device__ inline uint64_t foreign_word(uint32_t tag_bits, uint32_t low) {
+  return (static_cast<uint64_t>(kDescForeign | (tag_bits & kEpochMask)) << 32) | low;
+}
+
+__host__ __device__ inline size_t scan_ws_bytes(int64_t ntiles, int64_t ncounters) {
+  return kScanHeaderWords * sizeof(uint32_t) + static_cast<size_t>(ntiles) * static_cast<size_t>(ncounters) * sizeof(uint64_t);
 }
 
 inline ScanWs scan_ws_view(void* base) {
-  uint32_t* w = static_cast<uint32_t*>(base);
   ScanWs ws;
-  ws.ticket = w;
-  ws.error = w + 1;
-  ws.desc = w + kScanHeaderWords;
+  ws.hdr = static_cast<uint32_t*>(base);
+  ws.desc = reinterpret_cast<uint64_t*>(ws.hdr + kScanHeaderWords);
   return ws;
+}
+
+__device__ __forceinline__ uint64_t ld_desc(const uint64_t* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_desc(uint64_t* p, uint32_t tag, uint32_t low) {
+  __hip_atomic_store(p, (static_cast<uint64_t>(tag) << 32) | low, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ bool desc_is_current(uint64_t x, uint32_t epoch) {
+  return (static_cast<uint32_t>(x >> 32) & ~kDescPoison) == epoch;
+}
+__device__ __forceinline__ bool desc_is_poisoned(uint64_t x) { return (static_cast<uint32_t>(x >> 32) & kDescPoison) != 0; }
+
+// What a tile learns when it starts.  ok == false: the workspace is not set up (or its state is damaged); the
+// caller marks the outputs of tile `tile` (= its workgroup index then) and returns without tile_scan.
+struct TileStart {
+  uint32_t tile, epoch, spin;
+  bool ok;
+};
+
+// Must be called from uniform control flow by all kTile threads, first thing in the kernel.
+__device__ __forceinline__ TileStart tile_begin(const ScanWs& ws, int ntiles) {
+  __shared__ uint32_t s_start[4];
+  if (threadIdx.x == 0) {
+    uint32_t tile = blockIdx.x, epoch = 0u, spin = 0u, ok = 0u;
+    if (ld_agent(ws.hdr + kWsMagic) == kWsMagicValue) {
+      const uint32_t t = atomicAdd(ws.hdr + kWsTicket, 1u);
+      epoch = ld_agent(ws.hdr + kWsEpoch);
+      spin = ld_agent(ws.hdr + kWsSpin);
+      if (t < static_cast<uint32_t>(ntiles) && epoch != 0u && (epoch & ~kEpochMask) == 0u) {
+        tile = t;
+        ok = 1u;
+      }
+    }
+    if (!ok) st_agent(ws.hdr + kWsError, 1u);
+    s_start[0] = tile;
+    s_start[1] = epoch;
+    s_start[2] = spin ? spin : kDefaultScanSpin;
+    s_start[3] = ok;
+  }
+  __syncthreads();
+  TileStart r;
+  r.tile = s_start[0];
+  r.epoch = s_start[1];
+  r.spin = s_start[2];
+  r.ok = s_start[3] != 0u;
+  return r;
+}
+
+// What a tile learns when it ends.  last: it is the tile that finished last, the launch's totals (the
+// inclusive prefix of the last tile, per counter) are in the LDS array it passed and in the workspace's header;
+// failed (meaningful for the last tile, which knows about all tiles): some tile of the launch was poisoned,
+// or the totals could not be read.
+struct TileEnd {
+  bool last, failed;
+};
+
+// Last thing a tile that passed tile_begin does (uniform control flow, all threads; s_tot: LDS, ncounters
+// words, free for use).  A poisoned tile says so in the same counter that counts the finished tiles, so the
+// tile that finishes last knows whether any tile was.  That tile reads the totals, stores them and the
+// verdict in the header for a kernel that follows (the top-2 finalisation), and leaves the workspace ready for
+// the next launch.  Every tile has read the epoch before it gets here, so moving it on disturbs nobody.  When
+// the epoch wraps, the words of 2^30 launches ago would look current again: they are cleared first.
+__device__ __forceinline__ TileEnd tile_end(const ScanWs& ws, const TileStart& me, int ntiles, int ncounters,
+                                            bool tile_failed, uint32_t* s_tot) {
+  __shared__ uint32_t s_old;
+  __shared__ int s_bad;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    if (tile_failed) atomicOr(ws.hdr + kWsDone, kDoneFailed);  // same address, same thread: ordered before the add
+    s_old = atomicAdd(ws.hdr + kWsDone, 1u);
+    s_bad = 0;
+  }
+  __syncthreads();
+  TileEnd r;
+  r.last = (s_old & ~kDoneFailed) == static_cast<uint32_t>(ntiles) - 1u;
+  r.failed = tile_failed || (s_old & kDoneFailed) != 0u;
+  if (!r.last) return r;
+  // totals: the last tile has published its inclusive words before it counted itself done, but nothing
+  // orders the two for another workgroup; the words validate themselves, so wait for them (bounded)
+  const uint64_t* tot = ws.desc + static_cast<size_t>(ntiles - 1) * ncounters;
+  for (int c = threadIdx.x; c < ncounters; c += kTile) {
+    uint64_t x = ld_desc(tot + c);
+    uint32_t spins = 0;
+    while (!(desc_is_current(x, me.epoch) && (static_cast<uint32_t>(x) & kDescInclusive))) {
+      if (++spins > me.spin) {
+        st_agent(ws.hdr + kWsError, 1u);
+        s_bad = 1;
+        x = 0;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
+      x = ld_desc(tot + c);
+    }
+    s_tot[c] = static_cast<uint32_t>(x) & kDescCountMask;
+    st_agent(ws.hdr + kWsTotals + c, s_tot[c]);
+  }
+  __syncthreads();
+  r.failed = r.failed || s_bad != 0;
+  const uint32_t used = static_cast<uint32_t>(ntiles) * static_cast<uint32_t>(ncounters);
+  const uint32_t extent = max(ld_agent(ws.hdr + kWsExtent), used);
+  uint32_t next = (me.epoch + 1u) & kEpochMask;
+  if (next == 0u) {
+    for (uint32_t i = threadIdx.x; i < extent; i += kTile) st_desc(ws.desc + i, 0u, 0u);
+    next = 1u;
+  }
+  if (threadIdx.x == 0) {
+    st_agent(ws.hdr + kWsExtent, extent);
+    st_agent(ws.hdr + kWsFailed, r.failed ? 1u : 0u);
+    st_agent(ws.hdr + kWsTicket, 0u);
+    st_agent(ws.hdr + kWsDone, 0u);
+    st_agent(ws.hdr + kWsEpoch, next);
+  }
+  return r;
+}
+
+// One-time set-up of a workspace of nwords 32-bit words (a later launch may use any part of it).
+__global__ void scan_ws_init_kernel(uint32_t* ws, size_t nwords) {
+  for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < nwords;
+       i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+    uint32_t v = 0u;
+    if (i == kWsEpoch) v = 1u;
+    if (i == kWsMagic) v = kWsMagicValue;
+    ws[i] = v;
+  }
 }
 
 // LDS layout used by tile_scan: (kWavesPerTile + 3) rows of NC words:
@@ -65,20 +224,24 @@ constexpr int kLookbackLoads = 8;  // descriptor words in flight per thread and 
 // (negative = none); mem[j] says whether the token itself counts in that set.
 // On return rank[j] = number of earlier member tokens of class cls[j] in set j (0 when
 // cls[j] < 0); s_cnt row 5 holds the tile's exclusive base and row 4 its aggregate.
-// Must be called from uniform control flow by all kTile threads.
+// Returns true when the tile is poisoned (a wait gave up here or in a tile it builds on): its ranks mean
+// nothing.  Must be called from uniform control flow by all kTile threads.
 template <int NSETS>
-__device__ __forceinline__ void tile_scan(const int (&cls)[NSETS], const bool (&mem)[NSETS], int E,
-                                          uint32_t tile, const ScanWs& ws, uint32_t* s_cnt,
-                                          uint32_t spin_limit, uint32_t (&rank)[NSETS]) {
-  __shared__ int s_open;  // counters whose look-back has not reached an inclusive prefix yet
+__device__ __forceinline__ bool tile_scan(const int (&cls)[NSETS], const bool (&mem)[NSETS], int E,
+                                          const TileStart& me, const ScanWs& ws, uint32_t* s_cnt,
+                                          uint32_t (&rank)[NSETS]) {
+  __shared__ int s_open;    // counters whose look-back has not reached an inclusive prefix yet
+  __shared__ int s_poison;  // this tile's prefix cannot be trusted
   const int tid = threadIdx.x;
   const int w = tid / kWave;
   const int NC = NSETS * E;
+  const uint32_t tile = me.tile;
   uint32_t* s_agg = s_cnt + kWavesPerTile * NC;
   uint32_t* s_base = s_agg + NC;
   uint32_t* s_stop = s_base + NC;
 
   for (int c = tid; c < kScanLdsRows * NC; c += kTile) s_cnt[c] = 0;
+  if (tid == 0) s_poison = 0;
   __syncthreads();
 
   // 1. wave level
@@ -109,7 +272,7 @@ __device__ __forceinline__ void tile_scan(const int (&cls)[NSETS], const bool (&
       run += t;
     }
     s_agg[c] = run;
-    st_agent(ws.desc + static_cast<size_t>(tile) * NC + c, (tile == 0 ? kDescInclusive : kDescAggregate) | run);
+    st_desc(ws.desc + static_cast<size_t>(tile) * NC + c, me.epoch, (tile == 0 ? kDescInclusive : kDescAggregate) | run);
   }
 
   // 3. decoupled look-back
@@ -122,35 +285,35 @@ __device__ __forceinline__ void tile_scan(const int (&cls)[NSETS], const bool (&
     while (true) {
       const int nrows = min(win_rows, newest + 1);
       const int npairs = nrows * NC;
-      uint32_t word[kLookbackLoads];
+      uint64_t word[kLookbackLoads];
       // issue all loads of the window, then wait for the ones that are not published yet
 #pragma unroll
       for (int k = 0; k < kLookbackLoads; ++k) {
         const int i = tid + k * kTile;
-        word[k] = kDescAggregate;
+        word[k] = 0;
         if (i < npairs) {
           const int l = i / NC;
-          word[k] = ld_agent(ws.desc + static_cast<size_t>(newest - l) * NC + (i - l * NC));
+          word[k] = ld_desc(ws.desc + static_cast<size_t>(newest - l) * NC + (i - l * NC));
         }
       }
 #pragma unroll
       for (int k = 0; k < kLookbackLoads; ++k) {
         const int i = tid + k * kTile;
-        if (i < npairs && word[k] == 0) {
+        if (i < npairs && !desc_is_current(word[k], me.epoch)) {
           const int l = i / NC;
-          const uint32_t* ptr = ws.desc + static_cast<size_t>(newest - l) * NC + (i - l * NC);
+          const uint64_t* ptr = ws.desc + static_cast<size_t>(newest - l) * NC + (i - l * NC);
           uint32_t spins = 0;
           do {
-            if (++spins > spin_limit) {  // bounded wait: flag the workspace, carry on
-              st_agent(ws.error, 1u);
-              word[k] = kDescAggregate;
+            if (++spins > me.spin) {  // bounded wait: flag the workspace, poison the tile
+              st_agent(ws.hdr + kWsError, 1u);
+              word[k] = (static_cast<uint64_t>(me.epoch | kDescPoison) << 32) | kDescInclusive;
               break;
             }
             __builtin_amdgcn_s_sleep(1);
-            word[k] = ld_agent(ptr);
-          } while (word[k] == 0);
+            word[k] = ld_desc(ptr);
+          } while (!desc_is_current(word[k], me.epoch));
         }
-        if (i < npairs && (word[k] & kDescInclusive)) {
+        if (i < npairs && (static_cast<uint32_t>(word[k]) & kDescInclusive)) {
           const int l = i / NC;
           atomicMin(&s_stop[i - l * NC], static_cast<uint32_t>(static_cast<int>(tile) - 1 - (newest - l)));
         }
@@ -166,8 +329,9 @@ __device__ __forceinline__ void tile_scan(const int (&cls)[NSETS], const bool (&
           const uint32_t depth = static_cast<uint32_t>(static_cast<int>(tile) - 1 - (newest - l));
           const uint32_t stop = s_stop[c];
           if (depth <= stop) {
-            const uint32_t v = word[k] & kDescCountMask;
+            const uint32_t v = static_cast<uint32_t>(word[k]) & kDescCountMask;
             if (v) atomicAdd(&s_base[c], v);
+            if (desc_is_poisoned(word[k])) s_poison = 1;
             if (depth == stop) atomicSub(&s_open, 1);
           }
         }
@@ -177,8 +341,9 @@ __device__ __forceinline__ void tile_scan(const int (&cls)[NSETS], const bool (&
       newest -= nrows;
       __syncthreads();
     }
+    const uint32_t tag = me.epoch | (s_poison ? kDescPoison : 0u);
     for (int c = tid; c < NC; c += kTile)
-      st_agent(ws.desc + static_cast<size_t>(tile) * NC + c, kDescInclusive | ((s_base[c] + s_agg[c]) & kDescCountMask));
+      st_desc(ws.desc + static_cast<size_t>(tile) * NC + c, tag, kDescInclusive | ((s_base[c] + s_agg[c]) & kDescCountMask));
   }
   __syncthreads();
 
@@ -187,6 +352,7 @@ __device__ __forceinline__ void tile_scan(const int (&cls)[NSETS], const bool (&
     const int c = j * E + (cls[j] >= 0 ? cls[j] : 0);
     rank[j] = (cls[j] >= 0) ? s_base[c] + s_cnt[w * NC + c] + wrank[j] : 0u;
   }
+  return s_poison != 0;
 }
 
 }  // namespace lancet

@@ -8,9 +8,10 @@
 // The array's name is only a host-side stand-in for the symbol: the device address is looked up once
 // per device with hipGetSymbolAddress (with that device current) and kept; every launch gets that
 // pointer, never the name.  Nothing here calls hipMalloc, hipFree or an allocating library routine.
-// All calls on one GPU share the array, which keeps the last call's contents: the words that must be
-// zero are cleared by a fill kernel on the caller's stream at the start of every call, and calls that
-// overlap on one GPU (two streams, two host threads) race.
+// All calls on one GPU share the array, which keeps the last call's contents: it is a scan workspace, set
+// up (lancet_scan_workspace_init, a fill kernel on the caller's stream) by the first call on a device and
+// left ready for the next call by every call; calls that overlap on one GPU (two streams, two host
+// threads) race.
 #include "../../include/lancet_hip.h"
 #include "common.hpp"
 #include "launchers.hpp"
@@ -25,8 +26,9 @@ constexpr int kMaxDevices = 64;
 std::mutex g_lookup_mutex;
 std::atomic<void*> g_scratch_ptr[kMaxDevices];  // device address of `scratch` on device i, or null
 
-// Device address of this device's copy of the array; looked up on the first call on a device.
-int scratch_for_current_device(void** out) {
+// Device address of this device's copy of the array; looked up, and the workspace in it set up on `stream`,
+// on the first call on a device.
+int scratch_for_current_device(void** out, lancet_stream_t stream) {
   int device = -1;
   hipError_t e = hipGetDevice(&device);
   if (e != hipSuccess) return static_cast<int>(e);
@@ -39,6 +41,10 @@ int scratch_for_current_device(void** out) {
       e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
       if (e != hipSuccess) return static_cast<int>(e);
       if (!p) return static_cast<int>(hipErrorInvalidSymbol);
+      if (int r = lancet_scan_workspace_init(p, LANCET_NOALLOC_SCRATCH_BYTES, stream)) return r;
+      // later calls may come on other streams: the set-up is complete before any of them can start
+      e = hipStreamSynchronize(static_cast<hipStream_t>(stream));
+      if (e != hipSuccess) return static_cast<int>(e);
       g_scratch_ptr[device].store(p, std::memory_order_release);
     }
   }
@@ -58,9 +64,8 @@ extern "C" int lancet_moe_encode_noalloc(const void* data, const float* gate, co
   const size_t need = lancet_moe_encode_workspace_bytes(S, E, top_k);
   if (need > LANCET_NOALLOC_SCRATCH_BYTES) return LANCET_ERR_SCRATCH;
   void* ws = nullptr;
-  if (int r = scratch_for_current_device(&ws)) return r;
-  // the same kernels as lancet_moe_encode, which clears the words of the workspace it needs zero
-  // with a fill kernel before the scan
+  if (int r = scratch_for_current_device(&ws, stream)) return r;
+  // the same kernels as lancet_moe_encode
   return lancet_moe_encode(data, gate, gate2_noise, used_in, S, M, E, C, top_k, dtype, flags, gates_s,
                            indices_locations, used_out, elements_per_expert, dispatched, ws,
                            LANCET_NOALLOC_SCRATCH_BYTES, stream);

@@ -49,6 +49,63 @@ def _workspace(nbytes, device, given):
     return torch.empty(max(int(nbytes), 4), dtype=torch.uint8, device=device)
 
 
+class ScanWorkspace:
+    """Device memory of the position scan (moe_encode, moe_route, moe_encode_batch_prioritized, gen_location).
+
+    The scan keeps a few words of state in its workspace from call to call (launch epoch, ticket), so that no
+    call spends a launch on clearing it: the memory is set up once, here, on the current stream, and every call
+    leaves it ready for the next.  One workspace serves one call at a time: calls that may overlap (different
+    streams) need a workspace each.  No counterpart in the reference, whose scan kernel keeps no state
+    (tutel_moe_dispatch.cu:164-212)."""
+
+    def __init__(self, nbytes, device="cuda"):
+        nbytes = (max(int(nbytes), 8192) + 7) // 8 * 8
+        self.buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        capi.check(capi.load().lancet_scan_workspace_init(_p(self.buf), nbytes, _stream()), "lancet_scan_workspace_init")
+
+    @property
+    def nbytes(self):
+        return self.buf.numel()
+
+    def error(self):
+        """1 when a call on this workspace gave up a wait (its outputs then hold -1 for the tokens concerned and
+        for used_capacity) since the last read, else 0; synchronises the current stream and clears the word."""
+        err = C.c_int(0)
+        capi.check(capi.load().lancet_scan_workspace_error(_p(self.buf), _stream(), C.byref(err)),
+                   "lancet_scan_workspace_error")
+        return int(err.value)
+
+
+_scan_pool = {}
+
+
+def _scan_workspace(nbytes, device, given):
+    """The workspace a scan call uses: the caller's ScanWorkspace, or one kept per (device, stream) and grown on
+    demand (calls on one stream run one after the other, so they can share)."""
+    if given is not None:
+        if not isinstance(given, ScanWorkspace):
+            raise TypeError("workspace of a scan call must be an ops.ScanWorkspace (it is set up once and carries "
+                            "state from call to call), got %s" % type(given).__name__)
+        _need(given.buf.device == device and given.nbytes >= nbytes,
+              "workspace must live on the data's GPU and hold at least %d bytes" % nbytes)
+        return given
+    key = (device.index if device.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream(device).cuda_stream)
+    ws = _scan_pool.get(key)
+    if ws is None or ws.nbytes < nbytes:
+        with torch.cuda.device(device):
+            ws = ScanWorkspace(max(int(nbytes), 1 << 16), device)
+        _scan_pool[key] = ws
+    return ws
+
+
+def scan_errors():
+    """Number of scan workspaces kept by this module on which a wait gave up since the last check
+    (synchronises).  The reference aborts on any failure (src/common/cuda_utils.h:18-22); here the outputs of a
+    failed call hold -1 and this is the check a caller makes where it synchronises anyway."""
+    return sum(ws.error() for ws in list(_scan_pool.values()))
+
+
 def moe_capacity(S, E, capacity_factor):
     """C = int(float(cf) * ceil(S / E)) (src/op/dialect/cuda/moe.cc:107-109)."""
     return int(capi.load().lancet_moe_capacity(int(S), int(E), float(capacity_factor)))
@@ -113,11 +170,10 @@ def moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_
         disp = torch.empty((E, Cap, M), dtype=data.dtype, device=dev)
     else:
         gates_s, indloc, used_out, elems, disp = out
-    ws_bytes = moe_encode_workspace_bytes(S, E, top_k)
-    ws = _workspace(ws_bytes, dev, workspace)
+    ws = _scan_workspace(moe_encode_workspace_bytes(S, E, top_k), dev, workspace)
     st = lib.lancet_moe_encode(_p(data), _p(gate), _p(gate2_noise), _p(used_capacity), S, M, E, Cap, top_k, dt,
                                _flags(gate_is_logits, zero_tail, rows_at_used), _p(gates_s), _p(indloc),
-                               _p(used_out), _p(elems), _p(disp), _p(ws), ws.numel(), _stream())
+                               _p(used_out), _p(elems), _p(disp), _p(ws.buf), ws.nbytes, _stream())
     capi.check(st, "lancet_moe_encode")
     return gates_s, indloc, used_out, elems.view(torch.uint64) if elems.dtype == torch.int64 else elems, disp
 
@@ -140,9 +196,9 @@ def moe_route(gate, used_capacity, M, capacity_factor=1.0, top_k=1, gate_is_logi
                torch.empty((2, top_k * S), dtype=torch.int32, device=dev),
                torch.empty(E, dtype=torch.int32, device=dev), torch.empty(E, dtype=torch.int64, device=dev))
     gates_s, indloc, used_out, elems = out[:4]
-    ws = _workspace(moe_encode_workspace_bytes(S, E, top_k), dev, workspace)
+    ws = _scan_workspace(moe_encode_workspace_bytes(S, E, top_k), dev, workspace)
     st = lib.lancet_moe_route(_p(gate), _p(gate2_noise), _p(used_capacity), S, int(M), E, Cap, top_k, _flags(gate_is_logits, True),
-                              _p(gates_s), _p(indloc), _p(used_out), _p(elems), _p(ws), ws.numel(), _stream())
+                              _p(gates_s), _p(indloc), _p(used_out), _p(elems), _p(ws.buf), ws.nbytes, _stream())
     capi.check(st, "lancet_moe_route")
     return gates_s, indloc, used_out, elems
 
@@ -233,11 +289,10 @@ def moe_encode_batch_prioritized(data, gate, n_partitions=1, partition_id=0, cap
         disp = torch.empty((E, Cap, M), dtype=data.dtype, device=dev)
     else:
         gates_s, indloc, used_out, elems, disp = out
-    ws_bytes = moe_encode_bpr_workspace_bytes(S0, E, n_partitions)
-    ws = _workspace(ws_bytes, dev, workspace)
+    ws = _scan_workspace(moe_encode_bpr_workspace_bytes(S0, E, n_partitions), dev, workspace)
     st = lib.lancet_moe_encode_bpr(_p(data), _p(gate), S0, M, E, Cap, n_partitions, partition_id, dt,
                                    _flags(gate_is_logits, zero_tail), _p(gates_s), _p(indloc),
-                                   _p(used_out), _p(elems), _p(disp), _p(ws), ws.numel(), _stream())
+                                   _p(used_out), _p(elems), _p(disp), _p(ws.buf), ws.nbytes, _stream())
     capi.check(st, "lancet_moe_encode_bpr")
     return gates_s, indloc, used_out, elems.view(torch.uint64) if elems.dtype == torch.int64 else elems, disp
 

@@ -41,9 +41,11 @@ class PartitionedMoeLayer:
                      torch.empty(E, dtype=torch.int32, device=dev),
                      torch.empty(E, dtype=torch.int64, device=dev),
                      torch.empty((E, C, M), dtype=dtype, device=dev)) for _ in range(P)]
-        # one scan workspace per partition: encodes of neighbouring partitions never share one
-        self.ws = [torch.empty(ops.moe_encode_workspace_bytes(Sp, E, 1), dtype=torch.uint8, device=dev)
-                   for _ in range(P)]
+        # one scan workspace per partition: encodes of neighbouring partitions never share one; they are set up
+        # on the current stream and used on the routing / compute streams, hence the synchronisation
+        with torch.cuda.device(dev):
+            self.ws = [ops.ScanWorkspace(ops.moe_encode_workspace_bytes(Sp, E, 1), dev) for _ in range(P)]
+            torch.cuda.current_stream().synchronize()
         self.wire = [torch.empty(E * C * M, dtype=dtype, device=dev) for _ in range(P)]
         self.recv = [torch.empty((E, C, M), dtype=dtype, device=dev) for _ in range(P)]
         self.out = torch.empty((S, M), dtype=dtype, device=dev)
@@ -160,7 +162,9 @@ class RoutedOnceMoeLayer:
         P, K, Sp = n_partitions, top_k, self.Sp
         self.whole = (torch.empty(K * S, dtype=torch.float32, device=dev), torch.empty((2, K * S), dtype=torch.int32, device=dev),
                       torch.empty(E, dtype=torch.int32, device=dev), torch.empty(E, dtype=torch.int64, device=dev))
-        self.whole_ws = torch.empty(ops.moe_encode_workspace_bytes(S, E, K), dtype=torch.uint8, device=dev)
+        with torch.cuda.device(dev):   # set up on the current stream, used on the routing stream
+            self.whole_ws = ops.ScanWorkspace(ops.moe_encode_workspace_bytes(S, E, K), dev)
+            torch.cuda.current_stream().synchronize()
         self.ranges = (torch.empty((K * P, E), dtype=torch.int64, device=dev),
                        torch.empty((K * P, E), dtype=torch.int64, device=dev))
         self.ranges_ws = torch.empty(max(4, K * P * E * 4), dtype=torch.uint8, device=dev)

@@ -152,6 +152,7 @@ int raf_hip_bind_workspace(void* h, int i, void* data) {
     const auto& reqs = c->env->GetRequests();
     RAF_CHECK(i >= 0 && i < static_cast<int>(reqs.size()), "workspace index out of range");
     *reqs[i].dest = data;
+    c->env->WorkspaceBound();
   });
 }
 int raf_hip_num_arg_indices(void* h) { return static_cast<int>(static_cast<Call*>(h)->env->arg_indices.size()); }

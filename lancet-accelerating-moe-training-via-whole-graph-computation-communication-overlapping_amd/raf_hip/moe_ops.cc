@@ -40,6 +40,19 @@ void CheckStatus(int status, const char* what) {
                 std::to_string(status) + ")");
 }
 
+// The scan's workspace carries state from call to call and is set up once (lancet_scan_workspace_init).  The
+// executor binds the memory after the OpEnv is built and may bind other memory later (an interpreter keeps one
+// allocation per cached OpEnv, a VM allocates before every Execute, src/impl/vm/vm.cc:1260-1266): the OpEnv sets
+// up whatever address it has not set up yet, on the stream it executes on.
+struct ScanWorkspaceState {
+  void* ready = nullptr;  // the address lancet_scan_workspace_init has run on
+  void Ensure(void* ws, size_t nbytes, void* stream) {
+    if (ws == ready) return;
+    CheckStatus(lancet_scan_workspace_init(ws, nbytes, stream), "lancet_scan_workspace_init");
+    ready = ws;
+  }
+};
+
 Tensor MakeOut(int device_id, DTypeCode code, int bits, std::vector<int64_t> shape) {
   Tensor t;
   t.device_id = device_id;
@@ -146,6 +159,7 @@ class MoeEncode : public OpEnv {
     const float* noise = has_noise_ ? static_cast<const float*>(inputs[3].AsTensor().data) : nullptr;
     const auto& out = output.AsTuple();
     RAF_CHECK(out.size() == 5, "Expected output to be a 5-Tuple");
+    scan_ws_.Ensure(ws_, ws_bytes_, GetStream(device_id_));
     CheckStatus(lancet_moe_encode(data.data, static_cast<const float*>(gate.data), noise,
                                   static_cast<const int32_t*>(used.data), shape_.S, shape_.M, shape_.E, shape_.C,
                                   top_k_, dtype_, flags_, static_cast<float*>(out[0].AsTensor().data),
@@ -156,6 +170,7 @@ class MoeEncode : public OpEnv {
                 "lancet_moe_encode");
   }
 
+  void WorkspaceBound() override { scan_ws_.ready = nullptr; }
   std::string name() const override { return "raf.op.hip.moe_encode"; }
   static OpEnv* make(const CallValues& cv) { return new MoeEncode(cv); }
 
@@ -166,6 +181,7 @@ class MoeEncode : public OpEnv {
   bool has_noise_ = false;
   void* ws_ = nullptr;
   size_t ws_bytes_ = 0;
+  ScanWorkspaceState scan_ws_;
 };
 
 // =====================================================================================
@@ -207,6 +223,7 @@ class MoeEncodeBatchPrioritized : public OpEnv {
   void Execute(const std::vector<Value>& inputs, Value output) override {
     const auto& out = output.AsTuple();
     RAF_CHECK(out.size() == 5, "Expected output to be a 5-Tuple");
+    scan_ws_.Ensure(ws_, ws_bytes_, GetStream(device_id_));
     CheckStatus(lancet_moe_encode_bpr(inputs[0].AsTensor().data, static_cast<const float*>(inputs[1].AsTensor().data),
                                       orig_S_, shape_.M, shape_.E, shape_.C, n_partitions_, partition_id_, dtype_,
                                       flags_, static_cast<float*>(out[0].AsTensor().data),
@@ -217,6 +234,7 @@ class MoeEncodeBatchPrioritized : public OpEnv {
                 "lancet_moe_encode_bpr");
   }
 
+  void WorkspaceBound() override { scan_ws_.ready = nullptr; }
   std::string name() const override { return "raf.op.hip.moe_encode_batch_prioritized"; }
   static OpEnv* make(const CallValues& cv) { return new MoeEncodeBatchPrioritized(cv); }
 
@@ -227,6 +245,7 @@ class MoeEncodeBatchPrioritized : public OpEnv {
   unsigned flags_;
   void* ws_ = nullptr;
   size_t ws_bytes_ = 0;
+  ScanWorkspaceState scan_ws_;
 };
 
 // =====================================================================================

@@ -139,6 +139,9 @@ class OpEnv {
     workspace_.push_back({dest, device_id, nbytes});
   }
   const std::vector<WorkspaceRequest>& GetRequests() const { return workspace_; }
+  // Called by the executor after it has written a request's destination: the memory behind a workspace is
+  // new (or has been used by others since the last Execute), whatever its address.
+  virtual void WorkspaceBound() {}
 
   // Data input indices in the argument list (used by the VM executor).
   std::vector<int> arg_indices;

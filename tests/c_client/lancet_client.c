@@ -52,10 +52,11 @@ int main(void) {
   CHECK_HIP(hipMalloc((void**)&d_elems, E * sizeof(uint64_t)));
   CHECK_HIP(hipMalloc((void**)&d_disp, E * 2 * M * sizeof(float)));
   CHECK_HIP(hipMalloc((void**)&d_out, S * M * sizeof(float)));
-  CHECK_HIP(hipMalloc(&d_ws, ws_bytes ? ws_bytes : 4));
+  CHECK_HIP(hipMalloc(&d_ws, ws_bytes));
   CHECK_HIP(hipMemcpy(d_gate, gate, sizeof(gate), hipMemcpyHostToDevice));
   CHECK_HIP(hipMemcpy(d_data, data, sizeof(data), hipMemcpyHostToDevice));
   CHECK_HIP(hipMemset(d_disp, 0xff, E * 2 * M * sizeof(float))); /* stale contents must not survive */
+  CHECK_LANCET(lancet_scan_workspace_init(d_ws, ws_bytes, stream)); /* once per workspace */
 
   CHECK_LANCET(lancet_moe_encode(d_data, d_gate, NULL, NULL, S, M, E, C, 1, LANCET_F32, 0u, d_gates_s, d_il, d_used,
                                  d_elems, d_disp, d_ws, ws_bytes, stream));

@@ -91,5 +91,8 @@ def test_hip_path_reproduces_fixtures(pkg):
     for i in range(3):
         want = f["p3_%d" % i]
         assert np.abs(to_np(p[i]).astype(np.float64) - want).max() <= 1e-6 * np.abs(want).max()
-        np.testing.assert_allclose(to_np(m[i]), f["m3_%d" % i], rtol=1e-5, atol=1e-12)
-        np.testing.assert_allclose(to_np(v[i]), f["v3_%d" % i], rtol=1e-5, atol=1e-15)
+        # m and v: 1e-5 relative, with a floor of 1e-6 of the tensor's largest entry (an entry of m in which
+        # beta1 * m and (1 - beta1) * g / ||g|| cancel carries the last-place difference of ||g||, whose sum order
+        # differs between schedules, at its full absolute size)
+        for got_t, name in ((m[i], "m3_%d" % i), (v[i], "v3_%d" % i)):
+            np.testing.assert_allclose(to_np(got_t), f[name], rtol=1e-5, atol=1e-6 * np.abs(f[name]).max())

@@ -37,7 +37,7 @@ def test_encode_decode_graph_replays(pkg, k, dt):
     outs = (torch.empty(k * S, device="cuda"), torch.empty((2, k * S), dtype=torch.int32, device="cuda"),
             torch.empty(E, dtype=torch.int32, device="cuda"), torch.empty(E, dtype=torch.int64, device="cuda"),
             torch.empty((E, C, M), dtype=dt, device="cuda"))
-    ws = torch.empty(ops.moe_encode_workspace_bytes(S, E, k), dtype=torch.uint8, device="cuda")
+    ws = ops.ScanWorkspace(ops.moe_encode_workspace_bytes(S, E, k))
     dec = torch.empty((S, M), dtype=dt, device="cuda")
     zero = torch.zeros(E, dtype=torch.int32, device="cuda")
 

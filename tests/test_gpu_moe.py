@@ -272,6 +272,7 @@ def test_launch_gen_location_and_encode_forward(pkg):
     nws = lib.lancet_gen_location_workspace_bytes(S, E)
     ws = torch.empty(nws, dtype=torch.uint8, device="cuda")
     p = lambda t: C.c_void_p(t.data_ptr())
+    assert lib.lancet_scan_workspace_init(p(ws), nws, None) == 0
     st = lib.lancet_launch_gen_location(p(d_idx), p(d_used), p(d_loc), p(d_uo), p(d_el), Cap, S, E, M, p(ws), nws, None)
     assert st == 0
     torch.cuda.synchronize()
@@ -291,29 +292,125 @@ def test_launch_gen_location_and_encode_forward(pkg):
         np.testing.assert_array_equal(to_np(out), mo.scatter_rows(data, widx, wloc, E, Cap, avail))
 
 
-def test_bounded_wait_flags_the_workspace(pkg):
-    """A spin limit of 1 makes look-back waits give up at once: the kernel must still finish and
-    flag the workspace; the default limit must leave the flag clear."""
+@pytest.mark.parametrize("k", [1, 2])
+def test_bounded_wait_flags_the_workspace(pkg, k):
+    """A spin limit of 1 makes look-back waits give up at once: the kernels must still finish; a call in which a
+    wait gave up sets the workspace's sticky error word and shows it in its outputs without a synchronisation
+    (used_capacity = -1, and -1 for every token whose position depended on the wait); every token that is not
+    marked has its correct position; the default limit leaves the word clear and the next call is whole."""
     import ctypes as C
     lib = pkg.capi.load()
+    ops = pkg.ops
     S, M, E = 65536, 4, 8
     data, logits = make_inputs(1, S, M, E)
     d_data, d_gate = dev(data), dev(logits)
-    ws = torch.empty(pkg.ops.moe_encode_workspace_bytes(S, E, 1), dtype=torch.uint8, device="cuda")
-    err = C.c_int(-1)
-    pkg.ops.moe_encode(d_data, d_gate, None, 1.0, workspace=ws)
-    assert lib.lancet_scan_workspace_error(C.c_void_p(ws.data_ptr()), None, C.byref(err)) == 0 and err.value == 0
-    lib.lancet_debug_set_spin_limit(1)
-    try:
-        pkg.ops.moe_encode(d_data, d_gate, None, 1.0, workspace=ws)
+    enc = mo.moe_encode_top2 if k == 2 else mo.moe_encode
+    want = enc(data, logits, np.zeros(E, np.int32), 1.0, gate_is_logits=True, fast_scatter=True)
+    ws = ops.ScanWorkspace(ops.moe_encode_workspace_bytes(S, E, k))
+    ops.moe_encode(d_data, d_gate, None, 1.0, top_k=k, gate_is_logits=True, workspace=ws)
+    assert ws.error() == 0
+    gave_up = 0
+    for _ in range(3):
+        assert lib.lancet_debug_scan_workspace_spin_limit(C.c_void_p(ws.buf.data_ptr()), 1, None) == 0
+        got = ops.moe_encode(d_data, d_gate, None, 1.0, top_k=k, gate_is_logits=True, workspace=ws)
+        assert lib.lancet_debug_scan_workspace_spin_limit(C.c_void_p(ws.buf.data_ptr()), 0, None) == 0
         torch.cuda.synchronize()   # terminates
-        assert lib.lancet_scan_workspace_error(C.c_void_p(ws.data_ptr()), None, C.byref(err)) == 0
-        assert err.value in (0, 1)   # 1 whenever a predecessor was not ready at the first poll
-    finally:
-        lib.lancet_debug_set_spin_limit(0)
-    want = mo.moe_encode(data, logits, np.zeros(E, np.int32), 1.0, fast_scatter=True)
-    got = pkg.ops.moe_encode(d_data, d_gate, None, 1.0, workspace=ws)
-    np.testing.assert_array_equal(to_np(got[1]), want[1])
+        il, used = to_np(got[1]), to_np(got[2])
+        flagged = ws.error()       # 1 whenever a predecessor's word was not there at the first poll
+        assert ws.error() == 0     # the reader clears the word
+        marked = (il[0] == -1) & (il[1] == -1)
+        if marked.any():           # some position depended on a wait that gave up
+            gave_up += 1
+            assert flagged == 1
+            assert (used == -1).all(), "a failed scan must show in used_capacity"
+            if k == 2:
+                assert marked.all()
+            else:
+                # what is not marked is right (dropped tokens of the top-1 op keep idx -1 and their rank)
+                np.testing.assert_array_equal(il[:, ~marked], want[1][:, ~marked])
+        else:                      # no wait gave up, or nothing was built on one that did
+            np.testing.assert_array_equal(il, want[1])
+            np.testing.assert_array_equal(used, want[2])
+        # the workspace is ready for the next call whatever happened
+        got = ops.moe_encode(d_data, d_gate, None, 1.0, top_k=k, gate_is_logits=True, workspace=ws)
+        np.testing.assert_array_equal(to_np(got[1]), want[1])
+        np.testing.assert_array_equal(to_np(got[2]), want[2])
+        np.testing.assert_array_equal(to_np(got[4]), want[4])
+        assert ws.error() == 0
+    assert gave_up > 0, "256 tiles with a wait of one poll: some wait gives up"
+
+
+def test_scan_on_a_workspace_that_is_not_set_up(pkg):
+    """A call handed memory that lancet_scan_workspace_init never saw must not hang or run wild: it marks its
+    outputs (-1) and sets the error word; after the set-up the same memory works."""
+    import ctypes as C
+    lib = pkg.capi.load()
+    capi = pkg.capi
+    S, M, E = 3000, 8, 8
+    data, logits = make_inputs(2, S, M, E)
+    d_data, d_gate = dev(data), dev(logits)
+    p = lambda t: C.c_void_p(t.data_ptr())
+    for k in (1, 2):
+        nws = int(lib.lancet_moe_encode_workspace_bytes(S, E, k))
+        for fill in (0, 0xff):
+            ws = torch.full((nws,), fill, dtype=torch.uint8, device="cuda")
+            Cap = ops_cap = pkg.ops.moe_capacity(S, E, float(k))
+            outs = (torch.zeros(k * S, device="cuda"), torch.zeros((2, k * S), dtype=torch.int32, device="cuda"),
+                    torch.zeros(E, dtype=torch.int32, device="cuda"), torch.zeros(E, dtype=torch.int64, device="cuda"),
+                    torch.zeros((E, Cap, M), device="cuda"))
+            st = lib.lancet_moe_encode(p(d_data), p(d_gate), None, None, S, M, E, Cap, k, capi.F32, capi.GATE_IS_LOGITS,
+                                       *[p(t) for t in outs], p(ws), nws, None)
+            assert st == 0
+            torch.cuda.synchronize()
+            assert (to_np(outs[1]) == -1).all() and (to_np(outs[2]) == -1).all()
+            assert (to_np(outs[4]) == 0).all(), "no token has a place: the buffer is all tail"
+            err = C.c_int(0)
+            assert lib.lancet_scan_workspace_error(p(ws), None, C.byref(err)) == 0 and err.value == 1
+            assert lib.lancet_scan_workspace_init(p(ws), nws, None) == 0
+            st = lib.lancet_moe_encode(p(d_data), p(d_gate), None, None, S, M, E, Cap, k, capi.F32, capi.GATE_IS_LOGITS,
+                                       *[p(t) for t in outs], p(ws), nws, None)
+            assert st == 0
+            enc = mo.moe_encode_top2 if k == 2 else mo.moe_encode
+            want = enc(data, logits, np.zeros(E, np.int32), 1.0, gate_is_logits=True, fast_scatter=True)
+            np.testing.assert_array_equal(to_np(outs[1]), want[1])
+            np.testing.assert_array_equal(to_np(outs[4]), want[4])
+            assert lib.lancet_scan_workspace_error(p(ws), None, C.byref(err)) == 0 and err.value == 0
+
+
+def test_scan_workspace_is_reused_across_shapes(pkg):
+    """One workspace, calls of different token counts, expert counts and top_k one after the other: descriptor
+    words of earlier calls lie anywhere in the table and must never be taken for the running call's."""
+    ops = pkg.ops
+    ws = ops.ScanWorkspace(1 << 20)
+    rng = np.random.default_rng(5)
+    shapes = [(5000, 32, 2), (700, 8, 1), (5000, 32, 1), (2049, 64, 2), (256, 2, 2), (5000, 32, 2), (1, 4, 1), (4097, 16, 1)]
+    for i, (S, E, k) in enumerate(shapes * 2):
+        data, logits = make_inputs(200 + i, S, 8, E)
+        enc = mo.moe_encode_top2 if k == 2 else mo.moe_encode
+        want = enc(data, logits, np.zeros(E, np.int32), 1.0, gate_is_logits=True, fast_scatter=True)
+        got = ops.moe_encode(dev(data), dev(logits), None, 1.0, top_k=k, gate_is_logits=True, workspace=ws)
+        np.testing.assert_array_equal(to_np(got[1]), want[1])
+        np.testing.assert_array_equal(to_np(got[2]), want[2])
+        if i % 3 == 0:   # batch-prioritised calls share it too
+            gate = mo.softmax_rows(logits)
+            wb = mo.moe_encode_bpr(data, gate, 1, 0, 1.0, fast_scatter=True)
+            gb = ops.moe_encode_batch_prioritized(dev(data), dev(gate), 1, 0, 1.0, workspace=ws)
+            np.testing.assert_array_equal(to_np(gb[1]), wb[1])
+    # the batch-prioritised call keeps per-token data behind its descriptor table, where a later call with a
+    # larger table expects descriptors: small expert ids and arbitrary floats must not pass for them
+    data, logits = make_inputs(300, 32768, 8, 8)
+    gate = mo.softmax_rows(logits)
+    wb = mo.moe_encode_bpr(data, gate, 1, 0, 1.0, fast_scatter=True)
+    gb = ops.moe_encode_batch_prioritized(dev(data), dev(gate), 1, 0, 1.0, workspace=ws)
+    np.testing.assert_array_equal(to_np(gb[1]), wb[1])
+    for i, (S, E, k) in enumerate([(20000, 32, 2), (32768, 64, 1), (9000, 128, 2)]):
+        data, logits = make_inputs(310 + i, S, 8, E)
+        enc = mo.moe_encode_top2 if k == 2 else mo.moe_encode
+        want = enc(data, logits, np.zeros(E, np.int32), 1.0, gate_is_logits=True, fast_scatter=True)
+        got = ops.moe_encode(dev(data), dev(logits), None, 1.0, top_k=k, gate_is_logits=True, workspace=ws)
+        np.testing.assert_array_equal(to_np(got[1]), want[1])
+        np.testing.assert_array_equal(to_np(got[2]), want[2])
+    assert ws.error() == 0
 
 
 def test_encode_without_tail_zero_fill_feeds_redispatch(pkg):

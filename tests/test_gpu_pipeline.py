@@ -70,7 +70,8 @@ def test_concurrent_calls_on_separate_streams_share_no_state(pkg):
         alone_out = ops.moe_decode(alone[4], alone[0], alone[1], top_k=k)
         outs = tuple(torch.empty_like(t) if t.dtype != torch.uint64 else torch.empty(t.shape, dtype=torch.int64, device="cuda")
                      for t in alone)
-        ws = torch.empty(ops.moe_encode_workspace_bytes(S, E, k), dtype=torch.uint8, device="cuda")
+        ws = ops.ScanWorkspace(ops.moe_encode_workspace_bytes(S, E, k))
+        torch.cuda.synchronize()   # set up on this stream, used on the streams below
         jobs.append((k, d_data, d_logits, alone, alone_out, outs, ws, torch.empty_like(alone_out), torch.cuda.Stream()))
     torch.cuda.synchronize()
     for _ in range(3):

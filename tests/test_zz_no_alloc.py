@@ -35,6 +35,7 @@ def _encode_both(pkg, lib, data, gate, used_in, cf, k, flags):
     ref = _outputs(S, M, E, Cap, k, data.dtype)
     ws_bytes = lib.lancet_moe_encode_workspace_bytes(S, E, k)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+    assert lib.lancet_scan_workspace_init(_p(ws), ws_bytes, st) == 0
     rc = lib.lancet_moe_encode(_p(data), _p(gate), None, _p(used_in), S, M, E, Cap, k, dt, flags, *[_p(t) for t in ref],
                                _p(ws), ws_bytes, st)
     assert rc == 0, capi.status_string(rc)

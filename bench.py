@@ -649,7 +649,7 @@ def main():
 
     def route_only():
         st = lib.lancet_moe_route(p(logits), None, p(used_in), S, M, E, Cap, K, capi.GATE_IS_LOGITS, p(outs[0]),
-                                  p(outs[1]), p(outs[2]), p(outs[3]), p(ws), ws.numel(), stream)
+                                  p(outs[1]), p(outs[2]), p(outs[3]), p(ws.buf), ws.nbytes, stream)
         assert st == 0
 
     if args.only in ("scatter", "decode", "route"):

@@ -405,9 +405,11 @@ int lancet_lans_plan_norms(lancet_lans_plan_t plan, float* norms4xT, lancet_stre
  * allocation; every call that uses the workspace leaves it ready for the next, so that no call spends a
  * launch on clearing it.  A call that is handed a workspace that is not set up launches nothing harmful:
  * it sets every indices/locations entry and every used_out entry to -1 and the error word.
- * Every wait inside the scan is bounded.  A wait that gives up sets the workspace's sticky error word,
- * and the tokens whose positions depend on it get indices = locations = -1 and used_out = -1 (all of them,
- * for top_k = 2): a consumer sees the failure in the outputs without a synchronisation.
+ * Every wait inside the scan is bounded.  A wait that gives up sets the workspace's sticky error word, and
+ * every token whose position was built on it gets indices = locations = -1 (gates_s 0 for top_k = 2), as if
+ * dropped, so that no consumer moves a row on a wrong position; when the totals themselves were built on it,
+ * used_out = -1 for every expert (elements_per_expert 0; all tokens marked for top_k = 2).  What is not marked
+ * is right.  The workspace stays usable.
  * lancet_scan_workspace_error reads (synchronising `stream`) and clears the error word: *error_out = 1
  * when any call on this workspace gave up a wait, or found it not set up, since the last read. */
 int lancet_scan_workspace_init(void* workspace, size_t workspace_bytes, lancet_stream_t stream);

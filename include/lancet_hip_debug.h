@@ -36,6 +36,10 @@ int lancet_lans_plan_debug_last_resident(lancet_lans_plan_t plan, int* slots);
  * asynchronously on `stream`.  Lets a host test exercise the bounded wait while every kernel still exits
  * normally. */
 int lancet_debug_scan_workspace_spin_limit(void* workspace, unsigned limit, lancet_stream_t stream);
+/* Test hook: sets the launch epoch of a scan workspace that is set up and idle (1 .. 2^30 - 1), asynchronously on
+ * `stream`.  The epoch tags the scan's descriptor words and moves on by one per call; the call that runs with the
+ * last value clears the descriptor table before the epoch starts again at 1.  Lets a test reach that call. */
+int lancet_debug_scan_workspace_epoch(void* workspace, unsigned epoch, lancet_stream_t stream);
 /* Measurement aid (no counterpart in the reference): one plain streaming kernel over `bytes` bytes (a multiple
  * of 4096), one 16-byte non-temporal access per thread, workgroups in address order: the launch shape that
  * streams fastest on this device.  kind 0 reads src, 1 fills dst with zeros, 2 copies src to dst.  bench.py

@@ -97,6 +97,7 @@ SIGNATURES = {
     "lancet_lans_plan_debug_last_resident": (_int, [_vp, C.POINTER(_int)]),
     "lancet_lans_plan_resident_capacity": (_int, [_vp, C.POINTER(_int), C.POINTER(_int)]),
     "lancet_debug_scan_workspace_spin_limit": (_int, [_vp, _u32, _vp]),
+    "lancet_debug_scan_workspace_epoch": (_int, [_vp, _u32, _vp]),
     "lancet_scan_workspace_init": (_int, [_vp, _sz, _vp]),
     "lancet_scan_workspace_error": (_int, [_vp, _vp, C.POINTER(_int)]),
 }

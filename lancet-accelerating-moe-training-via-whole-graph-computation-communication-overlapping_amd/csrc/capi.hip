@@ -74,6 +74,13 @@ extern "C" int lancet_debug_scan_workspace_spin_limit(void* workspace, unsigned 
   return rc(run_scan_ws_set_spin(workspace, limit, S_(stream)));
 }
 
+extern "C" int lancet_debug_scan_workspace_epoch(void* workspace, unsigned epoch, lancet_stream_t stream) {
+  if (!workspace) return LANCET_ERR_NULL;
+  if (misaligned(workspace, 8)) return LANCET_ERR_ALIGN;
+  if (epoch < 1u || epoch > 0x3fffffffu) return LANCET_ERR_SHAPE;
+  return rc(run_scan_ws_set_epoch(workspace, epoch, S_(stream)));
+}
+
 extern "C" int lancet_scan_workspace_init(void* workspace, size_t workspace_bytes, lancet_stream_t stream) {
   if (!workspace) return LANCET_ERR_NULL;
   if (misaligned(workspace, 8)) return LANCET_ERR_ALIGN;

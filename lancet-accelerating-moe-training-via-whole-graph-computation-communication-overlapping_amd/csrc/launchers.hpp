@@ -17,6 +17,7 @@ size_t bpr_workspace_bytes(int64_t S0, int64_t S, int64_t E);
 // one-time set-up of a scan workspace; its bound for waits; its sticky error word, read and cleared
 hipError_t run_scan_ws_init(void* ws, size_t nbytes, hipStream_t st);
 hipError_t run_scan_ws_set_spin(void* ws, uint32_t limit, hipStream_t st);
+hipError_t run_scan_ws_set_epoch(void* ws, uint32_t epoch, hipStream_t st);
 hipError_t run_scan_ws_take_error(void* ws, int* error_out, hipStream_t st);
 
 hipError_t run_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t st);

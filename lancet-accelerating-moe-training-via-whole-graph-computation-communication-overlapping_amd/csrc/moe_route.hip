@@ -188,26 +188,30 @@ __global__ __launch_bounds__(kTile) void route_scan_kernel(RouteArgs a) {
       }
       if (a.gates_s) a.gates_s[s] = p[0];
     }
+    if (static_cast<int>(tile) == a.ntiles - 1) {
+      // the last tile's inclusive prefix is the total; poisoned, it is worth nothing
+      const uint32_t* s_agg = s_cnt + kWavesPerTile * a.E;
+      const uint32_t* s_base = s_agg + a.E;
+      for (int c = tid; c < a.E; c += kTile) {
+        const int64_t used = a.used_in ? a.used_in[c] : 0;
+        const int64_t total = static_cast<int64_t>(s_base[c]) + s_agg[c];
+        const int64_t uo = min(used + total, static_cast<int64_t>(a.C));
+        a.used_out[c] = poisoned ? -1 : static_cast<int32_t>(uo);
+        a.elems_out[c] = poisoned ? 0 : static_cast<uint64_t>((uo - used) * a.M);
+      }
+    }
   } else {
+    // raw values for finalize_top2_kernel; a poisoned tile marks its tokens, which that kernel passes on
     if (valid) {
 #pragma unroll
       for (int j = 0; j < K; ++j) {
-        a.idx_out[static_cast<size_t>(j) * a.S + s] = e[j];
-        a.loc_out[static_cast<size_t>(j) * a.S + s] = static_cast<int>(rank[j]);
+        a.idx_out[static_cast<size_t>(j) * a.S + s] = poisoned ? -1 : e[j];
+        a.loc_out[static_cast<size_t>(j) * a.S + s] = poisoned ? -1 : static_cast<int>(rank[j]);
         a.gates_s[static_cast<size_t>(j) * a.S + s] = p[j];
       }
     }
   }
-  // the tile that finishes last knows the totals and whether any tile was poisoned
-  const TileEnd te = tile_end(a.ws, me, a.ntiles, K * a.E, poisoned, s_cnt);
-  if (K == 1 && te.last) {
-    for (int c = tid; c < a.E; c += kTile) {
-      const int64_t used = a.used_in ? a.used_in[c] : 0;
-      const int64_t uo = min(used + static_cast<int64_t>(s_cnt[c]), static_cast<int64_t>(a.C));
-      a.used_out[c] = te.failed ? -1 : static_cast<int32_t>(uo);
-      a.elems_out[c] = te.failed ? 0 : static_cast<uint64_t>((uo - used) * a.M);
-    }
-  }
+  tile_end(a.ws, me, a.ntiles, K * a.E);
 }
 
 // Completes top-2 routing once all tiles are done: slot 1 is an ordinary top-1 encode with
@@ -218,9 +222,10 @@ __global__ __launch_bounds__(kTile) void finalize_top2_kernel(RouteArgs a) {
   const int s = blockIdx.x * kTile + threadIdx.x;
   // a workspace that is not set up: route_scan_kernel has marked every output already
   if (ld_agent(a.ws.hdr + kWsMagic) != kWsMagicValue) return;
-  // totals of both slots [2][E] and the verdict of the scan, as its last tile left them in the header
-  const uint32_t* tot = a.ws.hdr + kWsTotals;
-  const bool poisoned = ld_agent(a.ws.hdr + kWsFailed) != 0u;
+  // totals of both slots = the last tile's inclusive descriptors, [2][E]; if that tile was poisoned there are
+  // no totals and every token is marked, else the tokens of poisoned tiles carry marks of their own
+  const uint64_t* tot = a.ws.desc + static_cast<size_t>(a.ntiles - 1) * 2 * a.E;
+  const bool poisoned = desc_is_poisoned(ld_desc(tot));
   if (s < a.S) {
     if (poisoned) {
       a.idx_out[s] = a.idx_out[a.S + s] = -1;
@@ -233,7 +238,7 @@ __global__ __launch_bounds__(kTile) void finalize_top2_kernel(RouteArgs a) {
       const int u1 = (a.used_in && in1) ? a.used_in[e1] : 0;
       const int u2 = (a.used_in && in2) ? a.used_in[e2] : 0;
       const bool keep1 = in1 && r1 < a.C - u1;
-      const int64_t after1 = min(static_cast<int64_t>(u2) + (in2 ? tot[e2] : 0u),
+      const int64_t after1 = min(static_cast<int64_t>(u2) + (in2 ? static_cast<uint32_t>(ld_desc(tot + e2)) & kDescCountMask : 0u),
                                  static_cast<int64_t>(a.C));
       const bool keep2 = in2 && r2 < a.C - after1;
       a.idx_out[s] = keep1 ? e1 : -1;
@@ -250,7 +255,8 @@ __global__ __launch_bounds__(kTile) void finalize_top2_kernel(RouteArgs a) {
   if (blockIdx.x == 0) {
     for (int c = threadIdx.x; c < a.E; c += kTile) {
       const int64_t used = a.used_in ? a.used_in[c] : 0;
-      const int64_t total = static_cast<int64_t>(tot[c]) + tot[a.E + c];
+      const int64_t total = static_cast<int64_t>(static_cast<uint32_t>(ld_desc(tot + c)) & kDescCountMask) +
+                            (static_cast<uint32_t>(ld_desc(tot + a.E + c)) & kDescCountMask);
       const int64_t uo = min(used + total, static_cast<int64_t>(a.C));
       a.used_out[c] = poisoned ? -1 : static_cast<int32_t>(uo);
       a.elems_out[c] = poisoned ? 0 : static_cast<uint64_t>((uo - used) * a.M);
@@ -471,19 +477,21 @@ __global__ __launch_bounds__(kTile) void bpr_scan_kernel(BprArgs a) {
     a.loc_out[sl] = loc;
     a.gates_s[sl] = prio;
   }
-  const TileEnd te = tile_end(a.ws, me, a.ntiles, 2 * a.E, poisoned, s_cnt);
-  if (te.last) {
+  if (static_cast<int>(tile) == a.ntiles - 1) {
+    const uint32_t* s_agg = s_cnt + kWavesPerTile * 2 * a.E;
+    const uint32_t* s_base = s_agg + 2 * a.E;
     for (int c = tid; c < a.E; c += kTile) {
       const int64_t q = static_cast<int32_t>(par_value(a.par + a.E + c));
       const int64_t tb = static_cast<int32_t>(par_value(a.par + 2 * a.E + c));
-      const int64_t above = s_cnt[c];
-      const int64_t ties = s_cnt[a.E + c];
+      const int64_t above = static_cast<int64_t>(s_base[c]) + s_agg[c];
+      const int64_t ties = static_cast<int64_t>(s_base[a.E + c]) + s_agg[a.E + c];
       const int64_t kept = above + min(tb + ties, q) - min(tb, q);
       const int64_t uo = min(kept, static_cast<int64_t>(a.C));
-      a.used_out[c] = te.failed ? -1 : static_cast<int32_t>(uo);
-      a.elems_out[c] = te.failed ? 0 : static_cast<uint64_t>(uo * a.M);
+      a.used_out[c] = poisoned ? -1 : static_cast<int32_t>(uo);
+      a.elems_out[c] = poisoned ? 0 : static_cast<uint64_t>(uo * a.M);
     }
   }
+  tile_end(a.ws, me, a.ntiles, 2 * a.E);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -509,6 +517,10 @@ hipError_t run_scan_ws_init(void* ws, size_t nbytes, hipStream_t st) {
 
 hipError_t run_scan_ws_set_spin(void* ws, uint32_t limit, hipStream_t st) {
   return run_fill_u32(static_cast<uint32_t*>(ws) + kWsSpin, 1, limit, st);
+}
+
+hipError_t run_scan_ws_set_epoch(void* ws, uint32_t epoch, hipStream_t st) {
+  return run_fill_u32(static_cast<uint32_t*>(ws) + kWsEpoch, 1, epoch, st);
 }
 
 hipError_t run_scan_ws_take_error(void* ws, int* error_out, hipStream_t st) {

@@ -18,13 +18,13 @@
 // look-back is one round of parallel loads, not a serial chain.  Descriptor words are read
 // and written with agent-scope atomics (the eight XCDs of the chip have private L2 caches).
 //
-// The workspace carries its state from launch to launch (ticket, epoch): it is set up once
-// (scan_ws_init_kernel), every launch leaves it ready for the next (the tile that finishes
-// last resets the ticket and moves the epoch on), and a launch that finds no set-up workspace
-// flags it, marks its outputs and touches nothing else.  Every wait is bounded; a tile whose
-// wait gives up sets the workspace's sticky error word and poisons what it publishes, every
-// tile that builds on a poisoned word is poisoned too, and poisoned tiles write -1 for their
-// tokens: a consumer sees the failure in the outputs, without a synchronisation.
+// The workspace carries its state from launch to launch (ticket and epoch, one 64-bit word): it is set up once
+// (scan_ws_init_kernel), every launch leaves it ready for the next (the tile with the last ticket, which knows
+// that every tile has drawn ticket and epoch, resets the one and moves the other on), and a launch that finds no
+// set-up workspace flags it, marks its outputs and touches nothing else.  Every wait is bounded; a tile whose
+// wait gives up sets the workspace's sticky error word and poisons what it publishes, every tile that builds on
+// a poisoned word is poisoned too, and poisoned tiles write -1 for their tokens: a consumer sees the failure
+// in the outputs, without a synchronisation, and what carries no mark is right.
 //
 // Replaces the per-expert serial Blelloch scan of the reference
 // (src/op/dialect/cuda/kernels/tutel_moe_dispatch.cu:164-212: grid = E blocks, each
@@ -36,19 +36,15 @@ namespace lancet {
 
 // Header words of the workspace (uint32), followed by the descriptor table (uint64).
 enum : uint32_t {
-  kWsTicket = 0,  // next tile number; 0 between launches
-  kWsError = 1,   // sticky: a bounded wait gave up, or a launch found the workspace not set up
-  kWsEpoch = 2,   // tag of the running launch's descriptor words (1 .. 2^30-1)
-  kWsDone = 3,    // tiles of the running launch that have finished (and kDoneFailed); 0 between launches
+  kWsTicket = 0,  // next tile number, 0 between launches; with kWsEpoch ONE 64-bit word, so that a tile gets
+  kWsEpoch = 1,   // both with one atomic add: the tag of the running launch's descriptor words (1 .. 2^30-1)
+  kWsError = 2,   // sticky: a bounded wait gave up, or a launch found the workspace not set up
+  kWsDone = 3,    // finished tiles; counted only in the launch whose epoch is the last before the wrap
   kWsSpin = 4,    // polls a tile waits for a predecessor's word before it gives up (0: the default)
-  kWsMagic = 5,   // kWsMagicValue once the workspace is set up
+  kWsMagic = 5,   // kWsMagicValue once the workspace is set up (with kWsSpin one 8-byte load)
   kWsExtent = 6,  // largest number of descriptor words a launch has used
-  kWsFailed = 7,  // verdict of the last launch: 1 = a tile was poisoned (its outputs carry marks)
-  kWsTotals = 8,  // totals per counter of the last launch, kMaxScanCounters words
-  kScanHeaderWords = 8 + 1024
+  kScanHeaderWords = 8
 };
-constexpr int kMaxScanCounters = 1024;        // 2 counter sets x 512 experts
-constexpr uint32_t kDoneFailed = 0x80000000u;  // in kWsDone: a tile that has finished was poisoned
 constexpr uint32_t kWsMagicValue = 0x4c53434eu;  // "LSCN"
 constexpr uint32_t kDefaultScanSpin = 1u << 22;  // ~ seconds of polling; a healthy wait is microseconds
 
@@ -101,22 +97,20 @@ struct TileStart {
   bool ok;
 };
 
-// Must be called from uniform control flow by all kTile threads, first thing in the kernel.
+// Must be called from uniform control flow by all kTile threads, first thing in the kernel.  Two independent
+// memory round trips (the ticket fetch and the 8-byte load of spin limit and magic), issued together.
 __device__ __forceinline__ TileStart tile_begin(const ScanWs& ws, int ntiles) {
   __shared__ uint32_t s_start[4];
   if (threadIdx.x == 0) {
-    uint32_t tile = blockIdx.x, epoch = 0u, spin = 0u, ok = 0u;
-    if (ld_agent(ws.hdr + kWsMagic) == kWsMagicValue) {
-      const uint32_t t = atomicAdd(ws.hdr + kWsTicket, 1u);
-      epoch = ld_agent(ws.hdr + kWsEpoch);
-      spin = ld_agent(ws.hdr + kWsSpin);
-      if (t < static_cast<uint32_t>(ntiles) && epoch != 0u && (epoch & ~kEpochMask) == 0u) {
-        tile = t;
-        ok = 1u;
-      }
-    }
+    const uint64_t state = __hip_atomic_fetch_add(reinterpret_cast<uint64_t*>(ws.hdr + kWsTicket), 1ull,
+                                                  __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint64_t sm = __hip_atomic_load(reinterpret_cast<const uint64_t*>(ws.hdr + kWsSpin), __ATOMIC_RELAXED,
+                                          __HIP_MEMORY_SCOPE_AGENT);
+    const uint32_t t = static_cast<uint32_t>(state), epoch = static_cast<uint32_t>(state >> 32);
+    const uint32_t spin = static_cast<uint32_t>(sm), magic = static_cast<uint32_t>(sm >> 32);
+    const bool ok = magic == kWsMagicValue && t < static_cast<uint32_t>(ntiles) && epoch != 0u && (epoch & ~kEpochMask) == 0u;
     if (!ok) st_agent(ws.hdr + kWsError, 1u);
-    s_start[0] = tile;
+    s_start[0] = ok ? t : blockIdx.x;
     s_start[1] = epoch;
     s_start[2] = spin ? spin : kDefaultScanSpin;
     s_start[3] = ok;
@@ -130,71 +124,55 @@ __device__ __forceinline__ TileStart tile_begin(const ScanWs& ws, int ntiles) {
   return r;
 }
 
-// What a tile learns when it ends.  last: it is the tile that finished last, the launch's totals (the
-// inclusive prefix of the last tile, per counter) are in the LDS array it passed and in the workspace's header;
-// failed (meaningful for the last tile, which knows about all tiles): some tile of the launch was poisoned,
-// or the totals could not be read.
-struct TileEnd {
-  bool last, failed;
-};
-
-// Last thing a tile that passed tile_begin does (uniform control flow, all threads; s_tot: LDS, ncounters
-// words, free for use).  A poisoned tile says so in the same counter that counts the finished tiles, so the
-// tile that finishes last knows whether any tile was.  That tile reads the totals, stores them and the
-// verdict in the header for a kernel that follows (the top-2 finalisation), and leaves the workspace ready for
-// the next launch.  Every tile has read the epoch before it gets here, so moving it on disturbs nobody.  When
-// the epoch wraps, the words of 2^30 launches ago would look current again: they are cleared first.
-__device__ __forceinline__ TileEnd tile_end(const ScanWs& ws, const TileStart& me, int ntiles, int ncounters,
-                                            bool tile_failed, uint32_t* s_tot) {
-  __shared__ uint32_t s_old;
-  __shared__ int s_bad;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    if (tile_failed) atomicOr(ws.hdr + kWsDone, kDoneFailed);  // same address, same thread: ordered before the add
-    s_old = atomicAdd(ws.hdr + kWsDone, 1u);
-    s_bad = 0;
-  }
-  __syncthreads();
-  TileEnd r;
-  r.last = (s_old & ~kDoneFailed) == static_cast<uint32_t>(ntiles) - 1u;
-  r.failed = tile_failed || (s_old & kDoneFailed) != 0u;
-  if (!r.last) return r;
-  // totals: the last tile has published its inclusive words before it counted itself done, but nothing
-  // orders the two for another workgroup; the words validate themselves, so wait for them (bounded)
-  const uint64_t* tot = ws.desc + static_cast<size_t>(ntiles - 1) * ncounters;
-  for (int c = threadIdx.x; c < ncounters; c += kTile) {
-    uint64_t x = ld_desc(tot + c);
-    uint32_t spins = 0;
-    while (!(desc_is_current(x, me.epoch) && (static_cast<uint32_t>(x) & kDescInclusive))) {
-      if (++spins > me.spin) {
-        st_agent(ws.hdr + kWsError, 1u);
-        s_bad = 1;
-        x = 0;
-        break;
-      }
-      __builtin_amdgcn_s_sleep(1);
-      x = ld_desc(tot + c);
-    }
-    s_tot[c] = static_cast<uint32_t>(x) & kDescCountMask;
-    st_agent(ws.hdr + kWsTotals + c, s_tot[c]);
-  }
-  __syncthreads();
-  r.failed = r.failed || s_bad != 0;
+// Last thing a tile that passed tile_begin does (uniform control flow, all threads).  The tile with the last
+// ticket knows that every tile of the launch has its ticket and, with it, the epoch: it leaves the workspace
+// ready for the next launch (ticket 0, next epoch) without waiting for anybody.  Only in the launch whose
+// epoch is the last before the wrap the tiles are counted as they finish, and the one that finishes last
+// first clears the table (words of 2^30 launches ago would look current again), keeping the counts of the
+// totals row under a tag that is nobody's epoch for the kernel that reads them after this one.
+__device__ __forceinline__ void tile_end(const ScanWs& ws, const TileStart& me, int ntiles, int ncounters) {
   const uint32_t used = static_cast<uint32_t>(ntiles) * static_cast<uint32_t>(ncounters);
+  if (me.epoch != kEpochMask) {
+    if (me.tile == static_cast<uint32_t>(ntiles) - 1u && threadIdx.x == 0) {
+      atomicMax(ws.hdr + kWsExtent, used);
+      __hip_atomic_store(reinterpret_cast<uint64_t*>(ws.hdr + kWsTicket), static_cast<uint64_t>(me.epoch + 1u) << 32,
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return;
+  }
+  __shared__ uint32_t s_last;
+  __syncthreads();
+  if (threadIdx.x == 0) s_last = atomicAdd(ws.hdr + kWsDone, 1u) == static_cast<uint32_t>(ntiles) - 1u;
+  __syncthreads();
+  if (!s_last) return;
   const uint32_t extent = max(ld_agent(ws.hdr + kWsExtent), used);
-  uint32_t next = (me.epoch + 1u) & kEpochMask;
-  if (next == 0u) {
-    for (uint32_t i = threadIdx.x; i < extent; i += kTile) st_desc(ws.desc + i, 0u, 0u);
-    next = 1u;
+  const uint32_t tot_lo = used - static_cast<uint32_t>(ncounters);
+  for (uint32_t i = threadIdx.x; i < extent; i += kTile) {
+    uint32_t tag = 0u, low = 0u;
+    if (i >= tot_lo && i < used) {
+      // the last tile published these before it counted itself done, but nothing orders the two for another
+      // workgroup; the words validate themselves, so wait for them (bounded)
+      uint64_t x = ld_desc(ws.desc + i);
+      uint32_t spins = 0;
+      while (!(desc_is_current(x, me.epoch) && (static_cast<uint32_t>(x) & kDescInclusive))) {
+        if (++spins > me.spin) {
+          st_agent(ws.hdr + kWsError, 1u);
+          x = static_cast<uint64_t>(kDescPoison) << 32;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+        x = ld_desc(ws.desc + i);
+      }
+      tag = static_cast<uint32_t>(x >> 32) & kDescPoison;
+      low = static_cast<uint32_t>(x);
+    }
+    st_desc(ws.desc + i, tag, low);
   }
   if (threadIdx.x == 0) {
     st_agent(ws.hdr + kWsExtent, extent);
-    st_agent(ws.hdr + kWsFailed, r.failed ? 1u : 0u);
-    st_agent(ws.hdr + kWsTicket, 0u);
     st_agent(ws.hdr + kWsDone, 0u);
-    st_agent(ws.hdr + kWsEpoch, next);
+    __hip_atomic_store(reinterpret_cast<uint64_t*>(ws.hdr + kWsTicket), 1ull << 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
-  return r;
 }
 
 // One-time set-up of a workspace of nwords 32-bit words (a later launch may use any part of it).
@@ -218,7 +196,10 @@ __host__ __device__ inline size_t scan_lds_bytes(int ncounters) {
   return static_cast<size_t>(kScanLdsRows) * ncounters * sizeof(uint32_t);
 }
 
-constexpr int kLookbackLoads = 8;  // descriptor words in flight per thread and window
+// Descriptor words in flight per thread and window.  Measured at 256 tiles x 64 counters (all tiles running at
+// once, the deepest look-back): 4 loads 22.7 us, 8 loads 23.2, 16 loads 25.8, 32 loads 29.4 for the routing call;
+// at 16 to 64 tiles 8 is the fastest by 0.5 us.
+constexpr int kLookbackLoads = 8;
 
 // cls[j] in [0, E) is the class whose running count the token asks for in counter set j
 // (negative = none); mem[j] says whether the token itself counts in that set.
@@ -280,28 +261,39 @@ __device__ __forceinline__ bool tile_scan(const int (&cls)[NSETS], const bool (&
     if (tid == 0) s_open = NC;
     for (int c = tid; c < NC; c += kTile) s_stop[c] = 0xffffffffu;
     __syncthreads();
+    int newest = static_cast<int>(tile) - 1;  // newest row not looked at yet
     const int win_rows = max(1, (kTile * kLookbackLoads) / NC);  // rows examined per window
-    int newest = static_cast<int>(tile) - 1;                      // newest row of the window
+    // pair k of this thread is (row newest - lrow[k], counter lcol[k]), the same in every window: the one
+    // division by the run-time NC is done here and the pairs follow by addition
+    int lrow[kLookbackLoads], lcol[kLookbackLoads];
+    {
+      const int dl = kTile / NC, dc = kTile - dl * NC;
+      int l = tid / NC, c = tid - l * NC;
+#pragma unroll
+      for (int k = 0; k < kLookbackLoads; ++k) {
+        lrow[k] = l;
+        lcol[k] = c;
+        l += dl;
+        c += dc;
+        if (c >= NC) {
+          c -= NC;
+          l += 1;
+        }
+      }
+    }
     while (true) {
       const int nrows = min(win_rows, newest + 1);
-      const int npairs = nrows * NC;
       uint64_t word[kLookbackLoads];
       // issue all loads of the window, then wait for the ones that are not published yet
 #pragma unroll
       for (int k = 0; k < kLookbackLoads; ++k) {
-        const int i = tid + k * kTile;
         word[k] = 0;
-        if (i < npairs) {
-          const int l = i / NC;
-          word[k] = ld_desc(ws.desc + static_cast<size_t>(newest - l) * NC + (i - l * NC));
-        }
+        if (lrow[k] < nrows) word[k] = ld_desc(ws.desc + static_cast<size_t>(newest - lrow[k]) * NC + lcol[k]);
       }
 #pragma unroll
       for (int k = 0; k < kLookbackLoads; ++k) {
-        const int i = tid + k * kTile;
-        if (i < npairs && !desc_is_current(word[k], me.epoch)) {
-          const int l = i / NC;
-          const uint64_t* ptr = ws.desc + static_cast<size_t>(newest - l) * NC + (i - l * NC);
+        if (lrow[k] < nrows && !desc_is_current(word[k], me.epoch)) {
+          const uint64_t* ptr = ws.desc + static_cast<size_t>(newest - lrow[k]) * NC + lcol[k];
           uint32_t spins = 0;
           do {
             if (++spins > me.spin) {  // bounded wait: flag the workspace, poison the tile
@@ -313,20 +305,16 @@ __device__ __forceinline__ bool tile_scan(const int (&cls)[NSETS], const bool (&
             word[k] = ld_desc(ptr);
           } while (!desc_is_current(word[k], me.epoch));
         }
-        if (i < npairs && (static_cast<uint32_t>(word[k]) & kDescInclusive)) {
-          const int l = i / NC;
-          atomicMin(&s_stop[i - l * NC], static_cast<uint32_t>(static_cast<int>(tile) - 1 - (newest - l)));
-        }
+        if (lrow[k] < nrows && (static_cast<uint32_t>(word[k]) & kDescInclusive))
+          atomicMin(&s_stop[lcol[k]], static_cast<uint32_t>(static_cast<int>(tile) - 1 - (newest - lrow[k])));
       }
       __syncthreads();
       // add what counts: rows newer than the counter's stop row, and the stop row itself
 #pragma unroll
       for (int k = 0; k < kLookbackLoads; ++k) {
-        const int i = tid + k * kTile;
-        if (i < npairs) {
-          const int l = i / NC;
-          const int c = i - l * NC;
-          const uint32_t depth = static_cast<uint32_t>(static_cast<int>(tile) - 1 - (newest - l));
+        if (lrow[k] < nrows) {
+          const int c = lcol[k];
+          const uint32_t depth = static_cast<uint32_t>(static_cast<int>(tile) - 1 - (newest - lrow[k]));
           const uint32_t stop = s_stop[c];
           if (depth <= stop) {
             const uint32_t v = static_cast<uint32_t>(word[k]) & kDescCountMask;

@@ -38,8 +38,8 @@ def test_capacity_formula(pkg):
 
 def test_workspace_sizes_and_argument_rejection(pkg):
     lib, capi = pkg.capi.load(), pkg.capi
-    assert lib.lancet_moe_encode_workspace_bytes(65536, 32, 2) == 4128 + 256 * 64 * 8   # header + one 64-bit word per tile and counter
-    assert lib.lancet_moe_encode_workspace_bytes(0, 4, 1) == 4128 + 1 * 4 * 8
+    assert lib.lancet_moe_encode_workspace_bytes(65536, 32, 2) == 32 + 256 * 64 * 8   # header + one 64-bit word per tile and counter
+    assert lib.lancet_moe_encode_workspace_bytes(0, 4, 1) == 32 + 1 * 4 * 8
     assert lib.lancet_moe_encode_workspace_bytes(10, 0, 1) == 0
     one = C.c_void_p(16)  # never dereferenced: every call below is rejected before any launch
     st = lib.lancet_moe_encode(one, one, None, None, 8, 4, 2, 4, 1, 99, 0, one, one, one, one, one, one, 1 << 20, None)

@@ -257,7 +257,7 @@ def bench_config4_partitioned(pkg, ops, lib, capi, data, logits, S, M, E, cf, it
     Sp = S // P
     sel = torch.empty((2, S), dtype=torch.int32, device="cuda")
     val = torch.empty((2, S), dtype=torch.float32, device="cuda")
-    assert lib.lancet_gate_topk(C.c_void_p(logits.data_ptr()), None, S, E, 2, capi.GATE_IS_LOGITS,
+    assert lib.lancet_gate_topk(C.c_void_p(logits.data_ptr()), None, S, E, 2, capi.F32, capi.GATE_IS_LOGITS,
                                 C.c_void_p(sel.data_ptr()), C.c_void_p(val.data_ptr()), None) == 0
     gates, parts = [], []
     for slot in range(2):
@@ -648,7 +648,7 @@ def main():
         assert st == 0
 
     def route_only():
-        st = lib.lancet_moe_route(p(logits), None, p(used_in), S, M, E, Cap, K, capi.GATE_IS_LOGITS, p(outs[0]),
+        st = lib.lancet_moe_route(p(logits), None, p(used_in), S, M, E, Cap, K, capi.F32, capi.GATE_IS_LOGITS, p(outs[0]),
                                   p(outs[1]), p(outs[2]), p(outs[3]), p(ws.buf), ws.nbytes, stream)
         assert st == 0
 

@@ -22,8 +22,13 @@
  *     launched), > 0 = a hipError_t from the runtime.  Nothing aborts the process
  *     (the reference CHECK/LOG(FATAL)s, src/common/cuda_utils.h:18-22).
  *
- * Token rows are `dtype` (LANCET_F32 / LANCET_BF16 / LANCET_F16); gate values,
- * gates_s and LANS tensors are fp32; indices/locations/used capacity are int32 and
+ * Token rows are `dtype` (LANCET_F32 / LANCET_BF16 / LANCET_F16).  Gate arrays (gate and
+ * gate2_noise [S,E], gates_s [top_k*S], their gradients) are `gate_dtype`, one of the same three
+ * codes: the reference's kernels take the gate in the data type (`__dtype* gates1_s`,
+ * tutel_moe_dispatch.cu:110-116,126-157) and mixed-precision graphs feed a half gate
+ * (python/raf/amp/type_hints.py:97,105).  All arithmetic on gate values is fp32, with one rounding
+ * to gate_dtype where a value is stored; 16-bit gates tie often, and selection keeps its rule (first
+ * maximum wins).  LANS tensors are fp32; indices/locations/used capacity are int32 and
  * elements_per_expert is uint64, as in src/op/declare/moe.cc:48-58.
  */
 #ifndef LANCET_HIP_H_
@@ -36,9 +41,9 @@
 extern "C" {
 #endif
 
-#define LANCET_ABI_VERSION 5
+#define LANCET_ABI_VERSION 6
 
-/* element type of token rows */
+/* element type of token rows (dtype) and of gate arrays (gate_dtype) */
 #define LANCET_F32 0
 #define LANCET_BF16 1
 #define LANCET_F16 2
@@ -95,8 +100,8 @@ int64_t lancet_moe_capacity(int64_t S, int64_t E, float capacity_factor);
  * gate2_noise (top_k = 2 only, may be NULL): [S,E] values added to `gate` for the second choice alone,
  * the first choice masked out - the Gumbel noise of docker/resources/sharded_moe.py:275-278, drawn by
  * the caller; val is always read from `gate` itself. */
-int lancet_gate_topk(const float* gate, const float* gate2_noise, int64_t S, int64_t E, int top_k,
-                     unsigned flags, int32_t* idx, float* val, lancet_stream_t stream);
+int lancet_gate_topk(const void* gate, const void* gate2_noise, int64_t S, int64_t E, int top_k,
+                     int gate_dtype, unsigned flags, int32_t* idx, void* val, lancet_stream_t stream);
 
 /* ---- launcher level ----------------------------------------------------------------
  * Replaces launch_gen_location (kernel_util.cuh:60; tutel_moe_dispatch.cu:164-212,548-553).
@@ -123,11 +128,13 @@ int lancet_launch_encode_forward(const int32_t* indices, const int32_t* location
  * (docker/resources/sharded_moe.py:253-324, no noise): outputs are slot-major
  * (gates_s[2S], indices_locations[2, 2S]) in the layout moe_merge_masks produces for the two
  * chained top-1 encodes it is equivalent to, and gates_s holds the normalised combine weights.
- * used_in may be NULL (= zeros); gate2_noise as in lancet_gate_topk, NULL = none. */
+ * used_in may be NULL (= zeros); gate2_noise as in lancet_gate_topk, NULL = none.  With a 16-bit
+ * gate_dtype and top_k = 2 the two raw gate values are rounded to gate_dtype, as a gates_s array of that
+ * type holds them, before the combine weights are formed from them in fp32. */
 size_t lancet_moe_encode_workspace_bytes(int64_t S, int64_t E, int top_k);
-int lancet_moe_encode(const void* data, const float* gate, const float* gate2_noise, const int32_t* used_in,
-                      int64_t S, int64_t M, int64_t E, int64_t C, int top_k, int dtype,
-                      unsigned flags, float* gates_s, int32_t* indices_locations,
+int lancet_moe_encode(const void* data, const void* gate, const void* gate2_noise, const int32_t* used_in,
+                      int64_t S, int64_t M, int64_t E, int64_t C, int top_k, int dtype, int gate_dtype,
+                      unsigned flags, void* gates_s, int32_t* indices_locations,
                       int32_t* used_out, uint64_t* elements_per_expert, void* dispatched,
                       void* workspace, size_t workspace_bytes, lancet_stream_t stream);
 
@@ -143,9 +150,9 @@ int lancet_moe_encode(const void* data, const float* gate, const float* gate2_no
  * yourself.  The first call on a device looks the array's address up, sets the workspace up (one small
  * launch on `stream`, no allocation) and waits for `stream`; make that call once before recording a graph. */
 #define LANCET_NOALLOC_SCRATCH_BYTES ((2u << 20) + 4096u)
-int lancet_moe_encode_noalloc(const void* data, const float* gate, const float* gate2_noise,
+int lancet_moe_encode_noalloc(const void* data, const void* gate, const void* gate2_noise,
                               const int32_t* used_in, int64_t S, int64_t M, int64_t E, int64_t C, int top_k,
-                              int dtype, unsigned flags, float* gates_s, int32_t* indices_locations,
+                              int dtype, int gate_dtype, unsigned flags, void* gates_s, int32_t* indices_locations,
                               int32_t* used_out, uint64_t* elements_per_expert, void* dispatched,
                               lancet_stream_t stream);
 
@@ -157,8 +164,8 @@ int lancet_moe_encode_noalloc(const void* data, const float* gate, const float* 
  *                        except the buffer;
  *   lancet_moe_scatter = launch_encode_forward (moe.cc:381-395) on routing produced by
  *                        lancet_moe_route; zero-fills the rows past used_out - used_in. */
-int lancet_moe_route(const float* gate, const float* gate2_noise, const int32_t* used_in, int64_t S, int64_t M,
-                     int64_t E, int64_t C, int top_k, unsigned flags, float* gates_s,
+int lancet_moe_route(const void* gate, const void* gate2_noise, const int32_t* used_in, int64_t S, int64_t M,
+                     int64_t E, int64_t C, int top_k, int gate_dtype, unsigned flags, void* gates_s,
                      int32_t* indices_locations, int32_t* used_out, uint64_t* elements_per_expert,
                      void* workspace, size_t workspace_bytes, lancet_stream_t stream);
 int lancet_moe_scatter(const void* data, const int32_t* indices_locations, const int32_t* used_in,
@@ -172,9 +179,9 @@ int lancet_moe_scatter(const void* data, const int32_t* indices_locations, const
  * partition_id are encoded.  The per-expert keep set is the C best tokens by
  * (gate value descending, token index ascending), found with a radix select, not a sort. */
 size_t lancet_moe_encode_bpr_workspace_bytes(int64_t S0, int64_t E, int n_partitions);
-int lancet_moe_encode_bpr(const void* data, const float* gate, int64_t S0, int64_t M, int64_t E,
-                          int64_t C, int n_partitions, int partition_id, int dtype, unsigned flags,
-                          float* gates_s, int32_t* indices_locations, int32_t* used_out,
+int lancet_moe_encode_bpr(const void* data, const void* gate, int64_t S0, int64_t M, int64_t E,
+                          int64_t C, int n_partitions, int partition_id, int dtype, int gate_dtype, unsigned flags,
+                          void* gates_s, int32_t* indices_locations, int32_t* used_out,
                           uint64_t* elements_per_expert, void* dispatched,
                           void* workspace, size_t workspace_bytes, lancet_stream_t stream);
 
@@ -182,9 +189,9 @@ int lancet_moe_encode_bpr(const void* data, const float* gate, int64_t S0, int64
  * Replaces MoeDecode::Execute / launch_decode_forward (moe.cc:1262-1291; kernel_util.cuh:45;
  * tutel_moe_dispatch.cu:46-55,110-116,511-521).  top_k = 2 sums the two slots of the
  * slot-major layout in fp32 and rounds once. */
-int lancet_moe_decode(const void* expert_out, const float* gates_s,
+int lancet_moe_decode(const void* expert_out, const void* gates_s,
                       const int32_t* indices_locations, int64_t S, int64_t M, int64_t E,
-                      int64_t C, int top_k, int dtype, void* out, lancet_stream_t stream);
+                      int64_t C, int top_k, int dtype, int gate_dtype, void* out, lancet_stream_t stream);
 
 /* ---- token ranges of a whole-batch mask -------------------------------------------------
  * The partition pass cuts the token batch so that the exchange of one partition overlaps the work on
@@ -205,9 +212,9 @@ int lancet_moe_scatter_tokens(const void* data, const int32_t* indices_locations
                               const int32_t* used_out, int64_t S_total, int64_t token_first, int64_t n_tokens, int64_t M, int64_t E,
                               int64_t C, int top_k, int dtype, unsigned flags, void* dispatched,
                               lancet_stream_t stream);
-int lancet_moe_decode_tokens(const void* expert_out, const float* gates_s, const int32_t* indices_locations,
+int lancet_moe_decode_tokens(const void* expert_out, const void* gates_s, const int32_t* indices_locations,
                              int64_t S_total, int64_t token_first, int64_t n_tokens, int64_t M, int64_t E,
-                             int64_t C, int top_k, int dtype, void* out, lancet_stream_t stream);
+                             int64_t C, int top_k, int dtype, int gate_dtype, void* out, lancet_stream_t stream);
 
 /* ---- raf.op.moe_redispatch_expert_input ------------------------------------------------
  * Replaces MoeRedispatchExpertInput::Execute / launch_redispatch_expert_input (moe.cc:945-1073;
@@ -266,7 +273,7 @@ int lancet_moe_partition_ranges(const int32_t* indices_locations, int64_t S_tota
                                 size_t workspace_bytes, lancet_stream_t stream);
 
 /* ---- backward ops (raf.op.moe_encode_dx / _dg, raf.op.moe_decode_dx / _dg) ------------------
- * Gradients wired by src/op/grad/moe.cc:30-93.  Gate-side gradients are fp32 like gates_s; top_k = 2
+ * Gradients wired by src/op/grad/moe.cc:30-93.  Gate-side gradients are gate_dtype like gates_s; top_k = 2
  * takes the slot-major layout of the forward ops.
  *
  * moe_encode_dx: dx[s,:] = sum over slots of dy[idx, loc, :] (0 for dropped slots).  Replaces
@@ -277,27 +284,27 @@ int lancet_moe_encode_dx(const void* dy, const int32_t* indices_locations, int64
 /* moe_encode_dg: grad_gates[S,E] = 0 except grad_gates[s, idx] = dy_gates_s of that slot.  Replaces
  * MoeEncodeDg / launch_encode_backward_gate (moe.cc:1155-1225; kernel_util.cuh:43;
  * tutel_moe_dispatch.cu:96-105,499-506). */
-int lancet_moe_encode_dg(const float* dy_gates_s, const int32_t* indices_locations, int64_t S,
-                         int64_t E, int top_k, float* grad_gates, lancet_stream_t stream);
+int lancet_moe_encode_dg(const void* dy_gates_s, const int32_t* indices_locations, int64_t S,
+                         int64_t E, int top_k, int gate_dtype, void* grad_gates, lancet_stream_t stream);
 /* moe_decode_dx: grad_expert_out[idx, loc, :] = gates_s * dy[s, :], zero elsewhere.  Replaces
  * MoeDecodeDx / launch_decode_backward_data (moe.cc:1313-1395; kernel_util.cuh:47;
  * tutel_moe_dispatch.cu:118-124,523-533).  Workspace: an [E*C] int32 row -> token map. */
 size_t lancet_moe_decode_dx_workspace_bytes(int64_t E, int64_t C);
-int lancet_moe_decode_dx(const void* dy, const float* gates_s, const int32_t* indices_locations,
-                         int64_t S, int64_t M, int64_t E, int64_t C, int top_k, int dtype,
+int lancet_moe_decode_dx(const void* dy, const void* gates_s, const int32_t* indices_locations,
+                         int64_t S, int64_t M, int64_t E, int64_t C, int top_k, int dtype, int gate_dtype,
                          void* grad_expert_out, void* workspace, size_t workspace_bytes,
                          lancet_stream_t stream);
 /* moe_decode_dg: grad_gates_s[slot-token] = <expert_out[idx, loc, :], dy[s, :]>, 0 for dropped slots.
  * Replaces MoeDecodeDg / launch_decode_backward_gate (moe.cc:1397-1481; kernel_util.cuh:49;
  * tutel_moe_dispatch.cu:126-157,535-546). */
 int lancet_moe_decode_dg(const void* dy, const void* expert_out, const int32_t* indices_locations,
-                         int64_t S, int64_t M, int64_t E, int64_t C, int top_k, int dtype,
-                         float* grad_gates_s, lancet_stream_t stream);
+                         int64_t S, int64_t M, int64_t E, int64_t C, int top_k, int dtype, int gate_dtype,
+                         void* grad_gates_s, lancet_stream_t stream);
 
 /* Combine weights of the top-2 extension from raw per-slot gate values and merged indices
  * (docker/resources/sharded_moe.py:304-312); in place when gates_out == raw_gates. */
-int lancet_moe_top2_normalize_gates(const float* raw_gates, const int32_t* merged_indices,
-                                    int64_t S, float* gates_out, lancet_stream_t stream);
+int lancet_moe_top2_normalize_gates(const void* raw_gates, const int32_t* merged_indices,
+                                    int64_t S, int gate_dtype, void* gates_out, lancet_stream_t stream);
 
 /* ---- raf.op.moe_merge_masks --------------------------------------------------------
  * Replaces MoeMergeMasks::Execute / launch_merge_masks (moe.cc:772-802; kernel_util.cuh:62;

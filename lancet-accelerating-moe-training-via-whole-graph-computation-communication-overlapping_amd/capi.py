@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(HERE, "lib", "liblancet_hip.so")
 F32, BF16, F16 = 0, 1, 2
 GATE_IS_LOGITS = 1
 NO_TAIL_ZERO = 2
-ABI_VERSION = 5
+ABI_VERSION = 6
 ZERO_TAIL = 4
 ROWS_AT_USED = 8
 LANS_SWEEPS, LANS_RESIDENT = 0, 1
@@ -44,29 +44,29 @@ SIGNATURES = {
     "lancet_abi_version": (_int, []),
     "lancet_status_string": (C.c_char_p, [_int]),
     "lancet_moe_capacity": (_i64, [_i64, _i64, _f32]),
-    "lancet_gate_topk": (_int, [_vp, _vp, _i64, _i64, _int, _u32, _vp, _vp, _vp]),
+    "lancet_gate_topk": (_int, [_vp, _vp, _i64, _i64, _int, _int, _u32, _vp, _vp, _vp]),
     "lancet_gen_location_workspace_bytes": (_sz, [_i64, _i64]),
     "lancet_launch_gen_location": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _sz, _vp]),
     "lancet_launch_encode_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "lancet_moe_encode_workspace_bytes": (_sz, [_i64, _i64, _int]),
-    "lancet_moe_encode": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _u32,
+    "lancet_moe_encode": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _u32,
                                  _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
-    "lancet_moe_encode_noalloc": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _u32,
+    "lancet_moe_encode_noalloc": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _u32,
                                          _vp, _vp, _vp, _vp, _vp, _vp]),
-    "lancet_moe_route": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _u32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "lancet_moe_route": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _u32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "lancet_moe_scatter": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _u32, _vp, _vp]),
     "lancet_moe_encode_bpr_workspace_bytes": (_sz, [_i64, _i64, _int]),
-    "lancet_moe_encode_bpr": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _u32,
+    "lancet_moe_encode_bpr": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _u32,
                                      _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "lancet_moe_scatter_tokens": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _u32, _vp, _vp]),
-    "lancet_moe_decode_tokens": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp]),
+    "lancet_moe_decode_tokens": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _vp, _vp]),
     "lancet_memcpy_sparse_ranges_to_cont_3d": (_int, [_vp, _vp, _vp, _vp, _i64, _int, _int, _int, _i64, _i64, _i64, _i64, _int, _vp]),
     "lancet_memcpy_cont_to_sparse_ranges_3d": (_int, [_vp, _vp, _vp, _vp, _i64, _int, _int, _int, _i64, _i64, _i64, _i64, _int, _vp]),
     "lancet_moe_partition_ranges_workspace_bytes": (_sz, [_int, _int, _i64]),
     "lancet_moe_partition_ranges": (_int, [_vp, _i64, _int, _int, _i64, _i64, _vp, _vp, _vp, _sz, _vp]),
     "lancet_debug_stream": (_int, [_int, _vp, _vp, _sz, _vp]),
     "lancet_debug_stream_4r3w": (_int, [_vp, _vp, _vp, _vp, _sz, _vp]),
-    "lancet_moe_decode": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp]),
+    "lancet_moe_decode": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _vp, _vp]),
     "lancet_moe_redispatch_expert_input": (_int, [C.POINTER(_vp), C.POINTER(_vp), _int, _int, _int, _i64, _i64, _i64,
                                                   _int, _int, _vp, _vp]),
     "lancet_memcpy_sparse_to_cont_3d": (_int, [_vp, _vp, _vp, _i64, _int, _int, _int, _i64, _i64, _i64, _i64, _int, _int,
@@ -74,11 +74,11 @@ SIGNATURES = {
     "lancet_memcpy_cont_to_sparse_3d": (_int, [_vp, _vp, _vp, _i64, _int, _int, _int, _i64, _i64, _i64, _i64, _int, _int,
                                                _int, _u32, _vp]),
     "lancet_moe_encode_dx": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp]),
-    "lancet_moe_encode_dg": (_int, [_vp, _vp, _i64, _i64, _int, _vp, _vp]),
+    "lancet_moe_encode_dg": (_int, [_vp, _vp, _i64, _i64, _int, _int, _vp, _vp]),
     "lancet_moe_decode_dx_workspace_bytes": (_sz, [_i64, _i64]),
-    "lancet_moe_decode_dx": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp, _sz, _vp]),
-    "lancet_moe_decode_dg": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp]),
-    "lancet_moe_top2_normalize_gates": (_int, [_vp, _vp, _i64, _vp, _vp]),
+    "lancet_moe_decode_dx": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _vp, _vp, _sz, _vp]),
+    "lancet_moe_decode_dg": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _vp, _vp]),
+    "lancet_moe_top2_normalize_gates": (_int, [_vp, _vp, _i64, _int, _vp, _vp]),
     "lancet_moe_merge_masks_workspace_bytes": (_sz, [_int, _i64]),
     "lancet_moe_merge_masks": (_int, [C.POINTER(_vp), _int, _i64, _i64, _vp, _vp, _sz, _vp]),
     "lancet_moe_redispatch_workspace_bytes": (_sz, [_int, _i64]),

@@ -152,17 +152,19 @@ extern "C" int lancet_debug_stream(int kind, void* dst, const void* src, size_t 
 }
 
 // ---- routing front end ---------------------------------------------------------------
-extern "C" int lancet_gate_topk(const float* gate, const float* gate2_noise, int64_t S, int64_t E, int top_k,
-                                unsigned flags, int32_t* idx, float* val, lancet_stream_t stream) {
+extern "C" int lancet_gate_topk(const void* gate, const void* gate2_noise, int64_t S, int64_t E, int top_k,
+                                int gate_dtype, unsigned flags, int32_t* idx, void* val, lancet_stream_t stream) {
   if (!gate || !idx || !val) return LANCET_ERR_NULL;
+  const int gb = elem_bytes(gate_dtype);
+  if (!gb) return LANCET_ERR_DTYPE;
   if (int r = check_dims(S, 0, E, 0)) return r;
   if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
   if (top_k == 2 && E < 2) return LANCET_ERR_TOPK;
   if (gate2_noise && top_k != 2) return LANCET_ERR_TOPK;  // the noise only exists for the second choice
-  if (misaligned(gate, 4) || misaligned(gate2_noise, 4) || misaligned(idx, 4) || misaligned(val, 4))
+  if (misaligned(gate, gb) || misaligned(gate2_noise, gb) || misaligned(idx, 4) || misaligned(val, gb))
     return LANCET_ERR_ALIGN;
   return rc(run_gate_topk(gate, gate2_noise, static_cast<int>(S), static_cast<int>(E), top_k,
-                          (flags & LANCET_GATE_IS_LOGITS) != 0, idx, val, S_(stream)));
+                          (flags & LANCET_GATE_IS_LOGITS) != 0, gate_dtype, idx, val, S_(stream)));
 }
 
 // ---- launcher level ------------------------------------------------------------------
@@ -182,7 +184,7 @@ extern "C" int lancet_launch_gen_location(int32_t* indices, const int32_t* in_ca
       misaligned(out_elements_per_expert, 8) || misaligned(workspace, 8) || misaligned(in_capused, 4))
     return LANCET_ERR_ALIGN;
   return rc(run_route_scan(nullptr, nullptr, indices, in_capused, static_cast<int>(S), static_cast<int>(E),
-                           static_cast<int>(C), static_cast<int>(M), 1, false, nullptr, indices, locations,
+                           static_cast<int>(C), static_cast<int>(M), 1, false, LANCET_F32, nullptr, indices, locations,
                            out_capused, out_elements_per_expert, workspace, S_(stream)));
 }
 
@@ -211,23 +213,25 @@ extern "C" size_t lancet_moe_encode_workspace_bytes(int64_t S, int64_t E, int to
   return scan_workspace_bytes(S, E, top_k);
 }
 
-extern "C" int lancet_moe_route(const float* gate, const float* gate2_noise, const int32_t* used_in, int64_t S,
-                                int64_t M, int64_t E, int64_t C, int top_k, unsigned flags, float* gates_s,
+extern "C" int lancet_moe_route(const void* gate, const void* gate2_noise, const int32_t* used_in, int64_t S,
+                                int64_t M, int64_t E, int64_t C, int top_k, int gate_dtype, unsigned flags, void* gates_s,
                                 int32_t* indices_locations, int32_t* used_out, uint64_t* elements_per_expert,
                                 void* workspace, size_t workspace_bytes, lancet_stream_t stream) {
   if (((!gate || !gates_s || !indices_locations) && S > 0) || !used_out || !elements_per_expert)
     return LANCET_ERR_NULL;
+  const int gb = elem_bytes(gate_dtype);
+  if (!gb) return LANCET_ERR_DTYPE;
   if (int r = check_dims(S, M, E, C)) return r;
   if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
   if (top_k == 2 && E < 2) return LANCET_ERR_TOPK;
   if (gate2_noise && top_k != 2) return LANCET_ERR_TOPK;
   if (!workspace || workspace_bytes < lancet_moe_encode_workspace_bytes(S, E, top_k)) return LANCET_ERR_WORKSPACE;
-  if (misaligned(gate, 4) || misaligned(gate2_noise, 4) || misaligned(gates_s, 4) || misaligned(indices_locations, 4) || misaligned(used_in, 4) ||
+  if (misaligned(gate, gb) || misaligned(gate2_noise, gb) || misaligned(gates_s, gb) || misaligned(indices_locations, 4) || misaligned(used_in, 4) ||
       misaligned(used_out, 4) || misaligned(elements_per_expert, 8) || misaligned(workspace, 8))
     return LANCET_ERR_ALIGN;
   const int s = static_cast<int>(S);
   return rc(run_route_scan(gate, gate2_noise, nullptr, used_in, s, static_cast<int>(E), static_cast<int>(C),
-                           static_cast<int>(M), top_k, (flags & LANCET_GATE_IS_LOGITS) != 0, gates_s,
+                           static_cast<int>(M), top_k, (flags & LANCET_GATE_IS_LOGITS) != 0, gate_dtype, gates_s,
                            indices_locations, indices_locations + static_cast<size_t>(top_k) * s, used_out,
                            elements_per_expert, workspace, S_(stream)));
 }
@@ -254,10 +258,10 @@ extern "C" int lancet_moe_scatter(const void* data, const int32_t* indices_locat
                              static_cast<int>(E), static_cast<int>(C), top_k, eb, S_(stream)));
 }
 
-extern "C" int lancet_moe_encode(const void* data, const float* gate, const float* gate2_noise,
+extern "C" int lancet_moe_encode(const void* data, const void* gate, const void* gate2_noise,
                                  const int32_t* used_in, int64_t S, int64_t M, int64_t E, int64_t C, int top_k,
-                                 int dtype, unsigned flags,
-                                 float* gates_s, int32_t* indices_locations, int32_t* used_out,
+                                 int dtype, int gate_dtype, unsigned flags,
+                                 void* gates_s, int32_t* indices_locations, int32_t* used_out,
                                  uint64_t* elements_per_expert, void* dispatched, void* workspace,
                                  size_t workspace_bytes, lancet_stream_t stream) {
   // validate everything before the first launch
@@ -265,7 +269,7 @@ extern "C" int lancet_moe_encode(const void* data, const float* gate, const floa
   const int eb = elem_bytes(dtype);
   if (!eb) return LANCET_ERR_DTYPE;
   if (misaligned(data, eb) || misaligned(dispatched, eb)) return LANCET_ERR_ALIGN;
-  if (int r = lancet_moe_route(gate, gate2_noise, used_in, S, M, E, C, top_k, flags, gates_s, indices_locations, used_out,
+  if (int r = lancet_moe_route(gate, gate2_noise, used_in, S, M, E, C, top_k, gate_dtype, flags, gates_s, indices_locations, used_out,
                                elements_per_expert, workspace, workspace_bytes, stream))
     return r;
   return lancet_moe_scatter(data, indices_locations, used_in, used_out, S, M, E, C, top_k, dtype, flags, dispatched,
@@ -305,9 +309,9 @@ extern "C" int lancet_moe_scatter_tokens(const void* data, const int32_t* indice
                              static_cast<int>(E), static_cast<int>(C), top_k, eb, S_(stream), static_cast<int>(S_total)));
 }
 
-extern "C" int lancet_moe_decode_tokens(const void* expert_out, const float* gates_s, const int32_t* indices_locations,
+extern "C" int lancet_moe_decode_tokens(const void* expert_out, const void* gates_s, const int32_t* indices_locations,
                                         int64_t S_total, int64_t token_first, int64_t n_tokens, int64_t M, int64_t E,
-                                        int64_t C, int top_k, int dtype, void* out, lancet_stream_t stream) {
+                                        int64_t C, int top_k, int dtype, int gate_dtype, void* out, lancet_stream_t stream) {
   if ((!expert_out && C > 0 && M > 0) || ((!gates_s || !indices_locations) && n_tokens > 0) ||
       (!out && n_tokens > 0 && M > 0))
     return LANCET_ERR_NULL;
@@ -316,10 +320,13 @@ extern "C" int lancet_moe_decode_tokens(const void* expert_out, const float* gat
   if (int r = check_dims(S_total, M, E, C)) return r;
   if (int r = check_range(S_total, token_first, n_tokens)) return r;
   if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
-  if (misaligned(expert_out, eb) || misaligned(out, eb) || misaligned(gates_s, 4) || misaligned(indices_locations, 4))
+  const int gb = elem_bytes(gate_dtype);
+  if (!gb) return LANCET_ERR_DTYPE;
+  if (misaligned(expert_out, eb) || misaligned(out, eb) || misaligned(gates_s, gb) || misaligned(indices_locations, 4))
     return LANCET_ERR_ALIGN;
   const size_t st = static_cast<size_t>(S_total);
-  return rc(run_decode_rows(expert_out, gates_s + token_first, indices_locations + token_first,
+  return rc(run_decode_rows(expert_out, static_cast<const char*>(gates_s) + static_cast<size_t>(token_first) * gb, gate_dtype,
+                            indices_locations + token_first,
                             indices_locations + static_cast<size_t>(top_k) * st + token_first, out,
                             static_cast<int>(n_tokens), static_cast<int>(M), static_cast<int>(E), static_cast<int>(C),
                             top_k, dtype, S_(stream), static_cast<int>(S_total)));
@@ -331,22 +338,22 @@ extern "C" size_t lancet_moe_encode_bpr_workspace_bytes(int64_t S0, int64_t E, i
   return bpr_workspace_bytes(S0, S0 / n_partitions, E);
 }
 
-extern "C" int lancet_moe_encode_bpr(const void* data, const float* gate, int64_t S0, int64_t M, int64_t E,
-                                     int64_t C, int n_partitions, int partition_id, int dtype, unsigned flags,
-                                     float* gates_s, int32_t* indices_locations, int32_t* used_out,
+extern "C" int lancet_moe_encode_bpr(const void* data, const void* gate, int64_t S0, int64_t M, int64_t E,
+                                     int64_t C, int n_partitions, int partition_id, int dtype, int gate_dtype, unsigned flags,
+                                     void* gates_s, int32_t* indices_locations, int32_t* used_out,
                                      uint64_t* elements_per_expert, void* dispatched, void* workspace,
                                      size_t workspace_bytes, lancet_stream_t stream) {
   if ((!data && S0 > 0 && M > 0) || ((!gate || !gates_s || !indices_locations) && S0 > 0) || !used_out ||
       !elements_per_expert || (!dispatched && C > 0 && M > 0))
     return LANCET_ERR_NULL;
-  const int eb = elem_bytes(dtype);
-  if (!eb) return LANCET_ERR_DTYPE;
+  const int eb = elem_bytes(dtype), gb = elem_bytes(gate_dtype);
+  if (!eb || !gb) return LANCET_ERR_DTYPE;
   if (int r = check_dims(S0, M, E, C)) return r;
   // src/op/declare/moe.cc:74-75
   if (n_partitions < 1 || partition_id < 0 || partition_id >= n_partitions) return LANCET_ERR_PARTITION;
   if (!workspace || workspace_bytes < lancet_moe_encode_bpr_workspace_bytes(S0, E, n_partitions))
     return LANCET_ERR_WORKSPACE;
-  if (misaligned(data, eb) || misaligned(dispatched, eb) || misaligned(gate, 4) || misaligned(gates_s, 4) ||
+  if (misaligned(data, eb) || misaligned(dispatched, eb) || misaligned(gate, gb) || misaligned(gates_s, gb) ||
       misaligned(indices_locations, 4) || misaligned(used_out, 4) || misaligned(elements_per_expert, 8) ||
       misaligned(workspace, 8))
     return LANCET_ERR_ALIGN;
@@ -355,7 +362,7 @@ extern "C" int lancet_moe_encode_bpr(const void* data, const float* gate, int64_
   int32_t* idx = indices_locations;
   int32_t* loc = indices_locations + s;
   hipError_t e = run_bpr_route(gate, s0, static_cast<int>(E), static_cast<int>(C), static_cast<int>(M),
-                               n_partitions, partition_id, (flags & LANCET_GATE_IS_LOGITS) != 0, gates_s, idx,
+                               n_partitions, partition_id, (flags & LANCET_GATE_IS_LOGITS) != 0, gate_dtype, gates_s, idx,
                                loc, used_out, elements_per_expert, workspace, S_(stream));
   if (e != hipSuccess) return rc(e);
   const char* part = static_cast<const char*>(data) + static_cast<size_t>(partition_id) * s * M * eb;
@@ -365,8 +372,8 @@ extern "C" int lancet_moe_encode_bpr(const void* data, const float* gate, int64_
 }
 
 // ---- raf.op.moe_decode ---------------------------------------------------------------
-extern "C" int lancet_moe_decode(const void* expert_out, const float* gates_s, const int32_t* indices_locations,
-                                 int64_t S, int64_t M, int64_t E, int64_t C, int top_k, int dtype, void* out,
+extern "C" int lancet_moe_decode(const void* expert_out, const void* gates_s, const int32_t* indices_locations,
+                                 int64_t S, int64_t M, int64_t E, int64_t C, int top_k, int dtype, int gate_dtype, void* out,
                                  lancet_stream_t stream) {
   if ((!expert_out && C > 0 && M > 0) || ((!gates_s || !indices_locations) && S > 0) || (!out && S > 0 && M > 0))
     return LANCET_ERR_NULL;
@@ -374,10 +381,12 @@ extern "C" int lancet_moe_decode(const void* expert_out, const float* gates_s, c
   if (!eb) return LANCET_ERR_DTYPE;
   if (int r = check_dims(S, M, E, C)) return r;
   if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
-  if (misaligned(expert_out, eb) || misaligned(out, eb) || misaligned(gates_s, 4) || misaligned(indices_locations, 4))
+  const int gb = elem_bytes(gate_dtype);
+  if (!gb) return LANCET_ERR_DTYPE;
+  if (misaligned(expert_out, eb) || misaligned(out, eb) || misaligned(gates_s, gb) || misaligned(indices_locations, 4))
     return LANCET_ERR_ALIGN;
   const int s = static_cast<int>(S);
-  return rc(run_decode_rows(expert_out, gates_s, indices_locations, indices_locations + static_cast<size_t>(top_k) * s,
+  return rc(run_decode_rows(expert_out, gates_s, gate_dtype, indices_locations, indices_locations + static_cast<size_t>(top_k) * s,
                             out, s, static_cast<int>(M), static_cast<int>(E), static_cast<int>(C), top_k, dtype,
                             S_(stream)));
 }
@@ -525,17 +534,19 @@ extern "C" int lancet_moe_encode_dx(const void* dy, const int32_t* indices_locat
   if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
   if (misaligned(dy, eb) || misaligned(dx, eb) || misaligned(indices_locations, 4)) return LANCET_ERR_ALIGN;
   const int s = static_cast<int>(S);
-  return rc(run_decode_rows(dy, nullptr, indices_locations, indices_locations + static_cast<size_t>(top_k) * s, dx, s,
+  return rc(run_decode_rows(dy, nullptr, LANCET_F32, indices_locations, indices_locations + static_cast<size_t>(top_k) * s, dx, s,
                             static_cast<int>(M), static_cast<int>(E), static_cast<int>(C), top_k, dtype, S_(stream)));
 }
 
-extern "C" int lancet_moe_encode_dg(const float* dy_gates_s, const int32_t* indices_locations, int64_t S, int64_t E,
-                                    int top_k, float* grad_gates, lancet_stream_t stream) {
+extern "C" int lancet_moe_encode_dg(const void* dy_gates_s, const int32_t* indices_locations, int64_t S, int64_t E,
+                                    int top_k, int gate_dtype, void* grad_gates, lancet_stream_t stream) {
   if (S > 0 && (!dy_gates_s || !indices_locations || !grad_gates)) return LANCET_ERR_NULL;
+  const int gb = elem_bytes(gate_dtype);
+  if (!gb) return LANCET_ERR_DTYPE;
   if (int r = check_dims(S, 0, E, 0)) return r;
   if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
-  if (misaligned(dy_gates_s, 4) || misaligned(indices_locations, 4) || misaligned(grad_gates, 4)) return LANCET_ERR_ALIGN;
-  return rc(run_encode_dg(dy_gates_s, indices_locations, static_cast<int>(S), static_cast<int>(E), top_k, grad_gates,
+  if (misaligned(dy_gates_s, gb) || misaligned(indices_locations, 4) || misaligned(grad_gates, gb)) return LANCET_ERR_ALIGN;
+  return rc(run_encode_dg(dy_gates_s, indices_locations, static_cast<int>(S), static_cast<int>(E), top_k, gate_dtype, grad_gates,
                           S_(stream)));
 }
 
@@ -544,8 +555,8 @@ extern "C" size_t lancet_moe_decode_dx_workspace_bytes(int64_t E, int64_t C) {
   return static_cast<size_t>(E) * static_cast<size_t>(C) * sizeof(int32_t);
 }
 
-extern "C" int lancet_moe_decode_dx(const void* dy, const float* gates_s, const int32_t* indices_locations, int64_t S,
-                                    int64_t M, int64_t E, int64_t C, int top_k, int dtype, void* grad_expert_out,
+extern "C" int lancet_moe_decode_dx(const void* dy, const void* gates_s, const int32_t* indices_locations, int64_t S,
+                                    int64_t M, int64_t E, int64_t C, int top_k, int dtype, int gate_dtype, void* grad_expert_out,
                                     void* workspace, size_t workspace_bytes, lancet_stream_t stream) {
   if (((!dy && M > 0) || !gates_s || !indices_locations) && S > 0) return LANCET_ERR_NULL;
   if (!grad_expert_out && C > 0 && M > 0) return LANCET_ERR_NULL;
@@ -554,38 +565,44 @@ extern "C" int lancet_moe_decode_dx(const void* dy, const float* gates_s, const 
   if (int r = check_dims(S, M, E, C)) return r;
   if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
   if (C > 0 && (!workspace || workspace_bytes < lancet_moe_decode_dx_workspace_bytes(E, C))) return LANCET_ERR_WORKSPACE;
-  if (misaligned(dy, eb) || misaligned(grad_expert_out, eb) || misaligned(gates_s, 4) ||
+  const int gb = elem_bytes(gate_dtype);
+  if (!gb) return LANCET_ERR_DTYPE;
+  if (misaligned(dy, eb) || misaligned(grad_expert_out, eb) || misaligned(gates_s, gb) ||
       misaligned(indices_locations, 4) || misaligned(workspace, 4))
     return LANCET_ERR_ALIGN;
   const int s = static_cast<int>(S);
-  return rc(run_decode_dx(dy, gates_s, indices_locations, indices_locations + static_cast<size_t>(top_k) * s,
+  return rc(run_decode_dx(dy, gates_s, gate_dtype, indices_locations, indices_locations + static_cast<size_t>(top_k) * s,
                           grad_expert_out, static_cast<int32_t*>(workspace), s, static_cast<int>(M),
                           static_cast<int>(E), static_cast<int>(C), top_k, dtype, S_(stream)));
 }
 
 extern "C" int lancet_moe_decode_dg(const void* dy, const void* expert_out, const int32_t* indices_locations, int64_t S,
-                                    int64_t M, int64_t E, int64_t C, int top_k, int dtype, float* grad_gates_s,
+                                    int64_t M, int64_t E, int64_t C, int top_k, int dtype, int gate_dtype, void* grad_gates_s,
                                     lancet_stream_t stream) {
   if (S > 0 && (!indices_locations || !grad_gates_s || ((!dy || !expert_out) && M > 0))) return LANCET_ERR_NULL;
   const int eb = elem_bytes(dtype);
   if (!eb) return LANCET_ERR_DTYPE;
   if (int r = check_dims(S, M, E, C)) return r;
   if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
-  if (misaligned(dy, eb) || misaligned(expert_out, eb) || misaligned(grad_gates_s, 4) || misaligned(indices_locations, 4))
+  const int gb = elem_bytes(gate_dtype);
+  if (!gb) return LANCET_ERR_DTYPE;
+  if (misaligned(dy, eb) || misaligned(expert_out, eb) || misaligned(grad_gates_s, gb) || misaligned(indices_locations, 4))
     return LANCET_ERR_ALIGN;
   const int s = static_cast<int>(S);
   return rc(run_decode_dg(dy, expert_out, indices_locations, indices_locations + static_cast<size_t>(top_k) * s,
-                          grad_gates_s, s, static_cast<int>(M), static_cast<int>(E), static_cast<int>(C), top_k, dtype,
+                          grad_gates_s, gate_dtype, s, static_cast<int>(M), static_cast<int>(E), static_cast<int>(C), top_k, dtype,
                           S_(stream)));
 }
 
-extern "C" int lancet_moe_top2_normalize_gates(const float* raw_gates, const int32_t* merged_indices, int64_t S,
-                                               float* gates_out, lancet_stream_t stream) {
+extern "C" int lancet_moe_top2_normalize_gates(const void* raw_gates, const int32_t* merged_indices, int64_t S,
+                                               int gate_dtype, void* gates_out, lancet_stream_t stream) {
   if (S < 0 || S > 0x3fffffff) return LANCET_ERR_SHAPE;
   if (S == 0) return LANCET_OK;
   if (!raw_gates || !merged_indices || !gates_out) return LANCET_ERR_NULL;
-  if (misaligned(raw_gates, 4) || misaligned(merged_indices, 4) || misaligned(gates_out, 4)) return LANCET_ERR_ALIGN;
-  return rc(run_top2_normalize(raw_gates, merged_indices, static_cast<int>(S), gates_out, S_(stream)));
+  const int gb = elem_bytes(gate_dtype);
+  if (!gb) return LANCET_ERR_DTYPE;
+  if (misaligned(raw_gates, gb) || misaligned(merged_indices, 4) || misaligned(gates_out, gb)) return LANCET_ERR_ALIGN;
+  return rc(run_top2_normalize(raw_gates, merged_indices, static_cast<int>(S), gate_dtype, gates_out, S_(stream)));
 }
 
 // ---- raf.op.moe_merge_masks / raf.op.moe_redispatch -------------------------------------

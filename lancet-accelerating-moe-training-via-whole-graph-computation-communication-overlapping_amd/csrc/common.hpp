@@ -68,4 +68,22 @@ __device__ __forceinline__ uint32_t f32_to_f16(float f) {
   return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
 }
 
+// ---- gate values in their storage type ------------------------------------------------------
+// Gate arrays (gate [S,E], gates_s [k*S], their gradients) are fp32, bf16 or fp16 (the LANCET_F32 / _BF16 / _F16
+// codes 0 / 1 / 2); all arithmetic on them is fp32, with one rounding to the storage type on a store.
+__device__ __forceinline__ float ld_gate(const void* p, size_t i, int gd) {
+  if (gd == 0) return static_cast<const float*>(p)[i];
+  const uint32_t h = static_cast<const uint16_t*>(p)[i];
+  return gd == 1 ? bf16_to_f32(h) : f16_to_f32(h);
+}
+__device__ __forceinline__ void st_gate(void* p, size_t i, float v, int gd) {
+  if (gd == 0) static_cast<float*>(p)[i] = v;
+  else static_cast<uint16_t*>(p)[i] = static_cast<uint16_t>(gd == 1 ? f32_to_bf16(v) : f32_to_f16(v));
+}
+// the value a gate array of type gd holds after v is stored in it
+__device__ __forceinline__ float round_gate(float v, int gd) {
+  if (gd == 0) return v;
+  return gd == 1 ? bf16_to_f32(f32_to_bf16(v)) : f16_to_f32(f32_to_f16(v));
+}
+
 }  // namespace lancet

@@ -22,19 +22,20 @@ hipError_t run_scan_ws_take_error(void* ws, int* error_out, hipStream_t st);
 
 hipError_t run_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t st);
 // noise (top-2 only, may be null): [S,E] values added to the row for the second choice
-hipError_t run_gate_topk(const float* gate, const float* noise, int S, int E, int K, bool is_logits, int32_t* idx,
-                         float* val, hipStream_t st);
+// gate_dtype (LANCET_F32 / _BF16 / _F16): storage type of gate, noise, val / gates_s
+hipError_t run_gate_topk(const void* gate, const void* noise, int S, int E, int K, bool is_logits, int gate_dtype,
+                         int32_t* idx, void* val, hipStream_t st);
 // gate-driven (idx_in == nullptr) or index-driven (gate == nullptr, K == 1) routing + scan.
 // idx_out/loc_out are [K*S] each.
-hipError_t run_route_scan(const float* gate, const float* noise, const int32_t* idx_in, const int32_t* used_in, int S,
-                          int E, int C, int M, int K, bool is_logits, float* gates_s,
+hipError_t run_route_scan(const void* gate, const void* noise, const int32_t* idx_in, const int32_t* used_in, int S,
+                          int E, int C, int M, int K, bool is_logits, int gate_dtype, void* gates_s,
                           int32_t* idx_out, int32_t* loc_out, int32_t* used_out,
                           uint64_t* elems_out, void* ws, hipStream_t st);
-hipError_t run_bpr_route(const float* gate, int S0, int E, int C, int M, int n_partitions,
-                         int partition_id, bool is_logits, float* gates_s, int32_t* idx_out,
+hipError_t run_bpr_route(const void* gate, int S0, int E, int C, int M, int n_partitions,
+                         int partition_id, bool is_logits, int gate_dtype, void* gates_s, int32_t* idx_out,
                          int32_t* loc_out, int32_t* used_out, uint64_t* elems_out, void* ws,
                          hipStream_t st);
-hipError_t run_top2_normalize(const float* raw, const int32_t* idx, int S, float* out, hipStream_t st);
+hipError_t run_top2_normalize(const void* raw, const int32_t* idx, int S, int gate_dtype, void* out, hipStream_t st);
 
 // ---- row movers (moe_rows.hip) ------------------------------------------------------
 // Scatter of token rows into [E,C,M].  avail_used (may be null): only rows with
@@ -50,16 +51,16 @@ hipError_t run_scatter_rows(const void* data, void* out, const int32_t* idx, con
                             const int32_t* rows_hi,
                             int S, int M, int E, int C, int K, int elem_bytes, hipStream_t st, int slot_stride = -1);
 hipError_t run_zero_bytes(void* p, size_t nbytes, hipStream_t st);
-hipError_t run_decode_rows(const void* expert_out, const float* gates, const int32_t* idx,
+hipError_t run_decode_rows(const void* expert_out, const void* gates, int gate_dtype, const int32_t* idx,
                            const int32_t* loc, void* out, int S, int M, int E, int C, int K,
                            int dtype, hipStream_t st, int slot_stride = -1);
 
 // backward (gates == nullptr in run_decode_rows gives moe_encode_dx)
-hipError_t run_encode_dg(const float* dy, const int32_t* idx, int S, int E, int K, float* grad_gates, hipStream_t st);
-hipError_t run_decode_dx(const void* dy, const float* gates, const int32_t* idx, const int32_t* loc, void* out,
+hipError_t run_encode_dg(const void* dy, const int32_t* idx, int S, int E, int K, int gate_dtype, void* grad_gates, hipStream_t st);
+hipError_t run_decode_dx(const void* dy, const void* gates, int gate_dtype, const int32_t* idx, const int32_t* loc, void* out,
                          int32_t* src_map, int S, int M, int E, int C, int K, int dtype, hipStream_t st);
-hipError_t run_decode_dg(const void* dy, const void* expert_out, const int32_t* idx, const int32_t* loc, float* out,
-                         int S, int M, int E, int C, int K, int dtype, hipStream_t st);
+hipError_t run_decode_dg(const void* dy, const void* expert_out, const int32_t* idx, const int32_t* loc, void* out,
+                         int gate_dtype, int S, int M, int E, int C, int K, int dtype, hipStream_t st);
 
 struct PtrTable {
   const void* p[kMaxPartitions];

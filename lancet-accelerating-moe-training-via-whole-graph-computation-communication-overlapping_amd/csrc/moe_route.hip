@@ -2,6 +2,7 @@
 // position scan, the top-2 finalisation, and the batch-prioritised (radix select) variant.
 #include "launchers.hpp"
 #include "scan.hpp"
+#include "../../include/lancet_hip.h"
 #include <algorithm>
 
 namespace lancet {
@@ -39,33 +40,75 @@ struct Routed {
   float p0, p1;
 };
 
-// noise (K = 2 only, may be null): values added to the row for the second choice alone, the first
-// choice masked out (docker/resources/sharded_moe.py:275-278); gate values always come from the row.
-template <int K>
-__device__ __forceinline__ Routed route_token(const float* __restrict__ row, const float* __restrict__ noise, int E,
-                                              bool is_logits) {
-  typedef float f32x4 __attribute__((ext_vector_type(4)));
-  TopState t = {0.f, 0.f, -1, -1};
-  const bool vec = ((E & 3) == 0) && ((reinterpret_cast<uintptr_t>(row) & 15u) == 0);
+// ---- a gate row in its storage type (GD = LANCET_F32 / LANCET_BF16 / LANCET_F16), read as fp32 ----------
+template <int GD>
+__device__ __forceinline__ float gate_at(const void* row, int j) {
+  if (GD == LANCET_F32) return static_cast<const float*>(row)[j];
+  const uint32_t h = static_cast<const uint16_t*>(row)[j];
+  return GD == LANCET_BF16 ? bf16_to_f32(h) : f16_to_f32(h);
+}
+template <int GD>
+__device__ __forceinline__ float half_word(uint32_t h) {
+  return GD == LANCET_BF16 ? bf16_to_f32(h) : f16_to_f32(h);
+}
+
+// Calls f(x, j) for j = 0 .. E-1 in order and returns f (the functor carries its state by value, so that it
+// stays in registers).  16-byte granules (4 fp32 or 8 half values) when the row allows.
+template <int GD, typename F>
+__device__ __forceinline__ F walk_row(const void* row, int E, F f) {
+  constexpr int V = GD == LANCET_F32 ? 4 : 8;
+  const bool vec = ((E & (V - 1)) == 0) && ((reinterpret_cast<uintptr_t>(row) & 15u) == 0);
   if (vec) {
-    const f32x4* r4 = reinterpret_cast<const f32x4*>(row);
-    for (int j = 0; j < E / 4; ++j) {
-      const f32x4 x = r4[j];
-      t = consider<K>(t, x.x, 4 * j);
-      t = consider<K>(t, x.y, 4 * j + 1);
-      t = consider<K>(t, x.z, 4 * j + 2);
-      t = consider<K>(t, x.w, 4 * j + 3);
+    const u32x4* r = static_cast<const u32x4*>(row);
+    for (int g = 0; g < E / V; ++g) {
+      const u32x4 x = r[g];
+      if (GD == LANCET_F32) {
+        f(__uint_as_float(x.x), 4 * g);
+        f(__uint_as_float(x.y), 4 * g + 1);
+        f(__uint_as_float(x.z), 4 * g + 2);
+        f(__uint_as_float(x.w), 4 * g + 3);
+      } else {
+        f(half_word<GD>(x.x & 0xffffu), 8 * g);
+        f(half_word<GD>(x.x >> 16), 8 * g + 1);
+        f(half_word<GD>(x.y & 0xffffu), 8 * g + 2);
+        f(half_word<GD>(x.y >> 16), 8 * g + 3);
+        f(half_word<GD>(x.z & 0xffffu), 8 * g + 4);
+        f(half_word<GD>(x.z >> 16), 8 * g + 5);
+        f(half_word<GD>(x.w & 0xffffu), 8 * g + 6);
+        f(half_word<GD>(x.w >> 16), 8 * g + 7);
+      }
     }
   } else {
-    for (int j = 0; j < E; ++j) t = consider<K>(t, row[j], j);
+    for (int j = 0; j < E; ++j) f(gate_at<GD>(row, j), j);
   }
+  return f;
+}
+
+template <int K>
+struct SelectTop {
+  TopState t;
+  __device__ __forceinline__ void operator()(float x, int j) { t = consider<K>(t, x, j); }
+};
+struct SumExp {  // sequential sum in expert order
+  float top, sum;
+  __device__ __forceinline__ void operator()(float x, int) { sum += expf(x - top); }
+};
+
+// noise (K = 2 only, may be null): values added to the row for the second choice alone, the first
+// choice masked out (docker/resources/sharded_moe.py:275-278); gate values always come from the row.
+// Row and noise are stored as GD; 16-bit values tie massively, and the first maximum wins as always.
+template <int K, int GD>
+__device__ __forceinline__ Routed route_token(const void* __restrict__ row, const void* __restrict__ noise, int E,
+                                              bool is_logits) {
+  SelectTop<K> sel = {{0.f, 0.f, -1, -1}};
+  TopState t = walk_row<GD>(row, E, sel).t;
   if (K == 2 && noise) {
     // second choice again, on row + noise: first max over the experts other than the first choice
     float best = 0.f;
     t.i2 = -1;
     for (int j = 0; j < E; ++j) {
-      const float x = row[j];
-      const float y = x + noise[j];
+      const float x = gate_at<GD>(row, j);
+      const float y = x + gate_at<GD>(noise, j);
       const bool take = (j != t.i1) & ((t.i2 < 0) | (y > best));
       best = take ? y : best;
       t.v2 = take ? x : t.v2;
@@ -74,19 +117,8 @@ __device__ __forceinline__ Routed route_token(const float* __restrict__ row, con
   }
   float sum = 1.f;
   if (is_logits) {
-    sum = 0.f;  // sequential sum in expert order
-    if (vec) {
-      const f32x4* r4 = reinterpret_cast<const f32x4*>(row);
-      for (int j = 0; j < E / 4; ++j) {
-        const f32x4 x = r4[j];
-        sum += expf(x.x - t.v1);
-        sum += expf(x.y - t.v1);
-        sum += expf(x.z - t.v1);
-        sum += expf(x.w - t.v1);
-      }
-    } else {
-      for (int j = 0; j < E; ++j) sum += expf(row[j] - t.v1);
-    }
+    SumExp se = {t.v1, 0.f};
+    sum = walk_row<GD>(row, E, se).sum;
   }
   Routed r;
   r.e0 = t.i1;
@@ -96,12 +128,20 @@ __device__ __forceinline__ Routed route_token(const float* __restrict__ row, con
   return r;
 }
 
+// GD as a compile-time constant inside `...` for the run-time code gd
+#define LANCET_GATE_SWITCH(gd, ...)                                \
+  switch (gd) {                                                    \
+    case LANCET_BF16: { constexpr int GD = LANCET_BF16; __VA_ARGS__; } break; \
+    case LANCET_F16: { constexpr int GD = LANCET_F16; __VA_ARGS__; } break;   \
+    default: { constexpr int GD = LANCET_F32; __VA_ARGS__; } break;           \
+  }
+
 struct RouteArgs {
-  const float* gate;      // [S,E] (NULL when idx_in is given)
-  const float* noise;     // [S,E] or NULL: added for the second choice (K = 2)
+  const void* gate;       // [S,E] of gate_dtype (NULL when idx_in is given)
+  const void* noise;      // [S,E] of gate_dtype or NULL: added for the second choice (K = 2)
   const int32_t* idx_in;  // launcher-level entry: expert per token already chosen (may alias idx_out)
   const int32_t* used_in; // [E] or NULL (= zeros)
-  float* gates_s;         // [K*S] (NULL when idx_in is given)
+  void* gates_s;          // [K*S] of gate_dtype (NULL when idx_in is given)
   int32_t* idx_out;       // [K*S]
   int32_t* loc_out;       // [K*S]
   int32_t* used_out;      // [E]
@@ -110,13 +150,14 @@ struct RouteArgs {
   int S, E, C, M;
   int ntiles;
   int is_logits;
+  int gate_dtype;         // LANCET_F32 / _BF16 / _F16: storage type of gate, noise and gates_s
 };
 
 // K = 1: everything is final when the tile knows its prefix.
 // K = 2: ranks of both slots are produced in one pass (2E counters); slot-2 locations need the
 //        slot-1 totals of all tiles, so raw (expert, rank, value) are left in the output arrays
 //        and finalize_top2_kernel completes them.
-template <int K>
+template <int K, int GD>
 __global__ __launch_bounds__(kTile) void route_scan_kernel(RouteArgs a) {
   extern __shared__ uint32_t s_cnt[];
   const int tid = threadIdx.x;
@@ -131,7 +172,7 @@ __global__ __launch_bounds__(kTile) void route_scan_kernel(RouteArgs a) {
       for (int j = 0; j < K; ++j) {
         a.idx_out[static_cast<size_t>(j) * a.S + s] = -1;
         a.loc_out[static_cast<size_t>(j) * a.S + s] = -1;
-        if (a.gates_s) a.gates_s[static_cast<size_t>(j) * a.S + s] = 0.f;
+        if (a.gates_s) st_gate(a.gates_s, static_cast<size_t>(j) * a.S + s, 0.f, GD);
       }
     }
     if (blockIdx.x == 0) {
@@ -155,9 +196,11 @@ __global__ __launch_bounds__(kTile) void route_scan_kernel(RouteArgs a) {
       const int x = a.idx_in[s];
       e[0] = (x >= 0 && x < a.E) ? x : -1;
     } else {
-      const Routed r = route_token<K>(a.gate + static_cast<size_t>(s) * a.E,
-                                      a.noise ? a.noise + static_cast<size_t>(s) * a.E : nullptr, a.E,
-                                      a.is_logits != 0);
+      constexpr size_t gb = GD == LANCET_F32 ? 4 : 2;
+      const size_t off = static_cast<size_t>(s) * a.E * gb;
+      const Routed r = route_token<K, GD>(static_cast<const char*>(a.gate) + off,
+                                          a.noise ? static_cast<const char*>(a.noise) + off : nullptr, a.E,
+                                          a.is_logits != 0);
       e[0] = r.e0;
       p[0] = r.p0;
       if (K == 2) {
@@ -186,7 +229,7 @@ __global__ __launch_bounds__(kTile) void route_scan_kernel(RouteArgs a) {
         a.idx_out[s] = -1;
         a.loc_out[s] = 0;
       }
-      if (a.gates_s) a.gates_s[s] = p[0];
+      if (a.gates_s) st_gate(a.gates_s, s, p[0], GD);
     }
     if (static_cast<int>(tile) == a.ntiles - 1) {
       // the last tile's inclusive prefix is the total; poisoned, it is worth nothing
@@ -207,7 +250,7 @@ __global__ __launch_bounds__(kTile) void route_scan_kernel(RouteArgs a) {
       for (int j = 0; j < K; ++j) {
         a.idx_out[static_cast<size_t>(j) * a.S + s] = poisoned ? -1 : e[j];
         a.loc_out[static_cast<size_t>(j) * a.S + s] = poisoned ? -1 : static_cast<int>(rank[j]);
-        a.gates_s[static_cast<size_t>(j) * a.S + s] = p[j];
+        st_gate(a.gates_s, static_cast<size_t>(j) * a.S + s, p[j], GD);
       }
     }
   }
@@ -230,7 +273,8 @@ __global__ __launch_bounds__(kTile) void finalize_top2_kernel(RouteArgs a) {
     if (poisoned) {
       a.idx_out[s] = a.idx_out[a.S + s] = -1;
       a.loc_out[s] = a.loc_out[a.S + s] = -1;
-      a.gates_s[s] = a.gates_s[a.S + s] = 0.f;
+      st_gate(a.gates_s, s, 0.f, a.gate_dtype);
+      st_gate(a.gates_s, static_cast<size_t>(a.S) + s, 0.f, a.gate_dtype);
     } else {
       const int e1 = a.idx_out[s], e2 = a.idx_out[a.S + s];
       const int r1 = a.loc_out[s], r2 = a.loc_out[a.S + s];
@@ -245,11 +289,12 @@ __global__ __launch_bounds__(kTile) void finalize_top2_kernel(RouteArgs a) {
       a.loc_out[s] = keep1 ? r1 : -1;
       a.idx_out[a.S + s] = keep2 ? e2 : -1;
       a.loc_out[a.S + s] = keep2 ? r2 + static_cast<int>(after1 - u2) : -1;
-      const float g1 = keep1 ? a.gates_s[s] : 0.f;
-      const float g2 = keep2 ? a.gates_s[a.S + s] : 0.f;
+      // the raw values as the scan stored them (rounded to the gate type), normalised in fp32, rounded once
+      const float g1 = keep1 ? ld_gate(a.gates_s, s, a.gate_dtype) : 0.f;
+      const float g2 = keep2 ? ld_gate(a.gates_s, static_cast<size_t>(a.S) + s, a.gate_dtype) : 0.f;
       const float den = fmaxf(g1 + g2, 1.1920929e-07f);
-      a.gates_s[s] = g1 / den;
-      a.gates_s[a.S + s] = g2 / den;
+      st_gate(a.gates_s, s, g1 / den, a.gate_dtype);
+      st_gate(a.gates_s, static_cast<size_t>(a.S) + s, g2 / den, a.gate_dtype);
     }
   }
   if (blockIdx.x == 0) {
@@ -265,29 +310,31 @@ __global__ __launch_bounds__(kTile) void finalize_top2_kernel(RouteArgs a) {
 }
 
 // Selection only (no scan).
-template <int K>
-__global__ __launch_bounds__(kTile) void gate_topk_kernel(const float* gate, const float* noise, int S, int E,
-                                                          int is_logits, int32_t* idx, float* val) {
+template <int K, int GD>
+__global__ __launch_bounds__(kTile) void gate_topk_kernel(const void* gate, const void* noise, int S, int E,
+                                                          int is_logits, int32_t* idx, void* val) {
   const int s = blockIdx.x * kTile + threadIdx.x;
   if (s >= S) return;
-  const Routed r = route_token<K>(gate + static_cast<size_t>(s) * E, noise ? noise + static_cast<size_t>(s) * E : nullptr,
-                                  E, is_logits != 0);
+  constexpr size_t gb = GD == LANCET_F32 ? 4 : 2;
+  const size_t off = static_cast<size_t>(s) * E * gb;
+  const Routed r = route_token<K, GD>(static_cast<const char*>(gate) + off,
+                                      noise ? static_cast<const char*>(noise) + off : nullptr, E, is_logits != 0);
   idx[s] = r.e0;
-  val[s] = r.p0;
+  st_gate(val, s, r.p0, GD);
   if (K == 2) {
     idx[static_cast<size_t>(S) + s] = r.e1;
-    val[static_cast<size_t>(S) + s] = r.p1;
+    st_gate(val, static_cast<size_t>(S) + s, r.p1, GD);
   }
 }
 
-__global__ void top2_normalize_kernel(const float* raw, const int32_t* idx, int S, float* out) {
+__global__ void top2_normalize_kernel(const void* raw, const int32_t* idx, int S, void* out, int gd) {
   const int s = blockIdx.x * blockDim.x + threadIdx.x;
   if (s >= S) return;
-  const float g1 = idx[s] >= 0 ? raw[s] : 0.f;
-  const float g2 = idx[S + s] >= 0 ? raw[S + s] : 0.f;
+  const float g1 = idx[s] >= 0 ? ld_gate(raw, s, gd) : 0.f;
+  const float g2 = idx[S + s] >= 0 ? ld_gate(raw, static_cast<size_t>(S) + s, gd) : 0.f;
   const float den = fmaxf(g1 + g2, 1.1920929e-07f);
-  out[s] = g1 / den;
-  out[S + s] = g2 / den;
+  st_gate(out, s, g1 / den, gd);
+  st_gate(out, static_cast<size_t>(S) + s, g2 / den, gd);
 }
 
 __global__ void fill_u32_kernel(uint32_t* p, size_t n, uint32_t v) {
@@ -325,7 +372,8 @@ struct BprArgs {
   int S0, S, E, C, M;
   int part_lo;           // first token of the partition
   int ntiles;
-  float* gates_s;        // [S]
+  int gate_dtype;        // storage type of gates_s (and of the gate the priorities came from)
+  void* gates_s;         // [S]
   int32_t* idx_out;      // [S]
   int32_t* loc_out;      // [S]
   int32_t* used_out;     // [E]
@@ -340,11 +388,14 @@ __device__ __forceinline__ float tok_prio(uint64_t w) { return __uint_as_float(s
 __device__ __forceinline__ uint32_t par_value(const uint64_t* p) { return static_cast<uint32_t>(*p); }
 
 // first choice and its gate value (or softmax probability) of every token of the batch
-__global__ __launch_bounds__(kTile) void bpr_prepare_kernel(const float* gate, int S0, int E, int is_logits, uint64_t* tok) {
+// (the priority is the gate value as gates_s will hold it: rounded to the gate type)
+template <int GD>
+__global__ __launch_bounds__(kTile) void bpr_prepare_kernel(const void* gate, int S0, int E, int is_logits, uint64_t* tok) {
   const int s = blockIdx.x * kTile + threadIdx.x;
   if (s >= S0) return;
-  const Routed r = route_token<1>(gate + static_cast<size_t>(s) * E, nullptr, E, is_logits != 0);
-  tok[s] = foreign_word(static_cast<uint32_t>(r.e0 + 1), __float_as_uint(r.p0));
+  constexpr size_t gb = GD == LANCET_F32 ? 4 : 2;
+  const Routed r = route_token<1, GD>(static_cast<const char*>(gate) + static_cast<size_t>(s) * E * gb, nullptr, E, is_logits != 0);
+  tok[s] = foreign_word(static_cast<uint32_t>(r.e0 + 1), __float_as_uint(round_gate(r.p0, GD)));
 }
 
 __global__ __launch_bounds__(kSelectThreads) void bpr_select_kernel(BprArgs a) {
@@ -434,7 +485,7 @@ __global__ __launch_bounds__(kTile) void bpr_scan_kernel(BprArgs a) {
     if (valid) {
       a.idx_out[sl] = -1;
       a.loc_out[sl] = -1;
-      a.gates_s[sl] = 0.f;
+      st_gate(a.gates_s, sl, 0.f, a.gate_dtype);
     }
     if (blockIdx.x == 0) {
       for (int c = tid; c < a.E; c += kTile) {
@@ -475,7 +526,7 @@ __global__ __launch_bounds__(kTile) void bpr_scan_kernel(BprArgs a) {
     }
     a.idx_out[sl] = idx;
     a.loc_out[sl] = loc;
-    a.gates_s[sl] = prio;
+    st_gate(a.gates_s, sl, prio, a.gate_dtype);
   }
   if (static_cast<int>(tile) == a.ntiles - 1) {
     const uint32_t* s_agg = s_cnt + kWavesPerTile * 2 * a.E;
@@ -543,17 +594,18 @@ hipError_t run_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t st) {
   return hipGetLastError();
 }
 
-hipError_t run_gate_topk(const float* gate, const float* noise, int S, int E, int K, bool is_logits, int32_t* idx,
-                         float* val, hipStream_t st) {
+hipError_t run_gate_topk(const void* gate, const void* noise, int S, int E, int K, bool is_logits, int gate_dtype,
+                         int32_t* idx, void* val, hipStream_t st) {
   if (S == 0) return hipSuccess;
   const int blocks = (S + kTile - 1) / kTile;
-  if (K == 1) gate_topk_kernel<1><<<blocks, kTile, 0, st>>>(gate, nullptr, S, E, is_logits, idx, val);
-  else gate_topk_kernel<2><<<blocks, kTile, 0, st>>>(gate, noise, S, E, is_logits, idx, val);
+  LANCET_GATE_SWITCH(gate_dtype,
+    if (K == 1) gate_topk_kernel<1, GD><<<blocks, kTile, 0, st>>>(gate, nullptr, S, E, is_logits, idx, val);
+    else gate_topk_kernel<2, GD><<<blocks, kTile, 0, st>>>(gate, noise, S, E, is_logits, idx, val))
   return hipGetLastError();
 }
 
-hipError_t run_route_scan(const float* gate, const float* noise, const int32_t* idx_in, const int32_t* used_in, int S,
-                          int E, int C, int M, int K, bool is_logits, float* gates_s,
+hipError_t run_route_scan(const void* gate, const void* noise, const int32_t* idx_in, const int32_t* used_in, int S,
+                          int E, int C, int M, int K, bool is_logits, int gate_dtype, void* gates_s,
                           int32_t* idx_out, int32_t* loc_out, int32_t* used_out,
                           uint64_t* elems_out, void* ws, hipStream_t st) {
   RouteArgs a;
@@ -572,13 +624,14 @@ hipError_t run_route_scan(const float* gate, const float* noise, const int32_t* 
   a.M = M;
   a.ntiles = static_cast<int>(scan_num_tiles(S));
   a.is_logits = is_logits;
+  a.gate_dtype = gate_dtype;
   a.ws = scan_ws_view(ws);
   hipError_t err = hipSuccess;
   const size_t lds = scan_lds_bytes(K * E);
   if (K == 1) {
-    route_scan_kernel<1><<<a.ntiles, kTile, lds, st>>>(a);
+    LANCET_GATE_SWITCH(gate_dtype, (route_scan_kernel<1, GD><<<a.ntiles, kTile, lds, st>>>(a)))
   } else {
-    route_scan_kernel<2><<<a.ntiles, kTile, lds, st>>>(a);
+    LANCET_GATE_SWITCH(gate_dtype, (route_scan_kernel<2, GD><<<a.ntiles, kTile, lds, st>>>(a)))
     err = hipGetLastError();
     if (err != hipSuccess) return err;
     finalize_top2_kernel<<<a.ntiles, kTile, 0, st>>>(a);
@@ -586,8 +639,8 @@ hipError_t run_route_scan(const float* gate, const float* noise, const int32_t* 
   return hipGetLastError();
 }
 
-hipError_t run_bpr_route(const float* gate, int S0, int E, int C, int M, int n_partitions,
-                         int partition_id, bool is_logits, float* gates_s, int32_t* idx_out,
+hipError_t run_bpr_route(const void* gate, int S0, int E, int C, int M, int n_partitions,
+                         int partition_id, bool is_logits, int gate_dtype, void* gates_s, int32_t* idx_out,
                          int32_t* loc_out, int32_t* used_out, uint64_t* elems_out, void* ws,
                          hipStream_t st) {
   const int S = S0 / n_partitions;
@@ -603,13 +656,14 @@ hipError_t run_bpr_route(const float* gate, int S0, int E, int C, int M, int n_p
   a.tok = reinterpret_cast<uint64_t*>(static_cast<char*>(ws) + scan_ws_bytes(a.ntiles, 2 * E));
   a.par = a.tok + S0;
   a.gates_s = gates_s;
+  a.gate_dtype = gate_dtype;
   a.idx_out = idx_out;
   a.loc_out = loc_out;
   a.used_out = used_out;
   a.elems_out = elems_out;
   hipError_t err = hipSuccess;
   if (S0 > 0) {
-    bpr_prepare_kernel<<<(S0 + kTile - 1) / kTile, kTile, 0, st>>>(gate, S0, E, is_logits, a.tok);
+    LANCET_GATE_SWITCH(gate_dtype, (bpr_prepare_kernel<GD><<<(S0 + kTile - 1) / kTile, kTile, 0, st>>>(gate, S0, E, is_logits, a.tok)))
     err = hipGetLastError();
     if (err != hipSuccess) return err;
   }
@@ -620,9 +674,9 @@ hipError_t run_bpr_route(const float* gate, int S0, int E, int C, int M, int n_p
   return hipGetLastError();
 }
 
-hipError_t run_top2_normalize(const float* raw, const int32_t* idx, int S, float* out, hipStream_t st) {
+hipError_t run_top2_normalize(const void* raw, const int32_t* idx, int S, int gate_dtype, void* out, hipStream_t st) {
   if (S == 0) return hipSuccess;
-  top2_normalize_kernel<<<(S + 255) / 256, 256, 0, st>>>(raw, idx, S, out);
+  top2_normalize_kernel<<<(S + 255) / 256, 256, 0, st>>>(raw, idx, S, out, gate_dtype);
   return hipGetLastError();
 }
 

@@ -185,7 +185,8 @@ __device__ __forceinline__ u32x4 combine_vec(const u32x4 (&x)[K], const float (&
 
 struct DecodeArgs {
   const void* expert_out;
-  const float* gates;    // [K*S]; null = all ones (moe_encode_dx)
+  const void* gates;     // [K*S] of gate_dtype; null = all ones (moe_encode_dx)
+  int gate_dtype;
   const int32_t* idx;    // [K*S]
   const int32_t* loc;    // [K*S]
   void* out;             // [S, M]
@@ -213,7 +214,7 @@ __global__ __launch_bounds__(kTile) void decode_rows_kernel(DecodeArgs a) {
     const int e = a.idx[static_cast<size_t>(j) * a.slot_stride + s];
     const int l = a.loc[static_cast<size_t>(j) * a.slot_stride + s];
     ok[j] = e >= 0 && e < a.E && l >= 0 && l < a.C;
-    g[j] = ok[j] ? (a.gates ? a.gates[static_cast<size_t>(j) * a.slot_stride + s] : 1.f) : 0.f;
+    g[j] = ok[j] ? (a.gates ? ld_gate(a.gates, static_cast<size_t>(j) * a.slot_stride + s, a.gate_dtype) : 1.f) : 0.f;
     row[j] = ok[j] ? (static_cast<size_t>(e) * a.C + l) : 0;
     any = any || ok[j];
   }
@@ -442,17 +443,17 @@ __global__ __launch_bounds__(kTile) void redispatch_expert_input_kernel(PtrTable
 // encode_backward_gate_kernel (tutel_moe_dispatch.cu:96-105, 499-506) as one pass that writes every
 // element once.
 template <int K>
-__global__ __launch_bounds__(kTile) void encode_dg_kernel(const float* dy, const int32_t* idx, int S, int E,
-                                                          float* grad_gates) {
+__global__ __launch_bounds__(kTile) void encode_dg_kernel(const void* dy, const int32_t* idx, int S, int E,
+                                                          void* grad_gates, int gd) {
   const size_t n = static_cast<size_t>(S) * E;
   for (size_t i = blockIdx.x * static_cast<size_t>(kTile) + threadIdx.x; i < n;
        i += static_cast<size_t>(gridDim.x) * kTile) {
     const int s = static_cast<int>(i / E);
     const int e = static_cast<int>(i - static_cast<size_t>(s) * E);
     float v = 0.f;
-    if (idx[s] == e) v = dy[s];
-    if (K == 2 && idx[S + s] == e) v = dy[S + s];
-    grad_gates[i] = v;
+    if (idx[s] == e) v = ld_gate(dy, s, gd);
+    if (K == 2 && idx[S + s] == e) v = ld_gate(dy, static_cast<size_t>(S) + s, gd);
+    st_gate(grad_gates, i, v, gd);
   }
 }
 
@@ -469,7 +470,7 @@ __global__ __launch_bounds__(kTile) void inverse_map_kernel(const int32_t* idx, 
 // for rows nobody owns: decode_backward_data_kernel (tutel_moe_dispatch.cu:118-124, 523-533) without
 // the memset + atomicAdd; every output byte is written once.
 template <int DT, bool VEC>
-__global__ __launch_bounds__(kTile) void decode_dx_rows_kernel(const void* dy, const float* gates,
+__global__ __launch_bounds__(kTile) void decode_dx_rows_kernel(const void* dy, const void* gates, int gd,
                                                                const int32_t* src, void* out, int S, int M,
                                                                long rows, int wpr_shift) {
   typedef Codec<DT> Cd;
@@ -481,7 +482,7 @@ __global__ __launch_bounds__(kTile) void decode_dx_rows_kernel(const void* dy, c
   const int step = kWave << wpr_shift;
   if (r >= rows) return;
   const int i = src[r];
-  const float g1[1] = {i >= 0 ? gates[i] : 0.f};
+  const float g1[1] = {i >= 0 ? ld_gate(gates, i, gd) : 0.f};
   const size_t s = i >= 0 ? static_cast<size_t>(i % S) : 0;
   if (VEC) {
     const int row_vecs = M / Cd::kPerVec;
@@ -517,7 +518,7 @@ __global__ __launch_bounds__(kTile) void decode_dx_rows_kernel(const void* dy, c
 // sums per lane, xor-tree over the wave.
 template <int DT, bool VEC>
 __global__ __launch_bounds__(kTile) void decode_dg_kernel(const void* dy, const void* expert_out,
-                                                          const int32_t* idx, const int32_t* loc, float* out,
+                                                          const int32_t* idx, const int32_t* loc, void* out, int gd,
                                                           int S, int M, int E, int C, int n) {
   typedef Codec<DT> Cd;
   const int w = threadIdx.x / kWave;
@@ -526,7 +527,7 @@ __global__ __launch_bounds__(kTile) void decode_dg_kernel(const void* dy, const 
   if (i >= n) return;
   const int e = idx[i], l = loc[i];
   if (!(e >= 0 && e < E && l >= 0 && l < C)) {
-    if (lane == 0) out[i] = 0.f;
+    if (lane == 0) st_gate(out, i, 0.f, gd);
     return;
   }
   const size_t s = static_cast<size_t>(i % S);
@@ -555,7 +556,7 @@ __global__ __launch_bounds__(kTile) void decode_dg_kernel(const void* dy, const 
     for (int k = lane; k < M; k += kWave) acc += Cd::get(a[k]) * Cd::get(b[k]);
   }
   acc = wave_sum(acc);
-  if (lane == 0) out[i] = acc;
+  if (lane == 0) st_gate(out, i, acc, gd);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -657,12 +658,13 @@ static hipError_t decode_launch(DecodeArgs a, int K, bool vec, hipStream_t st) {
   return hipGetLastError();
 }
 
-hipError_t run_decode_rows(const void* expert_out, const float* gates, const int32_t* idx,
+hipError_t run_decode_rows(const void* expert_out, const void* gates, int gate_dtype, const int32_t* idx,
                            const int32_t* loc, void* out, int S, int M, int E, int C, int K,
                            int dtype, hipStream_t st, int slot_stride) {
   DecodeArgs a;
   a.expert_out = expert_out;
   a.gates = gates;
+  a.gate_dtype = gate_dtype;
   a.idx = idx;
   a.loc = loc;
   a.out = out;
@@ -717,26 +719,26 @@ hipError_t run_redispatch_rows(const PtrTable& bufs, int P, int M, int C, int E,
   return hipGetLastError();
 }
 
-hipError_t run_encode_dg(const float* dy, const int32_t* idx, int S, int E, int K, float* grad_gates, hipStream_t st) {
+hipError_t run_encode_dg(const void* dy, const int32_t* idx, int S, int E, int K, int gate_dtype, void* grad_gates, hipStream_t st) {
   const size_t n = static_cast<size_t>(S) * E;
   if (n == 0) return hipSuccess;
   const int blocks = static_cast<int>(std::min<size_t>((n + kTile - 1) / kTile, 65536));
-  if (K == 1) encode_dg_kernel<1><<<blocks, kTile, 0, st>>>(dy, idx, S, E, grad_gates);
-  else encode_dg_kernel<2><<<blocks, kTile, 0, st>>>(dy, idx, S, E, grad_gates);
+  if (K == 1) encode_dg_kernel<1><<<blocks, kTile, 0, st>>>(dy, idx, S, E, grad_gates, gate_dtype);
+  else encode_dg_kernel<2><<<blocks, kTile, 0, st>>>(dy, idx, S, E, grad_gates, gate_dtype);
   return hipGetLastError();
 }
 
 template <int DT>
-static hipError_t decode_dx_launch(const void* dy, const float* gates, const int32_t* src, void* out, int S, int M,
+static hipError_t decode_dx_launch(const void* dy, const void* gates, int gd, const int32_t* src, void* out, int S, int M,
                                    long rows, bool vec, hipStream_t st) {
   const int shift = split_waves(vec ? M / Codec<DT>::kPerVec : M, rows, 2);  // two granules per lane: 442 -> 408 us
   const unsigned blocks = static_cast<unsigned>(((rows << shift) + kRowsPerBlock - 1) / kRowsPerBlock);
-  if (vec) decode_dx_rows_kernel<DT, true><<<blocks, kTile, 0, st>>>(dy, gates, src, out, S, M, rows, shift);
-  else decode_dx_rows_kernel<DT, false><<<blocks, kTile, 0, st>>>(dy, gates, src, out, S, M, rows, shift);
+  if (vec) decode_dx_rows_kernel<DT, true><<<blocks, kTile, 0, st>>>(dy, gates, gd, src, out, S, M, rows, shift);
+  else decode_dx_rows_kernel<DT, false><<<blocks, kTile, 0, st>>>(dy, gates, gd, src, out, S, M, rows, shift);
   return hipGetLastError();
 }
 
-hipError_t run_decode_dx(const void* dy, const float* gates, const int32_t* idx, const int32_t* loc, void* out,
+hipError_t run_decode_dx(const void* dy, const void* gates, int gate_dtype, const int32_t* idx, const int32_t* loc, void* out,
                          int32_t* src_map, int S, int M, int E, int C, int K, int dtype, hipStream_t st) {
   const long rows = static_cast<long>(E) * C;
   if (rows == 0 || M == 0) return hipSuccess;
@@ -751,31 +753,31 @@ hipError_t run_decode_dx(const void* dy, const float* gates, const int32_t* idx,
   const int per_vec = (dtype == LANCET_F32) ? 4 : 8;
   const bool vec = (M % per_vec == 0) && aligned16(dy) && aligned16(out);
   switch (dtype) {
-    case LANCET_F32: return decode_dx_launch<LANCET_F32>(dy, gates, src_map, out, S, M, rows, vec, st);
-    case LANCET_BF16: return decode_dx_launch<LANCET_BF16>(dy, gates, src_map, out, S, M, rows, vec, st);
-    default: return decode_dx_launch<LANCET_F16>(dy, gates, src_map, out, S, M, rows, vec, st);
+    case LANCET_F32: return decode_dx_launch<LANCET_F32>(dy, gates, gate_dtype, src_map, out, S, M, rows, vec, st);
+    case LANCET_BF16: return decode_dx_launch<LANCET_BF16>(dy, gates, gate_dtype, src_map, out, S, M, rows, vec, st);
+    default: return decode_dx_launch<LANCET_F16>(dy, gates, gate_dtype, src_map, out, S, M, rows, vec, st);
   }
 }
 
 template <int DT>
 static hipError_t decode_dg_launch(const void* dy, const void* expert_out, const int32_t* idx, const int32_t* loc,
-                                   float* out, int S, int M, int E, int C, int n, bool vec, hipStream_t st) {
+                                   void* out, int gd, int S, int M, int E, int C, int n, bool vec, hipStream_t st) {
   const int blocks = (n + kRowsPerBlock - 1) / kRowsPerBlock;
-  if (vec) decode_dg_kernel<DT, true><<<blocks, kTile, 0, st>>>(dy, expert_out, idx, loc, out, S, M, E, C, n);
-  else decode_dg_kernel<DT, false><<<blocks, kTile, 0, st>>>(dy, expert_out, idx, loc, out, S, M, E, C, n);
+  if (vec) decode_dg_kernel<DT, true><<<blocks, kTile, 0, st>>>(dy, expert_out, idx, loc, out, gd, S, M, E, C, n);
+  else decode_dg_kernel<DT, false><<<blocks, kTile, 0, st>>>(dy, expert_out, idx, loc, out, gd, S, M, E, C, n);
   return hipGetLastError();
 }
 
-hipError_t run_decode_dg(const void* dy, const void* expert_out, const int32_t* idx, const int32_t* loc, float* out,
-                         int S, int M, int E, int C, int K, int dtype, hipStream_t st) {
+hipError_t run_decode_dg(const void* dy, const void* expert_out, const int32_t* idx, const int32_t* loc, void* out,
+                         int gate_dtype, int S, int M, int E, int C, int K, int dtype, hipStream_t st) {
   const int n = K * S;
   if (n == 0) return hipSuccess;
   const int per_vec = (dtype == LANCET_F32) ? 4 : 8;
   const bool vec = (M % per_vec == 0) && aligned16(dy) && aligned16(expert_out);
   switch (dtype) {
-    case LANCET_F32: return decode_dg_launch<LANCET_F32>(dy, expert_out, idx, loc, out, S, M, E, C, n, vec, st);
-    case LANCET_BF16: return decode_dg_launch<LANCET_BF16>(dy, expert_out, idx, loc, out, S, M, E, C, n, vec, st);
-    default: return decode_dg_launch<LANCET_F16>(dy, expert_out, idx, loc, out, S, M, E, C, n, vec, st);
+    case LANCET_F32: return decode_dg_launch<LANCET_F32>(dy, expert_out, idx, loc, out, gate_dtype, S, M, E, C, n, vec, st);
+    case LANCET_BF16: return decode_dg_launch<LANCET_BF16>(dy, expert_out, idx, loc, out, gate_dtype, S, M, E, C, n, vec, st);
+    default: return decode_dg_launch<LANCET_F16>(dy, expert_out, idx, loc, out, gate_dtype, S, M, E, C, n, vec, st);
   }
 }
 

@@ -54,9 +54,9 @@ int scratch_for_current_device(void** out, lancet_stream_t stream) {
 
 }  // namespace
 
-extern "C" int lancet_moe_encode_noalloc(const void* data, const float* gate, const float* gate2_noise,
+extern "C" int lancet_moe_encode_noalloc(const void* data, const void* gate, const void* gate2_noise,
                                          const int32_t* used_in, int64_t S, int64_t M, int64_t E, int64_t C,
-                                         int top_k, int dtype, unsigned flags, float* gates_s,
+                                         int top_k, int dtype, int gate_dtype, unsigned flags, void* gates_s,
                                          int32_t* indices_locations, int32_t* used_out,
                                          uint64_t* elements_per_expert, void* dispatched, lancet_stream_t stream) {
   if (S < 0 || E < 1 || E > LANCET_MAX_EXPERTS) return LANCET_ERR_SHAPE;
@@ -66,7 +66,7 @@ extern "C" int lancet_moe_encode_noalloc(const void* data, const float* gate, co
   void* ws = nullptr;
   if (int r = scratch_for_current_device(&ws, stream)) return r;
   // the same kernels as lancet_moe_encode
-  return lancet_moe_encode(data, gate, gate2_noise, used_in, S, M, E, C, top_k, dtype, flags, gates_s,
+  return lancet_moe_encode(data, gate, gate2_noise, used_in, S, M, E, C, top_k, dtype, gate_dtype, flags, gates_s,
                            indices_locations, used_out, elements_per_expert, dispatched, ws,
                            LANCET_NOALLOC_SCRATCH_BYTES, stream);
 }

@@ -40,7 +40,7 @@ class _MoeEncode(torch.autograd.Function):
             P, pid = ctx.bpr
             S = indloc.shape[1]
             full_x = torch.zeros(ctx.data_shape, dtype=ctx.data_dtype, device=dx.device)
-            full_g = torch.zeros((ctx.data_shape[0], ctx.n_experts), dtype=torch.float32, device=dx.device)
+            full_g = torch.zeros((ctx.data_shape[0], ctx.n_experts), dtype=dg.dtype, device=dx.device)
             full_x[pid * S:(pid + 1) * S] = dx
             full_g[pid * S:(pid + 1) * S] = dg
             dx, dg = full_x, full_g
@@ -58,7 +58,7 @@ class _MoeDecode(torch.autograd.Function):
         data, gate, indloc = ctx.saved_tensors
         E, C, _ = data.shape
         dy = dy.contiguous()
-        return ops.moe_decode_dx(dy, gate, indloc, E, C), ops.moe_decode_dg(dy, data, indloc), None
+        return ops.moe_decode_dx(dy, gate, indloc, E, C), ops.moe_decode_dg(dy, data, indloc, gate_dtype=gate.dtype), None
 
 
 def moe_encode(data, gate, used_capacity=None, capacity_factor=1.0):

@@ -31,6 +31,14 @@ def _dtype_code(t):
     return _DTYPES[t.dtype]
 
 
+def _gate_code(t, name="gate"):
+    """Gate arrays (gate, gate2_noise, gates_s and their gradients) are float32, or a half type as a
+    mixed-precision graph has them (python/raf/amp/type_hints.py:97,105); arithmetic on them is fp32."""
+    if t.dtype not in _DTYPES:
+        raise TypeError("%s must be float32, bfloat16 or float16, got %s" % (name, t.dtype))
+    return _DTYPES[t.dtype]
+
+
 def _need(cond, msg):
     if not cond:
         raise ValueError(msg)
@@ -116,7 +124,7 @@ def _check_encode_inputs(data, gate):
     _need(data.dim() == 2, "Expected input data to be 2D.")
     _need(gate.dim() == 2, "Expected input gate to be 2D.")
     _need(data.shape[0] == gate.shape[0], "Input data and gate should have matching shape in dim 0.")
-    _need(gate.dtype == torch.float32, "gate must be float32")
+    _gate_code(gate)
     return _dtype_code(data)
 
 
@@ -134,7 +142,7 @@ def _check_noise(gate2_noise, gate, top_k):
         return
     _dev(gate2_noise, "gate2_noise")
     _need(top_k == 2, "gate2_noise only exists for the second choice (top_k = 2)")
-    _need(gate2_noise.shape == gate.shape and gate2_noise.dtype == torch.float32, "gate2_noise must be float32 [S, E]")
+    _need(gate2_noise.shape == gate.shape and gate2_noise.dtype == gate.dtype, "gate2_noise must have the gate's shape and dtype")
 
 
 def moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_logits=False,
@@ -163,7 +171,7 @@ def moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_
               "Input used_capacity should be 1-D int32 of length E.")
     dev = data.device
     if out is None:
-        gates_s = torch.empty(top_k * S, dtype=torch.float32, device=dev)
+        gates_s = torch.empty(top_k * S, dtype=gate.dtype, device=dev)
         indloc = torch.empty((2, top_k * S), dtype=torch.int32, device=dev)
         used_out = torch.empty(E, dtype=torch.int32, device=dev)
         elems = torch.empty(E, dtype=torch.int64, device=dev)
@@ -171,8 +179,9 @@ def moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_
     else:
         gates_s, indloc, used_out, elems, disp = out
     ws = _scan_workspace(moe_encode_workspace_bytes(S, E, top_k), dev, workspace)
+    _need(gates_s.dtype == gate.dtype, "gates_s takes the gate's dtype")
     st = lib.lancet_moe_encode(_p(data), _p(gate), _p(gate2_noise), _p(used_capacity), S, M, E, Cap, top_k, dt,
-                               _flags(gate_is_logits, zero_tail, rows_at_used), _p(gates_s), _p(indloc),
+                               _gate_code(gate), _flags(gate_is_logits, zero_tail, rows_at_used), _p(gates_s), _p(indloc),
                                _p(used_out), _p(elems), _p(disp), _p(ws.buf), ws.nbytes, _stream())
     capi.check(st, "lancet_moe_encode")
     return gates_s, indloc, used_out, elems.view(torch.uint64) if elems.dtype == torch.int64 else elems, disp
@@ -185,19 +194,21 @@ def moe_route(gate, used_capacity, M, capacity_factor=1.0, top_k=1, gate_is_logi
     elements_per_expert.  Returns (gates_s, indices_locations, used_capacity, elements_per_expert)."""
     lib = capi.load()
     _dev(gate, "gate")
-    _need(gate.dim() == 2 and gate.dtype == torch.float32, "gate must be 2-D float32")
+    _need(gate.dim() == 2, "gate must be 2-D")
+    gd = _gate_code(gate)
     S, E = gate.shape
     _need(top_k in (1, 2), "top_k must be 1 or 2")
     _check_noise(gate2_noise, gate, top_k)
     Cap = moe_capacity(S, E, float(capacity_factor) * (2.0 if top_k == 2 else 1.0))
     dev = gate.device
     if out is None:
-        out = (torch.empty(top_k * S, dtype=torch.float32, device=dev),
+        out = (torch.empty(top_k * S, dtype=gate.dtype, device=dev),
                torch.empty((2, top_k * S), dtype=torch.int32, device=dev),
                torch.empty(E, dtype=torch.int32, device=dev), torch.empty(E, dtype=torch.int64, device=dev))
     gates_s, indloc, used_out, elems = out[:4]
     ws = _scan_workspace(moe_encode_workspace_bytes(S, E, top_k), dev, workspace)
-    st = lib.lancet_moe_route(_p(gate), _p(gate2_noise), _p(used_capacity), S, int(M), E, Cap, top_k, _flags(gate_is_logits, True),
+    _need(gates_s.dtype == gate.dtype, "gates_s takes the gate's dtype")
+    st = lib.lancet_moe_route(_p(gate), _p(gate2_noise), _p(used_capacity), S, int(M), E, Cap, top_k, gd, _flags(gate_is_logits, True),
                               _p(gates_s), _p(indloc), _p(used_out), _p(elems), _p(ws.buf), ws.nbytes, _stream())
     capi.check(st, "lancet_moe_route")
     return gates_s, indloc, used_out, elems
@@ -250,7 +261,7 @@ def moe_decode_tokens(data, gate, indices_locations, token_first, n_tokens, top_
     lib = capi.load()
     _dev(data, "data"), _dev(gate, "gate")
     _need(data.dim() == 3, "Expected input data to be 3D.")
-    _need(gate.dim() == 1 and gate.dtype == torch.float32, "gate must be 1-D float32")
+    _need(gate.dim() == 1, "gate must be 1-D")
     S_total = _check_indloc(indices_locations, top_k)
     _need(gate.shape[0] == top_k * S_total, "gate and indices_locations disagree on the token count")
     _need(0 <= token_first and 0 <= n_tokens and token_first + n_tokens <= S_total, "token range outside the routed batch")
@@ -258,7 +269,7 @@ def moe_decode_tokens(data, gate, indices_locations, token_first, n_tokens, top_
     if out is None:
         out = torch.empty((n_tokens, M), dtype=data.dtype, device=data.device)
     st = lib.lancet_moe_decode_tokens(_p(data), _p(gate), _p(indices_locations), S_total, int(token_first),
-                                      int(n_tokens), M, E, Cap, top_k, _dtype_code(data), _p(out), _stream())
+                                      int(n_tokens), M, E, Cap, top_k, _dtype_code(data), _gate_code(gate), _p(out), _stream())
     capi.check(st, "lancet_moe_decode_tokens")
     return out
 
@@ -282,7 +293,7 @@ def moe_encode_batch_prioritized(data, gate, n_partitions=1, partition_id=0, cap
     Cap = moe_capacity(S, E, capacity_factor)
     dev = data.device
     if out is None:
-        gates_s = torch.empty(S, dtype=torch.float32, device=dev)
+        gates_s = torch.empty(S, dtype=gate.dtype, device=dev)
         indloc = torch.empty((2, S), dtype=torch.int32, device=dev)
         used_out = torch.empty(E, dtype=torch.int32, device=dev)
         elems = torch.empty(E, dtype=torch.int64, device=dev)
@@ -290,7 +301,8 @@ def moe_encode_batch_prioritized(data, gate, n_partitions=1, partition_id=0, cap
     else:
         gates_s, indloc, used_out, elems, disp = out
     ws = _scan_workspace(moe_encode_bpr_workspace_bytes(S0, E, n_partitions), dev, workspace)
-    st = lib.lancet_moe_encode_bpr(_p(data), _p(gate), S0, M, E, Cap, n_partitions, partition_id, dt,
+    _need(gates_s.dtype == gate.dtype, "gates_s takes the gate's dtype")
+    st = lib.lancet_moe_encode_bpr(_p(data), _p(gate), S0, M, E, Cap, n_partitions, partition_id, dt, _gate_code(gate),
                                    _flags(gate_is_logits, zero_tail), _p(gates_s), _p(indloc),
                                    _p(used_out), _p(elems), _p(disp), _p(ws.buf), ws.nbytes, _stream())
     capi.check(st, "lancet_moe_encode_bpr")
@@ -298,12 +310,12 @@ def moe_encode_batch_prioritized(data, gate, n_partitions=1, partition_id=0, cap
 
 
 def moe_decode(data, gate, indices_locations, top_k=1, out=None):
-    """raf.op.moe_decode(data [E,C,M], gate [k*S] f32, indices_locations [2, k*S]) -> [S, M]."""
+    """raf.op.moe_decode(data [E,C,M], gate [k*S], indices_locations [2, k*S]) -> [S, M]."""
     lib = capi.load()
     _dev(data, "data"), _dev(gate, "gate"), _dev(indices_locations, "indices_locations")
     _need(data.dim() == 3, "Expected input data to be 3D.")
     _need(gate.dim() == 1, "Expected input gate to be 1D.")
-    _need(gate.dtype == torch.float32, "gate must be float32")
+    gd = _gate_code(gate)
     _need(indices_locations.dtype == torch.int32 and indices_locations.dim() == 2 and
           indices_locations.shape[0] == 2 and indices_locations.shape[1] == gate.shape[0],
           "indices_locations must be int32 [2, k*S]")
@@ -313,7 +325,7 @@ def moe_decode(data, gate, indices_locations, top_k=1, out=None):
     S = gate.shape[0] // top_k
     if out is None:
         out = torch.empty((S, M), dtype=data.dtype, device=data.device)
-    st = lib.lancet_moe_decode(_p(data), _p(gate), _p(indices_locations), S, M, E, Cap, top_k, dt, _p(out),
+    st = lib.lancet_moe_decode(_p(data), _p(gate), _p(indices_locations), S, M, E, Cap, top_k, dt, gd, _p(out),
                                _stream())
     capi.check(st, "lancet_moe_decode")
     return out
@@ -342,25 +354,26 @@ def moe_encode_dx(dy, indices_locations, top_k=1, out=None):
 
 
 def moe_encode_dg(dy, indices_locations, n_experts, top_k=1, out=None):
-    """raf.op.moe_encode_dg(dy [k*S] f32, indices_locations, n_experts) -> [S, E] f32."""
+    """raf.op.moe_encode_dg(dy [k*S], indices_locations, n_experts) -> [S, E] of dy's dtype."""
     lib = capi.load()
     _dev(dy, "dy")
-    _need(dy.dim() == 1 and dy.dtype == torch.float32, "Input dy should be 1-D float32.")
+    _need(dy.dim() == 1, "Input dy should be 1-D.")
     S = _check_indloc(indices_locations, top_k)
     _need(dy.shape[0] == top_k * S, "dy and indices_locations disagree")
     if out is None:
-        out = torch.empty((S, n_experts), dtype=torch.float32, device=dy.device)
-    st = lib.lancet_moe_encode_dg(_p(dy), _p(indices_locations), S, n_experts, top_k, _p(out), _stream())
+        out = torch.empty((S, n_experts), dtype=dy.dtype, device=dy.device)
+    _need(out.dtype == dy.dtype, "the gate gradient takes dy's dtype")
+    st = lib.lancet_moe_encode_dg(_p(dy), _p(indices_locations), S, n_experts, top_k, _gate_code(dy, "dy"), _p(out), _stream())
     capi.check(st, "lancet_moe_encode_dg")
     return out
 
 
 def moe_decode_dx(dy, gate, indices_locations, n_experts, capacity, top_k=1, workspace=None, out=None):
-    """raf.op.moe_decode_dx(dy [S,M], gate [k*S] f32, indices_locations, n_experts, capacity) -> [E, C, M]."""
+    """raf.op.moe_decode_dx(dy [S,M], gate [k*S], indices_locations, n_experts, capacity) -> [E, C, M]."""
     lib = capi.load()
     _dev(dy, "dy"), _dev(gate, "gate")
     _need(dy.dim() == 2, "Input dy should be 2-D.")
-    _need(gate.dim() == 1 and gate.dtype == torch.float32, "gate must be 1-D float32")
+    _need(gate.dim() == 1, "gate must be 1-D")
     S = _check_indloc(indices_locations, top_k)
     _need(dy.shape[0] == S and gate.shape[0] == top_k * S, "dy, gate and indices_locations disagree")
     M = dy.shape[1]
@@ -369,13 +382,14 @@ def moe_decode_dx(dy, gate, indices_locations, n_experts, capacity, top_k=1, wor
     ws_bytes = int(lib.lancet_moe_decode_dx_workspace_bytes(n_experts, capacity))
     ws = _workspace(ws_bytes, dy.device, workspace)
     st = lib.lancet_moe_decode_dx(_p(dy), _p(gate), _p(indices_locations), S, M, n_experts, capacity, top_k,
-                                  _dtype_code(dy), _p(out), _p(ws), ws.numel(), _stream())
+                                  _dtype_code(dy), _gate_code(gate), _p(out), _p(ws), ws.numel(), _stream())
     capi.check(st, "lancet_moe_decode_dx")
     return out
 
 
-def moe_decode_dg(dy, data, indices_locations, top_k=1, out=None):
-    """raf.op.moe_decode_dg(dy [S,M], data [E,C,M], indices_locations) -> [k*S] f32."""
+def moe_decode_dg(dy, data, indices_locations, top_k=1, gate_dtype=torch.float32, out=None):
+    """raf.op.moe_decode_dg(dy [S,M], data [E,C,M], indices_locations) -> [k*S] of gate_dtype (the dtype of the
+    gates_s the gradient belongs to; the reference gives it dy's dtype, src/op/declare/moe.cc:239)."""
     lib = capi.load()
     _dev(dy, "dy"), _dev(data, "data")
     _need(dy.dim() == 2 and data.dim() == 3 and dy.dtype == data.dtype and dy.shape[1] == data.shape[2],
@@ -384,9 +398,9 @@ def moe_decode_dg(dy, data, indices_locations, top_k=1, out=None):
     _need(dy.shape[0] == S, "dy and indices_locations disagree")
     E, Cap, M = data.shape
     if out is None:
-        out = torch.empty(top_k * S, dtype=torch.float32, device=dy.device)
+        out = torch.empty(top_k * S, dtype=gate_dtype, device=dy.device)
     st = lib.lancet_moe_decode_dg(_p(dy), _p(data), _p(indices_locations), S, M, E, Cap, top_k, _dtype_code(dy),
-                                  _p(out), _stream())
+                                  _gate_code(out, "the gate gradient"), _p(out), _stream())
     capi.check(st, "lancet_moe_decode_dg")
     return out
 
@@ -397,7 +411,8 @@ def moe_top2_normalize_gates(raw_gates, merged_indices_locations):
     lib = capi.load()
     S = raw_gates.shape[0] // 2
     out = torch.empty_like(raw_gates)
-    st = lib.lancet_moe_top2_normalize_gates(_p(raw_gates), _p(merged_indices_locations), S, _p(out), _stream())
+    st = lib.lancet_moe_top2_normalize_gates(_p(raw_gates), _p(merged_indices_locations), S, _gate_code(raw_gates, "raw_gates"),
+                                             _p(out), _stream())
     capi.check(st, "lancet_moe_top2_normalize_gates")
     return out
 

@@ -32,6 +32,14 @@ int DTypeToLancet(const DType& dt) {
 }
 
 bool IsF32(const DType& dt) { return dt.code == DTypeCode::kFloat && dt.bits == 32; }
+// Gate arrays come in the type the graph has them in: fp32, or a half type under mixed precision
+// (python/raf/amp/type_hints.py:97,105; the reference's kernels take `__dtype* gates1_s`).
+int GateDTypeToLancet(const DType& dt) {
+  if (dt.code == DTypeCode::kFloat && dt.bits == 32) return LANCET_F32;
+  if (dt.code == DTypeCode::kFloat && dt.bits == 16) return LANCET_F16;
+  if (dt.code == DTypeCode::kBFloat && dt.bits == 16) return LANCET_BF16;
+  throw Error("gate values must be float32, float16 or bfloat16");
+}
 bool IsI32(const DType& dt) { return dt.code == DTypeCode::kInt && dt.bits == 32; }
 
 void CheckStatus(int status, const char* what) {
@@ -69,6 +77,19 @@ double OptFloat(const CallValues& cv, size_t i, double dflt) {
   return cv.args.size() > i && cv.args[i].kind != Value::kNone ? cv.args[i].AsFloat() : dflt;
 }
 
+// dtype of a gate gradient that no gate-typed input fixes, from an optional trailing integer argument
+// (the LANCET_* code: 0 float32, the default; 1 bfloat16; 2 float16)
+DType GateGradDType(const CallValues& cv, size_t i) {
+  DType dt;
+  switch (OptInt(cv, i, LANCET_F32)) {
+    case LANCET_F32: dt.code = DTypeCode::kFloat, dt.bits = 32; break;
+    case LANCET_BF16: dt.code = DTypeCode::kBFloat, dt.bits = 16; break;
+    case LANCET_F16: dt.code = DTypeCode::kFloat, dt.bits = 16; break;
+    default: throw Error("gate_dtype must be 0 (float32), 1 (bfloat16) or 2 (float16)");
+  }
+  return dt;
+}
+
 struct EncodeShape {
   int64_t S, M, E, C;
 };
@@ -78,7 +99,7 @@ EncodeShape CheckEncodeInputs(const Tensor& data, const Tensor& gate, int64_t n_
   RAF_CHECK(data.shape.size() == 2, "Input data should be 2-D.");
   RAF_CHECK(gate.shape.size() == 2, "Input gate should be 2-D.");
   RAF_CHECK(data.shape[0] == gate.shape[0], "Input data and gate should have matching shape in dim 0.");
-  RAF_CHECK(IsF32(gate.dtype), "gate must be float32 in the hip dialect");
+  GateDTypeToLancet(gate.dtype);
   DTypeToLancet(data.dtype);
   EncodeShape s;
   s.S = data.shape[0] / n_partitions;
@@ -89,10 +110,11 @@ EncodeShape CheckEncodeInputs(const Tensor& data, const Tensor& gate, int64_t n_
   return s;
 }
 
-// the 5-tuple of declare/moe.cc:48-58; gates_s is fp32, the buffer has the data dtype
-Value EncodeOutputs(const Tensor& data, const EncodeShape& s, int64_t k) {
+// the 5-tuple of declare/moe.cc:48-58; gates_s has the gate's dtype (what the reference's kernels write,
+// tutel_moe_dispatch.cu:110-116; its declaration says fp32 whatever the gate is), the buffer the data dtype
+Value EncodeOutputs(const Tensor& data, const Tensor& gate, const EncodeShape& s, int64_t k) {
   std::vector<Value> ret;
-  ret.push_back(Value::MakeTensor(MakeOut(data.device_id, DTypeCode::kFloat, 32, {k * s.S})));
+  ret.push_back(Value::MakeTensor(MakeOut(data.device_id, gate.dtype.code, gate.dtype.bits, {k * s.S})));
   ret.push_back(Value::MakeTensor(MakeOut(data.device_id, DTypeCode::kInt, 32, {2, k * s.S})));
   ret.push_back(Value::MakeTensor(MakeOut(data.device_id, DTypeCode::kInt, 32, {s.E})));
   ret.push_back(Value::MakeTensor(MakeOut(data.device_id, DTypeCode::kUInt, 64, {s.E})));
@@ -117,7 +139,7 @@ void MoeEncodeDeclare(CallValues& call) {
   const float cf = static_cast<float>(OptFloat(call, 3, 1.0)) * (k == 2 ? 2.0f : 1.0f);
   const EncodeShape s = CheckEncodeInputs(data, gate, 1, cf);
   RAF_CHECK(used.shape[0] == s.E && IsI32(used.dtype), "used_capacity must be int32 [E]");
-  call.out = EncodeOutputs(data, s, k);
+  call.out = EncodeOutputs(data, gate, s, k);
   call.device_id = data.device_id;
 }
 
@@ -130,6 +152,7 @@ class MoeEncode : public OpEnv {
     shape_ = CheckEncodeInputs(data, cv.args[1].AsTensor(), 1, cf);
     flags_ = (OptInt(cv, 5, 0) ? LANCET_GATE_IS_LOGITS : 0u) | (OptInt(cv, 6, 1) ? 0u : LANCET_NO_TAIL_ZERO);
     dtype_ = DTypeToLancet(data.dtype);
+    gate_dtype_ = GateDTypeToLancet(cv.args[1].AsTensor().dtype);
     device_id_ = data.device_id;
     RAF_CHECK(cv.out.kind == Value::kTuple && cv.out.fields.size() == 5, "Expected output to be a 5-Tuple");
     ws_bytes_ = lancet_moe_encode_workspace_bytes(shape_.S, shape_.E, top_k_);
@@ -140,8 +163,8 @@ class MoeEncode : public OpEnv {
     if (has_noise_) {
       const Tensor& noise = cv.args[7].AsTensor();
       RAF_CHECK(top_k_ == 2, "gate2_noise only exists for the second choice (top_k = 2)");
-      RAF_CHECK(noise.shape == cv.args[1].AsTensor().shape && noise.dtype.code == DTypeCode::kFloat && noise.dtype.bits == 32,
-                "gate2_noise must be float32 [S, E]");
+      RAF_CHECK(noise.shape == cv.args[1].AsTensor().shape && noise.dtype == cv.args[1].AsTensor().dtype,
+                "gate2_noise must have the gate's shape and dtype");
       this->arg_indices.push_back(7);
     }
   }
@@ -156,13 +179,13 @@ class MoeEncode : public OpEnv {
     const Tensor& data = inputs[0].AsTensor();
     const Tensor& gate = inputs[1].AsTensor();
     const Tensor& used = inputs[2].AsTensor();
-    const float* noise = has_noise_ ? static_cast<const float*>(inputs[3].AsTensor().data) : nullptr;
+    const void* noise = has_noise_ ? inputs[3].AsTensor().data : nullptr;
     const auto& out = output.AsTuple();
     RAF_CHECK(out.size() == 5, "Expected output to be a 5-Tuple");
     scan_ws_.Ensure(ws_, ws_bytes_, GetStream(device_id_));
-    CheckStatus(lancet_moe_encode(data.data, static_cast<const float*>(gate.data), noise,
+    CheckStatus(lancet_moe_encode(data.data, gate.data, noise,
                                   static_cast<const int32_t*>(used.data), shape_.S, shape_.M, shape_.E, shape_.C,
-                                  top_k_, dtype_, flags_, static_cast<float*>(out[0].AsTensor().data),
+                                  top_k_, dtype_, gate_dtype_, flags_, out[0].AsTensor().data,
                                   static_cast<int32_t*>(out[1].AsTensor().data),
                                   static_cast<int32_t*>(out[2].AsTensor().data),
                                   static_cast<uint64_t*>(out[3].AsTensor().data), out[4].AsTensor().data, ws_,
@@ -176,7 +199,7 @@ class MoeEncode : public OpEnv {
 
  private:
   EncodeShape shape_;
-  int top_k_, dtype_, device_id_;
+  int top_k_, dtype_, gate_dtype_, device_id_;
   unsigned flags_;
   bool has_noise_ = false;
   void* ws_ = nullptr;
@@ -195,7 +218,7 @@ void MoeEncodeBatchPrioritizedDeclare(CallValues& call) {
   RAF_CHECK(pid >= 0 && pid < n_part, "partition_id should be less than n_partitions.");
   const EncodeShape s = CheckEncodeInputs(data, call.args[1].AsTensor(), n_part,
                                           static_cast<float>(OptFloat(call, 4, 1.0)));
-  call.out = EncodeOutputs(data, s, 1);
+  call.out = EncodeOutputs(data, call.args[1].AsTensor(), s, 1);
   call.device_id = data.device_id;
 }
 
@@ -210,6 +233,7 @@ class MoeEncodeBatchPrioritized : public OpEnv {
     orig_S_ = data.shape[0];
     flags_ = (OptInt(cv, 5, 0) ? LANCET_GATE_IS_LOGITS : 0u) | (OptInt(cv, 6, 1) ? 0u : LANCET_NO_TAIL_ZERO);
     dtype_ = DTypeToLancet(data.dtype);
+    gate_dtype_ = GateDTypeToLancet(cv.args[1].AsTensor().dtype);
     device_id_ = data.device_id;
     // sorted indices, dropping mask, indices and gate buffers of the reference (cuda/moe.cc:512-520)
     // are replaced by one workspace for the radix select and the scan
@@ -224,9 +248,9 @@ class MoeEncodeBatchPrioritized : public OpEnv {
     const auto& out = output.AsTuple();
     RAF_CHECK(out.size() == 5, "Expected output to be a 5-Tuple");
     scan_ws_.Ensure(ws_, ws_bytes_, GetStream(device_id_));
-    CheckStatus(lancet_moe_encode_bpr(inputs[0].AsTensor().data, static_cast<const float*>(inputs[1].AsTensor().data),
+    CheckStatus(lancet_moe_encode_bpr(inputs[0].AsTensor().data, inputs[1].AsTensor().data,
                                       orig_S_, shape_.M, shape_.E, shape_.C, n_partitions_, partition_id_, dtype_,
-                                      flags_, static_cast<float*>(out[0].AsTensor().data),
+                                      gate_dtype_, flags_, out[0].AsTensor().data,
                                       static_cast<int32_t*>(out[1].AsTensor().data),
                                       static_cast<int32_t*>(out[2].AsTensor().data),
                                       static_cast<uint64_t*>(out[3].AsTensor().data), out[4].AsTensor().data, ws_,
@@ -241,7 +265,7 @@ class MoeEncodeBatchPrioritized : public OpEnv {
  private:
   EncodeShape shape_;
   int64_t orig_S_;
-  int n_partitions_, partition_id_, dtype_, device_id_;
+  int n_partitions_, partition_id_, dtype_, gate_dtype_, device_id_;
   unsigned flags_;
   void* ws_ = nullptr;
   size_t ws_bytes_ = 0;
@@ -397,7 +421,7 @@ class MoeDecode : public OpEnv {
     const Tensor& gate = cv.args[1].AsTensor();
     RAF_CHECK(data.shape.size() == 3, "Expected input data to be 3D.");
     RAF_CHECK(gate.shape.size() == 1, "Expected input gate to be 1D.");
-    RAF_CHECK(IsF32(gate.dtype), "gate must be float32 in the hip dialect");
+    gate_dtype_ = GateDTypeToLancet(gate.dtype);
     top_k_ = static_cast<int>(OptInt(cv, 3, 1));
     dim_S_ = gate.shape[0] / top_k_;
     dim_E_ = data.shape[0], dim_C_ = data.shape[1], dim_M_ = data.shape[2];
@@ -411,9 +435,9 @@ class MoeDecode : public OpEnv {
   void Execute(const std::vector<Value>& inputs, Value output) override {
     const Tensor& il = inputs[2].AsTensor();
     RAF_CHECK(IsI32(il.dtype) && il.shape.size() == 2 && il.shape[1] == dim_S_ * top_k_, "indices_locations must be int32 [2, k*S]");
-    CheckStatus(lancet_moe_decode(inputs[0].AsTensor().data, static_cast<const float*>(inputs[1].AsTensor().data),
+    CheckStatus(lancet_moe_decode(inputs[0].AsTensor().data, inputs[1].AsTensor().data,
                                   static_cast<const int32_t*>(il.data), dim_S_, dim_M_, dim_E_, dim_C_, top_k_,
-                                  dtype_, output.AsTensor().data, GetStream(device_id_)),
+                                  dtype_, gate_dtype_, output.AsTensor().data, GetStream(device_id_)),
                 "lancet_moe_decode");
   }
 
@@ -422,7 +446,7 @@ class MoeDecode : public OpEnv {
 
  private:
   int64_t dim_S_, dim_E_, dim_C_, dim_M_;
-  int top_k_, dtype_, device_id_;
+  int top_k_, dtype_, gate_dtype_, device_id_;
 };
 
 // =====================================================================================
@@ -563,9 +587,9 @@ void MoeEncodeDgDeclare(CallValues& call) {
   RAF_CHECK(call.args.size() >= 3, "moe_encode_dg(dy, indices_locations, n_experts)");
   const Tensor& dy = call.args[0].AsTensor();
   RAF_CHECK(dy.shape.size() == 1, "Input dy should be 1-D.");
-  RAF_CHECK(IsF32(dy.dtype), "dy of moe_encode_dg must be float32 in the hip dialect");
+  GateDTypeToLancet(dy.dtype);
   const int64_t S = MaskTokens(call.args[1].AsTensor(), OptInt(call, 3, 1));
-  call.out = Value::MakeTensor(MakeOut(dy.device_id, DTypeCode::kFloat, 32, {S, call.args[2].AsInt()}));
+  call.out = Value::MakeTensor(MakeOut(dy.device_id, dy.dtype.code, dy.dtype.bits, {S, call.args[2].AsInt()}));  // declare/moe.cc:194
   call.device_id = dy.device_id;
 }
 
@@ -573,7 +597,8 @@ class MoeEncodeDg : public OpEnv {
  public:
   explicit MoeEncodeDg(const CallValues& cv) {
     const Tensor& dy = cv.args[0].AsTensor();
-    RAF_CHECK(dy.shape.size() == 1 && IsF32(dy.dtype), "Expected input dy to be 1D float32.");
+    RAF_CHECK(dy.shape.size() == 1, "Expected input dy to be 1D.");
+    gate_dtype_ = GateDTypeToLancet(dy.dtype);
     top_k_ = static_cast<int>(OptInt(cv, 3, 1));
     dim_S_ = MaskTokens(cv.args[1].AsTensor(), top_k_);
     RAF_CHECK(dy.shape[0] == dim_S_ * top_k_, "dy and indices_locations disagree");
@@ -583,9 +608,9 @@ class MoeEncodeDg : public OpEnv {
   }
   void Execute(const CallValues& cv) override { Execute({cv.args[0], cv.args[1]}, cv.out); }
   void Execute(const std::vector<Value>& inputs, Value output) override {
-    CheckStatus(lancet_moe_encode_dg(static_cast<const float*>(inputs[0].AsTensor().data),
+    CheckStatus(lancet_moe_encode_dg(inputs[0].AsTensor().data,
                                      static_cast<const int32_t*>(inputs[1].AsTensor().data), dim_S_, dim_E_, top_k_,
-                                     static_cast<float*>(output.AsTensor().data), GetStream(device_id_)),
+                                     gate_dtype_, output.AsTensor().data, GetStream(device_id_)),
                 "lancet_moe_encode_dg");
   }
   std::string name() const override { return "raf.op.hip.moe_encode_dg"; }
@@ -593,7 +618,7 @@ class MoeEncodeDg : public OpEnv {
 
  private:
   int64_t dim_S_, dim_E_;
-  int top_k_, device_id_;
+  int top_k_, gate_dtype_, device_id_;
 };
 
 void MoeDecodeDxDeclare(CallValues& call) {
@@ -612,7 +637,8 @@ class MoeDecodeDx : public OpEnv {
     const Tensor& dy = cv.args[0].AsTensor();
     const Tensor& gate = cv.args[1].AsTensor();
     RAF_CHECK(dy.shape.size() == 2, "Expected input dy to be 2D.");
-    RAF_CHECK(gate.shape.size() == 1 && IsF32(gate.dtype), "Expected input gate to be 1D float32.");
+    RAF_CHECK(gate.shape.size() == 1, "Expected input gate to be 1D.");
+    gate_dtype_ = GateDTypeToLancet(gate.dtype);
     top_k_ = static_cast<int>(OptInt(cv, 5, 1));
     dim_S_ = MaskTokens(cv.args[2].AsTensor(), top_k_);
     RAF_CHECK(dy.shape[0] == dim_S_ && gate.shape[0] == dim_S_ * top_k_, "dy, gate and indices_locations disagree");
@@ -627,9 +653,9 @@ class MoeDecodeDx : public OpEnv {
   }
   void Execute(const CallValues& cv) override { Execute({cv.args[0], cv.args[1], cv.args[2]}, cv.out); }
   void Execute(const std::vector<Value>& inputs, Value output) override {
-    CheckStatus(lancet_moe_decode_dx(inputs[0].AsTensor().data, static_cast<const float*>(inputs[1].AsTensor().data),
+    CheckStatus(lancet_moe_decode_dx(inputs[0].AsTensor().data, inputs[1].AsTensor().data,
                                      static_cast<const int32_t*>(inputs[2].AsTensor().data), dim_S_, dim_M_, dim_E_,
-                                     dim_C_, top_k_, dtype_, output.AsTensor().data, ws_, ws_bytes_,
+                                     dim_C_, top_k_, dtype_, gate_dtype_, output.AsTensor().data, ws_, ws_bytes_,
                                      GetStream(device_id_)),
                 "lancet_moe_decode_dx");
   }
@@ -638,7 +664,7 @@ class MoeDecodeDx : public OpEnv {
 
  private:
   int64_t dim_S_, dim_E_, dim_C_, dim_M_;
-  int top_k_, dtype_, device_id_;
+  int top_k_, dtype_, gate_dtype_, device_id_;
   void* ws_ = nullptr;
   size_t ws_bytes_ = 0;
 };
@@ -650,7 +676,10 @@ void MoeDecodeDgDeclare(CallValues& call) {
   DTypeToLancet(dy.dtype);
   const int64_t k = OptInt(call, 3, 1);
   const int64_t S = MaskTokens(call.args[2].AsTensor(), k);
-  call.out = Value::MakeTensor(MakeOut(dy.device_id, DTypeCode::kFloat, 32, {k * S}));
+  // the gradient of gates_s has the gate's dtype: fp32 by default, or what the trailing gate_dtype argument
+  // names (a mixed-precision graph passes the half type; the reference gives it dy's dtype, declare/moe.cc:239)
+  const DType gd = GateGradDType(call, 4);
+  call.out = Value::MakeTensor(MakeOut(dy.device_id, gd.code, gd.bits, {k * S}));
   call.device_id = dy.device_id;
 }
 
@@ -667,6 +696,7 @@ class MoeDecodeDg : public OpEnv {
     RAF_CHECK(dy.shape[0] == dim_S_, "dy and indices_locations disagree");
     dim_E_ = data.shape[0], dim_C_ = data.shape[1], dim_M_ = data.shape[2];
     dtype_ = DTypeToLancet(dy.dtype);
+    gate_dtype_ = GateDTypeToLancet(GateGradDType(cv, 4));
     device_id_ = dy.device_id;
     this->arg_indices = {0, 1, 2};
   }
@@ -674,7 +704,7 @@ class MoeDecodeDg : public OpEnv {
   void Execute(const std::vector<Value>& inputs, Value output) override {
     CheckStatus(lancet_moe_decode_dg(inputs[0].AsTensor().data, inputs[1].AsTensor().data,
                                      static_cast<const int32_t*>(inputs[2].AsTensor().data), dim_S_, dim_M_, dim_E_,
-                                     dim_C_, top_k_, dtype_, static_cast<float*>(output.AsTensor().data),
+                                     dim_C_, top_k_, dtype_, gate_dtype_, output.AsTensor().data,
                                      GetStream(device_id_)),
                 "lancet_moe_decode_dg");
   }
@@ -683,7 +713,7 @@ class MoeDecodeDg : public OpEnv {
 
  private:
   int64_t dim_S_, dim_E_, dim_C_, dim_M_;
-  int top_k_, dtype_, device_id_;
+  int top_k_, dtype_, gate_dtype_, device_id_;
 };
 
 // ---- registration (cuda/cuda_utils.cc:17; cuda/moe.cc:411-412,728-729,822-823,942-943,1310-1311) ----

@@ -281,19 +281,24 @@ def moe_decode(expert_out, gates_s, indloc, k=1, round_fn=None):
 # A.6: top-2 extension (docker/resources/sharded_moe.py:253-324, no Gumbel noise)
 # --------------------------------------------------------------------------
 def moe_encode_top2(data, gate, used_in, capacity_factor=1.0, gate_is_logits=False,
-                    C=None, fast_scatter=False, gate2_noise=None):
+                    C=None, fast_scatter=False, gate2_noise=None, gate_round=None):
     """GShard top-2 expressed as two chained reference top-1 encodes, merged:
     slot 1 with used_in, slot 2 with used_out(slot 1); merged layout is what
     moe_merge_masks/moe_redispatch give for the two calls.  Capacity follows the
     reference formula with capacity_factor' = 2*capacity_factor
     (sharded_moe.py:267).  Combine weights are taken after the drop and
-    normalised by max(g1+g2, eps) (:296-312)."""
+    normalised by max(g1+g2, eps) (:296-312).  gate_round (a 16-bit gate array: the
+    function that rounds fp32 to its type, result as fp32): the two raw gate values
+    are what a gates_s array of that type holds, i.e. rounded, before the fp32
+    normalisation; rounding the returned weights to the type is the caller's."""
     data = np.asarray(data)
     S, M = data.shape
     E = gate.shape[1]
     if C is None:
         C = capacity(S, E, 2.0 * capacity_factor)
     sel, val = select_topk(gate, 2, gate_is_logits, gate2_noise)
+    if gate_round is not None:
+        val = gate_round(val).astype(np.float32)
     used_in = np.asarray(used_in, dtype=np.int32)
     i1, l1, used1, _ = gen_location(sel[0], used_in, C, M, E)
     i2, l2, used2, _ = gen_location(sel[1], used1, C, M, E)
@@ -336,6 +341,11 @@ def bf16_bits_to_f32(b):
 def round_to_bf16(a):
     """fp32 -> nearest bf16 value, returned as fp32."""
     return bf16_bits_to_f32(f32_to_bf16_bits(a))
+
+
+def round_to_f16(a):
+    """fp32 -> nearest fp16 value (round to nearest even), returned as fp32."""
+    return np.asarray(a, dtype=np.float32).astype(np.float16).astype(np.float32)
 
 
 # --------------------------------------------------------------------------

@@ -58,9 +58,9 @@ int main(void) {
   CHECK_HIP(hipMemset(d_disp, 0xff, E * 2 * M * sizeof(float))); /* stale contents must not survive */
   CHECK_LANCET(lancet_scan_workspace_init(d_ws, ws_bytes, stream)); /* once per workspace */
 
-  CHECK_LANCET(lancet_moe_encode(d_data, d_gate, NULL, NULL, S, M, E, C, 1, LANCET_F32, 0u, d_gates_s, d_il, d_used,
+  CHECK_LANCET(lancet_moe_encode(d_data, d_gate, NULL, NULL, S, M, E, C, 1, LANCET_F32, LANCET_F32, 0u, d_gates_s, d_il, d_used,
                                  d_elems, d_disp, d_ws, ws_bytes, stream));
-  CHECK_LANCET(lancet_moe_decode(d_disp, d_gates_s, d_il, S, M, E, C, 1, LANCET_F32, d_out, stream));
+  CHECK_LANCET(lancet_moe_decode(d_disp, d_gates_s, d_il, S, M, E, C, 1, LANCET_F32, LANCET_F32, d_out, stream));
   CHECK_HIP(hipStreamSynchronize(stream));
 
   float gates_s[S], disp[E * 2 * M], out[S * M];
@@ -91,10 +91,10 @@ int main(void) {
   bad += memcmp(out, want_out, sizeof(out)) != 0;
 
   /* a rejected call launches nothing and says why */
-  if (lancet_moe_encode(d_data, d_gate, NULL, NULL, S, M, E, C, 3, LANCET_F32, 0u, d_gates_s, d_il, d_used, d_elems,
+  if (lancet_moe_encode(d_data, d_gate, NULL, NULL, S, M, E, C, 3, LANCET_F32, LANCET_F32, 0u, d_gates_s, d_il, d_used, d_elems,
                         d_disp, d_ws, ws_bytes, stream) != LANCET_ERR_TOPK)
     ++bad;
-  if (lancet_moe_decode(d_disp, d_gates_s, d_il, S, M, E, C, 1, 99, d_out, stream) != LANCET_ERR_DTYPE) ++bad;
+  if (lancet_moe_decode(d_disp, d_gates_s, d_il, S, M, E, C, 1, 99, LANCET_F32, d_out, stream) != LANCET_ERR_DTYPE) ++bad;
 
   hipFree(d_gate), hipFree(d_data), hipFree(d_gates_s), hipFree(d_il), hipFree(d_used);
   hipFree(d_elems), hipFree(d_disp), hipFree(d_out), hipFree(d_ws);

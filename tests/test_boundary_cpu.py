@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol(pkg):
     for n in names + hooks:
         assert hasattr(lib, n), "liblancet_hip.so does not export %s" % n
     assert sorted(pkg.capi.SIGNATURES) == sorted(names + hooks), "capi.SIGNATURES and the headers disagree"
-    assert lib.lancet_abi_version() == pkg.capi.ABI_VERSION == 5
+    assert lib.lancet_abi_version() == pkg.capi.ABI_VERSION == 6
     # test and measurement hooks live in their own header; the operator surface declares none
     assert not [n for n in names if "debug" in n] and all("debug" in n for n in hooks)
 
@@ -42,25 +42,35 @@ def test_workspace_sizes_and_argument_rejection(pkg):
     assert lib.lancet_moe_encode_workspace_bytes(0, 4, 1) == 32 + 1 * 4 * 8
     assert lib.lancet_moe_encode_workspace_bytes(10, 0, 1) == 0
     one = C.c_void_p(16)  # never dereferenced: every call below is rejected before any launch
-    st = lib.lancet_moe_encode(one, one, None, None, 8, 4, 2, 4, 1, 99, 0, one, one, one, one, one, one, 1 << 20, None)
+    st = lib.lancet_moe_encode(one, one, None, None, 8, 4, 2, 4, 1, 99, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
     assert st == capi.ERR_DTYPE
-    st = lib.lancet_moe_encode(one, one, None, None, 8, 4, 2, 4, 3, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
+    st = lib.lancet_moe_encode(one, one, None, None, 8, 4, 2, 4, 1, capi.F32, 7, 0, one, one, one, one, one, one, 1 << 20, None)
+    assert st == capi.ERR_DTYPE                     # gate dtype
+    st = lib.lancet_moe_encode(one, C.c_void_p(18), None, None, 8, 4, 2, 4, 1, capi.F32, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
+    assert st == capi.ERR_ALIGN                     # an fp32 gate at a 2-byte address ...
+    st = lib.lancet_moe_encode(one, C.c_void_p(18), None, None, 8, 4, 2, 4, 3, capi.F32, capi.BF16, 0, one, one, one, one, one, one, 1 << 20, None)
+    assert st == capi.ERR_TOPK                      # ... which a 16-bit gate may have (the next check rejects top_k)
+    assert lib.lancet_moe_decode(one, one, one, 8, 4, 2, 4, 1, capi.F32, 9, one, None) == capi.ERR_DTYPE
+    assert lib.lancet_moe_decode_dg(one, one, one, 8, 4, 2, 4, 1, capi.F32, 9, one, None) == capi.ERR_DTYPE
+    assert lib.lancet_moe_encode_dg(one, one, 8, 2, 1, 9, one, None) == capi.ERR_DTYPE
+    assert lib.lancet_gate_topk(one, None, 8, 2, 1, 9, 0, one, one, None) == capi.ERR_DTYPE
+    st = lib.lancet_moe_encode(one, one, None, None, 8, 4, 2, 4, 3, capi.F32, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
     assert st == capi.ERR_TOPK
-    st = lib.lancet_moe_encode(one, one, None, None, 8, 4, 1, 4, 2, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
+    st = lib.lancet_moe_encode(one, one, None, None, 8, 4, 1, 4, 2, capi.F32, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
     assert st == capi.ERR_TOPK                      # top-2 needs two experts
-    st = lib.lancet_moe_encode(one, one, None, None, 8, 4, 2, 4, 1, capi.F32, 0, one, one, one, one, one, one, 8, None)
+    st = lib.lancet_moe_encode(one, one, None, None, 8, 4, 2, 4, 1, capi.F32, capi.F32, 0, one, one, one, one, one, one, 8, None)
     assert st == capi.ERR_WORKSPACE
-    st = lib.lancet_moe_encode(one, one, None, None, 8, 4, 2, 4, 1, capi.F32, 0, one, None, one, one, one, one, 1 << 20, None)
+    st = lib.lancet_moe_encode(one, one, None, None, 8, 4, 2, 4, 1, capi.F32, capi.F32, 0, one, None, one, one, one, one, 1 << 20, None)
     assert st == capi.ERR_NULL
-    st = lib.lancet_moe_encode(one, one, None, None, -1, 4, 2, 4, 1, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
+    st = lib.lancet_moe_encode(one, one, None, None, -1, 4, 2, 4, 1, capi.F32, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
     assert st == capi.ERR_SHAPE
-    st = lib.lancet_moe_encode(one, one, None, None, 8, 4, 1000, 4, 1, capi.F32, 0, one, one, one, one, one, one, 1 << 30, None)
+    st = lib.lancet_moe_encode(one, one, None, None, 8, 4, 1000, 4, 1, capi.F32, capi.F32, 0, one, one, one, one, one, one, 1 << 30, None)
     assert st == capi.ERR_SHAPE                     # more experts than LANCET_MAX_EXPERTS
-    st = lib.lancet_moe_encode(C.c_void_p(18), one, None, None, 8, 4, 2, 4, 1, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
+    st = lib.lancet_moe_encode(C.c_void_p(18), one, None, None, 8, 4, 2, 4, 1, capi.F32, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
     assert st == capi.ERR_ALIGN
-    st = lib.lancet_moe_encode(one, one, one, None, 8, 4, 2, 4, 1, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
+    st = lib.lancet_moe_encode(one, one, one, None, 8, 4, 2, 4, 1, capi.F32, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
     assert st == capi.ERR_TOPK                      # noise for a second choice that does not exist
-    st = lib.lancet_moe_encode_bpr(one, one, 8, 4, 2, 4, 2, 2, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
+    st = lib.lancet_moe_encode_bpr(one, one, 8, 4, 2, 4, 2, 2, capi.F32, capi.F32, 0, one, one, one, one, one, one, 1 << 20, None)
     assert st == capi.ERR_PARTITION
     ptrs = capi.ptr_array([16] * 70)
     assert lib.lancet_moe_merge_masks(ptrs, 70, 8, 2, one, one, 1 << 20, None) == capi.ERR_PARTITION
@@ -78,9 +88,9 @@ def test_workspace_sizes_and_argument_rejection(pkg):
     assert sc(one, one, None, None, 64, 0, 8, 4, 2, 4, 1, capi.F32, 0, one, None) == capi.ERR_NULL   # tail fill needs used_out
     assert sc(one, one, None, one, 64, 0, 8, 4, 2, 4, 3, capi.F32, 0, one, None) == capi.ERR_TOPK
     assert sc(one, one, None, one, 64, 0, 8, 4, 2, 4, 1, 7, 0, one, None) == capi.ERR_DTYPE
-    assert dc(one, one, one, 64, 57, 8, 4, 2, 4, 1, capi.F32, one, None) == capi.ERR_SHAPE
-    assert dc(one, None, one, 64, 0, 8, 4, 2, 4, 1, capi.F32, one, None) == capi.ERR_NULL
-    assert dc(one, one, one, 64, 0, 8, 4, 2, 4, 1, capi.F32, C.c_void_p(6), None) == capi.ERR_ALIGN
+    assert dc(one, one, one, 64, 57, 8, 4, 2, 4, 1, capi.F32, capi.F32, one, None) == capi.ERR_SHAPE
+    assert dc(one, None, one, 64, 0, 8, 4, 2, 4, 1, capi.F32, capi.F32, one, None) == capi.ERR_NULL
+    assert dc(one, one, one, 64, 0, 8, 4, 2, 4, 1, capi.F32, capi.F32, C.c_void_p(6), None) == capi.ERR_ALIGN
     # row ranges of token partitions
     pr = lib.lancet_moe_partition_ranges
     assert lib.lancet_moe_partition_ranges_workspace_bytes(2, 4, 8) == 2 * 4 * 8 * 4

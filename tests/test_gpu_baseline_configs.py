@@ -121,7 +121,7 @@ def test_config4_lancet_forward_pipeline_bf16(pkg):
     import ctypes as C
     sel = torch.empty((2, S0), dtype=torch.int32, device="cuda")
     val = torch.empty((2, S0), dtype=torch.float32, device="cuda")
-    assert lib.lancet_gate_topk(C.c_void_p(logits.data_ptr()), None, S0, E, 2, pkg.capi.GATE_IS_LOGITS,
+    assert lib.lancet_gate_topk(C.c_void_p(logits.data_ptr()), None, S0, E, 2, pkg.capi.F32, pkg.capi.GATE_IS_LOGITS,
                                 C.c_void_p(sel.data_ptr()), C.c_void_p(val.data_ptr()), None) == 0
     used = torch.zeros(E, dtype=torch.int32, device="cuda")
     ils, bufs, raws = [], [], []

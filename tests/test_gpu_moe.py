@@ -403,7 +403,7 @@ def test_scan_on_a_workspace_that_is_not_set_up(pkg):
             outs = (torch.zeros(k * S, device="cuda"), torch.zeros((2, k * S), dtype=torch.int32, device="cuda"),
                     torch.zeros(E, dtype=torch.int32, device="cuda"), torch.zeros(E, dtype=torch.int64, device="cuda"),
                     torch.zeros((E, Cap, M), device="cuda"))
-            st = lib.lancet_moe_encode(p(d_data), p(d_gate), None, None, S, M, E, Cap, k, capi.F32, capi.GATE_IS_LOGITS,
+            st = lib.lancet_moe_encode(p(d_data), p(d_gate), None, None, S, M, E, Cap, k, capi.F32, capi.F32, capi.GATE_IS_LOGITS,
                                        *[p(t) for t in outs], p(ws), nws, None)
             assert st == 0
             torch.cuda.synchronize()
@@ -412,7 +412,7 @@ def test_scan_on_a_workspace_that_is_not_set_up(pkg):
             err = C.c_int(0)
             assert lib.lancet_scan_workspace_error(p(ws), None, C.byref(err)) == 0 and err.value == 1
             assert lib.lancet_scan_workspace_init(p(ws), nws, None) == 0
-            st = lib.lancet_moe_encode(p(d_data), p(d_gate), None, None, S, M, E, Cap, k, capi.F32, capi.GATE_IS_LOGITS,
+            st = lib.lancet_moe_encode(p(d_data), p(d_gate), None, None, S, M, E, Cap, k, capi.F32, capi.F32, capi.GATE_IS_LOGITS,
                                        *[p(t) for t in outs], p(ws), nws, None)
             assert st == 0
             enc = mo.moe_encode_top2 if k == 2 else mo.moe_encode

@@ -36,13 +36,13 @@ def _encode_both(pkg, lib, data, gate, used_in, cf, k, flags):
     ws_bytes = lib.lancet_moe_encode_workspace_bytes(S, E, k)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
     assert lib.lancet_scan_workspace_init(_p(ws), ws_bytes, st) == 0
-    rc = lib.lancet_moe_encode(_p(data), _p(gate), None, _p(used_in), S, M, E, Cap, k, dt, flags, *[_p(t) for t in ref],
+    rc = lib.lancet_moe_encode(_p(data), _p(gate), None, _p(used_in), S, M, E, Cap, k, dt, capi.F32, flags, *[_p(t) for t in ref],
                                _p(ws), ws_bytes, st)
     assert rc == 0, capi.status_string(rc)
     got = _outputs(S, M, E, Cap, k, data.dtype)
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
-    rc = lib.lancet_moe_encode_noalloc(_p(data), _p(gate), None, _p(used_in), S, M, E, Cap, k, dt, flags,
+    rc = lib.lancet_moe_encode_noalloc(_p(data), _p(gate), None, _p(used_in), S, M, E, Cap, k, dt, capi.F32, flags,
                                        *[_p(t) for t in got], st)
     assert rc == 0, capi.status_string(rc)
     torch.cuda.synchronize()
@@ -83,7 +83,7 @@ def test_noalloc_encode_rejects_sizes_beyond_its_scratch(pkg, lib):
     S, E, k = 1 << 20, 512, 2          # 4096 tiles x 1024 counters x 4 B = 16 MiB of descriptors
     assert lib.lancet_moe_encode_workspace_bytes(S, E, k) > capi.NOALLOC_SCRATCH_BYTES
     one = torch.zeros(1, device="cuda")
-    rc = lib.lancet_moe_encode_noalloc(_p(one), _p(one), None, None, S, 4, E, 8, k, capi.F32, 0, _p(one), _p(one), _p(one),
+    rc = lib.lancet_moe_encode_noalloc(_p(one), _p(one), None, None, S, 4, E, 8, k, capi.F32, capi.F32, 0, _p(one), _p(one), _p(one),
                                        _p(one), _p(one), None)
     assert rc == capi.ERR_SCRATCH
     assert "scratch" in capi.status_string(rc)

@@ -188,39 +188,64 @@ def profile_figure(key):
         return None
 
 
-def cpu_baseline(S, M, E, cf, budget_s=12.0):
-    """The CPU restatement of the reference's algorithm (oracle/c/lancet_oracle.c, OpenMP over the
-    host cores this process may use) timed on the headline workload itself: whole top-2
-    encode + decode passes over S tokens, repeated until the time budget is used (at least 2
-    passes).  The NumPy restatement (the style of the reference's test references, one core) is
-    timed on a 2048-token slice and quoted in `sample`."""
+def headline_inputs(S, M, E):
+    """The headline's host arrays: NumPy default_rng(0), generation order data then logits, both N(0,1) fp32; the token
+    rows rounded to bf16 (nearest even).  The same arrays are uploaded for the GPU legs and timed by the CPU baseline."""
+    import numpy as np
+    from oracle import moe_oracle as mo
+    rng = np.random.default_rng(0)
+    data_bits = mo.f32_to_bf16_bits(rng.standard_normal((S, M), dtype=np.float32))
+    logits = rng.standard_normal((S, E), dtype=np.float32)
+    return data_bits, logits
+
+
+def cpu_baseline(data_bits, logits, cf, budget_s=10.0):
+    """The CPU restatement of the reference's algorithm timed on the host cores of this box, on the arrays the GPU
+    legs ran on: whole top-2 encode + decode passes of the C restatement (oracle/c/lancet_oracle.c) with all the
+    cores this process may use (repeated until the time budget is used, at least 2 passes, median) and with one
+    thread (2 passes); and the NumPy restatement in the style of the reference's own test references (one-hot +
+    cumsum locations, Python scatter loop; one core) on BASELINE config 1, the case the reference's CPU path runs."""
     import numpy as np
     from oracle import c_oracle, moe_oracle as mo
+    S, M = data_bits.shape
+    E = logits.shape[1]
     cores = len(os.sched_getaffinity(0))
-    c_oracle.set_num_threads(cores)
-    rng = np.random.default_rng(0)
-    data = mo.f32_to_bf16_bits(rng.standard_normal((S, M), dtype=np.float32))
-    logits = rng.standard_normal((S, E), dtype=np.float32)
     Cap = mo.capacity(S, E, 2 * cf)
+
+    def c_passes(threads, budget, most):
+        c_oracle.set_num_threads(threads)
+        times = []
+        t_all = time.perf_counter()
+        while len(times) < 2 or (time.perf_counter() - t_all < budget and len(times) < most):
+            t0 = time.perf_counter()
+            g, il, _, _, disp = c_oracle.moe_encode(data_bits, logits, None, Cap, 2, True)
+            out = c_oracle.moe_decode(disp, g, il, 2)
+            times.append(time.perf_counter() - t0)
+            del out, disp
+        return sorted(times)[len(times) // 2], len(times)
+
+    t_all, n_all = c_passes(cores, budget_s, 50)
+    t_one, n_one = c_passes(1, 0.0, 2)
+    c_oracle.set_num_threads(cores)
+    # config 1: S=4096, M=768 fp32, E=8, top-1, cf 1.25 (C=640), seed 0, data then logits
+    rng = np.random.default_rng(0)
+    d1 = rng.standard_normal((4096, 768), dtype=np.float32)
+    l1 = rng.standard_normal((4096, 8), dtype=np.float32)
     times = []
-    t_all = time.perf_counter()
-    while len(times) < 2 or (time.perf_counter() - t_all < budget_s and len(times) < 50):
+    for _ in range(6):   # 1 warm-up + median of 5
         t0 = time.perf_counter()
-        g, il, _, _, disp = c_oracle.moe_encode(data, logits, None, Cap, 2, True)
-        out = c_oracle.moe_decode(disp, g, il, 2)
+        g, il, _, _, disp = mo.moe_encode(d1, l1, np.zeros(8, np.int32), 1.25, gate_is_logits=True)
+        mo.moe_decode(disp, g, il, k=1)
         times.append(time.perf_counter() - t0)
-        del out, disp
-    best = sorted(times)[len(times) // 2]
-    n = 2048
-    d32 = mo.bf16_bits_to_f32(data[:n])
-    t0 = time.perf_counter()
-    g, il, _, _, disp = mo.moe_encode_top2(d32, logits[:n], np.zeros(E, np.int32), cf, gate_is_logits=True)
-    mo.moe_decode(disp, g, il, k=2, round_fn=mo.round_to_bf16)
-    t_np = time.perf_counter() - t0
-    return {"value": round(S / best, 1), "unit": "tokens/s", "cores": cores, "kind": "port",
-            "sample": "C/OpenMP restatement, %d whole top-2 encode+decode passes over S=%d M=%d E=%d "
-                      "(median %.3f s per pass, %d threads); NumPy restatement on one core: %.0f tokens/s "
-                      "over a %d-token slice" % (len(times), S, M, E, best, cores, n / t_np, n)}
+    t_np = sorted(times[1:])[2]
+    return {"value": round(S / t_all, 1), "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": "C/OpenMP restatement, %d whole top-2 encode+decode passes over the headline's own arrays "
+                      "(S=%d M=%d E=%d, median %.3f s per pass, %d threads)" % (n_all, S, M, E, t_all, cores),
+            "threads_all": {"threads": cores, "s_per_pass": round(t_all, 4), "tokens_per_s": round(S / t_all, 1), "passes": n_all},
+            "threads_1": {"threads": 1, "s_per_pass": round(t_one, 4), "tokens_per_s": round(S / t_one, 1), "passes": n_one},
+            "numpy_config1": {"what": "NumPy restatement in the reference tests' style (one-hot + cumsum, Python scatter "
+                                      "loop), top-1 encode + decode, S=4096 M=768 fp32 E=8 C=640, one core, median of 5",
+                              "s_per_pass": round(t_np, 4), "tokens_per_s": round(4096 / t_np, 1)}}
 
 
 def cpu_baseline_lans(hyper_steps=2):
@@ -576,9 +601,9 @@ def main():
     S, M, E, K, cf = args.tokens, args.hidden, args.experts, 2, 1.25
     b = 2  # bf16
     Cap = ops.moe_capacity(S, E, 2 * cf)
-    gen = torch.Generator(device="cuda").manual_seed(0)
-    data = torch.empty((S, M), device="cuda").normal_(0, 1, generator=gen).to(torch.bfloat16)
-    logits = torch.empty((S, E), device="cuda").normal_(0, 1, generator=gen)
+    h_data_bits, h_logits = headline_inputs(S, M, E)
+    data = torch.from_numpy(h_data_bits.view(np.int16)).cuda().view(torch.bfloat16)
+    logits = torch.from_numpy(h_logits).cuda()
     used_in = torch.zeros(E, dtype=torch.int32, device="cuda")
     outs = (torch.empty(K * S, device="cuda"), torch.empty((2, K * S), dtype=torch.int32, device="cuda"),
             torch.empty(E, dtype=torch.int32, device="cuda"), torch.empty(E, dtype=torch.int64, device="cuda"),
@@ -600,7 +625,6 @@ def main():
     from oracle import moe_oracle as mo
     step()
     torch.cuda.synchronize()
-    h_logits = logits.cpu().numpy()
     sel, val = mo.select_topk(h_logits, 2, True)
     zero = np.zeros(E, np.int32)
     i1, l1, u1, _ = mo.gen_location(sel[0], zero, Cap, M, E)
@@ -619,9 +643,12 @@ def main():
     tail_mask = torch.arange(Cap, device="cuda")[None, :] >= used[:, None]
     assert not outs[4][tail_mask].any(), "rows past the used capacity are not zero"
     either = (il_t[0, :S] >= 0) | (il_t[0, S:] >= 0)
-    # identity expert + normalised weights: decode returns the token (g1 + g2 = 1) within 1 bf16 ulp
-    err = (dec[either].float() - data[either].float()).abs() / data[either].float().abs().clamp_min(1e-30)
-    assert float(err.max()) <= 2 ** -7, "encode -> decode round trip broken"
+    # identity expert + normalised weights: decode returns the token (g1 + g2 = 1) within 1 unit in the last place
+    # of bf16, counted on the bit patterns (sign-magnitude patterns mapped to integers in value order)
+    def ordered(t):
+        i = t.view(torch.int16).to(torch.int32)
+        return torch.where(i < 0, -(i & 0x7fff), i)
+    assert int((ordered(dec[either]) - ordered(data[either])).abs().max()) <= 1, "encode -> decode round trip broken"
     assert not dec[~either].any()
     log("parity gate ok: S=%d M=%d E=%d C=%d kept=%d of %d slots" % (S, M, E, Cap, kept, K * S))
 
@@ -715,7 +742,7 @@ def main():
         result["lans"] = bench_lans(ops, capi, max(3, min(args.steps, 10)), max(1, min(args.warmup, 2)),
                                     args.lans_scale)
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(S, M, E, cf)
+        result["cpu_baseline"] = cpu_baseline(h_data_bits, h_logits, cf)
         if "lans" in result:
             result["lans"]["cpu_baseline"] = cpu_baseline_lans()
     print(json.dumps(result), flush=True)

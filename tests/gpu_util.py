@@ -47,3 +47,12 @@ def to_np(t):
 def dev(a, dtype=None):
     t = torch.from_numpy(np.ascontiguousarray(a)).cuda()
     return t if dtype is None else t.to(dtype)
+
+
+def ulp_distance(a, b):
+    """Largest distance between two 16-bit float GPU tensors of one dtype, in units of the last place (the
+    sign-magnitude bit patterns mapped to integers in value order)."""
+    x, y = a.view(torch.int16).to(torch.int32), b.view(torch.int16).to(torch.int32)
+    x = torch.where(x < 0, -(x & 0x7fff), x)
+    y = torch.where(y < 0, -(y & 0x7fff), y)
+    return int((x - y).abs().max()) if x.numel() else 0

@@ -11,7 +11,7 @@ import pytest
 import torch
 
 from oracle import moe_oracle as mo
-from tests.gpu_util import dev, make_inputs, rows_to_torch, to_np
+from tests.gpu_util import ulp_distance, dev, make_inputs, rows_to_torch, to_np
 
 pytestmark = pytest.mark.gpu
 
@@ -71,8 +71,10 @@ def test_config2_gshard_top2_zipf(pkg, dt):
     # identity expert: out = (g1 + g2) * x with g1 + g2 = 1 where any slot was kept, else 0
     either = (got[1][0, :S] >= 0) | (got[1][0, S:] >= 0)
     x = d_data.float()
-    tol = 2e-6 if dt == "f32" else 2 ** -7
-    assert float(((out.float() - x)[either].abs() / x[either].abs().clamp_min(1e-20)).max()) <= tol
+    if dt == "f32":
+        assert float(((out.float() - x)[either].abs() / x[either].abs().clamp_min(1e-20)).max()) <= 2e-6
+    else:   # 1 unit in the last place of bf16 (north_star's bound for the combine), counted on the bit patterns
+        assert ulp_distance(out[either], d_data[either]) <= 1
     assert not out[~either].any() and (~either).any()
 
 
@@ -103,17 +105,22 @@ def test_config3_batch_prioritized_bf16(pkg, P, hot_experts):
     assert bool((cnt > 640).any()) == hot_experts
 
 
-def test_config4_lancet_forward_pipeline_bf16(pkg):
+@pytest.mark.parametrize("pressure", [False, True])
+def test_config4_lancet_forward_pipeline_bf16(pkg, pressure):
     """S=65536 (4 partitions of 16384), M=4096 bf16, E=32, top-2, cf=1.25 -> C=5120: encode per
     (slot, partition) in capacity order s1p0..s1p3, s2p0..s2p3 with chained used capacity, then
-    moe_merge_masks + moe_redispatch, then moe_decode; must equal the un-partitioned top-2 op."""
+    moe_merge_masks + moe_redispatch, then moe_decode; must equal the un-partitioned top-2 op.
+    Inputs as the configuration states them: NumPy default_rng(0), data then logits, both N(0,1), rows rounded
+    to bf16 (nothing is dropped at C = 5120 then); and the same with four favoured experts, so that slots overflow."""
     ops = pkg.ops
     S0, M, E, cf, P = 65536, 4096, 32, 1.25, 4
     S = S0 // P
-    gen = torch.Generator(device="cuda").manual_seed(0)
-    data = torch.empty((S0, M), device="cuda").normal_(0, 1, generator=gen).to(torch.bfloat16)
-    logits = torch.empty((S0, E), device="cuda").normal_(0, 1, generator=gen)
-    logits[:, :4] += 0.75            # some pressure so that slot 2 overflows
+    rng = np.random.default_rng(0)
+    data = torch.from_numpy(mo.f32_to_bf16_bits(rng.standard_normal((S0, M), dtype=np.float32)).view(np.int16)).cuda().view(torch.bfloat16)
+    h_logits = rng.standard_normal((S0, E), dtype=np.float32)
+    if pressure:
+        h_logits[:, :4] += np.float32(0.75)
+    logits = torch.from_numpy(h_logits).cuda()
     fused = ops.moe_encode(data, logits, None, cf, top_k=2, gate_is_logits=True)
     assert fused[4].shape == (E, 5120, M)
     # per-slot gate arrays: argmax = the slot's expert, max = its softmax probability
@@ -141,13 +148,12 @@ def test_config4_lancet_forward_pipeline_bf16(pkg):
     assert torch.equal(used, fused[2])
     assert torch.equal(red, fused[4])
     np.testing.assert_allclose(to_np(weights), to_np(fused[0]), rtol=1e-5)
-    assert int((merged[0] < 0).sum()) > 0
+    assert (int((merged[0] < 0).sum()) > 0) == pressure
     out_p = ops.moe_decode(red, weights, merged, top_k=2)
     out_f = ops.moe_decode(fused[4], fused[0], fused[1], top_k=2)
     diff = (out_p.view(torch.int16).int() - out_f.view(torch.int16).int()).abs().max()
     assert int(diff) <= 1
     # routing at full size against the oracle
-    h_logits = logits.cpu().numpy()
     osel, _ = mo.select_topk(h_logits, 2, True)
     zero = np.zeros(E, np.int32)
     i1, l1, u1, _ = mo.gen_location(osel[0], zero, 5120, M, E)
@@ -213,8 +219,16 @@ def test_config5_lans_full_size(pkg):
         assert plan.error() == 0
         for k, i in enumerate(sample):
             for got, want, tol, what in ((p[i], ref_p[k], 1e-6, "p"), (m[i], ref_m[k], 1e-5, "m"), (v[i], ref_v[k], 1e-5, "v")):
-                err = np.abs(to_np(got).astype(np.float64) - want).max()
+                diff = np.abs(to_np(got).astype(np.float64) - want)
+                err = diff.max()
                 assert err <= tol * np.abs(want).max(), "%s %s[%d]: %.3e" % (name, what, i, err)
+                if what == "p":
+                    # element by element: 1e-6 relative, with a floor of 1e-9 of the tensor's largest entry for the
+                    # entries near zero (an entry moves by about lr * |p| per step whatever its own size, so the
+                    # last place of that movement, not of the entry, bounds what two evaluation orders can differ by)
+                    bound = 1e-6 * np.abs(want) + 1e-9 * np.abs(want).max()
+                    assert (diff <= bound).all(), "%s p[%d]: %.3e relative at the worst entry" % (
+                        name, i, (diff / np.maximum(np.abs(want), 1e-30)).max())
     ps, pr = state["sweeps"][0], state["resident"][0]
     for i in range(len(shapes)):
         scale = float(ps[i].abs().max())

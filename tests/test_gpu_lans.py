@@ -69,6 +69,8 @@ def test_lans_reference_test_shapes(pkg):
     dict(mode=0), dict(weight_decay=0.0), dict(normalize_grad=False), dict(bias_correction=0),
     dict(grad_averaging=0), dict(mode=0, weight_decay=0.0, normalize_grad=False),
     dict(lr=5e-2, beta1=0.8, beta2=0.99, eps=1e-8),
+    # mode 0 with weight decay: wd * p joins the scaled gradient before the moments (multi_tensor_lans.cu:287-297)
+    dict(mode=0, weight_decay=0.25, lr=0.1, beta1=0.5, beta2=0.5, bias_correction=0),
 ])
 def test_lans_flags(pkg, hyper):
     run_both(pkg, [(300, 40), (129,), (64, 64)], 5, seed=3, **hyper)

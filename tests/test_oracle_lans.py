@@ -114,3 +114,34 @@ def test_flags(bias_correction, grad_averaging):
         np.testing.assert_allclose([bc1, bc2], [1 - 0.9 ** 5, 1 - 0.999 ** 5], rtol=1e-4)
     else:
         assert bc1 == 1 and bc2 == 1
+
+
+def test_mode0_weight_decay_two_elements_by_hand():
+    """Mode 0 adds weight_decay * p to the scaled gradient BEFORE the moments
+    (multi_tensor_lans.cu:287-297); mode 1 adds it to the two updates after them (:299-306).  With two
+    elements the placement shows in p, m and v.  Numbers worked out by hand for g = (0.3, -0.4),
+    p = (2, 1), m = v = 0, lr 0.1, beta1 = beta2 = 0.5, eps 0, no bias correction, wd 0.25:
+    ||g|| = 0.5, g/||g|| = (0.6, -0.8), + wd*p = (1.1, -0.55); m' = 0.5 * that, v' = 0.5 * that^2;
+    u_m = m'/sqrt(v') = (1, -1)/sqrt(2), u_g = (1, -1)*sqrt(2); ||u_m|| = 1, ||u_g|| = 2, ||p|| = sqrt(5);
+    p' = p - (0.1*sqrt(5)/1*0.5)*u_m - (0.1*sqrt(5)/2*0.5)*u_g = p -/+ 0.1*sqrt(5)/sqrt(2)."""
+    kw = dict(lr=0.1, beta1=0.5, beta2=0.5, eps=0.0, bias_correction=0, weight_decay=0.25, grad_averaging=1,
+              normalize_grad=True)
+    g = [np.array([0.3, -0.4], np.float32)]
+    p, m, v = [np.array([2.0, 1.0], np.float32)], [np.zeros(2, np.float32)], [np.zeros(2, np.float32)]
+    lo.lans_step(g, p, m, v, 1, mode=0, **kw)
+    np.testing.assert_allclose(m[0], [0.55, -0.275], rtol=1e-6)
+    np.testing.assert_allclose(v[0], [0.605, 0.15125], rtol=1e-6)
+    np.testing.assert_allclose(p[0], [2.0 - 0.15811388300841897, 1.0 + 0.15811388300841897], rtol=1e-6)
+    # the same input in mode 1: the moments see the bare scaled gradient, the updates get wd*p:
+    # m' = (0.3, -0.4), v' = (0.18, 0.32); u_m = (1/sqrt(2) + 0.5, -1/sqrt(2) + 0.25),
+    # u_g = (sqrt(2) + 0.5, -sqrt(2) + 0.25): a different step
+    p1, m1, v1 = [np.array([2.0, 1.0], np.float32)], [np.zeros(2, np.float32)], [np.zeros(2, np.float32)]
+    lo.lans_step(g, p1, m1, v1, 1, mode=1, **kw)
+    np.testing.assert_allclose(m1[0], [0.3, -0.4], rtol=1e-6)
+    np.testing.assert_allclose(v1[0], [0.18, 0.32], rtol=1e-6)
+    um = np.array([0.7071067811865476 + 0.5, -0.7071067811865476 + 0.25])
+    ug = np.array([1.4142135623730951 + 0.5, -1.4142135623730951 + 0.25])
+    rm = 0.1 * 2.23606797749979 / np.sqrt((um * um).sum()) * 0.5
+    rg = 0.1 * 2.23606797749979 / np.sqrt((ug * ug).sum()) * 0.5
+    np.testing.assert_allclose(p1[0], np.array([2.0, 1.0]) - rm * um - rg * ug, rtol=1e-6)
+    assert abs(p1[0][0] - p[0][0]) > 1e-3

@@ -31,7 +31,6 @@ int DTypeToLancet(const DType& dt) {
   throw Error("token rows must be float32, float16 or bfloat16");
 }
 
-bool IsF32(const DType& dt) { return dt.code == DTypeCode::kFloat && dt.bits == 32; }
 // Gate arrays come in the type the graph has them in: fp32, or a half type under mixed precision
 // (python/raf/amp/type_hints.py:97,105; the reference's kernels take `__dtype* gates1_s`).
 int GateDTypeToLancet(const DType& dt) {

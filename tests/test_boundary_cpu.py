@@ -375,3 +375,18 @@ def test_header_is_plain_c_and_the_c_client_links():
     build_dir = os.path.join(root, "tests", "c_client")
     subprocess.run(["make", "-C", build_dir, "-B"], check=True, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
     assert os.path.exists(os.path.join(build_dir, "lancet_client")) and shutil.which("gcc")
+
+
+def test_op_layer_under_address_and_undefined_behaviour_sanitizers():
+    """The C++ op layer (raf_hip/) built with -fsanitize=address,undefined and run on host memory for every operator
+    of the hip dialect, against a host-only stand-in for the C ABI whose calls touch every byte the kernels touch
+    (tests/c_client/op_layer_san.cc): a wrong shape, dtype or size in the op layer is a sanitizer report.  The
+    reference builds its host code under the same sanitizers (cmake/modules/Sanitizer.cmake:13-40)."""
+    import subprocess
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "c_client")
+    subprocess.run(["make", "-C", here, "op_layer_san"], check=True, stdout=subprocess.DEVNULL)
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0", UBSAN_OPTIONS="print_stacktrace=1")
+    proc = subprocess.run([os.path.join(here, "op_layer_san")], env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert proc.returncode == 0, proc.stdout[-4000:]
+    assert "every operator ran under the sanitizers" in proc.stdout
+    assert "ERROR: AddressSanitizer" not in proc.stdout and "runtime error" not in proc.stdout

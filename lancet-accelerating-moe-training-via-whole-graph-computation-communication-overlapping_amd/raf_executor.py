@@ -59,6 +59,7 @@ def load():
         "raf_hip_num_workspaces": (ci, [vp]),
         "raf_hip_workspace_bytes": (i64, [vp, ci]),
         "raf_hip_bind_workspace": (ci, [vp, ci, vp]),
+        "raf_hip_check_device_status": (ci, [vp]),
         "raf_hip_num_arg_indices": (ci, [vp]),
         "raf_hip_arg_index": (ci, [vp, ci]),
         "raf_hip_set_stream": (None, [ci, vp]),
@@ -180,6 +181,11 @@ class PreparedCall:
         _check(self._lib.raf_hip_execute(self._h))
         return self.outputs
 
+    def check(self):
+        """Raises if the device recorded a failure in work this call launched (a bounded wait that gave up);
+        synchronises the current stream."""
+        _check(self._lib.raf_hip_check_device_status(self._h))
+
     def close(self):
         if self._h is not None:
             self._lib.raf_hip_call_destroy(self._h)
@@ -199,7 +205,9 @@ class Executor:
     def __call__(self, op_name, *args):
         call = PreparedCall(op_name, args)
         try:
-            return call.run()
+            out = call.run()
+            call.check()          # synchronises; the reference would have aborted on a device-side failure
+            return out
         finally:
             # outputs are torch tensors and stay valid; the OpEnv (and, for lans, its plan) goes away.
             # Work already enqueued only touches caller-owned memory and the workspaces kept below.

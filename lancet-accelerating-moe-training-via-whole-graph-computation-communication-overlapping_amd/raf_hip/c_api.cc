@@ -168,6 +168,15 @@ int raf_hip_execute(void* h) {
   });
 }
 
+// the executor has synchronised (or is about to): failures the device recorded become an error here
+int raf_hip_check_device_status(void* h) {
+  return Guard([&] {
+    Call* c = static_cast<Call*>(h);
+    RAF_CHECK(c->env != nullptr, "dispatch the call before checking it");
+    c->env->CheckDeviceStatus(OpEnv::GetStream(c->cv.device_id));
+  });
+}
+
 // dialect preference scope + registry queries
 int raf_hip_push_dialect_preference(const char* comma_separated) {
   return Guard([&] {

@@ -91,6 +91,13 @@ class LansImpl : public OpEnv {
       throw Error(std::string("lancet_lans_step failed: ") + lancet_status_string(st) + " (status " + std::to_string(st) + ")");
   }
 
+  void CheckDeviceStatus(void* stream) override {
+    int err = 0;
+    int st = lancet_lans_plan_error(plan_, stream, &err);
+    if (st != LANCET_OK) throw Error(std::string("lancet_lans_plan_error failed: ") + lancet_status_string(st));
+    if (err) throw Error("lans: a step of the resident schedule gave up a wait; the parameters of that step were left unwritten");
+  }
+
   std::string name() const override { return "raf.op.hip.lans"; }
   static OpEnv* make(const CallValues& cv) { return new LansImpl(cv); }
 

@@ -58,6 +58,15 @@ struct ScanWorkspaceState {
     CheckStatus(lancet_scan_workspace_init(ws, nbytes, stream), "lancet_scan_workspace_init");
     ready = ws;
   }
+  // the workspace's sticky error word (read and cleared; synchronises the stream)
+  void Check(void* ws, void* stream, const char* op) {
+    if (!ws || ws != ready) return;
+    int err = 0;
+    CheckStatus(lancet_scan_workspace_error(ws, stream, &err), "lancet_scan_workspace_error");
+    if (err)
+      throw Error(std::string(op) + ": the position scan gave up a wait for another workgroup; the tokens concerned "
+                  "carry indices_locations = -1 (used_capacity = -1 if the totals were lost)");
+  }
 };
 
 Tensor MakeOut(int device_id, DTypeCode code, int bits, std::vector<int64_t> shape) {
@@ -193,6 +202,7 @@ class MoeEncode : public OpEnv {
   }
 
   void WorkspaceBound() override { scan_ws_.ready = nullptr; }
+  void CheckDeviceStatus(void* stream) override { scan_ws_.Check(ws_, stream, "moe_encode"); }
   std::string name() const override { return "raf.op.hip.moe_encode"; }
   static OpEnv* make(const CallValues& cv) { return new MoeEncode(cv); }
 
@@ -258,6 +268,7 @@ class MoeEncodeBatchPrioritized : public OpEnv {
   }
 
   void WorkspaceBound() override { scan_ws_.ready = nullptr; }
+  void CheckDeviceStatus(void* stream) override { scan_ws_.Check(ws_, stream, "moe_encode_batch_prioritized"); }
   std::string name() const override { return "raf.op.hip.moe_encode_batch_prioritized"; }
   static OpEnv* make(const CallValues& cv) { return new MoeEncodeBatchPrioritized(cv); }
 

@@ -142,6 +142,11 @@ class OpEnv {
   // Called by the executor after it has written a request's destination: the memory behind a workspace is
   // new (or has been used by others since the last Execute), whatever its address.
   virtual void WorkspaceBound() {}
+  // Called by the executor where it waits for the device anyway (after a run, at a synchronisation point of
+  // the schedule): throws if the device recorded a failure in work this OpEnv launched.  The reference aborts the
+  // process on any failure (src/common/cuda_utils.h:18-22); here failures that only show on the device (a
+  // bounded wait that gave up) mark the outputs at once and are reported here.  Synchronises `stream`.
+  virtual void CheckDeviceStatus(void* stream) { (void)stream; }
 
   // Data input indices in the argument list (used by the VM executor).
   std::vector<int> arg_indices;

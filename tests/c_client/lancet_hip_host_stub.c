@@ -46,6 +46,14 @@ int lancet_scan_workspace_init(void* ws, size_t nbytes, lancet_stream_t st) {
   return 0;
 }
 
+int lancet_scan_workspace_error(void* ws, lancet_stream_t st, int* error_out) {
+  (void)st;
+  if (!ws || !error_out) return LANCET_ERR_NULL;
+  touch_read(ws, 32);
+  *error_out = 0;
+  return 0;
+}
+
 int lancet_moe_encode(const void* data, const void* gate, const void* noise, const int32_t* used_in, int64_t S, int64_t M,
                       int64_t E, int64_t C, int top_k, int dtype, int gate_dtype, unsigned flags, void* gates_s,
                       int32_t* il, int32_t* used_out, uint64_t* elems, void* dispatched, void* ws, size_t ws_bytes,
@@ -200,6 +208,12 @@ int lancet_lans_plan_destroy(lancet_lans_plan_t plan) {
 int lancet_lans_plan_set_schedule(lancet_lans_plan_t plan, int schedule) {
   (void)schedule;
   return plan ? 0 : LANCET_ERR_PLAN;
+}
+int lancet_lans_plan_error(lancet_lans_plan_t plan, lancet_stream_t st, int* error_out) {
+  (void)st;
+  if (!plan || !error_out) return LANCET_ERR_PLAN;
+  *error_out = 0;
+  return 0;
 }
 int lancet_lans_step(lancet_lans_plan_t plan, const float* const* g, float* const* p, float* const* m, float* const* v,
                      int step_host, const float* step_dev, const lancet_lans_hyper* hyper, const float* grad_norms,

@@ -32,6 +32,7 @@ int raf_hip_num_workspaces(void* h);
 int64_t raf_hip_workspace_bytes(void* h, int i);
 int raf_hip_bind_workspace(void* h, int i, void* data);
 int raf_hip_execute(void* h);
+int raf_hip_check_device_status(void* h);
 }
 
 namespace {
@@ -87,6 +88,7 @@ void run(void* h, Arena& a, const char* what) {
       MUST(raf_hip_bind_workspace(h, i, a.get(static_cast<size_t>(raf_hip_workspace_bytes(h, i)))));
     MUST(raf_hip_execute(h));
     MUST(raf_hip_execute(h));
+    MUST(raf_hip_check_device_status(h));
   }
   printf("ok   %-40s %s\n", raf_hip_env_name(h), what);
 }

@@ -99,3 +99,41 @@ def test_plain_c_client_of_the_c_abi():
     proc = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=100)
     assert proc.returncode == 0, proc.stdout
     assert "match the hand-computed case" in proc.stdout
+
+
+def test_op_layer_reports_a_scan_that_gave_up(pkg, ex):
+    """A prepared call keeps its OpEnv and workspace across runs (RAF's interpreter cache): the workspace is set up
+    by the first run only; with a wait bound of one poll the scan gives up somewhere in 256 tiles, the outputs carry
+    the marks, and check() raises where the reference would have aborted; the next run is whole again."""
+    import ctypes as C
+    lib = pkg.capi.load()
+    S, M, E = 65536, 8, 8
+    data, logits = make_inputs(13, S, M, E)
+    gate = mo.softmax_rows(logits)
+    want = mo.moe_encode(data, gate, np.zeros(E, np.int32), 1.0, fast_scatter=True)
+    call = ex.prepare("raf.op.moe_encode", dev(data), dev(gate), dev(np.zeros(E, np.int32)), 1.0)
+    try:
+        got = call.run()
+        call.check()
+        np.testing.assert_array_equal(to_np(got[1]), want[1])
+        ws = C.c_void_p(call.workspaces[0].data_ptr())
+        raised = 0
+        for _ in range(3):
+            assert lib.lancet_debug_scan_workspace_spin_limit(ws, 1, None) == 0
+            got = call.run()
+            assert lib.lancet_debug_scan_workspace_spin_limit(ws, 0, None) == 0
+            il = to_np(got[1])
+            marked = ((il[0] == -1) & (il[1] == -1)).any()
+            try:
+                call.check()
+                assert not marked
+            except pkg.raf_executor.RafError as e:
+                raised += 1
+                assert "gave up a wait" in str(e)
+            got = call.run()
+            call.check()              # the word was cleared by the check that raised
+            np.testing.assert_array_equal(to_np(got[1]), want[1])
+            np.testing.assert_array_equal(to_np(got[4]), want[4])
+        assert raised > 0
+    finally:
+        call.close()

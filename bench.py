@@ -42,7 +42,7 @@ def parse():
     ap.add_argument("--lans-scale", type=float, default=1.0, help="fraction of the 24-layer LANS tensor list")
     ap.add_argument("--lans-schedule", default=None, choices=["sweeps", "resident"],
                     help="time only this LANS schedule (profiling)")
-    ap.add_argument("--only", default="all", choices=["all", "scatter", "decode", "route", "copy", "lans"],
+    ap.add_argument("--only", default="all", choices=["all", "scatter", "decode", "route", "copy", "stream_copy", "lans"],
                     help="profiling aid: run just one kernel family (prints a short JSON line)")
     return ap.parse_args()
 
@@ -590,6 +590,19 @@ def main():
             dst.copy_(src)
         ms = event_ms(lambda: dst.copy_(src), args.steps)
         print(json.dumps({"only": "copy", "bytes_read": n, "bytes_written": n, "ms": round(ms, 4),
+                          "GBps": round(2 * n / ms / 1e6, 1)}), flush=True)
+        return
+    if args.only == "stream_copy":
+        # the library's own plain copy (lancet_debug_stream: one 16-byte non-temporal access per thread, workgroups
+        # in address order) over 1 GiB: the kernel the scatter's counters are read against
+        n = 1 << 30
+        src = torch.zeros(n, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        run = lambda: lib.lancet_debug_stream(2, C.c_void_p(dst.data_ptr()), C.c_void_p(src.data_ptr()), n, None)
+        for _ in range(args.warmup):
+            assert run() == 0
+        ms = event_ms(run, args.steps)
+        print(json.dumps({"only": "stream_copy", "bytes_read": n, "bytes_written": n, "ms": round(ms, 4),
                           "GBps": round(2 * n / ms / 1e6, 1)}), flush=True)
         return
     if args.only == "lans":

@@ -146,7 +146,7 @@ def _check_noise(gate2_noise, gate, top_k):
 
 
 def moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_logits=False,
-               zero_tail=True, gate2_noise=None, rows_at_used=False, workspace=None, out=None):
+               zero_tail=True, gate2_noise=None, rows_at_used=False, workspace=None, out=None, capacity=None):
     """raf.op.moe_encode(data, gate, used_capacity, capacity_factor=1.0).
 
     Returns (gates_s [k*S] f32, indices_locations [2, k*S] i32, used_capacity [E] i32,
@@ -156,7 +156,11 @@ def moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_
     docker/resources/sharded_moe.py:275, drawn by the caller).  rows_at_used=True writes the rows of expert e
     from row used_capacity[e] on: chained partition encodes that pass the same `dispatched` buffer (out=) fill
     it the way moe_redispatch would, the last one with zero_tail=True, the others without.  zero_tail=False
-    leaves rows past the used capacity unwritten (partition buffers that only feed moe_redispatch)."""
+    leaves rows past the used capacity unwritten (partition buffers that only feed moe_redispatch).
+    capacity, if given, is used as it is instead of the reference formula: GShard's own top-2 capacity is
+    ceil(2 * S / E * capacity_factor) (docker/resources/sharded_moe.py:267), which differs from
+    int(2 * capacity_factor * ceil(S / E)) when E does not divide S or the factor is fractional
+    (S = 300, E = 8, factor 1: 75 against 76)."""
     lib = capi.load()
     dt = _check_encode_inputs(data, gate)
     S, M = data.shape
@@ -164,7 +168,8 @@ def moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_
     _need(top_k in (1, 2), "top_k must be 1 or 2")
     _check_noise(gate2_noise, gate, top_k)
     cf = float(capacity_factor) * (2.0 if top_k == 2 else 1.0)
-    Cap = moe_capacity(S, E, cf)
+    Cap = moe_capacity(S, E, cf) if capacity is None else int(capacity)
+    _need(Cap >= 0, "capacity must not be negative")
     if used_capacity is not None:
         _dev(used_capacity, "used_capacity")
         _need(used_capacity.dim() == 1 and used_capacity.numel() == E and used_capacity.dtype == torch.int32,
@@ -188,7 +193,7 @@ def moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_
 
 
 def moe_route(gate, used_capacity, M, capacity_factor=1.0, top_k=1, gate_is_logits=False, gate2_noise=None,
-              workspace=None, out=None):
+              workspace=None, out=None, capacity=None):
     """The routing half of moe_encode (selection + position scan, src/op/dialect/cuda/moe.cc:366-380), so that
     a caller can run it ahead of, or beside, the row movement of another partition.  M only scales
     elements_per_expert.  Returns (gates_s, indices_locations, used_capacity, elements_per_expert)."""
@@ -199,7 +204,7 @@ def moe_route(gate, used_capacity, M, capacity_factor=1.0, top_k=1, gate_is_logi
     S, E = gate.shape
     _need(top_k in (1, 2), "top_k must be 1 or 2")
     _check_noise(gate2_noise, gate, top_k)
-    Cap = moe_capacity(S, E, float(capacity_factor) * (2.0 if top_k == 2 else 1.0))
+    Cap = moe_capacity(S, E, float(capacity_factor) * (2.0 if top_k == 2 else 1.0)) if capacity is None else int(capacity)
     dev = gate.device
     if out is None:
         out = (torch.empty(top_k * S, dtype=gate.dtype, device=dev),

@@ -47,6 +47,14 @@ def capacity(S, E, capacity_factor):
     return int(np.float32(capacity_factor) * np.float32((S + E - 1) // E))
 
 
+def gshard_top2_capacity(S, E, capacity_factor):
+    """ceil(2 * S / E * cf) in double precision (docker/resources/sharded_moe.py:267): GShard's own top-2
+    capacity.  The top-2 extension here follows the reference op's formula with the factor doubled
+    (capacity(S, E, 2 * cf)); the two agree when E divides S and 2 * cf * S / E is whole."""
+    import math
+    return int(math.ceil((2 * S / E) * capacity_factor))
+
+
 # --------------------------------------------------------------------------
 # A0: gate softmax (outside the reference op; models/benchmark/pytorch/utils.py:565-573)
 # --------------------------------------------------------------------------

@@ -874,3 +874,18 @@ def test_range_copies_along_axis_1(pkg):
     wire2 = ops.memcpy_sparse_ranges_to_cont_3d(dev(buf), torch.zeros(2000, device="cuda"), dev(counts.astype(np.int64)),
                                                 dev(starts.astype(np.int64)), axis=1)
     np.testing.assert_array_equal(to_np(wire2), mo.memcpy_sparse_ranges_to_cont_3d(buf, np.zeros(2000, np.float32), counts, starts, axis=1))
+
+
+def test_capacity_override_gshard_formula(pkg):
+    """capacity= replaces the formula: GShard's ceil(2 S / E * cf) where E does not divide S (75 against 76)."""
+    S, M, E = 300, 16, 8
+    data, logits = make_inputs(71, S, M, E, zipf_bias=True)
+    C = mo.gshard_top2_capacity(S, E, 1.0)
+    assert C == 75 and pkg.ops.moe_capacity(S, E, 2.0) == 76
+    want = mo.moe_encode_top2(data, logits, np.zeros(E, np.int32), 1.0, gate_is_logits=True, C=C, fast_scatter=True)
+    got = pkg.ops.moe_encode(dev(data), dev(logits), None, 1.0, top_k=2, gate_is_logits=True, capacity=C)
+    assert got[4].shape == (E, 75, M)
+    for i in (1, 2, 3, 4):
+        np.testing.assert_array_equal(to_np(got[i]), want[i])
+    r = pkg.ops.moe_route(dev(logits), None, M, 1.0, top_k=2, gate_is_logits=True, capacity=C)
+    np.testing.assert_array_equal(to_np(r[1]), want[1])

@@ -499,3 +499,28 @@ def test_partition_ranges_of_a_top2_routing_hold_the_partitions_tokens_in_order(
                 np.testing.assert_array_equal(disp[e, r0:r0 + len(toks)], data[toks])
                 assert [int(il[1, j * S0 + s]) for s in toks] == list(range(r0, r0 + len(toks)))
     np.testing.assert_array_equal((starts + counts)[-1], used.astype(np.uint64) * np.uint64(M))
+
+
+def test_top2_capacity_formula_against_gshard():
+    """The top-2 extension sizes the buffer with the reference op's formula and a doubled factor,
+    int(2 cf * ceil(S / E)); GShard's own is ceil(2 S / E * cf) (sharded_moe.py:267).  They agree on every
+    BASELINE configuration and differ when E does not divide S or the factor is fractional; a caller that
+    wants GShard's passes it as the capacity override, and the drop set then is GShard's."""
+    for S, E, cf in [(16384, 16, 1.0), (65536, 32, 1.25), (4096, 8, 1.0)]:
+        assert mo.capacity(S, E, 2 * cf) == mo.gshard_top2_capacity(S, E, cf)
+    assert (mo.capacity(300, 8, 2.0), mo.gshard_top2_capacity(300, 8, 1.0)) == (76, 75)
+    assert (mo.capacity(1000, 7, 2 * 1.1), mo.gshard_top2_capacity(1000, 7, 1.1)) == (314, 315)
+    # with the override the oracle's drop set is that of the dense GShard form at that capacity
+    rng = np.random.default_rng(4)
+    S, E, M = 300, 8, 3
+    data = rng.standard_normal((S, M), dtype=np.float32)
+    logits = rng.standard_normal((S, E), dtype=np.float32)
+    logits[:, 0] += 2.0
+    C = mo.gshard_top2_capacity(S, E, 1.0)
+    g, il, used, _, disp = mo.moe_encode_top2(data, logits, np.zeros(E, np.int32), 1.0, gate_is_logits=True, C=C)
+    assert disp.shape == (E, 75, M) and used.max() == 75
+    kept1 = il[0, :S] >= 0
+    first = np.argmax(logits, axis=1)
+    for e in range(E):   # slot 1 keeps the first C tokens of every expert, in token order
+        tok = np.flatnonzero(first == e)
+        assert kept1[tok[:C]].all() and not kept1[tok[C:]].any()

@@ -8,6 +8,7 @@ gate_is_logits, workspace, out).  torch supplies device memory and the current
 stream; all computation is done by the HIP kernels behind the C ABI.
 """
 import ctypes as C
+import functools
 import os
 
 import torch
@@ -114,6 +115,7 @@ def scan_errors():
     return sum(ws.error() for ws in list(_scan_pool.values()))
 
 
+@functools.lru_cache(maxsize=256)
 def moe_capacity(S, E, capacity_factor):
     """C = int(float(cf) * ceil(S / E)) (src/op/dialect/cuda/moe.cc:107-109)."""
     return int(capi.load().lancet_moe_capacity(int(S), int(E), float(capacity_factor)))
@@ -128,6 +130,7 @@ def _check_encode_inputs(data, gate):
     return _dtype_code(data)
 
 
+@functools.lru_cache(maxsize=256)
 def moe_encode_workspace_bytes(S, E, top_k=1):
     return int(capi.load().lancet_moe_encode_workspace_bytes(int(S), int(E), int(top_k)))
 
@@ -279,6 +282,7 @@ def moe_decode_tokens(data, gate, indices_locations, token_first, n_tokens, top_
     return out
 
 
+@functools.lru_cache(maxsize=256)
 def moe_encode_bpr_workspace_bytes(S0, E, n_partitions=1):
     return int(capi.load().lancet_moe_encode_bpr_workspace_bytes(int(S0), int(E), int(n_partitions)))
 

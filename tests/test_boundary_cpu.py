@@ -354,6 +354,7 @@ def test_missing_library_is_an_error_not_a_fallback(pkg, monkeypatch, tmp_path):
     monkeypatch.setattr(capi, "LIB_PATH", str(tmp_path / "liblancet_hip.so"))
     with pytest.raises(RuntimeError, match="not built"):
         capi.load()
+    pkg.ops.moe_capacity.cache_clear()   # sizes are cached per shape; every operator loads the library first
     with pytest.raises(RuntimeError, match="not built"):
         pkg.ops.moe_capacity(16, 4, 1.0)
     src = open(os.path.join(os.path.dirname(capi.__file__), "ops.py")).read()

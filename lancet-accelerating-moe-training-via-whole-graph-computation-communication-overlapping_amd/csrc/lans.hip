@@ -5,10 +5,10 @@
 //   phase M  reads g, p, m, v      -> writes m, v; per-chunk sums of p^2, u_m^2 and u_g^2
 //   phase U  reads g, p, m, v      -> recomputes u_m, u_g (never stored) and writes p
 // and two schedules:
-//   * sweeps (default): three plain launches + two tiny per-tensor reductions.  Real HBM traffic
-//     is 48 B/param (g read three times, p, m, v twice).
-//   * resident (opt-in): ONE persistent kernel in which every array is read once and written once
-//     (28 B/param).  A workgroup runs a three-stage software pipeline over the chunks it draws from a
+//   * sweeps: three plain launches + two tiny per-tensor reductions.  Real HBM traffic
+//     is 48 B/param (g read three times, p, m, v twice).  No workgroup waits for another.
+//   * resident (what a new plan runs): ONE persistent kernel in which every array is read once and written
+//     once (28 B/param).  A workgroup runs a three-stage software pipeline over the chunks it draws from a
 //     ticket: stage N loads g of a chunk into registers and publishes its sum of squares; stage M, one
 //     iteration later, loads p, m, v of that chunk, writes m and v and keeps u_m, u_g in registers and p
 //     in LDS; stage U, another iteration later, writes p.  Between the stages of one chunk the workgroup

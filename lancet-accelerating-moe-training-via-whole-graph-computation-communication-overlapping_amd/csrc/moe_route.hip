@@ -257,6 +257,116 @@ __global__ __launch_bounds__(kTile) void route_scan_kernel(RouteArgs a) {
   tile_end(a.ws, me, a.ntiles, K * a.E);
 }
 
+// ---- the same routing as two kernels that wait for nothing (use_count_place) -----------------------------------
+// route_count_kernel: selection, ranks inside the tile, the tile's counts -> table.  Leaves expert, rank inside the
+// tile and raw gate value in idx_out / loc_out / gates_s (idx_out is not written when the experts are given).
+template <int K, int GD>
+__global__ __launch_bounds__(kTile) void route_count_kernel(RouteArgs a) {
+  extern __shared__ uint32_t s_cnt[];
+  const int tid = threadIdx.x;
+  const uint32_t tile = blockIdx.x;
+  const int s = static_cast<int>(tile) * kTile + tid;
+  const bool valid = s < a.S;
+  int e[K];
+  float p[K];
+#pragma unroll
+  for (int j = 0; j < K; ++j) {
+    e[j] = -1;
+    p[j] = 0.f;
+  }
+  if (valid) {
+    if (a.idx_in) {
+      const int x = a.idx_in[s];
+      e[0] = (x >= 0 && x < a.E) ? x : -1;
+    } else {
+      constexpr size_t gb = GD == LANCET_F32 ? 4 : 2;
+      const size_t off = static_cast<size_t>(s) * a.E * gb;
+      const Routed r = route_token<K, GD>(static_cast<const char*>(a.gate) + off,
+                                          a.noise ? static_cast<const char*>(a.noise) + off : nullptr, a.E,
+                                          a.is_logits != 0);
+      e[0] = r.e0;
+      p[0] = r.p0;
+      if (K == 2) {
+        e[K - 1] = r.e1;
+        p[K - 1] = r.p1;
+      }
+    }
+  }
+  uint32_t rank[K];
+  bool mem[K];
+#pragma unroll
+  for (int j = 0; j < K; ++j) mem[j] = e[j] >= 0;
+  TileStart me;
+  me.tile = tile, me.epoch = 0u, me.spin = 0u, me.ok = true;
+  tile_scan<K, false>(e, mem, a.E, me, a.ws, s_cnt, rank);
+  store_tile_counts(a.ws, tile, K * a.E, s_cnt);
+  if (valid) {
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+      if (!a.idx_in) a.idx_out[static_cast<size_t>(j) * a.S + s] = e[j];
+      if (!a.idx_in || e[j] >= 0) a.loc_out[static_cast<size_t>(j) * a.S + s] = static_cast<int>(rank[j]);
+      if (a.gates_s) st_gate(a.gates_s, static_cast<size_t>(j) * a.S + s, p[j], GD);
+    }
+  }
+}
+
+// route_place_kernel: every tile adds up what the tiles before it counted (and what all tiles counted) and finishes
+// its tokens: what route_scan_kernel does after its look-back and, for K = 2, what finalize_top2_kernel does.
+template <int K>
+__global__ __launch_bounds__(kTile) void route_place_kernel(RouteArgs a) {
+  extern __shared__ uint32_t s_sum[];  // [2][K * E]: before this tile, all tiles
+  const int NC = K * a.E;
+  uint32_t* s_before = s_sum;
+  uint32_t* s_total = s_sum + NC;
+  const uint32_t tile = blockIdx.x;
+  sum_tile_counts(a.ws, tile, a.ntiles, NC, s_before, s_total);
+  const int s = static_cast<int>(tile) * kTile + threadIdx.x;
+  if (s < a.S) {
+    if (K == 1) {
+      const int x = a.idx_in ? a.idx_in[s] : a.idx_out[s];
+      const int e = (x >= 0 && x < a.E) ? x : -1;
+      if (e >= 0) {
+        const int used = a.used_in ? a.used_in[e] : 0;
+        const int r = static_cast<int>(s_before[e]) + a.loc_out[s];
+        a.loc_out[s] = r;
+        a.idx_out[s] = (r >= a.C - used) ? -1 : e;
+      } else if (!a.idx_in) {
+        a.idx_out[s] = -1;
+        a.loc_out[s] = 0;
+      }
+    } else {
+      const int e1 = a.idx_out[s], e2 = a.idx_out[a.S + s];
+      const bool in1 = e1 >= 0 && e1 < a.E, in2 = e2 >= 0 && e2 < a.E;  // always (two experts at least)
+      const int r1 = (in1 ? static_cast<int>(s_before[e1]) : 0) + a.loc_out[s];
+      const int r2 = (in2 ? static_cast<int>(s_before[a.E + e2]) : 0) + a.loc_out[a.S + s];
+      const int u1 = (a.used_in && in1) ? a.used_in[e1] : 0;
+      const int u2 = (a.used_in && in2) ? a.used_in[e2] : 0;
+      const bool keep1 = in1 && r1 < a.C - u1;
+      const int64_t after1 = min(static_cast<int64_t>(u2) + (in2 ? s_total[e2] : 0u), static_cast<int64_t>(a.C));
+      const bool keep2 = in2 && r2 < a.C - after1;
+      a.idx_out[s] = keep1 ? e1 : -1;
+      a.loc_out[s] = keep1 ? r1 : -1;
+      a.idx_out[a.S + s] = keep2 ? e2 : -1;
+      a.loc_out[a.S + s] = keep2 ? r2 + static_cast<int>(after1 - u2) : -1;
+      // the raw values as the first kernel stored them (rounded to the gate type), normalised in fp32, rounded once
+      const float g1 = keep1 ? ld_gate(a.gates_s, s, a.gate_dtype) : 0.f;
+      const float g2 = keep2 ? ld_gate(a.gates_s, static_cast<size_t>(a.S) + s, a.gate_dtype) : 0.f;
+      const float den = fmaxf(g1 + g2, 1.1920929e-07f);
+      st_gate(a.gates_s, s, g1 / den, a.gate_dtype);
+      st_gate(a.gates_s, static_cast<size_t>(a.S) + s, g2 / den, a.gate_dtype);
+    }
+  }
+  if (tile == 0) {
+    for (int c = threadIdx.x; c < a.E; c += kTile) {
+      const int64_t used = a.used_in ? a.used_in[c] : 0;
+      const int64_t total = static_cast<int64_t>(s_total[c]) + (K == 2 ? s_total[a.E + c] : 0u);
+      const int64_t uo = min(used + total, static_cast<int64_t>(a.C));
+      a.used_out[c] = static_cast<int32_t>(uo);
+      a.elems_out[c] = static_cast<uint64_t>((uo - used) * a.M);
+    }
+  }
+}
+
 // Completes top-2 routing once all tiles are done: slot 1 is an ordinary top-1 encode with
 // used_in; slot 2 is a top-1 encode whose used capacity is slot 1's result; locations are in
 // the merged layout (slot-2 rows follow slot-1 rows of the same expert); combine weights are
@@ -628,6 +738,22 @@ hipError_t run_route_scan(const void* gate, const void* noise, const int32_t* id
   a.ws = scan_ws_view(ws);
   hipError_t err = hipSuccess;
   const size_t lds = scan_lds_bytes(K * E);
+  if (use_count_place(a.ntiles, static_cast<int64_t>(K) * E, K)) {
+    // two kernels that wait for nothing instead of a look-back between tiles that all run at once
+    const size_t lds2 = 2 * static_cast<size_t>(K) * E * sizeof(uint32_t);
+    if (K == 1) {
+      LANCET_GATE_SWITCH(gate_dtype, (route_count_kernel<1, GD><<<a.ntiles, kTile, lds, st>>>(a)))
+      err = hipGetLastError();
+      if (err != hipSuccess) return err;
+      route_place_kernel<1><<<a.ntiles, kTile, lds2, st>>>(a);
+    } else {
+      LANCET_GATE_SWITCH(gate_dtype, (route_count_kernel<2, GD><<<a.ntiles, kTile, lds, st>>>(a)))
+      err = hipGetLastError();
+      if (err != hipSuccess) return err;
+      route_place_kernel<2><<<a.ntiles, kTile, lds2, st>>>(a);
+    }
+    return hipGetLastError();
+  }
   if (K == 1) {
     LANCET_GATE_SWITCH(gate_dtype, (route_scan_kernel<1, GD><<<a.ntiles, kTile, lds, st>>>(a)))
   } else {

@@ -207,7 +207,10 @@ constexpr int kLookbackLoads = 8;
 // cls[j] < 0); s_cnt row 5 holds the tile's exclusive base and row 4 its aggregate.
 // Returns true when the tile is poisoned (a wait gave up here or in a tile it builds on): its ranks mean
 // nothing.  Must be called from uniform control flow by all kTile threads.
-template <int NSETS>
+// LOOKBACK = false: the first two levels only.  rank[j] is then the rank inside the tile, row 4 of s_cnt the
+// tile's counts, and neither `me` nor the descriptor table is touched: the caller stores the counts
+// (store_tile_counts) and a second kernel adds what the earlier tiles counted (sum_tile_counts).
+template <int NSETS, bool LOOKBACK = true>
 __device__ __forceinline__ bool tile_scan(const int (&cls)[NSETS], const bool (&mem)[NSETS], int E,
                                           const TileStart& me, const ScanWs& ws, uint32_t* s_cnt,
                                           uint32_t (&rank)[NSETS]) {
@@ -253,11 +256,12 @@ __device__ __forceinline__ bool tile_scan(const int (&cls)[NSETS], const bool (&
       run += t;
     }
     s_agg[c] = run;
-    st_desc(ws.desc + static_cast<size_t>(tile) * NC + c, me.epoch, (tile == 0 ? kDescInclusive : kDescAggregate) | run);
+    if (LOOKBACK)
+      st_desc(ws.desc + static_cast<size_t>(tile) * NC + c, me.epoch, (tile == 0 ? kDescInclusive : kDescAggregate) | run);
   }
 
   // 3. decoupled look-back
-  if (tile > 0) {
+  if (LOOKBACK && tile > 0) {
     if (tid == 0) s_open = NC;
     for (int c = tid; c < NC; c += kTile) s_stop[c] = 0xffffffffu;
     __syncthreads();
@@ -341,6 +345,124 @@ __device__ __forceinline__ bool tile_scan(const int (&cls)[NSETS], const bool (&
     rank[j] = (cls[j] >= 0) ? s_base[c] + s_cnt[w * NC + c] + wrank[j] : 0u;
   }
   return s_poison != 0;
+}
+
+// ---- two kernels instead of a look-back -------------------------------------------------------------------
+// When the tiles of a launch all run at once no inclusive prefix exists until the first tiles finish, and the
+// look-back degenerates into a chain of memory round trips from tile to tile (8 of the 21 us of a 256-tile
+// launch, and still 70 us at 1024 tiles).  Unless the batch is very long the scan is therefore cut in two
+// kernels that wait for nothing: the first stores every tile's counts, the second lets every tile add up the
+// counts of the tiles before it (and of all tiles: the totals) with plain loads, eight in flight per thread.
+// A tile's counts are stored two to a 64-bit word, the high half tagged "not a descriptor", so that the
+// workspace keeps its property that no word of it can pass for a descriptor of a later look-back launch.
+// Reading all rows costs T * NC words per tile, quadratic in the tile count T: measured faster than the look-back
+// up to 1024 tiles x 64 counters (41 against 70 us) and 2048 x 16 (31 against 87 us), slower beyond
+// T * NC of about 100k, where the launch keeps the look-back.
+constexpr int64_t kCountPlaceMaxWork = 98304;  // tiles x counters
+__host__ inline bool use_count_place(int64_t ntiles, int64_t ncounters, int nsets) {
+  // one counter set and few tiles: the look-back is a single short kernel
+  return ntiles * ncounters <= kCountPlaceMaxWork && (nsets > 1 || ntiles > 32);
+}
+
+__host__ __device__ inline int count_pairs(int ncounters) { return (ncounters + 1) / 2; }
+
+// after tile_scan<NSETS, false>: row 4 of s_cnt -> the tile's row of the table
+__device__ __forceinline__ void store_tile_counts(const ScanWs& ws, uint32_t tile, int NC, const uint32_t* s_cnt) {
+  const uint32_t* s_agg = s_cnt + kWavesPerTile * NC;
+  const int PP = count_pairs(NC);
+  for (int q = threadIdx.x; q < PP; q += kTile) {
+    const uint32_t lo = s_agg[2 * q], hi = (2 * q + 1 < NC) ? s_agg[2 * q + 1] : 0u;
+    ws.desc[static_cast<size_t>(tile) * PP + q] = foreign_word(hi, lo);
+  }
+}
+
+// s_before[c] = counts of tiles [0, tile), s_total[c] = counts of all ntiles tiles (LDS, NC words each, zeroed
+// here).  Uniform control flow, all kTile threads; the table was written by an earlier kernel.
+__device__ __forceinline__ void sum_tile_counts(const ScanWs& ws, uint32_t tile, int ntiles, int NC, uint32_t* s_before,
+                                                uint32_t* s_total) {
+  const int PP = count_pairs(NC);
+  for (int c = threadIdx.x; c < NC; c += kTile) s_before[c] = s_total[c] = 0u;
+  __syncthreads();
+  const int n = ntiles * PP;
+  const int dl = kTile / PP, dc = kTile - dl * PP;
+  int row = static_cast<int>(threadIdx.x) / PP, q = static_cast<int>(threadIdx.x) - row * PP;
+  if (PP > kTile && PP % kTile == 0 && PP / kTile <= 2) {
+    // two pairs per thread and row (more than 256 pairs: several hundred experts)
+    uint32_t tl[2] = {0, 0}, th[2] = {0, 0}, bl[2] = {0, 0}, bh[2] = {0, 0};
+    constexpr int kRows = 4;  // rows in flight per thread
+    int r = 0;
+    for (; r < ntiles; r += kRows) {
+      uint64_t w[kRows][2];
+#pragma unroll
+      for (int k = 0; k < kRows; ++k)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          w[k][j] = (r + k < ntiles) ? ws.desc[static_cast<size_t>(r + k) * PP + threadIdx.x + j * kTile] : 0ull;
+#pragma unroll
+      for (int k = 0; k < kRows; ++k)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const uint32_t lo = static_cast<uint32_t>(w[k][j]), hi = static_cast<uint32_t>(w[k][j] >> 32) & kEpochMask;
+          tl[j] += lo, th[j] += hi;
+          if (r + k < static_cast<int>(tile)) bl[j] += lo, bh[j] += hi;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int c = 2 * (static_cast<int>(threadIdx.x) + j * kTile);
+      s_total[c] = tl[j], s_before[c] = bl[j];
+      if (c + 1 < NC) s_total[c + 1] = th[j], s_before[c + 1] = bh[j];
+    }
+    __syncthreads();
+    return;
+  }
+  if (dc == 0) {
+    // the pairs of a row divide the workgroup: a thread meets the same pair in every row it reads, adds up in
+    // registers and goes to LDS once
+    uint32_t tl = 0, th = 0, bl = 0, bh = 0;
+    constexpr int kBatch = 8;  // loads in flight per thread (one at a time would be a chain of round trips)
+    int i = threadIdx.x;
+    for (; i + (kBatch - 1) * kTile < n; i += kBatch * kTile) {
+      uint64_t w[kBatch];
+#pragma unroll
+      for (int k = 0; k < kBatch; ++k) w[k] = ws.desc[i + k * kTile];
+#pragma unroll
+      for (int k = 0; k < kBatch; ++k) {
+        const uint32_t lo = static_cast<uint32_t>(w[k]), hi = static_cast<uint32_t>(w[k] >> 32) & kEpochMask;
+        tl += lo, th += hi;
+        if (row + k * dl < static_cast<int>(tile)) bl += lo, bh += hi;
+      }
+      row += kBatch * dl;
+    }
+    for (; i < n; i += kTile) {
+      const uint64_t w = ws.desc[i];
+      const uint32_t lo = static_cast<uint32_t>(w), hi = static_cast<uint32_t>(w >> 32) & kEpochMask;
+      tl += lo, th += hi;
+      if (row < static_cast<int>(tile)) bl += lo, bh += hi;
+      row += dl;
+    }
+    if (tl) atomicAdd(&s_total[2 * q], tl);
+    if (th) atomicAdd(&s_total[2 * q + 1], th);
+    if (bl) atomicAdd(&s_before[2 * q], bl);
+    if (bh) atomicAdd(&s_before[2 * q + 1], bh);
+    __syncthreads();
+    return;
+  }
+  for (int i = threadIdx.x; i < n; i += kTile) {
+    const uint64_t w = ws.desc[i];
+    const uint32_t lo = static_cast<uint32_t>(w), hi = static_cast<uint32_t>(w >> 32) & kEpochMask;
+    if (lo) {
+      atomicAdd(&s_total[2 * q], lo);
+      if (row < static_cast<int>(tile)) atomicAdd(&s_before[2 * q], lo);
+    }
+    if (hi) {
+      atomicAdd(&s_total[2 * q + 1], hi);
+      if (row < static_cast<int>(tile)) atomicAdd(&s_before[2 * q + 1], hi);
+    }
+    row += dl, q += dc;
+    if (q >= PP) q -= PP, row += 1;
+  }
+  __syncthreads();
 }
 
 }  // namespace lancet

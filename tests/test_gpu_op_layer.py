@@ -103,11 +103,11 @@ def test_plain_c_client_of_the_c_abi():
 
 def test_op_layer_reports_a_scan_that_gave_up(pkg, ex):
     """A prepared call keeps its OpEnv and workspace across runs (RAF's interpreter cache): the workspace is set up
-    by the first run only; with a wait bound of one poll the scan gives up somewhere in 256 tiles, the outputs carry
+    by the first run only; with a wait bound of one poll the scan gives up somewhere in 512 tiles, the outputs carry
     the marks, and check() raises where the reference would have aborted; the next run is whole again."""
     import ctypes as C
     lib = pkg.capi.load()
-    S, M, E = 65536, 8, 8
+    S, M, E = 131072, 8, 256         # 512 tiles x 256 counters: the scan with the look-back (smaller launches take a form without waits)
     data, logits = make_inputs(13, S, M, E)
     gate = mo.softmax_rows(logits)
     want = mo.moe_encode(data, gate, np.zeros(E, np.int32), 1.0, fast_scatter=True)

@@ -18,12 +18,21 @@ from . import capi
 _DTYPES = {torch.float32: capi.F32, torch.bfloat16: capi.BF16, torch.float16: capi.F16}
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream():
-    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    """Handle of the current device's current stream, as the integer a void* argument takes.  A small call costs
+    about as much on the host as on the device, so this goes straight to torch's C entry points where they exist."""
+    if _raw_stream is not None and _raw_device is not None:
+        return _raw_stream(_raw_device())
+    return torch.cuda.current_stream().cuda_stream
 
 
 def _p(t):
-    return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(None)
+    """Device address of a tensor (None = null pointer); the typed entry points of capi take it as void*."""
+    return t.data_ptr() if t is not None else None
 
 
 def _dtype_code(t):
@@ -98,8 +107,8 @@ def _scan_workspace(nbytes, device, given):
         _need(given.buf.device == device and given.nbytes >= nbytes,
               "workspace must live on the data's GPU and hold at least %d bytes" % nbytes)
         return given
-    key = (device.index if device.index is not None else torch.cuda.current_device(),
-           torch.cuda.current_stream(device).cuda_stream)
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    key = (idx, _raw_stream(idx) if _raw_stream is not None else torch.cuda.current_stream(device).cuda_stream)
     ws = _scan_pool.get(key)
     if ws is None or ws.nbytes < nbytes:
         with torch.cuda.device(device):

@@ -185,6 +185,10 @@ def test_top2_equals_two_chained_top1_encodes(pkg):
     (1024, 512, 16, 4, 4.0, False),                                    # test_cuda_moe.py:1316
     (2000, 16, 8, 1, 0.5, True), (1536, 8, 6, 3, 1.5, True), (4096, 8, 64, 4, 2.0, False),
     (700, 4, 3, 1, 5.0, False),                                        # nothing dropped
+    # more keys per expert than the select kernel keeps on chip (10240): it fetches them again in every pass
+    (36000, 4, 2, 1, 0.5, False), (40000, 4, 2, 4, 0.75, True),
+    (19000, 4, 2, 2, 0.6, True),                                       # about that limit: one expert over, one under
+    (1050000, 2, 4, 2, 0.5, True),                                     # more than 4096 tiles: the batch is read whole
 ])
 def test_encode_bpr(pkg, S0, M, E, P, cf, ties):
     data, logits = make_inputs(S0 + P, S0, M, E, logit_scale=2.0, ties=ties)

@@ -177,7 +177,9 @@ int lancet_moe_scatter(const void* data, const int32_t* indices_locations, const
  * (:701-719) and launch_gen_location_bpr (kernel_util.cuh:65; tutel_moe_dispatch.cu:259-363).
  * data[S0,M], gate[S0,E] are the whole batch; S = S0 / n_partitions tokens of partition
  * partition_id are encoded.  The per-expert keep set is the C best tokens by
- * (gate value descending, token index ascending), found with a radix select, not a sort. */
+ * (gate value descending, token index ascending), found with a radix select, not a sort.
+ * The workspace holds, behind the scan's table, 16 bytes per token of the batch (first choice and priority; the
+ * order keys of each tile of 256 tokens grouped by expert) and 8 bytes per (expert, tile of the batch). */
 size_t lancet_moe_encode_bpr_workspace_bytes(int64_t S0, int64_t E, int n_partitions);
 int lancet_moe_encode_bpr(const void* data, const void* gate, int64_t S0, int64_t M, int64_t E,
                           int64_t C, int n_partitions, int partition_id, int dtype, int gate_dtype, unsigned flags,

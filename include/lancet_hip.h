@@ -415,7 +415,7 @@ int lancet_lans_plan_norms(lancet_lans_plan_t plan, float* norms4xT, lancet_stre
  * launch on clearing it.  A call that is handed a workspace that is not set up launches nothing harmful:
  * it sets every indices/locations entry and every used_out entry to -1 and the error word.
  * The scan has two forms and a call picks one by its size.  Short and moderately long batches (tiles of 256
- * tokens x counters up to about 100k, e.g. 262144 tokens x 32 experts x top-2) run as two kernels in which no
+ * tokens x counters up to 131072, e.g. 524288 tokens x 32 experts x top-2) run as two kernels in which no
  * workgroup waits for another: they use the workspace as plain scratch (no state, no wait that could give up,
  * and memory that was never set up works as well).  Longer batches, and top-1 calls of at most 32 tiles (8192
  * tokens), run as one kernel with a look-back between tiles, to which everything said here about state and

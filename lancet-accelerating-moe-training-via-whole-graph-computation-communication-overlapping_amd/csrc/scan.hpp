@@ -355,10 +355,12 @@ __device__ __forceinline__ bool tile_scan(const int (&cls)[NSETS], const bool (&
 // counts of the tiles before it (and of all tiles: the totals) with plain loads, eight in flight per thread.
 // A tile's counts are stored two to a 64-bit word, the high half tagged "not a descriptor", so that the
 // workspace keeps its property that no word of it can pass for a descriptor of a later look-back launch.
-// Reading all rows costs T * NC words per tile, quadratic in the tile count T: measured faster than the look-back
-// up to 1024 tiles x 64 counters (41 against 70 us) and 2048 x 16 (31 against 87 us), slower beyond
-// T * NC of about 100k, where the launch keeps the look-back.
-constexpr int64_t kCountPlaceMaxWork = 98304;  // tiles x counters
+// Reading all rows costs T * NC words per tile, quadratic in the tile count T.  Measured against the look-back
+// (routing of T tiles x NC counters, us): 256 x 64: 14.5 / 23; 1024 x 64: 41 / 70; 2048 x 16: 31 / 87; at
+// T * NC = 131072 it still wins everywhere (256 x 512: 58 / 72; 1024 x 128: 89 / 108; 2048 x 64: 271 / 308;
+// 8192 x 16: 272 / 467); at 262144 it loses (512 x 512: 151 / 118; 4096 x 64: 700 / 622; 1024 x 256: 371 / 274),
+// so the launch keeps the look-back beyond 131072.
+constexpr int64_t kCountPlaceMaxWork = 131072;  // tiles x counters
 __host__ inline bool use_count_place(int64_t ntiles, int64_t ncounters, int nsets) {
   // one counter set and few tiles: the look-back is a single short kernel
   return ntiles * ncounters <= kCountPlaceMaxWork && (nsets > 1 || ntiles > 32);

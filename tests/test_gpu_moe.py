@@ -305,7 +305,7 @@ def test_bounded_wait_flags_the_workspace(pkg, k):
     import ctypes as C
     lib = pkg.capi.load()
     ops = pkg.ops
-    S, M, E = 131072, 4, 256         # 512 tiles x 256 counters: a launch that takes the look-back form of the scan
+    S, M, E = 131072, 4, 512         # 512 tiles x 512 or 1024 counters: a launch that takes the look-back form of the scan
     data, logits = make_inputs(1, S, M, E)
     d_data, d_gate = dev(data), dev(logits)
     enc = mo.moe_encode_top2 if k == 2 else mo.moe_encode

@@ -102,17 +102,17 @@ def test_routing_over_many_tiles(pkg, S, E, k, cf, skew):
     np.testing.assert_array_equal(to_np(got[4]), want[4])
 
 
-# tiles x counters at most 98304: two kernels without waits (unless one counter set on at most 32 tiles); beyond: look-back
+# tiles x counters at most 131072: two kernels without waits (unless one counter set on at most 32 tiles); beyond: look-back
 @pytest.mark.parametrize("S,E,k,cf,skew", [
-    (24576, 512, 2, 1.0, 2.0),    # 96 tiles x 1024 counters = the limit: two pairs of counters per thread and row
-    (24577, 512, 2, 1.0, 2.0),    # one tile more: look-back
+    (32768, 512, 2, 1.0, 2.0),    # 128 tiles x 1024 counters = the limit: two pairs of counters per thread and row
+    (32769, 512, 2, 1.0, 2.0),    # one tile more: look-back
     (49152, 256, 2, 0.5, 3.0),    # 192 x 512: one pair per thread, rows read eight at a time
     (8448, 100, 1, 1.5, 1.0),     # 33 tiles, 50 pairs (do not divide the workgroup: sums through LDS atomics)
     (8192, 100, 1, 1.5, 1.0),     # 32 tiles, one set: look-back
     (20000, 64, 1, 0.7, 2.0),     # 79 x 64: 32 pairs, several rows per thread and a remainder
     (9000, 7, 1, 1.0, 0.0),       # odd counter count: the last pair's high half is empty
     (5000, 3, 2, 1.0, 0.0), (300, 2, 2, 2.0, 0.0), (1, 2, 2, 1.0, 0.0),
-    (786432, 16, 1, 1.0, 1.0),    # 3072 tiles x 16 = 49152: the longest batch that still takes the two-kernel form
+    (786432, 16, 1, 1.0, 1.0),    # 3072 tiles x 16: more tiles than run at once, still the two-kernel form
 ])
 def test_both_forms_of_the_scan_at_their_boundaries(pkg, S, E, k, cf, skew):
     test_routing_over_many_tiles(pkg, S, E, k, cf, skew)

@@ -107,7 +107,7 @@ def test_op_layer_reports_a_scan_that_gave_up(pkg, ex):
     the marks, and check() raises where the reference would have aborted; the next run is whole again."""
     import ctypes as C
     lib = pkg.capi.load()
-    S, M, E = 131072, 8, 256         # 512 tiles x 256 counters: the scan with the look-back (smaller launches take a form without waits)
+    S, M, E = 131072, 8, 512         # 512 tiles x 512 counters: the scan with the look-back (smaller launches take a form without waits)
     data, logits = make_inputs(13, S, M, E)
     gate = mo.softmax_rows(logits)
     want = mo.moe_encode(data, gate, np.zeros(E, np.int32), 1.0, fast_scatter=True)

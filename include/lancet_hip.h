@@ -81,6 +81,11 @@ extern "C" {
  * (reference: redispatch_kernel, tutel_moe_dispatch.cu:365-408), without that second pass over the rows.
  * indices_locations are unchanged (locations stay relative to the call, as moe_merge_masks expects). */
 #define LANCET_ROWS_AT_USED 8u
+/* lancet_moe_encode / lancet_moe_route / lancet_moe_encode_bpr: run the position scan as ONE kernel with a
+ * decoupled look-back between its tiles, whatever the size.  By default only top-1 calls of at most 8192 tokens
+ * do; everything else is faster as two or three kernels in which no workgroup waits for another.  For callers
+ * that want the fewest launches, and for tests of the look-back's bounded waits. */
+#define LANCET_SCAN_LOOKBACK 16u
 
 typedef void* lancet_stream_t;
 
@@ -414,12 +419,11 @@ int lancet_lans_plan_norms(lancet_lans_plan_t plan, float* norms4xT, lancet_stre
  * allocation; every call that uses the workspace leaves it ready for the next, so that no call spends a
  * launch on clearing it.  A call that is handed a workspace that is not set up launches nothing harmful:
  * it sets every indices/locations entry and every used_out entry to -1 and the error word.
- * The scan has two forms and a call picks one by its size.  Short and moderately long batches (tiles of 256
- * tokens x counters up to 131072, e.g. 524288 tokens x 32 experts x top-2) run as two kernels in which no
- * workgroup waits for another: they use the workspace as plain scratch (no state, no wait that could give up,
- * and memory that was never set up works as well).  Longer batches, and top-1 calls of at most 32 tiles (8192
- * tokens), run as one kernel with a look-back between tiles, to which everything said here about state and
- * waits applies.
+ * The scan has two forms and a call picks one by its size.  Top-1 calls of at most 32 tiles of 256 tokens
+ * (8192 tokens), and calls with LANCET_SCAN_LOOKBACK, run as one kernel with a look-back between tiles, to which
+ * everything said here about state and waits applies.  All others run as two kernels (three on long batches: tiles
+ * x counters above 32768) in which no workgroup waits for another: they use the workspace as plain scratch (no
+ * state, no wait that could give up, and memory that was never set up works as well).
  * Every wait inside the scan is bounded.  A wait that gives up sets the workspace's sticky error word, and
  * every token whose position was built on it gets indices = locations = -1 (gates_s 0 for top_k = 2), as if
  * dropped, so that no consumer moves a row on a wrong position; when the totals themselves were built on it,

@@ -15,6 +15,7 @@ NO_TAIL_ZERO = 2
 ABI_VERSION = 6
 ZERO_TAIL = 4
 ROWS_AT_USED = 8
+SCAN_LOOKBACK = 16
 LANS_SWEEPS, LANS_RESIDENT = 0, 1
 MAX_EXPERTS = 512
 MAX_PARTITIONS = 64

@@ -233,7 +233,7 @@ extern "C" int lancet_moe_route(const void* gate, const void* gate2_noise, const
   return rc(run_route_scan(gate, gate2_noise, nullptr, used_in, s, static_cast<int>(E), static_cast<int>(C),
                            static_cast<int>(M), top_k, (flags & LANCET_GATE_IS_LOGITS) != 0, gate_dtype, gates_s,
                            indices_locations, indices_locations + static_cast<size_t>(top_k) * s, used_out,
-                           elements_per_expert, workspace, S_(stream)));
+                           elements_per_expert, workspace, S_(stream), (flags & LANCET_SCAN_LOOKBACK) != 0));
 }
 
 extern "C" int lancet_moe_scatter(const void* data, const int32_t* indices_locations, const int32_t* used_in,
@@ -363,7 +363,7 @@ extern "C" int lancet_moe_encode_bpr(const void* data, const void* gate, int64_t
   int32_t* loc = indices_locations + s;
   hipError_t e = run_bpr_route(gate, s0, static_cast<int>(E), static_cast<int>(C), static_cast<int>(M),
                                n_partitions, partition_id, (flags & LANCET_GATE_IS_LOGITS) != 0, gate_dtype, gates_s, idx,
-                               loc, used_out, elements_per_expert, workspace, S_(stream));
+                               loc, used_out, elements_per_expert, workspace, S_(stream), (flags & LANCET_SCAN_LOOKBACK) != 0);
   if (e != hipSuccess) return rc(e);
   const char* part = static_cast<const char*>(data) + static_cast<size_t>(partition_id) * s * M * eb;
   return rc(run_scatter_rows(part, dispatched, idx, loc, nullptr, nullptr, nullptr,

@@ -30,11 +30,11 @@ hipError_t run_gate_topk(const void* gate, const void* noise, int S, int E, int 
 hipError_t run_route_scan(const void* gate, const void* noise, const int32_t* idx_in, const int32_t* used_in, int S,
                           int E, int C, int M, int K, bool is_logits, int gate_dtype, void* gates_s,
                           int32_t* idx_out, int32_t* loc_out, int32_t* used_out,
-                          uint64_t* elems_out, void* ws, hipStream_t st);
+                          uint64_t* elems_out, void* ws, hipStream_t st, bool force_lookback = false);
 hipError_t run_bpr_route(const void* gate, int S0, int E, int C, int M, int n_partitions,
                          int partition_id, bool is_logits, int gate_dtype, void* gates_s, int32_t* idx_out,
                          int32_t* loc_out, int32_t* used_out, uint64_t* elems_out, void* ws,
-                         hipStream_t st);
+                         hipStream_t st, bool force_lookback = false);
 hipError_t run_top2_normalize(const void* raw, const int32_t* idx, int S, int gate_dtype, void* out, hipStream_t st);
 
 // ---- row movers (moe_rows.hip) ------------------------------------------------------

@@ -151,6 +151,7 @@ struct RouteArgs {
   int ntiles;
   int is_logits;
   int gate_dtype;         // LANCET_F32 / _BF16 / _F16: storage type of gate, noise and gates_s
+  int seg_rows;           // place kernel: tiles per segment of the segment sums, 0 = there are none
 };
 
 // K = 1: everything is final when the tile knows its prefix.
@@ -257,7 +258,7 @@ __global__ __launch_bounds__(kTile) void route_scan_kernel(RouteArgs a) {
   tile_end(a.ws, me, a.ntiles, K * a.E);
 }
 
-// ---- the same routing as two kernels that wait for nothing (use_count_place) -----------------------------------
+// ---- the same routing as two or three kernels that wait for nothing (scan_form) ------------------------------
 // route_count_kernel: selection, ranks inside the tile, the tile's counts -> table.  Leaves expert, rank inside the
 // tile and raw gate value in idx_out / loc_out / gates_s (idx_out is not written when the experts are given).
 template <int K, int GD>
@@ -319,7 +320,7 @@ __global__ __launch_bounds__(kTile) void route_place_kernel(RouteArgs a) {
   uint32_t* s_before = s_sum;
   uint32_t* s_total = s_sum + NC;
   const uint32_t tile = blockIdx.x;
-  sum_tile_counts(a.ws, tile, a.ntiles, NC, s_before, s_total);
+  sum_tile_counts(a.ws, tile, a.ntiles, NC, a.seg_rows, s_before, s_total);
   const int s = static_cast<int>(tile) * kTile + threadIdx.x;
   if (s < a.S) {
     if (K == 1) {
@@ -365,6 +366,12 @@ __global__ __launch_bounds__(kTile) void route_place_kernel(RouteArgs a) {
       a.elems_out[c] = static_cast<uint64_t>((uo - used) * a.M);
     }
   }
+}
+
+// Between count and place on long batches: one workgroup per segment of R tiles adds up the segment's rows.
+__global__ __launch_bounds__(kTile) void scan_segsum_kernel(ScanWs ws, int ntiles, int NC, int R) {
+  extern __shared__ uint32_t s_sum[];  // [NC]
+  tile_segsum(ws, blockIdx.x, ntiles, NC, R, s_sum);
 }
 
 // Completes top-2 routing once all tiles are done: slot 1 is an ordinary top-1 encode with
@@ -489,6 +496,7 @@ struct BprArgs {
   int S0, S, E, C, M;
   int part_lo;           // first token of the partition
   int ntiles;
+  int seg_rows;          // place kernel: tiles per segment of the segment sums, 0 = there are none
   int gate_dtype;        // storage type of gates_s (and of the gate the priorities came from)
   void* gates_s;         // [S]
   int32_t* idx_out;      // [S]
@@ -812,7 +820,7 @@ __global__ __launch_bounds__(kTile) void bpr_scan_kernel(BprArgs a) {
   tile_end(a.ws, me, a.ntiles, 2 * a.E);
 }
 
-// ---- the same scan as two kernels that wait for nothing (use_count_place) --------------------------------------
+// ---- the same scan as two or three kernels that wait for nothing (scan_form) ---------------------------------
 // class and membership of a partition token in the two counter sets, from its word and the expert's threshold
 struct BprClass {
   int e;        // expert, -1 = none
@@ -866,7 +874,7 @@ __global__ __launch_bounds__(kTile) void bpr_place_kernel(BprArgs a) {
   uint32_t* s_before = s_sum;
   uint32_t* s_total = s_sum + NC;
   const uint32_t tile = blockIdx.x;
-  sum_tile_counts(a.ws, tile, a.ntiles, NC, s_before, s_total);
+  sum_tile_counts(a.ws, tile, a.ntiles, NC, a.seg_rows, s_before, s_total);
   const int sl = static_cast<int>(tile) * kTile + threadIdx.x;
   if (sl < a.S) {
     const BprClass c = bpr_classify(a, sl);
@@ -904,7 +912,9 @@ __global__ __launch_bounds__(kTile) void bpr_place_kernel(BprArgs a) {
 int64_t scan_num_tiles(int64_t S) { return S > 0 ? (S + kTile - 1) / kTile : 1; }
 
 size_t scan_workspace_bytes(int64_t S, int64_t E, int nsets) {
-  return scan_ws_bytes(scan_num_tiles(S), nsets * E);
+  // (two words per tile at least: the forms without look-back keep the tiles' counts, two to a word, and the
+  // segments' sums in the room of the look-back's table)
+  return scan_ws_bytes(scan_num_tiles(S), std::max<int64_t>(nsets * E, 2));
 }
 
 size_t bpr_workspace_bytes(int64_t S0, int64_t S, int64_t E) {
@@ -963,7 +973,7 @@ hipError_t run_gate_topk(const void* gate, const void* noise, int S, int E, int 
 hipError_t run_route_scan(const void* gate, const void* noise, const int32_t* idx_in, const int32_t* used_in, int S,
                           int E, int C, int M, int K, bool is_logits, int gate_dtype, void* gates_s,
                           int32_t* idx_out, int32_t* loc_out, int32_t* used_out,
-                          uint64_t* elems_out, void* ws, hipStream_t st) {
+                          uint64_t* elems_out, void* ws, hipStream_t st, bool force_lookback) {
   RouteArgs a;
   a.gate = gate;
   a.noise = K == 2 ? noise : nullptr;
@@ -982,22 +992,29 @@ hipError_t run_route_scan(const void* gate, const void* noise, const int32_t* id
   a.is_logits = is_logits;
   a.gate_dtype = gate_dtype;
   a.ws = scan_ws_view(ws);
+  a.seg_rows = 0;
   hipError_t err = hipSuccess;
   const size_t lds = scan_lds_bytes(K * E);
-  if (use_count_place(a.ntiles, static_cast<int64_t>(K) * E, K)) {
-    // two kernels that wait for nothing instead of a look-back between tiles that all run at once
-    const size_t lds2 = 2 * static_cast<size_t>(K) * E * sizeof(uint32_t);
+  const ScanForm form = scan_form(a.ntiles, static_cast<int64_t>(K) * E, K, force_lookback);
+  if (form != kScanLookback) {
+    // two or three kernels that wait for nothing instead of a look-back between tiles that all run at once
+    const int NC = K * E;
+    const size_t lds2 = 2 * static_cast<size_t>(NC) * sizeof(uint32_t);
     if (K == 1) {
       LANCET_GATE_SWITCH(gate_dtype, (route_count_kernel<1, GD><<<a.ntiles, kTile, lds, st>>>(a)))
-      err = hipGetLastError();
-      if (err != hipSuccess) return err;
-      route_place_kernel<1><<<a.ntiles, kTile, lds2, st>>>(a);
     } else {
       LANCET_GATE_SWITCH(gate_dtype, (route_count_kernel<2, GD><<<a.ntiles, kTile, lds, st>>>(a)))
+    }
+    err = hipGetLastError();
+    if (err != hipSuccess) return err;
+    if (form == kScanCountSegPlace) {
+      a.seg_rows = seg_rows(a.ntiles);
+      scan_segsum_kernel<<<(a.ntiles + a.seg_rows - 1) / a.seg_rows, kTile, NC * sizeof(uint32_t), st>>>(a.ws, a.ntiles, NC, a.seg_rows);
       err = hipGetLastError();
       if (err != hipSuccess) return err;
-      route_place_kernel<2><<<a.ntiles, kTile, lds2, st>>>(a);
     }
+    if (K == 1) route_place_kernel<1><<<a.ntiles, kTile, lds2, st>>>(a);
+    else route_place_kernel<2><<<a.ntiles, kTile, lds2, st>>>(a);
     return hipGetLastError();
   }
   if (K == 1) {
@@ -1014,7 +1031,7 @@ hipError_t run_route_scan(const void* gate, const void* noise, const int32_t* id
 hipError_t run_bpr_route(const void* gate, int S0, int E, int C, int M, int n_partitions,
                          int partition_id, bool is_logits, int gate_dtype, void* gates_s, int32_t* idx_out,
                          int32_t* loc_out, int32_t* used_out, uint64_t* elems_out, void* ws,
-                         hipStream_t st) {
+                         hipStream_t st, bool force_lookback) {
   const int S = S0 / n_partitions;
   BprArgs a;
   a.S0 = S0;
@@ -1025,7 +1042,7 @@ hipError_t run_bpr_route(const void* gate, int S0, int E, int C, int M, int n_pa
   a.part_lo = partition_id * S;
   a.ntiles = static_cast<int>(scan_num_tiles(S));
   a.ws = scan_ws_view(ws);
-  a.tok = reinterpret_cast<uint64_t*>(static_cast<char*>(ws) + scan_ws_bytes(a.ntiles, 2 * E));
+  a.tok = reinterpret_cast<uint64_t*>(static_cast<char*>(ws) + scan_workspace_bytes(S, E, 2));
   a.par = a.tok + S0;
   a.ntiles0 = static_cast<int>(scan_num_tiles(S0));
   a.keys = a.par + 4 * static_cast<size_t>(E);
@@ -1044,10 +1061,18 @@ hipError_t run_bpr_route(const void* gate, int S0, int E, int C, int M, int n_pa
   bpr_select_kernel<<<E, kSelectThreads, 0, st>>>(a);
   err = hipGetLastError();
   if (err != hipSuccess) return err;
-  if (use_count_place(a.ntiles, 2 * static_cast<int64_t>(E), 2)) {
+  a.seg_rows = 0;
+  const ScanForm form = scan_form(a.ntiles, 2 * static_cast<int64_t>(E), 2, force_lookback);
+  if (form != kScanLookback) {
     bpr_count_kernel<<<a.ntiles, kTile, scan_lds_bytes(2 * E), st>>>(a);
     err = hipGetLastError();
     if (err != hipSuccess) return err;
+    if (form == kScanCountSegPlace) {
+      a.seg_rows = seg_rows(a.ntiles);
+      scan_segsum_kernel<<<(a.ntiles + a.seg_rows - 1) / a.seg_rows, kTile, 2 * E * sizeof(uint32_t), st>>>(a.ws, a.ntiles, 2 * E, a.seg_rows);
+      err = hipGetLastError();
+      if (err != hipSuccess) return err;
+    }
     bpr_place_kernel<<<a.ntiles, kTile, 4 * static_cast<size_t>(E) * sizeof(uint32_t), st>>>(a);
     return hipGetLastError();
   }

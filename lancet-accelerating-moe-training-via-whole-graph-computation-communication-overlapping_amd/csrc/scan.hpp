@@ -360,10 +360,23 @@ __device__ __forceinline__ bool tile_scan(const int (&cls)[NSETS], const bool (&
 // T * NC = 131072 it still wins everywhere (256 x 512: 58 / 72; 1024 x 128: 89 / 108; 2048 x 64: 271 / 308;
 // 8192 x 16: 272 / 467); at 262144 it loses (512 x 512: 151 / 118; 4096 x 64: 700 / 622; 1024 x 256: 371 / 274),
 // so the launch keeps the look-back beyond 131072.
-constexpr int64_t kCountPlaceMaxWork = 131072;  // tiles x counters
-__host__ inline bool use_count_place(int64_t ntiles, int64_t ncounters, int nsets) {
+// The third form, for long batches: adding up ALL rows in every tile is quadratic in the tile count, so a kernel
+// between the two adds the rows up in segments of R consecutive tiles (R about the square root of the tile
+// count), and a tile then reads the sums of the segments before its own and the rows of its own segment before
+// itself: about 2 * sqrt(T) rows instead of T.  Three launches, still no waits and no state.
+enum ScanForm { kScanLookback = 0, kScanCountPlace = 1, kScanCountSegPlace = 2 };
+constexpr int64_t kFlatPlaceMaxWork = 32768;  // tiles x counters up to which the extra launch costs more than it saves
+__host__ inline ScanForm scan_form(int64_t ntiles, int64_t ncounters, int nsets, bool force_lookback = false) {
+  if (force_lookback) return kScanLookback;
   // one counter set and few tiles: the look-back is a single short kernel
-  return ntiles * ncounters <= kCountPlaceMaxWork && (nsets > 1 || ntiles > 32);
+  if (nsets == 1 && ntiles <= 32) return kScanLookback;
+  return ntiles * ncounters <= kFlatPlaceMaxWork ? kScanCountPlace : kScanCountSegPlace;
+}
+// rows per segment: the smallest power of two from 32 on whose square covers the tiles
+__host__ __device__ inline int seg_rows(int64_t ntiles) {
+  int r = 32;
+  while (static_cast<int64_t>(r) * r < ntiles && r < (1 << 15)) r <<= 1;
+  return r;
 }
 
 __host__ __device__ inline int count_pairs(int ncounters) { return (ncounters + 1) / 2; }
@@ -378,42 +391,46 @@ __device__ __forceinline__ void store_tile_counts(const ScanWs& ws, uint32_t til
   }
 }
 
-// s_before[c] = counts of tiles [0, tile), s_total[c] = counts of all ntiles tiles (LDS, NC words each, zeroed
-// here).  Uniform control flow, all kTile threads; the table was written by an earlier kernel.
-__device__ __forceinline__ void sum_tile_counts(const ScanWs& ws, uint32_t tile, int ntiles, int NC, uint32_t* s_before,
-                                                uint32_t* s_total) {
+// Adds up nrows rows of a table of counts (count_pairs(NC) words per row): s_total[c] += all of them (TOTAL),
+// s_before[c] += the rows below `cut`.  The caller has zeroed (or pre-loaded) both arrays and synchronised; on
+// return the sums are complete and visible.  Uniform control flow, all kTile threads; the table was written by an
+// earlier kernel.
+template <bool TOTAL>
+__device__ __forceinline__ void sum_count_rows(const uint64_t* table, int nrows, int cut, int NC, uint32_t* s_before,
+                                               uint32_t* s_total) {
   const int PP = count_pairs(NC);
-  for (int c = threadIdx.x; c < NC; c += kTile) s_before[c] = s_total[c] = 0u;
-  __syncthreads();
-  const int n = ntiles * PP;
+  const int n = nrows * PP;
   const int dl = kTile / PP, dc = kTile - dl * PP;
   int row = static_cast<int>(threadIdx.x) / PP, q = static_cast<int>(threadIdx.x) - row * PP;
   if (PP > kTile && PP % kTile == 0 && PP / kTile <= 2) {
     // two pairs per thread and row (more than 256 pairs: several hundred experts)
     uint32_t tl[2] = {0, 0}, th[2] = {0, 0}, bl[2] = {0, 0}, bh[2] = {0, 0};
     constexpr int kRows = 4;  // rows in flight per thread
-    int r = 0;
-    for (; r < ntiles; r += kRows) {
+    for (int r = 0; r < nrows; r += kRows) {
       uint64_t w[kRows][2];
 #pragma unroll
       for (int k = 0; k < kRows; ++k)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
-          w[k][j] = (r + k < ntiles) ? ws.desc[static_cast<size_t>(r + k) * PP + threadIdx.x + j * kTile] : 0ull;
+          w[k][j] = (r + k < nrows) ? table[static_cast<size_t>(r + k) * PP + threadIdx.x + j * kTile] : 0ull;
 #pragma unroll
       for (int k = 0; k < kRows; ++k)
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
           const uint32_t lo = static_cast<uint32_t>(w[k][j]), hi = static_cast<uint32_t>(w[k][j] >> 32) & kEpochMask;
           tl[j] += lo, th[j] += hi;
-          if (r + k < static_cast<int>(tile)) bl[j] += lo, bh[j] += hi;
+          if (r + k < cut) bl[j] += lo, bh[j] += hi;
         }
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int c = 2 * (static_cast<int>(threadIdx.x) + j * kTile);
-      s_total[c] = tl[j], s_before[c] = bl[j];
-      if (c + 1 < NC) s_total[c + 1] = th[j], s_before[c + 1] = bh[j];
+      const int c = 2 * (static_cast<int>(threadIdx.x) + j * kTile);  // this thread alone owns the pair
+      if (TOTAL) s_total[c] += tl[j];
+      s_before[c] += bl[j];
+      if (c + 1 < NC) {
+        if (TOTAL) s_total[c + 1] += th[j];
+        s_before[c + 1] += bh[j];
+      }
     }
     __syncthreads();
     return;
@@ -427,44 +444,80 @@ __device__ __forceinline__ void sum_tile_counts(const ScanWs& ws, uint32_t tile,
     for (; i + (kBatch - 1) * kTile < n; i += kBatch * kTile) {
       uint64_t w[kBatch];
 #pragma unroll
-      for (int k = 0; k < kBatch; ++k) w[k] = ws.desc[i + k * kTile];
+      for (int k = 0; k < kBatch; ++k) w[k] = table[i + k * kTile];
 #pragma unroll
       for (int k = 0; k < kBatch; ++k) {
         const uint32_t lo = static_cast<uint32_t>(w[k]), hi = static_cast<uint32_t>(w[k] >> 32) & kEpochMask;
         tl += lo, th += hi;
-        if (row + k * dl < static_cast<int>(tile)) bl += lo, bh += hi;
+        if (row + k * dl < cut) bl += lo, bh += hi;
       }
       row += kBatch * dl;
     }
     for (; i < n; i += kTile) {
-      const uint64_t w = ws.desc[i];
+      const uint64_t w = table[i];
       const uint32_t lo = static_cast<uint32_t>(w), hi = static_cast<uint32_t>(w >> 32) & kEpochMask;
       tl += lo, th += hi;
-      if (row < static_cast<int>(tile)) bl += lo, bh += hi;
+      if (row < cut) bl += lo, bh += hi;
       row += dl;
     }
-    if (tl) atomicAdd(&s_total[2 * q], tl);
-    if (th) atomicAdd(&s_total[2 * q + 1], th);
+    if (TOTAL && tl) atomicAdd(&s_total[2 * q], tl);
+    if (TOTAL && th) atomicAdd(&s_total[2 * q + 1], th);
     if (bl) atomicAdd(&s_before[2 * q], bl);
     if (bh) atomicAdd(&s_before[2 * q + 1], bh);
     __syncthreads();
     return;
   }
   for (int i = threadIdx.x; i < n; i += kTile) {
-    const uint64_t w = ws.desc[i];
+    const uint64_t w = table[i];
     const uint32_t lo = static_cast<uint32_t>(w), hi = static_cast<uint32_t>(w >> 32) & kEpochMask;
     if (lo) {
-      atomicAdd(&s_total[2 * q], lo);
-      if (row < static_cast<int>(tile)) atomicAdd(&s_before[2 * q], lo);
+      if (TOTAL) atomicAdd(&s_total[2 * q], lo);
+      if (row < cut) atomicAdd(&s_before[2 * q], lo);
     }
     if (hi) {
-      atomicAdd(&s_total[2 * q + 1], hi);
-      if (row < static_cast<int>(tile)) atomicAdd(&s_before[2 * q + 1], hi);
+      if (TOTAL) atomicAdd(&s_total[2 * q + 1], hi);
+      if (row < cut) atomicAdd(&s_before[2 * q + 1], hi);
     }
     row += dl, q += dc;
     if (q >= PP) q -= PP, row += 1;
   }
   __syncthreads();
+}
+
+// the table of segment sums lies behind the tiles' rows (the look-back form's table has room for both)
+__device__ __forceinline__ uint64_t* seg_table(const ScanWs& ws, int ntiles, int NC) {
+  return ws.desc + static_cast<size_t>(ntiles) * count_pairs(NC);
+}
+
+// s_before[c] = counts of tiles [0, tile), s_total[c] = counts of all ntiles tiles (LDS, NC words each).
+// R = 0: every row is read; R > 0: the sums of segments of R tiles (tile_segsum) are there.
+__device__ __forceinline__ void sum_tile_counts(const ScanWs& ws, uint32_t tile, int ntiles, int NC, int R,
+                                                uint32_t* s_before, uint32_t* s_total) {
+  for (int c = threadIdx.x; c < NC; c += kTile) s_before[c] = s_total[c] = 0u;
+  __syncthreads();
+  if (R <= 0) {
+    sum_count_rows<true>(ws.desc, ntiles, static_cast<int>(tile), NC, s_before, s_total);
+    return;
+  }
+  const int seg = static_cast<int>(tile) / R, nseg = (ntiles + R - 1) / R;
+  sum_count_rows<true>(seg_table(ws, ntiles, NC), nseg, seg, NC, s_before, s_total);
+  const int first = seg * R;
+  sum_count_rows<false>(ws.desc + static_cast<size_t>(first) * count_pairs(NC), min(R, ntiles - first),
+                        static_cast<int>(tile) - first, NC, s_before, s_total);
+}
+
+// the segment's sums (LDS s_sum[NC], all kTile threads) -> its row of the segment table
+__device__ __forceinline__ void tile_segsum(const ScanWs& ws, int seg, int ntiles, int NC, int R, uint32_t* s_sum) {
+  for (int c = threadIdx.x; c < NC; c += kTile) s_sum[c] = 0u;
+  __syncthreads();
+  const int first = seg * R;
+  const int PP = count_pairs(NC);
+  sum_count_rows<true>(ws.desc + static_cast<size_t>(first) * PP, min(R, ntiles - first), 0, NC, s_sum, s_sum);
+  uint64_t* out = seg_table(ws, ntiles, NC) + static_cast<size_t>(seg) * PP;
+  for (int q = threadIdx.x; q < PP; q += kTile) {
+    const uint32_t lo = s_sum[2 * q], hi = (2 * q + 1 < NC) ? s_sum[2 * q + 1] : 0u;
+    out[q] = foreign_word(hi, lo);
+  }
 }
 
 }  // namespace lancet

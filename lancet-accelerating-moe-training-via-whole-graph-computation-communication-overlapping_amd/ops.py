@@ -144,9 +144,9 @@ def moe_encode_workspace_bytes(S, E, top_k=1):
     return int(capi.load().lancet_moe_encode_workspace_bytes(int(S), int(E), int(top_k)))
 
 
-def _flags(gate_is_logits, zero_tail, rows_at_used=False):
+def _flags(gate_is_logits, zero_tail, rows_at_used=False, scan_lookback=False):
     return ((capi.GATE_IS_LOGITS if gate_is_logits else 0) | (0 if zero_tail else capi.NO_TAIL_ZERO) |
-            (capi.ROWS_AT_USED if rows_at_used else 0))
+            (capi.ROWS_AT_USED if rows_at_used else 0) | (capi.SCAN_LOOKBACK if scan_lookback else 0))
 
 
 def _check_noise(gate2_noise, gate, top_k):
@@ -158,7 +158,8 @@ def _check_noise(gate2_noise, gate, top_k):
 
 
 def moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_logits=False,
-               zero_tail=True, gate2_noise=None, rows_at_used=False, workspace=None, out=None, capacity=None):
+               zero_tail=True, gate2_noise=None, rows_at_used=False, workspace=None, out=None, capacity=None,
+               scan_lookback=False):
     """raf.op.moe_encode(data, gate, used_capacity, capacity_factor=1.0).
 
     Returns (gates_s [k*S] f32, indices_locations [2, k*S] i32, used_capacity [E] i32,
@@ -172,7 +173,8 @@ def moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_
     capacity, if given, is used as it is instead of the reference formula: GShard's own top-2 capacity is
     ceil(2 * S / E * capacity_factor) (docker/resources/sharded_moe.py:267), which differs from
     int(2 * capacity_factor * ceil(S / E)) when E does not divide S or the factor is fractional
-    (S = 300, E = 8, factor 1: 75 against 76)."""
+    (S = 300, E = 8, factor 1: 75 against 76).  scan_lookback=True runs the position scan as one kernel with a
+    look-back between its tiles whatever the size (LANCET_SCAN_LOOKBACK)."""
     lib = capi.load()
     dt = _check_encode_inputs(data, gate)
     S, M = data.shape
@@ -198,14 +200,14 @@ def moe_encode(data, gate, used_capacity, capacity_factor=1.0, top_k=1, gate_is_
     ws = _scan_workspace(moe_encode_workspace_bytes(S, E, top_k), dev, workspace)
     _need(gates_s.dtype == gate.dtype, "gates_s takes the gate's dtype")
     st = lib.lancet_moe_encode(_p(data), _p(gate), _p(gate2_noise), _p(used_capacity), S, M, E, Cap, top_k, dt,
-                               _gate_code(gate), _flags(gate_is_logits, zero_tail, rows_at_used), _p(gates_s), _p(indloc),
+                               _gate_code(gate), _flags(gate_is_logits, zero_tail, rows_at_used, scan_lookback), _p(gates_s), _p(indloc),
                                _p(used_out), _p(elems), _p(disp), _p(ws.buf), ws.nbytes, _stream())
     capi.check(st, "lancet_moe_encode")
     return gates_s, indloc, used_out, elems.view(torch.uint64) if elems.dtype == torch.int64 else elems, disp
 
 
 def moe_route(gate, used_capacity, M, capacity_factor=1.0, top_k=1, gate_is_logits=False, gate2_noise=None,
-              workspace=None, out=None, capacity=None):
+              workspace=None, out=None, capacity=None, scan_lookback=False):
     """The routing half of moe_encode (selection + position scan, src/op/dialect/cuda/moe.cc:366-380), so that
     a caller can run it ahead of, or beside, the row movement of another partition.  M only scales
     elements_per_expert.  Returns (gates_s, indices_locations, used_capacity, elements_per_expert)."""
@@ -225,7 +227,7 @@ def moe_route(gate, used_capacity, M, capacity_factor=1.0, top_k=1, gate_is_logi
     gates_s, indloc, used_out, elems = out[:4]
     ws = _scan_workspace(moe_encode_workspace_bytes(S, E, top_k), dev, workspace)
     _need(gates_s.dtype == gate.dtype, "gates_s takes the gate's dtype")
-    st = lib.lancet_moe_route(_p(gate), _p(gate2_noise), _p(used_capacity), S, int(M), E, Cap, top_k, gd, _flags(gate_is_logits, True),
+    st = lib.lancet_moe_route(_p(gate), _p(gate2_noise), _p(used_capacity), S, int(M), E, Cap, top_k, gd, _flags(gate_is_logits, True, False, scan_lookback),
                               _p(gates_s), _p(indloc), _p(used_out), _p(elems), _p(ws.buf), ws.nbytes, _stream())
     capi.check(st, "lancet_moe_route")
     return gates_s, indloc, used_out, elems
@@ -297,7 +299,7 @@ def moe_encode_bpr_workspace_bytes(S0, E, n_partitions=1):
 
 
 def moe_encode_batch_prioritized(data, gate, n_partitions=1, partition_id=0, capacity_factor=1.0,
-                                 gate_is_logits=False, zero_tail=True, workspace=None, out=None):
+                                 gate_is_logits=False, zero_tail=True, workspace=None, out=None, scan_lookback=False):
     """raf.op.moe_encode_batch_prioritized(data, gate, n_partitions=1, partition_id=0,
     capacity_factor=1.0): data/gate are the whole batch, the outputs cover partition
     partition_id (S = S0 / n_partitions tokens)."""
@@ -321,7 +323,7 @@ def moe_encode_batch_prioritized(data, gate, n_partitions=1, partition_id=0, cap
     ws = _scan_workspace(moe_encode_bpr_workspace_bytes(S0, E, n_partitions), dev, workspace)
     _need(gates_s.dtype == gate.dtype, "gates_s takes the gate's dtype")
     st = lib.lancet_moe_encode_bpr(_p(data), _p(gate), S0, M, E, Cap, n_partitions, partition_id, dt, _gate_code(gate),
-                                   _flags(gate_is_logits, zero_tail), _p(gates_s), _p(indloc),
+                                   _flags(gate_is_logits, zero_tail, False, scan_lookback), _p(gates_s), _p(indloc),
                                    _p(used_out), _p(elems), _p(disp), _p(ws.buf), ws.nbytes, _stream())
     capi.check(st, "lancet_moe_encode_bpr")
     return gates_s, indloc, used_out, elems.view(torch.uint64) if elems.dtype == torch.int64 else elems, disp

@@ -159,6 +159,8 @@ class MoeEncode : public OpEnv {
     const float cf = static_cast<float>(OptFloat(cv, 3, 1.0)) * (top_k_ == 2 ? 2.0f : 1.0f);
     shape_ = CheckEncodeInputs(data, cv.args[1].AsTensor(), 1, cf);
     flags_ = (OptInt(cv, 5, 0) ? LANCET_GATE_IS_LOGITS : 0u) | (OptInt(cv, 6, 1) ? 0u : LANCET_NO_TAIL_ZERO);
+    // trailing extension (argument 8, after the optional noise tensor): the scan as one look-back kernel
+    if (cv.args.size() > 8 && cv.args[8].kind != Value::kTensor && OptInt(cv, 8, 0)) flags_ |= LANCET_SCAN_LOOKBACK;
     dtype_ = DTypeToLancet(data.dtype);
     gate_dtype_ = GateDTypeToLancet(cv.args[1].AsTensor().dtype);
     device_id_ = data.device_id;

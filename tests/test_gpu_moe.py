@@ -305,18 +305,18 @@ def test_bounded_wait_flags_the_workspace(pkg, k):
     import ctypes as C
     lib = pkg.capi.load()
     ops = pkg.ops
-    S, M, E = 131072, 4, 512         # 512 tiles x 512 or 1024 counters: a launch that takes the look-back form of the scan
+    S, M, E = 131072, 4, 256         # 512 tiles; scan_lookback asks for the look-back form (the default forms have no waits)
     data, logits = make_inputs(1, S, M, E)
     d_data, d_gate = dev(data), dev(logits)
     enc = mo.moe_encode_top2 if k == 2 else mo.moe_encode
     want = enc(data, logits, np.zeros(E, np.int32), 1.0, gate_is_logits=True, fast_scatter=True)
     ws = ops.ScanWorkspace(ops.moe_encode_workspace_bytes(S, E, k))
-    ops.moe_encode(d_data, d_gate, None, 1.0, top_k=k, gate_is_logits=True, workspace=ws)
+    ops.moe_encode(d_data, d_gate, None, 1.0, top_k=k, gate_is_logits=True, workspace=ws, scan_lookback=True)
     assert ws.error() == 0
     gave_up = 0
     for _ in range(3):
         assert lib.lancet_debug_scan_workspace_spin_limit(C.c_void_p(ws.buf.data_ptr()), 1, None) == 0
-        got = ops.moe_encode(d_data, d_gate, None, 1.0, top_k=k, gate_is_logits=True, workspace=ws)
+        got = ops.moe_encode(d_data, d_gate, None, 1.0, top_k=k, gate_is_logits=True, workspace=ws, scan_lookback=True)
         assert lib.lancet_debug_scan_workspace_spin_limit(C.c_void_p(ws.buf.data_ptr()), 0, None) == 0
         torch.cuda.synchronize()   # terminates
         il, used = to_np(got[1]), to_np(got[2])
@@ -339,7 +339,7 @@ def test_bounded_wait_flags_the_workspace(pkg, k):
             if k == 2:
                 assert (il == -1).all()
         # the workspace is ready for the next call whatever happened
-        got = ops.moe_encode(d_data, d_gate, None, 1.0, top_k=k, gate_is_logits=True, workspace=ws)
+        got = ops.moe_encode(d_data, d_gate, None, 1.0, top_k=k, gate_is_logits=True, workspace=ws, scan_lookback=True)
         np.testing.assert_array_equal(to_np(got[1]), want[1])
         np.testing.assert_array_equal(to_np(got[2]), want[2])
         np.testing.assert_array_equal(to_np(got[4]), want[4])
@@ -364,11 +364,14 @@ def test_scan_epoch_wraps(pkg):
         wants.append((dev(data), dev(logits), enc(data, logits, np.zeros(E, np.int32), 1.0, gate_is_logits=True, fast_scatter=True)))
 
     def run_all():
+        # every case as one look-back kernel (the form that draws epochs) and in the form it takes by default
+        # (no look-back at these sizes: its words in the table must never pass for descriptors)
         for (S, E, k), (d, g, want) in zip(cases, wants):
-            got = ops.moe_encode(d, g, None, 1.0, top_k=k, gate_is_logits=True, workspace=ws)
-            np.testing.assert_array_equal(to_np(got[1]), want[1])
-            np.testing.assert_array_equal(to_np(got[2]), want[2])
-            np.testing.assert_allclose(to_np(got[0]), want[0], rtol=1e-5)
+            for lookback in (True, False):
+                got = ops.moe_encode(d, g, None, 1.0, top_k=k, gate_is_logits=True, workspace=ws, scan_lookback=lookback)
+                np.testing.assert_array_equal(to_np(got[1]), want[1])
+                np.testing.assert_array_equal(to_np(got[2]), want[2])
+                np.testing.assert_allclose(to_np(got[0]), want[0], rtol=1e-5)
 
     run_all()                      # epochs 1..3: their words stay in the table
     for start in (last - 4, last - 1, last):
@@ -381,8 +384,8 @@ def test_scan_epoch_wraps(pkg):
     gate = mo.softmax_rows(logits)
     want = mo.moe_encode_bpr(data, gate, 1, 0, 1.0, fast_scatter=True)
     assert lib.lancet_debug_scan_workspace_epoch(C.c_void_p(ws.buf.data_ptr()), last, None) == 0
-    for _ in range(2):
-        got = ops.moe_encode_batch_prioritized(dev(data), dev(gate), 1, 0, 1.0, workspace=ws)
+    for lookback in (True, True, False, True):
+        got = ops.moe_encode_batch_prioritized(dev(data), dev(gate), 1, 0, 1.0, workspace=ws, scan_lookback=lookback)
         np.testing.assert_array_equal(to_np(got[1]), want[1])
         np.testing.assert_array_equal(to_np(got[2]), want[2])
     run_all()
@@ -443,13 +446,14 @@ def test_scan_workspace_is_reused_across_shapes(pkg):
         data, logits = make_inputs(200 + i, S, 8, E)
         enc = mo.moe_encode_top2 if k == 2 else mo.moe_encode
         want = enc(data, logits, np.zeros(E, np.int32), 1.0, gate_is_logits=True, fast_scatter=True)
-        got = ops.moe_encode(dev(data), dev(logits), None, 1.0, top_k=k, gate_is_logits=True, workspace=ws)
+        # the look-back form and the forms without waits alternate on the one workspace
+        got = ops.moe_encode(dev(data), dev(logits), None, 1.0, top_k=k, gate_is_logits=True, workspace=ws, scan_lookback=i % 2 == 0)
         np.testing.assert_array_equal(to_np(got[1]), want[1])
         np.testing.assert_array_equal(to_np(got[2]), want[2])
         if i % 3 == 0:   # batch-prioritised calls share it too
             gate = mo.softmax_rows(logits)
             wb = mo.moe_encode_bpr(data, gate, 1, 0, 1.0, fast_scatter=True)
-            gb = ops.moe_encode_batch_prioritized(dev(data), dev(gate), 1, 0, 1.0, workspace=ws)
+            gb = ops.moe_encode_batch_prioritized(dev(data), dev(gate), 1, 0, 1.0, workspace=ws, scan_lookback=i % 2 == 1)
             np.testing.assert_array_equal(to_np(gb[1]), wb[1])
     # the batch-prioritised call keeps per-token data behind its descriptor table, where a later call with a
     # larger table expects descriptors: small expert ids and arbitrary floats must not pass for them
@@ -462,9 +466,10 @@ def test_scan_workspace_is_reused_across_shapes(pkg):
         data, logits = make_inputs(310 + i, S, 8, E)
         enc = mo.moe_encode_top2 if k == 2 else mo.moe_encode
         want = enc(data, logits, np.zeros(E, np.int32), 1.0, gate_is_logits=True, fast_scatter=True)
-        got = ops.moe_encode(dev(data), dev(logits), None, 1.0, top_k=k, gate_is_logits=True, workspace=ws)
-        np.testing.assert_array_equal(to_np(got[1]), want[1])
-        np.testing.assert_array_equal(to_np(got[2]), want[2])
+        for lookback in (True, False):
+            got = ops.moe_encode(dev(data), dev(logits), None, 1.0, top_k=k, gate_is_logits=True, workspace=ws, scan_lookback=lookback)
+            np.testing.assert_array_equal(to_np(got[1]), want[1])
+            np.testing.assert_array_equal(to_np(got[2]), want[2])
     assert ws.error() == 0
 
 

@@ -81,7 +81,7 @@ def test_encode_bpr_random(pkg, seed):
 
 @pytest.mark.parametrize("S,E,k,cf,skew", [(300001, 512, 2, 1.0, 3.0), (262144, 2, 2, 0.3, 0.0), (100000, 100, 1, 2.5, 1.0),
                                            (65536, 256, 2, 0.3, 3.0), (300001, 3, 1, 1.0, 0.0), (262144, 64, 1, 0.3, 3.0)])
-def test_routing_over_many_tiles(pkg, S, E, k, cf, skew):
+def test_routing_over_many_tiles(pkg, S, E, k, cf, skew, scan_lookback=False):
     """Long batches: more than a thousand scan tiles, look-back windows of a couple of rows (E = 512, top-2) up
     to hundreds, a crowded expert, chained used capacity; every output against the oracle (M = 4 keeps the
     oracle's row movement small)."""
@@ -94,7 +94,7 @@ def test_routing_over_many_tiles(pkg, S, E, k, cf, skew):
     if k == 1:
         used0 = rng.integers(0, max(mo.capacity(S, E, cf), 1) + 1, E).astype(np.int32)
     want = (mo.moe_encode_top2 if k == 2 else mo.moe_encode)(data, logits, used0, cf, gate_is_logits=True, fast_scatter=True)
-    got = pkg.ops.moe_encode(dev(data), dev(logits), dev(used0), cf, top_k=k, gate_is_logits=True)
+    got = pkg.ops.moe_encode(dev(data), dev(logits), dev(used0), cf, top_k=k, gate_is_logits=True, scan_lookback=scan_lookback)
     np.testing.assert_array_equal(to_np(got[1]), want[1])
     np.testing.assert_array_equal(to_np(got[2]), want[2])
     np.testing.assert_array_equal(to_np(got[3]), want[3])
@@ -102,17 +102,22 @@ def test_routing_over_many_tiles(pkg, S, E, k, cf, skew):
     np.testing.assert_array_equal(to_np(got[4]), want[4])
 
 
-# tiles x counters at most 131072: two kernels without waits (unless one counter set on at most 32 tiles); beyond: look-back
+# one counter set on at most 32 tiles: one look-back kernel; tiles x counters up to 32768: two kernels without waits;
+# beyond: three (segment sums between count and place).  Every case also as one look-back kernel.
 @pytest.mark.parametrize("S,E,k,cf,skew", [
-    (32768, 512, 2, 1.0, 2.0),    # 128 tiles x 1024 counters = the limit: two pairs of counters per thread and row
-    (32769, 512, 2, 1.0, 2.0),    # one tile more: look-back
+    (32768, 512, 2, 1.0, 2.0),    # 128 tiles x 1024 counters: two pairs of counters per thread and row, segments of 32
+    (8192, 512, 2, 1.0, 2.0),     # 32 x 1024 = 32768: the last size at which every tile adds up all rows
+    (8193, 512, 2, 1.0, 2.0),     # one tile more: segment sums
     (49152, 256, 2, 0.5, 3.0),    # 192 x 512: one pair per thread, rows read eight at a time
     (8448, 100, 1, 1.5, 1.0),     # 33 tiles, 50 pairs (do not divide the workgroup: sums through LDS atomics)
     (8192, 100, 1, 1.5, 1.0),     # 32 tiles, one set: look-back
     (20000, 64, 1, 0.7, 2.0),     # 79 x 64: 32 pairs, several rows per thread and a remainder
     (9000, 7, 1, 1.0, 0.0),       # odd counter count: the last pair's high half is empty
     (5000, 3, 2, 1.0, 0.0), (300, 2, 2, 2.0, 0.0), (1, 2, 2, 1.0, 0.0),
-    (786432, 16, 1, 1.0, 1.0),    # 3072 tiles x 16: more tiles than run at once, still the two-kernel form
+    (786432, 16, 1, 1.0, 1.0),    # 3072 tiles: more tiles than run at once; segments of 64, the last one short
+    (300001, 1, 1, 0.5, 0.0),     # one expert: one counter per tile, 1172 tiles, segment table behind an odd-sized table
+    (262145, 33, 2, 1.0, 2.0),    # 1025 tiles in segments of 64 (the 17th holds one tile), 66 counters
 ])
-def test_both_forms_of_the_scan_at_their_boundaries(pkg, S, E, k, cf, skew):
+def test_every_form_of_the_scan_at_its_boundaries(pkg, S, E, k, cf, skew):
     test_routing_over_many_tiles(pkg, S, E, k, cf, skew)
+    test_routing_over_many_tiles(pkg, S, E, k, cf, skew, scan_lookback=True)

@@ -107,11 +107,12 @@ def test_op_layer_reports_a_scan_that_gave_up(pkg, ex):
     the marks, and check() raises where the reference would have aborted; the next run is whole again."""
     import ctypes as C
     lib = pkg.capi.load()
-    S, M, E = 131072, 8, 512         # 512 tiles x 512 counters: the scan with the look-back (smaller launches take a form without waits)
+    S, M, E = 131072, 8, 256         # 512 tiles; the look-back form of the scan is asked for below (the default forms have no waits)
     data, logits = make_inputs(13, S, M, E)
     gate = mo.softmax_rows(logits)
     want = mo.moe_encode(data, gate, np.zeros(E, np.int32), 1.0, fast_scatter=True)
-    call = ex.prepare("raf.op.moe_encode", dev(data), dev(gate), dev(np.zeros(E, np.int32)), 1.0)
+    # capacity_factor, top_k, gate_is_logits, zero_tail, no noise tensor, scan as one look-back kernel
+    call = ex.prepare("raf.op.moe_encode", dev(data), dev(gate), dev(np.zeros(E, np.int32)), 1.0, 1, 0, 1, 0, 1)
     try:
         got = call.run()
         call.check()

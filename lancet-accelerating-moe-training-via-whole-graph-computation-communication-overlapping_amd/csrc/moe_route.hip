@@ -89,6 +89,20 @@ struct SelectTop {
   TopState t;
   __device__ __forceinline__ void operator()(float x, int j) { t = consider<K>(t, x, j); }
 };
+// Selection and the softmax denominator in one walk: the sum is kept relative to the running maximum and
+// rescaled when a larger value comes (the values the two-pass form adds, exp(x - max), each within an ulp or two;
+// used where the row is staged through LDS and a second walk would move it through LDS again).
+template <int K>
+struct SelectSum {
+  TopState t;
+  float sum;
+  __device__ __forceinline__ void operator()(float x, int j) {
+    const bool first = (t.i1 < 0) | (x > t.v1);
+    if (first) sum = (t.i1 < 0 ? 0.f : sum * expf(t.v1 - x)) + 1.f;
+    else sum += expf(x - t.v1);
+    t = consider<K>(t, x, j);
+  }
+};
 struct SumExp {  // sequential sum in expert order
   float top, sum;
   __device__ __forceinline__ void operator()(float x, int) { sum += expf(x - top); }
@@ -125,6 +139,141 @@ __device__ __forceinline__ Routed route_token(const void* __restrict__ row, cons
   r.p0 = is_logits ? expf(t.v1 - t.v1) / sum : t.v1;
   r.e1 = K == 2 ? t.i2 : -1;
   r.p1 = K == 2 ? (is_logits ? expf(t.v2 - t.v1) / sum : t.v2) : 0.f;
+  return r;
+}
+
+// ---- rows longer than a cache line: staged through LDS ------------------------------------------------------
+// A lane that walks its own row touches each 128-byte line of it in eight loads, and every load of the wave
+// touches 64 different lines; with rows of several lines and many waves on a CU the lines are evicted between a
+// lane's visits and fetched again (1M tokens x 64 fp32 experts: 0.55 TB/s).  Such rows are therefore read the way
+// they lie in memory, a wave's 64 rows 128 bytes at a time (eight lanes per row and line, every line whole in one
+// load), passed through LDS and walked from there, each lane its own row as before: the values and their order
+// are the same, so is the result.  It pays from about two workgroups per CU on (512 tiles: routing of 1M tokens x
+// 64 experts 482 -> 98 us, 262144 x 256 274 -> 92); launches of fewer tiles keep the direct walk, whose lines survive
+// in the cache (65536 x 256 top-2: 50 against 64 us).
+constexpr int kStageMinTiles = 512;
+constexpr int kStageChunk = 128;                   // bytes of a row staged at a time
+constexpr int kStageRow = kStageChunk + 16;        // row pitch in LDS (the pad spreads the lanes' reads over the banks)
+constexpr int kStageWave = kWave * kStageRow;      // bytes per wave
+constexpr int kStageBytes = kWavesPerTile * kStageWave;
+
+template <int GD>
+__host__ __device__ inline bool rows_are_staged(const void* gate, const void* noise, int S, int E) {
+  constexpr int gb = GD == LANCET_F32 ? 4 : 2;
+  return noise == nullptr && (S + kTile - 1) / kTile >= kStageMinTiles && E * gb > kStageChunk && (E * gb) % 16 == 0 &&
+         (reinterpret_cast<uintptr_t>(gate) & 15u) == 0;
+}
+
+// Calls f(x, j), j = 0 .. E-1 in order, for the lane's row of the wave's rows (rows = first of them, nrows <= 64
+// valid ones, E * sizeof(value) a multiple of 16, 16-byte aligned).  All lanes of the wave, uniform control flow;
+// stage = the wave's kStageWave bytes of LDS.
+// the lane's eight granules of chunk c0 of the wave's rows (zeros beyond the rows and beyond the chunk)
+__device__ __forceinline__ void stage_load(const char* rows, int nrows, int row_bytes, int c0, u32x4 (&x)[8]) {
+  const int lane = lane_id();
+  const int gpr = min(kStageChunk, row_bytes - c0) / 16;  // granules per row in this chunk: 8, less in the last
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int g = i * kWave + lane;
+    const int r = gpr == 8 ? (g >> 3) : g / gpr;
+    const int part = gpr == 8 ? (g & 7) : g - r * gpr;
+    x[i] = u32x4{0u, 0u, 0u, 0u};
+    if (r < nrows) x[i] = *reinterpret_cast<const u32x4*>(rows + static_cast<size_t>(r) * row_bytes + c0 + part * 16);
+  }
+}
+
+template <int GD, typename F>
+__device__ __forceinline__ F walk_rows_staged(const char* rows, int nrows, int E, char* stage, F f) {
+  constexpr int gb = GD == LANCET_F32 ? 4 : 2;
+  constexpr int V = 16 / gb;  // values per 16-byte granule
+  const int row_bytes = E * gb;
+  const int lane = lane_id();
+  u32x4 x[8], nx[8];
+  stage_load(rows, nrows, row_bytes, 0, x);
+  for (int c0 = 0; c0 < row_bytes; c0 += kStageChunk) {
+    const int gpr = min(kStageChunk, row_bytes - c0) / 16;
+    // the next chunk's loads are in flight while this one is walked
+    const bool more = c0 + kStageChunk < row_bytes;
+    if (more) stage_load(rows, nrows, row_bytes, c0 + kStageChunk, nx);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int g = i * kWave + lane;
+      const int r = gpr == 8 ? (g >> 3) : g / gpr;
+      const int part = gpr == 8 ? (g & 7) : g - r * gpr;
+      if (r < kWave) *reinterpret_cast<u32x4*>(stage + r * kStageRow + part * 16) = x[i];
+    }
+    // the wave's own LDS traffic is in order; the fences keep the compiler from moving the reads above the writes
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int j0 = c0 / gb;
+    for (int p = 0; p < gpr; ++p) {
+      const u32x4 v = *reinterpret_cast<const u32x4*>(stage + lane * kStageRow + p * 16);
+      const int j = j0 + p * V;
+      if (GD == LANCET_F32) {
+        f(__uint_as_float(v.x), j);
+        f(__uint_as_float(v.y), j + 1);
+        f(__uint_as_float(v.z), j + 2);
+        f(__uint_as_float(v.w), j + 3);
+      } else {
+        f(half_word<GD>(v.x & 0xffffu), j);
+        f(half_word<GD>(v.x >> 16), j + 1);
+        f(half_word<GD>(v.y & 0xffffu), j + 2);
+        f(half_word<GD>(v.y >> 16), j + 3);
+        f(half_word<GD>(v.z & 0xffffu), j + 4);
+        f(half_word<GD>(v.z >> 16), j + 5);
+        f(half_word<GD>(v.w & 0xffffu), j + 6);
+        f(half_word<GD>(v.w >> 16), j + 7);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (more) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] = nx[i];
+    }
+  }
+  return f;
+}
+
+// Selection for token s of a workgroup whose thread t holds token s = first + t (kTile consecutive tokens): what
+// route_token gives, by the direct walk or through LDS.  All kTile threads, uniform control flow; lds = at least
+// kStageBytes when rows_are_staged (it may be reused after the call).  Threads with s >= S get {-1, -1, 0, 0}.
+template <int K, int GD>
+__device__ __forceinline__ Routed route_tile_token(const void* gate, const void* noise, int s, int S, int E, bool is_logits,
+                                                   void* lds) {
+  constexpr size_t gb = GD == LANCET_F32 ? 4 : 2;
+  Routed r = {-1, -1, 0.f, 0.f};
+  if (!rows_are_staged<GD>(gate, noise, S, E)) {
+    if (s < S) {
+      const size_t off = static_cast<size_t>(s) * E * gb;
+      r = route_token<K, GD>(static_cast<const char*>(gate) + off, noise ? static_cast<const char*>(noise) + off : nullptr, E,
+                             is_logits);
+    }
+    return r;
+  }
+  const int first = s - lane_id();  // the wave's first token
+  const int nrows = min(max(S - first, 0), kWave);
+  const char* rows = static_cast<const char*>(gate) + static_cast<size_t>(first) * E * gb;
+  char* stage = static_cast<char*>(lds) + (threadIdx.x / kWave) * kStageWave;
+  TopState t;
+  float sum = 1.f;
+  if (is_logits) {
+    SelectSum<K> sel = {{0.f, 0.f, -1, -1}, 0.f};
+    sel = walk_rows_staged<GD>(rows, nrows, E, stage, sel);
+    t = sel.t;
+    sum = sel.sum;
+  } else {
+    SelectTop<K> sel = {{0.f, 0.f, -1, -1}};
+    t = walk_rows_staged<GD>(rows, nrows, E, stage, sel).t;
+  }
+  if (s < S) {
+    r.e0 = t.i1;
+    r.p0 = is_logits ? expf(t.v1 - t.v1) / sum : t.v1;
+    r.e1 = K == 2 ? t.i2 : -1;
+    r.p1 = K == 2 ? (is_logits ? expf(t.v2 - t.v1) / sum : t.v2) : 0.f;
+  }
+  __syncthreads();  // the caller may use the LDS for something else now
   return r;
 }
 
@@ -192,16 +341,14 @@ __global__ __launch_bounds__(kTile) void route_scan_kernel(RouteArgs a) {
     e[j] = -1;
     p[j] = 0.f;
   }
-  if (valid) {
-    if (a.idx_in) {
+  if (a.idx_in) {
+    if (valid) {
       const int x = a.idx_in[s];
       e[0] = (x >= 0 && x < a.E) ? x : -1;
-    } else {
-      constexpr size_t gb = GD == LANCET_F32 ? 4 : 2;
-      const size_t off = static_cast<size_t>(s) * a.E * gb;
-      const Routed r = route_token<K, GD>(static_cast<const char*>(a.gate) + off,
-                                          a.noise ? static_cast<const char*>(a.noise) + off : nullptr, a.E,
-                                          a.is_logits != 0);
+    }
+  } else {
+    const Routed r = route_tile_token<K, GD>(a.gate, a.noise, s, a.S, a.E, a.is_logits != 0, s_cnt);
+    if (valid) {
       e[0] = r.e0;
       p[0] = r.p0;
       if (K == 2) {
@@ -275,16 +422,14 @@ __global__ __launch_bounds__(kTile) void route_count_kernel(RouteArgs a) {
     e[j] = -1;
     p[j] = 0.f;
   }
-  if (valid) {
-    if (a.idx_in) {
+  if (a.idx_in) {
+    if (valid) {
       const int x = a.idx_in[s];
       e[0] = (x >= 0 && x < a.E) ? x : -1;
-    } else {
-      constexpr size_t gb = GD == LANCET_F32 ? 4 : 2;
-      const size_t off = static_cast<size_t>(s) * a.E * gb;
-      const Routed r = route_token<K, GD>(static_cast<const char*>(a.gate) + off,
-                                          a.noise ? static_cast<const char*>(a.noise) + off : nullptr, a.E,
-                                          a.is_logits != 0);
+    }
+  } else {
+    const Routed r = route_tile_token<K, GD>(a.gate, a.noise, s, a.S, a.E, a.is_logits != 0, s_cnt);
+    if (valid) {
       e[0] = r.e0;
       p[0] = r.p0;
       if (K == 2) {
@@ -430,12 +575,10 @@ __global__ __launch_bounds__(kTile) void finalize_top2_kernel(RouteArgs a) {
 template <int K, int GD>
 __global__ __launch_bounds__(kTile) void gate_topk_kernel(const void* gate, const void* noise, int S, int E,
                                                           int is_logits, int32_t* idx, void* val) {
+  extern __shared__ uint32_t s_stage[];
   const int s = blockIdx.x * kTile + threadIdx.x;
+  const Routed r = route_tile_token<K, GD>(gate, noise, s, S, E, is_logits != 0, s_stage);
   if (s >= S) return;
-  constexpr size_t gb = GD == LANCET_F32 ? 4 : 2;
-  const size_t off = static_cast<size_t>(s) * E * gb;
-  const Routed r = route_token<K, GD>(static_cast<const char*>(gate) + off,
-                                      noise ? static_cast<const char*>(noise) + off : nullptr, E, is_logits != 0);
   idx[s] = r.e0;
   st_gate(val, s, r.p0, GD);
   if (K == 2) {
@@ -523,9 +666,8 @@ __global__ __launch_bounds__(kTile) void bpr_prepare_kernel(const void* gate, in
   const int s = static_cast<int>(tile) * kTile + tid;
   int cls[1] = {-1};
   uint32_t key = 0;
+  const Routed r = route_tile_token<1, GD>(gate, nullptr, s, a.S0, a.E, is_logits != 0, s_cnt);
   if (s < a.S0) {
-    constexpr size_t gb = GD == LANCET_F32 ? 4 : 2;
-    const Routed r = route_token<1, GD>(static_cast<const char*>(gate) + static_cast<size_t>(s) * a.E * gb, nullptr, a.E, is_logits != 0);
     const float prio = round_gate(r.p0, GD);
     a.tok[s] = foreign_word(static_cast<uint32_t>(r.e0 + 1), __float_as_uint(prio));
     cls[0] = r.e0;
@@ -911,6 +1053,13 @@ __global__ __launch_bounds__(kTile) void bpr_place_kernel(BprArgs a) {
 // ---------------------------------------------------------------------------------------
 int64_t scan_num_tiles(int64_t S) { return S > 0 ? (S + kTile - 1) / kTile : 1; }
 
+// LDS a selecting kernel needs for the rows it stages (0: it walks them directly)
+static size_t stage_lds_bytes(int gate_dtype, const void* gate, const void* noise, int S, int E) {
+  bool staged = false;
+  LANCET_GATE_SWITCH(gate_dtype, staged = rows_are_staged<GD>(gate, noise, S, E))
+  return staged ? kStageBytes : 0;
+}
+
 size_t scan_workspace_bytes(int64_t S, int64_t E, int nsets) {
   // (two words per tile at least: the forms without look-back keep the tiles' counts, two to a word, and the
   // segments' sums in the room of the look-back's table)
@@ -964,9 +1113,10 @@ hipError_t run_gate_topk(const void* gate, const void* noise, int S, int E, int 
                          int32_t* idx, void* val, hipStream_t st) {
   if (S == 0) return hipSuccess;
   const int blocks = (S + kTile - 1) / kTile;
+  const size_t lds = stage_lds_bytes(gate_dtype, gate, K == 2 ? noise : nullptr, S, E);
   LANCET_GATE_SWITCH(gate_dtype,
-    if (K == 1) gate_topk_kernel<1, GD><<<blocks, kTile, 0, st>>>(gate, nullptr, S, E, is_logits, idx, val);
-    else gate_topk_kernel<2, GD><<<blocks, kTile, 0, st>>>(gate, noise, S, E, is_logits, idx, val))
+    if (K == 1) gate_topk_kernel<1, GD><<<blocks, kTile, lds, st>>>(gate, nullptr, S, E, is_logits, idx, val);
+    else gate_topk_kernel<2, GD><<<blocks, kTile, lds, st>>>(gate, noise, S, E, is_logits, idx, val))
   return hipGetLastError();
 }
 
@@ -994,7 +1144,7 @@ hipError_t run_route_scan(const void* gate, const void* noise, const int32_t* id
   a.ws = scan_ws_view(ws);
   a.seg_rows = 0;
   hipError_t err = hipSuccess;
-  const size_t lds = scan_lds_bytes(K * E);
+  const size_t lds = std::max(scan_lds_bytes(K * E), idx_in ? size_t(0) : stage_lds_bytes(gate_dtype, gate, a.noise, S, E));
   const ScanForm form = scan_form(a.ntiles, static_cast<int64_t>(K) * E, K, force_lookback);
   if (form != kScanLookback) {
     // two or three kernels that wait for nothing instead of a look-back between tiles that all run at once
@@ -1055,7 +1205,7 @@ hipError_t run_bpr_route(const void* gate, int S0, int E, int C, int M, int n_pa
   a.elems_out = elems_out;
   hipError_t err = hipSuccess;
   // (an empty batch still runs one tile, which leaves empty groups for the select kernel)
-  LANCET_GATE_SWITCH(gate_dtype, (bpr_prepare_kernel<GD><<<a.ntiles0, kTile, scan_lds_bytes(E), st>>>(gate, is_logits, a)))
+  LANCET_GATE_SWITCH(gate_dtype, (bpr_prepare_kernel<GD><<<a.ntiles0, kTile, std::max(scan_lds_bytes(E), stage_lds_bytes(gate_dtype, gate, nullptr, S0, E)), st>>>(gate, is_logits, a)))
   err = hipGetLastError();
   if (err != hipSuccess) return err;
   bpr_select_kernel<<<E, kSelectThreads, 0, st>>>(a);

@@ -347,23 +347,22 @@ __device__ __forceinline__ bool tile_scan(const int (&cls)[NSETS], const bool (&
   return s_poison != 0;
 }
 
-// ---- two kernels instead of a look-back -------------------------------------------------------------------
+// ---- two or three kernels instead of a look-back -----------------------------------------------------------
 // When the tiles of a launch all run at once no inclusive prefix exists until the first tiles finish, and the
 // look-back degenerates into a chain of memory round trips from tile to tile (8 of the 21 us of a 256-tile
-// launch, and still 70 us at 1024 tiles).  Unless the batch is very long the scan is therefore cut in two
-// kernels that wait for nothing: the first stores every tile's counts, the second lets every tile add up the
-// counts of the tiles before it (and of all tiles: the totals) with plain loads, eight in flight per thread.
-// A tile's counts are stored two to a 64-bit word, the high half tagged "not a descriptor", so that the
-// workspace keeps its property that no word of it can pass for a descriptor of a later look-back launch.
-// Reading all rows costs T * NC words per tile, quadratic in the tile count T.  Measured against the look-back
-// (routing of T tiles x NC counters, us): 256 x 64: 14.5 / 23; 1024 x 64: 41 / 70; 2048 x 16: 31 / 87; at
-// T * NC = 131072 it still wins everywhere (256 x 512: 58 / 72; 1024 x 128: 89 / 108; 2048 x 64: 271 / 308;
-// 8192 x 16: 272 / 467); at 262144 it loses (512 x 512: 151 / 118; 4096 x 64: 700 / 622; 1024 x 256: 371 / 274),
-// so the launch keeps the look-back beyond 131072.
-// The third form, for long batches: adding up ALL rows in every tile is quadratic in the tile count, so a kernel
-// between the two adds the rows up in segments of R consecutive tiles (R about the square root of the tile
-// count), and a tile then reads the sums of the segments before its own and the rows of its own segment before
-// itself: about 2 * sqrt(T) rows instead of T.  Three launches, still no waits and no state.
+// launch, 70 us at 1024 tiles, 430 us at 8192).  Except for one counter set on at most 32 tiles (one short
+// kernel) the scan is therefore cut into kernels that wait for nothing: the first stores every tile's counts,
+// the last lets every tile add up the counts of the tiles before it (and of all tiles: the totals) with plain
+// loads, eight in flight per thread.  A tile's counts are stored two to a 64-bit word, the high half tagged "not
+// a descriptor", so that the workspace keeps its property that no word of it can pass for a descriptor of a
+// later look-back launch.
+// Adding up ALL rows in every tile costs T * NC words per tile, quadratic in the tile count T: beyond
+// T * NC = 32768 a kernel between the two adds the rows up in segments of R consecutive tiles (R about the
+// square root of T), and a tile then reads the sums of the segments before its own and the rows of its own
+// segment before itself: about 2 * sqrt(T) rows instead of T.  Three launches, still no waits and no state.
+// Routing of S tokens x E experts (us; two kernels / three kernels / look-back): 65536 x 32 top-2 12.7 / 15.7 / 24;
+// 131072 x 32 top-2 19 / 21 / 38; 262144 x 32 top-2 42 / 33 / 69; 1048576 x 16 top-1 88 / 39 / 208;
+// 2097152 x 16 top-1 275 / 68 / 432.
 enum ScanForm { kScanLookback = 0, kScanCountPlace = 1, kScanCountSegPlace = 2 };
 constexpr int64_t kFlatPlaceMaxWork = 32768;  // tiles x counters up to which the extra launch costs more than it saves
 __host__ inline ScanForm scan_form(int64_t ntiles, int64_t ncounters, int nsets, bool force_lookback = false) {

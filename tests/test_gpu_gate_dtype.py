@@ -157,3 +157,60 @@ def test_op_layer_takes_a_half_gate(pkg):
     np.testing.assert_array_equal(to_np(out[4]), want[4])
     dec = run("raf.op.moe_decode", out[4], out[0], out[1])
     np.testing.assert_array_equal(to_np(dec), mo.moe_decode(want[4], want[0], want[1], round_fn=mo.round_to_f16))
+
+
+# From 512 tiles of 256 tokens on, gate rows longer than a cache line are read a wave's 64 rows at a time, 128 bytes
+# of each, and passed through LDS; with logits the softmax denominator is then formed in the same walk as the
+# selection (rescaled sum).  Row lengths: whole 128-byte chunks, a short last chunk, a single granule in the last.
+@pytest.mark.parametrize("gd,E", [("f32", 64), ("f32", 100), ("f32", 36), ("bf16", 72), ("bf16", 128), ("f16", 200), ("f16", 68)])
+@pytest.mark.parametrize("k", [1, 2])
+@pytest.mark.parametrize("logits", [False, True])
+def test_selection_on_long_batches_of_long_rows(pkg, gd, E, k, logits):
+    import ctypes as C
+    ops, capi, lib = pkg.ops, pkg.capi, pkg.capi.load()
+    S, M, cf = 131072 + 37, 4, 0.7            # 513 tiles, the last one ragged
+    rng = np.random.default_rng(E + k)
+    raw = rng.standard_normal((S, E), dtype=np.float32) * np.float32(2.0)
+    raw[:, rng.integers(E)] += np.float32(1.5)
+    data = rng.standard_normal((S, M), dtype=np.float32)
+    gate32 = raw if logits else mo.softmax_rows(raw)
+    gate = gate32 if gd == "f32" else ROUND[gd](gate32)
+    rnd = None if gd == "f32" else ROUND[gd]
+    used_in = (np.arange(E, dtype=np.int32) % 5) if k == 1 else np.zeros(E, np.int32)
+    if k == 1:
+        want = mo.moe_encode(data, gate, used_in, cf, gate_is_logits=logits, fast_scatter=True)
+    else:
+        want = mo.moe_encode_top2(data, gate, used_in, cf, gate_is_logits=logits, fast_scatter=True, gate_round=rnd)
+    tdt = torch.float32 if gd == "f32" else TORCH_DT[gd]
+    d_gate = dev(gate).to(tdt)
+    got = ops.moe_encode(dev(data), d_gate, dev(used_in), cf, top_k=k, gate_is_logits=logits)
+    np.testing.assert_array_equal(to_np(got[1]), want[1])
+    np.testing.assert_array_equal(to_np(got[2]), want[2])
+    np.testing.assert_array_equal(to_np(got[4]), want[4])
+    if gd == "f32":
+        np.testing.assert_allclose(to_np(got[0]), want[0], rtol=1e-5, atol=0)
+    else:
+        assert ulp_diff(got[0], want[0], gd) <= (0 if (k == 1 and not logits) else 1)
+    # selection alone (lancet_gate_topk) takes the same path
+    code = {"f32": capi.F32, "bf16": capi.BF16, "f16": capi.F16}[gd]
+    p = lambda t: C.c_void_p(t.data_ptr())
+    idx = torch.empty((k, S), dtype=torch.int32, device="cuda")
+    val = torch.empty((k, S), dtype=tdt, device="cuda")
+    assert lib.lancet_gate_topk(p(d_gate), None, S, E, k, code, capi.GATE_IS_LOGITS if logits else 0, p(idx), p(val), None) == 0
+    wi, wv = mo.select_topk(gate, k, logits, None)
+    np.testing.assert_array_equal(to_np(idx), wi)
+    if not logits:
+        np.testing.assert_array_equal(to_np(val).astype(np.float32), wv)
+
+
+def test_batch_prioritized_on_a_long_batch_of_long_rows(pkg):
+    S0, M, E, P = 140000, 4, 96, 2
+    rng = np.random.default_rng(77)
+    gate = mo.softmax_rows(rng.standard_normal((S0, E), dtype=np.float32) * np.float32(2.0))
+    data = rng.standard_normal((S0, M), dtype=np.float32)
+    for pid in range(P):
+        want = mo.moe_encode_bpr(data, gate, P, pid, 0.8, fast_scatter=True)
+        got = pkg.ops.moe_encode_batch_prioritized(dev(data), dev(gate), P, pid, 0.8)
+        np.testing.assert_array_equal(to_np(got[1]), want[1])
+        np.testing.assert_array_equal(to_np(got[2]), want[2])
+        np.testing.assert_array_equal(to_np(got[0]), want[0])

@@ -41,7 +41,7 @@
 extern "C" {
 #endif
 
-#define LANCET_ABI_VERSION 6
+#define LANCET_ABI_VERSION 7
 
 /* element type of token rows (dtype) and of gate arrays (gate_dtype) */
 #define LANCET_F32 0

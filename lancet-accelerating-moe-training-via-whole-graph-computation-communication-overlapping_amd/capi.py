@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(HERE, "lib", "liblancet_hip.so")
 F32, BF16, F16 = 0, 1, 2
 GATE_IS_LOGITS = 1
 NO_TAIL_ZERO = 2
-ABI_VERSION = 6
+ABI_VERSION = 7
 ZERO_TAIL = 4
 ROWS_AT_USED = 8
 SCAN_LOOKBACK = 16

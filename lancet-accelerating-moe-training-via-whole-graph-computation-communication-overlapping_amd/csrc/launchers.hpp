@@ -31,6 +31,8 @@ hipError_t run_route_scan(const void* gate, const void* noise, const int32_t* id
                           int E, int C, int M, int K, bool is_logits, int gate_dtype, void* gates_s,
                           int32_t* idx_out, int32_t* loc_out, int32_t* used_out,
                           uint64_t* elems_out, void* ws, hipStream_t st, bool force_lookback = false);
+// between count and place on long batches: sums of the table's rows in segments of R tiles (scan.hpp)
+hipError_t run_scan_segsum(void* ws, int ntiles, int NC, int R, hipStream_t st);
 hipError_t run_bpr_route(const void* gate, int S0, int E, int C, int M, int n_partitions,
                          int partition_id, bool is_logits, int gate_dtype, void* gates_s, int32_t* idx_out,
                          int32_t* loc_out, int32_t* used_out, uint64_t* elems_out, void* ws,

@@ -175,17 +175,6 @@ __device__ __forceinline__ void tile_end(const ScanWs& ws, const TileStart& me, 
   }
 }
 
-// One-time set-up of a workspace of nwords 32-bit words (a later launch may use any part of it).
-__global__ void scan_ws_init_kernel(uint32_t* ws, size_t nwords) {
-  for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < nwords;
-       i += static_cast<size_t>(gridDim.x) * blockDim.x) {
-    uint32_t v = 0u;
-    if (i == kWsEpoch) v = 1u;
-    if (i == kWsMagic) v = kWsMagicValue;
-    ws[i] = v;
-  }
-}
-
 // LDS layout used by tile_scan: (kWavesPerTile + 3) rows of NC words:
 //   rows 0..3 : per-wave counts, turned into exclusive prefixes over the waves of the tile
 //   row  4    : tile aggregate

@@ -419,7 +419,7 @@ int lancet_lans_plan_norms(lancet_lans_plan_t plan, float* norms4xT, lancet_stre
  * allocation; every call that uses the workspace leaves it ready for the next, so that no call spends a
  * launch on clearing it.  A call that is handed a workspace that is not set up launches nothing harmful:
  * it sets every indices/locations entry and every used_out entry to -1 and the error word.
- * The scan has two forms and a call picks one by its size.  Top-1 calls of at most 32 tiles of 256 tokens
+ * The scan has several forms and a call picks one by its size.  Top-1 calls of at most 32 tiles of 256 tokens
  * (8192 tokens), and calls with LANCET_SCAN_LOOKBACK, run as one kernel with a look-back between tiles, to which
  * everything said here about state and waits applies.  All others run as two kernels (three on long batches: tiles
  * x counters above 32768) in which no workgroup waits for another: they use the workspace as plain scratch (no

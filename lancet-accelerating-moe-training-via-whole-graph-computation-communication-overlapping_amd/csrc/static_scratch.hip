@@ -1,7 +1,7 @@
 // lancet_moe_encode_noalloc: moe_encode for callers that cannot allocate device memory (code under
 // HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  The position scan needs
-// scratch memory beyond the inputs and outputs (ticket, error word and the descriptor table of the
-// decoupled look-back); lancet_moe_encode takes it as a caller-owned workspace, this entry point keeps
+// scratch memory beyond the inputs and outputs (the table of the tiles' counts; ticket, error word and
+// descriptors in its look-back form); lancet_moe_encode takes it as a caller-owned workspace, this entry point keeps
 // it in a file-scope device array of LANCET_NOALLOC_SCRATCH_BYTES instead.  Every GPU the library runs
 // on holds its own copy of the array, at its own address, until the process ends.
 //

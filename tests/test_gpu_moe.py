@@ -260,10 +260,12 @@ def test_decode_roundtrip_identity_expert(pkg):
 
 
 # ----------------------------------------------------------------------------- launcher level
-def test_launch_gen_location_and_encode_forward(pkg):
+# the scan in each of its forms: one look-back kernel (12 tiles), count + place (79), count + segment sums + place (1172)
+@pytest.mark.parametrize("S,E", [(3000, 12), (20000, 12), (300000, 64)])
+def test_launch_gen_location_and_encode_forward(pkg, S, E):
     import ctypes as C
     lib = pkg.capi.load()
-    S, M, E, cf = 3000, 16, 12, 0.7
+    M, cf = 16, 0.7
     data, logits = make_inputs(31, S, M, E)
     Cap = mo.capacity(S, E, cf)
     idx0 = np.argmax(logits, axis=1).astype(np.int32)

@@ -27,10 +27,13 @@ def _capture(fn):
     return g
 
 
+# (4096, 256, 16): the scan as one look-back kernel (top-1) or as count + place (top-2); (140000, 8, 64): count +
+# segment sums + place, gate rows staged through LDS
+@pytest.mark.parametrize("S,M,E", [(4096, 256, 16), (140000, 8, 64)])
 @pytest.mark.parametrize("k,dt", [(1, torch.float32), (2, torch.bfloat16)])
-def test_encode_decode_graph_replays(pkg, k, dt):
+def test_encode_decode_graph_replays(pkg, k, dt, S, M, E):
     ops = pkg.ops
-    S, M, E, cf = 4096, 256, 16, 0.8
+    cf = 0.8
     data = torch.empty((S, M), dtype=dt, device="cuda")
     logits = torch.empty((S, E), dtype=torch.float32, device="cuda")
     C = ops.moe_capacity(S, E, cf * k)

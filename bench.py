@@ -42,7 +42,7 @@ def parse():
     ap.add_argument("--lans-scale", type=float, default=1.0, help="fraction of the 24-layer LANS tensor list")
     ap.add_argument("--lans-schedule", default=None, choices=["sweeps", "resident"],
                     help="time only this LANS schedule (profiling)")
-    ap.add_argument("--only", default="all", choices=["all", "scatter", "decode", "route", "copy", "stream_copy", "lans"],
+    ap.add_argument("--only", default="all", choices=["all", "scatter", "decode", "route", "route_forms", "copy", "stream_copy", "lans"],
                     help="profiling aid: run just one kernel family (prints a short JSON line)")
     return ap.parse_args()
 
@@ -604,6 +604,33 @@ def main():
         ms = event_ms(run, args.steps)
         print(json.dumps({"only": "stream_copy", "bytes_read": n, "bytes_written": n, "ms": round(ms, 4),
                           "GBps": round(2 * n / ms / 1e6, 1)}), flush=True)
+        return
+    if args.only == "route_forms":
+        # Routing alone (selection + position scan, lancet_moe_route) over token and expert counts from the side
+        # configurations to long batches, in the form the library picks (look-back on few tiles of top-1, else two
+        # or three kernels without waits) and as one look-back kernel (LANCET_SCAN_LOOKBACK).
+        rows = []
+        for S, E, k in [(4096, 8, 1), (16384, 16, 2), (32768, 64, 1), (65536, 32, 2), (65536, 64, 1), (131072, 32, 2),
+                        (262144, 32, 2), (65536, 256, 2), (131072, 256, 2), (262144, 64, 2), (524288, 64, 1),
+                        (1048576, 16, 1), (1048576, 64, 1), (2097152, 16, 1), (262144, 256, 1), (131072, 512, 1)]:
+            gate = torch.randn((S, E), device="cuda")
+            out = ops.moe_route(gate, None, 8, 1.25, top_k=k, gate_is_logits=True)
+            ref = [t.clone() for t in out]
+            t = {}
+            for name, lb in (("default", False), ("look_back", True)):
+                run = lambda: ops.moe_route(gate, None, 8, 1.25, top_k=k, gate_is_logits=True, out=out, scan_lookback=lb)
+                for _ in range(max(args.warmup, 2)):
+                    run()
+                t[name] = event_ms(run, max(args.steps, 20))
+                assert all(torch.equal(a, b) for a, b in zip(out, ref)), "the forms of the scan disagree"
+            tiles = (S + 255) // 256
+            form = "look-back" if (k == 1 and tiles <= 32) else ("count+place" if tiles * k * E <= 32768 else "count+segsum+place")
+            rows.append({"tokens": S, "experts": E, "top_k": k, "tiles": tiles, "default_form": form,
+                         "gate_rows_staged": bool(tiles >= 512 and E * 4 > 128),
+                         "us_default": round(t["default"] * 1e3, 1), "us_look_back": round(t["look_back"] * 1e3, 1),
+                         "gate_GBps_default": round(S * E * 4 / t["default"] / 1e6, 1)})
+            del gate, out, ref
+        print(json.dumps({"only": "route_forms", "rows": rows}), flush=True)
         return
     if args.only == "lans":
         print(json.dumps({"only": "lans", "lans": bench_lans(ops, capi, args.steps, args.warmup, args.lans_scale,

@@ -112,14 +112,18 @@ struct SelectSum {
   float sum;
   __device__ __forceinline__ void operator()(float x, int j) {
     const bool first = (t.i1 < 0) | (x > t.v1);
-    if (first) sum = (t.i1 < 0 ? 0.f : sum * expf(t.v1 - x)) + 1.f;
-    else sum += expf(x - t.v1);
+    if (first) sum = (t.i1 < 0 ? 0.f : sum * __expf(t.v1 - x)) + 1.f;
+    else sum += __expf(x - t.v1);
     t = consider<K>(t, x, j);
   }
 };
+// The terms of the denominator go through the hardware exponential (__expf); the two gate values themselves
+// through expf.  Against an fp64 softmax the gates are as close as with expf in the sum (largest relative error
+// 4e-7 at 32 experts, 1.6e-6 at 512, either way: what shows is the rounding of the fp32 sum), and routing with
+// 64 experts or more takes 10-15 % less time.
 struct SumExp {  // sequential sum in expert order
   float top, sum;
-  __device__ __forceinline__ void operator()(float x, int) { sum += expf(x - top); }
+  __device__ __forceinline__ void operator()(float x, int) { sum += __expf(x - top); }
 };
 
 // noise (K = 2 only, may be null): values added to the row for the second choice alone, the first

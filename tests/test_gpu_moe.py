@@ -906,3 +906,29 @@ def test_capacity_override_gshard_formula(pkg):
         np.testing.assert_array_equal(to_np(got[i]), want[i])
     r = pkg.ops.moe_route(dev(logits), None, M, 1.0, top_k=2, gate_is_logits=True, capacity=C)
     np.testing.assert_array_equal(to_np(r[1]), want[1])
+
+
+def test_default_workspaces_are_kept_per_stream(pkg):
+    """Calls without a workspace argument share one kept per (device, stream): calls on two streams that run at the
+    same time must not share theirs (the look-back form keeps state in it), and scan_errors() reads them all."""
+    ops = pkg.ops
+    S, M, E = 6000, 32, 16           # top-1 on 24 tiles: the look-back form
+    data, logits = make_inputs(77, S, M, E)
+    want = mo.moe_encode(data, logits, np.zeros(E, np.int32), 1.0, gate_is_logits=True, fast_scatter=True)
+    d_data, d_gate = dev(data), dev(logits)
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    before = len(ops._scan_pool)
+    outs = []
+    for _ in range(20):
+        outs.append(ops.moe_encode(d_data, d_gate, None, 1.0, gate_is_logits=True))
+        with torch.cuda.stream(side):
+            outs.append(ops.moe_encode(d_data, d_gate, None, 1.0, gate_is_logits=True))
+    torch.cuda.synchronize()
+    assert len(ops._scan_pool) >= max(before, 2)
+    keys = {k for k in ops._scan_pool if k[1] in (side.cuda_stream, torch.cuda.current_stream().cuda_stream)}
+    assert len(keys) == 2
+    for got in outs:
+        np.testing.assert_array_equal(to_np(got[1]), want[1])
+        np.testing.assert_array_equal(to_np(got[4]), want[4])
+    assert ops.scan_errors() == 0

@@ -41,7 +41,7 @@
 extern "C" {
 #endif
 
-#define LANCET_ABI_VERSION 7
+#define LANCET_ABI_VERSION 8
 
 /* element type of token rows (dtype) and of gate arrays (gate_dtype) */
 #define LANCET_F32 0
@@ -293,6 +293,22 @@ int lancet_moe_encode_dx(const void* dy, const int32_t* indices_locations, int64
  * tutel_moe_dispatch.cu:96-105,499-506). */
 int lancet_moe_encode_dg(const void* dy_gates_s, const int32_t* indices_locations, int64_t S,
                          int64_t E, int top_k, int gate_dtype, void* grad_gates, lancet_stream_t stream);
+/* Gate gradient of moe_encode as a whole, for the forms of the op that do more to a gate value than select it:
+ * grad_gate[S,E] = d loss / d gate given dy_gates_s = d loss / d gates_s (the op's OUTPUT, [top_k*S]), through
+ *   - top_k = 2: the normalisation g_k / max(g_1 + g_2, eps) of the two kept values (docker/resources/sharded_moe.py:
+ *     304-312): d g_1 = (dy_1 - dy_2) * g_2 / (g_1 + g_2)^2, d g_2 = (dy_2 - dy_1) * g_1 / (g_1 + g_2)^2; below eps the
+ *     clamped denominator is a constant (d g_k = dy_k / eps); a dropped slot has g = 0 and gets no gradient, which
+ *     leaves the other slot's weight at the constant 1;
+ *   - LANCET_GATE_IS_LOGITS in flags: the softmax the op fused (sharded_moe.py:260): d x[e] = p[e] * (d p[e] - sum_j
+ *     p[i_j] * d p[i_j]), p recomputed from `gate` (the logits) in fp32.
+ * gate and indices_locations are the forward's input and output; second-choice noise (gate2_noise) only moved the
+ * selection and needs no gradient.  With top_k = 1 and no flag the result is moe_encode_dg's (gate may then be NULL).
+ * Extends MoeEncodeGrad (src/op/grad/moe.cc:30-58), which differentiates the op end to end for the one form the
+ * reference has (top-1 on probabilities), to the top-2 / fused-softmax forms of lancet_moe_encode.  One pass: reads
+ * and writes S*E gate elements. */
+int lancet_moe_encode_dgate(const void* dy_gates_s, const void* gate, const int32_t* indices_locations, int64_t S,
+                            int64_t E, int top_k, int gate_dtype, unsigned flags, void* grad_gate,
+                            lancet_stream_t stream);
 /* moe_decode_dx: grad_expert_out[idx, loc, :] = gates_s * dy[s, :], zero elsewhere.  Replaces
  * MoeDecodeDx / launch_decode_backward_data (moe.cc:1313-1395; kernel_util.cuh:47;
  * tutel_moe_dispatch.cu:118-124,523-533).  Workspace: an [E*C] int32 row -> token map. */

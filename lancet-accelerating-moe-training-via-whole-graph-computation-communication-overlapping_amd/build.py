@@ -15,7 +15,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 
-HIP_SOURCES = ["capi.hip", "moe_route.hip", "moe_bpr.hip", "moe_rows.hip", "sparse_copy.hip", "lans.hip", "static_scratch.hip"]
+HIP_SOURCES = ["capi.hip", "moe_route.hip", "moe_bpr.hip", "moe_rows.hip", "moe_gate_grad.hip", "sparse_copy.hip", "lans.hip", "static_scratch.hip"]
 HIP_FLAGS = [
     "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC",
     # Packed fp32 arithmetic stays off for every kernel of this library.  The option reaches both passes of

@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(HERE, "lib", "liblancet_hip.so")
 F32, BF16, F16 = 0, 1, 2
 GATE_IS_LOGITS = 1
 NO_TAIL_ZERO = 2
-ABI_VERSION = 7
+ABI_VERSION = 8
 ZERO_TAIL = 4
 ROWS_AT_USED = 8
 SCAN_LOOKBACK = 16
@@ -23,7 +23,7 @@ MAX_PARTITIONS = 64
 OK = 0
 (ERR_NULL, ERR_SHAPE, ERR_DTYPE, ERR_WORKSPACE, ERR_ALIGN, ERR_TOPK, ERR_PARTITION, ERR_PLAN, ERR_SCRATCH,
  ERR_STALLED) = range(-1, -11, -1)
-NOALLOC_SCRATCH_BYTES = 1 << 20
+NOALLOC_SCRATCH_BYTES = (2 << 20) + 4096
 
 
 class LansHyper(C.Structure):
@@ -76,6 +76,7 @@ SIGNATURES = {
                                                _int, _u32, _vp]),
     "lancet_moe_encode_dx": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp]),
     "lancet_moe_encode_dg": (_int, [_vp, _vp, _i64, _i64, _int, _int, _vp, _vp]),
+    "lancet_moe_encode_dgate": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _int, _u32, _vp, _vp]),
     "lancet_moe_decode_dx_workspace_bytes": (_sz, [_i64, _i64]),
     "lancet_moe_decode_dx": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _vp, _vp, _sz, _vp]),
     "lancet_moe_decode_dg": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _vp, _vp]),

@@ -550,6 +550,24 @@ extern "C" int lancet_moe_encode_dg(const void* dy_gates_s, const int32_t* indic
                           S_(stream)));
 }
 
+extern "C" int lancet_moe_encode_dgate(const void* dy_gates_s, const void* gate, const int32_t* indices_locations,
+                                       int64_t S, int64_t E, int top_k, int gate_dtype, unsigned flags, void* grad_gate,
+                                       lancet_stream_t stream) {
+  const bool is_logits = (flags & LANCET_GATE_IS_LOGITS) != 0;
+  const bool needs_gate = top_k == 2 || is_logits;
+  if (S > 0 && (!dy_gates_s || !indices_locations || !grad_gate || (needs_gate && !gate))) return LANCET_ERR_NULL;
+  const int gb = elem_bytes(gate_dtype);
+  if (!gb) return LANCET_ERR_DTYPE;
+  if (int r = check_dims(S, 0, E, 0)) return r;
+  if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
+  if (top_k == 2 && E < 2) return LANCET_ERR_TOPK;
+  if (S * E > 0x7fffffff) return LANCET_ERR_SHAPE;  // a tile's elements are indexed with 32 bits above its base
+  if (misaligned(dy_gates_s, gb) || misaligned(gate, gb) || misaligned(indices_locations, 4) || misaligned(grad_gate, gb))
+    return LANCET_ERR_ALIGN;
+  return rc(run_encode_dgate(dy_gates_s, gate, indices_locations, static_cast<int>(S), static_cast<int>(E), top_k,
+                             is_logits, gate_dtype, grad_gate, S_(stream)));
+}
+
 extern "C" size_t lancet_moe_decode_dx_workspace_bytes(int64_t E, int64_t C) {
   if (E < 1 || C < 0) return 0;
   return static_cast<size_t>(E) * static_cast<size_t>(C) * sizeof(int32_t);

@@ -59,6 +59,10 @@ hipError_t run_decode_rows(const void* expert_out, const void* gates, int gate_d
 
 // backward (gates == nullptr in run_decode_rows gives moe_encode_dx)
 hipError_t run_encode_dg(const void* dy, const int32_t* idx, int S, int E, int K, int gate_dtype, void* grad_gates, hipStream_t st);
+// moe_gate_grad.hip: gradient of gates_s [K*S] back to the [S,E] gate through the top-2 normalisation and, with
+// is_logits, the fused softmax; gate may be null for K == 1 on probabilities
+hipError_t run_encode_dgate(const void* dy, const void* gate, const int32_t* idx, int S, int E, int K, bool is_logits,
+                            int gate_dtype, void* out, hipStream_t st);
 hipError_t run_decode_dx(const void* dy, const void* gates, int gate_dtype, const int32_t* idx, const int32_t* loc, void* out,
                          int32_t* src_map, int S, int M, int E, int C, int K, int dtype, hipStream_t st);
 hipError_t run_decode_dg(const void* dy, const void* expert_out, const int32_t* idx, const int32_t* loc, void* out,

@@ -1,0 +1,172 @@
+// Gate gradient of moe_encode as a whole: from the gradient of the op's OUTPUT gates_s back to the [S,E] array
+// the op was given, through everything the op does to a gate value on the way:
+//   top_k = 1, probabilities   nothing: grad[s, idx] = dy            (encode_backward_gate_kernel,
+//                              src/op/dialect/cuda/kernels/tutel_moe_dispatch.cu:96-105; wired by
+//                              src/op/grad/moe.cc:30-58)
+//   top_k = 2                  the normalisation g_k / max(g_1 + g_2, eps) of the two kept values
+//                              (docker/resources/sharded_moe.py:304-312; the clamp passes no gradient to the sum
+//                              below eps)
+//   LANCET_GATE_IS_LOGITS      the softmax the op fuses in front of the selection (sharded_moe.py:260):
+//                              d x[e] = p[e] * (d p[e] - sum_j p[i_j] * d p[i_j])
+// Probabilities of a 16-bit softmax are taken as computed (fp32), not as a 16-bit gates_s array would hold them:
+// the difference is below that type's own rounding.  Dropped slots carry no gradient (their mask is zero,
+// sharded_moe.py:296-297,306-307).  One launch: a lane per token forms the token's few scalars (row maximum,
+// 1 / sum of exponentials, the two slot gradients), then the workgroup writes its tile's [256, E] block of the
+// result in memory order, every element once.
+#include "launchers.hpp"
+#include "select.hpp"
+#include <algorithm>
+
+namespace lancet {
+
+struct GateGradArgs {
+  const void* dy;        // [K*S] gradient of gates_s
+  const void* gate;      // [S,E] the forward's gate input (may be null for top-1 on probabilities)
+  const int32_t* idx;    // [K*S] expert per slot after the drop (row 0 of indices_locations)
+  void* out;             // [S,E]
+  int S, E;
+  int is_logits;
+  int vec;               // rows and pointers allow 16-byte granules
+};
+
+struct RowMax {
+  float top;
+  __device__ __forceinline__ void operator()(float x, int) { top = fmaxf(top, x); }
+};
+struct RowSumExp {  // sequential sum in expert order, as the forward forms it
+  float top, sum;
+  __device__ __forceinline__ void operator()(float x, int) { sum += expf(x - top); }
+};
+
+// per-token scalars of a tile, in LDS
+struct GateGradTile {
+  int i1[kTile], i2[kTile];      // experts that receive a slot gradient (-1: none)
+  float d1[kTile], d2[kTile];    // gradient with respect to the raw value of that expert (probability or array entry)
+  float top[kTile], inv[kTile];  // logits: row maximum and 1 / sum_e exp(x - max)
+  float dot[kTile];              // logits: sum_j p[i_j] * d_j
+};
+
+template <int K, int GD>
+__global__ __launch_bounds__(kTile) void encode_dgate_kernel(GateGradArgs a) {
+  __shared__ GateGradTile sh;
+  constexpr size_t gb = GD == LANCET_F32 ? 4 : 2;
+  constexpr int V = 16 / gb;
+  const int tid = threadIdx.x;
+  const int first = blockIdx.x * kTile;
+  const int s = first + tid;
+  // ---- a lane per token -----------------------------------------------------------------------------------
+  if (s < a.S) {
+    const char* row = static_cast<const char*>(a.gate) + static_cast<size_t>(s) * a.E * gb;
+    int e[2] = {-1, -1};
+    float dy[2] = {0.f, 0.f}, g[2] = {0.f, 0.f}, praw[2] = {0.f, 0.f};
+    float top = 0.f, inv = 1.f;
+    if (a.is_logits) {
+      RowMax mx = {-INFINITY};
+      top = walk_row<GD>(row, a.E, mx).top;
+      RowSumExp se = {top, 0.f};
+      inv = 1.f / walk_row<GD>(row, a.E, se).sum;
+    }
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+      const int x = a.idx[static_cast<size_t>(j) * a.S + s];
+      if (x >= 0 && x < a.E) {
+        e[j] = x;
+        dy[j] = ld_gate(a.dy, static_cast<size_t>(j) * a.S + s, GD);
+        const float raw = (K == 2 || a.is_logits) ? gate_at<GD>(row, x) : 0.f;  // top-1 on probabilities needs no gate
+        praw[j] = a.is_logits ? expf(raw - top) * inv : raw;
+        g[j] = praw[j];
+      }
+    }
+    float d[2] = {0.f, 0.f};
+    if (K == 1) {
+      d[0] = dy[0];
+    } else {
+      const float sum = g[0] + g[1];
+      if (sum >= 1.1920929e-07f) {
+        const float r = 1.f / (sum * sum);
+        d[0] = (dy[0] - dy[1]) * g[1] * r;
+        d[1] = (dy[1] - dy[0]) * g[0] * r;
+      } else {  // the clamped denominator is a constant
+        d[0] = dy[0] / 1.1920929e-07f;
+        d[1] = dy[1] / 1.1920929e-07f;
+      }
+      if (e[0] < 0) d[0] = 0.f;
+      if (e[1] < 0) d[1] = 0.f;
+    }
+    sh.i1[tid] = e[0];
+    sh.i2[tid] = e[1];
+    sh.d1[tid] = d[0];
+    sh.d2[tid] = d[1];
+    sh.top[tid] = top;
+    sh.inv[tid] = inv;
+    sh.dot[tid] = praw[0] * d[0] + praw[1] * d[1];
+  }
+  __syncthreads();
+  // ---- the tile's block of the result, in memory order ------------------------------------------------------
+  const int ntok = min(kTile, a.S - first);
+  const size_t base = static_cast<size_t>(first) * a.E;  // first element of the tile
+  auto value = [&](int t, int ex, float x) -> float {
+    float sel = 0.f;
+    if (ex == sh.i1[t]) sel = sh.d1[t];
+    if (K == 2 && ex == sh.i2[t]) sel = sh.d2[t];
+    if (!a.is_logits) return sel;
+    return expf(x - sh.top[t]) * sh.inv[t] * (sel - sh.dot[t]);
+  };
+  if (a.vec) {
+    const int gpr = a.E / V;  // granules per row
+    const int n = ntok * gpr;
+    const u32x4* src = reinterpret_cast<const u32x4*>(static_cast<const char*>(a.gate) + base * gb);
+    u32x4* dst = reinterpret_cast<u32x4*>(static_cast<char*>(a.out) + base * gb);
+    for (int q = tid; q < n; q += kTile) {
+      const int t = q / gpr;
+      const int e0 = (q - t * gpr) * V;
+      u32x4 x = {0u, 0u, 0u, 0u};
+      if (a.is_logits) x = src[q];
+      u32x4 r;
+      if (GD == LANCET_F32) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r[i] = __float_as_uint(value(t, e0 + i, __uint_as_float(x[i])));
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float lo = value(t, e0 + 2 * i, half_word<GD>(x[i] & 0xffffu));
+          const float hi = value(t, e0 + 2 * i + 1, half_word<GD>(x[i] >> 16));
+          const uint32_t l = GD == LANCET_BF16 ? f32_to_bf16(lo) : f32_to_f16(lo);
+          const uint32_t h = GD == LANCET_BF16 ? f32_to_bf16(hi) : f32_to_f16(hi);
+          r[i] = (l & 0xffffu) | (h << 16);
+        }
+      }
+      dst[q] = r;
+    }
+  } else {
+    const int n = ntok * a.E;
+    for (int q = tid; q < n; q += kTile) {
+      const int t = q / a.E;
+      const int ex = q - t * a.E;
+      const float x = a.is_logits ? ld_gate(a.gate, base + q, GD) : 0.f;
+      st_gate(a.out, base + q, value(t, ex, x), GD);
+    }
+  }
+}
+
+hipError_t run_encode_dgate(const void* dy, const void* gate, const int32_t* idx, int S, int E, int K, bool is_logits,
+                            int gate_dtype, void* out, hipStream_t st) {
+  if (S == 0) return hipSuccess;
+  GateGradArgs a;
+  a.dy = dy;
+  a.gate = gate;
+  a.idx = idx;
+  a.out = out;
+  a.S = S;
+  a.E = E;
+  a.is_logits = is_logits;
+  const int gb = gate_dtype == LANCET_F32 ? 4 : 2;
+  a.vec = (static_cast<size_t>(E) * gb) % 16 == 0 && ((reinterpret_cast<uintptr_t>(gate) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+  const int blocks = (S + kTile - 1) / kTile;
+  LANCET_GATE_SWITCH(gate_dtype,
+    if (K == 1) encode_dgate_kernel<1, GD><<<blocks, kTile, 0, st>>>(a);
+    else encode_dgate_kernel<2, GD><<<blocks, kTile, 0, st>>>(a))
+  return hipGetLastError();
+}
+
+}  // namespace lancet

@@ -249,9 +249,12 @@ __global__ __launch_bounds__(kTile) void finalize_top2_kernel(RouteArgs a) {
   // a workspace that is not set up: route_scan_kernel has marked every output already
   if (ld_agent(a.ws.hdr + kWsMagic) != kWsMagicValue) return;
   // totals of both slots = the last tile's inclusive descriptors, [2][E]; if that tile was poisoned there are
-  // no totals and every token is marked, else the tokens of poisoned tiles carry marks of their own
+  // no totals and every token is marked, else the tokens of poisoned tiles carry marks of their own.  A tile
+  // that could not take part (its ticket or epoch was out of range: the workspace's state is damaged, e.g. by a
+  // call that overlapped this one) has published nothing, and the row may be what an earlier launch left: no
+  // totals either.
   const uint64_t* tot = a.ws.desc + static_cast<size_t>(a.ntiles - 1) * 2 * a.E;
-  const bool poisoned = desc_is_poisoned(ld_desc(tot));
+  const bool poisoned = ld_agent(a.ws.hdr + kWsFailed) != 0u || desc_is_poisoned(ld_desc(tot));
   if (s < a.S) {
     if (poisoned) {
       a.idx_out[s] = a.idx_out[a.S + s] = -1;
@@ -453,6 +456,9 @@ hipError_t run_route_scan(const void* gate, const void* noise, const int32_t* id
     err = hipGetLastError();
     if (err != hipSuccess) return err;
     finalize_top2_kernel<<<a.ntiles, kTile, 0, st>>>(a);
+    err = hipGetLastError();
+    if (err != hipSuccess) return err;
+    return run_fill_u32(a.ws.hdr + kWsFailed, 1, 0u, st);  // read by the kernel before; the next launch starts clear
   }
   return hipGetLastError();
 }

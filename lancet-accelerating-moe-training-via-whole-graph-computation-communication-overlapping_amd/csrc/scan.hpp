@@ -43,6 +43,9 @@ enum : uint32_t {
   kWsSpin = 4,    // polls a tile waits for a predecessor's word before it gives up (0: the default)
   kWsMagic = 5,   // kWsMagicValue once the workspace is set up (with kWsSpin one 8-byte load)
   kWsExtent = 6,  // largest number of descriptor words a launch has used
+  kWsFailed = 7,  // a tile of the running launch found the workspace unusable (bad ticket or epoch) and published
+                  // nothing: read by the kernel that finishes a top-2 launch from the totals row, which would
+                  // otherwise take the row an earlier launch left there; cleared by the launch sequence behind it
   kScanHeaderWords = 8
 };
 constexpr uint32_t kWsMagicValue = 0x4c53434eu;  // "LSCN"
@@ -109,7 +112,10 @@ __device__ __forceinline__ TileStart tile_begin(const ScanWs& ws, int ntiles) {
     const uint32_t t = static_cast<uint32_t>(state), epoch = static_cast<uint32_t>(state >> 32);
     const uint32_t spin = static_cast<uint32_t>(sm), magic = static_cast<uint32_t>(sm >> 32);
     const bool ok = magic == kWsMagicValue && t < static_cast<uint32_t>(ntiles) && epoch != 0u && (epoch & ~kEpochMask) == 0u;
-    if (!ok) st_agent(ws.hdr + kWsError, 1u);
+    if (!ok) {
+      st_agent(ws.hdr + kWsError, 1u);
+      st_agent(ws.hdr + kWsFailed, 1u);
+    }
     s_start[0] = ok ? t : blockIdx.x;
     s_start[1] = epoch;
     s_start[2] = spin ? spin : kDefaultScanSpin;

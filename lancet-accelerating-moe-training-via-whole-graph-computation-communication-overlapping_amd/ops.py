@@ -388,6 +388,26 @@ def moe_encode_dg(dy, indices_locations, n_experts, top_k=1, out=None):
     return out
 
 
+def moe_encode_dgate(dy, gate, indices_locations, top_k=1, gate_is_logits=False, out=None):
+    """Gate gradient of moe_encode(..., top_k, gate_is_logits) as a whole: dy [k*S] is the gradient of the op's output
+    gates_s, gate [S, E] the op's gate input, the result [S, E] the gradient with respect to that input, through the
+    top-2 normalisation (docker/resources/sharded_moe.py:304-312) and, with gate_is_logits, the fused softmax.  With
+    top_k = 1 on probabilities it is moe_encode_dg (src/op/grad/moe.cc:30-58)."""
+    lib = capi.load()
+    _dev(dy, "dy"), _dev(gate, "gate")
+    _need(dy.dim() == 1 and gate.dim() == 2, "dy must be 1-D and gate 2-D")
+    S = _check_indloc(indices_locations, top_k)
+    _need(dy.shape[0] == top_k * S and gate.shape[0] == S, "dy, gate and indices_locations disagree")
+    _need(dy.dtype == gate.dtype, "dy takes the gate's dtype")
+    if out is None:
+        out = torch.empty_like(gate)
+    _need(out.dtype == gate.dtype and out.shape == gate.shape and out.is_contiguous(), "the gradient has the gate's shape and dtype")
+    st = lib.lancet_moe_encode_dgate(_p(dy), _p(gate), _p(indices_locations), S, gate.shape[1], top_k, _gate_code(gate),
+                                     capi.GATE_IS_LOGITS if gate_is_logits else 0, _p(out), _stream())
+    capi.check(st, "lancet_moe_encode_dgate")
+    return out
+
+
 def moe_decode_dx(dy, gate, indices_locations, n_experts, capacity, top_k=1, workspace=None, out=None):
     """raf.op.moe_decode_dx(dy [S,M], gate [k*S], indices_locations, n_experts, capacity) -> [E, C, M]."""
     lib = capi.load()

@@ -32,6 +32,10 @@ Parity status of each function (what pins it, beyond re-reading the source):
   moe_encode_top2     dense einsum form of docker/resources/sharded_moe.py:253-324
                       at tiny sizes; identity with two chained top-1 encodes
   moe_decode          round trip decode(encode(x), gate=1) == x on kept tokens
+  backward ops        torch autograd through dense einsum forms of the forward
+  moe_encode_dgate    torch autograd through a dense restatement of top2gating
+                      (docker/resources/sharded_moe.py:253-324: softmax, capacity masks, clamp,
+                      normalisation), incl. a case below the clamp
 """
 import numpy as np
 
@@ -382,6 +386,45 @@ def moe_encode_dg(dy_gates_s, indloc, n_experts, k=1):
         ok = (idx >= 0) & (idx < n_experts)
         out[np.arange(S)[ok], idx[ok]] = dy_gates_s[j * S:(j + 1) * S][ok]
     return out
+
+
+def moe_encode_dgate(dy_gates_s, gate, indloc, k=1, gate_is_logits=False):
+    """Gradient of the [S,E] gate input of moe_encode / moe_encode_top2 given the gradient of the op's OUTPUT
+    gates_s [k*S]; fp64 arithmetic on the fp32 inputs.  What MoeEncodeGrad (src/op/grad/moe.cc:30-58) gives for the
+    reference's one form (k = 1 on probabilities: moe_encode_dg), extended to what the top-2 op does to a gate
+    value (docker/resources/sharded_moe.py:296-312): g_j = p[s, i_j] * mask_j (masks after the capacity drop),
+    w_j = g_j / clamp(g_1 + g_2, min=eps); torch.clamp passes the gradient where the sum is >= eps and none
+    below.  With gate_is_logits the array holds logits and p = softmax(logits) (:260), differentiated too.
+    Pinned in tests/test_oracle_moe.py by torch autograd through a dense restatement of top2gating."""
+    gate = np.asarray(gate, np.float64)
+    S, E = gate.shape
+    dy = np.asarray(dy_gates_s, np.float64)
+    if gate_is_logits:
+        ex = np.exp(gate - gate.max(axis=1, keepdims=True))
+        p = ex / ex.sum(axis=1, keepdims=True)
+    else:
+        p = gate
+    rows = np.arange(S)
+    idx = [np.asarray(indloc[0, j * S:(j + 1) * S]) for j in range(k)]
+    kept = [(i >= 0) & (i < E) for i in idx]
+    safe = [np.where(m, i, 0) for i, m in zip(idx, kept)]
+    g = [np.where(m, p[rows, i], 0.0) for i, m in zip(safe, kept)]
+    if k == 1:
+        d = [np.where(kept[0], dy[:S], 0.0)]
+    else:
+        eps = float(F32_EPS)
+        tot = g[0] + g[1]
+        live = (g[0].astype(np.float32) + g[1].astype(np.float32)) >= F32_EPS   # the forward's own fp32 sum decides
+        den2 = np.where(live, tot * tot, 1.0)
+        d1 = np.where(live, (dy[:S] - dy[S:]) * g[1] / den2, dy[:S] / eps)
+        d2 = np.where(live, (dy[S:] - dy[:S]) * g[0] / den2, dy[S:] / eps)
+        d = [np.where(kept[0], d1, 0.0), np.where(kept[1], d2, 0.0)]
+    dp = np.zeros((S, E), np.float64)
+    for j in range(k):
+        np.add.at(dp, (rows, safe[j]), d[j])
+    if not gate_is_logits:
+        return dp
+    return p * (dp - (p * dp).sum(axis=1, keepdims=True))
 
 
 def moe_decode_dx(dy, gates_s, indloc, n_experts, capacity, k=1, round_fn=None):

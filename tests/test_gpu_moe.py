@@ -48,6 +48,65 @@ def test_encode_top1(pkg, S, M, E, cf, is_logits):
     check_encode(got, want, gate_exact=not is_logits)
 
 
+def _softmax64(logits):
+    x = logits.astype(np.float64)
+    ex = np.exp(x - x.max(axis=1, keepdims=True))
+    return ex / ex.sum(axis=1, keepdims=True)
+
+
+@pytest.mark.parametrize("k", [1, 2])
+@pytest.mark.parametrize("S,E,scale,close", [(4096, 32, 30.0, False), (4096, 512, 30.0, False), (4096, 32, 1.0, True),
+                                             (3000, 512, 4.0, True), (300000, 64, 30.0, False)])
+def test_softmax_gates_for_wide_rows_and_close_runner_ups(pkg, k, S, E, scale, close):
+    """The fused softmax where it is hardest: logits of scale 30 (|x - max| of 30 to 150: the terms of the
+    denominator span the whole fp32 range and the second probability is tiny), rows of 512 experts, and rows
+    whose runner-up lies within 1e-3 of the maximum (every second row: exactly equal, where the first must win).
+    Selection bit-exact against the oracle; probabilities (lancet_gate_topk) and the op's gates_s at 1e-5 against
+    the oracle AND against a float64 softmax evaluated here.  The last shape is long enough for the rows to be
+    staged through LDS (rescaled running sum)."""
+    import ctypes as C
+    ops, capi = pkg.ops, pkg.capi
+    TINY = 1.2e-38          # below the smallest normal fp32 a probability may be flushed or lose digits
+    _, logits = make_inputs(S + E + int(scale), S, 1, E, logit_scale=scale)
+    if close:
+        rng = np.random.default_rng(1)
+        top = logits.argmax(axis=1)
+        other = (top + 1 + rng.integers(0, E - 1, S)) % E
+        delta = (rng.random(S) * 1e-3).astype(np.float32)
+        delta[::2] = 0.0
+        logits[np.arange(S), other] = logits[np.arange(S), top] - delta
+    sel, val = mo.select_topk(logits, k, True)
+    p64 = _softmax64(logits)
+    idx = torch.empty((k, S), dtype=torch.int32, device="cuda")
+    prob = torch.empty((k, S), dtype=torch.float32, device="cuda")
+    d_logits = dev(logits)
+    st = capi.load().lancet_gate_topk(C.c_void_p(d_logits.data_ptr()), None, S, E, k, capi.F32, capi.GATE_IS_LOGITS,
+                                      C.c_void_p(idx.data_ptr()), C.c_void_p(prob.data_ptr()), None)
+    assert st == 0
+    np.testing.assert_array_equal(to_np(idx), sel)
+    np.testing.assert_allclose(to_np(prob), val, rtol=GATE_RTOL, atol=TINY)
+    rows = np.arange(S)
+    for j in range(k):
+        np.testing.assert_allclose(to_np(prob)[j], p64[rows, sel[j]], rtol=GATE_RTOL, atol=TINY)
+    # the op itself: routing bit-exact, gates_s (k = 2: normalised after the drop) at the same bar
+    zero = np.zeros(E, np.int32)
+    data = np.zeros((S, 4), np.float32)
+    if k == 1:
+        want = mo.moe_encode(data, logits, zero, 0.9, gate_is_logits=True, fast_scatter=True)
+    else:
+        want = mo.moe_encode_top2(data, logits, zero, 0.9, gate_is_logits=True, fast_scatter=True)
+    got = ops.moe_encode(dev(data), d_logits, None, 0.9, top_k=k, gate_is_logits=True)
+    np.testing.assert_array_equal(to_np(got[1]), want[1])
+    np.testing.assert_array_equal(to_np(got[2]), want[2])
+    np.testing.assert_allclose(to_np(got[0]), want[0], rtol=GATE_RTOL, atol=TINY)
+    if k == 1:
+        np.testing.assert_allclose(to_np(got[0]), p64[rows, sel[0]], rtol=GATE_RTOL, atol=TINY)
+    else:
+        g = [np.where(want[1][0, j * S:(j + 1) * S] >= 0, p64[rows, sel[j]], 0.0) for j in range(2)]
+        den = np.maximum(g[0] + g[1], float(mo.F32_EPS))
+        np.testing.assert_allclose(to_np(got[0]), np.concatenate([g[0] / den, g[1] / den]), rtol=GATE_RTOL, atol=TINY)
+
+
 @pytest.mark.parametrize("dt", ["bf16", "f16"])
 def test_encode_top1_16bit_rows(pkg, dt):
     S, M, E = 1500, 96, 16
@@ -435,6 +494,35 @@ def test_scan_on_a_workspace_that_is_not_set_up(pkg):
             np.testing.assert_array_equal(to_np(outs[1]), want[1])
             np.testing.assert_array_equal(to_np(outs[4]), want[4])
             assert lib.lancet_scan_workspace_error(p(ws), None, C.byref(err)) == 0 and err.value == 0
+
+
+def test_top2_lookback_on_a_workspace_with_a_damaged_ticket(pkg):
+    """A set-up workspace that served a healthy top-2 look-back call, then has only its ticket word damaged (as a
+    call that overlapped another on the same workspace leaves it): no tile of the next call can take part, none
+    publishes, and the totals row still holds the healthy call's words.  The finalisation must not take them:
+    every output is marked (-1, gates 0, used_capacity -1, no elements), the error word is set, and after a new
+    set-up the workspace works."""
+    ops = pkg.ops
+    S, M, E = 6000, 8, 16
+    data, logits = make_inputs(31, S, M, E)
+    d_data, d_gate = dev(data), dev(logits)
+    want = mo.moe_encode_top2(data, logits, np.zeros(E, np.int32), 1.0, gate_is_logits=True, fast_scatter=True)
+    ws = ops.ScanWorkspace(ops.moe_encode_workspace_bytes(S, E, 2))
+    for _ in range(2):
+        got = ops.moe_encode(d_data, d_gate, None, 1.0, top_k=2, gate_is_logits=True, workspace=ws, scan_lookback=True)
+        np.testing.assert_array_equal(to_np(got[1]), want[1])
+    assert ws.error() == 0
+    ws.buf.view(torch.int32)[0] = 1 << 20                       # the ticket: far beyond the launch's tiles
+    got = ops.moe_encode(d_data, d_gate, None, 1.0, top_k=2, gate_is_logits=True, workspace=ws, scan_lookback=True)
+    torch.cuda.synchronize()
+    assert (to_np(got[1]) == -1).all() and (to_np(got[2]) == -1).all()
+    assert not to_np(got[0]).any() and not to_np(got[3]).any() and not to_np(got[4]).any()
+    assert ws.error() == 1
+    ws = ops.ScanWorkspace(ops.moe_encode_workspace_bytes(S, E, 2))
+    got = ops.moe_encode(d_data, d_gate, None, 1.0, top_k=2, gate_is_logits=True, workspace=ws, scan_lookback=True)
+    np.testing.assert_array_equal(to_np(got[1]), want[1])
+    np.testing.assert_array_equal(to_np(got[2]), want[2])
+    assert ws.error() == 0
 
 
 def test_scan_workspace_is_reused_across_shapes(pkg):

@@ -70,6 +70,97 @@ def test_backward_ops(pkg, dt, k, S, M, E):
     assert not got[~ok].any()
 
 
+def _gate_rounder(gdt):
+    return {"f32": lambda a: a, "bf16": mo.round_to_bf16, "f16": mo.round_to_f16}[gdt]
+
+
+def _check_gate_gradient(pkg, logits, il, k, is_logits, gdt, seed):
+    """lancet_moe_encode_dgate against the oracle (fp64 on the same, rounded, inputs).  fp32 gates: 1e-5 relative,
+    plus 1e-6 of the row's largest slot gradient for the entries where the selected term and the row's mean cancel.
+    16-bit gates: one unit in the last place of the type, or that same absolute floor."""
+    ops = pkg.ops
+    S, E = logits.shape
+    rnd = _gate_rounder(gdt)
+    gate_in = rnd(logits if is_logits else mo.softmax_rows(logits)).astype(np.float32)
+    dy = rnd(np.random.default_rng(seed).standard_normal(k * S).astype(np.float32)).astype(np.float32)
+    want = mo.moe_encode_dgate(dy, gate_in, il, k, is_logits)
+    tdt = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}[gdt]
+    got = ops.moe_encode_dgate(dev(dy).to(tdt), dev(gate_in).to(tdt), dev(il), top_k=k, gate_is_logits=is_logits)
+    assert got.dtype == tdt and got.shape == (S, E)
+    scale = np.abs(want).max(axis=1, keepdims=True)          # the selected entries carry the row's largest values
+    if gdt == "f32":
+        err = np.abs(to_np(got).astype(np.float64) - want)
+        assert (err <= 1e-5 * np.abs(want) + 1e-6 * scale + 1e-30).all(), float((err / (np.abs(want) + 1e-30)).max())
+    else:
+        w16 = torch.from_numpy(want).to(tdt)
+        a, b = got.cpu().view(torch.int16).to(torch.int32), w16.view(torch.int16).to(torch.int32)
+        a, b = torch.where(a < 0, -(a & 0x7fff), a), torch.where(b < 0, -(b & 0x7fff), b)
+        close = torch.from_numpy(np.abs(to_np(got).astype(np.float64) - want) <= 1e-6 * scale)
+        assert bool((((a - b).abs() <= 1) | close).all())
+    dead = np.stack([il[0, j * S:(j + 1) * S] < 0 for j in range(k)]).all(axis=0)
+    assert not to_np(got)[dead].any()                         # a token with no kept slot gets no gradient
+    return got
+
+
+@pytest.mark.parametrize("gdt", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("is_logits", [False, True])
+@pytest.mark.parametrize("k", [1, 2])
+@pytest.mark.parametrize("S,E", [(1024, 32), (777, 6), (300, 5), (2048, 512)])
+def test_gate_gradient_of_the_whole_op(pkg, gdt, is_logits, k, S, E):
+    """E = 5 (rows that are no whole 16-byte granules) takes the element path, the others the 16-byte one."""
+    data, logits = make_inputs(S + E, S, 1, E, zipf_bias=True)
+    rnd = _gate_rounder(gdt)
+    gate_in = rnd(logits if is_logits else mo.softmax_rows(logits)).astype(np.float32)
+    used0 = np.zeros(E, np.int32)
+    if k == 1:
+        il = mo.moe_encode(data, gate_in, used0, 0.7, gate_is_logits=is_logits, fast_scatter=True)[1]
+    else:
+        il = mo.moe_encode_top2(data, gate_in, used0, 0.7, gate_is_logits=is_logits, fast_scatter=True)[1]
+    assert (il[0] < 0).any() and (il[0] >= 0).any()
+    got = _check_gate_gradient(pkg, logits, il, k, is_logits, gdt, S)
+    if k == 1 and not is_logits:     # the reference's own rule (moe_encode_dg) is this case
+        dy = dev(rnd(np.random.default_rng(S).standard_normal(S).astype(np.float32)).astype(np.float32)).to(got.dtype)
+        assert torch.equal(got, pkg.ops.moe_encode_dg(dy, dev(il), E))
+
+
+@pytest.mark.parametrize("shape", ["config2", "config4_pressure"])
+def test_gate_gradient_at_the_baseline_shapes(pkg, shape):
+    """Config 2 (S=16384, E=16, Zipf bias: more than 1000 dropped slots) and config 4's shape with four favoured
+    experts (S=65536, E=32, C=5120: slots overflow), top-2 on logits, fp32 gate; routing taken from the HIP op."""
+    if shape == "config2":
+        S, E, cf = 16384, 16, 1.0
+        _, logits = make_inputs(0, S, 1, E, zipf_bias=True)
+    else:
+        S, E, cf = 65536, 32, 1.25
+        rng = np.random.default_rng(0)
+        logits = rng.standard_normal((S, E), dtype=np.float32)
+        logits[:, :4] += np.float32(0.75)
+    _, il, _, _ = pkg.ops.moe_route(dev(logits), None, 8, cf, top_k=2, gate_is_logits=True)
+    il = to_np(il)
+    assert (il[0] < 0).sum() > (1000 if shape == "config2" else 0)
+    _check_gate_gradient(pkg, logits, il, 2, True, "f32", 11)
+
+
+def test_gate_gradient_below_the_clamp_and_for_large_logits(pkg):
+    """Rows whose two kept values add up to less than eps (the clamped denominator is a constant), and logits of
+    scale 30, where a row's probabilities span 60 orders of magnitude."""
+    S, E = 512, 8
+    rng = np.random.default_rng(4)
+    gate = (rng.random((S, E), dtype=np.float32) * np.linspace(1e-8, 3e-7, S, dtype=np.float32)[:, None]).astype(np.float32)
+    _, il, *_ = mo.moe_encode_top2(np.zeros((S, 1), np.float32), gate, np.zeros(E, np.int32), 1.0, fast_scatter=True)
+    sel, val = mo.select_topk(gate, 2)
+    tot = val[0].astype(np.float64) + val[1]
+    assert (tot < 1.19e-7).sum() > 10 and (tot > 1.2e-7).sum() > 10
+    dy = rng.standard_normal(2 * S).astype(np.float32)
+    got = to_np(pkg.ops.moe_encode_dgate(dev(dy), dev(gate), dev(il), top_k=2))
+    want = mo.moe_encode_dgate(dy, gate, il, 2, False)
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=0)
+    _, logits = make_inputs(3, 1024, 1, 32, logit_scale=30.0)
+    il = mo.moe_encode_top2(np.zeros((1024, 1), np.float32), logits, np.zeros(32, np.int32), 0.8, gate_is_logits=True,
+                            fast_scatter=True)[1]
+    _check_gate_gradient(pkg, logits, il, 2, True, "f32", 5)
+
+
 def test_backward_matches_autograd_through_forward_ops(pkg):
     """End to end: gradients of sum(decode(expert(encode(x))) * Y) with an elementwise expert, taken
     with the backward ops, against torch autograd of the same computation written with torch indexing."""
@@ -171,15 +262,19 @@ def test_autograd_wiring_of_a_prioritized_partition(pkg):
 
 
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
-def test_moe_layer_module_against_a_dense_layer(pkg, dt):
+@pytest.mark.parametrize("top_k,fused", [(1, False), (1, True), (2, False), (2, True)])
+def test_moe_layer_module_against_a_dense_layer(pkg, dt, top_k, fused):
     """Gate / Experts / MOELayerImpl (the reference's layer, models/benchmark/pytorch/utils.py:529-634) on the HIP
     operators: output and all parameter gradients against the same layer written densely with one-hot masks in
-    torch (the form of the reference's FakeMoeEncodeOp / FakeMoeDecodeOp, :349-370,454-462), in fp64."""
+    torch (the form of the reference's FakeMoeEncodeOp / FakeMoeDecodeOp, :349-370,454-462; for top_k = 2 the
+    masks, clamp and normalisation of docker/resources/sharded_moe.py:296-322), in fp64.  fused: the gate module
+    hands over logits and the operator runs the softmax."""
     ml = pkg.moe_layer
     torch.manual_seed(3)
     B, L, M, E, H = 4, 96, 32, 4, 48
     expert = torch.nn.Sequential(torch.nn.Linear(M, H), torch.nn.GELU(), torch.nn.Linear(H, M))
-    layer = ml.MOELayerImpl(ml.Gate(M, E), ml.Experts(expert, 1, M, E), 1, E, capacity_factor=0.75).cuda()
+    layer = ml.MOELayerImpl(ml.Gate(M, E, softmax=not fused), ml.Experts(expert, 1, M, E), 1, E, capacity_factor=0.75 / top_k,
+                            top_k=top_k, fused_softmax=fused).cuda()
     for i, e in enumerate(layer.experts.experts):            # the copies start equal: make the experts differ
         for p in e.parameters():
             p.data.add_(0.05 * (i + 1) * torch.randn_like(p))
@@ -198,16 +293,24 @@ def test_moe_layer_module_against_a_dense_layer(pkg, dt):
     S = flat.shape[0]
     C = pkg.ops.moe_capacity(S, E, 0.75)
     with torch.no_grad():
-        _, il, _, _, _ = pkg.ops.moe_encode(x.detach().reshape(-1, M).contiguous(), layer.gate(x.detach().reshape(-1, M)), None, 0.75)
-    idx, loc = il[0].long(), il[1].long()
-    kept = idx >= 0
-    assert bool((~kept).any())
-    mask = torch.zeros((S, E, C), dtype=torch.float64, device="cuda")
-    mask[torch.arange(S, device="cuda")[kept], idx[kept], loc[kept]] = 1.0
-    gates_s = (gate * mask.sum(2)).sum(1)
-    disp = torch.einsum("sec,sm->ecm", mask, flat)
+        _, il, _, _, _ = pkg.ops.moe_encode(x.detach().reshape(-1, M).contiguous(), layer.gate(x.detach().reshape(-1, M)), None,
+                                            0.75 / top_k, top_k=top_k, gate_is_logits=fused)
+    assert bool((il[0] < 0).any())
+    masks, weights = [], []
+    for j in range(top_k):
+        idx, loc = il[0, j * S:(j + 1) * S].long(), il[1, j * S:(j + 1) * S].long()
+        kept = idx >= 0
+        mask = torch.zeros((S, E, C), dtype=torch.float64, device="cuda")
+        mask[torch.arange(S, device="cuda")[kept], idx[kept], loc[kept]] = 1.0
+        masks.append(mask)
+        weights.append((gate * mask.sum(2)).sum(1))
+    if top_k == 2:
+        denom = torch.clamp(weights[0] + weights[1], min=torch.finfo(torch.float32).eps)
+        weights = [w / denom for w in weights]
+    disp = torch.einsum("sec,sm->ecm", sum(masks), flat)
     eo = torch.stack([ref.experts.experts[e](disp[e]) for e in range(E)])
-    want = torch.einsum("sec,ecm->sm", mask * gates_s[:, None, None], eo).reshape(B, L, M)
+    combine = sum(m * w[:, None, None] for m, w in zip(masks, weights))
+    want = torch.einsum("sec,ecm->sm", combine, eo).reshape(B, L, M)
     (want * Y.double()).sum().backward()
     tol = dict(rtol=1e-4, atol=1e-5) if dt == torch.float32 else dict(rtol=5e-2, atol=5e-2)
     torch.testing.assert_close(out.detach().double(), want.detach(), **tol)

@@ -354,6 +354,75 @@ def test_backward_ops_match_autograd_of_dense_forms(k):
     np.testing.assert_allclose(mo.moe_decode_dg(Y.astype(np.float32), eo32, il, k), gs.grad.numpy(), rtol=1e-5, atol=1e-6)
 
 
+def _dense_top2_weights(logits_or_probs, il, k, S, E, is_logits):
+    """The gate side of top2gating (docker/resources/sharded_moe.py:253-324) in torch, fp64, dense one-hot form,
+    with the selection and capacity decisions (which slots survive) taken from `il` as constants: gates = softmax
+    (:260), mask_j after the capacity drop (:296-297), gates_j_s = einsum('se,se->s', gates, mask_j) (:306-307),
+    denom clamped at finfo(float32).eps (:308-310), division (:311-312).  k = 1: the reference op's own
+    gates_s = sum_e gate * one_hot (src/op/dialect/cuda/moe.cc:232-250), kept tokens only as its gradient rule has it."""
+    import torch
+    gates = torch.softmax(logits_or_probs, dim=1) if is_logits else logits_or_probs
+    masks = []
+    for j in range(k):
+        idx = torch.as_tensor(np.asarray(il[0, j * S:(j + 1) * S]), dtype=torch.long)
+        kept = idx >= 0
+        m = torch.zeros((S, E), dtype=torch.float64)
+        m[torch.arange(S)[kept], idx[kept]] = 1.0
+        masks.append(m)
+    gs = [torch.einsum("se,se->s", gates, m) for m in masks]
+    if k == 1:
+        return gs[0]
+    denom = torch.clamp(gs[0] + gs[1], min=torch.finfo(torch.float32).eps)
+    return torch.cat([gs[0] / denom, gs[1] / denom])
+
+
+@pytest.mark.parametrize("is_logits", [False, True])
+@pytest.mark.parametrize("k", [1, 2])
+def test_gate_gradient_of_the_whole_op_matches_autograd_of_dense_top2gating(k, is_logits):
+    import torch
+    S, M, E = 96, 4, 6
+    data, logits = rng_case(77 + k, S, M, E)
+    logits[:, 1] += 1.5                                   # a hot expert: slots of both kinds get dropped
+    gate_in = logits if is_logits else mo.softmax_rows(logits)
+    used0 = np.zeros(E, np.int32)
+    if k == 1:
+        g, il, *_ = mo.moe_encode(data, gate_in, used0, 0.6, gate_is_logits=is_logits)
+    else:
+        g, il, *_ = mo.moe_encode_top2(data, gate_in, used0, 0.6, gate_is_logits=is_logits)
+        first, second = il[0, :S] >= 0, il[0, S:] >= 0
+        assert (first & ~second).any() and (~first & second).any() and (~first & ~second).any() and (first & second).any()
+    rng = np.random.default_rng(9)
+    w = rng.standard_normal(k * S).astype(np.float32)
+    x = torch.tensor(gate_in.astype(np.float64), requires_grad=True)
+    ws = _dense_top2_weights(x, il, k, S, E, is_logits)
+    if k == 2 or not is_logits:
+        # the dense form reproduces the forward's weights (k = 1 on logits: the forward keeps the value of dropped tokens too)
+        kept = np.concatenate([il[0, j * S:(j + 1) * S] >= 0 for j in range(k)])
+        np.testing.assert_allclose(ws.detach().numpy()[kept], g[kept], rtol=2e-6)
+    (ws * torch.tensor(w.astype(np.float64))).sum().backward()
+    got = mo.moe_encode_dgate(w, gate_in, il, k, is_logits)
+    np.testing.assert_allclose(got, x.grad.numpy(), rtol=1e-9, atol=1e-12)
+    if k == 1 and not is_logits:
+        np.testing.assert_array_equal(got.astype(np.float32), mo.moe_encode_dg(w, il, E, 1))
+
+
+def test_gate_gradient_below_the_clamp_of_the_denominator():
+    """Probabilities so small that g1 + g2 < eps: the clamped denominator is a constant, d g_k = dy_k / eps
+    (torch.clamp's gradient); and rows at either side of the threshold."""
+    import torch
+    S, E = 8, 4
+    gate = np.full((S, E), 1e-9, np.float32)
+    gate[:, 0] = np.float32(3e-8) * np.arange(1, S + 1, dtype=np.float32)      # g1 + g2 from 4e-8 to 2.5e-7: crosses eps
+    gate[:, 2] = np.float32(1e-8)
+    il = np.array([[0] * S + [2] * S, list(range(S)) * 2], np.int32)
+    tot = gate[:, 0].astype(np.float64) + gate[:, 2]
+    assert (tot < float(mo.F32_EPS)).any() and (tot > float(mo.F32_EPS)).any()
+    w = np.linspace(-1, 2, 2 * S).astype(np.float32)
+    x = torch.tensor(gate.astype(np.float64), requires_grad=True)
+    (_dense_top2_weights(x, il, 2, S, E, False) * torch.tensor(w.astype(np.float64))).sum().backward()
+    np.testing.assert_allclose(mo.moe_encode_dgate(w, gate, il, 2, False), x.grad.numpy(), rtol=1e-9, atol=0)
+
+
 # ---------------------------------------------------------------- redispatch_expert_input
 @pytest.mark.parametrize("P", [2, 4])
 def test_redispatch_expert_input_partitioned_equals_whole(P):

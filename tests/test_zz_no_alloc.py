@@ -1,6 +1,7 @@
 """lancet_moe_encode_noalloc (static device scratch, no allocation) against lancet_moe_encode, through the
-C ABI: identical outputs, bit for bit, on two calls in a row, the second with a smaller input (the shared
-scratch still holds the first call's descriptors), then once more with top-1 and a used capacity."""
+C ABI: identical outputs, bit for bit, on two calls in a row, the second with a smaller input, both in the scan's
+look-back form (the one form that keeps state: the shared scratch still holds the first call's descriptors under
+the second call's table), then once more with top-1 and a used capacity; and at the largest size the scratch holds."""
 import ctypes as C
 
 import numpy as np
@@ -57,7 +58,7 @@ def test_noalloc_encode_equals_encode_on_two_calls_in_a_row(pkg, lib):
     for seed, (S, M, E, k, dtype) in enumerate([(5000, 256, 32, 2, torch.bfloat16), (1300, 64, 8, 2, torch.bfloat16)]):
         data, logits = make_inputs(100 + seed, S, M, E)
         d_data = dev(data).to(dtype)
-        ref, got, Cap = _encode_both(pkg, lib, d_data, dev(logits), None, 1.0, k, capi.GATE_IS_LOGITS)
+        ref, got, Cap = _encode_both(pkg, lib, d_data, dev(logits), None, 1.0, k, capi.GATE_IS_LOGITS | capi.SCAN_LOOKBACK)
         for name, r, g in zip(("gates_s", "indices_locations", "used_capacity", "elements_per_expert", "dispatched"), ref, got):
             assert torch.equal(r.view(torch.uint8), g.view(torch.uint8)), (seed, name)
         # and both equal the oracle's routing
@@ -78,8 +79,29 @@ def test_noalloc_encode_equals_encode_on_two_calls_in_a_row(pkg, lib):
     np.testing.assert_array_equal(to_np(got[4]), want[4])
 
 
+def test_noalloc_encode_at_the_limit_of_its_scratch(pkg, lib):
+    """S = 65536, E = 512, top-2 is the largest power-of-two batch whose table fits (256 tiles x 1024 counters);
+    one tile more is rejected."""
+    capi = pkg.capi
+    S, M, E, k = 65536, 8, 512, 2
+    assert lib.lancet_moe_encode_workspace_bytes(S, E, k) <= capi.NOALLOC_SCRATCH_BYTES
+    assert lib.lancet_moe_encode_workspace_bytes(S + 1, E, k) > capi.NOALLOC_SCRATCH_BYTES
+    data, logits = make_inputs(12, S, M, E)
+    d_data, d_logits = dev(data).to(torch.bfloat16), dev(logits)
+    for flags in (capi.GATE_IS_LOGITS, capi.GATE_IS_LOGITS | capi.SCAN_LOOKBACK):
+        ref, got, Cap = _encode_both(pkg, lib, d_data, d_logits, None, 1.0, k, flags)
+        for r, g in zip(ref, got):
+            assert torch.equal(r.view(torch.uint8), g.view(torch.uint8))
+        assert int((got[1][0] >= 0).sum()) > S
+    one = torch.zeros(1, device="cuda")
+    rc = lib.lancet_moe_encode_noalloc(_p(one), _p(one), None, None, S + 1, M, E, 8, k, capi.BF16, capi.F32, 0, _p(one), _p(one),
+                                       _p(one), _p(one), _p(one), None)
+    assert rc == capi.ERR_SCRATCH
+
+
 def test_noalloc_encode_rejects_sizes_beyond_its_scratch(pkg, lib):
     capi = pkg.capi
+    assert capi.NOALLOC_SCRATCH_BYTES == (2 << 20) + 4096     # LANCET_NOALLOC_SCRATCH_BYTES of the header
     S, E, k = 1 << 20, 512, 2          # 4096 tiles x 1024 counters x 4 B = 16 MiB of descriptors
     assert lib.lancet_moe_encode_workspace_bytes(S, E, k) > capi.NOALLOC_SCRATCH_BYTES
     one = torch.zeros(1, device="cuda")

@@ -28,8 +28,9 @@
  * tutel_moe_dispatch.cu:110-116,126-157) and mixed-precision graphs feed a half gate
  * (python/raf/amp/type_hints.py:97,105).  All arithmetic on gate values is fp32, with one rounding
  * to gate_dtype where a value is stored; 16-bit gates tie often, and selection keeps its rule (first
- * maximum wins).  LANS tensors are fp32; indices/locations/used capacity are int32 and
- * elements_per_expert is uint64, as in src/op/declare/moe.cc:48-58.
+ * maximum wins).  LANS parameters and moments are fp32 (gradients may be 16-bit: lancet_lans_step_mixed);
+ * indices/locations/used capacity are int32 and elements_per_expert is uint64, as in
+ * src/op/declare/moe.cc:48-58.
  */
 #ifndef LANCET_HIP_H_
 #define LANCET_HIP_H_
@@ -383,6 +384,19 @@ int lancet_lans_plan_destroy(lancet_lans_plan_t plan);
 int lancet_lans_step(lancet_lans_plan_t plan, const float* const* g, float* const* p,
                      float* const* m, float* const* v, int step_host, const float* step_dev,
                      const lancet_lans_hyper* hyper, const float* grad_norms, lancet_stream_t stream);
+/* The step of a mixed-precision trainer: fp32 master parameters and moments, a 16-bit model.  The reference's
+ * traced optimizer casts every gradient to fp32 in front of the op and every new parameter back to the model type
+ * behind it (python/raf/optim/lans.py:256-257, 285-288): two more passes over the state, 6 + 6 bytes per parameter on
+ * top of the step's 28.  Here the step itself reads the gradients in g_dtype (LANCET_F32 / _BF16 / _F16; widened in
+ * registers, which is exact, so every value of the step is what the cast would have given) and, when p_lowp is not
+ * NULL, writes next to each new fp32 parameter its copy in lowp_dtype (LANCET_BF16 / _F16, round to nearest even:
+ * the cast's result, bit for bit).  g and p_lowp are HOST arrays of T device pointers like the others; with
+ * g_dtype = LANCET_F32 and p_lowp = NULL this is lancet_lans_step.  16-bit gradients and both 16-bit types in and
+ * out: 2 + 24 + 2 = 28 bytes per parameter. */
+int lancet_lans_step_mixed(lancet_lans_plan_t plan, const void* const* g, int g_dtype, float* const* p,
+                           float* const* m, float* const* v, void* const* p_lowp, int lowp_dtype, int step_host,
+                           const float* step_dev, const lancet_lans_hyper* hyper, const float* grad_norms,
+                           lancet_stream_t stream);
 /* A step may be recorded into a HIP graph (either schedule): with step_dev the step number is read on the
  * device, and everything else that changes from step to step lives in the plan's device memory, so each
  * replay is a new step.  The pointer tables are uploaded (one host-to-device copy) by the first call that
@@ -403,7 +417,9 @@ int lancet_lans_step(lancet_lans_plan_t plan, const float* const* g, float* cons
  * kernel that itself waits for this step) can stall it.  Every wait is bounded: a wait that gives up leaves
  * the parameters of the tensors concerned unwritten (their m and v may already hold the new moments), sets
  * the plan's sticky error, and the NEXT lancet_lans_step on the plan returns LANCET_ERR_STALLED without
- * launching anything, until lancet_lans_plan_error has been called.
+ * launching anything, until lancet_lans_plan_error has been called.  Steps that were already queued behind the
+ * one that stalled (a loop that never synchronises, a replayed graph) see the error word on the device when they
+ * begin and skip themselves as a whole, either schedule: no array is touched again before the error is read.
  * LANCET_LANS_SWEEPS: three whole-state sweeps with two per-tensor reductions between them (48 B/param of
  * traffic).  No workgroup waits for another: the schedule for a device that is shared with kernels of
  * unbounded duration.  set_schedule(LANCET_LANS_RESIDENT) on a plan with no tensor that fits returns
@@ -449,6 +465,13 @@ int lancet_lans_plan_norms(lancet_lans_plan_t plan, float* norms4xT, lancet_stre
  * when any call on this workspace gave up a wait, or found it not set up, since the last read. */
 int lancet_scan_workspace_init(void* workspace, size_t workspace_bytes, lancet_stream_t stream);
 int lancet_scan_workspace_error(void* workspace, lancet_stream_t stream, int* error_out);
+/* 1 when a call of these sizes and flags (batch_prioritized != 0: lancet_moe_encode_bpr, S = S0 / n_partitions; else
+ * lancet_moe_encode / lancet_moe_route) runs the scan in its look-back form, the only form that reads state from
+ * the workspace: such a call needs the first lancet_moe_encode_workspace_bytes(S, E, top_k or 2) bytes of its
+ * workspace set up and can give up a wait; 0: it uses the whole workspace as plain scratch, which needs neither
+ * set-up nor a look at the error word.  For executors that hand an operator fresh workspace memory before every
+ * call (src/impl/vm/vm.cc:1260-1266) and would otherwise pay a set-up launch each time. */
+int lancet_scan_call_is_stateful(int64_t S, int64_t E, int top_k, unsigned flags, int batch_prioritized);
 
 #ifdef __cplusplus
 }

@@ -90,6 +90,8 @@ SIGNATURES = {
     "lancet_lans_plan_destroy": (_int, [_vp]),
     "lancet_lans_step": (_int, [_vp, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),
                                 _int, _vp, C.POINTER(LansHyper), _vp, _vp]),
+    "lancet_lans_step_mixed": (_int, [_vp, C.POINTER(_vp), _int, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),
+                                      _int, _int, _vp, C.POINTER(LansHyper), _vp, _vp]),
     "lancet_lans_plan_norms": (_int, [_vp, _vp, _vp]),
     "lancet_lans_plan_schedule": (_int, [_vp, C.POINTER(_int)]),
     "lancet_lans_plan_set_schedule": (_int, [_vp, _int]),
@@ -101,6 +103,7 @@ SIGNATURES = {
     "lancet_debug_scan_workspace_spin_limit": (_int, [_vp, _u32, _vp]),
     "lancet_debug_scan_workspace_epoch": (_int, [_vp, _u32, _vp]),
     "lancet_scan_workspace_init": (_int, [_vp, _sz, _vp]),
+    "lancet_scan_call_is_stateful": (_int, [_i64, _i64, _int, _u32, _int]),
     "lancet_scan_workspace_error": (_int, [_vp, _vp, C.POINTER(_int)]),
 }
 

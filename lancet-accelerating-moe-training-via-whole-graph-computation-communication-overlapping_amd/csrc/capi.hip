@@ -3,6 +3,7 @@
 #include "../../include/lancet_hip_debug.h"
 #include "common.hpp"
 #include "launchers.hpp"
+#include "scan.hpp"
 
 using namespace lancet;
 
@@ -86,6 +87,12 @@ extern "C" int lancet_scan_workspace_init(void* workspace, size_t workspace_byte
   if (misaligned(workspace, 8)) return LANCET_ERR_ALIGN;
   if (workspace_bytes < scan_workspace_bytes(0, 1, 1)) return LANCET_ERR_WORKSPACE;
   return rc(run_scan_ws_init(workspace, workspace_bytes, S_(stream)));
+}
+
+extern "C" int lancet_scan_call_is_stateful(int64_t S, int64_t E, int top_k, unsigned flags, int batch_prioritized) {
+  if (S < 0 || E < 1 || (top_k != 1 && top_k != 2)) return 0;
+  const int nsets = batch_prioritized ? 2 : top_k;
+  return scan_form(scan_num_tiles(S), static_cast<int64_t>(nsets) * E, nsets, (flags & LANCET_SCAN_LOOKBACK) != 0) == kScanLookback;
 }
 
 extern "C" int lancet_scan_workspace_error(void* workspace, lancet_stream_t stream, int* error_out) {

@@ -47,14 +47,17 @@ constexpr int kLansChunk = LANCET_LANS_CHUNK;  // elements per task: kLansChunk 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // control words of a plan (uint32): [0] next ticket of the resident kernel, [1] error (sticky: only
-// lancet_lans_plan_error clears it), [2] step epoch, [3] unused
-constexpr int kCtlTicket = 0, kCtlError = 1, kCtlEpoch = 2, kCtlWords = 4;
+// lancet_lans_plan_error clears it), [2] step epoch, [3] skip: the step that is running found the error word set
+// when it began and leaves every array alone (a step queued behind one that stalled must not build on its
+// half-applied state: moments written, parameters not)
+constexpr int kCtlTicket = 0, kCtlError = 1, kCtlEpoch = 2, kCtlSkip = 3, kCtlWords = 4;
 
 struct LansTables {
-  const float* const* g;  // [T] device pointers
+  const void* const* g;   // [T] device pointers; elements of the step's gradient type (fp32, bf16 or fp16)
   float* const* p;
   float* const* m;
   float* const* v;
+  void* const* plow;      // [T] device pointers or unused: 16-bit copies of the new parameters, written with p
   const int64_t* numel;        // [T]
   const int32_t* chunk_tensor; // [nchunks] tensor of a chunk slot, -1 = padding slot of a round
   const int32_t* tensor_first; // [T] first chunk slot of each tensor (its chunks are consecutive)
@@ -71,7 +74,7 @@ struct LansTables {
   int T;
   int nchunks;                 // chunk slots, padding included
   int nres;                    // slots [0, nres) are handed out by the resident kernel
-  uint32_t debug_flags;        // bit 0: the last arriver withholds the norms (exercises the bounded waits)
+  uint32_t debug_flags;        // bit 0: nothing is published (exercises the bounded waits); bit 1 is the host's
 };
 
 struct LansScalars {
@@ -199,46 +202,113 @@ __device__ __forceinline__ void bias_corrections(const LansScalars& sc, float& b
 __device__ __forceinline__ f32x4 ldn(const LANCET_GLOBAL f32x4* p) { return __builtin_nontemporal_load(p); }
 __device__ __forceinline__ void stn(LANCET_GLOBAL f32x4* p, f32x4 x) { __builtin_nontemporal_store(x, p); }
 
+// ---- gradients and parameter copies of a 16-bit model ---------------------------------------------------------
+// A mixed-precision trainer keeps fp32 master parameters and moments and a 16-bit model: the reference casts every
+// gradient to fp32 in front of the op and every new parameter back behind it (python/raf/optim/lans.py:256-257,
+// 285-288), two more sweeps over the state.  Here the step reads the gradients in the type they have (GT: the
+// conversion to fp32 is exact, so every later value is what the cast would have given) and writes the 16-bit copy
+// of a new parameter (PL; round to nearest even, what the cast does) with the fp32 one.  Four consecutive
+// elements are one access: 16 bytes of fp32, 8 bytes of a 16-bit type.
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+constexpr int kNoLowp = -1;  // PL: no 16-bit copy
+
+template <int GT>
+struct Grad {  // GT = LANCET_F32
+  typedef float S;   // storage type of an element
+  typedef f32x4 R;   // four consecutive elements as they are kept in registers
+  static constexpr uintptr_t kAlign4 = 15u;  // alignment mask of a 4-element access
+  static __device__ __forceinline__ float ld1(const LANCET_GLOBAL S* p) { return *p; }
+  static __device__ __forceinline__ R ldr4(const LANCET_GLOBAL S* p) { return ldn((const LANCET_GLOBAL f32x4*)p); }
+  static __device__ __forceinline__ f32x4 wide(const R& x) { return x; }
+  static __device__ __forceinline__ f32x4 ld4(const LANCET_GLOBAL S* p) { return ldr4(p); }
+};
+template <int GT>
+__device__ __forceinline__ float half_to_f32(uint32_t h) {
+  return GT == LANCET_BF16 ? bf16_to_f32(h) : f16_to_f32(h);
+}
+template <int GT>
+struct GradHalf {
+  typedef uint16_t S;
+  typedef u32x2 R;   // kept packed: half the registers of the fp32 form, widened where a value is used
+  static constexpr uintptr_t kAlign4 = 7u;
+  static __device__ __forceinline__ float ld1(const LANCET_GLOBAL S* p) { return half_to_f32<GT>(*p); }
+  static __device__ __forceinline__ R ldr4(const LANCET_GLOBAL S* p) {
+    return __builtin_nontemporal_load((const LANCET_GLOBAL u32x2*)p);
+  }
+  static __device__ __forceinline__ f32x4 wide(const R& x) {
+    return f32x4{half_to_f32<GT>(x.x & 0xffffu), half_to_f32<GT>(x.x >> 16), half_to_f32<GT>(x.y & 0xffffu),
+                 half_to_f32<GT>(x.y >> 16)};
+  }
+  static __device__ __forceinline__ f32x4 ld4(const LANCET_GLOBAL S* p) { return wide(ldr4(p)); }
+};
+template <>
+struct Grad<LANCET_BF16> : GradHalf<LANCET_BF16> {};
+template <>
+struct Grad<LANCET_F16> : GradHalf<LANCET_F16> {};
+
+template <int PL>
+__device__ __forceinline__ uint32_t f32_to_half(float f) {
+  return PL == LANCET_BF16 ? f32_to_bf16(f) : f32_to_f16(f);
+}
+// the 16-bit copy of four consecutive new parameters (nothing for PL = kNoLowp)
+template <int PL>
+__device__ __forceinline__ void st_lowp4(LANCET_GLOBAL uint16_t* p, f32x4 x) {
+  if (PL == kNoLowp) return;
+  u32x2 y;
+  y.x = (f32_to_half<PL>(x.x) & 0xffffu) | (f32_to_half<PL>(x.y) << 16);
+  y.y = (f32_to_half<PL>(x.z) & 0xffffu) | (f32_to_half<PL>(x.w) << 16);
+  __builtin_nontemporal_store(y, (LANCET_GLOBAL u32x2*)p);
+}
+template <int PL>
+__device__ __forceinline__ void st_lowp1(LANCET_GLOBAL uint16_t* p, float x) {
+  if (PL != kNoLowp) *p = static_cast<uint16_t>(f32_to_half<PL>(x));
+}
+
 // ---- the three phases on one chunk, executed by one workgroup ------------------------------
 // phase 1: sum of squares of g (L2NormFunctor, multi_tensor_lans.cu:95-167); valid on thread 0.
 // (The sum of squares of p is not needed before phase 3 and is taken in phase 2, which reads p anyway.)
+template <int GT>
 __device__ __forceinline__ float chunk_norm_g(const LansTables& t, const ChunkView& c, float* s_red) {
-  const LANCET_GLOBAL float* g = as_global(t.g[c.tensor] + c.begin);
+  typedef Grad<GT> G;
+  const LANCET_GLOBAL typename G::S* g = as_global(static_cast<const typename G::S*>(t.g[c.tensor]) + c.begin);
   float ag = 0.f;
   int scalar_from = 0;
-  if (vec_ok(g, g, g, g)) {
+  if (((uintptr_t)g & G::kAlign4) == 0) {
     const int nv = c.n / 4;
-    const LANCET_GLOBAL f32x4* g4 = (const LANCET_GLOBAL f32x4*)g;
 #pragma unroll 8
     for (int i = threadIdx.x; i < nv; i += kLansThreads) {
-      const f32x4 x = ldn(g4 + i);
+      const f32x4 x = G::ld4(g + 4 * i);
       ag += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
     }
     scalar_from = nv * 4;
   }
-  for (int i = scalar_from + threadIdx.x; i < c.n; i += kLansThreads) ag += g[i] * g[i];
+  for (int i = scalar_from + threadIdx.x; i < c.n; i += kLansThreads) {
+    const float x = G::ld1(g + i);
+    ag += x * x;
+  }
   return block_sum(ag, s_red);
 }
 
 // phase 2: moments + sums of squares of p and of the two updates (LANSStage1Functor :207-322 and the
 // l2norm sweeps around it, :428-441); sums valid on thread 0
+template <int GT>
 __device__ __forceinline__ void chunk_moments(const LansTables& t, const ChunkView& c, const LansElem& el,
                                               float* s_red, float& sum_p, float& sum_um, float& sum_ug) {
-  const LANCET_GLOBAL float* g = as_global(t.g[c.tensor] + c.begin);
+  typedef Grad<GT> G;
+  const LANCET_GLOBAL typename G::S* g = as_global(static_cast<const typename G::S*>(t.g[c.tensor]) + c.begin);
   const LANCET_GLOBAL float* p = as_global(t.p[c.tensor] + c.begin);
   LANCET_GLOBAL float* m = as_global(t.m[c.tensor] + c.begin);
   LANCET_GLOBAL float* v = as_global(t.v[c.tensor] + c.begin);
   float ap = 0.f, am = 0.f, ag = 0.f;
   int scalar_from = 0;
-  if (vec_ok(g, p, m, v)) {
+  if (vec_ok(p, p, m, v) && ((uintptr_t)g & G::kAlign4) == 0) {
     const int nv = c.n / 4;
-    const LANCET_GLOBAL f32x4* g4 = (const LANCET_GLOBAL f32x4*)g;
     const LANCET_GLOBAL f32x4* p4 = (const LANCET_GLOBAL f32x4*)p;
     LANCET_GLOBAL f32x4* m4 = (LANCET_GLOBAL f32x4*)m;
     LANCET_GLOBAL f32x4* v4 = (LANCET_GLOBAL f32x4*)v;
 #pragma unroll 2
     for (int i = threadIdx.x; i < nv; i += kLansThreads) {
-      const f32x4 xg = ldn(g4 + i), xp = ldn(p4 + i);
+      const f32x4 xg = G::ld4(g + 4 * i), xp = ldn(p4 + i);
       f32x4 xm = ldn(m4 + i), xv = ldn(v4 + i);
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
@@ -258,7 +328,7 @@ __device__ __forceinline__ void chunk_moments(const LansTables& t, const ChunkVi
     scalar_from = nv * 4;
   }
   for (int i = scalar_from + threadIdx.x; i < c.n; i += kLansThreads) {
-    const float sg = el.scaled_grad(g[i], p[i]);
+    const float sg = el.scaled_grad(G::ld1(g + i), p[i]);
     float mm = m[i], vv = v[i], um, ug;
     el.moments(sg, mm, vv);
     el.updates(sg, p[i], mm, vv, um, ug);
@@ -274,26 +344,28 @@ __device__ __forceinline__ void chunk_moments(const LansTables& t, const ChunkVi
 }
 
 // phase 3: trust ratios and parameter update (LANSStage2Functor :326-399)
+template <int GT, int PL>
 __device__ __forceinline__ void chunk_update(const LansTables& t, const ChunkView& c, const LansElem& el,
                                              const LansScalars& sc, float pn, float umn, float ugn) {
+  typedef Grad<GT> G;
   float ratio_m = (umn != 0.f && pn != 0.f) ? sc.lr * (pn / umn) : sc.lr;
   float ratio_g = (ugn != 0.f && pn != 0.f) ? sc.lr * (pn / ugn) : sc.lr;
   ratio_m *= sc.beta1;
   ratio_g *= sc.beta3;
-  const LANCET_GLOBAL float* g = as_global(t.g[c.tensor] + c.begin);
+  const LANCET_GLOBAL typename G::S* g = as_global(static_cast<const typename G::S*>(t.g[c.tensor]) + c.begin);
+  LANCET_GLOBAL uint16_t* pl = PL == kNoLowp ? nullptr : as_global(static_cast<uint16_t*>(t.plow[c.tensor]) + c.begin);
   LANCET_GLOBAL float* p = as_global(t.p[c.tensor] + c.begin);
   const LANCET_GLOBAL float* m = as_global(t.m[c.tensor] + c.begin);
   const LANCET_GLOBAL float* v = as_global(t.v[c.tensor] + c.begin);
   int scalar_from = 0;
-  if (vec_ok(g, p, m, v)) {
+  if (vec_ok(p, p, m, v) && ((uintptr_t)g & G::kAlign4) == 0 && (PL == kNoLowp || ((uintptr_t)pl & 7u) == 0)) {
     const int nv = c.n / 4;
-    const LANCET_GLOBAL f32x4* g4 = (const LANCET_GLOBAL f32x4*)g;
     LANCET_GLOBAL f32x4* p4 = (LANCET_GLOBAL f32x4*)p;
     const LANCET_GLOBAL f32x4* m4 = (const LANCET_GLOBAL f32x4*)m;
     const LANCET_GLOBAL f32x4* v4 = (const LANCET_GLOBAL f32x4*)v;
 #pragma unroll 2
     for (int i = threadIdx.x; i < nv; i += kLansThreads) {
-      const f32x4 xg = ldn(g4 + i), xm = ldn(m4 + i), xv = ldn(v4 + i);
+      const f32x4 xg = G::ld4(g + 4 * i), xm = ldn(m4 + i), xv = ldn(v4 + i);
       f32x4 xp = ldn(p4 + i);
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
@@ -304,15 +376,18 @@ __device__ __forceinline__ void chunk_update(const LansTables& t, const ChunkVie
         xp[k] = xp[k] - (ratio_m * um) - (ratio_g * ug);
       }
       stn(p4 + i, xp);
+      st_lowp4<PL>(pl + 4 * i, xp);
     }
     scalar_from = nv * 4;
   }
   for (int i = scalar_from + threadIdx.x; i < c.n; i += kLansThreads) {
 #pragma clang fp contract(off)
-    const float sg = el.scaled_grad(g[i], p[i]);
+    const float sg = el.scaled_grad(G::ld1(g + i), p[i]);
     float um, ug;
     el.updates(sg, p[i], m[i], v[i], um, ug);
-    p[i] = p[i] - (ratio_m * um) - (ratio_g * ug);
+    const float np = p[i] - (ratio_m * um) - (ratio_g * ug);
+    p[i] = np;
+    st_lowp1<PL>(pl + i, np);
   }
 }
 
@@ -330,8 +405,19 @@ __device__ __forceinline__ float wave_norm(int lo, int hi, Get get) {
 // =======================================================================================
 // schedule "sweeps": three launches + two per-tensor reductions
 // =======================================================================================
+// A step begins by looking at the plan's sticky error word: if an earlier step gave up a wait, its tensors hold
+// new moments and old parameters, and a step queued behind it (enqueued before the host could see the failure, or
+// replayed from a graph) must not advance them again.  Such a step is skipped as a whole: every kernel of it reads
+// the skip word first and leaves when it is set, until lancet_lans_plan_error has cleared the error.
+__device__ __forceinline__ bool step_is_skipped(const LansTables& t) {
+  return __builtin_amdgcn_readfirstlane(static_cast<int>(ld_agent(t.ctl + kCtlSkip))) != 0;
+}
+
 __global__ void lans_prepare_kernel(LansTables t, LansScalars sc) {
-  if (threadIdx.x == 0 && blockIdx.x == 0) bias_corrections(sc, t.consts[0], t.consts[1]);
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    t.ctl[kCtlSkip] = ld_agent(t.ctl + kCtlError) != 0u ? 1u : 0u;
+    bias_corrections(sc, t.consts[0], t.consts[1]);
+  }
 }
 
 // The sweeps hand every chunk to kSweepSplit workgroups (a slice of kLansChunk / kSweepSplit elements each:
@@ -358,12 +444,14 @@ __device__ __forceinline__ ChunkView slice_view(const LansTables& t, int chunk_b
 // The sweep over g covers chunks [chunk_base, chunk_base + gridDim.x), the other two
 // [chunk_base, chunk_base + gridDim.x / kSweepSplit): all of them, or the ones the resident
 // kernel takes (first sweep only), or the ones it leaves (tensors too large for it).
+template <int GT>
 __global__ __launch_bounds__(kLansThreads) void lans_norm_g_kernel(LansTables t, int chunk_base) {
   __shared__ float s_red[kLansThreads / kWave];
+  if (step_is_skipped(t)) return;
   const int chunk = chunk_base + blockIdx.x;  // a whole chunk per workgroup: this sweep only reads, and splitting it costs more in reductions than it gains
   const ChunkView c = chunk_view(t, chunk);
   if (c.tensor < 0) return;  // padding slot (uniform over the workgroup)
-  const float sg = chunk_norm_g(t, c, s_red);
+  const float sg = chunk_norm_g<GT>(t, c, s_red);
   if (threadIdx.x == 0) t.partial[chunk] = sg;
 }
 
@@ -371,6 +459,7 @@ __global__ __launch_bounds__(kLansThreads) void lans_norm_g_kernel(LansTables t,
 // split: partial sums per chunk (1 after the sweep over g, kSweepSplit after the moments sweep)
 __global__ __launch_bounds__(kLansThreads) void lans_reduce_kernel(LansTables t, int first_norm, int tensor_base,
                                                                    int tensor_end, int count, int split) {
+  if (step_is_skipped(t)) return;  // the norms of the last step that ran stay
   const int tensor = tensor_base + blockIdx.x * (kLansThreads / kWave) + threadIdx.x / kWave;
   if (tensor >= tensor_end) return;
   const int lo = t.tensor_first[tensor], hi = lo + t.tensor_chunks[tensor];
@@ -381,14 +470,16 @@ __global__ __launch_bounds__(kLansThreads) void lans_reduce_kernel(LansTables t,
   }
 }
 
+template <int GT>
 __global__ __launch_bounds__(kLansThreads) void lans_moments_kernel(LansTables t, LansScalars sc, int chunk_base) {
   __shared__ float s_red[kLansThreads / kWave];
+  if (step_is_skipped(t)) return;
   int slot;
   const ChunkView c = slice_view(t, chunk_base, slot);
   if (c.tensor < 0) return;  // padding slot (uniform over the workgroup)
   const LansElem el = make_elem(sc, t.norms[c.tensor], t.consts[0], t.consts[1]);
   float sp, sm, sg;
-  chunk_moments(t, c, el, s_red, sp, sm, sg);
+  chunk_moments<GT>(t, c, el, s_red, sp, sm, sg);
   if (threadIdx.x == 0) {
     const size_t row = static_cast<size_t>(t.nchunks) * kSweepSplit;
     t.partial[slot] = sp;
@@ -397,17 +488,20 @@ __global__ __launch_bounds__(kLansThreads) void lans_moments_kernel(LansTables t
   }
 }
 
+template <int GT, int PL>
 __global__ __launch_bounds__(kLansThreads) void lans_update_kernel(LansTables t, LansScalars sc, int chunk_base) {
+  if (step_is_skipped(t)) return;
   int slot;
   const ChunkView c = slice_view(t, chunk_base, slot);
   if (c.tensor < 0) return;
   const LansElem el = make_elem(sc, t.norms[c.tensor], t.consts[0], t.consts[1]);
-  chunk_update(t, c, el, sc, t.norms[1 * t.T + c.tensor], t.norms[2 * t.T + c.tensor], t.norms[3 * t.T + c.tensor]);
+  chunk_update<GT, PL>(t, c, el, sc, t.norms[1 * t.T + c.tensor], t.norms[2 * t.T + c.tensor], t.norms[3 * t.T + c.tensor]);
 }
 
 // ||g|| per tensor supplied by the caller (in the order of its lists) instead of the sweep over g
 __global__ void lans_take_grad_norms_kernel(LansTables t) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (step_is_skipped(t)) return;
   if (i < t.T) t.norms[i] = t.grad_norms[t.order[i]];
 }
 
@@ -520,6 +614,15 @@ __device__ __forceinline__ f32x4 ld_chunk4(const LANCET_GLOBAL float* a, int k, 
 __device__ __forceinline__ void st_chunk4(LANCET_GLOBAL float* a, int k, f32x4 x, int wave) {
   __builtin_nontemporal_store(x, (LANCET_GLOBAL f32x4*)(a + k * (4 * kWave) + lane_offset(wave)));
 }
+// the same four elements of a gradient chunk in its own type, as fp32, and of the 16-bit parameter copy
+template <int GT>
+__device__ __forceinline__ typename Grad<GT>::R ld_grad4(const LANCET_GLOBAL typename Grad<GT>::S* a, int k, int wave) {
+  return Grad<GT>::ldr4(a + k * (4 * kWave) + lane_offset(wave));
+}
+template <int PL>
+__device__ __forceinline__ void st_lowp_chunk4(LANCET_GLOBAL uint16_t* a, int k, f32x4 x, int wave) {
+  st_lowp4<PL>(a + k * (4 * kWave) + lane_offset(wave), x);
+}
 
 // Thread 0: publishes the N chunk sums a[] of slot s as words first .. first+N-1 (fire and forget).
 template <int N>
@@ -560,9 +663,9 @@ __device__ __forceinline__ void gather_take(const LansScalars& sc, const Slot& s
 // around it, :428-441) of a chunk whose g sits in registers.  m and v are written; u_m, u_g stay in
 // registers and p in LDS for stage U.  The loads of float4 k+1 are issued before the stores of float4 k:
 // memory operations of a wave complete in order, so a load behind a store would wait for it.
-template <int PAR>
+template <int PAR, int GT>
 __device__ __forceinline__ void moments_chunk(const LansTables& t, const Slot& s, const LansElem& el,
-                                              const f32x4 (&g)[kVecPerThread], f32x4 (&um)[kVecPerThread],
+                                              const typename Grad<GT>::R (&g)[kVecPerThread], f32x4 (&um)[kVecPerThread],
                                               f32x4 (&ug)[kVecPerThread], PipeShared& sh, float (&a)[3], uint32_t ticket, int wave) {
   const LANCET_GLOBAL float* p = as_global(ld_table(t.p + s.tensor) + s.begin);
   LANCET_GLOBAL float* m = as_global(ld_table(t.m + s.tensor) + s.begin);
@@ -589,9 +692,10 @@ __device__ __forceinline__ void moments_chunk(const LansTables& t, const Slot& s
       nv[k % kPrefetch] = ld_chunk4(v, k + kPrefetch, wave);
     }
     sh.p[PAR][k][fresh_tid(wave)] = xp;
+    const f32x4 xg = Grad<GT>::wide(g[k]);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const float sg = el.scaled_grad(g[k][j], xp[j]);
+      const float sg = el.scaled_grad(xg[j], xp[j]);
       float mm = xm[j], vv = xv[j], u0, u1;
       el.moments(sg, mm, vv);
       el.updates(sg, xp[j], mm, vv, u0, u1);
@@ -709,10 +813,10 @@ __device__ __forceinline__ void forget(f32x4 (&a)[kVecPerThread], f32x4 (&b)[kVe
 // next pass (the norm is carried there in LDS; a register carried over would be looked at behind stage U's
 // stores).  Only a sum that is still missing then is polled for.  Returns false when the workgroup holds
 // nothing any more.
-template <int PAR>
+template <int PAR, int GT, int PL>
 __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansScalars& sc, float bc1, float bc2,
                                               Slot& s0, Slot& s1, Slot& s2,
-                                              f32x4 (&g)[kVecPerThread],
+                                              typename Grad<GT>::R (&g)[kVecPerThread],
                                               f32x4 (&um_new)[kVecPerThread], f32x4 (&ug_new)[kVecPerThread],
                                               const f32x4 (&um_old)[kVecPerThread], const f32x4 (&ug_old)[kVecPerThread],
                                               PipeShared& sh, int wave) {
@@ -736,7 +840,7 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
     float a[3] = {0.f, 0.f, 0.f};
     if (LIKELY(!bad)) {
       const LansElem el = make_elem(sc, g_norm, bc1, bc2);
-      moments_chunk<PAR>(t, s1, el, g, um_new, ug_new, sh, a, ticket, wave);
+      moments_chunk<PAR, GT>(t, s1, el, g, um_new, ug_new, sh, a, ticket, wave);
     } else {
       if (is_first(wave)) sh.chunk = static_cast<int>(ticket);
       s1.dead = 1;  // ||g|| is unknown: the chunk is left as it is, and so will its tensor's parameters be
@@ -793,9 +897,10 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
   // the sums other workgroups have published: read as late as possible, and still back before anything waits
   // for them alone
   if (LIKELY(s3.real())) {
-    const LANCET_GLOBAL float* src = as_global(ld_table(t.g + s3.tensor) + s3.begin);
+    typedef typename Grad<GT>::S GS;
+    const LANCET_GLOBAL GS* src = as_global(static_cast<const GS*>(ld_table(t.g + s3.tensor)) + s3.begin);
 #pragma unroll
-    for (int k = 0; k < kVecPerThread; ++k) g[k] = ld_chunk4(src, k, wave);
+    for (int k = 0; k < kVecPerThread; ++k) g[k] = ld_grad4<GT>(src, k, wave);
   }
   if (LIKELY(need_u)) {
 #pragma unroll
@@ -805,7 +910,10 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
   if (LIKELY(s3.real())) {
     float a = 0.f;
 #pragma unroll
-    for (int k = 0; k < kVecPerThread; ++k) a += g[k].x * g[k].x + g[k].y * g[k].y + g[k].z * g[k].z + g[k].w * g[k].w;
+    for (int k = 0; k < kVecPerThread; ++k) {
+      const f32x4 x = Grad<GT>::wide(g[k]);
+      a += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+    }
     a = wave_sum(a);
     if (fresh_lane() == 0) sh.red[0][wave] = a;
   }
@@ -868,6 +976,8 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
     ratio_m = uniform(ratio_m * sc.beta1);
     ratio_g = uniform(ratio_g * sc.beta3);
     LANCET_GLOBAL float* p = as_global(ld_table(t.p + s0.tensor) + s0.begin);
+    LANCET_GLOBAL uint16_t* pl = nullptr;
+    if (PL != kNoLowp) pl = as_global(static_cast<uint16_t*>(ld_table(t.plow + s0.tensor)) + s0.begin);
 #pragma unroll
     for (int k = 0; k < kVecPerThread; ++k) {
       f32x4 xp = sh.p[PAR ^ 1][k][fresh_tid(wave)];
@@ -877,6 +987,7 @@ __device__ __forceinline__ bool pipeline_pass(const LansTables& t, const LansSca
         xp[j] = xp[j] - (ratio_m * um_old[k][j]) - (ratio_g * ug_old[k][j]);
       }
       st_chunk4(p, k, xp, wave);
+      st_lowp_chunk4<PL>(pl, k, xp, wave);
     }
   }
   // ---- the slots move up ------------------------------------------------------------------------------------
@@ -904,18 +1015,21 @@ __global__ __launch_bounds__(kLansThreads) void lans_begin_kernel(LansTables t, 
   if (threadIdx.x == 0) {
     *ep = e == 0u ? 1u : e;
     t.ctl[kCtlTicket] = 0u;
+    t.ctl[kCtlSkip] = ld_agent(t.ctl + kCtlError) != 0u ? 1u : 0u;  // step_is_skipped
     bias_corrections(sc, t.consts[0], t.consts[1]);
   }
 }
 
+template <int GT, int PL>
 __global__ __launch_bounds__(kLansThreads, kResidentWavesPerSimd) void lans_resident_kernel(LansTables t, LansScalars sc) {
   __shared__ PipeShared sh;
+  if (step_is_skipped(t)) return;
   const int wave = static_cast<int>(static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(threadIdx.x)) / kWave);
   sc.epoch = __builtin_amdgcn_readfirstlane(t.ctl[kCtlEpoch]);
   const float bc1 = uniform(t.consts[0]), bc2 = uniform(t.consts[1]);  // lans_begin_kernel
   // s0: between stages M and U; s1, s2: between stages N and M, s1 the older.  Register arrays rotate with
   // the slots: g of s1 / s2 alternates between ga and gb, the updates between parity 0 and 1.
-  f32x4 ga[kVecPerThread], gb[kVecPerThread];
+  typename Grad<GT>::R ga[kVecPerThread], gb[kVecPerThread];
   f32x4 um0[kVecPerThread], ug0[kVecPerThread], um1[kVecPerThread], ug1[kVecPerThread];
   Slot s0, s1, s2;
   s0.chunk = s1.chunk = s2.chunk = -1;
@@ -929,8 +1043,8 @@ __global__ __launch_bounds__(kLansThreads, kResidentWavesPerSimd) void lans_resi
   // the first two passes find empty slots (their stages M and U have nothing to do) and fill the pipeline;
   // every pass draws a ticket, tickets run out, and every wait is bounded: all workgroups leave
   for (;;) {
-    if (!pipeline_pass<0>(t, sc, bc1, bc2, s0, s1, s2, ga, um0, ug0, um1, ug1, sh, wave)) break;
-    if (!pipeline_pass<1>(t, sc, bc1, bc2, s0, s1, s2, gb, um1, ug1, um0, ug0, sh, wave)) break;
+    if (!pipeline_pass<0, GT, PL>(t, sc, bc1, bc2, s0, s1, s2, ga, um0, ug0, um1, ug1, sh, wave)) break;
+    if (!pipeline_pass<1, GT, PL>(t, sc, bc1, bc2, s0, s1, s2, gb, um1, ug1, um0, ug0, sh, wave)) break;
   }
 }
 
@@ -947,7 +1061,7 @@ struct lancet_lans_plan {
   int T;
   int nchunks;                      // chunk slots, padding included
   std::vector<int64_t> numels;
-  std::vector<const void*> shadow;  // last uploaded 4T pointers
+  std::vector<const void*> shadow;  // last uploaded 5T pointers (g, p, m, v, 16-bit parameter copies or null)
   void* dev_block;                  // one allocation holding every table
   void** h_ptrs;                    // pinned staging for the pointer tables
   uint32_t* h_status;               // pinned word the resident kernel sets with its error word
@@ -1044,7 +1158,7 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
   pl->magic = kPlanMagic;
   pl->T = T;
   pl->numels.assign(numels, numels + T);
-  pl->shadow.assign(4 * static_cast<size_t>(T), nullptr);
+  pl->shadow.assign(5 * static_cast<size_t>(T), nullptr);
   pl->dev_block = nullptr;
   pl->h_ptrs = nullptr;
   pl->h_status = nullptr;
@@ -1061,7 +1175,13 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
   for (int i = 0; i < T; ++i) pl->max_tensor_chunks = std::max(pl->max_tensor_chunks, chunks_of(numels[i]));
   if (err == hipSuccess) {
     int per_cu = 0;
-    err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lans_resident_kernel, kLansThreads, 0);
+    // every variant of the kernel has the same launch bounds and LDS; the grid follows the variant that reads and
+    // writes the most (16-bit gradients in, 16-bit parameter copies out)
+    err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lans_resident_kernel<LANCET_F32, kNoLowp>, kLansThreads, 0);
+    int per_cu_mixed = 0;
+    if (err == hipSuccess)
+      err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_mixed, lans_resident_kernel<LANCET_BF16, LANCET_BF16>, kLansThreads, 0);
+    per_cu = std::min(per_cu, per_cu_mixed);
     pl->resident_grid = per_cu * cus;
   }
   // a tensor's chunks fit one round, so the kernel drains with half of its workgroups on the chip
@@ -1079,7 +1199,7 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
   const size_t n = static_cast<size_t>(pl->nchunks);
   const size_t n1 = n ? n : 1;
   size_t off = 0;
-  const size_t o_ptrs = off;      off = align_up(off + 4 * T * sizeof(void*), 256);
+  const size_t o_ptrs = off;      off = align_up(off + 5 * T * sizeof(void*), 256);
   const size_t o_numel = off;     off = align_up(off + T * sizeof(int64_t), 256);
   const size_t o_ctensor = off;   off = align_up(off + n1 * sizeof(int32_t), 256);
   const size_t o_first = off;     off = align_up(off + T * sizeof(int32_t), 256);
@@ -1093,7 +1213,7 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
   const size_t o_order = off;     off = align_up(off + T * sizeof(int32_t), 256);
   pl->words_bytes = 4 * (n1 + T) * sizeof(uint64_t);
   if (err == hipSuccess) err = hipMalloc(&pl->dev_block, off);
-  if (err == hipSuccess) err = hipHostMalloc(reinterpret_cast<void**>(&pl->h_ptrs), 4 * T * sizeof(void*), hipHostMallocDefault);
+  if (err == hipSuccess) err = hipHostMalloc(reinterpret_cast<void**>(&pl->h_ptrs), 5 * T * sizeof(void*), hipHostMallocDefault);
   if (err == hipSuccess) err = hipHostMalloc(reinterpret_cast<void**>(&pl->h_status), 64, hipHostMallocDefault);
   if (err == hipSuccess) err = hipEventCreateWithFlags(&pl->upload_done, hipEventDisableTiming);
   if (err == hipSuccess) {
@@ -1116,10 +1236,11 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
     t.host_status = nullptr;
     if (err == hipSuccess) err = hipHostGetDevicePointer(reinterpret_cast<void**>(&t.host_status), pl->h_status, 0);
     void** dptrs = reinterpret_cast<void**>(base + o_ptrs);
-    t.g = reinterpret_cast<const float* const*>(dptrs);
+    t.g = reinterpret_cast<const void* const*>(dptrs);
     t.p = reinterpret_cast<float* const*>(dptrs + T);
     t.m = reinterpret_cast<float* const*>(dptrs + 2 * T);
     t.v = reinterpret_cast<float* const*>(dptrs + 3 * T);
+    t.plow = reinterpret_cast<void* const*>(dptrs + 4 * T);
     t.numel = reinterpret_cast<const int64_t*>(base + o_numel);
     t.chunk_tensor = reinterpret_cast<const int32_t*>(base + o_ctensor);
     t.tensor_first = reinterpret_cast<const int32_t*>(base + o_first);
@@ -1163,32 +1284,55 @@ extern "C" int lancet_lans_plan_norms(lancet_lans_plan_t pl, float* norms, lance
   return static_cast<int>(hipGetLastError());
 }
 
-extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, float* const* p,
-                                float* const* m, float* const* v, int step_host,
-                                const float* step_dev, const lancet_lans_hyper* h,
-                                const float* grad_norms, lancet_stream_t stream) {
+namespace {
+
+// GT / PL as compile-time constants inside `...` for the run-time codes gt (LANCET_F32 / _BF16 / _F16) and pl (the
+// same 16-bit codes, or kNoLowp)
+#define LANS_TYPE_SWITCH(gt, pl, ...)                                                                      \
+  switch ((gt) * 4 + ((pl) == kNoLowp ? 0 : (pl))) {                                                       \
+    case LANCET_F32 * 4 + 0: { constexpr int GT = LANCET_F32, PL = kNoLowp; (void)PL; __VA_ARGS__; } break;          \
+    case LANCET_F32 * 4 + LANCET_BF16: { constexpr int GT = LANCET_F32, PL = LANCET_BF16; (void)PL; __VA_ARGS__; } break;   \
+    case LANCET_F32 * 4 + LANCET_F16: { constexpr int GT = LANCET_F32, PL = LANCET_F16; (void)PL; __VA_ARGS__; } break;     \
+    case LANCET_BF16 * 4 + 0: { constexpr int GT = LANCET_BF16, PL = kNoLowp; (void)PL; __VA_ARGS__; } break;        \
+    case LANCET_BF16 * 4 + LANCET_BF16: { constexpr int GT = LANCET_BF16, PL = LANCET_BF16; (void)PL; __VA_ARGS__; } break; \
+    case LANCET_BF16 * 4 + LANCET_F16: { constexpr int GT = LANCET_BF16, PL = LANCET_F16; (void)PL; __VA_ARGS__; } break;   \
+    case LANCET_F16 * 4 + 0: { constexpr int GT = LANCET_F16, PL = kNoLowp; (void)PL; __VA_ARGS__; } break;          \
+    case LANCET_F16 * 4 + LANCET_BF16: { constexpr int GT = LANCET_F16, PL = LANCET_BF16; (void)PL; __VA_ARGS__; } break;   \
+    default: { constexpr int GT = LANCET_F16, PL = LANCET_F16; (void)PL; __VA_ARGS__; } break;                       \
+  }
+
+int lans_step_impl(lancet_lans_plan_t pl, const void* const* g, int g_dtype, float* const* p, float* const* m,
+                   float* const* v, void* const* p_lowp, int lowp_dtype, int step_host, const float* step_dev,
+                   const lancet_lans_hyper* h, const float* grad_norms, lancet_stream_t stream) {
   if (!pl || pl->magic != kPlanMagic) return LANCET_ERR_PLAN;
   if (!g || !p || !m || !v || !h) return LANCET_ERR_NULL;
+  if (g_dtype != LANCET_F32 && g_dtype != LANCET_BF16 && g_dtype != LANCET_F16) return LANCET_ERR_DTYPE;
+  if (p_lowp && lowp_dtype != LANCET_BF16 && lowp_dtype != LANCET_F16) return LANCET_ERR_DTYPE;
+  const int plt = p_lowp ? lowp_dtype : kNoLowp;
   if (!step_dev && step_host < 1) return LANCET_ERR_SHAPE;
   if (h->mode != 0 && h->mode != 1) return LANCET_ERR_SHAPE;
   int current = -1;
   if (hipGetDevice(&current) != hipSuccess || current != pl->device) return LANCET_ERR_PLAN;  // tables live on pl->device
   // an earlier step of this plan gave up a wait: nothing more is launched until lancet_lans_plan_error
-  // has been called (the word is written by the device; reading it needs no synchronisation)
-  if (__atomic_load_n(pl->h_status, __ATOMIC_RELAXED) != 0u) return LANCET_ERR_STALLED;
+  // has been called (the word is written by the device; reading it needs no synchronisation).  Steps that were
+  // queued before the word arrived skip themselves on the device (step_is_skipped).
+  if (!(pl->tables.debug_flags & 2u) && __atomic_load_n(pl->h_status, __ATOMIC_RELAXED) != 0u) return LANCET_ERR_STALLED;
   if (reinterpret_cast<uintptr_t>(grad_norms) & 3u) return LANCET_ERR_ALIGN;
   const int T = pl->T;
   hipStream_t st = static_cast<hipStream_t>(stream);
+  const uintptr_t g_elem = g_dtype == LANCET_F32 ? 3u : 1u;   // alignment masks: one element, four elements
+  const uintptr_t g_vec = g_dtype == LANCET_F32 ? 15u : 7u;
   bool changed = false;
-  bool aligned16 = true;  // the resident kernel moves float4s: a step in which one of its tensors is not 16-byte aligned runs as sweeps
+  bool aligned16 = true;  // the resident kernel moves four elements per access: a step in which one of its tensors is not aligned to that runs as sweeps
   for (int i = 0; i < T; ++i) {
-    if (pl->numels[i] > 0 && (!g[i] || !p[i] || !m[i] || !v[i])) return LANCET_ERR_NULL;
-    const uintptr_t bits = reinterpret_cast<uintptr_t>(g[i]) | reinterpret_cast<uintptr_t>(p[i]) |
-                           reinterpret_cast<uintptr_t>(m[i]) | reinterpret_cast<uintptr_t>(v[i]);
-    if (bits & 3u) return LANCET_ERR_ALIGN;
-    aligned16 = aligned16 && (!pl->is_resident[i] || (bits & 15u) == 0);
+    void* const lo = p_lowp ? p_lowp[i] : nullptr;
+    if (pl->numels[i] > 0 && (!g[i] || !p[i] || !m[i] || !v[i] || (p_lowp && !lo))) return LANCET_ERR_NULL;
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(p[i]) | reinterpret_cast<uintptr_t>(m[i]) | reinterpret_cast<uintptr_t>(v[i]);
+    const uintptr_t gbits = reinterpret_cast<uintptr_t>(g[i]), lbits = reinterpret_cast<uintptr_t>(lo);
+    if ((bits & 3u) || (gbits & g_elem) || (lbits & 1u)) return LANCET_ERR_ALIGN;
+    aligned16 = aligned16 && (!pl->is_resident[i] || ((bits & 15u) == 0 && (gbits & g_vec) == 0 && (lbits & 7u) == 0));
     changed = changed || pl->shadow[i] != g[i] || pl->shadow[T + i] != p[i] ||
-              pl->shadow[2 * T + i] != m[i] || pl->shadow[3 * T + i] != v[i];
+              pl->shadow[2 * T + i] != m[i] || pl->shadow[3 * T + i] != v[i] || pl->shadow[4 * T + i] != lo;
   }
   hipError_t err = hipSuccess;
   if (changed) {
@@ -1198,18 +1342,20 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
       if (err != hipSuccess) return static_cast<int>(err);
     }
     for (int i = 0; i < T; ++i) {
-      pl->shadow[i] = const_cast<float*>(g[i]);
+      pl->shadow[i] = g[i];
       pl->shadow[T + i] = p[i];
       pl->shadow[2 * T + i] = m[i];
       pl->shadow[3 * T + i] = v[i];
+      pl->shadow[4 * T + i] = p_lowp ? p_lowp[i] : nullptr;
       const int u = pl->order[i];  // the plan's i-th tensor is the caller's u-th
-      pl->h_ptrs[i] = const_cast<float*>(g[u]);
+      pl->h_ptrs[i] = const_cast<void*>(g[u]);
       pl->h_ptrs[T + i] = p[u];
       pl->h_ptrs[2 * T + i] = m[u];
       pl->h_ptrs[3 * T + i] = v[u];
+      pl->h_ptrs[4 * T + i] = p_lowp ? p_lowp[u] : nullptr;
     }
     err = hipMemcpyAsync(pl->dev_block, pl->h_ptrs,
-                         4 * static_cast<size_t>(T) * sizeof(void*), hipMemcpyHostToDevice, st);
+                         5 * static_cast<size_t>(T) * sizeof(void*), hipMemcpyHostToDevice, st);
     if (err == hipSuccess) err = hipEventRecord(pl->upload_done, st);
     if (err != hipSuccess) return static_cast<int>(err);
     pl->upload_pending = true;
@@ -1231,15 +1377,18 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
   t.grad_norms = grad_norms;
   sc.spin_limit = pl->spin_limit;
   sc.epoch = 0;
-  if (grad_norms) lans_take_grad_norms_kernel<<<(T + 255) / 256, 256, 0, st>>>(t);
   // slots [0, chunk_base) and tensors [0, tensor_base) go through the resident kernel, the rest
   // (everything, under the sweeps schedule) through the three sweeps
   int chunk_base = 0, tensor_base = 0;
   pl->last_resident_slots = 0;
-  if (pl->schedule == LANCET_LANS_RESIDENT && pl->n_res_chunks > 0 && aligned16) {
-    lans_begin_kernel<<<1, kLansThreads, 0, st>>>(t, sc, pl->words_bytes / sizeof(uint64_t));
+  const bool resident = pl->schedule == LANCET_LANS_RESIDENT && pl->n_res_chunks > 0 && aligned16;
+  // the first kernel of a step forms the bias corrections and decides whether the step runs at all
+  if (resident) lans_begin_kernel<<<1, kLansThreads, 0, st>>>(t, sc, pl->words_bytes / sizeof(uint64_t));
+  else lans_prepare_kernel<<<1, 64, 0, st>>>(t, sc);
+  if (grad_norms) lans_take_grad_norms_kernel<<<(T + 255) / 256, 256, 0, st>>>(t);
+  if (resident) {
     const int grid = std::min(pl->resident_grid, pl->n_res_chunks);
-    lans_resident_kernel<<<grid, kLansThreads, 0, st>>>(t, sc);
+    LANS_TYPE_SWITCH(g_dtype, plt, (lans_resident_kernel<GT, PL><<<grid, kLansThreads, 0, st>>>(t, sc)))
     chunk_base = pl->n_res_chunks;
     tensor_base = pl->n_res_tensors;
     pl->last_resident_slots = chunk_base;
@@ -1248,16 +1397,32 @@ extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, fl
   if (nsweep > 0) {
     const int per_block = kLansThreads / kWave;
     const int rblocks = (T - tensor_base + per_block - 1) / per_block;
-    if (chunk_base == 0) lans_prepare_kernel<<<1, 64, 0, st>>>(t, sc);  // the bias corrections
     if (!grad_norms) {
-      lans_norm_g_kernel<<<nsweep, kLansThreads, 0, st>>>(t, chunk_base);
+      LANS_TYPE_SWITCH(g_dtype, kNoLowp, (lans_norm_g_kernel<GT><<<nsweep, kLansThreads, 0, st>>>(t, chunk_base)))
       lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 0, tensor_base, T, 1, 1);
     }
-    lans_moments_kernel<<<nsweep * kSweepSplit, kLansThreads, 0, st>>>(t, sc, chunk_base);
+    LANS_TYPE_SWITCH(g_dtype, kNoLowp, (lans_moments_kernel<GT><<<nsweep * kSweepSplit, kLansThreads, 0, st>>>(t, sc, chunk_base)))
     lans_reduce_kernel<<<rblocks, kLansThreads, 0, st>>>(t, 1, tensor_base, T, 3, kSweepSplit);
-    lans_update_kernel<<<nsweep * kSweepSplit, kLansThreads, 0, st>>>(t, sc, chunk_base);
+    LANS_TYPE_SWITCH(g_dtype, plt, (lans_update_kernel<GT, PL><<<nsweep * kSweepSplit, kLansThreads, 0, st>>>(t, sc, chunk_base)))
   }
   return static_cast<int>(hipGetLastError());
+}
+
+}  // namespace
+
+extern "C" int lancet_lans_step(lancet_lans_plan_t pl, const float* const* g, float* const* p,
+                                float* const* m, float* const* v, int step_host,
+                                const float* step_dev, const lancet_lans_hyper* h,
+                                const float* grad_norms, lancet_stream_t stream) {
+  return lans_step_impl(pl, reinterpret_cast<const void* const*>(g), LANCET_F32, p, m, v, nullptr, LANCET_F32, step_host,
+                        step_dev, h, grad_norms, stream);
+}
+
+extern "C" int lancet_lans_step_mixed(lancet_lans_plan_t pl, const void* const* g, int g_dtype, float* const* p,
+                                      float* const* m, float* const* v, void* const* p_lowp, int lowp_dtype,
+                                      int step_host, const float* step_dev, const lancet_lans_hyper* h,
+                                      const float* grad_norms, lancet_stream_t stream) {
+  return lans_step_impl(pl, g, g_dtype, p, m, v, p_lowp, lowp_dtype, step_host, step_dev, h, grad_norms, stream);
 }
 
 extern "C" int lancet_lans_plan_set_schedule(lancet_lans_plan_t pl, int schedule) {
@@ -1312,6 +1477,6 @@ extern "C" int lancet_lans_plan_debug_last_resident(lancet_lans_plan_t pl, int* 
 extern "C" int lancet_lans_plan_debug(lancet_lans_plan_t pl, unsigned spin_limit, unsigned flags) {
   if (!pl || pl->magic != kPlanMagic) return LANCET_ERR_PLAN;
   pl->spin_limit = spin_limit ? spin_limit : kDefaultSpinLimit;
-  pl->tables.debug_flags = flags;
+  pl->tables.debug_flags = flags;  // bit 1 (host only): lancet_lans_step does not look at the pinned status word
   return LANCET_OK;
 }

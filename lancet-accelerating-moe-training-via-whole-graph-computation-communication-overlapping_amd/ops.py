@@ -695,8 +695,12 @@ class LansPlan:
         except Exception:
             pass
 
-    def step(self, g, p, m, v, step, hyper, step_dev=None, grad_norms=None):
-        """One LANS step.  grad_norms: optional float32 GPU tensor [T] of ||g_i|| in list order (skips the
+    def step(self, g, p, m, v, step, hyper, step_dev=None, grad_norms=None, p_lowp=None):
+        """One LANS step.  p, m, v are float32 (the master parameters and the moments); g is float32, or bfloat16 /
+        float16 as the backward pass of a 16-bit model leaves it (one type for the whole list; widened inside the
+        step, which is what casting the gradients to float32 first would give); p_lowp: optional list of bfloat16 /
+        float16 tensors that receive the new parameters rounded to that type (the model's own copies), written in
+        the same pass as p.  grad_norms: optional float32 GPU tensor [T] of ||g_i|| in list order (skips the
         step's own pass over g).  Raises LancetError(ERR_STALLED) when an earlier step of the resident
         schedule gave up a wait, until error() has been read."""
         T = len(self.numels)
@@ -704,14 +708,27 @@ class LansPlan:
             _need(grad_norms.is_cuda and grad_norms.dtype == torch.float32 and grad_norms.numel() == T and
                   grad_norms.is_contiguous(), "grad_norms must be a contiguous float32 GPU tensor of T values")
         _need(len(g) == len(p) == len(m) == len(v) == T, "tensor lists must have one entry per planned tensor")
-        for lst in (g, p, m, v):
+        _need(p_lowp is None or len(p_lowp) == T, "p_lowp must have one entry per planned tensor")
+        g_dtype = g[0].dtype if T else torch.float32
+        _need(g_dtype in _DTYPES, "gradients must be float32, bfloat16 or float16")
+        lowp_dtype = p_lowp[0].dtype if p_lowp else torch.bfloat16
+        _need(lowp_dtype in (torch.bfloat16, torch.float16), "p_lowp must be bfloat16 or float16")
+        for lst, dt in ((g, g_dtype), (p, torch.float32), (m, torch.float32), (v, torch.float32)) + (((p_lowp, lowp_dtype),) if p_lowp else ()):
             for t, n in zip(lst, self.numels):
-                _need(t.is_cuda and t.is_contiguous() and t.dtype == torch.float32 and t.numel() == n,
-                      "LANS tensors must be contiguous float32 GPU tensors of the planned sizes")
+                _need(t.is_cuda and t.is_contiguous() and t.dtype == dt and t.numel() == n,
+                      "LANS tensors must be contiguous GPU tensors of the planned sizes: p, m, v float32, every gradient of "
+                      "one type, every 16-bit parameter copy of one type")
         arrs = [capi.ptr_array([t.data_ptr() for t in lst]) for lst in (g, p, m, v)]
-        st = self._lib.lancet_lans_step(self._h, arrs[0], arrs[1], arrs[2], arrs[3], int(step),
-                                        _p(step_dev), C.byref(hyper), _p(grad_norms), _stream())
-        capi.check(st, "lancet_lans_step")
+        if g_dtype == torch.float32 and not p_lowp:
+            st = self._lib.lancet_lans_step(self._h, arrs[0], arrs[1], arrs[2], arrs[3], int(step),
+                                            _p(step_dev), C.byref(hyper), _p(grad_norms), _stream())
+            capi.check(st, "lancet_lans_step")
+            return
+        low = capi.ptr_array([t.data_ptr() for t in p_lowp]) if p_lowp else None
+        st = self._lib.lancet_lans_step_mixed(self._h, arrs[0], _DTYPES[g_dtype], arrs[1], arrs[2], arrs[3], low,
+                                              _DTYPES[lowp_dtype], int(step), _p(step_dev), C.byref(hyper), _p(grad_norms),
+                                              _stream())
+        capi.check(st, "lancet_lans_step_mixed")
 
     def norms(self):
         """[4, T] float32: (||g||, ||p||, ||u_m||, ||u_g||) of the last step."""
@@ -724,13 +741,15 @@ _PLANS = {}
 
 
 def lans(tensor_list, step, learning_rate, beta1, beta2, eps, bias_correction, weight_decay, grad_averaging,
-         mode, normalize_grad):
+         mode, normalize_grad, p_lowp=None):
     """raf.op.lans(tensor_list, step, learning_rate, beta1, beta2, eps, bias_correction,
     weight_decay, grad_averaging, mode, normalize_grad).
 
     tensor_list = [g.. | p.. | m.. | v..] (python/raf/optim/lans.py:76-103); p, m, v are updated
     in place and the output tuple aliases the inputs (src/op/declare/optimizer.cc:46-62).  `step` is a Python number or a
-    0-dim float32 GPU tensor (the reference passes a tensor; it is read on the device)."""
+    0-dim float32 GPU tensor (the reference passes a tensor; it is read on the device).  Trailing extension for a
+    16-bit model: the gradients may be bfloat16 / float16 and p_lowp, a list of T 16-bit tensors, receives the new
+    parameters in that type (what the casts around the op do in python/raf/optim/lans.py:256-257, 285-288)."""
     n = len(tensor_list)
     _need(n % 4 == 0 and n > 0, "tensor_list must hold 4 lists of equal length")
     T = n // 4
@@ -746,9 +765,9 @@ def lans(tensor_list, step, learning_rate, beta1, beta2, eps, bias_correction, w
                            float(weight_decay), int(grad_averaging), int(mode), int(bool(normalize_grad)))
     if torch.is_tensor(step):
         _need(step.is_cuda and step.dtype == torch.float32 and step.numel() == 1, "step tensor must be a float32 GPU scalar")
-        plan.step(g, p, m, v, 0, hyper, step_dev=step)
+        plan.step(g, p, m, v, 0, hyper, step_dev=step, p_lowp=p_lowp)
     else:
-        plan.step(g, p, m, v, int(step), hyper)
+        plan.step(g, p, m, v, int(step), hyper, p_lowp=p_lowp)
     return tuple(tensor_list)
 
 
@@ -759,8 +778,14 @@ class LansStepper:
     def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), eps=1e-6, weight_decay=0.01, bias_correction=True,
                  grad_averaging=True, mode=True, normalize_grad=True):
         self.params = list(params)
-        self.m = [torch.zeros_like(p) for p in self.params]
-        self.v = [torch.zeros_like(p) for p in self.params]
+        # a 16-bit model: float32 master copies are what the step updates, and it writes the model's own
+        # parameters, rounded, in the same pass (the reference keeps float32 parameters and casts around the op,
+        # python/raf/optim/lans.py:256-257, 285-288)
+        self.mixed = bool(self.params) and self.params[0].dtype in (torch.bfloat16, torch.float16)
+        _need(all(p.dtype == self.params[0].dtype for p in self.params), "parameters must share one dtype")
+        self.master = [p.detach().float() for p in self.params] if self.mixed else None
+        self.m = [torch.zeros_like(p, dtype=torch.float32) for p in self.params]
+        self.v = [torch.zeros_like(p, dtype=torch.float32) for p in self.params]
         self.hyper = (lr, betas[0], betas[1], eps, int(bias_correction), weight_decay, int(grad_averaging),
                       int(mode), bool(normalize_grad))
         self._step = 1
@@ -776,6 +801,10 @@ class LansStepper:
         if live:
             pick = lambda lst: [lst[i] for i in live]
             # the update writes the parameters in place, outside autograd
-            lans(pick(grads) + [p.detach() for p in pick(self.params)] + pick(self.m) + pick(self.v), self._step,
-                 *self.hyper)
+            if self.mixed:
+                lans(pick(grads) + pick(self.master) + pick(self.m) + pick(self.v), self._step, *self.hyper,
+                     p_lowp=[p.detach() for p in pick(self.params)])
+            else:
+                lans(pick(grads) + [p.detach() for p in pick(self.params)] + pick(self.m) + pick(self.v), self._step,
+                     *self.hyper)
         self._step += 1

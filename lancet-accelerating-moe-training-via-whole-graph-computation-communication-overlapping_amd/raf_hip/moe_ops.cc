@@ -47,20 +47,30 @@ void CheckStatus(int status, const char* what) {
                 std::to_string(status) + ")");
 }
 
-// The scan's workspace carries state from call to call and is set up once (lancet_scan_workspace_init).  The
-// executor binds the memory after the OpEnv is built and may bind other memory later (an interpreter keeps one
-// allocation per cached OpEnv, a VM allocates before every Execute, src/impl/vm/vm.cc:1260-1266): the OpEnv sets
-// up whatever address it has not set up yet, on the stream it executes on.
+// Only the look-back form of the scan carries state in its workspace from call to call (ticket, epoch, descriptors)
+// and needs it set up once (lancet_scan_workspace_init); the forms most calls take use the workspace as plain
+// scratch (lancet_scan_call_is_stateful).  The executor binds the memory after the OpEnv is built and may bind other
+// memory later (an interpreter keeps one allocation per cached OpEnv, a VM allocates before every Execute,
+// src/impl/vm/vm.cc:1260-1266, and other operators may have used that memory in between): a stateful OpEnv sets up
+// whatever binding it has not set up yet, on the stream it executes on, and only the header and descriptor table
+// the scan reads (init_bytes), not the scratch behind them; a stateless one sets up nothing, and has nothing to
+// report at CheckDeviceStatus either (no waits, so no synchronisation there).
 struct ScanWorkspaceState {
-  void* ready = nullptr;  // the address lancet_scan_workspace_init has run on
+  bool stateful = false;  // the OpEnv's calls run the look-back form
+  size_t init_bytes = 0;  // header + descriptor table
+  void* ready = nullptr;  // the binding lancet_scan_workspace_init has run on
+  void Configure(int64_t S, int64_t E, int nsets, unsigned flags, bool bpr) {
+    stateful = lancet_scan_call_is_stateful(S, E, bpr ? 1 : nsets, flags, bpr ? 1 : 0) != 0;
+    init_bytes = lancet_moe_encode_workspace_bytes(S, E, nsets);
+  }
   void Ensure(void* ws, size_t nbytes, void* stream) {
-    if (ws == ready) return;
-    CheckStatus(lancet_scan_workspace_init(ws, nbytes, stream), "lancet_scan_workspace_init");
+    if (!stateful || ws == ready) return;
+    CheckStatus(lancet_scan_workspace_init(ws, init_bytes < nbytes ? init_bytes : nbytes, stream), "lancet_scan_workspace_init");
     ready = ws;
   }
   // the workspace's sticky error word (read and cleared; synchronises the stream)
   void Check(void* ws, void* stream, const char* op) {
-    if (!ws || ws != ready) return;
+    if (!stateful || !ws || ws != ready) return;
     int err = 0;
     CheckStatus(lancet_scan_workspace_error(ws, stream, &err), "lancet_scan_workspace_error");
     if (err)
@@ -166,6 +176,7 @@ class MoeEncode : public OpEnv {
     device_id_ = data.device_id;
     RAF_CHECK(cv.out.kind == Value::kTuple && cv.out.fields.size() == 5, "Expected output to be a 5-Tuple");
     ws_bytes_ = lancet_moe_encode_workspace_bytes(shape_.S, shape_.E, top_k_);
+    scan_ws_.Configure(shape_.S, shape_.E, top_k_, flags_, false);
     RequestWorkspace(&ws_, device_id_, static_cast<int64_t>(ws_bytes_));
     this->arg_indices = {0, 1, 2};  // data, gate, used_capacity
     // trailing extension: gate2_noise [S, E] for the second choice of top_k = 2
@@ -249,6 +260,7 @@ class MoeEncodeBatchPrioritized : public OpEnv {
     // sorted indices, dropping mask, indices and gate buffers of the reference (cuda/moe.cc:512-520)
     // are replaced by one workspace for the radix select and the scan
     ws_bytes_ = lancet_moe_encode_bpr_workspace_bytes(orig_S_, shape_.E, n_partitions_);
+    scan_ws_.Configure(shape_.S, shape_.E, 2, flags_, true);
     RequestWorkspace(&ws_, device_id_, static_cast<int64_t>(ws_bytes_));
     this->arg_indices = {0, 1};
   }
@@ -728,6 +740,294 @@ class MoeDecodeDg : public OpEnv {
   int top_k_, dtype_, gate_dtype_, device_id_;
 };
 
+// =====================================================================================
+// raf.op.moe_encode_dgate(dy, gate, indices_locations, top_k=1, gate_is_logits=false): gate gradient of moe_encode
+// as a whole, for the forms of the op that transform the gate value (top-2 normalisation, fused softmax).  Extends
+// MoeEncodeGrad (src/op/grad/moe.cc:30-58), whose moe_encode_dg covers the reference's one form.
+// =====================================================================================
+void MoeEncodeDgateDeclare(CallValues& call) {
+  RAF_CHECK(call.args.size() >= 3, "moe_encode_dgate(dy, gate, indices_locations, top_k=1, gate_is_logits=false)");
+  const Tensor& dy = call.args[0].AsTensor();
+  const Tensor& gate = call.args[1].AsTensor();
+  RAF_CHECK(dy.shape.size() == 1, "Input dy should be 1-D.");
+  RAF_CHECK(gate.shape.size() == 2, "Input gate should be 2-D.");
+  GateDTypeToLancet(gate.dtype);
+  RAF_CHECK(dy.dtype == gate.dtype, "dy takes the gate's dtype");
+  const int64_t k = OptInt(call, 3, 1);
+  const int64_t S = MaskTokens(call.args[2].AsTensor(), k);
+  RAF_CHECK(gate.shape[0] == S && dy.shape[0] == k * S, "dy, gate and indices_locations disagree");
+  call.out = Value::MakeTensor(MakeOut(gate.device_id, gate.dtype.code, gate.dtype.bits, gate.shape));
+  call.device_id = gate.device_id;
+}
+
+class MoeEncodeDgate : public OpEnv {
+ public:
+  explicit MoeEncodeDgate(const CallValues& cv) {
+    const Tensor& gate = cv.args[1].AsTensor();
+    RAF_CHECK(gate.shape.size() == 2, "Expected input gate to be 2D.");
+    gate_dtype_ = GateDTypeToLancet(gate.dtype);
+    top_k_ = static_cast<int>(OptInt(cv, 3, 1));
+    flags_ = OptInt(cv, 4, 0) ? LANCET_GATE_IS_LOGITS : 0u;
+    dim_S_ = MaskTokens(cv.args[2].AsTensor(), top_k_);
+    dim_E_ = gate.shape[1];
+    device_id_ = gate.device_id;
+    this->arg_indices = {0, 1, 2};
+  }
+  void Execute(const CallValues& cv) override { Execute({cv.args[0], cv.args[1], cv.args[2]}, cv.out); }
+  void Execute(const std::vector<Value>& inputs, Value output) override {
+    CheckStatus(lancet_moe_encode_dgate(inputs[0].AsTensor().data, inputs[1].AsTensor().data,
+                                        static_cast<const int32_t*>(inputs[2].AsTensor().data), dim_S_, dim_E_, top_k_,
+                                        gate_dtype_, flags_, output.AsTensor().data, GetStream(device_id_)),
+                "lancet_moe_encode_dgate");
+  }
+  std::string name() const override { return "raf.op.hip.moe_encode_dgate"; }
+  static OpEnv* make(const CallValues& cv) { return new MoeEncodeDgate(cv); }
+
+ private:
+  int64_t dim_S_, dim_E_;
+  int top_k_, gate_dtype_, device_id_;
+  unsigned flags_;
+};
+
+// =====================================================================================
+// The routed-once form of Lancet's partitioned dispatch.  The partition pass emits, per token partition p, a
+// moe_encode chained to the one before it through used_capacity, then moe_merge_masks and moe_redispatch over all
+// of them (src/pass/dist_optimization/partition_exprs.cc:1709-1874).  Routing only reads the [S, E] gate, and the
+// merged masks of the chained encodes are by construction the routing of the whole batch
+// (tests/python/op/cuda/test_cuda_moe.py:384-471), so a graph that has the whole gate can be rewritten to
+//   moe_route(gate_all, used, M, cf, top_k)                         -> (gates_s, indices_locations, used, elems)
+//   moe_scatter_tokens(data_p, indices_locations, used_in, used, buffer, token_first_p)   per partition, in place
+//   moe_partition_ranges(indices_locations, P, E, M, top_k)         -> (starts, counts) for the partitions' exchanges
+//   moe_decode_tokens(expert_out, gates_s, indices_locations, token_first_p, n_tokens)    per partition
+// with no merge or redispatch pass: rows go straight to their final places in ONE [E, C, M] buffer.
+// =====================================================================================
+void MoeRouteDeclare(CallValues& call) {
+  RAF_CHECK(call.args.size() >= 3, "moe_route(gate, used_capacity, M, capacity_factor=1.0, top_k=1, gate_is_logits=false)");
+  const Tensor& gate = call.args[0].AsTensor();
+  const Tensor& used = call.args[1].AsTensor();
+  RAF_CHECK(gate.shape.size() == 2, "Input gate should be 2-D.");
+  RAF_CHECK(used.shape.size() == 1 && used.shape[0] == gate.shape[1] && IsI32(used.dtype), "used_capacity must be int32 [E]");
+  GateDTypeToLancet(gate.dtype);
+  const int64_t k = OptInt(call, 4, 1);
+  RAF_CHECK(k == 1 || k == 2, "top_k must be 1 or 2");
+  const int64_t S = gate.shape[0], E = gate.shape[1];
+  std::vector<Value> ret;
+  ret.push_back(Value::MakeTensor(MakeOut(gate.device_id, gate.dtype.code, gate.dtype.bits, {k * S})));
+  ret.push_back(Value::MakeTensor(MakeOut(gate.device_id, DTypeCode::kInt, 32, {2, k * S})));
+  ret.push_back(Value::MakeTensor(MakeOut(gate.device_id, DTypeCode::kInt, 32, {E})));
+  ret.push_back(Value::MakeTensor(MakeOut(gate.device_id, DTypeCode::kUInt, 64, {E})));
+  call.out = Value::MakeTuple(std::move(ret));
+  call.device_id = gate.device_id;
+}
+
+class MoeRoute : public OpEnv {
+ public:
+  explicit MoeRoute(const CallValues& cv) {
+    const Tensor& gate = cv.args[0].AsTensor();
+    RAF_CHECK(gate.shape.size() == 2, "Expected input gate to be 2D.");
+    dim_S_ = gate.shape[0], dim_E_ = gate.shape[1];
+    dim_M_ = cv.args[2].AsInt();
+    top_k_ = static_cast<int>(OptInt(cv, 4, 1));
+    const float cf = static_cast<float>(OptFloat(cv, 3, 1.0)) * (top_k_ == 2 ? 2.0f : 1.0f);
+    dim_C_ = lancet_moe_capacity(dim_S_, dim_E_, cf);
+    RAF_CHECK(dim_C_ >= 0 && dim_M_ >= 0, "bad capacity or model dim");
+    flags_ = OptInt(cv, 5, 0) ? LANCET_GATE_IS_LOGITS : 0u;
+    if (cv.args.size() > 7 && cv.args[7].kind != Value::kTensor && OptInt(cv, 7, 0)) flags_ |= LANCET_SCAN_LOOKBACK;
+    gate_dtype_ = GateDTypeToLancet(gate.dtype);
+    device_id_ = gate.device_id;
+    ws_bytes_ = lancet_moe_encode_workspace_bytes(dim_S_, dim_E_, top_k_);
+    scan_ws_.Configure(dim_S_, dim_E_, top_k_, flags_, false);
+    RequestWorkspace(&ws_, device_id_, static_cast<int64_t>(ws_bytes_));
+    this->arg_indices = {0, 1};
+    has_noise_ = cv.args.size() > 6 && cv.args[6].kind == Value::kTensor;  // gate2_noise [S, E], top_k = 2
+    if (has_noise_) {
+      RAF_CHECK(top_k_ == 2, "gate2_noise only exists for the second choice (top_k = 2)");
+      RAF_CHECK(cv.args[6].AsTensor().shape == gate.shape && cv.args[6].AsTensor().dtype == gate.dtype,
+                "gate2_noise must have the gate's shape and dtype");
+      this->arg_indices.push_back(6);
+    }
+  }
+  void Execute(const CallValues& cv) override {
+    std::vector<Value> inputs = {cv.args[0], cv.args[1]};
+    if (has_noise_) inputs.push_back(cv.args[6]);
+    Execute(inputs, cv.out);
+  }
+  void Execute(const std::vector<Value>& inputs, Value output) override {
+    const auto& out = output.AsTuple();
+    RAF_CHECK(out.size() == 4, "Expected output to be a 4-Tuple");
+    scan_ws_.Ensure(ws_, ws_bytes_, GetStream(device_id_));
+    CheckStatus(lancet_moe_route(inputs[0].AsTensor().data, has_noise_ ? inputs[2].AsTensor().data : nullptr,
+                                 static_cast<const int32_t*>(inputs[1].AsTensor().data), dim_S_, dim_M_, dim_E_, dim_C_,
+                                 top_k_, gate_dtype_, flags_, out[0].AsTensor().data,
+                                 static_cast<int32_t*>(out[1].AsTensor().data), static_cast<int32_t*>(out[2].AsTensor().data),
+                                 static_cast<uint64_t*>(out[3].AsTensor().data), ws_, ws_bytes_, GetStream(device_id_)),
+                "lancet_moe_route");
+  }
+  void WorkspaceBound() override { scan_ws_.ready = nullptr; }
+  void CheckDeviceStatus(void* stream) override { scan_ws_.Check(ws_, stream, "moe_route"); }
+  std::string name() const override { return "raf.op.hip.moe_route"; }
+  static OpEnv* make(const CallValues& cv) { return new MoeRoute(cv); }
+
+ private:
+  int64_t dim_S_, dim_E_, dim_M_, dim_C_;
+  int top_k_, gate_dtype_, device_id_;
+  unsigned flags_;
+  bool has_noise_ = false;
+  void* ws_ = nullptr;
+  size_t ws_bytes_ = 0;
+  ScanWorkspaceState scan_ws_;
+};
+
+// moe_scatter_tokens(data [n, M], indices_locations [2, k*S_total], used_in [E], used_out [E], buffer [E, C, M],
+//                    token_first, top_k=1, zero_tail=true): in place on `buffer`, which is also the output (the way
+// lans aliases its tensor list, src/op/declare/optimizer.cc:46-62): every partition's call writes its own rows.
+void MoeScatterTokensDeclare(CallValues& call) {
+  RAF_CHECK(call.args.size() >= 6, "moe_scatter_tokens(data, indices_locations, used_in, used_out, buffer, token_first, top_k=1, zero_tail=true)");
+  const Tensor& data = call.args[0].AsTensor();
+  const Tensor& buf = call.args[4].AsTensor();
+  RAF_CHECK(data.shape.size() == 2, "Input data should be 2-D.");
+  RAF_CHECK(buf.shape.size() == 3 && buf.shape[2] == data.shape[1] && buf.dtype == data.dtype,
+            "buffer must be [E, C, M] of the data's dtype");
+  DTypeToLancet(data.dtype);
+  const int64_t S_total = MaskTokens(call.args[1].AsTensor(), OptInt(call, 6, 1));
+  const int64_t first = call.args[5].AsInt();
+  RAF_CHECK(first >= 0 && first + data.shape[0] <= S_total, "token range outside the routed batch");
+  call.out = call.args[4];  // in place
+  call.device_id = data.device_id;
+}
+
+class MoeScatterTokens : public OpEnv {
+ public:
+  explicit MoeScatterTokens(const CallValues& cv) {
+    const Tensor& data = cv.args[0].AsTensor();
+    const Tensor& buf = cv.args[4].AsTensor();
+    top_k_ = static_cast<int>(OptInt(cv, 6, 1));
+    dim_S_total_ = MaskTokens(cv.args[1].AsTensor(), top_k_);
+    n_tokens_ = data.shape[0], dim_M_ = data.shape[1];
+    dim_E_ = buf.shape[0], dim_C_ = buf.shape[1];
+    token_first_ = cv.args[5].AsInt();
+    flags_ = OptInt(cv, 7, 1) ? 0u : LANCET_NO_TAIL_ZERO;
+    for (int i : {2, 3})
+      RAF_CHECK(IsI32(cv.args[i].AsTensor().dtype) && cv.args[i].AsTensor().numel() == dim_E_, "used capacities must be int32 [E]");
+    dtype_ = DTypeToLancet(data.dtype);
+    device_id_ = data.device_id;
+    this->arg_indices = {0, 1, 2, 3, 4};
+  }
+  void Execute(const CallValues& cv) override { Execute({cv.args[0], cv.args[1], cv.args[2], cv.args[3], cv.args[4]}, cv.out); }
+  void Execute(const std::vector<Value>& inputs, Value /*output: the buffer itself*/) override {
+    CheckStatus(lancet_moe_scatter_tokens(inputs[0].AsTensor().data, static_cast<const int32_t*>(inputs[1].AsTensor().data),
+                                          static_cast<const int32_t*>(inputs[2].AsTensor().data),
+                                          static_cast<const int32_t*>(inputs[3].AsTensor().data), dim_S_total_, token_first_,
+                                          n_tokens_, dim_M_, dim_E_, dim_C_, top_k_, dtype_, flags_, inputs[4].AsTensor().data,
+                                          GetStream(device_id_)),
+                "lancet_moe_scatter_tokens");
+  }
+  std::string name() const override { return "raf.op.hip.moe_scatter_tokens"; }
+  static OpEnv* make(const CallValues& cv) { return new MoeScatterTokens(cv); }
+
+ private:
+  int64_t dim_S_total_, n_tokens_, token_first_, dim_M_, dim_E_, dim_C_;
+  int top_k_, dtype_, device_id_;
+  unsigned flags_;
+};
+
+// moe_decode_tokens(data [E, C, M], gate [k*S_total], indices_locations [2, k*S_total], token_first, n_tokens, top_k=1)
+void MoeDecodeTokensDeclare(CallValues& call) {
+  RAF_CHECK(call.args.size() >= 5, "moe_decode_tokens(data, gate, indices_locations, token_first, n_tokens, top_k=1)");
+  const Tensor& data = call.args[0].AsTensor();
+  const Tensor& gate = call.args[1].AsTensor();
+  RAF_CHECK(data.shape.size() == 3, "Input data should be 3-D.");
+  RAF_CHECK(gate.shape.size() == 1, "Input gate should be 1-D.");
+  DTypeToLancet(data.dtype);
+  GateDTypeToLancet(gate.dtype);
+  const int64_t k = OptInt(call, 5, 1);
+  const int64_t S_total = MaskTokens(call.args[2].AsTensor(), k);
+  RAF_CHECK(gate.shape[0] == k * S_total, "gate and indices_locations disagree on the token count");
+  const int64_t first = call.args[3].AsInt(), n = call.args[4].AsInt();
+  RAF_CHECK(first >= 0 && n >= 0 && first + n <= S_total, "token range outside the routed batch");
+  call.out = Value::MakeTensor(MakeOut(data.device_id, data.dtype.code, data.dtype.bits, {n, data.shape[2]}));
+  call.device_id = data.device_id;
+}
+
+class MoeDecodeTokens : public OpEnv {
+ public:
+  explicit MoeDecodeTokens(const CallValues& cv) {
+    const Tensor& data = cv.args[0].AsTensor();
+    top_k_ = static_cast<int>(OptInt(cv, 5, 1));
+    dim_S_total_ = MaskTokens(cv.args[2].AsTensor(), top_k_);
+    dim_E_ = data.shape[0], dim_C_ = data.shape[1], dim_M_ = data.shape[2];
+    token_first_ = cv.args[3].AsInt(), n_tokens_ = cv.args[4].AsInt();
+    dtype_ = DTypeToLancet(data.dtype);
+    gate_dtype_ = GateDTypeToLancet(cv.args[1].AsTensor().dtype);
+    device_id_ = data.device_id;
+    this->arg_indices = {0, 1, 2};
+  }
+  void Execute(const CallValues& cv) override { Execute({cv.args[0], cv.args[1], cv.args[2]}, cv.out); }
+  void Execute(const std::vector<Value>& inputs, Value output) override {
+    CheckStatus(lancet_moe_decode_tokens(inputs[0].AsTensor().data, inputs[1].AsTensor().data,
+                                         static_cast<const int32_t*>(inputs[2].AsTensor().data), dim_S_total_, token_first_,
+                                         n_tokens_, dim_M_, dim_E_, dim_C_, top_k_, dtype_, gate_dtype_,
+                                         output.AsTensor().data, GetStream(device_id_)),
+                "lancet_moe_decode_tokens");
+  }
+  std::string name() const override { return "raf.op.hip.moe_decode_tokens"; }
+  static OpEnv* make(const CallValues& cv) { return new MoeDecodeTokens(cv); }
+
+ private:
+  int64_t dim_S_total_, n_tokens_, token_first_, dim_M_, dim_E_, dim_C_;
+  int top_k_, dtype_, gate_dtype_, device_id_;
+};
+
+// moe_partition_ranges(indices_locations [2, k*S_total], n_partitions, n_experts, M, top_k=1) -> (starts, counts),
+// uint64 [k*P, E] in elements: what the partitions' exchanges (sparse copies on row ranges, all-to-allv counts) take
+void MoePartitionRangesDeclare(CallValues& call) {
+  RAF_CHECK(call.args.size() >= 4, "moe_partition_ranges(indices_locations, n_partitions, n_experts, M, top_k=1)");
+  const Tensor& il = call.args[0].AsTensor();
+  const int64_t k = OptInt(call, 4, 1);
+  const int64_t S_total = MaskTokens(il, k);
+  const int64_t P = call.args[1].AsInt(), E = call.args[2].AsInt();
+  RAF_CHECK(P >= 1 && S_total % P == 0 && k * P <= LANCET_MAX_PARTITIONS, "the token count must divide into n_partitions");
+  RAF_CHECK(E >= 1, "n_experts must be positive");
+  std::vector<Value> ret;
+  for (int i = 0; i < 2; ++i) ret.push_back(Value::MakeTensor(MakeOut(il.device_id, DTypeCode::kUInt, 64, {k * P, E})));
+  call.out = Value::MakeTuple(std::move(ret));
+  call.device_id = il.device_id;
+}
+
+class MoePartitionRanges : public OpEnv {
+ public:
+  explicit MoePartitionRanges(const CallValues& cv) {
+    const Tensor& il = cv.args[0].AsTensor();
+    top_k_ = static_cast<int>(OptInt(cv, 4, 1));
+    dim_S_total_ = MaskTokens(il, top_k_);
+    n_partitions_ = static_cast<int>(cv.args[1].AsInt());
+    dim_E_ = cv.args[2].AsInt();
+    dim_M_ = cv.args[3].AsInt();
+    device_id_ = il.device_id;
+    ws_bytes_ = lancet_moe_partition_ranges_workspace_bytes(top_k_, n_partitions_, dim_E_);
+    RequestWorkspace(&ws_, device_id_, static_cast<int64_t>(ws_bytes_));
+    this->arg_indices = {0};
+  }
+  void Execute(const CallValues& cv) override { Execute({cv.args[0]}, cv.out); }
+  void Execute(const std::vector<Value>& inputs, Value output) override {
+    const auto& out = output.AsTuple();
+    RAF_CHECK(out.size() == 2, "Expected output to be a 2-Tuple");
+    CheckStatus(lancet_moe_partition_ranges(static_cast<const int32_t*>(inputs[0].AsTensor().data), dim_S_total_, top_k_,
+                                            n_partitions_, dim_E_, dim_M_, static_cast<uint64_t*>(out[0].AsTensor().data),
+                                            static_cast<uint64_t*>(out[1].AsTensor().data), ws_, ws_bytes_,
+                                            GetStream(device_id_)),
+                "lancet_moe_partition_ranges");
+  }
+  std::string name() const override { return "raf.op.hip.moe_partition_ranges"; }
+  static OpEnv* make(const CallValues& cv) { return new MoePartitionRanges(cv); }
+
+ private:
+  int64_t dim_S_total_, dim_E_, dim_M_;
+  int top_k_, n_partitions_, device_id_;
+  void* ws_ = nullptr;
+  size_t ws_bytes_ = 0;
+};
+
 // ---- registration (cuda/cuda_utils.cc:17; cuda/moe.cc:411-412,728-729,822-823,942-943,1310-1311) ----
 RAF_REGISTER_DIALECT("hip").set_enable("hip");
 
@@ -763,6 +1063,22 @@ RAF_REGISTER_DIALECT_OP(hip, moe_decode_dx, 20);
 RAF_OP_ENV_MAKER("raf.op.hip.moe_decode_dx", MoeDecodeDx::make);
 RAF_REGISTER_DIALECT_OP(hip, moe_decode_dg, 20);
 RAF_OP_ENV_MAKER("raf.op.hip.moe_decode_dg", MoeDecodeDg::make);
+// no base op of these names exists in the reference: they are what a graph rewrite for this dialect introduces
+RAF_OP_DECLARE("raf.op.moe_encode_dgate", MoeEncodeDgateDeclare);
+RAF_REGISTER_DIALECT_OP(hip, moe_encode_dgate, 20);
+RAF_OP_ENV_MAKER("raf.op.hip.moe_encode_dgate", MoeEncodeDgate::make);
+RAF_OP_DECLARE("raf.op.moe_route", MoeRouteDeclare);
+RAF_REGISTER_DIALECT_OP(hip, moe_route, 20);
+RAF_OP_ENV_MAKER("raf.op.hip.moe_route", MoeRoute::make);
+RAF_OP_DECLARE("raf.op.moe_scatter_tokens", MoeScatterTokensDeclare);
+RAF_REGISTER_DIALECT_OP(hip, moe_scatter_tokens, 20);
+RAF_OP_ENV_MAKER("raf.op.hip.moe_scatter_tokens", MoeScatterTokens::make);
+RAF_OP_DECLARE("raf.op.moe_decode_tokens", MoeDecodeTokensDeclare);
+RAF_REGISTER_DIALECT_OP(hip, moe_decode_tokens, 20);
+RAF_OP_ENV_MAKER("raf.op.hip.moe_decode_tokens", MoeDecodeTokens::make);
+RAF_OP_DECLARE("raf.op.moe_partition_ranges", MoePartitionRangesDeclare);
+RAF_REGISTER_DIALECT_OP(hip, moe_partition_ranges, 20);
+RAF_OP_ENV_MAKER("raf.op.hip.moe_partition_ranges", MoePartitionRanges::make);
 
 }  // namespace hip
 }  // namespace op

@@ -84,3 +84,15 @@ def lans_step(g_list, p_list, m_list, v_list, step, lr=1e-3, beta1=0.9, beta2=0.
         p[...] = p - ratio_m * u_m - ratio_g * u_g               # :386
         norms.append((gn, pn, umn, ugn))
     return norms
+
+
+def lans_step_mixed(g_list, p_list, m_list, v_list, step, lowp_round=None, **hyper):
+    """The step as the reference's traced optimizer runs it for a 16-bit model (python/raf/optim/lans.py:256-257,
+    285-288): every gradient cast to float32, lans_step, every new parameter cast back to the model's type.
+    g_list holds the 16-bit gradients as the float32 values they denote (the cast is exact); p, m, v are the float32
+    master state, updated in place.  Returns the model's copies of the new parameters (float32 values of the 16-bit
+    type lowp_round rounds to), or None without lowp_round."""
+    lans_step([np.asarray(g, np.float32) for g in g_list], p_list, m_list, v_list, step, **hyper)
+    if lowp_round is None:
+        return None
+    return [lowp_round(p).astype(np.float32) for p in p_list]

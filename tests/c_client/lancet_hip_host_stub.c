@@ -46,6 +46,13 @@ int lancet_scan_workspace_init(void* ws, size_t nbytes, lancet_stream_t st) {
   return 0;
 }
 
+/* as the library decides it: top-1 on at most 32 tiles, or on request (the stub's OpEnvs then also run the set-up) */
+int lancet_scan_call_is_stateful(int64_t S, int64_t E, int top_k, unsigned flags, int bpr) {
+  (void)E;
+  if (flags & LANCET_SCAN_LOOKBACK) return 1;
+  return !bpr && top_k == 1 && tiles(S) <= 32;
+}
+
 int lancet_scan_workspace_error(void* ws, lancet_stream_t st, int* error_out) {
   (void)st;
   if (!ws || !error_out) return LANCET_ERR_NULL;
@@ -228,5 +235,93 @@ int lancet_lans_step(lancet_lans_plan_t plan, const float* const* g, float* cons
     touch_read(p[i], n), touch_read(m[i], n), touch_read(v[i], n);
     touch_write(p[i], n), touch_write(m[i], n), touch_write(v[i], n);
   }
+  return 0;
+}
+
+int lancet_lans_step_mixed(lancet_lans_plan_t plan, const void* const* g, int g_dtype, float* const* p, float* const* m,
+                           float* const* v, void* const* p_lowp, int lowp_dtype, int step_host, const float* step_dev,
+                           const lancet_lans_hyper* hyper, const float* grad_norms, lancet_stream_t st) {
+  (void)st, (void)step_host;
+  if (!plan || !hyper) return LANCET_ERR_PLAN;
+  if (!eb(g_dtype) || (p_lowp && eb(lowp_dtype) != 2)) return LANCET_ERR_DTYPE;
+  if (step_dev) touch_read(step_dev, 4);
+  if (grad_norms) touch_read(grad_norms, (size_t)plan->T * 4);
+  for (int i = 0; i < plan->T; ++i) {
+    const size_t n = (size_t)plan->numels[i];
+    touch_read(g[i], n * eb(g_dtype));
+    touch_read(p[i], n * 4), touch_read(m[i], n * 4), touch_read(v[i], n * 4);
+    touch_write(p[i], n * 4), touch_write(m[i], n * 4), touch_write(v[i], n * 4);
+    if (p_lowp) touch_write(p_lowp[i], n * 2);
+  }
+  return 0;
+}
+
+int lancet_moe_encode_dgate(const void* dy, const void* gate, const int32_t* il, int64_t S, int64_t E, int top_k,
+                            int gate_dtype, unsigned flags, void* grad, lancet_stream_t st) {
+  (void)st;
+  if (!eb(gate_dtype)) return LANCET_ERR_DTYPE;
+  touch_read(dy, (size_t)top_k * S * eb(gate_dtype));
+  touch_read(il, (size_t)top_k * S * 4);                      /* the index row only */
+  if (top_k == 2 || (flags & LANCET_GATE_IS_LOGITS)) touch_read(gate, (size_t)S * E * eb(gate_dtype));
+  touch_write(grad, (size_t)S * E * eb(gate_dtype));
+  return 0;
+}
+
+int lancet_moe_route(const void* gate, const void* noise, const int32_t* used_in, int64_t S, int64_t M, int64_t E, int64_t C,
+                     int top_k, int gate_dtype, unsigned flags, void* gates_s, int32_t* il, int32_t* used_out,
+                     uint64_t* elems, void* ws, size_t ws_bytes, lancet_stream_t st) {
+  (void)flags, (void)st, (void)M, (void)C;
+  if (!eb(gate_dtype)) return LANCET_ERR_DTYPE;
+  if (ws_bytes < lancet_moe_encode_workspace_bytes(S, E, top_k)) return LANCET_ERR_WORKSPACE;
+  touch_read(gate, (size_t)S * E * eb(gate_dtype));
+  if (noise) touch_read(noise, (size_t)S * E * eb(gate_dtype));
+  if (used_in) touch_read(used_in, (size_t)E * 4);
+  touch_write(gates_s, (size_t)top_k * S * eb(gate_dtype));
+  touch_write(il, (size_t)2 * top_k * S * 4);
+  touch_write(used_out, (size_t)E * 4);
+  touch_write(elems, (size_t)E * 8);
+  touch_write(ws, lancet_moe_encode_workspace_bytes(S, E, top_k));
+  return 0;
+}
+
+int lancet_moe_scatter_tokens(const void* data, const int32_t* il, const int32_t* used_in, const int32_t* used_out,
+                              int64_t S_total, int64_t token_first, int64_t n_tokens, int64_t M, int64_t E, int64_t C,
+                              int top_k, int dtype, unsigned flags, void* dispatched, lancet_stream_t st) {
+  (void)st;
+  if (!eb(dtype)) return LANCET_ERR_DTYPE;
+  if (token_first < 0 || n_tokens < 0 || token_first + n_tokens > S_total) return LANCET_ERR_SHAPE;
+  touch_read(data, (size_t)n_tokens * M * eb(dtype));
+  for (int j = 0; j < 2 * top_k; ++j) touch_read(il + (size_t)j * S_total + token_first, (size_t)n_tokens * 4);
+  if (!(flags & LANCET_NO_TAIL_ZERO)) {
+    if (used_in) touch_read(used_in, (size_t)E * 4);
+    touch_read(used_out, (size_t)E * 4);
+  }
+  touch_write(dispatched, (size_t)E * C * M * eb(dtype));      /* any row of the buffer may be this call's */
+  return 0;
+}
+
+int lancet_moe_decode_tokens(const void* expert_out, const void* gates_s, const int32_t* il, int64_t S_total,
+                             int64_t token_first, int64_t n_tokens, int64_t M, int64_t E, int64_t C, int top_k, int dtype,
+                             int gate_dtype, void* out, lancet_stream_t st) {
+  (void)st;
+  if (!eb(dtype) || !eb(gate_dtype)) return LANCET_ERR_DTYPE;
+  if (token_first < 0 || n_tokens < 0 || token_first + n_tokens > S_total) return LANCET_ERR_SHAPE;
+  touch_read(expert_out, (size_t)E * C * M * eb(dtype));
+  for (int j = 0; j < top_k; ++j)
+    touch_read((const char*)gates_s + ((size_t)j * S_total + token_first) * eb(gate_dtype), (size_t)n_tokens * eb(gate_dtype));
+  for (int j = 0; j < 2 * top_k; ++j) touch_read(il + (size_t)j * S_total + token_first, (size_t)n_tokens * 4);
+  touch_write(out, (size_t)n_tokens * M * eb(dtype));
+  return 0;
+}
+
+size_t lancet_moe_partition_ranges_workspace_bytes(int top_k, int P, int64_t E) { return (size_t)top_k * (size_t)P * (size_t)E * 4; }
+int lancet_moe_partition_ranges(const int32_t* il, int64_t S_total, int top_k, int P, int64_t E, int64_t M, uint64_t* starts,
+                                uint64_t* counts, void* ws, size_t ws_bytes, lancet_stream_t st) {
+  (void)st, (void)M;
+  if (ws_bytes < lancet_moe_partition_ranges_workspace_bytes(top_k, P, E)) return LANCET_ERR_WORKSPACE;
+  touch_read(il, (size_t)top_k * S_total * 4);
+  touch_write(starts, (size_t)top_k * P * E * 8);
+  touch_write(counts, (size_t)top_k * P * E * 8);
+  touch_write(ws, lancet_moe_partition_ranges_workspace_bytes(top_k, P, E));
   return 0;
 }

@@ -233,6 +233,89 @@ void all_ops() {
     raf_hip_push_bool(c.h, 1);
     run(c.h, a, "4 tensors, step tensor");
   }
+  for (int g_bits : {32, 16}) {  // a 16-bit model: 16-bit gradients in, 16-bit copies of the new parameters out
+    Arena a;
+    CallH c("raf.op.lans");
+    const std::vector<std::vector<int64_t>> shapes = {{17, 5}, {129}, {8192}};
+    raf_hip_begin_tuple(c.h);
+    for (int q = 0; q < 4; ++q)
+      for (const auto& s : shapes) tensor(c.h, a, q == 0 && g_bits == 16 ? kBFloat : kFloat, q == 0 ? g_bits : 32, s);
+    raf_hip_end_tuple(c.h);
+    raf_hip_push_int(c.h, 3);
+    raf_hip_push_float(c.h, 1e-3), raf_hip_push_float(c.h, 0.9), raf_hip_push_float(c.h, 0.999), raf_hip_push_float(c.h, 1e-6);
+    raf_hip_push_int(c.h, 1), raf_hip_push_float(c.h, 0.01), raf_hip_push_int(c.h, 1), raf_hip_push_int(c.h, 1);
+    raf_hip_push_bool(c.h, 1);
+    raf_hip_begin_tuple(c.h);
+    for (const auto& s : shapes) tensor(c.h, a, kBFloat, 16, s);
+    raf_hip_end_tuple(c.h);
+    run(c.h, a, g_bits == 16 ? "bf16 gradients, bf16 parameter copies" : "fp32 gradients, bf16 parameter copies");
+  }
+  // the routed-once form of the partitioned dispatch: one routing of the whole batch, per-partition row movement
+  for (int k : {1, 2}) {
+    const int64_t P = 3, Sp = S / P, C = 140 * k;
+    {
+      Arena a;
+      CallH c("raf.op.moe_route");
+      tensor(c.h, a, kFloat, 32, {S, E});
+      tensor(c.h, a, kInt, 32, {E});
+      raf_hip_push_int(c.h, M);
+      raf_hip_push_float(c.h, 1.25);
+      raf_hip_push_int(c.h, k);
+      raf_hip_push_int(c.h, 1);
+      run(c.h, a, k == 1 ? "top-1 on few tiles: the stateful form, workspace set up" : "top-2: plain scratch");
+    }
+    {
+      Arena a;
+      CallH c("raf.op.moe_scatter_tokens");
+      tensor(c.h, a, kBFloat, 16, {Sp, M});
+      tensor(c.h, a, kInt, 32, {2, k * S});
+      tensor(c.h, a, kInt, 32, {E});
+      tensor(c.h, a, kInt, 32, {E});
+      tensor(c.h, a, kBFloat, 16, {E, C, M});
+      raf_hip_push_int(c.h, 2 * Sp);  // the last partition
+      raf_hip_push_int(c.h, k);
+      run(c.h, a, "in place on the shared buffer");
+    }
+    {
+      Arena a;
+      CallH c("raf.op.moe_decode_tokens");
+      tensor(c.h, a, kBFloat, 16, {E, C, M});
+      tensor(c.h, a, kFloat, 32, {k * S});
+      tensor(c.h, a, kInt, 32, {2, k * S});
+      raf_hip_push_int(c.h, 2 * Sp);
+      raf_hip_push_int(c.h, Sp);
+      raf_hip_push_int(c.h, k);
+      run(c.h, a, "");
+    }
+    {
+      Arena a;
+      CallH c("raf.op.moe_partition_ranges");
+      tensor(c.h, a, kInt, 32, {2, k * S});
+      raf_hip_push_int(c.h, P), raf_hip_push_int(c.h, E), raf_hip_push_int(c.h, M), raf_hip_push_int(c.h, k);
+      run(c.h, a, "");
+    }
+    for (int logits : {0, 1}) {
+      Arena a;
+      CallH c("raf.op.moe_encode_dgate");
+      tensor(c.h, a, kBFloat, 16, {k * S});
+      tensor(c.h, a, kBFloat, 16, {S, E});
+      tensor(c.h, a, kInt, 32, {2, k * S});
+      raf_hip_push_int(c.h, k);
+      raf_hip_push_int(c.h, logits);
+      run(c.h, a, "gate gradient through the normalisation / the softmax");
+    }
+  }
+  {
+    Arena a;
+    CallH c("raf.op.moe_scatter_tokens");
+    tensor(c.h, a, kFloat, 32, {100, 4});
+    tensor(c.h, a, kInt, 32, {2, 300});
+    tensor(c.h, a, kInt, 32, {6});
+    tensor(c.h, a, kInt, 32, {6});
+    tensor(c.h, a, kFloat, 32, {6, 50, 4});
+    raf_hip_push_int(c.h, 250);
+    expect_rejected(c.h, "token range past the routed batch");
+  }
   // error paths: the message is built, the call object is destroyed with a half-built state
   {
     Arena a;

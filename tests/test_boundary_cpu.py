@@ -200,6 +200,64 @@ def test_declare_reproduces_the_output_contract(pkg):
     lib.raf_hip_call_destroy(h)
 
 
+def test_declare_of_the_routed_once_ops_and_the_gate_gradient(pkg):
+    """The operators a graph rewrite for this dialect introduces (no base op of these names in the reference):
+    moe_route, moe_scatter_tokens (in place on the shared buffer), moe_decode_tokens, moe_partition_ranges,
+    moe_encode_dgate."""
+    rx = pkg.raf_executor
+    lib, capi = rx.load(), pkg.capi.load()
+    S, M, E, P = 65536, 4096, 32, 4
+    h, rc, outs = _declare(rx, "raf.op.moe_route", [("t", (F32, (S, E))), ("t", (I32, (E,))), ("i", M), ("f", 1.25), ("i", 2), ("i", 1)])
+    assert rc == 0 and outs == [(F32, (2 * S,)), (I32, (2, 2 * S)), (I32, (E,)), (U64, (E,))]
+    assert lib.raf_hip_dispatch(h) == 0 and lib.raf_hip_env_name(h) == b"raf.op.hip.moe_route"
+    assert lib.raf_hip_workspace_bytes(h, 0) == capi.lancet_moe_encode_workspace_bytes(S, E, 2)
+    assert [lib.raf_hip_arg_index(h, i) for i in range(lib.raf_hip_num_arg_indices(h))] == [0, 1]
+    lib.raf_hip_call_destroy(h)
+    h, rc, outs = _declare(rx, "raf.op.moe_scatter_tokens",
+                           [("t", (BF16, (S // P, M))), ("t", (I32, (2, 2 * S))), ("t", (I32, (E,))), ("t", (I32, (E,))),
+                            ("t", (BF16, (E, 5120, M))), ("i", S // P), ("i", 2), ("i", 0)])
+    assert rc == 0 and outs == [(BF16, (E, 5120, M))]              # the buffer itself
+    assert lib.raf_hip_dispatch(h) == 0 and lib.raf_hip_num_workspaces(h) == 0
+    lib.raf_hip_call_destroy(h)
+    h, rc, outs = _declare(rx, "raf.op.moe_decode_tokens",
+                           [("t", (BF16, (E, 5120, M))), ("t", (F32, (2 * S,))), ("t", (I32, (2, 2 * S))), ("i", S // P), ("i", S // P), ("i", 2)])
+    assert rc == 0 and outs == [(BF16, (S // P, M))]
+    lib.raf_hip_call_destroy(h)
+    h, rc, outs = _declare(rx, "raf.op.moe_partition_ranges", [("t", (I32, (2, 2 * S))), ("i", P), ("i", E), ("i", M), ("i", 2)])
+    assert rc == 0 and outs == [(U64, (2 * P, E)), (U64, (2 * P, E))]
+    assert lib.raf_hip_dispatch(h) == 0
+    assert lib.raf_hip_workspace_bytes(h, 0) == capi.lancet_moe_partition_ranges_workspace_bytes(2, P, E)
+    lib.raf_hip_call_destroy(h)
+    for gd in (F32, BF16):
+        h, rc, outs = _declare(rx, "raf.op.moe_encode_dgate", [("t", (gd, (2 * S,))), ("t", (gd, (S, E))), ("t", (I32, (2, 2 * S))), ("i", 2), ("i", 1)])
+        assert rc == 0 and outs == [(gd, (S, E))]
+        lib.raf_hip_call_destroy(h)
+    h, rc, _ = _declare(rx, "raf.op.moe_decode_tokens",
+                        [("t", (F32, (8, 50, 64))), ("t", (F32, (100,))), ("t", (I32, (2, 100))), ("i", 90), ("i", 20)])
+    assert rc != 0 and b"token range outside the routed batch" in lib.raf_hip_last_error()
+    lib.raf_hip_call_destroy(h)
+
+
+def test_gate_typed_outputs_follow_the_gate(pkg):
+    """A deliberate difference from the reference's Declare, which types gates_s float32 whatever the gate is
+    (src/op/declare/moe.cc:54) and the gradient of gates_s like dy (:239): here gates_s and its gradient take the
+    gate's type, which is what the reference's kernels are instantiated on (`__dtype* gates1_s`,
+    tutel_moe_dispatch.cu:110-116).  With the float32 gate the reference's models feed, both rules give float32;
+    under mixed precision a graph typed by the reference's rule needs a cast behind the op."""
+    rx = pkg.raf_executor
+    lib = rx.load()
+    for gd in (F32, BF16):
+        h, rc, outs = _declare(rx, "raf.op.moe_encode", [("t", (BF16, (512, 64))), ("t", (gd, (512, 8))), ("t", (I32, (8,)))])
+        assert rc == 0 and outs[0] == (gd, (512,)) and outs[4] == (BF16, (8, 64, 64))
+        lib.raf_hip_call_destroy(h)
+    # moe_decode_dg: float32 unless the trailing gate_dtype argument names a half type (never dy's type by itself)
+    for code, want in ((None, F32), (1, BF16)):
+        args = [("t", (BF16, (100, 64))), ("t", (BF16, (8, 50, 64))), ("t", (I32, (2, 100)))] + ([("i", 1), ("i", code)] if code is not None else [])
+        h, rc, outs = _declare(rx, "raf.op.moe_decode_dg", args)
+        assert rc == 0 and outs == [(want, (100,))]
+        lib.raf_hip_call_destroy(h)
+
+
 def test_op_layer_errors_are_reported_not_fatal(pkg):
     rx = pkg.raf_executor
     lib = rx.load()

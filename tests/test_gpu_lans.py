@@ -235,6 +235,130 @@ def test_lans_resident_give_up_is_fail_safe_and_sticky(pkg):
     other.close()
 
 
+@pytest.mark.parametrize("with_grad_norms", [False, True])
+def test_lans_steps_queued_behind_a_stalled_step_touch_nothing(pkg, with_grad_norms):
+    """A training loop that never synchronises has steps 2 and 3 queued before the host can see that step 1 stalled
+    (and a replayed graph never asks the host): such steps must see the error on the device and leave every array
+    alone, in both schedules, until the error has been read.  With the caller's gradient norms stage M of step 1
+    runs (moments written) and only its parameters stay unwritten: the half-applied state a later step must not
+    build on.  The host-side refusal is switched off here (debug flag 2) so that the steps really are launched."""
+    capi = pkg.capi
+    numels = [1 << 20, 8192 * 3, 8192, 1000]             # the last one goes through the sweeps of the same step
+    hyper = capi.LansHyper(1e-3, 0.9, 0.999, 1e-6, 1, 0.01, 1, 1, 1)
+    state = _fresh_state(numels, 17)
+    before = [[t.clone() for t in lst] for lst in state]
+    norms = torch.stack([torch.linalg.vector_norm(g.double()).float() for g in state[0]]) if with_grad_norms else None
+    plan = pkg.ops.LansPlan(numels)
+    plan.debug(spin_limit=8, flags=1 | 2)                 # nothing is published: every wait gives up
+    plan.step(*state, 1, hyper, grad_norms=norms)
+    torch.cuda.synchronize()
+    after1 = [[t.clone() for t in lst] for lst in state]
+    for i in range(3):                                    # the resident kernel's tensors: no parameter was written
+        assert torch.equal(state[1][i], before[1][i])
+        assert torch.equal(state[2][i], before[2][i]) != with_grad_norms     # moments: written only when ||g|| was known
+    assert not torch.equal(state[1][3], before[1][3])     # the sweeps' tensor of step 1 is independent of the stall
+    plan.debug(spin_limit=0, flags=2)                     # a healthy device from here on; the host still does not look
+    plan.step(*state, 2, hyper, grad_norms=norms)
+    plan.step(*state, 3, hyper, grad_norms=norms)
+    plan.set_schedule(capi.LANS_SWEEPS)
+    plan.step(*state, 4, hyper, grad_norms=norms)
+    torch.cuda.synchronize()
+    for la, lb in zip(state, after1):
+        for a, b in zip(la, lb):
+            assert torch.equal(a, b)                      # steps 2 to 4 were skipped as a whole
+    plan.set_schedule(capi.LANS_RESIDENT)
+    plan.debug(spin_limit=0, flags=0)
+    with pytest.raises(capi.LancetError):                 # the host-side refusal is back
+        plan.step(*state, 2, hyper, grad_norms=norms)
+    assert plan.error() == 1 and plan.error() == 0
+    plan.step(*state, 2, hyper, grad_norms=norms)         # and the plan works again
+    torch.cuda.synchronize()
+    assert plan.error() == 0
+    for i in range(4):
+        assert not torch.equal(state[1][i], after1[1][i])
+    plan.close()
+
+
+def _rounder(name):
+    from oracle import moe_oracle as mo
+    return {"f32": (lambda a: a), "bf16": mo.round_to_bf16, "f16": mo.round_to_f16}[name]
+
+
+_TORCH = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
+
+
+@pytest.mark.parametrize("schedule", ["sweeps", "resident"])
+@pytest.mark.parametrize("gdt,pdt", [("bf16", "bf16"), ("f16", "f16"), ("f32", "bf16"), ("bf16", None), ("f16", "bf16")])
+def test_lans_mixed_precision_step(pkg, schedule, gdt, pdt):
+    """The step of a 16-bit model: gradients in bf16 / fp16, fp32 master parameters and moments, and the model's
+    16-bit copy of every new parameter written by the same step, against the oracle's restatement of what the
+    reference's optimizer does around its op (cast the gradients up, lans, cast the parameters down,
+    python/raf/optim/lans.py:256-257, 285-288).  Master parameters within 1e-6 after 10 steps as for the fp32 step;
+    the 16-bit copies bit-equal to the rounded master.  Shapes: the reference's own test lists
+    (tests/python/optim/test_lans.py:94-161) and tensors the resident kernel takes."""
+    capi = pkg.capi
+    for seed, shapes in enumerate([[(2, 2)], [(6, 3, 5, 5), (6,), (6,), (10, 84), (10,)],
+                                   [(3 * 8192,), (300, 70), (2, 8192), (8192 + 5,), (8192,)]]):
+        rng, p, m, v = make_state(20 + seed, shapes)
+        dp, dm, dv = [dev(a) for a in p], [dev(a) for a in m], [dev(a) for a in v]
+        dlow = [torch.full(s, 7.0, dtype=_TORCH[pdt], device="cuda") for s in shapes] if pdt else None
+        plan = pkg.ops.LansPlan([a.size for a in p], schedule=capi.LANS_SWEEPS if schedule == "sweeps" else None)
+        hyper = capi.LansHyper(1e-3, 0.9, 0.999, 1e-6, 1, 0.01, 1, 1, 1)
+        for step in range(1, 11):
+            g = [_rounder(gdt)(rng.normal(0, 1e-3, s).astype(np.float32)).astype(np.float32) for s in shapes]
+            dg = [dev(a).to(_TORCH[gdt]) for a in g]
+            for a, b in zip(dg, g):
+                np.testing.assert_array_equal(to_np(a), b)            # the device holds exactly the oracle's gradients
+            low = lo.lans_step_mixed(g, p, m, v, step, _rounder(pdt) if pdt else None)
+            plan.step(dg, dp, dm, dv, step, hyper, p_lowp=dlow)
+            if dlow is not None:
+                for a, b in zip(dlow, dp):                            # bit-equal to the rounded master, every step
+                    assert torch.equal(a, b.to(_TORCH[pdt]))
+        assert plan.error() == 0
+        if schedule == "resident" and seed == 2:
+            assert plan.last_resident_slots() >= 6
+        for i in range(len(shapes)):
+            assert_close_scaled(to_np(dp[i]), p[i], P_RTOL, "p[%d]" % i)
+            assert_close_scaled(to_np(dm[i]), m[i], 1e-5, "m[%d]" % i)
+            assert_close_scaled(to_np(dv[i]), v[i], 1e-5, "v[%d]" % i)
+            if pdt:                                                    # and against the oracle's casts: one ulp of the type
+                from tests.gpu_util import ulp_distance
+                assert ulp_distance(dlow[i], torch.from_numpy(low[i]).to(_TORCH[pdt]).cuda()) <= 1
+        plan.close()
+
+
+def test_lans_mixed_precision_rejects_and_aligns(pkg):
+    """p, m, v stay float32; 16-bit arrays of a resident tensor that are not 8-byte aligned send the step through
+    the sweeps (element path), with the same result."""
+    capi = pkg.capi
+    numels = [8192 * 2, 100]
+    hyper = capi.LansHyper(1e-3, 0.9, 0.999, 1e-6, 1, 0.01, 1, 1, 1)
+    out = []
+    for offset in (0, 1):
+        g, p, m, v = _fresh_state(numels, 23, 0)
+        store = [torch.zeros(n + offset, dtype=torch.bfloat16, device="cuda") for n in numels]
+        g16 = [s[offset:] for s in store]
+        for a, b in zip(g16, g):
+            a.copy_(b)
+        low_store = [torch.zeros(n + offset, dtype=torch.bfloat16, device="cuda") for n in numels]
+        low = [s[offset:] for s in low_store]
+        plan = pkg.ops.LansPlan(numels)
+        plan.step(g16, p, m, v, 1, hyper, p_lowp=low)
+        plan.step(g16, p, m, v, 2, hyper, p_lowp=low)
+        torch.cuda.synchronize()
+        assert plan.error() == 0
+        assert (plan.last_resident_slots() > 0) == (offset == 0)
+        out.append((p, low))
+        for a, b in zip(low, p):
+            assert torch.equal(a, b.to(torch.bfloat16))
+        with pytest.raises(ValueError):
+            plan.step(g16, [x.to(torch.bfloat16) for x in p], m, v, 3, hyper)
+        plan.close()
+    for a, b in zip(out[0][0], out[1][0]):
+        scale = float(a.abs().max())
+        assert float((a - b).abs().max()) <= 2e-6 * scale
+
+
 def test_lans_resident_schedule_against_oracle(pkg):
     capi = pkg.capi
     rng = np.random.default_rng(5)
@@ -367,3 +491,35 @@ def test_stepper_trains_a_small_model_like_the_reference_optimizer(pkg):
     np.testing.assert_array_equal(to_np(unused.detach()), np.ones(5, np.float32))
     with pytest.raises(ValueError):
         opt.step([None])
+
+
+def test_stepper_keeps_master_weights_for_a_16_bit_model(pkg):
+    """Parameters in bfloat16: the stepper keeps float32 master copies, feeds the 16-bit gradients as they are and
+    lets the step write the model's parameters (python/raf/optim/lans.py:256-257, 285-288 does it with casts around
+    the op).  Against the oracle's mixed step fed with the same gradients."""
+    from oracle import moe_oracle as mo
+    torch.manual_seed(1)
+    w1 = (torch.randn(64, 32, device="cuda") * 0.1).to(torch.bfloat16).requires_grad_(True)
+    w2 = (torch.randn(32, 8, device="cuda") * 0.1).to(torch.bfloat16).requires_grad_(True)
+    params = [w1, w2]
+    opt = pkg.ops.LansStepper(params, lr=2e-3, weight_decay=0.05)
+    assert opt.mixed and opt.master[0].dtype == torch.float32
+    ref_p = [to_np(p.detach()) for p in params]
+    ref_m = [np.zeros_like(a) for a in ref_p]
+    ref_v = [np.zeros_like(a) for a in ref_p]
+    x = torch.randn(128, 64, device="cuda").to(torch.bfloat16)
+    y = torch.randn(128, 8, device="cuda")
+    for step in range(1, 5):
+        for p in params:
+            p.grad = None
+        loss = ((torch.tanh(x @ w1) @ w2).float() - y).pow(2).mean()
+        loss.backward()
+        assert w1.grad.dtype == torch.bfloat16
+        low = lo.lans_step_mixed([to_np(p.grad) for p in params], ref_p, ref_m, ref_v, step, mo.round_to_bf16, lr=2e-3, weight_decay=0.05)
+        opt.step()
+        for p, master, want in zip(params, opt.master, low):
+            assert torch.equal(p.detach(), master.to(torch.bfloat16))
+        # the model's parameters feed the next gradients: keep the oracle on the device's values
+        for a, master in zip(ref_p, opt.master):
+            assert_close_scaled(to_np(master), a, 2e-6, "master parameter")
+            a[...] = to_np(master)

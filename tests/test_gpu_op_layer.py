@@ -80,6 +80,96 @@ def test_lans_through_the_op_layer_with_cached_openv(pkg, ex, monkeypatch, sched
     call.close()
 
 
+@pytest.mark.parametrize("full_size", [False, True])
+def test_config4_pattern_both_ways_through_the_op_layer(pkg, ex, full_size):
+    """Config 4's dispatch (4 token partitions, top-2) through the executor in the two forms the op layer offers:
+    as the partition pass emits it (src/pass/dist_optimization/partition_exprs.cc:1709-1874: one moe_encode per
+    (slot, partition) chained through used_capacity, moe_merge_masks, moe_redispatch) and rewritten to the
+    routed-once form (moe_route over the whole gate, moe_scatter_tokens per partition in place on one buffer,
+    moe_decode_tokens per partition).  Masks, capacities, the [E, C, M] buffer and the combined output must be
+    equal, bit for bit (the weights to 1e-5: the chained form normalises them in a separate op)."""
+    ops = pkg.ops
+    if full_size:
+        S0, M, E, cf, P, dt = 65536, 4096, 32, 1.25, 4, torch.bfloat16
+    else:
+        S0, M, E, cf, P, dt = 4096, 64, 8, 0.5, 4, torch.bfloat16
+    S = S0 // P
+    rng = np.random.default_rng(0)
+    data = torch.from_numpy(rng.standard_normal((S0, M), dtype=np.float32)).cuda().to(dt)
+    h_logits = rng.standard_normal((S0, E), dtype=np.float32)
+    h_logits[:, :2] += np.float32(0.75)                     # favoured experts: slots overflow
+    logits = torch.from_numpy(h_logits).cuda()
+    zero = torch.zeros(E, dtype=torch.int32, device="cuda")
+    # ---- routed once
+    gates_s, il, used, elems = ex("raf.op.moe_route", logits, zero, M, cf, 2, 1)
+    Cap = ops.moe_capacity(S0, E, 2 * cf)
+    buf = torch.full((E, Cap, M), 7.0, dtype=dt, device="cuda")
+    for p in range(P):
+        out = ex("raf.op.moe_scatter_tokens", data[p * S:(p + 1) * S], il, zero, used, buf, p * S, 2, p == P - 1)
+        assert out.data_ptr() == buf.data_ptr()            # in place
+    starts, counts = ex("raf.op.moe_partition_ranges", il, P, E, M, 2)
+    outs = [ex("raf.op.moe_decode_tokens", buf, gates_s, il, p * S, S, 2) for p in range(P)]
+    # ---- as the partition pass emits it
+    sel = torch.empty((2, S0), dtype=torch.int32, device="cuda")
+    val = torch.empty((2, S0), dtype=torch.float32, device="cuda")
+    import ctypes as C
+    assert pkg.capi.load().lancet_gate_topk(C.c_void_p(logits.data_ptr()), None, S0, E, 2, pkg.capi.F32, pkg.capi.GATE_IS_LOGITS,
+                                            C.c_void_p(sel.data_ptr()), C.c_void_p(val.data_ptr()), None) == 0
+    u = zero
+    ils, bufs, raws = [], [], []
+    for slot in range(2):
+        for p in range(P):
+            sl = slice(p * S, (p + 1) * S)
+            gate = torch.full((S, E), -1.0, device="cuda")
+            gate.scatter_(1, sel[slot, sl].long()[:, None], val[slot, sl][:, None])
+            g, pil, u, pel, disp = ex("raf.op.moe_encode", data[sl], gate, u, 2 * cf * P, 1, 0, 0)   # no tail zero-fill: feeds redispatch
+            ils.append(pil), bufs.append(disp), raws.append(g)
+    merged = ex("raf.op.moe_merge_masks", ils, E)
+    red = ex("raf.op.moe_redispatch", bufs, ils)
+    del bufs
+    weights = ops.moe_top2_normalize_gates(torch.cat(raws), merged)
+    assert bool((merged[0] < 0).any())
+    assert torch.equal(merged, il) and torch.equal(u, used) and torch.equal(red, buf)
+    np.testing.assert_allclose(to_np(weights), to_np(gates_s), rtol=1e-5)
+    whole = ex("raf.op.moe_decode", red, gates_s, merged, 2)
+    assert torch.equal(torch.cat(outs), whole)
+    # the ranges are the partitions' own element counts, in capacity order
+    kept = torch.stack([(il[0, j * S0 + p * S: j * S0 + (p + 1) * S].long().clamp_min(-1) + 1).bincount(minlength=E + 1)[1:]
+                        for j in range(2) for p in range(P)])
+    assert torch.equal(counts.view(torch.int64), kept * M)
+    assert torch.equal(starts.view(torch.int64), (torch.cumsum(kept, 0) - kept) * M)
+
+
+def test_gate_gradient_and_mixed_lans_through_the_op_layer(pkg, ex):
+    S, M, E = 3000, 16, 16
+    data, logits = make_inputs(17, S, M, E, zipf_bias=True)
+    want = mo.moe_encode_top2(data, logits, np.zeros(E, np.int32), 0.7, gate_is_logits=True, fast_scatter=True)
+    dy = np.random.default_rng(2).standard_normal(2 * S).astype(np.float32)
+    got = ex("raf.op.moe_encode_dgate", dev(dy), dev(logits), dev(want[1]), 2, 1)
+    ref = mo.moe_encode_dgate(dy, logits, want[1], 2, True)
+    scale = np.abs(ref).max(axis=1, keepdims=True)
+    assert (np.abs(to_np(got) - ref) <= 1e-5 * np.abs(ref) + 1e-6 * scale).all()
+    # lans with bf16 gradients and bf16 parameter copies (trailing tuple argument)
+    shapes = [(128, 64), (33,), (2, 8192)]
+    rng = np.random.default_rng(1)
+    p = [rng.normal(0, 0.02, s).astype(np.float32) for s in shapes]
+    m = [np.zeros(s, np.float32) for s in shapes]
+    v = [np.zeros(s, np.float32) for s in shapes]
+    g = [mo.round_to_bf16(rng.normal(0, 1e-3, s).astype(np.float32)) for s in shapes]
+    dg = [dev(a).to(torch.bfloat16) for a in g]
+    dp, dm, dv = ([dev(a) for a in l] for l in (p, m, v))
+    low = [torch.zeros(s, dtype=torch.bfloat16, device="cuda") for s in shapes]
+    call = ex.prepare("raf.op.lans", dg + dp + dm + dv, 1, 1e-3, 0.9, 0.999, 1e-6, 1, 0.01, 1, 1, True, low)
+    assert call.arg_indices == [0, 1, 11]
+    call.run()
+    torch.cuda.synchronize()
+    lo.lans_step_mixed(g, p, m, v, 1, mo.round_to_bf16)
+    for a, b, c in zip(dp, p, low):
+        assert np.abs(to_np(a).astype(np.float64) - b).max() <= 1e-6 * np.abs(b).max()
+        assert torch.equal(c, a.to(torch.bfloat16))
+    call.close()
+
+
 def test_executor_reports_op_errors(pkg, ex):
     with pytest.raises(pkg.raf_executor.RafError, match="matching shape in dim 0"):
         ex("raf.op.moe_encode", torch.zeros((8, 4), device="cuda"), torch.zeros((9, 2), device="cuda"),

@@ -42,7 +42,7 @@ def parse():
     ap.add_argument("--lans-scale", type=float, default=1.0, help="fraction of the 24-layer LANS tensor list")
     ap.add_argument("--lans-schedule", default=None, choices=["sweeps", "resident"],
                     help="time only this LANS schedule (profiling)")
-    ap.add_argument("--only", default="all", choices=["all", "scatter", "decode", "route", "route_forms", "copy", "stream_copy", "lans"],
+    ap.add_argument("--only", default="all", choices=["all", "scatter", "scatter_dest", "decode", "decode_dest", "route", "route_forms", "copy", "stream_copy", "lans", "lans_mixed", "dgate"],
                     help="profiling aid: run just one kernel family (prints a short JSON line)")
     return ap.parse_args()
 
@@ -145,6 +145,9 @@ def bench_lans(ops, capi, steps, warmup, scale, only_schedule=None):
     primary = default if default in timed else min(timed, key=timed.get)
     ms = timed[primary]
     gbs = 28.0 * total / (ms * 1e-3) / 1e9
+    mixed = None
+    if not only_schedule:
+        mixed = bench_lans_mixed(ops, capi, numels, flat, views, hyper, state, steps, warmup, ms)
     # the ceiling: what the memory system gives a kernel with the step's access pattern and none of its
     # dependencies (4 arrays read, 3 written, one float4 per thread and array), over the same number of elements
     import ctypes as C
@@ -174,7 +177,60 @@ def bench_lans(ops, capi, steps, warmup, scale, only_schedule=None):
             # HBM bytes per parameter from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this workload
             # (profiles/lans_traffic.json); null when that file is absent
             "bytes_per_param_traffic_measured": traffic,
+            "bytes_per_param_traffic_source": "profiles/lans_traffic.json (rocprofv3 --pmc runs of this workload; not measured by this process)",
+            "mixed_precision": mixed,
             "steps": steps}
+
+
+def bench_lans_mixed(ops, capi, numels, flat, views, hyper, state, steps, warmup, ms_fp32):
+    """The step of a bf16 model on the same tensor list: bf16 gradients read as they are, fp32 master parameters
+    and moments, and the bf16 copy of every new parameter written by the same kernel (lancet_lans_step_mixed):
+    2 + 24 + 2 = 28 bytes per parameter.  Beside it the three-pass form the reference's optimizer runs
+    (python/raf/optim/lans.py:256-257, 285-288): cast the gradients to fp32, the fp32 step, cast the new parameters
+    to bf16, here with one torch cast over each flat array (6 + 28 + 6 = 40 bytes per parameter)."""
+    import torch
+    total = sum(numels)
+    g16 = flat["g"].to(torch.bfloat16)
+    low = torch.empty(total, dtype=torch.bfloat16, device="cuda")
+    g16_views, low_views = list(torch.split(g16, numels)), list(torch.split(low, numels))
+    plan = ops.LansPlan(numels)
+
+    def one():
+        plan.step(g16_views, views["p"], views["m"], views["v"], state["step"], hyper, p_lowp=low_views)
+        state["step"] += 1
+
+    for _ in range(warmup):
+        one()
+    ms = event_ms(one, steps)
+    if plan.error() != 0:
+        raise RuntimeError("the mixed-precision LANS step flagged a wait that gave up")
+    if not torch.equal(low, flat["p"].to(torch.bfloat16)):
+        raise RuntimeError("16-bit parameter copies differ from the rounded master parameters")
+    schedule = "resident" if plan.schedule() == capi.LANS_RESIDENT else "sweeps"
+    plan.close()
+    g32 = torch.empty(total, device="cuda")
+    plan32 = ops.LansPlan(numels)
+    g32_views = list(torch.split(g32, numels))
+
+    def three_pass():
+        g32.copy_(g16)
+        plan32.step(g32_views, views["p"], views["m"], views["v"], state["step"], hyper)
+        low.copy_(flat["p"])
+        state["step"] += 1
+
+    for _ in range(warmup):
+        three_pass()
+    ms3 = event_ms(three_pass, steps)
+    plan32.close()
+    gbs = 28.0 * total / (ms * 1e-3) / 1e9
+    return {"what": "bf16 gradients in, fp32 master p / m / v, bf16 copies of the new parameters out, one pass",
+            "schedule": schedule, "ms_per_step": round(ms, 4), "bytes_per_param_algorithmic": 28,
+            "algorithmic_GBps": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+            "three_pass_form": {"what": "torch cast of the flat bf16 gradients to fp32, the fp32 step, torch cast of the "
+                                        "flat new parameters to bf16 (40 bytes per parameter)",
+                                "ms_per_step": round(ms3, 4), "bytes_per_param": 40,
+                                "GBps_of_its_own_bytes": round(40.0 * total / (ms3 * 1e-3) / 1e9, 1)},
+            "speedup_over_three_pass": round(ms3 / ms, 3), "ms_fp32_step": round(ms_fp32, 4)}
 
 
 def profile_figure(key):
@@ -238,6 +294,7 @@ def cpu_baseline(data_bits, logits, cf, budget_s=10.0):
         mo.moe_decode(disp, g, il, k=1)
         times.append(time.perf_counter() - t0)
     t_np = sorted(times[1:])[2]
+    numpy_more = numpy_side_configs()
     return {"value": round(S / t_all, 1), "unit": "tokens/s", "cores": cores, "kind": "port",
             "sample": "C/OpenMP restatement, %d whole top-2 encode+decode passes over the headline's own arrays "
                       "(S=%d M=%d E=%d, median %.3f s per pass, %d threads)" % (n_all, S, M, E, t_all, cores),
@@ -245,19 +302,93 @@ def cpu_baseline(data_bits, logits, cf, budget_s=10.0):
             "threads_1": {"threads": 1, "s_per_pass": round(t_one, 4), "tokens_per_s": round(S / t_one, 1), "passes": n_one},
             "numpy_config1": {"what": "NumPy restatement in the reference tests' style (one-hot + cumsum, Python scatter "
                                       "loop), top-1 encode + decode, S=4096 M=768 fp32 E=8 C=640, one core, median of 5",
-                              "s_per_pass": round(t_np, 4), "tokens_per_s": round(4096 / t_np, 1)}}
+                              "s_per_pass": round(t_np, 4), "tokens_per_s": round(4096 / t_np, 1)},
+            "numpy_config2": numpy_more.get("config2"), "numpy_config3": numpy_more.get("config3")}
+
+
+def numpy_side_configs(limit_s=60.0):
+    """The NumPy restatement (reference tests' style, one core) on BASELINE configs 2 and 3, encode + decode per pass:
+    one warm-up pass, then the median of 3, unless the warm-up alone shows that the leg would not finish within
+    limit_s (then the record says so)."""
+    import numpy as np
+    from oracle import moe_oracle as mo
+    out = {}
+
+    def leg(name, what, S, make, run):
+        args = make()
+        t0 = time.perf_counter()
+        run(*args)
+        first = time.perf_counter() - t0
+        if first * 4 > limit_s:
+            out[name] = {"what": what, "skipped": "one pass takes %.1f s: four would not finish within %.0f s" % (first, limit_s)}
+            return
+        times = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            run(*args)
+            times.append(time.perf_counter() - t0)
+        t = sorted(times)[1]
+        out[name] = {"what": what, "s_per_pass": round(t, 4), "tokens_per_s": round(S / t, 1)}
+
+    def make2():
+        rng = np.random.default_rng(0)
+        S, M, E = 16384, 1024, 16
+        data = rng.standard_normal((S, M), dtype=np.float32)
+        logits = rng.standard_normal((S, E), dtype=np.float32)
+        r = np.arange(1, E + 1, dtype=np.float64)
+        bias = 3.0 * (r ** -1.2 - E ** -1.2) / (1.0 - E ** -1.2)
+        return data, (logits + bias[rng.permutation(E)].astype(np.float32)[None, :]).astype(np.float32)
+
+    def run2(data, logits):
+        g, il, _, _, disp = mo.moe_encode_top2(data, logits, np.zeros(16, np.int32), 1.0, gate_is_logits=True)
+        mo.moe_decode(disp, g, il, k=2)
+
+    def make3():
+        rng = np.random.default_rng(0)
+        S, M, E = 32768, 2048, 64
+        data = mo.round_to_bf16(rng.standard_normal((S, M), dtype=np.float32))
+        return data, mo.softmax_rows(rng.standard_normal((S, E), dtype=np.float32) * np.float32(2.0))
+
+    def run3(data, gate):
+        g, il, _, _, disp = mo.moe_encode_bpr(data, gate, 1, 0, 1.25)
+        mo.moe_decode(disp, g, il, k=1)
+
+    leg("config2", "top-2 encode + decode, S=16384 M=1024 fp32 E=16 C=2048, Zipf expert bias, one core", 16384, make2, run2)
+    leg("config3", "batch-prioritised encode + decode, S=32768 M=2048 (bf16 values held as fp32) E=64 C=640, one core",
+        32768, make3, run3)
+    return out
+
+
+def host_memory_available_gb():
+    """MemAvailable of /proc/meminfo in GB (0 when it cannot be read)."""
+    try:
+        with open("/proc/meminfo") as f:
+            for line in f:
+                if line.startswith("MemAvailable:"):
+                    return int(line.split()[1]) * 1024 / 1e9
+    except (OSError, ValueError):
+        pass
+    return 0.0
 
 
 def cpu_baseline_lans(hyper_steps=2):
-    """C/OpenMP LANS on the 32 expert tensors of one MoE layer (134M parameters)."""
+    """C/OpenMP LANS on the host: the whole 674-tensor list of config 5 when the host has 48 GB available (the four
+    arrays take 27.4 GB), else the 32 expert tensors of one MoE layer (134M parameters); the record says which."""
     import numpy as np
     from oracle import c_oracle
     cores = len(os.sched_getaffinity(0))
     c_oracle.set_num_threads(cores)
-    shapes = [(1024, 4096), (4096, 1024)] * 16
+    avail = host_memory_available_gb()
+    full = avail >= 48.0
+    shapes = lans_shapes(1.0) if full else [(1024, 4096), (4096, 1024)] * 16
     rng = np.random.default_rng(0)
-    p = [rng.standard_normal(s, dtype=np.float32) * np.float32(0.02) for s in shapes]
-    g = [rng.standard_normal(s, dtype=np.float32) * np.float32(1e-3) for s in shapes]
+    # one random draw per distinct shape, copied to every tensor of that shape: the time of a step does not depend
+    # on the values, and drawing 3.4e9 normals would take longer than the timed steps
+    draw = {}
+    for sh in set(shapes):
+        draw[sh] = (rng.standard_normal(sh, dtype=np.float32) * np.float32(0.02), rng.standard_normal(sh, dtype=np.float32) * np.float32(1e-3))
+    p = [draw[sh][0].copy() for sh in shapes]
+    g = [draw[sh][1].copy() for sh in shapes]
     m = [np.zeros(s, np.float32) for s in shapes]
     v = [np.zeros(s, np.float32) for s in shapes]
     total = sum(a.size for a in p)
@@ -269,7 +400,9 @@ def cpu_baseline_lans(hyper_steps=2):
     dt = (time.perf_counter() - t0) / hyper_steps
     return {"params": total, "tensors": len(shapes), "ms_per_step": round(dt * 1e3, 2), "cores": cores,
             "algorithmic_GBps": round(28.0 * total / dt / 1e9, 2), "ns_per_param": round(dt / total * 1e9, 3),
-            "kind": "port", "sample": "C/OpenMP restatement, one MoE layer's 32 expert tensors"}
+            "kind": "port", "host_memory_available_GB": round(avail, 1),
+            "sample": ("C/OpenMP restatement, the whole config 5 list (674 tensors), %d timed steps after one warm-up" % hyper_steps) if full
+            else "C/OpenMP restatement, one MoE layer's 32 expert tensors (the host has less than 48 GB available for the whole list)"}
 
 
 def bench_config4_partitioned(pkg, ops, lib, capi, data, logits, S, M, E, cf, iters):
@@ -439,7 +572,12 @@ def bench_config4_partitioned(pkg, ops, lib, capi, data, logits, S, M, E, cf, it
                                 frac_of_hbm_peak=round((alg_shared - S * M * b - 2 * (2 * S) * 8) /
                                                        (seq_routed["ms_sequence"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)),
             "note": "token rows are read once per slot (two passes) in this call pattern; "
-                    "partition encodes write used rows only (zero_tail=False), redispatch zero-fills the merged tail"}
+                    "partition encodes write used rows only (zero_tail=False), redispatch zero-fills the merged tail.  "
+                    "The sequence is 8 encodes x (2 routing kernels + 1 scatter) + merge_masks (clear, count, merge) + redispatch "
+                    "(clear, count, row mover) + decode: 31 dependent launches of which 21 are minimum-length kernels of "
+                    "3-10 us that the used_capacity chain serialises, so 0.12-0.15 ms of the 1.15-1.2 ms moves no rows: "
+                    "0.59-0.61 of peak is this call pattern's floor, run to run.  routed_once (raf.op.moe_route + moe_scatter_tokens + "
+                    "moe_decode_tokens in the op layer) is the supported form of the same dispatch."}
 
 
 def bench_pipeline(pkg, data, logits, S, M, E, cf, iters):
@@ -530,10 +668,14 @@ def bench_backward(ops, data, outs, dec, S, M, E, Cap, K, kept, iters):
     dbuf = torch.empty_like(disp)
     dgs = torch.empty(K * S, device="cuda")
     ws = torch.empty(E * Cap * 4, dtype=torch.uint8, device="cuda")
+    logits = torch.randn((S, E), device="cuda")
     res = {}
     for name, fn, nbytes in (
             ("encode_dx", lambda: ops.moe_encode_dx(disp, il, top_k=K, out=dx), kept * M * b + S * M * b + K * S * 8),
             ("encode_dg", lambda: ops.moe_encode_dg(g, il, E, top_k=K, out=dgate), S * E * 4 + K * S * 8),
+            # the gate gradient of the op the headline runs (top-2 on logits): through the normalisation and the softmax
+            ("encode_dgate", lambda: ops.moe_encode_dgate(g, logits, il, top_k=K, gate_is_logits=True, out=dgate),
+             2 * S * E * 4 + K * S * 8),
             ("decode_dx", lambda: ops.moe_decode_dx(dec, g, il, E, Cap, top_k=K, workspace=ws, out=dbuf),
              kept * M * b + E * Cap * M * b + K * S * 12 + 2 * E * Cap * 4),
             ("decode_dg", lambda: ops.moe_decode_dg(dec, disp, il, top_k=K, out=dgs), 2 * kept * M * b + K * S * 12)):
@@ -637,6 +779,34 @@ def main():
                                                                args.lans_schedule)}),
               flush=True)
         return
+    if args.only == "lans_mixed":
+        # the mixed-precision step alone (bf16 gradients in, bf16 parameter copies out), for profiler runs
+        shapes = lans_shapes(args.lans_scale)
+        numels = [int(torch.Size(s).numel()) for s in shapes]
+        total = sum(numels)
+        gen = torch.Generator(device="cuda").manual_seed(0)
+        g16 = torch.empty(total, device="cuda").normal_(0, 1e-3, generator=gen).to(torch.bfloat16)
+        pm = torch.empty(total, device="cuda").normal_(0, 0.02, generator=gen)
+        m, v = torch.zeros(total, device="cuda"), torch.zeros(total, device="cuda")
+        low = torch.empty(total, dtype=torch.bfloat16, device="cuda")
+        lists = [list(torch.split(t, numels)) for t in (g16, pm, m, v, low)]
+        hyper = capi.LansHyper(1e-3, 0.9, 0.999, 1e-6, 1, 0.01, 1, 1, 1)
+        plan = ops.LansPlan(numels)
+        if args.lans_schedule:
+            plan.set_schedule(capi.LANS_SWEEPS if args.lans_schedule == "sweeps" else capi.LANS_RESIDENT)
+        state = {"step": 1}
+
+        def one():
+            plan.step(lists[0], lists[1], lists[2], lists[3], state["step"], hyper, p_lowp=lists[4])
+            state["step"] += 1
+
+        for _ in range(args.warmup):
+            one()
+        ms = event_ms(one, args.steps)
+        assert plan.error() == 0
+        print(json.dumps({"only": "lans_mixed", "params": total, "ms_per_step": round(ms, 4), "steps": args.steps + args.warmup,
+                          "algorithmic_GBps": round(28.0 * total / ms / 1e6, 1)}), flush=True)
+        return
 
     S, M, E, K, cf = args.tokens, args.hidden, args.experts, 2, 1.25
     b = 2  # bf16
@@ -719,6 +889,35 @@ def main():
                                   p(outs[1]), p(outs[2]), p(outs[3]), p(ws.buf), ws.nbytes, stream)
         assert st == 0
 
+    if args.only in ("scatter_dest", "decode_dest"):
+        # the row movers fed with one routing word per slot (lancet_debug_scatter_dest / _decode_dest): checked equal
+        # to the operator calls, then timed alone (for a counter run beside --only scatter / decode)
+        il_t = outs[1]
+        dest = torch.where(il_t[0] >= 0, il_t[0] * Cap + il_t[1], torch.full_like(il_t[0], -1)).contiguous()
+        want = (outs[4] if args.only == "scatter_dest" else dec).clone()
+
+        def one_word():
+            if args.only == "scatter_dest":
+                st = lib.lancet_debug_scatter_dest(p(data), p(dest), p(used_in), p(outs[2]), S, M, E, Cap, K, capi.BF16, p(outs[4]), stream)
+            else:
+                st = lib.lancet_debug_decode_dest(p(outs[4]), p(outs[0]), p(dest), S, M, E, Cap, K, capi.BF16, capi.F32, p(dec), stream)
+            assert st == 0
+
+        one_word()
+        assert torch.equal(outs[4] if args.only == "scatter_dest" else dec, want), "the one-word form differs from the operator"
+        for _ in range(args.warmup):
+            one_word()
+        ms = event_ms(one_word, args.steps)
+        print(json.dumps({"only": args.only, "ms": round(ms, 4), "steps": args.steps}), flush=True)
+        return
+    if args.only == "dgate":
+        grad = torch.empty_like(logits)
+        fn = lambda: ops.moe_encode_dgate(outs[0], logits, outs[1], top_k=K, gate_is_logits=True, out=grad)
+        for _ in range(args.warmup):
+            fn()
+        ms = event_ms(fn, args.steps)
+        print(json.dumps({"only": "dgate", "ms": round(ms, 4), "steps": args.steps, "algorithmic_bytes": 2 * S * E * 4 + K * S * 8}), flush=True)
+        return
     if args.only in ("scatter", "decode", "route"):
         fn = {"scatter": scatter_only, "decode": decode, "route": route_only}[args.only]
         for _ in range(args.warmup):
@@ -756,6 +955,8 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "scatter_rows_kernel<u32x4,2> (encode_forward)",
                      "achieved": round(scatter_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(scatter_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "traffic_source": "profiles/scatter_rows_headline_traffic.json: HBM bytes per launch from rocprofv3 --pmc "
+                                       "FETCH_SIZE / WRITE_SIZE runs of this workload (a stored figure, not measured by this process)",
                      "algorithmic_bytes_per_launch": scatter_bytes, "avg_launch_ms": round(ms_scatter, 4)},
         "ops": {
             "encode": {"ms": round(ms_enc, 4), "algorithmic_bytes": enc_bytes,

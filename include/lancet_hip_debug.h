@@ -51,6 +51,17 @@ int lancet_debug_stream(int kind, void* dst, const void* src, size_t bytes, lanc
  * 28 bytes per element, with a few multiply-adds in between, one float4 per thread and array.  bench.py times
  * it beside the LANS step: what the memory system delivers to a kernel that needs no norms. */
 int lancet_debug_stream_4r3w(const float* g, float* p, float* m, float* v, size_t n, lancet_stream_t stream);
+/* Measurement aid (no counterpart in the reference): lancet_moe_scatter and lancet_moe_decode fed with ONE routing
+ * word per slot instead of the four of indices_locations and the capacity arrays: dest[j*S + s] = e * C + location of
+ * slot j of token s, -1 when the slot moves no row.  Rows of whole 16-byte granules only.  Results are those of the
+ * operator calls.  Built to test whether the routing words a wave reads in front of its row cost the row movers
+ * their distance to a plain copy; measured slower than the four-word form (339 against 333 us, 258 against 256 at
+ * S = 65536, M = 4096 bf16, E = 32, top-2), so the operators keep indices_locations as their only format. */
+int lancet_debug_scatter_dest(const void* data, const int32_t* dest, const int32_t* used_in, const int32_t* used_out,
+                              int64_t S, int64_t M, int64_t E, int64_t C, int top_k, int dtype, void* dispatched,
+                              lancet_stream_t stream);
+int lancet_debug_decode_dest(const void* expert_out, const void* gates_s, const int32_t* dest, int64_t S, int64_t M,
+                             int64_t E, int64_t C, int top_k, int dtype, int gate_dtype, void* out, lancet_stream_t stream);
 #ifdef __cplusplus
 }
 #endif

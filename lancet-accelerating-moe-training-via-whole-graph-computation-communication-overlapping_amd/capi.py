@@ -65,6 +65,8 @@ SIGNATURES = {
     "lancet_memcpy_cont_to_sparse_ranges_3d": (_int, [_vp, _vp, _vp, _vp, _i64, _int, _int, _int, _i64, _i64, _i64, _i64, _int, _vp]),
     "lancet_moe_partition_ranges_workspace_bytes": (_sz, [_int, _int, _i64]),
     "lancet_moe_partition_ranges": (_int, [_vp, _i64, _int, _int, _i64, _i64, _vp, _vp, _vp, _sz, _vp]),
+    "lancet_debug_scatter_dest": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp]),
+    "lancet_debug_decode_dest": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _vp, _vp]),
     "lancet_debug_stream": (_int, [_int, _vp, _vp, _sz, _vp]),
     "lancet_debug_stream_4r3w": (_int, [_vp, _vp, _vp, _vp, _sz, _vp]),
     "lancet_moe_decode": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _vp, _vp]),

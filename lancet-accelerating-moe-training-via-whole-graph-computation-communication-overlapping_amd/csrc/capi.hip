@@ -158,6 +158,34 @@ extern "C" int lancet_debug_stream(int kind, void* dst, const void* src, size_t 
   return rc(hipGetLastError());
 }
 
+// Measurement aid: the scatter and the gather-combine fed with ONE routing word per slot (dest[j*S + s] = e * C + location,
+// -1 = none) instead of the four of indices_locations and the capacity arrays.
+extern "C" int lancet_debug_scatter_dest(const void* data, const int32_t* dest, const int32_t* used_in, const int32_t* used_out,
+                                         int64_t S, int64_t M, int64_t E, int64_t C, int top_k, int dtype, void* dispatched,
+                                         lancet_stream_t stream) {
+  if (!data || !dest || !used_out || !dispatched) return LANCET_ERR_NULL;
+  const int eb = elem_bytes(dtype);
+  if (!eb) return LANCET_ERR_DTYPE;
+  if (int r = check_dims(S, M, E, C)) return r;
+  if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
+  if ((M * eb) % 16 != 0 || misaligned(data, 16) || misaligned(dispatched, 16) || misaligned(dest, 4)) return LANCET_ERR_ALIGN;
+  return rc(run_scatter_rows(data, dispatched, nullptr, nullptr, nullptr, nullptr, used_in, used_out, static_cast<int>(S),
+                             static_cast<int>(M), static_cast<int>(E), static_cast<int>(C), top_k, eb, S_(stream), -1, dest));
+}
+
+extern "C" int lancet_debug_decode_dest(const void* expert_out, const void* gates_s, const int32_t* dest, int64_t S, int64_t M,
+                                        int64_t E, int64_t C, int top_k, int dtype, int gate_dtype, void* out,
+                                        lancet_stream_t stream) {
+  if (!expert_out || !gates_s || !dest || !out) return LANCET_ERR_NULL;
+  const int eb = elem_bytes(dtype), gb = elem_bytes(gate_dtype);
+  if (!eb || !gb) return LANCET_ERR_DTYPE;
+  if (int r = check_dims(S, M, E, C)) return r;
+  if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
+  if ((M * eb) % 16 != 0 || misaligned(expert_out, 16) || misaligned(out, 16) || misaligned(dest, 4)) return LANCET_ERR_ALIGN;
+  return rc(run_decode_rows(expert_out, gates_s, gate_dtype, nullptr, nullptr, out, static_cast<int>(S), static_cast<int>(M),
+                            static_cast<int>(E), static_cast<int>(C), top_k, dtype, S_(stream), -1, dest));
+}
+
 // ---- routing front end ---------------------------------------------------------------
 extern "C" int lancet_gate_topk(const void* gate, const void* gate2_noise, int64_t S, int64_t E, int top_k,
                                 int gate_dtype, unsigned flags, int32_t* idx, void* val, lancet_stream_t stream) {
@@ -553,6 +581,11 @@ extern "C" int lancet_moe_encode_dg(const void* dy_gates_s, const int32_t* indic
   if (int r = check_dims(S, 0, E, 0)) return r;
   if (top_k != 1 && top_k != 2) return LANCET_ERR_TOPK;
   if (misaligned(dy_gates_s, gb) || misaligned(indices_locations, 4) || misaligned(grad_gates, gb)) return LANCET_ERR_ALIGN;
+  // top-1: the kernel of lancet_moe_encode_dgate in its plainest form (same result; it writes the block of a
+  // workgroup's tokens in memory order, which streams several times faster on wide gates)
+  if (top_k == 1 && S * E <= 0x7fffffff)
+    return rc(run_encode_dgate(dy_gates_s, nullptr, indices_locations, static_cast<int>(S), static_cast<int>(E), 1, false,
+                               gate_dtype, grad_gates, S_(stream)));
   return rc(run_encode_dg(dy_gates_s, indices_locations, static_cast<int>(S), static_cast<int>(E), top_k, gate_dtype, grad_gates,
                           S_(stream)));
 }

@@ -47,15 +47,17 @@ hipError_t run_top2_normalize(const void* raw, const int32_t* idx, int S, int ga
 // (rows_lo may be null = zeros); otherwise the caller has cleared the buffer.  slot_stride: distance
 // between the K slots of one token in idx / loc (and gates, for decode); negative = S.  A call that
 // moves a token range of a larger mask passes pointers to the range's first token and the mask's
-// token count here.
+// token count here.  dest (may be null; rows of whole 16-byte granules only): [K*S] destination rows e * C + location,
+// -1 for none, ONE routing word per slot; idx, loc, avail_used and row_base are then not read.
 hipError_t run_scatter_rows(const void* data, void* out, const int32_t* idx, const int32_t* loc,
                             const int32_t* avail_used, const int32_t* row_base, const int32_t* rows_lo,
                             const int32_t* rows_hi,
-                            int S, int M, int E, int C, int K, int elem_bytes, hipStream_t st, int slot_stride = -1);
+                            int S, int M, int E, int C, int K, int elem_bytes, hipStream_t st, int slot_stride = -1,
+                            const int32_t* dest = nullptr);
 hipError_t run_zero_bytes(void* p, size_t nbytes, hipStream_t st);
 hipError_t run_decode_rows(const void* expert_out, const void* gates, int gate_dtype, const int32_t* idx,
                            const int32_t* loc, void* out, int S, int M, int E, int C, int K,
-                           int dtype, hipStream_t st, int slot_stride = -1);
+                           int dtype, hipStream_t st, int slot_stride = -1, const int32_t* dest = nullptr);
 
 // backward (gates == nullptr in run_decode_rows gives moe_encode_dx)
 hipError_t run_encode_dg(const void* dy, const int32_t* idx, int S, int E, int K, int gate_dtype, void* grad_gates, hipStream_t st);

@@ -10,8 +10,8 @@
 //                              d x[e] = p[e] * (d p[e] - sum_j p[i_j] * d p[i_j])
 // Probabilities of a 16-bit softmax are taken as computed (fp32), not as a 16-bit gates_s array would hold them:
 // the difference is below that type's own rounding.  Dropped slots carry no gradient (their mask is zero,
-// sharded_moe.py:296-297,306-307).  One launch: a lane per token forms the token's few scalars (row maximum,
-// 1 / sum of exponentials, the two slot gradients), then the workgroup writes its tile's [256, E] block of the
+// sharded_moe.py:296-297,306-307).  One launch: four lanes per token form the token's few scalars (row maximum,
+// 1 / sum of exponentials, the two slot gradients), then the workgroup writes its 64 tokens' block of the
 // result in memory order, every element once.
 #include "launchers.hpp"
 #include "select.hpp"
@@ -29,21 +29,31 @@ struct GateGradArgs {
   int vec;               // rows and pointers allow 16-byte granules
 };
 
-struct RowMax {
-  float top;
-  __device__ __forceinline__ void operator()(float x, int) { top = fmaxf(top, x); }
-};
-struct RowSumExp {  // sequential sum in expert order, as the forward forms it
+// A token's row is walked by kSub lanes, each taking every kSub-th 16-byte granule (or element), with the maximum
+// and the sum of exponentials kept together and rescaled when a larger value comes; the lanes' pairs are then
+// merged.  Few tokens per workgroup and few loads per lane: the launch is short (a 65536 x 32 gate is 8 MB) and
+// only gets up to the memory system's speed when many waves are in flight.
+constexpr int kSub = 4;                      // lanes per token
+constexpr int kGradTokens = kTile / kSub;    // tokens per workgroup
+
+struct MaxSum {
   float top, sum;
-  __device__ __forceinline__ void operator()(float x, int) { sum += expf(x - top); }
+  __device__ __forceinline__ void operator()(float x) {
+    if (x > top) {
+      sum = sum * expf(top - x) + 1.f;   // top = -inf at first: exp(-inf) * 0 = 0
+      top = x;
+    } else {
+      sum += expf(x - top);
+    }
+  }
 };
 
-// per-token scalars of a tile, in LDS
+// per-token scalars of a workgroup's tokens, in LDS
 struct GateGradTile {
-  int i1[kTile], i2[kTile];      // experts that receive a slot gradient (-1: none)
-  float d1[kTile], d2[kTile];    // gradient with respect to the raw value of that expert (probability or array entry)
-  float top[kTile], inv[kTile];  // logits: row maximum and 1 / sum_e exp(x - max)
-  float dot[kTile];              // logits: sum_j p[i_j] * d_j
+  int i1[kGradTokens], i2[kGradTokens];      // experts that receive a slot gradient (-1: none)
+  float d1[kGradTokens], d2[kGradTokens];    // gradient with respect to the raw value of that expert (probability or array entry)
+  float top[kGradTokens], inv[kGradTokens];  // logits: row maximum and 1 / sum_e exp(x - max)
+  float dot[kGradTokens];                    // logits: sum_j p[i_j] * d_j
 };
 
 template <int K, int GD>
@@ -52,20 +62,43 @@ __global__ __launch_bounds__(kTile) void encode_dgate_kernel(GateGradArgs a) {
   constexpr size_t gb = GD == LANCET_F32 ? 4 : 2;
   constexpr int V = 16 / gb;
   const int tid = threadIdx.x;
-  const int first = blockIdx.x * kTile;
-  const int s = first + tid;
-  // ---- a lane per token -----------------------------------------------------------------------------------
-  if (s < a.S) {
+  const int first = blockIdx.x * kGradTokens;
+  const int t = tid / kSub, sub = tid % kSub;
+  const int s = min(first + t, a.S - 1);  // lanes past the batch repeat its last token (their result is not stored)
+  // ---- kSub lanes per token ---------------------------------------------------------------------------------
+  {
     const char* row = static_cast<const char*>(a.gate) + static_cast<size_t>(s) * a.E * gb;
-    int e[2] = {-1, -1};
-    float dy[2] = {0.f, 0.f}, g[2] = {0.f, 0.f}, praw[2] = {0.f, 0.f};
     float top = 0.f, inv = 1.f;
     if (a.is_logits) {
-      RowMax mx = {-INFINITY};
-      top = walk_row<GD>(row, a.E, mx).top;
-      RowSumExp se = {top, 0.f};
-      inv = 1.f / walk_row<GD>(row, a.E, se).sum;
+      MaxSum ms = {-INFINITY, 0.f};
+      if (a.vec) {
+        const u32x4* r = reinterpret_cast<const u32x4*>(row);
+        const int n = a.E / V;
+        for (int g0 = sub; g0 < n; g0 += 2 * kSub) {  // two granules in flight per lane
+          const u32x4 x0 = r[g0];
+          const bool two = g0 + kSub < n;
+          const u32x4 x1 = two ? r[g0 + kSub] : x0;
+          auto eat = [&](float x, int) { ms(x); };
+          walk_granule<GD>(x0, 0, eat);
+          if (two) walk_granule<GD>(x1, 0, eat);
+        }
+      } else {
+        for (int j = sub; j < a.E; j += kSub) ms(gate_at<GD>(row, j));
+      }
+      // merge the kSub lanes' (max, sum) pairs: they are neighbours in the wave
+#pragma unroll
+      for (int o = 1; o < kSub; o <<= 1) {
+        const float ot = __shfl_xor(ms.top, o, kWave), os = __shfl_xor(ms.sum, o, kWave);
+        const float nt = fmaxf(ms.top, ot);
+        // a lane that saw no value holds (-inf, 0): its term is 0 whatever the other maximum is
+        ms.sum = (ms.sum > 0.f ? ms.sum * expf(ms.top - nt) : 0.f) + (os > 0.f ? os * expf(ot - nt) : 0.f);
+        ms.top = nt;
+      }
+      top = ms.top;
+      inv = 1.f / ms.sum;
     }
+    int e[2] = {-1, -1};
+    float dy[2] = {0.f, 0.f}, g[2] = {0.f, 0.f}, praw[2] = {0.f, 0.f};
 #pragma unroll
     for (int j = 0; j < K; ++j) {
       const int x = a.idx[static_cast<size_t>(j) * a.S + s];
@@ -93,24 +126,26 @@ __global__ __launch_bounds__(kTile) void encode_dgate_kernel(GateGradArgs a) {
       if (e[0] < 0) d[0] = 0.f;
       if (e[1] < 0) d[1] = 0.f;
     }
-    sh.i1[tid] = e[0];
-    sh.i2[tid] = e[1];
-    sh.d1[tid] = d[0];
-    sh.d2[tid] = d[1];
-    sh.top[tid] = top;
-    sh.inv[tid] = inv;
-    sh.dot[tid] = praw[0] * d[0] + praw[1] * d[1];
+    if (sub == 0) {
+      sh.i1[t] = e[0];
+      sh.i2[t] = e[1];
+      sh.d1[t] = d[0];
+      sh.d2[t] = d[1];
+      sh.top[t] = top;
+      sh.inv[t] = inv;
+      sh.dot[t] = praw[0] * d[0] + praw[1] * d[1];
+    }
   }
   __syncthreads();
-  // ---- the tile's block of the result, in memory order ------------------------------------------------------
-  const int ntok = min(kTile, a.S - first);
-  const size_t base = static_cast<size_t>(first) * a.E;  // first element of the tile
-  auto value = [&](int t, int ex, float x) -> float {
+  // ---- the workgroup's block of the result, in memory order ---------------------------------------------------
+  const int ntok = min(kGradTokens, a.S - first);
+  const size_t base = static_cast<size_t>(first) * a.E;  // first element of the block
+  auto value = [&](int tk, int ex, float x) -> float {
     float sel = 0.f;
-    if (ex == sh.i1[t]) sel = sh.d1[t];
-    if (K == 2 && ex == sh.i2[t]) sel = sh.d2[t];
+    if (ex == sh.i1[tk]) sel = sh.d1[tk];
+    if (K == 2 && ex == sh.i2[tk]) sel = sh.d2[tk];
     if (!a.is_logits) return sel;
-    return expf(x - sh.top[t]) * sh.inv[t] * (sel - sh.dot[t]);
+    return expf(x - sh.top[tk]) * sh.inv[tk] * (sel - sh.dot[tk]);
   };
   if (a.vec) {
     const int gpr = a.E / V;  // granules per row
@@ -118,19 +153,19 @@ __global__ __launch_bounds__(kTile) void encode_dgate_kernel(GateGradArgs a) {
     const u32x4* src = reinterpret_cast<const u32x4*>(static_cast<const char*>(a.gate) + base * gb);
     u32x4* dst = reinterpret_cast<u32x4*>(static_cast<char*>(a.out) + base * gb);
     for (int q = tid; q < n; q += kTile) {
-      const int t = q / gpr;
-      const int e0 = (q - t * gpr) * V;
+      const int tk = q / gpr;
+      const int e0 = (q - tk * gpr) * V;
       u32x4 x = {0u, 0u, 0u, 0u};
       if (a.is_logits) x = src[q];
       u32x4 r;
       if (GD == LANCET_F32) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) r[i] = __float_as_uint(value(t, e0 + i, __uint_as_float(x[i])));
+        for (int i = 0; i < 4; ++i) r[i] = __float_as_uint(value(tk, e0 + i, __uint_as_float(x[i])));
       } else {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float lo = value(t, e0 + 2 * i, half_word<GD>(x[i] & 0xffffu));
-          const float hi = value(t, e0 + 2 * i + 1, half_word<GD>(x[i] >> 16));
+          const float lo = value(tk, e0 + 2 * i, half_word<GD>(x[i] & 0xffffu));
+          const float hi = value(tk, e0 + 2 * i + 1, half_word<GD>(x[i] >> 16));
           const uint32_t l = GD == LANCET_BF16 ? f32_to_bf16(lo) : f32_to_f16(lo);
           const uint32_t h = GD == LANCET_BF16 ? f32_to_bf16(hi) : f32_to_f16(hi);
           r[i] = (l & 0xffffu) | (h << 16);
@@ -141,10 +176,10 @@ __global__ __launch_bounds__(kTile) void encode_dgate_kernel(GateGradArgs a) {
   } else {
     const int n = ntok * a.E;
     for (int q = tid; q < n; q += kTile) {
-      const int t = q / a.E;
-      const int ex = q - t * a.E;
+      const int tk = q / a.E;
+      const int ex = q - tk * a.E;
       const float x = a.is_logits ? ld_gate(a.gate, base + q, GD) : 0.f;
-      st_gate(a.out, base + q, value(t, ex, x), GD);
+      st_gate(a.out, base + q, value(tk, ex, x), GD);
     }
   }
 }
@@ -162,7 +197,7 @@ hipError_t run_encode_dgate(const void* dy, const void* gate, const int32_t* idx
   a.is_logits = is_logits;
   const int gb = gate_dtype == LANCET_F32 ? 4 : 2;
   a.vec = (static_cast<size_t>(E) * gb) % 16 == 0 && ((reinterpret_cast<uintptr_t>(gate) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
-  const int blocks = (S + kTile - 1) / kTile;
+  const int blocks = (S + kGradTokens - 1) / kGradTokens;
   LANCET_GATE_SWITCH(gate_dtype,
     if (K == 1) encode_dgate_kernel<1, GD><<<blocks, kTile, 0, st>>>(a);
     else encode_dgate_kernel<2, GD><<<blocks, kTile, 0, st>>>(a))

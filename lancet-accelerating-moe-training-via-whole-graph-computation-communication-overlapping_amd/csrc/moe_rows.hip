@@ -34,6 +34,8 @@ struct ScatterArgs {
   V* out;
   const int32_t* idx;         // [K*S]
   const int32_t* loc;         // [K*S]
+  const int32_t* dest;        // [K*S] or null: destination row e * C + location (-1: none) in ONE word per slot,
+                              // instead of idx / loc / avail_used / row_base
   const int32_t* avail_used;  // [E] or null
   const int32_t* row_base;    // [E] or null: row of expert e that location 0 maps to
   const int32_t* rows_lo;     // [E] or null
@@ -47,7 +49,7 @@ struct ScatterArgs {
   int tail_chunks;            // tail workgroups per expert
 };
 
-template <typename V, int K>
+template <typename V, int K, bool DEST = false>
 __global__ __launch_bounds__(kTile) void scatter_rows_kernel(ScatterArgs<V> a) {
   const int w = threadIdx.x / kWave;
   const int lane = threadIdx.x & (kWave - 1);
@@ -76,6 +78,12 @@ __global__ __launch_bounds__(kTile) void scatter_rows_kernel(ScatterArgs<V> a) {
     int nd = 0;
 #pragma unroll
     for (int j = 0; j < K; ++j) {
+      if (DEST) {
+        const int d = a.dest[static_cast<size_t>(j) * a.slot_stride + s];
+        dst[j] = as_global(a.out);
+        if (d >= 0 && d < a.E * a.C) dst[nd++] = as_global(a.out + static_cast<size_t>(d) * a.row_vecs);
+        continue;
+      }
       const int e = a.idx[static_cast<size_t>(j) * a.slot_stride + s];
       int l = a.loc[static_cast<size_t>(j) * a.slot_stride + s];
       bool ok = e >= 0 && e < a.E && l >= 0 && l < a.C;
@@ -206,13 +214,14 @@ struct DecodeArgs {
   int gate_dtype;
   const int32_t* idx;    // [K*S]
   const int32_t* loc;    // [K*S]
+  const int32_t* dest;   // [K*S] or null: row e * C + location of the slot (-1: none) instead of idx / loc
   void* out;             // [S, M]
   int S, M, E, C;
   int slot_stride;       // distance between the slots of one token in gates / idx / loc
   int wpr_shift;         // 2^wpr_shift waves share one token row (each takes every 2^wpr_shift-th run of 64 granules)
 };
 
-template <int DT, int K, bool VEC>
+template <int DT, int K, bool VEC, bool DEST = false>
 __global__ __launch_bounds__(kTile) void decode_rows_kernel(DecodeArgs a) {
   typedef Codec<DT> Cd;
   const int w = threadIdx.x / kWave;
@@ -228,11 +237,17 @@ __global__ __launch_bounds__(kTile) void decode_rows_kernel(DecodeArgs a) {
   bool any = false;
 #pragma unroll
   for (int j = 0; j < K; ++j) {
-    const int e = a.idx[static_cast<size_t>(j) * a.slot_stride + s];
-    const int l = a.loc[static_cast<size_t>(j) * a.slot_stride + s];
-    ok[j] = e >= 0 && e < a.E && l >= 0 && l < a.C;
+    if (DEST) {
+      const int d = a.dest[static_cast<size_t>(j) * a.slot_stride + s];
+      ok[j] = d >= 0 && d < a.E * a.C;
+      row[j] = ok[j] ? static_cast<size_t>(d) : 0;
+    } else {
+      const int e = a.idx[static_cast<size_t>(j) * a.slot_stride + s];
+      const int l = a.loc[static_cast<size_t>(j) * a.slot_stride + s];
+      ok[j] = e >= 0 && e < a.E && l >= 0 && l < a.C;
+      row[j] = ok[j] ? (static_cast<size_t>(e) * a.C + l) : 0;
+    }
     g[j] = ok[j] ? (a.gates ? ld_gate(a.gates, static_cast<size_t>(j) * a.slot_stride + s, a.gate_dtype) : 1.f) : 0.f;
-    row[j] = ok[j] ? (static_cast<size_t>(e) * a.C + l) : 0;
     any = any || ok[j];
   }
   if (VEC) {
@@ -598,8 +613,9 @@ template <typename V>
 static hipError_t scatter_launch(const void* data, void* out, const int32_t* idx, const int32_t* loc,
                                  const int32_t* avail_used, const int32_t* row_base, const int32_t* rows_lo,
                                  const int32_t* rows_hi, int S, int E, int C, int K, int row_vecs,
-                                 int slot_stride, hipStream_t st) {
+                                 int slot_stride, hipStream_t st, const int32_t* dest = nullptr) {
   ScatterArgs<V> a;
+  a.dest = dest;
   a.data = static_cast<const V*>(data);
   a.out = static_cast<V*>(out);
   a.idx = idx;
@@ -619,7 +635,10 @@ static hipError_t scatter_launch(const void* data, void* out, const int32_t* idx
   a.tail_chunks = rows_hi ? (C + kTailRows - 1) / kTailRows : 0;
   const long blocks = static_cast<long>(a.token_blocks) + static_cast<long>(a.tail_chunks) * E;
   if (blocks == 0) return hipSuccess;
-  if (K == 1) scatter_rows_kernel<V, 1><<<static_cast<unsigned>(blocks), kTile, 0, st>>>(a);
+  if (dest) {
+    if (K == 1) scatter_rows_kernel<V, 1, true><<<static_cast<unsigned>(blocks), kTile, 0, st>>>(a);
+    else scatter_rows_kernel<V, 2, true><<<static_cast<unsigned>(blocks), kTile, 0, st>>>(a);
+  } else if (K == 1) scatter_rows_kernel<V, 1><<<static_cast<unsigned>(blocks), kTile, 0, st>>>(a);
   else scatter_rows_kernel<V, 2><<<static_cast<unsigned>(blocks), kTile, 0, st>>>(a);
   return hipGetLastError();
 }
@@ -627,13 +646,15 @@ static hipError_t scatter_launch(const void* data, void* out, const int32_t* idx
 hipError_t run_scatter_rows(const void* data, void* out, const int32_t* idx, const int32_t* loc,
                             const int32_t* avail_used, const int32_t* row_base, const int32_t* rows_lo,
                             const int32_t* rows_hi,
-                            int S, int M, int E, int C, int K, int elem_bytes, hipStream_t st, int slot_stride) {
+                            int S, int M, int E, int C, int K, int elem_bytes, hipStream_t st, int slot_stride,
+                            const int32_t* dest) {
   const size_t row_bytes = static_cast<size_t>(M) * elem_bytes;
   if (row_bytes == 0) return hipSuccess;
   const int ss = slot_stride < 0 ? S : slot_stride;
   if (row_bytes % 16 == 0 && aligned16(data) && aligned16(out))
     return scatter_launch<u32x4>(data, out, idx, loc, avail_used, row_base, rows_lo, rows_hi, S, E, C, K,
-                                 static_cast<int>(row_bytes / 16), ss, st);
+                                 static_cast<int>(row_bytes / 16), ss, st, dest);
+  if (dest) return hipErrorInvalidValue;  // the one-word form is for rows of 16-byte granules
   if (elem_bytes == 4)
     return scatter_launch<uint32_t>(data, out, idx, loc, avail_used, row_base, rows_lo, rows_hi, S, E, C, K, M, ss, st);
   return scatter_launch<uint16_t>(data, out, idx, loc, avail_used, row_base, rows_lo, rows_hi, S, E, C, K, M, ss, st);
@@ -665,7 +686,11 @@ static hipError_t decode_launch(DecodeArgs a, int K, bool vec, hipStream_t st) {
   if (a.S == 0 || a.M == 0) return hipSuccess;
   a.wpr_shift = split_waves(vec ? a.M / Codec<DT>::kPerVec : a.M, a.S, 2);
   const unsigned blocks = static_cast<unsigned>(((static_cast<long>(a.S) << a.wpr_shift) + kRowsPerBlock - 1) / kRowsPerBlock);
-  if (K == 1) {
+  if (a.dest) {
+    if (!vec) return hipErrorInvalidValue;
+    if (K == 1) decode_rows_kernel<DT, 1, true, true><<<blocks, kTile, 0, st>>>(a);
+    else decode_rows_kernel<DT, 2, true, true><<<blocks, kTile, 0, st>>>(a);
+  } else if (K == 1) {
     if (vec) decode_rows_kernel<DT, 1, true><<<blocks, kTile, 0, st>>>(a);
     else decode_rows_kernel<DT, 1, false><<<blocks, kTile, 0, st>>>(a);
   } else {
@@ -677,8 +702,9 @@ static hipError_t decode_launch(DecodeArgs a, int K, bool vec, hipStream_t st) {
 
 hipError_t run_decode_rows(const void* expert_out, const void* gates, int gate_dtype, const int32_t* idx,
                            const int32_t* loc, void* out, int S, int M, int E, int C, int K,
-                           int dtype, hipStream_t st, int slot_stride) {
+                           int dtype, hipStream_t st, int slot_stride, const int32_t* dest) {
   DecodeArgs a;
+  a.dest = dest;
   a.expert_out = expert_out;
   a.gates = gates;
   a.gate_dtype = gate_dtype;

@@ -230,7 +230,9 @@ def bench_lans_mixed(ops, capi, numels, flat, views, hyper, state, steps, warmup
                                         "flat new parameters to bf16 (40 bytes per parameter)",
                                 "ms_per_step": round(ms3, 4), "bytes_per_param": 40,
                                 "GBps_of_its_own_bytes": round(40.0 * total / (ms3 * 1e-3) / 1e9, 1)},
-            "speedup_over_three_pass": round(ms3 / ms, 3), "ms_fp32_step": round(ms_fp32, 4)}
+            "speedup_over_three_pass": round(ms3 / ms, 3), "ms_fp32_step": round(ms_fp32, 4),
+            # from rocprofv3 --pmc runs of `--only lans_mixed` (profiles/lans_traffic.json), not measured by this process
+            "bytes_per_param_traffic_measured": (profile_figure("lans_traffic_bytes_per_param") or {}).get("resident_mixed_bf16")}
 
 
 def profile_figure(key):

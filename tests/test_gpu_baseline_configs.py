@@ -236,3 +236,45 @@ def test_config5_lans_full_size(pkg):
         assert bool((ps[i] != p0[i]).any())                         # every tensor was stepped
     for name in ("sweeps", "resident"):
         state[name][3].close()
+
+
+def test_config5_lans_mixed_precision_full_size(pkg):
+    """Config 5's 674 tensors as a bf16 model trains them: bf16 gradients, fp32 master parameters and moments, and the
+    model's bf16 parameters written by the same step (lancet_lans_step_mixed), resident schedule, 4 steps.  The oracle
+    (cast up, lans_step, cast down: python/raf/optim/lans.py:256-257, 285-288) follows a sample of tensors of every
+    shape; over the whole list every 16-bit copy must be the rounded master parameter, bit for bit."""
+    import importlib
+    lo = importlib.import_module("oracle.lans_oracle")
+    ops, capi = pkg.ops, pkg.capi
+    free, _ = torch.cuda.mem_get_info()
+    if free < 50 << 30:
+        pytest.skip("needs 50 GiB of free device memory")
+    shapes = _config5_shapes()
+    numels = [int(np.prod(s)) for s in shapes]
+    gen = torch.Generator(device="cuda").manual_seed(6)
+    p = [torch.randn(s, generator=gen, device="cuda") * 0.02 for s in shapes]
+    m = [torch.zeros_like(x) for x in p]
+    v = [torch.zeros_like(x) for x in p]
+    low = [torch.zeros(s, dtype=torch.bfloat16, device="cuda") for s in shapes]
+    g = [torch.empty(s, dtype=torch.bfloat16, device="cuda") for s in shapes]
+    sample = [0, 4, 12, 16, 24, 25, 300, 341, 672, 673]
+    ref_p = [to_np(p[i]) for i in sample]
+    ref_m = [np.zeros(shapes[i], np.float32) for i in sample]
+    ref_v = [np.zeros(shapes[i], np.float32) for i in sample]
+    plan = ops.LansPlan(numels)
+    assert plan.schedule() == capi.LANS_RESIDENT
+    hyper = capi.LansHyper(1e-3, 0.9, 0.999, 1e-6, 1, 0.01, 1, 1, 1)
+    for step in range(1, 5):
+        for x in g:
+            x.copy_(torch.empty(x.shape, device="cuda").normal_(0.0, 1e-3, generator=gen))
+        plan.step(g, p, m, v, step, hyper, p_lowp=low)
+        lo.lans_step_mixed([to_np(g[i]) for i in sample], ref_p, ref_m, ref_v, step, mo.round_to_bf16)
+    torch.cuda.synchronize()
+    assert plan.error() == 0 and plan.last_resident_slots() > 0
+    for i in range(len(shapes)):
+        assert torch.equal(low[i], p[i].to(torch.bfloat16)), i
+    for k, i in enumerate(sample):
+        for got, want, tol, what in ((p[i], ref_p[k], 1e-6, "p"), (m[i], ref_m[k], 1e-5, "m"), (v[i], ref_v[k], 1e-5, "v")):
+            err = np.abs(to_np(got).astype(np.float64) - want).max()
+            assert err <= tol * np.abs(want).max(), "%s[%d]: %.3e" % (what, i, err)
+    plan.close()

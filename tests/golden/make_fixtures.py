@@ -6,7 +6,8 @@ NumPy oracle after it has passed tests/test_oracle_*.py (brute force, dense GSha
 fp64 LANS).  They freeze the oracle's behaviour: a later edit of the oracle that changes any
 output fails tests/test_golden.py, and the HIP path is checked against the same files.
 
-    python tests/golden/make_fixtures.py
+    python tests/golden/make_fixtures.py            # writes the files that do not exist yet (existing ones stay frozen)
+    python tests/golden/make_fixtures.py --force    # rewrites all of them
 """
 import os
 import sys
@@ -90,8 +91,41 @@ def main():
     for i in range(3):
         lans["p3_%d" % i], lans["m3_%d" % i], lans["v3_%d" % i] = p[i], m[i], v[i]
     out["lans"] = lans
+    # gate gradient of the whole op: top-1 / top-2, on probabilities / on logits, with dropped slots of every kind
+    data, logits = inputs(7, 72, 2, 6, hot=True)
+    dgate = dict(logits=logits)
+    rng = np.random.default_rng(8)
+    for k in (1, 2):
+        for is_logits in (0, 1):
+            gate = logits if is_logits else mo.softmax_rows(logits)
+            enc = mo.moe_encode_top2 if k == 2 else mo.moe_encode
+            il = enc(data, gate, np.zeros(6, np.int32), 0.6, gate_is_logits=bool(is_logits))[1]
+            dy = rng.standard_normal(k * 72).astype(np.float32)
+            tag = "k%d_l%d" % (k, is_logits)
+            dgate["gate_" + tag], dgate["indloc_" + tag], dgate["dy_" + tag] = gate, il, dy
+            dgate["grad_" + tag] = mo.moe_encode_dgate(dy, gate, il, k, bool(is_logits))
+    out["encode_dgate"] = dgate
+    # LANS of a bf16 model: bf16 gradients, fp32 master state, bf16 copies of the new parameters; 3 tensors, 3 steps
+    rng = np.random.default_rng(9)
+    p = [rng.normal(0, 0.02, s).astype(np.float32) for s in shapes]
+    m = [np.zeros(s, np.float32) for s in shapes]
+    v = [np.zeros(s, np.float32) for s in shapes]
+    mixed = {"p0_%d" % i: a.copy() for i, a in enumerate(p)}
+    for step in (1, 2, 3):
+        g = [mo.round_to_bf16(rng.normal(0, 1e-3, s).astype(np.float32)) for s in shapes]
+        for i, a in enumerate(g):
+            mixed["g%d_%d" % (step, i)] = a
+        low = lo.lans_step_mixed(g, p, m, v, step, mo.round_to_bf16)
+    for i in range(3):
+        mixed["p3_%d" % i], mixed["m3_%d" % i], mixed["v3_%d" % i], mixed["low3_%d" % i] = p[i], m[i], v[i], low[i]
+    out["lans_mixed"] = mixed
+    force = "--force" in sys.argv[1:]
     for name, arrays in out.items():
-        np.savez_compressed(os.path.join(HERE, name + ".npz"), **arrays)
+        path = os.path.join(HERE, name + ".npz")
+        if os.path.exists(path) and not force:
+            print("kept ", name)
+            continue
+        np.savez_compressed(path, **arrays)
         print("wrote", name, sum(a.nbytes for a in arrays.values()), "bytes")
 
 

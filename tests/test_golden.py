@@ -54,6 +54,56 @@ def test_oracle_reproduces_fixtures():
         np.testing.assert_array_equal(v[i], f["v3_%d" % i])
 
 
+def test_oracle_reproduces_the_gradient_and_mixed_precision_fixtures():
+    f = gold("encode_dgate")
+    for k in (1, 2):
+        for is_logits in (0, 1):
+            tag = "k%d_l%d" % (k, is_logits)
+            got = mo.moe_encode_dgate(f["dy_" + tag], f["gate_" + tag], f["indloc_" + tag], k, bool(is_logits))
+            np.testing.assert_array_equal(got, f["grad_" + tag])
+            assert (f["indloc_" + tag][0] < 0).any() and np.abs(f["grad_" + tag]).max() > 0
+    f = gold("lans_mixed")
+    p = [f["p0_%d" % i].copy() for i in range(3)]
+    m = [np.zeros_like(a) for a in p]
+    v = [np.zeros_like(a) for a in p]
+    for step in (1, 2, 3):
+        low = lo.lans_step_mixed([f["g%d_%d" % (step, i)] for i in range(3)], p, m, v, step, mo.round_to_bf16)
+    for i in range(3):
+        np.testing.assert_array_equal(p[i], f["p3_%d" % i])
+        np.testing.assert_array_equal(low[i], f["low3_%d" % i])
+        np.testing.assert_array_equal(mo.round_to_bf16(f["p3_%d" % i]), f["low3_%d" % i])
+
+
+@pytest.mark.gpu
+def test_hip_path_reproduces_the_gradient_and_mixed_precision_fixtures(pkg):
+    import torch
+    from tests.gpu_util import dev, to_np
+    ops = pkg.ops
+    f = gold("encode_dgate")
+    for k in (1, 2):
+        for is_logits in (0, 1):
+            tag = "k%d_l%d" % (k, is_logits)
+            got = to_np(ops.moe_encode_dgate(dev(f["dy_" + tag]), dev(f["gate_" + tag]), dev(f["indloc_" + tag]), top_k=k,
+                                             gate_is_logits=bool(is_logits)))
+            want = f["grad_" + tag]
+            scale = np.abs(want).max(axis=1, keepdims=True)
+            assert (np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-6 * scale).all()
+    f = gold("lans_mixed")
+    p = [dev(f["p0_%d" % i]) for i in range(3)]
+    m = [torch.zeros_like(a) for a in p]
+    v = [torch.zeros_like(a) for a in p]
+    low = [torch.zeros_like(a, dtype=torch.bfloat16) for a in p]
+    for step in (1, 2, 3):
+        g = [dev(f["g%d_%d" % (step, i)]).to(torch.bfloat16) for i in range(3)]
+        ops.lans(g + p + m + v, step, 1e-3, 0.9, 0.999, 1e-6, 1, 0.01, 1, 1, True, p_lowp=low)
+    for i in range(3):
+        want = f["p3_%d" % i]
+        assert np.abs(to_np(p[i]).astype(np.float64) - want).max() <= 1e-6 * np.abs(want).max()
+        assert torch.equal(low[i], p[i].to(torch.bfloat16))
+        ulp = (low[i].cpu().view(torch.int16).int() - torch.from_numpy(f["low3_%d" % i]).to(torch.bfloat16).view(torch.int16).int()).abs().max()
+        assert int(ulp) <= 1
+
+
 @pytest.mark.gpu
 def test_hip_path_reproduces_fixtures(pkg):
     import torch

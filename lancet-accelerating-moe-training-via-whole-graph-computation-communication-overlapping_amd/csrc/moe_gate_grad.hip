@@ -36,9 +36,14 @@ struct GateGradArgs {
 constexpr int kSub = 4;                      // lanes per token
 constexpr int kGradTokens = kTile / kSub;    // tokens per workgroup
 
-struct MaxSum {
+// Maximum and sum of exponentials of a row WITHOUT the entries that carry a slot gradient: with those the sum would
+// hide how far a selected probability is from 1 (1 - p = rest / sum loses every digit to rounding once the row is
+// peaked; kept apart it is exact to a few ulp, and with it the gradient p (1 - p) dy of a saturated gate).
+struct MaxSumRest {
   float top, sum;
-  __device__ __forceinline__ void operator()(float x) {
+  int skip1, skip2;
+  __device__ __forceinline__ void operator()(float x, int j) {
+    if (j == skip1 || j == skip2) return;
     if (x > top) {
       sum = sum * expf(top - x) + 1.f;   // top = -inf at first: exp(-inf) * 0 = 0
       top = x;
@@ -51,9 +56,10 @@ struct MaxSum {
 // per-token scalars of a workgroup's tokens, in LDS
 struct GateGradTile {
   int i1[kGradTokens], i2[kGradTokens];      // experts that receive a slot gradient (-1: none)
-  float d1[kGradTokens], d2[kGradTokens];    // gradient with respect to the raw value of that expert (probability or array entry)
+  // factor of the entry of expert i1 / i2 / of every other expert: the gradient with respect to that array entry
+  // (probabilities), or what p[e] is multiplied with (logits: d_j (1 - p_j) - p_other d_other, and -sum_j p_j d_j)
+  float c1[kGradTokens], c2[kGradTokens], rest[kGradTokens];
   float top[kGradTokens], inv[kGradTokens];  // logits: row maximum and 1 / sum_e exp(x - max)
-  float dot[kGradTokens];                    // logits: sum_j p[i_j] * d_j
 };
 
 template <int K, int GD>
@@ -68,9 +74,21 @@ __global__ __launch_bounds__(kTile) void encode_dgate_kernel(GateGradArgs a) {
   // ---- kSub lanes per token ---------------------------------------------------------------------------------
   {
     const char* row = static_cast<const char*>(a.gate) + static_cast<size_t>(s) * a.E * gb;
-    float top = 0.f, inv = 1.f;
+    int e[2] = {-1, -1};
+    float dy[2] = {0.f, 0.f}, raw[2] = {0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+      const int x = a.idx[static_cast<size_t>(j) * a.S + s];
+      if (x >= 0 && x < a.E) {
+        e[j] = x;
+        dy[j] = ld_gate(a.dy, static_cast<size_t>(j) * a.S + s, GD);
+        if (K == 2 || a.is_logits) raw[j] = gate_at<GD>(row, x);  // top-1 on probabilities needs no gate
+      }
+    }
+    float top = 0.f, inv = 1.f, rest = 0.f;  // rest: sum of exponentials of the entries without a slot gradient
+    float g[2] = {raw[0], raw[1]};           // the two kept probabilities (0 for a dropped slot)
     if (a.is_logits) {
-      MaxSum ms = {-INFINITY, 0.f};
+      MaxSumRest ms = {-INFINITY, 0.f, e[0], e[1]};
       if (a.vec) {
         const u32x4* r = reinterpret_cast<const u32x4*>(row);
         const int n = a.E / V;
@@ -78,12 +96,11 @@ __global__ __launch_bounds__(kTile) void encode_dgate_kernel(GateGradArgs a) {
           const u32x4 x0 = r[g0];
           const bool two = g0 + kSub < n;
           const u32x4 x1 = two ? r[g0 + kSub] : x0;
-          auto eat = [&](float x, int) { ms(x); };
-          walk_granule<GD>(x0, 0, eat);
-          if (two) walk_granule<GD>(x1, 0, eat);
+          walk_granule<GD>(x0, g0, ms);
+          if (two) walk_granule<GD>(x1, g0 + kSub, ms);
         }
       } else {
-        for (int j = sub; j < a.E; j += kSub) ms(gate_at<GD>(row, j));
+        for (int j = sub; j < a.E; j += kSub) ms(gate_at<GD>(row, j), j);
       }
       // merge the kSub lanes' (max, sum) pairs: they are neighbours in the wave
 #pragma unroll
@@ -95,20 +112,15 @@ __global__ __launch_bounds__(kTile) void encode_dgate_kernel(GateGradArgs a) {
         ms.top = nt;
       }
       top = ms.top;
-      inv = 1.f / ms.sum;
-    }
-    int e[2] = {-1, -1};
-    float dy[2] = {0.f, 0.f}, g[2] = {0.f, 0.f}, praw[2] = {0.f, 0.f};
-#pragma unroll
-    for (int j = 0; j < K; ++j) {
-      const int x = a.idx[static_cast<size_t>(j) * a.S + s];
-      if (x >= 0 && x < a.E) {
-        e[j] = x;
-        dy[j] = ld_gate(a.dy, static_cast<size_t>(j) * a.S + s, GD);
-        const float raw = (K == 2 || a.is_logits) ? gate_at<GD>(row, x) : 0.f;  // top-1 on probabilities needs no gate
-        praw[j] = a.is_logits ? expf(raw - top) * inv : raw;
-        g[j] = praw[j];
-      }
+      if (e[0] >= 0) top = fmaxf(top, raw[0]);
+      if (e[1] >= 0) top = fmaxf(top, raw[1]);
+      rest = ms.sum > 0.f ? ms.sum * expf(ms.top - top) : 0.f;
+      g[0] = e[0] >= 0 ? expf(raw[0] - top) : 0.f;   // exponentials for now, probabilities below
+      g[1] = e[1] >= 0 ? expf(raw[1] - top) : 0.f;
+      inv = 1.f / (rest + g[0] + g[1]);              // a row has at least one entry, and the largest one adds 1
+      rest *= inv;
+      g[0] *= inv;
+      g[1] *= inv;
     }
     float d[2] = {0.f, 0.f};
     if (K == 1) {
@@ -129,11 +141,17 @@ __global__ __launch_bounds__(kTile) void encode_dgate_kernel(GateGradArgs a) {
     if (sub == 0) {
       sh.i1[t] = e[0];
       sh.i2[t] = e[1];
-      sh.d1[t] = d[0];
-      sh.d2[t] = d[1];
       sh.top[t] = top;
       sh.inv[t] = inv;
-      sh.dot[t] = praw[0] * d[0] + praw[1] * d[1];
+      if (a.is_logits) {  // 1 - p_1 = rest + p_2 and 1 - p_2 = rest + p_1: sums of positive terms
+        sh.c1[t] = d[0] * (rest + g[1]) - g[1] * d[1];
+        sh.c2[t] = d[1] * (rest + g[0]) - g[0] * d[0];
+        sh.rest[t] = -(g[0] * d[0] + g[1] * d[1]);
+      } else {
+        sh.c1[t] = d[0];
+        sh.c2[t] = d[1];
+        sh.rest[t] = 0.f;
+      }
     }
   }
   __syncthreads();
@@ -141,11 +159,11 @@ __global__ __launch_bounds__(kTile) void encode_dgate_kernel(GateGradArgs a) {
   const int ntok = min(kGradTokens, a.S - first);
   const size_t base = static_cast<size_t>(first) * a.E;  // first element of the block
   auto value = [&](int tk, int ex, float x) -> float {
-    float sel = 0.f;
-    if (ex == sh.i1[tk]) sel = sh.d1[tk];
-    if (K == 2 && ex == sh.i2[tk]) sel = sh.d2[tk];
-    if (!a.is_logits) return sel;
-    return expf(x - sh.top[tk]) * sh.inv[tk] * (sel - sh.dot[tk]);
+    float c = sh.rest[tk];
+    if (ex == sh.i1[tk]) c = sh.c1[tk];
+    if (K == 2 && ex == sh.i2[tk]) c = sh.c2[tk];
+    if (!a.is_logits) return c;
+    return expf(x - sh.top[tk]) * sh.inv[tk] * c;
   };
   if (a.vec) {
     const int gpr = a.E / V;  // granules per row

@@ -35,7 +35,8 @@ Parity status of each function (what pins it, beyond re-reading the source):
   backward ops        torch autograd through dense einsum forms of the forward
   moe_encode_dgate    torch autograd through a dense restatement of top2gating
                       (docker/resources/sharded_moe.py:253-324: softmax, capacity masks, clamp,
-                      normalisation), incl. a case below the clamp
+                      normalisation), incl. a case below the clamp; peaked rows by the
+                      closed form of a two-expert softmax
 """
 import numpy as np
 
@@ -395,7 +396,8 @@ def moe_encode_dgate(dy_gates_s, gate, indloc, k=1, gate_is_logits=False):
     value (docker/resources/sharded_moe.py:296-312): g_j = p[s, i_j] * mask_j (masks after the capacity drop),
     w_j = g_j / clamp(g_1 + g_2, min=eps); torch.clamp passes the gradient where the sum is >= eps and none
     below.  With gate_is_logits the array holds logits and p = softmax(logits) (:260), differentiated too.
-    Pinned in tests/test_oracle_moe.py by torch autograd through a dense restatement of top2gating."""
+    Pinned in tests/test_oracle_moe.py by torch autograd through a dense restatement of top2gating, and for peaked
+    rows by the closed form of a two-expert softmax."""
     gate = np.asarray(gate, np.float64)
     S, E = gate.shape
     dy = np.asarray(dy_gates_s, np.float64)
@@ -424,7 +426,19 @@ def moe_encode_dgate(dy_gates_s, gate, indloc, k=1, gate_is_logits=False):
         np.add.at(dp, (rows, safe[j]), d[j])
     if not gate_is_logits:
         return dp
-    return p * (dp - (p * dp).sum(axis=1, keepdims=True))
+    out = p * (dp - (p * dp).sum(axis=1, keepdims=True))
+    # The entries that carry a slot gradient again, without 1 - p_j as a difference: in a peaked row (p_j within
+    # 1e-11 of 1) that difference loses five of fp64's digits.  1 - p_j is the sum of the OTHER exponentials over
+    # the whole sum, and d_j (1 - p_j) - sum_{l != j} p_l d_l is the same number as d_j - sum_l p_l d_l.
+    tot = ex.sum(axis=1)
+    for j in range(k):
+        others = ex.copy()
+        others[rows, safe[j]] = 0.0
+        rest = others.sum(axis=1) / tot
+        cross = sum((p[rows, safe[l]] * d[l] for l in range(k) if l != j), np.zeros(S))
+        val = p[rows, safe[j]] * (d[j] * rest - cross)
+        out[rows[kept[j]], safe[j][kept[j]]] = val[kept[j]]
+    return out
 
 
 def moe_decode_dx(dy, gates_s, indloc, n_experts, capacity, k=1, round_fn=None):

@@ -161,6 +161,33 @@ def test_gate_gradient_below_the_clamp_and_for_large_logits(pkg):
     _check_gate_gradient(pkg, logits, il, 2, True, "f32", 5)
 
 
+@pytest.mark.parametrize("scale", [4.0, 12.0, 30.0])
+def test_gate_gradient_of_peaked_rows_keeps_its_relative_accuracy(pkg, scale):
+    """Top-1 on logits whose rows are peaked (the selected probability within 1e-3 ... 1e-30 of 1): the gradient
+    of the selected logit is dy p (1 - p).  The kernel forms 1 - p from the sum of the other exponentials, not as
+    a difference, so EVERY entry stays within 2e-5 relative of the oracle, with no floor tied to the row (a plain
+    fp32 softmax backward is off by 6e-8 / (1 - p) there); 1e-37 covers results that underflow."""
+    S, E = 2048, 32
+    _, logits = make_inputs(int(scale), S, 1, E, logit_scale=scale)
+    il = mo.moe_encode(np.zeros((S, 1), np.float32), logits, np.zeros(E, np.int32), 0.9, gate_is_logits=True, fast_scatter=True)[1]
+    p_top = mo.softmax_rows(logits).max(axis=1)
+    assert (p_top > 1 - 1e-4).sum() >= (50 if scale > 4 else 0)
+    dy = np.random.default_rng(9).standard_normal(S).astype(np.float32)
+    got = to_np(pkg.ops.moe_encode_dgate(dev(dy), dev(logits), dev(il), top_k=1, gate_is_logits=True))
+    want = mo.moe_encode_dgate(dy, logits, il, 1, True)
+    np.testing.assert_allclose(got, want, rtol=2e-5, atol=1e-37)
+    # two experts: the closed form dy exp(-t) / (1 + exp(-t))^2 for the selected logit, its negative for the other
+    t = np.linspace(0.25, 80.0, 320).astype(np.float32)
+    two = np.stack([np.zeros_like(t), t], axis=1)
+    il2 = np.array([[1] * t.size, list(range(t.size))], np.int32)
+    dy2 = np.random.default_rng(10).standard_normal(t.size).astype(np.float32)
+    got = to_np(pkg.ops.moe_encode_dgate(dev(dy2), dev(two), dev(il2), top_k=1, gate_is_logits=True))
+    z = np.exp(-t.astype(np.float64))
+    sel = dy2 * z / (1 + z) ** 2
+    np.testing.assert_allclose(got[:, 1], sel, rtol=2e-5, atol=1e-37)
+    np.testing.assert_allclose(got[:, 0], -sel, rtol=2e-5, atol=1e-37)
+
+
 def test_backward_matches_autograd_through_forward_ops(pkg):
     """End to end: gradients of sum(decode(expert(encode(x))) * Y) with an elementwise expert, taken
     with the backward ops, against torch autograd of the same computation written with torch indexing."""

@@ -423,6 +423,32 @@ def test_gate_gradient_below_the_clamp_of_the_denominator():
     np.testing.assert_allclose(mo.moe_encode_dgate(w, gate, il, 2, False), x.grad.numpy(), rtol=1e-9, atol=0)
 
 
+def test_gate_gradient_of_peaked_rows_has_the_closed_form_of_a_two_expert_softmax():
+    """Two experts, logits (t, 0) with t up to 60: p1 = 1 / (1 + exp(-t)) and the gradient of the selected logit is
+    dy p1 (1 - p1) = dy exp(-t) / (1 + exp(-t))^2, of the other one its negative; neither form subtracts.
+    Evaluating p (dp - sum p dp) as written would be off by 1e-16 / (1 - p1): 2e-5 at t = 27, everything at t = 40."""
+    t = np.array([0.5, 3.0, 12.0, 27.0, 40.0, 60.0])
+    S = t.size
+    logits = np.stack([t, np.zeros(S)], axis=1).astype(np.float32)
+    il = np.array([[0] * S, list(range(S))], np.int32)
+    dy = np.linspace(-2, 3, S).astype(np.float32)
+    z = np.exp(-t)
+    sel = dy.astype(np.float64) * z / (1 + z) ** 2
+    got = mo.moe_encode_dgate(dy, logits, il, 1, True)
+    np.testing.assert_allclose(got[:, 0], sel, rtol=1e-13, atol=0)
+    np.testing.assert_allclose(got[:, 1], -sel, rtol=1e-13, atol=0)
+    # top-2, both kept: w1 = p1 / (p1 + p2) = 1 / (1 + exp(-t)) again (a third expert far below changes nothing
+    # in the ratio), so d logit1 = (dy1 - dy2) exp(-t) / (1 + exp(-t))^2, d logit2 its negative, d logit3 = 0
+    logits3 = np.concatenate([logits, np.full((S, 1), -5.0, np.float32)], axis=1)
+    il2 = np.array([[0] * S + [1] * S, list(range(S)) * 2], np.int32)
+    dy2 = np.concatenate([dy, dy[::-1] * np.float32(0.5)]).astype(np.float32)
+    sel2 = (dy2[:S].astype(np.float64) - dy2[S:]) * z / (1 + z) ** 2
+    got = mo.moe_encode_dgate(dy2, logits3, il2, 2, True)
+    np.testing.assert_allclose(got[:, 0], sel2, rtol=1e-12, atol=0)
+    np.testing.assert_allclose(got[:, 1], -sel2, rtol=1e-12, atol=0)
+    assert np.abs(got[:, 2]).max() <= 1e-15 * np.abs(sel2).max()
+
+
 # ---------------------------------------------------------------- redispatch_expert_input
 @pytest.mark.parametrize("P", [2, 4])
 def test_redispatch_expert_input_partitioned_equals_whole(P):

@@ -1084,6 +1084,21 @@ struct lancet_lans_plan {
 static constexpr uint32_t kPlanMagic = 0x4c414e53u;  // "LANS"
 static constexpr uint32_t kDefaultSpinLimit = 1u << 20;  // about a second of polling; a healthy wait is microseconds
 
+// GT / PL as compile-time constants inside `...` for the run-time codes gt (LANCET_F32 / _BF16 / _F16) and pl (the
+// same 16-bit codes, or kNoLowp)
+#define LANS_TYPE_SWITCH(gt, pl, ...)                                                                      \
+  switch ((gt) * 4 + ((pl) == kNoLowp ? 0 : (pl))) {                                                       \
+    case LANCET_F32 * 4 + 0: { constexpr int GT = LANCET_F32, PL = kNoLowp; (void)PL; __VA_ARGS__; } break;          \
+    case LANCET_F32 * 4 + LANCET_BF16: { constexpr int GT = LANCET_F32, PL = LANCET_BF16; (void)PL; __VA_ARGS__; } break;   \
+    case LANCET_F32 * 4 + LANCET_F16: { constexpr int GT = LANCET_F32, PL = LANCET_F16; (void)PL; __VA_ARGS__; } break;     \
+    case LANCET_BF16 * 4 + 0: { constexpr int GT = LANCET_BF16, PL = kNoLowp; (void)PL; __VA_ARGS__; } break;        \
+    case LANCET_BF16 * 4 + LANCET_BF16: { constexpr int GT = LANCET_BF16, PL = LANCET_BF16; (void)PL; __VA_ARGS__; } break; \
+    case LANCET_BF16 * 4 + LANCET_F16: { constexpr int GT = LANCET_BF16, PL = LANCET_F16; (void)PL; __VA_ARGS__; } break;   \
+    case LANCET_F16 * 4 + 0: { constexpr int GT = LANCET_F16, PL = kNoLowp; (void)PL; __VA_ARGS__; } break;          \
+    case LANCET_F16 * 4 + LANCET_BF16: { constexpr int GT = LANCET_F16, PL = LANCET_BF16; (void)PL; __VA_ARGS__; } break;   \
+    default: { constexpr int GT = LANCET_F16, PL = LANCET_F16; (void)PL; __VA_ARGS__; } break;                       \
+  }
+
 static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 static inline int chunks_of(int64_t numel) { return static_cast<int>((numel + kLansChunk - 1) / kLansChunk); }
 
@@ -1174,14 +1189,18 @@ extern "C" int lancet_lans_plan_create(const int64_t* numels, int T, lancet_lans
   pl->max_tensor_chunks = 0;
   for (int i = 0; i < T; ++i) pl->max_tensor_chunks = std::max(pl->max_tensor_chunks, chunks_of(numels[i]));
   if (err == hipSuccess) {
-    int per_cu = 0;
-    // every variant of the kernel has the same launch bounds and LDS; the grid follows the variant that reads and
-    // writes the most (16-bit gradients in, 16-bit parameter copies out)
-    err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lans_resident_kernel<LANCET_F32, kNoLowp>, kLansThreads, 0);
-    int per_cu_mixed = 0;
-    if (err == hipSuccess)
-      err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_mixed, lans_resident_kernel<LANCET_BF16, LANCET_BF16>, kLansThreads, 0);
-    per_cu = std::min(per_cu, per_cu_mixed);
+    // every variant of the kernel has the same launch bounds and LDS but its own register count: the grid is what
+    // the variant with the fewest workgroups per CU runs at once, so that whichever variant a step launches, all of
+    // its workgroups are on the chip together (the waits between them rely on that)
+    int per_cu = 1 << 30;
+    for (int gt : {LANCET_F32, LANCET_BF16, LANCET_F16})
+      for (int plt : {static_cast<int>(kNoLowp), static_cast<int>(LANCET_BF16), static_cast<int>(LANCET_F16)}) {
+        int n = 0;
+        LANS_TYPE_SWITCH(gt, plt, if (err == hipSuccess) err = hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                                      &n, lans_resident_kernel<GT, PL>, kLansThreads, 0))
+        per_cu = std::min(per_cu, n);
+      }
+    if (err != hipSuccess) per_cu = 0;
     pl->resident_grid = per_cu * cus;
   }
   // a tensor's chunks fit one round, so the kernel drains with half of its workgroups on the chip
@@ -1285,21 +1304,6 @@ extern "C" int lancet_lans_plan_norms(lancet_lans_plan_t pl, float* norms, lance
 }
 
 namespace {
-
-// GT / PL as compile-time constants inside `...` for the run-time codes gt (LANCET_F32 / _BF16 / _F16) and pl (the
-// same 16-bit codes, or kNoLowp)
-#define LANS_TYPE_SWITCH(gt, pl, ...)                                                                      \
-  switch ((gt) * 4 + ((pl) == kNoLowp ? 0 : (pl))) {                                                       \
-    case LANCET_F32 * 4 + 0: { constexpr int GT = LANCET_F32, PL = kNoLowp; (void)PL; __VA_ARGS__; } break;          \
-    case LANCET_F32 * 4 + LANCET_BF16: { constexpr int GT = LANCET_F32, PL = LANCET_BF16; (void)PL; __VA_ARGS__; } break;   \
-    case LANCET_F32 * 4 + LANCET_F16: { constexpr int GT = LANCET_F32, PL = LANCET_F16; (void)PL; __VA_ARGS__; } break;     \
-    case LANCET_BF16 * 4 + 0: { constexpr int GT = LANCET_BF16, PL = kNoLowp; (void)PL; __VA_ARGS__; } break;        \
-    case LANCET_BF16 * 4 + LANCET_BF16: { constexpr int GT = LANCET_BF16, PL = LANCET_BF16; (void)PL; __VA_ARGS__; } break; \
-    case LANCET_BF16 * 4 + LANCET_F16: { constexpr int GT = LANCET_BF16, PL = LANCET_F16; (void)PL; __VA_ARGS__; } break;   \
-    case LANCET_F16 * 4 + 0: { constexpr int GT = LANCET_F16, PL = kNoLowp; (void)PL; __VA_ARGS__; } break;          \
-    case LANCET_F16 * 4 + LANCET_BF16: { constexpr int GT = LANCET_F16, PL = LANCET_BF16; (void)PL; __VA_ARGS__; } break;   \
-    default: { constexpr int GT = LANCET_F16, PL = LANCET_F16; (void)PL; __VA_ARGS__; } break;                       \
-  }
 
 int lans_step_impl(lancet_lans_plan_t pl, const void* const* g, int g_dtype, float* const* p, float* const* m,
                    float* const* v, void* const* p_lowp, int lowp_dtype, int step_host, const float* step_dev,

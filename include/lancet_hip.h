@@ -93,7 +93,7 @@ typedef void* lancet_stream_t;
 int lancet_abi_version(void);
 const char* lancet_status_string(int status);
 
-/* Capacity C = int(float(cf) * ((S + E - 1) / E)).
+/* Capacity C = int(float(cf) * ((S + E - 1) / E)); -1 for E <= 0, S < 0 or a product that no int holds.
  * Replaces: src/op/dialect/cuda/moe.cc:107-109, src/op/declare/moe.cc:46, src/op/ty/moe.cc:50. */
 int64_t lancet_moe_capacity(int64_t S, int64_t E, float capacity_factor);
 

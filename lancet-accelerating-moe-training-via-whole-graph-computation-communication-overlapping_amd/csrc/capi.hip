@@ -65,8 +65,11 @@ extern "C" const char* lancet_status_string(int status) {
 
 extern "C" int64_t lancet_moe_capacity(int64_t S, int64_t E, float capacity_factor) {
   if (E <= 0 || S < 0) return -1;
-  // float * integer in float, truncated: src/op/dialect/cuda/moe.cc:109
-  return static_cast<int64_t>(static_cast<int>(capacity_factor * static_cast<float>((S + E - 1) / E)));
+  // float * integer in float, truncated: src/op/dialect/cuda/moe.cc:109.  A product that no int holds (or a NaN
+  // factor) has no capacity: -1, which every entry point that takes a capacity rejects.
+  const float c = capacity_factor * static_cast<float>(S / E + (S % E != 0));
+  if (!(c > -2147483648.f && c < 2147483648.f)) return -1;
+  return static_cast<int64_t>(static_cast<int>(c));
 }
 
 extern "C" int lancet_debug_scan_workspace_spin_limit(void* workspace, unsigned limit, lancet_stream_t stream) {

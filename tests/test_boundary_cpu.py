@@ -35,6 +35,11 @@ def test_capacity_formula(pkg):
     cap = pkg.ops.moe_capacity
     assert cap(4096, 8, 1.25) == 640 and cap(16384, 16, 2.0) == 2048 and cap(32768, 64, 1.25) == 640
     assert cap(65536, 32, 2.5) == 5120 and cap(16384, 32, 10.0) == 5120 and cap(10, 4, 1.5) == 4
+    # no capacity: no experts, a negative token count, a product that no int holds, a factor that is no number
+    assert cap(16, 0, 1.0) == -1 and cap(-1, 4, 1.0) == -1 and cap(2 ** 62, 1, 3.0e30) == -1
+    assert cap(1 << 40, 1, 1.0) == -1 and cap(16, 4, float("nan")) == -1 and cap(16, 4, float("inf")) == -1
+    # the ceiling division itself cannot overflow
+    assert cap(2 ** 63 - 1, 3, 1e-10) == int(np.float32(1e-10) * np.float32((2 ** 63 - 1 + 2) // 3))
 
 
 def test_workspace_sizes_and_argument_rejection(pkg):

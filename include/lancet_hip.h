@@ -354,7 +354,7 @@ int lancet_moe_redispatch(const void* const* data, const int32_t* const* indices
  * Replaces LansImpl (src/op/dialect/cuda/lans.cc:26-180) and multi_tensor_lans_cuda
  * (kernel_util.cuh:25-33; multi_tensor_lans.cu:401-450).  A plan captures the tensor sizes of
  * one parameter set (what the LansImpl constructor captures) and owns the chunk tables,
- * per-chunk partial sums and norm vectors; it is created once and reused every step.
+ * per-chunk partial sums and norm vectors; it is created once and reused every step (T >= 1; a tensor may be empty).
  * g/p/m/v are HOST arrays of T device pointers to fp32 tensors (the four quarters of the
  * reference's tensor_list).  p, m, v are updated in place; g is not modified.
  * step: pass step_host >= 1, or a device pointer step_dev to the fp32 step scalar the
